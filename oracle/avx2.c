@@ -1,0 +1,578 @@
+// TEST INFRASTRUCTURE ONLY (see ora_common.h). AVX2+FMA+F16C restatement of the reference's vector kernels, in
+// their instruction order: the two activation encoders and the Q4_K / Q6_K / IQ2_XXS row dots, one column or a
+// tile of up to eight columns that unpacks each weight block once. It has two uses: the test suite holds it
+// bit-equal to the scalar restatement in qdot.c (two independently written paths through the same arithmetic,
+// the reference's own first gate, crates/qdot/tests/qdot.rs:346,738,818,2664), and the benchmark times it as the
+// CPU baseline. Build with -mavx2 -mfma -mf16c -ffp-contract=off.
+#include <immintrin.h>
+#include <pthread.h>
+#include <stdlib.h>
+
+#include "bm_oracle.h"
+#include "bm_oracle_avx2.h"
+#include "iq_tables.h"
+#include "ora_common.h"
+
+int ora_avx2_supported(void) {
+    return __builtin_cpu_supports("avx2") && __builtin_cpu_supports("fma") && __builtin_cpu_supports("f16c");
+}
+
+// ------------------------------------------------------------------------------------------------- small helpers
+
+// crates/qdot/src/lib.rs:1822-1832.
+static inline __m256i v_nearest_int(__m256 y) {
+    __m256 z = _mm256_add_ps(y, _mm256_set1_ps(12582912.0f));
+    __m256i b = _mm256_castps_si256(z);
+    return _mm256_sub_epi32(_mm256_and_si256(b, _mm256_set1_epi32(0x007fffff)), _mm256_set1_epi32(0x00400000));
+}
+
+// crates/qdot/src/lib.rs:1844-1851.
+static inline __m256i v_wrap_i8(__m256i q) {
+    __m256i t = _mm256_and_si256(q, _mm256_set1_epi32(0xFF));
+    __m256i ge = _mm256_cmpgt_epi32(t, _mm256_set1_epi32(127));
+    return _mm256_sub_epi32(t, _mm256_and_si256(ge, _mm256_set1_epi32(256)));
+}
+
+// crates/qdot/src/lib.rs:1862-1871.
+static inline float hmax_ps(__m256 v) {
+    __m128 lo = _mm256_castps256_ps128(v), hi = _mm256_extractf128_ps(v, 1);
+    __m128 m = _mm_max_ps(lo, hi);
+    m = _mm_max_ps(m, _mm_movehl_ps(m, m));
+    return _mm_cvtss_f32(_mm_max_ss(m, _mm_movehdup_ps(m)));
+}
+
+// crates/qdot/src/lib.rs:1978-1986.
+static inline int32_t hsum_i32(__m256i v) {
+    __m128i lo = _mm_add_epi32(_mm256_castsi256_si128(v), _mm256_extracti128_si256(v, 1));
+    lo = _mm_add_epi32(lo, _mm_shuffle_epi32(lo, 0x4E));
+    lo = _mm_add_epi32(lo, _mm_shuffle_epi32(lo, 0x8D));
+    return _mm_cvtsi128_si32(lo);
+}
+
+// crates/qdot/src/lib.rs:4128-4137. The order is load-bearing.
+static inline float hsum_float_8(__m256 x) {
+    __m128 res = _mm256_extractf128_ps(x, 1);
+    res = _mm_add_ps(res, _mm256_castps256_ps128(x));
+    res = _mm_add_ps(res, _mm_movehl_ps(res, res));
+    res = _mm_add_ss(res, _mm_movehdup_ps(res));
+    return _mm_cvtss_f32(res);
+}
+
+static inline float f16c_to_f32(uint16_t h) { return _mm_cvtss_f32(_mm_cvtph_ps(_mm_cvtsi32_si128(h))); }
+
+// ------------------------------------------------------------------------------------------- activation encoders
+
+// One 32-value q8_2 block (crates/qdot/src/lib.rs:3953-4002 under the bf16 rule, :3930-3939).
+static int q82_block_avx2(const float *x, uint8_t *codes, uint16_t *t_out, int16_t *isum_out) {
+    const __m256 sgn = _mm256_set1_ps(-0.0f);
+    __m256 m = _mm256_setzero_ps(), unord = _mm256_setzero_ps();
+    for (int j = 0; j < 4; j++) {
+        __m256 v = _mm256_loadu_ps(x + 8 * j);
+        m = _mm256_max_ps(_mm256_andnot_ps(sgn, v), m);
+        unord = _mm256_or_ps(unord, _mm256_cmp_ps(v, v, _CMP_UNORD_Q));
+    }
+    float amax = hmax_ps(m);
+    if (_mm256_movemask_ps(unord) != 0 || !isfinite(amax)) return ORA_ENONFINITE;
+    uint16_t t = ora_fp32_to_bf16_bits(amax / 127.0f);
+    __m256 idv = _mm256_set1_ps(ora_q82_inverse(t));
+    __m256i qi[4];
+    for (int j = 0; j < 4; j++) qi[j] = v_nearest_int(_mm256_mul_ps(_mm256_loadu_ps(x + 8 * j), idv));
+    __m256i p0 = _mm256_packs_epi32(qi[0], qi[1]), p1 = _mm256_packs_epi32(qi[2], qi[3]);
+    __m256i c = _mm256_packs_epi16(p0, p1);
+    c = _mm256_permutevar8x32_epi32(c, _mm256_setr_epi32(0, 4, 1, 5, 2, 6, 3, 7));
+    _mm256_storeu_si256((__m256i *)codes, c);
+    *t_out = t;
+    *isum_out =
+        (int16_t)hsum_i32(_mm256_add_epi32(_mm256_add_epi32(qi[0], qi[1]), _mm256_add_epi32(qi[2], qi[3])));
+    return 0;
+}
+
+// crates/qdot/src/lib.rs:4014-4036 (whole groups).
+int ora_avx2_quantize_q82x4(const float *x, int k, uint8_t *out) {
+    if (k <= 0 || k % 128 != 0) return ORA_EUNALIGNED;
+    for (int gi = 0; gi < k / 128; gi++) {
+        uint8_t *group = out + (size_t)gi * ORA_Q82X4_STRIDE;
+        memset(group, 0, ORA_Q82X4_STRIDE);
+        for (int ir = 0; ir < 4; ir++) {
+            uint16_t d;
+            int16_t isum;
+            int rc = q82_block_avx2(x + 128 * gi + 32 * ir, group + 16 + 32 * ir, &d, &isum);
+            if (rc) return rc;
+            ora_wr16(group + 2 * ir, d);
+            ora_wr16(group + 8 + 2 * ir, (uint16_t)isum);
+        }
+    }
+    return 0;
+}
+
+// crates/qdot/src/lib.rs:1885-1955.
+int ora_avx2_quantize_q8k(const float *x, int k, uint8_t *out) {
+    if (k <= 0 || k % 256 != 0) return ORA_EUNALIGNED;
+    const __m256 sgn = _mm256_set1_ps(-0.0f);
+    for (int b = 0; b < k / 256; b++) {
+        const float *xb = x + 256 * b;
+        uint8_t *o = out + (size_t)b * ORA_Q8K_STRIDE;
+        __m256 m = _mm256_setzero_ps(), unord = _mm256_setzero_ps();
+        for (int i = 0; i < 32; i++) {
+            __m256 v = _mm256_loadu_ps(xb + 8 * i);
+            m = _mm256_max_ps(_mm256_andnot_ps(sgn, v), m);
+            unord = _mm256_or_ps(unord, _mm256_cmp_ps(v, v, _CMP_UNORD_Q));
+        }
+        float amax = hmax_ps(m);
+        if (_mm256_movemask_ps(unord) != 0 || !isfinite(amax)) return ORA_ENONFINITE;
+        if (amax == 0.0f) {
+            memset(o, 0, ORA_Q8K_STRIDE);
+            continue;
+        }
+        __m256 amax_v = _mm256_set1_ps(amax);
+        int first = 256;
+        for (int i = 0; i < 32 && first == 256; i++) {
+            __m256 v = _mm256_loadu_ps(xb + 8 * i);
+            unsigned mask = (unsigned)_mm256_movemask_ps(_mm256_cmp_ps(_mm256_andnot_ps(sgn, v), amax_v, _CMP_EQ_OQ));
+            if (mask) first = 8 * i + __builtin_ctz(mask);
+        }
+        float max = xb[first];
+        float iscale = -127.0f / max;
+        __m256 iscale_v = _mm256_set1_ps(iscale);
+        __m256i clamp = _mm256_set1_epi32(127);
+        for (int g = 0; g < 8; g++) {
+            __m256i qi[4];
+            for (int j = 0; j < 4; j++) {
+                __m256 y = _mm256_mul_ps(_mm256_loadu_ps(xb + 32 * g + 8 * j), iscale_v);
+                qi[j] = v_wrap_i8(_mm256_min_epi32(v_nearest_int(y), clamp));
+            }
+            __m256i p0 = _mm256_packs_epi32(qi[0], qi[1]), p1 = _mm256_packs_epi32(qi[2], qi[3]);
+            __m256i c = _mm256_packs_epi16(p0, p1);
+            c = _mm256_permutevar8x32_epi32(c, _mm256_setr_epi32(0, 4, 1, 5, 2, 6, 3, 7));
+            _mm256_storeu_si256((__m256i *)(o + 8 + 32 * g), c);
+            ora_wr16(o + 264 + 4 * g, (uint16_t)(int16_t)hsum_i32(_mm256_add_epi32(qi[0], qi[1])));
+            ora_wr16(o + 266 + 4 * g, (uint16_t)(int16_t)hsum_i32(_mm256_add_epi32(qi[2], qi[3])));
+        }
+        float d = 1.0f / iscale;
+        memcpy(o, &d, 4);
+        memset(o + 4, 0, 4);
+    }
+    return 0;
+}
+
+int ora_avx2_quantize_col(int wtype, const float *x, int k, uint8_t *out) {
+    if (wtype == ORA_TYPE_Q4_K || wtype == ORA_TYPE_Q6_K) return ora_avx2_quantize_q82x4(x, k, out);
+    if (wtype == ORA_TYPE_IQ2_XXS) return ora_avx2_quantize_q8k(x, k, out);
+    return ORA_ETYPE;
+}
+
+// --------------------------------------------------------------------------------------------- shared dot pieces
+
+// The eight bf16 block scales of super-block i's two groups as f32 (crates/qdot/src/lib.rs:4149-4158).
+static inline __m256 q82x4_dy(const uint8_t *col, int i) {
+    const uint8_t *g0 = col + (size_t)(2 * i) * ORA_Q82X4_STRIDE, *g1 = g0 + ORA_Q82X4_STRIDE;
+    __m128i d4_1 = _mm_cvtepu16_epi32(_mm_loadl_epi64((const __m128i *)g0));
+    __m128i d4_2 = _mm_cvtepu16_epi32(_mm_loadl_epi64((const __m128i *)g1));
+    return _mm256_castsi256_ps(_mm256_slli_epi32(_mm256_set_m128i(d4_2, d4_1), 16));
+}
+
+// dy times the blocks' i16 sums (crates/qdot/src/lib.rs:4160-4168).
+static inline __m256 q82x4_my(const uint8_t *col, int i, __m256 dy) {
+    const uint8_t *g0 = col + (size_t)(2 * i) * ORA_Q82X4_STRIDE, *g1 = g0 + ORA_Q82X4_STRIDE;
+    __m128i m4_1 = _mm_cvtepi16_epi32(_mm_loadl_epi64((const __m128i *)(g0 + 8)));
+    __m128i m4_2 = _mm_cvtepi16_epi32(_mm_loadl_epi64((const __m128i *)(g1 + 8)));
+    return _mm256_mul_ps(dy, _mm256_cvtepi32_ps(_mm256_set_m128i(m4_2, m4_1)));
+}
+
+// Four maddubs results of a 128-value half reduced to eight i32 lanes: lane t the first 16 values of 32-block t,
+// lane 4 + t the second 16 (crates/qdot/src/lib.rs:4251-4261).
+static inline __m256i reduce4(__m256i s1, __m256i s2, __m256i s3, __m256i s4) {
+    __m256i t1 = _mm256_add_epi16(_mm256_unpacklo_epi32(s1, s2), _mm256_unpackhi_epi32(s1, s2));
+    __m256i t3 = _mm256_add_epi16(_mm256_unpacklo_epi32(s3, s4), _mm256_unpackhi_epi32(s3, s4));
+    __m256i t = _mm256_add_epi16(_mm256_unpacklo_epi64(t1, t3), _mm256_unpackhi_epi64(t1, t3));
+    return _mm256_madd_epi16(_mm256_set1_epi16(1), t);
+}
+
+static inline void q4_unpack_scales(const uint8_t *s12, uint32_t utmp[4]) {
+    uint32_t a0, a1, a2;
+    memcpy(&a0, s12, 4);
+    memcpy(&a1, s12 + 4, 4);
+    memcpy(&a2, s12 + 8, 4);
+    utmp[0] = a0 & 0x3f3f3f3fu;
+    utmp[1] = (a2 & 0x0f0f0f0fu) | ((a0 >> 2) & 0x30303030u);
+    utmp[2] = a1 & 0x3f3f3f3fu;
+    utmp[3] = ((a2 >> 4) & 0x0f0f0f0fu) | ((a1 >> 2) & 0x30303030u);
+}
+
+// -------------------------------------------------------------------------------------------------- Q4_K tile
+
+// One Q4_K row against C <= 8 columns, each column the one-column kernel's steps
+// (crates/qdot/src/lib.rs:4203-4272): weights unpacked once per block.
+static void dot_q4k_tile(const uint8_t *wrow, const uint8_t *const *acols, int C, int nb, float *out) {
+    const __m256i ml = _mm256_set1_epi8(0xF);
+    __m256 accd[8];
+    for (int c = 0; c < C; c++) accd[c] = _mm256_setzero_ps();
+    for (int i = 0; i < nb; i++) {
+        const uint8_t *wb = wrow + (size_t)i * ORA_Q4K_BLOCK;
+        uint16_t dh, mh;
+        memcpy(&dh, wb, 2);
+        memcpy(&mh, wb + 2, 2);
+        float d = f16c_to_f32(dh), dmin = f16c_to_f32(mh);
+        uint32_t utmp[4];
+        q4_unpack_scales(wb + 4, utmp);
+        __m256 mins_v = _mm256_cvtepi32_ps(_mm256_cvtepu8_epi32(_mm_loadl_epi64((const __m128i *)(utmp + 2))));
+        __m256 mins = _mm256_mul_ps(_mm256_set1_ps(-dmin), mins_v);
+        __m256 all_scales = _mm256_mul_ps(
+            _mm256_set1_ps(d), _mm256_cvtepi32_ps(_mm256_cvtepu8_epi32(_mm_loadl_epi64((const __m128i *)utmp))));
+        __m128 lo = _mm256_castps256_ps128(all_scales), hi = _mm256_extractf128_ps(all_scales, 1);
+        __m256 scales[2] = {_mm256_set_m128(lo, lo), _mm256_set_m128(hi, hi)};
+        __m256i values[2][4];
+        for (int j = 0; j < 2; j++) {
+            __m256i bits0 = _mm256_loadu_si256((const __m256i *)(wb + 16 + 64 * j));
+            __m256i bits1 = _mm256_loadu_si256((const __m256i *)(wb + 16 + 64 * j + 32));
+            values[j][0] = _mm256_and_si256(bits0, ml);
+            values[j][1] = _mm256_and_si256(_mm256_srli_epi16(bits0, 4), ml);
+            values[j][2] = _mm256_and_si256(bits1, ml);
+            values[j][3] = _mm256_and_si256(_mm256_srli_epi16(bits1, 4), ml);
+        }
+        for (int c = 0; c < C; c++) {
+            const uint8_t *acol = acols[c];
+            __m256 dy = q82x4_dy(acol, i);
+            __m256 my = q82x4_my(acol, i, dy);
+            __m128 dy4[2] = {_mm256_castps256_ps128(dy), _mm256_extractf128_ps(dy, 1)};
+            __m256 sumi_f[2], d4d8[2];
+            for (int j = 0; j < 2; j++) {
+                d4d8[j] = _mm256_mul_ps(scales[j], _mm256_set_m128(dy4[j], dy4[j]));
+                const uint8_t *qs = acol + (size_t)(2 * i + j) * ORA_Q82X4_STRIDE + 16;
+                __m256i s1 = _mm256_maddubs_epi16(values[j][0], _mm256_loadu_si256((const __m256i *)qs));
+                __m256i s2 = _mm256_maddubs_epi16(values[j][1], _mm256_loadu_si256((const __m256i *)(qs + 32)));
+                __m256i s3 = _mm256_maddubs_epi16(values[j][2], _mm256_loadu_si256((const __m256i *)(qs + 64)));
+                __m256i s4 = _mm256_maddubs_epi16(values[j][3], _mm256_loadu_si256((const __m256i *)(qs + 96)));
+                sumi_f[j] = _mm256_cvtepi32_ps(reduce4(s1, s2, s3, s4));
+            }
+            accd[c] = _mm256_fmadd_ps(my, mins, accd[c]);
+            accd[c] = _mm256_fmadd_ps(d4d8[0], sumi_f[0], accd[c]);
+            accd[c] = _mm256_fmadd_ps(d4d8[1], sumi_f[1], accd[c]);
+        }
+    }
+    for (int c = 0; c < C; c++) out[c] = hsum_float_8(accd[c]);
+}
+
+// -------------------------------------------------------------------------------------------------- Q6_K tile
+
+static const uint8_t K_SHUFFLE_Q6K[32] = {0, 1, 4, 5, 8, 9, 12, 13, 2, 3, 6, 7, 10, 11, 14, 15,
+                                          0, 1, 4, 5, 8, 9, 12, 13, 2, 3, 6, 7, 10, 11, 14, 15};
+
+// One Q6_K row against C <= 8 columns (crates/qdot/src/lib.rs:4469-4579).
+static void dot_q6k_tile(const uint8_t *wrow, const uint8_t *const *acols, int C, int nb, float *out) {
+    const __m256i ml = _mm256_set1_epi8(0xF), mh = _mm256_set1_epi8(0x30), m32n = _mm256_set1_epi8(-32);
+    const __m256i shuff = _mm256_loadu_si256((const __m256i *)K_SHUFFLE_Q6K);
+    __m256 accd[8];
+    for (int c = 0; c < C; c++) accd[c] = _mm256_setzero_ps();
+    for (int i = 0; i < nb; i++) {
+        const uint8_t *wb = wrow + (size_t)i * ORA_Q6K_BLOCK;
+        uint16_t dh;
+        memcpy(&dh, wb + 208, 2);
+        __m256 vd = _mm256_set1_ps(f16c_to_f32(dh));
+        __m256i sc16 =
+            _mm256_shuffle_epi8(_mm256_cvtepi8_epi16(_mm_loadu_si128((const __m128i *)(wb + 192))), shuff);
+        __m256 wscales[2] = {
+            _mm256_mul_ps(vd, _mm256_cvtepi32_ps(_mm256_cvtepi16_epi32(_mm256_castsi256_si128(sc16)))),
+            _mm256_mul_ps(vd, _mm256_cvtepi32_ps(_mm256_cvtepi16_epi32(_mm256_extracti128_si256(sc16, 1))))};
+        __m256i values[2][4], us[2][4];
+        for (int j = 0; j < 2; j++) {
+            __m256i lbits1 = _mm256_loadu_si256((const __m256i *)(wb + 64 * j));
+            __m256i lbits2 = _mm256_loadu_si256((const __m256i *)(wb + 64 * j + 32));
+            __m256i hbits = _mm256_loadu_si256((const __m256i *)(wb + 128 + 32 * j));
+            values[j][0] = _mm256_or_si256(_mm256_and_si256(lbits1, ml), _mm256_and_si256(_mm256_slli_epi16(hbits, 4), mh));
+            values[j][1] = _mm256_or_si256(_mm256_and_si256(lbits2, ml), _mm256_and_si256(_mm256_slli_epi16(hbits, 2), mh));
+            values[j][2] = _mm256_or_si256(_mm256_and_si256(_mm256_srli_epi16(lbits1, 4), ml), _mm256_and_si256(hbits, mh));
+            values[j][3] = _mm256_or_si256(_mm256_and_si256(_mm256_srli_epi16(lbits2, 4), ml),
+                                           _mm256_and_si256(_mm256_srli_epi16(hbits, 2), mh));
+            for (int q = 0; q < 4; q++) {
+                values[j][q] = _mm256_add_epi8(values[j][q], m32n);
+                us[j][q] = _mm256_sign_epi8(values[j][q], values[j][q]);
+            }
+        }
+        for (int c = 0; c < C; c++) {
+            const uint8_t *acol = acols[c];
+            __m256 dy = q82x4_dy(acol, i);
+            __m128 dyl = _mm256_castps256_ps128(dy), dyh = _mm256_extractf128_ps(dy, 1);
+            __m256 scales[2] = {_mm256_mul_ps(wscales[0], _mm256_set_m128(dyl, dyl)),
+                                _mm256_mul_ps(wscales[1], _mm256_set_m128(dyh, dyh))};
+            __m256i sumis[2];
+            for (int j = 0; j < 2; j++) {
+                const uint8_t *qs = acol + (size_t)(2 * i + j) * ORA_Q82X4_STRIDE + 16;
+                __m256i s[4];
+                for (int q = 0; q < 4; q++)
+                    s[q] = _mm256_maddubs_epi16(
+                        us[j][q], _mm256_sign_epi8(_mm256_loadu_si256((const __m256i *)(qs + 32 * q)), values[j][q]));
+                sumis[j] = reduce4(s[0], s[1], s[2], s[3]);
+            }
+            accd[c] = _mm256_fmadd_ps(scales[0], _mm256_cvtepi32_ps(sumis[0]), accd[c]);
+            accd[c] = _mm256_fmadd_ps(scales[1], _mm256_cvtepi32_ps(sumis[1]), accd[c]);
+        }
+    }
+    for (int c = 0; c < C; c++) out[c] = hsum_float_8(accd[c]);
+}
+
+// ------------------------------------------------------------------------------------------------ IQ2_XXS tile
+
+static uint64_t KEVEN_SIGNS[128]; // crates/qdot/src/lib.rs:7201-7218: 0xff where the sign bit is set, 0x01 where clear
+static pthread_once_t keven_once = PTHREAD_ONCE_INIT;
+
+static void keven_init(void) {
+    for (int i = 0; i < 128; i++) {
+        uint64_t t = 0;
+        for (int b = 0; b < 8; b++) t |= (uint64_t)(((ORA_KSIGNS_IQ2XS[i] >> b) & 1) ? 0xff : 0x01) << (8 * b);
+        KEVEN_SIGNS[i] = t;
+    }
+}
+
+// One IQ2_XXS row against C <= 8 columns (crates/qdot/src/lib.rs:8328-8354 per column; new_block :8494, prepare
+// :8558, half step :8599, group :8636).
+static void dot_iq2xxs_tile(const uint8_t *wrow, const uint8_t *const *acols, int C, int nb, float *out) {
+    const __m256i min_value = _mm256_set1_epi8(43);
+    __m256 accd[8];
+    for (int c = 0; c < C; c++) accd[c] = _mm256_setzero_ps();
+    for (int i = 0; i < nb; i++) {
+        const uint8_t *blk = wrow + (size_t)i * ORA_IQ2XXS_BLOCK;
+        size_t at = (size_t)i * ORA_Q8K_STRIDE;
+        uint16_t dh;
+        memcpy(&dh, blk, 2);
+        float d = 0.125f * f16c_to_f32(dh);
+        float dmin = -d * 43.0f;
+        __m256 lo = _mm256_castsi256_ps(_mm256_loadu_si256((const __m256i *)(blk + 2)));
+        __m256 hi = _mm256_castsi256_ps(_mm256_loadu_si256((const __m256i *)(blk + 34)));
+        __m256i words = _mm256_permute4x64_epi64(_mm256_castps_si256(_mm256_shuffle_ps(lo, hi, 0xDD)), 0xD8);
+        __m256i sc32 = _mm256_or_si256(_mm256_slli_epi32(_mm256_srli_epi32(words, 28), 1), _mm256_set1_epi32(1));
+        __m128i sc16 = _mm_packs_epi32(_mm256_castsi256_si128(sc32), _mm256_extracti128_si256(sc32, 1));
+        __m256i mins = _mm256_set_m128i(
+            _mm_shuffle_epi8(sc16, _mm_set_epi32(0x0f0e0f0e, 0x0d0c0d0c, 0x0b0a0b0a, 0x09080908)),
+            _mm_shuffle_epi8(sc16, _mm_set_epi32(0x07060706, 0x05040504, 0x03020302, 0x01000100)));
+        __m256i all_scales = _mm256_set_m128i(sc16, sc16);
+        __m256i sumi[8];
+        for (int c = 0; c < C; c++) {
+            const uint8_t *col = acols[c] + at;
+            float dy;
+            memcpy(&dy, col, 4);
+            __m256i bsums = _mm256_loadu_si256((const __m256i *)(col + 264));
+            accd[c] = _mm256_fmadd_ps(_mm256_set1_ps(dmin * dy), _mm256_cvtepi32_ps(_mm256_madd_epi16(mins, bsums)),
+                                      accd[c]);
+        }
+        for (int j = 0; j < 2; j++) {
+            __m256i values[4], scales[4];
+            for (int q = 0; q < 4; q++) {
+                const uint8_t *qs = blk + 2 + 8 * (4 * j + q);
+                uint32_t aux;
+                memcpy(&aux, qs + 4, 4);
+                __m256i q2 = _mm256_set_epi64x((long long)ORA_IQ2XXS_GRID[qs[3]], (long long)ORA_IQ2XXS_GRID[qs[2]],
+                                               (long long)ORA_IQ2XXS_GRID[qs[1]], (long long)ORA_IQ2XXS_GRID[qs[0]]);
+                __m256i sg = _mm256_set_epi64x((long long)KEVEN_SIGNS[(aux >> 21) & 127], (long long)KEVEN_SIGNS[(aux >> 14) & 127],
+                                               (long long)KEVEN_SIGNS[(aux >> 7) & 127], (long long)KEVEN_SIGNS[aux & 127]);
+                values[q] = _mm256_add_epi8(_mm256_sign_epi8(q2, sg), min_value);
+                int b = 8 * j + 2 * q;
+                scales[q] = _mm256_shuffle_epi8(all_scales, _mm256_set1_epi16((short)(b | ((b + 1) << 8))));
+            }
+            for (int c = 0; c < C; c++) {
+                const uint8_t *col = acols[c] + at;
+                __m256i p[4];
+                for (int q = 0; q < 4; q++) {
+                    __m256i q8 = _mm256_loadu_si256((const __m256i *)(col + 8 + 32 * (4 * j + q)));
+                    p[q] = _mm256_madd_epi16(scales[q], _mm256_maddubs_epi16(values[q], q8));
+                }
+                if (j == 0) {
+                    sumi[c] = _mm256_add_epi32(_mm256_add_epi32(p[0], p[2]), _mm256_add_epi32(p[1], p[3]));
+                } else {
+                    sumi[c] = _mm256_add_epi32(sumi[c], _mm256_add_epi32(p[0], p[2]));
+                    sumi[c] = _mm256_add_epi32(sumi[c], _mm256_add_epi32(p[1], p[3]));
+                }
+            }
+        }
+        for (int c = 0; c < C; c++) {
+            float dy;
+            memcpy(&dy, acols[c] + at, 4);
+            accd[c] = _mm256_fmadd_ps(_mm256_set1_ps(d * dy), _mm256_cvtepi32_ps(sumi[c]), accd[c]);
+        }
+    }
+    for (int c = 0; c < C; c++) out[c] = hsum_float_8(accd[c]);
+}
+
+// ----------------------------------------------------------------------------------------------------- dispatch
+
+// dot_row_cols (crates/qdot/src/lib.rs:905): 1..=8 columns, every value the one-column kernel's.
+int ora_avx2_dot_row_cols(int wtype, const uint8_t *wrow, const uint8_t *const *acols, int cols, int k, float *out) {
+    if (cols < 1 || cols > 8) return ORA_ESHAPE;
+    if (k <= 0 || k % 256 != 0) return ORA_EUNALIGNED;
+    int nb = k / 256;
+    switch (wtype) {
+    case ORA_TYPE_Q4_K:
+        dot_q4k_tile(wrow, acols, cols, nb, out);
+        return 0;
+    case ORA_TYPE_Q6_K:
+        dot_q6k_tile(wrow, acols, cols, nb, out);
+        return 0;
+    case ORA_TYPE_IQ2_XXS:
+        pthread_once(&keven_once, keven_init);
+        dot_iq2xxs_tile(wrow, acols, cols, nb, out);
+        return 0;
+    default:
+        return ORA_ETYPE;
+    }
+}
+
+int ora_avx2_dot_row(int wtype, const uint8_t *wrow, const uint8_t *acol, int k, float *out) {
+    return ora_avx2_dot_row_cols(wtype, wrow, &acol, 1, k, out);
+}
+
+// --------------------------------------------------------------------------------- multi-threaded layer baseline
+
+typedef struct {
+    int wtype, k, rows, cols;
+    const uint8_t *w;
+    const uint8_t *const *acols;
+    float *const *outs;
+} mt_gemv;
+
+typedef struct {
+    pthread_t th;
+    int tid, n_threads;
+    pthread_barrier_t *bar;
+    volatile int *quit;
+    const mt_gemv *volatile *job;
+} worker;
+
+static void run_slice(const mt_gemv *g, int tid, int n_threads) {
+    int per = (g->rows + n_threads - 1) / n_threads;
+    int r0 = tid * per, r1 = r0 + per > g->rows ? g->rows : r0 + per;
+    int rb = ora_row_bytes(g->wtype, g->k);
+    float tmp[8];
+    for (int r = r0; r < r1; r++) {
+        for (int c0 = 0; c0 < g->cols; c0 += 8) {
+            int c = g->cols - c0 < 8 ? g->cols - c0 : 8;
+            ora_avx2_dot_row_cols(g->wtype, g->w + (size_t)r * rb, g->acols + c0, c, g->k, tmp);
+            for (int j = 0; j < c; j++) g->outs[c0 + j][r] = tmp[j];
+        }
+    }
+}
+
+static void *worker_main(void *arg) {
+    worker *w = (worker *)arg;
+    for (;;) {
+        pthread_barrier_wait(w->bar);
+        if (*w->quit) return NULL;
+        run_slice((const mt_gemv *)*w->job, w->tid, w->n_threads);
+        pthread_barrier_wait(w->bar);
+    }
+}
+
+struct ora_pool {
+    int n_threads;
+    worker *ws;
+    pthread_barrier_t bar;
+    volatile int quit;
+    const mt_gemv *volatile job;
+};
+
+// A resident pool (the role of crates/threads): n_threads - 1 workers plus the caller.
+ora_pool *ora_pool_create(int n_threads) {
+    if (n_threads < 1) n_threads = 1;
+    ora_pool *p = (ora_pool *)calloc(1, sizeof(ora_pool));
+    p->n_threads = n_threads;
+    pthread_barrier_init(&p->bar, NULL, (unsigned)n_threads);
+    p->ws = (worker *)calloc((size_t)n_threads, sizeof(worker));
+    for (int t = 1; t < n_threads; t++) {
+        p->ws[t] = (worker){0, t, n_threads, &p->bar, &p->quit, &p->job};
+        pthread_create(&p->ws[t].th, NULL, worker_main, &p->ws[t]);
+    }
+    return p;
+}
+
+void ora_pool_destroy(ora_pool *p) {
+    if (!p) return;
+    p->quit = 1;
+    if (p->n_threads > 1) pthread_barrier_wait(&p->bar);
+    for (int t = 1; t < p->n_threads; t++) pthread_join(p->ws[t].th, NULL);
+    pthread_barrier_destroy(&p->bar);
+    free(p->ws);
+    free(p);
+}
+
+static void pool_gemv(ora_pool *p, const mt_gemv *g) {
+    if (p->n_threads == 1) {
+        run_slice(g, 0, 1);
+        return;
+    }
+    p->job = g;
+    pthread_barrier_wait(&p->bar);
+    run_slice(g, 0, p->n_threads);
+    pthread_barrier_wait(&p->bar);
+}
+
+// The layer step of ora_moe_forward on the AVX2 kernels and the pool, slots grouped by expert so a weight row is
+// read once for up to eight of its columns (crates/model/src/moe.rs:617-749 with dot_row_cols tiles). The values
+// are ora_moe_forward's bit for bit: every (row, column) dot is the one-column kernel's and the combine keeps
+// its slot order.
+int ora_avx2_moe_forward(ora_pool *p, const ora_moe_layer *L, const float *x, int m, const uint32_t *ids,
+                         const float *wts, int top_k, float *y, float *h_out) {
+    int hidden = L->hidden, ff = L->ff, n_slots = m * top_k;
+    int cb_g = ora_col_bytes(L->gate_type, hidden), cb_u = ora_col_bytes(L->up_type, hidden);
+    int cb_d = ora_col_bytes(L->down_type, ff);
+    int rb_g = ora_row_bytes(L->gate_type, hidden), rb_u = ora_row_bytes(L->up_type, hidden);
+    int rb_d = ora_row_bytes(L->down_type, ff);
+    if (cb_g < 0 || cb_u < 0 || cb_d < 0) return ORA_ESHAPE;
+    for (int s = 0; s < n_slots; s++)
+        if (ids[s] >= (uint32_t)L->n_experts) return ORA_ESHAPE;
+    int same_enc = (L->gate_type == ORA_TYPE_IQ2_XXS) == (L->up_type == ORA_TYPE_IQ2_XXS);
+    uint8_t *ag = (uint8_t *)malloc((size_t)cb_g * m), *au = same_enc ? ag : (uint8_t *)malloc((size_t)cb_u * m);
+    uint8_t *ad = (uint8_t *)malloc((size_t)cb_d * n_slots);
+    float *g = (float *)malloc(sizeof(float) * (size_t)ff * n_slots);
+    float *u = (float *)malloc(sizeof(float) * (size_t)ff * n_slots);
+    float *h = h_out ? h_out : (float *)malloc(sizeof(float) * (size_t)ff * n_slots);
+    float *down = (float *)malloc(sizeof(float) * (size_t)hidden * n_slots);
+    int *order = (int *)malloc(sizeof(int) * (size_t)n_slots);
+    const uint8_t **cols = (const uint8_t **)malloc(sizeof(void *) * (size_t)n_slots);
+    float **outs = (float **)malloc(sizeof(void *) * (size_t)n_slots);
+    int rc = 0;
+    for (int t = 0; t < m && !rc; t++) {
+        rc = ora_avx2_quantize_col(L->gate_type, x + (size_t)t * hidden, hidden, ag + (size_t)t * cb_g);
+        if (!rc && !same_enc)
+            rc = ora_avx2_quantize_col(L->up_type, x + (size_t)t * hidden, hidden, au + (size_t)t * cb_u);
+    }
+    // Slots grouped by expert, ascending slot order inside an expert (the bucket table, moe.rs:281-304).
+    int n = 0;
+    for (int e = 0; e < L->n_experts && !rc; e++) {
+        int first = n;
+        for (int s = 0; s < n_slots; s++)
+            if (ids[s] == (uint32_t)e) order[n++] = s;
+        int cnt = n - first;
+        if (!cnt) continue;
+        for (int pass = 0; pass < 2; pass++) {
+            for (int j = 0; j < cnt; j++) {
+                int s = order[first + j];
+                cols[j] = (pass ? au + (size_t)(s / top_k) * cb_u : ag + (size_t)(s / top_k) * cb_g);
+                outs[j] = (pass ? u : g) + (size_t)s * ff;
+            }
+            mt_gemv job = {pass ? L->up_type : L->gate_type, hidden, ff, cnt,
+                           (pass ? L->wu + (size_t)e * ff * rb_u : L->wg + (size_t)e * ff * rb_g), cols, outs};
+            pool_gemv(p, &job);
+        }
+        for (int j = 0; j < cnt && !rc; j++) {
+            int s = order[first + j];
+            ora_swiglu(g + (size_t)s * ff, u + (size_t)s * ff, ff, h + (size_t)s * ff);
+            rc = ora_avx2_quantize_col(L->down_type, h + (size_t)s * ff, ff, ad + (size_t)s * cb_d);
+            cols[j] = ad + (size_t)s * cb_d;
+            outs[j] = down + (size_t)s * hidden;
+        }
+        if (rc) break;
+        mt_gemv job = {L->down_type, ff, hidden, cnt, L->wd + (size_t)e * hidden * rb_d, cols, outs};
+        pool_gemv(p, &job);
+    }
+    if (!rc) ora_combine_tokens(down, wts, NULL, hidden, top_k, m, y);
+    free(ag);
+    if (!same_enc) free(au);
+    free(ad);
+    free(g);
+    free(u);
+    if (!h_out) free(h);
+    free(down);
+    free(order);
+    free(cols);
+    free(outs);
+    return rc;
+}

@@ -1,0 +1,93 @@
+// TEST INFRASTRUCTURE ONLY. CPU oracle of the quantized MoE expert-matmul path: a plain C restatement of the
+// reference's crates/qdot (activation encoders, Q4_K / Q6_K / IQ2_XXS row dots, SwiGLU), crates/gguf (block
+// layouts, dequantizers, K-quant and IQ2_XXS weight quantizers) and the caller-side router/combine order of
+// crates/model/src/moe.rs. Each function cites the reference lines it follows. The shipped library never links
+// or calls this; the test suite, the smoke check and the benchmark's CPU-baseline leg do.
+//
+// What pins each function (the reference itself cannot be built here: it is Rust and the image has no rustc):
+//   encoders        the reference tests' known answers (bf16 scale bits 0x3F80/0x4000/0x3F80/0x3F82, saturation
+//                   ends, 1e-40 / 1e-38 flushes, first-max ties, round-half-even codes), an independent
+//                   closed-form restatement in the test suite, and the isum / bsums invariants;
+//   integer sums    brute-force sums over independently decoded codes in the test suite;
+//   fp32 dots       bit-equality with an AVX2-intrinsics restatement of the reference's vector kernels (its own
+//                   first gate) and an f64 band around the dequantized dot;
+//   dequantizers    the reference's ggml-made IQ2_XXS block (66 bytes -> 256 f32 bit patterns), table digests;
+//   expf / SwiGLU   libm band and special-case paths;
+//   weight quantizers   PARITY UNPINNED as bytes: the reference holds no golden bytes for them (it pins them
+//                   against ggml on its own machine). They are held to the reference tests' round-trip bounds,
+//                   zero-row and on-grid properties. Their output is an input shared by the oracle and the GPU
+//                   path, so it does not enter any parity claim.
+#ifndef BM_ORACLE_H
+#define BM_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+// Refusals (the reference panics or returns QdotError, crates/qdot/src/lib.rs:127-160).
+#define ORA_EUNALIGNED (-1) // k is not a whole number of 256-value super-blocks
+#define ORA_ETYPE (-2)      // weight type outside {Q4_K = 12, Q6_K = 14, IQ2_XXS = 16}
+#define ORA_ESHORTROW (-3)
+#define ORA_ESHORTCOL (-4)
+#define ORA_ENONFINITE (-5) // an activation value that is not finite
+#define ORA_ESHAPE (-6)
+#define ORA_ESTATUS (-7) // the IQ2_XXS search left the grid (crates/gguf/src/iq_quant.rs:52-61)
+
+int ora_col_bytes(int wtype, int k);
+int ora_row_bytes(int wtype, int k);
+
+int ora_quantize_q82x4(const float *x, int k, uint8_t *out);
+int ora_quantize_q8k(const float *x, int k, uint8_t *out);
+int ora_quantize_col(int wtype, const float *x, int k, uint8_t *out);
+
+float ora_dot_q4k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb);
+float ora_dot_q6k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb);
+float ora_dot_iq2xxs_q8k(const uint8_t *wrow, const uint8_t *acol, int nb);
+int ora_dot_row(int wtype, const uint8_t *wrow, size_t wrow_len, const uint8_t *acol, size_t acol_len, int k,
+                float *out);
+int ora_gemv(int wtype, const uint8_t *w, int rows, int k, const uint8_t *act, int m, float *y);
+
+void ora_q4k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_t *a_out, int32_t *isum_out);
+void ora_q6k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int fold, int32_t *s_out);
+void ora_iq2xxs_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_t *i_out, int32_t *sc_out,
+                           int32_t *codes_out, int32_t *fold_out);
+
+int ora_dequant_row(int wtype, const uint8_t *src, int k, float *dst);
+int ora_dequant_col(int wtype, const uint8_t *acol, int k, float *dst);
+
+float ora_expf_ik(float x);
+void ora_swiglu(const float *gate, const float *up, int n, float *out);
+
+// Router and combine, in the caller's order (harness side of the path).
+int ora_route_softmax_topk(const float *logits, int n_experts, int top_k, int renorm, uint32_t *ids, float *w);
+void ora_combine_tokens(const float *down, const float *w, const float *resid, int rows, int n_slots, int m,
+                        float *y);
+
+// Weight quantizers (offline, host).
+int ora_quantize_row_q4k(const float *x, int k, uint8_t *out);
+int ora_quantize_row_q6k(const float *x, int k, uint8_t *out);
+int ora_quantize_row_iq2xxs(const float *x, const float *qw, int k, uint8_t *out);
+int ora_quantize_rows(int wtype, const float *x, int rows, int k, uint8_t *out, int n_threads);
+int ora_iq2xxs_grid_codes(uint32_t *codes256, int *kmap_neg_count, int *neighbour_words);
+
+// Whole layers, for parity tests and the CPU baseline. Weights are GGUF block bytes, expert-major, rows back to
+// back. `n_threads` splits rows statically; each (row, column) value is ora_dot_row's whatever the split.
+typedef struct {
+    int hidden, ff, n_experts;
+    int gate_type, up_type, down_type;
+    const uint8_t *wg, *wu, *wd;
+} ora_moe_layer;
+
+// One decode step of `m` tokens: x[m][hidden], ids/wts[m][top_k] -> y[m][hidden] (no residual),
+// optionally h[m*top_k][ff] (the SwiGLU outputs). Returns 0 or a refusal.
+int ora_moe_forward(const ora_moe_layer *L, const float *x, int m, const uint32_t *ids, const float *wts, int top_k,
+                    float *y, float *h_out, int n_threads);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif // BM_ORACLE_H

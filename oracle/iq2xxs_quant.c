@@ -1,0 +1,352 @@
+// TEST INFRASTRUCTURE ONLY (see ora_common.h). Host IQ2_XXS weight quantizer for synthetic expert stacks: ggml's
+// `quantize_row_iq2_xxs_impl` as the reference restates it (crates/gguf/src/iq_quant.rs), every f32 operation
+// rounded on its own (build with -ffp-contract=off), ggml's candidate order and strict tie-breaks.
+//
+// PARITY UNPINNED as bytes: the reference holds no golden bytes for it; it is held to the reference tests'
+// properties (grid tables equal a naive sort, every emitted word on the grid, cosine of the round trip).
+#include <pthread.h>
+#include <stdlib.h>
+
+#include "bm_oracle.h"
+#include "iq_tables.h"
+#include "ora_common.h"
+
+#define KMAP_SIZE 43692 // crates/gguf/src/iq_quant.rs:43
+#define EPS_IQ2_XXS 1e-15f
+#define NWANT 2
+
+typedef struct {
+    uint32_t codes[256]; // grid point g's eight 2-bit codes, value k at bits 2k..
+    int32_t *map;        // code word -> grid index, or -(offset + 1) into neighbours
+    uint32_t *neighbours; // lists [n, j_1 .. j_n]
+    int n_neighbour_words;
+} grid_tables;
+
+static grid_tables G;
+static pthread_once_t g_once = PTHREAD_ONCE_INIT;
+
+// iq2xs_init_impl's output for the IQ2_XXS grid (crates/gguf/src/iq_quant.rs:162-223): each point's codes from its
+// magnitudes (0x08, 0x19, 0x2b are codes 0, 1, 2), the map, and for every off-grid word the points at its two
+// smallest squared distances in (distance, index) order.
+static void build_tables(void) {
+    for (int g = 0; g < 256; g++) {
+        uint32_t acc = 0;
+        for (int k = 0; k < 8; k++) {
+            uint8_t b = (uint8_t)(ORA_IQ2XXS_GRID[g] >> (8 * k));
+            uint32_t l = b == 0x08 ? 0 : (b == 0x19 ? 1 : 2);
+            acc |= l << (2 * k);
+        }
+        G.codes[g] = acc;
+    }
+    G.map = (int32_t *)malloc(sizeof(int32_t) * KMAP_SIZE);
+    for (int i = 0; i < KMAP_SIZE; i++) G.map[i] = -1;
+    for (int g = 0; g < 256; g++) G.map[G.codes[g]] = g;
+    size_t cap = 1 << 20, len = 0;
+    G.neighbours = (uint32_t *)malloc(sizeof(uint32_t) * cap);
+    int d2s[256];
+    for (int i = 0; i < KMAP_SIZE; i++) {
+        if (G.map[i] >= 0) continue;
+        for (int j = 0; j < 256; j++) {
+            int d2 = 0;
+            for (int k = 0; k < 8; k++) {
+                int a = (i >> (2 * k)) & 3, b = (int)((G.codes[j] >> (2 * k)) & 3);
+                int d = 2 * (b - a);
+                d2 += d * d;
+            }
+            d2s[j] = d2;
+        }
+        if (len + 258 > cap) {
+            cap *= 2;
+            G.neighbours = (uint32_t *)realloc(G.neighbours, sizeof(uint32_t) * cap);
+        }
+        G.map[i] = -((int32_t)len + 1);
+        size_t start = len++;
+        int last = -1;
+        for (int want = 0; want < NWANT; want++) {
+            int best = 1 << 30;
+            for (int j = 0; j < 256; j++)
+                if (d2s[j] > last && d2s[j] < best) best = d2s[j];
+            if (best == 1 << 30) break;
+            for (int j = 0; j < 256; j++)
+                if (d2s[j] == best) G.neighbours[len++] = (uint32_t)j;
+            last = best;
+        }
+        G.neighbours[start] = (uint32_t)(len - start - 1);
+    }
+    G.n_neighbour_words = (int)len;
+}
+
+static inline int code_of(int g, int k) { return (int)((G.codes[g] >> (2 * k)) & 3); }
+static inline float gmax(float a, float b) { return a > b ? a : b; }
+
+// For the table test: the 256 point codes, how many map entries are off-grid, and the neighbour list length.
+int ora_iq2xxs_grid_codes(uint32_t *codes256, int *kmap_neg_count, int *neighbour_words) {
+    pthread_once(&g_once, build_tables);
+    memcpy(codes256, G.codes, sizeof(G.codes));
+    int neg = 0;
+    for (int i = 0; i < KMAP_SIZE; i++) neg += G.map[i] < 0;
+    *kmap_neg_count = neg;
+    *neighbour_words = G.n_neighbour_words;
+    return KMAP_SIZE;
+}
+
+// make_qp_quants(32, nmax, x, L, w), the scale only (crates/gguf/src/iq_quant.rs:326-403).
+static float make_qp_quants(int nmax, const float *x, const float *qw) {
+    float max = 0.0f;
+    for (int i = 0; i < 32; i++) max = gmax(max, x[i]);
+    if (max < EPS_IQ2_XXS) return 0.0f;
+    float nmaxf = (float)nmax;
+    uint8_t l[32];
+    float iscale = nmaxf / max;
+    for (int i = 0; i < 32; i++) l[i] = (uint8_t)ora_nearest_int(iscale * x[i]);
+    float scale = 1.0f / iscale;
+    float best_mse = 0.0f;
+    for (int i = 0; i < 32; i++) {
+        float diff = x[i] - scale * (float)l[i];
+        best_mse = best_mse + (qw[i] * diff) * diff;
+    }
+    for (int is = -4; is <= 4; is++) {
+        if (is == 0) continue;
+        float iscale_is = (0.1f * (float)is + nmaxf) / max;
+        float scale_is = 1.0f / iscale_is;
+        float mse = 0.0f;
+        for (int i = 0; i < 32; i++) {
+            int li = ora_nearest_int(iscale_is * x[i]);
+            if (li > nmax) li = nmax;
+            float diff = x[i] - scale_is * (float)li;
+            mse = mse + (qw[i] * diff) * diff;
+        }
+        if (mse < best_mse) {
+            best_mse = mse;
+            iscale = iscale_is;
+        }
+    }
+    float sumlx = 0.0f, suml2 = 0.0f;
+    for (int i = 0; i < 32; i++) {
+        int li = ora_nearest_int(iscale * x[i]);
+        if (li > nmax) li = nmax;
+        l[i] = (uint8_t)li;
+        float lf = (float)li;
+        sumlx = sumlx + (qw[i] * x[i]) * lf;
+        suml2 = suml2 + (qw[i] * lf) * lf;
+    }
+    for (int itry = 0; itry < 5; itry++) {
+        int n_changed = 0;
+        for (int i = 0; i < 32; i++) {
+            float w = qw[i];
+            float li = (float)l[i];
+            float slx = sumlx - (w * x[i]) * li;
+            float sl2 = suml2 - (w * li) * li;
+            if (slx > 0.0f && sl2 > 0.0f) {
+                int new_l = ora_nearest_int((x[i] * sl2) / slx);
+                if (new_l > nmax) new_l = nmax;
+                if (new_l != (int)l[i]) {
+                    float nl = (float)new_l;
+                    slx = slx + (w * x[i]) * nl;
+                    sl2 = sl2 + (w * nl) * nl;
+                    if ((slx * slx) * suml2 > (sumlx * sumlx) * sl2) {
+                        l[i] = (uint8_t)new_l;
+                        sumlx = slx;
+                        suml2 = sl2;
+                        n_changed++;
+                    }
+                }
+            }
+        }
+        if (n_changed == 0) break;
+    }
+    return suml2 > 0.0f ? sumlx / suml2 : 0.0f;
+}
+
+// iq2_find_best_neighbour over group k (crates/gguf/src/iq_quant.rs:409-439). Returns the grid index or -1.
+static int best_neighbour(int start, const float *xval, const float *waux, int k, float scale, int *l) {
+    int n = (int)G.neighbours[start];
+    float best_d2 = 3.402823466e+38f;
+    int best = -1;
+    for (int j = 1; j <= n; j++) {
+        int g = (int)G.neighbours[start + j];
+        float d2 = 0.0f;
+        for (int i = 0; i < 8; i++) {
+            float q = (float)(2 * code_of(g, i) + 1);
+            float diff = scale * q - xval[8 * k + i];
+            d2 = d2 + (waux[8 * k + i] * diff) * diff;
+        }
+        if (d2 < best_d2) {
+            best_d2 = d2;
+            best = g;
+        }
+    }
+    if (best < 0) return -1;
+    for (int i = 0; i < 8; i++) l[8 * k + i] = code_of(best, i);
+    return best;
+}
+
+// Group k's code word at 1/scale (crates/gguf/src/iq_quant.rs:443-453).
+static uint32_t iq2_word(const float *xval, int k, float id, int *l) {
+    uint32_t u = 0;
+    for (int i = 0; i < 8; i++) {
+        int v = ora_nearest_int(0.5f * (id * xval[8 * k + i] - 1.0f));
+        int c = v < 0 ? 0 : (v > 2 ? 2 : v);
+        l[8 * k + i] = c;
+        u |= (uint32_t)c << (2 * i);
+    }
+    return u;
+}
+
+static void iq2_sums(const float *w, const float *xval, const int *l, float *sumqx, float *sumq2) {
+    float sx = 0.0f, s2 = 0.0f;
+    for (int i = 0; i < 32; i++) {
+        float q = (float)(2 * l[i] + 1);
+        sx = sx + (w[i] * xval[i]) * q;
+        s2 = s2 + (w[i] * q) * q;
+    }
+    *sumqx = sx;
+    *sumq2 = s2;
+}
+
+typedef struct {
+    uint32_t w0, w1;
+    float scale;
+    uint32_t status;
+} sub_t;
+
+// One 32-value sub-block (crates/gguf/src/iq_quant.rs:471-637).
+static sub_t iq2_xxs_sub(const float *xb, const float *qw, float sigma2) {
+    const int KMAXQ = 3;
+    sub_t zero = {0, 0, 0.0f, 0};
+    for (int i = 0; i < 32; i++)
+        if (isnan(xb[i]) || isnan(qw[i])) return (sub_t){0, 0, 0.0f, 8};
+    float weight[32], waux[32], xval[32];
+    for (int i = 0; i < 32; i++) {
+        weight[i] = qw[i] * sqrtf(sigma2 + xb[i] * xb[i]);
+        waux[i] = sqrtf(weight[i]);
+    }
+    uint32_t block_signs[4];
+    for (int k = 0; k < 4; k++) {
+        int nflip = 0;
+        uint32_t s = 0;
+        for (int i = 0; i < 8; i++) {
+            float v = xb[8 * k + i];
+            if (v >= 0.0f) {
+                xval[8 * k + i] = v;
+            } else {
+                xval[8 * k + i] = -v;
+                nflip++;
+                s |= 1u << i;
+            }
+        }
+        if (nflip % 2 == 1) {
+            int imin = 0;
+            float min = (weight[8 * k] * xb[8 * k]) * xb[8 * k];
+            for (int i = 1; i < 8; i++) {
+                float ax = (weight[8 * k + i] * xb[8 * k + i]) * xb[8 * k + i];
+                if (ax < min) {
+                    min = ax;
+                    imin = i;
+                }
+            }
+            xval[8 * k + imin] = -xval[8 * k + imin];
+            s ^= 1u << imin;
+        }
+        block_signs[k] = s & 127;
+    }
+    float max = xval[0];
+    for (int i = 1; i < 32; i++) max = gmax(max, xval[i]);
+    if (max < EPS_IQ2_XXS) return zero;
+    float scale = make_qp_quants(KMAXQ + 1, xval, weight);
+    float eff_max = scale * (float)KMAXQ;
+    if (eff_max <= 0.0f) return zero;
+    int l[32] = {0}, laux[32] = {0};
+    float best = 0.0f;
+    for (int is = -6; is <= 6; is++) {
+        float id = ((float)(2 * KMAXQ - 1) + (float)is * 0.1f) / eff_max;
+        float this_scale = 1.0f / id;
+        for (int k = 0; k < 4; k++) {
+            uint32_t u = iq2_word(xval, k, id, laux);
+            if (u >= KMAP_SIZE) return (sub_t){0, 0, 0.0f, 1};
+            int32_t g = G.map[u];
+            if (g < 0 && best_neighbour(-g - 1, xval, waux, k, this_scale, laux) < 0) return (sub_t){0, 0, 0.0f, 4};
+        }
+        float sumqx, sumq2;
+        iq2_sums(weight, xval, laux, &sumqx, &sumq2);
+        if (sumq2 > 0.0f && sumqx * sumqx > best * sumq2) {
+            scale = sumqx / sumq2;
+            best = scale * sumqx;
+            memcpy(l, laux, sizeof(l));
+        }
+    }
+    if (scale > 0.0f) {
+        float id = 1.0f / scale;
+        for (int k = 0; k < 4; k++) {
+            uint32_t u = iq2_word(xval, k, id, l);
+            if (u >= KMAP_SIZE) return (sub_t){0, 0, 0.0f, 1};
+            int32_t g = G.map[u];
+            if (g < 0) {
+                g = best_neighbour(-g - 1, xval, waux, k, scale, l);
+                if (g < 0) return (sub_t){0, 0, 0.0f, 4};
+            }
+            for (int i = 0; i < 8; i++) l[8 * k + i] = code_of(g, i);
+        }
+        float sumqx, sumq2;
+        iq2_sums(weight, xval, l, &sumqx, &sumq2);
+        if (sumq2 > 0.0f) scale = sumqx / sumq2;
+    }
+    if (scale < 0.0f) {
+        scale = -scale;
+        for (int k = 0; k < 4; k++) block_signs[k] = ~block_signs[k] & 127;
+    }
+    uint32_t w0 = 0, w1 = 0;
+    for (int k = 0; k < 4; k++) {
+        uint32_t u = 0;
+        for (int i = 0; i < 8; i++) u |= ((uint32_t)l[8 * k + i] & 0xff) << (2 * i);
+        if (u >= KMAP_SIZE || G.map[u] < 0) return (sub_t){0, 0, 0.0f, 1};
+        w0 |= (uint32_t)G.map[u] << (8 * k);
+        w1 |= block_signs[k] << (7 * k);
+    }
+    if (isnan(scale)) return (sub_t){0, 0, 0.0f, 2};
+    return (sub_t){w0, w1, scale, 0};
+}
+
+// One row with importance `qw` (crates/gguf/src/iq_quant.rs:967-996; finish :867-881).
+int ora_quantize_row_iq2xxs(const float *x, const float *qw, int k, uint8_t *out) {
+    if (k <= 0 || k % 256 != 0) return ORA_EUNALIGNED;
+    pthread_once(&g_once, build_tables);
+    for (int ib = 0; ib < k / 256; ib++) {
+        const float *xbl = x + 256 * ib;
+        const float *qwbl = qw + 256 * ib;
+        float sumx2 = 0.0f;
+        for (int i = 0; i < 256; i++) sumx2 = sumx2 + xbl[i] * xbl[i];
+        float sigma2 = sumx2 / 256.0f;
+        sub_t subs[8];
+        uint32_t status = 0;
+        for (int s = 0; s < 8; s++) {
+            subs[s] = iq2_xxs_sub(xbl + 32 * s, qwbl + 32 * s, sigma2);
+            status |= subs[s].status;
+        }
+        if (status) return ORA_ESTATUS;
+        uint8_t *o = out + (size_t)ib * ORA_IQ2XXS_BLOCK;
+        uint32_t q2[16] = {0};
+        float m = 0.0f;
+        for (int s = 0; s < 8; s++) m = gmax(m, subs[s].scale);
+        uint16_t dbits = 0;
+        if (m != 0.0f) {
+            float d = m / 31.0f;
+            float id = 1.0f / d;
+            for (int s = 0; s < 8; s++) {
+                int l = ora_nearest_int(0.5f * (id * subs[s].scale - 1.0f));
+                l = l < 0 ? 0 : (l > 15 ? 15 : l);
+                q2[2 * s] = subs[s].w0;
+                q2[2 * s + 1] = subs[s].w1 | ((uint32_t)l << 28);
+            }
+            dbits = ora_f32_to_f16_bits(d);
+        }
+        ora_wr16(o, dbits);
+        for (int w = 0; w < 16; w++) {
+            o[2 + 4 * w] = (uint8_t)q2[w];
+            o[3 + 4 * w] = (uint8_t)(q2[w] >> 8);
+            o[4 + 4 * w] = (uint8_t)(q2[w] >> 16);
+            o[5 + 4 * w] = (uint8_t)(q2[w] >> 24);
+        }
+    }
+    return 0;
+}

@@ -1,0 +1,265 @@
+"""TEST INFRASTRUCTURE ONLY: ctypes view of the CPU oracle (oracle/libbm_oracle.so).
+
+Imported by the test suite, the smoke check and the benchmark's CPU-baseline leg; never by the package.
+The library is built by `make -C oracle` (or `__graft_entry__.build()`); loading it never compiles.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libbm_oracle.so")
+
+Q4_K, Q6_K, IQ2_XXS = 12, 14, 16
+BLOCK_BYTES = {Q4_K: 144, Q6_K: 210, IQ2_XXS: 66}
+
+EUNALIGNED, ETYPE, ESHORTROW, ESHORTCOL, ENONFINITE, ESHAPE, ESTATUS = -1, -2, -3, -4, -5, -6, -7
+
+_u8p = C.POINTER(C.c_uint8)
+_f32p = C.POINTER(C.c_float)
+_i32p = C.POINTER(C.c_int32)
+_u32p = C.POINTER(C.c_uint32)
+
+
+class MoeLayer(C.Structure):
+    _fields_ = [
+        ("hidden", C.c_int), ("ff", C.c_int), ("n_experts", C.c_int),
+        ("gate_type", C.c_int), ("up_type", C.c_int), ("down_type", C.c_int),
+        ("wg", C.c_void_p), ("wu", C.c_void_p), ("wd", C.c_void_p),
+    ]
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f"{LIB_PATH} is not built: run `make -C oracle`")
+    lib = C.CDLL(LIB_PATH)
+    sig = {
+        "ora_col_bytes": (C.c_int, [C.c_int, C.c_int]),
+        "ora_row_bytes": (C.c_int, [C.c_int, C.c_int]),
+        "ora_quantize_col": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_avx2_quantize_col": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_dot_row": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]),
+        "ora_gemv": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_avx2_dot_row": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_avx2_dot_row_cols": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+        "ora_avx2_supported": (C.c_int, []),
+        "ora_q4k_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+        "ora_q6k_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+        "ora_iq2xxs_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                         C.c_void_p]),
+        "ora_dequant_row": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_dequant_col": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_expf_ik": (C.c_float, [C.c_float]),
+        "ora_swiglu": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_route_softmax_topk": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
+        "ora_combine_tokens": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
+        "ora_quantize_row_q4k": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_quantize_row_q6k": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_quantize_row_iq2xxs": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_quantize_rows": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]),
+        "ora_iq2xxs_grid_codes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
+        "ora_moe_forward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
+                                      C.c_void_p, C.c_int]),
+        "ora_pool_create": (C.c_void_p, [C.c_int]),
+        "ora_pool_destroy": (None, [C.c_void_p]),
+        "ora_avx2_moe_forward": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
+                                           C.c_int, C.c_void_p, C.c_void_p]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _u8(a):
+    return np.ascontiguousarray(a, dtype=np.uint8)
+
+
+class OracleError(Exception):
+    def __init__(self, code):
+        super().__init__(f"oracle refusal {code}")
+        self.code = code
+
+
+def _check(rc):
+    if rc != 0:
+        raise OracleError(rc)
+
+
+def col_bytes(wtype, k):
+    n = lib.ora_col_bytes(wtype, k)
+    if n < 0:
+        raise OracleError(n)
+    return n
+
+
+def row_bytes(wtype, k):
+    n = lib.ora_row_bytes(wtype, k)
+    if n < 0:
+        raise OracleError(n)
+    return n
+
+
+def quantize_col(wtype, x, avx2=False):
+    """One f32 column -> the activation bytes the weight type `wtype` dots against."""
+    x = _f32(x)
+    out = np.empty(col_bytes(wtype, x.size), np.uint8)
+    fn = lib.ora_avx2_quantize_col if avx2 else lib.ora_quantize_col
+    _check(fn(wtype, _p(x), x.size, _p(out)))
+    return out
+
+
+def dot_row(wtype, wrow, acol, k, avx2=False):
+    wrow, acol = _u8(wrow), _u8(acol)
+    out = C.c_float()
+    if avx2:
+        if wrow.size < row_bytes(wtype, k) or acol.size < col_bytes(wtype, k):
+            raise OracleError(ESHAPE)
+        _check(lib.ora_avx2_dot_row(wtype, _p(wrow), _p(acol), k, C.byref(out)))
+    else:
+        _check(lib.ora_dot_row(wtype, _p(wrow), wrow.size, _p(acol), acol.size, k, C.byref(out)))
+    return np.float32(out.value)
+
+
+def dot_row_cols(wtype, wrow, acols, k):
+    """AVX2 tile: one row against 1..8 columns."""
+    wrow = _u8(wrow)
+    acols = [_u8(a) for a in acols]
+    ptrs = (C.c_void_p * len(acols))(*[a.ctypes.data for a in acols])
+    out = np.empty(len(acols), np.float32)
+    _check(lib.ora_avx2_dot_row_cols(wtype, _p(wrow), ptrs, len(acols), k, _p(out)))
+    return out
+
+
+def gemv(wtype, w, rows, k, act, m=1):
+    """y[r * m + c] = row r . column c; `act` holds m columns back to back."""
+    w, act = _u8(w), _u8(act)
+    assert w.size >= rows * row_bytes(wtype, k) and act.size >= m * col_bytes(wtype, k)
+    y = np.empty(rows * m, np.float32)
+    _check(lib.ora_gemv(wtype, _p(w), rows, k, _p(act), m, _p(y)))
+    return y
+
+
+def q4k_block_sums(wrow, acol, k):
+    nb = k // 256
+    a = np.empty(nb * 8, np.int32)
+    s = np.empty(nb * 8, np.int32)
+    lib.ora_q4k_block_sums(_p(_u8(wrow)), _p(_u8(acol)), nb, _p(a), _p(s))
+    return a, s
+
+
+def q6k_block_sums(wrow, acol, k, fold=False):
+    nb = k // 256
+    s = np.empty(nb * 16, np.int32)
+    lib.ora_q6k_block_sums(_p(_u8(wrow)), _p(_u8(acol)), nb, int(fold), _p(s))
+    return s
+
+
+def iq2xxs_block_sums(wrow, acol, k):
+    nb = k // 256
+    i = np.empty(nb * 8, np.int32)
+    sc = np.empty(nb * 8, np.int32)
+    codes = np.empty(nb, np.int32)
+    fold = np.empty(nb, np.int32)
+    lib.ora_iq2xxs_block_sums(_p(_u8(wrow)), _p(_u8(acol)), nb, _p(i), _p(sc), _p(codes), _p(fold))
+    return i, sc, codes, fold
+
+
+def dequant_row(wtype, src, k):
+    src = _u8(src)
+    out = np.empty(k, np.float32)
+    _check(lib.ora_dequant_row(wtype, _p(src), k, _p(out)))
+    return out
+
+
+def dequant_col(wtype, acol, k):
+    out = np.empty(k, np.float32)
+    _check(lib.ora_dequant_col(wtype, _p(_u8(acol)), k, _p(out)))
+    return out
+
+
+def expf_ik(x):
+    return np.float32(lib.ora_expf_ik(C.c_float(float(x))))
+
+
+def swiglu(gate, up):
+    gate, up = _f32(gate), _f32(up)
+    out = np.empty_like(gate)
+    lib.ora_swiglu(_p(gate), _p(up), gate.size, _p(out))
+    return out
+
+
+def route_softmax_topk(logits, top_k, renorm=True):
+    logits = _f32(logits)
+    ids = np.empty(top_k, np.uint32)
+    w = np.empty(top_k, np.float32)
+    _check(lib.ora_route_softmax_topk(_p(logits), logits.size, top_k, int(renorm), _p(ids), _p(w)))
+    return ids, w
+
+
+def combine_tokens(down, w, resid, rows, n_slots, m):
+    down, w = _f32(down), _f32(w)
+    y = np.empty(rows * m, np.float32)
+    rp = _p(_f32(resid)) if resid is not None else None
+    lib.ora_combine_tokens(_p(down), _p(w), rp, rows, n_slots, m, _p(y))
+    return y
+
+
+def quantize_rows(wtype, x, rows, k, n_threads=8):
+    """rows x k f32 -> GGUF block bytes, rows back to back."""
+    x = _f32(x).reshape(rows, k)
+    out = np.empty(rows * row_bytes(wtype, k), np.uint8)
+    _check(lib.ora_quantize_rows(wtype, _p(x), rows, k, _p(out), n_threads))
+    return out
+
+
+def quantize_row_iq2xxs(x, qw):
+    x, qw = _f32(x), _f32(qw)
+    out = np.empty(row_bytes(IQ2_XXS, x.size), np.uint8)
+    _check(lib.ora_quantize_row_iq2xxs(_p(x), _p(qw), x.size, _p(out)))
+    return out
+
+
+def iq2xxs_grid_codes():
+    codes = np.empty(256, np.uint32)
+    neg, words = C.c_int(), C.c_int()
+    size = lib.ora_iq2xxs_grid_codes(_p(codes), C.byref(neg), C.byref(words))
+    return codes, size, neg.value, words.value
+
+
+def _layer(hidden, ff, n_experts, types, wg, wu, wd):
+    L = MoeLayer(hidden, ff, n_experts, types[0], types[1], types[2], wg.ctypes.data, wu.ctypes.data, wd.ctypes.data)
+    return L
+
+
+def moe_forward(hidden, ff, n_experts, types, wg, wu, wd, x, ids, wts, top_k, n_threads=1, want_h=False,
+                avx2_pool=None):
+    """One layer step; x[m][hidden], ids/wts[m][top_k] -> y[m][hidden] (and h[m*top_k][ff])."""
+    wg, wu, wd = _u8(wg), _u8(wu), _u8(wd)
+    x = _f32(x)
+    m = x.size // hidden
+    ids = np.ascontiguousarray(ids, np.uint32)
+    wts = _f32(wts)
+    L = _layer(hidden, ff, n_experts, types, wg, wu, wd)
+    y = np.empty(m * hidden, np.float32)
+    h = np.empty(m * top_k * ff, np.float32) if want_h else None
+    hp = _p(h) if want_h else None
+    if avx2_pool is not None:
+        rc = lib.ora_avx2_moe_forward(avx2_pool, C.byref(L), _p(x), m, _p(ids), _p(wts), top_k, _p(y), hp)
+    else:
+        rc = lib.ora_moe_forward(C.byref(L), _p(x), m, _p(ids), _p(wts), top_k, _p(y), hp, n_threads)
+    _check(rc)
+    return (y, h) if want_h else y

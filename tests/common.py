@@ -1,0 +1,63 @@
+"""Shared generators for the parity tests: seeded inputs and independent (numpy / pure Python) restatements the
+oracle is checked against. Nothing here calls the HIP library."""
+import numpy as np
+
+
+class Lcg:
+    """Knuth MMIX LCG, the generator the reference's encoder sweeps use (crates/qdot/tests/qdot.rs:4510-4525)."""
+
+    def __init__(self, seed):
+        self.s = seed & 0xFFFFFFFFFFFFFFFF
+
+    def next_u32(self):
+        self.s = (self.s * 6364136223846793005 + 1442695040888963407) & 0xFFFFFFFFFFFFFFFF
+        return self.s >> 33
+
+    def unit(self):
+        return np.float32(np.float32(self.next_u32()) / np.float32(2147483648.0) - np.float32(1.0))
+
+
+def bf16_rne_bits(x):
+    u = int(np.float32(x).view(np.uint32))
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) & 0xFFFF
+
+
+def bf16_to_f32(bits):
+    return np.uint32(bits << 16).view(np.float32)
+
+
+def round_half_even(v):
+    """Independent of the magic-number form: numpy's rint rounds halves to even."""
+    return int(np.rint(np.float64(v)))
+
+
+def q82_block_closed_form(x):
+    """ik's q8_2 rule for one 32-value block, restated independently (crates/qdot/tests/qdot.rs:5093-5110).
+    Returns None where 1/d overflows (the encoders flush that block to zero)."""
+    x = np.asarray(x, np.float32)
+    amax = np.float32(np.max(np.abs(x)))
+    t = bf16_rne_bits(amax / np.float32(127.0))
+    d = bf16_to_f32(t)
+    with np.errstate(divide="ignore", over="ignore"):
+        inv = np.float32(1.0) / d if d > 0 else np.float32(0.0)
+    if not np.isfinite(inv):
+        return None
+    codes, isum = [], 0
+    for v in x:
+        q = round_half_even(np.float32(v * inv))
+        codes.append(max(-128, min(127, q)))
+        isum += q
+    isum = ((isum + 0x8000) & 0xFFFF) - 0x8000
+    return np.array(codes, np.int8), t, isum
+
+
+def normal_f32(rng, shape, sigma=1.0):
+    return (rng.standard_normal(shape) * sigma).astype(np.float32)
+
+
+def max_abs_normalised(got, want):
+    """max |got - want| / max |want|: the metric the fp32 tolerance of 1e-4 is stated in."""
+    want = np.asarray(want, np.float64)
+    got = np.asarray(got, np.float64)
+    denom = np.max(np.abs(want))
+    return float(np.max(np.abs(got - want)) / (denom if denom > 0 else 1.0))

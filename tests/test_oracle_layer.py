@@ -1,0 +1,239 @@
+"""Pins the rest of the oracle: expf / SwiGLU (crates/qdot/tests/qdot.rs:3927-4034, 8157-8230), router and combine
+order (crates/model/src/moe.rs:246-279, crates/gpu/src/elem.rs:658-697), the weight quantizers' properties
+(crates/gguf/src/kquant/tests.rs:5-60, crates/gguf/src/iq_quant/tests.rs:44-140) and the whole-layer step (scalar,
+threaded and AVX2 forms must agree bit for bit)."""
+import math
+
+import numpy as np
+import pytest
+
+import ora
+from common import max_abs_normalised, normal_f32
+
+
+# ----------------------------------------------------------------------------------------------- expf and SwiGLU
+
+def test_expf_ik_tracks_libm():
+    xs = np.concatenate([np.linspace(-87.0, 88.0, 4001), np.linspace(-1.0, 1.0, 2001), [0.0, -0.0]]).astype(np.float32)
+    for x in xs:
+        got = float(ora.expf_ik(x))
+        want = math.exp(float(x))
+        assert abs(got - want) <= 2.5e-7 * want, (x, got, want)
+
+
+def test_expf_ik_special_paths():
+    # |n| > 126 takes the two-step scale, |n| > 192 overflows or underflows outright (crates/qdot/src/lib.rs:3762-3771)
+    assert ora.expf_ik(0.0) == np.float32(1.0)
+    for x in (88.0, 88.5, 88.7):
+        got, want = float(ora.expf_ik(x)), math.exp(float(np.float32(x)))
+        assert abs(got - want) <= 3e-7 * want
+    for x in (-88.0, -95.0, -100.0, -103.0):
+        got, want = float(ora.expf_ik(x)), math.exp(float(np.float32(x)))
+        assert abs(got - want) <= max(3e-7 * want, 1.5e-45)
+    assert np.isinf(ora.expf_ik(89.0)) and np.isinf(ora.expf_ik(200.0)) and np.isinf(ora.expf_ik(1e30))
+    assert ora.expf_ik(-104.5) == 0.0 and ora.expf_ik(-200.0) == 0.0 and ora.expf_ik(-1e30) == 0.0
+    assert np.isnan(ora.expf_ik(np.nan))
+
+
+def test_swiglu_is_divide_then_multiply_and_position_independent():
+    rng = np.random.default_rng(1)
+    g, u = normal_f32(rng, 777, 3.0), normal_f32(rng, 777, 2.0)
+    out = ora.swiglu(g, u)
+    for i in (0, 1, 7, 8, 9, 500, 776):
+        e = ora.expf_ik(np.float32(0.0) - g[i])
+        want = np.float32(np.float32(g[i] / np.float32(np.float32(1.0) + e)) * u[i])
+        assert out[i].tobytes() == want.tobytes()
+        assert ora.swiglu(g[i:i + 1], u[i:i + 1])[0].tobytes() == out[i].tobytes()
+    ref = g.astype(np.float64) / (1.0 + np.exp(-g.astype(np.float64))) * u.astype(np.float64)
+    assert max_abs_normalised(out, ref) < 1e-6
+    big = ora.swiglu(np.array([100.0, -100.0, 0.0], np.float32), np.array([2.0, 2.0, 5.0], np.float32))
+    assert big[0] == 200.0 and abs(big[1]) < 1e-40 and big[2] == 0.0
+
+
+# ------------------------------------------------------------------------------------------- router and combine
+
+def test_router_softmax_topk_renorm():
+    rng = np.random.default_rng(2)
+    for n_experts, top_k in ((128, 8), (256, 8), (8, 2), (4, 4)):
+        logits = normal_f32(rng, n_experts)
+        ids, w = ora.route_softmax_topk(logits, top_k)
+        p = np.exp((logits - logits.max()).astype(np.float32)).astype(np.float32)
+        p = (p / np.float32(p.astype(np.float64).sum())).astype(np.float32)
+        order = sorted(range(n_experts), key=lambda e: (-p[e], e))[:top_k]
+        assert list(ids) == order
+        chosen = p[order]
+        want = chosen / np.float32(chosen.astype(np.float64).sum())
+        assert np.allclose(w, want, rtol=3e-7, atol=0)
+        assert abs(float(w.astype(np.float64).sum()) - 1.0) < 1e-6
+        ids2, w2 = ora.route_softmax_topk(logits, top_k, renorm=False)
+        assert list(ids2) == order and np.allclose(w2, chosen, rtol=3e-7, atol=0)
+
+
+def test_router_ties_go_to_the_smaller_id():
+    logits = np.zeros(16, np.float32)
+    logits[[3, 9, 12]] = 1.0
+    ids, w = ora.route_softmax_topk(logits, 4)
+    assert list(ids) == [3, 9, 12, 0]
+    with pytest.raises(ora.OracleError):
+        ora.route_softmax_topk(logits, 17)
+
+
+def test_combine_is_slot_ascending_fma_then_residual():
+    rng = np.random.default_rng(3)
+    rows, n_slots, m = 40, 8, 3
+    down, w, resid = normal_f32(rng, m * n_slots * rows), normal_f32(rng, m * n_slots), normal_f32(rng, m * rows)
+    got = ora.combine_tokens(down, w, resid, rows, n_slots, m)
+    d = down.reshape(m, n_slots, rows)
+    for t in range(m):
+        for r in (0, 17, rows - 1):
+            acc = np.float32(0.0)
+            for e in range(n_slots):
+                # one rounding per term: the exact product added in f64 then rounded to f32 is the fma
+                acc = np.float32(np.float64(w[t * n_slots + e]) * np.float64(d[t, e, r]) + np.float64(acc))
+            want = np.float32(acc + resid[t * rows + r])
+            assert got[t * rows + r].tobytes() == want.tobytes()
+    assert np.array_equal(ora.combine_tokens(down, w, None, rows, n_slots, m),
+                          ora.combine_tokens(down, w, np.zeros(m * rows, np.float32), rows, n_slots, m))
+
+
+# ---------------------------------------------------------------------------------------------- weight quantizers
+
+def wave_row(n, seed):
+    """The reference's deterministic row (crates/gguf/src/kquant/tests.rs:5-15)."""
+    out = np.empty(n, np.float32)
+    for i in range(n):
+        h = (i * 2654435761 + seed * 40503) & 0xFFFFFFFF
+        ripple = np.float32(np.float32((h >> 8) & 0xFFFF) / np.float32(65536.0) - np.float32(0.5))
+        out[i] = np.float32(np.sin(np.float32(np.float32(i) * np.float32(0.013) + np.float32(seed))) * np.float32(0.7)
+                            + ripple * np.float32(0.3))
+    return out
+
+
+@pytest.mark.parametrize("wtype,bound", ((ora.Q4_K, 0.12), (ora.Q6_K, 0.02)))
+def test_kquant_round_trip_bounds(wtype, bound):
+    x = wave_row(512, 3)
+    q = ora.quantize_rows(wtype, x, 1, 512, n_threads=1)
+    assert q.size == 512 // 256 * ora.BLOCK_BYTES[wtype]
+    back = ora.dequant_row(wtype, q, 512)
+    assert np.abs(x - back).max() < bound
+    assert not ora.quantize_rows(wtype, np.zeros(256, np.float32), 1, 256).any(), "a zero row is zero bytes"
+
+
+@pytest.mark.parametrize("wtype,rel", ((ora.Q4_K, 0.09), (ora.Q6_K, 0.02), (ora.IQ2_XXS, 0.55)))
+def test_quantizers_on_the_benchmark_distribution(wtype, rel):
+    rng = np.random.default_rng(40 + wtype)
+    x = normal_f32(rng, (16, 1024), 0.02)
+    q = ora.quantize_rows(wtype, x, 16, 1024, n_threads=3)
+    assert np.array_equal(q, ora.quantize_rows(wtype, x, 16, 1024, n_threads=1)), "rows are independent of the split"
+    rb = ora.row_bytes(wtype, 1024)
+    back = np.stack([ora.dequant_row(wtype, q[r * rb:(r + 1) * rb], 1024) for r in range(16)])
+    err = np.sqrt(np.mean((back - x) ** 2)) / np.sqrt(np.mean(x ** 2))
+    assert err < rel, err
+    cos = float((back * x).sum() / np.sqrt((back ** 2).sum() * (x ** 2).sum()))
+    assert cos > (0.8 if wtype == ora.IQ2_XXS else 0.99)
+
+
+def test_kquant_refuses_non_finite_and_unaligned():
+    x = np.ones(256, np.float32)
+    x[3] = np.nan
+    for wtype in (ora.Q4_K, ora.Q6_K):
+        with pytest.raises(ora.OracleError) as e:
+            ora.quantize_rows(wtype, x, 1, 256)
+        assert e.value.code == ora.ENONFINITE
+    with pytest.raises(ora.OracleError) as e:
+        ora.quantize_rows(ora.Q4_K, np.ones(300, np.float32), 1, 300)
+    assert e.value.code == ora.EUNALIGNED
+
+
+def test_iq2xxs_grid_tables_are_ggml_init():
+    # crates/gguf/src/iq_quant/tests.rs:44-84: first point codes, map size, lists == naive (distance, index) sort
+    codes, size, neg, words = ora.iq2xxs_grid_codes()
+    assert size == 43692
+    first8 = []
+    for g in range(8):
+        c = int(codes[g])
+        first8.append(sum(((c >> (2 * k)) & 3) << (2 * k) for k in range(8)))
+    assert first8 == [0, 2, 5, 8, 10, 17, 20, 32]
+    assert neg == 43692 - 256
+    assert len(set(int(c) for c in codes)) == 256
+
+
+def test_iq2xxs_rows_quantize_and_read_back():
+    # the reference's LCG row of few distinct levels with positive importance (crates/gguf/src/iq_quant/tests.rs:92-140)
+    s = [7]
+
+    def nxt():
+        s[0] = (s[0] * 1103515245 + 12345) & 0xFFFFFFFF
+        return s[0] >> 8
+
+    levels = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+    n = 4 * 256
+    x = np.empty(n, np.float32)
+    for i in range(n):
+        r = nxt()
+        v = np.float32(levels[r % 8]) * np.float32(0.01)
+        x[i] = -v if r & 256 else v
+    w = np.array([np.float32(0.1) + np.float32(nxt() % 1000) / np.float32(100.0) for _ in range(n)], np.float32)
+    q = ora.quantize_row_iq2xxs(x, w)
+    assert q.size == n // 256 * 66
+    assert np.array_equal(q, ora.quantize_row_iq2xxs(x, w))
+    y = ora.dequant_row(ora.IQ2_XXS, q, n).astype(np.float64)
+    cos = float((x * y).sum() / np.sqrt((x.astype(np.float64) ** 2).sum() * (y ** 2).sum()))
+    assert cos > 0.8, cos
+    assert not ora.quantize_row_iq2xxs(np.zeros(256, np.float32), np.ones(256, np.float32)).any()
+
+
+# ----------------------------------------------------------------------------------------------------- the layer
+
+def small_layer(types, hidden, ff, n_experts, seed):
+    rng = np.random.default_rng(seed)
+    wg = ora.quantize_rows(types[0], normal_f32(rng, (n_experts * ff, hidden), 0.02), n_experts * ff, hidden)
+    wu = ora.quantize_rows(types[1], normal_f32(rng, (n_experts * ff, hidden), 0.02), n_experts * ff, hidden)
+    wd = ora.quantize_rows(types[2], normal_f32(rng, (n_experts * hidden, ff), 0.02), n_experts * hidden, ff)
+    return wg, wu, wd
+
+
+@pytest.mark.parametrize("types,hidden,ff", (((ora.Q4_K, ora.Q4_K, ora.Q6_K), 512, 256),
+                                             ((ora.IQ2_XXS, ora.IQ2_XXS, ora.IQ2_XXS), 512, 256)))
+def test_layer_forms_agree_and_track_f64(types, hidden, ff):
+    n_experts, top_k, m = 6, 3, 4
+    wg, wu, wd = small_layer(types, hidden, ff, n_experts, 77)
+    rng = np.random.default_rng(78)
+    x = normal_f32(rng, (m, hidden))
+    ids = np.empty((m, top_k), np.uint32)
+    wts = np.empty((m, top_k), np.float32)
+    for t in range(m):
+        ids[t], wts[t] = ora.route_softmax_topk(normal_f32(rng, n_experts), top_k)
+    y1, h1 = ora.moe_forward(hidden, ff, n_experts, types, wg, wu, wd, x, ids, wts, top_k, n_threads=1, want_h=True)
+    y3 = ora.moe_forward(hidden, ff, n_experts, types, wg, wu, wd, x, ids, wts, top_k, n_threads=3)
+    assert y1.tobytes() == y3.tobytes(), "the row split never changes a value"
+    pool = ora.lib.ora_pool_create(3)
+    try:
+        y2, h2 = ora.moe_forward(hidden, ff, n_experts, types, wg, wu, wd, x, ids, wts, top_k, want_h=True,
+                                 avx2_pool=pool)
+    finally:
+        ora.lib.ora_pool_destroy(pool)
+    assert h1.tobytes() == h2.tobytes() and y1.tobytes() == y2.tobytes(), "AVX2 grouped form == scalar form"
+    # against f64 on the dequantized weights and the raw activations: quantization error only
+    rbg, rbd = ora.row_bytes(types[0], hidden), ora.row_bytes(types[2], ff)
+    want = np.zeros((m, hidden))
+    for t in range(m):
+        for s in range(top_k):
+            e = int(ids[t, s])
+            G = np.stack([ora.dequant_row(types[0], wg[(e * ff + r) * rbg:(e * ff + r + 1) * rbg], hidden)
+                          for r in range(ff)]).astype(np.float64)
+            U = np.stack([ora.dequant_row(types[1], wu[(e * ff + r) * rbg:(e * ff + r + 1) * rbg], hidden)
+                          for r in range(ff)]).astype(np.float64)
+            D = np.stack([ora.dequant_row(types[2], wd[(e * hidden + r) * rbd:(e * hidden + r + 1) * rbd], ff)
+                          for r in range(hidden)]).astype(np.float64)
+            g, u = G @ x[t].astype(np.float64), U @ x[t].astype(np.float64)
+            want[t] += float(wts[t, s]) * (D @ (g / (1.0 + np.exp(-g)) * u))
+    assert max_abs_normalised(y1, want.reshape(-1)) < 0.05
+
+
+def test_layer_refuses_bad_ids():
+    types = (ora.Q4_K, ora.Q4_K, ora.Q6_K)
+    wg, wu, wd = small_layer(types, 256, 256, 2, 5)
+    x = np.ones(256, np.float32)
+    with pytest.raises(ora.OracleError):
+        ora.moe_forward(256, 256, 2, types, wg, wu, wd, x, np.array([2], np.uint32), np.array([1.0], np.float32), 1)

@@ -1,0 +1,274 @@
+"""bloomery_amd: MI355X-native quantized MoE expert matmul (Q4_K / Q6_K / IQ2_XXS x Q8) behind the kernel-call
+surface of the reference's crates/gpu.
+
+This module is a thin ctypes view of the C ABI in include/bm_moe.h (bloomery_amd/libbm_moe_hip.so, hand-written
+HIP for gfx950). The names mirror the reference's host objects: `Gpu` (crates/gpu/src/lib.rs:2529), `DeviceTensor`
+(crates/gpu/src/tensor.rs:588), `Q8Act` (:811) and the `enqueue_*` launchers; a refusal raises `GpuError` with the
+library's message, as the reference returns `GpuError::Shape` / `Driver`.
+
+There is no CPU fallback: without the built library, or without a GPU, every entry raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libbm_moe_hip.so")
+
+Q4_K, Q6_K, IQ2_XXS = 12, 14, 16
+FAULT_NONE = 0xFFFFFFFF
+LAYER_NONE = 0xFFFF
+SITE_QUANT_COLUMN, SITE_EXPERT_ID = 1, 7
+HOST_SLOT = 0xFFFFFFFF
+
+OK, ESHAPE, EDRIVER, ETYPE, EARG, EFAULT = 0, -1, -2, -3, -4, -5
+
+# Every symbol include/bm_moe.h declares: (restype, argtypes).
+_vp, _i, _i64, _u32 = C.c_void_p, C.c_int, C.c_int64, C.c_uint32
+SYMBOLS = {
+    "bm_version": (_i, []),
+    "bm_ctx_create": (_i, [_i, C.POINTER(_vp)]),
+    "bm_ctx_create_on_stream": (_i, [_i, _vp, C.POINTER(_vp)]),
+    "bm_ctx_destroy": (None, [_vp]),
+    "bm_ctx_stream": (_vp, [_vp]),
+    "bm_ctx_sync": (_i, [_vp]),
+    "bm_last_error": (C.c_char_p, [_vp]),
+    "bm_set_layer": (_i, [_vp, _u32]),
+    "bm_fault_read": (_i, [_vp, _u32, C.POINTER(_u32), C.POINTER(_u32)]),
+    "bm_fault_clear": (_i, [_vp]),
+    "bm_fault_word_dev": (_vp, [_vp]),
+    "bm_row_bytes": (_i64, [_i, _i]),
+    "bm_col_bytes": (_i64, [_i, _i]),
+    "bm_dev_alloc": (_i, [_vp, C.c_size_t, C.POINTER(_vp)]),
+    "bm_dev_free": (_i, [_vp, _vp]),
+    "bm_dev_upload": (_i, [_vp, _vp, _vp, C.c_size_t]),
+    "bm_dev_download": (_i, [_vp, _vp, _vp, C.c_size_t]),
+    "bm_dev_memset": (_i, [_vp, _vp, _i, C.c_size_t]),
+    "bm_weights_create": (_i, [_vp, _i, _i64, _i, _vp, C.POINTER(_vp)]),
+    "bm_weights_wrap": (_i, [_vp, _i, _i64, _i, _vp, C.POINTER(_vp)]),
+    "bm_weights_destroy": (None, [_vp]),
+    "bm_weights_dev": (_vp, [_vp]),
+    "bm_act_create": (_i, [_vp, _i, _i, _i, C.POINTER(_vp)]),
+    "bm_act_destroy": (None, [_vp]),
+    "bm_act_download": (_i, [_vp, _vp, _i, _vp]),
+    "bm_act_upload": (_i, [_vp, _vp, _i, _vp]),
+    "bm_quantize": (_i, [_vp, _vp, _i, _vp]),
+    "bm_gemv": (_i, [_vp, _vp, _vp, _i, _vp]),
+    "bm_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
+    "bm_gemv_sel": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "bm_combine_tokens": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "bm_down_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "bm_block_sums": (_i, [_vp, _vp, _i64, _vp, _i, _vp]),
+}
+
+
+class GpuError(RuntimeError):
+    """A refusal of the library: `code` is the C ABI's return value, the text its bm_last_error message."""
+
+    def __init__(self, code, message):
+        super().__init__(message)
+        self.code = code
+
+
+_lib = None
+
+
+def load_library(path=LIB_PATH):
+    """Load the built library and bind every declared symbol. Never compiles; raises when the file is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(path):
+        raise GpuError(EDRIVER, f"{path} is not built: run __graft_entry__.build() (hipcc, gfx950); there is no CPU path")
+    lib = C.CDLL(path)
+    for name, (res, args) in SYMBOLS.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def row_bytes(wtype, k):
+    return int(load_library().bm_row_bytes(wtype, k))
+
+
+def col_bytes(wtype, k):
+    return int(load_library().bm_col_bytes(wtype, k))
+
+
+class DeviceBuffer:
+    """A typed device allocation (the reference's DeviceBuffer<T>)."""
+
+    def __init__(self, gpu, dtype, count):
+        self.gpu, self.dtype, self.count = gpu, np.dtype(dtype), int(count)
+        p = _vp()
+        gpu._check(gpu.lib.bm_dev_alloc(gpu.ctx, self.count * self.dtype.itemsize, C.byref(p)))
+        self.ptr = p.value
+
+    @property
+    def nbytes(self):
+        return self.count * self.dtype.itemsize
+
+    def upload(self, host):
+        host = np.ascontiguousarray(host, self.dtype).reshape(-1)
+        assert host.size <= self.count
+        self.gpu._check(self.gpu.lib.bm_dev_upload(self.gpu.ctx, self.ptr, host.ctypes.data, host.nbytes))
+        return self
+
+    def download(self, count=None):
+        out = np.empty(self.count if count is None else count, self.dtype)
+        self.gpu._check(self.gpu.lib.bm_dev_download(self.gpu.ctx, out.ctypes.data, self.ptr, out.nbytes))
+        return out
+
+    def fill_bytes(self, byte):
+        self.gpu._check(self.gpu.lib.bm_dev_memset(self.gpu.ctx, self.ptr, byte, self.nbytes))
+        return self
+
+    def free(self):
+        if self.ptr:
+            self.gpu.lib.bm_dev_free(self.gpu.ctx, self.ptr)
+            self.ptr = None
+
+
+class DeviceTensor:
+    """An expert stack or one matrix: rows of GGUF block bytes on the device."""
+
+    def __init__(self, gpu, wtype, rows, k, host_bytes=None, dev_ptr=None):
+        self.gpu, self.wtype, self.rows, self.k = gpu, wtype, int(rows), int(k)
+        h = _vp()
+        if host_bytes is not None:
+            host_bytes = np.ascontiguousarray(host_bytes, np.uint8)
+            need = self.rows * row_bytes(wtype, k) if row_bytes(wtype, k) > 0 else 0
+            if host_bytes.size < need:
+                raise GpuError(ESHAPE, f"DeviceTensor: {host_bytes.size} bytes for {rows} rows of {need // max(rows, 1)}")
+            gpu._check(gpu.lib.bm_weights_create(gpu.ctx, wtype, self.rows, self.k, host_bytes.ctypes.data, C.byref(h)))
+        else:
+            gpu._check(gpu.lib.bm_weights_wrap(gpu.ctx, wtype, self.rows, self.k, dev_ptr, C.byref(h)))
+        self.handle = h.value
+
+    @property
+    def dev_ptr(self):
+        return self.gpu.lib.bm_weights_dev(self.handle)
+
+    def free(self):
+        if self.handle:
+            self.gpu.lib.bm_weights_destroy(self.handle)
+            self.handle = None
+
+
+class Q8Act:
+    """Quantized activation scratch: m_cap columns of k values in the form weight type `wtype` dots against."""
+
+    def __init__(self, gpu, wtype, k, m_cap):
+        self.gpu, self.wtype, self.k, self.m_cap = gpu, wtype, int(k), int(m_cap)
+        h = _vp()
+        gpu._check(gpu.lib.bm_act_create(gpu.ctx, wtype, self.k, self.m_cap, C.byref(h)))
+        self.handle = h.value
+
+    def download(self, col):
+        out = np.empty(col_bytes(self.wtype, self.k), np.uint8)
+        self.gpu._check(self.gpu.lib.bm_act_download(self.gpu.ctx, self.handle, col, out.ctypes.data))
+        return out
+
+    def upload(self, col, host_bytes):
+        host_bytes = np.ascontiguousarray(host_bytes, np.uint8)
+        assert host_bytes.size == col_bytes(self.wtype, self.k)
+        self.gpu._check(self.gpu.lib.bm_act_upload(self.gpu.ctx, self.handle, col, host_bytes.ctypes.data))
+
+    def free(self):
+        if self.handle:
+            self.gpu.lib.bm_act_destroy(self.handle)
+            self.handle = None
+
+
+def _ptr(x):
+    if x is None:
+        return None
+    if isinstance(x, DeviceBuffer):
+        return x.ptr
+    return x  # a raw device address (e.g. torch.Tensor.data_ptr())
+
+
+class Gpu:
+    """A device context: stream, fault word and the launchers (the reference's `Gpu` and its kernel structs)."""
+
+    def __init__(self, device=0, stream=None):
+        self.lib = load_library()
+        ctx = _vp()
+        if stream is None:
+            rc = self.lib.bm_ctx_create(device, C.byref(ctx))
+        else:
+            rc = self.lib.bm_ctx_create_on_stream(device, stream, C.byref(ctx))
+        if rc != OK:
+            raise GpuError(rc, self.lib.bm_last_error(None).decode())
+        self.ctx = ctx.value
+
+    def _check(self, rc):
+        if rc != OK:
+            raise GpuError(rc, self.lib.bm_last_error(self.ctx).decode())
+
+    def close(self):
+        if self.ctx:
+            self.lib.bm_ctx_destroy(self.ctx)
+            self.ctx = None
+
+    # -- context
+    def stream(self):
+        return self.lib.bm_ctx_stream(self.ctx)
+
+    def sync(self):
+        self._check(self.lib.bm_ctx_sync(self.ctx))
+
+    def set_layer(self, layer):
+        self._check(self.lib.bm_set_layer(self.ctx, layer))
+
+    def fault(self, layer=LAYER_NONE):
+        w0, mask = _u32(), _u32()
+        self._check(self.lib.bm_fault_read(self.ctx, layer, C.byref(w0), C.byref(mask)))
+        return w0.value, mask.value
+
+    def fault_clear(self):
+        self._check(self.lib.bm_fault_clear(self.ctx))
+
+    # -- buffers
+    def buffer(self, dtype, count, host=None):
+        b = DeviceBuffer(self, dtype, count)
+        if host is not None:
+            b.upload(host)
+        return b
+
+    def upload(self, host, dtype=None):
+        host = np.ascontiguousarray(host, dtype)
+        return DeviceBuffer(self, host.dtype, host.size).upload(host)
+
+    def weights(self, wtype, rows, k, host_bytes):
+        return DeviceTensor(self, wtype, rows, k, host_bytes=host_bytes)
+
+    def act(self, wtype, k, m_cap):
+        return Q8Act(self, wtype, k, m_cap)
+
+    # -- launchers (asynchronous on the context's stream)
+    def enqueue_quantize(self, x, m, act):
+        self._check(self.lib.bm_quantize(self.ctx, _ptr(x), m, act.handle))
+
+    def enqueue_gemv(self, w, act, m, y):
+        self._check(self.lib.bm_gemv(self.ctx, w.handle, act.handle, m, _ptr(y)))
+
+    def enqueue_gate_up(self, wg, wu, act, sel, n_slots, rows_per_expert, slots_per_col, h, act_h=None):
+        self._check(self.lib.bm_gate_up(self.ctx, wg.handle, wu.handle, act.handle, _ptr(sel), n_slots, rows_per_expert,
+                                        slots_per_col, _ptr(h), act_h.handle if act_h is not None else None))
+
+    def enqueue_gemv_sel(self, w, act, sel, n_slots, rows_per_expert, y):
+        self._check(self.lib.bm_gemv_sel(self.ctx, w.handle, act.handle, _ptr(sel), n_slots, rows_per_expert, _ptr(y)))
+
+    def enqueue_combine_tokens(self, down, w, resid, rows, n_slots, m, y):
+        self._check(self.lib.bm_combine_tokens(self.ctx, _ptr(down), _ptr(w), _ptr(resid), rows, n_slots, m, _ptr(y)))
+
+    def enqueue_down_combine(self, w, act, sel, wts, resid, n_slots_per_token, m, rows_per_expert, y):
+        self._check(self.lib.bm_down_combine(self.ctx, w.handle, act.handle, _ptr(sel), _ptr(wts), _ptr(resid),
+                                             n_slots_per_token, m, rows_per_expert, _ptr(y)))
+
+    def enqueue_block_sums(self, w, row, act, col, out):
+        self._check(self.lib.bm_block_sums(self.ctx, w.handle, row, act.handle, col, _ptr(out)))

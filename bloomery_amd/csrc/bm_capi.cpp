@@ -1,0 +1,438 @@
+// The C ABI of libbm_moe_hip.so (include/bm_moe.h): handles, the host-side geometry checks the reference's
+// launchers make before a launch (crates/gpu/src/q4k_sel.rs:990-1042 and its siblings), and the calls into the
+// kernels. Refusals carry a message naming the entry point and the lengths, as GpuError::Shape does.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+
+#include <hip/hip_runtime.h>
+
+#include "../../include/bm_moe.h"
+#include "bm_kernels.h"
+
+struct bm_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool own_stream = false;
+    uint32_t *fault = nullptr;
+    uint32_t layer = BM_LAYER_NONE;
+    std::string err;
+};
+
+struct bm_weights {
+    bm_ctx *ctx;
+    int wtype;
+    int64_t rows;
+    int k;
+    uint8_t *dev;
+    bool owned;
+};
+
+struct bm_act {
+    bm_ctx *ctx;
+    int wtype; // the weight type whose activation form this is
+    int k, m_cap;
+    uint8_t *dev;
+};
+
+static thread_local std::string g_err;
+
+static int fail(bm_ctx *ctx, int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_err = buf;
+    if (ctx) ctx->err = buf;
+    return code;
+}
+
+static int driver(bm_ctx *ctx, const char *what, hipError_t e) {
+    if (e == hipSuccess) return BM_OK;
+    return fail(ctx, BM_EDRIVER, "%s: %s", what, hipGetErrorString(e));
+}
+
+static bool known_type(int t) { return t == BM_TYPE_Q4_K || t == BM_TYPE_Q6_K || t == BM_TYPE_IQ2_XXS; }
+// Q8_2_X4 for the K-quants, Q8_K for IQ2_XXS (crates/gguf/src/qtype.rs host_act).
+static int act_form(int t) { return t == BM_TYPE_IQ2_XXS ? 1 : 0; }
+
+extern "C" {
+
+int bm_version(void) { return 100; }
+
+int64_t bm_row_bytes(int wtype, int k) {
+    if (!known_type(wtype)) return BM_ETYPE;
+    if (k <= 0 || k % 256 != 0) return BM_ESHAPE;
+    const int bb = wtype == BM_TYPE_Q4_K ? 144 : (wtype == BM_TYPE_Q6_K ? 210 : 66);
+    return (int64_t)(k / 256) * bb;
+}
+
+int64_t bm_col_bytes(int wtype, int k) {
+    if (!known_type(wtype)) return BM_ETYPE;
+    if (k <= 0 || k % 256 != 0) return BM_ESHAPE;
+    return (int64_t)(k / 256) * (wtype == BM_TYPE_IQ2_XXS ? 296 : 288);
+}
+
+const char *bm_last_error(const bm_ctx *ctx) { return ctx ? ctx->err.c_str() : g_err.c_str(); }
+
+static int ctx_make(int device, hipStream_t stream, bool own, bm_ctx **out) {
+    if (!out) return fail(nullptr, BM_EARG, "bm_ctx_create: out is NULL");
+    *out = nullptr;
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) return fail(nullptr, BM_EDRIVER, "bm_ctx_create: hipSetDevice(%d): %s", device, hipGetErrorString(e));
+    bm_ctx *c = new (std::nothrow) bm_ctx();
+    if (!c) return fail(nullptr, BM_EDRIVER, "bm_ctx_create: out of host memory");
+    c->device = device;
+    if (own) {
+        e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking); // default priority
+        if (e != hipSuccess) {
+            delete c;
+            return fail(nullptr, BM_EDRIVER, "bm_ctx_create: hipStreamCreate: %s", hipGetErrorString(e));
+        }
+        c->own_stream = true;
+    } else {
+        c->stream = stream;
+    }
+    e = hipMalloc((void **)&c->fault, sizeof(uint32_t) * BM_FAULT_WORDS);
+    if (e == hipSuccess) {
+        // word 0 all ones, the masks zero: synchronous here, load time
+        e = hipMemset(c->fault, 0, sizeof(uint32_t) * BM_FAULT_WORDS);
+        if (e == hipSuccess) e = hipMemset(c->fault, 0xff, sizeof(uint32_t));
+    }
+    if (e != hipSuccess) {
+        if (c->fault) (void)hipFree(c->fault);
+        if (c->own_stream) (void)hipStreamDestroy(c->stream);
+        delete c;
+        return fail(nullptr, BM_EDRIVER, "bm_ctx_create: fault word: %s", hipGetErrorString(e));
+    }
+    *out = c;
+    return BM_OK;
+}
+
+int bm_ctx_create(int device, bm_ctx **out) { return ctx_make(device, nullptr, true, out); }
+
+int bm_ctx_create_on_stream(int device, void *hip_stream, bm_ctx **out) {
+    return ctx_make(device, (hipStream_t)hip_stream, false, out);
+}
+
+void bm_ctx_destroy(bm_ctx *ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(ctx->fault);
+    if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+void *bm_ctx_stream(bm_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+int bm_ctx_sync(bm_ctx *ctx) {
+    if (!ctx) return fail(nullptr, BM_EARG, "bm_ctx_sync: ctx is NULL");
+    return driver(ctx, "bm_ctx_sync", hipStreamSynchronize(ctx->stream));
+}
+
+int bm_set_layer(bm_ctx *ctx, uint32_t layer) {
+    if (!ctx) return fail(nullptr, BM_EARG, "bm_set_layer: ctx is NULL");
+    if (layer > BM_LAYER_NONE) return fail(ctx, BM_ESHAPE, "bm_set_layer: layer %u is past %u", layer, BM_LAYER_NONE);
+    ctx->layer = layer;
+    return BM_OK;
+}
+
+uint32_t *bm_fault_word_dev(bm_ctx *ctx) { return ctx ? ctx->fault : nullptr; }
+
+int bm_fault_read(bm_ctx *ctx, uint32_t layer, uint32_t *word0, uint32_t *mask) {
+    if (!ctx) return fail(nullptr, BM_EARG, "bm_fault_read: ctx is NULL");
+    if (layer > BM_LAYER_NONE) return fail(ctx, BM_ESHAPE, "bm_fault_read: layer %u is past %u", layer, BM_LAYER_NONE);
+    int rc = driver(ctx, "bm_fault_read: sync", hipStreamSynchronize(ctx->stream));
+    if (rc) return rc;
+    if (word0) rc = driver(ctx, "bm_fault_read", hipMemcpy(word0, ctx->fault, 4, hipMemcpyDeviceToHost));
+    if (!rc && mask) rc = driver(ctx, "bm_fault_read", hipMemcpy(mask, ctx->fault + 1 + layer, 4, hipMemcpyDeviceToHost));
+    return rc;
+}
+
+static bmk::Launch launch_of(bm_ctx *ctx) { return bmk::Launch{ctx->stream, ctx->fault, ctx->layer}; }
+
+int bm_fault_clear(bm_ctx *ctx) {
+    if (!ctx) return fail(nullptr, BM_EARG, "bm_fault_clear: ctx is NULL");
+    bmk::Launch L = launch_of(ctx);
+    hipError_t e = bmk::fill_u32(L, ctx->fault + 1, 0u, BM_FAULT_WORDS - 1);
+    if (e == hipSuccess) e = bmk::fill_u32(L, ctx->fault, BM_FAULT_NONE, 1);
+    return driver(ctx, "bm_fault_clear", e);
+}
+
+// ------------------------------------------------------------------------------------------------ buffers
+
+int bm_dev_alloc(bm_ctx *ctx, size_t bytes, void **out_dev) {
+    if (!ctx || !out_dev) return fail(ctx, BM_EARG, "bm_dev_alloc: NULL argument");
+    return driver(ctx, "bm_dev_alloc", hipMalloc(out_dev, bytes ? bytes : 1));
+}
+
+int bm_dev_free(bm_ctx *ctx, void *dev) {
+    if (!ctx) return fail(nullptr, BM_EARG, "bm_dev_free: ctx is NULL");
+    return driver(ctx, "bm_dev_free", hipFree(dev));
+}
+
+int bm_dev_upload(bm_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes) {
+    if (!ctx || !dst_dev || !src_host) return fail(ctx, BM_EARG, "bm_dev_upload: NULL argument");
+    int rc = driver(ctx, "bm_dev_upload: sync", hipStreamSynchronize(ctx->stream));
+    if (rc) return rc;
+    return driver(ctx, "bm_dev_upload", hipMemcpy(dst_dev, src_host, bytes, hipMemcpyHostToDevice));
+}
+
+int bm_dev_download(bm_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes) {
+    if (!ctx || !dst_host || !src_dev) return fail(ctx, BM_EARG, "bm_dev_download: NULL argument");
+    int rc = driver(ctx, "bm_dev_download: sync", hipStreamSynchronize(ctx->stream));
+    if (rc) return rc;
+    return driver(ctx, "bm_dev_download", hipMemcpy(dst_host, src_dev, bytes, hipMemcpyDeviceToHost));
+}
+
+int bm_dev_memset(bm_ctx *ctx, void *dst_dev, int byte, size_t bytes) {
+    if (!ctx || !dst_dev) return fail(ctx, BM_EARG, "bm_dev_memset: NULL argument");
+    int rc = driver(ctx, "bm_dev_memset: sync", hipStreamSynchronize(ctx->stream));
+    if (rc) return rc;
+    rc = driver(ctx, "bm_dev_memset", hipMemset(dst_dev, byte, bytes));
+    if (rc) return rc;
+    return driver(ctx, "bm_dev_memset: sync", hipDeviceSynchronize());
+}
+
+static int weights_make(bm_ctx *ctx, const char *what, int wtype, int64_t rows, int k, const void *host,
+                        const void *dev, bm_weights **out) {
+    if (!ctx || !out) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    *out = nullptr;
+    if (!known_type(wtype)) return fail(ctx, BM_ETYPE, "%s: weight type %d has no kernel (12 Q4_K, 14 Q6_K, 16 IQ2_XXS)", what, wtype);
+    if (k <= 0 || k % 256 != 0) return fail(ctx, BM_ESHAPE, "%s: k = %d is not a whole number of 256-value super-blocks", what, k);
+    if (rows <= 0) return fail(ctx, BM_ESHAPE, "%s: rows = %lld must be positive", what, (long long)rows);
+    const size_t bytes = (size_t)rows * (size_t)bm_row_bytes(wtype, k);
+    bm_weights *w = new (std::nothrow) bm_weights{ctx, wtype, rows, k, nullptr, false};
+    if (!w) return fail(ctx, BM_EDRIVER, "%s: out of host memory", what);
+    if (host) {
+        // 16 spare bytes: the last row's vector loads never leave the allocation
+        hipError_t e = hipMalloc((void **)&w->dev, bytes + 16);
+        if (e == hipSuccess) e = hipMemcpy(w->dev, host, bytes, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            if (w->dev) (void)hipFree(w->dev);
+            delete w;
+            return driver(ctx, what, e);
+        }
+        w->owned = true;
+    } else {
+        if (!dev) {
+            delete w;
+            return fail(ctx, BM_EARG, "%s: dev_bytes is NULL", what);
+        }
+        if (wtype == BM_TYPE_Q4_K && ((uintptr_t)dev & 15) != 0) {
+            delete w;
+            return fail(ctx, BM_ESHAPE, "%s: Q4_K rows are read with 16-byte loads, dev_bytes %p is not 16-byte aligned", what, dev);
+        }
+        if (((uintptr_t)dev & 1) != 0) {
+            delete w;
+            return fail(ctx, BM_ESHAPE, "%s: dev_bytes %p is not 2-byte aligned", what, dev);
+        }
+        w->dev = (uint8_t *)dev;
+    }
+    *out = w;
+    return BM_OK;
+}
+
+int bm_weights_create(bm_ctx *ctx, int wtype, int64_t rows, int k, const void *host_bytes, bm_weights **out) {
+    if (!host_bytes) return fail(ctx, BM_EARG, "bm_weights_create: host_bytes is NULL");
+    return weights_make(ctx, "bm_weights_create", wtype, rows, k, host_bytes, nullptr, out);
+}
+
+int bm_weights_wrap(bm_ctx *ctx, int wtype, int64_t rows, int k, const void *dev_bytes, bm_weights **out) {
+    return weights_make(ctx, "bm_weights_wrap", wtype, rows, k, nullptr, dev_bytes, out);
+}
+
+void bm_weights_destroy(bm_weights *w) {
+    if (!w) return;
+    if (w->owned) (void)hipFree(w->dev);
+    delete w;
+}
+
+const void *bm_weights_dev(const bm_weights *w) { return w ? w->dev : nullptr; }
+
+int bm_act_create(bm_ctx *ctx, int wtype, int k, int m_cap, bm_act **out) {
+    if (!ctx || !out) return fail(ctx, BM_EARG, "bm_act_create: NULL argument");
+    *out = nullptr;
+    if (!known_type(wtype)) return fail(ctx, BM_ETYPE, "bm_act_create: weight type %d has no activation form here", wtype);
+    if (k <= 0 || k % 256 != 0) return fail(ctx, BM_ESHAPE, "bm_act_create: activation columns are whole 256-value super-blocks, k = %d", k);
+    if (m_cap <= 0) return fail(ctx, BM_ESHAPE, "bm_act_create: m_cap = %d must be positive", m_cap);
+    bm_act *a = new (std::nothrow) bm_act{ctx, wtype, k, m_cap, nullptr};
+    if (!a) return fail(ctx, BM_EDRIVER, "bm_act_create: out of host memory");
+    const size_t bytes = (size_t)m_cap * (size_t)bm_col_bytes(wtype, k);
+    hipError_t e = hipMalloc((void **)&a->dev, bytes);
+    if (e == hipSuccess) e = hipMemset(a->dev, 0, bytes);
+    if (e != hipSuccess) {
+        if (a->dev) (void)hipFree(a->dev);
+        delete a;
+        return driver(ctx, "bm_act_create", e);
+    }
+    *out = a;
+    return BM_OK;
+}
+
+void bm_act_destroy(bm_act *act) {
+    if (!act) return;
+    (void)hipFree(act->dev);
+    delete act;
+}
+
+int bm_act_download(bm_ctx *ctx, const bm_act *act, int col, void *host_bytes) {
+    if (!ctx || !act || !host_bytes) return fail(ctx, BM_EARG, "bm_act_download: NULL argument");
+    if (col < 0 || col >= act->m_cap) return fail(ctx, BM_ESHAPE, "bm_act_download: column %d of %d", col, act->m_cap);
+    const size_t cb = (size_t)bm_col_bytes(act->wtype, act->k);
+    return bm_dev_download(ctx, host_bytes, act->dev + (size_t)col * cb, cb);
+}
+
+int bm_act_upload(bm_ctx *ctx, bm_act *act, int col, const void *host_bytes) {
+    if (!ctx || !act || !host_bytes) return fail(ctx, BM_EARG, "bm_act_upload: NULL argument");
+    if (col < 0 || col >= act->m_cap) return fail(ctx, BM_ESHAPE, "bm_act_upload: column %d of %d", col, act->m_cap);
+    const size_t cb = (size_t)bm_col_bytes(act->wtype, act->k);
+    return bm_dev_upload(ctx, act->dev + (size_t)col * cb, host_bytes, cb);
+}
+
+// ------------------------------------------------------------------------------------------------ launchers
+
+int bm_quantize(bm_ctx *ctx, const float *x_dev, int m, bm_act *act) {
+    const char *what = "bm_quantize";
+    if (!ctx || !x_dev || !act) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (m < 1 || m > act->m_cap) return fail(ctx, BM_ESHAPE, "%s: m = %d columns, act holds %d", what, m, act->m_cap);
+    return driver(ctx, what, bmk::quantize(launch_of(ctx), act->wtype, x_dev, m, act->k, act->dev));
+}
+
+// A weight stack and an activation of one form and one k.
+static int check_pair(bm_ctx *ctx, const char *what, const bm_weights *w, const bm_act *act) {
+    if (act_form(w->wtype) != act_form(act->wtype))
+        return fail(ctx, BM_ETYPE, "%s: weight type %d dots %s columns, act was made for type %d", what, w->wtype,
+                    act_form(w->wtype) ? "Q8_K" : "Q8_2_X4", act->wtype);
+    if (w->k != act->k) return fail(ctx, BM_ESHAPE, "%s: weight rows hold k = %d values, act columns %d", what, w->k, act->k);
+    return BM_OK;
+}
+
+int bm_gemv(bm_ctx *ctx, const bm_weights *w, const bm_act *act, int m, float *y_dev) {
+    const char *what = "bm_gemv";
+    if (!ctx || !w || !act || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    int rc = check_pair(ctx, what, w, act);
+    if (rc) return rc;
+    if (m < 1 || m > 8 || m > act->m_cap)
+        return fail(ctx, BM_ESHAPE, "%s: m = %d columns outside 1..=8 or past act's %d", what, m, act->m_cap);
+    const int per = bmk::gemv_max_cols(w->wtype, w->k);
+    if (per < 1) return fail(ctx, BM_ESHAPE, "%s: one column of k = %d does not fit the workgroup's LDS", what, w->k);
+    bmk::Launch L = launch_of(ctx);
+    for (int c0 = 0; c0 < m; c0 += per) {
+        const int mc = m - c0 < per ? m - c0 : per;
+        rc = driver(ctx, what, bmk::gemv(L, w->wtype, w->dev, w->rows, w->k, act->dev, m, c0, mc, y_dev));
+        if (rc) return rc;
+    }
+    return BM_OK;
+}
+
+// rows a positive multiple of rows_per_expert (crates/gpu/src/q4k_sel.rs:1013-1023).
+static int check_stack(bm_ctx *ctx, const char *what, const bm_weights *w, int rows_per_expert, int *n_experts) {
+    if (rows_per_expert <= 0 || w->rows % rows_per_expert != 0)
+        return fail(ctx, BM_ESHAPE, "%s: w.rows() %lld must be a positive multiple of rows_per_expert %d", what,
+                    (long long)w->rows, rows_per_expert);
+    const int64_t n = w->rows / rows_per_expert;
+    if (n > 0x7fffffff) return fail(ctx, BM_ESHAPE, "%s: %lld experts", what, (long long)n);
+    *n_experts = (int)n;
+    return BM_OK;
+}
+
+int bm_gate_up(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_act *act, const uint32_t *sel_dev,
+               int n_slots, int rows_per_expert, int slots_per_col, float *h_dev, bm_act *act_h) {
+    const char *what = "bm_gate_up";
+    if (!ctx || !wg || !wu || !act || !sel_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (!h_dev && !act_h) return fail(ctx, BM_EARG, "%s: neither h_dev nor act_h to write", what);
+    if (wg->wtype != wu->wtype)
+        return fail(ctx, BM_ETYPE, "%s: gate is type %d and up type %d; one launch reads one type", what, wg->wtype, wu->wtype);
+    int rc = check_pair(ctx, what, wg, act);
+    if (rc) return rc;
+    if (wu->k != wg->k || wu->rows != wg->rows)
+        return fail(ctx, BM_ESHAPE, "%s: gate is %lld x %d, up %lld x %d", what, (long long)wg->rows, wg->k, (long long)wu->rows, wu->k);
+    int n_experts = 0;
+    rc = check_stack(ctx, what, wg, rows_per_expert, &n_experts);
+    if (rc) return rc;
+    if (n_slots < 1) return fail(ctx, BM_ESHAPE, "%s: need n_slots >= 1, got %d", what, n_slots);
+    if (slots_per_col < 1) return fail(ctx, BM_ESHAPE, "%s: slots_per_col = %d must be at least 1", what, slots_per_col);
+    if ((int64_t)n_slots > (int64_t)act->m_cap * slots_per_col)
+        return fail(ctx, BM_ESHAPE, "%s: n_slots %d needs %d columns at %d slots a column, act holds %d", what, n_slots,
+                    (n_slots + slots_per_col - 1) / slots_per_col, slots_per_col, act->m_cap);
+    uint8_t *ah = nullptr;
+    if (act_h) {
+        if (act_form(act_h->wtype) != 0)
+            return fail(ctx, BM_ETYPE, "%s: the fused quantizer writes Q8_2_X4 columns; act_h was made for type %d (Q8_K)", what, act_h->wtype);
+        if (act_h->k != rows_per_expert)
+            return fail(ctx, BM_ESHAPE, "%s: act_h columns hold k = %d values, a slot writes rows_per_expert = %d", what, act_h->k, rows_per_expert);
+        if (act_h->m_cap < n_slots)
+            return fail(ctx, BM_ESHAPE, "%s: a column of act_h per slot: %d slots, act_h holds %d", what, n_slots, act_h->m_cap);
+        ah = act_h->dev;
+    }
+    return driver(ctx, what, bmk::gate_up(launch_of(ctx), wg->wtype, wg->dev, wu->dev, n_experts, wg->k, act->dev, sel_dev,
+                                          n_slots, rows_per_expert, slots_per_col, h_dev, ah));
+}
+
+int bm_gemv_sel(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const uint32_t *sel_dev, int n_slots,
+                int rows_per_expert, float *y_dev) {
+    const char *what = "bm_gemv_sel";
+    if (!ctx || !w || !act || !sel_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    int rc = check_pair(ctx, what, w, act);
+    if (rc) return rc;
+    int n_experts = 0;
+    rc = check_stack(ctx, what, w, rows_per_expert, &n_experts);
+    if (rc) return rc;
+    if (n_slots < 1) return fail(ctx, BM_ESHAPE, "%s: need n_slots >= 1, got %d", what, n_slots);
+    if (act->m_cap < n_slots)
+        return fail(ctx, BM_ESHAPE, "%s: an activation column per slot: act.m() = %d must be at least n_slots = %d", what, act->m_cap, n_slots);
+    return driver(ctx, what, bmk::gemv_sel(launch_of(ctx), w->wtype, w->dev, n_experts, w->k, act->dev, sel_dev, n_slots,
+                                           rows_per_expert, y_dev));
+}
+
+int bm_combine_tokens(bm_ctx *ctx, const float *down_dev, const float *w_dev, const float *resid_dev, int rows,
+                      int n_slots, int m, float *y_dev) {
+    const char *what = "bm_combine_tokens";
+    if (!ctx || !down_dev || !w_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (rows < 1 || n_slots < 1 || m < 1)
+        return fail(ctx, BM_ESHAPE, "%s: rows %d, n_slots %d and m %d must all be positive", what, rows, n_slots, m);
+    return driver(ctx, what, bmk::combine_tokens(launch_of(ctx), down_dev, w_dev, resid_dev, rows, n_slots, m, y_dev));
+}
+
+int bm_down_combine(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const uint32_t *sel_dev,
+                    const float *w_dev, const float *resid_dev, int n_slots_per_token, int m, int rows_per_expert,
+                    float *y_dev) {
+    const char *what = "bm_down_combine";
+    if (!ctx || !w || !act || !sel_dev || !w_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    int rc = check_pair(ctx, what, w, act);
+    if (rc) return rc;
+    int n_experts = 0;
+    rc = check_stack(ctx, what, w, rows_per_expert, &n_experts);
+    if (rc) return rc;
+    if (n_slots_per_token < 1 || n_slots_per_token > bmk::kMaxCombineSlots)
+        return fail(ctx, BM_ESHAPE, "%s: %d slots a token outside 1..=%d", what, n_slots_per_token, bmk::kMaxCombineSlots);
+    if (m < 1) return fail(ctx, BM_ESHAPE, "%s: need m >= 1 tokens, got %d", what, m);
+    if ((int64_t)m * n_slots_per_token > act->m_cap)
+        return fail(ctx, BM_ESHAPE, "%s: an activation column per slot: %d tokens x %d slots, act holds %d", what, m,
+                    n_slots_per_token, act->m_cap);
+    const size_t lds = (size_t)n_slots_per_token * (size_t)bm_col_bytes(act->wtype, act->k) + 4096;
+    if (lds > (size_t)bmk::kMaxLds)
+        return fail(ctx, BM_ESHAPE, "%s: %d columns of k = %d do not fit the workgroup's LDS; use bm_gemv_sel and bm_combine_tokens", what,
+                    n_slots_per_token, act->k);
+    return driver(ctx, what, bmk::down_combine(launch_of(ctx), w->wtype, w->dev, n_experts, w->k, act->dev, sel_dev, w_dev,
+                                               resid_dev, n_slots_per_token, m, rows_per_expert, y_dev));
+}
+
+int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *act, int col, int32_t *out_dev) {
+    const char *what = "bm_block_sums";
+    if (!ctx || !w || !act || !out_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    int rc = check_pair(ctx, what, w, act);
+    if (rc) return rc;
+    if (row < 0 || row >= w->rows) return fail(ctx, BM_ESHAPE, "%s: row %lld of %lld", what, (long long)row, (long long)w->rows);
+    if (col < 0 || col >= act->m_cap) return fail(ctx, BM_ESHAPE, "%s: column %d of %d", what, col, act->m_cap);
+    const uint8_t *wrow = w->dev + (size_t)row * (size_t)bm_row_bytes(w->wtype, w->k);
+    const uint8_t *c = act->dev + (size_t)col * (size_t)bm_col_bytes(act->wtype, act->k);
+    return driver(ctx, what, bmk::block_sums(launch_of(ctx), w->wtype, wrow, w->k, c, out_dev));
+}
+
+} // extern "C"

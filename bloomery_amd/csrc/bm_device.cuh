@@ -1,0 +1,434 @@
+// Device-side building blocks of the quantized row dots on gfx950 (wave64).
+//
+// Lane map ("quad"): one weight row is dotted by four consecutive lanes. The CPU path this library reproduces
+// (crates/qdot/src/lib.rs:4363-4447 Q4_K, :4776-4874 Q6_K, :8677-8724 IQ2_XXS) keeps eight f32 accumulators per
+// row and walks the super-blocks in order; here each lane of the quad owns two of the eight and walks every
+// super-block of the row itself, so each accumulator sees the reference's fused multiply-adds in the reference's
+// order and the final butterfly over the quad is the reference's closing sum ((t0+t2)+(t1+t3), t_l = acc_l +
+// acc_{l+4}). The integer sums are formed with v_dot4_i32_i8 over the same 16-value (Q4_K, Q6_K) or 4-value
+// (IQ2_XXS) spans the reference's i32 lanes cover; they are exact, so their inner order is free.
+//
+// Build: -ffp-contract=off (a product meets a sum in one rounding only where fmaf is written), f32 denormals
+// kept, correctly rounded f32 divide (hipcc's defaults for gfx950).
+#ifndef BM_DEVICE_CUH
+#define BM_DEVICE_CUH
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef uint32_t u32;
+
+#define BM_Q4K 12
+#define BM_Q6K 14
+#define BM_IQ2XXS 16
+
+#define BM_Q4K_BLOCK 144
+#define BM_Q6K_BLOCK 210
+#define BM_IQ2XXS_BLOCK 66
+#define BM_Q82X4_STRIDE 144
+#define BM_Q8K_STRIDE 296
+
+// ------------------------------------------------------------------------------------------------ scalars
+
+__device__ __forceinline__ float bm_bits_f32(u32 u) { return __uint_as_float(u); }
+__device__ __forceinline__ u32 bm_f32_bits(float f) { return __float_as_uint(f); }
+
+// f16 bits -> f32: v_cvt_f32_f16, exact for every f16 (subnormals included; f16 denormals are on).
+__device__ __forceinline__ float bm_half_to_f32(u32 h16) { return __half2float(__ushort_as_half((unsigned short)h16)); }
+
+__device__ __forceinline__ float bm_bf16_to_f32(u32 b16) { return bm_bits_f32(b16 << 16); }
+
+// crates/gguf/src/quant.rs:544-551.
+__device__ __forceinline__ u32 bm_fp32_to_bf16_bits(float s) {
+    u32 u = bm_f32_bits(s);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return ((u >> 16) | 64u) & 0xffffu;
+    return ((u + (0x7fffu + ((u >> 16) & 1u))) >> 16) & 0xffffu;
+}
+
+// Round to nearest even through one f32 add (crates/gguf/src/quant.rs:2222-2226). __fadd_rn keeps the add from
+// being folded or fused whatever the caller's surrounding arithmetic.
+__device__ __forceinline__ int bm_nearest_int(float v) {
+    float val = __fadd_rn(v, 12582912.0f);
+    return (int)(bm_f32_bits(val) & 0x007fffffu) - 0x00400000;
+}
+
+// crates/gguf/src/quant.rs:2237-2241.
+__device__ __forceinline__ float bm_q82_inverse(u32 t) {
+    float d = bm_bf16_to_f32(t);
+    float id = d > 0.0f ? __fdiv_rn(1.0f, d) : 0.0f;
+    return (bm_f32_bits(id) & 0x7fffffffu) < 0x7f800000u ? id : 0.0f;
+}
+
+__device__ __forceinline__ int bm_sdot4(u32 a, u32 b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
+
+// 16 bytes from an address of any alignment (global memory takes unaligned vector loads on this target).
+__device__ __forceinline__ uint4 bm_ld16u(const uint8_t *p) {
+    uint4 v;
+    __builtin_memcpy(&v, p, 16);
+    return v;
+}
+
+__device__ __forceinline__ uint4 bm_ld16(const uint8_t *p) { return *reinterpret_cast<const uint4 *>(p); }
+
+__device__ __forceinline__ u32 bm_ld2u(const uint8_t *p) {
+    unsigned short v;
+    __builtin_memcpy(&v, p, 2);
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------ quad exchange
+
+// Lane ^ 1 and lane ^ 2 inside a quad, through DPP quad_perm (no LDS traffic).
+__device__ __forceinline__ float bm_quad_xor1(float v) {
+    return bm_bits_f32((u32)__builtin_amdgcn_mov_dpp((int)bm_f32_bits(v), 0xB1, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float bm_quad_xor2(float v) {
+    return bm_bits_f32((u32)__builtin_amdgcn_mov_dpp((int)bm_f32_bits(v), 0x4E, 0xF, 0xF, true));
+}
+__device__ __forceinline__ u32 bm_quad_bcast(u32 v, int k) {
+    switch (k) {
+    case 0:
+        return (u32)__builtin_amdgcn_mov_dpp((int)v, 0x00, 0xF, 0xF, true);
+    case 1:
+        return (u32)__builtin_amdgcn_mov_dpp((int)v, 0x55, 0xF, 0xF, true);
+    case 2:
+        return (u32)__builtin_amdgcn_mov_dpp((int)v, 0xAA, 0xF, 0xF, true);
+    default:
+        return (u32)__builtin_amdgcn_mov_dpp((int)v, 0xFF, 0xF, 0xF, true);
+    }
+}
+
+// ------------------------------------------------------------------------------------------ fault raising
+
+// crates/device/src/fault.rs:9-60: word 0 takes (layer << 8) | site by atomic minimum, word 1 + layer the site bit.
+__device__ __forceinline__ void bm_raise(u32 *fault, u32 layer, u32 site) {
+    atomicMin(&fault[0], (layer << 8) | site);
+    atomicOr(&fault[1 + layer], 1u << site);
+}
+
+// -------------------------------------------------------------------------------------------------- taps
+
+// A tap sees the exact integers a core forms. The launchers pass NoTap (everything folds away); the
+// verification kernel passes one that stores them, so it checks the code the launchers run.
+struct NoTap {
+    __device__ __forceinline__ void q4k(int, int, int, int) const {}
+    __device__ __forceinline__ void q4k_isum(int, int, int) const {}
+    __device__ __forceinline__ void q6k(int, int, int) const {}
+    __device__ __forceinline__ void iq2(int, int, int, int) const {}
+};
+
+// ------------------------------------------------------------------------------------------------- cores
+
+template <int WT>
+struct Blk;
+
+// ---- Q4_K: lane (c = q & 1, h = q >> 1) owns accumulators l = 4h + 2c and 4h + 2c + 1 of the reference's eight.
+// It reads bytes [32c + 16h, +16) of the first and of the second 64 code bytes: low nibbles are the 16 values of
+// half h of sub-block 2c (resp. 4 + 2c), high nibbles those of sub-block 2c + 1 (resp. 5 + 2c).
+template <>
+struct Blk<BM_Q4K> {
+    uint4 hdr, qa, qb;
+};
+
+__device__ __forceinline__ Blk<BM_Q4K> bm_load_q4k(const uint8_t *wrow, int i, int c, int h) {
+    const uint8_t *wb = wrow + (size_t)i * BM_Q4K_BLOCK;
+    Blk<BM_Q4K> b;
+    b.hdr = bm_ld16(wb);
+    b.qa = bm_ld16(wb + 16 + 32 * c + 16 * h);
+    b.qb = bm_ld16(wb + 16 + 64 + 32 * c + 16 * h);
+    return b;
+}
+
+__device__ __forceinline__ void bm_q4_dot16(uint4 q, uint4 alo, uint4 ahi, int &lo, int &hi) {
+    const u32 m = 0x0f0f0f0fu;
+    lo = bm_sdot4(q.x & m, alo.x, 0);
+    lo = bm_sdot4(q.y & m, alo.y, lo);
+    lo = bm_sdot4(q.z & m, alo.z, lo);
+    lo = bm_sdot4(q.w & m, alo.w, lo);
+    hi = bm_sdot4((q.x >> 4) & m, ahi.x, 0);
+    hi = bm_sdot4((q.y >> 4) & m, ahi.y, hi);
+    hi = bm_sdot4((q.z >> 4) & m, ahi.z, hi);
+    hi = bm_sdot4((q.w >> 4) & m, ahi.w, hi);
+}
+
+// One super-block of one column. `col` points at the column's Q8_2_X4 bytes (LDS), `i` is the super-block.
+template <class Tap>
+__device__ __forceinline__ void bm_dot_q4k(const Blk<BM_Q4K> &b, const uint8_t *col, int i, int c, int h, float &acc0,
+                                           float &acc1, const Tap &tap) {
+    const uint8_t *g0 = col + (size_t)(2 * i) * BM_Q82X4_STRIDE;
+    const uint8_t *g1 = g0 + BM_Q82X4_STRIDE;
+    const uint4 h0 = *reinterpret_cast<const uint4 *>(g0); // d bf16[4], isum i16[4]
+    const uint4 h1 = *reinterpret_cast<const uint4 *>(g1);
+    const float d = bm_half_to_f32(b.hdr.x & 0xffffu), dmin = bm_half_to_f32(b.hdr.x >> 16);
+    const u32 a0 = b.hdr.y, a1 = b.hdr.z, a2 = b.hdr.w; // crates/qdot/src/lib.rs:3868-3878
+    const u32 sc03 = a0 & 0x3f3f3f3fu, sc47 = (a2 & 0x0f0f0f0fu) | ((a0 >> 2) & 0x30303030u);
+    const u32 mn03 = a1 & 0x3f3f3f3fu, mn47 = ((a2 >> 4) & 0x0f0f0f0fu) | ((a1 >> 2) & 0x30303030u);
+    const int t0 = 2 * c, t1 = 2 * c + 1;
+    // The eight bf16 scales: group 0 holds sub-blocks 0..3, group 1 sub-blocks 4..7.
+    const u32 dw0 = c ? h0.y : h0.x, dw1 = c ? h1.y : h1.x; // scales of sub-blocks (t0, t1) and (4 + t0, 4 + t1)
+    const float d8_0a = bm_bits_f32(dw0 << 16), d8_0b = bm_bits_f32(dw0 & 0xffff0000u);
+    const float d8_1a = bm_bits_f32(dw1 << 16), d8_1b = bm_bits_f32(dw1 & 0xffff0000u);
+    // Min term of accumulators l = 4h + t: sub-block l's scale, sum and 6-bit min (lib.rs:4389-4394).
+    {
+        const u32 dwh = h ? dw1 : dw0;
+        const u32 sw = h ? (c ? h1.w : h1.z) : (c ? h0.w : h0.z);
+        const u32 mnw = h ? mn47 : mn03;
+        const float d8a = bm_bits_f32(dwh << 16), d8b = bm_bits_f32(dwh & 0xffff0000u);
+        const int sa = (int)(short)(sw & 0xffffu), sb = (int)(short)(sw >> 16);
+        const float ma = -(dmin * (float)((mnw >> (8 * t0)) & 0xffu));
+        const float mb = -(dmin * (float)((mnw >> (8 * t1)) & 0xffu));
+        acc0 = fmaf(d8a * (float)sa, ma, acc0);
+        acc1 = fmaf(d8b * (float)sb, mb, acc1);
+        tap.q4k_isum(i, 4 * h + t0, sa);
+        tap.q4k_isum(i, 4 * h + t1, sb);
+    }
+    // j = 0: sub-blocks t0, t1 (group 0); j = 1: sub-blocks 4 + t0, 4 + t1 (group 1) (lib.rs:4402-4436).
+    {
+        const uint4 alo = *reinterpret_cast<const uint4 *>(g0 + 16 + 32 * t0 + 16 * h);
+        const uint4 ahi = *reinterpret_cast<const uint4 *>(g0 + 16 + 32 * t1 + 16 * h);
+        int lo, hi;
+        bm_q4_dot16(b.qa, alo, ahi, lo, hi);
+        const float sa = (d * (float)((sc03 >> (8 * t0)) & 0xffu)) * d8_0a;
+        const float sb = (d * (float)((sc03 >> (8 * t1)) & 0xffu)) * d8_0b;
+        acc0 = fmaf(sa, (float)lo, acc0);
+        acc1 = fmaf(sb, (float)hi, acc1);
+        tap.q4k(i, t0, h, lo);
+        tap.q4k(i, t1, h, hi);
+    }
+    {
+        const uint4 alo = *reinterpret_cast<const uint4 *>(g1 + 16 + 32 * t0 + 16 * h);
+        const uint4 ahi = *reinterpret_cast<const uint4 *>(g1 + 16 + 32 * t1 + 16 * h);
+        int lo, hi;
+        bm_q4_dot16(b.qb, alo, ahi, lo, hi);
+        const float sa = (d * (float)((sc47 >> (8 * t0)) & 0xffu)) * d8_1a;
+        const float sb = (d * (float)((sc47 >> (8 * t1)) & 0xffu)) * d8_1b;
+        acc0 = fmaf(sa, (float)lo, acc0);
+        acc1 = fmaf(sb, (float)hi, acc1);
+        tap.q4k(i, 4 + t0, h, lo);
+        tap.q4k(i, 4 + t1, h, hi);
+    }
+}
+
+// ---- Q6_K: lane (c, h) owns accumulators l = 4h + c and 4h + c + 2. Per 128-value half j it reads ql bytes
+// [64j + 32c + 16h, +16) (low nibbles: quarter c, high nibbles: quarter c + 2, both half h) and qh bytes
+// [32j + 16h, +16) (bits 2a of quarter a).
+template <>
+struct Blk<BM_Q6K> {
+    uint4 ql0, qh0, ql1, qh1, sc;
+    u32 d;
+};
+
+__device__ __forceinline__ Blk<BM_Q6K> bm_load_q6k(const uint8_t *wrow, int i, int c, int h) {
+    const uint8_t *wb = wrow + (size_t)i * BM_Q6K_BLOCK;
+    Blk<BM_Q6K> b;
+    b.ql0 = bm_ld16u(wb + 32 * c + 16 * h);
+    b.qh0 = bm_ld16u(wb + 128 + 16 * h);
+    b.ql1 = bm_ld16u(wb + 64 + 32 * c + 16 * h);
+    b.qh1 = bm_ld16u(wb + 128 + 32 + 16 * h);
+    b.sc = bm_ld16u(wb + 192);
+    b.d = bm_ld2u(wb + 208);
+    return b;
+}
+
+// sum (q6 - 32) * a over 16 values: the 6-bit code fits a signed byte, so dot it as is and take 32 * sum a off.
+__device__ __forceinline__ int bm_q6_dot16(uint4 ql, uint4 qh, int nib_shift, int hi_shift, uint4 a) {
+    const u32 ml = 0x0f0f0f0fu, mh = 0x03030303u, ones = 0x01010101u;
+    int s = 0, sa = 0;
+    s = bm_sdot4(((ql.x >> nib_shift) & ml) | (((qh.x >> hi_shift) & mh) << 4), a.x, s);
+    s = bm_sdot4(((ql.y >> nib_shift) & ml) | (((qh.y >> hi_shift) & mh) << 4), a.y, s);
+    s = bm_sdot4(((ql.z >> nib_shift) & ml) | (((qh.z >> hi_shift) & mh) << 4), a.z, s);
+    s = bm_sdot4(((ql.w >> nib_shift) & ml) | (((qh.w >> hi_shift) & mh) << 4), a.w, s);
+    sa = bm_sdot4(ones, a.x, sa);
+    sa = bm_sdot4(ones, a.y, sa);
+    sa = bm_sdot4(ones, a.z, sa);
+    sa = bm_sdot4(ones, a.w, sa);
+    return s - 32 * sa;
+}
+
+template <class Tap>
+__device__ __forceinline__ void bm_dot_q6k(const Blk<BM_Q6K> &b, const uint8_t *col, int i, int c, int h, float &acc0,
+                                           float &acc1, const Tap &tap) {
+    const uint8_t *g0 = col + (size_t)(2 * i) * BM_Q82X4_STRIDE;
+    const float d = bm_half_to_f32(b.d);
+    const int t0 = c, t1 = c + 2;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const uint8_t *g = g0 + j * BM_Q82X4_STRIDE;
+        const uint2 dd = *reinterpret_cast<const uint2 *>(g); // four bf16 scales
+        const u32 dwa = dd.x, dwb = dd.y;                     // sub-blocks (0, 1) and (2, 3) of this half
+        const float d8a = c ? bm_bits_f32(dwa & 0xffff0000u) : bm_bits_f32(dwa << 16); // block t0 = c
+        const float d8b = c ? bm_bits_f32(dwb & 0xffff0000u) : bm_bits_f32(dwb << 16); // block t1 = c + 2
+        const uint4 aa = *reinterpret_cast<const uint4 *>(g + 16 + 32 * t0 + 16 * h);
+        const uint4 ab = *reinterpret_cast<const uint4 *>(g + 16 + 32 * t1 + 16 * h);
+        const uint4 ql = j ? b.ql1 : b.ql0, qh = j ? b.qh1 : b.qh0;
+        const int s0 = bm_q6_dot16(ql, qh, 0, 2 * c, aa);
+        const int s1 = bm_q6_dot16(ql, qh, 4, 2 * c + 4, ab);
+        // scale byte 8j + 2t + h (crates/qdot/src/lib.rs:4455 K_SHUFFLE_Q6K, :4794-4809)
+        const u32 w01 = j ? b.sc.z : b.sc.x, w23 = j ? b.sc.w : b.sc.y; // scale bytes 8j + 0..3 and 8j + 4..7
+        const int i0 = 2 * t0 + h, i1 = 2 * t1 + h;                     // byte index inside the half: 0..7
+        const int sc0 = (int)(signed char)(((i0 < 4 ? w01 : w23) >> (8 * (i0 & 3))) & 0xffu);
+        const int sc1 = (int)(signed char)(((i1 < 4 ? w01 : w23) >> (8 * (i1 & 3))) & 0xffu);
+        const float f0 = (d * (float)sc0) * d8a;
+        const float f1 = (d * (float)sc1) * d8b;
+        acc0 = fmaf(f0, (float)s0, acc0);
+        acc1 = fmaf(f1, (float)s1, acc1);
+        tap.q6k(i, 8 * j + i0, s0);
+        tap.q6k(i, 8 * j + i1, s1);
+    }
+}
+
+// ---- IQ2_XXS: lane q owns accumulators l = 2q and 2q + 1: values 8q .. 8q + 8 (grid group q) of every
+// sub-block. The quad loads the block's 64 code bytes once (16 each) and shares them through DPP.
+template <>
+struct Blk<BM_IQ2XXS> {
+    uint4 q; // sub-blocks 2q' and 2q' + 1 of this lane's quarter q': (idx, aux, idx, aux)
+    u32 d;
+};
+
+__device__ __forceinline__ Blk<BM_IQ2XXS> bm_load_iq2xxs(const uint8_t *wrow, int i, int q) {
+    const uint8_t *blk = wrow + (size_t)i * BM_IQ2XXS_BLOCK;
+    Blk<BM_IQ2XXS> b;
+    b.q = bm_ld16u(blk + 2 + 16 * q);
+    b.d = bm_ld2u(blk);
+    return b;
+}
+
+// LDS tables of the IQ2_XXS decode: the 256-point grid (8 magnitudes a point), the 128 sign bytes, and the 16
+// nibble -> byte-mask words (bit k set -> byte k = 0xff).
+struct Iq2Tables {
+    const uint2 *grid;
+    const uint8_t *ksigns;
+    const u32 *nibmask;
+};
+
+template <class Tap>
+__device__ __forceinline__ void bm_dot_iq2xxs(const Blk<BM_IQ2XXS> &b, const uint8_t *col, int i, int q,
+                                              const Iq2Tables &tb, float &acc0, float &acc1, const Tap &tap) {
+    const uint8_t *blk = col + (size_t)i * BM_Q8K_STRIDE;
+    const float dy = *reinterpret_cast<const float *>(blk);
+    const float d = 0.125f * bm_half_to_f32(b.d);
+    const float dmin = -d * 43.0f;
+    // Fold first (crates/qdot/src/lib.rs:8691-8694): accumulator l takes sub-block l's scale on its two bsums.
+    {
+        const int sca = 2 * (int)(b.q.y >> 28) + 1, scb = 2 * (int)(b.q.w >> 28) + 1; // sub-blocks 2q, 2q + 1
+        const uint2 bs = *reinterpret_cast<const uint2 *>(blk + 264 + 8 * q);          // bsums 4q .. 4q + 3
+        const int b0 = (int)(short)(bs.x & 0xffffu), b1 = (int)(short)(bs.x >> 16);
+        const int b2 = (int)(short)(bs.y & 0xffffu), b3 = (int)(short)(bs.y >> 16);
+        const int ma = sca * b0 + sca * b1, mb = scb * b2 + scb * b3;
+        const float f = dmin * dy;
+        acc0 = fmaf(f, (float)ma, acc0);
+        acc1 = fmaf(f, (float)mb, acc1);
+    }
+    int sumi0 = 0, sumi1 = 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        // Quarter k of the block (sub-blocks 2k, 2k + 1) sits in lane k of the quad.
+        const u32 idx_a = bm_quad_bcast(b.q.x, k), aux_a = bm_quad_bcast(b.q.y, k);
+        const u32 idx_b = bm_quad_bcast(b.q.z, k), aux_b = bm_quad_bcast(b.q.w, k);
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const int sb = 2 * k + e;
+            const u32 idx = e ? idx_b : idx_a, aux = e ? aux_b : aux_a;
+            const int sc = 2 * (int)(aux >> 28) + 1;
+            const uint2 g = tb.grid[(idx >> (8 * q)) & 0xffu];
+            const u32 sg = tb.ksigns[(aux >> (7 * q)) & 127u];
+            const u32 m_lo = tb.nibmask[sg & 15u], m_hi = tb.nibmask[sg >> 4];
+            // -mag where the sign bit is set: (mag ^ 0xff) + 1 per byte, no carry leaves a byte (mag > 0).
+            const u32 v_lo = (g.x ^ m_lo) + (m_lo & 0x01010101u), v_hi = (g.y ^ m_hi) + (m_hi & 0x01010101u);
+            const uint2 a = *reinterpret_cast<const uint2 *>(blk + 8 + 32 * sb + 8 * q);
+            const int i_lo = bm_sdot4(v_lo, a.x, 0), i_hi = bm_sdot4(v_hi, a.y, 0);
+            const int s_lo = bm_sdot4(0x01010101u, a.x, 0), s_hi = bm_sdot4(0x01010101u, a.y, 0);
+            // the reference sums sc * (v + 43) * a: the offset comes back out through the fold above
+            sumi0 += sc * (i_lo + 43 * s_lo);
+            sumi1 += sc * (i_hi + 43 * s_hi);
+            tap.iq2(i, sb, q, i_lo + i_hi);
+        }
+    }
+    const float f = d * dy;
+    acc0 = fmaf(f, (float)sumi0, acc0);
+    acc1 = fmaf(f, (float)sumi1, acc1);
+}
+
+// ---- closing sums: (t0 + t2) + (t1 + t3) with t_l = acc_l + acc_{l+4}; every lane of the quad gets the value.
+template <int WT>
+__device__ __forceinline__ float bm_quad_finish(float acc0, float acc1) {
+    // lane ^ 2 holds acc_{l+4} (Q4_K, Q6_K: the other half h; IQ2_XXS: lane q + 2 owns l + 4)
+    const float x = acc0 + bm_quad_xor2(acc0), y = acc1 + bm_quad_xor2(acc1);
+    if (WT == BM_Q6K) {
+        // lane c holds t_c and t_{c+2}
+        const float z = x + y;
+        return z + bm_quad_xor1(z);
+    }
+    // lane c holds t_{2c} and t_{2c+1}
+    const float X = x + bm_quad_xor1(x), Y = y + bm_quad_xor1(y);
+    return X + Y;
+}
+
+// Uniform front over the three types.
+template <int WT>
+__device__ __forceinline__ Blk<WT> bm_load_blk(const uint8_t *wrow, int i, int q);
+template <>
+__device__ __forceinline__ Blk<BM_Q4K> bm_load_blk<BM_Q4K>(const uint8_t *wrow, int i, int q) {
+    return bm_load_q4k(wrow, i, q & 1, q >> 1);
+}
+template <>
+__device__ __forceinline__ Blk<BM_Q6K> bm_load_blk<BM_Q6K>(const uint8_t *wrow, int i, int q) {
+    return bm_load_q6k(wrow, i, q & 1, q >> 1);
+}
+template <>
+__device__ __forceinline__ Blk<BM_IQ2XXS> bm_load_blk<BM_IQ2XXS>(const uint8_t *wrow, int i, int q) {
+    return bm_load_iq2xxs(wrow, i, q);
+}
+
+template <int WT, class Tap>
+__device__ __forceinline__ void bm_dot_blk(const Blk<WT> &b, const uint8_t *col, int i, int q, const Iq2Tables &tb,
+                                           float &acc0, float &acc1, const Tap &tap) {
+    if constexpr (WT == BM_Q4K)
+        bm_dot_q4k(b, col, i, q & 1, q >> 1, acc0, acc1, tap);
+    else if constexpr (WT == BM_Q6K)
+        bm_dot_q6k(b, col, i, q & 1, q >> 1, acc0, acc1, tap);
+    else
+        bm_dot_iq2xxs(b, col, i, q, tb, acc0, acc1, tap);
+}
+
+template <int WT>
+__host__ __device__ constexpr int bm_block_bytes() {
+    return WT == BM_Q4K ? BM_Q4K_BLOCK : (WT == BM_Q6K ? BM_Q6K_BLOCK : BM_IQ2XXS_BLOCK);
+}
+
+// Bytes of one activation super-block (256 values) in the form type WT dots against.
+template <int WT>
+__host__ __device__ constexpr int bm_act_sb_bytes() {
+    return WT == BM_IQ2XXS ? BM_Q8K_STRIDE : 2 * BM_Q82X4_STRIDE;
+}
+
+// ---- SwiGLU: crates/qdot/src/lib.rs:3741-3773 (expf) and :11467-11478 (divide, then multiply).
+__device__ __forceinline__ float bm_expf_ik(float x) {
+    const float SHIFT = bm_bits_f32(0x4b400000u), LOG2E = bm_bits_f32(0x3fb8aa3bu);
+    const float LN2_HI = bm_bits_f32(0x3f317200u), LN2_LO = bm_bits_f32(0x35bfbe8eu);
+    const float C0 = bm_bits_f32(0x3f7ffff6u), C1 = bm_bits_f32(0x3efffedbu), C2 = bm_bits_f32(0x3e2aaf33u);
+    const float C3 = bm_bits_f32(0x3d2b9f17u), C4 = bm_bits_f32(0x3c072010u);
+    const float z = fmaf(x, LOG2E, SHIFT);
+    const float n = __fsub_rn(z, SHIFT);
+    const float b = fmaf(-n, LN2_LO, fmaf(-n, LN2_HI, x));
+    const u32 e = bm_f32_bits(z) << 23;
+    const float k = bm_bits_f32(e + 0x3f800000u);
+    const float u = __fmul_rn(b, b);
+    const float j = fmaf(fmaf(fmaf(C4, b, C3), u, fmaf(C2, b, C1)), u, __fmul_rn(C0, b));
+    if (fabsf(n) > 126.0f) {
+        const u32 g = (n <= 0.0f) ? 0x82000000u : 0u;
+        const float s1 = bm_bits_f32(g + 0x7f000000u);
+        const float s2 = bm_bits_f32(e - g);
+        if (fabsf(n) > 192.0f) return __fmul_rn(s1, s1);
+        return __fmul_rn(fmaf(s2, j, s2), s1);
+    }
+    return fmaf(j, k, k);
+}
+
+__device__ __forceinline__ float bm_swiglu(float g, float u) {
+    const float e = bm_expf_ik(__fsub_rn(0.0f, g));
+    return __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, e)), u);
+}
+
+#endif // BM_DEVICE_CUH

@@ -1,0 +1,174 @@
+/* bm_moe.h - C ABI of libbm_moe_hip.so: quantized MoE expert matmul on MI355X (gfx950).
+ *
+ * Q4_K / Q6_K / IQ2_XXS GGUF weight blocks dotted with Q8-quantized activations (Q8_2_X4 for the K-quants,
+ * Q8_K for IQ2_XXS), in the arithmetic of the reference's CPU path crates/qdot: activation bytes and per-block
+ * integer sums are bit-exact with it, and the decode kernels keep its fp32 operation order.
+ *
+ * The entry points stand where the reference's crates/gpu launchers stand (each declaration cites the one it
+ * replaces). Conventions shared by all of them, as in the reference (crates/gpu/src/q4k_sel.rs:926-936,973):
+ *   - every launcher is asynchronous on the context's stream, allocates nothing, never synchronises, and reads
+ *     expert ids from device memory, so it can be captured into a HIP graph and replayed over new ids;
+ *   - the caller owns every buffer; handles are created at load time and are not thread-safe;
+ *   - geometry the host can check is refused before launch with a negative code and a message naming the entry
+ *     point and the lengths (bm_last_error); conditions only the device can see raise the fault word.
+ * Pointers named *_dev are device pointers; weights are the file's block bytes verbatim, rows back to back
+ * (crates/gpu/src/weights.rs:69-86).
+ */
+#ifndef BM_MOE_H
+#define BM_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Weight types, numbered as ggml numbers them (crates/gguf/src/qtype.rs:94,98,105). */
+#define BM_TYPE_Q4_K 12    /* 144 B / 256 values; activations Q8_2_X4 */
+#define BM_TYPE_Q6_K 14    /* 210 B / 256 values; activations Q8_2_X4 */
+#define BM_TYPE_IQ2_XXS 16 /* 66 B / 256 values; activations Q8_K */
+
+/* Return codes: 0 is success (crates/gpu/src/lib.rs:175-313 GpuError). */
+#define BM_OK 0
+#define BM_ESHAPE (-1)   /* GpuError::Shape: lengths that do not fit the launch */
+#define BM_EDRIVER (-2)  /* GpuError::Driver: a HIP call failed */
+#define BM_ETYPE (-3)    /* a weight type or type combination with no kernel */
+#define BM_EARG (-4)     /* a null handle or pointer */
+#define BM_EFAULT (-5)   /* bm_fault_check: the fault word is raised */
+
+/* Fault word (crates/device/src/fault.rs:9-60): u32[BM_FAULT_WORDS] on the device. Word 0 holds
+ * (layer << 8) | site of the earliest layer and smallest site raised there (atomic minimum; BM_FAULT_NONE while
+ * clean); word 1 + layer is that layer's site mask. Sticky until bm_fault_clear. */
+#define BM_FAULT_NONE 0xFFFFFFFFu
+#define BM_LAYER_NONE 0xFFFFu
+#define BM_FAULT_WORDS (1 + 0xFFFF + 1)
+#define BM_SITE_QUANT_COLUMN 1 /* a quantizer met a value that is not finite: NaN scale, zero codes */
+#define BM_SITE_EXPERT_ID 7    /* an expert id at or past the stack */
+
+/* The id of a slot served elsewhere (crates/gpu/src/host/slots.rs:10): the down projections skip it silently. */
+#define BM_HOST_SLOT 0xFFFFFFFFu
+
+typedef struct bm_ctx bm_ctx;         /* crates/gpu/src/lib.rs:2529 Gpu: device, stream, fault word */
+typedef struct bm_weights bm_weights; /* crates/gpu/src/tensor.rs:588-616 DeviceTensor<u32>: rows of block bytes */
+typedef struct bm_act bm_act;         /* crates/gpu/src/tensor.rs:811-948 Q8Act: m quantized columns of k values */
+
+/* ------------------------------------------------------------------------------------------------ context */
+
+/* A context on `device` with a stream of its own (default priority) and a clean fault word. */
+int bm_ctx_create(int device, bm_ctx **out);
+/* As bm_ctx_create, on a stream the caller owns (a hipStream_t); the context never destroys it. */
+int bm_ctx_create_on_stream(int device, void *hip_stream, bm_ctx **out);
+void bm_ctx_destroy(bm_ctx *ctx);
+/* The context's hipStream_t. */
+void *bm_ctx_stream(bm_ctx *ctx);
+/* hipStreamSynchronize on the context's stream. */
+int bm_ctx_sync(bm_ctx *ctx);
+/* The message of the last refusal on this context (or on the creating thread when ctx is NULL). */
+const char *bm_last_error(const bm_ctx *ctx);
+/* The layer later launches raise faults with (default BM_LAYER_NONE). */
+int bm_set_layer(bm_ctx *ctx, uint32_t layer);
+/* Synchronise and read word 0 and the site mask of `layer` (either pointer may be NULL). */
+int bm_fault_read(bm_ctx *ctx, uint32_t layer, uint32_t *word0, uint32_t *mask);
+/* Reset the fault word to clean (asynchronous, a fill kernel on the stream). */
+int bm_fault_clear(bm_ctx *ctx);
+/* Device pointer of the fault word. */
+uint32_t *bm_fault_word_dev(bm_ctx *ctx);
+
+/* Bytes of one weight row / one activation column of k values (crates/qdot/src/lib.rs:381-422,1727-1762);
+ * negative for a type with no kernel or a k that is not a multiple of 256. */
+int64_t bm_row_bytes(int wtype, int k);
+int64_t bm_col_bytes(int wtype, int k);
+
+/* ------------------------------------------------------------------------------------------------ buffers */
+
+/* Device memory helpers for callers without a HIP binding of their own (the test suite). */
+int bm_dev_alloc(bm_ctx *ctx, size_t bytes, void **out_dev);
+int bm_dev_free(bm_ctx *ctx, void *dev);
+int bm_dev_upload(bm_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);   /* synchronous */
+int bm_dev_download(bm_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes); /* synchronous */
+int bm_dev_memset(bm_ctx *ctx, void *dst_dev, int byte, size_t bytes);               /* synchronous */
+
+/* An expert stack (or one matrix): `rows` rows of `k` values in `wtype` blocks, uploaded from `host_bytes`
+ * (rows * bm_row_bytes bytes). Load time only. */
+int bm_weights_create(bm_ctx *ctx, int wtype, int64_t rows, int k, const void *host_bytes, bm_weights **out);
+/* As bm_weights_create over device memory the caller already holds (no copy; the caller keeps ownership). */
+int bm_weights_wrap(bm_ctx *ctx, int wtype, int64_t rows, int k, const void *dev_bytes, bm_weights **out);
+void bm_weights_destroy(bm_weights *w);
+const void *bm_weights_dev(const bm_weights *w);
+
+/* Activation scratch for up to `m_cap` columns of `k` values in the form `wtype` dots against
+ * (Q8Act::with_k / with_slots). Load time only. The device layout is the reference CPU path's column bytes,
+ * columns back to back, so a column can be handed to or taken from a host tier unchanged. */
+int bm_act_create(bm_ctx *ctx, int wtype, int k, int m_cap, bm_act **out);
+void bm_act_destroy(bm_act *act);
+/* Synchronise and copy column `col`'s bytes (bm_col_bytes of them) to the host. */
+int bm_act_download(bm_ctx *ctx, const bm_act *act, int col, void *host_bytes);
+/* Upload column `col` from host bytes in the same layout. */
+int bm_act_upload(bm_ctx *ctx, bm_act *act, int col, const void *host_bytes);
+
+/* ------------------------------------------------------------------------------- decode: quantize and gemv */
+
+/* Gpu::enqueue_quantize_q8_1 (crates/gpu/src/lib.rs:3275), in the CPU path's rule (crates/qdot/src/lib.rs:434
+ * quantize_col): x_dev holds m columns of act's k values, column c at x_dev + c * k; columns 0..m of act are
+ * written. A block holding a value that is not finite raises BM_SITE_QUANT_COLUMN, gets a NaN scale and zero
+ * codes (crates/gpu/src/lib.rs:925-933). */
+int bm_quantize(bm_ctx *ctx, const float *x_dev, int m, bm_act *act);
+
+/* Gpu::enqueue_gemv_q4k / enqueue_gemv_q6k (crates/gpu/src/lib.rs:3495,3839) and the IQ2_XXS row kernel
+ * (crates/gpu/src/iq.rs:1405): y_dev[row * m + c] = row `row` of w . column c of act, m = `m` columns, 1..=8. */
+int bm_gemv(bm_ctx *ctx, const bm_weights *w, const bm_act *act, int m, float *y_dev);
+
+/* -------------------------------------------------------------------------- decode: the routed expert chain */
+
+/* ExpertKernels::enqueue_gate_up(GateUpArgs) (crates/gpu/src/arch/qwen3moe/experts.rs:326-335,462), for Q4_K,
+ * Q6_K (crates/gpu/src/q6k_sel.rs:633) and IQ2_XXS (crates/gpu/src/iq_sel.rs:1357) stacks of one type:
+ * slot s < n_slots reads expert sel_dev[s]'s rows of both stacks against activation column s / slots_per_col and
+ * writes h_dev[s * rows_per_expert + r] = silu(gate_r) * up_r in the CPU path's SwiGLU
+ * (crates/qdot/src/lib.rs:11467). An id at or past the stack raises BM_SITE_EXPERT_ID and writes NaN into the
+ * slot's rows. h_dev may be NULL when act_h is given.
+ * act_h (optional, NULL to skip): the down projection's activation, quantized in the same launch from the rows
+ * just written, column s of act_h for slot s, in the form of act_h's type (Q8_2_X4 only; rows_per_expert must
+ * then be act_h's k). The reference runs this as a separate quantizer launch (dispatch.rs:1343). */
+int bm_gate_up(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_act *act, const uint32_t *sel_dev,
+               int n_slots, int rows_per_expert, int slots_per_col, float *h_dev, bm_act *act_h);
+
+/* Q4kSelKernels::enqueue_gemv_q4k_sel (crates/gpu/src/q4k_sel.rs:978), Q6kSelKernels::enqueue_gemv_q6k_sel
+ * (crates/gpu/src/q6k_sel.rs:513), QuantSelKernels::enqueue_down (crates/gpu/src/iq_sel.rs:1557): slot s writes
+ * y_dev[s * rows_per_expert + r] = row r of expert sel_dev[s] . column s of act. An id at or past the stack
+ * leaves the slot's rows untouched and, unless it is BM_HOST_SLOT, raises BM_SITE_EXPERT_ID. */
+int bm_gemv_sel(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const uint32_t *sel_dev, int n_slots,
+                int rows_per_expert, float *y_dev);
+
+/* ExpertKernels::enqueue_combine_tokens(CombineArgs) (crates/gpu/src/arch/qwen3moe/experts.rs:341-349,529):
+ * y[t * rows + d] = (acc = 0; for slot e ascending: acc = fma(w[t * n_slots + e], down[(t * n_slots + e) * rows
+ * + d], acc)) + resid[t * rows + d] for t < m. resid_dev may be NULL (no residual add). */
+int bm_combine_tokens(bm_ctx *ctx, const float *down_dev, const float *w_dev, const float *resid_dev, int rows,
+                      int n_slots, int m, float *y_dev);
+
+/* bm_gemv_sel and bm_combine_tokens in one launch (no counterpart launch in the reference, which keeps the two
+ * apart: dispatch.rs:1346-1424): the slot values never reach memory. Same values as the two calls: every slot
+ * dot is bm_gemv_sel's and the sum keeps the slot order. A refused id contributes nothing to the sum. */
+int bm_down_combine(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const uint32_t *sel_dev,
+                    const float *w_dev, const float *resid_dev, int n_slots_per_token, int m, int rows_per_expert,
+                    float *y_dev);
+
+/* ------------------------------------------------------------------------------------------- verification */
+
+/* The exact per-block integers the kernels above form for row `row` of w against column `col` of act, written
+ * to out_dev as i32, through the same device code the launchers run:
+ *   Q4_K:    per super-block 8 sums A[s] = sum q4 * a over sub-block s, then the 8 activation isums (16 words);
+ *   Q6_K:    per super-block 16 sums S[g] = sum (q6 - 32) * a over 16-value group g (16 words);
+ *   IQ2_XXS: per super-block 8 sums I[b] = sum (+-grid) * a over sub-block b, then the 8 scales 2s + 1 (16 words).
+ * out_dev holds 16 * (k / 256) words. These are the integers crates/qdot's lanes hold (its gates pin them by
+ * bit identity, crates/qdot/tests/qdot.rs:738,818,2664). */
+int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *act, int col, int32_t *out_dev);
+
+/* Library version: major * 10000 + minor * 100 + patch. */
+int bm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* BM_MOE_H */

@@ -1,0 +1,447 @@
+"""GPU parity tests of the decode path, through the C ABI, against the CPU oracle on the same seeded inputs.
+
+Bars: activation bytes bit-exact; per-block integer sums bit-exact; fp32 outputs within 1e-4 (max-abs normalised)
+as the task states, and bit-exact where the kernels keep the reference's operation order (they do: every value
+here is compared bit for bit as well, and a difference is reported with both numbers).
+Mirrors the reference's gates: gate_q4k_sel (slot == one-expert gemv, duplicate ids, bad ids, HOST), gate_kquant,
+gate_iq_sel, gate_moe_fused (crates/gpu-gates/src/bin/)."""
+import numpy as np
+import pytest
+
+import bloomery_amd as bm
+import ora
+from common import Lcg, max_abs_normalised, normal_f32
+
+pytestmark = pytest.mark.gpu
+
+TYPES = (bm.Q4_K, bm.Q6_K, bm.IQ2_XXS)
+TIES = np.array([0.5, 1.5, 2.5, 3.5, -0.5, -1.5, -2.5, -3.5, 0.25, 7.5, -7.5, 63.5, -63.5, 120.5, -120.5,
+                 0.0, -0.0, 127.0, -127.0], np.float32)
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    g = bm.Gpu(0)
+    yield g
+    g.close()
+
+
+def assert_f32(got, want, what):
+    got, want = np.asarray(got, np.float32), np.asarray(want, np.float32)
+    err = max_abs_normalised(got, want)
+    assert err <= 1e-4, f"{what}: max-abs normalised error {err}"
+    same = got.view(np.uint32) == want.view(np.uint32)
+    assert same.all(), f"{what}: {np.count_nonzero(~same)} of {same.size} values differ in bits (err {err}); " \
+                       f"first at {int(np.argmin(same))}: {got[np.argmin(same)]!r} vs {want[np.argmin(same)]!r}"
+
+
+def random_blocks(wtype, rows, k, rng):
+    """Raw random block bytes with sane f16 scales: every code pattern is a legal block."""
+    bb = ora.BLOCK_BYTES[wtype]
+    nb = k // 256
+    w = rng.integers(0, 256, rows * nb * bb, dtype=np.uint8).reshape(rows * nb, bb)
+    off = {ora.Q4_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0}[wtype]
+    d = rng.uniform(-0.05, 0.05, rows * nb).astype(np.float16).view(np.uint16)
+    w[:, off] = d & 0xFF
+    w[:, off + 1] = d >> 8
+    if wtype == ora.Q4_K:
+        m = rng.uniform(0.0, 0.05, rows * nb).astype(np.float16).view(np.uint16)
+        w[:, 2] = m & 0xFF
+        w[:, 3] = m >> 8
+    return w.reshape(-1)
+
+
+def quantized(wtype, rows, k, seed):
+    rng = np.random.default_rng(seed)
+    return ora.quantize_rows(wtype, normal_f32(rng, (rows, k), 0.02), rows, k, n_threads=8)
+
+
+def stack(wtype, rows, k, seed):
+    """Weights for a test: the repo's quantizer for the K-quants, and for IQ2_XXS (whose search is slow) a few
+    quantized rows followed by raw random blocks."""
+    if wtype != bm.IQ2_XXS or rows <= 64:
+        return quantized(wtype, rows, k, seed)
+    rng = np.random.default_rng(seed)
+    head = quantized(wtype, 64, k, seed)
+    return np.concatenate([head, random_blocks(wtype, rows - 64, k, rng)])
+
+
+# ------------------------------------------------------------------------------------------------ quantizers
+
+def kat_columns(k):
+    """Edge columns of the reference's encoder tests (crates/qdot/tests/qdot.rs:4619-4944) at width k."""
+    rng = Lcg(0xC0FFEE)
+    cols = []
+    x = np.array([rng.unit() for _ in range(k)], np.float32)
+    cols.append(x)
+    t = np.array([TIES[i % len(TIES)] for i in range(k)], np.float32)
+    t[0::32] = 127.0
+    t[32] = 254.0
+    cols.append(t)
+    sat = np.array([254.0 if j % 2 == 0 else -254.0 for j in range(k)], np.float32)
+    sat[96:128] *= np.float32((127.0 - 127.0 / 512.0) / 254.0)
+    cols.append(sat)
+    cols.append(np.full(k, 1e-40, np.float32))
+    cols.append(np.full(k, 1e-38, np.float32))
+    z = np.array([rng.unit() * np.float32(3.0) for _ in range(k)], np.float32)
+    z[0:64] = 0.0
+    z[k // 2:k // 2 + 256] = 0.0
+    cols.append(z)
+    ties = np.array([rng.unit() * np.float32(0.4) for _ in range(k)], np.float32)
+    ties[9], ties[200], ties[137] = 3.0, -3.0, 3.0
+    ties[256 + 250], ties[256 + 3] = 3.0, -3.0
+    cols.append(ties)
+    sub = np.where(np.arange(k) % 2 == 0, 1.0, -1.0).astype(np.float32) * np.float32(127.0 * (64.49 / 64.0) * 2.0 ** -127)
+    cols.append(sub)
+    for mag in (1e-6, 1e-3, 1.0, 1e4):
+        cols.append(np.array([rng.unit() * np.float32(mag) for _ in range(k)], np.float32))
+    return np.stack(cols)
+
+
+@pytest.mark.parametrize("wtype", (bm.Q4_K, bm.IQ2_XXS))
+@pytest.mark.parametrize("k", (512, 2048))
+def test_quantize_bytes_are_the_cpu_paths(gpu, wtype, k):
+    x = kat_columns(k)
+    m = x.shape[0]
+    act = gpu.act(wtype, k, m)
+    xd = gpu.upload(x, np.float32)
+    gpu.enqueue_quantize(xd, m, act)
+    for c in range(m):
+        want = ora.quantize_col(wtype, x[c])
+        got = act.download(c)
+        assert np.array_equal(got, want), f"type {wtype} k {k} column {c}: {np.count_nonzero(got != want)} bytes differ"
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    act.free()
+    xd.free()
+
+
+def test_quantize_random_columns(gpu):
+    rng = np.random.default_rng(7)
+    for wtype, k in ((bm.Q4_K, 2048), (bm.Q6_K, 768), (bm.IQ2_XXS, 7168)):
+        m = 40
+        x = (normal_f32(rng, (m, k)) * (10.0 ** rng.uniform(-5, 4, (m, 1)))).astype(np.float32)
+        act = gpu.act(wtype, k, m)
+        xd = gpu.upload(x, np.float32)
+        gpu.enqueue_quantize(xd, m, act)
+        for c in range(m):
+            assert np.array_equal(act.download(c), ora.quantize_col(wtype, x[c])), (wtype, c)
+        act.free()
+        xd.free()
+
+
+def test_non_finite_activation_raises_quant_column(gpu):
+    # crates/gpu/src/lib.rs:925-933: NaN scale, zero codes, fault site 1; the CPU path refuses the column instead
+    for wtype, bb in ((bm.Q4_K, 144), (bm.IQ2_XXS, 296)):
+        gpu.fault_clear()
+        x = np.ones((1, 512), np.float32)
+        x[0, 300] = np.inf
+        act = gpu.act(wtype, 512, 1)
+        xd = gpu.upload(x, np.float32)
+        gpu.set_layer(3)
+        gpu.enqueue_quantize(xd, 1, act)
+        w0, mask = gpu.fault(3)
+        assert w0 == (3 << 8) | bm.SITE_QUANT_COLUMN and mask == 1 << bm.SITE_QUANT_COLUMN
+        col = act.download(0)
+        good = ora.quantize_col(wtype, np.ones(256, np.float32))
+        assert np.array_equal(col[:len(good)], good), "the clean block is untouched by its neighbour"
+        if wtype == bm.Q4_K:
+            grp = col[288:432]  # values 256..383; the bad block is the second of this group
+            assert grp[2:4].view(np.uint16)[0] == 0x7FC0 and not grp[16 + 32:16 + 64].any() and grp[10:12].view(np.int16)[0] == 0
+        else:
+            blk = col[296:592]
+            assert np.isnan(blk[0:4].view(np.float32)[0]) and not blk[4:].any()
+        gpu.set_layer(bm.LAYER_NONE)
+        gpu.fault_clear()
+        assert gpu.fault(3) == (bm.FAULT_NONE, 0)
+        act.free()
+        xd.free()
+
+
+# ------------------------------------------------------------------------------------------------ integer sums
+
+@pytest.mark.parametrize("wtype", TYPES)
+def test_block_sums_are_the_cpu_paths_integers(gpu, wtype):
+    rng = np.random.default_rng(20 + wtype)
+    for k in (256, 768, 2048):
+        rows = 6
+        w = np.concatenate([random_blocks(wtype, 3, k, rng), quantized(wtype, 3, k, 21)])
+        x = normal_f32(rng, (2, k), 10.0 ** rng.uniform(-2, 2))
+        wd, act = gpu.weights(wtype, rows, k, w), gpu.act(wtype, k, 2)
+        xd = gpu.upload(x, np.float32)
+        gpu.enqueue_quantize(xd, 2, act)
+        out = gpu.buffer(np.int32, 16 * (k // 256))
+        rb = ora.row_bytes(wtype, k)
+        for row in range(rows):
+            for col in range(2):
+                gpu.enqueue_block_sums(wd, row, act, col, out)
+                got = out.download().reshape(-1, 16)
+                wrow, acol = w[row * rb:(row + 1) * rb], ora.quantize_col(wtype, x[col])
+                if wtype == bm.Q4_K:
+                    a, isum = ora.q4k_block_sums(wrow, acol, k)
+                    assert np.array_equal(got[:, :8].reshape(-1), a) and np.array_equal(got[:, 8:].reshape(-1), isum)
+                elif wtype == bm.Q6_K:
+                    assert np.array_equal(got.reshape(-1), ora.q6k_block_sums(wrow, acol, k))
+                    assert np.array_equal(got.reshape(-1), ora.q6k_block_sums(wrow, acol, k, fold=True))
+                else:
+                    i_b, sc, _, _ = ora.iq2xxs_block_sums(wrow, acol, k)
+                    assert np.array_equal(got[:, :8].reshape(-1), i_b) and np.array_equal(got[:, 8:].reshape(-1), sc)
+        for b in (wd, act, xd, out):
+            b.free()
+
+
+# -------------------------------------------------------------------------------------------------------- gemv
+
+@pytest.mark.parametrize("wtype,rows,k", ((bm.Q4_K, 768, 2048), (bm.Q6_K, 2048, 768), (bm.IQ2_XXS, 300, 2048),
+                                          (bm.Q4_K, 70, 256), (bm.Q6_K, 65, 1792), (bm.IQ2_XXS, 33, 7168)))
+def test_gemv_matches_dot_row(gpu, wtype, rows, k):
+    # config 1 is the first case: 768 x 2048 Q4_K against one 2048-vector
+    rng = np.random.default_rng(30 + rows)
+    w = stack(wtype, rows, k, 31 + rows)
+    x = normal_f32(rng, (8, k))
+    wd, act = gpu.weights(wtype, rows, k, w), gpu.act(wtype, k, 8)
+    xd = gpu.upload(x, np.float32)
+    gpu.enqueue_quantize(xd, 8, act)
+    cols = np.concatenate([ora.quantize_col(wtype, x[c]) for c in range(8)])
+    for m in (1, 3, 8):
+        y = gpu.buffer(np.float32, rows * m).fill_bytes(0xFF)
+        gpu.enqueue_gemv(wd, act, m, y)
+        assert_f32(y.download(), ora.gemv(wtype, w, rows, k, cols, m), f"gemv type {wtype} {rows}x{k} m={m}")
+        y.free()
+    for b in (wd, act, xd):
+        b.free()
+
+
+def test_extreme_blocks(gpu):
+    """Every code at its ends, zero, subnormal and negative block scales (crates/qdot/tests/qdot.rs:2615-2655)."""
+    rng = np.random.default_rng(44)
+    for wtype in TYPES:
+        bb = ora.BLOCK_BYTES[wtype]
+        rows_bytes = []
+        for fill, dval in ((0xFF, 0.05), (0x00, 0.05), (0xFF, 0.0), (0xAA, 6e-8), (0x55, -0.03), (0x0F, 65504.0)):
+            w = np.full(2 * bb, fill, np.uint8)
+            for i in range(2):
+                h = np.array([dval, abs(dval)], np.float16).view(np.uint8)
+                off = {ora.Q4_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0}[wtype]
+                w[i * bb + off:i * bb + off + 2] = h[0:2]
+                if wtype == ora.Q4_K:
+                    w[i * bb + 2:i * bb + 4] = h[2:4]
+            rows_bytes.append(w)
+        w = np.concatenate(rows_bytes)
+        rows, k = len(rows_bytes), 512
+        x = np.stack([np.full(k, 3.0, np.float32), normal_f32(rng, k), -np.abs(normal_f32(rng, k)),
+                      normal_f32(rng, k, 1e-3)])
+        wd, act = gpu.weights(wtype, rows, k, w), gpu.act(wtype, k, 4)
+        xd = gpu.upload(x, np.float32)
+        gpu.enqueue_quantize(xd, 4, act)
+        y = gpu.buffer(np.float32, rows * 4)
+        gpu.enqueue_gemv(wd, act, 4, y)
+        cols = np.concatenate([ora.quantize_col(wtype, x[c]) for c in range(4)])
+        want = ora.gemv(wtype, w, rows, k, cols, 4)
+        got = y.download()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (wtype, got, want)
+        for b in (wd, act, xd, y):
+            b.free()
+
+
+# ------------------------------------------------------------------------------------------- the expert chain
+
+def route(rng, m, n_experts, top_k, bias=None):
+    ids = np.empty((m, top_k), np.uint32)
+    wts = np.empty((m, top_k), np.float32)
+    for t in range(m):
+        logits = normal_f32(rng, n_experts)
+        if bias is not None:
+            logits = (logits + bias).astype(np.float32)
+        ids[t], wts[t] = ora.route_softmax_topk(logits, top_k)
+    return ids, wts
+
+
+class Layer:
+    def __init__(self, gpu, types, hidden, ff, n_experts, seed):
+        self.types, self.hidden, self.ff, self.n_experts = types, hidden, ff, n_experts
+        self.wg = stack(types[0], n_experts * ff, hidden, seed)
+        self.wu = stack(types[1], n_experts * ff, hidden, seed + 1)
+        self.wd = stack(types[2], n_experts * hidden, ff, seed + 2)
+        self.dg = gpu.weights(types[0], n_experts * ff, hidden, self.wg)
+        self.du = gpu.weights(types[1], n_experts * ff, hidden, self.wu)
+        self.dd = gpu.weights(types[2], n_experts * hidden, ff, self.wd)
+
+    def oracle(self, x, ids, wts, top_k):
+        return ora.moe_forward(self.hidden, self.ff, self.n_experts, self.types, self.wg, self.wu, self.wd, x, ids,
+                               wts, top_k, n_threads=8, want_h=True)
+
+    def free(self):
+        for b in (self.dg, self.du, self.dd):
+            b.free()
+
+
+def run_chain(gpu, L, x, ids, wts, top_k, fused):
+    """quantize -> gate.up (-> quantize) -> down -> combine, as the reference's decode dispatch orders them
+    (crates/gpu/src/arch/qwen3moe/dispatch.rs:1245-1436); `fused` takes the two fused launches instead."""
+    m = x.shape[0]
+    n_slots = m * top_k
+    act = gpu.act(L.types[0], L.hidden, m)
+    act_h = gpu.act(L.types[2], L.ff, n_slots)
+    xd, sel, wd = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32)
+    h = gpu.buffer(np.float32, n_slots * L.ff).fill_bytes(0xFF)
+    y = gpu.buffer(np.float32, m * L.hidden).fill_bytes(0xFF)
+    gpu.enqueue_quantize(xd, m, act)
+    if fused and L.types[2] != bm.IQ2_XXS:
+        gpu.enqueue_gate_up(L.dg, L.du, act, sel, n_slots, L.ff, top_k, h, act_h)
+    else:
+        gpu.enqueue_gate_up(L.dg, L.du, act, sel, n_slots, L.ff, top_k, h)
+        gpu.enqueue_quantize(h, n_slots, act_h)
+    if fused:
+        gpu.enqueue_down_combine(L.dd, act_h, sel, wd, None, top_k, m, L.hidden, y)
+    else:
+        down = gpu.buffer(np.float32, n_slots * L.hidden).fill_bytes(0xFF)
+        gpu.enqueue_gemv_sel(L.dd, act_h, sel, n_slots, L.hidden, down)
+        gpu.enqueue_combine_tokens(down, wd, None, L.hidden, top_k, m, y)
+    out = y.download(), h.download(), [act_h.download(s) for s in range(n_slots)]
+    for b in (act, act_h, xd, sel, wd, h, y):
+        b.free()
+    return out
+
+
+@pytest.mark.parametrize("fused", (False, True))
+def test_qwen3_shaped_layer_one_token(gpu, fused):
+    """Config 2 at its full shape with 16 of the 128 experts resident: hidden 2048, ff 768, Q4_K gate/up, Q6_K
+    down, softmax top-8 renormalised, one token."""
+    L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 16, 100)
+    rng = np.random.default_rng(101)
+    x = normal_f32(rng, (1, 2048))
+    ids, wts = route(rng, 1, 16, 8)
+    y, h, act_h = run_chain(gpu, L, x, ids, wts, 8, fused)
+    want_y, want_h = L.oracle(x, ids, wts, 8)
+    assert_f32(h, want_h, "h")
+    for s in range(8):
+        assert np.array_equal(act_h[s], ora.quantize_col(bm.Q6_K, want_h[s * 768:(s + 1) * 768])), f"act_h slot {s}"
+    assert_f32(y, want_y, "y")
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    L.free()
+
+
+@pytest.mark.parametrize("types,hidden,ff,n_experts,m,top_k", (
+    ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 12, 5, 4),
+    ((bm.Q6_K, bm.Q6_K, bm.Q4_K), 512, 512, 5, 3, 2),
+    ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ2_XXS), 1024, 512, 6, 4, 3),
+    ((bm.IQ2_XXS, bm.IQ2_XXS, bm.Q6_K), 768, 256, 4, 2, 4),
+))
+@pytest.mark.parametrize("fused", (False, True))
+def test_layers_of_every_type_and_several_tokens(gpu, types, hidden, ff, n_experts, m, top_k, fused):
+    L = Layer(gpu, types, hidden, ff, n_experts, 200 + hidden)
+    rng = np.random.default_rng(201)
+    x = normal_f32(rng, (m, hidden))
+    ids, wts = route(rng, m, n_experts, top_k)
+    y, h, act_h = run_chain(gpu, L, x, ids, wts, top_k, fused)
+    want_y, want_h = L.oracle(x, ids, wts, top_k)
+    assert_f32(h, want_h, "h")
+    for s in range(m * top_k):
+        assert np.array_equal(act_h[s], ora.quantize_col(types[2], want_h[s * ff:(s + 1) * ff])), f"act_h slot {s}"
+    assert_f32(y, want_y, "y")
+    L.free()
+
+
+def test_slot_equals_one_expert_gemv_and_duplicate_ids(gpu):
+    # gate_q4k_sel's first clauses (crates/gpu-gates/src/bin/gate_q4k_sel.rs:1-48)
+    rng = np.random.default_rng(300)
+    for wtype, k, rpe in ((bm.Q4_K, 768, 96), (bm.Q6_K, 768, 2048 // 8), (bm.IQ2_XXS, 512, 80)):
+        n_experts, n_slots = 5, 7
+        w = stack(wtype, n_experts * rpe, k, 301)
+        sel = np.array([3, 0, 3, 4, 1, 3, 0], np.uint32)
+        x = normal_f32(rng, (n_slots, k))
+        wd, act = gpu.weights(wtype, n_experts * rpe, k, w), gpu.act(wtype, k, n_slots)
+        xd, seld = gpu.upload(x, np.float32), gpu.upload(sel, np.uint32)
+        gpu.enqueue_quantize(xd, n_slots, act)
+        y = gpu.buffer(np.float32, n_slots * rpe).fill_bytes(0xFF)
+        gpu.enqueue_gemv_sel(wd, act, seld, n_slots, rpe, y)
+        got = y.download().reshape(n_slots, rpe)
+        rb = ora.row_bytes(wtype, k)
+        for s in range(n_slots):
+            e = int(sel[s])
+            want = ora.gemv(wtype, w[e * rpe * rb:(e + 1) * rpe * rb], rpe, k, ora.quantize_col(wtype, x[s]), 1)
+            assert_f32(got[s], want, f"type {wtype} slot {s}")
+        for b in (wd, act, xd, seld, y):
+            b.free()
+
+
+def test_bad_ids_raise_expert_id_and_host_is_silent(gpu):
+    # crates/gpu/src/kquant/sel.rs:22-28, crates/gpu/src/q4k_sel.rs:968-972
+    rng = np.random.default_rng(400)
+    k, rpe, n_experts = 512, 64, 3
+    w = quantized(bm.Q4_K, n_experts * rpe, k, 401)
+    wd, act = gpu.weights(bm.Q4_K, n_experts * rpe, k, w), gpu.act(bm.Q4_K, k, 3)
+    x = normal_f32(rng, (3, k))
+    xd = gpu.upload(x, np.float32)
+    gpu.enqueue_quantize(xd, 3, act)
+    y = gpu.buffer(np.float32, 3 * rpe)
+    # HOST: skipped silently, rows untouched
+    gpu.fault_clear()
+    y.upload(np.full(3 * rpe, 7.0, np.float32))
+    seld = gpu.upload(np.array([1, bm.HOST_SLOT, 2], np.uint32))
+    gpu.enqueue_gemv_sel(wd, act, seld, 3, rpe, y)
+    got = y.download().reshape(3, rpe)
+    assert (got[1] == 7.0).all() and not (got[0] == 7.0).any() and gpu.fault() == (bm.FAULT_NONE, 0)
+    # an id past the stack: rows untouched and ExpertId raised under the launch's layer
+    gpu.set_layer(9)
+    y.upload(np.full(3 * rpe, 7.0, np.float32))
+    seld.upload(np.array([1, 3, 2], np.uint32))
+    gpu.enqueue_gemv_sel(wd, act, seld, 3, rpe, y)
+    got = y.download().reshape(3, rpe)
+    assert (got[1] == 7.0).all() and gpu.fault(9) == ((9 << 8) | bm.SITE_EXPERT_ID, 1 << bm.SITE_EXPERT_ID)
+    # gate.up writes NaN into the refused slot's rows
+    gpu.fault_clear()
+    h = gpu.buffer(np.float32, 3 * rpe).fill_bytes(0)
+    gpu.enqueue_gate_up(wd, wd, act, seld, 3, rpe, 1, h)
+    hh = h.download().reshape(3, rpe)
+    assert np.isnan(hh[1]).all() and np.isfinite(hh[0]).all() and np.isfinite(hh[2]).all()
+    assert gpu.fault(9)[0] == (9 << 8) | bm.SITE_EXPERT_ID
+    gpu.set_layer(bm.LAYER_NONE)
+    gpu.fault_clear()
+    for b in (wd, act, xd, y, seld, h):
+        b.free()
+
+
+def test_combine_adds_the_residual(gpu):
+    rng = np.random.default_rng(500)
+    rows, n_slots, m = 200, 8, 3
+    down, w, resid = normal_f32(rng, m * n_slots * rows), normal_f32(rng, m * n_slots), normal_f32(rng, m * rows)
+    dd, dw, dr = gpu.upload(down), gpu.upload(w), gpu.upload(resid)
+    y = gpu.buffer(np.float32, m * rows)
+    gpu.enqueue_combine_tokens(dd, dw, dr, rows, n_slots, m, y)
+    assert_f32(y.download(), ora.combine_tokens(down, w, resid, rows, n_slots, m), "combine + resid")
+    gpu.enqueue_combine_tokens(dd, dw, None, rows, n_slots, m, y)
+    assert_f32(y.download(), ora.combine_tokens(down, w, None, rows, n_slots, m), "combine")
+    for b in (dd, dw, dr, y):
+        b.free()
+
+
+def test_shape_refusals_are_named(gpu):
+    # crates/gpu/src/q4k_sel.rs:990-1042: refused on the host, before any launch, with the entry point's name
+    w4 = gpu.weights(bm.Q4_K, 64, 512, np.zeros(64 * bm.row_bytes(bm.Q4_K, 512), np.uint8))
+    a512, a256, aq8k = gpu.act(bm.Q4_K, 512, 2), gpu.act(bm.Q4_K, 256, 2), gpu.act(bm.IQ2_XXS, 512, 2)
+    buf = gpu.buffer(np.float32, 4096)
+    sel = gpu.upload(np.zeros(8, np.uint32))
+    cases = (
+        (lambda: gpu.enqueue_gemv(w4, a256, 1, buf), bm.ESHAPE, "bm_gemv"),
+        (lambda: gpu.enqueue_gemv(w4, aq8k, 1, buf), bm.ETYPE, "bm_gemv"),
+        (lambda: gpu.enqueue_gemv(w4, a512, 3, buf), bm.ESHAPE, "bm_gemv"),
+        (lambda: gpu.enqueue_gemv(w4, a512, 9, buf), bm.ESHAPE, "bm_gemv"),
+        (lambda: gpu.enqueue_gemv_sel(w4, a512, sel, 2, 48, buf), bm.ESHAPE, "rows_per_expert"),
+        (lambda: gpu.enqueue_gemv_sel(w4, a512, sel, 3, 32, buf), bm.ESHAPE, "n_slots"),
+        (lambda: gpu.enqueue_gemv_sel(w4, a512, sel, 0, 32, buf), bm.ESHAPE, "n_slots"),
+        (lambda: gpu.enqueue_gate_up(w4, w4, a512, sel, 5, 32, 2, buf), bm.ESHAPE, "bm_gate_up"),
+        (lambda: gpu.enqueue_gate_up(w4, w4, a512, sel, 2, 32, 0, buf), bm.ESHAPE, "slots_per_col"),
+        (lambda: gpu.enqueue_gate_up(w4, w4, a512, sel, 2, 32, 1, buf, a512), bm.ESHAPE, "act_h"),
+        (lambda: gpu.enqueue_quantize(buf, 3, a512), bm.ESHAPE, "bm_quantize"),
+        (lambda: gpu.enqueue_down_combine(w4, a512, sel, buf, None, 65, 1, 32, buf), bm.ESHAPE, "slots a token"),
+        (lambda: gpu.weights(7, 4, 256, np.zeros(1024, np.uint8)), bm.ETYPE, "weight type"),
+        (lambda: gpu.weights(bm.Q4_K, 4, 300, np.zeros(4096, np.uint8)), bm.ESHAPE, "256"),
+        (lambda: gpu.act(bm.Q6_K, 100, 1), bm.ESHAPE, "256"),
+    )
+    for call, code, word in cases:
+        with pytest.raises(bm.GpuError) as e:
+            call()
+        assert e.value.code == code and word in str(e.value), str(e.value)
+    for b in (w4, a512, a256, aq8k, buf, sel):
+        b.free()

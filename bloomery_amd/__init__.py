@@ -60,6 +60,14 @@ SYMBOLS = {
     "bm_combine_tokens": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_down_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_block_sums": (_i, [_vp, _vp, _i64, _vp, _i, _vp]),
+    "bm_capture_begin": (_i, [_vp]),
+    "bm_capture_end": (_i, [_vp, C.POINTER(_vp)]),
+    "bm_graph_launch": (_i, [_vp, _vp]),
+    "bm_graph_destroy": (None, [_vp]),
+    "bm_event_create": (_i, [_vp, C.POINTER(_vp)]),
+    "bm_event_record": (_i, [_vp, _vp]),
+    "bm_event_elapsed_ms": (_i, [_vp, _vp, _vp, C.POINTER(C.c_float)]),
+    "bm_event_destroy": (None, [_vp]),
 }
 
 
@@ -248,6 +256,37 @@ class Gpu:
 
     def act(self, wtype, k, m_cap):
         return Q8Act(self, wtype, k, m_cap)
+
+    # -- graphs and events
+    def capture_begin(self):
+        self._check(self.lib.bm_capture_begin(self.ctx))
+
+    def capture_end(self):
+        g = _vp()
+        self._check(self.lib.bm_capture_end(self.ctx, C.byref(g)))
+        return g.value
+
+    def graph_launch(self, graph):
+        self._check(self.lib.bm_graph_launch(self.ctx, graph))
+
+    def graph_destroy(self, graph):
+        self.lib.bm_graph_destroy(graph)
+
+    def event(self):
+        e = _vp()
+        self._check(self.lib.bm_event_create(self.ctx, C.byref(e)))
+        return e.value
+
+    def event_record(self, event):
+        self._check(self.lib.bm_event_record(self.ctx, event))
+
+    def event_elapsed_ms(self, start, stop):
+        ms = C.c_float()
+        self._check(self.lib.bm_event_elapsed_ms(self.ctx, start, stop, C.byref(ms)))
+        return ms.value
+
+    def event_destroy(self, event):
+        self.lib.bm_event_destroy(event)
 
     # -- launchers (asynchronous on the context's stream)
     def enqueue_quantize(self, x, m, act):

@@ -435,4 +435,86 @@ int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *a
     return driver(ctx, what, bmk::block_sums(launch_of(ctx), w->wtype, wrow, w->k, c, out_dev));
 }
 
+// ------------------------------------------------------------------------------------ graphs and events
+
+struct bm_graph {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+};
+
+struct bm_event {
+    hipEvent_t ev;
+};
+
+int bm_capture_begin(bm_ctx *ctx) {
+    if (!ctx) return fail(nullptr, BM_EARG, "bm_capture_begin: ctx is NULL");
+    return driver(ctx, "bm_capture_begin", hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+}
+
+int bm_capture_end(bm_ctx *ctx, bm_graph **out) {
+    if (!ctx || !out) return fail(ctx, BM_EARG, "bm_capture_end: NULL argument");
+    *out = nullptr;
+    hipGraph_t g = nullptr;
+    int rc = driver(ctx, "bm_capture_end", hipStreamEndCapture(ctx->stream, &g));
+    if (rc) return rc;
+    hipGraphExec_t x = nullptr;
+    rc = driver(ctx, "bm_capture_end: instantiate", hipGraphInstantiate(&x, g, nullptr, nullptr, 0));
+    if (rc) {
+        (void)hipGraphDestroy(g);
+        return rc;
+    }
+    bm_graph *bg = new (std::nothrow) bm_graph{g, x};
+    if (!bg) {
+        (void)hipGraphExecDestroy(x);
+        (void)hipGraphDestroy(g);
+        return fail(ctx, BM_EDRIVER, "bm_capture_end: out of host memory");
+    }
+    *out = bg;
+    return BM_OK;
+}
+
+int bm_graph_launch(bm_ctx *ctx, bm_graph *graph) {
+    if (!ctx || !graph) return fail(ctx, BM_EARG, "bm_graph_launch: NULL argument");
+    return driver(ctx, "bm_graph_launch", hipGraphLaunch(graph->exec, ctx->stream));
+}
+
+void bm_graph_destroy(bm_graph *graph) {
+    if (!graph) return;
+    (void)hipGraphExecDestroy(graph->exec);
+    (void)hipGraphDestroy(graph->graph);
+    delete graph;
+}
+
+int bm_event_create(bm_ctx *ctx, bm_event **out) {
+    if (!ctx || !out) return fail(ctx, BM_EARG, "bm_event_create: NULL argument");
+    *out = nullptr;
+    hipEvent_t e;
+    int rc = driver(ctx, "bm_event_create", hipEventCreate(&e));
+    if (rc) return rc;
+    *out = new (std::nothrow) bm_event{e};
+    if (!*out) {
+        (void)hipEventDestroy(e);
+        return fail(ctx, BM_EDRIVER, "bm_event_create: out of host memory");
+    }
+    return BM_OK;
+}
+
+int bm_event_record(bm_ctx *ctx, bm_event *event) {
+    if (!ctx || !event) return fail(ctx, BM_EARG, "bm_event_record: NULL argument");
+    return driver(ctx, "bm_event_record", hipEventRecord(event->ev, ctx->stream));
+}
+
+int bm_event_elapsed_ms(bm_ctx *ctx, bm_event *start, bm_event *stop, float *ms) {
+    if (!ctx || !start || !stop || !ms) return fail(ctx, BM_EARG, "bm_event_elapsed_ms: NULL argument");
+    int rc = driver(ctx, "bm_event_elapsed_ms: sync", hipEventSynchronize(stop->ev));
+    if (rc) return rc;
+    return driver(ctx, "bm_event_elapsed_ms", hipEventElapsedTime(ms, start->ev, stop->ev));
+}
+
+void bm_event_destroy(bm_event *event) {
+    if (!event) return;
+    (void)hipEventDestroy(event->ev);
+    delete event;
+}
+
 } // extern "C"

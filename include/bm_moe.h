@@ -164,6 +164,26 @@ int bm_down_combine(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const u
  * bit identity, crates/qdot/tests/qdot.rs:738,818,2664). */
 int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *act, int col, int32_t *out_dev);
 
+/* ------------------------------------------------------------------------------------ graphs and events */
+
+typedef struct bm_graph bm_graph; /* an instantiated HIP graph of launches captured on the context's stream */
+typedef struct bm_event bm_event; /* a HIP event on the context's stream */
+
+/* The reference replays each decode step as one captured graph (crates/gpu/src/arch/qwen3moe/dispatch.rs, the
+ * launchers' "capturable" contract, crates/gpu/src/q4k_sel.rs:973). bm_capture_begin starts capturing the
+ * context's stream (thread-local mode); the launchers called until bm_capture_end become the graph's nodes.
+ * Ids, activations and outputs are read and written through their device pointers at replay time. */
+int bm_capture_begin(bm_ctx *ctx);
+int bm_capture_end(bm_ctx *ctx, bm_graph **out);
+int bm_graph_launch(bm_ctx *ctx, bm_graph *graph);
+void bm_graph_destroy(bm_graph *graph);
+
+int bm_event_create(bm_ctx *ctx, bm_event **out);
+int bm_event_record(bm_ctx *ctx, bm_event *event);
+/* Waits for `stop`, then the milliseconds from `start` to `stop`. */
+int bm_event_elapsed_ms(bm_ctx *ctx, bm_event *start, bm_event *stop, float *ms);
+void bm_event_destroy(bm_event *event);
+
 /* Library version: major * 10000 + minor * 100 + patch. */
 int bm_version(void);
 

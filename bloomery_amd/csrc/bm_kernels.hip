@@ -1,9 +1,14 @@
 // HIP kernels of the quantized MoE expert matmul for gfx950, and their launch functions.
 //
-// Every dot kernel follows one plan: a quad of lanes per weight row (bm_device.cuh), the row's first batch of
-// super-blocks requested from HBM before anything else (128-bit loads, one batch = U super-blocks a lane), the
-// token's quantized activation column copied to LDS while those loads fly, then the arithmetic. Weights are read
-// once, straight from the file's block bytes; the kernels are bound by HBM bandwidth.
+// Every dot kernel follows one plan: a quad of lanes per weight row (bm_device.cuh); the token's quantized
+// activation column requested first, then the row's first batch of super-blocks (128-bit loads), all from
+// straight-line code so the hardware's in-order load counter lets the column be copied to LDS and the arithmetic
+// start on the first super-block while the later ones are still in flight. Weights are read once, straight from
+// the file's block bytes; the kernels are bound by HBM bandwidth.
+//
+// Variants: a kernel is instantiated per weight type and per (U, NB): U super-blocks a lane requests per batch,
+// NB the row's super-block count when it is known at compile time (0: a run-time count that U divides). The hot
+// shapes (Q4_K rows of 2048 values, Q6_K rows of 768) take NB = U = the whole row, one batch and no loop.
 #include "bm_kernels.h"
 
 #define BM_TABLE_QUAL __device__ const
@@ -52,35 +57,72 @@ __device__ __forceinline__ void stage_bytes(uint8_t *dst, const uint8_t *src, in
         *reinterpret_cast<uint2 *>(dst + o) = *reinterpret_cast<const uint2 *>(src + o);
 }
 
-template <int WT, int U>
-__device__ __forceinline__ void preload(Blk<WT> (&b)[U], const uint8_t *wrow, int nb, int q) {
+// The same copy in two halves: R unconditional loads a thread (offsets past the end are clamped onto the last
+// word, so no branch stands between them and the weight loads that follow), then the LDS stores. Memory returns
+// in order, so the stores wait for these loads only. Bytes past R * 8 * blockDim are copied afterwards by
+// stage_bytes' loop (that part waits for everything in flight).
+template <int R>
+struct Stage {
+    uint2 v[R];
+    __device__ __forceinline__ void load(const uint8_t *src, int bytes) {
 #pragma unroll
-    for (int u = 0; u < U; u++)
-        if (u < nb) b[u] = bm_load_blk<WT>(wrow, u, q);
+        for (int r = 0; r < R; r++) {
+            int o = (r * (int)blockDim.x + (int)threadIdx.x) * 8;
+            o = o < bytes ? o : bytes - 8;
+            v[r] = *reinterpret_cast<const uint2 *>(src + o);
+        }
+        // keep these loads ahead of whatever is requested next: the in-order wait depends on it
+        __asm__ volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    __device__ __forceinline__ void store(uint8_t *dst, const uint8_t *src, int bytes) const {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int o = (r * (int)blockDim.x + (int)threadIdx.x) * 8;
+            if (o < bytes) *reinterpret_cast<uint2 *>(dst + o) = v[r];
+        }
+        for (int o = (R * (int)blockDim.x + (int)threadIdx.x) * 8; o < bytes; o += (int)blockDim.x * 8)
+            *reinterpret_cast<uint2 *>(dst + o) = *reinterpret_cast<const uint2 *>(src + o);
+    }
+};
+
+// Super-blocks 0..U of the row, requested unconditionally (the launch functions pick U to divide the row).
+template <int WT, int U>
+__device__ __forceinline__ void preload(Blk<WT> (&b)[U], const uint8_t *wrow, int q) {
+#pragma unroll
+    for (int u = 0; u < U; u++) b[u] = bm_load_blk<WT>(wrow, u, q);
 }
 
 // Row `wrow` against `m` <= M columns (LDS, `col_stride` apart); b holds the first batch already.
-template <int WT, int U, int M, class Tap>
+// NB > 0: the row has NB super-blocks (a multiple of U); NB == 0: it has nb, a multiple of U.
+template <int WT, int U, int NB, int M, class Tap>
 __device__ __forceinline__ void row_dot(Blk<WT> (&b)[U], const uint8_t *wrow, const uint8_t *cols, int col_stride,
                                         int m, int nb, int q, const Iq2Tables &tb, float (&out)[M], const Tap &tap) {
     float a0[M], a1[M];
 #pragma unroll
     for (int c = 0; c < M; c++) a0[c] = a1[c] = 0.0f;
-    int i0 = 0;
-    for (;;) {
+    if constexpr (NB == U) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            if (i0 + u < nb) {
+#pragma unroll
+            for (int c = 0; c < M; c++)
+                if (M == 1 || c < m) bm_dot_blk<WT>(b[u], cols + (size_t)c * col_stride, u, q, tb, a0[c], a1[c], tap);
+        }
+    } else {
+        const int n = NB > 0 ? NB : nb;
+        for (int i0 = 0;;) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
 #pragma unroll
                 for (int c = 0; c < M; c++)
-                    if (c < m) bm_dot_blk<WT>(b[u], cols + (size_t)c * col_stride, i0 + u, q, tb, a0[c], a1[c], tap);
+                    if (M == 1 || c < m)
+                        bm_dot_blk<WT>(b[u], cols + (size_t)c * col_stride, i0 + u, q, tb, a0[c], a1[c], tap);
             }
-        }
-        i0 += U;
-        if (i0 >= nb) break;
+            i0 += U;
+            if (i0 >= n) break;
 #pragma unroll
-        for (int u = 0; u < U; u++)
-            if (i0 + u < nb) b[u] = bm_load_blk<WT>(wrow, i0 + u, q);
+            for (int u = 0; u < U; u++) b[u] = bm_load_blk<WT>(wrow, i0 + u, q);
+        }
     }
 #pragma unroll
     for (int c = 0; c < M; c++) out[c] = bm_quad_finish<WT>(a0[c], a1[c]);
@@ -101,7 +143,7 @@ hipError_t fill_u32(const Launch &L, uint32_t *dst, uint32_t value, size_t n) {
 
 // ------------------------------------------------------------------------------------------- quantizers
 
-// One 32-value q8_2 block on the 32 lanes `lane32` = 0..31 of a half wave (crates/qdot/src/lib.rs:3883-3904).
+// One 32-value q8_2 block on the 32 lanes of a half wave (crates/qdot/src/lib.rs:3883-3904).
 // Returns the code; *t_out / *isum_out are valid on every lane. `bad` reports a value that is not finite.
 __device__ __forceinline__ int q82_block(float v, u32 *t_out, int *isum_out, bool *bad) {
     u32 ab = bm_f32_bits(v) & 0x7fffffffu;
@@ -231,26 +273,26 @@ hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, ui
 // ------------------------------------------------------------------------------------------------ gemv
 
 // y[row * m_total + col0 + c] = row . column (col0 + c), c < m <= 8. A quad a row, 64 rows a workgroup.
-template <int WT, int U>
+template <int WT, int U, int NB>
 __global__ __launch_bounds__(256) void k_gemv(const uint8_t *w, long rows, int nb, const uint8_t *act, int m_total,
                                               int col0, int m, float *y) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, q = tid & 3;
     const long row = (long)blockIdx.x * 64 + (tid >> 2);
     const bool active = row < rows;
-    const size_t row_bytes = (size_t)nb * bm_block_bytes<WT>();
-    const int col_bytes = nb * bm_act_sb_bytes<WT>();
+    const int n = NB > 0 ? NB : nb;
+    const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
+    const int col_bytes = n * bm_act_sb_bytes<WT>();
     const uint8_t *wrow = w + (size_t)(active ? row : 0) * row_bytes;
     Blk<WT> b[U];
-    if (active) preload<WT, U>(b, wrow, nb, q);
+    preload<WT, U>(b, wrow, q);
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *cols = lds + tab_bytes<WT>();
     stage_bytes(cols, act + (size_t)col0 * col_bytes, m * col_bytes);
     __syncthreads();
-    if (!active) return;
     float out[8];
-    row_dot<WT, U, 8>(b, wrow, cols, col_bytes, m, nb, q, tb, out, NoTap{});
-    if (q == 0) {
+    row_dot<WT, U, NB, 8>(b, wrow, cols, col_bytes, m, n, q, tb, out, NoTap{});
+    if (q == 0 && active) {
 #pragma unroll
         for (int c = 0; c < 8; c++)
             if (c < m) y[(size_t)row * m_total + col0 + c] = out[c];
@@ -261,7 +303,7 @@ __global__ __launch_bounds__(256) void k_gemv(const uint8_t *w, long rows, int n
 
 // One workgroup = 32 consecutive rows of one slot; eight lanes a row: a quad on the gate row, a quad on the up row.
 // With act_h the 32 values are quantized to one q8_2 block of the slot's down activation in the same launch.
-template <int WT, int U>
+template <int WT, int U, int NB>
 __global__ __launch_bounds__(256) void k_gate_up(const uint8_t *wg, const uint8_t *wu, u32 n_experts, int nb,
                                                  const uint8_t *act, const u32 *sel, int rpe, int slots_per_col,
                                                  float *h, uint8_t *act_h, u32 *fault, u32 layer) {
@@ -272,24 +314,28 @@ __global__ __launch_bounds__(256) void k_gate_up(const uint8_t *wg, const uint8_
     const int r = rb * 32 + (tid >> 3);
     const bool active = r < rpe;
     const u32 id = sel[slot];
+    const int n = NB > 0 ? NB : nb;
     const int h_col_bytes = (rpe / 128) * BM_Q82X4_STRIDE;
+    const int col_bytes = n * bm_act_sb_bytes<WT>();
+    const uint8_t *act_col = act + (size_t)(slot / slots_per_col) * col_bytes;
+    Stage<2> st;
+    st.load(act_col, col_bytes);
     if (id >= n_experts) { // uniform over the workgroup: no weight is read (crates/gpu/src/kquant/sel.rs:22-28)
         if (tid == 0) bm_raise(fault, layer, kSiteExpertId);
         if (h && active && (tid & 7) == 0) h[(size_t)slot * rpe + r] = bm_bits_f32(0x7fc00000u);
         if (act_h && tid < 32) q82_store(act_h + (size_t)slot * h_col_bytes, rb, tid, 0, 0x7fc0u, 0);
         return;
     }
-    const size_t row_bytes = (size_t)nb * bm_block_bytes<WT>();
-    const int col_bytes = nb * bm_act_sb_bytes<WT>();
+    const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
     const uint8_t *wrow = (which ? wu : wg) + ((size_t)id * rpe + (active ? r : 0)) * row_bytes;
     Blk<WT> b[U];
-    if (active) preload<WT, U>(b, wrow, nb, q);
+    preload<WT, U>(b, wrow, q);
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *col = lds + tab_bytes<WT>();
-    stage_bytes(col, act + (size_t)(slot / slots_per_col) * col_bytes, col_bytes);
+    st.store(col, act_col, col_bytes);
     __syncthreads();
-    float v[1] = {0.0f};
-    if (active) row_dot<WT, U, 1>(b, wrow, col, col_bytes, 1, nb, q, tb, v, NoTap{});
+    float v[1];
+    row_dot<WT, U, NB, 1>(b, wrow, col, col_bytes, 1, n, q, tb, v, NoTap{});
     const float other = __shfl_xor(v[0], 4, 64);
     const float hv = bm_swiglu(which ? other : v[0], which ? v[0] : other);
     if (h && active && (tid & 7) == 0) h[(size_t)slot * rpe + r] = hv;
@@ -311,7 +357,7 @@ __global__ __launch_bounds__(256) void k_gate_up(const uint8_t *wg, const uint8_
 // ------------------------------------------------------------------------------------- down: gemv_sel
 
 // Slot s: rows of expert sel[s] against column s. A quad a row, 64 rows a workgroup.
-template <int WT, int U>
+template <int WT, int U, int NB>
 __global__ __launch_bounds__(256) void k_gemv_sel(const uint8_t *w, u32 n_experts, int nb, const uint8_t *act,
                                                   const u32 *sel, int rpe, float *y, u32 *fault, u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -321,23 +367,26 @@ __global__ __launch_bounds__(256) void k_gemv_sel(const uint8_t *w, u32 n_expert
     const int r = rb * 64 + (tid >> 2);
     const bool active = r < rpe;
     const u32 id = sel[slot];
+    const int n = NB > 0 ? NB : nb;
+    const int col_bytes = n * bm_act_sb_bytes<WT>();
+    const uint8_t *act_col = act + (size_t)slot * col_bytes;
+    Stage<2> st;
+    st.load(act_col, col_bytes);
     if (id >= n_experts) { // the slot's rows stay untouched; a host slot is skipped silently
         if (tid == 0 && rb == 0 && id != 0xffffffffu) bm_raise(fault, layer, kSiteExpertId);
         return;
     }
-    const size_t row_bytes = (size_t)nb * bm_block_bytes<WT>();
-    const int col_bytes = nb * bm_act_sb_bytes<WT>();
+    const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
     const uint8_t *wrow = w + ((size_t)id * rpe + (active ? r : 0)) * row_bytes;
     Blk<WT> b[U];
-    if (active) preload<WT, U>(b, wrow, nb, q);
+    preload<WT, U>(b, wrow, q);
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *col = lds + tab_bytes<WT>();
-    stage_bytes(col, act + (size_t)slot * col_bytes, col_bytes);
+    st.store(col, act_col, col_bytes);
     __syncthreads();
-    if (!active) return;
     float v[1];
-    row_dot<WT, U, 1>(b, wrow, col, col_bytes, 1, nb, q, tb, v, NoTap{});
-    if (q == 0) y[(size_t)slot * rpe + r] = v[0];
+    row_dot<WT, U, NB, 1>(b, wrow, col, col_bytes, 1, n, q, tb, v, NoTap{});
+    if (q == 0 && active) y[(size_t)slot * rpe + r] = v[0];
 }
 
 // --------------------------------------------------------------------------------------------- combine
@@ -366,7 +415,7 @@ hipError_t combine_tokens(const Launch &L, const float *down, const float *w, co
 
 // One workgroup = one token and D = 64 / slots_per_token output rows: a quad for every (row, slot). The slot values
 // meet in LDS and one thread a row folds them in slot order, then adds the residual.
-template <int WT, int U>
+template <int WT, int U, int NB>
 __global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_experts, int nb, const uint8_t *act,
                                                       const u32 *sel, const float *wts, const float *resid, int spt,
                                                       int rpe, float *y, u32 *fault, u32 layer) {
@@ -379,27 +428,41 @@ __global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_ex
     const int r = rb * D + dl;
     const int slot = t * spt + e;
     const u32 id = sel[slot];
+    // the token's ids and weights for the closing sum, requested now and parked in LDS
+    const int si = tid < spt ? tid : 0;
+    const u32 my_sel = sel[t * spt + si];
+    const float my_w = wts[t * spt + si];
     const bool live = id < n_experts;
     const bool active = dl < D && r < rpe && live;
     if (!live && id != 0xffffffffu && rb == 0 && dl == 0 && q == 0) bm_raise(fault, layer, kSiteExpertId);
-    const size_t row_bytes = (size_t)nb * bm_block_bytes<WT>();
-    const int col_bytes = nb * bm_act_sb_bytes<WT>();
+    const int n = NB > 0 ? NB : nb;
+    const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
+    const int col_bytes = n * bm_act_sb_bytes<WT>();
+    const uint8_t *act_cols = act + (size_t)t * spt * col_bytes;
+    Stage<4> st;
+    st.load(act_cols, spt * col_bytes);
     const uint8_t *wrow = w + ((size_t)(live ? id : 0) * rpe + (active ? r : 0)) * row_bytes;
     Blk<WT> b[U];
-    if (active) preload<WT, U>(b, wrow, nb, q);
+    preload<WT, U>(b, wrow, q);
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *cols = lds + tab_bytes<WT>();
-    stage_bytes(cols, act + (size_t)t * spt * col_bytes, spt * col_bytes);
+    st.store(cols, act_cols, spt * col_bytes);
     float *part = reinterpret_cast<float *>(cols + (size_t)spt * col_bytes); // [D][spt]
+    float *s_w = part + D * spt;                                              // [spt]
+    u32 *s_sel = reinterpret_cast<u32 *>(s_w + spt);                          // [spt]
+    if (tid < spt) {
+        s_w[tid] = my_w;
+        s_sel[tid] = my_sel;
+    }
     __syncthreads();
-    float v[1] = {0.0f};
-    if (active) row_dot<WT, U, 1>(b, wrow, cols + (size_t)e * col_bytes, col_bytes, 1, nb, q, tb, v, NoTap{});
+    float v[1];
+    row_dot<WT, U, NB, 1>(b, wrow, cols + (size_t)e * col_bytes, col_bytes, 1, n, q, tb, v, NoTap{});
     if (q == 0 && dl < D) part[dl * spt + e] = v[0];
     __syncthreads();
     if (tid < D && rb * D + tid < rpe) {
         float acc = 0.0f;
         for (int s = 0; s < spt; s++)
-            if (sel[t * spt + s] < n_experts) acc = fmaf(wts[t * spt + s], part[tid * spt + s], acc);
+            if (s_sel[s] < n_experts) acc = fmaf(s_w[s], part[tid * spt + s], acc);
         const size_t o = (size_t)t * rpe + rb * D + tid;
         y[o] = resid ? __fadd_rn(acc, resid[o]) : acc;
     }
@@ -418,12 +481,13 @@ struct StoreTap {
     }
 };
 
-template <int WT, int U>
+template <int WT, int U, int NB>
 __global__ __launch_bounds__(64) void k_block_sums(const uint8_t *wrow, int nb, const uint8_t *act_col, int *out) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, q = tid & 3;
-    const int col_bytes = nb * bm_act_sb_bytes<WT>();
-    for (int i = tid; i < 16 * nb; i += blockDim.x) out[i] = 0;
+    const int n = NB > 0 ? NB : nb;
+    const int col_bytes = n * bm_act_sb_bytes<WT>();
+    for (int i = tid; i < 16 * n; i += blockDim.x) out[i] = 0;
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *col = lds + tab_bytes<WT>();
     stage_bytes(col, act_col, col_bytes);
@@ -431,13 +495,13 @@ __global__ __launch_bounds__(64) void k_block_sums(const uint8_t *wrow, int nb, 
     __syncthreads();
     if (tid >= 4) return;
     Blk<WT> b[U];
-    preload<WT, U>(b, wrow, nb, q);
+    preload<WT, U>(b, wrow, q);
     float v[1];
-    row_dot<WT, U, 1>(b, wrow, col, col_bytes, 1, nb, q, tb, v, StoreTap{out});
+    row_dot<WT, U, NB, 1>(b, wrow, col, col_bytes, 1, n, q, tb, v, StoreTap{out});
     if constexpr (WT == BM_IQ2XXS) {
         // the eight scales 2s + 1 of each super-block, as the dot reads them
         if (q == 0)
-            for (int i = 0; i < nb; i++)
+            for (int i = 0; i < n; i++)
                 for (int s = 0; s < 8; s++) {
                     u32 aux;
                     __builtin_memcpy(&aux, wrow + (size_t)i * BM_IQ2XXS_BLOCK + 6 + 8 * s, 4);
@@ -448,13 +512,6 @@ __global__ __launch_bounds__(64) void k_block_sums(const uint8_t *wrow, int nb, 
 
 // ---------------------------------------------------------------------------------------- launch helpers
 
-// Super-blocks a lane requests per batch. Enough to keep every byte of a Qwen3-shaped row (8 super-blocks of
-// Q4_K, 3 of Q6_K) in flight at once; longer rows walk in batches.
-template <int WT>
-constexpr int batch() {
-    return WT == BM_Q4K ? 8 : 4;
-}
-
 template <typename K>
 static hipError_t allow_lds(K kernel, size_t lds) {
     if (lds <= 64 * 1024) return hipSuccess;
@@ -462,20 +519,30 @@ static hipError_t allow_lds(K kernel, size_t lds) {
                                (int)lds);
 }
 
-#define BM_DISPATCH_TYPE(wtype, CALL)                                                                                  \
+// Picks the kernel variant for a row of nb super-blocks and runs CALL with WT, U and NB as constants. Each type
+// lists its whole-row variant first (the hot shape), then a batch of four, then one super-block at a time, which
+// divides every row.
+#define BM_VARIANT(T, UU, NN)                                                                                          \
+    {                                                                                                                  \
+        constexpr int WT = T, U = UU, NB = NN;                                                                         \
+        CALL_BODY;                                                                                                     \
+    }
+#define BM_DISPATCH(wtype, nb)                                                                                         \
     switch (wtype) {                                                                                                   \
-    case BM_Q4K: {                                                                                                     \
-        constexpr int WT = BM_Q4K;                                                                                     \
-        CALL;                                                                                                          \
-    } break;                                                                                                           \
-    case BM_Q6K: {                                                                                                     \
-        constexpr int WT = BM_Q6K;                                                                                     \
-        CALL;                                                                                                          \
-    } break;                                                                                                           \
-    case BM_IQ2XXS: {                                                                                                  \
-        constexpr int WT = BM_IQ2XXS;                                                                                  \
-        CALL;                                                                                                          \
-    } break;                                                                                                           \
+    case BM_Q4K:                                                                                                       \
+        if ((nb) == 8) BM_VARIANT(BM_Q4K, 8, 8)                                                                        \
+        else if ((nb) % 4 == 0) BM_VARIANT(BM_Q4K, 4, 0)                                                               \
+        else BM_VARIANT(BM_Q4K, 1, 0)                                                                                  \
+        break;                                                                                                         \
+    case BM_Q6K:                                                                                                       \
+        if ((nb) == 3) BM_VARIANT(BM_Q6K, 3, 3)                                                                        \
+        else if ((nb) % 4 == 0) BM_VARIANT(BM_Q6K, 4, 0)                                                               \
+        else BM_VARIANT(BM_Q6K, 1, 0)                                                                                  \
+        break;                                                                                                         \
+    case BM_IQ2XXS:                                                                                                    \
+        if ((nb) % 4 == 0) BM_VARIANT(BM_IQ2XXS, 4, 0)                                                                 \
+        else BM_VARIANT(BM_IQ2XXS, 1, 0)                                                                               \
+        break;                                                                                                         \
     default:                                                                                                           \
         return hipErrorInvalidValue;                                                                                   \
     }
@@ -489,101 +556,84 @@ int gemv_max_cols(int wtype, int k) {
     return m > 8 ? 8 : m;
 }
 
-template <int WT>
-static hipError_t gemv_t(const Launch &L, const uint8_t *w, int64_t rows, int nb, const uint8_t *act, int m_total,
-                         int col0, int m, float *y) {
-    const size_t lds = tab_bytes<WT>() + (size_t)m * nb * bm_act_sb_bytes<WT>();
-    auto kern = k_gemv<WT, batch<WT>()>;
-    hipError_t e = allow_lds(kern, lds);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 63) / 64)), dim3(256), lds, L.stream, w, (long)rows, nb, act,
-                       m_total, col0, m, y);
-    return hipGetLastError();
-}
-
 hipError_t gemv(const Launch &L, int wtype, const uint8_t *w, int64_t rows, int k, const uint8_t *act, int m_total,
                 int col0, int m, float *y) {
-    BM_DISPATCH_TYPE(wtype, return gemv_t<WT>(L, w, rows, k / 256, act, m_total, col0, m, y));
-    return hipSuccess;
-}
-
-template <int WT>
-static hipError_t gate_up_t(const Launch &L, const uint8_t *wg, const uint8_t *wu, int n_experts, int nb,
-                            const uint8_t *act, const uint32_t *sel, int n_slots, int rpe, int slots_per_col, float *h,
-                            uint8_t *act_h) {
-    const size_t lds = tab_bytes<WT>() + (size_t)nb * bm_act_sb_bytes<WT>() + 32 * sizeof(float);
-    auto kern = k_gate_up<WT, batch<WT>()>;
-    hipError_t e = allow_lds(kern, lds);
-    if (e != hipSuccess) return e;
-    const unsigned grid = (unsigned)n_slots * (unsigned)((rpe + 31) / 32);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, wg, wu, (u32)n_experts, nb, act, sel, rpe,
-                       slots_per_col, h, act_h, L.fault, L.layer);
+    const int nb = k / 256;
+    const size_t lds = tab_bytes_rt(wtype) + (size_t)m * nb * act_sb_bytes(wtype);
+#define CALL_BODY                                                                                                      \
+    auto kern = k_gemv<WT, U, NB>;                                                                                     \
+    hipError_t e = allow_lds(kern, lds);                                                                               \
+    if (e != hipSuccess) return e;                                                                                     \
+    hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 63) / 64)), dim3(256), lds, L.stream, w, (long)rows, nb, act,     \
+                       m_total, col0, m, y);
+    BM_DISPATCH(wtype, nb)
+#undef CALL_BODY
     return hipGetLastError();
 }
 
 hipError_t gate_up(const Launch &L, int wtype, const uint8_t *wg, const uint8_t *wu, int n_experts, int k,
                    const uint8_t *act, const uint32_t *sel, int n_slots, int rows_per_expert, int slots_per_col,
                    float *h, uint8_t *act_h) {
-    BM_DISPATCH_TYPE(wtype, return gate_up_t<WT>(L, wg, wu, n_experts, k / 256, act, sel, n_slots, rows_per_expert,
-                                                 slots_per_col, h, act_h));
-    return hipSuccess;
-}
-
-template <int WT>
-static hipError_t gemv_sel_t(const Launch &L, const uint8_t *w, int n_experts, int nb, const uint8_t *act,
-                             const uint32_t *sel, int n_slots, int rpe, float *y) {
-    const size_t lds = tab_bytes<WT>() + (size_t)nb * bm_act_sb_bytes<WT>();
-    auto kern = k_gemv_sel<WT, batch<WT>()>;
-    hipError_t e = allow_lds(kern, lds);
-    if (e != hipSuccess) return e;
-    const unsigned grid = (unsigned)n_slots * (unsigned)((rpe + 63) / 64);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act, sel, rpe, y, L.fault,
-                       L.layer);
+    const int nb = k / 256, rpe = rows_per_expert;
+    const size_t lds = tab_bytes_rt(wtype) + (size_t)nb * act_sb_bytes(wtype) + 32 * sizeof(float);
+    const unsigned grid = (unsigned)n_slots * (unsigned)((rpe + 31) / 32);
+#define CALL_BODY                                                                                                      \
+    auto kern = k_gate_up<WT, U, NB>;                                                                                  \
+    hipError_t e = allow_lds(kern, lds);                                                                               \
+    if (e != hipSuccess) return e;                                                                                     \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, wg, wu, (u32)n_experts, nb, act, sel, rpe,          \
+                       slots_per_col, h, act_h, L.fault, L.layer);
+    BM_DISPATCH(wtype, nb)
+#undef CALL_BODY
     return hipGetLastError();
 }
 
 hipError_t gemv_sel(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const uint8_t *act,
                     const uint32_t *sel, int n_slots, int rows_per_expert, float *y) {
-    BM_DISPATCH_TYPE(wtype, return gemv_sel_t<WT>(L, w, n_experts, k / 256, act, sel, n_slots, rows_per_expert, y));
-    return hipSuccess;
-}
-
-template <int WT>
-static hipError_t down_combine_t(const Launch &L, const uint8_t *w, int n_experts, int nb, const uint8_t *act,
-                                 const uint32_t *sel, const float *wts, const float *resid, int spt, int m, int rpe,
-                                 float *y) {
-    const int D = 64 / spt;
-    const size_t lds = tab_bytes<WT>() + (size_t)spt * nb * bm_act_sb_bytes<WT>() + (size_t)D * spt * sizeof(float);
-    auto kern = k_down_combine<WT, batch<WT>()>;
-    hipError_t e = allow_lds(kern, lds);
-    if (e != hipSuccess) return e;
-    const unsigned grid = (unsigned)m * (unsigned)((rpe + D - 1) / D);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act, sel, wts, resid, spt,
-                       rpe, y, L.fault, L.layer);
+    const int nb = k / 256, rpe = rows_per_expert;
+    const size_t lds = tab_bytes_rt(wtype) + (size_t)nb * act_sb_bytes(wtype);
+    const unsigned grid = (unsigned)n_slots * (unsigned)((rpe + 63) / 64);
+#define CALL_BODY                                                                                                      \
+    auto kern = k_gemv_sel<WT, U, NB>;                                                                                 \
+    hipError_t e = allow_lds(kern, lds);                                                                               \
+    if (e != hipSuccess) return e;                                                                                     \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act, sel, rpe, y, L.fault,   \
+                       L.layer);
+    BM_DISPATCH(wtype, nb)
+#undef CALL_BODY
     return hipGetLastError();
 }
 
 hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const uint8_t *act,
                         const uint32_t *sel, const float *wts, const float *resid, int slots_per_token, int m,
                         int rows_per_expert, float *y) {
-    BM_DISPATCH_TYPE(wtype, return down_combine_t<WT>(L, w, n_experts, k / 256, act, sel, wts, resid, slots_per_token,
-                                                      m, rows_per_expert, y));
-    return hipSuccess;
-}
-
-template <int WT>
-static hipError_t block_sums_t(const Launch &L, const uint8_t *wrow, int nb, const uint8_t *col, int32_t *out) {
-    const size_t lds = tab_bytes<WT>() + (size_t)nb * bm_act_sb_bytes<WT>();
-    auto kern = k_block_sums<WT, batch<WT>()>;
-    hipError_t e = allow_lds(kern, lds);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3(1), dim3(64), lds, L.stream, wrow, nb, col, out);
+    const int nb = k / 256, rpe = rows_per_expert, spt = slots_per_token;
+    const int D = 64 / spt;
+    const size_t lds = tab_bytes_rt(wtype) + (size_t)spt * nb * act_sb_bytes(wtype) +
+                       ((size_t)D * spt + 2 * (size_t)spt) * sizeof(float);
+    const unsigned grid = (unsigned)m * (unsigned)((rpe + D - 1) / D);
+#define CALL_BODY                                                                                                      \
+    auto kern = k_down_combine<WT, U, NB>;                                                                             \
+    hipError_t e = allow_lds(kern, lds);                                                                               \
+    if (e != hipSuccess) return e;                                                                                     \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act, sel, wts, resid, spt,   \
+                       rpe, y, L.fault, L.layer);
+    BM_DISPATCH(wtype, nb)
+#undef CALL_BODY
     return hipGetLastError();
 }
 
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out) {
-    BM_DISPATCH_TYPE(wtype, return block_sums_t<WT>(L, wrow, k / 256, col, out));
-    return hipSuccess;
+    const int nb = k / 256;
+    const size_t lds = tab_bytes_rt(wtype) + (size_t)nb * act_sb_bytes(wtype);
+#define CALL_BODY                                                                                                      \
+    auto kern = k_block_sums<WT, U, NB>;                                                                               \
+    hipError_t e = allow_lds(kern, lds);                                                                               \
+    if (e != hipSuccess) return e;                                                                                     \
+    hipLaunchKernelGGL(kern, dim3(1), dim3(64), lds, L.stream, wrow, nb, col, out);
+    BM_DISPATCH(wtype, nb)
+#undef CALL_BODY
+    return hipGetLastError();
 }
 
 } // namespace bmk

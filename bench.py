@@ -70,6 +70,9 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--mode", choices=("two", "single", "chain"), default="two",
+                    help="two: bm_moe_decode in two launches (quantizers folded in); single: bm_moe_decode in one "
+                         "launch; chain: quantize, gate_up, down_combine")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus above 1 is not supported (nothing here shards)")
@@ -96,9 +99,22 @@ def main():
     act = gpu.act(bm.Q4_K, HIDDEN, 1)
     act_h = gpu.act(bm.Q6_K, FF, TOP_K)
 
-    def enqueue_step(i, which=("quant", "gate_up", "down")):
+    single = args.mode == "single"
+    kernels = {"single": ("step",), "two": ("gate_up_x", "down"), "chain": ("quant", "gate_up", "down")}[args.mode]
+    gpu.set_decode_plan(bm.PLAN_ONE_LAUNCH if single else bm.PLAN_TWO_LAUNCHES)
+
+    def enqueue_step(i, which=kernels):
         t = i % n_tok
         dg, du, dd = layers[i % len(layers)]
+        if "gate_up_x" in which and "down" in which:
+            gpu.enqueue_moe_decode(dg, du, dd, xd.ptr + 4 * t * HIDDEN, sel.ptr + 4 * t * TOP_K, wt.ptr + 4 * t * TOP_K,
+                                   None, TOP_K, 1, act_h, y.ptr + 4 * t * HIDDEN)
+            return
+        if "gate_up_x" in which:
+            gpu.enqueue_gate_up_x(dg, du, xd.ptr + 4 * t * HIDDEN, sel.ptr + 4 * t * TOP_K, TOP_K, 1, FF, act_h)
+        if "step" in which:
+            gpu.enqueue_moe_decode(dg, du, dd, xd.ptr + 4 * t * HIDDEN, sel.ptr + 4 * t * TOP_K, wt.ptr + 4 * t * TOP_K,
+                                   None, TOP_K, 1, act_h, y.ptr + 4 * t * HIDDEN)
         if "quant" in which:
             gpu.enqueue_quantize(xd.ptr + 4 * t * HIDDEN, 1, act)
         if "gate_up" in which:
@@ -150,7 +166,7 @@ def main():
     # per-kernel launch durations: a graph of one kernel only, over the same cycling inputs, between events on
     # the launch stream
     kernel_us = {}
-    for name in ("quant", "gate_up", "down"):
+    for name in kernels:
         gpu.capture_begin()
         for i in range(unit):
             enqueue_step(i, (name,))
@@ -166,7 +182,15 @@ def main():
         gpu.graph_destroy(g1)
     gate_up_bytes = TOP_K * 2 * FF * bm.row_bytes(bm.Q4_K, HIDDEN)
     down_bytes = TOP_K * HIDDEN * bm.row_bytes(bm.Q6_K, FF)
-    achieved = gate_up_bytes / (kernel_us["gate_up"] * 1e-6) / 1e9
+    if single:
+        dominant, dom_bytes = "k_moe_decode<Q4_K, Q6_K>", bytes_per_token
+        achieved = dom_bytes / (kernel_us["step"] * 1e-6) / 1e9
+        kernel_gbps = {"step": achieved}
+    else:
+        gk = "gate_up_x" if args.mode == "two" else "gate_up"
+        dominant, dom_bytes = ("k_gate_up_x<Q4_K>" if args.mode == "two" else "k_gate_up<Q4_K>"), gate_up_bytes
+        achieved = dom_bytes / (kernel_us[gk] * 1e-6) / 1e9
+        kernel_gbps = {gk: achieved, "down": down_bytes / (kernel_us["down"] * 1e-6) / 1e9}
     assert gpu.fault() == (bm.FAULT_NONE, 0)
 
     cpu = None
@@ -205,16 +229,16 @@ def main():
         "data": "synthetic",
         "config": {"workload": "Qwen3-30B-A3B-shaped MoE layer decode, 1 token: hidden 2048, 128 experts x ff 768, "
                                "Q4_K gate/up + Q6_K down, softmax top-8 renormalised (BASELINE.json configs[1])",
-                   "layer_copies": len(layers), "distinct_tokens": n_tok, "launches_per_step": 3, "mode": "hipGraph replay"},
+                   "layer_copies": len(layers), "distinct_tokens": n_tok, "launches_per_step": len(kernels), "mode": "hipGraph replay"},
         "hbm_tbps": bytes_per_token / (us_per_token * 1e-6) / 1e12,
         "algorithmic_bytes_per_token": bytes_per_token,
         "event_ms_per_step": ev_ms / steps,
         "kernel_us": kernel_us,
-        "kernel_gbps": {"gate_up": achieved, "down": down_bytes / (kernel_us["down"] * 1e-6) / 1e9},
+        "kernel_gbps": kernel_gbps,
         "parity": parity,
-        "roofline": {"bound": "hbm", "kernel": "k_gate_up<Q4_K>", "achieved": achieved, "peak": HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes_per_launch": gate_up_bytes},
+                     "algorithmic_bytes_per_launch": dom_bytes},
         "cpu_baseline": cpu,
     }
     print(json.dumps(out), flush=True)

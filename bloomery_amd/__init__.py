@@ -19,7 +19,8 @@ LIB_PATH = os.path.join(HERE, "libbm_moe_hip.so")
 Q4_K, Q6_K, IQ2_XXS = 12, 14, 16
 FAULT_NONE = 0xFFFFFFFF
 LAYER_NONE = 0xFFFF
-SITE_QUANT_COLUMN, SITE_EXPERT_ID = 1, 7
+SITE_QUANT_COLUMN, SITE_EXPERT_ID, SITE_STALLED = 1, 7, 31
+PLAN_ONE_LAUNCH, PLAN_TWO_LAUNCHES = 1, 2
 HOST_SLOT = 0xFFFFFFFF
 
 OK, ESHAPE, EDRIVER, ETYPE, EARG, EFAULT = 0, -1, -2, -3, -4, -5
@@ -59,6 +60,10 @@ SYMBOLS = {
     "bm_gemv_sel": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "bm_combine_tokens": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_down_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "bm_moe_decode": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp]),
+    "bm_set_spin_limit": (_i, [_vp, _u32]),
+    "bm_set_decode_plan": (_i, [_vp, _i]),
+    "bm_gate_up_x": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
     "bm_block_sums": (_i, [_vp, _vp, _i64, _vp, _i, _vp]),
     "bm_capture_begin": (_i, [_vp]),
     "bm_capture_end": (_i, [_vp, C.POINTER(_vp)]),
@@ -308,6 +313,23 @@ class Gpu:
     def enqueue_down_combine(self, w, act, sel, wts, resid, n_slots_per_token, m, rows_per_expert, y):
         self._check(self.lib.bm_down_combine(self.ctx, w.handle, act.handle, _ptr(sel), _ptr(wts), _ptr(resid),
                                              n_slots_per_token, m, rows_per_expert, _ptr(y)))
+
+    def enqueue_moe_decode(self, wg, wu, wd, x, sel, wts, resid, n_slots_per_token, m, act_h, y, act_x=None, h=None):
+        """The whole layer step in one launch (bm_moe_decode)."""
+        self._check(self.lib.bm_moe_decode(self.ctx, wg.handle, wu.handle, wd.handle, _ptr(x), _ptr(sel), _ptr(wts),
+                                           _ptr(resid), n_slots_per_token, m, act_h.handle,
+                                           act_x.handle if act_x is not None else None, _ptr(h), _ptr(y)))
+
+    def enqueue_gate_up_x(self, wg, wu, x, sel, n_slots_per_token, m, rows_per_expert, act_h, act_x=None, h=None):
+        self._check(self.lib.bm_gate_up_x(self.ctx, wg.handle, wu.handle, _ptr(x), _ptr(sel), n_slots_per_token, m,
+                                          rows_per_expert, act_h.handle, act_x.handle if act_x is not None else None,
+                                          _ptr(h)))
+
+    def set_decode_plan(self, plan):
+        self._check(self.lib.bm_set_decode_plan(self.ctx, plan))
+
+    def set_spin_limit(self, spins):
+        self._check(self.lib.bm_set_spin_limit(self.ctx, spins))
 
     def enqueue_block_sums(self, w, row, act, col, out):
         self._check(self.lib.bm_block_sums(self.ctx, w.handle, row, act.handle, col, _ptr(out)))

@@ -18,6 +18,9 @@ struct bm_ctx {
     bool own_stream = false;
     uint32_t *fault = nullptr;
     uint32_t layer = BM_LAYER_NONE;
+    uint32_t *counters = nullptr; // bm_moe_decode's producer/consumer counts, zero between launches
+    int decode_plan = BM_PLAN_TWO_LAUNCHES;
+    uint32_t spin_limit = 1u << 18; // a poll is a round trip to memory: some tenths of a second of waiting
     std::string err;
 };
 
@@ -58,10 +61,12 @@ static int driver(bm_ctx *ctx, const char *what, hipError_t e) {
 static bool known_type(int t) { return t == BM_TYPE_Q4_K || t == BM_TYPE_Q6_K || t == BM_TYPE_IQ2_XXS; }
 // Q8_2_X4 for the K-quants, Q8_K for IQ2_XXS (crates/gguf/src/qtype.rs host_act).
 static int act_form(int t) { return t == BM_TYPE_IQ2_XXS ? 1 : 0; }
+// Bytes between two columns of a bm_act on the device (the CPU path's bytes plus the dot kernels' tables).
+static size_t dev_col_bytes(int wtype, int k) { return (size_t)bmk::act_col_bytes(wtype, k); }
 
 extern "C" {
 
-int bm_version(void) { return 100; }
+int bm_version(void) { return 101; }
 
 int64_t bm_row_bytes(int wtype, int k) {
     if (!known_type(wtype)) return BM_ETYPE;
@@ -102,8 +107,15 @@ static int ctx_make(int device, hipStream_t stream, bool own, bm_ctx **out) {
         e = hipMemset(c->fault, 0, sizeof(uint32_t) * BM_FAULT_WORDS);
         if (e == hipSuccess) e = hipMemset(c->fault, 0xff, sizeof(uint32_t));
     }
+    if (e == hipSuccess) {
+        const size_t cb = sizeof(uint32_t) * (bmk::kMaxDecodeTokens + 1);
+        e = hipMalloc((void **)&c->counters, cb);
+        if (e == hipSuccess) e = hipMemset(c->counters, 0, cb);
+    }
+    if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
         if (c->fault) (void)hipFree(c->fault);
+        if (c->counters) (void)hipFree(c->counters);
         if (c->own_stream) (void)hipStreamDestroy(c->stream);
         delete c;
         return fail(nullptr, BM_EDRIVER, "bm_ctx_create: fault word: %s", hipGetErrorString(e));
@@ -123,6 +135,7 @@ void bm_ctx_destroy(bm_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(ctx->fault);
+    (void)hipFree(ctx->counters);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -160,6 +173,8 @@ int bm_fault_clear(bm_ctx *ctx) {
     bmk::Launch L = launch_of(ctx);
     hipError_t e = bmk::fill_u32(L, ctx->fault + 1, 0u, BM_FAULT_WORDS - 1);
     if (e == hipSuccess) e = bmk::fill_u32(L, ctx->fault, BM_FAULT_NONE, 1);
+    // a launch that gave up waiting may have left its counts behind
+    if (e == hipSuccess) e = bmk::fill_u32(L, ctx->counters, 0u, bmk::kMaxDecodeTokens + 1);
     return driver(ctx, "bm_fault_clear", e);
 }
 
@@ -262,7 +277,7 @@ int bm_act_create(bm_ctx *ctx, int wtype, int k, int m_cap, bm_act **out) {
     if (m_cap <= 0) return fail(ctx, BM_ESHAPE, "bm_act_create: m_cap = %d must be positive", m_cap);
     bm_act *a = new (std::nothrow) bm_act{ctx, wtype, k, m_cap, nullptr};
     if (!a) return fail(ctx, BM_EDRIVER, "bm_act_create: out of host memory");
-    const size_t bytes = (size_t)m_cap * (size_t)bm_col_bytes(wtype, k);
+    const size_t bytes = (size_t)m_cap * dev_col_bytes(wtype, k);
     hipError_t e = hipMalloc((void **)&a->dev, bytes);
     if (e == hipSuccess) e = hipMemset(a->dev, 0, bytes);
     if (e != hipSuccess) {
@@ -283,15 +298,18 @@ void bm_act_destroy(bm_act *act) {
 int bm_act_download(bm_ctx *ctx, const bm_act *act, int col, void *host_bytes) {
     if (!ctx || !act || !host_bytes) return fail(ctx, BM_EARG, "bm_act_download: NULL argument");
     if (col < 0 || col >= act->m_cap) return fail(ctx, BM_ESHAPE, "bm_act_download: column %d of %d", col, act->m_cap);
-    const size_t cb = (size_t)bm_col_bytes(act->wtype, act->k);
-    return bm_dev_download(ctx, host_bytes, act->dev + (size_t)col * cb, cb);
+    // a column starts with the CPU path's bytes
+    return bm_dev_download(ctx, host_bytes, act->dev + (size_t)col * dev_col_bytes(act->wtype, act->k),
+                           (size_t)bm_col_bytes(act->wtype, act->k));
 }
 
 int bm_act_upload(bm_ctx *ctx, bm_act *act, int col, const void *host_bytes) {
     if (!ctx || !act || !host_bytes) return fail(ctx, BM_EARG, "bm_act_upload: NULL argument");
     if (col < 0 || col >= act->m_cap) return fail(ctx, BM_ESHAPE, "bm_act_upload: column %d of %d", col, act->m_cap);
-    const size_t cb = (size_t)bm_col_bytes(act->wtype, act->k);
-    return bm_dev_upload(ctx, act->dev + (size_t)col * cb, host_bytes, cb);
+    uint8_t *dst = act->dev + (size_t)col * dev_col_bytes(act->wtype, act->k);
+    int rc = bm_dev_upload(ctx, dst, host_bytes, (size_t)bm_col_bytes(act->wtype, act->k));
+    if (rc || act_form(act->wtype) != 0) return rc;
+    return driver(ctx, "bm_act_upload: tables", bmk::q82_tables(launch_of(ctx), dst, 1, act->k));
 }
 
 // ------------------------------------------------------------------------------------------------ launchers
@@ -415,12 +433,98 @@ int bm_down_combine(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const u
     if ((int64_t)m * n_slots_per_token > act->m_cap)
         return fail(ctx, BM_ESHAPE, "%s: an activation column per slot: %d tokens x %d slots, act holds %d", what, m,
                     n_slots_per_token, act->m_cap);
-    const size_t lds = (size_t)n_slots_per_token * (size_t)bm_col_bytes(act->wtype, act->k) + 4096;
+    const size_t lds = (size_t)n_slots_per_token * dev_col_bytes(act->wtype, act->k) + 4096;
     if (lds > (size_t)bmk::kMaxLds)
         return fail(ctx, BM_ESHAPE, "%s: %d columns of k = %d do not fit the workgroup's LDS; use bm_gemv_sel and bm_combine_tokens", what,
                     n_slots_per_token, act->k);
     return driver(ctx, what, bmk::down_combine(launch_of(ctx), w->wtype, w->dev, n_experts, w->k, act->dev, sel_dev, w_dev,
                                                resid_dev, n_slots_per_token, m, rows_per_expert, y_dev));
+}
+
+int bm_set_spin_limit(bm_ctx *ctx, uint32_t spins) {
+    if (!ctx) return fail(nullptr, BM_EARG, "bm_set_spin_limit: ctx is NULL");
+    ctx->spin_limit = spins;
+    return BM_OK;
+}
+
+int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const float *x_dev, const uint32_t *sel_dev,
+                 int n_slots_per_token, int m, int rows_per_expert, bm_act *act_h, bm_act *act_x, float *h_dev) {
+    const char *what = "bm_gate_up_x";
+    if (!ctx || !wg || !wu || !x_dev || !sel_dev || !act_h) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (wg->wtype != BM_TYPE_Q4_K || wu->wtype != BM_TYPE_Q4_K)
+        return fail(ctx, BM_ETYPE, "%s: takes Q4_K gate and up stacks, got types %d and %d; use bm_quantize and bm_gate_up", what,
+                    wg->wtype, wu->wtype);
+    if (wu->k != wg->k || wu->rows != wg->rows)
+        return fail(ctx, BM_ESHAPE, "%s: gate is %lld x %d, up %lld x %d", what, (long long)wg->rows, wg->k, (long long)wu->rows, wu->k);
+    const int hidden = wg->k, ff = rows_per_expert;
+    int n_experts = 0;
+    int rc = check_stack(ctx, what, wg, ff, &n_experts);
+    if (rc) return rc;
+    if (ff % 256 != 0) return fail(ctx, BM_ESHAPE, "%s: rows_per_expert = %d is not a whole number of 256-value super-blocks", what, ff);
+    if (n_slots_per_token < 1 || m < 1 || m > bmk::kMaxDecodeTokens)
+        return fail(ctx, BM_ESHAPE, "%s: %d slots a token, m = %d tokens (1..=%d)", what, n_slots_per_token, m, bmk::kMaxDecodeTokens);
+    if (act_form(act_h->wtype) != 0 || act_h->k != ff || (int64_t)act_h->m_cap < (int64_t)m * n_slots_per_token)
+        return fail(ctx, BM_ESHAPE, "%s: act_h must hold %d Q8_2_X4 columns of k = %d; it holds %d of k = %d (type %d)", what,
+                    m * n_slots_per_token, ff, act_h->m_cap, act_h->k, act_h->wtype);
+    if (act_x && (act_form(act_x->wtype) != 0 || act_x->k != hidden || act_x->m_cap < m))
+        return fail(ctx, BM_ESHAPE, "%s: act_x must hold %d Q8_2_X4 columns of k = %d; it holds %d of k = %d (type %d)", what, m, hidden,
+                    act_x->m_cap, act_x->k, act_x->wtype);
+    if (((uintptr_t)x_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: x_dev %p is not 16-byte aligned", what, (const void *)x_dev);
+    if (dev_col_bytes(wg->wtype, hidden) + 128 > (size_t)bmk::kMaxLds)
+        return fail(ctx, BM_ESHAPE, "%s: a column of hidden = %d does not fit the workgroup's LDS", what, hidden);
+    return driver(ctx, what,
+                  bmk::gate_up_x(launch_of(ctx), wg->wtype, x_dev, wg->dev, wu->dev, n_experts, hidden, ff, sel_dev, n_slots_per_token, m,
+                                 act_x ? act_x->dev : nullptr, act_h->dev, h_dev));
+}
+
+int bm_set_decode_plan(bm_ctx *ctx, int plan) {
+    if (!ctx) return fail(nullptr, BM_EARG, "bm_set_decode_plan: ctx is NULL");
+    if (plan != BM_PLAN_ONE_LAUNCH && plan != BM_PLAN_TWO_LAUNCHES)
+        return fail(ctx, BM_EARG, "bm_set_decode_plan: plan %d is neither BM_PLAN_ONE_LAUNCH nor BM_PLAN_TWO_LAUNCHES", plan);
+    ctx->decode_plan = plan;
+    return BM_OK;
+}
+
+int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_weights *wd, const float *x_dev,
+                  const uint32_t *sel_dev, const float *w_dev, const float *resid_dev, int n_slots_per_token, int m,
+                  bm_act *act_h, bm_act *act_x, float *h_dev, float *y_dev) {
+    const char *what = "bm_moe_decode";
+    if (!ctx || !wg || !wu || !wd || !x_dev || !sel_dev || !w_dev || !act_h || !y_dev)
+        return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (wg->wtype != wu->wtype)
+        return fail(ctx, BM_ETYPE, "%s: gate is type %d and up type %d; one launch reads one type", what, wg->wtype, wu->wtype);
+    if (!bmk::moe_decode_supported(wg->wtype, wd->wtype))
+        return fail(ctx, BM_ETYPE, "%s: the single launch takes Q4_K gate/up with Q6_K or Q4_K down, got %d and %d; use the separate launches",
+                    what, wg->wtype, wd->wtype);
+    if (wu->k != wg->k || wu->rows != wg->rows)
+        return fail(ctx, BM_ESHAPE, "%s: gate is %lld x %d, up %lld x %d", what, (long long)wg->rows, wg->k, (long long)wu->rows, wu->k);
+    const int hidden = wg->k, ff = wd->k;
+    int n_experts = 0, n_down = 0;
+    int rc = check_stack(ctx, what, wg, ff, &n_experts);
+    if (!rc) rc = check_stack(ctx, what, wd, hidden, &n_down);
+    if (rc) return rc;
+    if (n_down != n_experts)
+        return fail(ctx, BM_ESHAPE, "%s: gate/up hold %d experts of %d rows, down %d experts of %d rows", what, n_experts, ff, n_down, hidden);
+    if (n_slots_per_token < 1 || n_slots_per_token > bmk::kMaxCombineSlots)
+        return fail(ctx, BM_ESHAPE, "%s: %d slots a token outside 1..=%d", what, n_slots_per_token, bmk::kMaxCombineSlots);
+    if (m < 1 || m > bmk::kMaxDecodeTokens)
+        return fail(ctx, BM_ESHAPE, "%s: m = %d tokens outside 1..=%d", what, m, bmk::kMaxDecodeTokens);
+    if (act_form(act_h->wtype) != 0 || act_h->k != ff || (int64_t)act_h->m_cap < (int64_t)m * n_slots_per_token)
+        return fail(ctx, BM_ESHAPE, "%s: act_h must hold %d Q8_2_X4 columns of k = %d; it holds %d of k = %d (type %d)", what,
+                    m * n_slots_per_token, ff, act_h->m_cap, act_h->k, act_h->wtype);
+    if (act_x && (act_form(act_x->wtype) != 0 || act_x->k != hidden || act_x->m_cap < m))
+        return fail(ctx, BM_ESHAPE, "%s: act_x must hold %d Q8_2_X4 columns of k = %d; it holds %d of k = %d (type %d)", what, m, hidden,
+                    act_x->m_cap, act_x->k, act_x->wtype);
+    if (((uintptr_t)x_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: x_dev %p is not 16-byte aligned", what, (const void *)x_dev);
+    const size_t lds_a = dev_col_bytes(wg->wtype, hidden) + 128;
+    const size_t lds_b = (size_t)n_slots_per_token * dev_col_bytes(wd->wtype, ff) + 4096;
+    if (lds_a > (size_t)bmk::kMaxLds || lds_b > (size_t)bmk::kMaxLds)
+        return fail(ctx, BM_ESHAPE, "%s: hidden = %d or %d columns of ff = %d do not fit the workgroup's LDS; use the separate launches", what,
+                    hidden, n_slots_per_token, ff);
+    return driver(ctx, what,
+                  bmk::moe_decode(launch_of(ctx), ctx->decode_plan, wg->wtype, wd->wtype, x_dev, wg->dev, wu->dev, wd->dev, n_experts, hidden, ff, sel_dev,
+                                  w_dev, resid_dev, n_slots_per_token, m, act_x ? act_x->dev : nullptr, act_h->dev, h_dev, y_dev,
+                                  ctx->counters, ctx->spin_limit));
 }
 
 int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *act, int col, int32_t *out_dev) {
@@ -431,7 +535,7 @@ int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *a
     if (row < 0 || row >= w->rows) return fail(ctx, BM_ESHAPE, "%s: row %lld of %lld", what, (long long)row, (long long)w->rows);
     if (col < 0 || col >= act->m_cap) return fail(ctx, BM_ESHAPE, "%s: column %d of %d", what, col, act->m_cap);
     const uint8_t *wrow = w->dev + (size_t)row * (size_t)bm_row_bytes(w->wtype, w->k);
-    const uint8_t *c = act->dev + (size_t)col * (size_t)bm_col_bytes(act->wtype, act->k);
+    const uint8_t *c = act->dev + (size_t)col * dev_col_bytes(act->wtype, act->k);
     return driver(ctx, what, bmk::block_sums(launch_of(ctx), w->wtype, wrow, w->k, c, out_dev));
 }
 

@@ -8,6 +8,13 @@
 // acc_{l+4}). The integer sums are formed with v_dot4_i32_i8 over the same 16-value (Q4_K, Q6_K) or 4-value
 // (IQ2_XXS) spans the reference's i32 lanes cover; they are exact, so their inner order is free.
 //
+// Activation columns on the device. A Q8_K column (IQ2_XXS weights) is the CPU path's bytes, 296 a super-block.
+// A Q8_2_X4 column (Q4_K, Q6_K weights) is the CPU path's bytes (288 a super-block) followed by two tables the
+// quantizers write beside them so the dots need no per-block unpacking: for each 32-value block the pair
+// (d8 as f32, d8 * (f32)isum) - the second is the product the reference forms first in its min term - and for each
+// 16 values the i32 sum of the stored codes (Q6_K's -32 offset comes out through it). nb super-blocks give
+// nb * 288 bytes, then nb * 64 table bytes, then nb * 64 sum bytes: 416 * nb in all.
+//
 // Build: -ffp-contract=off (a product meets a sum in one rounding only where fmaf is written), f32 denormals
 // kept, correctly rounded f32 divide (hipcc's defaults for gfx950).
 #ifndef BM_DEVICE_CUH
@@ -28,6 +35,8 @@ typedef uint32_t u32;
 #define BM_IQ2XXS_BLOCK 66
 #define BM_Q82X4_STRIDE 144
 #define BM_Q8K_STRIDE 296
+#define BM_Q82_SB_REF 288 // reference bytes of one super-block of a Q8_2_X4 column
+#define BM_Q82_SB_EXT 416 // with the two tables
 
 // ------------------------------------------------------------------------------------------------ scalars
 
@@ -77,26 +86,58 @@ __device__ __forceinline__ u32 bm_ld2u(const uint8_t *p) {
     return v;
 }
 
-// ------------------------------------------------------------------------------------------ quad exchange
+// ------------------------------------------------------------------------------------------ lane exchange
 
-// Lane ^ 1 and lane ^ 2 inside a quad, through DPP quad_perm (no LDS traffic).
-__device__ __forceinline__ float bm_quad_xor1(float v) {
-    return bm_bits_f32((u32)__builtin_amdgcn_mov_dpp((int)bm_f32_bits(v), 0xB1, 0xF, 0xF, true));
+// Data-parallel-primitive moves: no LDS traffic, a few cycles each. CTRL is the DPP control word.
+template <int CTRL>
+__device__ __forceinline__ u32 bm_dpp(u32 v) {
+    return (u32)__builtin_amdgcn_mov_dpp((int)v, CTRL, 0xF, 0xF, true);
 }
-__device__ __forceinline__ float bm_quad_xor2(float v) {
-    return bm_bits_f32((u32)__builtin_amdgcn_mov_dpp((int)bm_f32_bits(v), 0x4E, 0xF, 0xF, true));
+template <int CTRL>
+__device__ __forceinline__ float bm_dppf(float v) {
+    return bm_bits_f32(bm_dpp<CTRL>(bm_f32_bits(v)));
 }
+constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane i <-> 7 - i inside each 8
+constexpr int kDppMirror = 0x140;     // lane i <-> 15 - i inside each 16
+constexpr int kDppShl1 = 0x101, kDppShl2 = 0x102, kDppShl4 = 0x104; // lane i reads lane i + n of its row of 16
+constexpr int kDppShr4 = 0x114;                                     // lane i reads lane i - 4
+
+__device__ __forceinline__ float bm_quad_xor1(float v) { return bm_dppf<kDppXor1>(v); }
+__device__ __forceinline__ float bm_quad_xor2(float v) { return bm_dppf<kDppXor2>(v); }
 __device__ __forceinline__ u32 bm_quad_bcast(u32 v, int k) {
     switch (k) {
     case 0:
-        return (u32)__builtin_amdgcn_mov_dpp((int)v, 0x00, 0xF, 0xF, true);
+        return bm_dpp<0x00>(v);
     case 1:
-        return (u32)__builtin_amdgcn_mov_dpp((int)v, 0x55, 0xF, 0xF, true);
+        return bm_dpp<0x55>(v);
     case 2:
-        return (u32)__builtin_amdgcn_mov_dpp((int)v, 0xAA, 0xF, 0xF, true);
+        return bm_dpp<0xAA>(v);
     default:
-        return (u32)__builtin_amdgcn_mov_dpp((int)v, 0xFF, 0xF, 0xF, true);
+        return bm_dpp<0xFF>(v);
     }
+}
+
+// Lanes 16..31 <-> 0..15 of each half wave (ds_swizzle bit mode: xor 0x10; goes through the LDS crossbar only).
+__device__ __forceinline__ u32 bm_swap16(u32 v) { return (u32)__builtin_amdgcn_ds_swizzle((int)v, 0x401F); }
+
+// All-reduce over each aligned group of 32 lanes: every lane ends with the group's maximum / sum.
+__device__ __forceinline__ u32 bm_max32(u32 v) {
+    u32 o;
+    o = bm_dpp<kDppXor1>(v), v = o > v ? o : v;
+    o = bm_dpp<kDppXor2>(v), v = o > v ? o : v;
+    o = bm_dpp<kDppHalfMirror>(v), v = o > v ? o : v;
+    o = bm_dpp<kDppMirror>(v), v = o > v ? o : v;
+    o = bm_swap16(v), v = o > v ? o : v;
+    return v;
+}
+__device__ __forceinline__ int bm_sum16(int v) { // over each aligned group of 16 lanes
+    v += (int)bm_dpp<kDppXor1>((u32)v);
+    v += (int)bm_dpp<kDppXor2>((u32)v);
+    v += (int)bm_dpp<kDppHalfMirror>((u32)v);
+    v += (int)bm_dpp<kDppMirror>((u32)v);
+    return v;
 }
 
 // ------------------------------------------------------------------------------------------ fault raising
@@ -112,11 +153,33 @@ __device__ __forceinline__ void bm_raise(u32 *fault, u32 layer, u32 site) {
 // A tap sees the exact integers a core forms. The launchers pass NoTap (everything folds away); the
 // verification kernel passes one that stores them, so it checks the code the launchers run.
 struct NoTap {
+    static constexpr bool kActive = false;
     __device__ __forceinline__ void q4k(int, int, int, int) const {}
     __device__ __forceinline__ void q4k_isum(int, int, int) const {}
     __device__ __forceinline__ void q6k(int, int, int) const {}
     __device__ __forceinline__ void iq2(int, int, int, int) const {}
 };
+
+// ------------------------------------------------------------------------------------------ activation view
+
+// One activation column in LDS (or global memory): its reference bytes and, for the Q8_2_X4 form, the tables.
+struct ActView {
+    const uint8_t *col;
+    const uint8_t *tbl; // nb * 8 pairs (f32 d8, f32 d8 * isum)
+    const uint8_t *s16; // nb * 16 i32 sums of 16 stored codes
+};
+
+// Bytes of one column of nb super-blocks on the device, in the form type WT dots against.
+template <int WT>
+__host__ __device__ constexpr int bm_act_col_bytes(int nb) {
+    return WT == BM_IQ2XXS ? nb * BM_Q8K_STRIDE : nb * BM_Q82_SB_EXT;
+}
+
+template <int WT>
+__device__ __forceinline__ ActView bm_act_view(const uint8_t *col, int nb) {
+    if (WT == BM_IQ2XXS) return ActView{col, nullptr, nullptr};
+    return ActView{col, col + (size_t)nb * BM_Q82_SB_REF, col + (size_t)nb * (BM_Q82_SB_REF + 64)};
+}
 
 // ------------------------------------------------------------------------------------------------- cores
 
@@ -152,61 +215,52 @@ __device__ __forceinline__ void bm_q4_dot16(uint4 q, uint4 alo, uint4 ahi, int &
     hi = bm_sdot4((q.w >> 4) & m, ahi.w, hi);
 }
 
-// One super-block of one column. `col` points at the column's Q8_2_X4 bytes (LDS), `i` is the super-block.
+// One super-block `i` of one column.
 template <class Tap>
-__device__ __forceinline__ void bm_dot_q4k(const Blk<BM_Q4K> &b, const uint8_t *col, int i, int c, int h, float &acc0,
+__device__ __forceinline__ void bm_dot_q4k(const Blk<BM_Q4K> &b, const ActView &av, int i, int c, int h, float &acc0,
                                            float &acc1, const Tap &tap) {
-    const uint8_t *g0 = col + (size_t)(2 * i) * BM_Q82X4_STRIDE;
+    const uint8_t *g0 = av.col + (size_t)(2 * i) * BM_Q82X4_STRIDE;
     const uint8_t *g1 = g0 + BM_Q82X4_STRIDE;
-    const uint4 h0 = *reinterpret_cast<const uint4 *>(g0); // d bf16[4], isum i16[4]
-    const uint4 h1 = *reinterpret_cast<const uint4 *>(g1);
+    const uint8_t *te = av.tbl + (size_t)i * 64;
+    // (d8, d8 * isum) of sub-blocks (2c, 2c + 1), (4 + 2c, 5 + 2c) and of this lane's own pair (4h + 2c, 4h + 2c + 1)
+    const float4 e0 = *reinterpret_cast<const float4 *>(te + 16 * c);
+    const float4 e1 = *reinterpret_cast<const float4 *>(te + 32 + 16 * c);
+    const float4 em = *reinterpret_cast<const float4 *>(te + 32 * h + 16 * c);
     const float d = bm_half_to_f32(b.hdr.x & 0xffffu), dmin = bm_half_to_f32(b.hdr.x >> 16);
     const u32 a0 = b.hdr.y, a1 = b.hdr.z, a2 = b.hdr.w; // crates/qdot/src/lib.rs:3868-3878
-    const u32 sc03 = a0 & 0x3f3f3f3fu, sc47 = (a2 & 0x0f0f0f0fu) | ((a0 >> 2) & 0x30303030u);
-    const u32 mn03 = a1 & 0x3f3f3f3fu, mn47 = ((a2 >> 4) & 0x0f0f0f0fu) | ((a1 >> 2) & 0x30303030u);
-    const int t0 = 2 * c, t1 = 2 * c + 1;
-    // The eight bf16 scales: group 0 holds sub-blocks 0..3, group 1 sub-blocks 4..7.
-    const u32 dw0 = c ? h0.y : h0.x, dw1 = c ? h1.y : h1.x; // scales of sub-blocks (t0, t1) and (4 + t0, 4 + t1)
-    const float d8_0a = bm_bits_f32(dw0 << 16), d8_0b = bm_bits_f32(dw0 & 0xffff0000u);
-    const float d8_1a = bm_bits_f32(dw1 << 16), d8_1b = bm_bits_f32(dw1 & 0xffff0000u);
-    // Min term of accumulators l = 4h + t: sub-block l's scale, sum and 6-bit min (lib.rs:4389-4394).
-    {
-        const u32 dwh = h ? dw1 : dw0;
-        const u32 sw = h ? (c ? h1.w : h1.z) : (c ? h0.w : h0.z);
-        const u32 mnw = h ? mn47 : mn03;
-        const float d8a = bm_bits_f32(dwh << 16), d8b = bm_bits_f32(dwh & 0xffff0000u);
-        const int sa = (int)(short)(sw & 0xffffu), sb = (int)(short)(sw >> 16);
-        const float ma = -(dmin * (float)((mnw >> (8 * t0)) & 0xffu));
-        const float mb = -(dmin * (float)((mnw >> (8 * t1)) & 0xffu));
-        acc0 = fmaf(d8a * (float)sa, ma, acc0);
-        acc1 = fmaf(d8b * (float)sb, mb, acc1);
-        tap.q4k_isum(i, 4 * h + t0, sa);
-        tap.q4k_isum(i, 4 * h + t1, sb);
+    const int sh = 16 * c;                               // this lane's two sub-blocks sit in bytes 2c, 2c + 1
+    const u32 s0 = (a0 & 0x3f3f3f3fu) >> sh;             // scales of sub-blocks 2c, 2c + 1
+    const u32 s1 = ((a2 & 0x0f0f0f0fu) | ((a0 >> 2) & 0x30303030u)) >> sh; // 4 + 2c, 5 + 2c
+    const u32 mw = h ? (((a2 >> 4) & 0x0f0f0f0fu) | ((a1 >> 2) & 0x30303030u)) : (a1 & 0x3f3f3f3fu);
+    const u32 mm = mw >> sh; // mins of sub-blocks 4h + 2c, 4h + 2c + 1
+    // Min term of accumulators l = 4h + t (lib.rs:4389-4394): fma(d8 * isum, -(dmin * m), acc).
+    acc0 = fmaf(em.y, -(dmin * (float)(mm & 0xffu)), acc0);
+    acc1 = fmaf(em.w, -(dmin * (float)((mm >> 8) & 0xffu)), acc1);
+    if constexpr (Tap::kActive) {
+        const u32 sw = *reinterpret_cast<const u32 *>((h ? g1 : g0) + 8 + 4 * c);
+        tap.q4k_isum(i, 4 * h + 2 * c, (int)(short)(sw & 0xffffu));
+        tap.q4k_isum(i, 4 * h + 2 * c + 1, (int)(short)(sw >> 16));
     }
-    // j = 0: sub-blocks t0, t1 (group 0); j = 1: sub-blocks 4 + t0, 4 + t1 (group 1) (lib.rs:4402-4436).
+    // j = 0: sub-blocks 2c, 2c + 1 (group 0); j = 1: 4 + 2c, 5 + 2c (group 1) (lib.rs:4402-4436).
     {
-        const uint4 alo = *reinterpret_cast<const uint4 *>(g0 + 16 + 32 * t0 + 16 * h);
-        const uint4 ahi = *reinterpret_cast<const uint4 *>(g0 + 16 + 32 * t1 + 16 * h);
+        const uint4 alo = *reinterpret_cast<const uint4 *>(g0 + 16 + 64 * c + 16 * h);
+        const uint4 ahi = *reinterpret_cast<const uint4 *>(g0 + 16 + 64 * c + 32 + 16 * h);
         int lo, hi;
         bm_q4_dot16(b.qa, alo, ahi, lo, hi);
-        const float sa = (d * (float)((sc03 >> (8 * t0)) & 0xffu)) * d8_0a;
-        const float sb = (d * (float)((sc03 >> (8 * t1)) & 0xffu)) * d8_0b;
-        acc0 = fmaf(sa, (float)lo, acc0);
-        acc1 = fmaf(sb, (float)hi, acc1);
-        tap.q4k(i, t0, h, lo);
-        tap.q4k(i, t1, h, hi);
+        acc0 = fmaf((d * (float)(s0 & 0xffu)) * e0.x, (float)lo, acc0);
+        acc1 = fmaf((d * (float)((s0 >> 8) & 0xffu)) * e0.z, (float)hi, acc1);
+        tap.q4k(i, 2 * c, h, lo);
+        tap.q4k(i, 2 * c + 1, h, hi);
     }
     {
-        const uint4 alo = *reinterpret_cast<const uint4 *>(g1 + 16 + 32 * t0 + 16 * h);
-        const uint4 ahi = *reinterpret_cast<const uint4 *>(g1 + 16 + 32 * t1 + 16 * h);
+        const uint4 alo = *reinterpret_cast<const uint4 *>(g1 + 16 + 64 * c + 16 * h);
+        const uint4 ahi = *reinterpret_cast<const uint4 *>(g1 + 16 + 64 * c + 32 + 16 * h);
         int lo, hi;
         bm_q4_dot16(b.qb, alo, ahi, lo, hi);
-        const float sa = (d * (float)((sc47 >> (8 * t0)) & 0xffu)) * d8_1a;
-        const float sb = (d * (float)((sc47 >> (8 * t1)) & 0xffu)) * d8_1b;
-        acc0 = fmaf(sa, (float)lo, acc0);
-        acc1 = fmaf(sb, (float)hi, acc1);
-        tap.q4k(i, 4 + t0, h, lo);
-        tap.q4k(i, 4 + t1, h, hi);
+        acc0 = fmaf((d * (float)(s1 & 0xffu)) * e1.x, (float)lo, acc0);
+        acc1 = fmaf((d * (float)((s1 >> 8) & 0xffu)) * e1.z, (float)hi, acc1);
+        tap.q4k(i, 4 + 2 * c, h, lo);
+        tap.q4k(i, 5 + 2 * c, h, hi);
     }
 }
 
@@ -231,50 +285,48 @@ __device__ __forceinline__ Blk<BM_Q6K> bm_load_q6k(const uint8_t *wrow, int i, i
     return b;
 }
 
-// sum (q6 - 32) * a over 16 values: the 6-bit code fits a signed byte, so dot it as is and take 32 * sum a off.
-__device__ __forceinline__ int bm_q6_dot16(uint4 ql, uint4 qh, int nib_shift, int hi_shift, uint4 a) {
-    const u32 ml = 0x0f0f0f0fu, mh = 0x03030303u, ones = 0x01010101u;
-    int s = 0, sa = 0;
-    s = bm_sdot4(((ql.x >> nib_shift) & ml) | (((qh.x >> hi_shift) & mh) << 4), a.x, s);
-    s = bm_sdot4(((ql.y >> nib_shift) & ml) | (((qh.y >> hi_shift) & mh) << 4), a.y, s);
-    s = bm_sdot4(((ql.z >> nib_shift) & ml) | (((qh.z >> hi_shift) & mh) << 4), a.z, s);
-    s = bm_sdot4(((ql.w >> nib_shift) & ml) | (((qh.w >> hi_shift) & mh) << 4), a.w, s);
-    sa = bm_sdot4(ones, a.x, sa);
-    sa = bm_sdot4(ones, a.y, sa);
-    sa = bm_sdot4(ones, a.z, sa);
-    sa = bm_sdot4(ones, a.w, sa);
-    return s - 32 * sa;
+// The two 16-value dots of one half: quarter c (low nibbles, high bits 2c) against aa and quarter c + 2 (high
+// nibbles, high bits 2c + 4) against ab, each sum q6 * a with the 6-bit code taken as it is (it fits a signed byte).
+__device__ __forceinline__ void bm_q6_dot16x2(uint4 ql, uint4 qh, int hs, uint4 aa, uint4 ab, int &s0, int &s1) {
+    const u32 ml = 0x0f0f0f0fu, mh = 0x30303030u;
+    const u32 hx = qh.x >> hs, hy = qh.y >> hs, hz = qh.z >> hs, hw = qh.w >> hs; // this lane's bits at 0..1, 4..5
+    s0 = bm_sdot4((ql.x & ml) | ((hx << 4) & mh), aa.x, 0);
+    s0 = bm_sdot4((ql.y & ml) | ((hy << 4) & mh), aa.y, s0);
+    s0 = bm_sdot4((ql.z & ml) | ((hz << 4) & mh), aa.z, s0);
+    s0 = bm_sdot4((ql.w & ml) | ((hw << 4) & mh), aa.w, s0);
+    s1 = bm_sdot4(((ql.x >> 4) & ml) | (hx & mh), ab.x, 0);
+    s1 = bm_sdot4(((ql.y >> 4) & ml) | (hy & mh), ab.y, s1);
+    s1 = bm_sdot4(((ql.z >> 4) & ml) | (hz & mh), ab.z, s1);
+    s1 = bm_sdot4(((ql.w >> 4) & ml) | (hw & mh), ab.w, s1);
 }
 
 template <class Tap>
-__device__ __forceinline__ void bm_dot_q6k(const Blk<BM_Q6K> &b, const uint8_t *col, int i, int c, int h, float &acc0,
+__device__ __forceinline__ void bm_dot_q6k(const Blk<BM_Q6K> &b, const ActView &av, int i, int c, int h, float &acc0,
                                            float &acc1, const Tap &tap) {
-    const uint8_t *g0 = col + (size_t)(2 * i) * BM_Q82X4_STRIDE;
+    const uint8_t *g0 = av.col + (size_t)(2 * i) * BM_Q82X4_STRIDE;
+    const uint8_t *te = av.tbl + (size_t)i * 64;
+    const int *s16 = reinterpret_cast<const int *>(av.s16 + (size_t)i * 64);
     const float d = bm_half_to_f32(b.d);
-    const int t0 = c, t1 = c + 2;
+    const int bi = 8 * (2 * c + h); // this lane's scale byte inside each word of four
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const uint8_t *g = g0 + j * BM_Q82X4_STRIDE;
-        const uint2 dd = *reinterpret_cast<const uint2 *>(g); // four bf16 scales
-        const u32 dwa = dd.x, dwb = dd.y;                     // sub-blocks (0, 1) and (2, 3) of this half
-        const float d8a = c ? bm_bits_f32(dwa & 0xffff0000u) : bm_bits_f32(dwa << 16); // block t0 = c
-        const float d8b = c ? bm_bits_f32(dwb & 0xffff0000u) : bm_bits_f32(dwb << 16); // block t1 = c + 2
-        const uint4 aa = *reinterpret_cast<const uint4 *>(g + 16 + 32 * t0 + 16 * h);
-        const uint4 ab = *reinterpret_cast<const uint4 *>(g + 16 + 32 * t1 + 16 * h);
-        const uint4 ql = j ? b.ql1 : b.ql0, qh = j ? b.qh1 : b.qh0;
-        const int s0 = bm_q6_dot16(ql, qh, 0, 2 * c, aa);
-        const int s1 = bm_q6_dot16(ql, qh, 4, 2 * c + 4, ab);
-        // scale byte 8j + 2t + h (crates/qdot/src/lib.rs:4455 K_SHUFFLE_Q6K, :4794-4809)
-        const u32 w01 = j ? b.sc.z : b.sc.x, w23 = j ? b.sc.w : b.sc.y; // scale bytes 8j + 0..3 and 8j + 4..7
-        const int i0 = 2 * t0 + h, i1 = 2 * t1 + h;                     // byte index inside the half: 0..7
-        const int sc0 = (int)(signed char)(((i0 < 4 ? w01 : w23) >> (8 * (i0 & 3))) & 0xffu);
-        const int sc1 = (int)(signed char)(((i1 < 4 ? w01 : w23) >> (8 * (i1 & 3))) & 0xffu);
-        const float f0 = (d * (float)sc0) * d8a;
-        const float f1 = (d * (float)sc1) * d8b;
-        acc0 = fmaf(f0, (float)s0, acc0);
-        acc1 = fmaf(f1, (float)s1, acc1);
-        tap.q6k(i, 8 * j + i0, s0);
-        tap.q6k(i, 8 * j + i1, s1);
+        const float d8a = *reinterpret_cast<const float *>(te + 8 * (4 * j + c));     // 32-block c of this half
+        const float d8b = *reinterpret_cast<const float *>(te + 8 * (4 * j + c + 2)); // 32-block c + 2
+        const int sa = s16[2 * (4 * j + c) + h], sb = s16[2 * (4 * j + c + 2) + h];   // sum of the 16 codes dotted
+        const uint4 aa = *reinterpret_cast<const uint4 *>(g + 16 + 32 * c + 16 * h);
+        const uint4 ab = *reinterpret_cast<const uint4 *>(g + 16 + 32 * (c + 2) + 16 * h);
+        int s0, s1;
+        bm_q6_dot16x2(j ? b.ql1 : b.ql0, j ? b.qh1 : b.qh0, 2 * c, aa, ab, s0, s1);
+        s0 -= 32 * sa; // sum (q6 - 32) * a
+        s1 -= 32 * sb;
+        // scale bytes 8j + 2c + h and 8j + 4 + 2c + h (crates/qdot/src/lib.rs:4455 K_SHUFFLE_Q6K, :4794-4809)
+        const int sc0 = __builtin_amdgcn_sbfe((int)(j ? b.sc.z : b.sc.x), bi, 8);
+        const int sc1 = __builtin_amdgcn_sbfe((int)(j ? b.sc.w : b.sc.y), bi, 8);
+        acc0 = fmaf((d * (float)sc0) * d8a, (float)s0, acc0);
+        acc1 = fmaf((d * (float)sc1) * d8b, (float)s1, acc1);
+        tap.q6k(i, 8 * j + 2 * c + h, s0);
+        tap.q6k(i, 8 * j + 4 + 2 * c + h, s1);
     }
 }
 
@@ -303,9 +355,9 @@ struct Iq2Tables {
 };
 
 template <class Tap>
-__device__ __forceinline__ void bm_dot_iq2xxs(const Blk<BM_IQ2XXS> &b, const uint8_t *col, int i, int q,
+__device__ __forceinline__ void bm_dot_iq2xxs(const Blk<BM_IQ2XXS> &b, const ActView &av, int i, int q,
                                               const Iq2Tables &tb, float &acc0, float &acc1, const Tap &tap) {
-    const uint8_t *blk = col + (size_t)i * BM_Q8K_STRIDE;
+    const uint8_t *blk = av.col + (size_t)i * BM_Q8K_STRIDE;
     const float dy = *reinterpret_cast<const float *>(blk);
     const float d = 0.125f * bm_half_to_f32(b.d);
     const float dmin = -d * 43.0f;
@@ -382,25 +434,19 @@ __device__ __forceinline__ Blk<BM_IQ2XXS> bm_load_blk<BM_IQ2XXS>(const uint8_t *
 }
 
 template <int WT, class Tap>
-__device__ __forceinline__ void bm_dot_blk(const Blk<WT> &b, const uint8_t *col, int i, int q, const Iq2Tables &tb,
+__device__ __forceinline__ void bm_dot_blk(const Blk<WT> &b, const ActView &av, int i, int q, const Iq2Tables &tb,
                                            float &acc0, float &acc1, const Tap &tap) {
     if constexpr (WT == BM_Q4K)
-        bm_dot_q4k(b, col, i, q & 1, q >> 1, acc0, acc1, tap);
+        bm_dot_q4k(b, av, i, q & 1, q >> 1, acc0, acc1, tap);
     else if constexpr (WT == BM_Q6K)
-        bm_dot_q6k(b, col, i, q & 1, q >> 1, acc0, acc1, tap);
+        bm_dot_q6k(b, av, i, q & 1, q >> 1, acc0, acc1, tap);
     else
-        bm_dot_iq2xxs(b, col, i, q, tb, acc0, acc1, tap);
+        bm_dot_iq2xxs(b, av, i, q, tb, acc0, acc1, tap);
 }
 
 template <int WT>
 __host__ __device__ constexpr int bm_block_bytes() {
     return WT == BM_Q4K ? BM_Q4K_BLOCK : (WT == BM_Q6K ? BM_Q6K_BLOCK : BM_IQ2XXS_BLOCK);
-}
-
-// Bytes of one activation super-block (256 values) in the form type WT dots against.
-template <int WT>
-__host__ __device__ constexpr int bm_act_sb_bytes() {
-    return WT == BM_IQ2XXS ? BM_Q8K_STRIDE : 2 * BM_Q82X4_STRIDE;
 }
 
 // ---- SwiGLU: crates/qdot/src/lib.rs:3741-3773 (expf) and :11467-11478 (divide, then multiply).

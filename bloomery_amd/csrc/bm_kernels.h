@@ -19,7 +19,14 @@ constexpr int kMaxLds = 160 * 1024;
 
 hipError_t fill_u32(const Launch &L, uint32_t *dst, uint32_t value, size_t n);
 
+// Bytes of one activation column of k values on the device, in the form weight type `wtype` dots against: the CPU
+// path's bytes, and for the Q8_2_X4 form two tables after them (bm_device.cuh).
+int act_col_bytes(int wtype, int k);
+
 hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, uint8_t *act);
+
+// Rebuilds the tables of m Q8_2_X4 device columns whose reference bytes were just written by a copy.
+hipError_t q82_tables(const Launch &L, uint8_t *act, int m, int k);
 
 // Columns that fit one gemv launch's LDS for this type and k (at most 8).
 int gemv_max_cols(int wtype, int k);
@@ -41,6 +48,23 @@ constexpr int kMaxCombineSlots = 64;
 hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const uint8_t *act,
                         const uint32_t *sel, const float *wts, const float *resid, int slots_per_token, int m,
                         int rows_per_expert, float *y);
+
+// The whole decode step: quantize x, gate . up . SwiGLU, quantize h, down, weighted slot sum.
+//   kPlanOneLaunch:   one launch; the down workgroups stream their rows while gate . up runs and wait on device
+//                     counters (`counters`: m + 1 zeroed words, left zeroed; spin_limit bounds the wait);
+//   kPlanTwoLaunches: gate . up with the quantizers folded in, then down + combine (no counters).
+constexpr int kPlanOneLaunch = 1, kPlanTwoLaunches = 2;
+constexpr int kMaxDecodeTokens = 1024;
+bool moe_decode_supported(int gate_type, int down_type);
+// gate . up . SwiGLU from f32 token rows, both quantizers folded in (Q4_K gate/up): the first launch of
+// kPlanTwoLaunches.
+hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8_t *wg, const uint8_t *wu,
+                     int n_experts, int hidden, int ff, const uint32_t *sel, int slots_per_token, int m,
+                     uint8_t *act_x, uint8_t *act_h, float *h);
+hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, const float *x, const uint8_t *wg,
+                      const uint8_t *wu, const uint8_t *wd, int n_experts, int hidden, int ff, const uint32_t *sel,
+                      const float *wts, const float *resid, int slots_per_token, int m, uint8_t *act_x,
+                      uint8_t *act_h, float *h, float *y, uint32_t *counters, uint32_t spin_limit);
 
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out);
 

@@ -20,6 +20,7 @@ namespace bmk {
 
 constexpr u32 kSiteQuantColumn = 1; // crates/device/src/fault.rs:73-76
 constexpr u32 kSiteExpertId = 7;    // crates/device/src/fault.rs:89
+constexpr u32 kSiteStalled = 31;    // ours: a fused launch's down workgroup gave up waiting for its activations
 
 // LDS bytes of the IQ2_XXS tables: 2048 grid + 128 signs + 64 nibble masks, padded to a 16-byte multiple.
 constexpr int kTabBytes = 2048 + 128 + 64 + 64;
@@ -99,24 +100,27 @@ template <int WT, int U, int NB, int M, class Tap>
 __device__ __forceinline__ void row_dot(Blk<WT> (&b)[U], const uint8_t *wrow, const uint8_t *cols, int col_stride,
                                         int m, int nb, int q, const Iq2Tables &tb, float (&out)[M], const Tap &tap) {
     float a0[M], a1[M];
+    ActView av[M];
+    const int n = NB > 0 ? NB : nb;
 #pragma unroll
-    for (int c = 0; c < M; c++) a0[c] = a1[c] = 0.0f;
+    for (int c = 0; c < M; c++) {
+        a0[c] = a1[c] = 0.0f;
+        av[c] = bm_act_view<WT>(cols + (size_t)c * col_stride, n);
+    }
     if constexpr (NB == U) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
 #pragma unroll
             for (int c = 0; c < M; c++)
-                if (M == 1 || c < m) bm_dot_blk<WT>(b[u], cols + (size_t)c * col_stride, u, q, tb, a0[c], a1[c], tap);
+                if (M == 1 || c < m) bm_dot_blk<WT>(b[u], av[c], u, q, tb, a0[c], a1[c], tap);
         }
     } else {
-        const int n = NB > 0 ? NB : nb;
         for (int i0 = 0;;) {
 #pragma unroll
             for (int u = 0; u < U; u++) {
 #pragma unroll
                 for (int c = 0; c < M; c++)
-                    if (M == 1 || c < m)
-                        bm_dot_blk<WT>(b[u], cols + (size_t)c * col_stride, i0 + u, q, tb, a0[c], a1[c], tap);
+                    if (M == 1 || c < m) bm_dot_blk<WT>(b[u], av[c], i0 + u, q, tb, a0[c], a1[c], tap);
             }
             i0 += U;
             if (i0 >= n) break;
@@ -143,46 +147,55 @@ hipError_t fill_u32(const Launch &L, uint32_t *dst, uint32_t value, size_t n) {
 
 // ------------------------------------------------------------------------------------------- quantizers
 
-// One 32-value q8_2 block on the 32 lanes of a half wave (crates/qdot/src/lib.rs:3883-3904).
-// Returns the code; *t_out / *isum_out are valid on every lane. `bad` reports a value that is not finite.
-__device__ __forceinline__ int q82_block(float v, u32 *t_out, int *isum_out, bool *bad) {
-    u32 ab = bm_f32_bits(v) & 0x7fffffffu;
-#pragma unroll
-    for (int s = 16; s >= 1; s >>= 1) {
-        u32 o = (u32)__shfl_xor((int)ab, s, 32);
-        ab = o > ab ? o : ab;
-    }
+// What one q8_2 block's header needs beside its codes.
+struct Q82Head {
+    u32 t;    // bf16 scale bits
+    int isum; // sum of the unsaturated codes
+    bool bad; // a value that is not finite: NaN scale, zero codes (crates/gpu/src/lib.rs:925-933)
+};
+
+// One 32-value q8_2 block on an aligned group of 32 lanes, a value a lane (crates/qdot/src/lib.rs:3883-3904).
+// Returns the stored code; *s16 is the sum of the stored codes over the lane's aligned group of 16.
+__device__ __forceinline__ int q82_block(float v, Q82Head *hd, int *s16) {
+    const u32 ab = bm_max32(bm_f32_bits(v) & 0x7fffffffu);
     if (ab > 0x7f7fffffu) {
-        *bad = true;
-        *t_out = 0x7fc0u; // a NaN scale, zero codes (crates/gpu/src/lib.rs:925-933)
-        *isum_out = 0;
+        hd->t = 0x7fc0u;
+        hd->isum = 0;
+        hd->bad = true;
+        *s16 = 0;
         return 0;
     }
-    *bad = false;
-    const float amax = bm_bits_f32(ab);
-    const u32 t = bm_fp32_to_bf16_bits(__fdiv_rn(amax, 127.0f));
+    const u32 t = bm_fp32_to_bf16_bits(__fdiv_rn(bm_bits_f32(ab), 127.0f));
     const float id = bm_q82_inverse(t);
     const int q = bm_nearest_int(__fmul_rn(v, id));
-    int isum = q;
-#pragma unroll
-    for (int s = 16; s >= 1; s >>= 1) isum += __shfl_xor(isum, s, 32);
-    *t_out = t;
-    *isum_out = isum;
-    return q < -128 ? -128 : (q > 127 ? 127 : q);
+    const int code = q < -128 ? -128 : (q > 127 ? 127 : q);
+    const int s = bm_sum16(q);
+    hd->t = t;
+    hd->isum = s + (int)bm_swap16((u32)s);
+    hd->bad = false;
+    *s16 = bm_sum16(code);
+    return code;
 }
 
-// Stores one q8_2 block (its 32 codes, scale and sum) into a column's Q8_2_X4 bytes.
-__device__ __forceinline__ void q82_store(uint8_t *col, int blk, int lane32, int code, u32 t, int isum) {
+// Stores block `blk` of a device Q8_2_X4 column of nb super-blocks: codes, scale, sum and the two table entries.
+// Called by the block's 32 lanes with their `lane32`.
+__device__ __forceinline__ void q82_store(uint8_t *col, int nb, int blk, int lane32, int code, const Q82Head &hd,
+                                          int s16) {
     uint8_t *group = col + (size_t)(blk >> 2) * BM_Q82X4_STRIDE;
     const int ir = blk & 3;
     // four codes a lane-quad -> one dword store from its first lane
     u32 c = (u32)(code & 0xff);
-    c |= (u32)(__shfl_down((int)c, 1, 32) & 0xff) << 8;
-    c |= (u32)(__shfl_down((int)c, 2, 32) & 0xffff) << 16;
+    c |= (bm_dpp<kDppShl1>(c) & 0xffu) << 8;
+    c |= (bm_dpp<kDppShl2>(c) & 0xffffu) << 16;
     if ((lane32 & 3) == 0) *reinterpret_cast<u32 *>(group + 16 + 32 * ir + lane32) = c;
+    if ((lane32 & 15) == 0)
+        *reinterpret_cast<int *>(col + (size_t)nb * (BM_Q82_SB_REF + 64) + 4 * (2 * blk + (lane32 >> 4))) = s16;
     if (lane32 == 0) {
-        *reinterpret_cast<unsigned short *>(group + 2 * ir) = (unsigned short)t;
-        *reinterpret_cast<unsigned short *>(group + 8 + 2 * ir) = (unsigned short)(short)isum;
+        *reinterpret_cast<unsigned short *>(group + 2 * ir) = (unsigned short)hd.t;
+        *reinterpret_cast<unsigned short *>(group + 8 + 2 * ir) = (unsigned short)(short)hd.isum;
+        const float d8 = bm_bf16_to_f32(hd.t);
+        *reinterpret_cast<float2 *>(col + (size_t)nb * BM_Q82_SB_REF + 8 * blk) =
+            make_float2(d8, __fmul_rn(d8, (float)(short)hd.isum));
     }
 }
 
@@ -194,12 +207,11 @@ __global__ __launch_bounds__(256) void k_quantize_q82x4(const float *x, int m, i
     if (gblk >= (long)m * bpc) return;
     const int col = (int)(gblk / bpc), blk = (int)(gblk % bpc), lane32 = threadIdx.x & 31;
     const float v = x[(size_t)col * k + 32 * blk + lane32];
-    u32 t;
-    int isum;
-    bool bad;
-    const int code = q82_block(v, &t, &isum, &bad);
-    if (bad && lane32 == 0) bm_raise(fault, layer, kSiteQuantColumn);
-    q82_store(act + (size_t)col * (k / 128) * BM_Q82X4_STRIDE, blk, lane32, code, t, isum);
+    Q82Head hd;
+    int s16;
+    const int code = q82_block(v, &hd, &s16);
+    if (hd.bad && lane32 == 0) bm_raise(fault, layer, kSiteQuantColumn);
+    q82_store(act + (size_t)col * (k / 256) * BM_Q82_SB_EXT, k / 256, blk, lane32, code, hd, s16);
 }
 
 // x: m columns of k values -> Q8_K columns (crates/qdot/src/lib.rs:1787-1809). One workgroup a 256-value block.
@@ -270,6 +282,31 @@ hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, ui
     return hipGetLastError();
 }
 
+// Fills the two tables of `m` device Q8_2_X4 columns from their reference bytes (after an upload of those bytes).
+__global__ __launch_bounds__(256) void k_q82_tables(uint8_t *act, int m, int nb) {
+    const long g = (long)blockIdx.x * blockDim.x + threadIdx.x; // one 16-value group a thread
+    if (g >= (long)m * nb * 16) return;
+    const int col = (int)(g / (nb * 16)), g16 = (int)(g % (nb * 16)), blk = g16 >> 1, half = g16 & 1;
+    uint8_t *c = act + (size_t)col * nb * BM_Q82_SB_EXT;
+    const uint8_t *group = c + (size_t)(blk >> 2) * BM_Q82X4_STRIDE;
+    const signed char *codes = reinterpret_cast<const signed char *>(group + 16 + 32 * (blk & 3) + 16 * half);
+    int s = 0;
+    for (int n = 0; n < 16; n++) s += codes[n];
+    *reinterpret_cast<int *>(c + (size_t)nb * (BM_Q82_SB_REF + 64) + 4 * g16) = s;
+    if (half == 0) {
+        const float d8 = bm_bf16_to_f32(*reinterpret_cast<const unsigned short *>(group + 2 * (blk & 3)));
+        const int isum = *reinterpret_cast<const short *>(group + 8 + 2 * (blk & 3));
+        *reinterpret_cast<float2 *>(c + (size_t)nb * BM_Q82_SB_REF + 8 * blk) = make_float2(d8, __fmul_rn(d8, (float)isum));
+    }
+}
+
+hipError_t q82_tables(const Launch &L, uint8_t *act, int m, int k) {
+    const int nb = k / 256;
+    const long n = (long)m * nb * 16;
+    hipLaunchKernelGGL(k_q82_tables, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, L.stream, act, m, nb);
+    return hipGetLastError();
+}
+
 // ------------------------------------------------------------------------------------------------ gemv
 
 // y[row * m_total + col0 + c] = row . column (col0 + c), c < m <= 8. A quad a row, 64 rows a workgroup.
@@ -282,7 +319,7 @@ __global__ __launch_bounds__(256) void k_gemv(const uint8_t *w, long rows, int n
     const bool active = row < rows;
     const int n = NB > 0 ? NB : nb;
     const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
-    const int col_bytes = n * bm_act_sb_bytes<WT>();
+    const int col_bytes = bm_act_col_bytes<WT>(n);
     const uint8_t *wrow = w + (size_t)(active ? row : 0) * row_bytes;
     Blk<WT> b[U];
     preload<WT, U>(b, wrow, q);
@@ -301,6 +338,23 @@ __global__ __launch_bounds__(256) void k_gemv(const uint8_t *w, long rows, int n
 
 // --------------------------------------------------------------------------------- gate . up . SwiGLU
 
+// The gate/up exchange of the eight lanes of an output: lanes 0..3 hold the gate dot, 4..7 the up dot.
+__device__ __forceinline__ float swiglu_of_pair(float v, int which) {
+    // both moves run on every lane: a lane-crossing move under a divergent branch reads switched-off lanes as 0
+    const float from_above = bm_dppf<kDppShl4>(v), from_below = bm_dppf<kDppShr4>(v);
+    return bm_swiglu(which ? from_below : v, which ? v : from_above);
+}
+
+// The 32 values a workgroup produced (hbuf, LDS) as block `rb` of column `hcol`, by the first 32 threads.
+__device__ __forceinline__ void quantize_h_block(const float *hbuf, uint8_t *hcol, int nb_h, int rb, int tid,
+                                                 u32 *fault, u32 layer) {
+    Q82Head hd;
+    int s16;
+    const int code = q82_block(hbuf[tid], &hd, &s16);
+    if (hd.bad && tid == 0) bm_raise(fault, layer, kSiteQuantColumn);
+    q82_store(hcol, nb_h, rb, tid, code, hd, s16);
+}
+
 // One workgroup = 32 consecutive rows of one slot; eight lanes a row: a quad on the gate row, a quad on the up row.
 // With act_h the 32 values are quantized to one q8_2 block of the slot's down activation in the same launch.
 template <int WT, int U, int NB>
@@ -315,15 +369,16 @@ __global__ __launch_bounds__(256) void k_gate_up(const uint8_t *wg, const uint8_
     const bool active = r < rpe;
     const u32 id = sel[slot];
     const int n = NB > 0 ? NB : nb;
-    const int h_col_bytes = (rpe / 128) * BM_Q82X4_STRIDE;
-    const int col_bytes = n * bm_act_sb_bytes<WT>();
+    const int nb_h = rpe / 256;
+    const int col_bytes = bm_act_col_bytes<WT>(n);
     const uint8_t *act_col = act + (size_t)(slot / slots_per_col) * col_bytes;
+    uint8_t *hcol = act_h ? act_h + (size_t)slot * nb_h * BM_Q82_SB_EXT : nullptr;
     Stage<2> st;
     st.load(act_col, col_bytes);
     if (id >= n_experts) { // uniform over the workgroup: no weight is read (crates/gpu/src/kquant/sel.rs:22-28)
         if (tid == 0) bm_raise(fault, layer, kSiteExpertId);
         if (h && active && (tid & 7) == 0) h[(size_t)slot * rpe + r] = bm_bits_f32(0x7fc00000u);
-        if (act_h && tid < 32) q82_store(act_h + (size_t)slot * h_col_bytes, rb, tid, 0, 0x7fc0u, 0);
+        if (act_h && tid < 32) q82_store(hcol, nb_h, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);
         return;
     }
     const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
@@ -336,21 +391,13 @@ __global__ __launch_bounds__(256) void k_gate_up(const uint8_t *wg, const uint8_
     __syncthreads();
     float v[1];
     row_dot<WT, U, NB, 1>(b, wrow, col, col_bytes, 1, n, q, tb, v, NoTap{});
-    const float other = __shfl_xor(v[0], 4, 64);
-    const float hv = bm_swiglu(which ? other : v[0], which ? v[0] : other);
+    const float hv = swiglu_of_pair(v[0], which);
     if (h && active && (tid & 7) == 0) h[(size_t)slot * rpe + r] = hv;
     if (act_h) { // rpe is a multiple of 256 here, so every row of the block is live
         float *hbuf = reinterpret_cast<float *>(col + col_bytes);
         if ((tid & 7) == 0) hbuf[tid >> 3] = hv;
         __syncthreads();
-        if (tid < 32) {
-            u32 t;
-            int isum;
-            bool bad;
-            const int code = q82_block(hbuf[tid], &t, &isum, &bad);
-            if (bad && tid == 0) bm_raise(fault, layer, kSiteQuantColumn);
-            q82_store(act_h + (size_t)slot * h_col_bytes, rb, tid, code, t, isum);
-        }
+        if (tid < 32) quantize_h_block(hbuf, hcol, nb_h, rb, tid, fault, layer);
     }
 }
 
@@ -368,7 +415,7 @@ __global__ __launch_bounds__(256) void k_gemv_sel(const uint8_t *w, u32 n_expert
     const bool active = r < rpe;
     const u32 id = sel[slot];
     const int n = NB > 0 ? NB : nb;
-    const int col_bytes = n * bm_act_sb_bytes<WT>();
+    const int col_bytes = bm_act_col_bytes<WT>(n);
     const uint8_t *act_col = act + (size_t)slot * col_bytes;
     Stage<2> st;
     st.load(act_col, col_bytes);
@@ -413,17 +460,15 @@ hipError_t combine_tokens(const Launch &L, const float *down, const float *w, co
 
 // --------------------------------------------------------------------------- down + combine in one launch
 
-// One workgroup = one token and D = 64 / slots_per_token output rows: a quad for every (row, slot). The slot values
-// meet in LDS and one thread a row folds them in slot order, then adds the residual.
-template <int WT, int U, int NB>
-__global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_experts, int nb, const uint8_t *act,
-                                                      const u32 *sel, const float *wts, const float *resid, int spt,
-                                                      int rpe, float *y, u32 *fault, u32 layer) {
-    extern __shared__ __align__(16) uint8_t lds[];
+// The shared body of the down + combine workgroup: token t, output rows rb * D .. + D with D = 64 / spt, a quad for
+// every (row, slot). `wait` runs after the weight requests and before the activation columns are read.
+template <int WT, int U, int NB, class Wait>
+__device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w, u32 n_experts, int nb,
+                                                  const uint8_t *act, const u32 *sel, const float *wts,
+                                                  const float *resid, int spt, int rpe, float *y, int t, int rb,
+                                                  u32 *fault, u32 layer, const Wait &wait) {
     const int tid = threadIdx.x, q = tid & 3, quad = tid >> 2;
     const int D = 64 / spt;
-    const int blocks_per_token = (rpe + D - 1) / D;
-    const int t = blockIdx.x / blocks_per_token, rb = blockIdx.x % blocks_per_token;
     const int e = quad % spt, dl = quad / spt;
     const int r = rb * D + dl;
     const int slot = t * spt + e;
@@ -437,19 +482,26 @@ __global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_ex
     if (!live && id != 0xffffffffu && rb == 0 && dl == 0 && q == 0) bm_raise(fault, layer, kSiteExpertId);
     const int n = NB > 0 ? NB : nb;
     const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
-    const int col_bytes = n * bm_act_sb_bytes<WT>();
+    const int col_bytes = bm_act_col_bytes<WT>(n);
     const uint8_t *act_cols = act + (size_t)t * spt * col_bytes;
-    Stage<4> st;
-    st.load(act_cols, spt * col_bytes);
     const uint8_t *wrow = w + ((size_t)(live ? id : 0) * rpe + (active ? r : 0)) * row_bytes;
-    Blk<WT> b[U];
-    preload<WT, U>(b, wrow, q);
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *cols = lds + tab_bytes<WT>();
-    st.store(cols, act_cols, spt * col_bytes);
     float *part = reinterpret_cast<float *>(cols + (size_t)spt * col_bytes); // [D][spt]
     float *s_w = part + D * spt;                                              // [spt]
     u32 *s_sel = reinterpret_cast<u32 *>(s_w + spt);                          // [spt]
+    Blk<WT> b[U];
+    if constexpr (Wait::kWaits) {
+        // the rows do not depend on the activations: request them, then wait for the producers
+        preload<WT, U>(b, wrow, q);
+        wait();
+        stage_bytes(cols, act_cols, spt * col_bytes);
+    } else {
+        Stage<5> st;
+        st.load(act_cols, spt * col_bytes);
+        preload<WT, U>(b, wrow, q);
+        st.store(cols, act_cols, spt * col_bytes);
+    }
     if (tid < spt) {
         s_w[tid] = my_w;
         s_sel[tid] = my_sel;
@@ -468,9 +520,220 @@ __global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_ex
     }
 }
 
+struct NoWait {
+    static constexpr bool kWaits = false;
+    __device__ __forceinline__ void operator()() const {}
+};
+
+template <int WT, int U, int NB>
+__global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_experts, int nb, const uint8_t *act,
+                                                      const u32 *sel, const float *wts, const float *resid, int spt,
+                                                      int rpe, float *y, u32 *fault, u32 layer) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int D = 64 / spt;
+    const int blocks_per_token = (rpe + D - 1) / D;
+    down_combine_body<WT, U, NB>(lds, w, n_experts, nb, act, sel, wts, resid, spt, rpe, y,
+                                 blockIdx.x / blocks_per_token, blockIdx.x % blocks_per_token, fault, layer, NoWait{});
+}
+
+// ------------------------------------------------------------------------- the whole layer step, one launch
+
+// Waits until the token's gate.up workgroups have all published their activation blocks.
+struct CounterWait {
+    static constexpr bool kWaits = true;
+    u32 *counter;
+    u32 need, spin_limit;
+    u32 *fault;
+    u32 layer;
+    __device__ __forceinline__ void operator()() const {
+        if (threadIdx.x == 0) {
+            u32 spins = 0;
+            // relaxed polls (an acquiring poll would invalidate the caches on every turn); one fence afterwards
+            while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) {
+                __builtin_amdgcn_s_sleep(2);
+                if (++spins > spin_limit) { // every wave leaves: the launch ends with a fault, never a hang
+                    bm_raise(fault, layer, kSiteStalled);
+                    break;
+                }
+            }
+        }
+        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    }
+};
+
+// One 32-value q8_2 block held eight values a lane by four consecutive lanes (the in-kernel token quantizer).
+__device__ __forceinline__ void q82_quad8(const float (&v)[8], uint8_t *col, int nb, int blk, int lane4, u32 *fault,
+                                          u32 layer) {
+    u32 ab = 0;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const u32 a = bm_f32_bits(v[k]) & 0x7fffffffu;
+        ab = a > ab ? a : ab;
+    }
+    u32 o;
+    o = bm_dpp<kDppXor1>(ab), ab = o > ab ? o : ab;
+    o = bm_dpp<kDppXor2>(ab), ab = o > ab ? o : ab;
+    uint8_t *group = col + (size_t)(blk >> 2) * BM_Q82X4_STRIDE;
+    const int ir = blk & 3;
+    u32 t;
+    int isum = 0, csum = 0;
+    u32 c0 = 0, c1 = 0;
+    if (ab > 0x7f7fffffu) {
+        t = 0x7fc0u;
+        if (lane4 == 0) bm_raise(fault, layer, kSiteQuantColumn);
+    } else {
+        t = bm_fp32_to_bf16_bits(__fdiv_rn(bm_bits_f32(ab), 127.0f));
+        const float id = bm_q82_inverse(t);
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int qv = bm_nearest_int(__fmul_rn(v[k], id));
+            const int code = qv < -128 ? -128 : (qv > 127 ? 127 : qv);
+            isum += qv;
+            csum += code;
+            if (k < 4)
+                c0 |= (u32)(code & 0xff) << (8 * k);
+            else
+                c1 |= (u32)(code & 0xff) << (8 * (k - 4));
+        }
+    }
+    isum += (int)bm_dpp<kDppXor1>((u32)isum);
+    isum += (int)bm_dpp<kDppXor2>((u32)isum);
+    csum += (int)bm_dpp<kDppXor1>((u32)csum); // lanes (0,1): first 16 values, lanes (2,3): second
+    *reinterpret_cast<uint2 *>(group + 16 + 32 * ir + 8 * lane4) = make_uint2(c0, c1);
+    if ((lane4 & 1) == 0)
+        *reinterpret_cast<int *>(col + (size_t)nb * (BM_Q82_SB_REF + 64) + 4 * (2 * blk + (lane4 >> 1))) = csum;
+    if (lane4 == 0) {
+        *reinterpret_cast<unsigned short *>(group + 2 * ir) = (unsigned short)t;
+        *reinterpret_cast<unsigned short *>(group + 8 + 2 * ir) = (unsigned short)(short)isum;
+        const float d8 = bm_bf16_to_f32(t);
+        *reinterpret_cast<float2 *>(col + (size_t)nb * BM_Q82_SB_REF + 8 * blk) =
+            make_float2(d8, __fmul_rn(d8, (float)(short)isum));
+    }
+}
+
+// The gate . up . SwiGLU workgroup of the fused step: as k_gate_up's, except that it quantizes its token's f32 row
+// itself (into LDS; no quantizer launch, no activation column in memory) and always writes its q8_2 block of the
+// slot's down activation.
+template <int WA, int UA, int NBA>
+__device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, const uint8_t *wg, const uint8_t *wu,
+                                               u32 n_experts, int na, int nh, const u32 *sel, int spt, uint8_t *act_x,
+                                               uint8_t *act_h, float *h, int slot, int rb, u32 *fault, u32 layer) {
+    const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
+    const int hidden = na * 256, ff = nh * 256;
+    const int t = slot / spt;
+    const int r = rb * 32 + (tid >> 3);
+    const u32 id = sel[slot];
+    const int col_bytes = bm_act_col_bytes<WA>(na);
+    uint8_t *hcol = act_h + (size_t)slot * nh * BM_Q82_SB_EXT;
+    uint8_t *col = lds;
+    // the token's row: eight consecutive values a lane, 2048 a pass
+    constexpr int kPasses = NBA > 0 ? (NBA * 256 + 2047) / 2048 : 1;
+    float xv[kPasses][8];
+#pragma unroll
+    for (int p = 0; p < kPasses; p++) {
+        int o = p * 2048 + tid * 8;
+        o = o < hidden ? o : hidden - 8;
+        const float4 lo = *reinterpret_cast<const float4 *>(x + (size_t)t * hidden + o);
+        const float4 hi = *reinterpret_cast<const float4 *>(x + (size_t)t * hidden + o + 4);
+        xv[p][0] = lo.x, xv[p][1] = lo.y, xv[p][2] = lo.z, xv[p][3] = lo.w;
+        xv[p][4] = hi.x, xv[p][5] = hi.y, xv[p][6] = hi.z, xv[p][7] = hi.w;
+    }
+    __asm__ volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    if (id >= n_experts) { // uniform over the workgroup
+        if (tid == 0) bm_raise(fault, layer, kSiteExpertId);
+        if (h && (tid & 7) == 0) h[(size_t)slot * ff + r] = bm_bits_f32(0x7fc00000u);
+        if (tid < 32) q82_store(hcol, nh, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);
+        return;
+    }
+    const size_t row_bytes = (size_t)na * bm_block_bytes<WA>();
+    const uint8_t *wrow = (which ? wu : wg) + ((size_t)id * ff + r) * row_bytes;
+    Blk<WA> b[UA];
+    preload<WA, UA>(b, wrow, q);
+#pragma unroll
+    for (int p = 0; p < kPasses; p++) {
+        const int o = p * 2048 + tid * 8;
+        if (o < hidden) q82_quad8(xv[p], col, na, o >> 5, tid & 3, fault, layer);
+    }
+    if constexpr (NBA == 0) { // longer rows: the passes past the first, straight from memory
+        for (int o = 2048 + tid * 8; o < hidden; o += 2048) {
+            float v8[8];
+            for (int k = 0; k < 8; k++) v8[k] = x[(size_t)t * hidden + o + k];
+            q82_quad8(v8, col, na, o >> 5, tid & 3, fault, layer);
+        }
+    }
+    __syncthreads();
+    if (act_x && rb == 0 && slot % spt == 0) stage_bytes(act_x + (size_t)t * col_bytes, col, col_bytes);
+    float v[1];
+    row_dot<WA, UA, NBA, 1>(b, wrow, col, col_bytes, 1, na, q, Iq2Tables{}, v, NoTap{});
+    const float hv = swiglu_of_pair(v[0], which);
+    if (h && (tid & 7) == 0) h[(size_t)slot * ff + r] = hv;
+    float *hbuf = reinterpret_cast<float *>(col + col_bytes);
+    if ((tid & 7) == 0) hbuf[tid >> 3] = hv;
+    __syncthreads();
+    if (tid < 32) quantize_h_block(hbuf, hcol, nh, rb, tid, fault, layer);
+}
+
+// The first half of the fused step as a launch of its own: x -> quantized h, slot by slot.
+template <int WA, int UA, int NBA>
+__global__ __launch_bounds__(256) void k_gate_up_x(const float *x, const uint8_t *wg, const uint8_t *wu, u32 n_experts,
+                                                   int nba, int nh, const u32 *sel, int spt, uint8_t *act_x,
+                                                   uint8_t *act_h, float *h, u32 *fault, u32 layer) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int blocks_per_slot = nh * 8;
+    gate_up_x_body<WA, UA, NBA>(lds, x, wg, wu, n_experts, NBA > 0 ? NBA : nba, nh, sel, spt, act_x, act_h, h,
+                                blockIdx.x / blocks_per_slot, blockIdx.x % blocks_per_slot, fault, layer);
+}
+
+// The decode step of one MoE layer for m tokens in one launch. The first n_a workgroups are the gate . up ones
+// above; once its block of the down activation is written each bumps the token's counter. The workgroups after
+// them are the down + combine ones: they request their rows at once - the rows do not depend on the activations,
+// so the down stack streams from HBM while gate . up still runs - and read the activations when the counter says
+// all are there. Workgroups are dispatched in index order, so every producer is resident or finished before any
+// consumer waits. The last consumer resets the counters, so a replay starts clean without a memset node.
+template <int WA, int UA, int NBA, int WB, int UB, int NBB>
+__global__ __launch_bounds__(256) void k_moe_decode(const float *x, const uint8_t *wg, const uint8_t *wu,
+                                                    const uint8_t *wd, u32 n_experts, int nba, int nbb,
+                                                    const u32 *sel, const float *wts, const float *resid, int spt,
+                                                    int m, uint8_t *act_x, uint8_t *act_h, float *h, float *y,
+                                                    u32 *counters, u32 spin_limit, u32 *fault, u32 layer) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x;
+    const int na = NBA > 0 ? NBA : nba, nh = NBB > 0 ? NBB : nbb;
+    const int hidden = na * 256;
+    const int blocks_per_slot = nh * 8;
+    const int n_a = m * spt * blocks_per_slot;
+    if ((int)blockIdx.x < n_a) {
+        const int slot = blockIdx.x / blocks_per_slot;
+        gate_up_x_body<WA, UA, NBA>(lds, x, wg, wu, n_experts, na, nh, sel, spt, act_x, act_h, h, slot,
+                                    blockIdx.x % blocks_per_slot, fault, layer);
+        // publish: the block's stores (complete at the barrier), then the count with agent-scope release
+        __syncthreads();
+        if (tid == 0)
+            __hip_atomic_fetch_add(&counters[1 + slot / spt], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+    const int D = 64 / spt;
+    const int blocks_per_token = (hidden + D - 1) / D;
+    const int bi = (int)blockIdx.x - n_a;
+    const int t = bi / blocks_per_token, rb = bi % blocks_per_token;
+    down_combine_body<WB, UB, NBB>(lds, wd, n_experts, nh, act_h, sel, wts, resid, spt, hidden, y, t, rb, fault, layer,
+                                   CounterWait{&counters[1 + t], (u32)(spt * blocks_per_slot), spin_limit, fault, layer});
+    // the last consumer to finish leaves the counters clean for the next launch
+    __syncthreads();
+    if (tid == 0) {
+        const u32 done = __hip_atomic_fetch_add(&counters[0], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        if (done == (u32)(m * blocks_per_token) - 1) {
+            for (int i = 0; i <= m; i++) __hip_atomic_store(&counters[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------ verification
 
 struct StoreTap {
+    static constexpr bool kActive = true;
     int *out; // 16 words a super-block, zeroed before the quad runs
     __device__ __forceinline__ void q4k(int i, int s, int, int v) const { atomicAdd(&out[16 * i + s], v); }
     __device__ __forceinline__ void q4k_isum(int i, int s, int v) const { out[16 * i + 8 + s] = v; }
@@ -486,7 +749,7 @@ __global__ __launch_bounds__(64) void k_block_sums(const uint8_t *wrow, int nb, 
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, q = tid & 3;
     const int n = NB > 0 ? NB : nb;
-    const int col_bytes = n * bm_act_sb_bytes<WT>();
+    const int col_bytes = bm_act_col_bytes<WT>(n);
     for (int i = tid; i < 16 * n; i += blockDim.x) out[i] = 0;
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *col = lds + tab_bytes<WT>();
@@ -519,9 +782,9 @@ static hipError_t allow_lds(K kernel, size_t lds) {
                                (int)lds);
 }
 
-// Picks the kernel variant for a row of nb super-blocks and runs CALL with WT, U and NB as constants. Each type
-// lists its whole-row variant first (the hot shape), then a batch of four, then one super-block at a time, which
-// divides every row.
+// Picks the kernel variant for a row of nb super-blocks and runs CALL_BODY with WT, U and NB as constants. Each
+// type lists its whole-row variant first (the hot shape), then a batch of four, then one super-block at a time,
+// which divides every row.
 #define BM_VARIANT(T, UU, NN)                                                                                          \
     {                                                                                                                  \
         constexpr int WT = T, U = UU, NB = NN;                                                                         \
@@ -547,19 +810,21 @@ static hipError_t allow_lds(K kernel, size_t lds) {
         return hipErrorInvalidValue;                                                                                   \
     }
 
-static int act_sb_bytes(int wtype) { return wtype == BM_IQ2XXS ? BM_Q8K_STRIDE : 2 * BM_Q82X4_STRIDE; }
+int act_col_bytes(int wtype, int k) {
+    const int nb = k / 256;
+    return wtype == BM_IQ2XXS ? nb * BM_Q8K_STRIDE : nb * BM_Q82_SB_EXT;
+}
 static int tab_bytes_rt(int wtype) { return wtype == BM_IQ2XXS ? kTabBytes : 0; }
 
 int gemv_max_cols(int wtype, int k) {
-    const int col_bytes = (k / 256) * act_sb_bytes(wtype);
-    int m = (kMaxLds - tab_bytes_rt(wtype)) / col_bytes;
+    int m = (kMaxLds - tab_bytes_rt(wtype)) / act_col_bytes(wtype, k);
     return m > 8 ? 8 : m;
 }
 
 hipError_t gemv(const Launch &L, int wtype, const uint8_t *w, int64_t rows, int k, const uint8_t *act, int m_total,
                 int col0, int m, float *y) {
     const int nb = k / 256;
-    const size_t lds = tab_bytes_rt(wtype) + (size_t)m * nb * act_sb_bytes(wtype);
+    const size_t lds = tab_bytes_rt(wtype) + (size_t)m * act_col_bytes(wtype, k);
 #define CALL_BODY                                                                                                      \
     auto kern = k_gemv<WT, U, NB>;                                                                                     \
     hipError_t e = allow_lds(kern, lds);                                                                               \
@@ -575,7 +840,7 @@ hipError_t gate_up(const Launch &L, int wtype, const uint8_t *wg, const uint8_t 
                    const uint8_t *act, const uint32_t *sel, int n_slots, int rows_per_expert, int slots_per_col,
                    float *h, uint8_t *act_h) {
     const int nb = k / 256, rpe = rows_per_expert;
-    const size_t lds = tab_bytes_rt(wtype) + (size_t)nb * act_sb_bytes(wtype) + 32 * sizeof(float);
+    const size_t lds = tab_bytes_rt(wtype) + (size_t)act_col_bytes(wtype, k) + 32 * sizeof(float);
     const unsigned grid = (unsigned)n_slots * (unsigned)((rpe + 31) / 32);
 #define CALL_BODY                                                                                                      \
     auto kern = k_gate_up<WT, U, NB>;                                                                                  \
@@ -591,7 +856,7 @@ hipError_t gate_up(const Launch &L, int wtype, const uint8_t *wg, const uint8_t 
 hipError_t gemv_sel(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const uint8_t *act,
                     const uint32_t *sel, int n_slots, int rows_per_expert, float *y) {
     const int nb = k / 256, rpe = rows_per_expert;
-    const size_t lds = tab_bytes_rt(wtype) + (size_t)nb * act_sb_bytes(wtype);
+    const size_t lds = tab_bytes_rt(wtype) + (size_t)act_col_bytes(wtype, k);
     const unsigned grid = (unsigned)n_slots * (unsigned)((rpe + 63) / 64);
 #define CALL_BODY                                                                                                      \
     auto kern = k_gemv_sel<WT, U, NB>;                                                                                 \
@@ -604,13 +869,17 @@ hipError_t gemv_sel(const Launch &L, int wtype, const uint8_t *w, int n_experts,
     return hipGetLastError();
 }
 
+size_t down_combine_lds(int wtype, int k, int spt) {
+    const int D = 64 / spt;
+    return tab_bytes_rt(wtype) + (size_t)spt * act_col_bytes(wtype, k) + ((size_t)D * spt + 2 * (size_t)spt) * sizeof(float);
+}
+
 hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const uint8_t *act,
                         const uint32_t *sel, const float *wts, const float *resid, int slots_per_token, int m,
                         int rows_per_expert, float *y) {
     const int nb = k / 256, rpe = rows_per_expert, spt = slots_per_token;
     const int D = 64 / spt;
-    const size_t lds = tab_bytes_rt(wtype) + (size_t)spt * nb * act_sb_bytes(wtype) +
-                       ((size_t)D * spt + 2 * (size_t)spt) * sizeof(float);
+    const size_t lds = down_combine_lds(wtype, k, spt);
     const unsigned grid = (unsigned)m * (unsigned)((rpe + D - 1) / D);
 #define CALL_BODY                                                                                                      \
     auto kern = k_down_combine<WT, U, NB>;                                                                             \
@@ -623,9 +892,74 @@ hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_expe
     return hipGetLastError();
 }
 
+bool moe_decode_supported(int gate_type, int down_type) {
+    return gate_type == BM_Q4K && (down_type == BM_Q6K || down_type == BM_Q4K);
+}
+
+hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8_t *wg, const uint8_t *wu,
+                     int n_experts, int hidden, int ff, const uint32_t *sel, int slots_per_token, int m,
+                     uint8_t *act_x, uint8_t *act_h, float *h) {
+    const int nba = hidden / 256, nbb = ff / 256, spt = slots_per_token;
+    const size_t lds_a = (size_t)act_col_bytes(gate_type, hidden) + 32 * sizeof(float);
+    const unsigned grid_a = (unsigned)m * (unsigned)spt * (unsigned)(ff / 32);
+    if (gate_type != BM_Q4K) return hipErrorInvalidValue;
+#define BM_GUX(UA, NA)                                                                                                 \
+    {                                                                                                                  \
+        auto kern = k_gate_up_x<BM_Q4K, UA, NA>;                                                                       \
+        hipError_t e = allow_lds(kern, lds_a);                                                                         \
+        if (e != hipSuccess) return e;                                                                                 \
+        hipLaunchKernelGGL(kern, dim3(grid_a), dim3(256), lds_a, L.stream, x, wg, wu, (u32)n_experts, nba, nbb, sel,   \
+                           spt, act_x, act_h, h, L.fault, L.layer);                                                    \
+    }
+    if (nba == 8) BM_GUX(8, 8)
+    else BM_GUX(1, 0)
+#undef BM_GUX
+    return hipGetLastError();
+}
+
+hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, const float *x, const uint8_t *wg,
+                      const uint8_t *wu, const uint8_t *wd, int n_experts, int hidden, int ff, const uint32_t *sel,
+                      const float *wts, const float *resid, int slots_per_token, int m, uint8_t *act_x,
+                      uint8_t *act_h, float *h, float *y, uint32_t *counters, uint32_t spin_limit) {
+    const int nba = hidden / 256, nbb = ff / 256, spt = slots_per_token;
+    const int D = 64 / spt;
+    const size_t lds_a = (size_t)act_col_bytes(gate_type, hidden) + 32 * sizeof(float);
+    const size_t lds_b = down_combine_lds(down_type, ff, spt);
+    const unsigned grid_a = (unsigned)m * (unsigned)spt * (unsigned)(ff / 32);
+    if (gate_type != BM_Q4K) return hipErrorInvalidValue;
+    if (plan == kPlanTwoLaunches) {
+        hipError_t e = gate_up_x(L, gate_type, x, wg, wu, n_experts, hidden, ff, sel, spt, m, act_x, act_h, h);
+        if (e != hipSuccess) return e;
+        return down_combine(L, down_type, wd, n_experts, ff, act_h, sel, wts, resid, spt, m, hidden, y);
+    }
+    const size_t lds = lds_a > lds_b ? lds_a : lds_b;
+    const unsigned grid = grid_a + (unsigned)m * (unsigned)((hidden + D - 1) / D);
+#define BM_FUSED(WA, UA, NA, WB, UB, NBB_)                                                                             \
+    {                                                                                                                  \
+        auto kern = k_moe_decode<WA, UA, NA, WB, UB, NBB_>;                                                            \
+        hipError_t e = allow_lds(kern, lds);                                                                           \
+        if (e != hipSuccess) return e;                                                                                 \
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, x, wg, wu, wd, (u32)n_experts, nba, nbb, sel,   \
+                           wts, resid, spt, m, act_x, act_h, h, y, counters, spin_limit, L.fault, L.layer);            \
+    }
+    if (down_type == BM_Q6K) {
+        if (nba == 8 && nbb == 3) BM_FUSED(BM_Q4K, 8, 8, BM_Q6K, 3, 3)
+        else if (nba == 8) BM_FUSED(BM_Q4K, 8, 8, BM_Q6K, 1, 0)
+        else if (nbb == 3) BM_FUSED(BM_Q4K, 1, 0, BM_Q6K, 3, 3)
+        else BM_FUSED(BM_Q4K, 1, 0, BM_Q6K, 1, 0)
+    } else if (down_type == BM_Q4K) {
+        if (nba == 8) BM_FUSED(BM_Q4K, 8, 8, BM_Q4K, 1, 0)
+        else BM_FUSED(BM_Q4K, 1, 0, BM_Q4K, 1, 0)
+    } else {
+        return hipErrorInvalidValue;
+    }
+#undef BM_FUSED
+    return hipGetLastError();
+}
+
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out) {
     const int nb = k / 256;
-    const size_t lds = tab_bytes_rt(wtype) + (size_t)nb * act_sb_bytes(wtype);
+    const size_t lds = tab_bytes_rt(wtype) + (size_t)act_col_bytes(wtype, k);
 #define CALL_BODY                                                                                                      \
     auto kern = k_block_sums<WT, U, NB>;                                                                               \
     hipError_t e = allow_lds(kern, lds);                                                                               \

@@ -45,6 +45,7 @@ extern "C" {
 #define BM_FAULT_WORDS (1 + 0xFFFF + 1)
 #define BM_SITE_QUANT_COLUMN 1 /* a quantizer met a value that is not finite: NaN scale, zero codes */
 #define BM_SITE_EXPERT_ID 7    /* an expert id at or past the stack */
+#define BM_SITE_STALLED 31     /* ours: a bm_moe_decode consumer gave up waiting for its producers */
 
 /* The id of a slot served elsewhere (crates/gpu/src/host/slots.rs:10): the down projections skip it silently. */
 #define BM_HOST_SLOT 0xFFFFFFFFu
@@ -98,13 +99,15 @@ void bm_weights_destroy(bm_weights *w);
 const void *bm_weights_dev(const bm_weights *w);
 
 /* Activation scratch for up to `m_cap` columns of `k` values in the form `wtype` dots against
- * (Q8Act::with_k / with_slots). Load time only. The device layout is the reference CPU path's column bytes,
- * columns back to back, so a column can be handed to or taken from a host tier unchanged. */
+ * (Q8Act::with_k / with_slots). Load time only. On the device a column is the reference CPU path's column bytes
+ * followed, for the Q8_2_X4 form, by two small tables the dot kernels read (per-block f32 scale and scale * sum,
+ * per-16 code sums); bm_act_download / bm_act_upload move the reference bytes only, so a column can be handed to
+ * or taken from a host tier unchanged. */
 int bm_act_create(bm_ctx *ctx, int wtype, int k, int m_cap, bm_act **out);
 void bm_act_destroy(bm_act *act);
 /* Synchronise and copy column `col`'s bytes (bm_col_bytes of them) to the host. */
 int bm_act_download(bm_ctx *ctx, const bm_act *act, int col, void *host_bytes);
-/* Upload column `col` from host bytes in the same layout. */
+/* Upload column `col` from host bytes in the same layout (the tables are rebuilt on the device). */
 int bm_act_upload(bm_ctx *ctx, bm_act *act, int col, const void *host_bytes);
 
 /* ------------------------------------------------------------------------------- decode: quantize and gemv */
@@ -152,6 +155,35 @@ int bm_combine_tokens(bm_ctx *ctx, const float *down_dev, const float *w_dev, co
 int bm_down_combine(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const uint32_t *sel_dev,
                     const float *w_dev, const float *resid_dev, int n_slots_per_token, int m, int rows_per_expert,
                     float *y_dev);
+
+/* The whole decode step of one MoE layer for m tokens with every quantizer folded in (no counterpart in the
+ * reference, whose step is the chain quantize, gate_up, quantize, down, combine: dispatch.rs:1245-1436): x_dev
+ * holds m rows of hidden = wg's k f32 values (16-byte aligned); token t's slots are sel_dev / w_dev[t *
+ * n_slots_per_token ..]; y_dev[t * hidden + d] gets bm_combine_tokens' value. Same bits as bm_quantize, bm_gate_up
+ * (with act_h) and bm_down_combine run one after the other. Gate/up must be Q4_K, down Q6_K or Q4_K; other types
+ * take the separate launches. act_h is caller-held scratch (m * n_slots_per_token Q8_2_X4 columns of ff = wd's k)
+ * and holds the quantized h afterwards; act_x (optional) receives the quantized x columns; h_dev (optional) the
+ * f32 h rows. m <= 1024.
+ * Two plans (bm_set_decode_plan):
+ *   BM_PLAN_TWO_LAUNCHES (default): gate . up with both quantizers folded in, then down + combine;
+ *   BM_PLAN_ONE_LAUNCH: one launch; the down workgroups start streaming their rows at once and wait on a
+ *     per-token device counter for that token's gate/up workgroups. A wait that outlasts the context's spin
+ *     limit raises BM_SITE_STALLED and the launch still ends (y is then not valid; bm_fault_clear re-arms the
+ *     counters). Launches of this plan that share a context must not overlap. */
+#define BM_PLAN_ONE_LAUNCH 1
+#define BM_PLAN_TWO_LAUNCHES 2
+int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_weights *wd, const float *x_dev,
+                  const uint32_t *sel_dev, const float *w_dev, const float *resid_dev, int n_slots_per_token, int m,
+                  bm_act *act_h, bm_act *act_x, float *h_dev, float *y_dev);
+int bm_set_decode_plan(bm_ctx *ctx, int plan);
+/* The first launch of BM_PLAN_TWO_LAUNCHES on its own: bm_quantize, bm_gate_up and the quantizer of h in one
+ * launch, from the f32 token rows (Q4_K gate/up; rows_per_expert = ff a multiple of 256). Follow it with
+ * bm_down_combine or bm_gemv_sel over act_h. */
+int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const float *x_dev, const uint32_t *sel_dev,
+                 int n_slots_per_token, int m, int rows_per_expert, bm_act *act_h, bm_act *act_x, float *h_dev);
+/* Polls (a memory round trip each, about a microsecond) a BM_PLAN_ONE_LAUNCH consumer waits before it gives up;
+ * the default is 1 << 18. */
+int bm_set_spin_limit(bm_ctx *ctx, uint32_t spins);
 
 /* ------------------------------------------------------------------------------------------- verification */
 

@@ -342,6 +342,124 @@ def test_layers_of_every_type_and_several_tokens(gpu, types, hidden, ff, n_exper
     L.free()
 
 
+def run_single_launch(gpu, L, x, ids, wts, top_k, resid=None, replays=1, plan=bm.PLAN_ONE_LAUNCH):
+    """bm_moe_decode: the whole step with the quantizers folded in, in one launch or two. Returns (y, h, act_h
+    columns, act_x columns) of the last replay."""
+    gpu.set_decode_plan(plan)
+    m = x.shape[0]
+    n_slots = m * top_k
+    act_x = gpu.act(L.types[0], L.hidden, m)
+    act_h = gpu.act(L.types[2], L.ff, n_slots)
+    xd, sel, wd = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32)
+    rd = gpu.upload(resid, np.float32) if resid is not None else None
+    h = gpu.buffer(np.float32, n_slots * L.ff)
+    y = gpu.buffer(np.float32, m * L.hidden)
+    for _ in range(replays):
+        h.fill_bytes(0xFF)
+        y.fill_bytes(0xFF)
+        gpu.enqueue_moe_decode(L.dg, L.du, L.dd, xd, sel, wd, rd, top_k, m, act_h, y, act_x=act_x, h=h)
+    out = (y.download(), h.download(), [act_h.download(s) for s in range(n_slots)],
+           [act_x.download(t) for t in range(m)])
+    for b in (act_x, act_h, xd, sel, wd, h, y) + ((rd,) if rd is not None else ()):
+        b.free()
+    return out
+
+
+@pytest.mark.parametrize("types,hidden,ff,n_experts,m,top_k", (
+    ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 16, 1, 8),   # config 2's shape: the whole-row variants
+    ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 12, 5, 4),
+    ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 1024, 512, 6, 3, 6),    # 64 / 6 rows a consumer workgroup: a ragged tail
+    ((bm.Q4_K, bm.Q4_K, bm.Q4_K), 512, 512, 5, 4, 2),
+    ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 4096, 256, 4, 2, 3),    # rows longer than one quantizer pass
+))
+@pytest.mark.parametrize("plan", (bm.PLAN_ONE_LAUNCH, bm.PLAN_TWO_LAUNCHES))
+def test_single_launch_step_matches_the_chain_and_the_oracle(gpu, types, hidden, ff, n_experts, m, top_k, plan):
+    L = Layer(gpu, types, hidden, ff, n_experts, 600 + hidden + ff)
+    rng = np.random.default_rng(601)
+    x = normal_f32(rng, (m, hidden))
+    resid = normal_f32(rng, (m, hidden))
+    ids, wts = route(rng, m, n_experts, top_k)
+    gpu.fault_clear()
+    # three launches in a row: the counters must come back clean each time
+    y, h, act_h, act_x = run_single_launch(gpu, L, x, ids, wts, top_k, resid, replays=3, plan=plan)
+    want_y, want_h = L.oracle(x, ids, wts, top_k)
+    for t in range(m):
+        assert np.array_equal(act_x[t], ora.quantize_col(types[0], x[t])), f"act_x token {t}"
+    assert_f32(h, want_h, "h")
+    for s in range(m * top_k):
+        assert np.array_equal(act_h[s], ora.quantize_col(types[2], want_h[s * ff:(s + 1) * ff])), f"act_h slot {s}"
+    assert_f32(y, (want_y.reshape(m, hidden) + resid).astype(np.float32).reshape(-1), "y + resid")
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    L.free()
+
+
+@pytest.mark.parametrize("plan", (bm.PLAN_ONE_LAUNCH, bm.PLAN_TWO_LAUNCHES))
+def test_single_launch_refused_ids_and_host_slots(gpu, plan):
+    L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 4, 700)
+    rng = np.random.default_rng(701)
+    x = normal_f32(rng, (2, 512))
+    ids = np.array([[1, 9, 3], [2, 0, 1]], np.uint32)      # slot 1 names an expert past the stack
+    wts = np.array([[0.5, 0.3, 0.2], [0.2, 0.5, 0.3]], np.float32)
+    gpu.fault_clear()
+    gpu.set_layer(4)
+    y, h, _, _ = run_single_launch(gpu, L, x, ids, wts, 3, plan=plan)
+    assert gpu.fault(4) == ((4 << 8) | bm.SITE_EXPERT_ID, 1 << bm.SITE_EXPERT_ID)
+    assert np.isnan(h.reshape(6, 256)[1]).all()
+    # the refused slot adds nothing: the same as the oracle over the live slots with the same weights
+    live_ids, live_w = np.array([[1, 3], [2, 0]], np.uint32), np.array([[0.5, 0.2], [0.2, 0.5]], np.float32)
+    want0, _ = L.oracle(x[:1], live_ids[:1], live_w[:1], 2)
+    assert_f32(y[:512], want0, "token with a refused slot")
+    want1, _ = L.oracle(x[1:], ids[1:], wts[1:], 3)
+    assert_f32(y[512:], want1, "clean token")
+    gpu.set_layer(bm.LAYER_NONE)
+    gpu.fault_clear()
+    L.free()
+
+
+def test_single_launch_gives_up_waiting_and_recovers(gpu):
+    """A consumer that may not wait at all (spin limit 0) raises BM_SITE_STALLED and the launch still ends;
+    after bm_fault_clear the next launch is whole again."""
+    L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 8, 800)
+    rng = np.random.default_rng(801)
+    x = normal_f32(rng, (1, 2048))
+    ids, wts = route(rng, 1, 8, 8)
+    want_y, _ = L.oracle(x, ids, wts, 8)
+    gpu.fault_clear()
+    gpu.set_spin_limit(0)
+    y, _, _, _ = run_single_launch(gpu, L, x, ids, wts, 8)
+    word0, mask = gpu.fault()
+    gpu.set_spin_limit(1 << 18)
+    stalled = word0 == ((bm.LAYER_NONE << 8) | bm.SITE_STALLED)
+    if not stalled:  # every producer happened to finish first
+        assert word0 == bm.FAULT_NONE
+        assert_f32(y, want_y, "y of the launch that did not stall")
+    else:
+        assert mask == 1 << bm.SITE_STALLED
+    gpu.fault_clear()
+    y, _, _, _ = run_single_launch(gpu, L, x, ids, wts, 8, replays=2)
+    assert_f32(y, want_y, "y after recovery")
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    L.free()
+
+
+def test_uploaded_columns_dot_like_quantized_ones(gpu):
+    """A column that arrives as bytes from a host tier (bm_act_upload) has its tables rebuilt on the device."""
+    rng = np.random.default_rng(900)
+    for wtype, rows, k in ((bm.Q4_K, 64, 1024), (bm.Q6_K, 64, 768), (bm.IQ2_XXS, 64, 512)):
+        w = stack(wtype, rows, k, 901)
+        x = normal_f32(rng, (2, k))
+        cols = [ora.quantize_col(wtype, x[c]) for c in range(2)]
+        dw, act = gpu.weights(wtype, rows, k, w), gpu.act(wtype, k, 2)
+        for c in range(2):
+            act.upload(c, cols[c])
+            assert np.array_equal(act.download(c), cols[c])
+        y = gpu.buffer(np.float32, rows * 2)
+        gpu.enqueue_gemv(dw, act, 2, y)
+        assert_f32(y.download(), ora.gemv(wtype, w, rows, k, np.concatenate(cols), 2), f"type {wtype}")
+        for b in (dw, act, y):
+            b.free()
+
+
 def test_slot_equals_one_expert_gemv_and_duplicate_ids(gpu):
     # gate_q4k_sel's first clauses (crates/gpu-gates/src/bin/gate_q4k_sel.rs:1-48)
     rng = np.random.default_rng(300)

@@ -139,7 +139,7 @@ def main():
 
     # one graph of `unit` steps; the timed region replays it
     unit = max(len(layers) * n_tok // np.gcd(len(layers), n_tok), 1)
-    unit = min(int(unit), 256)
+    unit = min(max(int(unit), 64), 256)  # a graph of at least 64 steps: the replay call itself costs microseconds
     gpu.capture_begin()
     for i in range(unit):
         enqueue_step(i)

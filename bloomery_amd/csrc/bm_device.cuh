@@ -215,17 +215,40 @@ __device__ __forceinline__ void bm_q4_dot16(uint4 q, uint4 alo, uint4 ahi, int &
     hi = bm_sdot4((q.w >> 4) & m, ahi.w, hi);
 }
 
+// What the Q4_K core reads of one column for one super-block: read a super-block ahead of its use, the LDS
+// latency hides behind the previous super-block's arithmetic.
+template <int WT>
+struct Act;
+template <>
+struct Act<BM_Q4K> {
+    uint4 lo0, hi0, lo1, hi1; // codes against the low / high nibbles of the first and second 64 code bytes
+    float4 e0, e1, em;        // (d8, d8 * isum) of sub-blocks (2c, 2c + 1), (4 + 2c, 5 + 2c), (4h + 2c, 4h + 2c + 1)
+    u32 sw;                   // the two stored isums (taps only)
+};
+
+template <bool WithSums>
+__device__ __forceinline__ Act<BM_Q4K> bm_act_q4k(const ActView &av, int i, int c, int h) {
+    const uint8_t *g0 = av.col + (size_t)(2 * i) * BM_Q82X4_STRIDE + 16 + 64 * c + 16 * h;
+    const uint8_t *g1 = g0 + BM_Q82X4_STRIDE;
+    const uint8_t *te = av.tbl + (size_t)i * 64 + 16 * c;
+    Act<BM_Q4K> a;
+    a.lo0 = *reinterpret_cast<const uint4 *>(g0);
+    a.hi0 = *reinterpret_cast<const uint4 *>(g0 + 32);
+    a.lo1 = *reinterpret_cast<const uint4 *>(g1);
+    a.hi1 = *reinterpret_cast<const uint4 *>(g1 + 32);
+    a.e0 = *reinterpret_cast<const float4 *>(te);
+    a.e1 = *reinterpret_cast<const float4 *>(te + 32);
+    a.em = *reinterpret_cast<const float4 *>(te + 32 * h);
+    a.sw = 0;
+    if constexpr (WithSums)
+        a.sw = *reinterpret_cast<const u32 *>(av.col + (size_t)(2 * i + h) * BM_Q82X4_STRIDE + 8 + 4 * c);
+    return a;
+}
+
 // One super-block `i` of one column.
 template <class Tap>
-__device__ __forceinline__ void bm_dot_q4k(const Blk<BM_Q4K> &b, const ActView &av, int i, int c, int h, float &acc0,
-                                           float &acc1, const Tap &tap) {
-    const uint8_t *g0 = av.col + (size_t)(2 * i) * BM_Q82X4_STRIDE;
-    const uint8_t *g1 = g0 + BM_Q82X4_STRIDE;
-    const uint8_t *te = av.tbl + (size_t)i * 64;
-    // (d8, d8 * isum) of sub-blocks (2c, 2c + 1), (4 + 2c, 5 + 2c) and of this lane's own pair (4h + 2c, 4h + 2c + 1)
-    const float4 e0 = *reinterpret_cast<const float4 *>(te + 16 * c);
-    const float4 e1 = *reinterpret_cast<const float4 *>(te + 32 + 16 * c);
-    const float4 em = *reinterpret_cast<const float4 *>(te + 32 * h + 16 * c);
+__device__ __forceinline__ void bm_dot_q4k(const Blk<BM_Q4K> &b, const Act<BM_Q4K> &a, int i, int c, int h,
+                                           float &acc0, float &acc1, const Tap &tap) {
     const float d = bm_half_to_f32(b.hdr.x & 0xffffu), dmin = bm_half_to_f32(b.hdr.x >> 16);
     const u32 a0 = b.hdr.y, a1 = b.hdr.z, a2 = b.hdr.w; // crates/qdot/src/lib.rs:3868-3878
     const int sh = 16 * c;                               // this lane's two sub-blocks sit in bytes 2c, 2c + 1
@@ -234,31 +257,26 @@ __device__ __forceinline__ void bm_dot_q4k(const Blk<BM_Q4K> &b, const ActView &
     const u32 mw = h ? (((a2 >> 4) & 0x0f0f0f0fu) | ((a1 >> 2) & 0x30303030u)) : (a1 & 0x3f3f3f3fu);
     const u32 mm = mw >> sh; // mins of sub-blocks 4h + 2c, 4h + 2c + 1
     // Min term of accumulators l = 4h + t (lib.rs:4389-4394): fma(d8 * isum, -(dmin * m), acc).
-    acc0 = fmaf(em.y, -(dmin * (float)(mm & 0xffu)), acc0);
-    acc1 = fmaf(em.w, -(dmin * (float)((mm >> 8) & 0xffu)), acc1);
+    acc0 = fmaf(a.em.y, -(dmin * (float)(mm & 0xffu)), acc0);
+    acc1 = fmaf(a.em.w, -(dmin * (float)((mm >> 8) & 0xffu)), acc1);
     if constexpr (Tap::kActive) {
-        const u32 sw = *reinterpret_cast<const u32 *>((h ? g1 : g0) + 8 + 4 * c);
-        tap.q4k_isum(i, 4 * h + 2 * c, (int)(short)(sw & 0xffffu));
-        tap.q4k_isum(i, 4 * h + 2 * c + 1, (int)(short)(sw >> 16));
+        tap.q4k_isum(i, 4 * h + 2 * c, (int)(short)(a.sw & 0xffffu));
+        tap.q4k_isum(i, 4 * h + 2 * c + 1, (int)(short)(a.sw >> 16));
     }
     // j = 0: sub-blocks 2c, 2c + 1 (group 0); j = 1: 4 + 2c, 5 + 2c (group 1) (lib.rs:4402-4436).
     {
-        const uint4 alo = *reinterpret_cast<const uint4 *>(g0 + 16 + 64 * c + 16 * h);
-        const uint4 ahi = *reinterpret_cast<const uint4 *>(g0 + 16 + 64 * c + 32 + 16 * h);
         int lo, hi;
-        bm_q4_dot16(b.qa, alo, ahi, lo, hi);
-        acc0 = fmaf((d * (float)(s0 & 0xffu)) * e0.x, (float)lo, acc0);
-        acc1 = fmaf((d * (float)((s0 >> 8) & 0xffu)) * e0.z, (float)hi, acc1);
+        bm_q4_dot16(b.qa, a.lo0, a.hi0, lo, hi);
+        acc0 = fmaf((d * (float)(s0 & 0xffu)) * a.e0.x, (float)lo, acc0);
+        acc1 = fmaf((d * (float)((s0 >> 8) & 0xffu)) * a.e0.z, (float)hi, acc1);
         tap.q4k(i, 2 * c, h, lo);
         tap.q4k(i, 2 * c + 1, h, hi);
     }
     {
-        const uint4 alo = *reinterpret_cast<const uint4 *>(g1 + 16 + 64 * c + 16 * h);
-        const uint4 ahi = *reinterpret_cast<const uint4 *>(g1 + 16 + 64 * c + 32 + 16 * h);
         int lo, hi;
-        bm_q4_dot16(b.qb, alo, ahi, lo, hi);
-        acc0 = fmaf((d * (float)(s1 & 0xffu)) * e1.x, (float)lo, acc0);
-        acc1 = fmaf((d * (float)((s1 >> 8) & 0xffu)) * e1.z, (float)hi, acc1);
+        bm_q4_dot16(b.qb, a.lo1, a.hi1, lo, hi);
+        acc0 = fmaf((d * (float)(s1 & 0xffu)) * a.e1.x, (float)lo, acc0);
+        acc1 = fmaf((d * (float)((s1 >> 8) & 0xffu)) * a.e1.z, (float)hi, acc1);
         tap.q4k(i, 4 + 2 * c, h, lo);
         tap.q4k(i, 5 + 2 * c, h, hi);
     }
@@ -300,31 +318,46 @@ __device__ __forceinline__ void bm_q6_dot16x2(uint4 ql, uint4 qh, int hs, uint4 
     s1 = bm_sdot4(((ql.w >> 4) & ml) | (hw & mh), ab.w, s1);
 }
 
+template <>
+struct Act<BM_Q6K> {
+    uint4 aa[2], ab[2]; // per 128-value half j: the 16 codes of 32-block c and of 32-block c + 2, half h
+    float d8a[2], d8b[2];
+    int sa[2], sb[2]; // sums of those 16 codes
+};
+
+__device__ __forceinline__ Act<BM_Q6K> bm_act_q6k(const ActView &av, int i, int c, int h) {
+    const uint8_t *g0 = av.col + (size_t)(2 * i) * BM_Q82X4_STRIDE + 16 + 32 * c + 16 * h;
+    const uint8_t *te = av.tbl + (size_t)i * 64 + 8 * c;
+    const int *s16 = reinterpret_cast<const int *>(av.s16 + (size_t)i * 64) + 2 * c + h;
+    Act<BM_Q6K> a;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        a.aa[j] = *reinterpret_cast<const uint4 *>(g0 + j * BM_Q82X4_STRIDE);
+        a.ab[j] = *reinterpret_cast<const uint4 *>(g0 + j * BM_Q82X4_STRIDE + 64);
+        a.d8a[j] = *reinterpret_cast<const float *>(te + 32 * j);
+        a.d8b[j] = *reinterpret_cast<const float *>(te + 32 * j + 16);
+        a.sa[j] = s16[8 * j];
+        a.sb[j] = s16[8 * j + 4];
+    }
+    return a;
+}
+
 template <class Tap>
-__device__ __forceinline__ void bm_dot_q6k(const Blk<BM_Q6K> &b, const ActView &av, int i, int c, int h, float &acc0,
-                                           float &acc1, const Tap &tap) {
-    const uint8_t *g0 = av.col + (size_t)(2 * i) * BM_Q82X4_STRIDE;
-    const uint8_t *te = av.tbl + (size_t)i * 64;
-    const int *s16 = reinterpret_cast<const int *>(av.s16 + (size_t)i * 64);
+__device__ __forceinline__ void bm_dot_q6k(const Blk<BM_Q6K> &b, const Act<BM_Q6K> &a, int i, int c, int h,
+                                           float &acc0, float &acc1, const Tap &tap) {
     const float d = bm_half_to_f32(b.d);
     const int bi = 8 * (2 * c + h); // this lane's scale byte inside each word of four
 #pragma unroll
     for (int j = 0; j < 2; j++) {
-        const uint8_t *g = g0 + j * BM_Q82X4_STRIDE;
-        const float d8a = *reinterpret_cast<const float *>(te + 8 * (4 * j + c));     // 32-block c of this half
-        const float d8b = *reinterpret_cast<const float *>(te + 8 * (4 * j + c + 2)); // 32-block c + 2
-        const int sa = s16[2 * (4 * j + c) + h], sb = s16[2 * (4 * j + c + 2) + h];   // sum of the 16 codes dotted
-        const uint4 aa = *reinterpret_cast<const uint4 *>(g + 16 + 32 * c + 16 * h);
-        const uint4 ab = *reinterpret_cast<const uint4 *>(g + 16 + 32 * (c + 2) + 16 * h);
         int s0, s1;
-        bm_q6_dot16x2(j ? b.ql1 : b.ql0, j ? b.qh1 : b.qh0, 2 * c, aa, ab, s0, s1);
-        s0 -= 32 * sa; // sum (q6 - 32) * a
-        s1 -= 32 * sb;
+        bm_q6_dot16x2(j ? b.ql1 : b.ql0, j ? b.qh1 : b.qh0, 2 * c, a.aa[j], a.ab[j], s0, s1);
+        s0 -= 32 * a.sa[j]; // sum (q6 - 32) * a
+        s1 -= 32 * a.sb[j];
         // scale bytes 8j + 2c + h and 8j + 4 + 2c + h (crates/qdot/src/lib.rs:4455 K_SHUFFLE_Q6K, :4794-4809)
         const int sc0 = __builtin_amdgcn_sbfe((int)(j ? b.sc.z : b.sc.x), bi, 8);
         const int sc1 = __builtin_amdgcn_sbfe((int)(j ? b.sc.w : b.sc.y), bi, 8);
-        acc0 = fmaf((d * (float)sc0) * d8a, (float)s0, acc0);
-        acc1 = fmaf((d * (float)sc1) * d8b, (float)s1, acc1);
+        acc0 = fmaf((d * (float)sc0) * a.d8a[j], (float)s0, acc0);
+        acc1 = fmaf((d * (float)sc1) * a.d8b[j], (float)s1, acc1);
         tap.q6k(i, 8 * j + 2 * c + h, s0);
         tap.q6k(i, 8 * j + 4 + 2 * c + h, s1);
     }
@@ -354,17 +387,33 @@ struct Iq2Tables {
     const u32 *nibmask;
 };
 
-template <class Tap>
-__device__ __forceinline__ void bm_dot_iq2xxs(const Blk<BM_IQ2XXS> &b, const ActView &av, int i, int q,
-                                              const Iq2Tables &tb, float &acc0, float &acc1, const Tap &tap) {
+template <>
+struct Act<BM_IQ2XXS> {
+    float dy;
+    uint2 bs;   // bsums 4q .. 4q + 3
+    uint2 a[8]; // values 8q .. 8q + 8 of each of the eight sub-blocks
+};
+
+__device__ __forceinline__ Act<BM_IQ2XXS> bm_act_iq2xxs(const ActView &av, int i, int q) {
     const uint8_t *blk = av.col + (size_t)i * BM_Q8K_STRIDE;
-    const float dy = *reinterpret_cast<const float *>(blk);
+    Act<BM_IQ2XXS> a;
+    a.dy = *reinterpret_cast<const float *>(blk);
+    a.bs = *reinterpret_cast<const uint2 *>(blk + 264 + 8 * q);
+#pragma unroll
+    for (int sb = 0; sb < 8; sb++) a.a[sb] = *reinterpret_cast<const uint2 *>(blk + 8 + 32 * sb + 8 * q);
+    return a;
+}
+
+template <class Tap>
+__device__ __forceinline__ void bm_dot_iq2xxs(const Blk<BM_IQ2XXS> &b, const Act<BM_IQ2XXS> &act, int i, int q,
+                                              const Iq2Tables &tb, float &acc0, float &acc1, const Tap &tap) {
+    const float dy = act.dy;
     const float d = 0.125f * bm_half_to_f32(b.d);
     const float dmin = -d * 43.0f;
     // Fold first (crates/qdot/src/lib.rs:8691-8694): accumulator l takes sub-block l's scale on its two bsums.
     {
         const int sca = 2 * (int)(b.q.y >> 28) + 1, scb = 2 * (int)(b.q.w >> 28) + 1; // sub-blocks 2q, 2q + 1
-        const uint2 bs = *reinterpret_cast<const uint2 *>(blk + 264 + 8 * q);          // bsums 4q .. 4q + 3
+        const uint2 bs = act.bs;
         const int b0 = (int)(short)(bs.x & 0xffffu), b1 = (int)(short)(bs.x >> 16);
         const int b2 = (int)(short)(bs.y & 0xffffu), b3 = (int)(short)(bs.y >> 16);
         const int ma = sca * b0 + sca * b1, mb = scb * b2 + scb * b3;
@@ -388,7 +437,7 @@ __device__ __forceinline__ void bm_dot_iq2xxs(const Blk<BM_IQ2XXS> &b, const Act
             const u32 m_lo = tb.nibmask[sg & 15u], m_hi = tb.nibmask[sg >> 4];
             // -mag where the sign bit is set: (mag ^ 0xff) + 1 per byte, no carry leaves a byte (mag > 0).
             const u32 v_lo = (g.x ^ m_lo) + (m_lo & 0x01010101u), v_hi = (g.y ^ m_hi) + (m_hi & 0x01010101u);
-            const uint2 a = *reinterpret_cast<const uint2 *>(blk + 8 + 32 * sb + 8 * q);
+            const uint2 a = act.a[sb];
             const int i_lo = bm_sdot4(v_lo, a.x, 0), i_hi = bm_sdot4(v_hi, a.y, 0);
             const int s_lo = bm_sdot4(0x01010101u, a.x, 0), s_hi = bm_sdot4(0x01010101u, a.y, 0);
             // the reference sums sc * (v + 43) * a: the offset comes back out through the fold above
@@ -433,15 +482,25 @@ __device__ __forceinline__ Blk<BM_IQ2XXS> bm_load_blk<BM_IQ2XXS>(const uint8_t *
     return bm_load_iq2xxs(wrow, i, q);
 }
 
+template <int WT, bool WithSums>
+__device__ __forceinline__ Act<WT> bm_load_act(const ActView &av, int i, int q) {
+    if constexpr (WT == BM_Q4K)
+        return bm_act_q4k<WithSums>(av, i, q & 1, q >> 1);
+    else if constexpr (WT == BM_Q6K)
+        return bm_act_q6k(av, i, q & 1, q >> 1);
+    else
+        return bm_act_iq2xxs(av, i, q);
+}
+
 template <int WT, class Tap>
-__device__ __forceinline__ void bm_dot_blk(const Blk<WT> &b, const ActView &av, int i, int q, const Iq2Tables &tb,
+__device__ __forceinline__ void bm_dot_blk(const Blk<WT> &b, const Act<WT> &a, int i, int q, const Iq2Tables &tb,
                                            float &acc0, float &acc1, const Tap &tap) {
     if constexpr (WT == BM_Q4K)
-        bm_dot_q4k(b, av, i, q & 1, q >> 1, acc0, acc1, tap);
+        bm_dot_q4k(b, a, i, q & 1, q >> 1, acc0, acc1, tap);
     else if constexpr (WT == BM_Q6K)
-        bm_dot_q6k(b, av, i, q & 1, q >> 1, acc0, acc1, tap);
+        bm_dot_q6k(b, a, i, q & 1, q >> 1, acc0, acc1, tap);
     else
-        bm_dot_iq2xxs(b, av, i, q, tb, acc0, acc1, tap);
+        bm_dot_iq2xxs(b, a, i, q, tb, acc0, acc1, tap);
 }
 
 template <int WT>

@@ -1,14 +1,14 @@
 // HIP kernels of the quantized MoE expert matmul for gfx950, and their launch functions.
 //
 // Every dot kernel follows one plan: a quad of lanes per weight row (bm_device.cuh); the token's quantized
-// activation column requested first, then the row's first batch of super-blocks (128-bit loads), all from
-// straight-line code so the hardware's in-order load counter lets the column be copied to LDS and the arithmetic
-// start on the first super-block while the later ones are still in flight. Weights are read once, straight from
-// the file's block bytes; the kernels are bound by HBM bandwidth.
+// activation column requested first, then the row's super-blocks (128-bit loads) through a small ring of
+// registers, a few super-blocks ahead of the arithmetic, all from straight-line code so the hardware's in-order
+// load counter lets the arithmetic of one super-block run while the later ones are still in flight. Weights are
+// read once, straight from the file's block bytes.
 //
-// Variants: a kernel is instantiated per weight type and per (U, NB): U super-blocks a lane requests per batch,
-// NB the row's super-block count when it is known at compile time (0: a run-time count that U divides). The hot
-// shapes (Q4_K rows of 2048 values, Q6_K rows of 768) take NB = U = the whole row, one batch and no loop.
+// Variants: a kernel is instantiated per weight type and per (U, NB): U the ring's size in super-blocks, NB the
+// row's super-block count when it is known at compile time (0: a run-time count that U divides). The hot shapes
+// (Q4_K rows of 2048 values, Q6_K rows of 768) have NB set and their stages unrolled.
 #include "bm_kernels.h"
 
 #define BM_TABLE_QUAL __device__ const
@@ -87,15 +87,39 @@ struct Stage {
     }
 };
 
-// Super-blocks 0..U of the row, requested unconditionally (the launch functions pick U to divide the row).
+// The weight stream of a row is a ring of U super-blocks in registers: the first U - 1 are requested up front
+// (preload), and each stage requests the super-block U - 1 ahead of the one it is about to use before it starts its
+// arithmetic. A wave that asks for a whole row at once sits in the memory pipeline's queue until most of it has
+// arrived and only then starts to compute; with the ring the requests trickle out between the stages and the
+// arithmetic runs under the stream.
 template <int WT, int U>
 __device__ __forceinline__ void preload(Blk<WT> (&b)[U], const uint8_t *wrow, int q) {
 #pragma unroll
-    for (int u = 0; u < U; u++) b[u] = bm_load_blk<WT>(wrow, u, q);
+    for (int u = 0; u + 1 < U; u++) b[u] = bm_load_blk<WT>(wrow, u, q);
 }
 
-// Row `wrow` against `m` <= M columns (LDS, `col_stride` apart); b holds the first batch already.
-// NB > 0: the row has NB super-blocks (a multiple of U); NB == 0: it has nb, a multiple of U.
+// One stage: request super-block `ahead` into its ring slot, read the next stage's activation operands from LDS,
+// then the arithmetic of super-block i (ring slot `slot`). The asm statements pin that order: the compiler may
+// neither hoist the reads of later stages nor sink this stage's sums past them.
+template <int WT, int U, class Tap>
+__device__ __forceinline__ void stage_one(Blk<WT> (&b)[U], int slot, int fill, const uint8_t *wrow, int ahead,
+                                          const ActView &av, int i, int act_next, int q, const Iq2Tables &tb,
+                                          Act<WT> &cur, float &a0, float &a1, const Tap &tap) {
+    __asm__ volatile("" ::: "memory");
+    if (U > 1) b[fill] = bm_load_blk<WT>(wrow, ahead, q);
+    const Act<WT> next = bm_load_act<WT, Tap::kActive>(av, act_next, q);
+    __asm__ volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    if (U == 1) b[0] = bm_load_blk<WT>(wrow, i, q);
+    bm_dot_blk<WT>(b[slot], cur, i, q, tb, a0, a1, tap);
+    __asm__ volatile("" : "+v"(a0), "+v"(a1)::"memory");
+    __builtin_amdgcn_sched_barrier(0);
+    cur = next;
+}
+
+// Row `wrow` against `m` <= M columns (LDS, `col_stride` apart); b holds the ring, preloaded.
+// NB > 0: the row has NB super-blocks, the stages are unrolled; NB == 0: it has nb, a multiple of U.
+// Indices past the row's end are clamped onto its last super-block: a redundant read, no branch in the stream.
 template <int WT, int U, int NB, int M, class Tap>
 __device__ __forceinline__ void row_dot(Blk<WT> (&b)[U], const uint8_t *wrow, const uint8_t *cols, int col_stride,
                                         int m, int nb, int q, const Iq2Tables &tb, float (&out)[M], const Tap &tap) {
@@ -107,25 +131,46 @@ __device__ __forceinline__ void row_dot(Blk<WT> (&b)[U], const uint8_t *wrow, co
         a0[c] = a1[c] = 0.0f;
         av[c] = bm_act_view<WT>(cols + (size_t)c * col_stride, n);
     }
-    if constexpr (NB == U) {
+    if constexpr (M == 1) {
+        Act<WT> cur = bm_load_act<WT, Tap::kActive>(av[0], 0, q);
+        if constexpr (NB > 0) {
 #pragma unroll
-        for (int u = 0; u < U; u++) {
+            for (int i = 0; i < NB; i++) {
+                const int ahead = i + U - 1 < NB ? i + U - 1 : NB - 1;
+                stage_one<WT, U>(b, i % U, (i + U - 1) % U, wrow, ahead, av[0], i, i + 1 < NB ? i + 1 : i, q, tb, cur,
+                                 a0[0], a1[0], tap);
+            }
+        } else {
+            for (int i0 = 0; i0 < n; i0 += U) {
 #pragma unroll
-            for (int c = 0; c < M; c++)
-                if (M == 1 || c < m) bm_dot_blk<WT>(b[u], av[c], u, q, tb, a0[c], a1[c], tap);
+                for (int u = 0; u < U; u++) {
+                    const int i = i0 + u;
+                    const int ahead = i + U - 1 < n ? i + U - 1 : n - 1;
+                    stage_one<WT, U>(b, u, (u + U - 1) % U, wrow, ahead, av[0], i, i + 1 < n ? i + 1 : i, q, tb, cur,
+                                     a0[0], a1[0], tap);
+                }
+            }
         }
     } else {
-        for (int i0 = 0;;) {
+        // several columns: the same ring for the weights, the activation operands read where they are used
+        auto stage = [&](int slot, int fill, int i) {
+            const int ahead = i + U - 1 < n ? i + U - 1 : n - 1;
+            b[fill] = bm_load_blk<WT>(wrow, U > 1 ? ahead : i, q);
 #pragma unroll
-            for (int u = 0; u < U; u++) {
+            for (int c = 0; c < M; c++)
+                if (c < m) {
+                    const Act<WT> a = bm_load_act<WT, Tap::kActive>(av[c], i, q);
+                    bm_dot_blk<WT>(b[slot], a, i, q, tb, a0[c], a1[c], tap);
+                }
+        };
+        if constexpr (NB > 0) {
 #pragma unroll
-                for (int c = 0; c < M; c++)
-                    if (M == 1 || c < m) bm_dot_blk<WT>(b[u], av[c], i0 + u, q, tb, a0[c], a1[c], tap);
+            for (int i = 0; i < NB; i++) stage(i % U, (i + U - 1) % U, i);
+        } else {
+            for (int i0 = 0; i0 < n; i0 += U) {
+#pragma unroll
+                for (int u = 0; u < U; u++) stage(u, (u + U - 1) % U, i0 + u);
             }
-            i0 += U;
-            if (i0 >= n) break;
-#pragma unroll
-            for (int u = 0; u < U; u++) b[u] = bm_load_blk<WT>(wrow, i0 + u, q);
         }
     }
 #pragma unroll
@@ -783,8 +828,9 @@ static hipError_t allow_lds(K kernel, size_t lds) {
 }
 
 // Picks the kernel variant for a row of nb super-blocks and runs CALL_BODY with WT, U and NB as constants. Each
-// type lists its whole-row variant first (the hot shape), then a batch of four, then one super-block at a time,
-// which divides every row.
+// type lists the hot shape first (its count known at compile time, stages unrolled), then a ring of two for even
+// counts, then one super-block at a time, which divides every row.
+constexpr int kRingQ4K = 3, kRingQ6K = 2;
 #define BM_VARIANT(T, UU, NN)                                                                                          \
     {                                                                                                                  \
         constexpr int WT = T, U = UU, NB = NN;                                                                         \
@@ -793,17 +839,17 @@ static hipError_t allow_lds(K kernel, size_t lds) {
 #define BM_DISPATCH(wtype, nb)                                                                                         \
     switch (wtype) {                                                                                                   \
     case BM_Q4K:                                                                                                       \
-        if ((nb) == 8) BM_VARIANT(BM_Q4K, 8, 8)                                                                        \
-        else if ((nb) % 4 == 0) BM_VARIANT(BM_Q4K, 4, 0)                                                               \
+        if ((nb) == 8) BM_VARIANT(BM_Q4K, kRingQ4K, 8)                                                                 \
+        else if ((nb) % 2 == 0) BM_VARIANT(BM_Q4K, 2, 0)                                                               \
         else BM_VARIANT(BM_Q4K, 1, 0)                                                                                  \
         break;                                                                                                         \
     case BM_Q6K:                                                                                                       \
-        if ((nb) == 3) BM_VARIANT(BM_Q6K, 3, 3)                                                                        \
-        else if ((nb) % 4 == 0) BM_VARIANT(BM_Q6K, 4, 0)                                                               \
+        if ((nb) == 3) BM_VARIANT(BM_Q6K, kRingQ6K, 3)                                                                 \
+        else if ((nb) % 2 == 0) BM_VARIANT(BM_Q6K, 2, 0)                                                               \
         else BM_VARIANT(BM_Q6K, 1, 0)                                                                                  \
         break;                                                                                                         \
     case BM_IQ2XXS:                                                                                                    \
-        if ((nb) % 4 == 0) BM_VARIANT(BM_IQ2XXS, 4, 0)                                                                 \
+        if ((nb) % 2 == 0) BM_VARIANT(BM_IQ2XXS, 2, 0)                                                                 \
         else BM_VARIANT(BM_IQ2XXS, 1, 0)                                                                               \
         break;                                                                                                         \
     default:                                                                                                           \
@@ -911,7 +957,7 @@ hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8
         hipLaunchKernelGGL(kern, dim3(grid_a), dim3(256), lds_a, L.stream, x, wg, wu, (u32)n_experts, nba, nbb, sel,   \
                            spt, act_x, act_h, h, L.fault, L.layer);                                                    \
     }
-    if (nba == 8) BM_GUX(8, 8)
+    if (nba == 8) BM_GUX(kRingQ4K, 8)
     else BM_GUX(1, 0)
 #undef BM_GUX
     return hipGetLastError();
@@ -943,12 +989,12 @@ hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, c
                            wts, resid, spt, m, act_x, act_h, h, y, counters, spin_limit, L.fault, L.layer);            \
     }
     if (down_type == BM_Q6K) {
-        if (nba == 8 && nbb == 3) BM_FUSED(BM_Q4K, 8, 8, BM_Q6K, 3, 3)
-        else if (nba == 8) BM_FUSED(BM_Q4K, 8, 8, BM_Q6K, 1, 0)
-        else if (nbb == 3) BM_FUSED(BM_Q4K, 1, 0, BM_Q6K, 3, 3)
+        if (nba == 8 && nbb == 3) BM_FUSED(BM_Q4K, kRingQ4K, 8, BM_Q6K, kRingQ6K, 3)
+        else if (nba == 8) BM_FUSED(BM_Q4K, kRingQ4K, 8, BM_Q6K, 1, 0)
+        else if (nbb == 3) BM_FUSED(BM_Q4K, 1, 0, BM_Q6K, kRingQ6K, 3)
         else BM_FUSED(BM_Q4K, 1, 0, BM_Q6K, 1, 0)
     } else if (down_type == BM_Q4K) {
-        if (nba == 8) BM_FUSED(BM_Q4K, 8, 8, BM_Q4K, 1, 0)
+        if (nba == 8) BM_FUSED(BM_Q4K, kRingQ4K, 8, BM_Q4K, 1, 0)
         else BM_FUSED(BM_Q4K, 1, 0, BM_Q4K, 1, 0)
     } else {
         return hipErrorInvalidValue;

@@ -64,6 +64,12 @@ SYMBOLS = {
     "bm_set_spin_limit": (_i, [_vp, _u32]),
     "bm_set_decode_plan": (_i, [_vp, _i]),
     "bm_gate_up_x": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
+    "bm_tile_cap": (_i, [_i, _i]),
+    "bm_buckets": (_i, [_vp, _vp, _i, _i, _vp, _vp]),
+    "bm_tiles": (_i, [_vp, _vp, _i, _i, _vp]),
+    "bm_quantize_ord": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "bm_gate_up_tiles": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
+    "bm_gemv_tiles": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
     "bm_block_sums": (_i, [_vp, _vp, _i64, _vp, _i, _vp]),
     "bm_capture_begin": (_i, [_vp]),
     "bm_capture_end": (_i, [_vp, C.POINTER(_vp)]),
@@ -330,6 +336,29 @@ class Gpu:
 
     def set_spin_limit(self, spins):
         self._check(self.lib.bm_set_spin_limit(self.ctx, spins))
+
+    # -- grouped decode: the slot table by expert and the tile launchers
+    def tile_cap(self, n_slots, n_experts):
+        return self.lib.bm_tile_cap(n_slots, n_experts)
+
+    def enqueue_buckets(self, sel, n_slots, n_experts, order, start):
+        self._check(self.lib.bm_buckets(self.ctx, _ptr(sel), n_slots, n_experts, _ptr(order), _ptr(start)))
+
+    def enqueue_tiles(self, start, n_experts, n_slots, tiles):
+        self._check(self.lib.bm_tiles(self.ctx, _ptr(start), n_experts, n_slots, _ptr(tiles)))
+
+    def enqueue_quantize_ord(self, x, start, n_experts, m_cols, act):
+        self._check(self.lib.bm_quantize_ord(self.ctx, _ptr(x), _ptr(start), n_experts, m_cols, act.handle))
+
+    def enqueue_gate_up_tiles(self, wg, wu, act, order, start, tiles, n_slots, rows_per_expert, slots_per_col, h,
+                              act_h=None):
+        self._check(self.lib.bm_gate_up_tiles(self.ctx, wg.handle, wu.handle, act.handle, _ptr(order), _ptr(start),
+                                              _ptr(tiles), n_slots, rows_per_expert, slots_per_col, _ptr(h),
+                                              act_h.handle if act_h is not None else None))
+
+    def enqueue_gemv_tiles(self, w, act, order, start, tiles, n_slots, rows_per_expert, y):
+        self._check(self.lib.bm_gemv_tiles(self.ctx, w.handle, act.handle, _ptr(order), _ptr(start), _ptr(tiles),
+                                           n_slots, rows_per_expert, _ptr(y)))
 
     def enqueue_block_sums(self, w, row, act, col, out):
         self._check(self.lib.bm_block_sums(self.ctx, w.handle, row, act.handle, col, _ptr(out)))

@@ -527,6 +527,106 @@ int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const
                                   ctx->counters, ctx->spin_limit));
 }
 
+// ------------------------------------------------------------------------------------------ grouped decode
+
+int bm_tile_cap(int n_slots, int n_experts) {
+    if (n_slots < 0 || n_experts < 1) return BM_ESHAPE;
+    return bmk::tile_cap(n_slots, n_experts);
+}
+
+int bm_buckets(bm_ctx *ctx, const uint32_t *sel_dev, int n_slots, int n_experts, uint32_t *order_dev, uint32_t *start_dev) {
+    const char *what = "bm_buckets";
+    if (!ctx || !sel_dev || !order_dev || !start_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (n_experts < 1 || n_experts > bmk::kBucketExperts || n_slots < 1 || n_slots > bmk::kTileMaxSlots)
+        return fail(ctx, BM_ESHAPE, "%s: %d places over %d experts (1..=%d experts, 1..=%d places)", what, n_slots, n_experts,
+                    bmk::kBucketExperts, bmk::kTileMaxSlots);
+    return driver(ctx, what, bmk::buckets(launch_of(ctx), sel_dev, n_slots, n_experts, order_dev, start_dev));
+}
+
+int bm_tiles(bm_ctx *ctx, const uint32_t *start_dev, int n_experts, int n_slots, uint32_t *tiles_dev) {
+    const char *what = "bm_tiles";
+    if (!ctx || !start_dev || !tiles_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (n_experts < 1 || n_experts > bmk::kBucketExperts || n_slots < 1 || n_slots > bmk::kTileMaxSlots)
+        return fail(ctx, BM_ESHAPE, "%s: %d slots over %d experts (1..=%d experts, at most %d slots)", what, n_slots, n_experts,
+                    bmk::kBucketExperts, bmk::kTileMaxSlots);
+    return driver(ctx, what, bmk::tiles(launch_of(ctx), start_dev, n_experts, n_slots, tiles_dev));
+}
+
+int bm_quantize_ord(bm_ctx *ctx, const float *x_dev, const uint32_t *start_dev, int n_experts, int m_cols, bm_act *act) {
+    const char *what = "bm_quantize_ord";
+    if (!ctx || !x_dev || !start_dev || !act) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (n_experts < 1) return fail(ctx, BM_ESHAPE, "%s: n_experts = %d", what, n_experts);
+    if (m_cols < 1 || m_cols > act->m_cap)
+        return fail(ctx, BM_ESHAPE, "%s: %d columns of %d values into %d columns", what, m_cols, act->k, act->m_cap);
+    return driver(ctx, what, bmk::quantize(launch_of(ctx), act->wtype, x_dev, m_cols, act->k, act->dev, start_dev + n_experts));
+}
+
+// The table arguments every tile launcher takes.
+static int check_table(bm_ctx *ctx, const char *what, const uint32_t *order, const uint32_t *start, const uint32_t *tiles,
+                       int n_slots, int n_experts) {
+    if (!order || !start || !tiles) return fail(ctx, BM_EARG, "%s: NULL table", what);
+    if (n_experts > bmk::kBucketExperts)
+        return fail(ctx, BM_ESHAPE, "%s: the stack holds %d experts, a tile word names at most %d", what, n_experts, bmk::kBucketExperts);
+    if (n_slots < 1 || n_slots > bmk::kTileMaxSlots)
+        return fail(ctx, BM_ESHAPE, "%s: n_slots = %d outside 1..=%d", what, n_slots, bmk::kTileMaxSlots);
+    return BM_OK;
+}
+
+int bm_gate_up_tiles(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_act *act, const uint32_t *order_dev,
+                     const uint32_t *start_dev, const uint32_t *tiles_dev, int n_slots, int rows_per_expert,
+                     int slots_per_col, float *h_dev, bm_act *act_h) {
+    const char *what = "bm_gate_up_tiles";
+    if (!ctx || !wg || !wu || !act) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (!h_dev && !act_h) return fail(ctx, BM_EARG, "%s: neither h_dev nor act_h to write", what);
+    if (wg->wtype != wu->wtype)
+        return fail(ctx, BM_ETYPE, "%s: gate is type %d and up type %d; one launch reads one type", what, wg->wtype, wu->wtype);
+    int rc = check_pair(ctx, what, wg, act);
+    if (rc) return rc;
+    if (wu->k != wg->k || wu->rows != wg->rows)
+        return fail(ctx, BM_ESHAPE, "%s: gate is %lld x %d, up %lld x %d", what, (long long)wg->rows, wg->k, (long long)wu->rows, wu->k);
+    int n_experts = 0;
+    rc = check_stack(ctx, what, wg, rows_per_expert, &n_experts);
+    if (!rc) rc = check_table(ctx, what, order_dev, start_dev, tiles_dev, n_slots, n_experts);
+    if (rc) return rc;
+    if (slots_per_col < 1) return fail(ctx, BM_ESHAPE, "%s: slots_per_col = %d must be at least 1", what, slots_per_col);
+    if ((int64_t)n_slots > (int64_t)act->m_cap * slots_per_col)
+        return fail(ctx, BM_ESHAPE, "%s: n_slots %d needs %d columns at %d slots a column, act holds %d", what, n_slots,
+                    (n_slots + slots_per_col - 1) / slots_per_col, slots_per_col, act->m_cap);
+    uint8_t *ah = nullptr;
+    if (act_h) {
+        if (act_form(act_h->wtype) != 0)
+            return fail(ctx, BM_ETYPE, "%s: the fused quantizer writes Q8_2_X4 columns; act_h was made for type %d (Q8_K)", what, act_h->wtype);
+        if (act_h->k != rows_per_expert)
+            return fail(ctx, BM_ESHAPE, "%s: act_h columns hold k = %d values, an entry writes rows_per_expert = %d", what, act_h->k, rows_per_expert);
+        if (act_h->m_cap < n_slots)
+            return fail(ctx, BM_ESHAPE, "%s: a column of act_h per table entry: %d slots, act_h holds %d", what, n_slots, act_h->m_cap);
+        ah = act_h->dev;
+    }
+    if (bmk::tiles_lds(wg->wtype, wg->k) == 0)
+        return fail(ctx, BM_ESHAPE, "%s: eight columns of k = %d do not fit the workgroup's LDS; use bm_gate_up", what, wg->k);
+    return driver(ctx, what, bmk::gate_up_tiles(launch_of(ctx), wg->wtype, wg->dev, wu->dev, n_experts, wg->k, act->dev, act->m_cap,
+                                                order_dev, start_dev, tiles_dev, n_slots, rows_per_expert, slots_per_col, h_dev, ah));
+}
+
+int bm_gemv_tiles(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const uint32_t *order_dev, const uint32_t *start_dev,
+                  const uint32_t *tiles_dev, int n_slots, int rows_per_expert, float *y_dev) {
+    const char *what = "bm_gemv_tiles";
+    if (!ctx || !w || !act || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    int rc = check_pair(ctx, what, w, act);
+    if (rc) return rc;
+    int n_experts = 0;
+    rc = check_stack(ctx, what, w, rows_per_expert, &n_experts);
+    if (!rc) rc = check_table(ctx, what, order_dev, start_dev, tiles_dev, n_slots, n_experts);
+    if (rc) return rc;
+    if (act->m_cap < n_slots)
+        return fail(ctx, BM_ESHAPE, "%s: an activation column per table entry: act.m() = %d must be at least n_slots = %d", what,
+                    act->m_cap, n_slots);
+    if (bmk::tiles_lds(w->wtype, w->k) == 0)
+        return fail(ctx, BM_ESHAPE, "%s: eight columns of k = %d do not fit the workgroup's LDS; use bm_gemv_sel", what, w->k);
+    return driver(ctx, what, bmk::gemv_tiles(launch_of(ctx), w->wtype, w->dev, n_experts, w->k, act->dev, order_dev, start_dev,
+                                             tiles_dev, n_slots, rows_per_expert, y_dev));
+}
+
 int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *act, int col, int32_t *out_dev) {
     const char *what = "bm_block_sums";
     if (!ctx || !w || !act || !out_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);

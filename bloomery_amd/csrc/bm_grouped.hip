@@ -1,0 +1,278 @@
+// Grouped decode: the routed expert chain of several tokens with each expert's rows read once for up to eight of
+// its slots. The tables are the reference's (crates/gpu/src/q4k_sel.rs:20-41): `order` lists the card's slots by
+// expert, expert e's run is order[start[e] .. start[e + 1]], and the tile table cuts every run into tiles of up to
+// eight consecutive entries, tile g the word (e << 22) | j at tiles[1 + g], their count at tiles[0]. Every slot's
+// value is its slot-by-slot launch's, bit for bit: a column of the multi-column dot is the one-column dot.
+#include "bm_stream.cuh"
+
+namespace bmk {
+
+constexpr u32 kHostSlot = 0xffffffffu; // crates/gpu/src/host/slots.rs:10
+
+int tile_cap(int n_slots, int n_experts) { // crates/gpu/src/q4k_sel.rs:96-98
+    const long a = ((long)n_slots + (long)(kTileCols - 1) * n_experts) / kTileCols;
+    return (int)(a < n_slots ? a : n_slots);
+}
+
+// ---------------------------------------------------------------------------------------------- tables
+
+// crates/gpu/src/q4k_sel.rs:480-560 grouped_buckets: one workgroup of 1024 threads, a thread an expert. Slots keep
+// their order inside a run. An id at or past the stack that is not the host's raises ExpertId and joins no run.
+__global__ __launch_bounds__(1024) void k_buckets(const u32 *sel, u32 n_slots, u32 n_experts, u32 *order, u32 *start,
+                                                  u32 *fault, u32 layer) {
+    __shared__ u32 count[kBucketExperts];
+    const u32 tid = threadIdx.x;
+    for (u32 s = tid; s < n_slots; s += blockDim.x) {
+        const u32 p = sel[s];
+        if (p >= n_experts && p != kHostSlot) bm_raise(fault, layer, kSiteExpertId);
+    }
+    if (tid < n_experts) {
+        u32 c = 0;
+        for (u32 s = 0; s < n_slots; s++) c += sel[s] == tid;
+        count[tid] = c;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        u32 at = 0;
+        for (u32 e = 0; e < n_experts; e++) {
+            const u32 c = count[e];
+            start[e] = at;
+            count[e] = at;
+            at += c;
+        }
+        start[n_experts] = at;
+    }
+    __syncthreads();
+    if (tid < n_experts) {
+        u32 at = count[tid];
+        for (u32 s = 0; s < n_slots; s++)
+            if (sel[s] == tid) order[at++] = s;
+    }
+}
+
+// crates/gpu/src/q4k_sel.rs:562-680 grouped_tiles. A run outside 0 .. start[n_experts] <= n_slots, or more tiles
+// than `cap`, raise ExpertId and leave a count of 0.
+__global__ __launch_bounds__(1024) void k_tiles(const u32 *start, u32 n_experts, u32 n_slots, u32 cap, u32 *tiles,
+                                                u32 *fault, u32 layer) {
+    __shared__ u32 at[kBucketExperts];
+    __shared__ u32 total;
+    const u32 tid = threadIdx.x;
+    const u32 end = start[n_experts];
+    if (tid < n_experts) {
+        const u32 j0 = start[tid], j1 = start[tid + 1];
+        at[tid] = (j0 <= j1 && j1 <= end && end <= n_slots) ? (j1 - j0 + kTileCols - 1) / kTileCols : 0xffffffffu;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        u32 sum = 0;
+        for (u32 e = 0; e < n_experts; e++) {
+            const u32 c = at[e];
+            if (c == 0xffffffffu || c > cap - sum) {
+                sum = 0xffffffffu;
+                break;
+            }
+            at[e] = sum;
+            sum += c;
+        }
+        if (sum == 0xffffffffu) {
+            bm_raise(fault, layer, kSiteExpertId);
+            sum = 0;
+        }
+        total = sum;
+        tiles[0] = sum;
+    }
+    __syncthreads();
+    if (tid < n_experts && total != 0) {
+        u32 g = at[tid];
+        for (u32 j = start[tid], j1 = start[tid + 1]; j < j1; j += kTileCols) tiles[1 + g++] = (tid << kTileExpertShift) | j;
+    }
+}
+
+hipError_t buckets(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start) {
+    hipLaunchKernelGGL(k_buckets, dim3(1), dim3(1024), 0, L.stream, sel, (u32)n_slots, (u32)n_experts, order, start,
+                       L.fault, L.layer);
+    return hipGetLastError();
+}
+
+hipError_t tiles(const Launch &L, const uint32_t *start, int n_experts, int n_slots, uint32_t *tiles_out) {
+    hipLaunchKernelGGL(k_tiles, dim3(1), dim3(1024), 0, L.stream, start, (u32)n_experts, (u32)n_slots,
+                       (u32)tile_cap(n_slots, n_experts), tiles_out, L.fault, L.layer);
+    return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------- tile kernels
+
+// A launch's workgroup as every tile kernel reads it (crates/gpu/src/q4k_sel.rs:101-151 tile_at, :186-234
+// tile_block): workgroup b is tile g = b mod cap of row block b / cap. False: no tile (past the count, or a word
+// that names no run of the table, which raises ExpertId).
+struct Tile {
+    int e, j, m, row_block;
+};
+__device__ __forceinline__ bool tile_of_block(const u32 *tiles, const u32 *start, u32 n_experts, u32 n_slots, u32 cap,
+                                              Tile *t, u32 *fault, u32 layer) {
+    const u32 g = blockIdx.x % cap;
+    t->row_block = (int)(blockIdx.x / cap);
+    if (g >= tiles[0]) return false;
+    const u32 word = tiles[1 + g];
+    const u32 e = word >> kTileExpertShift, j = word & ((1u << kTileExpertShift) - 1);
+    const u32 j1 = e < n_experts ? start[e + 1] : 0;
+    if (!(j < j1 && j1 <= n_slots)) {
+        if (threadIdx.x == 0) bm_raise(fault, layer, kSiteExpertId);
+        return false;
+    }
+    t->e = (int)e;
+    t->j = (int)j;
+    t->m = (int)(j1 - j < (u32)kTileCols ? j1 - j : (u32)kTileCols);
+    return true;
+}
+
+// The tile's m activation columns into LDS, column c from `src_col(c)` of act (a column index, or -1: none).
+template <class ColOf>
+__device__ __forceinline__ void stage_tile_cols(uint8_t *cols, const uint8_t *act, int col_bytes, int m,
+                                                const ColOf &src_col) {
+    for (int c = 0; c < m; c++) {
+        const int sc = src_col(c);
+        if (sc >= 0) stage_bytes(cols + (size_t)c * col_bytes, act + (size_t)sc * col_bytes, col_bytes);
+    }
+}
+
+// crates/gpu/src/kquant/tiles.rs:62-118 GateUpTiles: workgroup = tile x 32 rows of the tile's expert, eight lanes a
+// row (a quad on the gate row, a quad on the up row), all m columns in one pass over the two rows. Entry j + c reads
+// the activation column of the token of slot order[j + c] and writes h[(j + c) * rpe + r]: by entry, not by slot.
+// With act_h the 32 values of each column become block rb of column j + c of act_h in the same launch.
+template <int WT, int U, int NB>
+__global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const uint8_t *wu, u32 n_experts, int nb,
+                                                       const uint8_t *act, int act_cols, const u32 *order,
+                                                       const u32 *start, const u32 *tiles, u32 n_slots, u32 cap,
+                                                       int rpe, int slots_per_col, float *h, uint8_t *act_h,
+                                                       u32 *fault, u32 layer) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
+    Tile t;
+    if (!tile_of_block(tiles, start, n_experts, n_slots, cap, &t, fault, layer)) return;
+    const int rb = t.row_block;
+    const int r = rb * 32 + (tid >> 3);
+    const bool active = r < rpe;
+    const int n = NB > 0 ? NB : nb;
+    const int nb_h = rpe / 256;
+    const int col_bytes = bm_act_col_bytes<WT>(n);
+    const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
+    const uint8_t *wrow = (which ? wu : wg) + ((size_t)t.e * rpe + (active ? r : 0)) * row_bytes;
+    Blk<WT> b[U];
+    preload<WT, U>(b, wrow, q);
+    const Iq2Tables tb = stage_tables<WT>(lds);
+    uint8_t *cols = lds + tab_bytes<WT>();
+    float *hbuf = reinterpret_cast<float *>(cols + (size_t)kTileCols * col_bytes); // [8][32]
+    u32 *bad = reinterpret_cast<u32 *>(hbuf + kTileCols * 32);                      // [8]: entry names no slot
+    if (tid < kTileCols) {
+        const u32 s = tid < t.m ? order[t.j + tid] : 0;
+        const bool none = tid < t.m && (s >= n_slots || (int)(s / slots_per_col) >= act_cols);
+        if (none) bm_raise(fault, layer, kSiteExpertId);
+        bad[tid] = none ? 0xffffffffu : s / slots_per_col;
+    }
+    __syncthreads();
+    stage_tile_cols(cols, act, col_bytes, t.m, [&](int c) { return bad[c] == 0xffffffffu ? 0 : (int)bad[c]; });
+    __syncthreads();
+    float v[kTileCols];
+    row_dot<WT, U, NB, kTileCols>(b, wrow, cols, col_bytes, t.m, n, q, tb, v, NoTap{});
+#pragma unroll
+    for (int c = 0; c < kTileCols; c++) {
+        float hv = swiglu_of_pair(v[c], which);
+        if (c < t.m) {
+            if (bad[c] == 0xffffffffu) hv = bm_bits_f32(0x7fc00000u);
+            if (h && active && (tid & 7) == 0) h[(size_t)(t.j + c) * rpe + r] = hv;
+            if (act_h && (tid & 7) == 0) hbuf[c * 32 + (tid >> 3)] = hv;
+        }
+    }
+    if (act_h) { // rpe is a multiple of 256 here, so every row of the block is live
+        __syncthreads();
+        const int c = tid >> 5; // half wave c: column c
+        if (c < t.m)
+            quantize_h_block(hbuf + c * 32, act_h + (size_t)(t.j + c) * nb_h * BM_Q82_SB_EXT, nb_h, rb, tid & 31, fault,
+                             layer);
+    }
+}
+
+// crates/gpu/src/kquant/tiles.rs:120-190 GemvTiles: workgroup = tile x 64 rows (a quad a row); entry j + c reads
+// column j + c of act and writes row r of its slot order[j + c]. An entry that names no slot raises ExpertId.
+template <int WT, int U, int NB>
+__global__ __launch_bounds__(256) void k_gemv_tiles(const uint8_t *w, u32 n_experts, int nb, const uint8_t *act,
+                                                    const u32 *order, const u32 *start, const u32 *tiles, u32 n_slots,
+                                                    u32 cap, int rpe, float *y, u32 *fault, u32 layer) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, q = tid & 3;
+    Tile t;
+    if (!tile_of_block(tiles, start, n_experts, n_slots, cap, &t, fault, layer)) return;
+    const int r = t.row_block * 64 + (tid >> 2);
+    const bool active = r < rpe;
+    const int n = NB > 0 ? NB : nb;
+    const int col_bytes = bm_act_col_bytes<WT>(n);
+    const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
+    const uint8_t *wrow = w + ((size_t)t.e * rpe + (active ? r : 0)) * row_bytes;
+    Blk<WT> b[U];
+    preload<WT, U>(b, wrow, q);
+    const Iq2Tables tb = stage_tables<WT>(lds);
+    uint8_t *cols = lds + tab_bytes<WT>();
+    u32 *slot_of = reinterpret_cast<u32 *>(cols + (size_t)kTileCols * col_bytes); // [8]
+    if (tid < kTileCols) {
+        const u32 s = tid < t.m ? order[t.j + tid] : 0;
+        if (tid < t.m && s >= n_slots && t.row_block == 0) bm_raise(fault, layer, kSiteExpertId);
+        slot_of[tid] = s;
+    }
+    stage_bytes(cols, act + (size_t)t.j * col_bytes, t.m * col_bytes); // the tile's columns lie side by side
+    __syncthreads();
+    float v[kTileCols];
+    row_dot<WT, U, NB, kTileCols>(b, wrow, cols, col_bytes, t.m, n, q, tb, v, NoTap{});
+    if (q == 0 && active) {
+#pragma unroll
+        for (int c = 0; c < kTileCols; c++)
+            if (c < t.m && slot_of[c] < n_slots) y[(size_t)slot_of[c] * rpe + r] = v[c];
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ launchers
+
+size_t tiles_lds(int wtype, int k) {
+    const size_t lds = tab_bytes_rt(wtype) + (size_t)kTileCols * act_col_bytes(wtype, k) + kTileCols * 32 * sizeof(float) +
+                       kTileCols * sizeof(u32);
+    return lds <= (size_t)kMaxLds ? lds : 0;
+}
+
+hipError_t gate_up_tiles(const Launch &L, int wtype, const uint8_t *wg, const uint8_t *wu, int n_experts, int k,
+                         const uint8_t *act, int act_cols, const uint32_t *order, const uint32_t *start,
+                         const uint32_t *tiles_dev, int n_slots, int rows_per_expert, int slots_per_col, float *h,
+                         uint8_t *act_h) {
+    const int nb = k / 256, rpe = rows_per_expert;
+    const size_t lds = tiles_lds(wtype, k);
+    const u32 cap = (u32)tile_cap(n_slots, n_experts);
+    const unsigned grid = cap * (unsigned)((rpe + 31) / 32);
+#define CALL_BODY                                                                                                      \
+    auto kern = k_gate_up_tiles<WT, U, NB>;                                                                            \
+    hipError_t e = allow_lds(kern, lds);                                                                               \
+    if (e != hipSuccess) return e;                                                                                     \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, wg, wu, (u32)n_experts, nb, act, act_cols, order,   \
+                       start, tiles_dev, (u32)n_slots, cap, rpe, slots_per_col, h, act_h, L.fault, L.layer);
+    BM_DISPATCH(wtype, nb)
+#undef CALL_BODY
+    return hipGetLastError();
+}
+
+hipError_t gemv_tiles(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const uint8_t *act,
+                      const uint32_t *order, const uint32_t *start, const uint32_t *tiles_dev, int n_slots,
+                      int rows_per_expert, float *y) {
+    const int nb = k / 256, rpe = rows_per_expert;
+    const size_t lds = tiles_lds(wtype, k);
+    const u32 cap = (u32)tile_cap(n_slots, n_experts);
+    const unsigned grid = cap * (unsigned)((rpe + 63) / 64);
+#define CALL_BODY                                                                                                      \
+    auto kern = k_gemv_tiles<WT, U, NB>;                                                                               \
+    hipError_t e = allow_lds(kern, lds);                                                                               \
+    if (e != hipSuccess) return e;                                                                                     \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act, order, start,           \
+                       tiles_dev, (u32)n_slots, cap, rpe, y, L.fault, L.layer);
+    BM_DISPATCH(wtype, nb)
+#undef CALL_BODY
+    return hipGetLastError();
+}
+
+} // namespace bmk

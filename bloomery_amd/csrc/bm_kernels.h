@@ -23,7 +23,9 @@ hipError_t fill_u32(const Launch &L, uint32_t *dst, uint32_t value, size_t n);
 // path's bytes, and for the Q8_2_X4 form two tables after them (bm_device.cuh).
 int act_col_bytes(int wtype, int k);
 
-hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, uint8_t *act);
+// `live` (optional): a device word holding how many of the m columns to quantize; the rest keep what they held.
+hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, uint8_t *act,
+                    const uint32_t *live = nullptr);
 
 // Rebuilds the tables of m Q8_2_X4 device columns whose reference bytes were just written by a copy.
 hipError_t q82_tables(const Launch &L, uint8_t *act, int m, int k);
@@ -65,6 +67,27 @@ hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, c
                       const uint8_t *wu, const uint8_t *wd, int n_experts, int hidden, int ff, const uint32_t *sel,
                       const float *wts, const float *resid, int slots_per_token, int m, uint8_t *act_x,
                       uint8_t *act_h, float *h, float *y, uint32_t *counters, uint32_t spin_limit);
+
+// ------------------------------------------------------------------------------ grouped decode (bm_grouped.hip)
+
+// crates/gpu/src/q4k_sel.rs:68-97: a tile is up to 8 consecutive entries of one expert's run; word (e << 22) | j.
+constexpr int kTileCols = 8;
+constexpr int kTileExpertShift = 22;
+constexpr int kBucketExperts = 1024;
+constexpr int kTileMaxSlots = 1 << kTileExpertShift;
+int tile_cap(int n_slots, int n_experts);
+
+hipError_t buckets(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start);
+hipError_t tiles(const Launch &L, const uint32_t *start, int n_experts, int n_slots, uint32_t *tiles);
+// LDS bytes a tile launch of this type and k asks for (0 if eight columns do not fit a workgroup's LDS).
+size_t tiles_lds(int wtype, int k);
+hipError_t gate_up_tiles(const Launch &L, int wtype, const uint8_t *wg, const uint8_t *wu, int n_experts, int k,
+                         const uint8_t *act, int act_cols, const uint32_t *order, const uint32_t *start,
+                         const uint32_t *tiles, int n_slots, int rows_per_expert, int slots_per_col, float *h,
+                         uint8_t *act_h);
+hipError_t gemv_tiles(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const uint8_t *act,
+                      const uint32_t *order, const uint32_t *start, const uint32_t *tiles, int n_slots,
+                      int rows_per_expert, float *y);
 
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out);
 

@@ -1,181 +1,11 @@
-// HIP kernels of the quantized MoE expert matmul for gfx950, and their launch functions.
-//
-// Every dot kernel follows one plan: a quad of lanes per weight row (bm_device.cuh); the token's quantized
-// activation column requested first, then the row's super-blocks (128-bit loads) through a small ring of
-// registers, a few super-blocks ahead of the arithmetic, all from straight-line code so the hardware's in-order
-// load counter lets the arithmetic of one super-block run while the later ones are still in flight. Weights are
-// read once, straight from the file's block bytes.
-//
-// Variants: a kernel is instantiated per weight type and per (U, NB): U the ring's size in super-blocks, NB the
-// row's super-block count when it is known at compile time (0: a run-time count that U divides). The hot shapes
-// (Q4_K rows of 2048 values, Q6_K rows of 768) have NB set and their stages unrolled.
+// HIP kernels of the quantized MoE expert matmul for gfx950, decode side, and their launch functions: the
+// activation quantizers, the dense gemv, the routed expert chain slot by slot (gate . up . SwiGLU, down, combine),
+// its fused forms, and the block-sum verification kernel.
 #include "bm_kernels.h"
 
-#define BM_TABLE_QUAL __device__ const
-#include "iq2xxs_tables.h"
-
-#include "bm_device.cuh"
+#include "bm_stream.cuh"
 
 namespace bmk {
-
-constexpr u32 kSiteQuantColumn = 1; // crates/device/src/fault.rs:73-76
-constexpr u32 kSiteExpertId = 7;    // crates/device/src/fault.rs:89
-constexpr u32 kSiteStalled = 31;    // ours: a fused launch's down workgroup gave up waiting for its activations
-
-// LDS bytes of the IQ2_XXS tables: 2048 grid + 128 signs + 64 nibble masks, padded to a 16-byte multiple.
-constexpr int kTabBytes = 2048 + 128 + 64 + 64;
-
-template <int WT>
-__host__ __device__ constexpr int tab_bytes() {
-    return WT == BM_IQ2XXS ? kTabBytes : 0;
-}
-
-template <int WT>
-__device__ __forceinline__ Iq2Tables stage_tables(uint8_t *lds) {
-    Iq2Tables tb{nullptr, nullptr, nullptr};
-    if constexpr (WT == BM_IQ2XXS) {
-        uint2 *grid = reinterpret_cast<uint2 *>(lds);
-        uint8_t *ks = lds + 2048;
-        u32 *nm = reinterpret_cast<u32 *>(lds + 2048 + 128);
-        for (int t = threadIdx.x; t < 256; t += blockDim.x) {
-            const uint64_t g = BM_IQ2XXS_GRID[t];
-            grid[t] = make_uint2((u32)g, (u32)(g >> 32));
-        }
-        for (int t = threadIdx.x; t < 128; t += blockDim.x) ks[t] = BM_KSIGNS_IQ2XS[t];
-        for (int t = threadIdx.x; t < 16; t += blockDim.x)
-            nm[t] = ((t & 1) ? 0xffu : 0u) | ((t & 2) ? 0xff00u : 0u) | ((t & 4) ? 0xff0000u : 0u) |
-                    ((t & 8) ? 0xff000000u : 0u);
-        tb.grid = grid;
-        tb.ksigns = ks;
-        tb.nibmask = nm;
-    }
-    return tb;
-}
-
-// `bytes` (a multiple of 8) from 8-byte aligned global memory to 8-byte aligned LDS, by the whole workgroup.
-__device__ __forceinline__ void stage_bytes(uint8_t *dst, const uint8_t *src, int bytes) {
-    for (int o = threadIdx.x * 8; o < bytes; o += blockDim.x * 8)
-        *reinterpret_cast<uint2 *>(dst + o) = *reinterpret_cast<const uint2 *>(src + o);
-}
-
-// The same copy in two halves: R unconditional loads a thread (offsets past the end are clamped onto the last
-// word, so no branch stands between them and the weight loads that follow), then the LDS stores. Memory returns
-// in order, so the stores wait for these loads only. Bytes past R * 8 * blockDim are copied afterwards by
-// stage_bytes' loop (that part waits for everything in flight).
-template <int R>
-struct Stage {
-    uint2 v[R];
-    __device__ __forceinline__ void load(const uint8_t *src, int bytes) {
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            int o = (r * (int)blockDim.x + (int)threadIdx.x) * 8;
-            o = o < bytes ? o : bytes - 8;
-            v[r] = *reinterpret_cast<const uint2 *>(src + o);
-        }
-        // keep these loads ahead of whatever is requested next: the in-order wait depends on it
-        __asm__ volatile("" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    __device__ __forceinline__ void store(uint8_t *dst, const uint8_t *src, int bytes) const {
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            const int o = (r * (int)blockDim.x + (int)threadIdx.x) * 8;
-            if (o < bytes) *reinterpret_cast<uint2 *>(dst + o) = v[r];
-        }
-        for (int o = (R * (int)blockDim.x + (int)threadIdx.x) * 8; o < bytes; o += (int)blockDim.x * 8)
-            *reinterpret_cast<uint2 *>(dst + o) = *reinterpret_cast<const uint2 *>(src + o);
-    }
-};
-
-// The weight stream of a row is a ring of U super-blocks in registers: the first U - 1 are requested up front
-// (preload), and each stage requests the super-block U - 1 ahead of the one it is about to use before it starts its
-// arithmetic. A wave that asks for a whole row at once sits in the memory pipeline's queue until most of it has
-// arrived and only then starts to compute; with the ring the requests trickle out between the stages and the
-// arithmetic runs under the stream.
-template <int WT, int U>
-__device__ __forceinline__ void preload(Blk<WT> (&b)[U], const uint8_t *wrow, int q) {
-#pragma unroll
-    for (int u = 0; u + 1 < U; u++) b[u] = bm_load_blk<WT>(wrow, u, q);
-}
-
-// One stage: request super-block `ahead` into its ring slot, read the next stage's activation operands from LDS,
-// then the arithmetic of super-block i (ring slot `slot`). The asm statements pin that order: the compiler may
-// neither hoist the reads of later stages nor sink this stage's sums past them.
-template <int WT, int U, class Tap>
-__device__ __forceinline__ void stage_one(Blk<WT> (&b)[U], int slot, int fill, const uint8_t *wrow, int ahead,
-                                          const ActView &av, int i, int act_next, int q, const Iq2Tables &tb,
-                                          Act<WT> &cur, float &a0, float &a1, const Tap &tap) {
-    __asm__ volatile("" ::: "memory");
-    if (U > 1) b[fill] = bm_load_blk<WT>(wrow, ahead, q);
-    const Act<WT> next = bm_load_act<WT, Tap::kActive>(av, act_next, q);
-    __asm__ volatile("" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-    if (U == 1) b[0] = bm_load_blk<WT>(wrow, i, q);
-    bm_dot_blk<WT>(b[slot], cur, i, q, tb, a0, a1, tap);
-    __asm__ volatile("" : "+v"(a0), "+v"(a1)::"memory");
-    __builtin_amdgcn_sched_barrier(0);
-    cur = next;
-}
-
-// Row `wrow` against `m` <= M columns (LDS, `col_stride` apart); b holds the ring, preloaded.
-// NB > 0: the row has NB super-blocks, the stages are unrolled; NB == 0: it has nb, a multiple of U.
-// Indices past the row's end are clamped onto its last super-block: a redundant read, no branch in the stream.
-template <int WT, int U, int NB, int M, class Tap>
-__device__ __forceinline__ void row_dot(Blk<WT> (&b)[U], const uint8_t *wrow, const uint8_t *cols, int col_stride,
-                                        int m, int nb, int q, const Iq2Tables &tb, float (&out)[M], const Tap &tap) {
-    float a0[M], a1[M];
-    ActView av[M];
-    const int n = NB > 0 ? NB : nb;
-#pragma unroll
-    for (int c = 0; c < M; c++) {
-        a0[c] = a1[c] = 0.0f;
-        av[c] = bm_act_view<WT>(cols + (size_t)c * col_stride, n);
-    }
-    if constexpr (M == 1) {
-        Act<WT> cur = bm_load_act<WT, Tap::kActive>(av[0], 0, q);
-        if constexpr (NB > 0) {
-#pragma unroll
-            for (int i = 0; i < NB; i++) {
-                const int ahead = i + U - 1 < NB ? i + U - 1 : NB - 1;
-                stage_one<WT, U>(b, i % U, (i + U - 1) % U, wrow, ahead, av[0], i, i + 1 < NB ? i + 1 : i, q, tb, cur,
-                                 a0[0], a1[0], tap);
-            }
-        } else {
-            for (int i0 = 0; i0 < n; i0 += U) {
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    const int i = i0 + u;
-                    const int ahead = i + U - 1 < n ? i + U - 1 : n - 1;
-                    stage_one<WT, U>(b, u, (u + U - 1) % U, wrow, ahead, av[0], i, i + 1 < n ? i + 1 : i, q, tb, cur,
-                                     a0[0], a1[0], tap);
-                }
-            }
-        }
-    } else {
-        // several columns: the same ring for the weights, the activation operands read where they are used
-        auto stage = [&](int slot, int fill, int i) {
-            const int ahead = i + U - 1 < n ? i + U - 1 : n - 1;
-            b[fill] = bm_load_blk<WT>(wrow, U > 1 ? ahead : i, q);
-#pragma unroll
-            for (int c = 0; c < M; c++)
-                if (c < m) {
-                    const Act<WT> a = bm_load_act<WT, Tap::kActive>(av[c], i, q);
-                    bm_dot_blk<WT>(b[slot], a, i, q, tb, a0[c], a1[c], tap);
-                }
-        };
-        if constexpr (NB > 0) {
-#pragma unroll
-            for (int i = 0; i < NB; i++) stage(i % U, (i + U - 1) % U, i);
-        } else {
-            for (int i0 = 0; i0 < n; i0 += U) {
-#pragma unroll
-                for (int u = 0; u < U; u++) stage(u, (u + U - 1) % U, i0 + u);
-            }
-        }
-    }
-#pragma unroll
-    for (int c = 0; c < M; c++) out[c] = bm_quad_finish<WT>(a0[c], a1[c]);
-}
 
 // ----------------------------------------------------------------------------------------------- fill
 
@@ -192,65 +22,14 @@ hipError_t fill_u32(const Launch &L, uint32_t *dst, uint32_t value, size_t n) {
 
 // ------------------------------------------------------------------------------------------- quantizers
 
-// What one q8_2 block's header needs beside its codes.
-struct Q82Head {
-    u32 t;    // bf16 scale bits
-    int isum; // sum of the unsaturated codes
-    bool bad; // a value that is not finite: NaN scale, zero codes (crates/gpu/src/lib.rs:925-933)
-};
-
-// One 32-value q8_2 block on an aligned group of 32 lanes, a value a lane (crates/qdot/src/lib.rs:3883-3904).
-// Returns the stored code; *s16 is the sum of the stored codes over the lane's aligned group of 16.
-__device__ __forceinline__ int q82_block(float v, Q82Head *hd, int *s16) {
-    const u32 ab = bm_max32(bm_f32_bits(v) & 0x7fffffffu);
-    if (ab > 0x7f7fffffu) {
-        hd->t = 0x7fc0u;
-        hd->isum = 0;
-        hd->bad = true;
-        *s16 = 0;
-        return 0;
-    }
-    const u32 t = bm_fp32_to_bf16_bits(__fdiv_rn(bm_bits_f32(ab), 127.0f));
-    const float id = bm_q82_inverse(t);
-    const int q = bm_nearest_int(__fmul_rn(v, id));
-    const int code = q < -128 ? -128 : (q > 127 ? 127 : q);
-    const int s = bm_sum16(q);
-    hd->t = t;
-    hd->isum = s + (int)bm_swap16((u32)s);
-    hd->bad = false;
-    *s16 = bm_sum16(code);
-    return code;
-}
-
-// Stores block `blk` of a device Q8_2_X4 column of nb super-blocks: codes, scale, sum and the two table entries.
-// Called by the block's 32 lanes with their `lane32`.
-__device__ __forceinline__ void q82_store(uint8_t *col, int nb, int blk, int lane32, int code, const Q82Head &hd,
-                                          int s16) {
-    uint8_t *group = col + (size_t)(blk >> 2) * BM_Q82X4_STRIDE;
-    const int ir = blk & 3;
-    // four codes a lane-quad -> one dword store from its first lane
-    u32 c = (u32)(code & 0xff);
-    c |= (bm_dpp<kDppShl1>(c) & 0xffu) << 8;
-    c |= (bm_dpp<kDppShl2>(c) & 0xffffu) << 16;
-    if ((lane32 & 3) == 0) *reinterpret_cast<u32 *>(group + 16 + 32 * ir + lane32) = c;
-    if ((lane32 & 15) == 0)
-        *reinterpret_cast<int *>(col + (size_t)nb * (BM_Q82_SB_REF + 64) + 4 * (2 * blk + (lane32 >> 4))) = s16;
-    if (lane32 == 0) {
-        *reinterpret_cast<unsigned short *>(group + 2 * ir) = (unsigned short)hd.t;
-        *reinterpret_cast<unsigned short *>(group + 8 + 2 * ir) = (unsigned short)(short)hd.isum;
-        const float d8 = bm_bf16_to_f32(hd.t);
-        *reinterpret_cast<float2 *>(col + (size_t)nb * BM_Q82_SB_REF + 8 * blk) =
-            make_float2(d8, __fmul_rn(d8, (float)(short)hd.isum));
-    }
-}
-
 // x: m columns of k values -> Q8_2_X4 columns. One half wave a 32-value block.
-__global__ __launch_bounds__(256) void k_quantize_q82x4(const float *x, int m, int k, uint8_t *act, u32 *fault,
-                                                        u32 layer) {
+__global__ __launch_bounds__(256) void k_quantize_q82x4(const float *x, int m, int k, uint8_t *act, const u32 *live,
+                                                        u32 *fault, u32 layer) {
     const int bpc = k / 32; // blocks a column
     const long gblk = (long)blockIdx.x * 8 + (threadIdx.x >> 5);
     if (gblk >= (long)m * bpc) return;
     const int col = (int)(gblk / bpc), blk = (int)(gblk % bpc), lane32 = threadIdx.x & 31;
+    if (live && (u32)col >= *live) return; // a device-side column count: the columns past it keep what they held
     const float v = x[(size_t)col * k + 32 * blk + lane32];
     Q82Head hd;
     int s16;
@@ -260,12 +39,13 @@ __global__ __launch_bounds__(256) void k_quantize_q82x4(const float *x, int m, i
 }
 
 // x: m columns of k values -> Q8_K columns (crates/qdot/src/lib.rs:1787-1809). One workgroup a 256-value block.
-__global__ __launch_bounds__(256) void k_quantize_q8k(const float *x, int m, int k, uint8_t *act, u32 *fault,
-                                                      u32 layer) {
+__global__ __launch_bounds__(256) void k_quantize_q8k(const float *x, int m, int k, uint8_t *act, const u32 *live,
+                                                      u32 *fault, u32 layer) {
     __shared__ unsigned long long s_key[4];
     __shared__ int s_codes[256];
     const int bpc = k / 256;
     const int col = blockIdx.x / bpc, blk = blockIdx.x % bpc, tid = threadIdx.x;
+    if (live && (u32)col >= *live) return;
     const float *xb = x + (size_t)col * k + 256 * blk;
     uint8_t *o = act + ((size_t)col * bpc + blk) * BM_Q8K_STRIDE;
     const float v = xb[tid];
@@ -315,14 +95,14 @@ __global__ __launch_bounds__(256) void k_quantize_q8k(const float *x, int m, int
     }
 }
 
-hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, uint8_t *act) {
+hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, uint8_t *act, const uint32_t *live) {
     if (wtype == BM_IQ2XXS) {
         hipLaunchKernelGGL(k_quantize_q8k, dim3((unsigned)(m * (k / 256))), dim3(256), 0, L.stream, x, m, k, act,
-                           L.fault, L.layer);
+                           live, L.fault, L.layer);
     } else {
         const long blocks = (long)m * (k / 32);
         hipLaunchKernelGGL(k_quantize_q82x4, dim3((unsigned)((blocks + 7) / 8)), dim3(256), 0, L.stream, x, m, k, act,
-                           L.fault, L.layer);
+                           live, L.fault, L.layer);
     }
     return hipGetLastError();
 }
@@ -382,23 +162,6 @@ __global__ __launch_bounds__(256) void k_gemv(const uint8_t *w, long rows, int n
 }
 
 // --------------------------------------------------------------------------------- gate . up . SwiGLU
-
-// The gate/up exchange of the eight lanes of an output: lanes 0..3 hold the gate dot, 4..7 the up dot.
-__device__ __forceinline__ float swiglu_of_pair(float v, int which) {
-    // both moves run on every lane: a lane-crossing move under a divergent branch reads switched-off lanes as 0
-    const float from_above = bm_dppf<kDppShl4>(v), from_below = bm_dppf<kDppShr4>(v);
-    return bm_swiglu(which ? from_below : v, which ? v : from_above);
-}
-
-// The 32 values a workgroup produced (hbuf, LDS) as block `rb` of column `hcol`, by the first 32 threads.
-__device__ __forceinline__ void quantize_h_block(const float *hbuf, uint8_t *hcol, int nb_h, int rb, int tid,
-                                                 u32 *fault, u32 layer) {
-    Q82Head hd;
-    int s16;
-    const int code = q82_block(hbuf[tid], &hd, &s16);
-    if (hd.bad && tid == 0) bm_raise(fault, layer, kSiteQuantColumn);
-    q82_store(hcol, nb_h, rb, tid, code, hd, s16);
-}
 
 // One workgroup = 32 consecutive rows of one slot; eight lanes a row: a quad on the gate row, a quad on the up row.
 // With act_h the 32 values are quantized to one q8_2 block of the slot's down activation in the same launch.
@@ -820,47 +583,10 @@ __global__ __launch_bounds__(64) void k_block_sums(const uint8_t *wrow, int nb, 
 
 // ---------------------------------------------------------------------------------------- launch helpers
 
-template <typename K>
-static hipError_t allow_lds(K kernel, size_t lds) {
-    if (lds <= 64 * 1024) return hipSuccess;
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                               (int)lds);
-}
-
-// Picks the kernel variant for a row of nb super-blocks and runs CALL_BODY with WT, U and NB as constants. Each
-// type lists the hot shape first (its count known at compile time, stages unrolled), then a ring of two for even
-// counts, then one super-block at a time, which divides every row.
-constexpr int kRingQ4K = 3, kRingQ6K = 2;
-#define BM_VARIANT(T, UU, NN)                                                                                          \
-    {                                                                                                                  \
-        constexpr int WT = T, U = UU, NB = NN;                                                                         \
-        CALL_BODY;                                                                                                     \
-    }
-#define BM_DISPATCH(wtype, nb)                                                                                         \
-    switch (wtype) {                                                                                                   \
-    case BM_Q4K:                                                                                                       \
-        if ((nb) == 8) BM_VARIANT(BM_Q4K, kRingQ4K, 8)                                                                 \
-        else if ((nb) % 2 == 0) BM_VARIANT(BM_Q4K, 2, 0)                                                               \
-        else BM_VARIANT(BM_Q4K, 1, 0)                                                                                  \
-        break;                                                                                                         \
-    case BM_Q6K:                                                                                                       \
-        if ((nb) == 3) BM_VARIANT(BM_Q6K, kRingQ6K, 3)                                                                 \
-        else if ((nb) % 2 == 0) BM_VARIANT(BM_Q6K, 2, 0)                                                               \
-        else BM_VARIANT(BM_Q6K, 1, 0)                                                                                  \
-        break;                                                                                                         \
-    case BM_IQ2XXS:                                                                                                    \
-        if ((nb) % 2 == 0) BM_VARIANT(BM_IQ2XXS, 2, 0)                                                                 \
-        else BM_VARIANT(BM_IQ2XXS, 1, 0)                                                                               \
-        break;                                                                                                         \
-    default:                                                                                                           \
-        return hipErrorInvalidValue;                                                                                   \
-    }
-
 int act_col_bytes(int wtype, int k) {
     const int nb = k / 256;
     return wtype == BM_IQ2XXS ? nb * BM_Q8K_STRIDE : nb * BM_Q82_SB_EXT;
 }
-static int tab_bytes_rt(int wtype) { return wtype == BM_IQ2XXS ? kTabBytes : 0; }
 
 int gemv_max_cols(int wtype, int k) {
     int m = (kMaxLds - tab_bytes_rt(wtype)) / act_col_bytes(wtype, k);

@@ -185,6 +185,42 @@ int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const 
  * the default is 1 << 18. */
 int bm_set_spin_limit(bm_ctx *ctx, uint32_t spins);
 
+/* ------------------------------------------------------------- decode of several tokens: grouped by expert */
+
+/* The grouped slot table (crates/gpu/src/q4k_sel.rs:20-41). Buffers the caller holds on the device:
+ *   order[n_slots]      the card's slots listed by expert, ascending inside a run;
+ *   start[n_experts+1]  expert e's run is order[start[e] .. start[e + 1]]; start[n_experts] = slots listed;
+ *   tiles[cap + 1]      cap = bm_tile_cap(n_slots, n_experts): tiles[0] = count, tiles[1 + g] = (e << 22) | j,
+ *                       tile g = up to 8 consecutive entries of expert e's run from entry j.
+ * The layouts are the reference's, so a caller's tables interchange. At most 1024 experts, 2^22 slots. */
+
+/* tile_cap (crates/gpu/src/q4k_sel.rs:96): min(n_slots, (n_slots + 7 * n_experts) / 8). */
+int bm_tile_cap(int n_slots, int n_experts);
+/* Q4kSelKernels::enqueue_buckets (crates/gpu/src/q4k_sel.rs:1103): order and start from sel_dev[n_slots]. An id
+ * at or past n_experts joins no run and, unless it is BM_HOST_SLOT, raises BM_SITE_EXPERT_ID. */
+int bm_buckets(bm_ctx *ctx, const uint32_t *sel_dev, int n_slots, int n_experts, uint32_t *order_dev, uint32_t *start_dev);
+/* Q4kSelKernels::enqueue_grouped_tiles (crates/gpu/src/q4k_sel.rs:1152): the tile table of start_dev. A run
+ * outside the table raises BM_SITE_EXPERT_ID and leaves a count of 0. */
+int bm_tiles(bm_ctx *ctx, const uint32_t *start_dev, int n_experts, int n_slots, uint32_t *tiles_dev);
+/* Q4kSelKernels::enqueue_quantize_ord (crates/gpu/src/q4k_sel.rs:1255): the first start_dev[n_experts] columns
+ * of x_dev (at most m_cols, the columns launched) into the same columns of act, bm_quantize's bytes; every other
+ * column keeps what it held. */
+int bm_quantize_ord(bm_ctx *ctx, const float *x_dev, const uint32_t *start_dev, int n_experts, int m_cols, bm_act *act);
+/* The grouped gate . up (crates/gpu/src/kquant/tiles.rs:62-118,1055; kq_card_gather :10-14 folded in): table
+ * entry j is slot order[j]; it reads the activation column of its token (column order[j] / slots_per_col of act)
+ * and writes h_dev[j * rows_per_expert + r] - by entry, not by slot - bm_gate_up's value for that slot. An expert's
+ * rows are read once for up to eight of its slots. act_h (optional, Q8_2_X4, k = rows_per_expert): column j gets
+ * the quantized rows of entry j in the same launch (the reference's bm_quantize_ord step). An entry that names no
+ * slot raises BM_SITE_EXPERT_ID and writes NaN. */
+int bm_gate_up_tiles(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_act *act, const uint32_t *order_dev,
+                     const uint32_t *start_dev, const uint32_t *tiles_dev, int n_slots, int rows_per_expert,
+                     int slots_per_col, float *h_dev, bm_act *act_h);
+/* Q4kSelKernels::enqueue_gemv_q4k_tiles (crates/gpu/src/q4k_sel.rs:1208; Q5K/Q6K/IQ forms kquant/tiles.rs:120-190):
+ * the grouped down. Entry j reads column j of act and writes y_dev[order[j] * rows_per_expert + r], bm_gemv_sel's
+ * value for that slot. An entry that names no slot raises BM_SITE_EXPERT_ID and writes nothing. */
+int bm_gemv_tiles(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const uint32_t *order_dev, const uint32_t *start_dev,
+                  const uint32_t *tiles_dev, int n_slots, int rows_per_expert, float *y_dev);
+
 /* ------------------------------------------------------------------------------------------- verification */
 
 /* The exact per-block integers the kernels above form for row `row` of w against column `col` of act, written

@@ -218,6 +218,39 @@ def combine_tokens(down, w, resid, rows, n_slots, m):
     return y
 
 
+TILE_COLS, TILE_E_SHIFT, HOST_SLOT = 8, 22, 0xFFFFFFFF
+
+
+def tile_cap(n_slots, n_experts):
+    """crates/gpu/src/q4k_sel.rs:96-98."""
+    return min(n_slots, (n_slots + (TILE_COLS - 1) * n_experts) // TILE_COLS)
+
+
+def grouped_table(sel, n_experts):
+    """The grouped slot table and its tile table by definition (crates/gpu/src/q4k_sel.rs:20-41, grouped_buckets
+    :480-560, grouped_tiles :562-680): order = the slots by expert, ascending inside a run; start = the runs' bounds;
+    tiles = [count, (e << 22) | j ...] with j stepping by 8 through each run, padded with zeros to tile_cap + 1
+    words. Ids at or past n_experts (the host's included) join no run. Returns (order, start, tiles, refused) with
+    refused = an id past the stack that is not the host's was met."""
+    sel = np.asarray(sel, np.uint32).reshape(-1)
+    n_slots = sel.size
+    order = [s for e in range(n_experts) for s in range(n_slots) if int(sel[s]) == e]
+    start = [0]
+    for e in range(n_experts):
+        start.append(start[-1] + int(np.count_nonzero(sel == e)))
+    words = []
+    for e in range(n_experts):
+        for j in range(start[e], start[e + 1], TILE_COLS):
+            words.append((e << TILE_E_SHIFT) | j)
+    cap = tile_cap(n_slots, n_experts)
+    assert len(words) <= cap
+    tiles = np.zeros(cap + 1, np.uint32)
+    tiles[0] = len(words)
+    tiles[1:1 + len(words)] = words
+    refused = bool(np.any((sel >= n_experts) & (sel != HOST_SLOT)))
+    return (np.asarray(order + [0] * (n_slots - len(order)), np.uint32), np.asarray(start, np.uint32), tiles, refused)
+
+
 def quantize_rows(wtype, x, rows, k, n_threads=8):
     """rows x k f32 -> GGUF block bytes, rows back to back."""
     x = _f32(x).reshape(rows, k)

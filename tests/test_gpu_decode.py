@@ -257,11 +257,17 @@ def route(rng, m, n_experts, top_k, bias=None):
 
 
 class Layer:
-    def __init__(self, gpu, types, hidden, ff, n_experts, seed):
+    def __init__(self, gpu, types, hidden, ff, n_experts, seed, cheap=False):
         self.types, self.hidden, self.ff, self.n_experts = types, hidden, ff, n_experts
-        self.wg = stack(types[0], n_experts * ff, hidden, seed)
-        self.wu = stack(types[1], n_experts * ff, hidden, seed + 1)
-        self.wd = stack(types[2], n_experts * hidden, ff, seed + 2)
+        if cheap:  # random legal blocks: a large stack without the quantizers' search
+            rng = np.random.default_rng(seed)
+            self.wg = random_blocks(types[0], n_experts * ff, hidden, rng)
+            self.wu = random_blocks(types[1], n_experts * ff, hidden, rng)
+            self.wd = random_blocks(types[2], n_experts * hidden, ff, rng)
+        else:
+            self.wg = stack(types[0], n_experts * ff, hidden, seed)
+            self.wu = stack(types[1], n_experts * ff, hidden, seed + 1)
+            self.wd = stack(types[2], n_experts * hidden, ff, seed + 2)
         self.dg = gpu.weights(types[0], n_experts * ff, hidden, self.wg)
         self.du = gpu.weights(types[1], n_experts * ff, hidden, self.wu)
         self.dd = gpu.weights(types[2], n_experts * hidden, ff, self.wd)
@@ -458,6 +464,139 @@ def test_uploaded_columns_dot_like_quantized_ones(gpu):
         assert_f32(y.download(), ora.gemv(wtype, w, rows, k, np.concatenate(cols), 2), f"type {wtype}")
         for b in (dw, act, y):
             b.free()
+
+
+# ------------------------------------------------------------------------------- several tokens, grouped by expert
+
+def grouped_tables_on_device(gpu, ids_flat, n_experts):
+    n_slots = ids_flat.size
+    cap = gpu.tile_cap(n_slots, n_experts)
+    assert cap == ora.tile_cap(n_slots, n_experts)
+    sel = gpu.upload(ids_flat, np.uint32)
+    order, start = gpu.buffer(np.uint32, n_slots).fill_bytes(0), gpu.buffer(np.uint32, n_experts + 1).fill_bytes(0xFF)
+    tiles = gpu.buffer(np.uint32, cap + 1).fill_bytes(0)
+    gpu.enqueue_buckets(sel, n_slots, n_experts, order, start)
+    gpu.enqueue_tiles(start, n_experts, n_slots, tiles)
+    return sel, order, start, tiles
+
+
+@pytest.mark.parametrize("n_experts,n_slots,seed", ((128, 128, 1), (7, 40, 2), (1, 9, 3), (1024, 64, 4), (16, 1, 5)))
+def test_grouped_tables_are_the_definition(gpu, n_experts, n_slots, seed):
+    """order, start and the tile words against the table's definition (gate_q4k_sel's table clauses,
+    crates/gpu-gates/src/bin/gate_q4k_sel.rs)."""
+    rng = np.random.default_rng(seed)
+    ids = rng.integers(0, n_experts, n_slots).astype(np.uint32)
+    if n_slots > 8:
+        ids[3] = bm.HOST_SLOT      # served elsewhere: in no run, silently
+    gpu.fault_clear()
+    sel, order, start, tiles = grouped_tables_on_device(gpu, ids, n_experts)
+    want_order, want_start, want_tiles, refused = ora.grouped_table(ids, n_experts)
+    listed = int(want_start[-1])
+    assert np.array_equal(start.download(), want_start)
+    assert np.array_equal(order.download()[:listed], want_order[:listed])
+    got_tiles = tiles.download()
+    assert got_tiles[0] == want_tiles[0] and np.array_equal(got_tiles[1:1 + got_tiles[0]], want_tiles[1:1 + want_tiles[0]])
+    assert not refused and gpu.fault() == (bm.FAULT_NONE, 0)
+    for b in (sel, order, start, tiles):
+        b.free()
+
+
+def test_grouped_tables_refuse_bad_ids_and_bad_runs(gpu):
+    ids = np.array([2, 9, 1, 2], np.uint32)   # 9 is past a stack of 4
+    gpu.fault_clear()
+    gpu.set_layer(3)
+    sel, order, start, tiles = grouped_tables_on_device(gpu, ids, 4)
+    assert gpu.fault(3) == ((3 << 8) | bm.SITE_EXPERT_ID, 1 << bm.SITE_EXPERT_ID)
+    assert np.array_equal(start.download(), [0, 0, 1, 3, 3]) and np.array_equal(order.download()[:3], [2, 0, 3])
+    # a run that ends past the table: no tiles, ExpertId (crates/gpu/src/q4k_sel.rs:606-651)
+    gpu.fault_clear()
+    start.upload(np.array([0, 2, 9, 3, 3], np.uint32))
+    gpu.enqueue_tiles(start, 4, 4, tiles)
+    assert tiles.download()[0] == 0 and gpu.fault(3)[0] == (3 << 8) | bm.SITE_EXPERT_ID
+    gpu.set_layer(bm.LAYER_NONE)
+    gpu.fault_clear()
+    for b in (sel, order, start, tiles):
+        b.free()
+
+
+def run_grouped(gpu, L, x, ids, wts, top_k, fused_quant):
+    """buckets -> tiles -> gate.up by tiles (-> quantize_ord) -> down by tiles -> combine: the reference's grouped
+    decode (crates/gpu/src/arch/qwen3moe/dispatch.rs grouped branch; crates/gpu/src/kquant/tiles.rs)."""
+    m = x.shape[0]
+    n_slots = m * top_k
+    sel, order, start, tiles = grouped_tables_on_device(gpu, ids.reshape(-1), L.n_experts)
+    act = gpu.act(L.types[0], L.hidden, m)
+    act_h = gpu.act(L.types[2], L.ff, n_slots)
+    xd, wd = gpu.upload(x, np.float32), gpu.upload(wts, np.float32)
+    h = gpu.buffer(np.float32, n_slots * L.ff).fill_bytes(0xFF)
+    down = gpu.buffer(np.float32, n_slots * L.hidden).fill_bytes(0xFF)
+    y = gpu.buffer(np.float32, m * L.hidden).fill_bytes(0xFF)
+    gpu.enqueue_quantize(xd, m, act)
+    if fused_quant and L.types[2] != bm.IQ2_XXS:
+        gpu.enqueue_gate_up_tiles(L.dg, L.du, act, order, start, tiles, n_slots, L.ff, top_k, h, act_h)
+    else:
+        gpu.enqueue_gate_up_tiles(L.dg, L.du, act, order, start, tiles, n_slots, L.ff, top_k, h)
+        gpu.enqueue_quantize_ord(h, start, L.n_experts, n_slots, act_h)
+    gpu.enqueue_gemv_tiles(L.dd, act_h, order, start, tiles, n_slots, L.hidden, down)
+    gpu.enqueue_combine_tokens(down, wd, None, L.hidden, top_k, m, y)
+    out = y.download(), h.download(), order.download(), down.download()
+    for b in (sel, order, start, tiles, act, act_h, xd, wd, h, down, y):
+        b.free()
+    return out
+
+
+@pytest.mark.parametrize("types,hidden,ff,n_experts,m,top_k", (
+    ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 16, 16, 8),   # config 3's shape with 16 experts resident: long runs
+    ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 128, 16, 8),  # config 3: 128 slots over 128 experts, skewed
+    ((bm.Q6_K, bm.Q6_K, bm.Q4_K), 512, 512, 3, 7, 2),
+    ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ2_XXS), 1024, 512, 5, 6, 3),
+    ((bm.IQ2_XXS, bm.IQ2_XXS, bm.Q6_K), 768, 256, 4, 5, 4),
+))
+@pytest.mark.parametrize("fused_quant", (False, True))
+def test_grouped_layer_matches_slot_by_slot(gpu, types, hidden, ff, n_experts, m, top_k, fused_quant):
+    """Every slot of the grouped path holds its slot-by-slot value bit for bit (crates/gpu/src/kquant/tiles.rs:5-9);
+    here against the oracle's slot-major layer on the same tokens."""
+    if n_experts == 128:
+        L = Layer(gpu, types, hidden, ff, n_experts, 1100, cheap=True)
+    else:
+        L = Layer(gpu, types, hidden, ff, n_experts, 1000 + hidden + n_experts)
+    rng = np.random.default_rng(1001)
+    x = normal_f32(rng, (m, hidden))
+    bias = normal_f32(rng, n_experts, 0.5) if n_experts == 128 else None
+    ids, wts = route(rng, m, n_experts, top_k, bias)
+    gpu.fault_clear()
+    y, h, order, down = run_grouped(gpu, L, x, ids, wts, top_k, fused_quant)
+    want_y, want_h = L.oracle(x, ids, wts, top_k)
+    n_slots = m * top_k
+    h, want_h = h.reshape(n_slots, ff), want_h.reshape(n_slots, ff)
+    assert_f32(h, want_h[order], "h by table entry")   # entry j holds slot order[j]
+    assert_f32(y, want_y, "y")
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    L.free()
+
+
+def test_grouped_skips_host_slots_and_refuses_stale_entries(gpu):
+    L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 4, 1200)
+    rng = np.random.default_rng(1201)
+    m, top_k = 3, 2
+    x = normal_f32(rng, (m, 512))
+    ids = np.array([[1, bm.HOST_SLOT], [2, 1], [0, 3]], np.uint32)
+    wts = normal_f32(rng, (m, top_k))
+    gpu.fault_clear()
+    y, h, order, down = run_grouped(gpu, L, x, ids, wts, top_k, True)
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    down = down.reshape(m * top_k, 512)
+    assert np.all(down[1].view(np.uint32) == 0xFFFFFFFF), "the host's slot keeps what it held"
+    live = ids.copy()
+    live[0, 1] = 1   # any live id: the slot's value is not compared
+    _, want_h = L.oracle(x, live, wts, top_k)
+    for s in (0, 2, 3, 4, 5):
+        e = int(ids.reshape(-1)[s])
+        rb = ora.row_bytes(bm.Q6_K, 256)
+        want = ora.gemv(bm.Q6_K, L.wd[e * 512 * rb:(e + 1) * 512 * rb], 512, 256,
+                        ora.quantize_col(bm.Q6_K, want_h[s * 256:(s + 1) * 256]), 1)
+        assert_f32(down[s], want, f"slot {s}")
+    L.free()
 
 
 def test_slot_equals_one_expert_gemv_and_duplicate_ids(gpu):

@@ -237,3 +237,16 @@ def test_layer_refuses_bad_ids():
     x = np.ones(256, np.float32)
     with pytest.raises(ora.OracleError):
         ora.moe_forward(256, 256, 2, types, wg, wu, wd, x, np.array([2], np.uint32), np.array([1.0], np.float32), 1)
+
+
+def test_grouped_table_by_hand():
+    """The slot table and tile words of crates/gpu/src/q4k_sel.rs:20-41,562-680 on cases small enough to write out."""
+    order, start, tiles, refused = ora.grouped_table([2, 0, 2, 1, 2], 3)
+    assert list(order) == [1, 3, 0, 2, 4] and list(start) == [0, 1, 2, 5] and not refused
+    assert list(tiles[:4]) == [3, (0 << 22) | 0, (1 << 22) | 1, (2 << 22) | 2]
+    # a run of nine entries cuts into a tile of eight and a tile of one; the host's slot and a stale id join no run
+    sel = [1] * 9 + [0xFFFFFFFF, 7]
+    order, start, tiles, refused = ora.grouped_table(sel, 2)
+    assert list(start) == [0, 0, 9] and list(order[:9]) == list(range(9)) and refused
+    assert list(tiles[:3]) == [2, (1 << 22) | 0, (1 << 22) | 8]
+    assert ora.tile_cap(11, 2) == 3 and ora.tile_cap(128, 128) == 128 and ora.tile_cap(16384, 128) == 2160

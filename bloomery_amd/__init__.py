@@ -70,6 +70,12 @@ SYMBOLS = {
     "bm_quantize_ord": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "bm_gate_up_tiles": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "bm_gemv_tiles": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "bm_route_create": (_i, [_vp, _i, _i, C.POINTER(_vp)]),
+    "bm_route_destroy": (None, [_vp]),
+    "bm_route_fill": (_i, [_vp, _vp, _i, _vp]),
+    "bm_route_read": (_i, [_vp, _vp, _vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
+    "bm_gemm": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp]),
+    "bm_swiglu_quant": (_i, [_vp, _vp, _vp, _i, _vp]),
     "bm_block_sums": (_i, [_vp, _vp, _i64, _vp, _i, _vp]),
     "bm_capture_begin": (_i, [_vp]),
     "bm_capture_end": (_i, [_vp, C.POINTER(_vp)]),
@@ -199,6 +205,36 @@ class Q8Act:
     def free(self):
         if self.handle:
             self.gpu.lib.bm_act_destroy(self.handle)
+            self.handle = None
+
+
+class Route:
+    """A prefill route table (GemmRoute, crates/gpu/src/gemm/route.rs:109)."""
+
+    def __init__(self, gpu, max_slots, n_experts):
+        self.gpu, self.max_slots, self.n_experts = gpu, max_slots, n_experts
+        h = _vp()
+        gpu._check(gpu.lib.bm_route_create(gpu.ctx, max_slots, n_experts, C.byref(h)))
+        self.handle = h
+
+    def fill(self, ids, n_slots):
+        self.gpu._check(self.gpu.lib.bm_route_fill(self.gpu.ctx, _ptr(ids), n_slots, self.handle))
+        self.n_slots = n_slots
+
+    def read(self):
+        """(cols, tiles as rows of (expert, start, len), refused count) of the last fill."""
+        cap = self.n_slots // 64 + min(self.n_experts, self.n_slots)
+        cols = np.empty(self.n_slots, np.uint32)
+        tiles = np.zeros(2 * cap, np.uint32)
+        n, r = _i(), _i()
+        self.gpu._check(self.gpu.lib.bm_route_read(self.gpu.ctx, self.handle, cols.ctypes.data_as(_vp),
+                                                   tiles.ctypes.data_as(_vp), C.byref(n), C.byref(r)))
+        t = tiles[:2 * n.value].reshape(-1, 2)
+        return cols, np.stack([t[:, 0], t[:, 1] & 0xFFFF, t[:, 1] >> 16], axis=1), r.value
+
+    def free(self):
+        if self.handle:
+            self.gpu.lib.bm_route_destroy(self.handle)
             self.handle = None
 
 
@@ -359,6 +395,17 @@ class Gpu:
     def enqueue_gemv_tiles(self, w, act, order, start, tiles, n_slots, rows_per_expert, y):
         self._check(self.lib.bm_gemv_tiles(self.ctx, w.handle, act.handle, _ptr(order), _ptr(start), _ptr(tiles),
                                            n_slots, rows_per_expert, _ptr(y)))
+
+    # -- prefill
+    def route(self, max_slots, n_experts):
+        return Route(self, max_slots, n_experts)
+
+    def enqueue_gemm(self, w, rows_per_expert, act, route, top_k, y):
+        """top_k > 0: every slot of a token reads the token's column; 0: a column a slot."""
+        self._check(self.lib.bm_gemm(self.ctx, w.handle, rows_per_expert, act.handle, route.handle, top_k, _ptr(y)))
+
+    def enqueue_swiglu_quant(self, g, u, n_cols, act):
+        self._check(self.lib.bm_swiglu_quant(self.ctx, _ptr(g), _ptr(u), n_cols, act.handle))
 
     def enqueue_block_sums(self, w, row, act, col, out):
         self._check(self.lib.bm_block_sums(self.ctx, w.handle, row, act.handle, col, _ptr(out)))

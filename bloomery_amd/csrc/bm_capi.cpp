@@ -627,6 +627,110 @@ int bm_gemv_tiles(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const uin
                                              tiles_dev, n_slots, rows_per_expert, y_dev));
 }
 
+// ------------------------------------------------------------------------------------------------ prefill
+
+struct bm_route {
+    bm_ctx *ctx;
+    int max_slots, n_experts;
+    int filled; // the slot count of the last fill, 0: never filled
+    uint32_t *cols, *tiles, *n_tiles;
+};
+
+int bm_route_create(bm_ctx *ctx, int max_slots, int n_experts, bm_route **out) {
+    const char *what = "bm_route_create";
+    if (!ctx || !out) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    *out = nullptr;
+    if (max_slots < 1 || max_slots > bmk::kGemmMaxSlots)
+        return fail(ctx, BM_ESHAPE, "%s: 1 <= max_slots <= %d, got %d", what, bmk::kGemmMaxSlots, max_slots);
+    if (n_experts < 1 || n_experts > bmk::kGemmMaxExperts)
+        return fail(ctx, BM_ESHAPE, "%s: 1 <= n_experts <= %d, got %d", what, bmk::kGemmMaxExperts, n_experts);
+    bm_route *r = new (std::nothrow) bm_route{ctx, max_slots, n_experts, 0, nullptr, nullptr, nullptr};
+    if (!r) return fail(ctx, BM_EDRIVER, "%s: out of host memory", what);
+    const size_t words = (size_t)max_slots + 2 * (size_t)bmk::gemm_max_tiles(max_slots, n_experts) + 2;
+    hipError_t e = hipMalloc((void **)&r->cols, words * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMemset(r->cols, 0, words * sizeof(uint32_t));
+    if (e != hipSuccess) {
+        if (r->cols) (void)hipFree(r->cols);
+        delete r;
+        return driver(ctx, what, e);
+    }
+    r->tiles = r->cols + max_slots;
+    r->n_tiles = r->tiles + 2 * (size_t)bmk::gemm_max_tiles(max_slots, n_experts);
+    *out = r;
+    return BM_OK;
+}
+
+void bm_route_destroy(bm_route *route) {
+    if (!route) return;
+    (void)hipFree(route->cols);
+    delete route;
+}
+
+int bm_route_fill(bm_ctx *ctx, const uint32_t *ids_dev, int n_slots, bm_route *route) {
+    const char *what = "bm_route_fill";
+    if (!ctx || !ids_dev || !route) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (n_slots < 1 || n_slots > route->max_slots)
+        return fail(ctx, BM_ESHAPE, "%s: 1 <= n_slots <= the table's %d slots, got %d", what, route->max_slots, n_slots);
+    int rc = driver(ctx, what, bmk::route(launch_of(ctx), ids_dev, n_slots, route->n_experts, route->cols, route->tiles, route->n_tiles));
+    if (!rc) route->filled = n_slots;
+    return rc;
+}
+
+int bm_route_read(bm_ctx *ctx, const bm_route *route, uint32_t *cols_host, uint32_t *tiles_host, int *n_tiles, int *n_refused) {
+    const char *what = "bm_route_read";
+    if (!ctx || !route || !n_tiles || !n_refused) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (!route->filled) return fail(ctx, BM_ESHAPE, "%s: the table was never filled", what);
+    uint32_t counts[2];
+    int rc = bm_dev_download(ctx, counts, route->n_tiles, sizeof counts);
+    if (rc) return rc;
+    const int cap = bmk::gemm_max_tiles(route->filled, route->n_experts);
+    if ((int)counts[0] > cap || (int)counts[1] > route->filled)
+        return fail(ctx, BM_ESHAPE, "%s: tile count %u (of %d) or refused count %u (of %d slots) is past the table", what, counts[0], cap,
+                    counts[1], route->filled);
+    *n_tiles = (int)counts[0];
+    *n_refused = (int)counts[1];
+    if (cols_host) rc = bm_dev_download(ctx, cols_host, route->cols, sizeof(uint32_t) * (size_t)route->filled);
+    if (!rc && tiles_host && counts[0]) rc = bm_dev_download(ctx, tiles_host, route->tiles, sizeof(uint32_t) * 2 * counts[0]);
+    return rc;
+}
+
+int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act *act, const bm_route *route, int top_k, float *y_dev) {
+    const char *what = "bm_gemm";
+    if (!ctx || !w || !act || !route || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (!route->filled) return fail(ctx, BM_ESHAPE, "%s: a filled route table (bm_route_fill first)", what);
+    if (!bmk::gemm_supported(w->wtype))
+        return fail(ctx, BM_ETYPE, "%s: weight type %d has no grouped GEMM here (Q4_K and Q6_K do); use the tile launchers", what, w->wtype);
+    int rc = check_pair(ctx, what, w, act);
+    if (rc) return rc;
+    if (rows_per_expert <= 0 || rows_per_expert % 16 != 0)
+        return fail(ctx, BM_ESHAPE, "%s: rows_per_expert must be a positive multiple of 16, got %d", what, rows_per_expert);
+    if (w->rows != (int64_t)route->n_experts * rows_per_expert)
+        return fail(ctx, BM_ESHAPE, "%s: the stack has %lld rows, the route %d experts of %d rows", what, (long long)w->rows,
+                    route->n_experts, rows_per_expert);
+    const int n_slots = route->filled;
+    int slot_div = 1;
+    if (top_k > 0) {
+        if (n_slots % top_k != 0) return fail(ctx, BM_ESHAPE, "%s: %d slots are not whole tokens of top_k %d", what, n_slots, top_k);
+        slot_div = top_k;
+    } else if (top_k < 0) {
+        return fail(ctx, BM_ESHAPE, "%s: top_k = %d (0: a column a slot)", what, top_k);
+    }
+    if (act->m_cap < n_slots / slot_div)
+        return fail(ctx, BM_ESHAPE, "%s: %d slots read %d activation columns, act holds %d", what, n_slots, n_slots / slot_div, act->m_cap);
+    return driver(ctx, what, bmk::gemm(launch_of(ctx), w->wtype, w->dev, route->n_experts, rows_per_expert, w->k, act->dev, route->cols,
+                                       route->tiles, route->n_tiles, n_slots, slot_div, y_dev));
+}
+
+int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, bm_act *act) {
+    const char *what = "bm_swiglu_quant";
+    if (!ctx || !g_dev || !u_dev || !act) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (act_form(act->wtype) != 0)
+        return fail(ctx, BM_ETYPE, "%s: writes Q8_2_X4 columns; act was made for type %d (Q8_K)", what, act->wtype);
+    if (n_cols < 1 || n_cols > act->m_cap)
+        return fail(ctx, BM_ESHAPE, "%s: n_cols = %d columns, act holds %d", what, n_cols, act->m_cap);
+    return driver(ctx, what, bmk::swiglu_quant(launch_of(ctx), g_dev, u_dev, n_cols, act->k, act->dev));
+}
+
 int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *act, int col, int32_t *out_dev) {
     const char *what = "bm_block_sums";
     if (!ctx || !w || !act || !out_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);

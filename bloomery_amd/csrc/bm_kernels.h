@@ -89,6 +89,22 @@ hipError_t gemv_tiles(const Launch &L, int wtype, const uint8_t *w, int n_expert
                       const uint32_t *order, const uint32_t *start, const uint32_t *tiles, int n_slots,
                       int rows_per_expert, float *y);
 
+// ------------------------------------------------------------------------------------- prefill (bm_prefill.hip)
+
+// crates/gpu/src/gemm/mod.rs:97-101, route.rs:11-13.
+constexpr int kGemmBN = 64, kGemmBM = 64;
+constexpr int kGemmMaxSlots = 40960, kGemmMaxExperts = 1024;
+int gemm_max_tiles(int n_slots, int n_experts);
+// cols[n_slots], tiles[2 * gemm_max_tiles], n_tiles[2]
+hipError_t route(const Launch &L, const uint32_t *ids, int n_slots, int n_experts, uint32_t *cols, uint32_t *tiles,
+                 uint32_t *n_tiles);
+hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act);
+bool gemm_supported(int wtype);
+// slot_div: slots a token when every slot of a token reads the token's column, 1 when each slot reads its own.
+hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int rows_per_expert, int k,
+                const uint8_t *act, const uint32_t *cols, const uint32_t *tiles, const uint32_t *n_tiles, int n_slots,
+                int slot_div, float *y);
+
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out);
 
 } // namespace bmk

@@ -1,0 +1,435 @@
+// Prefill: the grouped expert GEMM over a route table, on the int8 matrix cores, and the SwiGLU quantizer between
+// a gate/up pair and its down (crates/gpu/src/gemm/mod.rs:1-50).
+//
+// The route table is the reference's (crates/gpu/src/gemm/route.rs:1-60,109-125): `cols` lists the slots grouped by
+// expert, ascending slot order inside an expert, the refused slots (an id past the stack) at its end; `tiles` holds
+// a pair of words a tile, (expert, first index | length << 16), tiles of at most 64 slots; `n_tiles` = {tile count,
+// refused count}.
+//
+// The GEMM's numbers are the decode path's, bit for bit: every (row, slot) value is the one-column row dot of
+// bm_device.cuh. The integer sums of each 16-value group come out of v_mfma_i32_32x32x16_i8 (one instruction a
+// group: 32 rows x 32 slots x 16 values, exact), and each enters the f32 accumulator of the CPU path's lane that
+// owns it, in the CPU path's order (crates/qdot/src/lib.rs:4363-4447 Q4_K, :4776-4874 Q6_K): eight accumulators a
+// value, the min term first, then the groups in increasing k, and the closing sum (t0 + t2) + (t1 + t3).
+// Activation scales come per 32 values in this form, so every group's sum is scaled on the vector ALU before it is
+// added: three operations a (row, slot, group) against one matrix instruction per 1024 of them. The kernel is bound
+// by that arithmetic, not by the matrix cores.
+#include "bm_stream.cuh"
+
+namespace bmk {
+
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr u32 kNoExpert = 0xffffffffu;
+constexpr int kRouteThreads = 1024, kRouteWaves = kRouteThreads / 64, kRouteHist = 8192;
+
+int gemm_max_tiles(int n_slots, int n_experts) { // crates/gpu/src/gemm/route.rs:55-57
+    return n_slots / kGemmBN + (n_experts < n_slots ? n_experts : n_slots);
+}
+
+// ------------------------------------------------------------------------------------------------ route
+
+// One workgroup. The slots are cut into up to 16 chunks, a wave a chunk; counts per (chunk, expert) in LDS give
+// every chunk its place inside every expert's run, so the waves place their slots independently and each run stays
+// in ascending slot order. Bucket n_experts collects the refused slots.
+__global__ __launch_bounds__(kRouteThreads) void k_route(const u32 *ids, u32 n_slots, u32 n_experts, u32 *cols,
+                                                         u32 *tiles, u32 *n_tiles, u32 *fault, u32 layer) {
+    __shared__ u32 hist[kRouteHist + kRouteWaves]; // [chunk][bucket], bucket in 0..=n_experts
+    __shared__ u32 base[kGemmMaxExperts + 2];      // first index of every bucket's run
+    __shared__ u32 tile_at[kGemmMaxExperts + 1];
+    const u32 tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const u32 nbk = n_experts + 1;
+    u32 chunks = kRouteHist / nbk;
+    chunks = chunks < (u32)kRouteWaves ? chunks : (u32)kRouteWaves;
+    const u32 per = (n_slots + chunks - 1) / chunks;
+    for (u32 i = tid; i < chunks * nbk; i += blockDim.x) hist[i] = 0;
+    __syncthreads();
+    if (wave < chunks) {
+        const u32 lo = wave * per, hi = lo + per < n_slots ? lo + per : n_slots;
+        for (u32 s = lo + lane; s < hi; s += 64) {
+            const u32 id = ids[s];
+            const u32 b = id < n_experts ? id : n_experts;
+            if (b == n_experts) bm_raise(fault, layer, kSiteExpertId);
+            atomicAdd(&hist[wave * nbk + b], 1u);
+        }
+    }
+    __syncthreads();
+    for (u32 b = tid; b < nbk; b += blockDim.x) { // counts a chunk -> the chunk's offset inside the bucket's run
+        u32 sum = 0;
+        for (u32 c = 0; c < chunks; c++) {
+            const u32 v = hist[c * nbk + b];
+            hist[c * nbk + b] = sum;
+            sum += v;
+        }
+        base[b] = sum; // the bucket's count, for now
+    }
+    __syncthreads();
+    if (tid == 0) {
+        u32 at = 0, t = 0;
+        for (u32 e = 0; e < n_experts; e++) {
+            const u32 c = base[e];
+            base[e] = at;
+            tile_at[e] = t;
+            at += c;
+            t += (c + kGemmBN - 1) / kGemmBN;
+        }
+        const u32 refused = base[n_experts];
+        base[n_experts] = at;      // the refused slots close the list
+        base[n_experts + 1] = at + refused;
+        tile_at[n_experts] = t;
+        n_tiles[0] = t;
+        n_tiles[1] = refused;
+    }
+    __syncthreads();
+    if (wave < chunks) {
+        volatile u32 *off = &hist[wave * nbk];
+        const u32 lo = wave * per, hi = lo + per < n_slots ? lo + per : n_slots;
+        for (u32 s0 = lo; s0 < hi; s0 += 64) {
+            const u32 s = s0 + lane;
+            u32 b = kNoExpert;
+            if (s < hi) {
+                const u32 id = ids[s];
+                b = id < n_experts ? id : n_experts;
+            }
+            unsigned long long todo = __ballot(b != kNoExpert);
+            while (todo) { // the lanes of one bucket at a time, in lane (= slot) order
+                const int leader = __builtin_ctzll(todo);
+                const u32 lb = (u32)__builtin_amdgcn_readlane((int)b, leader);
+                const unsigned long long same = __ballot(b == lb);
+                const u32 first = off[lb];
+                if (b == lb) cols[base[lb] + first + (u32)__builtin_popcountll(same & ((1ull << lane) - 1ull))] = s;
+                __builtin_amdgcn_wave_barrier();
+                if (lane == (u32)leader) off[lb] = first + (u32)__builtin_popcountll(same);
+                __builtin_amdgcn_wave_barrier();
+                todo &= ~same;
+            }
+        }
+    }
+    if (tid < n_experts) {
+        const u32 j0 = base[tid], j1 = base[tid + 1];
+        u32 t = tile_at[tid];
+        for (u32 j = j0; j < j1; j += kGemmBN, t++) {
+            const u32 len = j1 - j < (u32)kGemmBN ? j1 - j : (u32)kGemmBN;
+            tiles[2 * t] = tid;
+            tiles[2 * t + 1] = j | (len << 16);
+        }
+    }
+}
+
+hipError_t route(const Launch &L, const uint32_t *ids, int n_slots, int n_experts, uint32_t *cols, uint32_t *tiles_out,
+                 uint32_t *n_tiles) {
+    hipLaunchKernelGGL(k_route, dim3(1), dim3(kRouteThreads), 0, L.stream, ids, (u32)n_slots, (u32)n_experts, cols,
+                       tiles_out, n_tiles, L.fault, L.layer);
+    return hipGetLastError();
+}
+
+// --------------------------------------------------------------------------------------- SwiGLU + quantize
+
+// crates/gpu/src/gemm/swiglu.rs:46-58 in the CPU path's rules: column c of act = Q8_2_X4(swiglu(g, u)) over the k
+// values g[c * k ..], u[c * k ..]. One half wave a 32-value block.
+__global__ __launch_bounds__(256) void k_swiglu_quant(const float *g, const float *u, int m, int k, uint8_t *act,
+                                                      u32 *fault, u32 layer) {
+    const int bpc = k / 32;
+    const long gblk = (long)blockIdx.x * 8 + (threadIdx.x >> 5);
+    if (gblk >= (long)m * bpc) return;
+    const int col = (int)(gblk / bpc), blk = (int)(gblk % bpc), lane32 = threadIdx.x & 31;
+    const size_t at = (size_t)col * k + 32 * blk + lane32;
+    const float v = bm_swiglu(g[at], u[at]);
+    Q82Head hd;
+    int s16;
+    const int code = q82_block(v, &hd, &s16);
+    if (hd.bad && lane32 == 0) bm_raise(fault, layer, kSiteQuantColumn);
+    q82_store(act + (size_t)col * (k / 256) * BM_Q82_SB_EXT, k / 256, blk, lane32, code, hd, s16);
+}
+
+hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act) {
+    const long blocks = (long)m * (k / 32);
+    hipLaunchKernelGGL(k_swiglu_quant, dim3((unsigned)((blocks + 7) / 8)), dim3(256), 0, L.stream, g, u, m, k, act,
+                       L.fault, L.layer);
+    return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------------- GEMM
+
+// LDS of one workgroup: a super-block of the tile's 64 activation columns and of the slab's 64 weight rows, and the
+// rows' scale products. Strides are padded off the 128-byte bank period.
+constexpr int kActSb = BM_Q82_SB_REF + 64;   // a column's super-block: its two groups and its (d8, d8 * isum) pairs
+constexpr int kActStride = kActSb + 8;       // 360
+template <int WT>
+__host__ __device__ constexpr int wt_stride() {
+    return WT == BM_Q4K ? 152 : 232; // 144 and 224 (14 chunks of 16) padded
+}
+template <int WT>
+__host__ __device__ constexpr int wt_chunks() {
+    return WT == BM_Q4K ? 9 : 14;
+}
+
+struct GemmLds {
+    u32 col[kGemmBN];  // the tile's activation columns
+    u32 slot[kGemmBN]; // and slots
+};
+
+template <int WT>
+__host__ __device__ constexpr size_t gemm_lds_bytes() {
+    return sizeof(GemmLds) + (size_t)kGemmBN * kActStride + (size_t)kGemmBM * wt_stride<WT>() + 16 * kGemmBM * sizeof(float);
+}
+
+// (q6 - 32) of four codes a word, as signed bytes: q6 in 0..63.
+__device__ __forceinline__ u32 q6_minus_32(u32 q) {
+    const u32 t = q ^ 0x20202020u;        // q >= 32: q - 32; q < 32: q + 32
+    const u32 m = ~q & 0x20202020u;       // the bytes that went up: they want -64, the two top bits
+    return t | (m << 1) | (m << 2);
+}
+
+template <int WT>
+__global__ __launch_bounds__(256) void k_gemm(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
+                                              const u32 *tiles, const u32 *n_tiles, u32 max_tiles, u32 slot_div,
+                                              u32 n_slots, float *y) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
+    uint8_t *acts = lds + sizeof(GemmLds);
+    uint8_t *wts = acts + (size_t)kGemmBN * kActStride;
+    float *rs = reinterpret_cast<float *>(wts + (size_t)kGemmBM * wt_stride<WT>()); // [16][64]
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const u32 g = blockIdx.x % max_tiles;
+    const int row0 = (int)(blockIdx.x / max_tiles) * kGemmBM;
+    const u32 count = n_tiles[0];
+    if (g > count) return;
+    if (g == count) { // the refused slots' rows: NaN (crates/gpu/src/gemm/grouped.rs:2283-2287)
+        const u32 refused = n_tiles[1];
+        for (u32 i = tid; i < refused * kGemmBM; i += blockDim.x) {
+            const u32 s = cols[n_slots - refused + i / kGemmBM];
+            const int r = row0 + (int)(i % kGemmBM);
+            if (r < rpe) y[(size_t)s * rpe + r] = bm_bits_f32(0x7fc00000u);
+        }
+        return;
+    }
+    const u32 e = tiles[2 * g], word = tiles[2 * g + 1];
+    const int start = (int)(word & 0xffffu), len = (int)(word >> 16);
+    if (tid < kGemmBN) {
+        const u32 s = cols[start + (tid < len ? tid : 0)];
+        tab->slot[tid] = s;
+        tab->col[tid] = s / slot_div;
+    }
+    __syncthreads();
+    constexpr int kBlock = WT == BM_Q4K ? BM_Q4K_BLOCK : BM_Q6K_BLOCK;
+    constexpr int kWc = wt_chunks<WT>();
+    const size_t row_bytes = (size_t)nb * kBlock;
+    const int col_bytes = nb * BM_Q82_SB_EXT;
+    // staging: kGemmBN * 22 chunks of 16 bytes of activations, kGemmBM * kWc of weights, a super-block
+    constexpr int kAc = kActSb / 16; // 22
+    constexpr int kActLoads = (kGemmBN * kAc + 255) / 256, kWtLoads = (kGemmBM * kWc + 255) / 256;
+    uint4 ra[kActLoads], rw[kWtLoads];
+    auto fetch = [&](int i) {
+#pragma unroll
+        for (int t = 0; t < kActLoads; t++) {
+            int c = t * 256 + tid;
+            c = c < kGemmBN * kAc ? c : kGemmBN * kAc - 1;
+            const int n = c / kAc, k = c % kAc;
+            const uint8_t *colp = act + (size_t)tab->col[n] * col_bytes;
+            const uint8_t *src = k < 18 ? colp + (size_t)i * BM_Q82_SB_REF + 16 * k
+                                        : colp + (size_t)nb * BM_Q82_SB_REF + (size_t)i * 64 + 16 * (k - 18);
+            ra[t] = *reinterpret_cast<const uint4 *>(src);
+        }
+#pragma unroll
+        for (int t = 0; t < kWtLoads; t++) {
+            int c = t * 256 + tid;
+            c = c < kGemmBM * kWc ? c : kGemmBM * kWc - 1;
+            int r = row0 + c / kWc;
+            const int k = c % kWc;
+            r = r < rpe ? r : rpe - 1;
+            const uint8_t *blk = w + ((size_t)e * rpe + r) * row_bytes + (size_t)i * kBlock;
+            // Q6_K: 210 bytes are 13 chunks and a last one that ends with the block (bytes 194 .. 210)
+            rw[t] = bm_ld16u(blk + ((WT == BM_Q6K && k == 13) ? 194 : 16 * k));
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int t = 0; t < kActLoads; t++) {
+            const int c = t * 256 + tid;
+            if (c < kGemmBN * kAc) {
+                uint8_t *dst = acts + (c / kAc) * kActStride + 16 * (c % kAc);
+                *reinterpret_cast<uint2 *>(dst) = make_uint2(ra[t].x, ra[t].y);
+                *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(ra[t].z, ra[t].w);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < kWtLoads; t++) {
+            const int c = t * 256 + tid;
+            if (c < kGemmBM * kWc) {
+                uint8_t *dst = wts + (c / kWc) * wt_stride<WT>() + 16 * (c % kWc);
+                *reinterpret_cast<uint2 *>(dst) = make_uint2(rw[t].x, rw[t].y);
+                *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(rw[t].z, rw[t].w);
+            }
+        }
+    };
+    // this lane in its wave's 32 x 32 product: operand row / column lane % 32, value half lane / 32; the sixteen
+    // results it holds are rows 8 * (v / 4) + 4 * (lane / 32) + v % 4 of column lane % 32
+    const int wr = wv & 1, wc = wv >> 1, l32 = lane & 31, kh = lane >> 5;
+    const uint8_t *my_act = acts + (32 * wc + l32) * kActStride;
+    const uint8_t *my_wt = wts + (32 * wr + l32) * wt_stride<WT>();
+    const int rbase = 32 * wr + 4 * kh; // result v sits in row rbase + 8 * (v / 4) + v % 4 of the slab
+    float acc[16][8];
+#pragma unroll
+    for (int v = 0; v < 16; v++)
+#pragma unroll
+        for (int l = 0; l < 8; l++) acc[v][l] = 0.0f;
+
+    fetch(0);
+    for (int i = 0; i < nb; i++) {
+        __syncthreads(); // the previous super-block's readers are done
+        stash();
+        __syncthreads();
+        if (i + 1 < nb) fetch(i + 1);
+        // the rows' scale products: rs[s][row]
+        {
+            const int r = tid >> 2, part = tid & 3;
+            const uint8_t *blk = wts + r * wt_stride<WT>();
+            if constexpr (WT == BM_Q4K) {
+                const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk));
+                const float dmin = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk + 2));
+                const uint8_t *sc = blk + 4;
+#pragma unroll
+                for (int t = 0; t < 2; t++) { // crates/gguf/src/quant.rs:620-628 get_scale_min_k4
+                    const int s = 2 * part + t;
+                    int scv, mv;
+                    if (s < 4) {
+                        scv = sc[s] & 63;
+                        mv = sc[s + 4] & 63;
+                    } else {
+                        scv = (sc[s + 4] & 15) | ((sc[s - 4] >> 6) << 4);
+                        mv = (sc[s + 4] >> 4) | ((sc[s] >> 6) << 4);
+                    }
+                    rs[s * kGemmBM + r] = d * (float)scv;
+                    rs[(8 + s) * kGemmBM + r] = -(dmin * (float)mv);
+                }
+            } else {
+                const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk + 222));
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const int gq = 4 * part + t;
+                    rs[gq * kGemmBM + r] = d * (float)(int)(signed char)blk[192 + gq];
+                }
+            }
+        }
+        __syncthreads();
+        const float2 *pair = reinterpret_cast<const float2 *>(my_act + BM_Q82_SB_REF); // (d8, d8 * isum) a 32-block
+        if constexpr (WT == BM_Q4K) {
+            // the min terms first: accumulator l takes sub-block l's (crates/qdot/src/lib.rs:4389-4394)
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                const float my = pair[s].y;
+#pragma unroll
+                for (int qd = 0; qd < 4; qd++) {
+                    const float4 mn = *reinterpret_cast<const float4 *>(&rs[(8 + s) * kGemmBM + rbase + 8 * qd]);
+                    acc[4 * qd + 0][s] = fmaf(my, mn.x, acc[4 * qd + 0][s]);
+                    acc[4 * qd + 1][s] = fmaf(my, mn.y, acc[4 * qd + 1][s]);
+                    acc[4 * qd + 2][s] = fmaf(my, mn.z, acc[4 * qd + 2][s]);
+                    acc[4 * qd + 3][s] = fmaf(my, mn.w, acc[4 * qd + 3][s]);
+                }
+            }
+#pragma unroll
+            for (int p = 0; p < 4; p++) { // code bytes 32p ..: low nibbles sub-block 2p, high nibbles 2p + 1
+                uint2 wq[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) wq[h] = *reinterpret_cast<const uint2 *>(my_wt + 16 + 32 * p + 16 * h + 8 * kh);
+#pragma unroll
+                for (int en = 0; en < 2; en++) {
+                    const int s = 2 * p + en;
+                    const float d8 = pair[s].x;
+                    float f[16];
+#pragma unroll
+                    for (int qd = 0; qd < 4; qd++) {
+                        const float4 sv = *reinterpret_cast<const float4 *>(&rs[s * kGemmBM + rbase + 8 * qd]);
+                        f[4 * qd + 0] = sv.x * d8;
+                        f[4 * qd + 1] = sv.y * d8;
+                        f[4 * qd + 2] = sv.z * d8;
+                        f[4 * qd + 3] = sv.w * d8;
+                    }
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const u32 ax = (wq[h].x >> (4 * en)) & 0x0f0f0f0fu, ay = (wq[h].y >> (4 * en)) & 0x0f0f0f0fu;
+                        const uint2 bq = *reinterpret_cast<const uint2 *>(my_act + (s >> 2) * BM_Q82X4_STRIDE + 16 +
+                                                                          32 * (s & 3) + 16 * h + 8 * kh);
+                        const long a = (long)(((unsigned long long)ay << 32) | ax);
+                        const long b = (long)(((unsigned long long)bq.y << 32) | bq.x);
+                        v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                        const v16i sum = __builtin_amdgcn_mfma_i32_32x32x16_i8(a, b, z, 0, 0, 0);
+                        const int l = 4 * h + (s & 3);
+#pragma unroll
+                        for (int v = 0; v < 16; v++) acc[v][l] = fmaf(f[v], (float)sum[v], acc[v][l]);
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int gq = 0; gq < 16; gq++) { // 16-value group gq: 32-block gq / 2, half gq % 2
+                const int c2 = gq >> 3, a4 = (gq & 7) >> 1, hh = gq & 1, bk = gq >> 1;
+                const int l0 = 16 * hh + 8 * kh;
+                const uint2 ql = *reinterpret_cast<const uint2 *>(my_wt + 64 * c2 + 32 * (a4 & 1) + l0);
+                const uint2 qh = *reinterpret_cast<const uint2 *>(my_wt + 128 + 32 * c2 + l0);
+                const int ns = 4 * (a4 >> 1), hs = 2 * a4;
+                const u32 ax = q6_minus_32(((ql.x >> ns) & 0x0f0f0f0fu) | (((qh.x >> hs) & 0x03030303u) << 4));
+                const u32 ay = q6_minus_32(((ql.y >> ns) & 0x0f0f0f0fu) | (((qh.y >> hs) & 0x03030303u) << 4));
+                const uint2 bq = *reinterpret_cast<const uint2 *>(my_act + (bk >> 2) * BM_Q82X4_STRIDE + 16 + 32 * (bk & 3) +
+                                                                  16 * hh + 8 * kh);
+                const float d8 = pair[bk].x;
+                const long a = (long)(((unsigned long long)ay << 32) | ax);
+                const long b = (long)(((unsigned long long)bq.y << 32) | bq.x);
+                v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                const v16i sum = __builtin_amdgcn_mfma_i32_32x32x16_i8(a, b, z, 0, 0, 0);
+                const int l = 4 * hh + (bk & 3); // crates/qdot/src/lib.rs:4794-4809: lane l < 4 scale 2l, lane 4 + l scale 2l + 1
+#pragma unroll
+                for (int qd = 0; qd < 4; qd++) {
+                    const float4 sv = *reinterpret_cast<const float4 *>(&rs[gq * kGemmBM + rbase + 8 * qd]);
+                    acc[4 * qd + 0][l] = fmaf(sv.x * d8, (float)sum[4 * qd + 0], acc[4 * qd + 0][l]);
+                    acc[4 * qd + 1][l] = fmaf(sv.y * d8, (float)sum[4 * qd + 1], acc[4 * qd + 1][l]);
+                    acc[4 * qd + 2][l] = fmaf(sv.z * d8, (float)sum[4 * qd + 2], acc[4 * qd + 2][l]);
+                    acc[4 * qd + 3][l] = fmaf(sv.w * d8, (float)sum[4 * qd + 3], acc[4 * qd + 3][l]);
+                }
+            }
+        }
+    }
+    // the closing sum of the eight lanes (crates/qdot/src/lib.rs:4128 hsum_float_8's order) and the store
+    const int n = 32 * wc + l32;
+    if (n < len) {
+        const size_t out = (size_t)tab->slot[n] * rpe + row0;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int r = rbase + 8 * (v >> 2) + (v & 3);
+            const float t0 = acc[v][0] + acc[v][4], t1 = acc[v][1] + acc[v][5];
+            const float t2 = acc[v][2] + acc[v][6], t3 = acc[v][3] + acc[v][7];
+            if (row0 + r < rpe) y[out + r] = (t0 + t2) + (t1 + t3);
+        }
+    }
+}
+
+bool gemm_supported(int wtype) { return wtype == BM_Q4K || wtype == BM_Q6K; }
+
+hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int rows_per_expert, int k,
+                const uint8_t *act, const uint32_t *cols, const uint32_t *tiles_dev, const uint32_t *n_tiles, int n_slots,
+                int slot_div, float *y) {
+    const int nb = k / 256;
+    const u32 max_tiles = (u32)gemm_max_tiles(n_slots, n_experts) + 1; // one more: the block that fills refused slots
+    const unsigned grid = max_tiles * (unsigned)((rows_per_expert + kGemmBM - 1) / kGemmBM);
+    if (wtype == BM_Q4K) {
+        auto kern = k_gemm<BM_Q4K>;
+        const size_t lds = gemm_lds_bytes<BM_Q4K>();
+        hipError_t e = allow_lds(kern, lds);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
+                           n_tiles, max_tiles, (u32)slot_div, (u32)n_slots, y);
+    } else if (wtype == BM_Q6K) {
+        auto kern = k_gemm<BM_Q6K>;
+        const size_t lds = gemm_lds_bytes<BM_Q6K>();
+        hipError_t e = allow_lds(kern, lds);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
+                           n_tiles, max_tiles, (u32)slot_div, (u32)n_slots, y);
+    } else {
+        return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+} // namespace bmk

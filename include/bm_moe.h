@@ -221,6 +221,35 @@ int bm_gate_up_tiles(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, co
 int bm_gemv_tiles(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const uint32_t *order_dev, const uint32_t *start_dev,
                   const uint32_t *tiles_dev, int n_slots, int rows_per_expert, float *y_dev);
 
+/* -------------------------------------------------------------------- prefill: route table and grouped GEMM */
+
+typedef struct bm_route bm_route; /* crates/gpu/src/gemm/route.rs:109-125 GemmRoute */
+
+/* GemmRoute::new (crates/gpu/src/gemm/route.rs:127-155): a table for up to max_slots (1..=40960) slots over a
+ * stack of n_experts (1..=1024) experts. Load time only. */
+int bm_route_create(bm_ctx *ctx, int max_slots, int n_experts, bm_route **out);
+void bm_route_destroy(bm_route *route);
+/* GemmKernels::enqueue_route (crates/gpu/src/gemm/route.rs:351): the table of ids_dev[0 .. n_slots) (slot =
+ * token * top_k + k), built on the device: the slots grouped by expert, ascending inside an expert, cut into
+ * tiles of at most 64. An id at or past the stack raises BM_SITE_EXPERT_ID; its slot is left out of the tiles
+ * and listed as refused, and every bm_gemm over the table writes NaN into its rows. */
+int bm_route_fill(bm_ctx *ctx, const uint32_t *ids_dev, int n_slots, bm_route *route);
+/* GemmRoute::read_back / refused_back (route.rs:188-245): synchronise and copy the table out. cols_host (optional)
+ * takes the n_slots slot list (refused slots last); tiles_host (optional) two words a tile: expert, then
+ * first index | length << 16. */
+int bm_route_read(bm_ctx *ctx, const bm_route *route, uint32_t *cols_host, uint32_t *tiles_host, int *n_tiles, int *n_refused);
+/* GemmKernels::enqueue_gemm(GemmArgs) (crates/gpu/src/gemm/grouped.rs:2125-2133,2300), Q4_K and Q6_K stacks:
+ * y_dev[s * rows_per_expert + r] = row r of expert e(s) . column c(s) of act for every slot s of the table's last
+ * fill; c(s) = s / top_k (GemmInput::Shared) or s when top_k is 0 (GemmInput::PerSlot). rows_per_expert a
+ * multiple of 16. Every value is bm_gemv_sel's for that slot, bit for bit; the integer sums are formed on the int8
+ * matrix cores. A refused slot gets NaN in every row. */
+int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act *act, const bm_route *route, int top_k,
+            float *y_dev);
+/* GemmKernels::enqueue_swiglu_quant (crates/gpu/src/gemm/swiglu.rs:46): column c of act = the quantized
+ * silu(g) * u of g_dev / u_dev[c * k .. (c + 1) * k), k = act's k, slot-major as the gate and up GEMMs write them;
+ * bm_quantize's bytes of the CPU path's SwiGLU. Q8_2_X4 columns only. */
+int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, bm_act *act);
+
 /* ------------------------------------------------------------------------------------------- verification */
 
 /* The exact per-block integers the kernels above form for row `row` of w against column `col` of act, written

@@ -251,6 +251,24 @@ def grouped_table(sel, n_experts):
     return (np.asarray(order + [0] * (n_slots - len(order)), np.uint32), np.asarray(start, np.uint32), tiles, refused)
 
 
+GEMM_BN = 64
+
+
+def gemm_route(ids, n_experts):
+    """The prefill route table by definition (crates/gpu/src/gemm/route.rs:1-4,109-125,351-362): the slots grouped
+    by expert, ascending slot order inside an expert, the refused slots (an id at or past the stack) at the end in
+    ascending order; tiles of at most 64 slots as rows (expert, start, len). Returns (cols, tiles, refused count)."""
+    ids = np.asarray(ids, np.uint32).reshape(-1)
+    cols, tiles = [], []
+    for e in range(n_experts):
+        run = [s for s in range(ids.size) if int(ids[s]) == e]
+        for j in range(0, len(run), GEMM_BN):
+            tiles.append((e, len(cols) + j, min(GEMM_BN, len(run) - j)))
+        cols += run
+    refused = [s for s in range(ids.size) if int(ids[s]) >= n_experts]
+    return (np.asarray(cols + refused, np.uint32), np.asarray(tiles, np.uint32).reshape(-1, 3), len(refused))
+
+
 def quantize_rows(wtype, x, rows, k, n_threads=8):
     """rows x k f32 -> GGUF block bytes, rows back to back."""
     x = _f32(x).reshape(rows, k)

@@ -1,0 +1,154 @@
+"""GPU parity tests of the prefill path (route table, grouped GEMM on the int8 matrix cores, SwiGLU quantizer),
+through the C ABI, against the CPU oracle on the same seeded inputs. Every value of the grouped GEMM is the
+one-column row dot's, so everything is compared bit for bit (and within the stated 1e-4 first).
+Mirrors the reference's gate_gemm clauses (crates/gpu-gates/src/bin/gate_gemm.rs): table by definition, refused ids
+-> NaN rows and ExpertId, Shared and PerSlot inputs, rows_per_expert a multiple of 16 that is not a whole slab."""
+import numpy as np
+import pytest
+
+import bloomery_amd as bm
+import ora
+from common import normal_f32
+from test_gpu_decode import Layer, assert_f32, gpu, route, stack  # noqa: F401  (gpu is the module fixture)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n_experts,n_slots,seed", ((128, 16384, 1), (3, 500, 2), (1, 64, 3), (1024, 4096, 4), (7, 1, 5)))
+def test_route_table_is_the_definition(gpu, n_experts, n_slots, seed):
+    rng = np.random.default_rng(seed)
+    ids = rng.integers(0, n_experts, n_slots).astype(np.uint32)
+    if n_experts == 128:  # skewed popularity, as a prefill batch has
+        p = 1.0 / np.arange(1, n_experts + 1) ** 1.1
+        ids = rng.choice(n_experts, n_slots, p=p / p.sum()).astype(np.uint32)
+    gpu.fault_clear()
+    table = gpu.route(n_slots, n_experts)
+    ids_d = gpu.upload(ids, np.uint32)
+    table.fill(ids_d, n_slots)
+    cols, tiles, refused = table.read()
+    want_cols, want_tiles, want_refused = ora.gemm_route(ids, n_experts)
+    assert refused == want_refused == 0
+    assert np.array_equal(cols, want_cols)
+    assert np.array_equal(tiles, want_tiles)
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    table.free()
+    ids_d.free()
+
+
+def run_prefill(gpu, L, x, ids, wts, top_k):
+    """quantize -> route -> gate GEMM, up GEMM (Shared) -> swiglu_quant -> down GEMM (PerSlot) -> combine
+    (crates/gpu/src/arch/qwen3moe/wide.rs:1171-1225)."""
+    m = x.shape[0]
+    n_slots = m * top_k
+    act = gpu.act(L.types[0], L.hidden, m)
+    act_h = gpu.act(L.types[2], L.ff, n_slots)
+    xd, sel, wd = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32)
+    table = gpu.route(n_slots, L.n_experts)
+    g = gpu.buffer(np.float32, n_slots * L.ff).fill_bytes(0xFF)
+    u = gpu.buffer(np.float32, n_slots * L.ff).fill_bytes(0xFF)
+    down = gpu.buffer(np.float32, n_slots * L.hidden).fill_bytes(0xFF)
+    y = gpu.buffer(np.float32, m * L.hidden).fill_bytes(0xFF)
+    gpu.enqueue_quantize(xd, m, act)
+    table.fill(sel, n_slots)
+    gpu.enqueue_gemm(L.dg, L.ff, act, table, top_k, g)
+    gpu.enqueue_gemm(L.du, L.ff, act, table, top_k, u)
+    gpu.enqueue_swiglu_quant(g, u, n_slots, act_h)
+    gpu.enqueue_gemm(L.dd, L.hidden, act_h, table, 0, down)
+    gpu.enqueue_combine_tokens(down, wd, None, L.hidden, top_k, m, y)
+    out = y.download(), g.download(), u.download(), [act_h.download(s) for s in range(n_slots)], down.download()
+    for b in (act, act_h, xd, sel, wd, table, g, u, down, y):
+        b.free()
+    return out
+
+
+@pytest.mark.parametrize("types,hidden,ff,n_experts,m,top_k,cheap", (
+    ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 6, 70, 3, False),      # runs past 64 slots: several tiles an expert
+    ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 16, 48, 8, True),     # config 4's layer shape, 384 slots
+    ((bm.Q6_K, bm.Q6_K, bm.Q4_K), 768, 512, 3, 9, 2, False),       # the other type on each side; ragged tiles
+))
+def test_prefill_layer_matches_the_oracle(gpu, types, hidden, ff, n_experts, m, top_k, cheap):
+    L = Layer(gpu, types, hidden, ff, n_experts, 2000 + hidden, cheap=cheap)
+    rng = np.random.default_rng(2001)
+    x = normal_f32(rng, (m, hidden))
+    ids, wts = route(rng, m, n_experts, top_k)
+    gpu.fault_clear()
+    y, g, u, act_h, down = run_prefill(gpu, L, x, ids, wts, top_k)
+    want_y, want_h = L.oracle(x, ids, wts, top_k)
+    # gate and up rows against the one-column dots
+    rb = ora.row_bytes(types[0], hidden)
+    for s in (0, m * top_k // 2, m * top_k - 1):
+        e, col = int(ids.reshape(-1)[s]), ora.quantize_col(types[0], x[s // top_k])
+        assert_f32(g[s * ff:(s + 1) * ff], ora.gemv(types[0], L.wg[e * ff * rb:(e + 1) * ff * rb], ff, hidden, col, 1), f"gate slot {s}")
+        assert_f32(u[s * ff:(s + 1) * ff], ora.gemv(types[1], L.wu[e * ff * rb:(e + 1) * ff * rb], ff, hidden, col, 1), f"up slot {s}")
+    for s in range(m * top_k):
+        assert np.array_equal(act_h[s], ora.quantize_col(types[2], want_h[s * ff:(s + 1) * ff])), f"act_h slot {s}"
+    assert_f32(y, want_y, "y")
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    L.free()
+
+
+def test_gemm_rows_not_a_whole_slab_and_refused_slots(gpu):
+    """rows_per_expert = 80 (a multiple of 16, a slab and a quarter); a refused id gets NaN rows and ExpertId."""
+    rng = np.random.default_rng(2100)
+    for wtype, k in ((bm.Q4_K, 1024), (bm.Q6_K, 768)):
+        rpe, n_experts, n_slots = 80, 4, 23
+        w = stack(wtype, n_experts * rpe, k, 2101)
+        ids = rng.integers(0, n_experts, n_slots).astype(np.uint32)
+        ids[5] = 9   # past the stack
+        x = normal_f32(rng, (n_slots, k))
+        dw, act = gpu.weights(wtype, n_experts * rpe, k, w), gpu.act(wtype, k, n_slots)
+        xd, sel = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32)
+        table = gpu.route(n_slots, n_experts)
+        gpu.fault_clear()
+        gpu.set_layer(2)
+        gpu.enqueue_quantize(xd, n_slots, act)
+        table.fill(sel, n_slots)
+        y = gpu.buffer(np.float32, n_slots * rpe).fill_bytes(0)
+        gpu.enqueue_gemm(dw, rpe, act, table, 0, y)
+        got = y.download().reshape(n_slots, rpe)
+        cols, tiles, refused = table.read()
+        assert refused == 1 and cols[-1] == 5 and gpu.fault(2) == ((2 << 8) | bm.SITE_EXPERT_ID, 1 << bm.SITE_EXPERT_ID)
+        assert np.isnan(got[5]).all()
+        rb = ora.row_bytes(wtype, k)
+        for s in range(n_slots):
+            if s == 5:
+                continue
+            e = int(ids[s])
+            want = ora.gemv(wtype, w[e * rpe * rb:(e + 1) * rpe * rb], rpe, k, ora.quantize_col(wtype, x[s]), 1)
+            assert_f32(got[s], want, f"type {wtype} slot {s}")
+        gpu.set_layer(bm.LAYER_NONE)
+        gpu.fault_clear()
+        for b in (dw, act, xd, sel, table, y):
+            b.free()
+
+
+def test_prefill_refusals_are_named(gpu):
+    w4 = gpu.weights(bm.Q4_K, 64, 512, np.zeros(64 * bm.row_bytes(bm.Q4_K, 512), np.uint8))
+    wi = gpu.weights(bm.IQ2_XXS, 64, 512, np.zeros(64 * bm.row_bytes(bm.IQ2_XXS, 512), np.uint8))
+    a512, aq8k = gpu.act(bm.Q4_K, 512, 8), gpu.act(bm.IQ2_XXS, 512, 8)
+    buf = gpu.buffer(np.float32, 4096)
+    ids = gpu.upload(np.zeros(8, np.uint32))
+    table = gpu.route(8, 2)
+    cases = [(lambda: gpu.enqueue_gemm(w4, 32, a512, table, 0, buf), bm.ESHAPE, "filled")]
+    for call, code, word in cases:
+        with pytest.raises(bm.GpuError) as e:
+            call()
+        assert e.value.code == code and word in str(e.value), str(e.value)
+    table.fill(ids, 8)
+    cases = (
+        (lambda: gpu.enqueue_gemm(w4, 24, a512, table, 0, buf), bm.ESHAPE, "multiple of 16"),
+        (lambda: gpu.enqueue_gemm(w4, 16, a512, table, 0, buf), bm.ESHAPE, "experts"),
+        (lambda: gpu.enqueue_gemm(w4, 32, a512, table, 3, buf), bm.ESHAPE, "whole tokens"),
+        (lambda: gpu.enqueue_gemm(wi, 32, aq8k, table, 0, buf), bm.ETYPE, "bm_gemm"),
+        (lambda: gpu.enqueue_swiglu_quant(buf, buf, 9, a512), bm.ESHAPE, "n_cols"),
+        (lambda: gpu.enqueue_swiglu_quant(buf, buf, 2, aq8k), bm.ETYPE, "Q8_2_X4"),
+        (lambda: table.fill(ids, 9), bm.ESHAPE, "n_slots"),
+        (lambda: gpu.route(50000, 2), bm.ESHAPE, "max_slots"),
+        (lambda: gpu.route(8, 2000), bm.ESHAPE, "n_experts"),
+    )
+    for call, code, word in cases:
+        with pytest.raises(bm.GpuError) as e:
+            call()
+        assert e.value.code == code and word in str(e.value), str(e.value)
+    for b in (w4, wi, a512, aq8k, buf, ids, table):
+        b.free()

@@ -250,3 +250,12 @@ def test_grouped_table_by_hand():
     assert list(start) == [0, 0, 9] and list(order[:9]) == list(range(9)) and refused
     assert list(tiles[:3]) == [2, (1 << 22) | 0, (1 << 22) | 8]
     assert ora.tile_cap(11, 2) == 3 and ora.tile_cap(128, 128) == 128 and ora.tile_cap(16384, 128) == 2160
+
+
+def test_gemm_route_by_hand():
+    """crates/gpu/src/gemm/route.rs: grouped by expert, ascending inside, tiles of at most 64, refused slots last."""
+    cols, tiles, refused = ora.gemm_route([1, 0, 5, 1, 1, 0], 3)
+    assert list(cols) == [1, 5, 0, 3, 4, 2] and refused == 1
+    assert tiles.tolist() == [[0, 0, 2], [1, 2, 3]]
+    cols, tiles, refused = ora.gemm_route([2] * 130, 3)
+    assert tiles.tolist() == [[2, 0, 64], [2, 64, 64], [2, 128, 2]] and refused == 0

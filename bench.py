@@ -60,8 +60,335 @@ def make_tokens(ora, n_tokens, seed):
     return x, ids, wts
 
 
+def timed_graph(gpu, enqueue, unit, steps, warmup):
+    """Capture `unit` steps into one graph, replay it for about `steps` timed steps; ms per step by wall clock
+    (bracketed by synchronisation) and by events on the launch stream."""
+    gpu.capture_begin()
+    for i in range(unit):
+        enqueue(i)
+    graph = gpu.capture_end()
+    reps_w, reps = max(1, -(-warmup // unit)), max(1, -(-steps // unit))
+    for _ in range(reps_w):
+        gpu.graph_launch(graph)
+    gpu.sync()
+    e0, e1 = gpu.event(), gpu.event()
+    t0 = time.perf_counter()
+    gpu.event_record(e0)
+    for _ in range(reps):
+        gpu.graph_launch(graph)
+    gpu.event_record(e1)
+    gpu.sync()
+    wall = (time.perf_counter() - t0) * 1e3 / (reps * unit)
+    ev = gpu.event_elapsed_ms(e0, e1) / (reps * unit)
+    gpu.graph_destroy(graph)
+    gpu.event_destroy(e0)
+    gpu.event_destroy(e1)
+    return wall, ev, reps * unit, reps_w * unit
+
+
+def emit(metric, value, unit, steps, warmup, ms_per_step, workload, extra, roofline, cpu, higher=False):
+    out = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
+           "ms_per_step": ms_per_step, "higher_is_better": higher, "scaling": "weak", "vs_baseline": None,
+           "dtype": "i8", "data": "synthetic", "config": {"workload": workload, "mode": "hipGraph replay"}}
+    out.update(extra)
+    out["roofline"] = roofline
+    out["cpu_baseline"] = cpu
+    print(json.dumps(out), flush=True)
+
+
+def cpu_layer_baseline(ora, args, threads, types, shape, stacks, x, ids, wts, top_k, per_call_tokens, bytes_per_call):
+    """The AVX2 restatement of the reference's qdot path on the host cores, a bounded sample of the same workload."""
+    if args.no_cpu:
+        return None
+    hidden, ff, n_experts = shape
+    pool = ora.lib.ora_pool_create(threads)
+    try:
+        n, t0 = 0, time.perf_counter()
+        while True:
+            lo = (n * per_call_tokens) % max(1, x.shape[0] - per_call_tokens + 1)
+            ora.moe_forward(hidden, ff, n_experts, types, *stacks, x[lo:lo + per_call_tokens], ids[lo:lo + per_call_tokens],
+                            wts[lo:lo + per_call_tokens], top_k, avx2_pool=pool)
+            n += 1
+            el = time.perf_counter() - t0
+            if el >= args.cpu_seconds and n >= 3:
+                break
+    finally:
+        ora.lib.ora_pool_destroy(pool)
+    return {"value": el / (n * per_call_tokens) * 1e6, "unit": "us/token", "cores": threads, "kind": "port",
+            "sample": f"{n} passes of {per_call_tokens} tokens of the same layer and routings, AVX2 restatement of qdot on "
+                      f"{threads} threads, {el:.1f}s"}
+
+
+def biased_routes(ora, n_tokens, n_experts, top_k, seed, bias_sigma=0.0, zipf=0.0):
+    """Router draws: logits N(0, 1) (+ a fixed expert bias N(0, sigma), or + log of a Zipf popularity over a random
+    expert permutation), softmax, top-k renormalised."""
+    rng = np.random.default_rng(seed)
+    bias = np.zeros(n_experts, np.float32)
+    if bias_sigma:
+        bias = (rng.standard_normal(n_experts) * bias_sigma).astype(np.float32)
+    if zipf:
+        pop = 1.0 / np.arange(1, n_experts + 1) ** zipf
+        bias = np.log(pop / pop.sum())[rng.permutation(n_experts)].astype(np.float32)
+    ids = np.empty((n_tokens, top_k), np.uint32)
+    wts = np.empty((n_tokens, top_k), np.float32)
+    for t in range(n_tokens):
+        logits = (rng.standard_normal(n_experts, dtype=np.float32) + bias).astype(np.float32)
+        ids[t], wts[t] = ora.route_softmax_topk(logits, top_k)
+    return ids, wts
+
+
+def parity_of(got, want):
+    err = float(np.max(np.abs(got.astype(np.float64) - want)) / np.max(np.abs(want)))
+    p = {"max_abs_normalised_err": err, "bit_identical": bool(np.array_equal(got, want))}
+    log(f"[bench] parity {p}")
+    assert err <= 1e-4, p
+    return p
+
+
+def bench_gemv(args, bm, ora, threads):
+    """Config 1: one Q4_K gemv, 768 x 2048, one column."""
+    rng = np.random.default_rng(0xB1000001)
+    w = ora.quantize_rows(ora.Q4_K, rng.standard_normal((FF, HIDDEN), dtype=np.float32) * np.float32(0.02), FF, HIDDEN,
+                          n_threads=threads)
+    x = np.random.default_rng(0xAC70001).standard_normal((64, HIDDEN), dtype=np.float32)
+    gpu = bm.Gpu(0)
+    copies = [gpu.weights(bm.Q4_K, FF, HIDDEN, w) for _ in range(64)]
+    xd, y = gpu.upload(x, np.float32), gpu.buffer(np.float32, 64 * FF)
+    acts = [gpu.act(bm.Q4_K, HIDDEN, 1) for _ in range(4)]
+
+    def step(i):
+        gpu.enqueue_quantize(xd.ptr + 4 * (i % 64) * HIDDEN, 1, acts[i % 4])
+        gpu.enqueue_gemv(copies[i % 64], acts[i % 4], 1, y.ptr + 4 * (i % 64) * FF)
+
+    for i in range(4):
+        step(i)
+    got = y.download()[:4 * FF].reshape(4, FF)
+    want = np.stack([ora.gemv(ora.Q4_K, w, FF, HIDDEN, ora.quantize_col(ora.Q4_K, x[i]), 1) for i in range(4)])
+    parity = parity_of(got, want)
+    wall, ev, steps, warm = timed_graph(gpu, step, 64, args.steps, args.warmup)
+    only = timed_graph(gpu, lambda i: gpu.enqueue_gemv(copies[i % 64], acts[i % 4], 1, y.ptr + 4 * (i % 64) * FF), 64, 1024, 64)[1]
+    nbytes = FF * bm.row_bytes(bm.Q4_K, HIDDEN)
+    ach = nbytes / (only * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu:
+        col, n, t0 = ora.quantize_col(ora.Q4_K, x[0], avx2=True), 0, time.perf_counter()
+        while time.perf_counter() - t0 < min(args.cpu_seconds, 3.0):
+            ora.quantize_col(ora.Q4_K, x[n % 64], avx2=True)
+            ora.gemv(ora.Q4_K, w, FF, HIDDEN, col, 1)
+            n += 1
+        cpu = {"value": (time.perf_counter() - t0) / n * 1e6, "unit": "us/gemv", "cores": 1, "kind": "port",
+               "sample": f"{n} quantize + gemv calls of the same matrix, scalar restatement of qdot on 1 thread"}
+    emit("q4k_gemv_us", wall * 1e3, "us/gemv", steps, warm, wall,
+         "single Q4_K gemv 768 x 2048, one column, quantizer included (BASELINE.json configs[0])",
+         {"event_ms_per_step": ev, "kernel_us": {"gemv": only * 1e3}, "parity": parity, "algorithmic_bytes_per_launch": nbytes},
+         {"bound": "hbm", "kernel": "k_gemv<Q4_K>", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+          "frac": ach / HBM_PEAK_GBS, "traffic": None}, cpu)
+    gpu.close()
+
+
+def bench_grouped(args, bm, ora, threads):
+    """Config 3: the same layer, 16 tokens, expert-biased routing, grouped by expert."""
+    m, sets = 16, 8
+    wg, wu, wd = make_layer(ora, 0xB1000001, threads)
+    x = np.random.default_rng(0xAC70001).standard_normal((m * sets, HIDDEN), dtype=np.float32)
+    ids, wts = biased_routes(ora, m * sets, N_EXPERTS, TOP_K, 0x707E0001, bias_sigma=0.5)
+    gpu = bm.Gpu(0)
+    layers = [(gpu.weights(bm.Q4_K, N_EXPERTS * FF, HIDDEN, wg), gpu.weights(bm.Q4_K, N_EXPERTS * FF, HIDDEN, wu),
+               gpu.weights(bm.Q6_K, N_EXPERTS * HIDDEN, FF, wd)) for _ in range(args.layers)]
+    n_slots = m * TOP_K
+    xd, sel, wt = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32)
+    y = gpu.buffer(np.float32, m * sets * HIDDEN)
+    down = gpu.buffer(np.float32, n_slots * HIDDEN)
+    act, act_h = gpu.act(bm.Q4_K, HIDDEN, m), gpu.act(bm.Q6_K, FF, n_slots)
+    order, start = gpu.buffer(np.uint32, n_slots), gpu.buffer(np.uint32, N_EXPERTS + 1)
+    tiles = gpu.buffer(np.uint32, gpu.tile_cap(n_slots, N_EXPERTS) + 1)
+
+    def step(i, which=("tables", "quant", "gate_up", "down", "combine")):
+        st = i % sets
+        dg, du, dd = layers[i % len(layers)]
+        s_ptr = sel.ptr + 4 * st * n_slots
+        if "tables" in which:
+            gpu.enqueue_buckets(s_ptr, n_slots, N_EXPERTS, order, start)
+            gpu.enqueue_tiles(start, N_EXPERTS, n_slots, tiles)
+        if "quant" in which:
+            gpu.enqueue_quantize(xd.ptr + 4 * st * m * HIDDEN, m, act)
+        if "gate_up" in which:
+            gpu.enqueue_gate_up_tiles(dg, du, act, order, start, tiles, n_slots, FF, TOP_K, None, act_h)
+        if "down" in which:
+            gpu.enqueue_gemv_tiles(dd, act_h, order, start, tiles, n_slots, HIDDEN, down)
+        if "combine" in which:
+            gpu.enqueue_combine_tokens(down, wt.ptr + 4 * st * n_slots, None, HIDDEN, TOP_K, m, y.ptr + 4 * st * m * HIDDEN)
+
+    step(0)
+    want = ora.moe_forward(HIDDEN, FF, N_EXPERTS, (ora.Q4_K, ora.Q4_K, ora.Q6_K), wg, wu, wd, x[:m], ids[:m], wts[:m], TOP_K,
+                           n_threads=threads).reshape(m, HIDDEN)
+    parity = parity_of(y.download()[:m * HIDDEN].reshape(m, HIDDEN), want)
+    wall, ev, steps, warm = timed_graph(gpu, step, 64, args.steps, args.warmup)
+    step(0)  # leave set 0's tables for the single-kernel graphs
+    kernel_us = {k: timed_graph(gpu, lambda i, k=k: step(i - i % sets, (k,)) if k in ("gate_up", "down") else step(i, (k,)),
+                                64, 512, 64)[1] * 1e3 for k in ("tables", "quant", "gate_up", "down", "combine")}
+    hit = np.mean([len(np.unique(ids[s * m:(s + 1) * m])) for s in range(sets)])
+    per_expert = 2 * FF * bm.row_bytes(bm.Q4_K, HIDDEN) + HIDDEN * bm.row_bytes(bm.Q6_K, FF)
+    nbytes = hit * per_expert
+    ach = hit * 2 * FF * bm.row_bytes(bm.Q4_K, HIDDEN) / (kernel_us["gate_up"] * 1e-6) / 1e9
+    cpu = cpu_layer_baseline(ora, args, threads, (ora.Q4_K, ora.Q4_K, ora.Q6_K), (HIDDEN, FF, N_EXPERTS), (wg, wu, wd), x, ids, wts,
+                             TOP_K, m, nbytes)
+    emit("moe_layer_decode_us_per_token", wall * 1e3 / m, "us/token", steps, warm, wall,
+         "Qwen3-30B-A3B-shaped MoE layer, batched decode of 16 tokens grouped by expert, router logits N(0,1) + expert bias "
+         "N(0,0.5) (BASELINE.json configs[2])",
+         {"event_ms_per_step": ev, "kernel_us": kernel_us, "parity": parity, "distinct_experts_per_step": float(hit),
+          "algorithmic_bytes_per_step": nbytes, "hbm_tbps": nbytes / (wall * 1e-3) / 1e12, "launches_per_step": 6},
+         {"bound": "hbm", "kernel": "k_gate_up_tiles<Q4_K>", "achieved": ach,
+          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None}, cpu)
+    gpu.close()
+
+
+def bench_prefill(args, bm, ora, threads):
+    """Config 4: the same layer, prefill of 2048 tokens, Zipf(1.1) expert popularity."""
+    m = args.prefill_tokens
+    wg, wu, wd = make_layer(ora, 0xB1000001, threads)
+    x = np.random.default_rng(0xAC70001).standard_normal((m, HIDDEN), dtype=np.float32)
+    ids, wts = biased_routes(ora, m, N_EXPERTS, TOP_K, 0x707E0001, zipf=1.1)
+    gpu = bm.Gpu(0)
+    dg, du, dd = (gpu.weights(bm.Q4_K, N_EXPERTS * FF, HIDDEN, wg), gpu.weights(bm.Q4_K, N_EXPERTS * FF, HIDDEN, wu),
+                  gpu.weights(bm.Q6_K, N_EXPERTS * HIDDEN, FF, wd))
+    n_slots = m * TOP_K
+    xd, sel, wt = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32)
+    act, act_h = gpu.act(bm.Q4_K, HIDDEN, m), gpu.act(bm.Q6_K, FF, n_slots)
+    g, u = gpu.buffer(np.float32, n_slots * FF), gpu.buffer(np.float32, n_slots * FF)
+    down, y = gpu.buffer(np.float32, n_slots * HIDDEN), gpu.buffer(np.float32, m * HIDDEN)
+    table = gpu.route(n_slots, N_EXPERTS)
+
+    def step(i, which=("quant", "route", "gate", "up", "swiglu_quant", "down", "combine")):
+        if "quant" in which:
+            gpu.enqueue_quantize(xd, m, act)
+        if "route" in which:
+            table.fill(sel, n_slots)
+        if "gate" in which:
+            gpu.enqueue_gemm(dg, FF, act, table, TOP_K, g)
+        if "up" in which:
+            gpu.enqueue_gemm(du, FF, act, table, TOP_K, u)
+        if "swiglu_quant" in which:
+            gpu.enqueue_swiglu_quant(g, u, n_slots, act_h)
+        if "down" in which:
+            gpu.enqueue_gemm(dd, HIDDEN, act_h, table, 0, down)
+        if "combine" in which:
+            gpu.enqueue_combine_tokens(down, wt, None, HIDDEN, TOP_K, m, y)
+
+    step(0)
+    n_chk = 4
+    want = ora.moe_forward(HIDDEN, FF, N_EXPERTS, (ora.Q4_K, ora.Q4_K, ora.Q6_K), wg, wu, wd, x[:n_chk], ids[:n_chk], wts[:n_chk],
+                           TOP_K, n_threads=threads).reshape(n_chk, HIDDEN)
+    parity = parity_of(y.download()[:n_chk * HIDDEN].reshape(n_chk, HIDDEN), want)
+    wall, ev, steps, warm = timed_graph(gpu, step, 2, min(args.steps, 20), min(args.warmup, 4))
+    kernel_us = {k: timed_graph(gpu, lambda i, k=k: step(i, (k,)), 2, 10, 2)[1] * 1e3
+                 for k in ("quant", "route", "gate", "up", "swiglu_quant", "down", "combine")}
+    ops = 2.0 * n_slots * (2 * FF * HIDDEN + HIDDEN * FF)
+    gate_ops = 2.0 * n_slots * FF * HIDDEN
+    ach = gate_ops / (kernel_us["gate"] * 1e-6) / 1e12
+    hit = len(np.unique(ids))
+    cpu = cpu_layer_baseline(ora, args, threads, (ora.Q4_K, ora.Q4_K, ora.Q6_K), (HIDDEN, FF, N_EXPERTS), (wg, wu, wd), x, ids, wts,
+                             TOP_K, min(m, 64), 0)
+    emit("prefill_int8_tops", ops / (wall * 1e-3) / 1e12, "TOP/s", steps, warm, wall,
+         f"Qwen3-30B-A3B-shaped MoE layer, prefill of {m} tokens, top-8 of 128 experts, Zipf(1.1) popularity "
+         "(BASELINE.json configs[3])",
+         {"event_ms_per_step": ev, "kernel_us": kernel_us, "parity": parity, "int8_ops_per_step": ops,
+          "us_per_token": wall * 1e3 / m, "distinct_experts": hit,
+          "weight_bytes_hit": hit * (2 * FF * bm.row_bytes(bm.Q4_K, HIDDEN) + HIDDEN * bm.row_bytes(bm.Q6_K, FF))},
+         {"bound": "mfma", "kernel": "k_gemm<Q4_K> (gate)", "achieved": ach, "peak": 5000.0, "unit": "TOP/s", "frac": ach / 5000.0,
+          "traffic": None}, cpu, higher=True)
+    gpu.close()
+
+
+def random_blocks(rng, wtype, rows, k, block_bytes, d_off):
+    """Random legal blocks with small f16 scales (IQ2_XXS stacks: the quantizer's search is too slow for 2.9 GB)."""
+    nb = rows * (k // 256)
+    w = rng.integers(0, 256, nb * block_bytes, dtype=np.uint8).reshape(nb, block_bytes)
+    d = rng.uniform(0.001, 0.02, nb).astype(np.float16).view(np.uint16)
+    w[:, d_off] = d & 0xFF
+    w[:, d_off + 1] = d >> 8
+    return w.reshape(-1)
+
+
+def bench_dsv3(args, bm, ora, threads):
+    """Config 5: DeepSeek-V3-shaped layer, 4 tokens, IQ2_XXS routed experts (grouped) + one Q6_K shared expert."""
+    hidden, ff, n_experts, m, sets = 7168, 2048, 256, 4, 8
+    rng = np.random.default_rng(0xB1000005)
+    t0 = time.time()
+    wg = random_blocks(rng, ora.IQ2_XXS, n_experts * ff, hidden, 66, 0)
+    wu = random_blocks(rng, ora.IQ2_XXS, n_experts * ff, hidden, 66, 0)
+    wd = random_blocks(rng, ora.IQ2_XXS, n_experts * hidden, ff, 66, 0)
+    sg = random_blocks(rng, ora.Q6_K, ff, hidden, 210, 208)
+    su = random_blocks(rng, ora.Q6_K, ff, hidden, 210, 208)
+    sd = random_blocks(rng, ora.Q6_K, hidden, ff, 210, 208)
+    log(f"[bench] stacks drawn ({(wg.nbytes * 2 + wd.nbytes) / 1e9:.2f} GB routed) in {time.time() - t0:.1f}s")
+    x = np.random.default_rng(0xAC70005).standard_normal((m * sets, hidden), dtype=np.float32)
+    ids, wts = biased_routes(ora, m * sets, n_experts, TOP_K, 0x707E0005)
+    gpu = bm.Gpu(0)
+    dg, du, dd = (gpu.weights(bm.IQ2_XXS, n_experts * ff, hidden, wg), gpu.weights(bm.IQ2_XXS, n_experts * ff, hidden, wu),
+                  gpu.weights(bm.IQ2_XXS, n_experts * hidden, ff, wd))
+    dsg, dsu, dsd = gpu.weights(bm.Q6_K, ff, hidden, sg), gpu.weights(bm.Q6_K, ff, hidden, su), gpu.weights(bm.Q6_K, hidden, ff, sd)
+    n_slots = m * TOP_K
+    xd, sel, wt = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32)
+    zeros, ones = gpu.upload(np.zeros(m, np.uint32)), gpu.upload(np.ones(m, np.float32))
+    act, act6 = gpu.act(bm.IQ2_XXS, hidden, m), gpu.act(bm.Q6_K, hidden, m)
+    act_h, act_sh = gpu.act(bm.IQ2_XXS, ff, n_slots), gpu.act(bm.Q6_K, ff, m)
+    h, down = gpu.buffer(np.float32, n_slots * ff), gpu.buffer(np.float32, n_slots * hidden)
+    sdown, yr = gpu.buffer(np.float32, m * hidden), gpu.buffer(np.float32, m * hidden)
+    y = gpu.buffer(np.float32, m * sets * hidden)
+    order, start = gpu.buffer(np.uint32, n_slots), gpu.buffer(np.uint32, n_experts + 1)
+    tiles = gpu.buffer(np.uint32, gpu.tile_cap(n_slots, n_experts) + 1)
+
+    def step(i, which=("routed", "shared", "combine")):
+        st = i % sets
+        s_ptr, x_ptr = sel.ptr + 4 * st * n_slots, xd.ptr + 4 * st * m * hidden
+        if "routed" in which:
+            gpu.enqueue_buckets(s_ptr, n_slots, n_experts, order, start)
+            gpu.enqueue_tiles(start, n_experts, n_slots, tiles)
+            gpu.enqueue_quantize(x_ptr, m, act)
+            gpu.enqueue_gate_up_tiles(dg, du, act, order, start, tiles, n_slots, ff, TOP_K, h)
+            gpu.enqueue_quantize_ord(h, start, n_experts, n_slots, act_h)
+            gpu.enqueue_gemv_tiles(dd, act_h, order, start, tiles, n_slots, hidden, down)
+        if "shared" in which:
+            gpu.enqueue_quantize(x_ptr, m, act6)
+            gpu.enqueue_gate_up(dsg, dsu, act6, zeros, m, ff, 1, None, act_sh)
+            gpu.enqueue_gemv_sel(dsd, act_sh, zeros, m, hidden, sdown)
+        if "combine" in which:
+            gpu.enqueue_combine_tokens(down, wt.ptr + 4 * st * n_slots, None, hidden, TOP_K, m, yr)
+            gpu.enqueue_combine_tokens(sdown, ones, yr, hidden, 1, m, y.ptr + 4 * st * m * hidden)
+
+    step(0)
+    types = (ora.IQ2_XXS, ora.IQ2_XXS, ora.IQ2_XXS)
+    routed = ora.moe_forward(hidden, ff, n_experts, types, wg, wu, wd, x[:m], ids[:m], wts[:m], TOP_K, n_threads=threads)
+    shared = ora.moe_forward(hidden, ff, 1, (ora.Q6_K, ora.Q6_K, ora.Q6_K), sg, su, sd, x[:m], np.zeros((m, 1), np.uint32),
+                             np.ones((m, 1), np.float32), 1, n_threads=threads)
+    want = ora.combine_tokens(np.asarray(shared).reshape(-1), np.ones(m, np.float32), np.asarray(routed).reshape(-1), hidden, 1,
+                              m).reshape(m, hidden)
+    parity = parity_of(y.download()[:m * hidden].reshape(m, hidden), want)
+    wall, ev, steps, warm = timed_graph(gpu, step, 16, min(args.steps, 256), min(args.warmup, 32))
+    kernel_us = {k: timed_graph(gpu, lambda i, k=k: step(i, (k,)), 16, 64, 16)[1] * 1e3 for k in ("routed", "shared", "combine")}
+    hit = np.mean([len(np.unique(ids[s * m:(s + 1) * m])) for s in range(sets)])
+    per_expert = (2 * ff * bm.row_bytes(bm.IQ2_XXS, hidden) + hidden * bm.row_bytes(bm.IQ2_XXS, ff))
+    shared_bytes = 2 * ff * bm.row_bytes(bm.Q6_K, hidden) + hidden * bm.row_bytes(bm.Q6_K, ff)
+    nbytes = hit * per_expert + shared_bytes
+    ach = nbytes / (wall * 1e-3) / 1e9
+    cpu = None
+    emit("moe_layer_decode_us_per_token", wall * 1e3 / m, "us/token", steps, warm, wall,
+         "DeepSeek-V3-shaped MoE layer decode, 4 tokens: hidden 7168, 256 IQ2_XXS experts of ff 2048 top-8 grouped by expert + one "
+         "Q6_K shared expert; random legal blocks (BASELINE.json configs[4])",
+         {"event_ms_per_step": ev, "kernel_us": kernel_us, "parity": parity, "distinct_experts_per_step": float(hit),
+          "algorithmic_bytes_per_step": nbytes, "hbm_tbps": ach / 1e3},
+         {"bound": "hbm", "kernel": "whole step (11 launches)", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+          "frac": ach / HBM_PEAK_GBS, "traffic": None}, cpu)
+    gpu.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5),
+                    help="1: one Q4_K gemv; 2 (default, the headline): Qwen3-shaped layer, 1 token; 3: the same layer, 16 tokens "
+                         "grouped by expert; 4: prefill of 2048 tokens (int8 MFMA GEMM); 5: DeepSeek-V3-shaped layer, 4 tokens")
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2048)
     ap.add_argument("--warmup", type=int, default=256)
@@ -81,6 +408,8 @@ def main():
     import ora
 
     threads = min(os.cpu_count() or 1, 16)
+    if args.config != 2:
+        return {1: bench_gemv, 3: bench_grouped, 4: bench_prefill, 5: bench_dsv3}[args.config](args, bm, ora, threads)
     t0 = time.time()
     wg, wu, wd = make_layer(ora, 0xB1000001, threads)
     x, ids, wts = make_tokens(ora, args.tokens, 0xAC70001)

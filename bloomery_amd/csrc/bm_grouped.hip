@@ -16,76 +16,48 @@ int tile_cap(int n_slots, int n_experts) { // crates/gpu/src/q4k_sel.rs:96-98
 
 // ---------------------------------------------------------------------------------------------- tables
 
-// crates/gpu/src/q4k_sel.rs:480-560 grouped_buckets: one workgroup of 1024 threads, a thread an expert. Slots keep
-// their order inside a run. An id at or past the stack that is not the host's raises ExpertId and joins no run.
+// crates/gpu/src/q4k_sel.rs:480-560 grouped_buckets: one workgroup of 1024 threads. Slots keep their order inside
+// a run. An id at or past the stack that is not the host's raises ExpertId and joins no run.
 __global__ __launch_bounds__(1024) void k_buckets(const u32 *sel, u32 n_slots, u32 n_experts, u32 *order, u32 *start,
                                                   u32 *fault, u32 layer) {
-    __shared__ u32 count[kBucketExperts];
-    const u32 tid = threadIdx.x;
-    for (u32 s = tid; s < n_slots; s += blockDim.x) {
+    __shared__ GroupLds g;
+    group_slots(g, n_slots, n_experts, order, [&](u32 s) {
         const u32 p = sel[s];
-        if (p >= n_experts && p != kHostSlot) bm_raise(fault, layer, kSiteExpertId);
-    }
-    if (tid < n_experts) {
-        u32 c = 0;
-        for (u32 s = 0; s < n_slots; s++) c += sel[s] == tid;
-        count[tid] = c;
-    }
-    __syncthreads();
-    if (tid == 0) {
-        u32 at = 0;
-        for (u32 e = 0; e < n_experts; e++) {
-            const u32 c = count[e];
-            start[e] = at;
-            count[e] = at;
-            at += c;
-        }
-        start[n_experts] = at;
-    }
-    __syncthreads();
-    if (tid < n_experts) {
-        u32 at = count[tid];
-        for (u32 s = 0; s < n_slots; s++)
-            if (sel[s] == tid) order[at++] = s;
-    }
+        if (p < n_experts) return p;
+        if (p != kHostSlot) bm_raise(fault, layer, kSiteExpertId);
+        return kNoBucket;
+    });
+    for (u32 e = threadIdx.x; e <= n_experts; e += blockDim.x) start[e] = g.base[e];
 }
 
 // crates/gpu/src/q4k_sel.rs:562-680 grouped_tiles. A run outside 0 .. start[n_experts] <= n_slots, or more tiles
 // than `cap`, raise ExpertId and leave a count of 0.
 __global__ __launch_bounds__(1024) void k_tiles(const u32 *start, u32 n_experts, u32 n_slots, u32 cap, u32 *tiles,
                                                 u32 *fault, u32 layer) {
-    __shared__ u32 at[kBucketExperts];
-    __shared__ u32 total;
+    __shared__ u32 scan[17];
+    __shared__ u32 bad;
     const u32 tid = threadIdx.x;
     const u32 end = start[n_experts];
+    if (tid == 0) bad = 0;
+    __syncthreads();
+    u32 j0 = 0, j1 = 0, c = 0;
     if (tid < n_experts) {
-        const u32 j0 = start[tid], j1 = start[tid + 1];
-        at[tid] = (j0 <= j1 && j1 <= end && end <= n_slots) ? (j1 - j0 + kTileCols - 1) / kTileCols : 0xffffffffu;
+        j0 = start[tid];
+        j1 = start[tid + 1];
+        if (j0 <= j1 && j1 <= end && end <= n_slots)
+            c = (j1 - j0 + kTileCols - 1) / kTileCols; // at most 2^19: the sum of 1024 of them fits a word
+        else
+            bad = 1;
     }
-    __syncthreads();
+    u32 total;
+    u32 g = block_scan_1024(c, scan, &total); // its barriers publish `bad`
+    const bool refuse = bad != 0 || total > cap;
     if (tid == 0) {
-        u32 sum = 0;
-        for (u32 e = 0; e < n_experts; e++) {
-            const u32 c = at[e];
-            if (c == 0xffffffffu || c > cap - sum) {
-                sum = 0xffffffffu;
-                break;
-            }
-            at[e] = sum;
-            sum += c;
-        }
-        if (sum == 0xffffffffu) {
-            bm_raise(fault, layer, kSiteExpertId);
-            sum = 0;
-        }
-        total = sum;
-        tiles[0] = sum;
+        if (refuse) bm_raise(fault, layer, kSiteExpertId);
+        tiles[0] = refuse ? 0 : total;
     }
-    __syncthreads();
-    if (tid < n_experts && total != 0) {
-        u32 g = at[tid];
-        for (u32 j = start[tid], j1 = start[tid + 1]; j < j1; j += kTileCols) tiles[1 + g++] = (tid << kTileExpertShift) | j;
-    }
+    if (tid < n_experts && !refuse)
+        for (u32 j = j0; j < j1; j += kTileCols) tiles[1 + g++] = (tid << kTileExpertShift) | j;
 }
 
 hipError_t buckets(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start) {

@@ -20,8 +20,7 @@ namespace bmk {
 
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr u32 kNoExpert = 0xffffffffu;
-constexpr int kRouteThreads = 1024, kRouteWaves = kRouteThreads / 64, kRouteHist = 8192;
+constexpr int kRouteThreads = 1024;
 
 int gemm_max_tiles(int n_slots, int n_experts) { // crates/gpu/src/gemm/route.rs:55-57
     return n_slots / kGemmBN + (n_experts < n_slots ? n_experts : n_slots);
@@ -29,90 +28,33 @@ int gemm_max_tiles(int n_slots, int n_experts) { // crates/gpu/src/gemm/route.rs
 
 // ------------------------------------------------------------------------------------------------ route
 
-// One workgroup. The slots are cut into up to 16 chunks, a wave a chunk; counts per (chunk, expert) in LDS give
-// every chunk its place inside every expert's run, so the waves place their slots independently and each run stays
-// in ascending slot order. Bucket n_experts collects the refused slots.
+// One workgroup: the slots listed by expert in ascending slot order (group_slots), bucket n_experts collecting the
+// refused ones at the list's end; then the tiles, an expert's run cut into runs of at most 64.
 __global__ __launch_bounds__(kRouteThreads) void k_route(const u32 *ids, u32 n_slots, u32 n_experts, u32 *cols,
                                                          u32 *tiles, u32 *n_tiles, u32 *fault, u32 layer) {
-    __shared__ u32 hist[kRouteHist + kRouteWaves]; // [chunk][bucket], bucket in 0..=n_experts
-    __shared__ u32 base[kGemmMaxExperts + 2];      // first index of every bucket's run
-    __shared__ u32 tile_at[kGemmMaxExperts + 1];
-    const u32 tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const u32 nbk = n_experts + 1;
-    u32 chunks = kRouteHist / nbk;
-    chunks = chunks < (u32)kRouteWaves ? chunks : (u32)kRouteWaves;
-    const u32 per = (n_slots + chunks - 1) / chunks;
-    for (u32 i = tid; i < chunks * nbk; i += blockDim.x) hist[i] = 0;
-    __syncthreads();
-    if (wave < chunks) {
-        const u32 lo = wave * per, hi = lo + per < n_slots ? lo + per : n_slots;
-        for (u32 s = lo + lane; s < hi; s += 64) {
-            const u32 id = ids[s];
-            const u32 b = id < n_experts ? id : n_experts;
-            if (b == n_experts) bm_raise(fault, layer, kSiteExpertId);
-            atomicAdd(&hist[wave * nbk + b], 1u);
-        }
-    }
-    __syncthreads();
-    for (u32 b = tid; b < nbk; b += blockDim.x) { // counts a chunk -> the chunk's offset inside the bucket's run
-        u32 sum = 0;
-        for (u32 c = 0; c < chunks; c++) {
-            const u32 v = hist[c * nbk + b];
-            hist[c * nbk + b] = sum;
-            sum += v;
-        }
-        base[b] = sum; // the bucket's count, for now
-    }
-    __syncthreads();
-    if (tid == 0) {
-        u32 at = 0, t = 0;
-        for (u32 e = 0; e < n_experts; e++) {
-            const u32 c = base[e];
-            base[e] = at;
-            tile_at[e] = t;
-            at += c;
-            t += (c + kGemmBN - 1) / kGemmBN;
-        }
-        const u32 refused = base[n_experts];
-        base[n_experts] = at;      // the refused slots close the list
-        base[n_experts + 1] = at + refused;
-        tile_at[n_experts] = t;
-        n_tiles[0] = t;
-        n_tiles[1] = refused;
-    }
-    __syncthreads();
-    if (wave < chunks) {
-        volatile u32 *off = &hist[wave * nbk];
-        const u32 lo = wave * per, hi = lo + per < n_slots ? lo + per : n_slots;
-        for (u32 s0 = lo; s0 < hi; s0 += 64) {
-            const u32 s = s0 + lane;
-            u32 b = kNoExpert;
-            if (s < hi) {
-                const u32 id = ids[s];
-                b = id < n_experts ? id : n_experts;
-            }
-            unsigned long long todo = __ballot(b != kNoExpert);
-            while (todo) { // the lanes of one bucket at a time, in lane (= slot) order
-                const int leader = __builtin_ctzll(todo);
-                const u32 lb = (u32)__builtin_amdgcn_readlane((int)b, leader);
-                const unsigned long long same = __ballot(b == lb);
-                const u32 first = off[lb];
-                if (b == lb) cols[base[lb] + first + (u32)__builtin_popcountll(same & ((1ull << lane) - 1ull))] = s;
-                __builtin_amdgcn_wave_barrier();
-                if (lane == (u32)leader) off[lb] = first + (u32)__builtin_popcountll(same);
-                __builtin_amdgcn_wave_barrier();
-                todo &= ~same;
-            }
-        }
-    }
+    __shared__ GroupLds g;
+    const u32 tid = threadIdx.x;
+    group_slots(g, n_slots, n_experts + 1, cols, [&](u32 s) {
+        const u32 id = ids[s];
+        return id < n_experts ? id : n_experts;
+    });
+    u32 j0 = 0, j1 = 0;
     if (tid < n_experts) {
-        const u32 j0 = base[tid], j1 = base[tid + 1];
-        u32 t = tile_at[tid];
-        for (u32 j = j0; j < j1; j += kGemmBN, t++) {
-            const u32 len = j1 - j < (u32)kGemmBN ? j1 - j : (u32)kGemmBN;
-            tiles[2 * t] = tid;
-            tiles[2 * t + 1] = j | (len << 16);
-        }
+        j0 = g.base[tid];
+        j1 = g.base[tid + 1];
+    }
+    u32 total;
+    u32 t = block_scan_1024((j1 - j0 + kGemmBN - 1) / kGemmBN, g.scan, &total);
+    for (u32 j = j0; j < j1; j += kGemmBN, t++) {
+        const u32 len = j1 - j < (u32)kGemmBN ? j1 - j : (u32)kGemmBN;
+        tiles[2 * t] = tid;
+        tiles[2 * t + 1] = j | (len << 16);
+    }
+    if (tid == 0) {
+        const u32 refused = g.base[n_experts + 1] - g.base[n_experts];
+        if (refused) bm_raise(fault, layer, kSiteExpertId);
+        n_tiles[0] = total;
+        n_tiles[1] = refused;
     }
 }
 

@@ -250,6 +250,110 @@ __device__ __forceinline__ void quantize_h_block(const float *hbuf, uint8_t *hco
     q82_store(hcol, nb_h, rb, tid, code, hd, s16);
 }
 
+// ------------------------------------------------------------------------------------- grouping by expert
+
+// Exclusive prefix sum over the 1024 threads of a workgroup (value v of thread tid); *total gets the sum.
+// `scratch` holds 17 words of LDS. Every thread calls it.
+__device__ __forceinline__ u32 block_scan_1024(u32 v, u32 *scratch, u32 *total) {
+    const u32 tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    u32 inc = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const u32 o = (u32)__shfl_up((int)inc, d, 64);
+        if (lane >= (u32)d) inc += o;
+    }
+    if (lane == 63) scratch[wave] = inc;
+    __syncthreads();
+    if (tid == 0) {
+        u32 at = 0;
+        for (int w = 0; w < 16; w++) {
+            const u32 c = scratch[w];
+            scratch[w] = at;
+            at += c;
+        }
+        scratch[16] = at;
+    }
+    __syncthreads();
+    *total = scratch[16];
+    return scratch[wave] + inc - v;
+}
+
+
+// The slots 0 .. n of a workgroup of 1024 threads listed by bucket (an expert, or one more bucket a caller adds),
+// ascending slot order inside a bucket - the stable counting sort both slot tables are. The slots are cut into up
+// to 16 chunks, a wave a chunk: counts per (chunk, bucket) give every chunk its place inside every bucket's run, so
+// the waves place their slots independently; inside a wave 64 consecutive slots are placed at a time, each lane's
+// rank among the lanes of its bucket read off the ballots of the bucket's bits.
+constexpr u32 kNoBucket = 0xffffffffu;
+constexpr int kGroupHist = 8192, kGroupWaves = 16, kGroupBuckets = 1025;
+struct GroupLds {
+    u32 hist[kGroupHist + kGroupWaves]; // [chunk][bucket]: the chunk's next place inside the bucket's run
+    u32 base[kGroupBuckets + 1];        // bucket b's run is list[base[b] .. base[b + 1]]
+    u32 scan[17];
+};
+
+// bucket_of(s): slot s's bucket below n_buckets, or kNoBucket for a slot that joins no run. Called twice a slot.
+// Every thread of the workgroup calls group_slots; afterwards g.base holds the runs' bounds.
+template <class BucketOf>
+__device__ __forceinline__ void group_slots(GroupLds &g, u32 n, u32 n_buckets, u32 *list, const BucketOf &bucket_of) {
+    const u32 tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    u32 chunks = (u32)kGroupHist / n_buckets;
+    chunks = chunks < (u32)kGroupWaves ? chunks : (u32)kGroupWaves;
+    const u32 per = ((n + chunks - 1) / chunks + 63) & ~63u; // whole batches of 64 a chunk
+    const u32 lo = wave * per, hi = lo + per < n ? lo + per : n;
+    for (u32 i = tid; i < chunks * n_buckets; i += blockDim.x) g.hist[i] = 0;
+    __syncthreads();
+    if (wave < chunks)
+        for (u32 s = lo + lane; s < hi; s += 64) {
+            const u32 b = bucket_of(s);
+            if (b != kNoBucket) atomicAdd(&g.hist[wave * n_buckets + b], 1u);
+        }
+    __syncthreads();
+    u32 count = 0;
+    for (u32 b = tid; b < n_buckets; b += blockDim.x) { // a chunk's count -> its offset inside the bucket's run
+        u32 sum = 0;
+        for (u32 c = 0; c < chunks; c++) {
+            const u32 v = g.hist[c * n_buckets + b];
+            g.hist[c * n_buckets + b] = sum;
+            sum += v;
+        }
+        if (b < 1024) count = sum;
+        else g.base[kGroupBuckets] = sum; // bucket 1024's count, parked
+    }
+    u32 total;
+    const u32 at = block_scan_1024(count, g.scan, &total);
+    if (tid < n_buckets) g.base[tid] = at;
+    if (tid == 0) {
+        if (n_buckets == (u32)kGroupBuckets) {
+            const u32 last = g.base[kGroupBuckets];
+            g.base[1024] = total;
+            g.base[kGroupBuckets] = total + last;
+        } else {
+            g.base[n_buckets] = total;
+        }
+    }
+    __syncthreads();
+    if (wave < chunks) {
+        const int bits = 32 - __builtin_clz(n_buckets | 1u);
+        for (u32 s0 = lo; s0 < hi; s0 += 64) {
+            const u32 s = s0 + lane;
+            const u32 b = s < hi ? bucket_of(s) : kNoBucket;
+            const bool live = b != kNoBucket;
+            unsigned long long same = __ballot(live);
+            for (int k = 0; k < bits; k++) {
+                const unsigned long long set = __ballot((b >> k) & 1u);
+                same &= ((b >> k) & 1u) ? set : ~set;
+            }
+            const int leader = live ? __builtin_ctzll(same) : (int)lane;
+            u32 first = 0;
+            if (live && lane == (u32)leader) first = atomicAdd(&g.hist[wave * n_buckets + b], (u32)__builtin_popcountll(same));
+            first = (u32)__shfl((int)first, leader, 64);
+            if (live) list[g.base[b] + first + (u32)__builtin_popcountll(same & ((1ull << lane) - 1ull))] = s;
+        }
+    }
+    __syncthreads();
+}
+
 // ---------------------------------------------------------------------------------------- launch helpers
 
 template <typename K>

@@ -124,7 +124,7 @@ __device__ __forceinline__ u32 q6_minus_32(u32 q) {
 }
 
 template <int WT>
-__global__ __launch_bounds__(256) void k_gemm(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
+__global__ __launch_bounds__(256, 2) void k_gemm(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
                                               const u32 *tiles, const u32 *n_tiles, u32 max_tiles, u32 slot_div,
                                               u32 n_slots, float *y) {
     extern __shared__ __align__(16) uint8_t lds[];

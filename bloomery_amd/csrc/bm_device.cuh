@@ -404,9 +404,39 @@ __device__ __forceinline__ Act<BM_IQ2XXS> bm_act_iq2xxs(const ActView &av, int i
     return a;
 }
 
+// The block's codes as this lane dots them: per sub-block the eight signed grid values (two words) and the
+// scale 2s + 1. Decoded once a super-block, whatever the number of columns.
+struct Iq2Dec {
+    u32 v_lo[8], v_hi[8];
+    int sc[8];
+};
+
+__device__ __forceinline__ Iq2Dec bm_decode_iq2xxs(const Blk<BM_IQ2XXS> &b, int q, const Iq2Tables &tb) {
+    Iq2Dec dec;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        // Quarter k of the block (sub-blocks 2k, 2k + 1) sits in lane k of the quad.
+        const u32 idx_a = bm_quad_bcast(b.q.x, k), aux_a = bm_quad_bcast(b.q.y, k);
+        const u32 idx_b = bm_quad_bcast(b.q.z, k), aux_b = bm_quad_bcast(b.q.w, k);
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const int sb = 2 * k + e;
+            const u32 idx = e ? idx_b : idx_a, aux = e ? aux_b : aux_a;
+            dec.sc[sb] = 2 * (int)(aux >> 28) + 1;
+            const uint2 g = tb.grid[(idx >> (8 * q)) & 0xffu];
+            const u32 sg = tb.ksigns[(aux >> (7 * q)) & 127u];
+            const u32 m_lo = tb.nibmask[sg & 15u], m_hi = tb.nibmask[sg >> 4];
+            // -mag where the sign bit is set: (mag ^ 0xff) + 1 per byte, no carry leaves a byte (mag > 0).
+            dec.v_lo[sb] = (g.x ^ m_lo) + (m_lo & 0x01010101u);
+            dec.v_hi[sb] = (g.y ^ m_hi) + (m_hi & 0x01010101u);
+        }
+    }
+    return dec;
+}
+
 template <class Tap>
-__device__ __forceinline__ void bm_dot_iq2xxs(const Blk<BM_IQ2XXS> &b, const Act<BM_IQ2XXS> &act, int i, int q,
-                                              const Iq2Tables &tb, float &acc0, float &acc1, const Tap &tap) {
+__device__ __forceinline__ void bm_dot_iq2xxs_dec(const Blk<BM_IQ2XXS> &b, const Iq2Dec &dec, const Act<BM_IQ2XXS> &act,
+                                                  int i, int q, float &acc0, float &acc1, const Tap &tap) {
     const float dy = act.dy;
     const float d = 0.125f * bm_half_to_f32(b.d);
     const float dmin = -d * 43.0f;
@@ -423,32 +453,25 @@ __device__ __forceinline__ void bm_dot_iq2xxs(const Blk<BM_IQ2XXS> &b, const Act
     }
     int sumi0 = 0, sumi1 = 0;
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
-        // Quarter k of the block (sub-blocks 2k, 2k + 1) sits in lane k of the quad.
-        const u32 idx_a = bm_quad_bcast(b.q.x, k), aux_a = bm_quad_bcast(b.q.y, k);
-        const u32 idx_b = bm_quad_bcast(b.q.z, k), aux_b = bm_quad_bcast(b.q.w, k);
-#pragma unroll
-        for (int e = 0; e < 2; e++) {
-            const int sb = 2 * k + e;
-            const u32 idx = e ? idx_b : idx_a, aux = e ? aux_b : aux_a;
-            const int sc = 2 * (int)(aux >> 28) + 1;
-            const uint2 g = tb.grid[(idx >> (8 * q)) & 0xffu];
-            const u32 sg = tb.ksigns[(aux >> (7 * q)) & 127u];
-            const u32 m_lo = tb.nibmask[sg & 15u], m_hi = tb.nibmask[sg >> 4];
-            // -mag where the sign bit is set: (mag ^ 0xff) + 1 per byte, no carry leaves a byte (mag > 0).
-            const u32 v_lo = (g.x ^ m_lo) + (m_lo & 0x01010101u), v_hi = (g.y ^ m_hi) + (m_hi & 0x01010101u);
-            const uint2 a = act.a[sb];
-            const int i_lo = bm_sdot4(v_lo, a.x, 0), i_hi = bm_sdot4(v_hi, a.y, 0);
-            const int s_lo = bm_sdot4(0x01010101u, a.x, 0), s_hi = bm_sdot4(0x01010101u, a.y, 0);
-            // the reference sums sc * (v + 43) * a: the offset comes back out through the fold above
-            sumi0 += sc * (i_lo + 43 * s_lo);
-            sumi1 += sc * (i_hi + 43 * s_hi);
-            tap.iq2(i, sb, q, i_lo + i_hi);
-        }
+    for (int sb = 0; sb < 8; sb++) {
+        const uint2 a = act.a[sb];
+        const int i_lo = bm_sdot4(dec.v_lo[sb], a.x, 0), i_hi = bm_sdot4(dec.v_hi[sb], a.y, 0);
+        const int s_lo = bm_sdot4(0x01010101u, a.x, 0), s_hi = bm_sdot4(0x01010101u, a.y, 0);
+        // the reference sums sc * (v + 43) * a: the offset comes back out through the fold above
+        sumi0 += dec.sc[sb] * (i_lo + 43 * s_lo);
+        sumi1 += dec.sc[sb] * (i_hi + 43 * s_hi);
+        tap.iq2(i, sb, q, i_lo + i_hi);
     }
     const float f = d * dy;
     acc0 = fmaf(f, (float)sumi0, acc0);
     acc1 = fmaf(f, (float)sumi1, acc1);
+}
+
+template <class Tap>
+__device__ __forceinline__ void bm_dot_iq2xxs(const Blk<BM_IQ2XXS> &b, const Act<BM_IQ2XXS> &act, int i, int q,
+                                              const Iq2Tables &tb, float &acc0, float &acc1, const Tap &tap) {
+    const Iq2Dec dec = bm_decode_iq2xxs(b, q, tb);
+    bm_dot_iq2xxs_dec(b, dec, act, i, q, acc0, acc1, tap);
 }
 
 // ---- closing sums: (t0 + t2) + (t1 + t3) with t_l = acc_l + acc_{l+4}; every lane of the quad gets the value.

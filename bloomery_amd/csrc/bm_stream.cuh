@@ -160,12 +160,22 @@ __device__ __forceinline__ void row_dot(Blk<WT> (&b)[U], const uint8_t *wrow, co
         auto stage = [&](int slot, int fill, int i) {
             const int ahead = i + U - 1 < n ? i + U - 1 : n - 1;
             b[fill] = bm_load_blk<WT>(wrow, U > 1 ? ahead : i, q);
+            if constexpr (WT == BM_IQ2XXS) { // the table lookups once, not once a column
+                const Iq2Dec dec = bm_decode_iq2xxs(b[slot], q, tb);
 #pragma unroll
-            for (int c = 0; c < M; c++)
-                if (c < m) {
-                    const Act<WT> a = bm_load_act<WT, Tap::kActive>(av[c], i, q);
-                    bm_dot_blk<WT>(b[slot], a, i, q, tb, a0[c], a1[c], tap);
-                }
+                for (int c = 0; c < M; c++)
+                    if (c < m) {
+                        const Act<WT> a = bm_load_act<WT, Tap::kActive>(av[c], i, q);
+                        bm_dot_iq2xxs_dec(b[slot], dec, a, i, q, a0[c], a1[c], tap);
+                    }
+            } else {
+#pragma unroll
+                for (int c = 0; c < M; c++)
+                    if (c < m) {
+                        const Act<WT> a = bm_load_act<WT, Tap::kActive>(av[c], i, q);
+                        bm_dot_blk<WT>(b[slot], a, i, q, tb, a0[c], a1[c], tap);
+                    }
+            }
         };
         if constexpr (NB > 0) {
 #pragma unroll

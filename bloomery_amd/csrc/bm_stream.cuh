@@ -376,7 +376,7 @@ static hipError_t allow_lds(K kernel, size_t lds) {
 // Picks the kernel variant for a row of nb super-blocks and runs CALL_BODY with WT, U and NB as constants. Each
 // type lists the hot shape first (its count known at compile time, stages unrolled), then a ring of two for even
 // counts, then one super-block at a time, which divides every row.
-constexpr int kRingQ4K = 3, kRingQ6K = 2;
+constexpr int kRingQ4K = 4, kRingQ6K = 3;
 #define BM_VARIANT(T, UU, NN)                                                                                          \
     {                                                                                                                  \
         constexpr int WT = T, U = UU, NB = NN;                                                                         \

@@ -27,6 +27,9 @@ for p in (ROOT, os.path.join(ROOT, "oracle")):
 
 HIDDEN, FF, N_EXPERTS, TOP_K = 2048, 768, 128, 8
 HBM_PEAK_GBS = 8000.0
+# HBM bytes a launch of the headline configuration's dominant kernel moves (read + written), from the rocprofv3
+# FETCH_SIZE / WRITE_SIZE summary under profiles/ (counter x the copy-kernel calibration measured in the same run).
+GATE_UP_X_TRAFFIC_BYTES = 14398180
 
 
 def log(*a):
@@ -389,6 +392,9 @@ def main():
                     help="1: one Q4_K gemv; 2 (default, the headline): Qwen3-shaped layer, 1 token; 3: the same layer, 16 tokens "
                          "grouped by expert; 4: prefill of 2048 tokens (int8 MFMA GEMM); 5: DeepSeek-V3-shaped layer, 4 tokens")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="config 2 only: no timing; 8 copies of 64 MiB by a plain kernel (the counters' calibration), then "
+                         "256 eager steps - the run to put under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2048)
     ap.add_argument("--warmup", type=int, default=256)
@@ -451,6 +457,18 @@ def main():
         if "down" in which:
             gpu.enqueue_down_combine(dd, act_h, sel.ptr + 4 * t * TOP_K, wt.ptr + 4 * t * TOP_K, None, TOP_K, 1, HIDDEN,
                                      y.ptr + 4 * t * HIDDEN)
+
+    if args.traffic_probe:
+        n = 1 << 24  # 64 MiB of f32 in, 64 MiB out: combine over one slot of weight 1 is a copy
+        src, dst, one = gpu.buffer(np.float32, n).fill_bytes(0), gpu.buffer(np.float32, n), gpu.upload(np.ones(16, np.float32))
+        for _ in range(8):
+            gpu.enqueue_combine_tokens(src, one, None, n // 16, 1, 16, dst)
+        for i in range(256):
+            enqueue_step(i)
+        gpu.sync()
+        log("[bench] traffic probe done: 8 x k_combine copies of 67108864 B each way, 256 steps")
+        gpu.close()
+        return
 
     # parity first: the first tokens against the oracle, same seeded inputs
     parity = None
@@ -566,7 +584,8 @@ def main():
         "kernel_gbps": kernel_gbps,
         "parity": parity,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": GATE_UP_X_TRAFFIC_BYTES if args.mode == "two" else None,
                      "algorithmic_bytes_per_launch": dom_bytes},
         "cpu_baseline": cpu,
     }

@@ -7,8 +7,8 @@
 // refused count}.
 //
 // The GEMM's numbers are the decode path's, bit for bit: every (row, slot) value is the one-column row dot of
-// bm_device.cuh. The integer sums of each 16-value group come out of v_mfma_i32_32x32x16_i8 (one instruction a
-// group: 32 rows x 32 slots x 16 values, exact), and each enters the f32 accumulator of the CPU path's lane that
+// bm_device.cuh. The integer sums of each 16-value group come out of v_mfma_i32_16x16x32_i8 (16 rows x 16 slots,
+// exact; the other half of the 32 values zeroed on the weight side), and each enters the f32 accumulator of the CPU path's lane that
 // owns it, in the CPU path's order (crates/qdot/src/lib.rs:4363-4447 Q4_K, :4776-4874 Q6_K): eight accumulators a
 // value, the min term first, then the groups in increasing k, and the closing sum (t0 + t2) + (t1 + t3).
 // Activation scales come per 32 values in this form, so every group's sum is scaled on the vector ALU before it is
@@ -18,7 +18,7 @@
 
 namespace bmk {
 
-typedef int v16i __attribute__((ext_vector_type(16)));
+typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr int kRouteThreads = 1024;
 
@@ -123,10 +123,15 @@ __device__ __forceinline__ u32 q6_minus_32(u32 q) {
     return t | (m << 1) | (m << 2);
 }
 
-template <int WT>
-__global__ __launch_bounds__(256, 2) void k_gemm(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
-                                              const u32 *tiles, const u32 *n_tiles, u32 max_tiles, u32 slot_div,
-                                              u32 n_slots, float *y) {
+// A workgroup of 1024 / T threads takes a tile of <= 64 slots and a slab of 64 rows. Wave w works on rows
+// 16 * (w & 3) .. and slots 16 T * (w >> 2) ..: T 16 x 16 products a 32-value block and half. v_mfma_i32_16x16x32_i8 sums over 32
+// values; a 16-value half comes out of it by zeroing the other half's weight codes, the lanes of one half of the
+// k range holding them (lane / 16 = k / 8). 4 T results a lane, 32 T accumulators: two to four waves a SIMD
+// stay resident and hide each other's LDS and matrix latencies.
+template <int WT, int T>
+__global__ __launch_bounds__(1024 / T) void k_gemm(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
+                                                 const u32 *tiles, const u32 *n_tiles, u32 max_tiles, u32 slot_div,
+                                                 u32 n_slots, float *y) {
     extern __shared__ __align__(16) uint8_t lds[];
     GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
     uint8_t *acts = lds + sizeof(GemmLds);
@@ -160,12 +165,13 @@ __global__ __launch_bounds__(256, 2) void k_gemm(const uint8_t *w, int rpe, int 
     const int col_bytes = nb * BM_Q82_SB_EXT;
     // staging: kGemmBN * 22 chunks of 16 bytes of activations, kGemmBM * kWc of weights, a super-block
     constexpr int kAc = kActSb / 16; // 22
-    constexpr int kActLoads = (kGemmBN * kAc + 255) / 256, kWtLoads = (kGemmBM * kWc + 255) / 256;
+    constexpr int kThreads = 1024 / T; // 16 / T waves: four row groups x (4 / T) slot groups of 16 T slots
+    constexpr int kActLoads = (kGemmBN * kAc + kThreads - 1) / kThreads, kWtLoads = (kGemmBM * kWc + kThreads - 1) / kThreads;
     uint4 ra[kActLoads], rw[kWtLoads];
     auto fetch = [&](int i) {
 #pragma unroll
         for (int t = 0; t < kActLoads; t++) {
-            int c = t * 256 + tid;
+            int c = t * kThreads + tid;
             c = c < kGemmBN * kAc ? c : kGemmBN * kAc - 1;
             const int n = c / kAc, k = c % kAc;
             const uint8_t *colp = act + (size_t)tab->col[n] * col_bytes;
@@ -175,7 +181,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm(const uint8_t *w, int rpe, int 
         }
 #pragma unroll
         for (int t = 0; t < kWtLoads; t++) {
-            int c = t * 256 + tid;
+            int c = t * kThreads + tid;
             c = c < kGemmBM * kWc ? c : kGemmBM * kWc - 1;
             int r = row0 + c / kWc;
             const int k = c % kWc;
@@ -188,7 +194,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm(const uint8_t *w, int rpe, int 
     auto stash = [&]() {
 #pragma unroll
         for (int t = 0; t < kActLoads; t++) {
-            const int c = t * 256 + tid;
+            const int c = t * kThreads + tid;
             if (c < kGemmBN * kAc) {
                 uint8_t *dst = acts + (c / kAc) * kActStride + 16 * (c % kAc);
                 *reinterpret_cast<uint2 *>(dst) = make_uint2(ra[t].x, ra[t].y);
@@ -197,7 +203,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm(const uint8_t *w, int rpe, int 
         }
 #pragma unroll
         for (int t = 0; t < kWtLoads; t++) {
-            const int c = t * 256 + tid;
+            const int c = t * kThreads + tid;
             if (c < kGemmBM * kWc) {
                 uint8_t *dst = wts + (c / kWc) * wt_stride<WT>() + 16 * (c % kWc);
                 *reinterpret_cast<uint2 *>(dst) = make_uint2(rw[t].x, rw[t].y);
@@ -205,17 +211,22 @@ __global__ __launch_bounds__(256, 2) void k_gemm(const uint8_t *w, int rpe, int 
             }
         }
     };
-    // this lane in its wave's 32 x 32 product: operand row / column lane % 32, value half lane / 32; the sixteen
-    // results it holds are rows 8 * (v / 4) + 4 * (lane / 32) + v % 4 of column lane % 32
-    const int wr = wv & 1, wc = wv >> 1, l32 = lane & 31, kh = lane >> 5;
-    const uint8_t *my_act = acts + (32 * wc + l32) * kActStride;
-    const uint8_t *my_wt = wts + (32 * wr + l32) * wt_stride<WT>();
-    const int rbase = 32 * wr + 4 * kh; // result v sits in row rbase + 8 * (v / 4) + v % 4 of the slab
-    float acc[16][8];
+    // this lane in its wave's two 16 x 16 products: operand row / slot lane % 16, values 8 * (lane / 16) .. + 8 of
+    // a 32-value block; its four results of each product are rows 4 * (lane / 16) + v of slot lane % 16
+    const int rg = wv & 3, ch = wv >> 2, l16 = lane & 15, kg = lane >> 4;
+    const uint8_t *my_act[T];
 #pragma unroll
-    for (int v = 0; v < 16; v++)
+    for (int t = 0; t < T; t++) my_act[t] = acts + (16 * T * ch + 16 * t + l16) * kActStride;
+    const uint8_t *my_wt = wts + (16 * rg + l16) * wt_stride<WT>();
+    const int rbase = 16 * rg + 4 * kg; // result v sits in row rbase + v of the slab
+    const u32 keep[2] = {kg < 2 ? 0xffffffffu : 0u, kg < 2 ? 0u : 0xffffffffu}; // this lane's codes are of half kg / 2
+    float acc[T][4][8];
 #pragma unroll
-        for (int l = 0; l < 8; l++) acc[v][l] = 0.0f;
+    for (int t = 0; t < T; t++)
+#pragma unroll
+        for (int v = 0; v < 4; v++)
+#pragma unroll
+            for (int l = 0; l < 8; l++) acc[t][v][l] = 0.0f;
 
     fetch(0);
     for (int i = 0; i < nb; i++) {
@@ -225,15 +236,14 @@ __global__ __launch_bounds__(256, 2) void k_gemm(const uint8_t *w, int rpe, int 
         if (i + 1 < nb) fetch(i + 1);
         // the rows' scale products: rs[s][row]
         {
-            const int r = tid >> 2, part = tid & 3;
+            const int r = (tid >> 3) & 63, part = tid & 7;
             const uint8_t *blk = wts + r * wt_stride<WT>();
-            if constexpr (WT == BM_Q4K) {
-                const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk));
-                const float dmin = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk + 2));
-                const uint8_t *sc = blk + 4;
-#pragma unroll
-                for (int t = 0; t < 2; t++) { // crates/gguf/src/quant.rs:620-628 get_scale_min_k4
-                    const int s = 2 * part + t;
+            if (tid < 512) {
+                if constexpr (WT == BM_Q4K) {
+                    const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk));
+                    const float dmin = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk + 2));
+                    const uint8_t *sc = blk + 4;
+                    const int s = part; // crates/gguf/src/quant.rs:620-628 get_scale_min_k4
                     int scv, mv;
                     if (s < 4) {
                         scv = sc[s] & 63;
@@ -244,104 +254,118 @@ __global__ __launch_bounds__(256, 2) void k_gemm(const uint8_t *w, int rpe, int 
                     }
                     rs[s * kGemmBM + r] = d * (float)scv;
                     rs[(8 + s) * kGemmBM + r] = -(dmin * (float)mv);
-                }
-            } else {
-                const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk + 222));
+                } else {
+                    const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk + 222));
 #pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    const int gq = 4 * part + t;
-                    rs[gq * kGemmBM + r] = d * (float)(int)(signed char)blk[192 + gq];
+                    for (int t = 0; t < 2; t++) {
+                        const int gq = 2 * part + t;
+                        rs[gq * kGemmBM + r] = d * (float)(int)(signed char)blk[192 + gq];
+                    }
                 }
             }
         }
         __syncthreads();
-        const float2 *pair = reinterpret_cast<const float2 *>(my_act + BM_Q82_SB_REF); // (d8, d8 * isum) a 32-block
+        const float2 *pair[T]; // (d8, d8 * isum) a 32-block
+#pragma unroll
+        for (int t = 0; t < T; t++) pair[t] = reinterpret_cast<const float2 *>(my_act[t] + BM_Q82_SB_REF);
         if constexpr (WT == BM_Q4K) {
             // the min terms first: accumulator l takes sub-block l's (crates/qdot/src/lib.rs:4389-4394)
 #pragma unroll
             for (int s = 0; s < 8; s++) {
-                const float my = pair[s].y;
+                const float4 mn = *reinterpret_cast<const float4 *>(&rs[(8 + s) * kGemmBM + rbase]);
 #pragma unroll
-                for (int qd = 0; qd < 4; qd++) {
-                    const float4 mn = *reinterpret_cast<const float4 *>(&rs[(8 + s) * kGemmBM + rbase + 8 * qd]);
-                    acc[4 * qd + 0][s] = fmaf(my, mn.x, acc[4 * qd + 0][s]);
-                    acc[4 * qd + 1][s] = fmaf(my, mn.y, acc[4 * qd + 1][s]);
-                    acc[4 * qd + 2][s] = fmaf(my, mn.z, acc[4 * qd + 2][s]);
-                    acc[4 * qd + 3][s] = fmaf(my, mn.w, acc[4 * qd + 3][s]);
+                for (int t = 0; t < T; t++) {
+                    const float my = pair[t][s].y;
+                    acc[t][0][s] = fmaf(my, mn.x, acc[t][0][s]);
+                    acc[t][1][s] = fmaf(my, mn.y, acc[t][1][s]);
+                    acc[t][2][s] = fmaf(my, mn.z, acc[t][2][s]);
+                    acc[t][3][s] = fmaf(my, mn.w, acc[t][3][s]);
                 }
             }
 #pragma unroll
             for (int p = 0; p < 4; p++) { // code bytes 32p ..: low nibbles sub-block 2p, high nibbles 2p + 1
-                uint2 wq[2];
-#pragma unroll
-                for (int h = 0; h < 2; h++) wq[h] = *reinterpret_cast<const uint2 *>(my_wt + 16 + 32 * p + 16 * h + 8 * kh);
+                const uint2 wq = *reinterpret_cast<const uint2 *>(my_wt + 16 + 32 * p + 8 * kg);
 #pragma unroll
                 for (int en = 0; en < 2; en++) {
                     const int s = 2 * p + en;
-                    const float d8 = pair[s].x;
-                    float f[16];
+                    const u32 ax = (wq.x >> (4 * en)) & 0x0f0f0f0fu, ay = (wq.y >> (4 * en)) & 0x0f0f0f0fu;
+                    const float4 sv = *reinterpret_cast<const float4 *>(&rs[s * kGemmBM + rbase]);
+                    float f[T][4];
+                    long b[T];
 #pragma unroll
-                    for (int qd = 0; qd < 4; qd++) {
-                        const float4 sv = *reinterpret_cast<const float4 *>(&rs[s * kGemmBM + rbase + 8 * qd]);
-                        f[4 * qd + 0] = sv.x * d8;
-                        f[4 * qd + 1] = sv.y * d8;
-                        f[4 * qd + 2] = sv.z * d8;
-                        f[4 * qd + 3] = sv.w * d8;
+                    for (int t = 0; t < T; t++) {
+                        const float d8 = pair[t][s].x;
+                        f[t][0] = sv.x * d8;
+                        f[t][1] = sv.y * d8;
+                        f[t][2] = sv.z * d8;
+                        f[t][3] = sv.w * d8;
+                        const uint2 bq = *reinterpret_cast<const uint2 *>(my_act[t] + (s >> 2) * BM_Q82X4_STRIDE + 16 +
+                                                                          32 * (s & 3) + 8 * kg);
+                        b[t] = (long)(((unsigned long long)bq.y << 32) | bq.x);
                     }
 #pragma unroll
                     for (int h = 0; h < 2; h++) {
-                        const u32 ax = (wq[h].x >> (4 * en)) & 0x0f0f0f0fu, ay = (wq[h].y >> (4 * en)) & 0x0f0f0f0fu;
-                        const uint2 bq = *reinterpret_cast<const uint2 *>(my_act + (s >> 2) * BM_Q82X4_STRIDE + 16 +
-                                                                          32 * (s & 3) + 16 * h + 8 * kh);
-                        const long a = (long)(((unsigned long long)ay << 32) | ax);
-                        const long b = (long)(((unsigned long long)bq.y << 32) | bq.x);
-                        v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                        const v16i sum = __builtin_amdgcn_mfma_i32_32x32x16_i8(a, b, z, 0, 0, 0);
+                        const long a = (long)(((unsigned long long)(ay & keep[h]) << 32) | (ax & keep[h]));
                         const int l = 4 * h + (s & 3);
 #pragma unroll
-                        for (int v = 0; v < 16; v++) acc[v][l] = fmaf(f[v], (float)sum[v], acc[v][l]);
+                        for (int t = 0; t < T; t++) {
+                            const v4i z = {0, 0, 0, 0};
+                            const v4i sum = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b[t], z, 0, 0, 0);
+#pragma unroll
+                            for (int v = 0; v < 4; v++) acc[t][v][l] = fmaf(f[t][v], (float)sum[v], acc[t][v][l]);
+                        }
                     }
                 }
             }
         } else {
 #pragma unroll
-            for (int gq = 0; gq < 16; gq++) { // 16-value group gq: 32-block gq / 2, half gq % 2
-                const int c2 = gq >> 3, a4 = (gq & 7) >> 1, hh = gq & 1, bk = gq >> 1;
-                const int l0 = 16 * hh + 8 * kh;
-                const uint2 ql = *reinterpret_cast<const uint2 *>(my_wt + 64 * c2 + 32 * (a4 & 1) + l0);
-                const uint2 qh = *reinterpret_cast<const uint2 *>(my_wt + 128 + 32 * c2 + l0);
+            for (int bk = 0; bk < 8; bk++) { // 32-block bk of the super-block: quarter bk % 4 of half bk / 4
+                const int c2 = bk >> 2, a4 = bk & 3;
+                const uint2 ql = *reinterpret_cast<const uint2 *>(my_wt + 64 * c2 + 32 * (a4 & 1) + 8 * kg);
+                const uint2 qh = *reinterpret_cast<const uint2 *>(my_wt + 128 + 32 * c2 + 8 * kg);
                 const int ns = 4 * (a4 >> 1), hs = 2 * a4;
                 const u32 ax = q6_minus_32(((ql.x >> ns) & 0x0f0f0f0fu) | (((qh.x >> hs) & 0x03030303u) << 4));
                 const u32 ay = q6_minus_32(((ql.y >> ns) & 0x0f0f0f0fu) | (((qh.y >> hs) & 0x03030303u) << 4));
-                const uint2 bq = *reinterpret_cast<const uint2 *>(my_act + (bk >> 2) * BM_Q82X4_STRIDE + 16 + 32 * (bk & 3) +
-                                                                  16 * hh + 8 * kh);
-                const float d8 = pair[bk].x;
-                const long a = (long)(((unsigned long long)ay << 32) | ax);
-                const long b = (long)(((unsigned long long)bq.y << 32) | bq.x);
-                v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                const v16i sum = __builtin_amdgcn_mfma_i32_32x32x16_i8(a, b, z, 0, 0, 0);
-                const int l = 4 * hh + (bk & 3); // crates/qdot/src/lib.rs:4794-4809: lane l < 4 scale 2l, lane 4 + l scale 2l + 1
+                long b[T];
+                float d8[T];
 #pragma unroll
-                for (int qd = 0; qd < 4; qd++) {
-                    const float4 sv = *reinterpret_cast<const float4 *>(&rs[gq * kGemmBM + rbase + 8 * qd]);
-                    acc[4 * qd + 0][l] = fmaf(sv.x * d8, (float)sum[4 * qd + 0], acc[4 * qd + 0][l]);
-                    acc[4 * qd + 1][l] = fmaf(sv.y * d8, (float)sum[4 * qd + 1], acc[4 * qd + 1][l]);
-                    acc[4 * qd + 2][l] = fmaf(sv.z * d8, (float)sum[4 * qd + 2], acc[4 * qd + 2][l]);
-                    acc[4 * qd + 3][l] = fmaf(sv.w * d8, (float)sum[4 * qd + 3], acc[4 * qd + 3][l]);
+                for (int t = 0; t < T; t++) {
+                    const uint2 bq = *reinterpret_cast<const uint2 *>(my_act[t] + (bk >> 2) * BM_Q82X4_STRIDE + 16 + 32 * (bk & 3) +
+                                                                      8 * kg);
+                    b[t] = (long)(((unsigned long long)bq.y << 32) | bq.x);
+                    d8[t] = pair[t][bk].x;
+                }
+#pragma unroll
+                for (int hh = 0; hh < 2; hh++) { // 16-value group 2 bk + hh
+                    const long a = (long)(((unsigned long long)(ay & keep[hh]) << 32) | (ax & keep[hh]));
+                    const float4 sv = *reinterpret_cast<const float4 *>(&rs[(2 * bk + hh) * kGemmBM + rbase]);
+                    const int l = 4 * hh + (bk & 3); // crates/qdot/src/lib.rs:4794-4809
+#pragma unroll
+                    for (int t = 0; t < T; t++) {
+                        const v4i z = {0, 0, 0, 0};
+                        const v4i sum = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b[t], z, 0, 0, 0);
+                        acc[t][0][l] = fmaf(sv.x * d8[t], (float)sum[0], acc[t][0][l]);
+                        acc[t][1][l] = fmaf(sv.y * d8[t], (float)sum[1], acc[t][1][l]);
+                        acc[t][2][l] = fmaf(sv.z * d8[t], (float)sum[2], acc[t][2][l]);
+                        acc[t][3][l] = fmaf(sv.w * d8[t], (float)sum[3], acc[t][3][l]);
+                    }
                 }
             }
         }
     }
     // the closing sum of the eight lanes (crates/qdot/src/lib.rs:4128 hsum_float_8's order) and the store
-    const int n = 32 * wc + l32;
-    if (n < len) {
-        const size_t out = (size_t)tab->slot[n] * rpe + row0;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int r = rbase + 8 * (v >> 2) + (v & 3);
-            const float t0 = acc[v][0] + acc[v][4], t1 = acc[v][1] + acc[v][5];
-            const float t2 = acc[v][2] + acc[v][6], t3 = acc[v][3] + acc[v][7];
-            if (row0 + r < rpe) y[out + r] = (t0 + t2) + (t1 + t3);
+    for (int t = 0; t < T; t++) {
+        const int n = 16 * T * ch + 16 * t + l16;
+        if (n < len) {
+            const size_t out = (size_t)tab->slot[n] * rpe + row0;
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int r = rbase + v;
+                const float t0 = acc[t][v][0] + acc[t][v][4], t1 = acc[t][v][1] + acc[t][v][5];
+                const float t2 = acc[t][v][2] + acc[t][v][6], t3 = acc[t][v][3] + acc[t][v][7];
+                if (row0 + r < rpe) y[out + r] = (t0 + t2) + (t1 + t3);
+            }
         }
     }
 }
@@ -354,19 +378,20 @@ hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int
     const int nb = k / 256;
     const u32 max_tiles = (u32)gemm_max_tiles(n_slots, n_experts) + 1; // one more: the block that fills refused slots
     const unsigned grid = max_tiles * (unsigned)((rows_per_expert + kGemmBM - 1) / kGemmBM);
+    // slot groups of 16 a wave (T): 1 -> 1024 threads a workgroup, 2 -> 512; the faster of the two for each type
     if (wtype == BM_Q4K) {
-        auto kern = k_gemm<BM_Q4K>;
+        auto kern = k_gemm<BM_Q4K, 1>;
         const size_t lds = gemm_lds_bytes<BM_Q4K>();
         hipError_t e = allow_lds(kern, lds);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(1024), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
                            n_tiles, max_tiles, (u32)slot_div, (u32)n_slots, y);
     } else if (wtype == BM_Q6K) {
-        auto kern = k_gemm<BM_Q6K>;
+        auto kern = k_gemm<BM_Q6K, 2>;
         const size_t lds = gemm_lds_bytes<BM_Q6K>();
         hipError_t e = allow_lds(kern, lds);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
                            n_tiles, max_tiles, (u32)slot_div, (u32)n_slots, y);
     } else {
         return hipErrorInvalidValue;

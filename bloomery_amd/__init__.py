@@ -21,6 +21,7 @@ FAULT_NONE = 0xFFFFFFFF
 LAYER_NONE = 0xFFFF
 SITE_QUANT_COLUMN, SITE_EXPERT_ID, SITE_STALLED = 1, 7, 31
 PLAN_ONE_LAUNCH, PLAN_TWO_LAUNCHES = 1, 2
+GEMM_EXACT, GEMM_FAST = 0, 1
 HOST_SLOT = 0xFFFFFFFF
 
 OK, ESHAPE, EDRIVER, ETYPE, EARG, EFAULT = 0, -1, -2, -3, -4, -5
@@ -76,6 +77,7 @@ SYMBOLS = {
     "bm_route_read": (_i, [_vp, _vp, _vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
     "bm_gemm": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp]),
     "bm_swiglu_quant": (_i, [_vp, _vp, _vp, _i, _vp]),
+    "bm_set_gemm_mode": (_i, [_vp, _i]),
     "bm_block_sums": (_i, [_vp, _vp, _i64, _vp, _i, _vp]),
     "bm_capture_begin": (_i, [_vp]),
     "bm_capture_end": (_i, [_vp, C.POINTER(_vp)]),
@@ -403,6 +405,9 @@ class Gpu:
     def enqueue_gemm(self, w, rows_per_expert, act, route, top_k, y):
         """top_k > 0: every slot of a token reads the token's column; 0: a column a slot."""
         self._check(self.lib.bm_gemm(self.ctx, w.handle, rows_per_expert, act.handle, route.handle, top_k, _ptr(y)))
+
+    def set_gemm_mode(self, mode):
+        self._check(self.lib.bm_set_gemm_mode(self.ctx, mode))
 
     def enqueue_swiglu_quant(self, g, u, n_cols, act):
         self._check(self.lib.bm_swiglu_quant(self.ctx, _ptr(g), _ptr(u), n_cols, act.handle))

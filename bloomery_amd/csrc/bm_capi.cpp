@@ -20,6 +20,7 @@ struct bm_ctx {
     uint32_t layer = BM_LAYER_NONE;
     uint32_t *counters = nullptr; // bm_moe_decode's producer/consumer counts, zero between launches
     int decode_plan = BM_PLAN_TWO_LAUNCHES;
+    int gemm_mode = BM_GEMM_EXACT;
     uint32_t spin_limit = 1u << 18; // a poll is a round trip to memory: some tenths of a second of waiting
     std::string err;
 };
@@ -718,7 +719,15 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
     if (act->m_cap < n_slots / slot_div)
         return fail(ctx, BM_ESHAPE, "%s: %d slots read %d activation columns, act holds %d", what, n_slots, n_slots / slot_div, act->m_cap);
     return driver(ctx, what, bmk::gemm(launch_of(ctx), w->wtype, w->dev, route->n_experts, rows_per_expert, w->k, act->dev, route->cols,
-                                       route->tiles, route->n_tiles, n_slots, slot_div, y_dev));
+                                       route->tiles, route->n_tiles, n_slots, slot_div, y_dev, ctx->gemm_mode == BM_GEMM_EXACT));
+}
+
+int bm_set_gemm_mode(bm_ctx *ctx, int mode) {
+    if (!ctx) return fail(nullptr, BM_EARG, "bm_set_gemm_mode: ctx is NULL");
+    if (mode != BM_GEMM_EXACT && mode != BM_GEMM_FAST)
+        return fail(ctx, BM_EARG, "bm_set_gemm_mode: mode %d is neither BM_GEMM_EXACT nor BM_GEMM_FAST", mode);
+    ctx->gemm_mode = mode;
+    return BM_OK;
 }
 
 int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, bm_act *act) {

@@ -370,14 +370,238 @@ __global__ __launch_bounds__(1024 / T) void k_gemm(const uint8_t *w, int rpe, in
     }
 }
 
+// The same product with one accumulator a value: each 32-value block's integer sum (Q4_K: two chained matrix
+// instructions) or 16-value group's (Q6_K) is scaled and added in increasing k, a block's min term just before it.
+// The integers are the exact ones; the f32 sum is not in the CPU path's eight-lane order, so a value differs from
+// the exact kernel's by rounding only (a few 1e-7 of the row's magnitude; the contract's tolerance is 1e-4). A third
+// fewer vector operations and an eighth of the accumulator registers: 32 x 32 tiles, four waves, several
+// workgroups a CU.
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+template <int WT>
+__global__ __launch_bounds__(256) void k_gemm_fast(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
+                                                   const u32 *tiles, const u32 *n_tiles, u32 max_tiles, u32 slot_div,
+                                                   u32 n_slots, float *y) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
+    uint8_t *acts = lds + sizeof(GemmLds);
+    uint8_t *wts = acts + (size_t)kGemmBN * kActStride;
+    float *rs = reinterpret_cast<float *>(wts + (size_t)kGemmBM * wt_stride<WT>()); // [16][64]
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const u32 g = blockIdx.x % max_tiles;
+    const int row0 = (int)(blockIdx.x / max_tiles) * kGemmBM;
+    const u32 count = n_tiles[0];
+    if (g > count) return;
+    if (g == count) {
+        const u32 refused = n_tiles[1];
+        for (u32 i = tid; i < refused * kGemmBM; i += blockDim.x) {
+            const u32 s = cols[n_slots - refused + i / kGemmBM];
+            const int r = row0 + (int)(i % kGemmBM);
+            if (r < rpe) y[(size_t)s * rpe + r] = bm_bits_f32(0x7fc00000u);
+        }
+        return;
+    }
+    const u32 e = tiles[2 * g], word = tiles[2 * g + 1];
+    const int start = (int)(word & 0xffffu), len = (int)(word >> 16);
+    if (tid < kGemmBN) {
+        const u32 s = cols[start + (tid < len ? tid : 0)];
+        tab->slot[tid] = s;
+        tab->col[tid] = s / slot_div;
+    }
+    __syncthreads();
+    constexpr int kBlock = WT == BM_Q4K ? BM_Q4K_BLOCK : BM_Q6K_BLOCK;
+    constexpr int kWc = wt_chunks<WT>();
+    const size_t row_bytes = (size_t)nb * kBlock;
+    const int col_bytes = nb * BM_Q82_SB_EXT;
+    constexpr int kAc = kActSb / 16; // 22
+    constexpr int kActLoads = (kGemmBN * kAc + 255) / 256, kWtLoads = (kGemmBM * kWc + 255) / 256;
+    uint4 ra[kActLoads], rw[kWtLoads];
+    auto fetch = [&](int i) {
+#pragma unroll
+        for (int t = 0; t < kActLoads; t++) {
+            int c = t * 256 + tid;
+            c = c < kGemmBN * kAc ? c : kGemmBN * kAc - 1;
+            const int n = c / kAc, k = c % kAc;
+            const uint8_t *colp = act + (size_t)tab->col[n] * col_bytes;
+            const uint8_t *src = k < 18 ? colp + (size_t)i * BM_Q82_SB_REF + 16 * k
+                                        : colp + (size_t)nb * BM_Q82_SB_REF + (size_t)i * 64 + 16 * (k - 18);
+            ra[t] = *reinterpret_cast<const uint4 *>(src);
+        }
+#pragma unroll
+        for (int t = 0; t < kWtLoads; t++) {
+            int c = t * 256 + tid;
+            c = c < kGemmBM * kWc ? c : kGemmBM * kWc - 1;
+            int r = row0 + c / kWc;
+            const int k = c % kWc;
+            r = r < rpe ? r : rpe - 1;
+            const uint8_t *blk = w + ((size_t)e * rpe + r) * row_bytes + (size_t)i * kBlock;
+            rw[t] = bm_ld16u(blk + ((WT == BM_Q6K && k == 13) ? 194 : 16 * k));
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int t = 0; t < kActLoads; t++) {
+            const int c = t * 256 + tid;
+            if (c < kGemmBN * kAc) {
+                uint8_t *dst = acts + (c / kAc) * kActStride + 16 * (c % kAc);
+                *reinterpret_cast<uint2 *>(dst) = make_uint2(ra[t].x, ra[t].y);
+                *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(ra[t].z, ra[t].w);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < kWtLoads; t++) {
+            const int c = t * 256 + tid;
+            if (c < kGemmBM * kWc) {
+                uint8_t *dst = wts + (c / kWc) * wt_stride<WT>() + 16 * (c % kWc);
+                *reinterpret_cast<uint2 *>(dst) = make_uint2(rw[t].x, rw[t].y);
+                *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(rw[t].z, rw[t].w);
+            }
+        }
+    };
+    // v_mfma_i32_32x32x16_i8: operand row / slot lane % 32, values 8 * (lane / 32) .. + 8 of a 16-value group; result v
+    // is row 8 * (v / 4) + 4 * (lane / 32) + v % 4 of slot lane % 32
+    const int wr = wv & 1, wc = wv >> 1, l32 = lane & 31, kh = lane >> 5;
+    const uint8_t *my_act = acts + (32 * wc + l32) * kActStride;
+    const uint8_t *my_wt = wts + (32 * wr + l32) * wt_stride<WT>();
+    const int rbase = 32 * wr + 4 * kh;
+    float acc[16];
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+
+    fetch(0);
+    for (int i = 0; i < nb; i++) {
+        __syncthreads();
+        stash();
+        __syncthreads();
+        if (i + 1 < nb) fetch(i + 1);
+        {
+            const int r = tid >> 2, part = tid & 3;
+            const uint8_t *blk = wts + r * wt_stride<WT>();
+            if constexpr (WT == BM_Q4K) {
+                const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk));
+                const float dmin = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk + 2));
+                const uint8_t *sc = blk + 4;
+#pragma unroll
+                for (int t = 0; t < 2; t++) { // crates/gguf/src/quant.rs:620-628 get_scale_min_k4
+                    const int s = 2 * part + t;
+                    int scv, mv;
+                    if (s < 4) {
+                        scv = sc[s] & 63;
+                        mv = sc[s + 4] & 63;
+                    } else {
+                        scv = (sc[s + 4] & 15) | ((sc[s - 4] >> 6) << 4);
+                        mv = (sc[s + 4] >> 4) | ((sc[s] >> 6) << 4);
+                    }
+                    rs[s * kGemmBM + r] = d * (float)scv;
+                    rs[(8 + s) * kGemmBM + r] = -(dmin * (float)mv);
+                }
+            } else {
+                const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk + 222));
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const int gq = 4 * part + t;
+                    rs[gq * kGemmBM + r] = d * (float)(int)(signed char)blk[192 + gq];
+                }
+            }
+        }
+        __syncthreads();
+        const float2 *pair = reinterpret_cast<const float2 *>(my_act + BM_Q82_SB_REF);
+        if constexpr (WT == BM_Q4K) {
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                uint2 wq[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) wq[h] = *reinterpret_cast<const uint2 *>(my_wt + 16 + 32 * p + 16 * h + 8 * kh);
+#pragma unroll
+                for (int en = 0; en < 2; en++) {
+                    const int s = 2 * p + en;
+                    v16i sum = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const u32 ax = (wq[h].x >> (4 * en)) & 0x0f0f0f0fu, ay = (wq[h].y >> (4 * en)) & 0x0f0f0f0fu;
+                        const uint2 bq = *reinterpret_cast<const uint2 *>(my_act + (s >> 2) * BM_Q82X4_STRIDE + 16 +
+                                                                          32 * (s & 3) + 16 * h + 8 * kh);
+                        sum = __builtin_amdgcn_mfma_i32_32x32x16_i8((long)(((unsigned long long)ay << 32) | ax),
+                                                                    (long)(((unsigned long long)bq.y << 32) | bq.x), sum, 0, 0, 0);
+                    }
+                    const float d8 = pair[s].x, my = pair[s].y;
+#pragma unroll
+                    for (int qd = 0; qd < 4; qd++) {
+                        const float4 mn = *reinterpret_cast<const float4 *>(&rs[(8 + s) * kGemmBM + rbase + 8 * qd]);
+                        const float4 sv = *reinterpret_cast<const float4 *>(&rs[s * kGemmBM + rbase + 8 * qd]);
+                        acc[4 * qd + 0] = fmaf(sv.x * d8, (float)sum[4 * qd + 0], fmaf(my, mn.x, acc[4 * qd + 0]));
+                        acc[4 * qd + 1] = fmaf(sv.y * d8, (float)sum[4 * qd + 1], fmaf(my, mn.y, acc[4 * qd + 1]));
+                        acc[4 * qd + 2] = fmaf(sv.z * d8, (float)sum[4 * qd + 2], fmaf(my, mn.z, acc[4 * qd + 2]));
+                        acc[4 * qd + 3] = fmaf(sv.w * d8, (float)sum[4 * qd + 3], fmaf(my, mn.w, acc[4 * qd + 3]));
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int gq = 0; gq < 16; gq++) {
+                const int c2 = gq >> 3, a4 = (gq & 7) >> 1, hh = gq & 1, bk = gq >> 1;
+                const int l0 = 16 * hh + 8 * kh;
+                const uint2 ql = *reinterpret_cast<const uint2 *>(my_wt + 64 * c2 + 32 * (a4 & 1) + l0);
+                const uint2 qh = *reinterpret_cast<const uint2 *>(my_wt + 128 + 32 * c2 + l0);
+                const int ns = 4 * (a4 >> 1), hs = 2 * a4;
+                const u32 ax = q6_minus_32(((ql.x >> ns) & 0x0f0f0f0fu) | (((qh.x >> hs) & 0x03030303u) << 4));
+                const u32 ay = q6_minus_32(((ql.y >> ns) & 0x0f0f0f0fu) | (((qh.y >> hs) & 0x03030303u) << 4));
+                const uint2 bq = *reinterpret_cast<const uint2 *>(my_act + (bk >> 2) * BM_Q82X4_STRIDE + 16 + 32 * (bk & 3) +
+                                                                  16 * hh + 8 * kh);
+                const float d8 = pair[bk].x;
+                const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                const v16i sum = __builtin_amdgcn_mfma_i32_32x32x16_i8((long)(((unsigned long long)ay << 32) | ax),
+                                                                       (long)(((unsigned long long)bq.y << 32) | bq.x), z, 0, 0, 0);
+#pragma unroll
+                for (int qd = 0; qd < 4; qd++) {
+                    const float4 sv = *reinterpret_cast<const float4 *>(&rs[gq * kGemmBM + rbase + 8 * qd]);
+                    acc[4 * qd + 0] = fmaf(sv.x * d8, (float)sum[4 * qd + 0], acc[4 * qd + 0]);
+                    acc[4 * qd + 1] = fmaf(sv.y * d8, (float)sum[4 * qd + 1], acc[4 * qd + 1]);
+                    acc[4 * qd + 2] = fmaf(sv.z * d8, (float)sum[4 * qd + 2], acc[4 * qd + 2]);
+                    acc[4 * qd + 3] = fmaf(sv.w * d8, (float)sum[4 * qd + 3], acc[4 * qd + 3]);
+                }
+            }
+        }
+    }
+    const int n = 32 * wc + l32;
+    if (n < len) {
+        const size_t out = (size_t)tab->slot[n] * rpe + row0;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int r = rbase + 8 * (v >> 2) + (v & 3);
+            if (row0 + r < rpe) y[out + r] = acc[v];
+        }
+    }
+}
+
 bool gemm_supported(int wtype) { return wtype == BM_Q4K || wtype == BM_Q6K; }
 
 hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int rows_per_expert, int k,
                 const uint8_t *act, const uint32_t *cols, const uint32_t *tiles_dev, const uint32_t *n_tiles, int n_slots,
-                int slot_div, float *y) {
+                int slot_div, float *y, bool exact) {
     const int nb = k / 256;
     const u32 max_tiles = (u32)gemm_max_tiles(n_slots, n_experts) + 1; // one more: the block that fills refused slots
     const unsigned grid = max_tiles * (unsigned)((rows_per_expert + kGemmBM - 1) / kGemmBM);
+    if (!exact) {
+        if (wtype == BM_Q4K) {
+            auto kern = k_gemm_fast<BM_Q4K>;
+            const size_t lds = gemm_lds_bytes<BM_Q4K>();
+            hipError_t e = allow_lds(kern, lds);
+            if (e != hipSuccess) return e;
+            hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
+                               n_tiles, max_tiles, (u32)slot_div, (u32)n_slots, y);
+        } else if (wtype == BM_Q6K) {
+            auto kern = k_gemm_fast<BM_Q6K>;
+            const size_t lds = gemm_lds_bytes<BM_Q6K>();
+            hipError_t e = allow_lds(kern, lds);
+            if (e != hipSuccess) return e;
+            hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
+                               n_tiles, max_tiles, (u32)slot_div, (u32)n_slots, y);
+        } else {
+            return hipErrorInvalidValue;
+        }
+        return hipGetLastError();
+    }
     // slot groups of 16 a wave (T): 1 -> 1024 threads a workgroup, 2 -> 512; the faster of the two for each type
     if (wtype == BM_Q4K) {
         auto kern = k_gemm<BM_Q4K, 1>;

@@ -245,6 +245,14 @@ int bm_route_read(bm_ctx *ctx, const bm_route *route, uint32_t *cols_host, uint3
  * matrix cores. A refused slot gets NaN in every row. */
 int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act *act, const bm_route *route, int top_k,
             float *y_dev);
+/* How bm_gemm sums in f32 (the integer block sums are exact either way):
+ *   BM_GEMM_EXACT (default): the CPU path's eight accumulators and closing order; bit-identical to bm_gemv_sel;
+ *   BM_GEMM_FAST: one accumulator a value, blocks in increasing k; differs from the exact value by f32 rounding
+ *     only (observed below 1e-6 of the row's largest magnitude; the contract's tolerance is 1e-4), about 2.5x the
+ *     speed. No counterpart in the reference, whose grouped GEMM has one order (gemm/grouped.rs:33-58). */
+#define BM_GEMM_EXACT 0
+#define BM_GEMM_FAST 1
+int bm_set_gemm_mode(bm_ctx *ctx, int mode);
 /* GemmKernels::enqueue_swiglu_quant (crates/gpu/src/gemm/swiglu.rs:46): column c of act = the quantized
  * silu(g) * u of g_dev / u_dev[c * k .. (c + 1) * k), k = act's k, slot-major as the gate and up GEMMs write them;
  * bm_quantize's bytes of the CPU path's SwiGLU. Q8_2_X4 columns only. */

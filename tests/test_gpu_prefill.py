@@ -61,6 +61,43 @@ def run_prefill(gpu, L, x, ids, wts, top_k):
     return out
 
 
+def test_gemm_fast_mode_is_within_the_tolerance(gpu):
+    """BM_GEMM_FAST keeps the exact integers and sums them in another f32 order: every value of one GEMM is within
+    1e-4 (max-abs normalised over its row vector, the contract's tolerance) of the one-column dot, in practice far
+    inside it. (Chained through the Q8 quantizer of h a last-bit difference can flip a code, which is why the exact
+    mode is the default and the one the layer tests use.)"""
+    from common import max_abs_normalised
+    rng = np.random.default_rng(2200)
+    worst = 0.0
+    for wtype, k, rpe in ((bm.Q4_K, 2048, 768), (bm.Q6_K, 768, 2048)):
+        n_experts, n_slots = 6, 150
+        w = stack(wtype, n_experts * rpe, k, 2201)
+        ids = rng.integers(0, n_experts, n_slots).astype(np.uint32)
+        x = normal_f32(rng, (n_slots, k))
+        dw, act = gpu.weights(wtype, n_experts * rpe, k, w), gpu.act(wtype, k, n_slots)
+        xd, sel = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32)
+        table = gpu.route(n_slots, n_experts)
+        gpu.enqueue_quantize(xd, n_slots, act)
+        table.fill(sel, n_slots)
+        y = gpu.buffer(np.float32, n_slots * rpe).fill_bytes(0)
+        gpu.set_gemm_mode(bm.GEMM_FAST)
+        try:
+            gpu.enqueue_gemm(dw, rpe, act, table, 0, y)
+            got = y.download().reshape(n_slots, rpe)
+        finally:
+            gpu.set_gemm_mode(bm.GEMM_EXACT)
+        rb = ora.row_bytes(wtype, k)
+        for s in range(0, n_slots, 7):
+            e = int(ids[s])
+            want = ora.gemv(wtype, w[e * rpe * rb:(e + 1) * rpe * rb], rpe, k, ora.quantize_col(wtype, x[s]), 1)
+            err = max_abs_normalised(got[s], want)
+            worst = max(worst, err)
+            assert err <= 1e-4, f"type {wtype} slot {s}: max-abs normalised error {err}"
+        for b in (dw, act, xd, sel, table, y):
+            b.free()
+    assert worst <= 1e-5, f"fast mode drifted further than f32 rounding explains: {worst}"
+
+
 @pytest.mark.parametrize("types,hidden,ff,n_experts,m,top_k,cheap", (
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 6, 70, 3, False),      # runs past 64 slots: several tiles an expert
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 16, 48, 8, True),     # config 4's layer shape, 384 slots

@@ -719,7 +719,7 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
     if (act->m_cap < n_slots / slot_div)
         return fail(ctx, BM_ESHAPE, "%s: %d slots read %d activation columns, act holds %d", what, n_slots, n_slots / slot_div, act->m_cap);
     return driver(ctx, what, bmk::gemm(launch_of(ctx), w->wtype, w->dev, route->n_experts, rows_per_expert, w->k, act->dev, route->cols,
-                                       route->tiles, route->n_tiles, n_slots, slot_div, y_dev, ctx->gemm_mode == BM_GEMM_EXACT));
+                                       route->tiles, route->n_tiles, n_slots, slot_div, y_dev, ctx->gemm_mode));
 }
 
 int bm_set_gemm_mode(bm_ctx *ctx, int mode) {

@@ -101,10 +101,10 @@ hipError_t route(const Launch &L, const uint32_t *ids, int n_slots, int n_expert
 hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act);
 bool gemm_supported(int wtype);
 // slot_div: slots a token when every slot of a token reads the token's column, 1 when each slot reads its own.
-// exact: the CPU path's eight-accumulator f32 order (bit-identical to the row dots); else one accumulator a value.
+// mode 0: the CPU path's eight-accumulator f32 order (bit-identical to the row dots); 1: one accumulator a value.
 hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int rows_per_expert, int k,
                 const uint8_t *act, const uint32_t *cols, const uint32_t *tiles, const uint32_t *n_tiles, int n_slots,
-                int slot_div, float *y, bool exact);
+                int slot_div, float *y, int mode);
 
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out);
 

@@ -116,6 +116,12 @@ __host__ __device__ constexpr size_t gemm_lds_bytes() {
     return sizeof(GemmLds) + (size_t)kGemmBN * kActStride + (size_t)kGemmBM * wt_stride<WT>() + 16 * kGemmBM * sizeof(float);
 }
 
+// Workgroup b of a GEMM grid: tile and row slab. Workgroups go to the chip's eight dies in turn (b to die b % 8,
+// each with its own L2), so a tile's row slabs are consecutive workgroups of one die: the tile's activation columns
+// come from memory once and serve all the slabs from that L2. The grid is 8 * ceil(tiles / 8) * n_slabs workgroups.
+__device__ __forceinline__ u32 tile_of_block(u32 b, u32 n_slabs) { return ((b >> 3) / n_slabs) * 8 + (b & 7); }
+__device__ __forceinline__ u32 slab_of_block(u32 b, u32 n_slabs) { return (b >> 3) % n_slabs; }
+
 // (q6 - 32) of four codes a word, as signed bytes: q6 in 0..63.
 __device__ __forceinline__ u32 q6_minus_32(u32 q) {
     const u32 t = q ^ 0x20202020u;        // q >= 32: q - 32; q < 32: q + 32
@@ -130,7 +136,7 @@ __device__ __forceinline__ u32 q6_minus_32(u32 q) {
 // stay resident and hide each other's LDS and matrix latencies.
 template <int WT, int T>
 __global__ __launch_bounds__(1024 / T) void k_gemm(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
-                                                 const u32 *tiles, const u32 *n_tiles, u32 max_tiles, u32 slot_div,
+                                                 const u32 *tiles, const u32 *n_tiles, u32 n_slabs, u32 slot_div,
                                                  u32 n_slots, float *y) {
     extern __shared__ __align__(16) uint8_t lds[];
     GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
@@ -138,8 +144,8 @@ __global__ __launch_bounds__(1024 / T) void k_gemm(const uint8_t *w, int rpe, in
     uint8_t *wts = acts + (size_t)kGemmBN * kActStride;
     float *rs = reinterpret_cast<float *>(wts + (size_t)kGemmBM * wt_stride<WT>()); // [16][64]
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    const u32 g = blockIdx.x % max_tiles;
-    const int row0 = (int)(blockIdx.x / max_tiles) * kGemmBM;
+    const u32 g = tile_of_block(blockIdx.x, n_slabs);
+    const int row0 = (int)slab_of_block(blockIdx.x, n_slabs) * kGemmBM;
     const u32 count = n_tiles[0];
     if (g > count) return;
     if (g == count) { // the refused slots' rows: NaN (crates/gpu/src/gemm/grouped.rs:2283-2287)
@@ -265,6 +271,7 @@ __global__ __launch_bounds__(1024 / T) void k_gemm(const uint8_t *w, int rpe, in
             }
         }
         __syncthreads();
+        if (16 * T * ch >= len) continue; // none of this wave's slots is real (the barriers above are the loop's only ones)
         const float2 *pair[T]; // (d8, d8 * isum) a 32-block
 #pragma unroll
         for (int t = 0; t < T; t++) pair[t] = reinterpret_cast<const float2 *>(my_act[t] + BM_Q82_SB_REF);
@@ -380,7 +387,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 template <int WT>
 __global__ __launch_bounds__(256) void k_gemm_fast(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
-                                                   const u32 *tiles, const u32 *n_tiles, u32 max_tiles, u32 slot_div,
+                                                   const u32 *tiles, const u32 *n_tiles, u32 n_slabs, u32 slot_div,
                                                    u32 n_slots, float *y) {
     extern __shared__ __align__(16) uint8_t lds[];
     GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
@@ -388,8 +395,8 @@ __global__ __launch_bounds__(256) void k_gemm_fast(const uint8_t *w, int rpe, in
     uint8_t *wts = acts + (size_t)kGemmBN * kActStride;
     float *rs = reinterpret_cast<float *>(wts + (size_t)kGemmBM * wt_stride<WT>()); // [16][64]
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    const u32 g = blockIdx.x % max_tiles;
-    const int row0 = (int)(blockIdx.x / max_tiles) * kGemmBM;
+    const u32 g = tile_of_block(blockIdx.x, n_slabs);
+    const int row0 = (int)slab_of_block(blockIdx.x, n_slabs) * kGemmBM;
     const u32 count = n_tiles[0];
     if (g > count) return;
     if (g == count) {
@@ -505,6 +512,7 @@ __global__ __launch_bounds__(256) void k_gemm_fast(const uint8_t *w, int rpe, in
             }
         }
         __syncthreads();
+        if (32 * wc >= len) continue; // none of this wave's slots is real (the barriers above are the loop's only ones)
         const float2 *pair = reinterpret_cast<const float2 *>(my_act + BM_Q82_SB_REF);
         if constexpr (WT == BM_Q4K) {
 #pragma unroll
@@ -578,49 +586,27 @@ bool gemm_supported(int wtype) { return wtype == BM_Q4K || wtype == BM_Q6K; }
 
 hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int rows_per_expert, int k,
                 const uint8_t *act, const uint32_t *cols, const uint32_t *tiles_dev, const uint32_t *n_tiles, int n_slots,
-                int slot_div, float *y, bool exact) {
+                int slot_div, float *y, int mode) {
     const int nb = k / 256;
     const u32 max_tiles = (u32)gemm_max_tiles(n_slots, n_experts) + 1; // one more: the block that fills refused slots
-    const unsigned grid = max_tiles * (unsigned)((rows_per_expert + kGemmBM - 1) / kGemmBM);
-    if (!exact) {
-        if (wtype == BM_Q4K) {
-            auto kern = k_gemm_fast<BM_Q4K>;
-            const size_t lds = gemm_lds_bytes<BM_Q4K>();
-            hipError_t e = allow_lds(kern, lds);
-            if (e != hipSuccess) return e;
-            hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
-                               n_tiles, max_tiles, (u32)slot_div, (u32)n_slots, y);
-        } else if (wtype == BM_Q6K) {
-            auto kern = k_gemm_fast<BM_Q6K>;
-            const size_t lds = gemm_lds_bytes<BM_Q6K>();
-            hipError_t e = allow_lds(kern, lds);
-            if (e != hipSuccess) return e;
-            hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
-                               n_tiles, max_tiles, (u32)slot_div, (u32)n_slots, y);
-        } else {
-            return hipErrorInvalidValue;
-        }
+    const u32 n_slabs = (u32)((rows_per_expert + kGemmBM - 1) / kGemmBM);
+    const unsigned grid = ((max_tiles + 7) / 8) * 8 * n_slabs;
+    auto launch = [&](auto kern, unsigned threads, size_t lds) {
+        hipError_t e = allow_lds(kern, lds);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev, n_tiles,
+                           n_slabs, (u32)slot_div, (u32)n_slots, y);
         return hipGetLastError();
-    }
-    // slot groups of 16 a wave (T): 1 -> 1024 threads a workgroup, 2 -> 512; the faster of the two for each type
-    if (wtype == BM_Q4K) {
-        auto kern = k_gemm<BM_Q4K, 1>;
-        const size_t lds = gemm_lds_bytes<BM_Q4K>();
-        hipError_t e = allow_lds(kern, lds);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(1024), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
-                           n_tiles, max_tiles, (u32)slot_div, (u32)n_slots, y);
-    } else if (wtype == BM_Q6K) {
-        auto kern = k_gemm<BM_Q6K, 2>;
-        const size_t lds = gemm_lds_bytes<BM_Q6K>();
-        hipError_t e = allow_lds(kern, lds);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
-                           n_tiles, max_tiles, (u32)slot_div, (u32)n_slots, y);
-    } else {
+    };
+    if (mode == 1) {
+        if (wtype == BM_Q4K) return launch(k_gemm_fast<BM_Q4K>, 256, gemm_lds_bytes<BM_Q4K>());
+        if (wtype == BM_Q6K) return launch(k_gemm_fast<BM_Q6K>, 256, gemm_lds_bytes<BM_Q6K>());
         return hipErrorInvalidValue;
     }
-    return hipGetLastError();
+    // slot groups of 16 a wave (T): 1 -> 1024 threads a workgroup, 2 -> 512; the faster of the two for each type
+    if (wtype == BM_Q4K) return launch(k_gemm<BM_Q4K, 1>, 1024, gemm_lds_bytes<BM_Q4K>());
+    if (wtype == BM_Q6K) return launch(k_gemm<BM_Q6K, 2>, 512, gemm_lds_bytes<BM_Q6K>());
+    return hipErrorInvalidValue;
 }
 
 } // namespace bmk

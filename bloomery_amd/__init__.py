@@ -19,7 +19,7 @@ LIB_PATH = os.path.join(HERE, "libbm_moe_hip.so")
 Q4_K, Q6_K, IQ2_XXS = 12, 14, 16
 FAULT_NONE = 0xFFFFFFFF
 LAYER_NONE = 0xFFFF
-SITE_QUANT_COLUMN, SITE_EXPERT_ID, SITE_STALLED = 1, 7, 31
+SITE_QUANT_COLUMN, SITE_ROUTER, SITE_EXPERT_ID, SITE_STALLED = 1, 5, 7, 31
 PLAN_ONE_LAUNCH, PLAN_TWO_LAUNCHES = 1, 2
 GEMM_EXACT, GEMM_FAST = 0, 1
 HOST_SLOT = 0xFFFFFFFF
@@ -77,6 +77,7 @@ SYMBOLS = {
     "bm_route_read": (_i, [_vp, _vp, _vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
     "bm_gemm": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp]),
     "bm_swiglu_quant": (_i, [_vp, _vp, _vp, _i, _vp]),
+    "bm_route_softmax": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "bm_set_gemm_mode": (_i, [_vp, _i]),
     "bm_block_sums": (_i, [_vp, _vp, _i64, _vp, _i, _vp]),
     "bm_capture_begin": (_i, [_vp]),
@@ -411,6 +412,11 @@ class Gpu:
 
     def enqueue_swiglu_quant(self, g, u, n_cols, act):
         self._check(self.lib.bm_swiglu_quant(self.ctx, _ptr(g), _ptr(u), n_cols, act.handle))
+
+    def enqueue_route_softmax(self, logits, n_tokens, n_experts, top_k, renorm, probs, ids, weights):
+        """RouterKernels::enqueue_route (crates/gpu/src/route_softmax.rs:1643): softmax, top-k, renormalised weights."""
+        self._check(self.lib.bm_route_softmax(self.ctx, _ptr(logits), n_tokens, n_experts, top_k, int(bool(renorm)),
+                                              _ptr(probs) if probs is not None else None, _ptr(ids), _ptr(weights)))
 
     def enqueue_block_sums(self, w, row, act, col, out):
         self._check(self.lib.bm_block_sums(self.ctx, w.handle, row, act.handle, col, _ptr(out)))

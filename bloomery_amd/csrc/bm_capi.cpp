@@ -740,6 +740,20 @@ int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_c
     return driver(ctx, what, bmk::swiglu_quant(launch_of(ctx), g_dev, u_dev, n_cols, act->k, act->dev));
 }
 
+int bm_route_softmax(bm_ctx *ctx, const float *logits_dev, int n_tokens, int n_experts, int top_k, int renorm, float *probs_dev,
+                     uint32_t *ids_dev, float *weights_dev) {
+    const char *what = "bm_route_softmax";
+    if (!ctx || !logits_dev || !ids_dev || !weights_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (n_tokens < 1) return fail(ctx, BM_ESHAPE, "%s: n_tokens = %d must be positive", what, n_tokens);
+    if (n_experts < 1 || n_experts > bmk::kRouteMaxExperts)
+        return fail(ctx, BM_ESHAPE, "%s: n_experts = %d, the router takes 1 to %d", what, n_experts, bmk::kRouteMaxExperts);
+    if (top_k < 1 || top_k > bmk::kRouteMaxPicks || top_k > n_experts)
+        return fail(ctx, BM_ESHAPE, "%s: top_k = %d of %d experts, the router picks 1 to %d", what, top_k, n_experts,
+                    bmk::kRouteMaxPicks);
+    return driver(ctx, what, bmk::route_softmax(launch_of(ctx), logits_dev, n_tokens, n_experts, top_k, renorm != 0, probs_dev,
+                                                ids_dev, weights_dev));
+}
+
 int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *act, int col, int32_t *out_dev) {
     const char *what = "bm_block_sums";
     if (!ctx || !w || !act || !out_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);

@@ -106,6 +106,13 @@ hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int
                 const uint8_t *act, const uint32_t *cols, const uint32_t *tiles, const uint32_t *n_tiles, int n_slots,
                 int slot_div, float *y, int mode);
 
+// ---------------------------------------------------------------------------------------- router (bm_router.hip)
+
+constexpr int kRouteMaxExperts = 1024, kRouteMaxPicks = 32;
+// probs may be NULL. logits[n_tok * n_exp], ids / weights[n_tok * used].
+hipError_t route_softmax(const Launch &L, const float *logits, int n_tok, int n_exp, int used, int renorm, float *probs,
+                         uint32_t *ids, float *weights);
+
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out);
 
 } // namespace bmk

@@ -44,6 +44,7 @@ extern "C" {
 #define BM_LAYER_NONE 0xFFFFu
 #define BM_FAULT_WORDS (1 + 0xFFFF + 1)
 #define BM_SITE_QUANT_COLUMN 1 /* a quantizer met a value that is not finite: NaN scale, zero codes */
+#define BM_SITE_ROUTER 5       /* a token's logits hold a value that is not finite */
 #define BM_SITE_EXPERT_ID 7    /* an expert id at or past the stack */
 #define BM_SITE_STALLED 31     /* ours: a bm_moe_decode consumer gave up waiting for its producers */
 
@@ -248,7 +249,7 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
 /* How bm_gemm sums in f32 (the integer block sums are exact either way):
  *   BM_GEMM_EXACT (default): the CPU path's eight accumulators and closing order; bit-identical to bm_gemv_sel;
  *   BM_GEMM_FAST: one accumulator a value, blocks in increasing k; differs from the exact value by f32 rounding
- *     only (observed below 1e-6 of the row's largest magnitude; the contract's tolerance is 1e-4), about 2.5x the
+ *     only (observed below 1e-6 of the row's largest magnitude; the contract's tolerance is 1e-4), about 1.4x the
  *     speed. No counterpart in the reference, whose grouped GEMM has one order (gemm/grouped.rs:33-58). */
 #define BM_GEMM_EXACT 0
 #define BM_GEMM_FAST 1
@@ -257,6 +258,20 @@ int bm_set_gemm_mode(bm_ctx *ctx, int mode);
  * silu(g) * u of g_dev / u_dev[c * k .. (c + 1) * k), k = act's k, slot-major as the gate and up GEMMs write them;
  * bm_quantize's bytes of the CPU path's SwiGLU. Q8_2_X4 columns only. */
 int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, bm_act *act);
+
+/* ------------------------------------------------------------------------------------------------- router */
+
+/* The step before the experts: RouterKernels::enqueue_route, kernel softmax_router_route
+ * (crates/gpu/src/route_softmax.rs:1643, :1203), in the CPU path's numbers (crates/model/src/moe.rs:246-279).
+ * logits_dev: n_tokens rows of n_experts f32 (1 .. 1024 experts). Per token: the softmax probabilities (exp of
+ * logit - max in f32, their sum in f64, one f32 divide) into probs_dev[t * n_experts ..] (probs_dev may be NULL),
+ * the top_k (1 .. 32) experts by descending probability, ties toward the smaller id, into ids_dev[t * top_k ..],
+ * and their weights into weights_dev[t * top_k ..]: with renorm != 0 each probability over the f32 rounding of the
+ * chosen probabilities' f64 sum in slot order (norm_topk_prob), else the probability itself. The outputs are the
+ * sel / weights arguments of the entries above. A token with a logit that is not finite raises BM_SITE_ROUTER, gets
+ * NaN probabilities and weights, and keeps its ids as they stand. */
+int bm_route_softmax(bm_ctx *ctx, const float *logits_dev, int n_tokens, int n_experts, int top_k, int renorm,
+                     float *probs_dev, uint32_t *ids_dev, float *weights_dev);
 
 /* ------------------------------------------------------------------------------------------- verification */
 

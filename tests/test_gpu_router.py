@@ -1,0 +1,141 @@
+"""GPU parity tests of the softmax router (bm_route_softmax) through the C ABI, against the CPU oracle's restatement
+of the CPU path's router (crates/model/src/moe.rs:246-279) on the same seeded logits: ids exactly; weights and
+probabilities within two units in the last place and bit for bit in all but a few per thousand (the CPU path's exp is
+the host library's expf, the kernel's the f64 exp rounded to f32: each the correctly rounded value in all but rare
+cases, and not the same rare cases; the stated tolerance of the path is 1e-4). Clauses follow the reference's router tests
+(crates/gpu/src/route_softmax.rs:2035-2110): the rule's picks, ties toward the smaller id, a token with a logit that
+is not finite."""
+import numpy as np
+import pytest
+
+import bloomery_amd as bm
+import ora
+from common import normal_f32
+from test_gpu_decode import Layer, assert_f32, gpu  # noqa: F401  (gpu is the module fixture)
+
+pytestmark = pytest.mark.gpu
+
+
+def assert_ulp(got, want, what, ulps=2, odd_share=0.005):
+    got, want = np.asarray(got, np.float32).ravel(), np.asarray(want, np.float32).ravel()
+    assert np.isfinite(got).all(), what
+    d = np.abs(got.view(np.int32).astype(np.int64) - want.view(np.int32).astype(np.int64))  # positive floats: ordered bits
+    assert d.max() <= ulps, f"{what}: {int(d.max())} units in the last place apart"
+    assert np.count_nonzero(d) <= max(1, int(odd_share * d.size)), f"{what}: {np.count_nonzero(d)} of {d.size} differ in bits"
+
+
+def run_router(gpu, logits, top_k, renorm=True, want_probs=True):
+    m, n_experts = logits.shape
+    ld = gpu.upload(logits, np.float32)
+    probs = gpu.buffer(np.float32, m * n_experts).fill_bytes(0xFF) if want_probs else None
+    ids = gpu.buffer(np.uint32, m * top_k).fill_bytes(0xEE)
+    wts = gpu.buffer(np.float32, m * top_k).fill_bytes(0xFF)
+    gpu.enqueue_route_softmax(ld, m, n_experts, top_k, renorm, probs, ids, wts)
+    out = (ids.download().reshape(m, top_k), wts.download().reshape(m, top_k),
+           probs.download().reshape(m, n_experts) if want_probs else None)
+    for b in (ld, probs, ids, wts):
+        if b is not None:
+            b.free()
+    return out
+
+
+def oracle_probs(logits):
+    """The CPU path's softmax row: exp(l - max) in f32 (the host library's expf, as the oracle's C uses), the sum in
+    f64 in expert order, one f32 divide."""
+    one = ora.route_softmax_topk  # the top-1 weight without renormalising is the largest probability: pins the divide
+    e = np.empty_like(logits)
+    for t, row in enumerate(logits):
+        # every probability through the oracle: route with top_k = n_experts, no renorm, then scatter by id
+        ids, w = one(row, row.size, renorm=False)
+        e[t, ids] = w
+    return e
+
+
+@pytest.mark.parametrize("n_experts,top_k,m,seed,renorm", ((128, 8, 512, 1, True), (256, 8, 64, 2, True), (100, 4, 33, 3, True),
+                                                           (128, 8, 16, 4, False), (1024, 32, 8, 5, True), (5, 5, 7, 6, True),
+                                                           (64, 1, 9, 7, True)))
+def test_router_is_the_cpu_paths(gpu, n_experts, top_k, m, seed, renorm):
+    rng = np.random.default_rng(seed)
+    logits = np.stack([normal_f32(rng, n_experts) * np.float32(1 + (t % 5)) for t in range(m)])
+    gpu.fault_clear()
+    ids, wts, probs = run_router(gpu, logits, top_k, renorm)
+    want_all = np.empty_like(wts)
+    for t in range(m):
+        want_ids, want_all[t] = ora.route_softmax_topk(logits[t], top_k, renorm=renorm)
+        assert np.array_equal(ids[t], want_ids), t
+    assert_ulp(wts, want_all, "weights")
+    if n_experts <= 256:
+        assert_ulp(probs, oracle_probs(logits), "probabilities")
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+
+
+def test_router_ties_go_to_the_smaller_id(gpu):
+    logits = np.zeros((3, 128), np.float32)
+    logits[1, [5, 77, 100]] = 2.0          # three equal winners, then equal losers
+    logits[2] = np.float32(-3.5)
+    logits[2, 127] = np.float32(-3.0)
+    ids, wts, _ = run_router(gpu, logits, 4, want_probs=False)
+    assert ids[0].tolist() == [0, 1, 2, 3]
+    assert ids[1].tolist() == [5, 77, 100, 0]
+    assert ids[2].tolist() == [127, 0, 1, 2]
+    for t in range(3):
+        want_ids, want_w = ora.route_softmax_topk(logits[t], 4)
+        assert np.array_equal(ids[t], want_ids)
+        assert_ulp(wts[t], want_w, f"weights of token {t}", odd_share=1.0)
+
+
+@pytest.mark.parametrize("poison", (np.nan, np.inf, -np.inf))
+def test_router_raises_on_a_logit_that_is_not_finite(gpu, poison):
+    rng = np.random.default_rng(11)
+    logits = np.stack([normal_f32(rng, 128) for _ in range(6)])
+    logits[4, 93] = poison
+    gpu.fault_clear()
+    gpu.set_layer(3)
+    ids, wts, probs = run_router(gpu, logits, 8)
+    gpu.set_layer(0)
+    w0, mask = gpu.fault(3)
+    assert w0 == (3 << 8) + bm.SITE_ROUTER and mask == 1 << bm.SITE_ROUTER
+    assert np.isnan(wts[4]).all() and np.isnan(probs[4]).all()
+    assert (ids[4] == 0xEEEEEEEE).all()  # left as they stood
+    for t in (0, 1, 2, 3, 5):
+        want_ids, want_w = ora.route_softmax_topk(logits[t], 8)
+        assert np.array_equal(ids[t], want_ids)
+        assert_ulp(wts[t], want_w, f"weights of token {t}", odd_share=1.0)
+    gpu.fault_clear()
+
+
+def test_router_feeds_the_decode_step(gpu):
+    """logits -> bm_route_softmax -> bm_moe_decode, ids and weights never leaving the device: the oracle's layer."""
+    rng = np.random.default_rng(21)
+    L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 16, 22)
+    m, top_k = 3, 4
+    x = np.stack([normal_f32(rng, L.hidden) for _ in range(m)])
+    logits = np.stack([normal_f32(rng, L.n_experts) for _ in range(m)])
+    ld, xd = gpu.upload(logits, np.float32), gpu.upload(x, np.float32)
+    sel, wts = gpu.buffer(np.uint32, m * top_k), gpu.buffer(np.float32, m * top_k)
+    act_h = gpu.act(L.types[2], L.ff, m * top_k)
+    y = gpu.buffer(np.float32, m * L.hidden).fill_bytes(0xFF)
+    gpu.enqueue_route_softmax(ld, m, L.n_experts, top_k, True, None, sel, wts)
+    gpu.enqueue_moe_decode(L.dg, L.du, L.dd, xd, sel, wts, None, top_k, m, act_h, y)
+    got = y.download().reshape(m, L.hidden)
+    routes = [ora.route_softmax_topk(logits[t], top_k) for t in range(m)]
+    ids = np.stack([r[0] for r in routes])
+    w = np.stack([r[1] for r in routes])
+    want_y, _ = L.oracle(x, ids, w, top_k)
+    assert (sel.download().reshape(m, top_k) == ids).all()
+    err = np.max(np.abs(got.astype(np.float64) - np.asarray(want_y).reshape(m, L.hidden))) / np.max(np.abs(want_y))
+    assert err <= 1e-6, err  # the weights may differ in their last place, nothing else does
+    for b in (ld, xd, sel, wts, act_h, y):
+        b.free()
+    L.free()
+
+
+def test_router_refusals_are_named(gpu):
+    buf = gpu.buffer(np.float32, 4096)
+    ids = gpu.buffer(np.uint32, 64)
+    for args, word in (((1, 2048, 8), "n_experts"), ((1, 128, 33), "top_k"), ((1, 4, 5), "top_k"), ((0, 128, 8), "n_tokens")):
+        with pytest.raises(bm.GpuError) as e:
+            gpu.enqueue_route_softmax(buf, args[0], args[1], args[2], True, None, ids, buf)
+        assert e.value.code == bm.ESHAPE and word in str(e.value) and "bm_route_softmax" in str(e.value)
+    buf.free()
+    ids.free()

@@ -78,6 +78,17 @@ SYMBOLS = {
     "bm_gemm": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp]),
     "bm_swiglu_quant": (_i, [_vp, _vp, _vp, _i, _vp]),
     "bm_route_softmax": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "bm_gguf_open": (_i, [C.c_char_p, C.POINTER(_vp)]),
+    "bm_gguf_close": (None, [_vp]),
+    "bm_gguf_last_error": (C.c_char_p, []),
+    "bm_gguf_version": (_i, [_vp]),
+    "bm_gguf_tensor_count": (_i64, [_vp]),
+    "bm_gguf_tensor_at": (_i, [_vp, _i64, _vp]),
+    "bm_gguf_find": (_i, [_vp, C.c_char_p, _vp]),
+    "bm_gguf_get_u64": (_i, [_vp, C.c_char_p, C.POINTER(C.c_uint64)]),
+    "bm_gguf_get_f32": (_i, [_vp, C.c_char_p, C.POINTER(C.c_float)]),
+    "bm_gguf_get_str": (C.c_char_p, [_vp, C.c_char_p]),
+    "bm_weights_from_gguf": (_i, [_vp, _vp, C.c_char_p, C.POINTER(_vp), C.POINTER(_i), C.POINTER(_i)]),
     "bm_set_gemm_mode": (_i, [_vp, _i]),
     "bm_block_sums": (_i, [_vp, _vp, _i64, _vp, _i, _vp]),
     "bm_capture_begin": (_i, [_vp]),
@@ -183,6 +194,87 @@ class DeviceTensor:
     def free(self):
         if self.handle:
             self.gpu.lib.bm_weights_destroy(self.handle)
+            self.handle = None
+
+
+class _GgufTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("type", _i), ("n_dims", _i), ("dims", C.c_uint64 * 4), ("offset", C.c_uint64),
+                ("nbytes", C.c_uint64), ("data", _vp)]
+
+
+class Gguf:
+    """A model file's header and mapping (crates/gguf/src/lib.rs Gguf): tensors by name, key-values, and a tensor as a
+    weight stack on a Gpu. Host code: opening and reading need no GPU."""
+
+    def __init__(self, path):
+        self.lib = load_library()
+        h = _vp()
+        rc = self.lib.bm_gguf_open(os.fsencode(path), C.byref(h))
+        if rc:
+            raise GpuError(rc, self.lib.bm_gguf_last_error().decode())
+        self.handle = h.value
+
+    def _tensor(self, t):
+        return {"name": t.name.decode(), "type": t.type, "dims": [int(t.dims[d]) for d in range(t.n_dims)],
+                "offset": int(t.offset), "nbytes": int(t.nbytes), "data": t.data}
+
+    @property
+    def version(self):
+        return self.lib.bm_gguf_version(self.handle)
+
+    def tensors(self):
+        out = []
+        for i in range(self.lib.bm_gguf_tensor_count(self.handle)):
+            t = _GgufTensor()
+            rc = self.lib.bm_gguf_tensor_at(self.handle, i, C.byref(t))
+            if rc:
+                raise GpuError(rc, self.lib.bm_gguf_last_error().decode())
+            out.append(self._tensor(t))
+        return out
+
+    def find(self, name):
+        t = _GgufTensor()
+        rc = self.lib.bm_gguf_find(self.handle, name.encode(), C.byref(t))
+        if rc:
+            raise GpuError(rc, self.lib.bm_gguf_last_error().decode())
+        return self._tensor(t)
+
+    def data(self, name):
+        """The tensor's bytes, copied out of the mapping."""
+        t = self.find(name)
+        return np.ctypeslib.as_array(C.cast(t["data"], C.POINTER(C.c_uint8)), (t["nbytes"],)).copy() if t["nbytes"] else \
+            np.empty(0, np.uint8)
+
+    def get_u64(self, key):
+        v = C.c_uint64()
+        rc = self.lib.bm_gguf_get_u64(self.handle, key.encode(), C.byref(v))
+        if rc:
+            raise GpuError(rc, self.lib.bm_gguf_last_error().decode())
+        return v.value
+
+    def get_f32(self, key):
+        v = C.c_float()
+        rc = self.lib.bm_gguf_get_f32(self.handle, key.encode(), C.byref(v))
+        if rc:
+            raise GpuError(rc, self.lib.bm_gguf_last_error().decode())
+        return v.value
+
+    def get_str(self, key):
+        v = self.lib.bm_gguf_get_str(self.handle, key.encode())
+        return v.decode() if v is not None else None
+
+    def weights(self, gpu, name):
+        """The tensor as a DeviceTensor on `gpu`, with (rows_per_expert, n_experts) of an expert stack."""
+        h, rpe, ne = _vp(), _i(), _i()
+        gpu._check(self.lib.bm_weights_from_gguf(gpu.ctx, self.handle, name.encode(), C.byref(h), C.byref(rpe), C.byref(ne)))
+        t = self.find(name)
+        w = DeviceTensor.__new__(DeviceTensor)
+        w.gpu, w.wtype, w.rows, w.k, w.handle = gpu, t["type"], rpe.value * ne.value, t["dims"][0], h.value
+        return w, rpe.value, ne.value
+
+    def close(self):
+        if self.handle:
+            self.lib.bm_gguf_close(self.handle)
             self.handle = None
 
 

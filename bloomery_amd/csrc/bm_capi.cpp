@@ -740,6 +740,30 @@ int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_c
     return driver(ctx, what, bmk::swiglu_quant(launch_of(ctx), g_dev, u_dev, n_cols, act->k, act->dev));
 }
 
+int bm_weights_from_gguf(bm_ctx *ctx, const bm_gguf *g, const char *name, bm_weights **out, int *rows_per_expert, int *n_experts) {
+    const char *what = "bm_weights_from_gguf";
+    if (!ctx || !g || !name || !out) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    *out = nullptr;
+    bm_gguf_tensor t;
+    if (bm_gguf_find(g, name, &t) != BM_OK) return fail(ctx, BM_ESHAPE, "%s: %s", what, bm_gguf_last_error());
+    if (!known_type(t.type))
+        return fail(ctx, BM_ETYPE, "%s: %s is of ggml type %d; this library computes in Q4_K (12), Q6_K (14) and IQ2_XXS (16)", what,
+                    name, t.type);
+    if (t.n_dims < 2 || t.n_dims > 3)
+        return fail(ctx, BM_ESHAPE, "%s: %s has %d dimensions; a matrix has 2, an expert stack 3", what, name, t.n_dims);
+    if (t.dims[0] > (1u << 30) || t.dims[1] > (1u << 30) || t.dims[2] > (1u << 20))
+        return fail(ctx, BM_ESHAPE, "%s: %s is {%llu, %llu, %llu}: past what a stack holds", what, name, (unsigned long long)t.dims[0],
+                    (unsigned long long)t.dims[1], (unsigned long long)t.dims[2]);
+    const int k = (int)t.dims[0];
+    const int64_t rows = (int64_t)t.dims[1] * (int64_t)t.dims[2];
+    if ((uint64_t)rows * (uint64_t)bm_row_bytes(t.type, k) != t.nbytes)
+        return fail(ctx, BM_ESHAPE, "%s: %s holds %llu bytes, %lld rows of %d values take %lld", what, name, (unsigned long long)t.nbytes,
+                    (long long)rows, k, (long long)(rows * bm_row_bytes(t.type, k)));
+    if (rows_per_expert) *rows_per_expert = (int)t.dims[1];
+    if (n_experts) *n_experts = (int)t.dims[2];
+    return bm_weights_create(ctx, t.type, rows, k, t.data, out);
+}
+
 int bm_route_softmax(bm_ctx *ctx, const float *logits_dev, int n_tokens, int n_experts, int top_k, int renorm, float *probs_dev,
                      uint32_t *ids_dev, float *weights_dev) {
     const char *what = "bm_route_softmax";

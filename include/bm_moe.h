@@ -273,6 +273,42 @@ int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_c
 int bm_route_softmax(bm_ctx *ctx, const float *logits_dev, int n_tokens, int n_experts, int top_k, int renorm,
                      float *probs_dev, uint32_t *ids_dev, float *weights_dev);
 
+/* ------------------------------------------------------------------------------------------- model files */
+
+/* A GGUF file's header and a read-only mapping of it: the part of the reference's reader (crates/gguf/src/lib.rs:
+ * Gguf::open :319, find :540, data :557, value :439; TensorInfo :103) that hands a model file's expert stacks to
+ * bm_weights_create. Host code; no context is needed. Versions 2 and 3, little-endian. Every length, count and
+ * offset of the file is checked against its size at open (LoadError::OutOfBounds and friends are refusals here);
+ * bm_gguf_last_error() holds the message of the calling thread's last refusal. */
+typedef struct bm_gguf bm_gguf;
+typedef struct bm_gguf_tensor {
+    const char *name;  /* owned by the bm_gguf */
+    int type;          /* the ggml type id as the file states it (BM_TYPE_Q4_K = 12, BM_TYPE_Q6_K = 14, BM_TYPE_IQ2_XXS = 16, 0 = F32 ...) */
+    int n_dims;        /* 1 .. 4 */
+    uint64_t dims[4];  /* ggml ne[] order: dims[0] is the contiguous axis; unused dims are 1 */
+    uint64_t offset;   /* from the file's data section */
+    uint64_t nbytes;   /* type_size * (dims[0] / block) * dims[1] * ...; 0 for a type this build cannot size */
+    const void *data;  /* the tensor's bytes in the mapping (valid until bm_gguf_close); NULL when nbytes is 0 */
+} bm_gguf_tensor;
+int bm_gguf_open(const char *path, bm_gguf **out);
+void bm_gguf_close(bm_gguf *g);
+const char *bm_gguf_last_error(void);
+int bm_gguf_version(const bm_gguf *g);
+int64_t bm_gguf_tensor_count(const bm_gguf *g);
+int bm_gguf_tensor_at(const bm_gguf *g, int64_t i, bm_gguf_tensor *out);
+int bm_gguf_find(const bm_gguf *g, const char *name, bm_gguf_tensor *out);
+/* Key-values: an integer of any width that is not negative (Value::as_u64, crates/gguf/src/lib.rs:1510), an f32, a
+ * string (NULL when the key is absent or not a string). "<arch>.expert_count", "<arch>.expert_used_count" and
+ * "general.architecture" are what the MoE caller reads (crates/gguf/src/lib.rs:512-516,453). */
+int bm_gguf_get_u64(const bm_gguf *g, const char *key, uint64_t *out);
+int bm_gguf_get_f32(const bm_gguf *g, const char *key, float *out);
+const char *bm_gguf_get_str(const bm_gguf *g, const char *key);
+/* The tensor `name` of the file as a weight stack on the device: a matrix {k, rows} or an expert stack
+ * {k, rows_per_expert, n_experts} (crates/model/src/moe.rs:330 expert_view: expert e's matrix is the e-th equal part),
+ * rows back to back as bm_weights_create takes them. The tensor's type must be one this library computes in
+ * (BM_TYPE_Q4_K, BM_TYPE_Q6_K, BM_TYPE_IQ2_XXS); rows_per_expert and n_experts (either may be NULL) receive dims[1] and dims[2]. */
+int bm_weights_from_gguf(bm_ctx *ctx, const bm_gguf *g, const char *name, bm_weights **out, int *rows_per_expert, int *n_experts);
+
 /* ------------------------------------------------------------------------------------------- verification */
 
 /* The exact per-block integers the kernels above form for row `row` of w against column `col` of act, written

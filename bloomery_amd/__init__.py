@@ -22,6 +22,8 @@ LAYER_NONE = 0xFFFF
 SITE_QUANT_COLUMN, SITE_ROUTER, SITE_EXPERT_ID, SITE_STALLED = 1, 5, 7, 31
 PLAN_ONE_LAUNCH, PLAN_TWO_LAUNCHES = 1, 2
 GEMM_EXACT, GEMM_FAST = 0, 1
+ACT_SILU_MUL, ACT_SWIGLU_CLAMP, ACT_SWIGLU_OAI, ACT_SWIGLU_GCLAMP = 0, 1, 2, 4
+SITE_F32_PRODUCT = 21
 HOST_SLOT = 0xFFFFFFFF
 
 OK, ESHAPE, EDRIVER, ETYPE, EARG, EFAULT = 0, -1, -2, -3, -4, -5
@@ -77,6 +79,7 @@ SYMBOLS = {
     "bm_route_read": (_i, [_vp, _vp, _vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
     "bm_gemm": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp]),
     "bm_swiglu_quant": (_i, [_vp, _vp, _vp, _i, _vp]),
+    "bm_set_gate_rule": (_i, [_vp, _i, C.c_float]),
     "bm_route_softmax": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "bm_gguf_open": (_i, [C.c_char_p, C.POINTER(_vp)]),
     "bm_gguf_close": (None, [_vp]),
@@ -498,6 +501,10 @@ class Gpu:
     def enqueue_gemm(self, w, rows_per_expert, act, route, top_k, y):
         """top_k > 0: every slot of a token reads the token's column; 0: a column a slot."""
         self._check(self.lib.bm_gemm(self.ctx, w.handle, rows_per_expert, act.handle, route.handle, top_k, _ptr(y)))
+
+    def set_gate_rule(self, rule, limit=0.0):
+        """The Act of the gate . up launches that follow (crates/gpu/src/kquant/act.rs:21-57)."""
+        self._check(self.lib.bm_set_gate_rule(self.ctx, rule, float(limit)))
 
     def set_gemm_mode(self, mode):
         self._check(self.lib.bm_set_gemm_mode(self.ctx, mode))

@@ -1,6 +1,7 @@
 // The C ABI of libbm_moe_hip.so (include/bm_moe.h): handles, the host-side geometry checks the reference's
 // launchers make before a launch (crates/gpu/src/q4k_sel.rs:990-1042 and its siblings), and the calls into the
 // kernels. Refusals carry a message naming the entry point and the lengths, as GpuError::Shape does.
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -21,6 +22,7 @@ struct bm_ctx {
     uint32_t *counters = nullptr; // bm_moe_decode's producer/consumer counts, zero between launches
     int decode_plan = BM_PLAN_TWO_LAUNCHES;
     int gemm_mode = BM_GEMM_EXACT;
+    bmk::GateRule rule = {0u, 0.0f}; // silu(g) * u
     uint32_t spin_limit = 1u << 18; // a poll is a round trip to memory: some tenths of a second of waiting
     std::string err;
 };
@@ -167,7 +169,7 @@ int bm_fault_read(bm_ctx *ctx, uint32_t layer, uint32_t *word0, uint32_t *mask) 
     return rc;
 }
 
-static bmk::Launch launch_of(bm_ctx *ctx) { return bmk::Launch{ctx->stream, ctx->fault, ctx->layer}; }
+static bmk::Launch launch_of(bm_ctx *ctx) { return bmk::Launch{ctx->stream, ctx->fault, ctx->layer, ctx->rule}; }
 
 int bm_fault_clear(bm_ctx *ctx) {
     if (!ctx) return fail(nullptr, BM_EARG, "bm_fault_clear: ctx is NULL");
@@ -720,6 +722,35 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
         return fail(ctx, BM_ESHAPE, "%s: %d slots read %d activation columns, act holds %d", what, n_slots, n_slots / slot_div, act->m_cap);
     return driver(ctx, what, bmk::gemm(launch_of(ctx), w->wtype, w->dev, route->n_experts, rows_per_expert, w->k, act->dev, route->cols,
                                        route->tiles, route->n_tiles, n_slots, slot_div, y_dev, ctx->gemm_mode));
+}
+
+int bm_set_gate_rule(bm_ctx *ctx, int rule, float limit) {
+    const char *what = "bm_set_gate_rule";
+    if (!ctx) return fail(nullptr, BM_EARG, "%s: ctx is NULL", what);
+    // crates/gpu/src/kquant/act.rs:71-125 Act::code: what the device rules can run
+    switch (rule) {
+    case BM_ACT_SILU_MUL:
+        limit = 0.0f;
+        break;
+    case BM_ACT_SWIGLU_CLAMP:
+        if (!std::isfinite(limit)) return fail(ctx, BM_ESHAPE, "%s: the clamp limit must be finite, got %g", what, (double)limit);
+        break;
+    case BM_ACT_SWIGLU_OAI:
+        if (!std::isfinite(limit) || limit < 0.0f)
+            return fail(ctx, BM_ESHAPE, "%s: swigluoai runs at alpha 1.702 and a finite limit of at least 0, got limit %g", what,
+                        (double)limit);
+        break;
+    case BM_ACT_SWIGLU_GCLAMP:
+        if (!std::isfinite(limit) || !(limit > 0.0f))
+            return fail(ctx, BM_ESHAPE, "%s: the gate-first clamp limit must be finite and positive, got %g; a caller that clamps "
+                        "nothing runs BM_ACT_SWIGLU_CLAMP", what, (double)limit);
+        break;
+    default:
+        return fail(ctx, BM_ETYPE, "%s: rule %d is not one of BM_ACT_SILU_MUL, BM_ACT_SWIGLU_CLAMP, BM_ACT_SWIGLU_OAI, "
+                    "BM_ACT_SWIGLU_GCLAMP (SiTU-GLU, code 3, is not built)", what, rule);
+    }
+    ctx->rule = bmk::GateRule{(uint32_t)rule, limit};
+    return BM_OK;
 }
 
 int bm_set_gemm_mode(bm_ctx *ctx, int mode) {

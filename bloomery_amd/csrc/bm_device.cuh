@@ -554,9 +554,57 @@ __device__ __forceinline__ float bm_expf_ik(float x) {
     return fmaf(j, k, k);
 }
 
-__device__ __forceinline__ float bm_swiglu(float g, float u) {
+__device__ __forceinline__ float bm_silu(float g) {
     const float e = bm_expf_ik(__fsub_rn(0.0f, g));
-    return __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, e)), u);
+    return __fdiv_rn(g, __fadd_rn(1.0f, e));
+}
+
+__device__ __forceinline__ float bm_swiglu(float g, float u) { return __fmul_rn(bm_silu(g), u); }
+
+// The clamped rules, comparison for comparison as the CPU path spells them (a NaN falls through each the same way).
+// ik's: min(silu(g), limit) * clamp(u, -limit, limit), nothing clamped at limit <= 1e-6
+// (crates/qdot/src/lib.rs:11492-11523 swiglu_clamp).
+__device__ __forceinline__ float bm_swiglu_clamp(float g, float u, float limit) {
+    float s = bm_silu(g), c = u;
+    if (limit > 1e-6f) {
+        s = limit < s ? limit : s;
+        c = u < limit ? u : limit;
+        c = -limit < c ? c : -limit;
+    }
+    return __fmul_rn(c, s);
+}
+// gpt-oss / MiniMax: x = min(g, limit), y = clamp(u, -limit, limit), x / (1 + e^(-alpha x)) * (y + 1), alpha 1.702
+// (crates/qdot/src/lib.rs swiglu_oai_1, crates/gpu/src/kquant/act.rs:213-223).
+__device__ __forceinline__ float bm_swiglu_oai(float g, float u, float limit) {
+    const float x = limit < g ? limit : g;
+    const float y = u < -limit ? -limit : (limit < u ? limit : u);
+    const float e = bm_expf_ik(__fmul_rn(1.702f, __fsub_rn(0.0f, x)));
+    return __fmul_rn(__fdiv_rn(x, __fadd_rn(1.0f, e)), __fadd_rn(y, 1.0f));
+}
+// ggml's gate-first clamp: silu(min(g, limit)) * clamp(u, -limit, limit), nothing clamped at limit <= 1e-6
+// (crates/qdot/src/lib.rs:11617-11660 swiglu_gclamp, swiglu_gclamp_1).
+__device__ __forceinline__ float bm_swiglu_gclamp(float g, float u, float limit) {
+    float x = g, y = u;
+    if (limit > 1e-6f) {
+        x = limit < g ? limit : g;
+        y = u < -limit ? -limit : (limit < u ? limit : u);
+    }
+    return __fmul_rn(bm_silu(x), y);
+}
+
+// A row's value under rule `act` (crates/gpu/src/kquant/act.rs:136-149 apply). Under the clamped rules a sum that is
+// not finite would come out finite: `odd` reports it and the value is NaN (:166-175 apply_checked; the CPU path's
+// rules return false for such a block). The plain rule lets it through as it is, as the CPU path's swiglu does.
+__device__ __forceinline__ float bm_gate_rule(u32 act, float limit, float g, float u, bool &odd) {
+    odd = false;
+    if (act == 0u) return bm_swiglu(g, u);
+    if (!(fabsf(g) <= 3.402823466e38f && fabsf(u) <= 3.402823466e38f)) {
+        odd = true;
+        return bm_bits_f32(0x7fc00000u);
+    }
+    if (act == 1u) return bm_swiglu_clamp(g, u, limit);
+    if (act == 2u) return bm_swiglu_oai(g, u, limit);
+    return bm_swiglu_gclamp(g, u, limit);
 }
 
 #endif // BM_DEVICE_CUH

@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
                                                        const uint8_t *act, int act_cols, const u32 *order,
                                                        const u32 *start, const u32 *tiles, u32 n_slots, u32 cap,
                                                        int rpe, int slots_per_col, float *h, uint8_t *act_h,
-                                                       u32 *fault, u32 layer) {
+                                                       GateRule rule, u32 *fault, u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
     Tile t;
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
     row_dot<WT, U, NB, kTileCols>(b, wrow, cols, col_bytes, t.m, n, q, tb, v, NoTap{});
 #pragma unroll
     for (int c = 0; c < kTileCols; c++) {
-        float hv = swiglu_of_pair(v[c], which);
+        float hv = swiglu_of_pair(c < t.m ? v[c] : 0.0f, which, rule, fault, layer);
         if (c < t.m) {
             if (bad[c] == 0xffffffffu) hv = bm_bits_f32(0x7fc00000u);
             if (h && active && (tid & 7) == 0) h[(size_t)(t.j + c) * rpe + r] = hv;
@@ -223,7 +223,7 @@ hipError_t gate_up_tiles(const Launch &L, int wtype, const uint8_t *wg, const ui
     hipError_t e = allow_lds(kern, lds);                                                                               \
     if (e != hipSuccess) return e;                                                                                     \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, wg, wu, (u32)n_experts, nb, act, act_cols, order,   \
-                       start, tiles_dev, (u32)n_slots, cap, rpe, slots_per_col, h, act_h, L.fault, L.layer);
+                       start, tiles_dev, (u32)n_slots, cap, rpe, slots_per_col, h, act_h, L.rule, L.fault, L.layer);
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
     return hipGetLastError();

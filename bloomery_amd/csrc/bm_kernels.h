@@ -8,10 +8,19 @@
 
 namespace bmk {
 
+// The rule a gate . up launch applies to a row's two sums (crates/gpu/src/kquant/act.rs:21-57 Act and its device
+// codes): silu(g) * u, ik's clamped SwiGLU, the gpt-oss / MiniMax SwiGLU at alpha 1.702, ggml's gate-first clamp.
+struct GateRule {
+    uint32_t act;
+    float limit;
+};
+constexpr uint32_t kActSiluMul = 0, kActSwigluClamp = 1, kActSwigluOai = 2, kActSwigluGclamp = 4;
+
 struct Launch {
     hipStream_t stream;
     uint32_t *fault; // device fault word, u32[BM_FAULT_WORDS]
     uint32_t layer;  // layer the launch raises with
+    GateRule rule;   // what the gate . up launches apply
 };
 
 // Largest dynamic LDS a launch may ask for (gfx950 has 160 KiB a workgroup).

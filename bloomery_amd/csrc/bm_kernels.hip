@@ -168,7 +168,7 @@ __global__ __launch_bounds__(256) void k_gemv(const uint8_t *w, long rows, int n
 template <int WT, int U, int NB>
 __global__ __launch_bounds__(256) void k_gate_up(const uint8_t *wg, const uint8_t *wu, u32 n_experts, int nb,
                                                  const uint8_t *act, const u32 *sel, int rpe, int slots_per_col,
-                                                 float *h, uint8_t *act_h, u32 *fault, u32 layer) {
+                                                 float *h, uint8_t *act_h, GateRule rule, u32 *fault, u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
     const int blocks_per_slot = (rpe + 31) / 32;
@@ -199,7 +199,7 @@ __global__ __launch_bounds__(256) void k_gate_up(const uint8_t *wg, const uint8_
     __syncthreads();
     float v[1];
     row_dot<WT, U, NB, 1>(b, wrow, col, col_bytes, 1, n, q, tb, v, NoTap{});
-    const float hv = swiglu_of_pair(v[0], which);
+    const float hv = swiglu_of_pair(v[0], which, rule, fault, layer);
     if (h && active && (tid & 7) == 0) h[(size_t)slot * rpe + r] = hv;
     if (act_h) { // rpe is a multiple of 256 here, so every row of the block is live
         float *hbuf = reinterpret_cast<float *>(col + col_bytes);
@@ -426,7 +426,8 @@ __device__ __forceinline__ void q82_quad8(const float (&v)[8], uint8_t *col, int
 template <int WA, int UA, int NBA>
 __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, const uint8_t *wg, const uint8_t *wu,
                                                u32 n_experts, int na, int nh, const u32 *sel, int spt, uint8_t *act_x,
-                                               uint8_t *act_h, float *h, int slot, int rb, u32 *fault, u32 layer) {
+                                               uint8_t *act_h, float *h, int slot, int rb, GateRule rule, u32 *fault,
+                                               u32 layer) {
     const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
     const int hidden = na * 256, ff = nh * 256;
     const int t = slot / spt;
@@ -475,7 +476,7 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
     if (act_x && rb == 0 && slot % spt == 0) stage_bytes(act_x + (size_t)t * col_bytes, col, col_bytes);
     float v[1];
     row_dot<WA, UA, NBA, 1>(b, wrow, col, col_bytes, 1, na, q, Iq2Tables{}, v, NoTap{});
-    const float hv = swiglu_of_pair(v[0], which);
+    const float hv = swiglu_of_pair(v[0], which, rule, fault, layer);
     if (h && (tid & 7) == 0) h[(size_t)slot * ff + r] = hv;
     float *hbuf = reinterpret_cast<float *>(col + col_bytes);
     if ((tid & 7) == 0) hbuf[tid >> 3] = hv;
@@ -487,11 +488,11 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
 template <int WA, int UA, int NBA>
 __global__ __launch_bounds__(256) void k_gate_up_x(const float *x, const uint8_t *wg, const uint8_t *wu, u32 n_experts,
                                                    int nba, int nh, const u32 *sel, int spt, uint8_t *act_x,
-                                                   uint8_t *act_h, float *h, u32 *fault, u32 layer) {
+                                                   uint8_t *act_h, float *h, GateRule rule, u32 *fault, u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int blocks_per_slot = nh * 8;
     gate_up_x_body<WA, UA, NBA>(lds, x, wg, wu, n_experts, NBA > 0 ? NBA : nba, nh, sel, spt, act_x, act_h, h,
-                                blockIdx.x / blocks_per_slot, blockIdx.x % blocks_per_slot, fault, layer);
+                                blockIdx.x / blocks_per_slot, blockIdx.x % blocks_per_slot, rule, fault, layer);
 }
 
 // The decode step of one MoE layer for m tokens in one launch. The first n_a workgroups are the gate . up ones
@@ -505,7 +506,8 @@ __global__ __launch_bounds__(256) void k_moe_decode(const float *x, const uint8_
                                                     const uint8_t *wd, u32 n_experts, int nba, int nbb,
                                                     const u32 *sel, const float *wts, const float *resid, int spt,
                                                     int m, uint8_t *act_x, uint8_t *act_h, float *h, float *y,
-                                                    u32 *counters, u32 spin_limit, u32 *fault, u32 layer) {
+                                                    u32 *counters, u32 spin_limit, GateRule rule, u32 *fault,
+                                                    u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x;
     const int na = NBA > 0 ? NBA : nba, nh = NBB > 0 ? NBB : nbb;
@@ -515,7 +517,7 @@ __global__ __launch_bounds__(256) void k_moe_decode(const float *x, const uint8_
     if ((int)blockIdx.x < n_a) {
         const int slot = blockIdx.x / blocks_per_slot;
         gate_up_x_body<WA, UA, NBA>(lds, x, wg, wu, n_experts, na, nh, sel, spt, act_x, act_h, h, slot,
-                                    blockIdx.x % blocks_per_slot, fault, layer);
+                                    blockIdx.x % blocks_per_slot, rule, fault, layer);
         // publish: the block's stores (complete at the barrier), then the count with agent-scope release
         __syncthreads();
         if (tid == 0)
@@ -619,7 +621,7 @@ hipError_t gate_up(const Launch &L, int wtype, const uint8_t *wg, const uint8_t 
     hipError_t e = allow_lds(kern, lds);                                                                               \
     if (e != hipSuccess) return e;                                                                                     \
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, wg, wu, (u32)n_experts, nb, act, sel, rpe,          \
-                       slots_per_col, h, act_h, L.fault, L.layer);
+                       slots_per_col, h, act_h, L.rule, L.fault, L.layer);
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
     return hipGetLastError();
@@ -681,7 +683,7 @@ hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8
         hipError_t e = allow_lds(kern, lds_a);                                                                         \
         if (e != hipSuccess) return e;                                                                                 \
         hipLaunchKernelGGL(kern, dim3(grid_a), dim3(256), lds_a, L.stream, x, wg, wu, (u32)n_experts, nba, nbb, sel,   \
-                           spt, act_x, act_h, h, L.fault, L.layer);                                                    \
+                           spt, act_x, act_h, h, L.rule, L.fault, L.layer);                                            \
     }
     if (nba == 8) BM_GUX(kRingQ4K, 8)
     else BM_GUX(1, 0)
@@ -712,7 +714,7 @@ hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, c
         hipError_t e = allow_lds(kern, lds);                                                                           \
         if (e != hipSuccess) return e;                                                                                 \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, x, wg, wu, wd, (u32)n_experts, nba, nbb, sel,   \
-                           wts, resid, spt, m, act_x, act_h, h, y, counters, spin_limit, L.fault, L.layer);            \
+                           wts, resid, spt, m, act_x, act_h, h, y, counters, spin_limit, L.rule, L.fault, L.layer);    \
     }
     if (down_type == BM_Q6K) {
         if (nba == 8 && nbb == 3) BM_FUSED(BM_Q4K, kRingQ4K, 8, BM_Q6K, kRingQ6K, 3)

@@ -70,13 +70,15 @@ hipError_t route(const Launch &L, const uint32_t *ids, int n_slots, int n_expert
 // crates/gpu/src/gemm/swiglu.rs:46-58 in the CPU path's rules: column c of act = Q8_2_X4(swiglu(g, u)) over the k
 // values g[c * k ..], u[c * k ..]. One half wave a 32-value block.
 __global__ __launch_bounds__(256) void k_swiglu_quant(const float *g, const float *u, int m, int k, uint8_t *act,
-                                                      u32 *fault, u32 layer) {
+                                                      GateRule rule, u32 *fault, u32 layer) {
     const int bpc = k / 32;
     const long gblk = (long)blockIdx.x * 8 + (threadIdx.x >> 5);
     if (gblk >= (long)m * bpc) return;
     const int col = (int)(gblk / bpc), blk = (int)(gblk % bpc), lane32 = threadIdx.x & 31;
     const size_t at = (size_t)col * k + 32 * blk + lane32;
-    const float v = bm_swiglu(g[at], u[at]);
+    bool odd;
+    const float v = bm_gate_rule(rule.act, rule.limit, g[at], u[at], odd);
+    if (odd) bm_raise(fault, layer, kSiteF32Product);
     Q82Head hd;
     int s16;
     const int code = q82_block(v, &hd, &s16);
@@ -87,7 +89,7 @@ __global__ __launch_bounds__(256) void k_swiglu_quant(const float *g, const floa
 hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act) {
     const long blocks = (long)m * (k / 32);
     hipLaunchKernelGGL(k_swiglu_quant, dim3((unsigned)((blocks + 7) / 8)), dim3(256), 0, L.stream, g, u, m, k, act,
-                       L.fault, L.layer);
+                       L.rule, L.fault, L.layer);
     return hipGetLastError();
 }
 

@@ -24,6 +24,7 @@ namespace bmk {
 
 constexpr u32 kSiteQuantColumn = 1; // crates/device/src/fault.rs:73-76
 constexpr u32 kSiteExpertId = 7;    // crates/device/src/fault.rs:89
+constexpr u32 kSiteF32Product = 21; // crates/device/src/fault.rs:151-155: a gate or up sum that is not finite under a clamp
 constexpr u32 kSiteStalled = 31;    // ours: a fused launch's down workgroup gave up waiting for its activations
 
 // LDS bytes of the IQ2_XXS tables: 2048 grid + 128 signs + 64 nibble masks, padded to a 16-byte multiple.
@@ -244,10 +245,13 @@ __device__ __forceinline__ void q82_store(uint8_t *col, int nb, int blk, int lan
 }
 
 // The gate/up exchange of the eight lanes of an output: lanes 0..3 hold the gate dot, 4..7 the up dot.
-__device__ __forceinline__ float swiglu_of_pair(float v, int which) {
+__device__ __forceinline__ float swiglu_of_pair(float v, int which, GateRule rule, u32 *fault, u32 layer) {
     // both moves run on every lane: a lane-crossing move under a divergent branch reads switched-off lanes as 0
     const float from_above = bm_dppf<kDppShl4>(v), from_below = bm_dppf<kDppShr4>(v);
-    return bm_swiglu(which ? from_below : v, which ? v : from_above);
+    bool odd;
+    const float hv = bm_gate_rule(rule.act, rule.limit, which ? from_below : v, which ? v : from_above, odd);
+    if (odd) bm_raise(fault, layer, kSiteF32Product);
+    return hv;
 }
 
 // The 32 values a workgroup produced (hbuf, LDS) as block `rb` of column `hcol`, by the first 32 threads.

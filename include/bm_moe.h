@@ -46,6 +46,7 @@ extern "C" {
 #define BM_SITE_QUANT_COLUMN 1 /* a quantizer met a value that is not finite: NaN scale, zero codes */
 #define BM_SITE_ROUTER 5       /* a token's logits hold a value that is not finite */
 #define BM_SITE_EXPERT_ID 7    /* an expert id at or past the stack */
+#define BM_SITE_F32_PRODUCT 21 /* a gate or up sum that is not finite met a clamped gate rule: the value is NaN */
 #define BM_SITE_STALLED 31     /* ours: a bm_moe_decode consumer gave up waiting for its producers */
 
 /* The id of a slot served elsewhere (crates/gpu/src/host/slots.rs:10): the down projections skip it silently. */
@@ -258,6 +259,22 @@ int bm_set_gemm_mode(bm_ctx *ctx, int mode);
  * silu(g) * u of g_dev / u_dev[c * k .. (c + 1) * k), k = act's k, slot-major as the gate and up GEMMs write them;
  * bm_quantize's bytes of the CPU path's SwiGLU. Q8_2_X4 columns only. */
 int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, bm_act *act);
+
+/* The rule the gate . up entries (bm_gate_up, bm_gate_up_x, bm_moe_decode, bm_gate_up_tiles, bm_swiglu_quant) apply to
+ * a row's gate sum g and up sum u: the Act argument of the reference's launchers (crates/gpu/src/kquant/act.rs:21-57,
+ * device codes :46-56), set on the context and read by each launch as it is enqueued. The numbers are the CPU path's
+ * (crates/qdot/src/lib.rs:11467 swiglu, :11492 swiglu_clamp, swiglu_oai, :11617 swiglu_gclamp), every exponential ik's.
+ *   BM_ACT_SILU_MUL       silu(g) * u (the default; limit ignored)
+ *   BM_ACT_SWIGLU_CLAMP   min(silu(g), limit) * clamp(u, -limit, limit); limit <= 1e-6 clamps nothing; limit finite
+ *   BM_ACT_SWIGLU_OAI     x = min(g, limit), y = clamp(u, -limit, limit): x / (1 + e^(-1.702 x)) * (y + 1); limit finite, >= 0
+ *   BM_ACT_SWIGLU_GCLAMP  silu(min(g, limit)) * clamp(u, -limit, limit); limit finite and positive
+ * Under the three clamped rules a sum that is not finite raises BM_SITE_F32_PRODUCT and its value is NaN (act.rs:166-175
+ * apply_checked; the CPU path's rules return false for such a block). SiTU-GLU (code 3) is not built. */
+#define BM_ACT_SILU_MUL 0
+#define BM_ACT_SWIGLU_CLAMP 1
+#define BM_ACT_SWIGLU_OAI 2
+#define BM_ACT_SWIGLU_GCLAMP 4
+int bm_set_gate_rule(bm_ctx *ctx, int rule, float limit);
 
 /* ------------------------------------------------------------------------------------------------- router */
 

@@ -60,6 +60,7 @@ int ora_dequant_col(int wtype, const uint8_t *acol, int k, float *dst);
 
 float ora_expf_ik(float x);
 void ora_swiglu(const float *gate, const float *up, int n, float *out);
+int ora_gate_rule(int rule, float limit, const float *gate, const float *up, int n, float *out);
 
 // Router and combine, in the caller's order (harness side of the path).
 int ora_route_softmax_topk(const float *logits, int n_experts, int top_k, int renorm, uint32_t *ids, float *w);

@@ -52,6 +52,7 @@ def _load():
         "ora_dequant_col": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
         "ora_expf_ik": (C.c_float, [C.c_float]),
         "ora_swiglu": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_gate_rule": (C.c_int, [C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
         "ora_route_softmax_topk": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
         "ora_combine_tokens": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
         "ora_quantize_row_q4k": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
@@ -200,6 +201,16 @@ def swiglu(gate, up):
     out = np.empty_like(gate)
     lib.ora_swiglu(_p(gate), _p(up), gate.size, _p(out))
     return out
+
+
+def gate_rule(rule, limit, gate, up):
+    """(out, finite): a gate . up rule of the CPU path over two vectors; `finite` is the reference functions' flag."""
+    gate, up = _f32(gate), _f32(up)
+    out = np.empty_like(gate)
+    rc = lib.ora_gate_rule(int(rule), float(limit), _p(gate), _p(up), gate.size, _p(out))
+    if rc < 0:
+        raise ValueError(f"no gate rule {rule}")
+    return out, bool(rc)
 
 
 def route_softmax_topk(logits, top_k, renorm=True):

@@ -469,3 +469,42 @@ float ora_expf_ik(float x) {
 void ora_swiglu(const float *gate, const float *up, int n, float *out) {
     for (int i = 0; i < n; i++) out[i] = gate[i] / (1.0f + ora_expf_ik(0.0f - gate[i])) * up[i];
 }
+
+// The other gate . up rules of the CPU path, each comparison spelled as the reference spells it (so a NaN falls
+// through the same way), the exponential ik's. rule 1: swiglu_clamp (crates/qdot/src/lib.rs:11492-11523): min(silu(g),
+// limit) * clamp(u), nothing clamped at limit <= 1e-6. rule 2: swiglu_oai / swiglu_oai_1 at alpha 1.702 (the value the
+// launchers run, crates/gpu/src/kquant/act.rs:58-60): x = min(g, limit), y = clamp(u), x / (1 + e^(alpha (0 - x))) *
+// (y + 1). rule 4: swiglu_gclamp / swiglu_gclamp_1 (:11617-11660): silu(min(g, limit)) * clamp(u), nothing clamped at
+// limit <= 1e-6. rule 0: ora_swiglu. Returns what the reference's functions return: 0 when a clamping rule met a gate
+// or up value that is not finite (the caller refuses the block), else 1; -1 for a rule this file does not hold.
+int ora_gate_rule(int rule, float limit, const float *gate, const float *up, int n, float *out) {
+    if (rule == 0) {
+        ora_swiglu(gate, up, n, out);
+        return 1;
+    }
+    if (rule != 1 && rule != 2 && rule != 4) return -1;
+    if ((rule == 1 || rule == 4) && !(limit > 1e-6f)) { // a NaN limit clamps nothing either
+        ora_swiglu(gate, up, n, out);
+        return 1;
+    }
+    int finite = 1;
+    for (int i = 0; i < n; i++) {
+        const float g = gate[i], u = up[i];
+        if (!isfinite(g) || !isfinite(u)) finite = 0;
+        if (rule == 1) {
+            float s = g / (1.0f + ora_expf_ik(0.0f - g));
+            s = limit < s ? limit : s;
+            float c = u < limit ? u : limit;
+            c = -limit < c ? c : -limit;
+            out[i] = c * s;
+        } else {
+            const float x = limit < g ? limit : g;
+            const float y = u < -limit ? -limit : (limit < u ? limit : u);
+            if (rule == 2)
+                out[i] = x / (1.0f + ora_expf_ik(1.702f * (0.0f - x))) * (y + 1.0f);
+            else
+                out[i] = x / (1.0f + ora_expf_ik(0.0f - x)) * y;
+        }
+    }
+    return finite;
+}

@@ -50,6 +50,72 @@ def test_swiglu_is_divide_then_multiply_and_position_independent():
     assert big[0] == 200.0 and abs(big[1]) < 1e-40 and big[2] == 0.0
 
 
+def silu64(g):
+    g = np.asarray(g, np.float64)
+    return g / (1.0 + np.exp(-g))
+
+
+def test_gate_rules_by_their_definitions():
+    """The clamped rules against what their definitions fix (crates/qdot/tests/qdot.rs:4035-4046 ik_swiglu_clamp,
+    :4158-4169 ref_swiglu_oai are transcriptions of the sources; here the cases a transcription could get wrong are
+    worked by hand): which quantity each limit bites on, the +1 of the OAI rule, its alpha, the no-clamp threshold,
+    NaN through every comparison, and the finite flag."""
+    f = np.float32
+    L = f(7.0)
+    g = np.array([20.0, 20.0, 20.0, 1.0, 1.0, -30.0, 0.0, 7.0, 6.9999], f)
+    u = np.array([3.0, 9.0, -9.0, 9.0, -0.5, 2.0, 5.0, 7.0, -7.0], f)
+    s = ora.swiglu(g, np.ones_like(g))  # silu(g), pinned above
+    # ik's clamp: the limit bites on silu(g), not on g
+    out, ok = ora.gate_rule(1, L, g, u)
+    want = np.minimum(s, L) * np.clip(u, -L, L)
+    assert ok and out.tobytes() == want.astype(f).tobytes()
+    assert out[0] == 21.0 and out[1] == 49.0 and out[2] == -49.0  # silu(20) = 20 > 7
+    # the gate-first clamp: the limit bites on g before the activation: silu(7) < 7
+    out4, ok = ora.gate_rule(4, L, g, u)
+    s7 = ora.swiglu(np.array([7.0], f), np.ones(1, f))[0]
+    assert ok and out4[0] == f(s7 * f(3.0)) and out4[1] == f(s7 * L) and out4[2] == f(s7 * -L)
+    assert out4[3:].tobytes() == (ora.swiglu(np.minimum(g, L), np.ones_like(g)) * np.clip(u, -L, L))[3:].astype(f).tobytes()
+    assert s7 < 7.0 and out4[0] != out[0]
+    # the OAI rule: x / (1 + e^(-1.702 x)) * (y + 1), gate clamped from above only
+    out2, ok = ora.gate_rule(2, L, g, u)
+    x, y = np.minimum(g, L).astype(np.float64), np.clip(u, -L, L).astype(np.float64)
+    ref = x / (1.0 + np.exp(-1.702 * x)) * (y + 1.0)
+    assert ok and np.max(np.abs(out2 - ref)) <= 2e-6 * np.max(np.abs(ref))
+    assert abs(out2[4] - 1.0 / (1.0 + np.exp(-1.702)) * 0.5) < 1e-6      # y + 1 with y = -0.5
+    assert abs(out2[5] - (-30.0 / (1.0 + np.exp(1.702 * 30.0)) * 3.0)) < 1e-20  # no clamp from below on the gate
+    e = ora.expf_ik(f(1.702) * (f(0.0) - f(1.0)))
+    assert out2[3].tobytes() == f(f(f(1.0) / f(f(1.0) + e)) * f(8.0)).tobytes()  # op order: divide, then (y + 1)
+    # a limit at or below 1e-6 (or NaN) clamps nothing under rules 1 and 4: the plain rule's bits
+    plain = ora.swiglu(g, u)
+    for lim in (0.0, 1e-6, -1.0, np.nan):
+        for rule in (1, 4):
+            o, ok = ora.gate_rule(rule, lim, g, u)
+            assert ok and o.tobytes() == plain.tobytes()
+    o, ok = ora.gate_rule(1, 2e-6, g, u)
+    assert o.tobytes() != plain.tobytes()
+    # rule 0 is swiglu; an unknown rule is refused
+    assert ora.gate_rule(0, 5.0, g, u)[0].tobytes() == plain.tobytes()
+    with pytest.raises(ValueError):
+        ora.gate_rule(3, 1.0, g, u)
+    # NaN through the comparisons: ik's clamp turns a NaN up into the limit and lets a NaN silu through; the other two
+    # let a NaN up through (std::clamp); every clamping rule reports the block
+    nan, inf = f(np.nan), f(np.inf)
+    o, ok = ora.gate_rule(1, L, np.array([1.0, nan, inf], f), np.array([nan, 2.0, 2.0], f))
+    assert not ok and o[0] == f(s[3] * L) and np.isnan(o[1]) and o[2] == 14.0
+    for rule in (2, 4):
+        o, ok = ora.gate_rule(rule, L, np.array([1.0, nan, inf, 1.0], f), np.array([nan, 2.0, 2.0, -inf], f))
+        assert not ok and np.isnan(o[0]) and np.isnan(o[1]) and np.isfinite(o[2]) and np.isfinite(o[3])
+    o, ok = ora.gate_rule(1, 0.0, np.array([inf], f), np.array([1.0], f))
+    assert ok and not np.isfinite(o[0])  # below the threshold nothing is hidden, so nothing is reported
+    # position independence
+    rng = np.random.default_rng(5)
+    gg, uu = normal_f32(rng, 333, 6.0), normal_f32(rng, 333, 6.0)
+    for rule in (1, 2, 4):
+        o, _ = ora.gate_rule(rule, 5.0, gg, uu)
+        for i in (0, 7, 8, 332):
+            assert ora.gate_rule(rule, 5.0, gg[i:i + 1], uu[i:i + 1])[0][0].tobytes() == o[i].tobytes()
+
+
 # ------------------------------------------------------------------------------------------- router and combine
 
 def test_router_softmax_topk_renorm():

@@ -131,27 +131,41 @@ __device__ __forceinline__ u32 q6_minus_32(u32 q) {
     return t | (m << 1) | (m << 2);
 }
 
-// A workgroup of 1024 / T threads takes a tile of <= 64 slots and a slab of 64 rows. Wave w works on rows
-// 16 * (w & 3) .. and slots 16 T * (w >> 2) ..: T 16 x 16 products a 32-value block and half. v_mfma_i32_16x16x32_i8 sums over 32
-// values; a 16-value half comes out of it by zeroing the other half's weight codes, the lanes of one half of the
-// k range holding them (lane / 16 = k / 8). 4 T results a lane, 32 T accumulators: two to four waves a SIMD
-// stay resident and hide each other's LDS and matrix latencies.
-template <int WT, int T>
-__global__ __launch_bounds__(1024 / T) void k_gemm(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
-                                                 const u32 *tiles, const u32 *n_tiles, u32 n_slabs, u32 slot_div,
+// LDS of the exact kernel: the weight rows arrive unpacked, a signed byte a code (Q4_K 0..15, Q6_K q6 - 32), behind a
+// 24-byte header (Q4_K: d, dmin, the twelve scale bytes; Q6_K: the sixteen scales, d), so the arithmetic waves read
+// matrix operands as they are; a page of zeros stands in for the half of an operand that must not count.
+constexpr int kRowCodesAt = 24, kRowStride = kRowCodesAt + 256; // 280: off the bank period
+constexpr int kZeroPage = 256 + 32;
+__host__ __device__ constexpr size_t gemm_exact_lds_bytes(int slots) {
+    return sizeof(GemmLds) + (size_t)slots * kActStride + (size_t)kGemmBM * kRowStride + kZeroPage + 16 * kGemmBM * sizeof(float);
+}
+
+// A workgroup of 4 CH waves takes 16 T CH slots of a tile (all 64, or a part of it: a tile's parts are workgroups of
+// their own) and a slab of 64 rows. Wave w works on rows 16 * (w & 3) .. and slots 16 T * (w >> 2) ..: T 16 x 16
+// products a 16-value group. Parts of 32 slots put two workgroups on a CU, and one's loads, LDS stores and barriers
+// then run under the other's arithmetic. v_mfma_i32_16x16x32_i8 sums over
+// 32 values, lane / 16 = k / 8; a 16-value half comes out of it when the lanes of the other half hand in zeros: those
+// lanes read their weight operand from the zero page (an address picked once, no instruction a product). 4 T results
+// a lane, 32 T accumulators: two to four waves a SIMD stay resident and hide each other's LDS and matrix latencies.
+template <int WT, int T, int CH>
+__global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
+                                                 const u32 *tiles, const u32 *n_tiles, u32 n_units, u32 slot_div,
                                                  u32 n_slots, float *y) {
+    constexpr int kSlots = 16 * T * CH, kParts = kGemmBN / kSlots, kThreads = 256 * CH;
     extern __shared__ __align__(16) uint8_t lds[];
     GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
     uint8_t *acts = lds + sizeof(GemmLds);
-    uint8_t *wts = acts + (size_t)kGemmBN * kActStride;
-    float *rs = reinterpret_cast<float *>(wts + (size_t)kGemmBM * wt_stride<WT>()); // [16][64]
+    uint8_t *wts = acts + (size_t)kSlots * kActStride;
+    uint8_t *zeros = wts + (size_t)kGemmBM * kRowStride;
+    float *rs = reinterpret_cast<float *>(zeros + kZeroPage); // [16][64]
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    const u32 g = tile_of_block(blockIdx.x, n_slabs);
-    const int row0 = (int)slab_of_block(blockIdx.x, n_slabs) * kGemmBM;
+    const u32 g = tile_of_block(blockIdx.x, n_units); // a unit: a row slab and a part of the tile
+    const u32 unit = slab_of_block(blockIdx.x, n_units);
+    const int row0 = (int)(unit / kParts) * kGemmBM, part0 = (int)(unit % kParts) * kSlots;
     const u32 count = n_tiles[0];
     if (g > count) return;
     if (g == count) { // the refused slots' rows: NaN (crates/gpu/src/gemm/grouped.rs:2283-2287)
-        const u32 refused = n_tiles[1];
+        const u32 refused = part0 == 0 ? n_tiles[1] : 0u;
         for (u32 i = tid; i < refused * kGemmBM; i += blockDim.x) {
             const u32 s = cols[n_slots - refused + i / kGemmBM];
             const int r = row0 + (int)(i % kGemmBM);
@@ -160,27 +174,33 @@ __global__ __launch_bounds__(1024 / T) void k_gemm(const uint8_t *w, int rpe, in
         return;
     }
     const u32 e = tiles[2 * g], word = tiles[2 * g + 1];
-    const int start = (int)(word & 0xffffu), len = (int)(word >> 16);
-    if (tid < kGemmBN) {
+    const int start = (int)(word & 0xffffu) + part0, len = (int)(word >> 16) - part0;
+    if (len <= 0) return; // the tile ends before this part
+    if (tid < kSlots) {
         const u32 s = cols[start + (tid < len ? tid : 0)];
         tab->slot[tid] = s;
         tab->col[tid] = s / slot_div;
     }
+    if (tid < kZeroPage / 4) reinterpret_cast<u32 *>(zeros)[tid] = 0u;
     __syncthreads();
     constexpr int kBlock = WT == BM_Q4K ? BM_Q4K_BLOCK : BM_Q6K_BLOCK;
-    constexpr int kWc = wt_chunks<WT>();
     const size_t row_bytes = (size_t)nb * kBlock;
     const int col_bytes = nb * BM_Q82_SB_EXT;
-    // staging: kGemmBN * 22 chunks of 16 bytes of activations, kGemmBM * kWc of weights, a super-block
+    // staging, a super-block: kGemmBN * 22 chunks of 16 bytes of activations; of the weights 64 rows x 8 pieces of 16
+    // code bytes (Q6_K: with the 16 bytes of high bits that go with them) and the rows' headers
     constexpr int kAc = kActSb / 16; // 22
-    constexpr int kThreads = 1024 / T; // 16 / T waves: four row groups x (4 / T) slot groups of 16 T slots
-    constexpr int kActLoads = (kGemmBN * kAc + kThreads - 1) / kThreads, kWtLoads = (kGemmBM * kWc + kThreads - 1) / kThreads;
-    uint4 ra[kActLoads], rw[kWtLoads];
+    constexpr int kActLoads = (kSlots * kAc + kThreads - 1) / kThreads, kWtLoads = (kGemmBM * 8 + kThreads - 1) / kThreads;
+    uint4 ra[kActLoads], rw[kWtLoads], rqh[kWtLoads], rhd;
+    u32 rhd2 = 0;
+    auto row_ptr = [&](int r, int i) {
+        r += row0;
+        return w + ((size_t)e * rpe + (r < rpe ? r : rpe - 1)) * row_bytes + (size_t)i * kBlock;
+    };
     auto fetch = [&](int i) {
 #pragma unroll
         for (int t = 0; t < kActLoads; t++) {
             int c = t * kThreads + tid;
-            c = c < kGemmBN * kAc ? c : kGemmBN * kAc - 1;
+            c = c < kSlots * kAc ? c : kSlots * kAc - 1;
             const int n = c / kAc, k = c % kAc;
             const uint8_t *colp = act + (size_t)tab->col[n] * col_bytes;
             const uint8_t *src = k < 18 ? colp + (size_t)i * BM_Q82_SB_REF + 16 * k
@@ -189,45 +209,78 @@ __global__ __launch_bounds__(1024 / T) void k_gemm(const uint8_t *w, int rpe, in
         }
 #pragma unroll
         for (int t = 0; t < kWtLoads; t++) {
-            int c = t * kThreads + tid;
-            c = c < kGemmBM * kWc ? c : kGemmBM * kWc - 1;
-            int r = row0 + c / kWc;
-            const int k = c % kWc;
-            r = r < rpe ? r : rpe - 1;
-            const uint8_t *blk = w + ((size_t)e * rpe + r) * row_bytes + (size_t)i * kBlock;
-            // Q6_K: 210 bytes are 13 chunks and a last one that ends with the block (bytes 194 .. 210)
-            rw[t] = bm_ld16u(blk + ((WT == BM_Q6K && k == 13) ? 194 : 16 * k));
+            const int c = (t * kThreads + tid) & (kGemmBM * 8 - 1), pc = c & 7;
+            const uint8_t *blk = row_ptr(c >> 3, i);
+            if constexpr (WT == BM_Q4K) {
+                rw[t] = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * pc);
+            } else { // half pc / 4: its ql bytes 16 (pc % 4) .. and the qh bytes that go with them
+                rw[t] = bm_ld16u(blk + 64 * (pc >> 2) + 16 * (pc & 3));
+                rqh[t] = bm_ld16u(blk + 128 + 32 * (pc >> 2) + 16 * (pc & 1));
+            }
         }
+        if (tid < kGemmBM) {
+            const uint8_t *blk = row_ptr(tid, i);
+            if constexpr (WT == BM_Q4K) {
+                rhd = *reinterpret_cast<const uint4 *>(blk);
+            } else {
+                rhd = bm_ld16u(blk + 192);
+                rhd2 = bm_ld2u(blk + 208);
+            }
+        }
+    };
+    auto put16 = [](uint8_t *dst, u32 a, u32 b, u32 c, u32 d) {
+        *reinterpret_cast<uint2 *>(dst) = make_uint2(a, b);
+        *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(c, d);
     };
     auto stash = [&]() {
 #pragma unroll
         for (int t = 0; t < kActLoads; t++) {
             const int c = t * kThreads + tid;
-            if (c < kGemmBN * kAc) {
-                uint8_t *dst = acts + (c / kAc) * kActStride + 16 * (c % kAc);
-                *reinterpret_cast<uint2 *>(dst) = make_uint2(ra[t].x, ra[t].y);
-                *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(ra[t].z, ra[t].w);
-            }
+            if (c < kSlots * kAc) put16(acts + (c / kAc) * kActStride + 16 * (c % kAc), ra[t].x, ra[t].y, ra[t].z, ra[t].w);
         }
+        const u32 ml = 0x0f0f0f0fu;
 #pragma unroll
         for (int t = 0; t < kWtLoads; t++) {
             const int c = t * kThreads + tid;
-            if (c < kGemmBM * kWc) {
-                uint8_t *dst = wts + (c / kWc) * wt_stride<WT>() + 16 * (c % kWc);
-                *reinterpret_cast<uint2 *>(dst) = make_uint2(rw[t].x, rw[t].y);
-                *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(rw[t].z, rw[t].w);
+            if (c < kGemmBM * 8) {
+                const int pc = c & 7;
+                uint8_t *codes = wts + (c >> 3) * kRowStride + kRowCodesAt;
+                if constexpr (WT == BM_Q4K) {
+                    // code bytes 16 pc ..: values 64 (pc / 2) + 16 (pc % 2) .. (low nibbles) and 32 on (high nibbles)
+                    uint8_t *dst = codes + 64 * (pc >> 1) + 16 * (pc & 1);
+                    put16(dst, rw[t].x & ml, rw[t].y & ml, rw[t].z & ml, rw[t].w & ml);
+                    put16(dst + 32, (rw[t].x >> 4) & ml, (rw[t].y >> 4) & ml, (rw[t].z >> 4) & ml, (rw[t].w >> 4) & ml);
+                } else {
+                    // low nibbles are quarter (pc % 4) / 2 of the half, high nibbles that quarter + 2; values 16 (pc % 2) ..
+#pragma unroll
+                    for (int hn = 0; hn < 2; hn++) {
+                        const int a4 = ((pc & 3) >> 1) + 2 * hn, ns = 4 * hn, hs = 2 * a4;
+                        uint8_t *dst = codes + 128 * (pc >> 2) + 32 * a4 + 16 * (pc & 1);
+                        const u32 mh = 0x03030303u;
+                        put16(dst, q6_minus_32(((rw[t].x >> ns) & ml) | (((rqh[t].x >> hs) & mh) << 4)),
+                              q6_minus_32(((rw[t].y >> ns) & ml) | (((rqh[t].y >> hs) & mh) << 4)),
+                              q6_minus_32(((rw[t].z >> ns) & ml) | (((rqh[t].z >> hs) & mh) << 4)),
+                              q6_minus_32(((rw[t].w >> ns) & ml) | (((rqh[t].w >> hs) & mh) << 4)));
+                    }
+                }
             }
         }
+        if (tid < kGemmBM) {
+            uint8_t *hd = wts + tid * kRowStride;
+            put16(hd, rhd.x, rhd.y, rhd.z, rhd.w);
+            if constexpr (WT == BM_Q6K) *reinterpret_cast<u32 *>(hd + 16) = rhd2;
+        }
     };
-    // this lane in its wave's two 16 x 16 products: operand row / slot lane % 16, values 8 * (lane / 16) .. + 8 of
-    // a 32-value block; its four results of each product are rows 4 * (lane / 16) + v of slot lane % 16
+    // this lane in its wave's 16 x 16 products: operand row / slot lane % 16, values 8 * (lane / 16) .. + 8 of a
+    // 32-value block; its four results of each product are rows 4 * (lane / 16) + v of slot lane % 16
     const int rg = wv & 3, ch = wv >> 2, l16 = lane & 15, kg = lane >> 4;
     const uint8_t *my_act[T];
 #pragma unroll
     for (int t = 0; t < T; t++) my_act[t] = acts + (16 * T * ch + 16 * t + l16) * kActStride;
-    const uint8_t *my_wt = wts + (16 * rg + l16) * wt_stride<WT>();
+    // the weight operand of half h of a block: this lane's eight codes when they are of that half, else zeros
+    const uint8_t *my_row = wts + (16 * rg + l16) * kRowStride + kRowCodesAt + 8 * kg;
+    const uint8_t *my_a[2] = {kg < 2 ? my_row : zeros, kg < 2 ? zeros : my_row};
     const int rbase = 16 * rg + 4 * kg; // result v sits in row rbase + v of the slab
-    const u32 keep[2] = {kg < 2 ? 0xffffffffu : 0u, kg < 2 ? 0u : 0xffffffffu}; // this lane's codes are of half kg / 2
     float acc[T][4][8];
 #pragma unroll
     for (int t = 0; t < T; t++)
@@ -243,14 +296,14 @@ __global__ __launch_bounds__(1024 / T) void k_gemm(const uint8_t *w, int rpe, in
         __syncthreads();
         if (i + 1 < nb) fetch(i + 1);
         // the rows' scale products: rs[s][row]
-        {
-            const int r = (tid >> 3) & 63, part = tid & 7;
-            const uint8_t *blk = wts + r * wt_stride<WT>();
-            if (tid < 512) {
+        for (int it = tid; it < 8 * kGemmBM; it += kThreads) {
+            const int r = it >> 3, part = it & 7;
+            const uint8_t *hd = wts + r * kRowStride;
+            {
                 if constexpr (WT == BM_Q4K) {
-                    const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk));
-                    const float dmin = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk + 2));
-                    const uint8_t *sc = blk + 4;
+                    const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(hd));
+                    const float dmin = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(hd + 2));
+                    const uint8_t *sc = hd + 4;
                     const int s = part; // crates/gguf/src/quant.rs:620-628 get_scale_min_k4
                     int scv, mv;
                     if (s < 4) {
@@ -263,11 +316,11 @@ __global__ __launch_bounds__(1024 / T) void k_gemm(const uint8_t *w, int rpe, in
                     rs[s * kGemmBM + r] = d * (float)scv;
                     rs[(8 + s) * kGemmBM + r] = -(dmin * (float)mv);
                 } else {
-                    const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk + 222));
+                    const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(hd + 16));
 #pragma unroll
                     for (int t = 0; t < 2; t++) {
                         const int gq = 2 * part + t;
-                        rs[gq * kGemmBM + r] = d * (float)(int)(signed char)blk[192 + gq];
+                        rs[gq * kGemmBM + r] = d * (float)(int)(signed char)hd[gq];
                     }
                 }
             }
@@ -291,73 +344,31 @@ __global__ __launch_bounds__(1024 / T) void k_gemm(const uint8_t *w, int rpe, in
                     acc[t][3][s] = fmaf(my, mn.w, acc[t][3][s]);
                 }
             }
+        }
 #pragma unroll
-            for (int p = 0; p < 4; p++) { // code bytes 32p ..: low nibbles sub-block 2p, high nibbles 2p + 1
-                const uint2 wq = *reinterpret_cast<const uint2 *>(my_wt + 16 + 32 * p + 8 * kg);
+        for (int bk = 0; bk < 8; bk++) { // 32-value block bk of the super-block: groups 2 bk (half 0) and 2 bk + 1
+            long a[2], b[T];
 #pragma unroll
-                for (int en = 0; en < 2; en++) {
-                    const int s = 2 * p + en;
-                    const u32 ax = (wq.x >> (4 * en)) & 0x0f0f0f0fu, ay = (wq.y >> (4 * en)) & 0x0f0f0f0fu;
-                    const float4 sv = *reinterpret_cast<const float4 *>(&rs[s * kGemmBM + rbase]);
-                    float f[T][4];
-                    long b[T];
+            for (int h = 0; h < 2; h++) a[h] = *reinterpret_cast<const long *>(my_a[h] + 32 * bk);
+            float d8[T];
 #pragma unroll
-                    for (int t = 0; t < T; t++) {
-                        const float d8 = pair[t][s].x;
-                        f[t][0] = sv.x * d8;
-                        f[t][1] = sv.y * d8;
-                        f[t][2] = sv.z * d8;
-                        f[t][3] = sv.w * d8;
-                        const uint2 bq = *reinterpret_cast<const uint2 *>(my_act[t] + (s >> 2) * BM_Q82X4_STRIDE + 16 +
-                                                                          32 * (s & 3) + 8 * kg);
-                        b[t] = (long)(((unsigned long long)bq.y << 32) | bq.x);
-                    }
-#pragma unroll
-                    for (int h = 0; h < 2; h++) {
-                        const long a = (long)(((unsigned long long)(ay & keep[h]) << 32) | (ax & keep[h]));
-                        const int l = 4 * h + (s & 3);
-#pragma unroll
-                        for (int t = 0; t < T; t++) {
-                            const v4i z = {0, 0, 0, 0};
-                            const v4i sum = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b[t], z, 0, 0, 0);
-#pragma unroll
-                            for (int v = 0; v < 4; v++) acc[t][v][l] = fmaf(f[t][v], (float)sum[v], acc[t][v][l]);
-                        }
-                    }
-                }
+            for (int t = 0; t < T; t++) {
+                b[t] = *reinterpret_cast<const long *>(my_act[t] + (bk >> 2) * BM_Q82X4_STRIDE + 16 + 32 * (bk & 3) + 8 * kg);
+                d8[t] = pair[t][bk].x;
             }
-        } else {
 #pragma unroll
-            for (int bk = 0; bk < 8; bk++) { // 32-block bk of the super-block: quarter bk % 4 of half bk / 4
-                const int c2 = bk >> 2, a4 = bk & 3;
-                const uint2 ql = *reinterpret_cast<const uint2 *>(my_wt + 64 * c2 + 32 * (a4 & 1) + 8 * kg);
-                const uint2 qh = *reinterpret_cast<const uint2 *>(my_wt + 128 + 32 * c2 + 8 * kg);
-                const int ns = 4 * (a4 >> 1), hs = 2 * a4;
-                const u32 ax = q6_minus_32(((ql.x >> ns) & 0x0f0f0f0fu) | (((qh.x >> hs) & 0x03030303u) << 4));
-                const u32 ay = q6_minus_32(((ql.y >> ns) & 0x0f0f0f0fu) | (((qh.y >> hs) & 0x03030303u) << 4));
-                long b[T];
-                float d8[T];
+            for (int h = 0; h < 2; h++) {
+                // Q4_K: one scale a block; Q6_K: one a group (crates/qdot/src/lib.rs:4403-4440, :4794-4809)
+                const float4 sv = *reinterpret_cast<const float4 *>(&rs[(WT == BM_Q4K ? bk : 2 * bk + h) * kGemmBM + rbase]);
+                const int l = 4 * h + (bk & 3);
 #pragma unroll
                 for (int t = 0; t < T; t++) {
-                    const uint2 bq = *reinterpret_cast<const uint2 *>(my_act[t] + (bk >> 2) * BM_Q82X4_STRIDE + 16 + 32 * (bk & 3) +
-                                                                      8 * kg);
-                    b[t] = (long)(((unsigned long long)bq.y << 32) | bq.x);
-                    d8[t] = pair[t][bk].x;
-                }
-#pragma unroll
-                for (int hh = 0; hh < 2; hh++) { // 16-value group 2 bk + hh
-                    const long a = (long)(((unsigned long long)(ay & keep[hh]) << 32) | (ax & keep[hh]));
-                    const float4 sv = *reinterpret_cast<const float4 *>(&rs[(2 * bk + hh) * kGemmBM + rbase]);
-                    const int l = 4 * hh + (bk & 3); // crates/qdot/src/lib.rs:4794-4809
-#pragma unroll
-                    for (int t = 0; t < T; t++) {
-                        const v4i z = {0, 0, 0, 0};
-                        const v4i sum = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b[t], z, 0, 0, 0);
-                        acc[t][0][l] = fmaf(sv.x * d8[t], (float)sum[0], acc[t][0][l]);
-                        acc[t][1][l] = fmaf(sv.y * d8[t], (float)sum[1], acc[t][1][l]);
-                        acc[t][2][l] = fmaf(sv.z * d8[t], (float)sum[2], acc[t][2][l]);
-                        acc[t][3][l] = fmaf(sv.w * d8[t], (float)sum[3], acc[t][3][l]);
-                    }
+                    const v4i z = {0, 0, 0, 0};
+                    const v4i sum = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[h], b[t], z, 0, 0, 0);
+                    acc[t][0][l] = fmaf(sv.x * d8[t], (float)sum[0], acc[t][0][l]);
+                    acc[t][1][l] = fmaf(sv.y * d8[t], (float)sum[1], acc[t][1][l]);
+                    acc[t][2][l] = fmaf(sv.z * d8[t], (float)sum[2], acc[t][2][l]);
+                    acc[t][3][l] = fmaf(sv.w * d8[t], (float)sum[3], acc[t][3][l]);
                 }
             }
         }
@@ -592,22 +603,26 @@ hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int
     const int nb = k / 256;
     const u32 max_tiles = (u32)gemm_max_tiles(n_slots, n_experts) + 1; // one more: the block that fills refused slots
     const u32 n_slabs = (u32)((rows_per_expert + kGemmBM - 1) / kGemmBM);
-    const unsigned grid = ((max_tiles + 7) / 8) * 8 * n_slabs;
-    auto launch = [&](auto kern, unsigned threads, size_t lds) {
+    // parts: workgroups a tile's 64 slots are shared among (each takes every row slab)
+    auto launch = [&](auto kern, unsigned threads, size_t lds, unsigned parts) {
         hipError_t e = allow_lds(kern, lds);
         if (e != hipSuccess) return e;
+        const u32 n_units = n_slabs * parts;
+        const unsigned grid = ((max_tiles + 7) / 8) * 8 * n_units;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev, n_tiles,
-                           n_slabs, (u32)slot_div, (u32)n_slots, y);
+                           n_units, (u32)slot_div, (u32)n_slots, y);
         return hipGetLastError();
     };
     if (mode == 1) {
-        if (wtype == BM_Q4K) return launch(k_gemm_fast<BM_Q4K>, 256, gemm_lds_bytes<BM_Q4K>());
-        if (wtype == BM_Q6K) return launch(k_gemm_fast<BM_Q6K>, 256, gemm_lds_bytes<BM_Q6K>());
+        if (wtype == BM_Q4K) return launch(k_gemm_fast<BM_Q4K>, 256, gemm_lds_bytes<BM_Q4K>(), 1);
+        if (wtype == BM_Q6K) return launch(k_gemm_fast<BM_Q6K>, 256, gemm_lds_bytes<BM_Q6K>(), 1);
         return hipErrorInvalidValue;
     }
-    // slot groups of 16 a wave (T): 1 -> 1024 threads a workgroup, 2 -> 512; the faster of the two for each type
-    if (wtype == BM_Q4K) return launch(k_gemm<BM_Q4K, 1>, 1024, gemm_lds_bytes<BM_Q4K>());
-    if (wtype == BM_Q6K) return launch(k_gemm<BM_Q6K, 2>, 512, gemm_lds_bytes<BM_Q6K>());
+    // 512 threads on 32 slots of a tile for both types (Q4_K 114 registers, Q6_K 121): two workgroups a CU. Measured
+    // against 1024 threads on all 64 slots (Q4_K gate 362 -> 342 us), 512 threads with two slot groups a wave on 64
+    // (Q6_K down 489 -> 407 us), and 256 threads on 16 or 32 slots (slower: the rows are staged once a workgroup).
+    if (wtype == BM_Q4K) return launch(k_gemm<BM_Q4K, 1, 2>, 512, gemm_exact_lds_bytes(32), 2);
+    if (wtype == BM_Q6K) return launch(k_gemm<BM_Q6K, 1, 2>, 512, gemm_exact_lds_bytes(32), 2);
     return hipErrorInvalidValue;
 }
 

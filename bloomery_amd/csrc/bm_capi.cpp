@@ -720,6 +720,11 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
     }
     if (act->m_cap < n_slots / slot_div)
         return fail(ctx, BM_ESHAPE, "%s: %d slots read %d activation columns, act holds %d", what, n_slots, n_slots / slot_div, act->m_cap);
+    // the kernels address the columns and an expert's rows by 32-bit offsets
+    if ((uint64_t)(n_slots / slot_div) * dev_col_bytes(act->wtype, act->k) >= (1ull << 32) ||
+        (uint64_t)rows_per_expert * (uint64_t)bm_row_bytes(w->wtype, w->k) >= (1ull << 32))
+        return fail(ctx, BM_ESHAPE, "%s: %d columns of k = %d or %d rows an expert pass 4 GiB, the kernels' offset range", what,
+                    n_slots / slot_div, act->k, rows_per_expert);
     return driver(ctx, what, bmk::gemm(launch_of(ctx), w->wtype, w->dev, route->n_experts, rows_per_expert, w->k, act->dev, route->cols,
                                        route->tiles, route->n_tiles, n_slots, slot_div, y_dev, ctx->gemm_mode));
 }

@@ -131,33 +131,45 @@ __device__ __forceinline__ u32 q6_minus_32(u32 q) {
     return t | (m << 1) | (m << 2);
 }
 
-// LDS of the exact kernel: the weight rows arrive unpacked, a signed byte a code (Q4_K 0..15, Q6_K q6 - 32), behind a
-// 24-byte header (Q4_K: d, dmin, the twelve scale bytes; Q6_K: the sixteen scales, d), so the arithmetic waves read
-// matrix operands as they are; a page of zeros stands in for the half of an operand that must not count.
-constexpr int kRowCodesAt = 24, kRowStride = kRowCodesAt + 256; // 280: off the bank period
-constexpr int kZeroPage = 256 + 32;
+// LDS of the exact kernel, two buffers of: the part's activation columns (a super-block each), the slab's 64 weight
+// rows unpacked to a signed byte a code (Q4_K 0..15, Q6_K q6 - 32), so the arithmetic reads matrix operands as they
+// are, and the rows' 16 x 64 scale products. A page of zeros stands in for the half of an operand that must not count.
+constexpr int kRowStride = 256 + 8; // off the bank period
+constexpr int kZeroPage = 256;
+__host__ __device__ constexpr size_t gemm_exact_buf_bytes(int slots) {
+    return (size_t)slots * kActStride + (size_t)kGemmBM * kRowStride + 16 * kGemmBM * sizeof(float);
+}
 __host__ __device__ constexpr size_t gemm_exact_lds_bytes(int slots) {
-    return sizeof(GemmLds) + (size_t)slots * kActStride + (size_t)kGemmBM * kRowStride + kZeroPage + 16 * kGemmBM * sizeof(float);
+    return sizeof(GemmLds) + kZeroPage + 2 * gemm_exact_buf_bytes(slots);
+}
+
+// Byte j (0..11) of the twelve scale bytes a Q4_K block holds after d and dmin, the bytes given as three words.
+__device__ __forceinline__ u32 q4k_scale_byte(u32 y, u32 z, u32 w, int j) {
+    const unsigned long long yz = ((unsigned long long)z << 32) | y;
+    const u32 a = (u32)(yz >> ((8 * j) & 63)), b = w >> ((8 * j) & 31);
+    return (j < 8 ? a : b) & 0xffu;
 }
 
 // A workgroup of 4 CH waves takes 16 T CH slots of a tile (all 64, or a part of it: a tile's parts are workgroups of
 // their own) and a slab of 64 rows. Wave w works on rows 16 * (w & 3) .. and slots 16 T * (w >> 2) ..: T 16 x 16
-// products a 16-value group. Parts of 32 slots put two workgroups on a CU, and one's loads, LDS stores and barriers
-// then run under the other's arithmetic. v_mfma_i32_16x16x32_i8 sums over
-// 32 values, lane / 16 = k / 8; a 16-value half comes out of it when the lanes of the other half hand in zeros: those
-// lanes read their weight operand from the zero page (an address picked once, no instruction a product). 4 T results
-// a lane, 32 T accumulators: two to four waves a SIMD stay resident and hide each other's LDS and matrix latencies.
+// products a 16-value group. v_mfma_i32_16x16x32_i8 sums over 32 values, lane / 16 = k / 8; a 16-value half comes out
+// of it when the lanes of the other half hand in zeros: those lanes read their weight operand from the zero page (an
+// address picked once, no instruction a product). 4 T results a lane, 32 T accumulators.
+// The next super-block is loaded to registers before the arithmetic on the present one and stored to the other
+// buffer after it: one barrier a super-block. Parts of 32 slots put two workgroups on a CU, and one's loads, LDS
+// stores and barrier then run under the other's arithmetic.
 template <int WT, int T, int CH>
 __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
                                                  const u32 *tiles, const u32 *n_tiles, u32 n_units, u32 slot_div,
                                                  u32 n_slots, float *y) {
     constexpr int kSlots = 16 * T * CH, kParts = kGemmBN / kSlots, kThreads = 256 * CH;
+    static_assert(kThreads == 8 * kGemmBM, "a thread a (row, eighth of the row's codes)");
+    constexpr size_t kBuf = gemm_exact_buf_bytes(kSlots);
+    constexpr int kWtsAt = kSlots * kActStride, kRsAt = kWtsAt + kGemmBM * kRowStride;
     extern __shared__ __align__(16) uint8_t lds[];
     GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
-    uint8_t *acts = lds + sizeof(GemmLds);
-    uint8_t *wts = acts + (size_t)kSlots * kActStride;
-    uint8_t *zeros = wts + (size_t)kGemmBM * kRowStride;
-    float *rs = reinterpret_cast<float *>(zeros + kZeroPage); // [16][64]
+    uint8_t *zeros = lds + sizeof(GemmLds);
+    uint8_t *buf0 = zeros + kZeroPage;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const u32 g = tile_of_block(blockIdx.x, n_units); // a unit: a row slab and a part of the tile
     const u32 unit = slab_of_block(blockIdx.x, n_units);
@@ -184,103 +196,103 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
     if (tid < kZeroPage / 4) reinterpret_cast<u32 *>(zeros)[tid] = 0u;
     __syncthreads();
     constexpr int kBlock = WT == BM_Q4K ? BM_Q4K_BLOCK : BM_Q6K_BLOCK;
-    const size_t row_bytes = (size_t)nb * kBlock;
-    const int col_bytes = nb * BM_Q82_SB_EXT;
-    // staging, a super-block: kGemmBN * 22 chunks of 16 bytes of activations; of the weights 64 rows x 8 pieces of 16
-    // code bytes (Q6_K: with the 16 bytes of high bits that go with them) and the rows' headers
+    const u32 row_bytes = (u32)nb * kBlock, col_bytes = (u32)nb * BM_Q82_SB_EXT;
+
+    // What a thread stages of every super-block: kActLoads 16-byte chunks of the activations (a column's super-block
+    // is 18 chunks of codes and 4 of (d8, d8 * isum) pairs), 16 code bytes of row tid / 8 (Q6_K: with the 16 bytes of
+    // high bits that go with them), and two of that row's sixteen scale products. The sources are fixed but for the
+    // super-block's offset: 32-bit offsets from the activations and from the expert's rows.
     constexpr int kAc = kActSb / 16; // 22
-    constexpr int kActLoads = (kSlots * kAc + kThreads - 1) / kThreads, kWtLoads = (kGemmBM * 8 + kThreads - 1) / kThreads;
-    uint4 ra[kActLoads], rw[kWtLoads], rqh[kWtLoads], rhd;
-    u32 rhd2 = 0;
-    auto row_ptr = [&](int r, int i) {
-        r += row0;
-        return w + ((size_t)e * rpe + (r < rpe ? r : rpe - 1)) * row_bytes + (size_t)i * kBlock;
-    };
+    constexpr int kActLoads = (kSlots * kAc + kThreads - 1) / kThreads;
+    u32 src_a[kActLoads], step_a[kActLoads]; // a chunk's offset in super-block 0 and its step a super-block
+    int dst_a[kActLoads];
+#pragma unroll
+    for (int t = 0; t < kActLoads; t++) {
+        int c = t * kThreads + tid;
+        c = c < kSlots * kAc ? c : kSlots * kAc - 1;
+        const int n = c / kAc, k = c % kAc;
+        const u32 colp = tab->col[n] * col_bytes;
+        // chunk k < 18: the codes, a step of 288 a super-block; else the pairs behind all the codes, a step of 64
+        src_a[t] = k < 18 ? colp + 16 * k : colp + (u32)nb * BM_Q82_SB_REF + 16 * (k - 18);
+        step_a[t] = k < 18 ? BM_Q82_SB_REF : 64;
+        dst_a[t] = n * kActStride + 16 * k;
+    }
+    const uint8_t *we = w + (size_t)e * rpe * row_bytes;
+    const int wr = tid >> 3, pc = tid & 7; // the row and the eighth of its codes
+    const u32 src_w = (u32)(row0 + wr < rpe ? row0 + wr : rpe - 1) * row_bytes;
+    uint4 ra[kActLoads], rw, rqh, rhd = make_uint4(0, 0, 0, 0);
     auto fetch = [&](int i) {
 #pragma unroll
-        for (int t = 0; t < kActLoads; t++) {
-            int c = t * kThreads + tid;
-            c = c < kSlots * kAc ? c : kSlots * kAc - 1;
-            const int n = c / kAc, k = c % kAc;
-            const uint8_t *colp = act + (size_t)tab->col[n] * col_bytes;
-            const uint8_t *src = k < 18 ? colp + (size_t)i * BM_Q82_SB_REF + 16 * k
-                                        : colp + (size_t)nb * BM_Q82_SB_REF + (size_t)i * 64 + 16 * (k - 18);
-            ra[t] = *reinterpret_cast<const uint4 *>(src);
-        }
-#pragma unroll
-        for (int t = 0; t < kWtLoads; t++) {
-            const int c = (t * kThreads + tid) & (kGemmBM * 8 - 1), pc = c & 7;
-            const uint8_t *blk = row_ptr(c >> 3, i);
-            if constexpr (WT == BM_Q4K) {
-                rw[t] = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * pc);
-            } else { // half pc / 4: its ql bytes 16 (pc % 4) .. and the qh bytes that go with them
-                rw[t] = bm_ld16u(blk + 64 * (pc >> 2) + 16 * (pc & 3));
-                rqh[t] = bm_ld16u(blk + 128 + 32 * (pc >> 2) + 16 * (pc & 1));
-            }
-        }
-        if (tid < kGemmBM) {
-            const uint8_t *blk = row_ptr(tid, i);
-            if constexpr (WT == BM_Q4K) {
-                rhd = *reinterpret_cast<const uint4 *>(blk);
-            } else {
-                rhd = bm_ld16u(blk + 192);
-                rhd2 = bm_ld2u(blk + 208);
-            }
+        for (int t = 0; t < kActLoads; t++) ra[t] = *reinterpret_cast<const uint4 *>(act + (src_a[t] + (u32)i * step_a[t]));
+        const uint8_t *blk = we + (src_w + (u32)i * kBlock);
+        if constexpr (WT == BM_Q4K) {
+            rw = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * pc);
+            if (pc == 0) rhd = *reinterpret_cast<const uint4 *>(blk); // d, dmin, the twelve scale bytes
+        } else { // half pc / 4: its ql bytes 16 (pc % 4) .. and the qh bytes that go with them
+            rw = bm_ld16u(blk + 64 * (pc >> 2) + 16 * (pc & 3));
+            rqh = bm_ld16u(blk + 128 + 32 * (pc >> 2) + 16 * (pc & 1));
+            rhd.x = bm_ld2u(blk + 208);          // d
+            rhd.y = bm_ld2u(blk + 192 + 2 * pc); // scales 2 pc, 2 pc + 1
         }
     };
     auto put16 = [](uint8_t *dst, u32 a, u32 b, u32 c, u32 d) {
         *reinterpret_cast<uint2 *>(dst) = make_uint2(a, b);
         *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(c, d);
     };
-    auto stash = [&]() {
+    auto stash = [&](uint8_t *buf) {
 #pragma unroll
-        for (int t = 0; t < kActLoads; t++) {
-            const int c = t * kThreads + tid;
-            if (c < kSlots * kAc) put16(acts + (c / kAc) * kActStride + 16 * (c % kAc), ra[t].x, ra[t].y, ra[t].z, ra[t].w);
-        }
+        for (int t = 0; t < kActLoads; t++)
+            if (t * kThreads + tid < kSlots * kAc) put16(buf + dst_a[t], ra[t].x, ra[t].y, ra[t].z, ra[t].w);
         const u32 ml = 0x0f0f0f0fu;
+        uint8_t *codes = buf + kWtsAt + wr * kRowStride;
+        float *rs = reinterpret_cast<float *>(buf + kRsAt); // [16][64]
+        if constexpr (WT == BM_Q4K) {
+            // code bytes 16 pc ..: values 64 (pc / 2) + 16 (pc % 2) .. (low nibbles) and 32 on (high nibbles)
+            uint8_t *dst = codes + 64 * (pc >> 1) + 16 * (pc & 1);
+            put16(dst, rw.x & ml, rw.y & ml, rw.z & ml, rw.w & ml);
+            put16(dst + 32, (rw.x >> 4) & ml, (rw.y >> 4) & ml, (rw.z >> 4) & ml, (rw.w >> 4) & ml);
+            // the row's header from the lane that read it; scale and min of sub-block pc
+            // (crates/gguf/src/quant.rs:620-628 get_scale_min_k4)
+            const int from = 4 * (lane & ~7);
+            const u32 h0 = (u32)__builtin_amdgcn_ds_bpermute(from, (int)rhd.x), h1 = (u32)__builtin_amdgcn_ds_bpermute(from, (int)rhd.y),
+                      h2 = (u32)__builtin_amdgcn_ds_bpermute(from, (int)rhd.z), h3 = (u32)__builtin_amdgcn_ds_bpermute(from, (int)rhd.w);
+            const float d = bm_half_to_f32((unsigned short)(h0 & 0xffffu));
+            const float dmin = bm_half_to_f32((unsigned short)(h0 >> 16));
+            const u32 lo = q4k_scale_byte(h1, h2, h3, pc < 4 ? pc : pc + 4);     // pc < 4: sc[pc]; else sc[pc + 4]
+            const u32 b4 = q4k_scale_byte(h1, h2, h3, pc < 4 ? pc + 4 : pc - 4); // pc < 4: sc[pc + 4]; else sc[pc - 4]
+            const u32 b0 = q4k_scale_byte(h1, h2, h3, pc);                       // sc[pc]
+            const u32 scv = pc < 4 ? (lo & 63u) : ((lo & 15u) | ((b4 >> 6) << 4));
+            const u32 mv = pc < 4 ? (b4 & 63u) : ((lo >> 4) | ((b0 >> 6) << 4));
+            rs[pc * kGemmBM + wr] = d * (float)scv;
+            rs[(8 + pc) * kGemmBM + wr] = -(dmin * (float)mv);
+        } else {
+            // low nibbles are quarter (pc % 4) / 2 of the half, high nibbles that quarter + 2; values 16 (pc % 2) ..
 #pragma unroll
-        for (int t = 0; t < kWtLoads; t++) {
-            const int c = t * kThreads + tid;
-            if (c < kGemmBM * 8) {
-                const int pc = c & 7;
-                uint8_t *codes = wts + (c >> 3) * kRowStride + kRowCodesAt;
-                if constexpr (WT == BM_Q4K) {
-                    // code bytes 16 pc ..: values 64 (pc / 2) + 16 (pc % 2) .. (low nibbles) and 32 on (high nibbles)
-                    uint8_t *dst = codes + 64 * (pc >> 1) + 16 * (pc & 1);
-                    put16(dst, rw[t].x & ml, rw[t].y & ml, rw[t].z & ml, rw[t].w & ml);
-                    put16(dst + 32, (rw[t].x >> 4) & ml, (rw[t].y >> 4) & ml, (rw[t].z >> 4) & ml, (rw[t].w >> 4) & ml);
-                } else {
-                    // low nibbles are quarter (pc % 4) / 2 of the half, high nibbles that quarter + 2; values 16 (pc % 2) ..
-#pragma unroll
-                    for (int hn = 0; hn < 2; hn++) {
-                        const int a4 = ((pc & 3) >> 1) + 2 * hn, ns = 4 * hn, hs = 2 * a4;
-                        uint8_t *dst = codes + 128 * (pc >> 2) + 32 * a4 + 16 * (pc & 1);
-                        const u32 mh = 0x03030303u;
-                        put16(dst, q6_minus_32(((rw[t].x >> ns) & ml) | (((rqh[t].x >> hs) & mh) << 4)),
-                              q6_minus_32(((rw[t].y >> ns) & ml) | (((rqh[t].y >> hs) & mh) << 4)),
-                              q6_minus_32(((rw[t].z >> ns) & ml) | (((rqh[t].z >> hs) & mh) << 4)),
-                              q6_minus_32(((rw[t].w >> ns) & ml) | (((rqh[t].w >> hs) & mh) << 4)));
-                    }
-                }
+            for (int hn = 0; hn < 2; hn++) {
+                const int a4 = ((pc & 3) >> 1) + 2 * hn, ns = 4 * hn, hs = 2 * a4;
+                uint8_t *dst = codes + 128 * (pc >> 2) + 32 * a4 + 16 * (pc & 1);
+                const u32 mh = 0x03030303u;
+                put16(dst, q6_minus_32(((rw.x >> ns) & ml) | (((rqh.x >> hs) & mh) << 4)),
+                      q6_minus_32(((rw.y >> ns) & ml) | (((rqh.y >> hs) & mh) << 4)),
+                      q6_minus_32(((rw.z >> ns) & ml) | (((rqh.z >> hs) & mh) << 4)),
+                      q6_minus_32(((rw.w >> ns) & ml) | (((rqh.w >> hs) & mh) << 4)));
             }
-        }
-        if (tid < kGemmBM) {
-            uint8_t *hd = wts + tid * kRowStride;
-            put16(hd, rhd.x, rhd.y, rhd.z, rhd.w);
-            if constexpr (WT == BM_Q6K) *reinterpret_cast<u32 *>(hd + 16) = rhd2;
+            const float d = bm_half_to_f32((unsigned short)rhd.x);
+            rs[(2 * pc) * kGemmBM + wr] = d * (float)(int)(signed char)(rhd.y & 0xffu);
+            rs[(2 * pc + 1) * kGemmBM + wr] = d * (float)(int)(signed char)(rhd.y >> 8);
         }
     };
     // this lane in its wave's 16 x 16 products: operand row / slot lane % 16, values 8 * (lane / 16) .. + 8 of a
     // 32-value block; its four results of each product are rows 4 * (lane / 16) + v of slot lane % 16
     const int rg = wv & 3, ch = wv >> 2, l16 = lane & 15, kg = lane >> 4;
-    const uint8_t *my_act[T];
+    int my_act[T];
 #pragma unroll
-    for (int t = 0; t < T; t++) my_act[t] = acts + (16 * T * ch + 16 * t + l16) * kActStride;
+    for (int t = 0; t < T; t++) my_act[t] = (16 * T * ch + 16 * t + l16) * kActStride;
     // the weight operand of half h of a block: this lane's eight codes when they are of that half, else zeros
-    const uint8_t *my_row = wts + (16 * rg + l16) * kRowStride + kRowCodesAt + 8 * kg;
-    const uint8_t *my_a[2] = {kg < 2 ? my_row : zeros, kg < 2 ? zeros : my_row};
+    // (offsets from the buffer; the zero page lies below both buffers)
+    const int my_row = kWtsAt + (16 * rg + l16) * kRowStride + 8 * kg;
     const int rbase = 16 * rg + 4 * kg; // result v sits in row rbase + v of the slab
+    const bool live = 16 * T * ch < len; // else none of this wave's slots is real
     float acc[T][4][8];
 #pragma unroll
     for (int t = 0; t < T; t++)
@@ -289,47 +301,12 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
 #pragma unroll
             for (int l = 0; l < 8; l++) acc[t][v][l] = 0.0f;
 
-    fetch(0);
-    for (int i = 0; i < nb; i++) {
-        __syncthreads(); // the previous super-block's readers are done
-        stash();
-        __syncthreads();
-        if (i + 1 < nb) fetch(i + 1);
-        // the rows' scale products: rs[s][row]
-        for (int it = tid; it < 8 * kGemmBM; it += kThreads) {
-            const int r = it >> 3, part = it & 7;
-            const uint8_t *hd = wts + r * kRowStride;
-            {
-                if constexpr (WT == BM_Q4K) {
-                    const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(hd));
-                    const float dmin = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(hd + 2));
-                    const uint8_t *sc = hd + 4;
-                    const int s = part; // crates/gguf/src/quant.rs:620-628 get_scale_min_k4
-                    int scv, mv;
-                    if (s < 4) {
-                        scv = sc[s] & 63;
-                        mv = sc[s + 4] & 63;
-                    } else {
-                        scv = (sc[s + 4] & 15) | ((sc[s - 4] >> 6) << 4);
-                        mv = (sc[s + 4] >> 4) | ((sc[s] >> 6) << 4);
-                    }
-                    rs[s * kGemmBM + r] = d * (float)scv;
-                    rs[(8 + s) * kGemmBM + r] = -(dmin * (float)mv);
-                } else {
-                    const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(hd + 16));
-#pragma unroll
-                    for (int t = 0; t < 2; t++) {
-                        const int gq = 2 * part + t;
-                        rs[gq * kGemmBM + r] = d * (float)(int)(signed char)hd[gq];
-                    }
-                }
-            }
-        }
-        __syncthreads();
-        if (16 * T * ch >= len) continue; // none of this wave's slots is real (the barriers above are the loop's only ones)
+    auto arithmetic = [&](const uint8_t *buf) __attribute__((always_inline)) {
+        const float *rs = reinterpret_cast<const float *>(buf + kRsAt);
+        const uint8_t *my_a[2] = {kg < 2 ? buf + my_row : zeros, kg < 2 ? zeros : buf + my_row};
         const float2 *pair[T]; // (d8, d8 * isum) a 32-block
 #pragma unroll
-        for (int t = 0; t < T; t++) pair[t] = reinterpret_cast<const float2 *>(my_act[t] + BM_Q82_SB_REF);
+        for (int t = 0; t < T; t++) pair[t] = reinterpret_cast<const float2 *>(buf + my_act[t] + BM_Q82_SB_REF);
         if constexpr (WT == BM_Q4K) {
             // the min terms first: accumulator l takes sub-block l's (crates/qdot/src/lib.rs:4389-4394)
 #pragma unroll
@@ -353,7 +330,7 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
             float d8[T];
 #pragma unroll
             for (int t = 0; t < T; t++) {
-                b[t] = *reinterpret_cast<const long *>(my_act[t] + (bk >> 2) * BM_Q82X4_STRIDE + 16 + 32 * (bk & 3) + 8 * kg);
+                b[t] = *reinterpret_cast<const long *>(buf + my_act[t] + (bk >> 2) * BM_Q82X4_STRIDE + 16 + 32 * (bk & 3) + 8 * kg);
                 d8[t] = pair[t][bk].x;
             }
 #pragma unroll
@@ -372,6 +349,18 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
                 }
             }
         }
+    };
+
+    fetch(0);
+    stash(buf0);
+    __syncthreads();
+    for (int i = 0; i < nb; i++) {
+        const bool more = i + 1 < nb;
+        if (more) fetch(i + 1);
+        if (live) arithmetic(buf0 + (size_t)(i & 1) * kBuf);
+        // the other buffer's last readers passed the barrier that ended the super-block before this one
+        if (more) stash(buf0 + (size_t)((i + 1) & 1) * kBuf);
+        __syncthreads();
     }
     // the closing sum of the eight lanes (crates/qdot/src/lib.rs:4128 hsum_float_8's order) and the store
 #pragma unroll

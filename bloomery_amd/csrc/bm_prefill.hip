@@ -134,10 +134,16 @@ __device__ __forceinline__ u32 q6_minus_32(u32 q) {
 // LDS of the exact kernel, two buffers of: the part's activation columns (a super-block each), the slab's 64 weight
 // rows unpacked to a signed byte a code (Q4_K 0..15, Q6_K q6 - 32), so the arithmetic reads matrix operands as they
 // are, and the rows' 16 x 64 scale products. A page of zeros stands in for the half of an operand that must not count.
-constexpr int kRowStride = 256 + 8; // off the bank period
+// Strides: an operand read is 8 bytes a lane, served sixteen lanes at a time, the sixteen a wave's rows (or slots) at
+// one piece of a block: a stride of 8 x an odd number puts them on sixteen different bank pairs (rows 8 x 33, columns
+// 8 x 45). Strides of 16-byte multiples, which would let the staging store 16 bytes a lane, measured slower: the reads
+// then collide in pairs.
+constexpr int kRowStride = 256 + 8;
+constexpr int kColStride = kActStride; // 360
+constexpr int kRsStride = 68; // floats a row of the 16 x 64 scale products
 constexpr int kZeroPage = 256;
 __host__ __device__ constexpr size_t gemm_exact_buf_bytes(int slots) {
-    return (size_t)slots * kActStride + (size_t)kGemmBM * kRowStride + 16 * kGemmBM * sizeof(float);
+    return (size_t)slots * kColStride + (size_t)kGemmBM * kRowStride + 16 * kRsStride * sizeof(float);
 }
 __host__ __device__ constexpr size_t gemm_exact_lds_bytes(int slots) {
     return sizeof(GemmLds) + kZeroPage + 2 * gemm_exact_buf_bytes(slots);
@@ -165,7 +171,7 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
     constexpr int kSlots = 16 * T * CH, kParts = kGemmBN / kSlots, kThreads = 256 * CH;
     static_assert(kThreads == 8 * kGemmBM, "a thread a (row, eighth of the row's codes)");
     constexpr size_t kBuf = gemm_exact_buf_bytes(kSlots);
-    constexpr int kWtsAt = kSlots * kActStride, kRsAt = kWtsAt + kGemmBM * kRowStride;
+    constexpr int kWtsAt = kSlots * kColStride, kRsAt = kWtsAt + kGemmBM * kRowStride;
     extern __shared__ __align__(16) uint8_t lds[];
     GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
     uint8_t *zeros = lds + sizeof(GemmLds);
@@ -215,7 +221,7 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
         // chunk k < 18: the codes, a step of 288 a super-block; else the pairs behind all the codes, a step of 64
         src_a[t] = k < 18 ? colp + 16 * k : colp + (u32)nb * BM_Q82_SB_REF + 16 * (k - 18);
         step_a[t] = k < 18 ? BM_Q82_SB_REF : 64;
-        dst_a[t] = n * kActStride + 16 * k;
+        dst_a[t] = n * kColStride + 16 * k;
     }
     const uint8_t *we = w + (size_t)e * rpe * row_bytes;
     const int wr = tid >> 3, pc = tid & 7; // the row and the eighth of its codes
@@ -245,7 +251,7 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
             if (t * kThreads + tid < kSlots * kAc) put16(buf + dst_a[t], ra[t].x, ra[t].y, ra[t].z, ra[t].w);
         const u32 ml = 0x0f0f0f0fu;
         uint8_t *codes = buf + kWtsAt + wr * kRowStride;
-        float *rs = reinterpret_cast<float *>(buf + kRsAt); // [16][64]
+        float *rs = reinterpret_cast<float *>(buf + kRsAt); // [16][kRsStride]
         if constexpr (WT == BM_Q4K) {
             // code bytes 16 pc ..: values 64 (pc / 2) + 16 (pc % 2) .. (low nibbles) and 32 on (high nibbles)
             uint8_t *dst = codes + 64 * (pc >> 1) + 16 * (pc & 1);
@@ -263,8 +269,8 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
             const u32 b0 = q4k_scale_byte(h1, h2, h3, pc);                       // sc[pc]
             const u32 scv = pc < 4 ? (lo & 63u) : ((lo & 15u) | ((b4 >> 6) << 4));
             const u32 mv = pc < 4 ? (b4 & 63u) : ((lo >> 4) | ((b0 >> 6) << 4));
-            rs[pc * kGemmBM + wr] = d * (float)scv;
-            rs[(8 + pc) * kGemmBM + wr] = -(dmin * (float)mv);
+            rs[pc * kRsStride + wr] = d * (float)scv;
+            rs[(8 + pc) * kRsStride + wr] = -(dmin * (float)mv);
         } else {
             // low nibbles are quarter (pc % 4) / 2 of the half, high nibbles that quarter + 2; values 16 (pc % 2) ..
 #pragma unroll
@@ -278,8 +284,8 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
                       q6_minus_32(((rw.w >> ns) & ml) | (((rqh.w >> hs) & mh) << 4)));
             }
             const float d = bm_half_to_f32((unsigned short)rhd.x);
-            rs[(2 * pc) * kGemmBM + wr] = d * (float)(int)(signed char)(rhd.y & 0xffu);
-            rs[(2 * pc + 1) * kGemmBM + wr] = d * (float)(int)(signed char)(rhd.y >> 8);
+            rs[(2 * pc) * kRsStride + wr] = d * (float)(int)(signed char)(rhd.y & 0xffu);
+            rs[(2 * pc + 1) * kRsStride + wr] = d * (float)(int)(signed char)(rhd.y >> 8);
         }
     };
     // this lane in its wave's 16 x 16 products: operand row / slot lane % 16, values 8 * (lane / 16) .. + 8 of a
@@ -287,7 +293,7 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
     const int rg = wv & 3, ch = wv >> 2, l16 = lane & 15, kg = lane >> 4;
     int my_act[T];
 #pragma unroll
-    for (int t = 0; t < T; t++) my_act[t] = (16 * T * ch + 16 * t + l16) * kActStride;
+    for (int t = 0; t < T; t++) my_act[t] = (16 * T * ch + 16 * t + l16) * kColStride;
     // the weight operand of half h of a block: this lane's eight codes when they are of that half, else zeros
     // (offsets from the buffer; the zero page lies below both buffers)
     const int my_row = kWtsAt + (16 * rg + l16) * kRowStride + 8 * kg;
@@ -311,7 +317,7 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
             // the min terms first: accumulator l takes sub-block l's (crates/qdot/src/lib.rs:4389-4394)
 #pragma unroll
             for (int s = 0; s < 8; s++) {
-                const float4 mn = *reinterpret_cast<const float4 *>(&rs[(8 + s) * kGemmBM + rbase]);
+                const float4 mn = *reinterpret_cast<const float4 *>(&rs[(8 + s) * kRsStride + rbase]);
 #pragma unroll
                 for (int t = 0; t < T; t++) {
                     const float my = pair[t][s].y;
@@ -336,7 +342,7 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
 #pragma unroll
             for (int h = 0; h < 2; h++) {
                 // Q4_K: one scale a block; Q6_K: one a group (crates/qdot/src/lib.rs:4403-4440, :4794-4809)
-                const float4 sv = *reinterpret_cast<const float4 *>(&rs[(WT == BM_Q4K ? bk : 2 * bk + h) * kGemmBM + rbase]);
+                const float4 sv = *reinterpret_cast<const float4 *>(&rs[(WT == BM_Q4K ? bk : 2 * bk + h) * kRsStride + rbase]);
                 const int l = 4 * h + (bk & 3);
 #pragma unroll
                 for (int t = 0; t < T; t++) {

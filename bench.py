@@ -347,7 +347,7 @@ def bench_dsv3(args, bm, ora, threads):
     act, act6 = gpu.act(bm.IQ2_XXS, hidden, m), gpu.act(bm.Q6_K, hidden, m)
     act_h, act_sh = gpu.act(bm.IQ2_XXS, ff, n_slots), gpu.act(bm.Q6_K, ff, m)
     h, down = gpu.buffer(np.float32, n_slots * ff), gpu.buffer(np.float32, n_slots * hidden)
-    sdown, yr = gpu.buffer(np.float32, m * hidden), gpu.buffer(np.float32, m * hidden)
+    sdown = gpu.buffer(np.float32, m * hidden)
     y = gpu.buffer(np.float32, m * sets * hidden)
     order, start = gpu.buffer(np.uint32, n_slots), gpu.buffer(np.uint32, n_experts + 1)
     tiles = gpu.buffer(np.uint32, gpu.tile_cap(n_slots, n_experts) + 1)
@@ -367,16 +367,15 @@ def bench_dsv3(args, bm, ora, threads):
             gpu.enqueue_gate_up(dsg, dsu, act6, zeros, m, ff, 1, None, act_sh)
             gpu.enqueue_gemv_sel(dsd, act_sh, zeros, m, hidden, sdown)
         if "combine" in which:
-            gpu.enqueue_combine_tokens(down, wt.ptr + 4 * st * n_slots, None, hidden, TOP_K, m, yr)
-            gpu.enqueue_combine_tokens(sdown, ones, yr, hidden, 1, m, y.ptr + 4 * st * m * hidden)
+            gpu.enqueue_moe_combine(down, wt.ptr + 4 * st * n_slots, sdown, None, hidden, TOP_K, m, y.ptr + 4 * st * m * hidden)
 
     step(0)
     types = (ora.IQ2_XXS, ora.IQ2_XXS, ora.IQ2_XXS)
     routed = ora.moe_forward(hidden, ff, n_experts, types, wg, wu, wd, x[:m], ids[:m], wts[:m], TOP_K, n_threads=threads)
     shared = ora.moe_forward(hidden, ff, 1, (ora.Q6_K, ora.Q6_K, ora.Q6_K), sg, su, sd, x[:m], np.zeros((m, 1), np.uint32),
                              np.ones((m, 1), np.float32), 1, n_threads=threads)
-    want = ora.combine_tokens(np.asarray(shared).reshape(-1), np.ones(m, np.float32), np.asarray(routed).reshape(-1), hidden, 1,
-                              m).reshape(m, hidden)
+    # (routed sum + shared expert), the reference's grouping (crates/gpu/src/moe_fused.rs:129-170)
+    want = (np.asarray(routed, np.float32).reshape(m, hidden) + np.asarray(shared, np.float32).reshape(m, hidden)).astype(np.float32)
     parity = parity_of(y.download()[:m * hidden].reshape(m, hidden), want)
     wall, ev, steps, warm = timed_graph(gpu, step, 16, min(args.steps, 256), min(args.warmup, 32))
     kernel_us = {k: timed_graph(gpu, lambda i, k=k: step(i, (k,)), 16, 64, 16)[1] * 1e3 for k in ("routed", "shared", "combine")}

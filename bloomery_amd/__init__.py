@@ -79,6 +79,7 @@ SYMBOLS = {
     "bm_route_read": (_i, [_vp, _vp, _vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
     "bm_gemm": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp]),
     "bm_swiglu_quant": (_i, [_vp, _vp, _vp, _i, _vp]),
+    "bm_moe_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_set_gate_rule": (_i, [_vp, _i, C.c_float]),
     "bm_route_softmax": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "bm_gguf_open": (_i, [C.c_char_p, C.POINTER(_vp)]),
@@ -449,6 +450,11 @@ class Gpu:
 
     def enqueue_combine_tokens(self, down, w, resid, rows, n_slots, m, y):
         self._check(self.lib.bm_combine_tokens(self.ctx, _ptr(down), _ptr(w), _ptr(resid), rows, n_slots, m, _ptr(y)))
+
+    def enqueue_moe_combine(self, down, w, shexp, resid, rows, n_slots, m, y):
+        """moe_combine (crates/gpu/src/moe_fused.rs:129-170): (slot sum + shared expert) + residual."""
+        self._check(self.lib.bm_moe_combine(self.ctx, _ptr(down), _ptr(w), _ptr(shexp), _ptr(resid) if resid is not None else None,
+                                            rows, n_slots, m, _ptr(y)))
 
     def enqueue_down_combine(self, w, act, sel, wts, resid, n_slots_per_token, m, rows_per_expert, y):
         self._check(self.lib.bm_down_combine(self.ctx, w.handle, act.handle, _ptr(sel), _ptr(wts), _ptr(resid),

@@ -417,7 +417,16 @@ int bm_combine_tokens(bm_ctx *ctx, const float *down_dev, const float *w_dev, co
     if (!ctx || !down_dev || !w_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
     if (rows < 1 || n_slots < 1 || m < 1)
         return fail(ctx, BM_ESHAPE, "%s: rows %d, n_slots %d and m %d must all be positive", what, rows, n_slots, m);
-    return driver(ctx, what, bmk::combine_tokens(launch_of(ctx), down_dev, w_dev, resid_dev, rows, n_slots, m, y_dev));
+    return driver(ctx, what, bmk::combine_tokens(launch_of(ctx), down_dev, w_dev, nullptr, resid_dev, rows, n_slots, m, y_dev));
+}
+
+int bm_moe_combine(bm_ctx *ctx, const float *down_dev, const float *w_dev, const float *shexp_dev, const float *resid_dev,
+                   int rows, int n_slots, int m, float *y_dev) {
+    const char *what = "bm_moe_combine";
+    if (!ctx || !down_dev || !w_dev || !shexp_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (rows < 1 || n_slots < 1 || m < 1)
+        return fail(ctx, BM_ESHAPE, "%s: rows %d, n_slots %d and m %d must all be positive", what, rows, n_slots, m);
+    return driver(ctx, what, bmk::combine_tokens(launch_of(ctx), down_dev, w_dev, shexp_dev, resid_dev, rows, n_slots, m, y_dev));
 }
 
 int bm_down_combine(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const uint32_t *sel_dev,

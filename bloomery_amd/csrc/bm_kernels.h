@@ -51,8 +51,8 @@ hipError_t gate_up(const Launch &L, int wtype, const uint8_t *wg, const uint8_t 
 hipError_t gemv_sel(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const uint8_t *act,
                     const uint32_t *sel, int n_slots, int rows_per_expert, float *y);
 
-hipError_t combine_tokens(const Launch &L, const float *down, const float *w, const float *resid, int rows,
-                          int n_slots, int m, float *y);
+hipError_t combine_tokens(const Launch &L, const float *down, const float *w, const float *shexp, const float *resid,
+                          int rows, int n_slots, int m, float *y);
 
 // Slots a token may have in the fused down + combine launch.
 constexpr int kMaxCombineSlots = 64;

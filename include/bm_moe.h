@@ -150,6 +150,11 @@ int bm_gemv_sel(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const uint3
  * + d], acc)) + resid[t * rows + d] for t < m. resid_dev may be NULL (no residual add). */
 int bm_combine_tokens(bm_ctx *ctx, const float *down_dev, const float *w_dev, const float *resid_dev, int rows,
                       int n_slots, int m, float *y_dev);
+/* The combine of a layer with a shared expert, MoeFusedKernels' moe_combine (crates/gpu/src/moe_fused.rs:129-170), for m
+ * tokens: y[t * rows + d] = (the slot sum above + shexp[t * rows + d]) + resid[t * rows + d], the two adds grouped as
+ * the reference groups them (f32 addition is not associative). resid_dev may be NULL. */
+int bm_moe_combine(bm_ctx *ctx, const float *down_dev, const float *w_dev, const float *shexp_dev, const float *resid_dev,
+                   int rows, int n_slots, int m, float *y_dev);
 
 /* bm_gemv_sel and bm_combine_tokens in one launch (no counterpart launch in the reference, which keeps the two
  * apart: dispatch.rs:1346-1424): the slot values never reach memory. Same values as the two calls: every slot

@@ -66,6 +66,8 @@ int ora_gate_rule(int rule, float limit, const float *gate, const float *up, int
 int ora_route_softmax_topk(const float *logits, int n_experts, int top_k, int renorm, uint32_t *ids, float *w);
 void ora_combine_tokens(const float *down, const float *w, const float *resid, int rows, int n_slots, int m,
                         float *y);
+void ora_moe_combine(const float *down, const float *w, const float *shexp, const float *resid, int rows, int n_slots,
+                     int m, float *y);
 
 // Weight quantizers (offline, host).
 int ora_quantize_row_q4k(const float *x, int k, uint8_t *out);

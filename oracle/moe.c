@@ -61,6 +61,20 @@ void ora_combine_tokens(const float *down, const float *w, const float *resid, i
         }
 }
 
+// y[t][d] = (the slot sum above + shexp[t][d]) + resid[t][d], the adds grouped as crates/gpu/src/moe_fused.rs:129-170
+// groups them. `resid` may be NULL.
+void ora_moe_combine(const float *down, const float *w, const float *shexp, const float *resid, int rows, int n_slots,
+                     int m, float *y) {
+    for (int t = 0; t < m; t++)
+        for (int d = 0; d < rows; d++) {
+            float acc = 0.0f;
+            for (int e = 0; e < n_slots; e++)
+                acc = fmaf(w[t * n_slots + e], down[((size_t)(t * n_slots + e)) * rows + d], acc);
+            acc = acc + shexp[(size_t)t * rows + d];
+            y[(size_t)t * rows + d] = resid ? acc + resid[(size_t)t * rows + d] : acc;
+        }
+}
+
 typedef struct {
     int wtype, k, r0, r1, m;
     const uint8_t *w;         // expert's rows

@@ -55,6 +55,7 @@ def _load():
         "ora_gate_rule": (C.c_int, [C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
         "ora_route_softmax_topk": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
         "ora_combine_tokens": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
+        "ora_moe_combine": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
         "ora_quantize_row_q4k": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
         "ora_quantize_row_q6k": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
         "ora_quantize_row_iq2xxs": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
@@ -226,6 +227,14 @@ def combine_tokens(down, w, resid, rows, n_slots, m):
     y = np.empty(rows * m, np.float32)
     rp = _p(_f32(resid)) if resid is not None else None
     lib.ora_combine_tokens(_p(down), _p(w), rp, rows, n_slots, m, _p(y))
+    return y
+
+
+def moe_combine(down, w, shexp, resid, rows, n_slots, m):
+    down, w, shexp = _f32(down), _f32(w), _f32(shexp)
+    y = np.empty(rows * m, np.float32)
+    rp = _p(_f32(resid)) if resid is not None else None
+    lib.ora_moe_combine(_p(down), _p(w), _p(shexp), rp, rows, n_slots, m, _p(y))
     return y
 
 

@@ -669,7 +669,19 @@ def test_combine_adds_the_residual(gpu):
     assert_f32(y.download(), ora.combine_tokens(down, w, resid, rows, n_slots, m), "combine + resid")
     gpu.enqueue_combine_tokens(dd, dw, None, rows, n_slots, m, y)
     assert_f32(y.download(), ora.combine_tokens(down, w, None, rows, n_slots, m), "combine")
-    for b in (dd, dw, dr, y):
+    # with a shared expert's rows (crates/gpu/src/moe_fused.rs:129-170): (sum + shexp) + resid, values chosen so that
+    # the other grouping rounds differently
+    shexp = (normal_f32(rng, m * rows) * np.float32(1e4)).astype(np.float32)
+    big = (-shexp + normal_f32(rng, m * rows) * np.float32(1e-3)).astype(np.float32)
+    ds, db = gpu.upload(shexp), gpu.upload(big)
+    gpu.enqueue_moe_combine(dd, dw, ds, db, rows, n_slots, m, y)
+    want = ora.moe_combine(down, w, shexp, big, rows, n_slots, m)
+    assert_f32(y.download(), want, "moe_combine")
+    other = ora.combine_tokens(down, w, (shexp + big).astype(np.float32), rows, n_slots, m)  # sum + (shexp + resid)
+    assert np.count_nonzero(want != other) > rows  # the grouping matters on these values
+    gpu.enqueue_moe_combine(dd, dw, ds, None, rows, n_slots, m, y)
+    assert_f32(y.download(), ora.moe_combine(down, w, shexp, None, rows, n_slots, m), "moe_combine without resid")
+    for b in (dd, dw, dr, y, ds, db):
         b.free()
 
 

@@ -160,6 +160,16 @@ def test_combine_is_slot_ascending_fma_then_residual():
             assert got[t * rows + r].tobytes() == want.tobytes()
     assert np.array_equal(ora.combine_tokens(down, w, None, rows, n_slots, m),
                           ora.combine_tokens(down, w, np.zeros(m * rows, np.float32), rows, n_slots, m))
+    # with a shared expert (crates/gpu/src/moe_fused.rs:129-170): (sum + shexp) + resid, not sum + (shexp + resid)
+    one = np.ones(1, np.float32)
+    got = ora.moe_combine(np.array([1e8], np.float32), one, np.array([-1e8], np.float32), one, 1, 1, 1)
+    assert got[0] == 1.0  # the other grouping gives 1e8 + (-1e8 + 1) = 0
+    got = ora.moe_combine(np.array([3.0], np.float32), np.array([0.5], np.float32), np.array([2.0], np.float32), None, 1, 1, 1)
+    assert got[0] == 3.5
+    sh = normal_f32(rng, m * rows)
+    full = ora.moe_combine(down, w, sh, resid, rows, n_slots, m)
+    base = ora.combine_tokens(down, w, None, rows, n_slots, m)
+    assert np.array_equal(full, ((base + sh).astype(np.float32) + resid).astype(np.float32))
 
 
 # ---------------------------------------------------------------------------------------------- weight quantizers

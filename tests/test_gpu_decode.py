@@ -399,6 +399,30 @@ def test_single_launch_step_matches_the_chain_and_the_oracle(gpu, types, hidden,
     L.free()
 
 
+def test_fused_step_at_the_token_limit(gpu):
+    """bm_moe_decode takes 1..=1024 tokens a launch: the limit itself against the oracle, one more refused by name."""
+    L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), 256, 256, 9, 650)
+    rng = np.random.default_rng(651)
+    m, top_k = 1024, 2
+    x = normal_f32(rng, (m, L.hidden))
+    ids, wts = route(rng, m, L.n_experts, top_k)
+    gpu.fault_clear()
+    y, h, _, _ = run_single_launch(gpu, L, x, ids, wts, top_k, plan=bm.PLAN_TWO_LAUNCHES)
+    want_y, want_h = L.oracle(x, ids, wts, top_k)
+    assert_f32(h, want_h, "h")
+    assert_f32(y, want_y, "y")
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    xd, sel, wd = gpu.upload(np.zeros((m + 1, L.hidden), np.float32)), gpu.upload(np.zeros((m + 1, top_k), np.uint32)), \
+        gpu.upload(np.zeros((m + 1, top_k), np.float32))
+    act_h, yb = gpu.act(L.types[2], L.ff, (m + 1) * top_k), gpu.buffer(np.float32, (m + 1) * L.hidden)
+    with pytest.raises(bm.GpuError) as e:
+        gpu.enqueue_moe_decode(L.dg, L.du, L.dd, xd, sel, wd, None, top_k, m + 1, act_h, yb)
+    assert e.value.code == bm.ESHAPE and "1025" in str(e.value)
+    for b in (xd, sel, wd, act_h, yb):
+        b.free()
+    L.free()
+
+
 @pytest.mark.parametrize("plan", (bm.PLAN_ONE_LAUNCH, bm.PLAN_TWO_LAUNCHES))
 def test_single_launch_refused_ids_and_host_slots(gpu, plan):
     L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 4, 700)

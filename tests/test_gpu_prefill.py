@@ -189,3 +189,39 @@ def test_prefill_refusals_are_named(gpu):
         assert e.value.code == code and word in str(e.value), str(e.value)
     for b in (w4, wi, a512, aq8k, buf, ids, table):
         b.free()
+
+
+def test_gemm_at_the_largest_route(gpu):
+    """The route's limits (crates/gpu/src/gemm/mod.rs:97-101): 40960 slots over 1024 experts, one column a slot, with
+    runs from empty to many tiles; every slot's 16 rows against the one-column dot, and the table by definition."""
+    from test_gpu_decode import random_blocks
+    n_experts, n_slots, rpe, k = 1024, 40960, 16, 256
+    rng = np.random.default_rng(2600)
+    w = random_blocks(bm.Q4_K, n_experts * rpe, k, rng)
+    p = 1.0 / np.arange(1, n_experts + 1) ** 1.3     # skewed: the first experts own thousands of slots, the last none
+    ids = rng.choice(n_experts, n_slots, p=p / p.sum()).astype(np.uint32)
+    x = normal_f32(rng, (n_slots, k))
+    dw, act = gpu.weights(bm.Q4_K, n_experts * rpe, k, w), gpu.act(bm.Q4_K, k, n_slots)
+    xd, sel = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32)
+    table = gpu.route(n_slots, n_experts)
+    y = gpu.buffer(np.float32, n_slots * rpe).fill_bytes(0xFF)
+    gpu.fault_clear()
+    gpu.enqueue_quantize(xd, n_slots, act)
+    table.fill(sel, n_slots)
+    gpu.enqueue_gemm(dw, rpe, act, table, 0, y)
+    got = y.download().reshape(n_slots, rpe)
+    cols, tiles, refused = table.read()
+    want_cols, want_tiles, want_refused = ora.gemm_route(ids, n_experts)
+    assert refused == want_refused == 0 and np.array_equal(cols, want_cols) and np.array_equal(tiles, want_tiles)
+    assert len(np.unique(ids)) < n_experts and np.bincount(ids).max() > 64 * 20
+    rb = ora.row_bytes(bm.Q4_K, k)
+    for s in np.concatenate([np.arange(0, n_slots, 97), [n_slots - 1]]):
+        e = int(ids[s])
+        want = ora.gemv(bm.Q4_K, w[e * rpe * rb:(e + 1) * rpe * rb], rpe, k, ora.quantize_col(bm.Q4_K, x[s]), 1)
+        assert_f32(got[s], want, f"slot {s}")
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    with pytest.raises(bm.GpuError) as e:
+        gpu.route(n_slots + 1, n_experts)
+    assert e.value.code == bm.ESHAPE and "max_slots" in str(e.value)
+    for b in (dw, act, xd, sel, table, y):
+        b.free()

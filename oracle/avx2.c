@@ -156,7 +156,7 @@ int ora_avx2_quantize_q8k(const float *x, int k, uint8_t *out) {
 }
 
 int ora_avx2_quantize_col(int wtype, const float *x, int k, uint8_t *out) {
-    if (wtype == ORA_TYPE_Q4_K || wtype == ORA_TYPE_Q6_K) return ora_avx2_quantize_q82x4(x, k, out);
+    if (wtype == ORA_TYPE_Q4_K || wtype == ORA_TYPE_Q5_K || wtype == ORA_TYPE_Q6_K) return ora_avx2_quantize_q82x4(x, k, out);
     if (wtype == ORA_TYPE_IQ2_XXS) return ora_avx2_quantize_q8k(x, k, out);
     return ORA_ETYPE;
 }
@@ -202,17 +202,21 @@ static inline void q4_unpack_scales(const uint8_t *s12, uint32_t utmp[4]) {
 // -------------------------------------------------------------------------------------------------- Q4_K tile
 
 // One Q4_K row against C <= 8 columns, each column the one-column kernel's steps
-// (crates/qdot/src/lib.rs:4203-4272): weights unpacked once per block.
-static void dot_q4k_tile(const uint8_t *wrow, const uint8_t *const *acols, int C, int nb, float *out) {
-    const __m256i ml = _mm256_set1_epi8(0xF);
+// (crates/qdot/src/lib.rs:4203-4272): weights unpacked once per block. With `q5` a Q5_K row, the twin kernel
+// (:4895-4990): the wider block, the codes at 48, and bit 4 of each code folded in from the 32 high bytes at 16 (in
+// half j, value 128 j + 32 b + l takes bit 4 j + b of qh[l]: qh at j = 0, qh >> 4 in 16-bit lanes at j = 1, shifted
+// left by 4 - b onto bit 4).
+static void dot_q45k_tile(const uint8_t *wrow, const uint8_t *const *acols, int C, int nb, int q5, float *out) {
+    const __m256i ml = _mm256_set1_epi8(0xF), mh = _mm256_set1_epi8(0x10);
+    const int block = q5 ? ORA_Q5K_BLOCK : ORA_Q4K_BLOCK, codes_at = q5 ? 48 : 16;
     __m256 accd[8];
     for (int c = 0; c < C; c++) accd[c] = _mm256_setzero_ps();
     for (int i = 0; i < nb; i++) {
-        const uint8_t *wb = wrow + (size_t)i * ORA_Q4K_BLOCK;
-        uint16_t dh, mh;
+        const uint8_t *wb = wrow + (size_t)i * block;
+        uint16_t dh, mnh;
         memcpy(&dh, wb, 2);
-        memcpy(&mh, wb + 2, 2);
-        float d = f16c_to_f32(dh), dmin = f16c_to_f32(mh);
+        memcpy(&mnh, wb + 2, 2);
+        float d = f16c_to_f32(dh), dmin = f16c_to_f32(mnh);
         uint32_t utmp[4];
         q4_unpack_scales(wb + 4, utmp);
         __m256 mins_v = _mm256_cvtepi32_ps(_mm256_cvtepu8_epi32(_mm_loadl_epi64((const __m128i *)(utmp + 2))));
@@ -223,12 +227,20 @@ static void dot_q4k_tile(const uint8_t *wrow, const uint8_t *const *acols, int C
         __m256 scales[2] = {_mm256_set_m128(lo, lo), _mm256_set_m128(hi, hi)};
         __m256i values[2][4];
         for (int j = 0; j < 2; j++) {
-            __m256i bits0 = _mm256_loadu_si256((const __m256i *)(wb + 16 + 64 * j));
-            __m256i bits1 = _mm256_loadu_si256((const __m256i *)(wb + 16 + 64 * j + 32));
+            __m256i bits0 = _mm256_loadu_si256((const __m256i *)(wb + codes_at + 64 * j));
+            __m256i bits1 = _mm256_loadu_si256((const __m256i *)(wb + codes_at + 64 * j + 32));
             values[j][0] = _mm256_and_si256(bits0, ml);
             values[j][1] = _mm256_and_si256(_mm256_srli_epi16(bits0, 4), ml);
             values[j][2] = _mm256_and_si256(bits1, ml);
             values[j][3] = _mm256_and_si256(_mm256_srli_epi16(bits1, 4), ml);
+            if (q5) {
+                __m256i qh = _mm256_loadu_si256((const __m256i *)(wb + 16));
+                __m256i hbits = j == 0 ? qh : _mm256_srli_epi16(qh, 4);
+                values[j][0] = _mm256_or_si256(values[j][0], _mm256_and_si256(_mm256_slli_epi16(hbits, 4), mh));
+                values[j][1] = _mm256_or_si256(values[j][1], _mm256_and_si256(_mm256_slli_epi16(hbits, 3), mh));
+                values[j][2] = _mm256_or_si256(values[j][2], _mm256_and_si256(_mm256_slli_epi16(hbits, 2), mh));
+                values[j][3] = _mm256_or_si256(values[j][3], _mm256_and_si256(_mm256_slli_epi16(hbits, 1), mh));
+            }
         }
         for (int c = 0; c < C; c++) {
             const uint8_t *acol = acols[c];
@@ -402,7 +414,10 @@ int ora_avx2_dot_row_cols(int wtype, const uint8_t *wrow, const uint8_t *const *
     int nb = k / 256;
     switch (wtype) {
     case ORA_TYPE_Q4_K:
-        dot_q4k_tile(wrow, acols, cols, nb, out);
+        dot_q45k_tile(wrow, acols, cols, nb, 0, out);
+        return 0;
+    case ORA_TYPE_Q5_K:
+        dot_q45k_tile(wrow, acols, cols, nb, 1, out);
         return 0;
     case ORA_TYPE_Q6_K:
         dot_q6k_tile(wrow, acols, cols, nb, out);

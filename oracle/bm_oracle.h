@@ -29,7 +29,7 @@ extern "C" {
 
 // Refusals (the reference panics or returns QdotError, crates/qdot/src/lib.rs:127-160).
 #define ORA_EUNALIGNED (-1) // k is not a whole number of 256-value super-blocks
-#define ORA_ETYPE (-2)      // weight type outside {Q4_K = 12, Q6_K = 14, IQ2_XXS = 16}
+#define ORA_ETYPE (-2)      // weight type outside {Q4_K = 12, Q5_K = 13, Q6_K = 14, IQ2_XXS = 16}
 #define ORA_ESHORTROW (-3)
 #define ORA_ESHORTCOL (-4)
 #define ORA_ENONFINITE (-5) // an activation value that is not finite
@@ -44,6 +44,7 @@ int ora_quantize_q8k(const float *x, int k, uint8_t *out);
 int ora_quantize_col(int wtype, const float *x, int k, uint8_t *out);
 
 float ora_dot_q4k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb);
+float ora_dot_q5k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb);
 float ora_dot_q6k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb);
 float ora_dot_iq2xxs_q8k(const uint8_t *wrow, const uint8_t *acol, int nb);
 int ora_dot_row(int wtype, const uint8_t *wrow, size_t wrow_len, const uint8_t *acol, size_t acol_len, int k,
@@ -51,6 +52,7 @@ int ora_dot_row(int wtype, const uint8_t *wrow, size_t wrow_len, const uint8_t *
 int ora_gemv(int wtype, const uint8_t *w, int rows, int k, const uint8_t *act, int m, float *y);
 
 void ora_q4k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_t *a_out, int32_t *isum_out);
+void ora_q5k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_t *a_out, int32_t *isum_out);
 void ora_q6k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int fold, int32_t *s_out);
 void ora_iq2xxs_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_t *i_out, int32_t *sc_out,
                            int32_t *codes_out, int32_t *fold_out);
@@ -71,6 +73,7 @@ void ora_moe_combine(const float *down, const float *w, const float *shexp, cons
 
 // Weight quantizers (offline, host).
 int ora_quantize_row_q4k(const float *x, int k, uint8_t *out);
+int ora_quantize_row_q5k(const float *x, int k, uint8_t *out);
 int ora_quantize_row_q6k(const float *x, int k, uint8_t *out);
 int ora_quantize_row_iq2xxs(const float *x, const float *qw, int k, uint8_t *out);
 int ora_quantize_rows(int wtype, const float *x, int rows, int k, uint8_t *out, int n_threads);

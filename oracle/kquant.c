@@ -148,8 +148,10 @@ static void get_scale_min_k4(int j, const uint8_t *q, uint8_t *d, uint8_t *m) {
     }
 }
 
-// One Q4_K block by the `_ref` rule (crates/gguf/src/kquant.rs:528-660, the branch without importance).
-static void q4k_block(const float *x, uint8_t *out) {
+// One Q4_K or Q5_K block by the `_ref` rule (crates/gguf/src/kquant.rs:528-660 kquant45_block, the branch without
+// importance): `q5` takes the 5-bit levels, their search grid and the block's plane of high bits.
+static void q45k_block(const float *x, uint8_t *out, int q5) {
+    const int nmax = q5 ? 31 : 15;
     uint8_t l[256] = {0}, laux[32];
     float scales[8], mins[8], weights[32];
     float max_scale = 0.0f, max_min = 0.0f;
@@ -160,7 +162,8 @@ static void q4k_block(const float *x, uint8_t *out) {
         float av_x = sqrtf(sum_x2 / 32.0f);
         for (int k = 0; k < 32; k++) weights[k] = av_x + fabsf(xs[k]);
         float m;
-        float s = make_qkx2_quants(15, xs, weights, l + 32 * j, laux, -1.0f, 0.1f, 20, &m);
+        float s = q5 ? make_qkx2_quants(nmax, xs, weights, l + 32 * j, laux, -0.5f, 0.1f, 15, &m)
+                     : make_qkx2_quants(nmax, xs, weights, l + 32 * j, laux, -1.0f, 0.1f, 20, &m);
         scales[j] = s;
         mins[j] = m;
         if (s > max_scale) max_scale = s;
@@ -195,12 +198,30 @@ static void q4k_block(const float *x, uint8_t *out) {
         float dm = dmin * (float)m6;
         for (int ii = 0; ii < 32; ii++) {
             int li = nint((x[32 * j + ii] + dm) / dd);
-            l[32 * j + ii] = (uint8_t)imax(0, imin(15, li));
+            l[32 * j + ii] = (uint8_t)imax(0, imin(nmax, li));
         }
     }
     ora_wr16(out, d_bits);
     ora_wr16(out + 2, dmin_bits);
     memcpy(out + 4, sc, 12);
+    if (q5) { // :627-650: bit 4 of a level goes to bit n / 32 of high byte n % 32
+        uint8_t *qh = out + 16, *ql = out + 48;
+        memset(qh, 0, 32);
+        for (int p = 0; p < 4; p++)
+            for (int j = 0; j < 32; j++) {
+                uint8_t l1 = l[64 * p + j], l2 = l[64 * p + j + 32];
+                if (l1 > 15) {
+                    l1 -= 16;
+                    qh[j] |= (uint8_t)(1u << (2 * p));
+                }
+                if (l2 > 15) {
+                    l2 -= 16;
+                    qh[j] |= (uint8_t)(2u << (2 * p));
+                }
+                ql[32 * p + j] = (uint8_t)(l1 | (l2 << 4));
+            }
+        return;
+    }
     uint8_t *q = out + 16;
     for (int j = 0; j < 256; j += 64)
         for (int k = 0; k < 32; k++) *q++ = (uint8_t)(l[j + k] | (l[j + k + 32] << 4));
@@ -262,7 +283,14 @@ static int finite_row(const float *x, int k) {
 int ora_quantize_row_q4k(const float *x, int k, uint8_t *out) {
     if (k <= 0 || k % 256 != 0) return ORA_EUNALIGNED;
     if (!finite_row(x, k)) return ORA_ENONFINITE;
-    for (int i = 0; i < k / 256; i++) q4k_block(x + 256 * i, out + (size_t)i * ORA_Q4K_BLOCK);
+    for (int i = 0; i < k / 256; i++) q45k_block(x + 256 * i, out + (size_t)i * ORA_Q4K_BLOCK, 0);
+    return 0;
+}
+
+int ora_quantize_row_q5k(const float *x, int k, uint8_t *out) {
+    if (k <= 0 || k % 256 != 0) return ORA_EUNALIGNED;
+    if (!finite_row(x, k)) return ORA_ENONFINITE;
+    for (int i = 0; i < k / 256; i++) q45k_block(x + 256 * i, out + (size_t)i * ORA_Q5K_BLOCK, 1);
     return 0;
 }
 
@@ -293,6 +321,8 @@ static void *qworker(void *arg) {
         uint8_t *o = j->out + (size_t)r * rb;
         if (j->wtype == ORA_TYPE_Q4_K)
             j->rc = ora_quantize_row_q4k(xr, j->k, o);
+        else if (j->wtype == ORA_TYPE_Q5_K)
+            j->rc = ora_quantize_row_q5k(xr, j->k, o);
         else if (j->wtype == ORA_TYPE_Q6_K)
             j->rc = ora_quantize_row_q6k(xr, j->k, o);
         else

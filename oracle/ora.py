@@ -11,8 +11,8 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libbm_oracle.so")
 
-Q4_K, Q6_K, IQ2_XXS = 12, 14, 16
-BLOCK_BYTES = {Q4_K: 144, Q6_K: 210, IQ2_XXS: 66}
+Q4_K, Q5_K, Q6_K, IQ2_XXS = 12, 13, 14, 16
+BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ2_XXS: 66}
 
 EUNALIGNED, ETYPE, ESHORTROW, ESHORTCOL, ENONFINITE, ESHAPE, ESTATUS = -1, -2, -3, -4, -5, -6, -7
 
@@ -45,6 +45,7 @@ def _load():
         "ora_avx2_dot_row_cols": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
         "ora_avx2_supported": (C.c_int, []),
         "ora_q4k_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+        "ora_q5k_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
         "ora_q6k_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
         "ora_iq2xxs_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
                                          C.c_void_p]),
@@ -155,11 +156,12 @@ def gemv(wtype, w, rows, k, act, m=1):
     return y
 
 
-def q4k_block_sums(wrow, acol, k):
+def q4k_block_sums(wrow, acol, k, q5=False):
+    """Per 32-value sub-block: sum of code * activation, and the column's stored isum (Q4_K; with q5 a Q5_K row)."""
     nb = k // 256
     a = np.empty(nb * 8, np.int32)
     s = np.empty(nb * 8, np.int32)
-    lib.ora_q4k_block_sums(_p(_u8(wrow)), _p(_u8(acol)), nb, _p(a), _p(s))
+    (lib.ora_q5k_block_sums if q5 else lib.ora_q4k_block_sums)(_p(_u8(wrow)), _p(_u8(acol)), nb, _p(a), _p(s))
     return a, s
 
 

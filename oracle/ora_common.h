@@ -12,6 +12,7 @@
 #include <string.h>
 
 #define ORA_Q4K_BLOCK 144    // crates/qdot/src/lib.rs:3864
+#define ORA_Q5K_BLOCK 176    // crates/qdot/src/lib.rs:4880: d, dmin, scales[12], qh[32] @16, qs[128] @48
 #define ORA_Q6K_BLOCK 210    // crates/qdot/src/lib.rs:4452
 #define ORA_IQ2XXS_BLOCK 66  // crates/qdot/src/lib.rs:8298
 #define ORA_Q8K_STRIDE 296   // crates/qdot/src/lib.rs:108
@@ -19,6 +20,7 @@
 
 // Weight types, numbered as ggml numbers them (crates/gguf/src/qtype.rs:94,98,105).
 #define ORA_TYPE_Q4_K 12
+#define ORA_TYPE_Q5_K 13
 #define ORA_TYPE_Q6_K 14
 #define ORA_TYPE_IQ2_XXS 16
 

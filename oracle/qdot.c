@@ -74,6 +74,7 @@ int ora_col_bytes(int wtype, int k) {
     if (k <= 0 || k % 256 != 0) return ORA_EUNALIGNED; // crates/qdot/src/lib.rs:381-422
     switch (wtype) {
     case ORA_TYPE_Q4_K:
+    case ORA_TYPE_Q5_K:
     case ORA_TYPE_Q6_K:
         return k / 128 * ORA_Q82X4_STRIDE;
     case ORA_TYPE_IQ2_XXS:
@@ -88,6 +89,8 @@ int ora_row_bytes(int wtype, int k) {
     switch (wtype) {
     case ORA_TYPE_Q4_K:
         return k / 256 * ORA_Q4K_BLOCK;
+    case ORA_TYPE_Q5_K:
+        return k / 256 * ORA_Q5K_BLOCK;
     case ORA_TYPE_Q6_K:
         return k / 256 * ORA_Q6K_BLOCK;
     case ORA_TYPE_IQ2_XXS:
@@ -100,6 +103,7 @@ int ora_row_bytes(int wtype, int k) {
 int ora_quantize_col(int wtype, const float *x, int k, uint8_t *out) {
     switch (wtype) { // crates/qdot/src/lib.rs:500-534
     case ORA_TYPE_Q4_K:
+    case ORA_TYPE_Q5_K:
     case ORA_TYPE_Q6_K:
         return ora_quantize_q82x4(x, k, out);
     case ORA_TYPE_IQ2_XXS:
@@ -130,27 +134,48 @@ static inline int q4k_code(const uint8_t *qs, int n) {
     return r < 32 ? (b & 0xf) : (b >> 4);
 }
 
-// The exact integers of super-block `i`: halves[s][h] = sum over the 16 values 32s+16h.. of q4 * a, the two i32
+// Value n of a Q5_K super-block's 5-bit codes: the Q4_K nibble of its code bytes (at 48) and bit n / 32 of high byte
+// n % 32 (at 16) on top (crates/gguf/src/quant.rs dequant_q5_k; crates/qdot/src/lib.rs:4882-4893: "value 128 j + 32 b +
+// l takes bit 4 j + b of qh[l]").
+static inline int q5k_code(const uint8_t *wb, int n) {
+    return q4k_code(wb + 48, n) | (((wb[16 + (n & 31)] >> (n >> 5)) & 1) << 4);
+}
+
+// The exact integers of super-block `i`: halves[s][h] = sum over the 16 values 32s+16h.. of q * a, the two i32
 // lanes `s & 3` and `4 + (s & 3)` of the reference's sumi for j = s / 4 (crates/qdot/src/lib.rs:4402-4430: with
-// codes <= 15 and |a| <= 128 neither maddubs nor the i16 adds saturate or wrap, so the lanes are plain sums).
-static void q4k_halves(const uint8_t *wb, const uint8_t *acol, int i, int32_t halves[8][2]) {
-    const uint8_t *qs = wb + 16;
+// codes <= 15 (Q5_K: <= 31, :4889-4891) and |a| <= 128 neither maddubs nor the i16 adds saturate or wrap, so the
+// lanes are plain sums). Q5_K is the same walk over 5-bit codes (:4882-4893).
+static void q45k_halves(const uint8_t *wb, const uint8_t *acol, int i, int q5, int32_t halves[8][2]) {
     for (int s = 0; s < 8; s++) {
         const uint8_t *g = acol + (size_t)(2 * i + s / 4) * ORA_Q82X4_STRIDE;
         const int8_t *a = (const int8_t *)(g + 16 + 32 * (s & 3));
         for (int h = 0; h < 2; h++) {
             int32_t sum = 0;
-            for (int n = 0; n < 16; n++) sum += q4k_code(qs, 32 * s + 16 * h + n) * a[16 * h + n];
+            for (int n = 0; n < 16; n++) {
+                int at = 32 * s + 16 * h + n;
+                sum += (q5 ? q5k_code(wb, at) : q4k_code(wb + 16, at)) * a[16 * h + n];
+            }
             halves[s][h] = sum;
         }
     }
 }
+static void q4k_halves(const uint8_t *wb, const uint8_t *acol, int i, int32_t halves[8][2]) {
+    q45k_halves(wb, acol, i, 0, halves);
+}
+
+static float dot_q45k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb, int q5);
 
 // Q4_K x Q8_2_X4, the scalar mirror's float steps in its order (crates/qdot/src/lib.rs:4363-4447).
-float ora_dot_q4k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb) {
+float ora_dot_q4k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb) { return dot_q45k_q82x4(wrow, acol, nb, 0); }
+
+// Q5_K x Q8_2_X4 (crates/qdot/src/lib.rs:4991-5090 dot_q5k_q82x4_emul): the Q4_K walk, block for block and lane for
+// lane, over the wider block and its 5-bit codes.
+float ora_dot_q5k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb) { return dot_q45k_q82x4(wrow, acol, nb, 1); }
+
+static float dot_q45k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb, int q5) {
     float accd[8] = {0};
     for (int i = 0; i < nb; i++) {
-        const uint8_t *wb = wrow + (size_t)i * ORA_Q4K_BLOCK;
+        const uint8_t *wb = wrow + (size_t)i * (q5 ? ORA_Q5K_BLOCK : ORA_Q4K_BLOCK);
         const uint8_t *g0 = acol + (size_t)(2 * i) * ORA_Q82X4_STRIDE;
         const uint8_t *g1 = g0 + ORA_Q82X4_STRIDE;
         float d = ora_half_to_f32(ora_rd16(wb));
@@ -171,7 +196,7 @@ float ora_dot_q4k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb) {
         }
         for (int l = 0; l < 8; l++) all_scales[l] = d * (float)sc[l];
         int32_t halves[8][2];
-        q4k_halves(wb, acol, i, halves);
+        q45k_halves(wb, acol, i, q5, halves);
         for (int j = 0; j < 2; j++) {
             for (int l = 0; l < 8; l++) {
                 int idx = 4 * j + (l & 3);
@@ -190,6 +215,18 @@ void ora_q4k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_
     for (int i = 0; i < nb; i++) {
         int32_t halves[8][2];
         q4k_halves(wrow + (size_t)i * ORA_Q4K_BLOCK, acol, i, halves);
+        for (int s = 0; s < 8; s++) {
+            const uint8_t *g = acol + (size_t)(2 * i + s / 4) * ORA_Q82X4_STRIDE;
+            a_out[8 * i + s] = halves[s][0] + halves[s][1];
+            isum_out[8 * i + s] = (int16_t)ora_rd16(g + 8 + 2 * (s & 3));
+        }
+    }
+}
+
+void ora_q5k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_t *a_out, int32_t *isum_out) {
+    for (int i = 0; i < nb; i++) {
+        int32_t halves[8][2];
+        q45k_halves(wrow + (size_t)i * ORA_Q5K_BLOCK, acol, i, 1, halves);
         for (int s = 0; s < 8; s++) {
             const uint8_t *g = acol + (size_t)(2 * i + s / 4) * ORA_Q82X4_STRIDE;
             a_out[8 * i + s] = halves[s][0] + halves[s][1];
@@ -355,6 +392,9 @@ int ora_dot_row(int wtype, const uint8_t *wrow, size_t wrow_len, const uint8_t *
     case ORA_TYPE_Q4_K:
         *out = ora_dot_q4k_q82x4(wrow, acol, nb);
         return 0;
+    case ORA_TYPE_Q5_K:
+        *out = ora_dot_q5k_q82x4(wrow, acol, nb);
+        return 0;
     case ORA_TYPE_Q6_K:
         *out = ora_dot_q6k_q82x4(wrow, acol, nb);
         return 0;
@@ -395,6 +435,15 @@ int ora_dequant_row(int wtype, const uint8_t *src, int k, float *dst) {
                 float d1 = d * (float)sc[n / 32], m1 = dmin * (float)mn[n / 32];
                 out[n] = fmaf((float)q4k_code(blk + 16, n), d1, -m1);
             }
+        } else if (wtype == ORA_TYPE_Q5_K) { // crates/gguf/src/quant.rs:780-816
+            const uint8_t *blk = src + (size_t)i * ORA_Q5K_BLOCK;
+            float d = ora_half_to_f32(ora_rd16(blk)), dmin = ora_half_to_f32(ora_rd16(blk + 2));
+            uint8_t sc[8], mn[8];
+            q4k_scales_mins(blk + 4, sc, mn);
+            for (int n = 0; n < 256; n++) {
+                float d1 = d * (float)sc[n / 32], m1 = dmin * (float)mn[n / 32];
+                out[n] = fmaf((float)q5k_code(blk, n), d1, -m1);
+            }
         } else if (wtype == ORA_TYPE_Q6_K) { // crates/gguf/src/quant.rs:826-859
             const uint8_t *blk = src + (size_t)i * ORA_Q6K_BLOCK;
             float d = ora_half_to_f32(ora_rd16(blk + 208));
@@ -429,7 +478,7 @@ int ora_dequant_col(int wtype, const uint8_t *acol, int k, float *dst) {
         }
         return 0;
     }
-    if (wtype != ORA_TYPE_Q4_K && wtype != ORA_TYPE_Q6_K) return ORA_ETYPE;
+    if (wtype != ORA_TYPE_Q4_K && wtype != ORA_TYPE_Q5_K && wtype != ORA_TYPE_Q6_K) return ORA_ETYPE;
     for (int g = 0; g < k / 128; g++) {
         const uint8_t *grp = acol + (size_t)g * ORA_Q82X4_STRIDE;
         for (int ir = 0; ir < 4; ir++) {

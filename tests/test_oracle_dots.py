@@ -16,7 +16,7 @@ import ora
 from common import normal_f32
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-TYPES = (ora.Q4_K, ora.Q6_K, ora.IQ2_XXS)
+TYPES = (ora.Q4_K, ora.Q5_K, ora.Q6_K, ora.IQ2_XXS)
 
 
 # ---------------------------------------------------------------- independent numpy decoders (written from the
@@ -61,6 +61,15 @@ def q4k_decode(blk):
     return codes, vals, (d, dmin, sc, mn)
 
 
+def q5k_decode(blk):
+    """block_q5_K (crates/gguf/src/quant.rs:769-816): Q4_K's header, 32 high-bit bytes, then Q4_K's nibbles."""
+    low, _, (d, dmin, sc, mn) = q4k_decode(np.concatenate([blk[0:16], blk[48:176]]))
+    qh = blk[16:48]
+    codes = low + np.array([((int(qh[n % 32]) >> (n // 32)) & 1) << 4 for n in range(256)], np.int64)
+    vals = np.array([d * sc[n // 32] * codes[n] - dmin * mn[n // 32] for n in range(256)], np.float64)
+    return codes, vals, (d, dmin, sc, mn)
+
+
 def q6k_decode(blk):
     ql, qh, scb = blk[0:128], blk[128:192], blk[192:208].view(np.int8)
     d = f16(blk[208], blk[209])
@@ -95,7 +104,7 @@ def iq2xxs_decode(blk):
     return codes, vals, (d, scs)
 
 
-DECODE = {ora.Q4_K: q4k_decode, ora.Q6_K: q6k_decode, ora.IQ2_XXS: iq2xxs_decode}
+DECODE = {ora.Q4_K: q4k_decode, ora.Q5_K: q5k_decode, ora.Q6_K: q6k_decode, ora.IQ2_XXS: iq2xxs_decode}
 
 
 def act_codes(wtype, col, k):
@@ -118,9 +127,9 @@ def random_blocks(wtype, nb, rng):
     w = rng.integers(0, 256, nb * bb, dtype=np.uint8)
     for i in range(nb):
         h = np.array([rng.uniform(-0.1, 0.1), rng.uniform(0.0, 0.1)], np.float16).view(np.uint8)
-        off = {ora.Q4_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0}[wtype]
+        off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0}[wtype]
         w[i * bb + off:i * bb + off + 2] = h[0:2]
-        if wtype == ora.Q4_K:
+        if wtype in (ora.Q4_K, ora.Q5_K):
             w[i * bb + 2:i * bb + 4] = h[2:4]
     return w
 
@@ -177,8 +186,8 @@ def test_block_sums_equal_brute_force(wtype):
         a, _ = act_codes(wtype, col, k)
         wc = np.concatenate([DECODE[wtype](w[i * bb:(i + 1) * bb])[0] for i in range(nb)])
         prod = wc * a
-        if wtype == ora.Q4_K:
-            got_a, got_isum = ora.q4k_block_sums(w, col, k)
+        if wtype in (ora.Q4_K, ora.Q5_K):
+            got_a, got_isum = ora.q4k_block_sums(w, col, k, q5=wtype == ora.Q5_K)
             assert list(got_a) == [int(prod[32 * s:32 * s + 32].sum()) for s in range(nb * 8)]
             assert list(got_isum) == [int(a[32 * s:32 * s + 32].sum()) for s in range(nb * 8)]
         elif wtype == ora.Q6_K:
@@ -225,9 +234,9 @@ def extreme_cases(wtype, rng):
         w = np.full(2 * bb, fill, np.uint8)
         for i in range(2):
             h = np.array([dval, abs(dval)], np.float16).view(np.uint8)
-            off = {ora.Q4_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0}[wtype]
+            off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0}[wtype]
             w[i * bb + off:i * bb + off + 2] = h[0:2]
-            if wtype == ora.Q4_K:
+            if wtype in (ora.Q4_K, ora.Q5_K):
                 w[i * bb + 2:i * bb + 4] = h[2:4]
         out.append(w)
     out.append(random_blocks(wtype, 2, rng))
@@ -312,11 +321,11 @@ def test_dot_within_f64_band_of_dequantized_dot(wtype):
                 terms = 2 * nb + 10
             else:
                 wv = np.concatenate([DECODE[wtype](w[i * bb:(i + 1) * bb])[1] for i in range(nb)])
-                if wtype == ora.Q4_K:
+                if wtype in (ora.Q4_K, ora.Q5_K):
                     # value = d*sc*q - dmin*m: bound with both parts' magnitudes
                     parts = []
                     for i in range(nb):
-                        codes, _, (d, dmin, sc, mn) = q4k_decode(w[i * bb:(i + 1) * bb])
+                        codes, _, (d, dmin, sc, mn) = DECODE[wtype](w[i * bb:(i + 1) * bb])
                         parts.append(np.array([abs(d) * sc[n // 32] * codes[n] + abs(dmin) * mn[n // 32]
                                                for n in range(256)]))
                     mag = np.sum(np.concatenate(parts) * np.abs(act))

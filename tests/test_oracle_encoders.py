@@ -32,6 +32,8 @@ def test_sizes():
     assert ora.col_bytes(ora.IQ2_XXS, 7168) == 8288 and ora.col_bytes(ora.IQ2_XXS, 2048) == 2368
     assert ora.row_bytes(ora.Q4_K, 2048) == 1152 and ora.row_bytes(ora.Q6_K, 768) == 630
     assert ora.row_bytes(ora.IQ2_XXS, 7168) == 1848
+    # crates/qdot/tests/qdot.rs:478-479: Q5_K pairs the Q8_2_X4 column with 176 weight bytes a super-block
+    assert ora.col_bytes(ora.Q5_K, 2304) == 144 * 18 and ora.row_bytes(ora.Q5_K, 2304) == 176 * 9
     for k in (0, 100, 255, 257, 2048 + 128):
         with pytest.raises(ora.OracleError) as e:
             ora.col_bytes(ora.Q4_K, k)

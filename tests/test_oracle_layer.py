@@ -185,7 +185,7 @@ def wave_row(n, seed):
     return out
 
 
-@pytest.mark.parametrize("wtype,bound", ((ora.Q4_K, 0.12), (ora.Q6_K, 0.02)))
+@pytest.mark.parametrize("wtype,bound", ((ora.Q4_K, 0.12), (ora.Q5_K, 0.06), (ora.Q6_K, 0.02)))
 def test_kquant_round_trip_bounds(wtype, bound):
     x = wave_row(512, 3)
     q = ora.quantize_rows(wtype, x, 1, 512, n_threads=1)
@@ -195,7 +195,7 @@ def test_kquant_round_trip_bounds(wtype, bound):
     assert not ora.quantize_rows(wtype, np.zeros(256, np.float32), 1, 256).any(), "a zero row is zero bytes"
 
 
-@pytest.mark.parametrize("wtype,rel", ((ora.Q4_K, 0.09), (ora.Q6_K, 0.02), (ora.IQ2_XXS, 0.55)))
+@pytest.mark.parametrize("wtype,rel", ((ora.Q4_K, 0.09), (ora.Q5_K, 0.045), (ora.Q6_K, 0.02), (ora.IQ2_XXS, 0.55)))
 def test_quantizers_on_the_benchmark_distribution(wtype, rel):
     rng = np.random.default_rng(40 + wtype)
     x = normal_f32(rng, (16, 1024), 0.02)
@@ -212,7 +212,7 @@ def test_quantizers_on_the_benchmark_distribution(wtype, rel):
 def test_kquant_refuses_non_finite_and_unaligned():
     x = np.ones(256, np.float32)
     x[3] = np.nan
-    for wtype in (ora.Q4_K, ora.Q6_K):
+    for wtype in (ora.Q4_K, ora.Q5_K, ora.Q6_K):
         with pytest.raises(ora.OracleError) as e:
             ora.quantize_rows(wtype, x, 1, 256)
         assert e.value.code == ora.ENONFINITE

@@ -61,7 +61,9 @@ static int driver(bm_ctx *ctx, const char *what, hipError_t e) {
     return fail(ctx, BM_EDRIVER, "%s: %s", what, hipGetErrorString(e));
 }
 
-static bool known_type(int t) { return t == BM_TYPE_Q4_K || t == BM_TYPE_Q6_K || t == BM_TYPE_IQ2_XXS; }
+static bool known_type(int t) {
+    return t == BM_TYPE_Q4_K || t == BM_TYPE_Q5_K || t == BM_TYPE_Q6_K || t == BM_TYPE_IQ2_XXS;
+}
 // Q8_2_X4 for the K-quants, Q8_K for IQ2_XXS (crates/gguf/src/qtype.rs host_act).
 static int act_form(int t) { return t == BM_TYPE_IQ2_XXS ? 1 : 0; }
 // Bytes between two columns of a bm_act on the device (the CPU path's bytes plus the dot kernels' tables).
@@ -74,7 +76,7 @@ int bm_version(void) { return 101; }
 int64_t bm_row_bytes(int wtype, int k) {
     if (!known_type(wtype)) return BM_ETYPE;
     if (k <= 0 || k % 256 != 0) return BM_ESHAPE;
-    const int bb = wtype == BM_TYPE_Q4_K ? 144 : (wtype == BM_TYPE_Q6_K ? 210 : 66);
+    const int bb = wtype == BM_TYPE_Q4_K ? 144 : wtype == BM_TYPE_Q5_K ? 176 : wtype == BM_TYPE_Q6_K ? 210 : 66;
     return (int64_t)(k / 256) * bb;
 }
 
@@ -220,7 +222,7 @@ static int weights_make(bm_ctx *ctx, const char *what, int wtype, int64_t rows, 
                         const void *dev, bm_weights **out) {
     if (!ctx || !out) return fail(ctx, BM_EARG, "%s: NULL argument", what);
     *out = nullptr;
-    if (!known_type(wtype)) return fail(ctx, BM_ETYPE, "%s: weight type %d has no kernel (12 Q4_K, 14 Q6_K, 16 IQ2_XXS)", what, wtype);
+    if (!known_type(wtype)) return fail(ctx, BM_ETYPE, "%s: weight type %d has no kernel (12 Q4_K, 13 Q5_K, 14 Q6_K, 16 IQ2_XXS)", what, wtype);
     if (k <= 0 || k % 256 != 0) return fail(ctx, BM_ESHAPE, "%s: k = %d is not a whole number of 256-value super-blocks", what, k);
     if (rows <= 0) return fail(ctx, BM_ESHAPE, "%s: rows = %lld must be positive", what, (long long)rows);
     const size_t bytes = (size_t)rows * (size_t)bm_row_bytes(wtype, k);
@@ -241,9 +243,9 @@ static int weights_make(bm_ctx *ctx, const char *what, int wtype, int64_t rows, 
             delete w;
             return fail(ctx, BM_EARG, "%s: dev_bytes is NULL", what);
         }
-        if (wtype == BM_TYPE_Q4_K && ((uintptr_t)dev & 15) != 0) {
+        if ((wtype == BM_TYPE_Q4_K || wtype == BM_TYPE_Q5_K) && ((uintptr_t)dev & 15) != 0) {
             delete w;
-            return fail(ctx, BM_ESHAPE, "%s: Q4_K rows are read with 16-byte loads, dev_bytes %p is not 16-byte aligned", what, dev);
+            return fail(ctx, BM_ESHAPE, "%s: Q4_K and Q5_K rows are read with 16-byte loads, dev_bytes %p is not 16-byte aligned", what, dev);
         }
         if (((uintptr_t)dev & 1) != 0) {
             delete w;

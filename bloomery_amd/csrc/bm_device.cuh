@@ -1,15 +1,15 @@
 // Device-side building blocks of the quantized row dots on gfx950 (wave64).
 //
 // Lane map ("quad"): one weight row is dotted by four consecutive lanes. The CPU path this library reproduces
-// (crates/qdot/src/lib.rs:4363-4447 Q4_K, :4776-4874 Q6_K, :8677-8724 IQ2_XXS) keeps eight f32 accumulators per
+// (crates/qdot/src/lib.rs:4363-4447 Q4_K, :4991-5090 Q5_K, :4776-4874 Q6_K, :8677-8724 IQ2_XXS) keeps eight f32 accumulators per
 // row and walks the super-blocks in order; here each lane of the quad owns two of the eight and walks every
 // super-block of the row itself, so each accumulator sees the reference's fused multiply-adds in the reference's
 // order and the final butterfly over the quad is the reference's closing sum ((t0+t2)+(t1+t3), t_l = acc_l +
-// acc_{l+4}). The integer sums are formed with v_dot4_i32_i8 over the same 16-value (Q4_K, Q6_K) or 4-value
+// acc_{l+4}). The integer sums are formed with v_dot4_i32_i8 over the same 16-value (Q4_K, Q5_K, Q6_K) or 4-value
 // (IQ2_XXS) spans the reference's i32 lanes cover; they are exact, so their inner order is free.
 //
 // Activation columns on the device. A Q8_K column (IQ2_XXS weights) is the CPU path's bytes, 296 a super-block.
-// A Q8_2_X4 column (Q4_K, Q6_K weights) is the CPU path's bytes (288 a super-block) followed by two tables the
+// A Q8_2_X4 column (Q4_K, Q5_K, Q6_K weights) is the CPU path's bytes (288 a super-block) followed by two tables the
 // quantizers write beside them so the dots need no per-block unpacking: for each 32-value block the pair
 // (d8 as f32, d8 * (f32)isum) - the second is the product the reference forms first in its min term - and for each
 // 16 values the i32 sum of the stored codes (Q6_K's -32 offset comes out through it). nb super-blocks give
@@ -27,10 +27,12 @@
 typedef uint32_t u32;
 
 #define BM_Q4K 12
+#define BM_Q5K 13
 #define BM_Q6K 14
 #define BM_IQ2XXS 16
 
 #define BM_Q4K_BLOCK 144
+#define BM_Q5K_BLOCK 176
 #define BM_Q6K_BLOCK 210
 #define BM_IQ2XXS_BLOCK 66
 #define BM_Q82X4_STRIDE 144
@@ -226,6 +228,9 @@ struct Act<BM_Q4K> {
     u32 sw;                   // the two stored isums (taps only)
 };
 
+template <>
+struct Act<BM_Q5K> : Act<BM_Q4K> {};
+
 template <bool WithSums>
 __device__ __forceinline__ Act<BM_Q4K> bm_act_q4k(const ActView &av, int i, int c, int h) {
     const uint8_t *g0 = av.col + (size_t)(2 * i) * BM_Q82X4_STRIDE + 16 + 64 * c + 16 * h;
@@ -245,14 +250,15 @@ __device__ __forceinline__ Act<BM_Q4K> bm_act_q4k(const ActView &av, int i, int 
     return a;
 }
 
-// One super-block `i` of one column.
-template <class Tap>
-__device__ __forceinline__ void bm_dot_q4k(const Blk<BM_Q4K> &b, const Act<BM_Q4K> &a, int i, int c, int h,
-                                           float &acc0, float &acc1, const Tap &tap) {
-    const float d = bm_half_to_f32(b.hdr.x & 0xffffu), dmin = bm_half_to_f32(b.hdr.x >> 16);
-    const u32 a0 = b.hdr.y, a1 = b.hdr.z, a2 = b.hdr.w; // crates/qdot/src/lib.rs:3868-3878
-    const int sh = 16 * c;                               // this lane's two sub-blocks sit in bytes 2c, 2c + 1
-    const u32 s0 = (a0 & 0x3f3f3f3fu) >> sh;             // scales of sub-blocks 2c, 2c + 1
+// One super-block `i` of one column, from the header word, the two code words and the column's reads. `Bits` adds
+// a code's fifth bit (Q5_K) before the integer dots; Q4_K passes none.
+template <class Bits, class Tap>
+__device__ __forceinline__ void bm_dot_q45k(uint4 hdr, uint4 qa, uint4 qb, const Bits &bits, const Act<BM_Q4K> &a, int i,
+                                            int c, int h, float &acc0, float &acc1, const Tap &tap) {
+    const float d = bm_half_to_f32(hdr.x & 0xffffu), dmin = bm_half_to_f32(hdr.x >> 16);
+    const u32 a0 = hdr.y, a1 = hdr.z, a2 = hdr.w; // crates/qdot/src/lib.rs:3868-3878
+    const int sh = 16 * c;                         // this lane's two sub-blocks sit in bytes 2c, 2c + 1
+    const u32 s0 = (a0 & 0x3f3f3f3fu) >> sh;       // scales of sub-blocks 2c, 2c + 1
     const u32 s1 = ((a2 & 0x0f0f0f0fu) | ((a0 >> 2) & 0x30303030u)) >> sh; // 4 + 2c, 5 + 2c
     const u32 mw = h ? (((a2 >> 4) & 0x0f0f0f0fu) | ((a1 >> 2) & 0x30303030u)) : (a1 & 0x3f3f3f3fu);
     const u32 mm = mw >> sh; // mins of sub-blocks 4h + 2c, 4h + 2c + 1
@@ -266,7 +272,7 @@ __device__ __forceinline__ void bm_dot_q4k(const Blk<BM_Q4K> &b, const Act<BM_Q4
     // j = 0: sub-blocks 2c, 2c + 1 (group 0); j = 1: 4 + 2c, 5 + 2c (group 1) (lib.rs:4402-4436).
     {
         int lo, hi;
-        bm_q4_dot16(b.qa, a.lo0, a.hi0, lo, hi);
+        bits.dot16(qa, 2 * c, a.lo0, a.hi0, lo, hi);
         acc0 = fmaf((d * (float)(s0 & 0xffu)) * a.e0.x, (float)lo, acc0);
         acc1 = fmaf((d * (float)((s0 >> 8) & 0xffu)) * a.e0.z, (float)hi, acc1);
         tap.q4k(i, 2 * c, h, lo);
@@ -274,12 +280,64 @@ __device__ __forceinline__ void bm_dot_q4k(const Blk<BM_Q4K> &b, const Act<BM_Q4
     }
     {
         int lo, hi;
-        bm_q4_dot16(b.qb, a.lo1, a.hi1, lo, hi);
+        bits.dot16(qb, 4 + 2 * c, a.lo1, a.hi1, lo, hi);
         acc0 = fmaf((d * (float)(s1 & 0xffu)) * a.e1.x, (float)lo, acc0);
         acc1 = fmaf((d * (float)((s1 >> 8) & 0xffu)) * a.e1.z, (float)hi, acc1);
         tap.q4k(i, 4 + 2 * c, h, lo);
         tap.q4k(i, 5 + 2 * c, h, hi);
     }
+}
+
+struct NoFifthBit {
+    __device__ __forceinline__ void dot16(uint4 q, int, uint4 alo, uint4 ahi, int &lo, int &hi) const {
+        bm_q4_dot16(q, alo, ahi, lo, hi);
+    }
+};
+
+template <class Tap>
+__device__ __forceinline__ void bm_dot_q4k(const Blk<BM_Q4K> &b, const Act<BM_Q4K> &a, int i, int c, int h,
+                                           float &acc0, float &acc1, const Tap &tap) {
+    bm_dot_q45k(b.hdr, b.qa, b.qb, NoFifthBit{}, a, i, c, h, acc0, acc1, tap);
+}
+
+// ---- Q5_K (crates/qdot/src/lib.rs:4876-4893): Q4_K's lane map over the 176-byte block. The lane also reads high
+// bytes [16h, +16): value 32s + 16h + t takes bit s of high byte 16h + t as its fifth bit, so the low nibbles of the
+// first code word (sub-block 2c) take bit 2c, its high nibbles bit 2c + 1, the second word's bits 4 + 2c and 5 + 2c.
+template <>
+struct Blk<BM_Q5K> {
+    uint4 hdr, qh, qa, qb;
+};
+
+__device__ __forceinline__ Blk<BM_Q5K> bm_load_q5k(const uint8_t *wrow, int i, int c, int h) {
+    const uint8_t *wb = wrow + (size_t)i * BM_Q5K_BLOCK;
+    Blk<BM_Q5K> b;
+    b.hdr = bm_ld16(wb);
+    b.qh = bm_ld16(wb + 16 + 16 * h);
+    b.qa = bm_ld16(wb + 48 + 32 * c + 16 * h);
+    b.qb = bm_ld16(wb + 48 + 64 + 32 * c + 16 * h);
+    return b;
+}
+
+struct FifthBit {
+    uint4 qh;
+    // `s`: the sub-block of q's low nibbles; its high nibbles are sub-block s + 1
+    __device__ __forceinline__ void dot16(uint4 q, int s, uint4 alo, uint4 ahi, int &lo, int &hi) const {
+        const u32 m = 0x0f0f0f0fu, one = 0x01010101u;
+        lo = bm_sdot4((q.x & m) | (((qh.x >> s) & one) << 4), alo.x, 0);
+        lo = bm_sdot4((q.y & m) | (((qh.y >> s) & one) << 4), alo.y, lo);
+        lo = bm_sdot4((q.z & m) | (((qh.z >> s) & one) << 4), alo.z, lo);
+        lo = bm_sdot4((q.w & m) | (((qh.w >> s) & one) << 4), alo.w, lo);
+        hi = bm_sdot4(((q.x >> 4) & m) | (((qh.x >> (s + 1)) & one) << 4), ahi.x, 0);
+        hi = bm_sdot4(((q.y >> 4) & m) | (((qh.y >> (s + 1)) & one) << 4), ahi.y, hi);
+        hi = bm_sdot4(((q.z >> 4) & m) | (((qh.z >> (s + 1)) & one) << 4), ahi.z, hi);
+        hi = bm_sdot4(((q.w >> 4) & m) | (((qh.w >> (s + 1)) & one) << 4), ahi.w, hi);
+    }
+};
+
+template <class Tap>
+__device__ __forceinline__ void bm_dot_q5k(const Blk<BM_Q5K> &b, const Act<BM_Q5K> &a, int i, int c, int h,
+                                           float &acc0, float &acc1, const Tap &tap) {
+    bm_dot_q45k(b.hdr, b.qa, b.qb, FifthBit{b.qh}, a, i, c, h, acc0, acc1, tap);
 }
 
 // ---- Q6_K: lane (c, h) owns accumulators l = 4h + c and 4h + c + 2. Per 128-value half j it reads ql bytes
@@ -489,12 +547,16 @@ __device__ __forceinline__ float bm_quad_finish(float acc0, float acc1) {
     return X + Y;
 }
 
-// Uniform front over the three types.
+// Uniform front over the types.
 template <int WT>
 __device__ __forceinline__ Blk<WT> bm_load_blk(const uint8_t *wrow, int i, int q);
 template <>
 __device__ __forceinline__ Blk<BM_Q4K> bm_load_blk<BM_Q4K>(const uint8_t *wrow, int i, int q) {
     return bm_load_q4k(wrow, i, q & 1, q >> 1);
+}
+template <>
+__device__ __forceinline__ Blk<BM_Q5K> bm_load_blk<BM_Q5K>(const uint8_t *wrow, int i, int q) {
+    return bm_load_q5k(wrow, i, q & 1, q >> 1);
 }
 template <>
 __device__ __forceinline__ Blk<BM_Q6K> bm_load_blk<BM_Q6K>(const uint8_t *wrow, int i, int q) {
@@ -509,7 +571,11 @@ template <int WT, bool WithSums>
 __device__ __forceinline__ Act<WT> bm_load_act(const ActView &av, int i, int q) {
     if constexpr (WT == BM_Q4K)
         return bm_act_q4k<WithSums>(av, i, q & 1, q >> 1);
-    else if constexpr (WT == BM_Q6K)
+    else if constexpr (WT == BM_Q5K) {
+        Act<BM_Q5K> a;
+        static_cast<Act<BM_Q4K> &>(a) = bm_act_q4k<WithSums>(av, i, q & 1, q >> 1);
+        return a;
+    } else if constexpr (WT == BM_Q6K)
         return bm_act_q6k(av, i, q & 1, q >> 1);
     else
         return bm_act_iq2xxs(av, i, q);
@@ -520,6 +586,8 @@ __device__ __forceinline__ void bm_dot_blk(const Blk<WT> &b, const Act<WT> &a, i
                                            float &acc0, float &acc1, const Tap &tap) {
     if constexpr (WT == BM_Q4K)
         bm_dot_q4k(b, a, i, q & 1, q >> 1, acc0, acc1, tap);
+    else if constexpr (WT == BM_Q5K)
+        bm_dot_q5k(b, a, i, q & 1, q >> 1, acc0, acc1, tap);
     else if constexpr (WT == BM_Q6K)
         bm_dot_q6k(b, a, i, q & 1, q >> 1, acc0, acc1, tap);
     else
@@ -528,7 +596,7 @@ __device__ __forceinline__ void bm_dot_blk(const Blk<WT> &b, const Act<WT> &a, i
 
 template <int WT>
 __host__ __device__ constexpr int bm_block_bytes() {
-    return WT == BM_Q4K ? BM_Q4K_BLOCK : (WT == BM_Q6K ? BM_Q6K_BLOCK : BM_IQ2XXS_BLOCK);
+    return WT == BM_Q4K ? BM_Q4K_BLOCK : WT == BM_Q5K ? BM_Q5K_BLOCK : WT == BM_Q6K ? BM_Q6K_BLOCK : BM_IQ2XXS_BLOCK;
 }
 
 // ---- SwiGLU: crates/qdot/src/lib.rs:3741-3773 (expf) and :11467-11478 (divide, then multiply).

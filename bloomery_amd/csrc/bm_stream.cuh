@@ -393,6 +393,10 @@ constexpr int kRingQ4K = 4, kRingQ6K = 3;
         else if ((nb) % 2 == 0) BM_VARIANT(BM_Q4K, 2, 0)                                                               \
         else BM_VARIANT(BM_Q4K, 1, 0)                                                                                  \
         break;                                                                                                         \
+    case BM_Q5K:                                                                                                       \
+        if ((nb) % 2 == 0) BM_VARIANT(BM_Q5K, 2, 0)                                                                    \
+        else BM_VARIANT(BM_Q5K, 1, 0)                                                                                  \
+        break;                                                                                                         \
     case BM_Q6K:                                                                                                       \
         if ((nb) == 3) BM_VARIANT(BM_Q6K, kRingQ6K, 3)                                                                 \
         else if ((nb) % 2 == 0) BM_VARIANT(BM_Q6K, 2, 0)                                                               \

@@ -1,5 +1,5 @@
 // TEST INFRASTRUCTURE ONLY. CPU oracle of the quantized MoE expert-matmul path: a plain C restatement of the
-// reference's crates/qdot (activation encoders, Q4_K / Q6_K / IQ2_XXS row dots, SwiGLU), crates/gguf (block
+// reference's crates/qdot (activation encoders, Q4_K / Q5_K / Q6_K / IQ2_XXS row dots, SwiGLU), crates/gguf (block
 // layouts, dequantizers, K-quant and IQ2_XXS weight quantizers) and the caller-side router/combine order of
 // crates/model/src/moe.rs. Each function cites the reference lines it follows. The shipped library never links
 // or calls this; the test suite, the smoke check and the benchmark's CPU-baseline leg do.

@@ -14,7 +14,7 @@ from common import Lcg, max_abs_normalised, normal_f32
 
 pytestmark = pytest.mark.gpu
 
-TYPES = (bm.Q4_K, bm.Q6_K, bm.IQ2_XXS)
+TYPES = (bm.Q4_K, bm.Q5_K, bm.Q6_K, bm.IQ2_XXS)
 TIES = np.array([0.5, 1.5, 2.5, 3.5, -0.5, -1.5, -2.5, -3.5, 0.25, 7.5, -7.5, 63.5, -63.5, 120.5, -120.5,
                  0.0, -0.0, 127.0, -127.0], np.float32)
 
@@ -40,11 +40,11 @@ def random_blocks(wtype, rows, k, rng):
     bb = ora.BLOCK_BYTES[wtype]
     nb = k // 256
     w = rng.integers(0, 256, rows * nb * bb, dtype=np.uint8).reshape(rows * nb, bb)
-    off = {ora.Q4_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0}[wtype]
+    off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0}[wtype]
     d = rng.uniform(-0.05, 0.05, rows * nb).astype(np.float16).view(np.uint16)
     w[:, off] = d & 0xFF
     w[:, off + 1] = d >> 8
-    if wtype == ora.Q4_K:
+    if wtype in (ora.Q4_K, ora.Q5_K):
         m = rng.uniform(0.0, 0.05, rows * nb).astype(np.float16).view(np.uint16)
         w[:, 2] = m & 0xFF
         w[:, 3] = m >> 8
@@ -117,7 +117,7 @@ def test_quantize_bytes_are_the_cpu_paths(gpu, wtype, k):
 
 def test_quantize_random_columns(gpu):
     rng = np.random.default_rng(7)
-    for wtype, k in ((bm.Q4_K, 2048), (bm.Q6_K, 768), (bm.IQ2_XXS, 7168)):
+    for wtype, k in ((bm.Q4_K, 2048), (bm.Q5_K, 2304), (bm.Q6_K, 768), (bm.IQ2_XXS, 7168)):
         m = 40
         x = (normal_f32(rng, (m, k)) * (10.0 ** rng.uniform(-5, 4, (m, 1)))).astype(np.float32)
         act = gpu.act(wtype, k, m)
@@ -176,8 +176,8 @@ def test_block_sums_are_the_cpu_paths_integers(gpu, wtype):
                 gpu.enqueue_block_sums(wd, row, act, col, out)
                 got = out.download().reshape(-1, 16)
                 wrow, acol = w[row * rb:(row + 1) * rb], ora.quantize_col(wtype, x[col])
-                if wtype == bm.Q4_K:
-                    a, isum = ora.q4k_block_sums(wrow, acol, k)
+                if wtype in (bm.Q4_K, bm.Q5_K):
+                    a, isum = ora.q4k_block_sums(wrow, acol, k, q5=wtype == bm.Q5_K)
                     assert np.array_equal(got[:, :8].reshape(-1), a) and np.array_equal(got[:, 8:].reshape(-1), isum)
                 elif wtype == bm.Q6_K:
                     assert np.array_equal(got.reshape(-1), ora.q6k_block_sums(wrow, acol, k))
@@ -192,7 +192,8 @@ def test_block_sums_are_the_cpu_paths_integers(gpu, wtype):
 # -------------------------------------------------------------------------------------------------------- gemv
 
 @pytest.mark.parametrize("wtype,rows,k", ((bm.Q4_K, 768, 2048), (bm.Q6_K, 2048, 768), (bm.IQ2_XXS, 300, 2048),
-                                          (bm.Q4_K, 70, 256), (bm.Q6_K, 65, 1792), (bm.IQ2_XXS, 33, 7168)))
+                                          (bm.Q4_K, 70, 256), (bm.Q6_K, 65, 1792), (bm.IQ2_XXS, 33, 7168),
+                                          (bm.Q5_K, 96, 2304), (bm.Q5_K, 67, 1280)))
 def test_gemv_matches_dot_row(gpu, wtype, rows, k):
     # config 1 is the first case: 768 x 2048 Q4_K against one 2048-vector
     rng = np.random.default_rng(30 + rows)
@@ -221,9 +222,9 @@ def test_extreme_blocks(gpu):
             w = np.full(2 * bb, fill, np.uint8)
             for i in range(2):
                 h = np.array([dval, abs(dval)], np.float16).view(np.uint8)
-                off = {ora.Q4_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0}[wtype]
+                off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0}[wtype]
                 w[i * bb + off:i * bb + off + 2] = h[0:2]
-                if wtype == ora.Q4_K:
+                if wtype in (ora.Q4_K, ora.Q5_K):
                     w[i * bb + 2:i * bb + 4] = h[2:4]
             rows_bytes.append(w)
         w = np.concatenate(rows_bytes)
@@ -330,6 +331,8 @@ def test_qwen3_shaped_layer_one_token(gpu, fused):
 @pytest.mark.parametrize("types,hidden,ff,n_experts,m,top_k", (
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 12, 5, 4),
     ((bm.Q6_K, bm.Q6_K, bm.Q4_K), 512, 512, 5, 3, 2),
+    ((bm.Q5_K, bm.Q5_K, bm.Q5_K), 768, 512, 4, 3, 2),
+    ((bm.Q4_K, bm.Q4_K, bm.Q5_K), 512, 2304, 3, 2, 2),          # a Q5_K down stack over 2304-value rows
     ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ2_XXS), 1024, 512, 6, 4, 3),
     ((bm.IQ2_XXS, bm.IQ2_XXS, bm.Q6_K), 768, 256, 4, 2, 4),
 ))
@@ -573,6 +576,7 @@ def run_grouped(gpu, L, x, ids, wts, top_k, fused_quant):
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 16, 16, 8),   # config 3's shape with 16 experts resident: long runs
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 128, 16, 8),  # config 3: 128 slots over 128 experts, skewed
     ((bm.Q6_K, bm.Q6_K, bm.Q4_K), 512, 512, 3, 7, 2),
+    ((bm.Q5_K, bm.Q5_K, bm.Q5_K), 768, 512, 3, 9, 2),
     ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ2_XXS), 1024, 512, 5, 6, 3),
     ((bm.IQ2_XXS, bm.IQ2_XXS, bm.Q6_K), 768, 256, 4, 5, 4),
 ))
@@ -626,7 +630,7 @@ def test_grouped_skips_host_slots_and_refuses_stale_entries(gpu):
 def test_slot_equals_one_expert_gemv_and_duplicate_ids(gpu):
     # gate_q4k_sel's first clauses (crates/gpu-gates/src/bin/gate_q4k_sel.rs:1-48)
     rng = np.random.default_rng(300)
-    for wtype, k, rpe in ((bm.Q4_K, 768, 96), (bm.Q6_K, 768, 2048 // 8), (bm.IQ2_XXS, 512, 80)):
+    for wtype, k, rpe in ((bm.Q4_K, 768, 96), (bm.Q5_K, 1024, 72), (bm.Q6_K, 768, 2048 // 8), (bm.IQ2_XXS, 512, 80)):
         n_experts, n_slots = 5, 7
         w = stack(wtype, n_experts * rpe, k, 301)
         sel = np.array([3, 0, 3, 4, 1, 3, 0], np.uint32)

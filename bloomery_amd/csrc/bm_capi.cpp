@@ -465,9 +465,9 @@ int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const 
                  int n_slots_per_token, int m, int rows_per_expert, bm_act *act_h, bm_act *act_x, float *h_dev) {
     const char *what = "bm_gate_up_x";
     if (!ctx || !wg || !wu || !x_dev || !sel_dev || !act_h) return fail(ctx, BM_EARG, "%s: NULL argument", what);
-    if (wg->wtype != BM_TYPE_Q4_K || wu->wtype != BM_TYPE_Q4_K)
-        return fail(ctx, BM_ETYPE, "%s: takes Q4_K gate and up stacks, got types %d and %d; use bm_quantize and bm_gate_up", what,
-                    wg->wtype, wu->wtype);
+    if (wg->wtype != wu->wtype || (wg->wtype != BM_TYPE_Q4_K && wg->wtype != BM_TYPE_Q5_K))
+        return fail(ctx, BM_ETYPE, "%s: takes Q4_K or Q5_K gate and up stacks of one type, got types %d and %d; use bm_quantize and bm_gate_up",
+                    what, wg->wtype, wu->wtype);
     if (wu->k != wg->k || wu->rows != wg->rows)
         return fail(ctx, BM_ESHAPE, "%s: gate is %lld x %d, up %lld x %d", what, (long long)wg->rows, wg->k, (long long)wu->rows, wu->k);
     const int hidden = wg->k, ff = rows_per_expert;
@@ -507,8 +507,10 @@ int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const
         return fail(ctx, BM_EARG, "%s: NULL argument", what);
     if (wg->wtype != wu->wtype)
         return fail(ctx, BM_ETYPE, "%s: gate is type %d and up type %d; one launch reads one type", what, wg->wtype, wu->wtype);
-    if (!bmk::moe_decode_supported(wg->wtype, wd->wtype))
-        return fail(ctx, BM_ETYPE, "%s: the single launch takes Q4_K gate/up with Q6_K or Q4_K down, got %d and %d; use the separate launches",
+    if (!bmk::moe_decode_supported(ctx->decode_plan, wg->wtype, wd->wtype))
+        return fail(ctx, BM_ETYPE,
+                    "%s: the fused step takes Q4_K or Q5_K gate/up with Q4_K, Q5_K or Q6_K down (as one launch: Q4_K with Q6_K or Q4_K), got %d "
+                    "and %d; use the separate launches",
                     what, wg->wtype, wd->wtype);
     if (wu->k != wg->k || wu->rows != wg->rows)
         return fail(ctx, BM_ESHAPE, "%s: gate is %lld x %d, up %lld x %d", what, (long long)wg->rows, wg->k, (long long)wu->rows, wu->k);
@@ -713,7 +715,7 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
     if (!ctx || !w || !act || !route || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
     if (!route->filled) return fail(ctx, BM_ESHAPE, "%s: a filled route table (bm_route_fill first)", what);
     if (!bmk::gemm_supported(w->wtype))
-        return fail(ctx, BM_ETYPE, "%s: weight type %d has no grouped GEMM here (Q4_K and Q6_K do); use the tile launchers", what, w->wtype);
+        return fail(ctx, BM_ETYPE, "%s: weight type %d has no grouped GEMM here (Q4_K, Q5_K and Q6_K do); use the tile launchers", what, w->wtype);
     int rc = check_pair(ctx, what, w, act);
     if (rc) return rc;
     if (rows_per_expert <= 0 || rows_per_expert % 16 != 0)

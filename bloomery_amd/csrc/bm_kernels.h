@@ -66,8 +66,8 @@ hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_expe
 //   kPlanTwoLaunches: gate . up with the quantizers folded in, then down + combine (no counters).
 constexpr int kPlanOneLaunch = 1, kPlanTwoLaunches = 2;
 constexpr int kMaxDecodeTokens = 1024;
-bool moe_decode_supported(int gate_type, int down_type);
-// gate . up . SwiGLU from f32 token rows, both quantizers folded in (Q4_K gate/up): the first launch of
+bool moe_decode_supported(int plan, int gate_type, int down_type);
+// gate . up . SwiGLU from f32 token rows, both quantizers folded in (Q4_K or Q5_K gate/up): the first launch of
 // kPlanTwoLaunches.
 hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8_t *wg, const uint8_t *wu,
                      int n_experts, int hidden, int ff, const uint32_t *sel, int slots_per_token, int m,

@@ -669,8 +669,9 @@ hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_expe
     return hipGetLastError();
 }
 
-bool moe_decode_supported(int gate_type, int down_type) {
-    return gate_type == BM_Q4K && (down_type == BM_Q6K || down_type == BM_Q4K);
+bool moe_decode_supported(int plan, int gate_type, int down_type) {
+    if (plan == kPlanOneLaunch) return gate_type == BM_Q4K && (down_type == BM_Q6K || down_type == BM_Q4K);
+    return (gate_type == BM_Q4K || gate_type == BM_Q5K) && (down_type == BM_Q4K || down_type == BM_Q5K || down_type == BM_Q6K);
 }
 
 hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8_t *wg, const uint8_t *wu,
@@ -679,17 +680,23 @@ hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8
     const int nba = hidden / 256, nbb = ff / 256, spt = slots_per_token;
     const size_t lds_a = (size_t)act_col_bytes(gate_type, hidden) + 32 * sizeof(float);
     const unsigned grid_a = (unsigned)m * (unsigned)spt * (unsigned)(ff / 32);
-    if (gate_type != BM_Q4K) return hipErrorInvalidValue;
-#define BM_GUX(UA, NA)                                                                                                 \
+#define BM_GUX(WA, UA, NA)                                                                                             \
     {                                                                                                                  \
-        auto kern = k_gate_up_x<BM_Q4K, UA, NA>;                                                                       \
+        auto kern = k_gate_up_x<WA, UA, NA>;                                                                           \
         hipError_t e = allow_lds(kern, lds_a);                                                                         \
         if (e != hipSuccess) return e;                                                                                 \
         hipLaunchKernelGGL(kern, dim3(grid_a), dim3(256), lds_a, L.stream, x, wg, wu, (u32)n_experts, nba, nbb, sel,   \
                            spt, act_x, act_h, h, L.rule, L.fault, L.layer);                                            \
     }
-    if (nba == 8) BM_GUX(kRingQ4K, 8)
-    else BM_GUX(1, 0)
+    if (gate_type == BM_Q4K) {
+        if (nba == 8) BM_GUX(BM_Q4K, kRingQ4K, 8)
+        else BM_GUX(BM_Q4K, 1, 0)
+    } else if (gate_type == BM_Q5K) {
+        if (nba == 8) BM_GUX(BM_Q5K, kRingQ5K, 8)
+        else BM_GUX(BM_Q5K, 1, 0)
+    } else {
+        return hipErrorInvalidValue;
+    }
 #undef BM_GUX
     return hipGetLastError();
 }
@@ -703,7 +710,7 @@ hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, c
     const size_t lds_a = (size_t)act_col_bytes(gate_type, hidden) + 32 * sizeof(float);
     const size_t lds_b = down_combine_lds(down_type, ff, spt);
     const unsigned grid_a = (unsigned)m * (unsigned)spt * (unsigned)(ff / 32);
-    if (gate_type != BM_Q4K) return hipErrorInvalidValue;
+    if (!moe_decode_supported(plan, gate_type, down_type)) return hipErrorInvalidValue;
     if (plan == kPlanTwoLaunches) {
         hipError_t e = gate_up_x(L, gate_type, x, wg, wu, n_experts, hidden, ff, sel, spt, m, act_x, act_h, h);
         if (e != hipSuccess) return e;

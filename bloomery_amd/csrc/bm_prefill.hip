@@ -201,7 +201,9 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
     }
     if (tid < kZeroPage / 4) reinterpret_cast<u32 *>(zeros)[tid] = 0u;
     __syncthreads();
-    constexpr int kBlock = WT == BM_Q4K ? BM_Q4K_BLOCK : BM_Q6K_BLOCK;
+    constexpr int kBlock = bm_block_bytes<WT>();
+    constexpr bool kQ45 = WT == BM_Q4K || WT == BM_Q5K; // one walk: Q5_K is Q4_K with a fifth bit a code
+    constexpr int kCodesAt = WT == BM_Q5K ? 48 : 16;    // where a Q4_K / Q5_K block's nibbles start
     const u32 row_bytes = (u32)nb * kBlock, col_bytes = (u32)nb * BM_Q82_SB_EXT;
 
     // What a thread stages of every super-block: kActLoads 16-byte chunks of the activations (a column's super-block
@@ -231,9 +233,12 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
 #pragma unroll
         for (int t = 0; t < kActLoads; t++) ra[t] = *reinterpret_cast<const uint4 *>(act + (src_a[t] + (u32)i * step_a[t]));
         const uint8_t *blk = we + (src_w + (u32)i * kBlock);
-        if constexpr (WT == BM_Q4K) {
-            rw = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * pc);
+        if constexpr (kQ45) {
+            rw = *reinterpret_cast<const uint4 *>(blk + kCodesAt + 16 * pc);
             if (pc == 0) rhd = *reinterpret_cast<const uint4 *>(blk); // d, dmin, the twelve scale bytes
+            // Q5_K: value n's fifth bit is bit n / 32 of high byte n % 32 (crates/gguf/src/quant.rs:769-816); these
+            // code bytes hold values 64 (pc / 2) + 16 (pc % 2) .. and the values 32 on
+            if constexpr (WT == BM_Q5K) rqh = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * (pc & 1));
         } else { // half pc / 4: its ql bytes 16 (pc % 4) .. and the qh bytes that go with them
             rw = bm_ld16u(blk + 64 * (pc >> 2) + 16 * (pc & 3));
             rqh = bm_ld16u(blk + 128 + 32 * (pc >> 2) + 16 * (pc & 1));
@@ -252,11 +257,20 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
         const u32 ml = 0x0f0f0f0fu;
         uint8_t *codes = buf + kWtsAt + wr * kRowStride;
         float *rs = reinterpret_cast<float *>(buf + kRsAt); // [16][kRsStride]
-        if constexpr (WT == BM_Q4K) {
+        if constexpr (kQ45) {
             // code bytes 16 pc ..: values 64 (pc / 2) + 16 (pc % 2) .. (low nibbles) and 32 on (high nibbles)
             uint8_t *dst = codes + 64 * (pc >> 1) + 16 * (pc & 1);
-            put16(dst, rw.x & ml, rw.y & ml, rw.z & ml, rw.w & ml);
-            put16(dst + 32, (rw.x >> 4) & ml, (rw.y >> 4) & ml, (rw.z >> 4) & ml, (rw.w >> 4) & ml);
+            if constexpr (WT == BM_Q5K) {
+                const u32 one = 0x01010101u;
+                const int s0 = 2 * (pc >> 1), s1 = s0 + 1; // the sub-blocks of the low and of the high nibbles
+                put16(dst, (rw.x & ml) | (((rqh.x >> s0) & one) << 4), (rw.y & ml) | (((rqh.y >> s0) & one) << 4),
+                      (rw.z & ml) | (((rqh.z >> s0) & one) << 4), (rw.w & ml) | (((rqh.w >> s0) & one) << 4));
+                put16(dst + 32, ((rw.x >> 4) & ml) | (((rqh.x >> s1) & one) << 4), ((rw.y >> 4) & ml) | (((rqh.y >> s1) & one) << 4),
+                      ((rw.z >> 4) & ml) | (((rqh.z >> s1) & one) << 4), ((rw.w >> 4) & ml) | (((rqh.w >> s1) & one) << 4));
+            } else {
+                put16(dst, rw.x & ml, rw.y & ml, rw.z & ml, rw.w & ml);
+                put16(dst + 32, (rw.x >> 4) & ml, (rw.y >> 4) & ml, (rw.z >> 4) & ml, (rw.w >> 4) & ml);
+            }
             // the row's header from the lane that read it; scale and min of sub-block pc
             // (crates/gguf/src/quant.rs:620-628 get_scale_min_k4)
             const int from = 4 * (lane & ~7);
@@ -313,7 +327,7 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
         const float2 *pair[T]; // (d8, d8 * isum) a 32-block
 #pragma unroll
         for (int t = 0; t < T; t++) pair[t] = reinterpret_cast<const float2 *>(buf + my_act[t] + BM_Q82_SB_REF);
-        if constexpr (WT == BM_Q4K) {
+        if constexpr (kQ45) {
             // the min terms first: accumulator l takes sub-block l's (crates/qdot/src/lib.rs:4389-4394)
 #pragma unroll
             for (int s = 0; s < 8; s++) {
@@ -341,8 +355,8 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
             }
 #pragma unroll
             for (int h = 0; h < 2; h++) {
-                // Q4_K: one scale a block; Q6_K: one a group (crates/qdot/src/lib.rs:4403-4440, :4794-4809)
-                const float4 sv = *reinterpret_cast<const float4 *>(&rs[(WT == BM_Q4K ? bk : 2 * bk + h) * kRsStride + rbase]);
+                // Q4_K, Q5_K: one scale a block; Q6_K: one a group (crates/qdot/src/lib.rs:4403-4440, :4794-4809)
+                const float4 sv = *reinterpret_cast<const float4 *>(&rs[(kQ45 ? bk : 2 * bk + h) * kRsStride + rbase]);
                 const int l = 4 * h + (bk & 3);
 #pragma unroll
                 for (int t = 0; t < T; t++) {
@@ -590,7 +604,7 @@ __global__ __launch_bounds__(256) void k_gemm_fast(const uint8_t *w, int rpe, in
     }
 }
 
-bool gemm_supported(int wtype) { return wtype == BM_Q4K || wtype == BM_Q6K; }
+bool gemm_supported(int wtype) { return wtype == BM_Q4K || wtype == BM_Q5K || wtype == BM_Q6K; }
 
 hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int rows_per_expert, int k,
                 const uint8_t *act, const uint32_t *cols, const uint32_t *tiles_dev, const uint32_t *n_tiles, int n_slots,
@@ -608,15 +622,15 @@ hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int
                            n_units, (u32)slot_div, (u32)n_slots, y);
         return hipGetLastError();
     };
-    if (mode == 1) {
+    if (mode == 1) { // Q5_K has no kernel of this kind and takes the exact one
         if (wtype == BM_Q4K) return launch(k_gemm_fast<BM_Q4K>, 256, gemm_lds_bytes<BM_Q4K>(), 1);
         if (wtype == BM_Q6K) return launch(k_gemm_fast<BM_Q6K>, 256, gemm_lds_bytes<BM_Q6K>(), 1);
-        return hipErrorInvalidValue;
     }
     // 512 threads on 32 slots of a tile for both types (Q4_K 114 registers, Q6_K 121): two workgroups a CU. Measured
     // against 1024 threads on all 64 slots (Q4_K gate 362 -> 342 us), 512 threads with two slot groups a wave on 64
     // (Q6_K down 489 -> 407 us), and 256 threads on 16 or 32 slots (slower: the rows are staged once a workgroup).
     if (wtype == BM_Q4K) return launch(k_gemm<BM_Q4K, 1, 2>, 512, gemm_exact_lds_bytes(32), 2);
+    if (wtype == BM_Q5K) return launch(k_gemm<BM_Q5K, 1, 2>, 512, gemm_exact_lds_bytes(32), 2);
     if (wtype == BM_Q6K) return launch(k_gemm<BM_Q6K, 1, 2>, 512, gemm_exact_lds_bytes(32), 2);
     return hipErrorInvalidValue;
 }

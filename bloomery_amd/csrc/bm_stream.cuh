@@ -380,7 +380,7 @@ static hipError_t allow_lds(K kernel, size_t lds) {
 // Picks the kernel variant for a row of nb super-blocks and runs CALL_BODY with WT, U and NB as constants. Each
 // type lists the hot shape first (its count known at compile time, stages unrolled), then a ring of two for even
 // counts, then one super-block at a time, which divides every row.
-constexpr int kRingQ4K = 4, kRingQ6K = 3;
+constexpr int kRingQ4K = 4, kRingQ5K = 4, kRingQ6K = 3;
 #define BM_VARIANT(T, UU, NN)                                                                                          \
     {                                                                                                                  \
         constexpr int WT = T, U = UU, NB = NN;                                                                         \
@@ -394,7 +394,8 @@ constexpr int kRingQ4K = 4, kRingQ6K = 3;
         else BM_VARIANT(BM_Q4K, 1, 0)                                                                                  \
         break;                                                                                                         \
     case BM_Q5K:                                                                                                       \
-        if ((nb) % 2 == 0) BM_VARIANT(BM_Q5K, 2, 0)                                                                    \
+        if ((nb) == 8) BM_VARIANT(BM_Q5K, kRingQ5K, 8)                                                                 \
+        else if ((nb) % 2 == 0) BM_VARIANT(BM_Q5K, 2, 0)                                                                    \
         else BM_VARIANT(BM_Q5K, 1, 0)                                                                                  \
         break;                                                                                                         \
     case BM_Q6K:                                                                                                       \

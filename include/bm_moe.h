@@ -168,8 +168,8 @@ int bm_down_combine(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const u
  * reference, whose step is the chain quantize, gate_up, quantize, down, combine: dispatch.rs:1245-1436): x_dev
  * holds m rows of hidden = wg's k f32 values (16-byte aligned); token t's slots are sel_dev / w_dev[t *
  * n_slots_per_token ..]; y_dev[t * hidden + d] gets bm_combine_tokens' value. Same bits as bm_quantize, bm_gate_up
- * (with act_h) and bm_down_combine run one after the other. Gate/up must be Q4_K, down Q6_K or Q4_K; other types
- * take the separate launches. act_h is caller-held scratch (m * n_slots_per_token Q8_2_X4 columns of ff = wd's k)
+ * (with act_h) and bm_down_combine run one after the other. Gate/up must be Q4_K or Q5_K, down Q4_K, Q5_K or Q6_K
+ * (BM_PLAN_ONE_LAUNCH: Q4_K gate/up, Q6_K or Q4_K down); other types take the separate launches. act_h is caller-held scratch (m * n_slots_per_token Q8_2_X4 columns of ff = wd's k)
  * and holds the quantized h afterwards; act_x (optional) receives the quantized x columns; h_dev (optional) the
  * f32 h rows. m <= 1024.
  * Two plans (bm_set_decode_plan):
@@ -185,7 +185,7 @@ int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const
                   bm_act *act_h, bm_act *act_x, float *h_dev, float *y_dev);
 int bm_set_decode_plan(bm_ctx *ctx, int plan);
 /* The first launch of BM_PLAN_TWO_LAUNCHES on its own: bm_quantize, bm_gate_up and the quantizer of h in one
- * launch, from the f32 token rows (Q4_K gate/up; rows_per_expert = ff a multiple of 256). Follow it with
+ * launch, from the f32 token rows (Q4_K or Q5_K gate/up; rows_per_expert = ff a multiple of 256). Follow it with
  * bm_down_combine or bm_gemv_sel over act_h. */
 int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const float *x_dev, const uint32_t *sel_dev,
                  int n_slots_per_token, int m, int rows_per_expert, bm_act *act_h, bm_act *act_x, float *h_dev);
@@ -246,7 +246,7 @@ int bm_route_fill(bm_ctx *ctx, const uint32_t *ids_dev, int n_slots, bm_route *r
  * takes the n_slots slot list (refused slots last); tiles_host (optional) two words a tile: expert, then
  * first index | length << 16. */
 int bm_route_read(bm_ctx *ctx, const bm_route *route, uint32_t *cols_host, uint32_t *tiles_host, int *n_tiles, int *n_refused);
-/* GemmKernels::enqueue_gemm(GemmArgs) (crates/gpu/src/gemm/grouped.rs:2125-2133,2300), Q4_K and Q6_K stacks:
+/* GemmKernels::enqueue_gemm(GemmArgs) (crates/gpu/src/gemm/grouped.rs:2125-2133,2300), Q4_K, Q5_K and Q6_K stacks:
  * y_dev[s * rows_per_expert + r] = row r of expert e(s) . column c(s) of act for every slot s of the table's last
  * fill; c(s) = s / top_k (GemmInput::Shared) or s when top_k is 0 (GemmInput::PerSlot). rows_per_expert a
  * multiple of 16. Every value is bm_gemv_sel's for that slot, bit for bit; the integer sums are formed on the int8

@@ -380,9 +380,20 @@ def run_single_launch(gpu, L, x, ids, wts, top_k, resid=None, replays=1, plan=bm
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 1024, 512, 6, 3, 6),    # 64 / 6 rows a consumer workgroup: a ragged tail
     ((bm.Q4_K, bm.Q4_K, bm.Q4_K), 512, 512, 5, 4, 2),
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 4096, 256, 4, 2, 3),    # rows longer than one quantizer pass
+    ((bm.Q5_K, bm.Q5_K, bm.Q6_K), 2048, 512, 4, 3, 4),    # Q5_K gate/up at the whole-row shape (two launches only)
+    ((bm.Q5_K, bm.Q5_K, bm.Q5_K), 768, 256, 3, 2, 2),
 ))
 @pytest.mark.parametrize("plan", (bm.PLAN_ONE_LAUNCH, bm.PLAN_TWO_LAUNCHES))
 def test_single_launch_step_matches_the_chain_and_the_oracle(gpu, types, hidden, ff, n_experts, m, top_k, plan):
+    if types[0] == bm.Q5_K and plan == bm.PLAN_ONE_LAUNCH:  # that plan takes Q4_K gate/up only and says so
+        L = Layer(gpu, types, hidden, ff, n_experts, 600 + hidden + ff, cheap=True)
+        x = np.zeros((m, hidden), np.float32)
+        with pytest.raises(bm.GpuError) as e:
+            run_single_launch(gpu, L, x, np.zeros((m, top_k), np.uint32), np.ones((m, top_k), np.float32), top_k, plan=plan)
+        assert e.value.code == bm.ETYPE and "bm_moe_decode" in str(e.value)
+        gpu.set_decode_plan(bm.PLAN_TWO_LAUNCHES)
+        L.free()
+        return
     L = Layer(gpu, types, hidden, ff, n_experts, 600 + hidden + ff)
     rng = np.random.default_rng(601)
     x = normal_f32(rng, (m, hidden))

@@ -102,6 +102,7 @@ def test_gemm_fast_mode_is_within_the_tolerance(gpu):
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 6, 70, 3, False),      # runs past 64 slots: several tiles an expert
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 16, 48, 8, True),     # config 4's layer shape, 384 slots
     ((bm.Q6_K, bm.Q6_K, bm.Q4_K), 768, 512, 3, 9, 2, False),       # the other type on each side; ragged tiles
+    ((bm.Q5_K, bm.Q5_K, bm.Q5_K), 768, 512, 3, 40, 2, False),      # Q5_K on both sides: the Q4_K walk with a fifth bit
 ))
 def test_prefill_layer_matches_the_oracle(gpu, types, hidden, ff, n_experts, m, top_k, cheap):
     L = Layer(gpu, types, hidden, ff, n_experts, 2000 + hidden, cheap=cheap)
@@ -127,7 +128,7 @@ def test_prefill_layer_matches_the_oracle(gpu, types, hidden, ff, n_experts, m, 
 def test_gemm_rows_not_a_whole_slab_and_refused_slots(gpu):
     """rows_per_expert = 80 (a multiple of 16, a slab and a quarter); a refused id gets NaN rows and ExpertId."""
     rng = np.random.default_rng(2100)
-    for wtype, k in ((bm.Q4_K, 1024), (bm.Q6_K, 768)):
+    for wtype, k in ((bm.Q4_K, 1024), (bm.Q5_K, 512), (bm.Q6_K, 768)):
         rpe, n_experts, n_slots = 80, 4, 23
         w = stack(wtype, n_experts * rpe, k, 2101)
         ids = rng.integers(0, n_experts, n_slots).astype(np.uint32)

@@ -1,5 +1,5 @@
 // TEST INFRASTRUCTURE ONLY (see ora_common.h). AVX2+FMA+F16C restatement of the reference's vector kernels, in
-// their instruction order: the two activation encoders and the Q4_K / Q6_K / IQ2_XXS row dots, one column or a
+// their instruction order: the two activation encoders and the Q4_K / Q5_K / Q6_K / IQ2_XXS / IQ4_XS row dots, one column or a
 // tile of up to eight columns that unpacks each weight block once. It has two uses: the test suite holds it
 // bit-equal to the scalar restatement in qdot.c (two independently written paths through the same arithmetic,
 // the reference's own first gate, crates/qdot/tests/qdot.rs:346,738,818,2664), and the benchmark times it as the
@@ -157,7 +157,7 @@ int ora_avx2_quantize_q8k(const float *x, int k, uint8_t *out) {
 
 int ora_avx2_quantize_col(int wtype, const float *x, int k, uint8_t *out) {
     if (wtype == ORA_TYPE_Q4_K || wtype == ORA_TYPE_Q5_K || wtype == ORA_TYPE_Q6_K) return ora_avx2_quantize_q82x4(x, k, out);
-    if (wtype == ORA_TYPE_IQ2_XXS) return ora_avx2_quantize_q8k(x, k, out);
+    if (ora_takes_q8k(wtype)) return ora_avx2_quantize_q8k(x, k, out);
     return ORA_ETYPE;
 }
 
@@ -405,6 +405,46 @@ static void dot_iq2xxs_tile(const uint8_t *wrow, const uint8_t *const *acols, in
     for (int c = 0; c < C; c++) out[c] = hsum_float_8(accd[c]);
 }
 
+// -------------------------------------------------------------------------------------------------- IQ4_XS tile
+
+// One IQ4_XS row against C <= 8 columns (crates/qdot/src/lib.rs:11062-11145): a sub-block's 32 levels come out of one
+// byte shuffle of the sixteen-entry table (low nibbles in the low half, high nibbles in the high half), a level's
+// magnitude goes to maddubs' unsigned side and its sign onto the activation byte, the pairs are scaled by the
+// sub-block's scale in madd and added into eight i32 lanes; one fmadd a super-block.
+static void dot_iq4xs_tile(const uint8_t *wrow, const uint8_t *const *acols, int C, int nb, float *out) {
+    const __m256i m4 = _mm256_set1_epi8(0x0f);
+    const __m128i t128 = _mm_loadu_si128((const __m128i *)ORA_KVALUES_IQ4NL);
+    const __m256i table = _mm256_set_m128i(t128, t128);
+    __m256 accd[8];
+    for (int c = 0; c < C; c++) accd[c] = _mm256_setzero_ps();
+    for (int i = 0; i < nb; i++) {
+        const uint8_t *blk = wrow + (size_t)i * ORA_IQ4XS_BLOCK;
+        float d = ora_half_to_f32(ora_rd16(blk));
+        uint32_t scales_h = ora_rd16(blk + 2);
+        __m256i values[8], scales[8];
+        for (int b = 0; b < 8; b++) {
+            __m128i aux = _mm_loadu_si128((const __m128i *)(blk + 8 + 16 * b));
+            __m256i nib = _mm256_and_si256(_mm256_set_m128i(_mm_srli_epi16(aux, 4), aux), m4);
+            values[b] = _mm256_shuffle_epi8(table, nib);
+            int ls = ((blk[4 + b / 2] >> (4 * (b % 2))) & 0x0f) | (int)(((scales_h >> (2 * b)) & 3) << 4);
+            scales[b] = _mm256_set1_epi16((short)(ls - 32));
+        }
+        for (int c = 0; c < C; c++) {
+            const uint8_t *col = acols[c] + (size_t)i * ORA_Q8K_STRIDE;
+            float dy;
+            memcpy(&dy, col, 4);
+            __m256i sumi = _mm256_setzero_si256();
+            for (int b = 0; b < 8; b++) {
+                __m256i q8 = _mm256_loadu_si256((const __m256i *)(col + 8 + 32 * b));
+                __m256i pair = _mm256_maddubs_epi16(_mm256_sign_epi8(values[b], values[b]), _mm256_sign_epi8(q8, values[b]));
+                sumi = _mm256_add_epi32(sumi, _mm256_madd_epi16(scales[b], pair));
+            }
+            accd[c] = _mm256_fmadd_ps(_mm256_set1_ps(d * dy), _mm256_cvtepi32_ps(sumi), accd[c]);
+        }
+    }
+    for (int c = 0; c < C; c++) out[c] = hsum_float_8(accd[c]);
+}
+
 // ----------------------------------------------------------------------------------------------------- dispatch
 
 // dot_row_cols (crates/qdot/src/lib.rs:905): 1..=8 columns, every value the one-column kernel's.
@@ -425,6 +465,9 @@ int ora_avx2_dot_row_cols(int wtype, const uint8_t *wrow, const uint8_t *const *
     case ORA_TYPE_IQ2_XXS:
         pthread_once(&keven_once, keven_init);
         dot_iq2xxs_tile(wrow, acols, cols, nb, out);
+        return 0;
+    case ORA_TYPE_IQ4_XS:
+        dot_iq4xs_tile(wrow, acols, cols, nb, out);
         return 0;
     default:
         return ORA_ETYPE;
@@ -533,7 +576,7 @@ int ora_avx2_moe_forward(ora_pool *p, const ora_moe_layer *L, const float *x, in
     if (cb_g < 0 || cb_u < 0 || cb_d < 0) return ORA_ESHAPE;
     for (int s = 0; s < n_slots; s++)
         if (ids[s] >= (uint32_t)L->n_experts) return ORA_ESHAPE;
-    int same_enc = (L->gate_type == ORA_TYPE_IQ2_XXS) == (L->up_type == ORA_TYPE_IQ2_XXS);
+    int same_enc = ora_takes_q8k(L->gate_type) == ora_takes_q8k(L->up_type);
     uint8_t *ag = (uint8_t *)malloc((size_t)cb_g * m), *au = same_enc ? ag : (uint8_t *)malloc((size_t)cb_u * m);
     uint8_t *ad = (uint8_t *)malloc((size_t)cb_d * n_slots);
     float *g = (float *)malloc(sizeof(float) * (size_t)ff * n_slots);

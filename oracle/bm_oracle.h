@@ -29,7 +29,7 @@ extern "C" {
 
 // Refusals (the reference panics or returns QdotError, crates/qdot/src/lib.rs:127-160).
 #define ORA_EUNALIGNED (-1) // k is not a whole number of 256-value super-blocks
-#define ORA_ETYPE (-2)      // weight type outside {Q4_K = 12, Q5_K = 13, Q6_K = 14, IQ2_XXS = 16}
+#define ORA_ETYPE (-2)      // weight type outside {Q4_K = 12, Q5_K = 13, Q6_K = 14, IQ2_XXS = 16, IQ4_XS = 23}
 #define ORA_ESHORTROW (-3)
 #define ORA_ESHORTCOL (-4)
 #define ORA_ENONFINITE (-5) // an activation value that is not finite
@@ -47,6 +47,7 @@ float ora_dot_q4k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb);
 float ora_dot_q5k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb);
 float ora_dot_q6k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb);
 float ora_dot_iq2xxs_q8k(const uint8_t *wrow, const uint8_t *acol, int nb);
+float ora_dot_iq4xs_q8k(const uint8_t *wrow, const uint8_t *acol, int nb);
 int ora_dot_row(int wtype, const uint8_t *wrow, size_t wrow_len, const uint8_t *acol, size_t acol_len, int k,
                 float *out);
 int ora_gemv(int wtype, const uint8_t *w, int rows, int k, const uint8_t *act, int m, float *y);
@@ -56,6 +57,8 @@ void ora_q5k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_
 void ora_q6k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int fold, int32_t *s_out);
 void ora_iq2xxs_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_t *i_out, int32_t *sc_out,
                            int32_t *codes_out, int32_t *fold_out);
+void ora_iq4xs_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int fold, int32_t *i_out,
+                          int32_t *lanes_out);
 
 int ora_dequant_row(int wtype, const uint8_t *src, int k, float *dst);
 int ora_dequant_col(int wtype, const uint8_t *acol, int k, float *dst);

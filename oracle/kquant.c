@@ -325,8 +325,10 @@ static void *qworker(void *arg) {
             j->rc = ora_quantize_row_q5k(xr, j->k, o);
         else if (j->wtype == ORA_TYPE_Q6_K)
             j->rc = ora_quantize_row_q6k(xr, j->k, o);
-        else
+        else if (j->wtype == ORA_TYPE_IQ2_XXS)
             j->rc = ora_quantize_row_iq2xxs(xr, ones, j->k, o);
+        else
+            j->rc = ORA_ETYPE; // IQ4_XS has no quantizer in the reference's gguf crate, so none here
     }
     free(ones);
     return NULL;

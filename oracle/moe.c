@@ -132,7 +132,7 @@ int ora_moe_forward(const ora_moe_layer *L, const float *x, int m, const uint32_
     for (int s = 0; s < n_slots; s++)
         if (ids[s] >= (uint32_t)L->n_experts) return ORA_ESHAPE;
     // x quantized once per (token, encoding) (crates/model/src/ops.rs:554).
-    int same_enc = (L->gate_type == ORA_TYPE_IQ2_XXS) == (L->up_type == ORA_TYPE_IQ2_XXS);
+    int same_enc = ora_takes_q8k(L->gate_type) == ora_takes_q8k(L->up_type);
     uint8_t *ag = (uint8_t *)malloc((size_t)cb_g * m), *au = same_enc ? ag : (uint8_t *)malloc((size_t)cb_u * m);
     uint8_t *ad = (uint8_t *)malloc((size_t)cb_d);
     float *g = (float *)malloc(sizeof(float) * ff), *u = (float *)malloc(sizeof(float) * ff);

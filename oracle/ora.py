@@ -11,8 +11,9 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libbm_oracle.so")
 
-Q4_K, Q5_K, Q6_K, IQ2_XXS = 12, 13, 14, 16
-BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ2_XXS: 66}
+Q4_K, Q5_K, Q6_K, IQ2_XXS, IQ4_XS = 12, 13, 14, 16, 23
+BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ2_XXS: 66, IQ4_XS: 136}
+Q8K_TYPES = (IQ2_XXS, IQ4_XS)  # the types whose activation column is ik's Q8_K; the others take Q8_2_X4
 
 EUNALIGNED, ETYPE, ESHORTROW, ESHORTCOL, ENONFINITE, ESHAPE, ESTATUS = -1, -2, -3, -4, -5, -6, -7
 
@@ -49,6 +50,7 @@ def _load():
         "ora_q6k_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
         "ora_iq2xxs_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
                                          C.c_void_p]),
+        "ora_iq4xs_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
         "ora_dequant_row": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
         "ora_dequant_col": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
         "ora_expf_ik": (C.c_float, [C.c_float]),
@@ -180,6 +182,15 @@ def iq2xxs_block_sums(wrow, acol, k):
     fold = np.empty(nb, np.int32)
     lib.ora_iq2xxs_block_sums(_p(_u8(wrow)), _p(_u8(acol)), nb, _p(i), _p(sc), _p(codes), _p(fold))
     return i, sc, codes, fold
+
+
+def iq4xs_block_sums(wrow, acol, k, fold=False):
+    """Per sub-block the sum of level * activation; per super-block the eight scaled lane sums the CPU path holds."""
+    nb = k // 256
+    i = np.empty(nb * 8, np.int32)
+    lanes = np.empty(nb * 8, np.int32)
+    lib.ora_iq4xs_block_sums(_p(_u8(wrow)), _p(_u8(acol)), nb, int(fold), _p(i), _p(lanes))
+    return i, lanes
 
 
 def dequant_row(wtype, src, k):

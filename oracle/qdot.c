@@ -78,6 +78,7 @@ int ora_col_bytes(int wtype, int k) {
     case ORA_TYPE_Q6_K:
         return k / 128 * ORA_Q82X4_STRIDE;
     case ORA_TYPE_IQ2_XXS:
+    case ORA_TYPE_IQ4_XS:
         return k / 256 * ORA_Q8K_STRIDE;
     default:
         return ORA_ETYPE;
@@ -95,6 +96,8 @@ int ora_row_bytes(int wtype, int k) {
         return k / 256 * ORA_Q6K_BLOCK;
     case ORA_TYPE_IQ2_XXS:
         return k / 256 * ORA_IQ2XXS_BLOCK;
+    case ORA_TYPE_IQ4_XS:
+        return k / 256 * ORA_IQ4XS_BLOCK;
     default:
         return ORA_ETYPE;
     }
@@ -107,6 +110,7 @@ int ora_quantize_col(int wtype, const float *x, int k, uint8_t *out) {
     case ORA_TYPE_Q6_K:
         return ora_quantize_q82x4(x, k, out);
     case ORA_TYPE_IQ2_XXS:
+    case ORA_TYPE_IQ4_XS:
         return ora_quantize_q8k(x, k, out);
     default:
         return ORA_ETYPE;
@@ -377,6 +381,69 @@ void ora_iq2xxs_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int
     }
 }
 
+// ---------------------------------------------------------------------------------------------------- IQ4_XS dot
+
+// Sub-block b's 6-bit scale less 32: nibble b % 2 of scales_l[b / 2] under bits 2b.. of scales_h
+// (crates/gguf/src/quant.rs:1989-1991, crates/qdot/src/lib.rs:11158-11160).
+static inline int iq4xs_scale(const uint8_t *blk, int b) {
+    int lo = (blk[4 + b / 2] >> (4 * (b % 2))) & 0x0f, hi = (ora_rd16(blk + 2) >> (2 * b)) & 3;
+    return (lo | (hi << 4)) - 32;
+}
+
+// Level n (0..32) of sub-block b: values 0..15 are the low nibbles of its sixteen bytes, 16..31 the high ones.
+static inline int iq4xs_value(const uint8_t *blk, int b, int n) {
+    uint8_t byte = blk[8 + 16 * b + (n % 16)];
+    return ORA_KVALUES_IQ4NL[n < 16 ? (byte & 0x0f) : (byte >> 4)];
+}
+
+// IQ4_XS x Q8_K, the scalar mirror's steps in its order (crates/qdot/src/lib.rs:11147-11180). The vector kernel puts
+// a level's magnitude on the unsigned side and folds its sign into the activation byte; -(-128) wraps there, so a
+// -128 code under a negative level counts as -128 (ik's Q8_K encoder never writes one).
+float ora_dot_iq4xs_q8k(const uint8_t *wrow, const uint8_t *acol, int nb) {
+    float accd[8] = {0};
+    for (int i = 0; i < nb; i++) {
+        const uint8_t *blk = wrow + (size_t)i * ORA_IQ4XS_BLOCK;
+        const uint8_t *col = acol + (size_t)i * ORA_Q8K_STRIDE;
+        float d = ora_half_to_f32(ora_rd16(blk));
+        float dy = ora_bits_f32(ora_rd32(col));
+        int32_t sumi[8] = {0};
+        for (int b = 0; b < 8; b++) {
+            int scale = iq4xs_scale(blk, b);
+            for (int n = 0; n < 32; n++) {
+                int w = iq4xs_value(blk, b, n);
+                int8_t a = (int8_t)col[8 + 32 * b + n];
+                int8_t q = w < 0 ? (int8_t)(uint8_t)(0u - (uint8_t)a) : (w == 0 ? 0 : a);
+                sumi[n / 4] += scale * (w < 0 ? -w : w) * (int32_t)q;
+            }
+        }
+        for (int l = 0; l < 8; l++) accd[l] = fmaf(d * dy, (float)sumi[l], accd[l]);
+    }
+    float t[4] = {accd[0] + accd[4], accd[1] + accd[5], accd[2] + accd[6], accd[3] + accd[7]};
+    return (t[0] + t[2]) + (t[1] + t[3]);
+}
+
+// Per super-block: I[b] = sum over sub-block b of level * a, and the eight lane sums L[l] = sum_b scale_b * (sum over
+// values 4l .. 4l + 3 of sub-block b of level * a) the reference's i32 lanes hold. `fold` counts a -128 code under a
+// negative level as the vector kernel's sign fold does (see the dot above); without it the products are plain.
+void ora_iq4xs_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int fold, int32_t *i_out,
+                          int32_t *lanes_out) {
+    for (int i = 0; i < nb; i++) {
+        const uint8_t *blk = wrow + (size_t)i * ORA_IQ4XS_BLOCK;
+        const uint8_t *col = acol + (size_t)i * ORA_Q8K_STRIDE;
+        for (int l = 0; l < 8; l++) lanes_out[8 * i + l] = 0;
+        for (int b = 0; b < 8; b++) {
+            int32_t sum = 0;
+            for (int n = 0; n < 32; n++) {
+                int32_t w = iq4xs_value(blk, b, n), a = (int8_t)col[8 + 32 * b + n];
+                int32_t p = (fold && w < 0 && a == -128) ? w * 128 : w * a;
+                sum += p;
+                lanes_out[8 * i + n / 4] += iq4xs_scale(blk, b) * p;
+            }
+            i_out[8 * i + b] = sum;
+        }
+    }
+}
+
 // ----------------------------------------------------------------------------------------------------- dispatch
 
 // crates/qdot/src/lib.rs:691-723 with check_row's refusals (:1727-1779) as return codes.
@@ -400,6 +467,9 @@ int ora_dot_row(int wtype, const uint8_t *wrow, size_t wrow_len, const uint8_t *
         return 0;
     case ORA_TYPE_IQ2_XXS:
         *out = ora_dot_iq2xxs_q8k(wrow, acol, nb);
+        return 0;
+    case ORA_TYPE_IQ4_XS:
+        *out = ora_dot_iq4xs_q8k(wrow, acol, nb);
         return 0;
     default:
         return ORA_ETYPE;
@@ -460,6 +530,13 @@ int ora_dequant_row(int wtype, const uint8_t *src, int k, float *dst) {
                     out[32 * b + n] = db * mag * (v < 0 ? -1.0f : 1.0f);
                 }
             }
+        } else if (wtype == ORA_TYPE_IQ4_XS) { // crates/gguf/src/quant.rs:1977-1999
+            const uint8_t *blk = src + (size_t)i * ORA_IQ4XS_BLOCK;
+            float d = ora_half_to_f32(ora_rd16(blk));
+            for (int b = 0; b < 8; b++) {
+                float dl = d * (float)iq4xs_scale(blk, b);
+                for (int n = 0; n < 32; n++) out[32 * b + n] = dl * (float)iq4xs_value(blk, b, n);
+            }
         } else {
             return ORA_ETYPE;
         }
@@ -470,7 +547,7 @@ int ora_dequant_row(int wtype, const uint8_t *src, int k, float *dst) {
 // Decoded value of one activation column (code times its block scale), for the f64 band checks.
 int ora_dequant_col(int wtype, const uint8_t *acol, int k, float *dst) {
     if (k <= 0 || k % 256 != 0) return ORA_EUNALIGNED;
-    if (wtype == ORA_TYPE_IQ2_XXS) {
+    if (ora_takes_q8k(wtype)) {
         for (int b = 0; b < k / 256; b++) {
             const uint8_t *o = acol + (size_t)b * ORA_Q8K_STRIDE;
             float d = ora_bits_f32(ora_rd32(o));

@@ -61,3 +61,34 @@ def max_abs_normalised(got, want):
     got = np.asarray(got, np.float64)
     denom = np.max(np.abs(want))
     return float(np.max(np.abs(got - want)) / (denom if denom > 0 else 1.0))
+
+
+KVALUES_IQ4NL = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.int64)
+
+
+def iq4xs_rows(x):
+    """IQ4_XS blocks (136 bytes a 256 values, crates/gguf/src/quant.rs:1969-1976) standing for the f32 rows x: a
+    test-side generator, nearest level under one scale a 32 values. The reference's gguf crate has no IQ4_XS
+    quantizer to follow; the tests only need blocks whose values look like weights, and every byte pattern is a legal
+    block."""
+    x = np.asarray(x, np.float32).reshape(-1, 256)
+    out = np.zeros((x.shape[0], 136), np.uint8)
+    for i, blk in enumerate(x):
+        sub = blk.reshape(8, 32).astype(np.float64)
+        amax = np.abs(sub).max(axis=1)
+        d = np.float16(amax.max() / (127.0 * 31.0))
+        df = float(d)
+        ls = np.zeros(8, np.int64) if df == 0.0 else np.clip(np.rint(amax / (127.0 * df)), 1, 31).astype(np.int64)
+        codes = np.zeros((8, 32), np.int64)
+        for b in range(8):
+            if df != 0.0:
+                codes[b] = np.abs(sub[b][:, None] / (df * ls[b]) - KVALUES_IQ4NL[None, :]).argmin(axis=1)
+        stored = ls + 32
+        out[i, 0:2] = np.array([d], np.float16).view(np.uint8)
+        sh = 0
+        for b in range(8):
+            sh |= int(stored[b] >> 4) << (2 * b)
+            out[i, 4 + b // 2] |= int(stored[b] & 15) << (4 * (b % 2))
+        out[i, 2], out[i, 3] = sh & 0xFF, sh >> 8
+        out[i, 8:136] = (codes[:, :16] | (codes[:, 16:] << 4)).astype(np.uint8).reshape(-1)
+    return out.reshape(-1)

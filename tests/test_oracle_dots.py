@@ -13,10 +13,10 @@ import numpy as np
 import pytest
 
 import ora
-from common import normal_f32
+from common import KVALUES_IQ4NL, iq4xs_rows, normal_f32
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-TYPES = (ora.Q4_K, ora.Q5_K, ora.Q6_K, ora.IQ2_XXS)
+TYPES = (ora.Q4_K, ora.Q5_K, ora.Q6_K, ora.IQ2_XXS, ora.IQ4_XS)
 
 
 # ---------------------------------------------------------------- independent numpy decoders (written from the
@@ -104,12 +104,27 @@ def iq2xxs_decode(blk):
     return codes, vals, (d, scs)
 
 
-DECODE = {ora.Q4_K: q4k_decode, ora.Q5_K: q5k_decode, ora.Q6_K: q6k_decode, ora.IQ2_XXS: iq2xxs_decode}
+def iq4xs_decode(blk):
+    """block_iq4_xs (crates/gguf/src/quant.rs:1969-1976): d, scales_h, scales_l[4], then sixteen bytes a sub-block,
+    low nibbles its first sixteen values, high nibbles the other sixteen."""
+    d = f16(blk[0], blk[1])
+    sh = int(blk[2]) | (int(blk[3]) << 8)
+    ls = [(((int(blk[4 + b // 2]) >> (4 * (b % 2))) & 15) | (((sh >> (2 * b)) & 3) << 4)) - 32 for b in range(8)]
+    codes = np.zeros(256, np.int64)
+    for b in range(8):
+        q = blk[8 + 16 * b:24 + 16 * b].astype(np.int64)
+        codes[32 * b:32 * b + 16] = KVALUES_IQ4NL[q & 15]
+        codes[32 * b + 16:32 * b + 32] = KVALUES_IQ4NL[q >> 4]
+    vals = np.array([d * ls[n // 32] * codes[n] for n in range(256)], np.float64)
+    return codes, vals, (d, ls)
+
+
+DECODE = {ora.IQ4_XS: iq4xs_decode, ora.Q4_K: q4k_decode, ora.Q5_K: q5k_decode, ora.Q6_K: q6k_decode, ora.IQ2_XXS: iq2xxs_decode}
 
 
 def act_codes(wtype, col, k):
     """Integer codes and f64 scales of an activation column, read from its bytes."""
-    if wtype == ora.IQ2_XXS:
+    if wtype in ora.Q8K_TYPES:
         blocks = col.reshape(-1, 296)
         codes = np.concatenate([b[8:264].view(np.int8).astype(np.int64) for b in blocks])
         scale = np.concatenate([np.full(256, float(b[0:4].view(np.float32)[0])) for b in blocks])
@@ -127,7 +142,7 @@ def random_blocks(wtype, nb, rng):
     w = rng.integers(0, 256, nb * bb, dtype=np.uint8)
     for i in range(nb):
         h = np.array([rng.uniform(-0.1, 0.1), rng.uniform(0.0, 0.1)], np.float16).view(np.uint8)
-        off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0}[wtype]
+        off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ4_XS: 0}[wtype]
         w[i * bb + off:i * bb + off + 2] = h[0:2]
         if wtype in (ora.Q4_K, ora.Q5_K):
             w[i * bb + 2:i * bb + 4] = h[2:4]
@@ -137,6 +152,8 @@ def random_blocks(wtype, nb, rng):
 def quantized_rows(wtype, rows, k, seed):
     rng = np.random.default_rng(seed)
     x = normal_f32(rng, (rows, k), 0.02)
+    if wtype == ora.IQ4_XS:
+        return iq4xs_rows(x), x
     return ora.quantize_rows(wtype, x, rows, k, n_threads=4), x
 
 
@@ -149,6 +166,24 @@ def test_codebook_digests_and_closed_form():
         assert hashlib.md5(struct.pack("<256Q", *grid)).hexdigest() == "fff55639176d84643cf2facd7a655c4d", path
         assert all(ks[i] == (i | ((bin(i).count("1") & 1) << 7)) for i in range(128)), path
         assert all(((g >> (8 * j)) & 0xFF) in (8, 25, 43) for g in grid for j in range(8)), path
+
+
+def test_iq4_levels_digest():
+    # crates/gguf/src/iq_tables.rs:432-436: md5 over the sixteen bytes; the shipped headers hold the same sixteen
+    assert hashlib.md5(KVALUES_IQ4NL.astype(np.int8).tobytes()).hexdigest() == "5dc4c90c34afd4f896578cb08cb33249"
+    import re
+    for path in ("oracle/iq_tables.h", "bloomery_amd/csrc/iq2xxs_tables.h"):
+        text = open(os.path.join(HERE, "..", path)).read()
+        body = re.search(r"KVALUES_IQ4NL\[16\] = \{(.*?)\};", text, re.S).group(1)
+        assert [int(v) for v in re.findall(r"-?\d+", body)] == list(KVALUES_IQ4NL), path
+    # every level times every block scale is exact in f32 (crates/gguf/src/quant.rs:2693-2700), so the decoder's f64
+    # product and the oracle's f32 one agree to the bit
+    for bits in range(0, 0x7C00, 37):
+        d = np.array([bits], np.uint16).view(np.float16).astype(np.float32)[0]
+        for ls in (-32, -7, 1, 31):
+            dl = np.float32(d * np.float32(ls))
+            assert float(dl) == float(d) * ls
+            assert all(float(np.float32(dl * np.float32(kv))) == float(dl) * int(kv) for kv in KVALUES_IQ4NL)
 
 
 def test_iq2xxs_decodes_the_ggml_made_block():
@@ -194,6 +229,15 @@ def test_block_sums_equal_brute_force(wtype):
             want = [int(prod[16 * g:16 * g + 16].sum()) for g in range(nb * 16)]
             assert list(ora.q6k_block_sums(w, col, k)) == want
             assert list(ora.q6k_block_sums(w, col, k, fold=True)) == want, "no -128 code on these inputs"
+        elif wtype == ora.IQ4_XS:
+            i_b, lanes = ora.iq4xs_block_sums(w, col, k)
+            assert list(i_b) == [int(prod[32 * b:32 * b + 32].sum()) for b in range(nb * 8)]
+            for i in range(nb):
+                ls = DECODE[wtype](w[i * bb:(i + 1) * bb])[2][1]
+                want = [sum(ls[b] * int(prod[256 * i + 32 * b + 4 * l:256 * i + 32 * b + 4 * l + 4].sum()) for b in range(8))
+                        for l in range(8)]
+                assert list(lanes[8 * i:8 * i + 8]) == want
+            assert ora.iq4xs_block_sums(w, col, k, fold=True)[1].tolist() == lanes.tolist(), "no -128 code on these inputs"
         else:
             i_b, sc, codes, fold = ora.iq2xxs_block_sums(w, col, k)
             assert list(i_b) == [int(prod[32 * b:32 * b + 32].sum()) for b in range(nb * 8)]
@@ -224,6 +268,40 @@ def test_q6k_sign_fold_differs_only_at_minus_128():
     assert not np.array_equal(plain, fold)
 
 
+def test_iq4xs_sign_fold_differs_only_at_minus_128():
+    # The reference's IQ4_XS kernel folds a level's sign into the activation byte (crates/qdot/src/lib.rs:11127-11131);
+    # -(-128) wraps, so a -128 code under a negative level counts with the wrong sign there and nowhere else. ik's
+    # Q8_K encoder never writes -128, so the column is hand-made: random codes with -128 among them.
+    rng = np.random.default_rng(6)
+    w = random_blocks(ora.IQ4_XS, 2, rng)
+    col = np.zeros(2 * 296, np.uint8)
+    for i in range(2):
+        col[296 * i:296 * i + 4] = np.array([0.01 * (i + 1)], np.float32).view(np.uint8)
+        codes = rng.integers(-128, 128, 256).astype(np.int8)
+        codes[rng.integers(0, 256, 24)] = -128
+        col[296 * i + 8:296 * i + 264] = codes.view(np.uint8)
+    a, _ = act_codes(ora.IQ4_XS, col, 512)
+    plain = ora.iq4xs_block_sums(w, col, 512)[1]
+    fold = ora.iq4xs_block_sums(w, col, 512, fold=True)[1]
+    want = np.zeros(16, np.int64)
+    for i in range(2):
+        lv, _, (_, ls) = iq4xs_decode(w[136 * i:136 * (i + 1)])
+        for n in range(256):
+            if a[256 * i + n] == -128 and lv[n] < 0:
+                want[8 * i + (n % 32) // 4] += -256 * ls[n // 32] * int(lv[n])
+    assert (plain.astype(np.int64) - fold).tolist() == want.tolist() and want.any()
+    # both restatements of the dot carry the fold: same bits, and the value the folded lanes give
+    got = ora.dot_row(ora.IQ4_XS, w, col, 512)
+    assert got.tobytes() == ora.dot_row(ora.IQ4_XS, w, col, 512, avx2=True).tobytes()
+    acc = np.zeros(8, np.float32)
+    for i in range(2):
+        d = np.float32(f16(w[136 * i], w[136 * i + 1])) * col[296 * i:296 * i + 4].view(np.float32)[0]
+        for l in range(8):
+            acc[l] = np.float32(np.float64(d) * np.float64(np.float32(fold[8 * i + l])) + np.float64(acc[l]))
+    t = [np.float32(acc[l] + acc[l + 4]) for l in range(4)]
+    assert np.float32(np.float32(t[0] + t[2]) + np.float32(t[1] + t[3])) == got
+
+
 # ------------------------------------------------------------------------------------------------------ fp32 dots
 
 def extreme_cases(wtype, rng):
@@ -234,7 +312,7 @@ def extreme_cases(wtype, rng):
         w = np.full(2 * bb, fill, np.uint8)
         for i in range(2):
             h = np.array([dval, abs(dval)], np.float16).view(np.uint8)
-            off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0}[wtype]
+            off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ4_XS: 0}[wtype]
             w[i * bb + off:i * bb + off + 2] = h[0:2]
             if wtype in (ora.Q4_K, ora.Q5_K):
                 w[i * bb + 2:i * bb + 4] = h[2:4]
@@ -307,7 +385,7 @@ def test_dot_within_f64_band_of_dequantized_dot(wtype):
             a_codes, a_scale = act_codes(wtype, col, k)
             act = a_codes * a_scale
             dq = ora.dequant_col(wtype, col, k).astype(np.float64)
-            if wtype == ora.IQ2_XXS:
+            if wtype in ora.Q8K_TYPES:
                 assert np.allclose(dq, act, rtol=1e-7, atol=0)  # an f32 scale times a code rounds once
             else:
                 assert np.array_equal(dq, act), "a bf16 scale times an 8-bit code is exact in f32"

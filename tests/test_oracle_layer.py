@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import ora
-from common import max_abs_normalised, normal_f32
+from common import iq4xs_rows, max_abs_normalised, normal_f32
 
 
 # ----------------------------------------------------------------------------------------------- expf and SwiGLU
@@ -263,14 +263,17 @@ def test_iq2xxs_rows_quantize_and_read_back():
 
 def small_layer(types, hidden, ff, n_experts, seed):
     rng = np.random.default_rng(seed)
-    wg = ora.quantize_rows(types[0], normal_f32(rng, (n_experts * ff, hidden), 0.02), n_experts * ff, hidden)
-    wu = ora.quantize_rows(types[1], normal_f32(rng, (n_experts * ff, hidden), 0.02), n_experts * ff, hidden)
-    wd = ora.quantize_rows(types[2], normal_f32(rng, (n_experts * hidden, ff), 0.02), n_experts * hidden, ff)
-    return wg, wu, wd
+
+    def rows(wtype, n, k):
+        x = normal_f32(rng, (n, k), 0.02)
+        return iq4xs_rows(x) if wtype == ora.IQ4_XS else ora.quantize_rows(wtype, x, n, k)
+
+    return rows(types[0], n_experts * ff, hidden), rows(types[1], n_experts * ff, hidden), rows(types[2], n_experts * hidden, ff)
 
 
 @pytest.mark.parametrize("types,hidden,ff", (((ora.Q4_K, ora.Q4_K, ora.Q6_K), 512, 256),
-                                             ((ora.IQ2_XXS, ora.IQ2_XXS, ora.IQ2_XXS), 512, 256)))
+                                             ((ora.IQ2_XXS, ora.IQ2_XXS, ora.IQ2_XXS), 512, 256),
+                                             ((ora.IQ4_XS, ora.IQ4_XS, ora.Q5_K), 512, 256)))
 def test_layer_forms_agree_and_track_f64(types, hidden, ff):
     n_experts, top_k, m = 6, 3, 4
     wg, wu, wd = small_layer(types, hidden, ff, n_experts, 77)

@@ -30,11 +30,13 @@ typedef uint32_t u32;
 #define BM_Q5K 13
 #define BM_Q6K 14
 #define BM_IQ2XXS 16
+#define BM_IQ4XS 23
 
 #define BM_Q4K_BLOCK 144
 #define BM_Q5K_BLOCK 176
 #define BM_Q6K_BLOCK 210
 #define BM_IQ2XXS_BLOCK 66
+#define BM_IQ4XS_BLOCK 136
 #define BM_Q82X4_STRIDE 144
 #define BM_Q8K_STRIDE 296
 #define BM_Q82_SB_REF 288 // reference bytes of one super-block of a Q8_2_X4 column
@@ -160,6 +162,8 @@ struct NoTap {
     __device__ __forceinline__ void q4k_isum(int, int, int) const {}
     __device__ __forceinline__ void q6k(int, int, int) const {}
     __device__ __forceinline__ void iq2(int, int, int, int) const {}
+    __device__ __forceinline__ void iq4_sub(int, int, int) const {}
+    __device__ __forceinline__ void iq4_lane(int, int, int) const {}
 };
 
 // ------------------------------------------------------------------------------------------ activation view
@@ -171,15 +175,18 @@ struct ActView {
     const uint8_t *s16; // nb * 16 i32 sums of 16 stored codes
 };
 
+// The types that dot against a Q8_K column (crates/gguf/src/qtype.rs host_act); the others take Q8_2_X4.
+__host__ __device__ constexpr bool bm_takes_q8k(int wt) { return wt == BM_IQ2XXS || wt == BM_IQ4XS; }
+
 // Bytes of one column of nb super-blocks on the device, in the form type WT dots against.
 template <int WT>
 __host__ __device__ constexpr int bm_act_col_bytes(int nb) {
-    return WT == BM_IQ2XXS ? nb * BM_Q8K_STRIDE : nb * BM_Q82_SB_EXT;
+    return bm_takes_q8k(WT) ? nb * BM_Q8K_STRIDE : nb * BM_Q82_SB_EXT;
 }
 
 template <int WT>
 __device__ __forceinline__ ActView bm_act_view(const uint8_t *col, int nb) {
-    if (WT == BM_IQ2XXS) return ActView{col, nullptr, nullptr};
+    if (bm_takes_q8k(WT)) return ActView{col, nullptr, nullptr};
     return ActView{col, col + (size_t)nb * BM_Q82_SB_REF, col + (size_t)nb * (BM_Q82_SB_REF + 64)};
 }
 
@@ -532,10 +539,122 @@ __device__ __forceinline__ void bm_dot_iq2xxs(const Blk<BM_IQ2XXS> &b, const Act
     bm_dot_iq2xxs_dec(b, dec, act, i, q, acc0, acc1, tap);
 }
 
+// ---- IQ4_XS (crates/qdot/src/lib.rs:11033-11180): lane q reads sub-blocks 2q and 2q + 1 whole (32 consecutive code
+// bytes) and their 64 activation codes, turns the nibbles into levels with byte permutes of the sixteen-entry table,
+// and forms its share of the CPU path's eight i32 lanes: lane l of those sums, scale by scale, the values 4l .. 4l + 3
+// of every sub-block (low nibbles of code bytes 4l .., then for l >= 4 the high nibbles of bytes 4 (l - 4) ..). The
+// quad adds the shares up (integers: any order) and lane q applies the f32 step to accumulators 2q and 2q + 1.
+template <>
+struct Blk<BM_IQ4XS> {
+    uint4 qa, qb; // the code bytes of sub-blocks 2q and 2q + 1
+    uint2 hd;     // d | scales_h << 16, scales_l
+};
+
+__device__ __forceinline__ Blk<BM_IQ4XS> bm_load_iq4xs(const uint8_t *wrow, int i, int q) {
+    const uint8_t *blk = wrow + (size_t)i * BM_IQ4XS_BLOCK;
+    Blk<BM_IQ4XS> b;
+    b.hd = *reinterpret_cast<const uint2 *>(blk);
+    b.qa = bm_ld16u(blk + 8 + 32 * q);
+    b.qb = bm_ld16u(blk + 24 + 32 * q);
+    return b;
+}
+
+template <>
+struct Act<BM_IQ4XS> {
+    float dy;
+    uint2 a[8]; // the 64 codes of sub-blocks 2q and 2q + 1
+};
+
+__device__ __forceinline__ Act<BM_IQ4XS> bm_act_iq4xs(const ActView &av, int i, int q) {
+    const uint8_t *blk = av.col + (size_t)i * BM_Q8K_STRIDE;
+    Act<BM_IQ4XS> a;
+    a.dy = *reinterpret_cast<const float *>(blk);
+#pragma unroll
+    for (int k = 0; k < 8; k++) a.a[k] = *reinterpret_cast<const uint2 *>(blk + 8 + 64 * q + 8 * k);
+    return a;
+}
+
+// Four 4-bit codes, one in the low nibble of each byte of x >> shift, as four levels: the table's low and high halves
+// through one byte permute each (selector: the code's low three bits), then a third that takes byte k from the high
+// half where code k has its top bit set.
+template <int SHIFT>
+__device__ __forceinline__ u32 bm_iq4_levels(u32 x) {
+    constexpr u32 t0 = bm_iq4_levels_word(0), t1 = bm_iq4_levels_word(1), t2 = bm_iq4_levels_word(2), t3 = bm_iq4_levels_word(3);
+    const u32 s = (x >> SHIFT) & 0x07070707u;
+    const u32 lo = __builtin_amdgcn_perm(t1, t0, s), hi = __builtin_amdgcn_perm(t3, t2, s);
+    const u32 pick = ((x >> (SHIFT + 1)) & 0x04040404u) | 0x03020100u;
+    return __builtin_amdgcn_perm(hi, lo, pick);
+}
+
+// The block's levels as this lane dots them, decoded once a super-block whatever the number of columns.
+struct Iq4Dec {
+    u32 lo[2][4], hi[2][4]; // sub-block 2q + e: levels of values 4j .. (low nibbles) and 16 + 4j .. (high nibbles)
+    int sc[2];
+};
+
+__device__ __forceinline__ Iq4Dec bm_decode_iq4xs(const Blk<BM_IQ4XS> &b, int q) {
+    Iq4Dec dec;
+    const u32 qw[2][4] = {{b.qa.x, b.qa.y, b.qa.z, b.qa.w}, {b.qb.x, b.qb.y, b.qb.z, b.qb.w}};
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            dec.lo[e][j] = bm_iq4_levels<0>(qw[e][j]);
+            dec.hi[e][j] = bm_iq4_levels<4>(qw[e][j]);
+        }
+        // crates/gguf/src/quant.rs:1989-1991: nibble b % 2 of scales_l[b / 2] under bits 2b .. of scales_h, less 32;
+        // sub-blocks 2q, 2q + 1 are the two nibbles of scales_l[q]
+        const u32 sl = (b.hd.y >> (8 * q + 4 * e)) & 15u, sh = (b.hd.x >> (16 + 4 * q + 2 * e)) & 3u;
+        dec.sc[e] = (int)(sl | (sh << 4)) - 32;
+    }
+    return dec;
+}
+
+template <class Tap>
+__device__ __forceinline__ void bm_dot_iq4xs_dec(const Blk<BM_IQ4XS> &b, const Iq4Dec &dec, const Act<BM_IQ4XS> &act, int i,
+                                                 int q, float &acc0, float &acc1, const Tap &tap) {
+    int lanes[8];
+#pragma unroll
+    for (int e = 0; e < 2; e++) {
+        int sub = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            // values 4j .. 4j + 3 of the sub-block are word j % 2 of its code group j / 2; 16 + 4j .. of group 2 + j / 2
+            const uint2 alo = act.a[4 * e + (j >> 1)], ahi = act.a[4 * e + 2 + (j >> 1)];
+            const int p_lo = bm_sdot4(dec.lo[e][j], (j & 1) ? alo.y : alo.x, 0);
+            const int p_hi = bm_sdot4(dec.hi[e][j], (j & 1) ? ahi.y : ahi.x, 0);
+            lanes[j] = e ? lanes[j] + dec.sc[1] * p_lo : dec.sc[0] * p_lo;
+            lanes[4 + j] = e ? lanes[4 + j] + dec.sc[1] * p_hi : dec.sc[0] * p_hi;
+            sub += p_lo + p_hi;
+        }
+        tap.iq4_sub(i, 2 * q + e, sub);
+    }
+    // the quad's four shares of each lane sum
+#pragma unroll
+    for (int l = 0; l < 8; l++) {
+        lanes[l] += (int)bm_dpp<kDppXor1>((u32)lanes[l]);
+        lanes[l] += (int)bm_dpp<kDppXor2>((u32)lanes[l]);
+        if (q == 0) tap.iq4_lane(i, l, lanes[l]);
+    }
+    const int s0 = q == 0 ? lanes[0] : (q == 1 ? lanes[2] : (q == 2 ? lanes[4] : lanes[6]));
+    const int s1 = q == 0 ? lanes[1] : (q == 1 ? lanes[3] : (q == 2 ? lanes[5] : lanes[7]));
+    // one fused multiply-add a super-block and lane (crates/qdot/src/lib.rs:11171-11173)
+    const float f = bm_half_to_f32(b.hd.x & 0xffffu) * act.dy;
+    acc0 = fmaf(f, (float)s0, acc0);
+    acc1 = fmaf(f, (float)s1, acc1);
+}
+
+template <class Tap>
+__device__ __forceinline__ void bm_dot_iq4xs(const Blk<BM_IQ4XS> &b, const Act<BM_IQ4XS> &act, int i, int q, float &acc0,
+                                             float &acc1, const Tap &tap) {
+    const Iq4Dec dec = bm_decode_iq4xs(b, q);
+    bm_dot_iq4xs_dec(b, dec, act, i, q, acc0, acc1, tap);
+}
+
 // ---- closing sums: (t0 + t2) + (t1 + t3) with t_l = acc_l + acc_{l+4}; every lane of the quad gets the value.
 template <int WT>
 __device__ __forceinline__ float bm_quad_finish(float acc0, float acc1) {
-    // lane ^ 2 holds acc_{l+4} (Q4_K, Q6_K: the other half h; IQ2_XXS: lane q + 2 owns l + 4)
+    // lane ^ 2 holds acc_{l+4} (Q4_K, Q5_K, Q6_K: the other half h; IQ2_XXS, IQ4_XS: lane q + 2 owns l + 4)
     const float x = acc0 + bm_quad_xor2(acc0), y = acc1 + bm_quad_xor2(acc1);
     if (WT == BM_Q6K) {
         // lane c holds t_c and t_{c+2}
@@ -566,6 +685,10 @@ template <>
 __device__ __forceinline__ Blk<BM_IQ2XXS> bm_load_blk<BM_IQ2XXS>(const uint8_t *wrow, int i, int q) {
     return bm_load_iq2xxs(wrow, i, q);
 }
+template <>
+__device__ __forceinline__ Blk<BM_IQ4XS> bm_load_blk<BM_IQ4XS>(const uint8_t *wrow, int i, int q) {
+    return bm_load_iq4xs(wrow, i, q);
+}
 
 template <int WT, bool WithSums>
 __device__ __forceinline__ Act<WT> bm_load_act(const ActView &av, int i, int q) {
@@ -577,6 +700,8 @@ __device__ __forceinline__ Act<WT> bm_load_act(const ActView &av, int i, int q) 
         return a;
     } else if constexpr (WT == BM_Q6K)
         return bm_act_q6k(av, i, q & 1, q >> 1);
+    else if constexpr (WT == BM_IQ4XS)
+        return bm_act_iq4xs(av, i, q);
     else
         return bm_act_iq2xxs(av, i, q);
 }
@@ -590,13 +715,15 @@ __device__ __forceinline__ void bm_dot_blk(const Blk<WT> &b, const Act<WT> &a, i
         bm_dot_q5k(b, a, i, q & 1, q >> 1, acc0, acc1, tap);
     else if constexpr (WT == BM_Q6K)
         bm_dot_q6k(b, a, i, q & 1, q >> 1, acc0, acc1, tap);
+    else if constexpr (WT == BM_IQ4XS)
+        bm_dot_iq4xs(b, a, i, q, acc0, acc1, tap);
     else
         bm_dot_iq2xxs(b, a, i, q, tb, acc0, acc1, tap);
 }
 
 template <int WT>
 __host__ __device__ constexpr int bm_block_bytes() {
-    return WT == BM_Q4K ? BM_Q4K_BLOCK : WT == BM_Q5K ? BM_Q5K_BLOCK : WT == BM_Q6K ? BM_Q6K_BLOCK : BM_IQ2XXS_BLOCK;
+    return WT == BM_Q4K ? BM_Q4K_BLOCK : WT == BM_Q5K ? BM_Q5K_BLOCK : WT == BM_Q6K ? BM_Q6K_BLOCK : WT == BM_IQ4XS ? BM_IQ4XS_BLOCK : BM_IQ2XXS_BLOCK;
 }
 
 // ---- SwiGLU: crates/qdot/src/lib.rs:3741-3773 (expf) and :11467-11478 (divide, then multiply).

@@ -96,7 +96,7 @@ __global__ __launch_bounds__(256) void k_quantize_q8k(const float *x, int m, int
 }
 
 hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, uint8_t *act, const uint32_t *live) {
-    if (wtype == BM_IQ2XXS) {
+    if (bm_takes_q8k(wtype)) {
         hipLaunchKernelGGL(k_quantize_q8k, dim3((unsigned)(m * (k / 256))), dim3(256), 0, L.stream, x, m, k, act,
                            live, L.fault, L.layer);
     } else {
@@ -555,6 +555,8 @@ struct StoreTap {
         atomicAdd(&out[16 * i + b], v);
         (void)q;
     }
+    __device__ __forceinline__ void iq4_sub(int i, int b, int v) const { out[16 * i + b] = v; }
+    __device__ __forceinline__ void iq4_lane(int i, int l, int v) const { out[16 * i + 8 + l] = v; }
 };
 
 template <int WT, int U, int NB>
@@ -590,7 +592,7 @@ __global__ __launch_bounds__(64) void k_block_sums(const uint8_t *wrow, int nb, 
 
 int act_col_bytes(int wtype, int k) {
     const int nb = k / 256;
-    return wtype == BM_IQ2XXS ? nb * BM_Q8K_STRIDE : nb * BM_Q82_SB_EXT;
+    return bm_takes_q8k(wtype) ? nb * BM_Q8K_STRIDE : nb * BM_Q82_SB_EXT;
 }
 
 int gemv_max_cols(int wtype, int k) {

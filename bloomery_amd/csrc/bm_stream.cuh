@@ -169,6 +169,14 @@ __device__ __forceinline__ void row_dot(Blk<WT> (&b)[U], const uint8_t *wrow, co
                         const Act<WT> a = bm_load_act<WT, Tap::kActive>(av[c], i, q);
                         bm_dot_iq2xxs_dec(b[slot], dec, a, i, q, a0[c], a1[c], tap);
                     }
+            } else if constexpr (WT == BM_IQ4XS) { // likewise the level permutes
+                const Iq4Dec dec = bm_decode_iq4xs(b[slot], q);
+#pragma unroll
+                for (int c = 0; c < M; c++)
+                    if (c < m) {
+                        const Act<WT> a = bm_load_act<WT, Tap::kActive>(av[c], i, q);
+                        bm_dot_iq4xs_dec(b[slot], dec, a, i, q, a0[c], a1[c], tap);
+                    }
             } else {
 #pragma unroll
                 for (int c = 0; c < M; c++)
@@ -406,6 +414,10 @@ constexpr int kRingQ4K = 4, kRingQ5K = 4, kRingQ6K = 3;
     case BM_IQ2XXS:                                                                                                    \
         if ((nb) % 2 == 0) BM_VARIANT(BM_IQ2XXS, 2, 0)                                                                 \
         else BM_VARIANT(BM_IQ2XXS, 1, 0)                                                                               \
+        break;                                                                                                         \
+    case BM_IQ4XS:                                                                                                     \
+        if ((nb) % 2 == 0) BM_VARIANT(BM_IQ4XS, 2, 0)                                                                  \
+        else BM_VARIANT(BM_IQ4XS, 1, 0)                                                                                \
         break;                                                                                                         \
     default:                                                                                                           \
         return hipErrorInvalidValue;                                                                                   \

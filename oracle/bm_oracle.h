@@ -1,5 +1,5 @@
 // TEST INFRASTRUCTURE ONLY. CPU oracle of the quantized MoE expert-matmul path: a plain C restatement of the
-// reference's crates/qdot (activation encoders, Q4_K / Q5_K / Q6_K / IQ2_XXS row dots, SwiGLU), crates/gguf (block
+// reference's crates/qdot (activation encoders, Q4_K / Q5_K / Q6_K / IQ2_XXS / IQ4_XS row dots, SwiGLU), crates/gguf (block
 // layouts, dequantizers, K-quant and IQ2_XXS weight quantizers) and the caller-side router/combine order of
 // crates/model/src/moe.rs. Each function cites the reference lines it follows. The shipped library never links
 // or calls this; the test suite, the smoke check and the benchmark's CPU-baseline leg do.
@@ -11,7 +11,8 @@
 //   integer sums    brute-force sums over independently decoded codes in the test suite;
 //   fp32 dots       bit-equality with an AVX2-intrinsics restatement of the reference's vector kernels (its own
 //                   first gate) and an f64 band around the dequantized dot;
-//   dequantizers    the reference's ggml-made IQ2_XXS block (66 bytes -> 256 f32 bit patterns), table digests;
+//   dequantizers    the reference's ggml-made IQ2_XXS block (66 bytes -> 256 f32 bit patterns), table digests,
+//                   independent decoders written from the layout text in the test suite (all five types);
 //   expf / SwiGLU   libm band and special-case paths;
 //   weight quantizers   PARITY UNPINNED as bytes: the reference holds no golden bytes for them (it pins them
 //                   against ggml on its own machine). They are held to the reference tests' round-trip bounds,

@@ -36,13 +36,23 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def make_layer(ora, seed, threads):
-    """The layer's expert stacks: fp32 N(0, 0.02) quantized by the repo's K-quant rules (Q4_K, Q6_K `_ref`)."""
+def make_layer(ora, seed, threads, gate_type=None, down_type=None):
+    """The layer's expert stacks: fp32 N(0, 0.02) quantized by the repo's K-quant rules (Q4_K, Q5_K, Q6_K `_ref`);
+    IQ4_XS, for which the reference has no quantizer, as random legal blocks with small scales."""
     rng = np.random.default_rng(seed)
+    gate_type = ora.Q4_K if gate_type is None else gate_type
+    down_type = ora.Q6_K if down_type is None else down_type
     out = []
-    for wtype, rows, k in ((ora.Q4_K, N_EXPERTS * FF, HIDDEN), (ora.Q4_K, N_EXPERTS * FF, HIDDEN),
-                           (ora.Q6_K, N_EXPERTS * HIDDEN, FF)):
+    for wtype, rows, k in ((gate_type, N_EXPERTS * FF, HIDDEN), (gate_type, N_EXPERTS * FF, HIDDEN),
+                           (down_type, N_EXPERTS * HIDDEN, FF)):
         rb = ora.row_bytes(wtype, k)
+        if wtype == ora.IQ4_XS:
+            nb = rows * (k // 256)
+            w = rng.integers(0, 256, nb * 136, dtype=np.uint8).reshape(nb, 136)
+            d = rng.uniform(2e-6, 8e-6, nb).astype(np.float16).view(np.uint16)  # values d * (ls - 32) * level ~ 0.01
+            w[:, 0], w[:, 1] = d & 0xFF, d >> 8
+            out.append(w.reshape(-1))
+            continue
         q = np.empty(rows * rb, np.uint8)
         chunk = 8192
         for r0 in range(0, rows, chunk):
@@ -412,6 +422,9 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--types", default="q4_k,q6_k",
+                    help="config 2 only: gate/up and down weight types (q4_k, q5_k, q6_k, iq4_xs); other than the default is "
+                         "a side measurement of that type, not the headline workload")
     ap.add_argument("--mode", choices=("two", "single", "chain"), default="two",
                     help="two: bm_moe_decode in two launches (quantizers folded in); single: bm_moe_decode in one "
                          "launch; chain: quantize, gate_up, down_combine")
@@ -425,26 +438,43 @@ def main():
     threads = min(os.cpu_count() or 1, 16)
     if args.config != 2:
         return {1: bench_gemv, 3: bench_grouped, 4: bench_prefill, 5: bench_dsv3}[args.config](args, bm, ora, threads)
+    names = {"q4_k": bm.Q4_K, "q5_k": bm.Q5_K, "q6_k": bm.Q6_K, "iq4_xs": bm.IQ4_XS}
+    try:
+        gate_t, down_t = (names[v] for v in args.types.lower().split(","))
+    except (KeyError, ValueError):
+        sys.exit(f"bench.py: --types takes two of {sorted(names)} separated by a comma, got {args.types!r}")
+    label = {v: k.upper() for k, v in names.items()}
+    gate_n, down_n = label[gate_t], label[down_t]
+    q8k = (bm.IQ2_XXS, bm.IQ4_XS)
+    if args.mode != "chain" and (gate_t in q8k or down_t in q8k or gate_t == bm.Q6_K):
+        log(f"[bench] {gate_n} gate/up with {down_n} down has no fused step: timing the chain of launches")
+        args.mode = "chain"
+    if args.mode == "single" and (gate_t, down_t) != (bm.Q4_K, bm.Q6_K):
+        sys.exit("bench.py: --mode single takes the default types")
+    types3 = (gate_t, gate_t, down_t)
     t0 = time.time()
-    wg, wu, wd = make_layer(ora, 0xB1000001, threads)
+    wg, wu, wd = make_layer(ora, 0xB1000001, threads, gate_t, down_t)
     x, ids, wts = make_tokens(ora, args.tokens, 0xAC70001)
     log(f"[bench] layer quantized ({(wg.nbytes + wu.nbytes + wd.nbytes) / 1e6:.1f} MB) in {time.time() - t0:.1f}s")
 
     gpu = bm.Gpu(0)
     layers = []
     for _ in range(args.layers):
-        layers.append((gpu.weights(bm.Q4_K, N_EXPERTS * FF, HIDDEN, wg), gpu.weights(bm.Q4_K, N_EXPERTS * FF, HIDDEN, wu),
-                       gpu.weights(bm.Q6_K, N_EXPERTS * HIDDEN, FF, wd)))
+        layers.append((gpu.weights(gate_t, N_EXPERTS * FF, HIDDEN, wg), gpu.weights(gate_t, N_EXPERTS * FF, HIDDEN, wu),
+                       gpu.weights(down_t, N_EXPERTS * HIDDEN, FF, wd)))
     n_tok = args.tokens
     xd = gpu.upload(x, np.float32)
     sel = gpu.upload(ids, np.uint32)
     wt = gpu.upload(wts, np.float32)
     y = gpu.buffer(np.float32, n_tok * HIDDEN)
-    act = gpu.act(bm.Q4_K, HIDDEN, 1)
-    act_h = gpu.act(bm.Q6_K, FF, TOP_K)
+    act = gpu.act(gate_t, HIDDEN, 1)
+    act_h = gpu.act(down_t, FF, TOP_K)
+    fold_h = down_t not in q8k  # gate . up writes the down activation itself when that is a Q8_2_X4 column
+    h = None if fold_h else gpu.buffer(np.float32, TOP_K * FF)
 
     single = args.mode == "single"
-    kernels = {"single": ("step",), "two": ("gate_up_x", "down"), "chain": ("quant", "gate_up", "down")}[args.mode]
+    kernels = {"single": ("step",), "two": ("gate_up_x", "down"),
+               "chain": ("quant", "gate_up", "down") if fold_h else ("quant", "gate_up", "quant_h", "down")}[args.mode]
     gpu.set_decode_plan(bm.PLAN_ONE_LAUNCH if single else bm.PLAN_TWO_LAUNCHES)
 
     def enqueue_step(i, which=kernels):
@@ -462,7 +492,9 @@ def main():
         if "quant" in which:
             gpu.enqueue_quantize(xd.ptr + 4 * t * HIDDEN, 1, act)
         if "gate_up" in which:
-            gpu.enqueue_gate_up(dg, du, act, sel.ptr + 4 * t * TOP_K, TOP_K, FF, TOP_K, None, act_h)
+            gpu.enqueue_gate_up(dg, du, act, sel.ptr + 4 * t * TOP_K, TOP_K, FF, TOP_K, h, act_h if fold_h else None)
+        if "quant_h" in which:
+            gpu.enqueue_quantize(h, TOP_K, act_h)
         if "down" in which:
             gpu.enqueue_down_combine(dd, act_h, sel.ptr + 4 * t * TOP_K, wt.ptr + 4 * t * TOP_K, None, TOP_K, 1, HIDDEN,
                                      y.ptr + 4 * t * HIDDEN)
@@ -486,7 +518,7 @@ def main():
         for i in range(n_chk):
             enqueue_step(i)
         got = y.download()[:n_chk * HIDDEN].reshape(n_chk, HIDDEN)
-        want = ora.moe_forward(HIDDEN, FF, N_EXPERTS, (ora.Q4_K, ora.Q4_K, ora.Q6_K), wg, wu, wd, x[:n_chk], ids[:n_chk],
+        want = ora.moe_forward(HIDDEN, FF, N_EXPERTS, types3, wg, wu, wd, x[:n_chk], ids[:n_chk],
                                wts[:n_chk], TOP_K, n_threads=threads).reshape(n_chk, HIDDEN)
         err = float(np.max(np.abs(got.astype(np.float64) - want)) / np.max(np.abs(want)))
         parity = {"tokens": n_chk, "max_abs_normalised_err": err, "bit_identical": bool(np.array_equal(got, want))}
@@ -517,7 +549,7 @@ def main():
     ev_ms = gpu.event_elapsed_ms(e0, e1)
     ms_per_step = wall_ms / steps
     us_per_token = ms_per_step * 1e3
-    bytes_per_token = TOP_K * (2 * FF * bm.row_bytes(bm.Q4_K, HIDDEN) + HIDDEN * bm.row_bytes(bm.Q6_K, FF))
+    bytes_per_token = TOP_K * (2 * FF * bm.row_bytes(gate_t, HIDDEN) + HIDDEN * bm.row_bytes(down_t, FF))
 
     # per-kernel launch durations: a graph of one kernel only, over the same cycling inputs, between events on
     # the launch stream
@@ -536,15 +568,15 @@ def main():
         gpu.event_record(e1)
         kernel_us[name] = gpu.event_elapsed_ms(e0, e1) * 1e3 / (r * unit)
         gpu.graph_destroy(g1)
-    gate_up_bytes = TOP_K * 2 * FF * bm.row_bytes(bm.Q4_K, HIDDEN)
-    down_bytes = TOP_K * HIDDEN * bm.row_bytes(bm.Q6_K, FF)
+    gate_up_bytes = TOP_K * 2 * FF * bm.row_bytes(gate_t, HIDDEN)
+    down_bytes = TOP_K * HIDDEN * bm.row_bytes(down_t, FF)
     if single:
         dominant, dom_bytes = "k_moe_decode<Q4_K, Q6_K>", bytes_per_token
         achieved = dom_bytes / (kernel_us["step"] * 1e-6) / 1e9
         kernel_gbps = {"step": achieved}
     else:
         gk = "gate_up_x" if args.mode == "two" else "gate_up"
-        dominant, dom_bytes = ("k_gate_up_x<Q4_K>" if args.mode == "two" else "k_gate_up<Q4_K>"), gate_up_bytes
+        dominant, dom_bytes = (f"k_gate_up_x<{gate_n}>" if args.mode == "two" else f"k_gate_up<{gate_n}>"), gate_up_bytes
         achieved = dom_bytes / (kernel_us[gk] * 1e-6) / 1e9
         kernel_gbps = {gk: achieved, "down": down_bytes / (kernel_us["down"] * 1e-6) / 1e9}
     assert gpu.fault() == (bm.FAULT_NONE, 0)
@@ -554,11 +586,11 @@ def main():
         pool = ora.lib.ora_pool_create(threads)
         try:
             for i in range(3):
-                ora.moe_forward(HIDDEN, FF, N_EXPERTS, (ora.Q4_K, ora.Q4_K, ora.Q6_K), wg, wu, wd, x[i % n_tok],
+                ora.moe_forward(HIDDEN, FF, N_EXPERTS, types3, wg, wu, wd, x[i % n_tok],
                                 ids[i % n_tok], wts[i % n_tok], TOP_K, avx2_pool=pool)
             n, t_cpu = 0, time.perf_counter()
             while True:
-                ora.moe_forward(HIDDEN, FF, N_EXPERTS, (ora.Q4_K, ora.Q4_K, ora.Q6_K), wg, wu, wd, x[n % n_tok],
+                ora.moe_forward(HIDDEN, FF, N_EXPERTS, types3, wg, wu, wd, x[n % n_tok],
                                 ids[n % n_tok], wts[n % n_tok], TOP_K, avx2_pool=pool)
                 n += 1
                 el = time.perf_counter() - t_cpu
@@ -584,7 +616,9 @@ def main():
         "dtype": "i8",
         "data": "synthetic",
         "config": {"workload": "Qwen3-30B-A3B-shaped MoE layer decode, 1 token: hidden 2048, 128 experts x ff 768, "
-                               "Q4_K gate/up + Q6_K down, softmax top-8 renormalised (BASELINE.json configs[1])",
+                               f"{gate_n} gate/up + {down_n} down, softmax top-8 renormalised "
+                               + ("(BASELINE.json configs[1])" if (gate_t, down_t) == (bm.Q4_K, bm.Q6_K)
+                                  else "(BASELINE.json configs[1]'s shape with other weight types: a side measurement)"),
                    "layer_copies": len(layers), "distinct_tokens": n_tok, "launches_per_step": len(kernels), "mode": "hipGraph replay"},
         "hbm_tbps": bytes_per_token / (us_per_token * 1e-6) / 1e12,
         "algorithmic_bytes_per_token": bytes_per_token,
@@ -594,7 +628,7 @@ def main():
         "parity": parity,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": GATE_UP_X_TRAFFIC_BYTES if args.mode == "two" else None,
+                     "traffic": GATE_UP_X_TRAFFIC_BYTES if args.mode == "two" and gate_t == bm.Q4_K else None,
                      "algorithmic_bytes_per_launch": dom_bytes},
         "cpu_baseline": cpu,
     }

@@ -112,16 +112,19 @@ __device__ __forceinline__ void stage_tile_cols(uint8_t *cols, const uint8_t *ac
 // row (a quad on the gate row, a quad on the up row), all m columns in one pass over the two rows. Entry j + c reads
 // the activation column of the token of slot order[j + c] and writes h[(j + c) * rpe + r]: by entry, not by slot.
 // With act_h the 32 values of each column become block rb of column j + c of act_h in the same launch.
-template <int WT, int U, int NB>
+// MC: the columns this launch has LDS for; it takes the tiles of m_lo < m <= MC columns and leaves the others to the
+// launch of the other width (see tile_widths below).
+template <int WT, int U, int NB, int MC>
 __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const uint8_t *wu, u32 n_experts, int nb,
                                                        const uint8_t *act, int act_cols, const u32 *order,
                                                        const u32 *start, const u32 *tiles, u32 n_slots, u32 cap,
-                                                       int rpe, int slots_per_col, float *h, uint8_t *act_h,
+                                                       int rpe, int slots_per_col, float *h, uint8_t *act_h, int m_lo,
                                                        GateRule rule, u32 *fault, u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
     Tile t;
-    if (!tile_of_block(tiles, start, n_experts, n_slots, cap, &t, fault, layer)) return;
+    if (!tile_of_block(tiles, start, n_experts, n_slots, cap, &t, fault, layer)) return; // raising twice is raising once
+    if (t.m <= m_lo || t.m > MC) return;
     const int rb = t.row_block;
     const int r = rb * 32 + (tid >> 3);
     const bool active = r < rpe;
@@ -134,9 +137,9 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
     preload<WT, U>(b, wrow, q);
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *cols = lds + tab_bytes<WT>();
-    float *hbuf = reinterpret_cast<float *>(cols + (size_t)kTileCols * col_bytes); // [8][32]
-    u32 *bad = reinterpret_cast<u32 *>(hbuf + kTileCols * 32);                      // [8]: entry names no slot
-    if (tid < kTileCols) {
+    float *hbuf = reinterpret_cast<float *>(cols + (size_t)MC * col_bytes); // [MC][32]
+    u32 *bad = reinterpret_cast<u32 *>(hbuf + MC * 32);                      // [MC]: entry names no slot
+    if (tid < MC) {
         const u32 s = tid < t.m ? order[t.j + tid] : 0;
         const bool none = tid < t.m && (s >= n_slots || (int)(s / slots_per_col) >= act_cols);
         if (none) bm_raise(fault, layer, kSiteExpertId);
@@ -145,10 +148,10 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
     __syncthreads();
     stage_tile_cols(cols, act, col_bytes, t.m, [&](int c) { return bad[c] == 0xffffffffu ? 0 : (int)bad[c]; });
     __syncthreads();
-    float v[kTileCols];
-    row_dot<WT, U, NB, kTileCols>(b, wrow, cols, col_bytes, t.m, n, q, tb, v, NoTap{});
+    float v[MC];
+    row_dot<WT, U, NB, MC>(b, wrow, cols, col_bytes, t.m, n, q, tb, v, NoTap{});
 #pragma unroll
-    for (int c = 0; c < kTileCols; c++) {
+    for (int c = 0; c < MC; c++) {
         float hv = swiglu_of_pair(c < t.m ? v[c] : 0.0f, which, rule, fault, layer);
         if (c < t.m) {
             if (bad[c] == 0xffffffffu) hv = bm_bits_f32(0x7fc00000u);
@@ -167,14 +170,15 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
 
 // crates/gpu/src/kquant/tiles.rs:120-190 GemvTiles: workgroup = tile x 64 rows (a quad a row); entry j + c reads
 // column j + c of act and writes row r of its slot order[j + c]. An entry that names no slot raises ExpertId.
-template <int WT, int U, int NB>
+template <int WT, int U, int NB, int MC>
 __global__ __launch_bounds__(256) void k_gemv_tiles(const uint8_t *w, u32 n_experts, int nb, const uint8_t *act,
                                                     const u32 *order, const u32 *start, const u32 *tiles, u32 n_slots,
-                                                    u32 cap, int rpe, float *y, u32 *fault, u32 layer) {
+                                                    u32 cap, int rpe, float *y, int m_lo, u32 *fault, u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, q = tid & 3;
     Tile t;
     if (!tile_of_block(tiles, start, n_experts, n_slots, cap, &t, fault, layer)) return;
+    if (t.m <= m_lo || t.m > MC) return;
     const int r = t.row_block * 64 + (tid >> 2);
     const bool active = r < rpe;
     const int n = NB > 0 ? NB : nb;
@@ -185,47 +189,66 @@ __global__ __launch_bounds__(256) void k_gemv_tiles(const uint8_t *w, u32 n_expe
     preload<WT, U>(b, wrow, q);
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *cols = lds + tab_bytes<WT>();
-    u32 *slot_of = reinterpret_cast<u32 *>(cols + (size_t)kTileCols * col_bytes); // [8]
-    if (tid < kTileCols) {
+    u32 *slot_of = reinterpret_cast<u32 *>(cols + (size_t)MC * col_bytes); // [MC]
+    if (tid < MC) {
         const u32 s = tid < t.m ? order[t.j + tid] : 0;
         if (tid < t.m && s >= n_slots && t.row_block == 0) bm_raise(fault, layer, kSiteExpertId);
         slot_of[tid] = s;
     }
     stage_bytes(cols, act + (size_t)t.j * col_bytes, t.m * col_bytes); // the tile's columns lie side by side
     __syncthreads();
-    float v[kTileCols];
-    row_dot<WT, U, NB, kTileCols>(b, wrow, cols, col_bytes, t.m, n, q, tb, v, NoTap{});
+    float v[MC];
+    row_dot<WT, U, NB, MC>(b, wrow, cols, col_bytes, t.m, n, q, tb, v, NoTap{});
     if (q == 0 && active) {
 #pragma unroll
-        for (int c = 0; c < kTileCols; c++)
+        for (int c = 0; c < MC; c++)
             if (c < t.m && slot_of[c] < n_slots) y[(size_t)slot_of[c] * rpe + r] = v[c];
     }
 }
 
 // ------------------------------------------------------------------------------------------------ launchers
 
+static size_t tiles_lds_of(int wtype, int k, int cols) {
+    return tab_bytes_rt(wtype) + (size_t)cols * act_col_bytes(wtype, k) + (size_t)cols * 32 * sizeof(float) + cols * sizeof(u32);
+}
 size_t tiles_lds(int wtype, int k) {
-    const size_t lds = tab_bytes_rt(wtype) + (size_t)kTileCols * act_col_bytes(wtype, k) + kTileCols * 32 * sizeof(float) +
-                       kTileCols * sizeof(u32);
+    const size_t lds = tiles_lds_of(wtype, k, kTileCols);
     return lds <= (size_t)kMaxLds ? lds : 0;
 }
+
+// Eight columns of a long row take most of a CU's LDS (IQ2_XXS at 7168 values: 66 KB, two workgroups a CU), and with
+// few tokens over many experts most tiles hold one or two slots. Past kTileSplitLds a tile launch therefore goes as two:
+// one with LDS for two columns takes the tiles of up to two slots at several times the occupancy, one with LDS for
+// eight takes the rest; a workgroup whose tile is the other launch's returns at once. Values do not depend on the
+// width: every column is its own row dot.
+constexpr size_t kTileSplitLds = 40 * 1024;
+constexpr int kTileNarrow = 2;
+static bool tile_widths_split(int wtype, int k) { return tiles_lds_of(wtype, k, kTileCols) > kTileSplitLds; }
 
 hipError_t gate_up_tiles(const Launch &L, int wtype, const uint8_t *wg, const uint8_t *wu, int n_experts, int k,
                          const uint8_t *act, int act_cols, const uint32_t *order, const uint32_t *start,
                          const uint32_t *tiles_dev, int n_slots, int rows_per_expert, int slots_per_col, float *h,
                          uint8_t *act_h) {
     const int nb = k / 256, rpe = rows_per_expert;
-    const size_t lds = tiles_lds(wtype, k);
+    const bool split = tile_widths_split(wtype, k);
     const u32 cap = (u32)tile_cap(n_slots, n_experts);
     const unsigned grid = cap * (unsigned)((rpe + 31) / 32);
+#define BM_TILE_LAUNCH(MC, M_LO)                                                                                       \
+    {                                                                                                                  \
+        const size_t lds = tiles_lds_of(wtype, k, MC);                                                                 \
+        auto kern = k_gate_up_tiles<WT, U, NB, MC>;                                                                    \
+        hipError_t e = allow_lds(kern, lds);                                                                           \
+        if (e != hipSuccess) return e;                                                                                 \
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, wg, wu, (u32)n_experts, nb, act, act_cols,      \
+                           order, start, tiles_dev, (u32)n_slots, cap, rpe, slots_per_col, h, act_h, M_LO, L.rule,     \
+                           L.fault, L.layer);                                                                          \
+    }
 #define CALL_BODY                                                                                                      \
-    auto kern = k_gate_up_tiles<WT, U, NB>;                                                                            \
-    hipError_t e = allow_lds(kern, lds);                                                                               \
-    if (e != hipSuccess) return e;                                                                                     \
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, wg, wu, (u32)n_experts, nb, act, act_cols, order,   \
-                       start, tiles_dev, (u32)n_slots, cap, rpe, slots_per_col, h, act_h, L.rule, L.fault, L.layer);
+    if (split) BM_TILE_LAUNCH(kTileNarrow, 0)                                                                          \
+    BM_TILE_LAUNCH(kTileCols, split ? kTileNarrow : 0)
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
+#undef BM_TILE_LAUNCH
     return hipGetLastError();
 }
 
@@ -233,17 +256,24 @@ hipError_t gemv_tiles(const Launch &L, int wtype, const uint8_t *w, int n_expert
                       const uint32_t *order, const uint32_t *start, const uint32_t *tiles_dev, int n_slots,
                       int rows_per_expert, float *y) {
     const int nb = k / 256, rpe = rows_per_expert;
-    const size_t lds = tiles_lds(wtype, k);
+    const bool split = tile_widths_split(wtype, k);
     const u32 cap = (u32)tile_cap(n_slots, n_experts);
     const unsigned grid = cap * (unsigned)((rpe + 63) / 64);
+#define BM_TILE_LAUNCH(MC, M_LO)                                                                                       \
+    {                                                                                                                  \
+        const size_t lds = tiles_lds_of(wtype, k, MC);                                                                 \
+        auto kern = k_gemv_tiles<WT, U, NB, MC>;                                                                       \
+        hipError_t e = allow_lds(kern, lds);                                                                           \
+        if (e != hipSuccess) return e;                                                                                 \
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act, order, start,       \
+                           tiles_dev, (u32)n_slots, cap, rpe, y, M_LO, L.fault, L.layer);                              \
+    }
 #define CALL_BODY                                                                                                      \
-    auto kern = k_gemv_tiles<WT, U, NB>;                                                                               \
-    hipError_t e = allow_lds(kern, lds);                                                                               \
-    if (e != hipSuccess) return e;                                                                                     \
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act, order, start,           \
-                       tiles_dev, (u32)n_slots, cap, rpe, y, L.fault, L.layer);
+    if (split) BM_TILE_LAUNCH(kTileNarrow, 0)                                                                          \
+    BM_TILE_LAUNCH(kTileCols, split ? kTileNarrow : 0)
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
+#undef BM_TILE_LAUNCH
     return hipGetLastError();
 }
 

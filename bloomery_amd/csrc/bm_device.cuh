@@ -75,6 +75,11 @@ __device__ __forceinline__ float bm_q82_inverse(u32 t) {
 
 __device__ __forceinline__ int bm_sdot4(u32 a, u32 b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
 
+// a * b + c for factors inside 24 signed bits (every integer the IQ cores scale is): one full-rate instruction where
+// the 32-bit multiply takes four times as long.
+__device__ __forceinline__ int bm_mad24(int a, int b, int c) { return __mul24(a, b) + c; }
+__device__ __forceinline__ int bm_mul24(int a, int b) { return __mul24(a, b); }
+
 // 16 bytes from an address of any alignment (global memory takes unaligned vector loads on this target).
 __device__ __forceinline__ uint4 bm_ld16u(const uint8_t *p) {
     uint4 v;
@@ -444,12 +449,13 @@ __device__ __forceinline__ Blk<BM_IQ2XXS> bm_load_iq2xxs(const uint8_t *wrow, in
     return b;
 }
 
-// LDS tables of the IQ2_XXS decode: the 256-point grid (8 magnitudes a point), the 128 sign bytes, and the 16
-// nibble -> byte-mask words (bit k set -> byte k = 0xff).
+// LDS tables of the IQ2_XXS decode. The CPU path dots the unsigned bytes u = +-mag + 43 (0 .. 86) and takes the 43s
+// back out through the column's sums, so the tables give u with two operations a word: a grid point is kept as its
+// eight magnitudes + 43 (x, y) and its eight doubled magnitudes (z, w), a sign index as eight byte masks (0xff where
+// the value is negative): u = (mag + 43) - (2 mag & mask), byte by byte without a borrow.
 struct Iq2Tables {
-    const uint2 *grid;
-    const uint8_t *ksigns;
-    const u32 *nibmask;
+    const uint4 *grid;
+    const uint2 *signs;
 };
 
 template <>
@@ -472,7 +478,7 @@ __device__ __forceinline__ Act<BM_IQ2XXS> bm_act_iq2xxs(const ActView &av, int i
 // The block's codes as this lane dots them: per sub-block the eight signed grid values (two words) and the
 // scale 2s + 1. Decoded once a super-block, whatever the number of columns.
 struct Iq2Dec {
-    u32 v_lo[8], v_hi[8];
+    u32 u_lo[8], u_hi[8]; // the bytes +-mag + 43
     int sc[8];
 };
 
@@ -488,12 +494,10 @@ __device__ __forceinline__ Iq2Dec bm_decode_iq2xxs(const Blk<BM_IQ2XXS> &b, int 
             const int sb = 2 * k + e;
             const u32 idx = e ? idx_b : idx_a, aux = e ? aux_b : aux_a;
             dec.sc[sb] = 2 * (int)(aux >> 28) + 1;
-            const uint2 g = tb.grid[(idx >> (8 * q)) & 0xffu];
-            const u32 sg = tb.ksigns[(aux >> (7 * q)) & 127u];
-            const u32 m_lo = tb.nibmask[sg & 15u], m_hi = tb.nibmask[sg >> 4];
-            // -mag where the sign bit is set: (mag ^ 0xff) + 1 per byte, no carry leaves a byte (mag > 0).
-            dec.v_lo[sb] = (g.x ^ m_lo) + (m_lo & 0x01010101u);
-            dec.v_hi[sb] = (g.y ^ m_hi) + (m_hi & 0x01010101u);
+            const uint4 g = tb.grid[(idx >> (8 * q)) & 0xffu];
+            const uint2 sg = tb.signs[(aux >> (7 * q)) & 127u];
+            dec.u_lo[sb] = g.x - (g.z & sg.x);
+            dec.u_hi[sb] = g.y - (g.w & sg.y);
         }
     }
     return dec;
@@ -511,7 +515,7 @@ __device__ __forceinline__ void bm_dot_iq2xxs_dec(const Blk<BM_IQ2XXS> &b, const
         const uint2 bs = act.bs;
         const int b0 = (int)(short)(bs.x & 0xffffu), b1 = (int)(short)(bs.x >> 16);
         const int b2 = (int)(short)(bs.y & 0xffffu), b3 = (int)(short)(bs.y >> 16);
-        const int ma = sca * b0 + sca * b1, mb = scb * b2 + scb * b3;
+        const int ma = bm_mad24(sca, b0, bm_mul24(sca, b1)), mb = bm_mad24(scb, b2, bm_mul24(scb, b3)); // bsums: 16 bits
         const float f = dmin * dy;
         acc0 = fmaf(f, (float)ma, acc0);
         acc1 = fmaf(f, (float)mb, acc1);
@@ -520,12 +524,13 @@ __device__ __forceinline__ void bm_dot_iq2xxs_dec(const Blk<BM_IQ2XXS> &b, const
 #pragma unroll
     for (int sb = 0; sb < 8; sb++) {
         const uint2 a = act.a[sb];
-        const int i_lo = bm_sdot4(dec.v_lo[sb], a.x, 0), i_hi = bm_sdot4(dec.v_hi[sb], a.y, 0);
-        const int s_lo = bm_sdot4(0x01010101u, a.x, 0), s_hi = bm_sdot4(0x01010101u, a.y, 0);
-        // the reference sums sc * (v + 43) * a: the offset comes back out through the fold above
-        sumi0 += dec.sc[sb] * (i_lo + 43 * s_lo);
-        sumi1 += dec.sc[sb] * (i_hi + 43 * s_hi);
-        tap.iq2(i, sb, q, i_lo + i_hi);
+        // the reference sums sc * u * a (the 43s come back out through the fold above); sums within 4 * 86 * 128 and
+        // sc <= 31 lie inside 24 bits
+        const int d_lo = bm_sdot4(dec.u_lo[sb], a.x, 0), d_hi = bm_sdot4(dec.u_hi[sb], a.y, 0);
+        sumi0 = bm_mad24(dec.sc[sb], d_lo, sumi0);
+        sumi1 = bm_mad24(dec.sc[sb], d_hi, sumi1);
+        if constexpr (Tap::kActive) // the signed sum: less 43 times the eight codes
+            tap.iq2(i, sb, q, d_lo + d_hi - 43 * (bm_sdot4(0x01010101u, a.x, 0) + bm_sdot4(0x01010101u, a.y, 0)));
     }
     const float f = d * dy;
     acc0 = fmaf(f, (float)sumi0, acc0);
@@ -623,8 +628,9 @@ __device__ __forceinline__ void bm_dot_iq4xs_dec(const Blk<BM_IQ4XS> &b, const I
             const uint2 alo = act.a[4 * e + (j >> 1)], ahi = act.a[4 * e + 2 + (j >> 1)];
             const int p_lo = bm_sdot4(dec.lo[e][j], (j & 1) ? alo.y : alo.x, 0);
             const int p_hi = bm_sdot4(dec.hi[e][j], (j & 1) ? ahi.y : ahi.x, 0);
-            lanes[j] = e ? lanes[j] + dec.sc[1] * p_lo : dec.sc[0] * p_lo;
-            lanes[4 + j] = e ? lanes[4 + j] + dec.sc[1] * p_hi : dec.sc[0] * p_hi;
+            // |p| <= 4 * 127 * 128 and |scale| <= 32: inside 24 bits
+            lanes[j] = e ? bm_mad24(dec.sc[1], p_lo, lanes[j]) : bm_mul24(dec.sc[0], p_lo);
+            lanes[4 + j] = e ? bm_mad24(dec.sc[1], p_hi, lanes[4 + j]) : bm_mul24(dec.sc[0], p_hi);
             sub += p_lo + p_hi;
         }
         tap.iq4_sub(i, 2 * q + e, sub);

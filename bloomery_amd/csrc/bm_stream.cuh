@@ -27,8 +27,8 @@ constexpr u32 kSiteExpertId = 7;    // crates/device/src/fault.rs:89
 constexpr u32 kSiteF32Product = 21; // crates/device/src/fault.rs:151-155: a gate or up sum that is not finite under a clamp
 constexpr u32 kSiteStalled = 31;    // ours: a fused launch's down workgroup gave up waiting for its activations
 
-// LDS bytes of the IQ2_XXS tables: 2048 grid + 128 signs + 64 nibble masks, padded to a 16-byte multiple.
-constexpr int kTabBytes = 2048 + 128 + 64 + 64;
+// LDS bytes of the IQ2_XXS tables: 256 grid entries of 16 + 128 sign entries of 8.
+constexpr int kTabBytes = 256 * 16 + 128 * 8;
 
 template <int WT>
 __host__ __device__ constexpr int tab_bytes() {
@@ -37,22 +37,27 @@ __host__ __device__ constexpr int tab_bytes() {
 
 template <int WT>
 __device__ __forceinline__ Iq2Tables stage_tables(uint8_t *lds) {
-    Iq2Tables tb{nullptr, nullptr, nullptr};
+    Iq2Tables tb{nullptr, nullptr};
     if constexpr (WT == BM_IQ2XXS) {
-        uint2 *grid = reinterpret_cast<uint2 *>(lds);
-        uint8_t *ks = lds + 2048;
-        u32 *nm = reinterpret_cast<u32 *>(lds + 2048 + 128);
+        uint4 *grid = reinterpret_cast<uint4 *>(lds);
+        uint2 *signs = reinterpret_cast<uint2 *>(lds + 256 * 16);
         for (int t = threadIdx.x; t < 256; t += blockDim.x) {
-            const uint64_t g = BM_IQ2XXS_GRID[t];
-            grid[t] = make_uint2((u32)g, (u32)(g >> 32));
+            const uint64_t g = BM_IQ2XXS_GRID[t]; // bytes 8, 25 or 43: + 43 and doubled stay inside a byte
+            const u32 lo = (u32)g, hi = (u32)(g >> 32);
+            grid[t] = make_uint4(lo + 0x2b2b2b2bu, hi + 0x2b2b2b2bu, lo << 1, hi << 1);
         }
-        for (int t = threadIdx.x; t < 128; t += blockDim.x) ks[t] = BM_KSIGNS_IQ2XS[t];
-        for (int t = threadIdx.x; t < 16; t += blockDim.x)
-            nm[t] = ((t & 1) ? 0xffu : 0u) | ((t & 2) ? 0xff00u : 0u) | ((t & 4) ? 0xff0000u : 0u) |
-                    ((t & 8) ? 0xff000000u : 0u);
+        for (int t = threadIdx.x; t < 128; t += blockDim.x) {
+            const u32 sg = BM_KSIGNS_IQ2XS[t];
+            u32 m[2];
+            for (int half = 0; half < 2; half++) {
+                const u32 nib = (sg >> (4 * half)) & 15u;
+                m[half] = ((nib & 1) ? 0xffu : 0u) | ((nib & 2) ? 0xff00u : 0u) | ((nib & 4) ? 0xff0000u : 0u) |
+                          ((nib & 8) ? 0xff000000u : 0u);
+            }
+            signs[t] = make_uint2(m[0], m[1]);
+        }
         tb.grid = grid;
-        tb.ksigns = ks;
-        tb.nibmask = nm;
+        tb.signs = signs;
     }
     return tb;
 }

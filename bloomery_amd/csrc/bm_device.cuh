@@ -272,7 +272,10 @@ __device__ __forceinline__ void bm_dot_q45k(uint4 hdr, uint4 qa, uint4 qb, const
     const int sh = 16 * c;                         // this lane's two sub-blocks sit in bytes 2c, 2c + 1
     const u32 s0 = (a0 & 0x3f3f3f3fu) >> sh;       // scales of sub-blocks 2c, 2c + 1
     const u32 s1 = ((a2 & 0x0f0f0f0fu) | ((a0 >> 2) & 0x30303030u)) >> sh; // 4 + 2c, 5 + 2c
-    const u32 mw = h ? (((a2 >> 4) & 0x0f0f0f0fu) | ((a1 >> 2) & 0x30303030u)) : (a1 & 0x3f3f3f3fu);
+    // both forms and a bitwise pick: a conditional here compiles to a branch a super-block, which also fences the
+    // scheduling of the loads around it
+    const u32 hm = 0u - (u32)h;
+    const u32 mw = ((((a2 >> 4) & 0x0f0f0f0fu) | ((a1 >> 2) & 0x30303030u)) & hm) | ((a1 & 0x3f3f3f3fu) & ~hm);
     const u32 mm = mw >> sh; // mins of sub-blocks 4h + 2c, 4h + 2c + 1
     // Min term of accumulators l = 4h + t (lib.rs:4389-4394): fma(d8 * isum, -(dmin * m), acc).
     acc0 = fmaf(a.em.y, -(dmin * (float)(mm & 0xffu)), acc0);

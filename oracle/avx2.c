@@ -405,6 +405,78 @@ static void dot_iq2xxs_tile(const uint8_t *wrow, const uint8_t *const *acols, in
     for (int c = 0; c < C; c++) out[c] = hsum_float_8(accd[c]);
 }
 
+// ------------------------------------------------------------------------------------------------- IQ3_XXS tile
+
+// One IQ3_XXS row against C <= 8 columns (crates/qdot/src/lib.rs:7259-7345 per column, :7412 the tile): the IQ2_XXS
+// tile with eight four-magnitude grid words a sub-block, the sign/scale words behind the 64 index bytes, the
+// offset 64 and d = f16 / 4.
+static void dot_iq3xxs_tile(const uint8_t *wrow, const uint8_t *const *acols, int C, int nb, float *out) {
+    const __m256i min_value = _mm256_set1_epi8(64);
+    __m256 accd[8];
+    for (int c = 0; c < C; c++) accd[c] = _mm256_setzero_ps();
+    for (int i = 0; i < nb; i++) {
+        const uint8_t *blk = wrow + (size_t)i * ORA_IQ3XXS_BLOCK;
+        const uint8_t *qs = blk + 2;
+        size_t at = (size_t)i * ORA_Q8K_STRIDE;
+        uint16_t dh;
+        memcpy(&dh, blk, 2);
+        float d = 0.25f * f16c_to_f32(dh);
+        float dmin = -d * 64.0f;
+        __m256i words = _mm256_loadu_si256((const __m256i *)(qs + 64));
+        __m256i sc32 = _mm256_or_si256(_mm256_slli_epi32(_mm256_srli_epi32(words, 28), 1), _mm256_set1_epi32(1));
+        __m128i sc16 = _mm_packs_epi32(_mm256_castsi256_si128(sc32), _mm256_extracti128_si256(sc32, 1));
+        __m256i mins = _mm256_set_m128i(
+            _mm_shuffle_epi8(sc16, _mm_set_epi32(0x0f0e0f0e, 0x0d0c0d0c, 0x0b0a0b0a, 0x09080908)),
+            _mm_shuffle_epi8(sc16, _mm_set_epi32(0x07060706, 0x05040504, 0x03020302, 0x01000100)));
+        __m256i all_scales = _mm256_set_m128i(sc16, sc16);
+        __m256i sumi[8];
+        for (int c = 0; c < C; c++) {
+            const uint8_t *col = acols[c] + at;
+            float dy;
+            memcpy(&dy, col, 4);
+            __m256i bsums = _mm256_loadu_si256((const __m256i *)(col + 264));
+            accd[c] = _mm256_fmadd_ps(_mm256_set1_ps(dmin * dy), _mm256_cvtepi32_ps(_mm256_madd_epi16(mins, bsums)),
+                                      accd[c]);
+        }
+        for (int j = 0; j < 2; j++) {
+            __m256i values[4], scales[4];
+            for (int q = 0; q < 4; q++) {
+                int b = 4 * j + q;
+                const uint8_t *g = qs + 8 * b;
+                uint32_t aux;
+                memcpy(&aux, qs + 64 + 4 * b, 4);
+                __m256i q3 = _mm256_set_epi32((int)ORA_IQ3XXS_GRID[g[7]], (int)ORA_IQ3XXS_GRID[g[6]], (int)ORA_IQ3XXS_GRID[g[5]],
+                                              (int)ORA_IQ3XXS_GRID[g[4]], (int)ORA_IQ3XXS_GRID[g[3]], (int)ORA_IQ3XXS_GRID[g[2]],
+                                              (int)ORA_IQ3XXS_GRID[g[1]], (int)ORA_IQ3XXS_GRID[g[0]]);
+                __m256i sg = _mm256_set_epi64x((long long)KEVEN_SIGNS[(aux >> 21) & 127], (long long)KEVEN_SIGNS[(aux >> 14) & 127],
+                                               (long long)KEVEN_SIGNS[(aux >> 7) & 127], (long long)KEVEN_SIGNS[aux & 127]);
+                values[q] = _mm256_add_epi8(_mm256_sign_epi8(q3, sg), min_value);
+                scales[q] = _mm256_shuffle_epi8(all_scales, _mm256_set1_epi16((short)((2 * b) | ((2 * b + 1) << 8))));
+            }
+            for (int c = 0; c < C; c++) {
+                const uint8_t *col = acols[c] + at;
+                __m256i p[4];
+                for (int q = 0; q < 4; q++) {
+                    __m256i q8 = _mm256_loadu_si256((const __m256i *)(col + 8 + 32 * (4 * j + q)));
+                    p[q] = _mm256_madd_epi16(scales[q], _mm256_maddubs_epi16(values[q], q8));
+                }
+                if (j == 0) {
+                    sumi[c] = _mm256_add_epi32(_mm256_add_epi32(p[0], p[2]), _mm256_add_epi32(p[1], p[3]));
+                } else {
+                    sumi[c] = _mm256_add_epi32(sumi[c], _mm256_add_epi32(p[0], p[2]));
+                    sumi[c] = _mm256_add_epi32(sumi[c], _mm256_add_epi32(p[1], p[3]));
+                }
+            }
+        }
+        for (int c = 0; c < C; c++) {
+            float dy;
+            memcpy(&dy, acols[c] + at, 4);
+            accd[c] = _mm256_fmadd_ps(_mm256_set1_ps(d * dy), _mm256_cvtepi32_ps(sumi[c]), accd[c]);
+        }
+    }
+    for (int c = 0; c < C; c++) out[c] = hsum_float_8(accd[c]);
+}
+
 // -------------------------------------------------------------------------------------------------- IQ4_XS tile
 
 // One IQ4_XS row against C <= 8 columns (crates/qdot/src/lib.rs:11062-11145): a sub-block's 32 levels come out of one
@@ -465,6 +537,10 @@ int ora_avx2_dot_row_cols(int wtype, const uint8_t *wrow, const uint8_t *const *
     case ORA_TYPE_IQ2_XXS:
         pthread_once(&keven_once, keven_init);
         dot_iq2xxs_tile(wrow, acols, cols, nb, out);
+        return 0;
+    case ORA_TYPE_IQ3_XXS:
+        pthread_once(&keven_once, keven_init);
+        dot_iq3xxs_tile(wrow, acols, cols, nb, out);
         return 0;
     case ORA_TYPE_IQ4_XS:
         dot_iq4xs_tile(wrow, acols, cols, nb, out);

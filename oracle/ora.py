@@ -11,9 +11,9 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libbm_oracle.so")
 
-Q4_K, Q5_K, Q6_K, IQ2_XXS, IQ4_XS = 12, 13, 14, 16, 23
-BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ2_XXS: 66, IQ4_XS: 136}
-Q8K_TYPES = (IQ2_XXS, IQ4_XS)  # the types whose activation column is ik's Q8_K; the others take Q8_2_X4
+Q4_K, Q5_K, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_XS = 12, 13, 14, 16, 18, 23
+BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ2_XXS: 66, IQ3_XXS: 98, IQ4_XS: 136}
+Q8K_TYPES = (IQ2_XXS, IQ3_XXS, IQ4_XS)  # the types whose activation column is ik's Q8_K; the others take Q8_2_X4
 
 EUNALIGNED, ETYPE, ESHORTROW, ESHORTCOL, ENONFINITE, ESHAPE, ESTATUS = -1, -2, -3, -4, -5, -6, -7
 
@@ -49,6 +49,8 @@ def _load():
         "ora_q5k_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
         "ora_q6k_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
         "ora_iq2xxs_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                         C.c_void_p]),
+        "ora_iq3xxs_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
                                          C.c_void_p]),
         "ora_iq4xs_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
         "ora_dequant_row": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
@@ -174,13 +176,16 @@ def q6k_block_sums(wrow, acol, k, fold=False):
     return s
 
 
-def iq2xxs_block_sums(wrow, acol, k):
+def iq2xxs_block_sums(wrow, acol, k, iq3=False):
+    """Per sub-block the signed sum and the scale 2s + 1, per super-block the CPU lanes' two aggregates (IQ2_XXS; with
+    iq3 an IQ3_XXS row)."""
     nb = k // 256
     i = np.empty(nb * 8, np.int32)
     sc = np.empty(nb * 8, np.int32)
     codes = np.empty(nb, np.int32)
     fold = np.empty(nb, np.int32)
-    lib.ora_iq2xxs_block_sums(_p(_u8(wrow)), _p(_u8(acol)), nb, _p(i), _p(sc), _p(codes), _p(fold))
+    (lib.ora_iq3xxs_block_sums if iq3 else lib.ora_iq2xxs_block_sums)(_p(_u8(wrow)), _p(_u8(acol)), nb, _p(i), _p(sc),
+                                                                      _p(codes), _p(fold))
     return i, sc, codes, fold
 
 

@@ -15,6 +15,7 @@
 #define ORA_Q5K_BLOCK 176    // crates/qdot/src/lib.rs:4880: d, dmin, scales[12], qh[32] @16, qs[128] @48
 #define ORA_Q6K_BLOCK 210    // crates/qdot/src/lib.rs:4452
 #define ORA_IQ2XXS_BLOCK 66  // crates/qdot/src/lib.rs:8298
+#define ORA_IQ3XXS_BLOCK 98  // crates/qdot/src/lib.rs IQ3XXS_BLOCK: d, 64 grid indices @2, eight sign/scale words @66
 #define ORA_IQ4XS_BLOCK 136  // crates/qdot/src/lib.rs:11033-11037: d, scales_h u16 @2, scales_l[4] @4, qs[128] @8
 #define ORA_Q8K_STRIDE 296   // crates/qdot/src/lib.rs:108
 #define ORA_Q82X4_STRIDE 144 // crates/qdot/src/lib.rs:110
@@ -24,10 +25,13 @@
 #define ORA_TYPE_Q5_K 13
 #define ORA_TYPE_Q6_K 14
 #define ORA_TYPE_IQ2_XXS 16
+#define ORA_TYPE_IQ3_XXS 18
 #define ORA_TYPE_IQ4_XS 23
 
 // The types whose activation column is ik's Q8_K (crates/gguf/src/qtype.rs host_act); the others here take Q8_2_X4.
-static inline int ora_takes_q8k(int wtype) { return wtype == ORA_TYPE_IQ2_XXS || wtype == ORA_TYPE_IQ4_XS; }
+static inline int ora_takes_q8k(int wtype) {
+    return wtype == ORA_TYPE_IQ2_XXS || wtype == ORA_TYPE_IQ3_XXS || wtype == ORA_TYPE_IQ4_XS;
+}
 
 static inline uint32_t ora_f32_bits(float f) {
     uint32_t u;

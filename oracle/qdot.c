@@ -78,6 +78,7 @@ int ora_col_bytes(int wtype, int k) {
     case ORA_TYPE_Q6_K:
         return k / 128 * ORA_Q82X4_STRIDE;
     case ORA_TYPE_IQ2_XXS:
+    case ORA_TYPE_IQ3_XXS:
     case ORA_TYPE_IQ4_XS:
         return k / 256 * ORA_Q8K_STRIDE;
     default:
@@ -96,6 +97,8 @@ int ora_row_bytes(int wtype, int k) {
         return k / 256 * ORA_Q6K_BLOCK;
     case ORA_TYPE_IQ2_XXS:
         return k / 256 * ORA_IQ2XXS_BLOCK;
+    case ORA_TYPE_IQ3_XXS:
+        return k / 256 * ORA_IQ3XXS_BLOCK;
     case ORA_TYPE_IQ4_XS:
         return k / 256 * ORA_IQ4XS_BLOCK;
     default:
@@ -110,6 +113,7 @@ int ora_quantize_col(int wtype, const float *x, int k, uint8_t *out) {
     case ORA_TYPE_Q6_K:
         return ora_quantize_q82x4(x, k, out);
     case ORA_TYPE_IQ2_XXS:
+    case ORA_TYPE_IQ3_XXS:
     case ORA_TYPE_IQ4_XS:
         return ora_quantize_q8k(x, k, out);
     default:
@@ -381,6 +385,72 @@ void ora_iq2xxs_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int
     }
 }
 
+// --------------------------------------------------------------------------------------------------- IQ3_XXS dot
+
+// Signed grid value n (0..32) of sub-block b: group n / 8 takes grid words qs[8b + 2 (n / 8)] (its values 0..3) and the
+// next (4..7), four magnitudes a word, and bit n % 8 of the group's sign byte (crates/gguf/src/quant.rs:1739-1772).
+static inline int iq3xxs_value(const uint8_t *blk, int b, int n) {
+    uint32_t word = ora_rd32(blk + 66 + 4 * b);
+    int mag = (int)((ORA_IQ3XXS_GRID[blk[2 + 8 * b + n / 4]] >> (8 * (n % 4))) & 0xff);
+    uint8_t signs = ORA_KSIGNS_IQ2XS[(word >> (7 * (n / 8))) & 127];
+    return ((signs >> (n % 8)) & 1) ? -mag : mag;
+}
+
+// IQ3_XXS x Q8_K, the scalar mirror's float steps in its order (crates/qdot/src/lib.rs:7494-7541): IQ2_XXS's walk with
+// d = f16 / 4, the offset 64 and four-magnitude grid words.
+float ora_dot_iq3xxs_q8k(const uint8_t *wrow, const uint8_t *acol, int nb) {
+    float accd[8] = {0};
+    for (int i = 0; i < nb; i++) {
+        const uint8_t *blk = wrow + (size_t)i * ORA_IQ3XXS_BLOCK;
+        const uint8_t *col = acol + (size_t)i * ORA_Q8K_STRIDE;
+        float d = 0.25f * ora_half_to_f32(ora_rd16(blk));
+        int32_t sc[8];
+        for (int b = 0; b < 8; b++) sc[b] = 2 * (int32_t)(ora_rd32(blk + 66 + 4 * b) >> 28) + 1;
+        float dmin = -d * 64.0f;
+        float dy = ora_bits_f32(ora_rd32(col));
+        for (int l = 0; l < 8; l++) {
+            int32_t b0 = (int16_t)ora_rd16(col + 264 + 4 * l);
+            int32_t b1 = (int16_t)ora_rd16(col + 266 + 4 * l);
+            int32_t m = sc[l] * b0 + sc[l] * b1;
+            accd[l] = fmaf(dmin * dy, (float)m, accd[l]);
+        }
+        int32_t sumi[8] = {0};
+        for (int b = 0; b < 8; b++) {
+            for (int n = 0; n < 32; n++) {
+                int v = iq3xxs_value(blk, b, n);
+                int32_t u = (uint8_t)(int8_t)(v + 64);
+                int32_t a = (int8_t)col[8 + 32 * b + n];
+                sumi[n / 4] += sc[b] * u * a;
+            }
+        }
+        for (int l = 0; l < 8; l++) accd[l] = fmaf(d * dy, (float)sumi[l], accd[l]);
+    }
+    float t[4] = {accd[0] + accd[4], accd[1] + accd[5], accd[2] + accd[6], accd[3] + accd[7]};
+    return (t[0] + t[2]) + (t[1] + t[3]);
+}
+
+// As ora_iq2xxs_block_sums, with the offset 64.
+void ora_iq3xxs_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_t *i_out, int32_t *sc_out,
+                           int32_t *codes_out, int32_t *fold_out) {
+    for (int i = 0; i < nb; i++) {
+        const uint8_t *blk = wrow + (size_t)i * ORA_IQ3XXS_BLOCK;
+        const uint8_t *col = acol + (size_t)i * ORA_Q8K_STRIDE;
+        int32_t codes = 0, fold = 0;
+        for (int b = 0; b < 8; b++) {
+            int32_t s = 2 * (int32_t)(ora_rd32(blk + 66 + 4 * b) >> 28) + 1;
+            int32_t sum = 0;
+            for (int n = 0; n < 32; n++) sum += iq3xxs_value(blk, b, n) * (int32_t)(int8_t)col[8 + 32 * b + n];
+            int32_t bs = (int16_t)ora_rd16(col + 264 + 4 * b) + (int16_t)ora_rd16(col + 266 + 4 * b);
+            i_out[8 * i + b] = sum;
+            sc_out[8 * i + b] = s;
+            codes += s * (sum + 64 * bs);
+            fold += s * bs;
+        }
+        codes_out[i] = codes;
+        fold_out[i] = fold;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------- IQ4_XS dot
 
 // Sub-block b's 6-bit scale less 32: nibble b % 2 of scales_l[b / 2] under bits 2b.. of scales_h
@@ -468,6 +538,9 @@ int ora_dot_row(int wtype, const uint8_t *wrow, size_t wrow_len, const uint8_t *
     case ORA_TYPE_IQ2_XXS:
         *out = ora_dot_iq2xxs_q8k(wrow, acol, nb);
         return 0;
+    case ORA_TYPE_IQ3_XXS:
+        *out = ora_dot_iq3xxs_q8k(wrow, acol, nb);
+        return 0;
     case ORA_TYPE_IQ4_XS:
         *out = ora_dot_iq4xs_q8k(wrow, acol, nb);
         return 0;
@@ -526,6 +599,18 @@ int ora_dequant_row(int wtype, const uint8_t *src, int k, float *dst) {
                 float db = d * (0.5f + (float)(aux >> 28)) * 0.25f;
                 for (int n = 0; n < 32; n++) {
                     int v = iq2xxs_value(blk, b, n);
+                    float mag = (float)(v < 0 ? -v : v);
+                    out[32 * b + n] = db * mag * (v < 0 ? -1.0f : 1.0f);
+                }
+            }
+        } else if (wtype == ORA_TYPE_IQ3_XXS) { // crates/gguf/src/quant.rs:1748-1772
+            const uint8_t *blk = src + (size_t)i * ORA_IQ3XXS_BLOCK;
+            float d = ora_half_to_f32(ora_rd16(blk));
+            for (int b = 0; b < 8; b++) {
+                uint32_t aux = ora_rd32(blk + 66 + 4 * b);
+                float db = d * (0.5f + (float)(aux >> 28)) * 0.5f;
+                for (int n = 0; n < 32; n++) {
+                    int v = iq3xxs_value(blk, b, n);
                     float mag = (float)(v < 0 ? -v : v);
                     out[32 * b + n] = db * mag * (v < 0 ? -1.0f : 1.0f);
                 }

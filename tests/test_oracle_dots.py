@@ -16,7 +16,7 @@ import ora
 from common import KVALUES_IQ4NL, iq4xs_rows, normal_f32
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-TYPES = (ora.Q4_K, ora.Q5_K, ora.Q6_K, ora.IQ2_XXS, ora.IQ4_XS)
+TYPES = (ora.Q4_K, ora.Q5_K, ora.Q6_K, ora.IQ2_XXS, ora.IQ3_XXS, ora.IQ4_XS)
 
 
 # ---------------------------------------------------------------- independent numpy decoders (written from the
@@ -39,6 +39,19 @@ def parse_tables():
 
 
 GRID, KSIGNS = parse_tables()["oracle/iq_tables.h"]
+
+
+def parse_grid3():
+    import re
+    out = {}
+    for path in ("oracle/iq_tables.h", "bloomery_amd/csrc/iq2xxs_tables.h"):
+        text = open(os.path.join(HERE, "..", path)).read()
+        body = re.search(r"IQ3XXS_GRID\[256\] = \{(.*?)\};", text, re.S).group(1)
+        out[path] = [int(v, 16) for v in re.findall(r"0x([0-9a-f]{8})u", body)]
+    return out
+
+
+GRID3 = parse_grid3()["oracle/iq_tables.h"]
 
 
 def q4k_decode(blk):
@@ -104,6 +117,25 @@ def iq2xxs_decode(blk):
     return codes, vals, (d, scs)
 
 
+def iq3xxs_decode(blk):
+    """block_iq3_xxs (crates/gguf/src/quant.rs:1739-1747): d, 64 grid indices (eight a sub-block, four magnitudes a
+    word), then a word a sub-block: four 7-bit sign indices and the scale in the top nibble."""
+    d = f16(blk[0], blk[1])
+    codes = np.zeros(256, np.int64)
+    scs = []
+    for b in range(8):
+        aux = int(blk[66 + 4 * b]) | (int(blk[67 + 4 * b]) << 8) | (int(blk[68 + 4 * b]) << 16) | (int(blk[69 + 4 * b]) << 24)
+        scs.append(aux >> 28)
+        for l in range(4):
+            s = KSIGNS[(aux >> (7 * l)) & 127]
+            for j in range(8):
+                g = GRID3[int(blk[2 + 8 * b + 2 * l + j // 4])]
+                mag = (g >> (8 * (j % 4))) & 0xFF
+                codes[32 * b + 8 * l + j] = -mag if (s >> j) & 1 else mag
+    vals = np.array([d * (0.5 + scs[n // 32]) * 0.5 * codes[n] for n in range(256)], np.float64)
+    return codes, vals, (d, scs)
+
+
 def iq4xs_decode(blk):
     """block_iq4_xs (crates/gguf/src/quant.rs:1969-1976): d, scales_h, scales_l[4], then sixteen bytes a sub-block,
     low nibbles its first sixteen values, high nibbles the other sixteen."""
@@ -119,7 +151,7 @@ def iq4xs_decode(blk):
     return codes, vals, (d, ls)
 
 
-DECODE = {ora.IQ4_XS: iq4xs_decode, ora.Q4_K: q4k_decode, ora.Q5_K: q5k_decode, ora.Q6_K: q6k_decode, ora.IQ2_XXS: iq2xxs_decode}
+DECODE = {ora.IQ3_XXS: iq3xxs_decode, ora.IQ4_XS: iq4xs_decode, ora.Q4_K: q4k_decode, ora.Q5_K: q5k_decode, ora.Q6_K: q6k_decode, ora.IQ2_XXS: iq2xxs_decode}
 
 
 def act_codes(wtype, col, k):
@@ -142,7 +174,7 @@ def random_blocks(wtype, nb, rng):
     w = rng.integers(0, 256, nb * bb, dtype=np.uint8)
     for i in range(nb):
         h = np.array([rng.uniform(-0.1, 0.1), rng.uniform(0.0, 0.1)], np.float16).view(np.uint8)
-        off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ4_XS: 0}[wtype]
+        off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ3_XXS: 0, ora.IQ4_XS: 0}[wtype]
         w[i * bb + off:i * bb + off + 2] = h[0:2]
         if wtype in (ora.Q4_K, ora.Q5_K):
             w[i * bb + 2:i * bb + 4] = h[2:4]
@@ -154,6 +186,8 @@ def quantized_rows(wtype, rows, k, seed):
     x = normal_f32(rng, (rows, k), 0.02)
     if wtype == ora.IQ4_XS:
         return iq4xs_rows(x), x
+    if wtype == ora.IQ3_XXS:  # no quantizer of this type in the reference's gguf crate: random legal blocks
+        return random_blocks(wtype, rows * (k // 256), rng), x
     return ora.quantize_rows(wtype, x, rows, k, n_threads=4), x
 
 
@@ -166,6 +200,14 @@ def test_codebook_digests_and_closed_form():
         assert hashlib.md5(struct.pack("<256Q", *grid)).hexdigest() == "fff55639176d84643cf2facd7a655c4d", path
         assert all(ks[i] == (i | ((bin(i).count("1") & 1) << 7)) for i in range(128)), path
         assert all(((g >> (8 * j)) & 0xFF) in (8, 25, 43) for g in grid for j in range(8)), path
+
+
+def test_iq3xxs_grid_digest_and_structure():
+    # crates/gguf/src/iq_tables.rs:293-295; every byte 4 + 8k or 62 (crates/gguf/src/quant.rs iq_tables_have_ggml_structure)
+    for path, grid in parse_grid3().items():
+        assert len(grid) == 256, path
+        assert hashlib.md5(struct.pack("<256I", *grid)).hexdigest() == "0ee1848d3f04a5720691cb6e7daee92e", path
+        assert all(((g >> (8 * j)) & 0xFF) in (4, 12, 20, 28, 36, 44, 52, 62) for g in grid for j in range(4)), path
 
 
 def test_iq4_levels_digest():
@@ -239,13 +281,14 @@ def test_block_sums_equal_brute_force(wtype):
                 assert list(lanes[8 * i:8 * i + 8]) == want
             assert ora.iq4xs_block_sums(w, col, k, fold=True)[1].tolist() == lanes.tolist(), "no -128 code on these inputs"
         else:
-            i_b, sc, codes, fold = ora.iq2xxs_block_sums(w, col, k)
+            off = 64 if wtype == ora.IQ3_XXS else 43
+            i_b, sc, codes, fold = ora.iq2xxs_block_sums(w, col, k, iq3=wtype == ora.IQ3_XXS)
             assert list(i_b) == [int(prod[32 * b:32 * b + 32].sum()) for b in range(nb * 8)]
             for i in range(nb):
                 s = [2 * DECODE[wtype](w[i * bb:(i + 1) * bb])[2][1][b] + 1 for b in range(8)]
                 assert list(sc[8 * i:8 * i + 8]) == s
                 bs = [int(a[256 * i + 32 * b:256 * i + 32 * b + 32].sum()) for b in range(8)]
-                assert codes[i] == sum(s[b] * (int(i_b[8 * i + b]) + 43 * bs[b]) for b in range(8))
+                assert codes[i] == sum(s[b] * (int(i_b[8 * i + b]) + off * bs[b]) for b in range(8))
                 assert fold[i] == sum(s[b] * bs[b] for b in range(8))
 
 
@@ -312,7 +355,7 @@ def extreme_cases(wtype, rng):
         w = np.full(2 * bb, fill, np.uint8)
         for i in range(2):
             h = np.array([dval, abs(dval)], np.float16).view(np.uint8)
-            off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ4_XS: 0}[wtype]
+            off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ3_XXS: 0, ora.IQ4_XS: 0}[wtype]
             w[i * bb + off:i * bb + off + 2] = h[0:2]
             if wtype in (ora.Q4_K, ora.Q5_K):
                 w[i * bb + 2:i * bb + 4] = h[2:4]
@@ -389,11 +432,12 @@ def test_dot_within_f64_band_of_dequantized_dot(wtype):
                 assert np.allclose(dq, act, rtol=1e-7, atol=0)  # an f32 scale times a code rounds once
             else:
                 assert np.array_equal(dq, act), "a bf16 scale times an 8-bit code is exact in f32"
-            if wtype == ora.IQ2_XXS:
-                # the kernel's own grouping: d/8 * (2s+1) * grid, with the +43 offset folded out exactly
+            if wtype in (ora.IQ2_XXS, ora.IQ3_XXS):
+                # the kernel's own grouping: d/8 * (2s+1) * grid (IQ3_XXS: d/4), with the +43 (+64) offset folded out
+                unit, both = (0.125, 86) if wtype == ora.IQ2_XXS else (0.25, 128)
                 wv = np.concatenate([DECODE[wtype](w[i * bb:(i + 1) * bb])[1] for i in range(nb)])
-                extra = np.concatenate([np.repeat([0.125 * abs(DECODE[wtype](w[i * bb:(i + 1) * bb])[2][0]) *
-                                                   (2 * s + 1) * 86 for s in DECODE[wtype](w[i * bb:(i + 1) * bb])[2][1]],
+                extra = np.concatenate([np.repeat([unit * abs(DECODE[wtype](w[i * bb:(i + 1) * bb])[2][0]) *
+                                                   (2 * s + 1) * both for s in DECODE[wtype](w[i * bb:(i + 1) * bb])[2][1]],
                                                   32) for i in range(nb)])
                 mag = np.sum((np.abs(wv) + extra) * np.abs(act))
                 terms = 2 * nb + 10

@@ -30,12 +30,14 @@ typedef uint32_t u32;
 #define BM_Q5K 13
 #define BM_Q6K 14
 #define BM_IQ2XXS 16
+#define BM_IQ3XXS 18
 #define BM_IQ4XS 23
 
 #define BM_Q4K_BLOCK 144
 #define BM_Q5K_BLOCK 176
 #define BM_Q6K_BLOCK 210
 #define BM_IQ2XXS_BLOCK 66
+#define BM_IQ3XXS_BLOCK 98
 #define BM_IQ4XS_BLOCK 136
 #define BM_Q82X4_STRIDE 144
 #define BM_Q8K_STRIDE 296
@@ -181,7 +183,7 @@ struct ActView {
 };
 
 // The types that dot against a Q8_K column (crates/gguf/src/qtype.rs host_act); the others take Q8_2_X4.
-__host__ __device__ constexpr bool bm_takes_q8k(int wt) { return wt == BM_IQ2XXS || wt == BM_IQ4XS; }
+__host__ __device__ constexpr bool bm_takes_q8k(int wt) { return wt == BM_IQ2XXS || wt == BM_IQ3XXS || wt == BM_IQ4XS; }
 
 // Bytes of one column of nb super-blocks on the device, in the form type WT dots against.
 template <int WT>
@@ -456,8 +458,10 @@ __device__ __forceinline__ Blk<BM_IQ2XXS> bm_load_iq2xxs(const uint8_t *wrow, in
 // back out through the column's sums, so the tables give u with two operations a word: a grid point is kept as its
 // eight magnitudes + 43 (x, y) and its eight doubled magnitudes (z, w), a sign index as eight byte masks (0xff where
 // the value is negative): u = (mag + 43) - (2 mag & mask), byte by byte without a borrow.
+// IQ3_XXS: the same with the offset 64 and grid points of four magnitudes: an entry is (magnitudes + 64, doubled).
 struct Iq2Tables {
-    const uint4 *grid;
+    const uint4 *grid;  // IQ2_XXS
+    const uint2 *grid3; // IQ3_XXS
     const uint2 *signs;
 };
 
@@ -506,15 +510,16 @@ __device__ __forceinline__ Iq2Dec bm_decode_iq2xxs(const Blk<BM_IQ2XXS> &b, int 
     return dec;
 }
 
-template <class Tap>
-__device__ __forceinline__ void bm_dot_iq2xxs_dec(const Blk<BM_IQ2XXS> &b, const Iq2Dec &dec, const Act<BM_IQ2XXS> &act,
-                                                  int i, int q, float &acc0, float &acc1, const Tap &tap) {
+// The float and integer steps IQ2_XXS and IQ3_XXS share (crates/qdot/src/lib.rs:8677-8724, :7494-7541): the fold of
+// the offset through the column's 16-value sums first, then the scaled sums of offset byte x code. `off`: 43 / 64;
+// d: f16 / 8 or f16 / 4; sca, scb: the scales 2s + 1 of the lane's own sub-blocks 2q and 2q + 1.
+template <int OFF, class Tap>
+__device__ __forceinline__ void bm_dot_iqx_dec(float d, int sca, int scb, const Iq2Dec &dec, const Act<BM_IQ2XXS> &act,
+                                               int i, int q, float &acc0, float &acc1, const Tap &tap) {
     const float dy = act.dy;
-    const float d = 0.125f * bm_half_to_f32(b.d);
-    const float dmin = -d * 43.0f;
+    const float dmin = -d * (float)OFF;
     // Fold first (crates/qdot/src/lib.rs:8691-8694): accumulator l takes sub-block l's scale on its two bsums.
     {
-        const int sca = 2 * (int)(b.q.y >> 28) + 1, scb = 2 * (int)(b.q.w >> 28) + 1; // sub-blocks 2q, 2q + 1
         const uint2 bs = act.bs;
         const int b0 = (int)(short)(bs.x & 0xffffu), b1 = (int)(short)(bs.x >> 16);
         const int b2 = (int)(short)(bs.y & 0xffffu), b3 = (int)(short)(bs.y >> 16);
@@ -527,13 +532,13 @@ __device__ __forceinline__ void bm_dot_iq2xxs_dec(const Blk<BM_IQ2XXS> &b, const
 #pragma unroll
     for (int sb = 0; sb < 8; sb++) {
         const uint2 a = act.a[sb];
-        // the reference sums sc * u * a (the 43s come back out through the fold above); sums within 4 * 86 * 128 and
-        // sc <= 31 lie inside 24 bits
+        // the reference sums sc * u * a (the offsets come back out through the fold above); sums within 4 * 126 * 128
+        // and sc <= 31 lie inside 24 bits
         const int d_lo = bm_sdot4(dec.u_lo[sb], a.x, 0), d_hi = bm_sdot4(dec.u_hi[sb], a.y, 0);
         sumi0 = bm_mad24(dec.sc[sb], d_lo, sumi0);
         sumi1 = bm_mad24(dec.sc[sb], d_hi, sumi1);
-        if constexpr (Tap::kActive) // the signed sum: less 43 times the eight codes
-            tap.iq2(i, sb, q, d_lo + d_hi - 43 * (bm_sdot4(0x01010101u, a.x, 0) + bm_sdot4(0x01010101u, a.y, 0)));
+        if constexpr (Tap::kActive) // the signed sum: less the offset times the eight codes
+            tap.iq2(i, sb, q, d_lo + d_hi - OFF * (bm_sdot4(0x01010101u, a.x, 0) + bm_sdot4(0x01010101u, a.y, 0)));
     }
     const float f = d * dy;
     acc0 = fmaf(f, (float)sumi0, acc0);
@@ -541,10 +546,78 @@ __device__ __forceinline__ void bm_dot_iq2xxs_dec(const Blk<BM_IQ2XXS> &b, const
 }
 
 template <class Tap>
+__device__ __forceinline__ void bm_dot_iq2xxs_dec(const Blk<BM_IQ2XXS> &b, const Iq2Dec &dec, const Act<BM_IQ2XXS> &act,
+                                                  int i, int q, float &acc0, float &acc1, const Tap &tap) {
+    bm_dot_iqx_dec<43>(0.125f * bm_half_to_f32(b.d), 2 * (int)(b.q.y >> 28) + 1, 2 * (int)(b.q.w >> 28) + 1, dec, act, i, q,
+                       acc0, acc1, tap);
+}
+
+template <class Tap>
 __device__ __forceinline__ void bm_dot_iq2xxs(const Blk<BM_IQ2XXS> &b, const Act<BM_IQ2XXS> &act, int i, int q,
                                               const Iq2Tables &tb, float &acc0, float &acc1, const Tap &tap) {
     const Iq2Dec dec = bm_decode_iq2xxs(b, q, tb);
     bm_dot_iq2xxs_dec(b, dec, act, i, q, acc0, acc1, tap);
+}
+
+// ---- IQ3_XXS (crates/qdot/src/lib.rs:7494-7541): IQ2_XXS's lane map. Lane q owns accumulators 2q and 2q + 1: the
+// values 8q .. 8q + 7 of every sub-block, i.e. the two four-magnitude grid words its index bytes 2q and 2q + 1 name
+// and the sub-block's sign group q. The quad loads the block's 64 index bytes and eight sign/scale words once
+// (16 + 8 bytes a lane: sub-blocks 2q and 2q + 1) and shares them through DPP.
+template <>
+struct Blk<BM_IQ3XXS> {
+    uint4 qi;  // the index bytes of sub-blocks 2q (x, y) and 2q + 1 (z, w)
+    uint2 aux; // their sign/scale words
+    u32 d;
+};
+
+__device__ __forceinline__ Blk<BM_IQ3XXS> bm_load_iq3xxs(const uint8_t *wrow, int i, int q) {
+    const uint8_t *blk = wrow + (size_t)i * BM_IQ3XXS_BLOCK;
+    Blk<BM_IQ3XXS> b;
+    b.qi = bm_ld16u(blk + 2 + 16 * q);
+    __builtin_memcpy(&b.aux, blk + 66 + 8 * q, 8);
+    b.d = bm_ld2u(blk);
+    return b;
+}
+
+template <>
+struct Act<BM_IQ3XXS> : Act<BM_IQ2XXS> {};
+
+__device__ __forceinline__ Iq2Dec bm_decode_iq3xxs(const Blk<BM_IQ3XXS> &b, int q, const Iq2Tables &tb) {
+    Iq2Dec dec;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        // sub-blocks 2k and 2k + 1 sit in lane k of the quad; this lane's two index bytes are bytes 2q, 2q + 1 of a
+        // sub-block's eight: the first word's for q < 2, the second's otherwise
+        const u32 ia0 = bm_quad_bcast(b.qi.x, k), ia1 = bm_quad_bcast(b.qi.y, k);
+        const u32 ib0 = bm_quad_bcast(b.qi.z, k), ib1 = bm_quad_bcast(b.qi.w, k);
+        const u32 aux_a = bm_quad_bcast(b.aux.x, k), aux_b = bm_quad_bcast(b.aux.y, k);
+#pragma unroll
+        for (int e = 0; e < 2; e++) {
+            const int sb = 2 * k + e;
+            const u32 word = (q & 2) ? (e ? ib1 : ia1) : (e ? ib0 : ia0), aux = e ? aux_b : aux_a;
+            const u32 pair = word >> (16 * (q & 1));
+            dec.sc[sb] = 2 * (int)(aux >> 28) + 1;
+            const uint2 g0 = tb.grid3[pair & 0xffu], g1 = tb.grid3[(pair >> 8) & 0xffu];
+            const uint2 sg = tb.signs[(aux >> (7 * q)) & 127u];
+            dec.u_lo[sb] = g0.x - (g0.y & sg.x);
+            dec.u_hi[sb] = g1.x - (g1.y & sg.y);
+        }
+    }
+    return dec;
+}
+
+template <class Tap>
+__device__ __forceinline__ void bm_dot_iq3xxs_dec(const Blk<BM_IQ3XXS> &b, const Iq2Dec &dec, const Act<BM_IQ3XXS> &act,
+                                                  int i, int q, float &acc0, float &acc1, const Tap &tap) {
+    bm_dot_iqx_dec<64>(0.25f * bm_half_to_f32(b.d), 2 * (int)(b.aux.x >> 28) + 1, 2 * (int)(b.aux.y >> 28) + 1, dec, act, i,
+                       q, acc0, acc1, tap);
+}
+
+template <class Tap>
+__device__ __forceinline__ void bm_dot_iq3xxs(const Blk<BM_IQ3XXS> &b, const Act<BM_IQ3XXS> &act, int i, int q,
+                                              const Iq2Tables &tb, float &acc0, float &acc1, const Tap &tap) {
+    const Iq2Dec dec = bm_decode_iq3xxs(b, q, tb);
+    bm_dot_iq3xxs_dec(b, dec, act, i, q, acc0, acc1, tap);
 }
 
 // ---- IQ4_XS (crates/qdot/src/lib.rs:11033-11180): lane q reads sub-blocks 2q and 2q + 1 whole (32 consecutive code
@@ -695,6 +768,10 @@ __device__ __forceinline__ Blk<BM_IQ2XXS> bm_load_blk<BM_IQ2XXS>(const uint8_t *
     return bm_load_iq2xxs(wrow, i, q);
 }
 template <>
+__device__ __forceinline__ Blk<BM_IQ3XXS> bm_load_blk<BM_IQ3XXS>(const uint8_t *wrow, int i, int q) {
+    return bm_load_iq3xxs(wrow, i, q);
+}
+template <>
 __device__ __forceinline__ Blk<BM_IQ4XS> bm_load_blk<BM_IQ4XS>(const uint8_t *wrow, int i, int q) {
     return bm_load_iq4xs(wrow, i, q);
 }
@@ -711,7 +788,11 @@ __device__ __forceinline__ Act<WT> bm_load_act(const ActView &av, int i, int q) 
         return bm_act_q6k(av, i, q & 1, q >> 1);
     else if constexpr (WT == BM_IQ4XS)
         return bm_act_iq4xs(av, i, q);
-    else
+    else if constexpr (WT == BM_IQ3XXS) {
+        Act<BM_IQ3XXS> a;
+        static_cast<Act<BM_IQ2XXS> &>(a) = bm_act_iq2xxs(av, i, q);
+        return a;
+    } else
         return bm_act_iq2xxs(av, i, q);
 }
 
@@ -726,13 +807,15 @@ __device__ __forceinline__ void bm_dot_blk(const Blk<WT> &b, const Act<WT> &a, i
         bm_dot_q6k(b, a, i, q & 1, q >> 1, acc0, acc1, tap);
     else if constexpr (WT == BM_IQ4XS)
         bm_dot_iq4xs(b, a, i, q, acc0, acc1, tap);
+    else if constexpr (WT == BM_IQ3XXS)
+        bm_dot_iq3xxs(b, a, i, q, tb, acc0, acc1, tap);
     else
         bm_dot_iq2xxs(b, a, i, q, tb, acc0, acc1, tap);
 }
 
 template <int WT>
 __host__ __device__ constexpr int bm_block_bytes() {
-    return WT == BM_Q4K ? BM_Q4K_BLOCK : WT == BM_Q5K ? BM_Q5K_BLOCK : WT == BM_Q6K ? BM_Q6K_BLOCK : WT == BM_IQ4XS ? BM_IQ4XS_BLOCK : BM_IQ2XXS_BLOCK;
+    return WT == BM_Q4K ? BM_Q4K_BLOCK : WT == BM_Q5K ? BM_Q5K_BLOCK : WT == BM_Q6K ? BM_Q6K_BLOCK : WT == BM_IQ4XS ? BM_IQ4XS_BLOCK : WT == BM_IQ3XXS ? BM_IQ3XXS_BLOCK : BM_IQ2XXS_BLOCK;
 }
 
 // ---- SwiGLU: crates/qdot/src/lib.rs:3741-3773 (expf) and :11467-11478 (divide, then multiply).

@@ -576,13 +576,16 @@ __global__ __launch_bounds__(64) void k_block_sums(const uint8_t *wrow, int nb, 
     preload<WT, U>(b, wrow, q);
     float v[1];
     row_dot<WT, U, NB, 1>(b, wrow, col, col_bytes, 1, n, q, tb, v, StoreTap{out});
-    if constexpr (WT == BM_IQ2XXS) {
+    if constexpr (WT == BM_IQ2XXS || WT == BM_IQ3XXS) {
         // the eight scales 2s + 1 of each super-block, as the dot reads them
         if (q == 0)
             for (int i = 0; i < n; i++)
                 for (int s = 0; s < 8; s++) {
                     u32 aux;
-                    __builtin_memcpy(&aux, wrow + (size_t)i * BM_IQ2XXS_BLOCK + 6 + 8 * s, 4);
+                    if constexpr (WT == BM_IQ2XXS)
+                        __builtin_memcpy(&aux, wrow + (size_t)i * BM_IQ2XXS_BLOCK + 6 + 8 * s, 4);
+                    else
+                        __builtin_memcpy(&aux, wrow + (size_t)i * BM_IQ3XXS_BLOCK + 66 + 4 * s, 4);
                     out[16 * i + 8 + s] = 2 * (int)(aux >> 28) + 1;
                 }
     }

@@ -30,14 +30,28 @@ constexpr u32 kSiteStalled = 31;    // ours: a fused launch's down workgroup gav
 // LDS bytes of the IQ2_XXS tables: 256 grid entries of 16 + 128 sign entries of 8.
 constexpr int kTabBytes = 256 * 16 + 128 * 8;
 
+constexpr int kTabBytes3 = 256 * 8 + 128 * 8; // IQ3_XXS: 256 grid entries of 8 + 128 sign entries of 8
+
 template <int WT>
 __host__ __device__ constexpr int tab_bytes() {
-    return WT == BM_IQ2XXS ? kTabBytes : 0;
+    return WT == BM_IQ2XXS ? kTabBytes : WT == BM_IQ3XXS ? kTabBytes3 : 0;
+}
+
+// A sign index's eight signs as two words of byte masks: 0xff where the value is negative.
+__device__ __forceinline__ uint2 iq_sign_masks(int t) {
+    const u32 sg = BM_KSIGNS_IQ2XS[t];
+    u32 m[2];
+    for (int half = 0; half < 2; half++) {
+        const u32 nib = (sg >> (4 * half)) & 15u;
+        m[half] = ((nib & 1) ? 0xffu : 0u) | ((nib & 2) ? 0xff00u : 0u) | ((nib & 4) ? 0xff0000u : 0u) |
+                  ((nib & 8) ? 0xff000000u : 0u);
+    }
+    return make_uint2(m[0], m[1]);
 }
 
 template <int WT>
 __device__ __forceinline__ Iq2Tables stage_tables(uint8_t *lds) {
-    Iq2Tables tb{nullptr, nullptr};
+    Iq2Tables tb{nullptr, nullptr, nullptr};
     if constexpr (WT == BM_IQ2XXS) {
         uint4 *grid = reinterpret_cast<uint4 *>(lds);
         uint2 *signs = reinterpret_cast<uint2 *>(lds + 256 * 16);
@@ -46,17 +60,19 @@ __device__ __forceinline__ Iq2Tables stage_tables(uint8_t *lds) {
             const u32 lo = (u32)g, hi = (u32)(g >> 32);
             grid[t] = make_uint4(lo + 0x2b2b2b2bu, hi + 0x2b2b2b2bu, lo << 1, hi << 1);
         }
-        for (int t = threadIdx.x; t < 128; t += blockDim.x) {
-            const u32 sg = BM_KSIGNS_IQ2XS[t];
-            u32 m[2];
-            for (int half = 0; half < 2; half++) {
-                const u32 nib = (sg >> (4 * half)) & 15u;
-                m[half] = ((nib & 1) ? 0xffu : 0u) | ((nib & 2) ? 0xff00u : 0u) | ((nib & 4) ? 0xff0000u : 0u) |
-                          ((nib & 8) ? 0xff000000u : 0u);
-            }
-            signs[t] = make_uint2(m[0], m[1]);
-        }
+        for (int t = threadIdx.x; t < 128; t += blockDim.x) signs[t] = iq_sign_masks(t);
         tb.grid = grid;
+        tb.signs = signs;
+    }
+    if constexpr (WT == BM_IQ3XXS) {
+        uint2 *grid = reinterpret_cast<uint2 *>(lds);
+        uint2 *signs = reinterpret_cast<uint2 *>(lds + 256 * 8);
+        for (int t = threadIdx.x; t < 256; t += blockDim.x) {
+            const u32 g = BM_IQ3XXS_GRID[t]; // bytes 4 .. 62: + 64 and doubled stay inside a byte
+            grid[t] = make_uint2(g + 0x40404040u, g << 1);
+        }
+        for (int t = threadIdx.x; t < 128; t += blockDim.x) signs[t] = iq_sign_masks(t);
+        tb.grid3 = grid;
         tb.signs = signs;
     }
     return tb;
@@ -173,6 +189,14 @@ __device__ __forceinline__ void row_dot(Blk<WT> (&b)[U], const uint8_t *wrow, co
                     if (c < m) {
                         const Act<WT> a = bm_load_act<WT, Tap::kActive>(av[c], i, q);
                         bm_dot_iq2xxs_dec(b[slot], dec, a, i, q, a0[c], a1[c], tap);
+                    }
+            } else if constexpr (WT == BM_IQ3XXS) {
+                const Iq2Dec dec = bm_decode_iq3xxs(b[slot], q, tb);
+#pragma unroll
+                for (int c = 0; c < M; c++)
+                    if (c < m) {
+                        const Act<WT> a = bm_load_act<WT, Tap::kActive>(av[c], i, q);
+                        bm_dot_iq3xxs_dec(b[slot], dec, a, i, q, a0[c], a1[c], tap);
                     }
             } else if constexpr (WT == BM_IQ4XS) { // likewise the level permutes
                 const Iq4Dec dec = bm_decode_iq4xs(b[slot], q);
@@ -420,6 +444,10 @@ constexpr int kRingQ4K = 4, kRingQ5K = 4, kRingQ6K = 3;
         if ((nb) % 2 == 0) BM_VARIANT(BM_IQ2XXS, 2, 0)                                                                 \
         else BM_VARIANT(BM_IQ2XXS, 1, 0)                                                                               \
         break;                                                                                                         \
+    case BM_IQ3XXS:                                                                                                    \
+        if ((nb) % 2 == 0) BM_VARIANT(BM_IQ3XXS, 2, 0)                                                                 \
+        else BM_VARIANT(BM_IQ3XXS, 1, 0)                                                                               \
+        break;                                                                                                         \
     case BM_IQ4XS:                                                                                                     \
         if ((nb) % 2 == 0) BM_VARIANT(BM_IQ4XS, 2, 0)                                                                  \
         else BM_VARIANT(BM_IQ4XS, 1, 0)                                                                                \
@@ -428,7 +456,7 @@ constexpr int kRingQ4K = 4, kRingQ5K = 4, kRingQ6K = 3;
         return hipErrorInvalidValue;                                                                                   \
     }
 
-static inline int tab_bytes_rt(int wtype) { return wtype == BM_IQ2XXS ? kTabBytes : 0; }
+static inline int tab_bytes_rt(int wtype) { return wtype == BM_IQ2XXS ? kTabBytes : wtype == BM_IQ3XXS ? kTabBytes3 : 0; }
 
 } // namespace bmk
 

@@ -1,4 +1,4 @@
-"""bloomery_amd: MI355X-native quantized MoE expert matmul (Q4_K / Q5_K / Q6_K / IQ2_XXS / IQ3_XXS / IQ4_XS x Q8) behind the kernel-call
+"""bloomery_amd: MI355X-native quantized MoE expert matmul (Q3_K / Q4_K / Q5_K / Q6_K / IQ2_XXS / IQ3_XXS / IQ4_XS x Q8) behind the kernel-call
 surface of the reference's crates/gpu.
 
 This module is a thin ctypes view of the C ABI in include/bm_moe.h (bloomery_amd/libbm_moe_hip.so, hand-written
@@ -16,7 +16,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libbm_moe_hip.so")
 
-Q4_K, Q5_K, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_XS = 12, 13, 14, 16, 18, 23
+Q3_K, Q4_K, Q5_K, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_XS = 11, 12, 13, 14, 16, 18, 23
 FAULT_NONE = 0xFFFFFFFF
 LAYER_NONE = 0xFFFF
 SITE_QUANT_COLUMN, SITE_ROUTER, SITE_EXPERT_ID, SITE_STALLED = 1, 5, 7, 31

@@ -62,10 +62,10 @@ static int driver(bm_ctx *ctx, const char *what, hipError_t e) {
 }
 
 static bool known_type(int t) {
-    return t == BM_TYPE_Q4_K || t == BM_TYPE_Q5_K || t == BM_TYPE_Q6_K || t == BM_TYPE_IQ2_XXS || t == BM_TYPE_IQ3_XXS || t == BM_TYPE_IQ4_XS;
+    return t == BM_TYPE_Q3_K || t == BM_TYPE_Q4_K || t == BM_TYPE_Q5_K || t == BM_TYPE_Q6_K || t == BM_TYPE_IQ2_XXS || t == BM_TYPE_IQ3_XXS || t == BM_TYPE_IQ4_XS;
 }
-// Q8_2_X4 for the K-quants, Q8_K for IQ2_XXS, IQ3_XXS and IQ4_XS (crates/gguf/src/qtype.rs host_act).
-static int act_form(int t) { return t == BM_TYPE_IQ2_XXS || t == BM_TYPE_IQ3_XXS || t == BM_TYPE_IQ4_XS ? 1 : 0; }
+// Q8_2_X4 for Q4_K, Q5_K and Q6_K, Q8_K for Q3_K, IQ2_XXS, IQ3_XXS and IQ4_XS (crates/gguf/src/qtype.rs host_act).
+static int act_form(int t) { return t == BM_TYPE_Q3_K || t == BM_TYPE_IQ2_XXS || t == BM_TYPE_IQ3_XXS || t == BM_TYPE_IQ4_XS ? 1 : 0; }
 // Bytes between two columns of a bm_act on the device (the CPU path's bytes plus the dot kernels' tables).
 static size_t dev_col_bytes(int wtype, int k) { return (size_t)bmk::act_col_bytes(wtype, k); }
 
@@ -76,7 +76,7 @@ int bm_version(void) { return 101; }
 int64_t bm_row_bytes(int wtype, int k) {
     if (!known_type(wtype)) return BM_ETYPE;
     if (k <= 0 || k % 256 != 0) return BM_ESHAPE;
-    const int bb = wtype == BM_TYPE_Q4_K ? 144 : wtype == BM_TYPE_Q5_K ? 176 : wtype == BM_TYPE_Q6_K ? 210 : wtype == BM_TYPE_IQ4_XS ? 136 : wtype == BM_TYPE_IQ3_XXS ? 98 : 66;
+    const int bb = wtype == BM_TYPE_Q3_K ? 110 : wtype == BM_TYPE_Q4_K ? 144 : wtype == BM_TYPE_Q5_K ? 176 : wtype == BM_TYPE_Q6_K ? 210 : wtype == BM_TYPE_IQ4_XS ? 136 : wtype == BM_TYPE_IQ3_XXS ? 98 : 66;
     return (int64_t)(k / 256) * bb;
 }
 
@@ -222,7 +222,7 @@ static int weights_make(bm_ctx *ctx, const char *what, int wtype, int64_t rows, 
                         const void *dev, bm_weights **out) {
     if (!ctx || !out) return fail(ctx, BM_EARG, "%s: NULL argument", what);
     *out = nullptr;
-    if (!known_type(wtype)) return fail(ctx, BM_ETYPE, "%s: weight type %d has no kernel (12 Q4_K, 13 Q5_K, 14 Q6_K, 16 IQ2_XXS, 18 IQ3_XXS, 23 IQ4_XS)", what, wtype);
+    if (!known_type(wtype)) return fail(ctx, BM_ETYPE, "%s: weight type %d has no kernel (11 Q3_K, 12 Q4_K, 13 Q5_K, 14 Q6_K, 16 IQ2_XXS, 18 IQ3_XXS, 23 IQ4_XS)", what, wtype);
     if (k <= 0 || k % 256 != 0) return fail(ctx, BM_ESHAPE, "%s: k = %d is not a whole number of 256-value super-blocks", what, k);
     if (rows <= 0) return fail(ctx, BM_ESHAPE, "%s: rows = %lld must be positive", what, (long long)rows);
     const size_t bytes = (size_t)rows * (size_t)bm_row_bytes(wtype, k);
@@ -800,7 +800,7 @@ int bm_weights_from_gguf(bm_ctx *ctx, const bm_gguf *g, const char *name, bm_wei
     bm_gguf_tensor t;
     if (bm_gguf_find(g, name, &t) != BM_OK) return fail(ctx, BM_ESHAPE, "%s: %s", what, bm_gguf_last_error());
     if (!known_type(t.type))
-        return fail(ctx, BM_ETYPE, "%s: %s is of ggml type %d; this library computes in Q4_K (12), Q5_K (13), Q6_K (14), IQ2_XXS (16), IQ3_XXS (18) and IQ4_XS (23)", what,
+        return fail(ctx, BM_ETYPE, "%s: %s is of ggml type %d; this library computes in Q3_K (11), Q4_K (12), Q5_K (13), Q6_K (14), IQ2_XXS (16), IQ3_XXS (18) and IQ4_XS (23)", what,
                     name, t.type);
     if (t.n_dims < 2 || t.n_dims > 3)
         return fail(ctx, BM_ESHAPE, "%s: %s has %d dimensions; a matrix has 2, an expert stack 3", what, name, t.n_dims);

@@ -26,6 +26,7 @@
 
 typedef uint32_t u32;
 
+#define BM_Q3K 11
 #define BM_Q4K 12
 #define BM_Q5K 13
 #define BM_Q6K 14
@@ -33,6 +34,7 @@ typedef uint32_t u32;
 #define BM_IQ3XXS 18
 #define BM_IQ4XS 23
 
+#define BM_Q3K_BLOCK 110
 #define BM_Q4K_BLOCK 144
 #define BM_Q5K_BLOCK 176
 #define BM_Q6K_BLOCK 210
@@ -183,7 +185,9 @@ struct ActView {
 };
 
 // The types that dot against a Q8_K column (crates/gguf/src/qtype.rs host_act); the others take Q8_2_X4.
-__host__ __device__ constexpr bool bm_takes_q8k(int wt) { return wt == BM_IQ2XXS || wt == BM_IQ3XXS || wt == BM_IQ4XS; }
+__host__ __device__ constexpr bool bm_takes_q8k(int wt) {
+    return wt == BM_Q3K || wt == BM_IQ2XXS || wt == BM_IQ3XXS || wt == BM_IQ4XS;
+}
 
 // Bytes of one column of nb super-blocks on the device, in the form type WT dots against.
 template <int WT>
@@ -620,6 +624,82 @@ __device__ __forceinline__ void bm_dot_iq3xxs(const Blk<BM_IQ3XXS> &b, const Act
     bm_dot_iq3xxs_dec(b, dec, act, i, q, acc0, acc1, tap);
 }
 
+// ---- Q3_K (crates/qdot/src/lib.rs:2223-2245, layout crates/gguf/src/quant.rs:671-678): one integer a super-block
+// and one f32 accumulator a row. Lane q takes the 16 field bytes 16q .. of qs: half j = q / 2, cells 16 (q % 2) .. + 15,
+// whose four two-bit fields are the 16-value groups 8j + 2f + q % 2, with the high bits of hmask bytes 16 (q % 2) ..
+// (bit 4j + f). A code u = low | high << 2 becomes the signed byte u - 4 through a byte permute of the eight levels;
+// the lane scales its four group sums, the quad adds the four shares, and every lane applies the same float step,
+// acc + (dcol * d) * sum with each operation rounded on its own.
+template <>
+struct Blk<BM_Q3K> {
+    uint4 qs, hm; // the lane's field bytes and the high-bit bytes of their cells
+    uint4 tail;   // block bytes 94 .. 109: the twelve scale bytes at 2 .., d at 14
+};
+
+__device__ __forceinline__ Blk<BM_Q3K> bm_load_q3k(const uint8_t *wrow, int i, int q) {
+    const uint8_t *blk = wrow + (size_t)i * BM_Q3K_BLOCK;
+    Blk<BM_Q3K> b;
+    b.qs = bm_ld16u(blk + 32 + 16 * q);
+    b.hm = bm_ld16u(blk + 16 * (q & 1));
+    b.tail = bm_ld16u(blk + 94);
+    return b;
+}
+
+template <>
+struct Act<BM_Q3K> {
+    float dcol;
+    uint2 a[8]; // field f's 16 codes: a[2f], a[2f + 1]
+};
+
+__device__ __forceinline__ Act<BM_Q3K> bm_act_q3k(const ActView &av, int i, int q) {
+    const uint8_t *blk = av.col + (size_t)i * BM_Q8K_STRIDE;
+    Act<BM_Q3K> a;
+    a.dcol = *reinterpret_cast<const float *>(blk);
+    const uint8_t *at = blk + 8 + 128 * (q >> 1) + 16 * (q & 1);
+#pragma unroll
+    for (int f = 0; f < 4; f++) {
+        a.a[2 * f] = *reinterpret_cast<const uint2 *>(at + 32 * f);
+        a.a[2 * f + 1] = *reinterpret_cast<const uint2 *>(at + 32 * f + 8);
+    }
+    return a;
+}
+
+template <class Tap>
+__device__ __forceinline__ void bm_dot_q3k(const Blk<BM_Q3K> &b, const Act<BM_Q3K> &act, int i, int q, float &acc0,
+                                           const Tap &tap) {
+    const int j = q >> 1, odd = q & 1;
+    // the sixteen six-bit scales (crates/qdot/src/lib.rs:2162-2174); this lane's are bytes 2 (f % 2) + q % 2 of words
+    // 2j + f / 2
+    const u32 a0 = (b.tail.x >> 16) | (b.tail.y << 16), a1 = (b.tail.y >> 16) | (b.tail.z << 16);
+    const u32 a2 = (b.tail.z >> 16) | (b.tail.w << 16);
+    const u32 lo = j ? (a0 >> 4) : a0, lo1 = j ? (a1 >> 4) : a1, hi = a2 >> (4 * j);
+    const u32 w0 = (lo & 0x0f0f0f0fu) | ((hi & 0x03030303u) << 4);
+    const u32 w1 = (lo1 & 0x0f0f0f0fu) | (((hi >> 2) & 0x03030303u) << 4);
+    const u32 qw[4] = {b.qs.x, b.qs.y, b.qs.z, b.qs.w}, hw[4] = {b.hm.x, b.hm.y, b.hm.z, b.hm.w};
+    int sum = 0;
+#pragma unroll
+    for (int f = 0; f < 4; f++) {
+        int g = 0;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const u32 low = (qw[t] >> (2 * f)) & 0x03030303u;
+            const u32 high = (hw[t] >> (4 * j + f)) & 0x01010101u;
+            // u = low | high << 2 picks its level: bytes -4, -3, -2, -1 then 0, 1, 2, 3
+            const u32 v = __builtin_amdgcn_perm(0x03020100u, 0xfffefdfcu, (high << 2) | low);
+            const uint2 a = act.a[2 * f + (t >> 1)];
+            g = bm_sdot4(v, (t & 1) ? a.y : a.x, g);
+        }
+        tap.q6k(i, 8 * j + 2 * f + odd, g);
+        const u32 word = (f >> 1) ? w1 : w0;
+        const int sc = (int)((word >> (8 * (2 * (f & 1) + odd))) & 0xffu) - 32;
+        sum = bm_mad24(sc, g, sum); // |g| <= 16 * 4 * 128, |sc| <= 32
+    }
+    sum += (int)bm_dpp<kDppXor1>((u32)sum);
+    sum += (int)bm_dpp<kDppXor2>((u32)sum);
+    const float d = bm_half_to_f32(b.tail.w >> 16);
+    acc0 = __fadd_rn(acc0, __fmul_rn(__fmul_rn(act.dcol, d), (float)sum));
+}
+
 // ---- IQ4_XS (crates/qdot/src/lib.rs:11033-11180): lane q reads sub-blocks 2q and 2q + 1 whole (32 consecutive code
 // bytes) and their 64 activation codes, turns the nibbles into levels with byte permutes of the sixteen-entry table,
 // and forms its share of the CPU path's eight i32 lanes: lane l of those sums, scale by scale, the values 4l .. 4l + 3
@@ -737,6 +817,7 @@ __device__ __forceinline__ void bm_dot_iq4xs(const Blk<BM_IQ4XS> &b, const Act<B
 template <int WT>
 __device__ __forceinline__ float bm_quad_finish(float acc0, float acc1) {
     // lane ^ 2 holds acc_{l+4} (Q4_K, Q5_K, Q6_K: the other half h; IQ2_XXS, IQ4_XS: lane q + 2 owns l + 4)
+    if (WT == BM_Q3K) return acc0; // one accumulator a row, the same in the four lanes
     const float x = acc0 + bm_quad_xor2(acc0), y = acc1 + bm_quad_xor2(acc1);
     if (WT == BM_Q6K) {
         // lane c holds t_c and t_{c+2}
@@ -751,6 +832,10 @@ __device__ __forceinline__ float bm_quad_finish(float acc0, float acc1) {
 // Uniform front over the types.
 template <int WT>
 __device__ __forceinline__ Blk<WT> bm_load_blk(const uint8_t *wrow, int i, int q);
+template <>
+__device__ __forceinline__ Blk<BM_Q3K> bm_load_blk<BM_Q3K>(const uint8_t *wrow, int i, int q) {
+    return bm_load_q3k(wrow, i, q);
+}
 template <>
 __device__ __forceinline__ Blk<BM_Q4K> bm_load_blk<BM_Q4K>(const uint8_t *wrow, int i, int q) {
     return bm_load_q4k(wrow, i, q & 1, q >> 1);
@@ -788,6 +873,8 @@ __device__ __forceinline__ Act<WT> bm_load_act(const ActView &av, int i, int q) 
         return bm_act_q6k(av, i, q & 1, q >> 1);
     else if constexpr (WT == BM_IQ4XS)
         return bm_act_iq4xs(av, i, q);
+    else if constexpr (WT == BM_Q3K)
+        return bm_act_q3k(av, i, q);
     else if constexpr (WT == BM_IQ3XXS) {
         Act<BM_IQ3XXS> a;
         static_cast<Act<BM_IQ2XXS> &>(a) = bm_act_iq2xxs(av, i, q);
@@ -807,6 +894,8 @@ __device__ __forceinline__ void bm_dot_blk(const Blk<WT> &b, const Act<WT> &a, i
         bm_dot_q6k(b, a, i, q & 1, q >> 1, acc0, acc1, tap);
     else if constexpr (WT == BM_IQ4XS)
         bm_dot_iq4xs(b, a, i, q, acc0, acc1, tap);
+    else if constexpr (WT == BM_Q3K)
+        bm_dot_q3k(b, a, i, q, acc0, tap);
     else if constexpr (WT == BM_IQ3XXS)
         bm_dot_iq3xxs(b, a, i, q, tb, acc0, acc1, tap);
     else
@@ -815,7 +904,7 @@ __device__ __forceinline__ void bm_dot_blk(const Blk<WT> &b, const Act<WT> &a, i
 
 template <int WT>
 __host__ __device__ constexpr int bm_block_bytes() {
-    return WT == BM_Q4K ? BM_Q4K_BLOCK : WT == BM_Q5K ? BM_Q5K_BLOCK : WT == BM_Q6K ? BM_Q6K_BLOCK : WT == BM_IQ4XS ? BM_IQ4XS_BLOCK : WT == BM_IQ3XXS ? BM_IQ3XXS_BLOCK : BM_IQ2XXS_BLOCK;
+    return WT == BM_Q3K ? BM_Q3K_BLOCK : WT == BM_Q4K ? BM_Q4K_BLOCK : WT == BM_Q5K ? BM_Q5K_BLOCK : WT == BM_Q6K ? BM_Q6K_BLOCK : WT == BM_IQ4XS ? BM_IQ4XS_BLOCK : WT == BM_IQ3XXS ? BM_IQ3XXS_BLOCK : BM_IQ2XXS_BLOCK;
 }
 
 // ---- SwiGLU: crates/qdot/src/lib.rs:3741-3773 (expf) and :11467-11478 (divide, then multiply).

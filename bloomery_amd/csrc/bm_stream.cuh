@@ -425,6 +425,10 @@ constexpr int kRingQ4K = 4, kRingQ5K = 4, kRingQ6K = 3;
     }
 #define BM_DISPATCH(wtype, nb)                                                                                         \
     switch (wtype) {                                                                                                   \
+    case BM_Q3K:                                                                                                       \
+        if ((nb) % 2 == 0) BM_VARIANT(BM_Q3K, 2, 0)                                                                    \
+        else BM_VARIANT(BM_Q3K, 1, 0)                                                                                  \
+        break;                                                                                                         \
     case BM_Q4K:                                                                                                       \
         if ((nb) == 8) BM_VARIANT(BM_Q4K, kRingQ4K, 8)                                                                 \
         else if ((nb) % 2 == 0) BM_VARIANT(BM_Q4K, 2, 0)                                                               \

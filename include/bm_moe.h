@@ -1,7 +1,7 @@
 /* bm_moe.h - C ABI of libbm_moe_hip.so: quantized MoE expert matmul on MI355X (gfx950).
  *
- * Q4_K / Q5_K / Q6_K / IQ2_XXS / IQ3_XXS / IQ4_XS GGUF weight blocks dotted with Q8-quantized activations (Q8_2_X4 for the K-quants,
- * Q8_K for the IQ types), in the arithmetic of the reference's CPU path crates/qdot: activation bytes and per-block
+ * Q3_K / Q4_K / Q5_K / Q6_K / IQ2_XXS / IQ3_XXS / IQ4_XS GGUF weight blocks dotted with Q8-quantized activations (Q8_2_X4 for Q4_K, Q5_K and
+ * Q6_K, Q8_K for Q3_K and the IQ types), in the arithmetic of the reference's CPU path crates/qdot: activation bytes and per-block
  * integer sums are bit-exact with it, and the decode kernels keep its fp32 operation order.
  *
  * The entry points stand where the reference's crates/gpu launchers stand (each declaration cites the one it
@@ -25,6 +25,7 @@ extern "C" {
 #endif
 
 /* Weight types, numbered as ggml numbers them (crates/gguf/src/qtype.rs:94,98,105). */
+#define BM_TYPE_Q3_K 11    /* 110 B / 256 values; activations Q8_K */
 #define BM_TYPE_Q4_K 12    /* 144 B / 256 values; activations Q8_2_X4 */
 #define BM_TYPE_Q5_K 13    /* 176 B / 256 values; activations Q8_2_X4 */
 #define BM_TYPE_Q6_K 14    /* 210 B / 256 values; activations Q8_2_X4 */
@@ -308,7 +309,7 @@ int bm_route_softmax(bm_ctx *ctx, const float *logits_dev, int n_tokens, int n_e
 typedef struct bm_gguf bm_gguf;
 typedef struct bm_gguf_tensor {
     const char *name;  /* owned by the bm_gguf */
-    int type;          /* the ggml type id as the file states it (BM_TYPE_Q4_K = 12, BM_TYPE_Q5_K = 13, BM_TYPE_Q6_K = 14, BM_TYPE_IQ2_XXS = 16, BM_TYPE_IQ3_XXS = 18, BM_TYPE_IQ4_XS = 23, 0 = F32 ...) */
+    int type;          /* the ggml type id as the file states it (BM_TYPE_Q3_K = 11, BM_TYPE_Q4_K = 12, BM_TYPE_Q5_K = 13, BM_TYPE_Q6_K = 14, BM_TYPE_IQ2_XXS = 16, BM_TYPE_IQ3_XXS = 18, BM_TYPE_IQ4_XS = 23, 0 = F32 ...) */
     int n_dims;        /* 1 .. 4 */
     uint64_t dims[4];  /* ggml ne[] order: dims[0] is the contiguous axis; unused dims are 1 */
     uint64_t offset;   /* from the file's data section */
@@ -331,7 +332,7 @@ const char *bm_gguf_get_str(const bm_gguf *g, const char *key);
 /* The tensor `name` of the file as a weight stack on the device: a matrix {k, rows} or an expert stack
  * {k, rows_per_expert, n_experts} (crates/model/src/moe.rs:330 expert_view: expert e's matrix is the e-th equal part),
  * rows back to back as bm_weights_create takes them. The tensor's type must be one this library computes in
- * (BM_TYPE_Q4_K, BM_TYPE_Q5_K, BM_TYPE_Q6_K, BM_TYPE_IQ2_XXS, BM_TYPE_IQ3_XXS, BM_TYPE_IQ4_XS); rows_per_expert and n_experts (either may be NULL) receive dims[1] and dims[2]. */
+ * (BM_TYPE_Q3_K, BM_TYPE_Q4_K, BM_TYPE_Q5_K, BM_TYPE_Q6_K, BM_TYPE_IQ2_XXS, BM_TYPE_IQ3_XXS, BM_TYPE_IQ4_XS); rows_per_expert and n_experts (either may be NULL) receive dims[1] and dims[2]. */
 int bm_weights_from_gguf(bm_ctx *ctx, const bm_gguf *g, const char *name, bm_weights **out, int *rows_per_expert, int *n_experts);
 
 /* ------------------------------------------------------------------------------------------- verification */
@@ -341,6 +342,7 @@ int bm_weights_from_gguf(bm_ctx *ctx, const bm_gguf *g, const char *name, bm_wei
  *   Q4_K, Q5_K: per super-block 8 sums A[s] = sum q * a over sub-block s (q the 4- or 5-bit code), then the 8
  *            activation isums (16 words);
  *   Q6_K:    per super-block 16 sums S[g] = sum (q6 - 32) * a over 16-value group g (16 words);
+ *   Q3_K:    per super-block 16 sums S[g] = sum (q3 - 4) * a over 16-value group g (16 words);
  *   IQ2_XXS, IQ3_XXS: per super-block 8 sums I[b] = sum (+-grid) * a over sub-block b, then the 8 scales 2s + 1
  *            (16 words);
  *   IQ4_XS:  per super-block 8 sums I[b] = sum level * a over sub-block b, then the CPU path's 8 i32 lanes

@@ -405,6 +405,62 @@ static void dot_iq2xxs_tile(const uint8_t *wrow, const uint8_t *const *acols, in
     for (int c = 0; c < C; c++) out[c] = hsum_float_8(accd[c]);
 }
 
+// --------------------------------------------------------------------------------------------------- Q3_K tile
+
+static inline int hsum_i32_8(__m256i v) {
+    __m128i s = _mm_add_epi32(_mm256_castsi256_si128(v), _mm256_extracti128_si256(v, 1));
+    s = _mm_add_epi32(s, _mm_shuffle_epi32(s, 0x4e));
+    s = _mm_add_epi32(s, _mm_shuffle_epi32(s, 0xb1));
+    return _mm_cvtsi128_si32(s);
+}
+
+// One Q3_K row against C <= 8 columns, each column by the one-column kernel's steps (crates/qdot/src/lib.rs:2036-2157,
+// field_dot :1997-2030): a field's two low bits on maddubs' unsigned side, the 4 of a clear high bit likewise and
+// subtracted, the pairs scaled per 16 values in madd; one integer a super-block, then acc += (dcol * d) * sum, each
+// operation rounded on its own.
+static void dot_q3k_tile(const uint8_t *wrow, const uint8_t *const *acols, int C, int nb, float *out) {
+    const __m256i m3 = _mm256_set1_epi8(3), mone = _mm256_set1_epi8(1);
+    float acc[8] = {0};
+    for (int i = 0; i < nb; i++) {
+        const uint8_t *blk = wrow + (size_t)i * ORA_Q3K_BLOCK;
+        __m256i hbits = _mm256_loadu_si256((const __m256i *)blk);
+        uint32_t a0 = ora_rd32(blk + 96), a1 = ora_rd32(blk + 100), a2 = ora_rd32(blk + 104);
+        uint32_t w[4] = {(a0 & 0x0f0f0f0fu) | ((a2 & 0x03030303u) << 4), (a1 & 0x0f0f0f0fu) | (((a2 >> 2) & 0x03030303u) << 4),
+                         ((a0 >> 4) & 0x0f0f0f0fu) | (((a2 >> 4) & 0x03030303u) << 4),
+                         ((a1 >> 4) & 0x0f0f0f0fu) | (((a2 >> 6) & 0x03030303u) << 4)};
+        short sc[16];
+        for (int j = 0; j < 16; j++) sc[j] = (short)((int)((w[j / 4] >> (8 * (j % 4))) & 0xff) - 32);
+        uint16_t dh;
+        memcpy(&dh, blk + 108, 2);
+        float d = f16c_to_f32(dh);
+        __m256i sumi[8];
+        for (int c = 0; c < C; c++) sumi[c] = _mm256_setzero_si256();
+        for (int j = 0; j < 2; j++) {
+            __m256i q3bits = _mm256_loadu_si256((const __m256i *)(blk + 32 + 32 * j));
+            for (int f = 0; f < 4; f++) {
+                int bit = 4 * j + f, g = 8 * j + 2 * f;
+                __m256i q3l = _mm256_and_si256(_mm256_srl_epi16(q3bits, _mm_cvtsi32_si128(2 * f)), m3);
+                __m256i clear = _mm256_andnot_si256(hbits, _mm256_sll_epi16(mone, _mm_cvtsi32_si128(bit)));
+                __m256i q3h = _mm256_slli_epi16(_mm256_srl_epi16(clear, _mm_cvtsi32_si128(bit)), 2);
+                __m256i scv = _mm256_set_m128i(_mm_set1_epi16(sc[g + 1]), _mm_set1_epi16(sc[g]));
+                for (int c = 0; c < C; c++) {
+                    __m256i q8 = _mm256_loadu_si256((const __m256i *)(acols[c] + (size_t)i * ORA_Q8K_STRIDE + 8 + 128 * j + 32 * f));
+                    __m256i p = _mm256_sub_epi16(_mm256_maddubs_epi16(q3l, q8), _mm256_maddubs_epi16(q3h, q8));
+                    sumi[c] = _mm256_add_epi32(sumi[c], _mm256_madd_epi16(scv, p));
+                }
+            }
+        }
+        for (int c = 0; c < C; c++) {
+            float dcol;
+            memcpy(&dcol, acols[c] + (size_t)i * ORA_Q8K_STRIDE, 4);
+            float t = dcol * d;
+            t = t * (float)hsum_i32_8(sumi[c]);
+            acc[c] = acc[c] + t;
+        }
+    }
+    for (int c = 0; c < C; c++) out[c] = acc[c];
+}
+
 // ------------------------------------------------------------------------------------------------- IQ3_XXS tile
 
 // One IQ3_XXS row against C <= 8 columns (crates/qdot/src/lib.rs:7259-7345 per column, :7412 the tile): the IQ2_XXS
@@ -525,6 +581,9 @@ int ora_avx2_dot_row_cols(int wtype, const uint8_t *wrow, const uint8_t *const *
     if (k <= 0 || k % 256 != 0) return ORA_EUNALIGNED;
     int nb = k / 256;
     switch (wtype) {
+    case ORA_TYPE_Q3_K:
+        dot_q3k_tile(wrow, acols, cols, nb, out);
+        return 0;
     case ORA_TYPE_Q4_K:
         dot_q45k_tile(wrow, acols, cols, nb, 0, out);
         return 0;

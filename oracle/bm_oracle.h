@@ -1,5 +1,5 @@
 // TEST INFRASTRUCTURE ONLY. CPU oracle of the quantized MoE expert-matmul path: a plain C restatement of the
-// reference's crates/qdot (activation encoders, Q4_K / Q5_K / Q6_K / IQ2_XXS / IQ3_XXS / IQ4_XS row dots, SwiGLU), crates/gguf (block
+// reference's crates/qdot (activation encoders, Q3_K / Q4_K / Q5_K / Q6_K / IQ2_XXS / IQ3_XXS / IQ4_XS row dots, SwiGLU), crates/gguf (block
 // layouts, dequantizers, K-quant and IQ2_XXS weight quantizers) and the caller-side router/combine order of
 // crates/model/src/moe.rs. Each function cites the reference lines it follows. The shipped library never links
 // or calls this; the test suite, the smoke check and the benchmark's CPU-baseline leg do.
@@ -30,7 +30,7 @@ extern "C" {
 
 // Refusals (the reference panics or returns QdotError, crates/qdot/src/lib.rs:127-160).
 #define ORA_EUNALIGNED (-1) // k is not a whole number of 256-value super-blocks
-#define ORA_ETYPE (-2)      // weight type outside {Q4_K = 12, Q5_K = 13, Q6_K = 14, IQ2_XXS = 16, IQ3_XXS = 18, IQ4_XS = 23}
+#define ORA_ETYPE (-2)      // weight type outside {Q3_K = 11, Q4_K = 12, Q5_K = 13, Q6_K = 14, IQ2_XXS = 16, IQ3_XXS = 18, IQ4_XS = 23}
 #define ORA_ESHORTROW (-3)
 #define ORA_ESHORTCOL (-4)
 #define ORA_ENONFINITE (-5) // an activation value that is not finite
@@ -47,6 +47,7 @@ int ora_quantize_col(int wtype, const float *x, int k, uint8_t *out);
 float ora_dot_q4k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb);
 float ora_dot_q5k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb);
 float ora_dot_q6k_q82x4(const uint8_t *wrow, const uint8_t *acol, int nb);
+float ora_dot_q3k_q8k(const uint8_t *wrow, const uint8_t *acol, int nb);
 float ora_dot_iq2xxs_q8k(const uint8_t *wrow, const uint8_t *acol, int nb);
 float ora_dot_iq3xxs_q8k(const uint8_t *wrow, const uint8_t *acol, int nb);
 float ora_dot_iq4xs_q8k(const uint8_t *wrow, const uint8_t *acol, int nb);
@@ -54,6 +55,7 @@ int ora_dot_row(int wtype, const uint8_t *wrow, size_t wrow_len, const uint8_t *
                 float *out);
 int ora_gemv(int wtype, const uint8_t *w, int rows, int k, const uint8_t *act, int m, float *y);
 
+void ora_q3k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_t *s_out);
 void ora_q4k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_t *a_out, int32_t *isum_out);
 void ora_q5k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_t *a_out, int32_t *isum_out);
 void ora_q6k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int fold, int32_t *s_out);

@@ -11,9 +11,9 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libbm_oracle.so")
 
-Q4_K, Q5_K, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_XS = 12, 13, 14, 16, 18, 23
-BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ2_XXS: 66, IQ3_XXS: 98, IQ4_XS: 136}
-Q8K_TYPES = (IQ2_XXS, IQ3_XXS, IQ4_XS)  # the types whose activation column is ik's Q8_K; the others take Q8_2_X4
+Q3_K, Q4_K, Q5_K, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_XS = 11, 12, 13, 14, 16, 18, 23
+BLOCK_BYTES = {Q3_K: 110, Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ2_XXS: 66, IQ3_XXS: 98, IQ4_XS: 136}
+Q8K_TYPES = (Q3_K, IQ2_XXS, IQ3_XXS, IQ4_XS)  # the types whose activation column is ik's Q8_K; the others take Q8_2_X4
 
 EUNALIGNED, ETYPE, ESHORTROW, ESHORTCOL, ENONFINITE, ESHAPE, ESTATUS = -1, -2, -3, -4, -5, -6, -7
 
@@ -45,6 +45,7 @@ def _load():
         "ora_avx2_dot_row": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
         "ora_avx2_dot_row_cols": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
         "ora_avx2_supported": (C.c_int, []),
+        "ora_q3k_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
         "ora_q4k_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
         "ora_q5k_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
         "ora_q6k_block_sums": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
@@ -173,6 +174,14 @@ def q6k_block_sums(wrow, acol, k, fold=False):
     nb = k // 256
     s = np.empty(nb * 16, np.int32)
     lib.ora_q6k_block_sums(_p(_u8(wrow)), _p(_u8(acol)), nb, int(fold), _p(s))
+    return s
+
+
+def q3k_block_sums(wrow, acol, k):
+    """Per 16-value group the sum of (code - 4) * activation."""
+    nb = k // 256
+    s = np.empty(nb * 16, np.int32)
+    lib.ora_q3k_block_sums(_p(_u8(wrow)), _p(_u8(acol)), nb, _p(s))
     return s
 
 

@@ -11,6 +11,7 @@
 #include <stdint.h>
 #include <string.h>
 
+#define ORA_Q3K_BLOCK 110    // crates/gguf/src/quant.rs:671-673: hmask[32], qs[64] @32, scales[12] @96, d @108
 #define ORA_Q4K_BLOCK 144    // crates/qdot/src/lib.rs:3864
 #define ORA_Q5K_BLOCK 176    // crates/qdot/src/lib.rs:4880: d, dmin, scales[12], qh[32] @16, qs[128] @48
 #define ORA_Q6K_BLOCK 210    // crates/qdot/src/lib.rs:4452
@@ -21,6 +22,7 @@
 #define ORA_Q82X4_STRIDE 144 // crates/qdot/src/lib.rs:110
 
 // Weight types, numbered as ggml numbers them (crates/gguf/src/qtype.rs:94,98,105).
+#define ORA_TYPE_Q3_K 11
 #define ORA_TYPE_Q4_K 12
 #define ORA_TYPE_Q5_K 13
 #define ORA_TYPE_Q6_K 14
@@ -30,7 +32,7 @@
 
 // The types whose activation column is ik's Q8_K (crates/gguf/src/qtype.rs host_act); the others here take Q8_2_X4.
 static inline int ora_takes_q8k(int wtype) {
-    return wtype == ORA_TYPE_IQ2_XXS || wtype == ORA_TYPE_IQ3_XXS || wtype == ORA_TYPE_IQ4_XS;
+    return wtype == ORA_TYPE_Q3_K || wtype == ORA_TYPE_IQ2_XXS || wtype == ORA_TYPE_IQ3_XXS || wtype == ORA_TYPE_IQ4_XS;
 }
 
 static inline uint32_t ora_f32_bits(float f) {

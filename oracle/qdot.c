@@ -77,6 +77,7 @@ int ora_col_bytes(int wtype, int k) {
     case ORA_TYPE_Q5_K:
     case ORA_TYPE_Q6_K:
         return k / 128 * ORA_Q82X4_STRIDE;
+    case ORA_TYPE_Q3_K:
     case ORA_TYPE_IQ2_XXS:
     case ORA_TYPE_IQ3_XXS:
     case ORA_TYPE_IQ4_XS:
@@ -89,6 +90,8 @@ int ora_col_bytes(int wtype, int k) {
 int ora_row_bytes(int wtype, int k) {
     if (k <= 0 || k % 256 != 0) return ORA_EUNALIGNED; // crates/qdot/src/lib.rs:1727-1762
     switch (wtype) {
+    case ORA_TYPE_Q3_K:
+        return k / 256 * ORA_Q3K_BLOCK;
     case ORA_TYPE_Q4_K:
         return k / 256 * ORA_Q4K_BLOCK;
     case ORA_TYPE_Q5_K:
@@ -112,12 +115,66 @@ int ora_quantize_col(int wtype, const float *x, int k, uint8_t *out) {
     case ORA_TYPE_Q5_K:
     case ORA_TYPE_Q6_K:
         return ora_quantize_q82x4(x, k, out);
+    case ORA_TYPE_Q3_K:
     case ORA_TYPE_IQ2_XXS:
     case ORA_TYPE_IQ3_XXS:
     case ORA_TYPE_IQ4_XS:
         return ora_quantize_q8k(x, k, out);
     default:
         return ORA_ETYPE;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------ Q3_K dot
+
+// A super-block's sixteen scales as stored, six bits each, s + 32 (crates/qdot/src/lib.rs:2162-2174).
+static void q3k_scales6(const uint8_t *blk, uint8_t sc[16]) {
+    uint32_t a0 = ora_rd32(blk + 96), a1 = ora_rd32(blk + 100), a2 = ora_rd32(blk + 104);
+    uint32_t w[4] = {(a0 & 0x0f0f0f0fu) | ((a2 & 0x03030303u) << 4), (a1 & 0x0f0f0f0fu) | (((a2 >> 2) & 0x03030303u) << 4),
+                     ((a0 >> 4) & 0x0f0f0f0fu) | (((a2 >> 4) & 0x03030303u) << 4),
+                     ((a1 >> 4) & 0x0f0f0f0fu) | (((a2 >> 6) & 0x03030303u) << 4)};
+    for (int j = 0; j < 16; j++) sc[j] = (uint8_t)(w[j / 4] >> (8 * (j % 4)));
+}
+
+// Value n of a super-block less its offset: u - 4 with u = two low bits of qs | the hmask bit << 2
+// (crates/qdot/src/lib.rs:2176-2185, crates/gguf/src/quant.rs:671-727).
+static inline int q3k_value(const uint8_t *blk, int n) {
+    int half = n / 128, field = (n / 32) % 4, cell = n % 32;
+    int low = (blk[32 + 32 * half + cell] >> (2 * field)) & 3;
+    int high = (blk[cell] >> (4 * half + field)) & 1;
+    return (low | (high << 2)) - 4;
+}
+
+// Q3_K x Q8_K (crates/qdot/src/lib.rs:2223-2245): one exact integer a super-block, one f32 accumulator a row, a
+// product and a sum each rounded on its own.
+float ora_dot_q3k_q8k(const uint8_t *wrow, const uint8_t *acol, int nb) {
+    float acc = 0.0f;
+    for (int i = 0; i < nb; i++) {
+        const uint8_t *blk = wrow + (size_t)i * ORA_Q3K_BLOCK;
+        const uint8_t *col = acol + (size_t)i * ORA_Q8K_STRIDE;
+        uint8_t sc[16];
+        q3k_scales6(blk, sc);
+        float d = ora_half_to_f32(ora_rd16(blk + 108));
+        float dcol = ora_bits_f32(ora_rd32(col));
+        int32_t sumi = 0;
+        for (int n = 0; n < 256; n++) sumi += ((int32_t)sc[n / 16] - 32) * q3k_value(blk, n) * (int32_t)(int8_t)col[8 + n];
+        float t = dcol * d;
+        t = t * (float)sumi;
+        acc = acc + t;
+    }
+    return acc;
+}
+
+// Per super-block the sixteen sums S[g] = sum over 16-value group g of (u - 4) * a.
+void ora_q3k_block_sums(const uint8_t *wrow, const uint8_t *acol, int nb, int32_t *s_out) {
+    for (int i = 0; i < nb; i++) {
+        const uint8_t *blk = wrow + (size_t)i * ORA_Q3K_BLOCK;
+        const uint8_t *col = acol + (size_t)i * ORA_Q8K_STRIDE;
+        for (int g = 0; g < 16; g++) {
+            int32_t sum = 0;
+            for (int n = 16 * g; n < 16 * g + 16; n++) sum += q3k_value(blk, n) * (int32_t)(int8_t)col[8 + n];
+            s_out[16 * i + g] = sum;
+        }
     }
 }
 
@@ -526,6 +583,9 @@ int ora_dot_row(int wtype, const uint8_t *wrow, size_t wrow_len, const uint8_t *
     if (acol_len < (size_t)need_a) return ORA_ESHORTCOL;
     int nb = k / 256;
     switch (wtype) {
+    case ORA_TYPE_Q3_K:
+        *out = ora_dot_q3k_q8k(wrow, acol, nb);
+        return 0;
     case ORA_TYPE_Q4_K:
         *out = ora_dot_q4k_q82x4(wrow, acol, nb);
         return 0;
@@ -569,7 +629,13 @@ int ora_dequant_row(int wtype, const uint8_t *src, int k, float *dst) {
     if (k <= 0 || k % 256 != 0) return ORA_EUNALIGNED;
     for (int i = 0; i < k / 256; i++) {
         float *out = dst + 256 * i;
-        if (wtype == ORA_TYPE_Q4_K) { // crates/gguf/src/quant.rs:738-767
+        if (wtype == ORA_TYPE_Q3_K) { // crates/gguf/src/quant.rs:679-727
+            const uint8_t *blk = src + (size_t)i * ORA_Q3K_BLOCK;
+            float d = ora_half_to_f32(ora_rd16(blk + 108));
+            uint8_t sc[16];
+            q3k_scales6(blk, sc);
+            for (int n = 0; n < 256; n++) out[n] = (d * (float)((int)sc[n / 16] - 32)) * (float)q3k_value(blk, n);
+        } else if (wtype == ORA_TYPE_Q4_K) { // crates/gguf/src/quant.rs:738-767
             const uint8_t *blk = src + (size_t)i * ORA_Q4K_BLOCK;
             float d = ora_half_to_f32(ora_rd16(blk)), dmin = ora_half_to_f32(ora_rd16(blk + 2));
             uint8_t sc[8], mn[8];

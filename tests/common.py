@@ -92,3 +92,31 @@ def iq4xs_rows(x):
         out[i, 2], out[i, 3] = sh & 0xFF, sh >> 8
         out[i, 8:136] = (codes[:, :16] | (codes[:, 16:] << 4)).astype(np.uint8).reshape(-1)
     return out.reshape(-1)
+
+
+def q3k_rows(x):
+    """Q3_K blocks (110 bytes a 256 values, crates/gguf/src/quant.rs:671-678) standing for the f32 rows x: a test-side
+    generator, nearest of the eight levels -4 .. 3 under one six-bit scale a 16 values. (The reference quantizes Q3_K
+    with ggml's search; the tests only need blocks whose values look like weights, every byte pattern being legal.)"""
+    x = np.asarray(x, np.float32).reshape(-1, 256)
+    out = np.zeros((x.shape[0], 110), np.uint8)
+    for i, blk in enumerate(x):
+        grp = blk.reshape(16, 16).astype(np.float64)
+        amax = np.abs(grp).max(axis=1)
+        d = np.float16(amax.max() / (4.0 * 31.0))
+        df = float(d)
+        sc = np.zeros(16, np.int64) if df == 0.0 else np.clip(np.rint(amax / (4.0 * df)), 1, 31).astype(np.int64)
+        u = np.full(256, 4, np.int64)
+        if df != 0.0:
+            u = (np.clip(np.rint(grp / (df * sc[:, None])), -4, 3).astype(np.int64) + 4).reshape(-1)
+        for n in range(256):
+            half, field, cell = n // 128, (n // 32) % 4, n % 32
+            out[i, 32 + 32 * half + cell] |= int(u[n] & 3) << (2 * field)
+            out[i, cell] |= int(u[n] >> 2) << (4 * half + field)
+        s6 = sc + 32
+        for k in range(4):  # crates/qdot/src/lib.rs:2187-2198
+            out[i, 96 + k] = int(s6[k] & 15) | (int(s6[8 + k] & 15) << 4)
+            out[i, 100 + k] = int(s6[4 + k] & 15) | (int(s6[12 + k] & 15) << 4)
+            out[i, 104 + k] = int(s6[k] >> 4) | (int(s6[4 + k] >> 4) << 2) | (int(s6[8 + k] >> 4) << 4) | (int(s6[12 + k] >> 4) << 6)
+        out[i, 108:110] = np.array([d], np.float16).view(np.uint8)
+    return out.reshape(-1)

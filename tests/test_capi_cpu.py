@@ -36,13 +36,13 @@ def test_size_rules_match_the_block_layouts():
     for k in (0, -256, 100, 257):
         assert bm.row_bytes(bm.Q4_K, k) == bm.ESHAPE and bm.col_bytes(bm.Q6_K, k) == bm.ESHAPE
     assert bm.row_bytes(bm.Q5_K, 2304) == 176 * 9 and bm.col_bytes(bm.Q5_K, 2304) == 144 * 18
-    assert bm.row_bytes(3, 256) == bm.ETYPE and bm.col_bytes(11, 256) == bm.ETYPE
+    assert bm.row_bytes(3, 256) == bm.ETYPE and bm.col_bytes(10, 256) == bm.ETYPE
     assert bm.load_library().bm_version() >= 100
 
 
 def test_oracle_and_library_agree_on_sizes():
     import ora
-    for wtype in (bm.Q4_K, bm.Q5_K, bm.Q6_K, bm.IQ2_XXS):
+    for wtype in (bm.Q3_K, bm.Q4_K, bm.Q5_K, bm.Q6_K, bm.IQ2_XXS, bm.IQ3_XXS, bm.IQ4_XS):
         for k in (256, 768, 2048, 7168):
             assert bm.row_bytes(wtype, k) == ora.row_bytes(wtype, k)
             assert bm.col_bytes(wtype, k) == ora.col_bytes(wtype, k)

@@ -10,12 +10,12 @@ import pytest
 
 import bloomery_amd as bm
 import ora
-from common import Lcg, iq4xs_rows, max_abs_normalised, normal_f32
+from common import Lcg, iq4xs_rows, max_abs_normalised, normal_f32, q3k_rows
 
 pytestmark = pytest.mark.gpu
 
-TYPES = (bm.Q4_K, bm.Q5_K, bm.Q6_K, bm.IQ2_XXS, bm.IQ3_XXS, bm.IQ4_XS)
-Q8K_TYPES = (bm.IQ2_XXS, bm.IQ3_XXS, bm.IQ4_XS)  # their activation columns are Q8_K, the others' Q8_2_X4
+TYPES = (bm.Q3_K, bm.Q4_K, bm.Q5_K, bm.Q6_K, bm.IQ2_XXS, bm.IQ3_XXS, bm.IQ4_XS)
+Q8K_TYPES = (bm.Q3_K, bm.IQ2_XXS, bm.IQ3_XXS, bm.IQ4_XS)  # their activation columns are Q8_K, the others' Q8_2_X4
 TIES = np.array([0.5, 1.5, 2.5, 3.5, -0.5, -1.5, -2.5, -3.5, 0.25, 7.5, -7.5, 63.5, -63.5, 120.5, -120.5,
                  0.0, -0.0, 127.0, -127.0], np.float32)
 
@@ -41,7 +41,7 @@ def random_blocks(wtype, rows, k, rng):
     bb = ora.BLOCK_BYTES[wtype]
     nb = k // 256
     w = rng.integers(0, 256, rows * nb * bb, dtype=np.uint8).reshape(rows * nb, bb)
-    off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ3_XXS: 0, ora.IQ4_XS: 0}[wtype]
+    off = {ora.Q3_K: 108, ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ3_XXS: 0, ora.IQ4_XS: 0}[wtype]
     d = rng.uniform(-0.05, 0.05, rows * nb).astype(np.float16).view(np.uint16)
     w[:, off] = d & 0xFF
     w[:, off + 1] = d >> 8
@@ -59,6 +59,8 @@ def quantized(wtype, rows, k, seed):
         return iq4xs_rows(x)
     if wtype == bm.IQ3_XXS:  # nor an IQ3_XXS one: raw random blocks, every one of which is legal
         return random_blocks(wtype, rows, k, rng)
+    if wtype == bm.Q3_K:  # a test-side generator: the oracle restates the quantizers of the benchmark's types only
+        return q3k_rows(x)
     return ora.quantize_rows(wtype, x, rows, k, n_threads=8)
 
 
@@ -185,6 +187,8 @@ def test_block_sums_are_the_cpu_paths_integers(gpu, wtype):
                 if wtype in (bm.Q4_K, bm.Q5_K):
                     a, isum = ora.q4k_block_sums(wrow, acol, k, q5=wtype == bm.Q5_K)
                     assert np.array_equal(got[:, :8].reshape(-1), a) and np.array_equal(got[:, 8:].reshape(-1), isum)
+                elif wtype == bm.Q3_K:
+                    assert np.array_equal(got.reshape(-1), ora.q3k_block_sums(wrow, acol, k))
                 elif wtype == bm.Q6_K:
                     assert np.array_equal(got.reshape(-1), ora.q6k_block_sums(wrow, acol, k))
                     assert np.array_equal(got.reshape(-1), ora.q6k_block_sums(wrow, acol, k, fold=True))
@@ -204,7 +208,8 @@ def test_block_sums_are_the_cpu_paths_integers(gpu, wtype):
 @pytest.mark.parametrize("wtype,rows,k", ((bm.Q4_K, 768, 2048), (bm.Q6_K, 2048, 768), (bm.IQ2_XXS, 300, 2048),
                                           (bm.Q4_K, 70, 256), (bm.Q6_K, 65, 1792), (bm.IQ2_XXS, 33, 7168),
                                           (bm.Q5_K, 96, 2304), (bm.Q5_K, 67, 1280), (bm.IQ4_XS, 200, 2560),
-                                          (bm.IQ4_XS, 66, 768), (bm.IQ3_XXS, 130, 2048), (bm.IQ3_XXS, 40, 1280)))
+                                          (bm.IQ4_XS, 66, 768), (bm.IQ3_XXS, 130, 2048), (bm.IQ3_XXS, 40, 1280),
+                                          (bm.Q3_K, 150, 2048), (bm.Q3_K, 70, 768)))
 def test_gemv_matches_dot_row(gpu, wtype, rows, k):
     # config 1 is the first case: 768 x 2048 Q4_K against one 2048-vector
     rng = np.random.default_rng(30 + rows)
@@ -233,7 +238,7 @@ def test_extreme_blocks(gpu):
             w = np.full(2 * bb, fill, np.uint8)
             for i in range(2):
                 h = np.array([dval, abs(dval)], np.float16).view(np.uint8)
-                off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ3_XXS: 0, ora.IQ4_XS: 0}[wtype]
+                off = {ora.Q3_K: 108, ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ3_XXS: 0, ora.IQ4_XS: 0}[wtype]
                 w[i * bb + off:i * bb + off + 2] = h[0:2]
                 if wtype in (ora.Q4_K, ora.Q5_K):
                     w[i * bb + 2:i * bb + 4] = h[2:4]
@@ -347,6 +352,8 @@ def test_qwen3_shaped_layer_one_token(gpu, fused):
     ((bm.IQ4_XS, bm.IQ4_XS, bm.IQ4_XS), 768, 512, 4, 3, 2),
     ((bm.IQ4_XS, bm.IQ4_XS, bm.Q5_K), 512, 256, 3, 2, 3),       # Q8_K columns into gate / up, Q8_2_X4 into down
     ((bm.IQ3_XXS, bm.IQ3_XXS, bm.IQ3_XXS), 768, 512, 4, 3, 2),
+    ((bm.Q3_K, bm.Q3_K, bm.Q3_K), 768, 512, 4, 3, 2),
+    ((bm.Q3_K, bm.Q3_K, bm.Q5_K), 512, 256, 3, 2, 3),
     ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ3_XXS), 512, 768, 3, 2, 3),
     ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ2_XXS), 1024, 512, 6, 4, 3),
     ((bm.IQ2_XXS, bm.IQ2_XXS, bm.Q6_K), 768, 256, 4, 2, 4),
@@ -605,6 +612,7 @@ def run_grouped(gpu, L, x, ids, wts, top_k, fused_quant):
     ((bm.Q5_K, bm.Q5_K, bm.Q5_K), 768, 512, 3, 9, 2),
     ((bm.IQ4_XS, bm.IQ4_XS, bm.IQ4_XS), 768, 512, 3, 9, 2),
     ((bm.IQ3_XXS, bm.IQ3_XXS, bm.IQ3_XXS), 768, 512, 3, 9, 2),
+    ((bm.Q3_K, bm.Q3_K, bm.Q3_K), 768, 512, 3, 9, 2),
     ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ2_XXS), 1024, 512, 5, 6, 3),
     ((bm.IQ2_XXS, bm.IQ2_XXS, bm.Q6_K), 768, 256, 4, 5, 4),
     # rows long enough that eight Q8_K columns pass the LDS mark where a tile launch goes as two, one for the tiles of
@@ -667,7 +675,7 @@ def test_slot_equals_one_expert_gemv_and_duplicate_ids(gpu):
     # gate_q4k_sel's first clauses (crates/gpu-gates/src/bin/gate_q4k_sel.rs:1-48)
     rng = np.random.default_rng(300)
     for wtype, k, rpe in ((bm.Q4_K, 768, 96), (bm.Q5_K, 1024, 72), (bm.Q6_K, 768, 2048 // 8), (bm.IQ2_XXS, 512, 80),
-                          (bm.IQ4_XS, 1280, 40), (bm.IQ3_XXS, 768, 48)):
+                          (bm.IQ4_XS, 1280, 40), (bm.IQ3_XXS, 768, 48), (bm.Q3_K, 512, 56)):
         n_experts, n_slots = 5, 7
         w = stack(wtype, n_experts * rpe, k, 301)
         sel = np.array([3, 0, 3, 4, 1, 3, 0], np.uint32)

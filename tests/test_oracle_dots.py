@@ -13,10 +13,10 @@ import numpy as np
 import pytest
 
 import ora
-from common import KVALUES_IQ4NL, iq4xs_rows, normal_f32
+from common import KVALUES_IQ4NL, iq4xs_rows, normal_f32, q3k_rows
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-TYPES = (ora.Q4_K, ora.Q5_K, ora.Q6_K, ora.IQ2_XXS, ora.IQ3_XXS, ora.IQ4_XS)
+TYPES = (ora.Q3_K, ora.Q4_K, ora.Q5_K, ora.Q6_K, ora.IQ2_XXS, ora.IQ3_XXS, ora.IQ4_XS)
 
 
 # ---------------------------------------------------------------- independent numpy decoders (written from the
@@ -52,6 +52,26 @@ def parse_grid3():
 
 
 GRID3 = parse_grid3()["oracle/iq_tables.h"]
+
+
+def q3k_decode(blk):
+    """block_q3_K (crates/gguf/src/quant.rs:671-678): 32 high-bit bytes, 64 bytes of two-bit fields, twelve scale bytes
+    (sixteen six-bit scales: four low bits in bytes 96..103, the two high bits in 104..107), d."""
+    d = f16(blk[108], blk[109])
+    sb = [int(v) for v in blk[96:108]]
+    sc = []
+    for j in range(16):
+        low = (sb[j % 8] >> (4 * (j // 8))) & 15
+        high = (sb[8 + j % 4] >> (2 * (j // 4))) & 3
+        sc.append((low | (high << 4)) - 32)
+    codes = np.zeros(256, np.int64)
+    for n in range(256):
+        half, field, cell = n // 128, (n // 32) % 4, n % 32
+        low = (int(blk[32 + 32 * half + cell]) >> (2 * field)) & 3
+        high = (int(blk[cell]) >> (4 * half + field)) & 1
+        codes[n] = low - (0 if high else 4)
+    vals = np.array([d * sc[n // 16] * codes[n] for n in range(256)], np.float64)
+    return codes, vals, (d, sc)
 
 
 def q4k_decode(blk):
@@ -151,7 +171,7 @@ def iq4xs_decode(blk):
     return codes, vals, (d, ls)
 
 
-DECODE = {ora.IQ3_XXS: iq3xxs_decode, ora.IQ4_XS: iq4xs_decode, ora.Q4_K: q4k_decode, ora.Q5_K: q5k_decode, ora.Q6_K: q6k_decode, ora.IQ2_XXS: iq2xxs_decode}
+DECODE = {ora.Q3_K: q3k_decode, ora.IQ3_XXS: iq3xxs_decode, ora.IQ4_XS: iq4xs_decode, ora.Q4_K: q4k_decode, ora.Q5_K: q5k_decode, ora.Q6_K: q6k_decode, ora.IQ2_XXS: iq2xxs_decode}
 
 
 def act_codes(wtype, col, k):
@@ -174,7 +194,7 @@ def random_blocks(wtype, nb, rng):
     w = rng.integers(0, 256, nb * bb, dtype=np.uint8)
     for i in range(nb):
         h = np.array([rng.uniform(-0.1, 0.1), rng.uniform(0.0, 0.1)], np.float16).view(np.uint8)
-        off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ3_XXS: 0, ora.IQ4_XS: 0}[wtype]
+        off = {ora.Q3_K: 108, ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ3_XXS: 0, ora.IQ4_XS: 0}[wtype]
         w[i * bb + off:i * bb + off + 2] = h[0:2]
         if wtype in (ora.Q4_K, ora.Q5_K):
             w[i * bb + 2:i * bb + 4] = h[2:4]
@@ -186,6 +206,8 @@ def quantized_rows(wtype, rows, k, seed):
     x = normal_f32(rng, (rows, k), 0.02)
     if wtype == ora.IQ4_XS:
         return iq4xs_rows(x), x
+    if wtype == ora.Q3_K:  # a test-side generator: the oracle restates the quantizers of the benchmark's types only
+        return q3k_rows(x), x
     if wtype == ora.IQ3_XXS:  # no quantizer of this type in the reference's gguf crate: random legal blocks
         return random_blocks(wtype, rows * (k // 256), rng), x
     return ora.quantize_rows(wtype, x, rows, k, n_threads=4), x
@@ -267,6 +289,8 @@ def test_block_sums_equal_brute_force(wtype):
             got_a, got_isum = ora.q4k_block_sums(w, col, k, q5=wtype == ora.Q5_K)
             assert list(got_a) == [int(prod[32 * s:32 * s + 32].sum()) for s in range(nb * 8)]
             assert list(got_isum) == [int(a[32 * s:32 * s + 32].sum()) for s in range(nb * 8)]
+        elif wtype == ora.Q3_K:
+            assert list(ora.q3k_block_sums(w, col, k)) == [int(prod[16 * g:16 * g + 16].sum()) for g in range(nb * 16)]
         elif wtype == ora.Q6_K:
             want = [int(prod[16 * g:16 * g + 16].sum()) for g in range(nb * 16)]
             assert list(ora.q6k_block_sums(w, col, k)) == want
@@ -355,7 +379,7 @@ def extreme_cases(wtype, rng):
         w = np.full(2 * bb, fill, np.uint8)
         for i in range(2):
             h = np.array([dval, abs(dval)], np.float16).view(np.uint8)
-            off = {ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ3_XXS: 0, ora.IQ4_XS: 0}[wtype]
+            off = {ora.Q3_K: 108, ora.Q4_K: 0, ora.Q5_K: 0, ora.Q6_K: 208, ora.IQ2_XXS: 0, ora.IQ3_XXS: 0, ora.IQ4_XS: 0}[wtype]
             w[i * bb + off:i * bb + off + 2] = h[0:2]
             if wtype in (ora.Q4_K, ora.Q5_K):
                 w[i * bb + 2:i * bb + 4] = h[2:4]

@@ -38,7 +38,7 @@ def log(*a):
 
 def make_layer(ora, seed, threads, gate_type=None, down_type=None):
     """The layer's expert stacks: fp32 N(0, 0.02) quantized by the repo's K-quant rules (Q4_K, Q5_K, Q6_K `_ref`);
-    IQ4_XS, for which the reference has no quantizer, as random legal blocks with small scales."""
+    the other types as random legal blocks with small scales."""
     rng = np.random.default_rng(seed)
     gate_type = ora.Q4_K if gate_type is None else gate_type
     down_type = ora.Q6_K if down_type is None else down_type
@@ -46,11 +46,16 @@ def make_layer(ora, seed, threads, gate_type=None, down_type=None):
     for wtype, rows, k in ((gate_type, N_EXPERTS * FF, HIDDEN), (gate_type, N_EXPERTS * FF, HIDDEN),
                            (down_type, N_EXPERTS * HIDDEN, FF)):
         rb = ora.row_bytes(wtype, k)
-        if wtype == ora.IQ4_XS:
+        raw = {ora.IQ4_XS: (136, 0, 2e-6, 8e-6),   # values d * (ls - 32) * level ~ 0.01
+               ora.Q3_K: (110, 108, 1e-4, 4e-4),   # d * (scale - 32) * (code - 4)
+               ora.IQ2_XXS: (66, 0, 1e-3, 4e-3),   # d * (0.5 + s) / 4 * magnitude
+               ora.IQ3_XXS: (98, 0, 2e-4, 8e-4)}   # d * (0.5 + s) / 2 * magnitude
+        if wtype in raw:  # types the oracle has no (fast) quantizer for: random legal blocks with small scales
+            bb, d_off, lo, hi = raw[wtype]
             nb = rows * (k // 256)
-            w = rng.integers(0, 256, nb * 136, dtype=np.uint8).reshape(nb, 136)
-            d = rng.uniform(2e-6, 8e-6, nb).astype(np.float16).view(np.uint16)  # values d * (ls - 32) * level ~ 0.01
-            w[:, 0], w[:, 1] = d & 0xFF, d >> 8
+            w = rng.integers(0, 256, nb * bb, dtype=np.uint8).reshape(nb, bb)
+            d = rng.uniform(lo, hi, nb).astype(np.float16).view(np.uint16)
+            w[:, d_off], w[:, d_off + 1] = d & 0xFF, d >> 8
             out.append(w.reshape(-1))
             continue
         q = np.empty(rows * rb, np.uint8)
@@ -423,7 +428,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
     ap.add_argument("--types", default="q4_k,q6_k",
-                    help="config 2 only: gate/up and down weight types (q4_k, q5_k, q6_k, iq4_xs); other than the default is "
+                    help="config 2 only: gate/up and down weight types (q3_k, q4_k, q5_k, q6_k, iq2_xxs, iq3_xxs, iq4_xs); other than the default is "
                          "a side measurement of that type, not the headline workload")
     ap.add_argument("--mode", choices=("two", "single", "chain"), default="two",
                     help="two: bm_moe_decode in two launches (quantizers folded in); single: bm_moe_decode in one "
@@ -438,17 +443,15 @@ def main():
     threads = min(os.cpu_count() or 1, 16)
     if args.config != 2:
         return {1: bench_gemv, 3: bench_grouped, 4: bench_prefill, 5: bench_dsv3}[args.config](args, bm, ora, threads)
-    names = {"q4_k": bm.Q4_K, "q5_k": bm.Q5_K, "q6_k": bm.Q6_K, "iq4_xs": bm.IQ4_XS}
+    names = {"q3_k": bm.Q3_K, "q4_k": bm.Q4_K, "q5_k": bm.Q5_K, "q6_k": bm.Q6_K, "iq2_xxs": bm.IQ2_XXS,
+             "iq3_xxs": bm.IQ3_XXS, "iq4_xs": bm.IQ4_XS}
     try:
         gate_t, down_t = (names[v] for v in args.types.lower().split(","))
     except (KeyError, ValueError):
         sys.exit(f"bench.py: --types takes two of {sorted(names)} separated by a comma, got {args.types!r}")
     label = {v: k.upper() for k, v in names.items()}
     gate_n, down_n = label[gate_t], label[down_t]
-    q8k = (bm.IQ2_XXS, bm.IQ4_XS)
-    if args.mode != "chain" and (gate_t in q8k or down_t in q8k or gate_t == bm.Q6_K):
-        log(f"[bench] {gate_n} gate/up with {down_n} down has no fused step: timing the chain of launches")
-        args.mode = "chain"
+    q8k = (bm.Q3_K, bm.IQ2_XXS, bm.IQ3_XXS, bm.IQ4_XS)
     if args.mode == "single" and (gate_t, down_t) != (bm.Q4_K, bm.Q6_K):
         sys.exit("bench.py: --mode single takes the default types")
     types3 = (gate_t, gate_t, down_t)
@@ -470,7 +473,7 @@ def main():
     act = gpu.act(gate_t, HIDDEN, 1)
     act_h = gpu.act(down_t, FF, TOP_K)
     fold_h = down_t not in q8k  # gate . up writes the down activation itself when that is a Q8_2_X4 column
-    h = None if fold_h else gpu.buffer(np.float32, TOP_K * FF)
+    h = None if fold_h else gpu.buffer(np.float32, TOP_K * FF)  # else f32 rows, quantized by the down launch
 
     single = args.mode == "single"
     kernels = {"single": ("step",), "two": ("gate_up_x", "down"),
@@ -482,10 +485,15 @@ def main():
         dg, du, dd = layers[i % len(layers)]
         if "gate_up_x" in which and "down" in which:
             gpu.enqueue_moe_decode(dg, du, dd, xd.ptr + 4 * t * HIDDEN, sel.ptr + 4 * t * TOP_K, wt.ptr + 4 * t * TOP_K,
-                                   None, TOP_K, 1, act_h, y.ptr + 4 * t * HIDDEN)
+                                   None, TOP_K, 1, act_h, y.ptr + 4 * t * HIDDEN, h=h)
             return
         if "gate_up_x" in which:
-            gpu.enqueue_gate_up_x(dg, du, xd.ptr + 4 * t * HIDDEN, sel.ptr + 4 * t * TOP_K, TOP_K, 1, FF, act_h)
+            gpu.enqueue_gate_up_x(dg, du, xd.ptr + 4 * t * HIDDEN, sel.ptr + 4 * t * TOP_K, TOP_K, 1, FF,
+                                  act_h if fold_h else None, h=h)
+        if "down" in which and not fold_h and args.mode == "two":
+            gpu.enqueue_down_combine_h(dd, h, act_h, sel.ptr + 4 * t * TOP_K, wt.ptr + 4 * t * TOP_K, None, TOP_K, 1, HIDDEN,
+                                       y.ptr + 4 * t * HIDDEN)
+            return
         if "step" in which:
             gpu.enqueue_moe_decode(dg, du, dd, xd.ptr + 4 * t * HIDDEN, sel.ptr + 4 * t * TOP_K, wt.ptr + 4 * t * TOP_K,
                                    None, TOP_K, 1, act_h, y.ptr + 4 * t * HIDDEN)

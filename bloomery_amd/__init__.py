@@ -63,6 +63,7 @@ SYMBOLS = {
     "bm_gemv_sel": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "bm_combine_tokens": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_down_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "bm_down_combine_h": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_moe_decode": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp]),
     "bm_set_spin_limit": (_i, [_vp, _u32]),
     "bm_set_decode_plan": (_i, [_vp, _i]),
@@ -460,16 +461,23 @@ class Gpu:
         self._check(self.lib.bm_down_combine(self.ctx, w.handle, act.handle, _ptr(sel), _ptr(wts), _ptr(resid),
                                              n_slots_per_token, m, rows_per_expert, _ptr(y)))
 
+    def enqueue_down_combine_h(self, w, h, act_h, sel, wts, resid, n_slots_per_token, m, rows_per_expert, y):
+        """bm_down_combine from the f32 rows of h, for a down stack on Q8_K columns (act_h may be None)."""
+        self._check(self.lib.bm_down_combine_h(self.ctx, w.handle, _ptr(h), act_h.handle if act_h is not None else None,
+                                               _ptr(sel), _ptr(wts), _ptr(resid), n_slots_per_token, m, rows_per_expert,
+                                               _ptr(y)))
+
     def enqueue_moe_decode(self, wg, wu, wd, x, sel, wts, resid, n_slots_per_token, m, act_h, y, act_x=None, h=None):
-        """The whole layer step in one launch (bm_moe_decode)."""
+        """The whole layer step with the quantizers folded in (bm_moe_decode): two launches, or one under
+        PLAN_ONE_LAUNCH. A down stack on Q8_K columns needs h (f32 scratch of m * n_slots_per_token * ff values)."""
         self._check(self.lib.bm_moe_decode(self.ctx, wg.handle, wu.handle, wd.handle, _ptr(x), _ptr(sel), _ptr(wts),
                                            _ptr(resid), n_slots_per_token, m, act_h.handle,
                                            act_x.handle if act_x is not None else None, _ptr(h), _ptr(y)))
 
     def enqueue_gate_up_x(self, wg, wu, x, sel, n_slots_per_token, m, rows_per_expert, act_h, act_x=None, h=None):
         self._check(self.lib.bm_gate_up_x(self.ctx, wg.handle, wu.handle, _ptr(x), _ptr(sel), n_slots_per_token, m,
-                                          rows_per_expert, act_h.handle, act_x.handle if act_x is not None else None,
-                                          _ptr(h)))
+                                          rows_per_expert, act_h.handle if act_h is not None else None,
+                                          act_x.handle if act_x is not None else None, _ptr(h)))
 
     def set_decode_plan(self, plan):
         self._check(self.lib.bm_set_decode_plan(self.ctx, plan))

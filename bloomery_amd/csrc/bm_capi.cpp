@@ -459,6 +459,32 @@ int bm_down_combine(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const u
                                                resid_dev, n_slots_per_token, m, rows_per_expert, y_dev));
 }
 
+int bm_down_combine_h(bm_ctx *ctx, const bm_weights *w, const float *h_dev, bm_act *act_h, const uint32_t *sel_dev,
+                      const float *w_dev, const float *resid_dev, int n_slots_per_token, int m, int rows_per_expert,
+                      float *y_dev) {
+    const char *what = "bm_down_combine_h";
+    if (!ctx || !w || !h_dev || !sel_dev || !w_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (act_form(w->wtype) == 0)
+        return fail(ctx, BM_ETYPE, "%s: folds the Q8_K quantizer; weight type %d takes Q8_2_X4 columns, which bm_gate_up and "
+                    "bm_gate_up_x already write: use bm_down_combine", what, w->wtype);
+    int n_experts = 0;
+    int rc = check_stack(ctx, what, w, rows_per_expert, &n_experts);
+    if (rc) return rc;
+    if (n_slots_per_token < 1 || n_slots_per_token > bmk::kMaxCombineSlots)
+        return fail(ctx, BM_ESHAPE, "%s: %d slots a token outside 1..=%d", what, n_slots_per_token, bmk::kMaxCombineSlots);
+    if (m < 1) return fail(ctx, BM_ESHAPE, "%s: need m >= 1 tokens, got %d", what, m);
+    if (act_h && (act_form(act_h->wtype) != 1 || act_h->k != w->k || (int64_t)act_h->m_cap < (int64_t)m * n_slots_per_token))
+        return fail(ctx, BM_ESHAPE, "%s: act_h must hold %d Q8_K columns of k = %d; it holds %d of k = %d (type %d)", what,
+                    m * n_slots_per_token, w->k, act_h->m_cap, act_h->k, act_h->wtype);
+    if (((uintptr_t)h_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: h_dev %p is not 16-byte aligned", what, (const void *)h_dev);
+    const size_t lds = (size_t)n_slots_per_token * dev_col_bytes(w->wtype, w->k) + 12288;
+    if (lds > (size_t)bmk::kMaxLds)
+        return fail(ctx, BM_ESHAPE, "%s: %d columns of k = %d do not fit the workgroup's LDS; use bm_quantize, bm_gemv_sel and "
+                    "bm_combine_tokens", what, n_slots_per_token, w->k);
+    return driver(ctx, what, bmk::down_combine_hq(launch_of(ctx), w->wtype, w->dev, n_experts, w->k, h_dev, act_h ? act_h->dev : nullptr,
+                                                  sel_dev, w_dev, resid_dev, n_slots_per_token, m, rows_per_expert, y_dev));
+}
+
 int bm_set_spin_limit(bm_ctx *ctx, uint32_t spins) {
     if (!ctx) return fail(nullptr, BM_EARG, "bm_set_spin_limit: ctx is NULL");
     ctx->spin_limit = spins;
@@ -468,10 +494,10 @@ int bm_set_spin_limit(bm_ctx *ctx, uint32_t spins) {
 int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const float *x_dev, const uint32_t *sel_dev,
                  int n_slots_per_token, int m, int rows_per_expert, bm_act *act_h, bm_act *act_x, float *h_dev) {
     const char *what = "bm_gate_up_x";
-    if (!ctx || !wg || !wu || !x_dev || !sel_dev || !act_h) return fail(ctx, BM_EARG, "%s: NULL argument", what);
-    if (wg->wtype != wu->wtype || (wg->wtype != BM_TYPE_Q4_K && wg->wtype != BM_TYPE_Q5_K))
-        return fail(ctx, BM_ETYPE, "%s: takes Q4_K or Q5_K gate and up stacks of one type, got types %d and %d; use bm_quantize and bm_gate_up",
-                    what, wg->wtype, wu->wtype);
+    if (!ctx || !wg || !wu || !x_dev || !sel_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (!act_h && !h_dev) return fail(ctx, BM_EARG, "%s: neither act_h nor h_dev: the launch would have no output", what);
+    if (wg->wtype != wu->wtype)
+        return fail(ctx, BM_ETYPE, "%s: gate is type %d and up type %d; one launch reads one type", what, wg->wtype, wu->wtype);
     if (wu->k != wg->k || wu->rows != wg->rows)
         return fail(ctx, BM_ESHAPE, "%s: gate is %lld x %d, up %lld x %d", what, (long long)wg->rows, wg->k, (long long)wu->rows, wu->k);
     const int hidden = wg->k, ff = rows_per_expert;
@@ -481,18 +507,20 @@ int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const 
     if (ff % 256 != 0) return fail(ctx, BM_ESHAPE, "%s: rows_per_expert = %d is not a whole number of 256-value super-blocks", what, ff);
     if (n_slots_per_token < 1 || m < 1 || m > bmk::kMaxDecodeTokens)
         return fail(ctx, BM_ESHAPE, "%s: %d slots a token, m = %d tokens (1..=%d)", what, n_slots_per_token, m, bmk::kMaxDecodeTokens);
-    if (act_form(act_h->wtype) != 0 || act_h->k != ff || (int64_t)act_h->m_cap < (int64_t)m * n_slots_per_token)
-        return fail(ctx, BM_ESHAPE, "%s: act_h must hold %d Q8_2_X4 columns of k = %d; it holds %d of k = %d (type %d)", what,
-                    m * n_slots_per_token, ff, act_h->m_cap, act_h->k, act_h->wtype);
-    if (act_x && (act_form(act_x->wtype) != 0 || act_x->k != hidden || act_x->m_cap < m))
-        return fail(ctx, BM_ESHAPE, "%s: act_x must hold %d Q8_2_X4 columns of k = %d; it holds %d of k = %d (type %d)", what, m, hidden,
-                    act_x->m_cap, act_x->k, act_x->wtype);
+    if (act_h && (act_form(act_h->wtype) != 0 || act_h->k != ff || (int64_t)act_h->m_cap < (int64_t)m * n_slots_per_token))
+        return fail(ctx, BM_ESHAPE,
+                    "%s: act_h must hold %d Q8_2_X4 columns of k = %d (the launch folds that quantizer only; pass NULL and h_dev for a "
+                    "down stack on Q8_K columns); it holds %d of k = %d (type %d)",
+                    what, m * n_slots_per_token, ff, act_h->m_cap, act_h->k, act_h->wtype);
+    if (act_x && (act_form(act_x->wtype) != act_form(wg->wtype) || act_x->k != hidden || act_x->m_cap < m))
+        return fail(ctx, BM_ESHAPE, "%s: act_x must hold %d %s columns of k = %d; it holds %d of k = %d (type %d)", what, m,
+                    act_form(wg->wtype) ? "Q8_K" : "Q8_2_X4", hidden, act_x->m_cap, act_x->k, act_x->wtype);
     if (((uintptr_t)x_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: x_dev %p is not 16-byte aligned", what, (const void *)x_dev);
-    if (dev_col_bytes(wg->wtype, hidden) + 128 > (size_t)bmk::kMaxLds)
+    if (dev_col_bytes(wg->wtype, hidden) + 8192 > (size_t)bmk::kMaxLds)
         return fail(ctx, BM_ESHAPE, "%s: a column of hidden = %d does not fit the workgroup's LDS", what, hidden);
     return driver(ctx, what,
                   bmk::gate_up_x(launch_of(ctx), wg->wtype, x_dev, wg->dev, wu->dev, n_experts, hidden, ff, sel_dev, n_slots_per_token, m,
-                                 act_x ? act_x->dev : nullptr, act_h->dev, h_dev));
+                                 act_x ? act_x->dev : nullptr, act_h ? act_h->dev : nullptr, h_dev));
 }
 
 int bm_set_decode_plan(bm_ctx *ctx, int plan) {
@@ -513,8 +541,8 @@ int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const
         return fail(ctx, BM_ETYPE, "%s: gate is type %d and up type %d; one launch reads one type", what, wg->wtype, wu->wtype);
     if (!bmk::moe_decode_supported(ctx->decode_plan, wg->wtype, wd->wtype))
         return fail(ctx, BM_ETYPE,
-                    "%s: the fused step takes Q4_K or Q5_K gate/up with Q4_K, Q5_K or Q6_K down (as one launch: Q4_K with Q6_K or Q4_K), got %d "
-                    "and %d; use the separate launches",
+                    "%s: as one launch the fused step takes Q4_K gate/up with Q6_K or Q4_K down (as two: every type), got %d and %d; "
+                    "use BM_PLAN_TWO_LAUNCHES or the separate launches",
                     what, wg->wtype, wd->wtype);
     if (wu->k != wg->k || wu->rows != wg->rows)
         return fail(ctx, BM_ESHAPE, "%s: gate is %lld x %d, up %lld x %d", what, (long long)wg->rows, wg->k, (long long)wu->rows, wu->k);
@@ -529,15 +557,19 @@ int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const
         return fail(ctx, BM_ESHAPE, "%s: %d slots a token outside 1..=%d", what, n_slots_per_token, bmk::kMaxCombineSlots);
     if (m < 1 || m > bmk::kMaxDecodeTokens)
         return fail(ctx, BM_ESHAPE, "%s: m = %d tokens outside 1..=%d", what, m, bmk::kMaxDecodeTokens);
-    if (act_form(act_h->wtype) != 0 || act_h->k != ff || (int64_t)act_h->m_cap < (int64_t)m * n_slots_per_token)
-        return fail(ctx, BM_ESHAPE, "%s: act_h must hold %d Q8_2_X4 columns of k = %d; it holds %d of k = %d (type %d)", what,
-                    m * n_slots_per_token, ff, act_h->m_cap, act_h->k, act_h->wtype);
-    if (act_x && (act_form(act_x->wtype) != 0 || act_x->k != hidden || act_x->m_cap < m))
-        return fail(ctx, BM_ESHAPE, "%s: act_x must hold %d Q8_2_X4 columns of k = %d; it holds %d of k = %d (type %d)", what, m, hidden,
-                    act_x->m_cap, act_x->k, act_x->wtype);
+    if (act_form(act_h->wtype) != act_form(wd->wtype) || act_h->k != ff || (int64_t)act_h->m_cap < (int64_t)m * n_slots_per_token)
+        return fail(ctx, BM_ESHAPE, "%s: act_h must hold %d %s columns of k = %d; it holds %d of k = %d (type %d)", what,
+                    m * n_slots_per_token, act_form(wd->wtype) ? "Q8_K" : "Q8_2_X4", ff, act_h->m_cap, act_h->k, act_h->wtype);
+    if (act_x && (act_form(act_x->wtype) != act_form(wg->wtype) || act_x->k != hidden || act_x->m_cap < m))
+        return fail(ctx, BM_ESHAPE, "%s: act_x must hold %d %s columns of k = %d; it holds %d of k = %d (type %d)", what, m,
+                    act_form(wg->wtype) ? "Q8_K" : "Q8_2_X4", hidden, act_x->m_cap, act_x->k, act_x->wtype);
+    if (act_form(wd->wtype) != 0 && !h_dev)
+        return fail(ctx, BM_EARG, "%s: a down stack on Q8_K columns needs h_dev: the gate . up launch leaves h there as f32 rows and "
+                    "the down launch quantizes them", what);
     if (((uintptr_t)x_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: x_dev %p is not 16-byte aligned", what, (const void *)x_dev);
-    const size_t lds_a = dev_col_bytes(wg->wtype, hidden) + 128;
-    const size_t lds_b = (size_t)n_slots_per_token * dev_col_bytes(wd->wtype, ff) + 4096;
+    if (h_dev && ((uintptr_t)h_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: h_dev %p is not 16-byte aligned", what, (const void *)h_dev);
+    const size_t lds_a = dev_col_bytes(wg->wtype, hidden) + 8192;
+    const size_t lds_b = (size_t)n_slots_per_token * dev_col_bytes(wd->wtype, ff) + 12288;
     if (lds_a > (size_t)bmk::kMaxLds || lds_b > (size_t)bmk::kMaxLds)
         return fail(ctx, BM_ESHAPE, "%s: hidden = %d or %d columns of ff = %d do not fit the workgroup's LDS; use the separate launches", what,
                     hidden, n_slots_per_token, ff);

@@ -67,11 +67,15 @@ hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_expe
 constexpr int kPlanOneLaunch = 1, kPlanTwoLaunches = 2;
 constexpr int kMaxDecodeTokens = 1024;
 bool moe_decode_supported(int plan, int gate_type, int down_type);
-// gate . up . SwiGLU from f32 token rows, both quantizers folded in (Q4_K or Q5_K gate/up): the first launch of
-// kPlanTwoLaunches.
+// gate . up . SwiGLU from f32 token rows, the token quantizer folded in: the first launch of kPlanTwoLaunches. act_h
+// (Q8_2_X4 columns, or NULL when the down stack takes Q8_K ones) is quantized in the same launch; h (f32 rows) is
+// optional beside act_h and the output without it.
 hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8_t *wg, const uint8_t *wu,
                      int n_experts, int hidden, int ff, const uint32_t *sel, int slots_per_token, int m,
                      uint8_t *act_x, uint8_t *act_h, float *h);
+hipError_t down_combine_hq(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const float *h,
+                           uint8_t *act_h, const uint32_t *sel, const float *wts, const float *resid,
+                           int slots_per_token, int m, int rows_per_expert, float *y);
 hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, const float *x, const uint8_t *wg,
                       const uint8_t *wu, const uint8_t *wd, int n_experts, int hidden, int ff, const uint32_t *sel,
                       const float *wts, const float *resid, int slots_per_token, int m, uint8_t *act_x,

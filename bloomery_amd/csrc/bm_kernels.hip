@@ -437,7 +437,7 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
     const int r = rb * 32 + (tid >> 3);
     const u32 id = sel[slot];
     const int col_bytes = bm_act_col_bytes<WA>(na);
-    uint8_t *hcol = act_h + (size_t)slot * nh * BM_Q82_SB_EXT;
+    uint8_t *hcol = act_h ? act_h + (size_t)slot * nh * BM_Q82_SB_EXT : nullptr; // none: the down stack takes Q8_K columns
     uint8_t *col = lds;
     // the token's row: eight consecutive values a lane, 2048 a pass
     constexpr int kPasses = NBA > 0 ? (NBA * 256 + 2047) / 2048 : 1;
@@ -456,7 +456,7 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
     if (id >= n_experts) { // uniform over the workgroup
         if (tid == 0) bm_raise(fault, layer, kSiteExpertId);
         if (h && (tid & 7) == 0) h[(size_t)slot * ff + r] = bm_bits_f32(0x7fc00000u);
-        if (tid < 32) q82_store(hcol, nh, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);
+        if (hcol && tid < 32) q82_store(hcol, nh, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);
         return;
     }
     const size_t row_bytes = (size_t)na * bm_block_bytes<WA>();
@@ -481,6 +481,7 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
     row_dot<WA, UA, NBA, 1>(b, wrow, col, col_bytes, 1, na, q, Iq2Tables{}, v, NoTap{});
     const float hv = swiglu_of_pair(v[0], which, rule, fault, layer);
     if (h && (tid & 7) == 0) h[(size_t)slot * ff + r] = hv;
+    if (!hcol) return;
     float *hbuf = reinterpret_cast<float *>(col + col_bytes);
     if ((tid & 7) == 0) hbuf[tid >> 3] = hv;
     __syncthreads();
@@ -540,6 +541,182 @@ __global__ __launch_bounds__(256) void k_moe_decode(const float *x, const uint8_
         if (done == (u32)(m * blocks_per_token) - 1) {
             for (int i = 0; i <= m; i++) __hip_atomic_store(&counters[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+    }
+}
+
+// ------------------------------------------------------------- the fused step for the types that take Q8_K columns
+
+// One 256-value block of a Q8_K column by one wave, four consecutive values a lane: k_quantize_q8k's operations on the
+// same operands (crates/qdot/src/lib.rs:1787-1809), the block's maximum and the sums met through lane exchanges.
+// `o` is the block's 296 bytes (LDS or global memory).
+__device__ __forceinline__ void q8k_wave_block(const float4 x4, uint8_t *o, int lane, u32 *fault, u32 layer) {
+    const float v[4] = {x4.x, x4.y, x4.z, x4.w};
+    // the largest magnitude: a maximum of the sign-less bit patterns over the wave
+    u32 mine_ab = 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const u32 a = bm_f32_bits(v[k]) & 0x7fffffffu;
+        mine_ab = a > mine_ab ? a : mine_ab;
+    }
+    const u32 half_ab = bm_max32(mine_ab); // over each half of the wave
+    const u32 lo_ab = (u32)__builtin_amdgcn_readlane((int)half_ab, 0), hi_ab = (u32)__builtin_amdgcn_readlane((int)half_ab, 32);
+    const u32 ab = lo_ab > hi_ab ? lo_ab : hi_ab;
+    // its first holder (value 4 * lane + k): the lowest lane among those that hold it at k, the lowest such value
+    int first = 1 << 20;
+    float max = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const unsigned long long holders = __ballot((bm_f32_bits(v[k]) & 0x7fffffffu) == ab);
+        if (holders) { // uniform over the wave
+            const int at = __builtin_ctzll(holders);
+            const float val = bm_bits_f32((u32)__builtin_amdgcn_readlane((int)bm_f32_bits(v[k]), at));
+            if (4 * at + k < first) first = 4 * at + k, max = val;
+        }
+    }
+    float d;
+    int code[4] = {0, 0, 0, 0};
+    if (ab > 0x7f7fffffu) {
+        if (lane == 0) bm_raise(fault, layer, kSiteQuantColumn);
+        d = bm_bits_f32(0x7fc00000u);
+    } else if (ab == 0) {
+        d = 0.0f;
+    } else {
+        const float iscale = __fdiv_rn(-127.0f, max);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            int qv = bm_nearest_int(__fmul_rn(iscale, v[k]));
+            qv = qv > 127 ? 127 : qv;
+            code[k] = (int)(signed char)(qv & 0xff); // `as i8`: the low byte
+        }
+        d = __fdiv_rn(1.0f, iscale);
+    }
+    *reinterpret_cast<u32 *>(o + 8 + 4 * lane) = (u32)(code[0] & 0xff) | ((u32)(code[1] & 0xff) << 8) |
+                                                 ((u32)(code[2] & 0xff) << 16) | ((u32)(code[3] & 0xff) << 24);
+    int sum = code[0] + code[1] + code[2] + code[3]; // sixteen codes a sum: four lanes
+    sum += (int)bm_dpp<kDppXor1>((u32)sum);
+    sum += (int)bm_dpp<kDppXor2>((u32)sum);
+    if ((lane & 3) == 0) *reinterpret_cast<unsigned short *>(o + 264 + 2 * (lane >> 2)) = (unsigned short)(short)sum;
+    if (lane == 0) {
+        *reinterpret_cast<float *>(o) = d;
+        *reinterpret_cast<u32 *>(o + 4) = 0u;
+    }
+}
+
+// `cols` columns of nb blocks each, f32 rows at x (column c at x + c * nb * 256), into LDS at `dst` by the workgroup's
+// waves, block by block.
+__device__ __forceinline__ void q8k_stage_cols(const float *x, uint8_t *dst, int cols, int nb, u32 *fault, u32 layer) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+    const int total = cols * nb;
+    constexpr int kAhead = 6; // blocks whose loads a wave has in flight
+    for (int b0 = wave; b0 < total; b0 += kAhead * n_waves) {
+        float4 x4[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; u++) {
+            const int b = b0 + u * n_waves;
+            x4[u] = *reinterpret_cast<const float4 *>(x + (size_t)(b < total ? b : b0) * 256 + 4 * lane);
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; u++) {
+            const int b = b0 + u * n_waves;
+            if (b < total) q8k_wave_block(x4[u], dst + (size_t)b * BM_Q8K_STRIDE, lane, fault, layer);
+        }
+    }
+}
+
+// k_gate_up_x for gate / up stacks that dot against Q8_K columns (Q3_K, IQ2_XXS, IQ3_XXS, IQ4_XS): the token's row is
+// quantized by every workgroup into LDS, h is written as f32 rows, and where the down stack takes Q8_2_X4 columns
+// (act_h given) the workgroup's 32 values also become their block of the slot's column.
+template <int WA, int UA, int NBA>
+__global__ __launch_bounds__(256) void k_gate_up_xq(const float *x, const uint8_t *wg, const uint8_t *wu, u32 n_experts,
+                                                    int nba, int nh, const u32 *sel, int spt, uint8_t *act_x,
+                                                    uint8_t *act_h, float *h, GateRule rule, u32 *fault, u32 layer) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
+    const int blocks_per_slot = nh * 8;
+    const int slot = blockIdx.x / blocks_per_slot, rb = blockIdx.x % blocks_per_slot;
+    const int na = NBA > 0 ? NBA : nba;
+    const int hidden = na * 256, ff = nh * 256;
+    const int t = slot / spt;
+    const int r = rb * 32 + (tid >> 3);
+    const u32 id = sel[slot];
+    uint8_t *hcol = act_h ? act_h + (size_t)slot * nh * BM_Q82_SB_EXT : nullptr;
+    if (id >= n_experts) { // uniform over the workgroup
+        if (tid == 0) bm_raise(fault, layer, kSiteExpertId);
+        if (h && (tid & 7) == 0) h[(size_t)slot * ff + r] = bm_bits_f32(0x7fc00000u);
+        if (hcol && tid < 32) q82_store(hcol, nh, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);
+        return;
+    }
+    const size_t row_bytes = (size_t)na * bm_block_bytes<WA>();
+    const uint8_t *wrow = (which ? wu : wg) + ((size_t)id * ff + r) * row_bytes;
+    Blk<WA> b[UA];
+    preload<WA, UA>(b, wrow, q);
+    const Iq2Tables tb = stage_tables<WA>(lds);
+    uint8_t *col = lds + tab_bytes<WA>();
+    const int col_bytes = bm_act_col_bytes<WA>(na);
+    q8k_stage_cols(x + (size_t)t * hidden, col, 1, na, fault, layer);
+    __syncthreads();
+    if (act_x && rb == 0 && slot % spt == 0) stage_bytes(act_x + (size_t)t * col_bytes, col, col_bytes);
+    float v[1];
+    row_dot<WA, UA, NBA, 1>(b, wrow, col, col_bytes, 1, na, q, tb, v, NoTap{});
+    const float hv = swiglu_of_pair(v[0], which, rule, fault, layer);
+    if (h && (tid & 7) == 0) h[(size_t)slot * ff + r] = hv;
+    if (hcol) {
+        float *hbuf = reinterpret_cast<float *>(col + col_bytes);
+        if ((tid & 7) == 0) hbuf[tid >> 3] = hv;
+        __syncthreads();
+        if (tid < 32) quantize_h_block(hbuf, hcol, nh, rb, tid, fault, layer);
+    }
+}
+
+// k_down_combine for down stacks that dot against Q8_K columns: the token's slot rows of h (f32) are quantized by
+// every workgroup into LDS; the first workgroup of a token also leaves the columns in act_h.
+template <int WT, int U, int NB>
+__global__ __launch_bounds__(256) void k_down_combine_hq(const uint8_t *w, u32 n_experts, int nb, const float *h,
+                                                         uint8_t *act_h, const u32 *sel, const float *wts,
+                                                         const float *resid, int spt, int rpe, float *y, u32 *fault,
+                                                         u32 layer) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, q = tid & 3, quad = tid >> 2;
+    const int D = 64 / spt;
+    const int blocks_per_token = (rpe + D - 1) / D;
+    const int t = blockIdx.x / blocks_per_token, rb = blockIdx.x % blocks_per_token;
+    const int e = quad % spt, dl = quad / spt;
+    const int r = rb * D + dl;
+    const u32 id = sel[t * spt + e];
+    const int si = tid < spt ? tid : 0;
+    const u32 my_sel = sel[t * spt + si];
+    const float my_w = wts[t * spt + si];
+    const bool live = id < n_experts;
+    const bool active = dl < D && r < rpe && live;
+    if (!live && id != 0xffffffffu && rb == 0 && dl == 0 && q == 0) bm_raise(fault, layer, kSiteExpertId);
+    const int n = NB > 0 ? NB : nb;
+    const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
+    const int col_bytes = bm_act_col_bytes<WT>(n);
+    const uint8_t *wrow = w + ((size_t)(live ? id : 0) * rpe + (active ? r : 0)) * row_bytes;
+    Blk<WT> b[U];
+    preload<WT, U>(b, wrow, q);
+    const Iq2Tables tb = stage_tables<WT>(lds);
+    uint8_t *cols = lds + tab_bytes<WT>();
+    float *part = reinterpret_cast<float *>(cols + (size_t)spt * col_bytes); // [D][spt]
+    float *s_w = part + D * spt;                                              // [spt]
+    u32 *s_sel = reinterpret_cast<u32 *>(s_w + spt);                          // [spt]
+    q8k_stage_cols(h + (size_t)t * spt * n * 256, cols, spt, n, fault, layer);
+    if (tid < spt) {
+        s_w[tid] = my_w;
+        s_sel[tid] = my_sel;
+    }
+    __syncthreads();
+    if (act_h && rb == 0) stage_bytes(act_h + (size_t)t * spt * col_bytes, cols, spt * col_bytes);
+    float v[1];
+    row_dot<WT, U, NB, 1>(b, wrow, cols + (size_t)e * col_bytes, col_bytes, 1, n, q, tb, v, NoTap{});
+    if (q == 0 && dl < D) part[dl * spt + e] = v[0];
+    __syncthreads();
+    if (tid < D && rb * D + tid < rpe) {
+        float acc = 0.0f;
+        for (int s = 0; s < spt; s++)
+            if (s_sel[s] < n_experts) acc = fmaf(s_w[s], part[tid * spt + s], acc);
+        const size_t o = (size_t)t * rpe + rb * D + tid;
+        y[o] = resid ? __fadd_rn(acc, resid[o]) : acc;
     }
 }
 
@@ -674,9 +851,14 @@ hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_expe
     return hipGetLastError();
 }
 
+static bool tab_known(int t) {
+    return t == BM_Q3K || t == BM_Q4K || t == BM_Q5K || t == BM_Q6K || t == BM_IQ2XXS || t == BM_IQ3XXS || t == BM_IQ4XS;
+}
+
 bool moe_decode_supported(int plan, int gate_type, int down_type) {
     if (plan == kPlanOneLaunch) return gate_type == BM_Q4K && (down_type == BM_Q6K || down_type == BM_Q4K);
-    return (gate_type == BM_Q4K || gate_type == BM_Q5K) && (down_type == BM_Q4K || down_type == BM_Q5K || down_type == BM_Q6K);
+    // two launches: every type this library has a row dot for, on either side
+    return tab_known(gate_type) && tab_known(down_type);
 }
 
 hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8_t *wg, const uint8_t *wu,
@@ -699,10 +881,44 @@ hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8
     } else if (gate_type == BM_Q5K) {
         if (nba == 8) BM_GUX(BM_Q5K, kRingQ5K, 8)
         else BM_GUX(BM_Q5K, 1, 0)
+    } else if (gate_type == BM_Q6K) {
+        if (nba % 2 == 0) BM_GUX(BM_Q6K, 2, 0)
+        else BM_GUX(BM_Q6K, 1, 0)
+    } else if (bm_takes_q8k(gate_type)) {
+        const int nb = nba;
+        const size_t lds_q = tab_bytes_rt(gate_type) + (size_t)act_col_bytes(gate_type, hidden) + 32 * sizeof(float);
+#define CALL_BODY                                                                                                      \
+    auto kern = k_gate_up_xq<WT, U, NB>;                                                                               \
+    hipError_t e = allow_lds(kern, lds_q);                                                                             \
+    if (e != hipSuccess) return e;                                                                                     \
+    hipLaunchKernelGGL(kern, dim3(grid_a), dim3(256), lds_q, L.stream, x, wg, wu, (u32)n_experts, nba, nbb, sel, spt,  \
+                       act_x, act_h, h, L.rule, L.fault, L.layer);
+        BM_DISPATCH(gate_type, nb)
+#undef CALL_BODY
     } else {
         return hipErrorInvalidValue;
     }
 #undef BM_GUX
+    return hipGetLastError();
+}
+
+// Down + combine from the f32 rows of h, for a down stack that takes Q8_K columns; act_h (optional) receives them.
+hipError_t down_combine_hq(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const float *h,
+                           uint8_t *act_h, const uint32_t *sel, const float *wts, const float *resid,
+                           int slots_per_token, int m, int rows_per_expert, float *y) {
+    const int nb = k / 256, rpe = rows_per_expert, spt = slots_per_token;
+    const int D = 64 / spt;
+    const size_t lds = down_combine_lds(wtype, k, spt);
+    const unsigned grid = (unsigned)m * (unsigned)((rpe + D - 1) / D);
+    if (!bm_takes_q8k(wtype)) return hipErrorInvalidValue;
+#define CALL_BODY                                                                                                      \
+    auto kern = k_down_combine_hq<WT, U, NB>;                                                                          \
+    hipError_t e = allow_lds(kern, lds);                                                                               \
+    if (e != hipSuccess) return e;                                                                                     \
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, (u32)n_experts, nb, h, act_h, sel, wts, resid,   \
+                       spt, rpe, y, L.fault, L.layer);
+    BM_DISPATCH(wtype, nb)
+#undef CALL_BODY
     return hipGetLastError();
 }
 
@@ -717,8 +933,12 @@ hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, c
     const unsigned grid_a = (unsigned)m * (unsigned)spt * (unsigned)(ff / 32);
     if (!moe_decode_supported(plan, gate_type, down_type)) return hipErrorInvalidValue;
     if (plan == kPlanTwoLaunches) {
-        hipError_t e = gate_up_x(L, gate_type, x, wg, wu, n_experts, hidden, ff, sel, spt, m, act_x, act_h, h);
+        // a down stack on Q8_K columns cannot get them from the gate . up launch (a column's block spans eight of
+        // its workgroups): that launch leaves h as f32 rows and the down launch quantizes them itself
+        const bool hq = bm_takes_q8k(down_type);
+        hipError_t e = gate_up_x(L, gate_type, x, wg, wu, n_experts, hidden, ff, sel, spt, m, act_x, hq ? nullptr : act_h, h);
         if (e != hipSuccess) return e;
+        if (hq) return down_combine_hq(L, down_type, wd, n_experts, ff, h, act_h, sel, wts, resid, spt, m, hidden, y);
         return down_combine(L, down_type, wd, n_experts, ff, act_h, sel, wts, resid, spt, m, hidden, y);
     }
     const size_t lds = lds_a > lds_b ? lds_a : lds_b;

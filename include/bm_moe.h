@@ -167,14 +167,24 @@ int bm_down_combine(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const u
                     const float *w_dev, const float *resid_dev, int n_slots_per_token, int m, int rows_per_expert,
                     float *y_dev);
 
+/* bm_quantize of the slots' f32 rows of h and bm_down_combine in one launch, for a down stack that takes Q8_K
+ * columns (Q3_K and the IQ types; the K-quants on Q8_2_X4 columns get theirs from bm_gate_up / bm_gate_up_x): slot s
+ * reads h_dev[s * k .. (s + 1) * k), k = w's k, 16-byte aligned. act_h (optional) receives the quantized columns.
+ * Same bits as the two calls. No counterpart launch in the reference. */
+int bm_down_combine_h(bm_ctx *ctx, const bm_weights *w, const float *h_dev, bm_act *act_h, const uint32_t *sel_dev,
+                      const float *w_dev, const float *resid_dev, int n_slots_per_token, int m, int rows_per_expert,
+                      float *y_dev);
+
 /* The whole decode step of one MoE layer for m tokens with every quantizer folded in (no counterpart in the
  * reference, whose step is the chain quantize, gate_up, quantize, down, combine: dispatch.rs:1245-1436): x_dev
  * holds m rows of hidden = wg's k f32 values (16-byte aligned); token t's slots are sel_dev / w_dev[t *
  * n_slots_per_token ..]; y_dev[t * hidden + d] gets bm_combine_tokens' value. Same bits as bm_quantize, bm_gate_up
- * (with act_h) and bm_down_combine run one after the other. Gate/up must be Q4_K or Q5_K, down Q4_K, Q5_K or Q6_K
- * (BM_PLAN_ONE_LAUNCH: Q4_K gate/up, Q6_K or Q4_K down); other types take the separate launches. act_h is caller-held scratch (m * n_slots_per_token Q8_2_X4 columns of ff = wd's k)
- * and holds the quantized h afterwards; act_x (optional) receives the quantized x columns; h_dev (optional) the
- * f32 h rows. m <= 1024.
+ * (with act_h) and bm_down_combine run one after the other. Gate and up are of one type; every type of this library
+ * goes on either side (BM_PLAN_ONE_LAUNCH: Q4_K gate/up with Q6_K or Q4_K down only). act_h is caller-held scratch
+ * (m * n_slots_per_token columns of ff = wd's k, in the form wd dots against) and holds the quantized h afterwards;
+ * act_x (optional, in the form wg dots against) receives the quantized x columns; h_dev receives the f32 h rows:
+ * optional, except that a down stack on Q8_K columns needs it (16-byte aligned): a Q8_K block spans eight gate . up
+ * workgroups, so that launch leaves f32 rows and the down launch quantizes them (bm_down_combine_h). m <= 1024.
  * Two plans (bm_set_decode_plan):
  *   BM_PLAN_TWO_LAUNCHES (default): gate . up with both quantizers folded in, then down + combine;
  *   BM_PLAN_ONE_LAUNCH: one launch; the down workgroups start streaming their rows at once and wait on a
@@ -188,8 +198,9 @@ int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const
                   bm_act *act_h, bm_act *act_x, float *h_dev, float *y_dev);
 int bm_set_decode_plan(bm_ctx *ctx, int plan);
 /* The first launch of BM_PLAN_TWO_LAUNCHES on its own: bm_quantize, bm_gate_up and the quantizer of h in one
- * launch, from the f32 token rows (Q4_K or Q5_K gate/up; rows_per_expert = ff a multiple of 256). Follow it with
- * bm_down_combine or bm_gemv_sel over act_h. */
+ * launch, from the f32 token rows (gate and up of one type; rows_per_expert = ff a multiple of 256). act_h: Q8_2_X4
+ * columns for the down stack, or NULL; h_dev: the f32 h rows, or NULL; one of the two at least. Follow it with
+ * bm_down_combine or bm_gemv_sel over act_h, or bm_down_combine_h over h_dev. */
 int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const float *x_dev, const uint32_t *sel_dev,
                  int n_slots_per_token, int m, int rows_per_expert, bm_act *act_h, bm_act *act_x, float *h_dev);
 /* Polls (a memory round trip each, about a microsecond) a BM_PLAN_ONE_LAUNCH consumer waits before it gives up;

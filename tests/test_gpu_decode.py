@@ -404,10 +404,19 @@ def run_single_launch(gpu, L, x, ids, wts, top_k, resid=None, replays=1, plan=bm
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 4096, 256, 4, 2, 3),    # rows longer than one quantizer pass
     ((bm.Q5_K, bm.Q5_K, bm.Q6_K), 2048, 512, 4, 3, 4),    # Q5_K gate/up at the whole-row shape (two launches only)
     ((bm.Q5_K, bm.Q5_K, bm.Q5_K), 768, 256, 3, 2, 2),
+    # the types on Q8_K columns: their quantizers folded into the two launches (the token's in every gate . up
+    # workgroup, h's in every down workgroup), and the mixes of the two column forms
+    ((bm.IQ4_XS, bm.IQ4_XS, bm.IQ4_XS), 2048, 768, 6, 3, 4),
+    ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ3_XXS), 1024, 512, 5, 2, 4),
+    ((bm.Q3_K, bm.Q3_K, bm.Q6_K), 768, 512, 4, 5, 2),
+    ((bm.Q4_K, bm.Q4_K, bm.IQ4_XS), 2048, 512, 4, 3, 4),
+    ((bm.Q5_K, bm.Q5_K, bm.Q3_K), 512, 768, 3, 2, 3),
+    ((bm.Q6_K, bm.Q6_K, bm.Q4_K), 768, 256, 3, 2, 2),
 ))
 @pytest.mark.parametrize("plan", (bm.PLAN_ONE_LAUNCH, bm.PLAN_TWO_LAUNCHES))
 def test_single_launch_step_matches_the_chain_and_the_oracle(gpu, types, hidden, ff, n_experts, m, top_k, plan):
-    if types[0] == bm.Q5_K and plan == bm.PLAN_ONE_LAUNCH:  # that plan takes Q4_K gate/up only and says so
+    # the one-launch plan takes Q4_K gate/up with Q6_K or Q4_K down only, and says so
+    if (types[0] != bm.Q4_K or types[2] not in (bm.Q4_K, bm.Q6_K)) and plan == bm.PLAN_ONE_LAUNCH:
         L = Layer(gpu, types, hidden, ff, n_experts, 600 + hidden + ff, cheap=True)
         x = np.zeros((m, hidden), np.float32)
         with pytest.raises(bm.GpuError) as e:

@@ -576,6 +576,31 @@ def main():
         gpu.event_record(e1)
         kernel_us[name] = gpu.event_elapsed_ms(e0, e1) * 1e3 / (r * unit)
         gpu.graph_destroy(g1)
+    # the step before the layer, timed beside it (not part of `value`): norm + router logits, then softmax top-k
+    rng_r = np.random.default_rng(0x707E0001)
+    router_d = gpu.upload(rng_r.standard_normal((N_EXPERTS, HIDDEN), dtype=np.float32) * np.float32(0.05), np.float32)
+    gain_d = gpu.upload(np.ones(HIDDEN, np.float32), np.float32)
+    normed_d, logits_d = gpu.buffer(np.float32, HIDDEN), gpu.buffer(np.float32, N_EXPERTS)
+    ids_d, wts_d = gpu.buffer(np.uint32, TOP_K), gpu.buffer(np.float32, TOP_K)
+    router_us = {}
+    for name in ("router_logits", "route_softmax"):
+        gpu.capture_begin()
+        for i in range(unit):
+            if name == "router_logits":
+                gpu.enqueue_router_logits(router_d, xd.ptr + 4 * (i % n_tok) * HIDDEN, gain_d, 1e-6, 1, N_EXPERTS, HIDDEN,
+                                          normed_d, logits_d)
+            else:
+                gpu.enqueue_route_softmax(logits_d, 1, N_EXPERTS, TOP_K, True, None, ids_d, wts_d)
+        g1 = gpu.capture_end()
+        gpu.graph_launch(g1)
+        gpu.sync()
+        gpu.event_record(e0)
+        r = max(1, 1024 // unit)
+        for _ in range(r):
+            gpu.graph_launch(g1)
+        gpu.event_record(e1)
+        router_us[name] = gpu.event_elapsed_ms(e0, e1) * 1e3 / (r * unit)
+        gpu.graph_destroy(g1)
     gate_up_bytes = TOP_K * 2 * FF * bm.row_bytes(gate_t, HIDDEN)
     down_bytes = TOP_K * HIDDEN * bm.row_bytes(down_t, FF)
     if single:
@@ -633,6 +658,7 @@ def main():
         "event_ms_per_step": ev_ms / steps,
         "kernel_us": kernel_us,
         "kernel_gbps": kernel_gbps,
+        "router_kernel_us": router_us,
         "parity": parity,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,

@@ -83,6 +83,7 @@ SYMBOLS = {
     "bm_moe_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_set_gate_rule": (_i, [_vp, _i, C.c_float]),
     "bm_route_softmax": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "bm_router_logits": (_i, [_vp, _vp, _vp, _vp, C.c_float, _i, _i, _i, _vp, _vp]),
     "bm_gguf_open": (_i, [C.c_char_p, C.POINTER(_vp)]),
     "bm_gguf_close": (None, [_vp]),
     "bm_gguf_last_error": (C.c_char_p, []),
@@ -530,6 +531,13 @@ class Gpu:
         """RouterKernels::enqueue_route (crates/gpu/src/route_softmax.rs:1643): softmax, top-k, renormalised weights."""
         self._check(self.lib.bm_route_softmax(self.ctx, _ptr(logits), n_tokens, n_experts, top_k, int(bool(renorm)),
                                               _ptr(probs) if probs is not None else None, _ptr(ids), _ptr(weights)))
+
+    def enqueue_router_logits(self, router, x, gain, eps, n_tokens, n_experts, hidden, normed, logits):
+        """The FFN norm (gain None: none) and the router's f32 logits, the step before enqueue_route_softmax
+        (bm_router_logits); normed (optional) receives the normed rows."""
+        self._check(self.lib.bm_router_logits(self.ctx, _ptr(router), _ptr(x), _ptr(gain) if gain is not None else None,
+                                              float(eps), n_tokens, n_experts, hidden,
+                                              _ptr(normed) if normed is not None else None, _ptr(logits)))
 
     def enqueue_block_sums(self, w, row, act, col, out):
         self._check(self.lib.bm_block_sums(self.ctx, w.handle, row, act.handle, col, _ptr(out)))

@@ -863,6 +863,23 @@ int bm_route_softmax(bm_ctx *ctx, const float *logits_dev, int n_tokens, int n_e
                                                 ids_dev, weights_dev));
 }
 
+int bm_router_logits(bm_ctx *ctx, const float *router_dev, const float *x_dev, const float *gain_dev, float eps, int n_tokens,
+                     int n_experts, int hidden, float *normed_dev, float *logits_dev) {
+    const char *what = "bm_router_logits";
+    if (!ctx || !router_dev || !x_dev || !logits_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (n_tokens < 1 || n_experts < 1) return fail(ctx, BM_ESHAPE, "%s: %d tokens, %d experts: both must be positive", what, n_tokens, n_experts);
+    if (hidden < 8 || hidden % 8 != 0)
+        return fail(ctx, BM_ESHAPE, "%s: hidden = %d is not a positive multiple of 8 (the f32 row dot's eight lanes)", what, hidden);
+    if ((int64_t)n_tokens * n_experts > (1 << 30)) return fail(ctx, BM_ESHAPE, "%s: %d tokens x %d experts is past what a launch takes", what, n_tokens, n_experts);
+    if (!bmk::router_logits_fits(hidden)) return fail(ctx, BM_ESHAPE, "%s: two rows of hidden = %d do not fit the workgroup's LDS", what, hidden);
+    if ((((uintptr_t)router_dev | (uintptr_t)x_dev | (uintptr_t)gain_dev | (uintptr_t)normed_dev) & 15) != 0)
+        return fail(ctx, BM_ESHAPE, "%s: router_dev %p, x_dev %p, gain_dev %p and normed_dev %p must be 16-byte aligned", what,
+                    (const void *)router_dev, (const void *)x_dev, (const void *)gain_dev, (const void *)normed_dev);
+    if (gain_dev && !(eps >= 0.0f)) return fail(ctx, BM_EARG, "%s: eps = %g is negative or not a number", what, (double)eps);
+    return driver(ctx, what, bmk::router_logits(launch_of(ctx), router_dev, x_dev, gain_dev, eps, n_tokens, n_experts, hidden, normed_dev,
+                                                logits_dev));
+}
+
 int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *act, int col, int32_t *out_dev) {
     const char *what = "bm_block_sums";
     if (!ctx || !w || !act || !out_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);

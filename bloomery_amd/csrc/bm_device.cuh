@@ -77,6 +77,19 @@ __device__ __forceinline__ float bm_q82_inverse(u32 t) {
     return (bm_f32_bits(id) & 0x7fffffffu) < 0x7f800000u ? id : 0.0f;
 }
 
+// The correctly rounded square root of a positive normal f32. The hardware's is within a unit in the last place (and
+// the runtime's "rn" form compiles to it as it stands), so the two neighbours are tried against the exact residuals:
+// x <= s_down * s puts sqrt(x) below the midpoint of s_down and s, x > s_up * s above that of s and s_up.
+__device__ __forceinline__ float bm_sqrt_rn(float x) {
+    float s = __builtin_amdgcn_sqrtf(x);
+    if (!(x > 0.0f) || bm_f32_bits(x) >= 0x7f800000u) return s; // zero, negative, infinite, NaN: the instruction's own result
+    const float s_dn = bm_bits_f32(bm_f32_bits(s) - 1u), s_up = bm_bits_f32(bm_f32_bits(s) + 1u);
+    const float vp = fmaf(-s_dn, s, x), vs = fmaf(-s_up, s, x);
+    s = vp <= 0.0f ? s_dn : s;
+    s = vs > 0.0f ? s_up : s;
+    return s;
+}
+
 __device__ __forceinline__ int bm_sdot4(u32 a, u32 b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
 
 // a * b + c for factors inside 24 signed bits (every integer the IQ cores scale is): one full-rate instruction where

@@ -126,6 +126,12 @@ constexpr int kRouteMaxExperts = 1024, kRouteMaxPicks = 32;
 hipError_t route_softmax(const Launch &L, const float *logits, int n_tok, int n_exp, int used, int renorm, float *probs,
                          uint32_t *ids, float *weights);
 
+// The FFN norm (gain NULL: none) and the router's f32 logits: router[n_exp * hidden], x[m * hidden], logits[m * n_exp],
+// normed_out (optional) [m * hidden]. hidden a multiple of 8.
+bool router_logits_fits(int hidden);
+hipError_t router_logits(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
+                         int hidden, float *normed_out, float *logits);
+
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out);
 
 } // namespace bmk

@@ -26,6 +26,13 @@ __device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
     return __hiloint2double(hi, lo);
 }
 
+// The larger of two (high, low) keys into the first.
+__device__ __forceinline__ void key_max(u32 &hi, u32 &lo, u32 ohi, u32 olo) {
+    const bool take = ohi > hi || (ohi == hi && olo > lo);
+    hi = take ? ohi : hi;
+    lo = take ? olo : lo;
+}
+
 // One wave a token; lane L owns experts L + 64 j, j < PER.
 template <int PER>
 __global__ __launch_bounds__(256) void k_route_softmax(const float *logits, u32 n_tok, u32 n_exp, u32 used, u32 renorm,
@@ -77,25 +84,27 @@ __global__ __launch_bounds__(256) void k_route_softmax(const float *logits, u32 
     double chosen = 0.0;
     float mine = 0.0f;
     for (u32 s = 0; s < used; s++) {
-        float bv = -INFINITY;
-        u32 bi = 0xffffffffu;
+        // the order as one unsigned key: a probability's bits (not negative, so ordered as its value) over the
+        // complement of the id; none left: key 0, which reads back as id 0xffffffff
+        u32 khi = 0, klo = 0;
 #pragma unroll
         for (int j = 0; j < PER; j++) {
             const u32 e = lane + 64 * j;
-            if (e < n_exp && !((taken >> j) & 1u) && p[j] > bv) { // strict: a lane's ids ascend with j
-                bv = p[j];
-                bi = e;
-            }
+            if (e < n_exp && !((taken >> j) & 1u)) key_max(khi, klo, bm_f32_bits(p[j]), 0xffffffffu - e);
         }
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ov = __shfl_xor(bv, off);
-            const u32 oi = (u32)__shfl_xor((int)bi, off);
-            if (ov > bv || (ov == bv && oi < bi)) {
-                bv = ov;
-                bi = oi;
-            }
-        }
+        // the wave's maximum: four exchanges inside each row of sixteen lanes, one between the rows of a half, the two
+        // halves through their first lanes
+        key_max(khi, klo, bm_dpp<kDppXor1>(khi), bm_dpp<kDppXor1>(klo));
+        key_max(khi, klo, bm_dpp<kDppXor2>(khi), bm_dpp<kDppXor2>(klo));
+        key_max(khi, klo, bm_dpp<kDppHalfMirror>(khi), bm_dpp<kDppHalfMirror>(klo));
+        key_max(khi, klo, bm_dpp<kDppMirror>(khi), bm_dpp<kDppMirror>(klo));
+        key_max(khi, klo, bm_swap16(khi), bm_swap16(klo));
+        const u32 h0 = (u32)__builtin_amdgcn_readlane((int)khi, 0), l0 = (u32)__builtin_amdgcn_readlane((int)klo, 0);
+        const u32 h1 = (u32)__builtin_amdgcn_readlane((int)khi, 32), l1 = (u32)__builtin_amdgcn_readlane((int)klo, 32);
+        khi = h0, klo = l0;
+        key_max(khi, klo, h1, l1);
+        const float bv = bm_bits_f32(khi);
+        const u32 bi = 0xffffffffu - klo;
         if ((bi & 63u) == lane && bi != 0xffffffffu) taken |= 1u << (bi >> 6);
         if (lane == 0) ids[(size_t)t * used + s] = bi;
         chosen += (double)bv;
@@ -116,6 +125,156 @@ hipError_t route_softmax(const Launch &L, const float *logits, int n_tok, int n_
     else
         hipLaunchKernelGGL(k_route_softmax<16>, grid, block, 0, L.stream, logits, (u32)n_tok, (u32)n_exp, (u32)used,
                            (u32)renorm, probs, ids, weights, L.fault, L.layer);
+    return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------- the norm and the router's logits
+
+// The FFN norm and the router's f32 logits of m tokens (crates/gpu/src/route_softmax.rs:1667-1674 enqueue_norm_fused does
+// norm, quantizer and routing in one launch; here the norm and the logits are this launch, the routing
+// k_route_softmax's, and the quantizer is folded into the expert launches). Numbers, op for op: the norm
+// (crates/model/src/ops.rs:350-368) sums the f32 squares in f64 - lane by lane and then over the lanes; any order gives
+// the same f32 mean except on an exact tie of that rounding, as the reference notes of its own two orders - narrows the
+// mean to f32, takes scale = 1 / sqrt(mean + eps) and writes (scale * gain) * x; a logit is the f32 row dot of
+// crates/qdot/src/lib.rs:11349-11386: eight lane accumulators (a product, then fused multiply-adds in increasing k) and
+// (l0 + l4 + l2 + l6) + (l1 + l5 + l3 + l7).
+//
+// A workgroup takes one token and R router rows: the token's row is normed into LDS by all 256 threads while the rows'
+// bytes arrive (both requested at once), then eight lanes a row walk it, lane l the accumulator l.
+template <int R>
+__global__ __launch_bounds__(256) void k_router_logits(const float *router, const float *x, const float *gain, float eps,
+                                                       int n_exp, int hidden, float *normed_out, float *logits) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    float *xs = reinterpret_cast<float *>(lds);  // [hidden]
+    float *ws = xs + hidden;                     // [R][hidden + 8]: rows eight banks apart, the R x 8 readers on 8 R banks
+    __shared__ double s_part[4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int blocks_per_token = (n_exp + R - 1) / R;
+    const int t = blockIdx.x / blocks_per_token, e0 = (blockIdx.x % blocks_per_token) * R;
+    const float *xt = x + (size_t)t * hidden;
+    // the rows' bytes on their way first: they do not depend on the norm
+    const int n4 = hidden / 4;
+    for (int i = tid; i < R * n4; i += 256) {
+        const int r = i / n4, c = i % n4;
+        const int e = e0 + r < n_exp ? e0 + r : n_exp - 1;
+        reinterpret_cast<float4 *>(ws + (size_t)r * (hidden + 8))[c] = reinterpret_cast<const float4 *>(router + (size_t)e * hidden)[c];
+    }
+    double sum = 0.0;
+    constexpr int kInRegs = 8; // float4s of the row a thread can hold: rows of up to 8192 values stay in registers
+    if (gain && n4 <= 256 * kInRegs) {
+        // the row and the gain requested together and kept in registers: one pass, no second wait on memory
+        float4 xv[kInRegs], gv[kInRegs];
+#pragma unroll
+        for (int j = 0; j < kInRegs; j++) {
+            const int i = tid + 256 * j;
+            if (i < n4) {
+                xv[j] = reinterpret_cast<const float4 *>(xt)[i];
+                gv[j] = reinterpret_cast<const float4 *>(gain)[i];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kInRegs; j++)
+            if (tid + 256 * j < n4) {
+                sum += (double)__fmul_rn(xv[j].x, xv[j].x);
+                sum += (double)__fmul_rn(xv[j].y, xv[j].y);
+                sum += (double)__fmul_rn(xv[j].z, xv[j].z);
+                sum += (double)__fmul_rn(xv[j].w, xv[j].w);
+            }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) sum += shfl_xor_f64(sum, off);
+        if (lane == 0) s_part[wave] = sum;
+        __syncthreads();
+        const double total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+        const float mean = (float)(total / (double)hidden);
+        const float scale = __fdiv_rn(1.0f, bm_sqrt_rn(__fadd_rn(mean, eps)));
+#pragma unroll
+        for (int j = 0; j < kInRegs; j++) {
+            const int i = tid + 256 * j;
+            if (i < n4) {
+                const float4 v = make_float4(__fmul_rn(__fmul_rn(scale, gv[j].x), xv[j].x), __fmul_rn(__fmul_rn(scale, gv[j].y), xv[j].y),
+                                             __fmul_rn(__fmul_rn(scale, gv[j].z), xv[j].z), __fmul_rn(__fmul_rn(scale, gv[j].w), xv[j].w));
+                reinterpret_cast<float4 *>(xs)[i] = v;
+                if (normed_out && e0 == 0) reinterpret_cast<float4 *>(normed_out + (size_t)t * hidden)[i] = v;
+            }
+        }
+    } else {
+        for (int i = tid; i < n4; i += 256) {
+            const float4 v = reinterpret_cast<const float4 *>(xt)[i];
+            reinterpret_cast<float4 *>(xs)[i] = v;
+            if (gain) {
+                sum += (double)__fmul_rn(v.x, v.x);
+                sum += (double)__fmul_rn(v.y, v.y);
+                sum += (double)__fmul_rn(v.z, v.z);
+                sum += (double)__fmul_rn(v.w, v.w);
+            }
+        }
+        if (gain) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) sum += shfl_xor_f64(sum, off);
+            if (lane == 0) s_part[wave] = sum;
+            __syncthreads();
+            const double total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+            const float mean = (float)(total / (double)hidden);
+            const float scale = __fdiv_rn(1.0f, bm_sqrt_rn(__fadd_rn(mean, eps)));
+            for (int i = tid; i < hidden; i += 256) {
+                const float v = __fmul_rn(__fmul_rn(scale, gain[i]), xs[i]); // written before the barrier above
+                xs[i] = v;
+                if (normed_out && e0 == 0) normed_out[(size_t)t * hidden + i] = v;
+            }
+        }
+    }
+    __syncthreads();
+    if (!gain && normed_out && e0 == 0) // the rows as they are (read after the barrier: other threads staged them)
+        for (int i = tid; i < hidden; i += 256) normed_out[(size_t)t * hidden + i] = xs[i];
+    if (tid >= 8 * R) return;
+    const int r = tid >> 3, l = tid & 7;
+    const float *wr = ws + (size_t)r * (hidden + 8);
+    float acc = __fmul_rn(xs[l], wr[l]);
+    // the chain is serial by the order's definition; the reads are not: sixteen steps' operands a batch
+    const int steps = hidden / 8;
+    int i = 1;
+    for (; i + 16 <= steps; i += 16) {
+        float a[16], b[16];
+#pragma unroll
+        for (int u = 0; u < 16; u++) a[u] = xs[8 * (i + u) + l], b[u] = wr[8 * (i + u) + l];
+#pragma unroll
+        for (int u = 0; u < 16; u++) acc = fmaf(a[u], b[u], acc);
+    }
+    for (; i < steps; i++) acc = fmaf(xs[8 * i + l], wr[8 * i + l], acc);
+    // s_l = acc_l + acc_{l+4} on lanes 0..3 of the row's eight, then (s0 + s2) + (s1 + s3)
+    const float s = __fadd_rn(acc, __shfl_down(acc, 4, 8));
+    const float pair = __fadd_rn(s, __shfl_down(s, 2, 8)); // lane 0: s0 + s2, lane 1: s1 + s3
+    const float out = __fadd_rn(pair, __shfl_down(pair, 1, 8));
+    if (l == 0 && e0 + r < n_exp) logits[(size_t)t * n_exp + e0 + r] = out;
+}
+
+// Rows a workgroup takes: four where they fit the LDS beside the token's row, else two, else one.
+static int router_rows(int hidden) {
+    for (int r = 4; r >= 1; r >>= 1)
+        if (((size_t)(r + 1) * hidden + 8 * r) * sizeof(float) <= (size_t)kMaxLds - 1024) return r;
+    return 0;
+}
+
+bool router_logits_fits(int hidden) { return router_rows(hidden) > 0; }
+
+hipError_t router_logits(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
+                         int hidden, float *normed_out, float *logits) {
+    const int rows = router_rows(hidden);
+    if (rows == 0) return hipErrorInvalidValue;
+    const size_t lds = ((size_t)(rows + 1) * hidden + 8 * rows) * sizeof(float);
+    const unsigned grid = (unsigned)m * (unsigned)((n_exp + rows - 1) / rows);
+#define BM_RL(R)                                                                                                       \
+    {                                                                                                                  \
+        auto kern = k_router_logits<R>;                                                                                \
+        hipError_t e = allow_lds(kern, lds);                                                                           \
+        if (e != hipSuccess) return e;                                                                                 \
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, router, x, gain, eps, n_exp, hidden, normed_out, \
+                           logits);                                                                                    \
+    }
+    if (rows == 4) BM_RL(4)
+    else if (rows == 2) BM_RL(2)
+    else BM_RL(1)
+#undef BM_RL
     return hipGetLastError();
 }
 

@@ -309,6 +309,17 @@ int bm_set_gate_rule(bm_ctx *ctx, int rule, float limit);
  * NaN probabilities and weights, and keeps its ids as they stand. */
 int bm_route_softmax(bm_ctx *ctx, const float *logits_dev, int n_tokens, int n_experts, int top_k, int renorm,
                      float *probs_dev, uint32_t *ids_dev, float *weights_dev);
+/* The FFN norm and the router's logits, the step before bm_route_softmax (RouterKernels::enqueue_norm_fused,
+ * crates/gpu/src/route_softmax.rs:1667-1674, does norm, quantizer and routing in one launch; here: this launch, then
+ * bm_route_softmax, and the quantizer rides in bm_moe_decode / bm_gate_up_x over normed_dev). In the CPU path's numbers:
+ * normed[t] = (scale * gain) * x[t] with scale = 1 / sqrt(mean of squares + eps), the squares summed in f64 and the mean
+ * narrowed to f32 (crates/model/src/ops.rs:350-368); logits[t * n_experts + e] = router row e . normed[t] in
+ * qdot::dot_f32's eight-lane order (crates/qdot/src/lib.rs:11349-11386). gain_dev NULL: no norm, the rows are dotted as
+ * they are. router_dev: n_experts rows of hidden f32, x_dev: n_tokens rows; hidden a multiple of 8; normed_dev
+ * (optional) receives the normed rows; every pointer 16-byte aligned. */
+int bm_router_logits(bm_ctx *ctx, const float *router_dev, const float *x_dev, const float *gain_dev, float eps, int n_tokens,
+                     int n_experts, int hidden, float *normed_dev, float *logits_dev);
+
 
 /* ------------------------------------------------------------------------------------------- model files */
 

@@ -101,6 +101,14 @@ typedef struct {
 int ora_moe_forward(const ora_moe_layer *L, const float *x, int m, const uint32_t *ids, const float *wts, int top_k,
                     float *y, float *h_out, int n_threads);
 
+// The step before the path: the FFN norm and the router's f32 logits (crates/model/src/ops.rs:350-368,
+// crates/qdot/src/lib.rs:11349-11456).
+double ora_sum_sq_f64(const float *x, int n);
+void ora_rms_norm(const float *x, const float *gain, float eps, int n, float *out);
+int ora_dot_f32(const float *w, const float *x, int n, float *out);
+int ora_router_logits(const float *router, int n_experts, int hidden, const float *x, const float *gain, float eps, int m,
+                      float *normed_out, float *logits);
+
 #ifdef __cplusplus
 }
 #endif

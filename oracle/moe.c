@@ -169,3 +169,74 @@ int ora_moe_forward(const ora_moe_layer *L, const float *x, int m, const uint32_
     free(down);
     return rc;
 }
+
+// ------------------------------------------------------------------------------- the norm and the router's logits
+
+// sum of (x[i] * x[i]) as f64, f32 squares, in the vector kernel's lane order (crates/qdot/src/lib.rs:11418-11456): two
+// registers of four f64 lanes take values 8i .. 8i + 3 and 8i + 4 .. 8i + 7, are added lane by lane, the upper pair
+// onto the lower, then the two; a tail past the last eight is added left to right.
+double ora_sum_sq_f64(const float *x, int n) {
+    double a0[4] = {0, 0, 0, 0}, a1[4] = {0, 0, 0, 0};
+    int full = n / 8 * 8;
+    for (int i = 0; i < full; i += 8)
+        for (int l = 0; l < 4; l++) {
+            float s0 = x[i + l] * x[i + l], s1 = x[i + 4 + l] * x[i + 4 + l];
+            a0[l] += (double)s0;
+            a1[l] += (double)s1;
+        }
+    double a[4], lo[2];
+    for (int l = 0; l < 4; l++) a[l] = a0[l] + a1[l];
+    lo[0] = a[0] + a[2];
+    lo[1] = a[1] + a[3];
+    double total = lo[0] + lo[1];
+    for (int i = full; i < n; i++) {
+        float s = x[i] * x[i];
+        total += (double)s;
+    }
+    return total;
+}
+
+// RMS norm with a gain (crates/model/src/ops.rs:350-368): the mean of the squares narrowed to f32, eps inside the
+// square root, then (scale * gain) * x in that order.
+void ora_rms_norm(const float *x, const float *gain, float eps, int n, float *out) {
+    float mean = (float)(ora_sum_sq_f64(x, n) / (double)n);
+    float scale = 1.0f / sqrtf(mean + eps);
+    for (int i = 0; i < n; i++) {
+        float sg = scale * gain[i];
+        out[i] = sg * x[i];
+    }
+}
+
+// One f32 weight row . an f32 column in the reference's float-kernel order (crates/qdot/src/lib.rs:11349-11386): eight
+// lane accumulators, the first block a product, every later one a fused multiply-add, then (l0 + l4 + l2 + l6) +
+// (l1 + l5 + l3 + l7). n a positive multiple of eight (the reference hands other widths back to its caller).
+int ora_dot_f32(const float *w, const float *x, int n, float *out) {
+    if (n <= 0 || n % 8 != 0) return ORA_EUNALIGNED;
+    float acc[8];
+    for (int l = 0; l < 8; l++) acc[l] = x[l] * w[l];
+    for (int i = 1; i < n / 8; i++)
+        for (int l = 0; l < 8; l++) acc[l] = fmaf(x[8 * i + l], w[8 * i + l], acc[l]);
+    float s[4] = {acc[0] + acc[4], acc[1] + acc[5], acc[2] + acc[6], acc[3] + acc[7]};
+    *out = (s[0] + s[2]) + (s[1] + s[3]);
+    return 0;
+}
+
+// The router's logits of m tokens (crates/model/src/moe.rs:246: matmul_q over the f32 gate_inp rows): logits[t *
+// n_experts + e] = row e . token t's row, after the norm when a gain is given.
+int ora_router_logits(const float *router, int n_experts, int hidden, const float *x, const float *gain, float eps, int m,
+                      float *normed_out, float *logits) {
+    float *row = (float *)malloc(sizeof(float) * (size_t)hidden);
+    int rc = 0;
+    for (int t = 0; t < m && !rc; t++) {
+        const float *xt = x + (size_t)t * hidden;
+        if (gain)
+            ora_rms_norm(xt, gain, eps, hidden, row);
+        else
+            memcpy(row, xt, sizeof(float) * (size_t)hidden);
+        if (normed_out) memcpy(normed_out + (size_t)t * hidden, row, sizeof(float) * (size_t)hidden);
+        for (int e = 0; e < n_experts && !rc; e++)
+            rc = ora_dot_f32(router + (size_t)e * hidden, row, hidden, &logits[(size_t)t * n_experts + e]);
+    }
+    free(row);
+    return rc;
+}

@@ -59,6 +59,11 @@ def _load():
         "ora_expf_ik": (C.c_float, [C.c_float]),
         "ora_swiglu": (None, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
         "ora_gate_rule": (C.c_int, [C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_sum_sq_f64": (C.c_double, [C.c_void_p, C.c_int]),
+        "ora_rms_norm": (None, [C.c_void_p, C.c_void_p, C.c_float, C.c_int, C.c_void_p]),
+        "ora_dot_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_router_logits": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_float, C.c_int, C.c_void_p,
+                                        C.c_void_p]),
         "ora_route_softmax_topk": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
         "ora_combine_tokens": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
         "ora_moe_combine": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
@@ -361,3 +366,35 @@ def moe_forward(hidden, ff, n_experts, types, wg, wu, wd, x, ids, wts, top_k, n_
         rc = lib.ora_moe_forward(C.byref(L), _p(x), m, _p(ids), _p(wts), top_k, _p(y), hp, n_threads)
     _check(rc)
     return (y, h) if want_h else y
+
+
+def sum_sq_f64(x):
+    x = np.ascontiguousarray(x, np.float32)
+    return float(lib.ora_sum_sq_f64(_p(x), x.size))
+
+
+def rms_norm(x, gain, eps):
+    x, gain = np.ascontiguousarray(x, np.float32), np.ascontiguousarray(gain, np.float32)
+    out = np.empty(x.size, np.float32)
+    lib.ora_rms_norm(_p(x), _p(gain), float(eps), x.size, _p(out))
+    return out
+
+
+def dot_f32(w, x):
+    w, x = np.ascontiguousarray(w, np.float32), np.ascontiguousarray(x, np.float32)
+    out = np.empty(1, np.float32)
+    _check(lib.ora_dot_f32(_p(w), _p(x), x.size, _p(out)))
+    return out[0]
+
+
+def router_logits(router, x, gain=None, eps=0.0):
+    """(normed rows, logits) of the tokens x[m, hidden] against the f32 router rows router[n_experts, hidden]."""
+    router, x = np.ascontiguousarray(router, np.float32), np.ascontiguousarray(x, np.float32)
+    n_experts, hidden = router.shape
+    m = x.size // hidden
+    g = None if gain is None else np.ascontiguousarray(gain, np.float32)
+    normed = np.empty((m, hidden), np.float32)
+    logits = np.empty((m, n_experts), np.float32)
+    _check(lib.ora_router_logits(_p(router), n_experts, hidden, _p(x), _p(g) if g is not None else None, float(eps), m,
+                                 _p(normed), _p(logits)))
+    return normed, logits

@@ -139,3 +139,69 @@ def test_router_refusals_are_named(gpu):
         assert e.value.code == bm.ESHAPE and word in str(e.value) and "bm_route_softmax" in str(e.value)
     buf.free()
     ids.free()
+
+
+# ------------------------------------------------------------------------- the norm and the router's logits
+
+@pytest.mark.parametrize("n_experts,hidden,m,with_gain,seed", ((128, 2048, 5, True, 11), (256, 7168, 2, True, 12),
+                                                               (128, 2048, 3, False, 13), (10, 64, 4, True, 14),
+                                                               (7, 16384, 1, True, 15), (3, 64, 2000, True, 16)))
+def test_router_logits_are_the_cpu_paths(gpu, n_experts, hidden, m, with_gain, seed):
+    """bm_router_logits: the normed rows and the f32 logits bit for bit against the oracle's restatement of the CPU
+    path's norm (crates/model/src/ops.rs:350-368) and eight-lane f32 row dot (crates/qdot/src/lib.rs:11349-11386).
+    Shapes: the two benchmark layers', rows that are not a whole number of a workgroup's four, a row so long that a
+    workgroup takes one router row at a time, and two thousand short rows for as many square roots (the hardware's is
+    not the correctly rounded one)."""
+    rng = np.random.default_rng(seed)
+    router = normal_f32(rng, (n_experts, hidden), 0.05)
+    x = np.stack([normal_f32(rng, hidden) * np.float32(10.0 ** rng.uniform(-2, 2)) for _ in range(m)])
+    gain = (1.0 + normal_f32(rng, hidden, 0.2)).astype(np.float32) if with_gain else None
+    eps = 1e-6
+    rd, xd = gpu.upload(router, np.float32), gpu.upload(x, np.float32)
+    gd = gpu.upload(gain, np.float32) if with_gain else None
+    normed = gpu.buffer(np.float32, m * hidden).fill_bytes(0xFF)
+    logits = gpu.buffer(np.float32, m * n_experts).fill_bytes(0xFF)
+    gpu.enqueue_router_logits(rd, xd, gd, eps, m, n_experts, hidden, normed, logits)
+    want_n, want_l = ora.router_logits(router, x, gain, eps)
+    assert_f32(normed.download(), want_n.reshape(-1), "normed rows")
+    assert_f32(logits.download(), want_l.reshape(-1), "logits")
+    # without the normed rows the logits are the same
+    logits.fill_bytes(0xFF)
+    gpu.enqueue_router_logits(rd, xd, gd, eps, m, n_experts, hidden, None, logits)
+    assert np.array_equal(logits.download().view(np.uint32), want_l.reshape(-1).view(np.uint32))
+    for b in (rd, xd, gd, normed, logits):
+        if b is not None:
+            b.free()
+
+
+def test_layer_from_the_residual_row(gpu):
+    """The layer from its input residual rows: norm and logits, routing, then the fused expert step on the normed rows,
+    four launches, nothing through the host. The ids are the oracle's; with the kernel's own weights (within two units
+    in the last place of the oracle's, see above) the layer's output is the oracle's bit for bit."""
+    hidden, ff, n_experts, top_k, m = 2048, 768, 16, 4, 6
+    L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), hidden, ff, n_experts, 4400)
+    rng = np.random.default_rng(4401)
+    router = normal_f32(rng, (n_experts, hidden), 0.05)
+    gain = (1.0 + normal_f32(rng, hidden, 0.1)).astype(np.float32)
+    x = normal_f32(rng, (m, hidden), 2.0)
+    rd, xd, gd = gpu.upload(router, np.float32), gpu.upload(x, np.float32), gpu.upload(gain, np.float32)
+    normed, logits = gpu.buffer(np.float32, m * hidden), gpu.buffer(np.float32, m * n_experts)
+    ids, wts = gpu.buffer(np.uint32, m * top_k), gpu.buffer(np.float32, m * top_k)
+    act_h, y = gpu.act(bm.Q6_K, ff, m * top_k), gpu.buffer(np.float32, m * hidden).fill_bytes(0xFF)
+    gpu.fault_clear()
+    gpu.set_decode_plan(bm.PLAN_TWO_LAUNCHES)
+    gpu.enqueue_router_logits(rd, xd, gd, 1e-6, m, n_experts, hidden, normed, logits)
+    gpu.enqueue_route_softmax(logits, m, n_experts, top_k, True, None, ids, wts)
+    gpu.enqueue_moe_decode(L.dg, L.du, L.dd, normed, ids, wts, xd, top_k, m, act_h, y)   # the residual: the input rows
+    want_n, want_l = ora.router_logits(router, x, gain, 1e-6)
+    got_ids, got_w = ids.download().reshape(m, top_k), wts.download().reshape(m, top_k)
+    for t in range(m):
+        want_ids, want_w = ora.route_softmax_topk(want_l[t], top_k)
+        assert list(got_ids[t]) == list(want_ids)
+        assert_ulp(got_w[t], want_w, f"weights of token {t}", odd_share=1.0)
+    want_y, _ = L.oracle(want_n, got_ids, got_w, top_k)
+    assert_f32(y.download(), (want_y.reshape(m, hidden) + x).astype(np.float32).reshape(-1), "y + residual")
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    for b in (rd, xd, gd, normed, logits, ids, wts, act_h, y):
+        b.free()
+    L.free()

@@ -338,3 +338,69 @@ def test_gemm_route_by_hand():
     assert tiles.tolist() == [[0, 0, 2], [1, 2, 3]]
     cols, tiles, refused = ora.gemm_route([2] * 130, 3)
     assert tiles.tolist() == [[2, 0, 64], [2, 64, 64], [2, 128, 2]] and refused == 0
+
+
+# ------------------------------------------------------------------------- the norm and the router's logits
+
+def fma32(a, b, c):
+    """a * b + c rounded once to f32, exactly: the sum as a fraction, then the nearest of the f32 values around it
+    (ties to the even mantissa)."""
+    from fractions import Fraction
+    r = Fraction(float(a)) * Fraction(float(b)) + Fraction(float(c))
+    near = np.float32(float(r))
+    best = None
+    for cand in (np.nextafter(near, np.float32(-np.inf)), near, np.nextafter(near, np.float32(np.inf))):
+        dist = abs(Fraction(float(cand)) - r)
+        even = (int(np.float32(cand).view(np.uint32)) & 1) == 0
+        if best is None or dist < best[0] or (dist == best[0] and even and not best[2]):
+            best = (dist, cand, even)
+    return np.float32(best[1])
+
+
+def test_sum_of_squares_narrows_to_the_sequential_sum():
+    # crates/qdot/tests/qdot.rs:4438-4455: the laned f64 sum against the left-to-right one, on its generator
+    for n in (8, 512, 2048, 2048 + 5):
+        x = ((np.arange(n) * 37 % 2001).astype(np.float32) - np.float32(1000.0)) * np.float32(0.0137)
+        seq = 0.0
+        for v in x:
+            seq += float(np.float32(v * v))
+        got = ora.sum_sq_f64(x)
+        assert abs((got - seq) / seq) < 1e-14
+        assert np.float32(got / n).tobytes() == np.float32(seq / n).tobytes()
+
+
+def test_f32_row_dot_is_the_eight_lane_order():
+    # crates/qdot/tests/qdot.rs:4460-4485, on its generators; the lanes re-derived with an exact fused multiply-add
+    k = 2048
+    w = ((np.arange(k) * 37 % 2001).astype(np.float32) - np.float32(1000.0)) * np.float32(0.0013)
+    x = ((np.arange(k) * 91 % 1777).astype(np.float32) - np.float32(888.0)) * np.float32(0.0071)
+    lane = [np.float32(x[l] * w[l]) for l in range(8)]
+    for i in range(1, k // 8):
+        for l in range(8):
+            lane[l] = fma32(x[8 * i + l], w[8 * i + l], lane[l])
+    s = [np.float32(lane[l] + lane[l + 4]) for l in range(4)]
+    want = np.float32(np.float32(s[0] + s[2]) + np.float32(s[1] + s[3]))
+    assert ora.dot_f32(w, x).tobytes() == want.tobytes()
+    with pytest.raises(ora.OracleError) as e:
+        ora.dot_f32(w[:12], x[:12])  # a width the lanes cannot take is the caller's
+    assert e.value.code == ora.EUNALIGNED
+
+
+def test_rms_norm_is_the_stated_formula():
+    # crates/model/src/ops.rs:350-368: mean of squares narrowed to f32, eps inside the root, (scale * gain) * x
+    rng = np.random.default_rng(91)
+    for n, eps in ((256, 1e-6), (2048, 1e-5), (7168, 1e-6)):
+        x, gain = normal_f32(rng, n, 3.0), normal_f32(rng, n, 1.0)
+        mean = np.float32(np.sum(np.float32(x * x).astype(np.float64)) / n)
+        scale = np.float32(1.0) / np.sqrt(np.float32(mean + np.float32(eps)), dtype=np.float32)
+        want = (np.float32(scale) * gain).astype(np.float32) * x
+        assert ora.rms_norm(x, gain, eps).tobytes() == want.astype(np.float32).tobytes()
+    router = normal_f32(rng, (5, 64), 0.1)
+    xs = normal_f32(rng, (3, 64))
+    gain = normal_f32(rng, 64)
+    normed, logits = ora.router_logits(router, xs, gain, 1e-6)
+    for t in range(3):
+        assert normed[t].tobytes() == ora.rms_norm(xs[t], gain, 1e-6).tobytes()
+        assert [ora.dot_f32(router[e], normed[t]).tobytes() for e in range(5)] == [logits[t, e].tobytes() for e in range(5)]
+    plain, logits0 = ora.router_logits(router, xs)
+    assert plain.tobytes() == xs.tobytes() and logits0[1, 2] == ora.dot_f32(router[2], xs[1])

@@ -85,6 +85,7 @@ SYMBOLS = {
     "bm_route_softmax": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "bm_router_logits": (_i, [_vp, _vp, _vp, _vp, C.c_float, _i, _i, _i, _vp, _vp]),
     "bm_gguf_open": (_i, [C.c_char_p, C.POINTER(_vp)]),
+    "bm_gguf_open_split": (_i, [C.c_char_p, C.POINTER(_vp)]),
     "bm_gguf_close": (None, [_vp]),
     "bm_gguf_last_error": (C.c_char_p, []),
     "bm_gguf_version": (_i, [_vp]),
@@ -210,12 +211,13 @@ class _GgufTensor(C.Structure):
 
 class Gguf:
     """A model file's header and mapping (crates/gguf/src/lib.rs Gguf): tensors by name, key-values, and a tensor as a
-    weight stack on a Gpu. Host code: opening and reading need no GPU."""
+    weight stack on a Gpu. Host code: opening and reading need no GPU. With split=True the path is a model's first
+    shard and the object answers for the whole split set (crates/gguf/src/lib.rs Split)."""
 
-    def __init__(self, path):
+    def __init__(self, path, split=False):
         self.lib = load_library()
         h = _vp()
-        rc = self.lib.bm_gguf_open(os.fsencode(path), C.byref(h))
+        rc = (self.lib.bm_gguf_open_split if split else self.lib.bm_gguf_open)(os.fsencode(path), C.byref(h))
         if rc:
             raise GpuError(rc, self.lib.bm_gguf_last_error().decode())
         self.handle = h.value

@@ -135,6 +135,7 @@ struct bm_gguf {
     std::vector<bm_gguf_tensor> tensors;
     std::vector<std::string> names;
     std::unordered_map<std::string, size_t> by_name;
+    std::vector<bm_gguf *> more; // the other shards of a split set, owned by the first
 };
 
 extern "C" {
@@ -143,13 +144,16 @@ const char *bm_gguf_last_error(void) { return g_gguf_err.c_str(); }
 
 void bm_gguf_close(bm_gguf *g) {
     if (!g) return;
+    for (bm_gguf *shard : g->more) bm_gguf_close(shard);
     if (g->map) munmap(const_cast<uint8_t *>(g->map), (size_t)g->len);
     if (g->fd >= 0) close(g->fd);
     delete g;
 }
 
-int bm_gguf_open(const char *path, bm_gguf **out) {
-    if (!path || !out) return refuse(BM_EARG, "bm_gguf_open: NULL argument");
+} // extern "C"
+
+// One file.
+static int open_one(const char *path, bm_gguf **out) {
     *out = nullptr;
     bm_gguf *g = new (std::nothrow) bm_gguf;
     if (!g) return refuse(BM_EDRIVER, "bm_gguf_open: out of host memory");
@@ -253,6 +257,114 @@ int bm_gguf_open(const char *path, bm_gguf **out) {
                                (unsigned long long)t.nbytes, (unsigned long long)g->data_base, (unsigned long long)t.offset,
                                (unsigned long long)g->len));
         t.data = t.nbytes ? g->map + start : nullptr;
+    }
+    *out = g;
+    return BM_OK;
+}
+
+static const Value *value_of(const bm_gguf *g, const char *key);
+
+// A split key as a count (llama.cpp's splitter writes split.no and split.count as u16, split.tensors.count as i32).
+static bool split_count(const bm_gguf *g, const char *key, uint64_t *out) {
+    const Value *v = value_of(g, key);
+    if (!v) return false;
+    switch (v->type) {
+    case 0: case 2: case 4: case 10: // u8, u16, u32, u64
+        *out = v->bits;
+        return true;
+    case 1: case 3: case 5: case 11: { // i8, i16, i32, i64: a count is not negative
+        const uint64_t sz = scalar_size(v->type);
+        const int64_t sv = (int64_t)(v->bits << (64 - 8 * sz)) >> (64 - 8 * sz);
+        if (sv < 0) return false;
+        *out = (uint64_t)sv;
+        return true;
+    }
+    default:
+        return false;
+    }
+}
+
+extern "C" {
+
+// One file, whatever split keys it holds (crates/gguf/src/lib.rs:359 Gguf::open_split_shard reads one shard so).
+int bm_gguf_open(const char *path, bm_gguf **out) {
+    if (!path || !out) return refuse(BM_EARG, "bm_gguf_open: NULL argument");
+    return open_one(path, out);
+}
+
+// A model as one file or as llama.cpp's split set named by its first shard (crates/gguf/src/lib.rs:835-875
+// Split::open_model): a file without split.count is a set of one. Otherwise split.count is a count above 0, the first
+// file's split.no is 0, a set of several is named <prefix>-00001-of-%05d.gguf and its siblings
+// <prefix>-%05d-of-%05d.gguf all open, every shard's split.no is its place, every split.count agrees, the shards'
+// tensor counts sum to the first shard's split.tensors.count and no tensor name appears twice, or the set is refused.
+// The metadata is the first shard's: the splitter writes the model's keys there alone.
+int bm_gguf_open_split(const char *first, bm_gguf **out) {
+    if (!first || !out) return refuse(BM_EARG, "bm_gguf_open_split: NULL argument");
+    bm_gguf *g = nullptr;
+    int rc = open_one(first, &g);
+    *out = nullptr;
+    if (rc) return rc;
+    if (!value_of(g, "split.count")) {
+        *out = g;
+        return BM_OK;
+    }
+    auto fail = [&](int code) {
+        bm_gguf_close(g);
+        return code;
+    };
+    auto place_of = [&](const bm_gguf *shard, const char *path, uint64_t place) {
+        uint64_t no = 0;
+        if (!split_count(shard, "split.no", &no)) return refuse(BM_ESHAPE, "bm_gguf_open_split: %s: split.no is absent or not a count", path);
+        if (no != place)
+            return refuse(BM_ESHAPE, "bm_gguf_open_split: %s: split.no is %llu, but the file is shard %llu of its set (from 0)", path,
+                          (unsigned long long)no, (unsigned long long)place);
+        return (int)BM_OK;
+    };
+    uint64_t count = 0;
+    if (!split_count(g, "split.count", &count) || count == 0 || count > 99999)
+        return fail(refuse(BM_ESHAPE, "bm_gguf_open_split: %s: split.count is not a count from 1 to 99999", first));
+    if ((rc = place_of(g, first, 0)) != BM_OK) return fail(rc);
+    uint64_t seen = g->tensors.size();
+    if (count > 1) {
+        char suffix[32];
+        snprintf(suffix, sizeof suffix, "-%05d-of-%05d.gguf", 1, (int)count);
+        const std::string name(first);
+        const size_t ns = strlen(suffix);
+        if (name.size() <= ns || name.compare(name.size() - ns, ns, suffix) != 0)
+            return fail(refuse(BM_ESHAPE, "bm_gguf_open_split: %s holds split.count = %llu, but its name does not end in %s", first,
+                               (unsigned long long)count, suffix));
+        const std::string prefix = name.substr(0, name.size() - ns);
+        for (uint64_t i = 1; i < count; i++) {
+            snprintf(suffix, sizeof suffix, "-%05d-of-%05d.gguf", (int)i + 1, (int)count);
+            const std::string sib = prefix + suffix;
+            bm_gguf *shard = nullptr;
+            rc = open_one(sib.c_str(), &shard);
+            if (rc) {
+                const std::string why = g_gguf_err; // names the shard's file
+                return fail(refuse(rc, "bm_gguf_open_split: shard %llu of %llu: %s", (unsigned long long)i + 1, (unsigned long long)count, why.c_str()));
+            }
+            g->more.push_back(shard);
+            if ((rc = place_of(shard, sib.c_str(), i)) != BM_OK) return fail(rc);
+            uint64_t theirs = 0;
+            if (!split_count(shard, "split.count", &theirs) || theirs != count)
+                return fail(refuse(BM_ESHAPE, "bm_gguf_open_split: %s: split.count is not the first shard's %llu", sib.c_str(), (unsigned long long)count));
+            seen += shard->tensors.size();
+        }
+    }
+    uint64_t want = 0;
+    if (!split_count(g, "split.tensors.count", &want))
+        return fail(refuse(BM_ESHAPE, "bm_gguf_open_split: %s: split.tensors.count is absent or not a count", first));
+    if (seen != want)
+        return fail(refuse(BM_ESHAPE, "bm_gguf_open_split: %s: split.tensors.count is %llu, but the %llu shards hold %llu tensors", first,
+                           (unsigned long long)want, (unsigned long long)count, (unsigned long long)seen));
+    // the set's tensors behind the first shard's: an entry's name and data point into its own shard, which g owns
+    for (bm_gguf *shard : g->more) {
+        for (size_t t = 0; t < shard->tensors.size(); t++) {
+            const std::string &tn = shard->names[t];
+            if (g->by_name.count(tn)) return fail(refuse(BM_ESHAPE, "bm_gguf_open_split: tensor %s is in two shards of the set", tn.c_str()));
+            g->by_name.emplace(tn, g->tensors.size());
+            g->tensors.push_back(shard->tensors[t]);
+        }
     }
     *out = g;
     return BM_OK;

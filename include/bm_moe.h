@@ -339,6 +339,14 @@ typedef struct bm_gguf_tensor {
     const void *data;  /* the tensor's bytes in the mapping (valid until bm_gguf_close); NULL when nbytes is 0 */
 } bm_gguf_tensor;
 int bm_gguf_open(const char *path, bm_gguf **out);
+/* A model as one file or as llama.cpp's split set, opened by its first shard (crates/gguf/src/lib.rs:617-630 Split,
+ * :835-875 Split::open_model): a file without "split.count" is a set of one. The siblings of
+ * <prefix>-00001-of-%05d.gguf are <prefix>-%05d-of-%05d.gguf; every shard's "split.no" is its place (from 0), every
+ * "split.count" agrees, the shards' tensor counts sum to the first shard's "split.tensors.count" and no tensor name
+ * appears twice, or the set is refused with the file and key named. The handle then answers for the whole set: tensors
+ * in shard order, each one's offset and data within its own shard, key-values from the first shard (the splitter
+ * writes the model's keys there alone). bm_gguf_open on a shard reads that one file (Gguf::open_split_shard, :359). */
+int bm_gguf_open_split(const char *first_shard_path, bm_gguf **out);
 void bm_gguf_close(bm_gguf *g);
 const char *bm_gguf_last_error(void);
 int bm_gguf_version(const bm_gguf *g);

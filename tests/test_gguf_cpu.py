@@ -121,3 +121,120 @@ def test_a_bad_alignment_is_refused(tmp_path):
         with pytest.raises(bm.GpuError) as e:
             bm.Gguf(bad)
         assert "general.alignment" in str(e.value)
+
+
+# --- split sets (crates/gguf/src/lib.rs:835-875 Split::open_model; its own tests, :2290 on, write shards the same way)
+
+def shard_name(prefix, i, count):
+    return f"{prefix}-{i + 1:05d}-of-{count:05d}.gguf"
+
+
+def split_set(tmp_path, count=3, per=(2, 1, 3), prefix="model", edit=None):
+    """`count` shards with per[i] F32 tensors each; edit(i, kvs, tensors) may damage shard i's lists before writing.
+    The model's keys are in the first shard alone, as the splitter leaves them."""
+    rng = np.random.default_rng(11)
+    total, made, n = sum(per), {}, 0
+    for i in range(count):
+        kvs = [("split.no", gf.U16, i), ("split.count", gf.U16, count), ("split.tensors.count", gf.I32, total)]
+        if i == 0:
+            kvs = [("general.architecture", gf.STR, "qwen3moe"), ("qwen3moe.expert_count", gf.U32, 8)] + kvs
+        tensors = []
+        for _ in range(per[i]):
+            data = rng.standard_normal(32 * (n + 1)).astype(np.float32)
+            tensors.append((f"blk.{n}.w", [data.size], 0, data.view(np.uint8)))
+            n += 1
+        if edit:
+            edit(i, kvs, tensors)
+        gf.write(os.path.join(tmp_path, shard_name(prefix, i, count)), kvs, tensors)
+        made.update({t[0]: t[3] for t in tensors})
+    return os.path.join(tmp_path, shard_name(prefix, 0, count)), made
+
+
+def test_a_split_set_reads_as_one_model(tmp_path):
+    first, made = split_set(str(tmp_path))
+    g = bm.Gguf(first, split=True)
+    assert g.get_str("general.architecture") == "qwen3moe" and g.get_u64("qwen3moe.expert_count") == 8
+    assert [t["name"] for t in g.tensors()] == list(made)  # shard order, then each shard's own
+    for name, data in made.items():
+        assert np.array_equal(g.data(name), data) and g.find(name)["nbytes"] == data.size
+    g.close()
+    # one shard read alone is that file: its own tensors, no siblings
+    alone = bm.Gguf(os.path.join(str(tmp_path), shard_name("model", 1, 3)))
+    assert [t["name"] for t in alone.tensors()] == ["blk.2.w"] and alone.get_u64("split.no") == 1
+    alone.close()
+
+
+def test_a_file_without_split_keys_is_a_set_of_one(tmp_path):
+    path, tensors, _ = sample(str(tmp_path))
+    g = bm.Gguf(path, split=True)
+    assert [t["name"] for t in g.tensors()] == [t[0] for t in tensors]
+    g.close()
+    first, made = split_set(str(tmp_path), count=1, per=(2,), prefix="anyname")
+    g = bm.Gguf(first, split=True)  # split.count = 1: the name is free, the keys are still checked
+    assert len(g.tensors()) == 2
+    g.close()
+
+
+def set_kv(kvs, key, vtype, v):
+    at = [k for k, _, _ in kvs].index(key)
+    if v is None:
+        del kvs[at]
+    else:
+        kvs[at] = (key, vtype, v)
+
+
+@pytest.mark.parametrize("case,words", (
+    ("missing_shard", ("shard 3 of 3", "cannot open", "-00003-of-00003.gguf")),
+    ("wrong_no", ("-00002-of-00003.gguf", "split.no is 2", "shard 1")),
+    ("no_absent", ("-00003-of-00003.gguf", "split.no is absent")),
+    ("first_not_first", ("split.no is 1", "shard 0")),
+    ("count_differs", ("-00002-of-00003.gguf", "split.count is not the first shard's 3")),
+    ("count_zero", ("split.count is not a count",)),
+    ("count_a_string", ("split.count is not a count",)),
+    ("tensors_count", ("split.tensors.count is 7", "3 shards hold 6")),
+    ("tensors_absent", ("split.tensors.count is absent",)),
+    ("tensors_negative", ("split.tensors.count is absent or not a count",)),
+    ("duplicate", ("blk.0.w", "two shards")),
+    ("damaged_shard", ("shard 2 of 3", "does not start with GGUF")),
+))
+def test_a_broken_split_set_is_refused_by_name(tmp_path, case, words):
+    def edit(i, kvs, tensors):
+        if case == "wrong_no" and i == 1:
+            set_kv(kvs, "split.no", gf.U16, 2)
+        if case == "no_absent" and i == 2:
+            set_kv(kvs, "split.no", gf.U16, None)
+        if case == "first_not_first" and i == 0:
+            set_kv(kvs, "split.no", gf.U16, 1)
+        if case == "count_differs" and i == 1:
+            set_kv(kvs, "split.count", gf.U16, 4)
+        if case == "count_zero" and i == 0:
+            set_kv(kvs, "split.count", gf.U16, 0)
+        if case == "count_a_string" and i == 0:
+            set_kv(kvs, "split.count", gf.STR, "3")
+        if case == "tensors_count" and i == 0:
+            set_kv(kvs, "split.tensors.count", gf.I32, 7)
+        if case == "tensors_absent" and i == 0:
+            set_kv(kvs, "split.tensors.count", gf.I32, None)
+        if case == "tensors_negative" and i == 0:
+            set_kv(kvs, "split.tensors.count", gf.I32, -6)
+        if case == "duplicate" and i == 2:
+            tensors[0] = ("blk.0.w",) + tensors[0][1:]
+    first, _ = split_set(str(tmp_path), edit=edit)
+    if case == "missing_shard":
+        os.remove(os.path.join(str(tmp_path), shard_name("model", 2, 3)))
+    if case == "damaged_shard":
+        with open(os.path.join(str(tmp_path), shard_name("model", 1, 3)), "r+b") as f:
+            f.write(b"GGUX")
+    with pytest.raises(bm.GpuError) as e:
+        bm.Gguf(first, split=True)
+    for w in words:
+        assert w in str(e.value), str(e.value)
+
+
+def test_a_split_sets_first_shard_must_carry_the_sets_name(tmp_path):
+    first, _ = split_set(str(tmp_path))
+    odd = os.path.join(str(tmp_path), "model.gguf")
+    os.rename(first, odd)
+    with pytest.raises(bm.GpuError) as e:
+        bm.Gguf(odd, split=True)
+    assert "does not end in -00001-of-00003.gguf" in str(e.value)

@@ -109,6 +109,14 @@ int ora_dot_f32(const float *w, const float *x, int n, float *out);
 int ora_router_logits(const float *router, int n_experts, int hidden, const float *x, const float *gain, float eps, int m,
                       float *normed_out, float *logits);
 
+// The card rule (card.c): the reference's CPU mirrors of its GPU tier's q8_1 activations and 32-lane row walks
+// (crates/qdot/src/lib.rs:2885-3620). ora_card_q8_1 returns the number of refused (non-finite) blocks.
+int ora_card_q8_1(const float *x, int k, int8_t *codes, float *d8, int32_t *s8, uint8_t *refused);
+int ora_card_dot_row(int wtype, const uint8_t *wrow, int k, const int8_t *codes, const float *d8, const int32_t *s8, float *out);
+int ora_card_gemv(int wtype, const uint8_t *w, int rows, int k, const int8_t *codes, const float *d8, const int32_t *s8, int m, float *y);
+int ora_card_gemv_sel(int wtype, const uint8_t *w, int n_experts, int rows_per_expert, int k, const int8_t *codes, const float *d8,
+                      const int32_t *s8, const uint32_t *sel, int n_slots, float *y);
+
 #ifdef __cplusplus
 }
 #endif

@@ -62,6 +62,11 @@ def _load():
         "ora_sum_sq_f64": (C.c_double, [C.c_void_p, C.c_int]),
         "ora_rms_norm": (None, [C.c_void_p, C.c_void_p, C.c_float, C.c_int, C.c_void_p]),
         "ora_dot_f32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_card_q8_1": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+        "ora_card_dot_row": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+        "ora_card_gemv": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
+        "ora_card_gemv_sel": (C.c_int, [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                        C.c_void_p, C.c_int, C.c_void_p]),
         "ora_router_logits": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_float, C.c_int, C.c_void_p,
                                         C.c_void_p]),
         "ora_route_softmax_topk": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
@@ -398,3 +403,45 @@ def router_logits(router, x, gain=None, eps=0.0):
     _check(lib.ora_router_logits(_p(router), n_experts, hidden, _p(x), _p(g) if g is not None else None, float(eps), m,
                                  _p(normed), _p(logits)))
     return normed, logits
+
+
+# ------------------------------------------------------------------------------------------------ the card rule
+
+def card_q8_1(x):
+    """The GPU tier's q8_1 form of the columns x[m, k] (crates/qdot/src/lib.rs:2885 card_q8_1): (codes i8 [m, k],
+    d8 f32 [m, k / 128], s8 i32 [m, k / 32], refused bool [m, k / 128])."""
+    x = np.atleast_2d(_f32(x))
+    m, k = x.shape
+    codes, d8 = np.empty((m, k), np.int8), np.empty((m, k // 128), np.float32)
+    s8, refused = np.empty((m, k // 32), np.int32), np.empty((m, k // 128), np.uint8)
+    for c in range(m):
+        rc = lib.ora_card_q8_1(_p(x[c]), k, _p(codes[c]), _p(d8[c]), _p(s8[c]), _p(refused[c]))
+        if rc < 0:
+            raise OracleError(rc)
+    return codes, d8, s8, refused.astype(bool)
+
+
+def card_dot_row(wtype, wrow, k, codes, d8, s8):
+    out = np.empty(1, np.float32)
+    _check(lib.ora_card_dot_row(wtype, _p(_u8(wrow)), k, _p(np.ascontiguousarray(codes, np.int8)), _p(_f32(d8)),
+                                _p(np.ascontiguousarray(s8, np.int32)), _p(out)))
+    return out[0]
+
+
+def card_gemv(wtype, w, rows, k, codes, d8, s8):
+    """y[r * m + c] over the m columns of (codes, d8, s8) as card_q8_1 returns them."""
+    codes, d8, s8 = np.ascontiguousarray(codes, np.int8), _f32(d8), np.ascontiguousarray(s8, np.int32)
+    m = codes.size // k
+    y = np.empty(rows * m, np.float32)
+    _check(lib.ora_card_gemv(wtype, _p(_u8(w)), rows, k, _p(codes), _p(d8), _p(s8), m, _p(y)))
+    return y
+
+
+def card_gemv_sel(wtype, w, n_experts, rows_per_expert, k, codes, d8, s8, sel):
+    """y[s * rows_per_expert + r]: slot s's column against the rows of expert sel[s]."""
+    codes, d8, s8 = np.ascontiguousarray(codes, np.int8), _f32(d8), np.ascontiguousarray(s8, np.int32)
+    sel = np.ascontiguousarray(sel, np.uint32)
+    y = np.empty(sel.size * rows_per_expert, np.float32)
+    _check(lib.ora_card_gemv_sel(wtype, _p(_u8(w)), n_experts, rows_per_expert, k, _p(codes), _p(d8), _p(s8), _p(sel),
+                                 sel.size, _p(y)))
+    return y

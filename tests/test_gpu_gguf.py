@@ -69,3 +69,36 @@ def test_an_iq2_xxs_matrix_from_a_file(gpu, tmp_path):
     g.close()
     for b in (dw, act, xd, y):
         b.free()
+
+
+def test_a_layer_from_a_split_set(gpu, tmp_path):
+    """A layer whose three stacks lie in three shards of a split set (Q5_K gate / up, IQ4_XS down): the set opens by
+    its first shard, each stack is found in its own shard, and the step over them is the oracle's."""
+    hidden, ff, ne, top_k, m = 512, 256, 6, 2, 2
+    wg, wu = stack(bm.Q5_K, ne * ff, hidden, 51), stack(bm.Q5_K, ne * ff, hidden, 52)
+    wd = stack(bm.IQ4_XS, ne * hidden, ff, 53)
+    parts = ([("blk.0.ffn_gate_exps.weight", [hidden, ff, ne], bm.Q5_K, wg)],
+             [("blk.0.ffn_up_exps.weight", [hidden, ff, ne], bm.Q5_K, wu)],
+             [("blk.0.ffn_down_exps.weight", [ff, hidden, ne], bm.IQ4_XS, wd)])
+    for i, tensors in enumerate(parts):
+        kvs = [("split.no", gf.U16, i), ("split.count", gf.U16, 3), ("split.tensors.count", gf.I32, 3)]
+        if i == 0:
+            kvs.insert(0, ("qwen3moe.expert_count", gf.U32, ne))
+        gf.write(os.path.join(str(tmp_path), f"layer-{i + 1:05d}-of-00003.gguf"), kvs, tensors)
+    g = bm.Gguf(os.path.join(str(tmp_path), "layer-00001-of-00003.gguf"), split=True)
+    assert g.get_u64("qwen3moe.expert_count") == ne and len(g.tensors()) == 3
+    (dg, _, _), (du, _, _), (dd, rpe_d, ne_d) = (g.weights(gpu, f"blk.0.ffn_{n}_exps.weight") for n in ("gate", "up", "down"))
+    assert (dg.wtype, dd.wtype, rpe_d, ne_d) == (bm.Q5_K, bm.IQ4_XS, hidden, ne)
+    g.close()
+    rng = np.random.default_rng(54)
+    x = normal_f32(rng, (m, hidden))
+    ids, wts = route(rng, m, ne, top_k)
+    xd, sel, wt = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32)
+    act_h = gpu.act(bm.IQ4_XS, ff, m * top_k)
+    h = gpu.buffer(np.float32, m * top_k * ff)
+    y = gpu.buffer(np.float32, m * hidden).fill_bytes(0xFF)
+    gpu.enqueue_moe_decode(dg, du, dd, xd, sel, wt, None, top_k, m, act_h, y, h=h)
+    want = ora.moe_forward(hidden, ff, ne, (bm.Q5_K, bm.Q5_K, bm.IQ4_XS), wg, wu, wd, x, ids, wts, top_k, n_threads=4)
+    assert_f32(y.download(), want, "y")
+    for b in (dg, du, dd, xd, sel, wt, act_h, h, y):
+        b.free()

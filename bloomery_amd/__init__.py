@@ -84,6 +84,9 @@ SYMBOLS = {
     "bm_set_gate_rule": (_i, [_vp, _i, C.c_float]),
     "bm_route_softmax": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "bm_router_logits": (_i, [_vp, _vp, _vp, _vp, C.c_float, _i, _i, _i, _vp, _vp]),
+    "bm_card_quantize": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp]),
+    "bm_card_gemv": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp]),
+    "bm_card_gemv_sel": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
     "bm_gguf_open": (_i, [C.c_char_p, C.POINTER(_vp)]),
     "bm_gguf_open_split": (_i, [C.c_char_p, C.POINTER(_vp)]),
     "bm_gguf_close": (None, [_vp]),
@@ -481,6 +484,17 @@ class Gpu:
         self._check(self.lib.bm_gate_up_x(self.ctx, wg.handle, wu.handle, _ptr(x), _ptr(sel), n_slots_per_token, m,
                                           rows_per_expert, act_h.handle if act_h is not None else None,
                                           act_x.handle if act_x is not None else None, _ptr(h)))
+
+    # -- the card rule: the reference GPU tier's q8_1 columns and 32-lane row walks
+    def enqueue_card_quantize(self, x, m, k, codes, d8, s8):
+        self._check(self.lib.bm_card_quantize(self.ctx, _ptr(x), m, k, _ptr(codes), _ptr(d8), _ptr(s8)))
+
+    def enqueue_card_gemv(self, w, codes, d8, s8, m, y):
+        self._check(self.lib.bm_card_gemv(self.ctx, w.handle, _ptr(codes), _ptr(d8), _ptr(s8), m, _ptr(y)))
+
+    def enqueue_card_gemv_sel(self, w, codes, d8, s8, sel, n_slots, rows_per_expert, y):
+        self._check(self.lib.bm_card_gemv_sel(self.ctx, w.handle, _ptr(codes), _ptr(d8), _ptr(s8), _ptr(sel), n_slots,
+                                              rows_per_expert, _ptr(y)))
 
     def set_decode_plan(self, plan):
         self._check(self.lib.bm_set_decode_plan(self.ctx, plan))

@@ -892,6 +892,61 @@ int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *a
     return driver(ctx, what, bmk::block_sums(launch_of(ctx), w->wtype, wrow, w->k, c, out_dev));
 }
 
+// ------------------------------------------------------------------------------------ the card rule
+
+static int check_card_planes(bm_ctx *ctx, const char *what, const void *codes, const void *d8, const void *s8) {
+    if (((uintptr_t)codes & 15) != 0 || (((uintptr_t)d8 | (uintptr_t)s8) & 3) != 0)
+        return fail(ctx, BM_ESHAPE, "%s: codes_dev %p must be 16-byte aligned, d8_dev %p and s8_dev %p 4-byte aligned", what, codes, d8, s8);
+    return BM_OK;
+}
+
+int bm_card_quantize(bm_ctx *ctx, const float *x_dev, int m, int k, int8_t *codes_dev, float *d8_dev, int32_t *s8_dev) {
+    const char *what = "bm_card_quantize";
+    if (!ctx || !x_dev || !codes_dev || !d8_dev || !s8_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (k <= 0 || k % 256 != 0) return fail(ctx, BM_ESHAPE, "%s: card q8_1 columns are whole 256-value super-blocks, k = %d", what, k);
+    if (m < 1) return fail(ctx, BM_ESHAPE, "%s: need m >= 1, got %d", what, m);
+    if (((uintptr_t)x_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: x_dev %p must be 16-byte aligned", what, (const void *)x_dev);
+    int rc = check_card_planes(ctx, what, codes_dev, d8_dev, s8_dev);
+    if (rc) return rc;
+    return driver(ctx, what, bmk::card_quantize(launch_of(ctx), x_dev, m, k, codes_dev, d8_dev, s8_dev));
+}
+
+static int check_card_weights(bm_ctx *ctx, const char *what, const bm_weights *w) {
+    if (!bmk::card_type(w->wtype))
+        return fail(ctx, BM_ETYPE, "%s: the card rule walks Q4_K (12) and Q3_K (11) rows; the weights are type %d", what, w->wtype);
+    return BM_OK;
+}
+
+int bm_card_gemv(bm_ctx *ctx, const bm_weights *w, const int8_t *codes_dev, const float *d8_dev, const int32_t *s8_dev, int m,
+                 float *y_dev) {
+    const char *what = "bm_card_gemv";
+    if (!ctx || !w || !codes_dev || !d8_dev || !s8_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    int rc = check_card_weights(ctx, what, w);
+    if (rc) return rc;
+    if (m < 1 || m > 65535) return fail(ctx, BM_ESHAPE, "%s: m = %d columns (1 .. 65535)", what, m);
+    rc = check_card_planes(ctx, what, codes_dev, d8_dev, s8_dev);
+    if (rc) return rc;
+    return driver(ctx, what, bmk::card_gemv(launch_of(ctx), w->wtype, w->dev, (long)w->rows, w->k, codes_dev, d8_dev, s8_dev, m, y_dev));
+}
+
+int bm_card_gemv_sel(bm_ctx *ctx, const bm_weights *w, const int8_t *codes_dev, const float *d8_dev, const int32_t *s8_dev,
+                     const uint32_t *sel_dev, int n_slots, int rows_per_expert, float *y_dev) {
+    const char *what = "bm_card_gemv_sel";
+    if (!ctx || !w || !codes_dev || !d8_dev || !s8_dev || !sel_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    int rc = check_card_weights(ctx, what, w);
+    if (rc) return rc;
+    int n_experts = 0;
+    rc = check_stack(ctx, what, w, rows_per_expert, &n_experts);
+    if (rc) return rc;
+    if (n_slots < 1) return fail(ctx, BM_ESHAPE, "%s: need n_slots >= 1, got %d", what, n_slots);
+    if ((int64_t)n_slots * ((rows_per_expert + 7) / 8) > 0x7fffffff)
+        return fail(ctx, BM_ESHAPE, "%s: %d slots of %d rows are past what a launch takes", what, n_slots, rows_per_expert);
+    rc = check_card_planes(ctx, what, codes_dev, d8_dev, s8_dev);
+    if (rc) return rc;
+    return driver(ctx, what, bmk::card_gemv_sel(launch_of(ctx), w->wtype, w->dev, n_experts, w->k, codes_dev, d8_dev, s8_dev, sel_dev,
+                                                n_slots, rows_per_expert, y_dev));
+}
+
 // ------------------------------------------------------------------------------------ graphs and events
 
 struct bm_graph {

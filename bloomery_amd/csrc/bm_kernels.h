@@ -134,6 +134,15 @@ hipError_t router_logits(const Launch &L, const float *router, const float *x, c
 
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out);
 
+// The card rule (bm_card.hip): the reference GPU tier's q8_1 columns (codes[m * k], d8[m * k / 128], s8[m * k / 32]) and
+// its 32-lane Q4_K / Q3_K row walks. codes must be 16-byte aligned.
+bool card_type(int wtype);
+hipError_t card_quantize(const Launch &L, const float *x, int m, int k, int8_t *codes, float *d8, int32_t *s8);
+hipError_t card_gemv(const Launch &L, int wtype, const uint8_t *w, long rows, int k, const int8_t *codes, const float *d8,
+                     const int32_t *s8, int m, float *y);
+hipError_t card_gemv_sel(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const int8_t *codes, const float *d8,
+                         const int32_t *s8, const uint32_t *sel, int n_slots, int rows_per_expert, float *y);
+
 } // namespace bmk
 
 #endif // BM_KERNELS_H

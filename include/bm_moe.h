@@ -321,6 +321,28 @@ int bm_router_logits(bm_ctx *ctx, const float *router_dev, const float *x_dev, c
                      int n_experts, int hidden, float *normed_dev, float *logits_dev);
 
 
+/* ------------------------------------------------------------------------------------------- the card rule */
+
+/* The reference's GPU tier has an activation form and row walks of its own, and its CPU crate restates them so the
+ * tiers can be compared bit for bit (crates/qdot/src/lib.rs:2885 card_q8_1, :3558 card_q4k_dot_row, :3346
+ * card_q3k_dot_row; the device side: q3k_quantize_q8_1 crates/gpu/src/lib.rs:1448, q4k_gemv :1617, q4k_gemv_sel
+ * crates/gpu/src/q4k_sel.rs:358). These entries give those values on this GPU, so a caller holding outputs of the
+ * reference's CUDA tier can compare them with this library's bit for bit. They are a second arithmetic beside the
+ * CPU path's that every other entry follows, not a faster one.
+ *
+ * A card q8_1 column of k values (a multiple of 256) is three planes in value order: codes i8[k]; d8 f32[k / 128],
+ * a 128-value block's amax / 127 (1 for a zero block); s8 i32[k / 32], the code sum of 32 values. Codes are
+ * v / d rounded half away from zero and held to +-127. A block holding a value that is not finite is refused: NaN
+ * scale, zero codes and sums, and the fault word takes QuantColumn. m columns lie back to back in each plane. */
+int bm_card_quantize(bm_ctx *ctx, const float *x_dev, int m, int k, int8_t *codes_dev, float *d8_dev, int32_t *s8_dev);
+/* y_dev[r * m + c] = row r of w (Q4_K or Q3_K) against column c, by the 32-lane walk and its butterfly. */
+int bm_card_gemv(bm_ctx *ctx, const bm_weights *w, const int8_t *codes_dev, const float *d8_dev, const int32_t *s8_dev, int m,
+                 float *y_dev);
+/* The MoE down step of the card tier: y_dev[s * rows_per_expert + r] = row r of expert sel_dev[s] against column s.
+ * Ids as bm_gemv_sel takes them (past the stack: ExpertId raised, the slot's rows untouched; 0xffffffff skipped). */
+int bm_card_gemv_sel(bm_ctx *ctx, const bm_weights *w, const int8_t *codes_dev, const float *d8_dev, const int32_t *s8_dev,
+                     const uint32_t *sel_dev, int n_slots, int rows_per_expert, float *y_dev);
+
 /* ------------------------------------------------------------------------------------------- model files */
 
 /* A GGUF file's header and a read-only mapping of it: the part of the reference's reader (crates/gguf/src/lib.rs:

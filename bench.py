@@ -410,11 +410,90 @@ def bench_dsv3(args, bm, ora, threads):
     gpu.close()
 
 
+def bench_card(args, bm, ora, threads):
+    """Config 6 (a side measurement, not a BASELINE.json line): the card rule. The MoE down step of the reference's GPU
+    tier at the headline layer's down shape (8 slots of 768 values against 2048 Q4_K rows of 8 of 128 resident experts:
+    the q8_1 quantizer, then the 32-lane row walks), and one large Q4_K gemv by the same walk for its streaming rate."""
+    rng = np.random.default_rng(0xB1000006)
+    def q4k_blocks(rows, k):  # a finite dmin beside the finite d
+        w = random_blocks(rng, bm.Q4_K, rows, k, 144, 0).reshape(-1, 144)
+        w[:, 2:4] = rng.uniform(0.001, 0.02, w.shape[0]).astype(np.float16).view(np.uint8).reshape(-1, 2)
+        return w.reshape(-1)
+
+    wd = q4k_blocks(N_EXPERTS * HIDDEN, FF)
+    n_tok = args.tokens
+    h = rng.uniform(-2, 2, (n_tok * TOP_K, FF)).astype(np.float32)
+    ids = np.stack([rng.choice(N_EXPERTS, TOP_K, replace=False) for _ in range(n_tok)]).astype(np.uint32)
+    gpu = bm.Gpu(0)
+    copies = [gpu.weights(bm.Q4_K, N_EXPERTS * HIDDEN, FF, wd) for _ in range(args.layers)]
+    hd, sel = gpu.upload(h, np.float32), gpu.upload(ids, np.uint32)
+    codes, d8, s8 = gpu.buffer(np.int8, n_tok * TOP_K * FF), gpu.buffer(np.float32, n_tok * TOP_K * FF // 128), \
+        gpu.buffer(np.int32, n_tok * TOP_K * FF // 32)
+    y = gpu.buffer(np.float32, n_tok * TOP_K * HIDDEN)
+
+    def planes(t):
+        return codes.ptr + t * TOP_K * FF, d8.ptr + 4 * t * TOP_K * FF // 128, s8.ptr + 4 * t * TOP_K * FF // 32
+
+    def quant(i):
+        t = i % n_tok
+        gpu.enqueue_card_quantize(hd.ptr + 4 * t * TOP_K * FF, TOP_K, FF, *planes(t))
+
+    def down(i):
+        t = i % n_tok
+        gpu.enqueue_card_gemv_sel(copies[i % len(copies)], *planes(t), sel.ptr + 4 * t * TOP_K, TOP_K, HIDDEN,
+                                  y.ptr + 4 * t * TOP_K * HIDDEN)
+
+    def step(i):
+        quant(i)
+        down(i)
+
+    for i in range(2):
+        step(i)
+    got = y.download()[:2 * TOP_K * HIDDEN]
+    c, d, s, _ = ora.card_q8_1(h[:2 * TOP_K])
+    want = ora.card_gemv_sel(ora.Q4_K, wd, N_EXPERTS, HIDDEN, FF, c, d, s, ids[:2].reshape(-1))
+    parity = parity_of(got, want)
+    wall, ev, steps, warm = timed_graph(gpu, step, n_tok, args.steps, args.warmup)
+    kernel_us = {"card_quantize": timed_graph(gpu, quant, n_tok, 1024, 64)[1] * 1e3,
+                 "card_gemv_sel": timed_graph(gpu, down, n_tok, 1024, 64)[1] * 1e3}
+    nbytes = TOP_K * HIDDEN * bm.row_bytes(bm.Q4_K, FF)
+    ach = nbytes / (kernel_us["card_gemv_sel"] * 1e-6) / 1e9
+    # the walk's streaming rate: 32768 rows of 4096 values, four copies cycled
+    rows_big, k_big = 32768, 4096
+    wb = q4k_blocks(rows_big, k_big)
+    big = [gpu.weights(bm.Q4_K, rows_big, k_big, wb) for _ in range(4)]
+    xb = gpu.upload(rng.uniform(-2, 2, k_big).astype(np.float32), np.float32)
+    cb, db, sb = gpu.buffer(np.int8, k_big), gpu.buffer(np.float32, k_big // 128), gpu.buffer(np.int32, k_big // 32)
+    yb = gpu.buffer(np.float32, rows_big)
+    gpu.enqueue_card_quantize(xb, 1, k_big, cb, db, sb)
+    big_ms = timed_graph(gpu, lambda i: gpu.enqueue_card_gemv(big[i % 4], cb, db, sb, 1, yb), 8, 64, 8)[1]
+    big_gbs = rows_big * bm.row_bytes(bm.Q4_K, k_big) / (big_ms * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu:
+        n, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < min(args.cpu_seconds, 10.0):
+            t = n % n_tok
+            c, d, s, _ = ora.card_q8_1(h[t * TOP_K:(t + 1) * TOP_K])
+            ora.card_gemv_sel(ora.Q4_K, wd, N_EXPERTS, HIDDEN, FF, c, d, s, ids[t])
+            n += 1
+        cpu = {"value": (time.perf_counter() - t0) / n * 1e6, "unit": "us/token", "cores": 1, "kind": "port",
+               "sample": f"{n} tokens' quantize + down step, scalar restatement of qdot's card mirrors on 1 thread"}
+    emit("card_rule_down_step_us_per_token", wall * 1e3, "us/token", steps, warm, wall,
+         "the card rule's MoE down step: 8 slots x 768 values, q8_1 quantizer + 32-lane Q4_K walks over 2048 rows of 8 of 128 "
+         "experts; random legal blocks (not a BASELINE.json configuration)",
+         {"event_ms_per_step": ev, "kernel_us": kernel_us, "parity": parity, "algorithmic_bytes_per_launch": nbytes,
+          "large_gemv": {"rows": rows_big, "k": k_big, "ms": big_ms, "gb_per_s": big_gbs}},
+         {"bound": "hbm", "kernel": "k_card_gemv_sel<Q4_K>", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+          "frac": ach / HBM_PEAK_GBS, "traffic": None}, cpu)
+    gpu.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5),
+    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5, 6),
                     help="1: one Q4_K gemv; 2 (default, the headline): Qwen3-shaped layer, 1 token; 3: the same layer, 16 tokens "
-                         "grouped by expert; 4: prefill of 2048 tokens (int8 MFMA GEMM); 5: DeepSeek-V3-shaped layer, 4 tokens")
+                         "grouped by expert; 4: prefill of 2048 tokens (int8 MFMA GEMM); 5: DeepSeek-V3-shaped layer, 4 tokens; "
+                         "6: the card rule's down step (a side measurement)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--traffic-probe", action="store_true",
                     help="config 2 only: no timing; 8 copies of 64 MiB by a plain kernel (the counters' calibration), then "
@@ -442,7 +521,7 @@ def main():
 
     threads = min(os.cpu_count() or 1, 16)
     if args.config != 2:
-        return {1: bench_gemv, 3: bench_grouped, 4: bench_prefill, 5: bench_dsv3}[args.config](args, bm, ora, threads)
+        return {1: bench_gemv, 3: bench_grouped, 4: bench_prefill, 5: bench_dsv3, 6: bench_card}[args.config](args, bm, ora, threads)
     names = {"q3_k": bm.Q3_K, "q4_k": bm.Q4_K, "q5_k": bm.Q5_K, "q6_k": bm.Q6_K, "iq2_xxs": bm.IQ2_XXS,
              "iq3_xxs": bm.IQ3_XXS, "iq4_xs": bm.IQ4_XS}
     try:

@@ -374,6 +374,82 @@ __device__ __forceinline__ void bm_dot_q5k(const Blk<BM_Q5K> &b, const Act<BM_Q5
     bm_dot_q45k(b.hdr, b.qa, b.qb, FifthBit{b.qh}, a, i, c, h, acc0, acc1, tap);
 }
 
+// A Q4_K / Q5_K super-block's weight side, formed once and dotted against several columns: the code words as the dot
+// takes them (the fifth bit joined), the four scale products d * sc and the two min products -(dmin * m), each the
+// value bm_dot_q45k forms for every column anew.
+struct Q45Dec {
+    u32 lo0[4], hi0[4], lo1[4], hi1[4];
+    float w00, w01, w10, w11, n0, n1;
+};
+
+template <bool Fifth>
+__device__ __forceinline__ Q45Dec bm_decode_q45k(uint4 hdr, uint4 qa, uint4 qb, uint4 qh, int c, int h) {
+    const float d = bm_half_to_f32(hdr.x & 0xffffu), dmin = bm_half_to_f32(hdr.x >> 16);
+    const u32 a0 = hdr.y, a1 = hdr.z, a2 = hdr.w;
+    const int sh = 16 * c;
+    const u32 s0 = (a0 & 0x3f3f3f3fu) >> sh;
+    const u32 s1 = ((a2 & 0x0f0f0f0fu) | ((a0 >> 2) & 0x30303030u)) >> sh;
+    const u32 hm = 0u - (u32)h;
+    const u32 mw = ((((a2 >> 4) & 0x0f0f0f0fu) | ((a1 >> 2) & 0x30303030u)) & hm) | ((a1 & 0x3f3f3f3fu) & ~hm);
+    const u32 mm = mw >> sh;
+    Q45Dec x;
+    x.n0 = -(dmin * (float)(mm & 0xffu));
+    x.n1 = -(dmin * (float)((mm >> 8) & 0xffu));
+    x.w00 = d * (float)(s0 & 0xffu);
+    x.w01 = d * (float)((s0 >> 8) & 0xffu);
+    x.w10 = d * (float)(s1 & 0xffu);
+    x.w11 = d * (float)((s1 >> 8) & 0xffu);
+    const u32 m = 0x0f0f0f0fu, one = 0x01010101u;
+    const u32 wa[4] = {qa.x, qa.y, qa.z, qa.w}, wb[4] = {qb.x, qb.y, qb.z, qb.w}, wh[4] = {qh.x, qh.y, qh.z, qh.w};
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        x.lo0[t] = wa[t] & m;
+        x.hi0[t] = (wa[t] >> 4) & m;
+        x.lo1[t] = wb[t] & m;
+        x.hi1[t] = (wb[t] >> 4) & m;
+        if constexpr (Fifth) { // sub-blocks 2c, 2c + 1 of the first word, 4 + 2c, 5 + 2c of the second
+            x.lo0[t] |= ((wh[t] >> (2 * c)) & one) << 4;
+            x.hi0[t] |= ((wh[t] >> (2 * c + 1)) & one) << 4;
+            x.lo1[t] |= ((wh[t] >> (4 + 2 * c)) & one) << 4;
+            x.hi1[t] |= ((wh[t] >> (5 + 2 * c)) & one) << 4;
+        }
+    }
+    return x;
+}
+
+__device__ __forceinline__ int bm_dot16_words(const u32 (&w)[4], uint4 a) {
+    int s = bm_sdot4(w[0], a.x, 0);
+    s = bm_sdot4(w[1], a.y, s);
+    s = bm_sdot4(w[2], a.z, s);
+    return bm_sdot4(w[3], a.w, s);
+}
+
+// bm_dot_q45k's column side over a decoded super-block: the same products and sums in the same order.
+template <class Tap>
+__device__ __forceinline__ void bm_dot_q45k_dec(const Q45Dec &x, const Act<BM_Q4K> &a, int i, int c, int h, float &acc0,
+                                                float &acc1, const Tap &tap) {
+    acc0 = fmaf(a.em.y, x.n0, acc0);
+    acc1 = fmaf(a.em.w, x.n1, acc1);
+    if constexpr (Tap::kActive) {
+        tap.q4k_isum(i, 4 * h + 2 * c, (int)(short)(a.sw & 0xffffu));
+        tap.q4k_isum(i, 4 * h + 2 * c + 1, (int)(short)(a.sw >> 16));
+    }
+    {
+        const int lo = bm_dot16_words(x.lo0, a.lo0), hi = bm_dot16_words(x.hi0, a.hi0);
+        acc0 = fmaf(x.w00 * a.e0.x, (float)lo, acc0);
+        acc1 = fmaf(x.w01 * a.e0.z, (float)hi, acc1);
+        tap.q4k(i, 2 * c, h, lo);
+        tap.q4k(i, 2 * c + 1, h, hi);
+    }
+    {
+        const int lo = bm_dot16_words(x.lo1, a.lo1), hi = bm_dot16_words(x.hi1, a.hi1);
+        acc0 = fmaf(x.w10 * a.e1.x, (float)lo, acc0);
+        acc1 = fmaf(x.w11 * a.e1.z, (float)hi, acc1);
+        tap.q4k(i, 4 + 2 * c, h, lo);
+        tap.q4k(i, 5 + 2 * c, h, hi);
+    }
+}
+
 // ---- Q6_K: lane (c, h) owns accumulators l = 4h + c and 4h + c + 2. Per 128-value half j it reads ql bytes
 // [64j + 32c + 16h, +16) (low nibbles: quarter c, high nibbles: quarter c + 2, both half h) and qh bytes
 // [32j + 16h, +16) (bits 2a of quarter a).
@@ -450,6 +526,49 @@ __device__ __forceinline__ void bm_dot_q6k(const Blk<BM_Q6K> &b, const Act<BM_Q6
         const int sc1 = __builtin_amdgcn_sbfe((int)(j ? b.sc.w : b.sc.y), bi, 8);
         acc0 = fmaf((d * (float)sc0) * a.d8a[j], (float)s0, acc0);
         acc1 = fmaf((d * (float)sc1) * a.d8b[j], (float)s1, acc1);
+        tap.q6k(i, 8 * j + 2 * c + h, s0);
+        tap.q6k(i, 8 * j + 4 + 2 * c + h, s1);
+    }
+}
+
+// A Q6_K super-block's weight side, formed once for several columns: the 6-bit code words of the lane's four
+// 16-value groups and the four products d * scale.
+struct Q6Dec {
+    u32 wa[2][4], wb[2][4];
+    float fa[2], fb[2];
+};
+
+__device__ __forceinline__ Q6Dec bm_decode_q6k(const Blk<BM_Q6K> &b, int c, int h) {
+    const float d = bm_half_to_f32(b.d);
+    const int bi = 8 * (2 * c + h), hs = 2 * c;
+    const u32 ml = 0x0f0f0f0fu, mh = 0x30303030u;
+    Q6Dec x;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const uint4 ql = j ? b.ql1 : b.ql0, qh = j ? b.qh1 : b.qh0;
+        const u32 l[4] = {ql.x, ql.y, ql.z, ql.w}, hh[4] = {qh.x >> hs, qh.y >> hs, qh.z >> hs, qh.w >> hs};
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            x.wa[j][t] = (l[t] & ml) | ((hh[t] << 4) & mh);
+            x.wb[j][t] = ((l[t] >> 4) & ml) | (hh[t] & mh);
+        }
+        const int sc0 = __builtin_amdgcn_sbfe((int)(j ? b.sc.z : b.sc.x), bi, 8); // the builtin's type is unsigned
+        const int sc1 = __builtin_amdgcn_sbfe((int)(j ? b.sc.w : b.sc.y), bi, 8);
+        x.fa[j] = d * (float)sc0;
+        x.fb[j] = d * (float)sc1;
+    }
+    return x;
+}
+
+template <class Tap>
+__device__ __forceinline__ void bm_dot_q6k_dec(const Q6Dec &x, const Act<BM_Q6K> &a, int i, int c, int h, float &acc0,
+                                               float &acc1, const Tap &tap) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int s0 = bm_dot16_words(x.wa[j], a.aa[j]) - 32 * a.sa[j];
+        const int s1 = bm_dot16_words(x.wb[j], a.ab[j]) - 32 * a.sb[j];
+        acc0 = fmaf(x.fa[j] * a.d8a[j], (float)s0, acc0);
+        acc1 = fmaf(x.fb[j] * a.d8b[j], (float)s1, acc1);
         tap.q6k(i, 8 * j + 2 * c + h, s0);
         tap.q6k(i, 8 * j + 4 + 2 * c + h, s1);
     }

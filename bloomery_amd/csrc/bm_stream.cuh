@@ -206,6 +206,24 @@ __device__ __forceinline__ void row_dot(Blk<WT> (&b)[U], const uint8_t *wrow, co
                         const Act<WT> a = bm_load_act<WT, Tap::kActive>(av[c], i, q);
                         bm_dot_iq4xs_dec(b[slot], dec, a, i, q, a0[c], a1[c], tap);
                     }
+            } else if constexpr (WT == BM_Q4K || WT == BM_Q5K) { // the nibble words and the scale products
+                Q45Dec dec;
+                if constexpr (WT == BM_Q5K) dec = bm_decode_q45k<true>(b[slot].hdr, b[slot].qa, b[slot].qb, b[slot].qh, q & 1, q >> 1);
+                else dec = bm_decode_q45k<false>(b[slot].hdr, b[slot].qa, b[slot].qb, b[slot].hdr, q & 1, q >> 1);
+#pragma unroll
+                for (int c = 0; c < M; c++)
+                    if (c < m) {
+                        const Act<WT> a = bm_load_act<WT, Tap::kActive>(av[c], i, q);
+                        bm_dot_q45k_dec(dec, a, i, q & 1, q >> 1, a0[c], a1[c], tap);
+                    }
+            } else if constexpr (WT == BM_Q6K) {
+                const Q6Dec dec = bm_decode_q6k(b[slot], q & 1, q >> 1);
+#pragma unroll
+                for (int c = 0; c < M; c++)
+                    if (c < m) {
+                        const Act<WT> a = bm_load_act<WT, Tap::kActive>(av[c], i, q);
+                        bm_dot_q6k_dec(dec, a, i, q & 1, q >> 1, a0[c], a1[c], tap);
+                    }
             } else {
 #pragma unroll
                 for (int c = 0; c < M; c++)

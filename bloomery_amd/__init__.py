@@ -60,6 +60,7 @@ SYMBOLS = {
     "bm_quantize": (_i, [_vp, _vp, _i, _vp]),
     "bm_gemv": (_i, [_vp, _vp, _vp, _i, _vp]),
     "bm_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
+    "bm_gemv_x": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
     "bm_gemv_sel": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "bm_combine_tokens": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_down_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -484,6 +485,10 @@ class Gpu:
         self._check(self.lib.bm_gate_up_x(self.ctx, wg.handle, wu.handle, _ptr(x), _ptr(sel), n_slots_per_token, m,
                                           rows_per_expert, act_h.handle if act_h is not None else None,
                                           act_x.handle if act_x is not None else None, _ptr(h)))
+
+    def enqueue_gemv_x(self, w, x, m, y, act_out=None):
+        """Quantizer and gemv in one launch: y[r * m + c] from the f32 columns x[m, k]."""
+        self._check(self.lib.bm_gemv_x(self.ctx, w.handle, _ptr(x), m, act_out.handle if act_out is not None else None, _ptr(y)))
 
     # -- the card rule: the reference GPU tier's q8_1 columns and 32-lane row walks
     def enqueue_card_quantize(self, x, m, k, codes, d8, s8):

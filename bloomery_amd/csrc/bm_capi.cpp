@@ -357,6 +357,21 @@ int bm_gemv(bm_ctx *ctx, const bm_weights *w, const bm_act *act, int m, float *y
     return BM_OK;
 }
 
+int bm_gemv_x(bm_ctx *ctx, const bm_weights *w, const float *x_dev, int m, bm_act *act_out, float *y_dev) {
+    const char *what = "bm_gemv_x";
+    if (!ctx || !w || !x_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (m < 1 || m > 65535) return fail(ctx, BM_ESHAPE, "%s: m = %d columns (1 .. 65535)", what, m);
+    if (((uintptr_t)x_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: x_dev %p must be 16-byte aligned", what, (const void *)x_dev);
+    if (act_out) {
+        int rc = check_pair(ctx, what, w, act_out);
+        if (rc) return rc;
+        if (act_out->m_cap < m) return fail(ctx, BM_ESHAPE, "%s: act_out holds %d columns, m = %d", what, act_out->m_cap, m);
+    }
+    if (bmk::gemv_x_lds(w->wtype, w->k) > (size_t)bmk::kMaxLds)
+        return fail(ctx, BM_ESHAPE, "%s: one column of k = %d does not fit the workgroup's LDS", what, w->k);
+    return driver(ctx, what, bmk::gemv_x(launch_of(ctx), w->wtype, w->dev, w->rows, w->k, x_dev, m, act_out ? act_out->dev : nullptr, y_dev));
+}
+
 // rows a positive multiple of rows_per_expert (crates/gpu/src/q4k_sel.rs:1013-1023).
 static int check_stack(bm_ctx *ctx, const char *what, const bm_weights *w, int rows_per_expert, int *n_experts) {
     if (rows_per_expert <= 0 || w->rows % rows_per_expert != 0)

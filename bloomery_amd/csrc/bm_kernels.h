@@ -132,6 +132,12 @@ bool router_logits_fits(int hidden);
 hipError_t router_logits(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                          int hidden, float *normed_out, float *logits);
 
+// gemv from f32 columns x[m * k], the quantizer folded in: y[row * m + c]; act_out (optional) receives the columns' bytes
+// in the device form of an activation column.
+size_t gemv_x_lds(int wtype, int k);
+hipError_t gemv_x(const Launch &L, int wtype, const uint8_t *w, int64_t rows, int k, const float *x, int m, uint8_t *act_out,
+                  float *y);
+
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out);
 
 // The card rule (bm_card.hip): the reference GPU tier's q8_1 columns (codes[m * k], d8[m * k / 128], s8[m * k / 32]) and

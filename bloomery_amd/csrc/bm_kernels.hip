@@ -668,6 +668,42 @@ __global__ __launch_bounds__(256) void k_gate_up_xq(const float *x, const uint8_
     }
 }
 
+// k_gemv with the activation quantizer folded in: grid row c is column c, an f32 row of k values that every workgroup
+// quantizes into LDS for itself (the form its weight type dots against), so a matrix-vector product from f32 is one
+// launch and no column passes through memory. With act_out the first workgroup of a column leaves its bytes there.
+template <int WT, int U, int NB>
+__global__ __launch_bounds__(256) void k_gemv_x(const float *x, const uint8_t *w, long rows, int nb, int m, uint8_t *act_out,
+                                                float *y, u32 *fault, u32 layer) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, q = tid & 3, c = blockIdx.y;
+    const long row = (long)blockIdx.x * 64 + (tid >> 2);
+    const bool active = row < rows;
+    const int n = NB > 0 ? NB : nb;
+    const int k = n * 256;
+    const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
+    const int col_bytes = bm_act_col_bytes<WT>(n);
+    const uint8_t *wrow = w + (size_t)(active ? row : 0) * row_bytes;
+    Blk<WT> b[U];
+    preload<WT, U>(b, wrow, q);
+    const Iq2Tables tb = stage_tables<WT>(lds);
+    uint8_t *col = lds + tab_bytes<WT>();
+    const float *xc = x + (size_t)c * k;
+    if constexpr (bm_takes_q8k(WT)) {
+        q8k_stage_cols(xc, col, 1, n, fault, layer);
+    } else { // a q8_2 block is four lanes of eight values; 2048 values a pass
+        for (int o = tid * 8; o < k; o += 2048) {
+            const float4 lo = *reinterpret_cast<const float4 *>(xc + o), hi = *reinterpret_cast<const float4 *>(xc + o + 4);
+            float v8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            q82_quad8(v8, col, n, o >> 5, tid & 3, fault, layer);
+        }
+    }
+    __syncthreads();
+    if (act_out && blockIdx.x == 0) stage_bytes(act_out + (size_t)c * col_bytes, col, col_bytes);
+    float v[1];
+    row_dot<WT, U, NB, 1>(b, wrow, col, col_bytes, 1, n, q, tb, v, NoTap{});
+    if (q == 0 && active) y[(size_t)row * m + c] = v[0];
+}
+
 // k_down_combine for down stacks that dot against Q8_K columns: the token's slot rows of h (f32) are quantized by
 // every workgroup into LDS; the first workgroup of a token also leaves the columns in act_h.
 template <int WT, int U, int NB>
@@ -790,6 +826,23 @@ hipError_t gemv(const Launch &L, int wtype, const uint8_t *w, int64_t rows, int 
     if (e != hipSuccess) return e;                                                                                     \
     hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 63) / 64)), dim3(256), lds, L.stream, w, (long)rows, nb, act,     \
                        m_total, col0, m, y);
+    BM_DISPATCH(wtype, nb)
+#undef CALL_BODY
+    return hipGetLastError();
+}
+
+size_t gemv_x_lds(int wtype, int k) { return tab_bytes_rt(wtype) + (size_t)act_col_bytes(wtype, k); }
+
+hipError_t gemv_x(const Launch &L, int wtype, const uint8_t *w, int64_t rows, int k, const float *x, int m, uint8_t *act_out,
+                  float *y) {
+    const int nb = k / 256;
+    const size_t lds = gemv_x_lds(wtype, k);
+#define CALL_BODY                                                                                                      \
+    auto kern = k_gemv_x<WT, U, NB>;                                                                                   \
+    hipError_t e = allow_lds(kern, lds);                                                                               \
+    if (e != hipSuccess) return e;                                                                                     \
+    hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 63) / 64), (unsigned)m), dim3(256), lds, L.stream, x, w,          \
+                       (long)rows, nb, m, act_out, y, L.fault, L.layer);
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
     return hipGetLastError();

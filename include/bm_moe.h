@@ -127,6 +127,12 @@ int bm_quantize(bm_ctx *ctx, const float *x_dev, int m, bm_act *act);
 /* Gpu::enqueue_gemv_q4k / enqueue_gemv_q6k (crates/gpu/src/lib.rs:3495,3839) and the IQ2_XXS row kernel
  * (crates/gpu/src/iq.rs:1405): y_dev[row * m + c] = row `row` of w . column c of act, m = `m` columns, 1..=8. */
 int bm_gemv(bm_ctx *ctx, const bm_weights *w, const bm_act *act, int m, float *y_dev);
+/* bm_quantize + bm_gemv in one launch (the reference issues the two, crates/gpu/src/lib.rs:3275 then :3495): column c is
+ * the f32 row x_dev + c * k, quantized by every workgroup for itself, so y_dev[r * m + c] holds bm_gemv's bits of
+ * bm_quantize's columns without a column passing through memory. act_out (optional, made for w's type, m_cap >= m)
+ * receives the columns as bm_quantize would leave them. A value that is not finite raises QuantColumn as bm_quantize
+ * does. x_dev 16-byte aligned. */
+int bm_gemv_x(bm_ctx *ctx, const bm_weights *w, const float *x_dev, int m, bm_act *act_out, float *y_dev);
 
 /* -------------------------------------------------------------------------- decode: the routed expert chain */
 

@@ -228,6 +228,47 @@ def test_gemv_matches_dot_row(gpu, wtype, rows, k):
         b.free()
 
 
+@pytest.mark.parametrize("wtype,rows,k", ((bm.Q4_K, 768, 2048), (bm.Q6_K, 2048, 768), (bm.Q5_K, 67, 1280), (bm.Q4_K, 70, 4352),
+                                          (bm.IQ2_XXS, 33, 7168), (bm.IQ4_XS, 66, 768), (bm.IQ3_XXS, 40, 1280),
+                                          (bm.Q3_K, 150, 2048)))
+def test_gemv_from_f32_folds_the_quantizer(gpu, wtype, rows, k):
+    """bm_gemv_x: the quantizer and the gemv in one launch give the two launches' bits, for y and for the columns it
+    leaves in act_out; a value that is not finite raises QuantColumn as bm_quantize does."""
+    rng = np.random.default_rng(300 + rows)
+    w = stack(wtype, rows, k, 301 + rows)
+    x = normal_f32(rng, (3, k))
+    x[1] *= np.float32(1e-3)
+    wd, xd = gpu.weights(wtype, rows, k, w), gpu.upload(x, np.float32)
+    cols = np.concatenate([ora.quantize_col(wtype, x[c]) for c in range(3)])
+    gpu.fault_clear()
+    for m, keep in ((1, False), (3, True)):
+        y = gpu.buffer(np.float32, rows * m).fill_bytes(0xFF)
+        act = gpu.act(wtype, k, 3) if keep else None
+        gpu.enqueue_gemv_x(wd, xd, m, y, act)
+        assert_f32(y.download(), ora.gemv(wtype, w, rows, k, cols, m), f"gemv_x type {wtype} {rows}x{k} m={m}")
+        if keep:
+            for c in range(m):
+                assert np.array_equal(act.download(c), ora.quantize_col(wtype, x[c])), f"column {c} left in act_out"
+            y2 = gpu.buffer(np.float32, rows * m).fill_bytes(0xFF)
+            gpu.enqueue_gemv(wd, act, m, y2)  # the columns it left are whole: tables and all
+            assert np.array_equal(y2.download().view(np.uint32), y.download().view(np.uint32))
+            y2.free()
+            act.free()
+        y.free()
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    x[0, 5] = np.nan
+    xd.upload(x)
+    y = gpu.buffer(np.float32, rows)
+    gpu.enqueue_gemv_x(wd, xd, 1, y)
+    assert (gpu.fault()[0] & 0xFF) == bm.SITE_QUANT_COLUMN
+    gpu.fault_clear()
+    with pytest.raises(bm.GpuError) as e:
+        gpu.enqueue_gemv_x(wd, xd, 0, y)
+    assert e.value.code == bm.ESHAPE
+    for b in (wd, xd, y):
+        b.free()
+
+
 def test_extreme_blocks(gpu):
     """Every code at its ends, zero, subnormal and negative block scales (crates/qdot/tests/qdot.rs:2615-2655)."""
     rng = np.random.default_rng(44)

@@ -134,8 +134,9 @@ hipError_t q82_tables(const Launch &L, uint8_t *act, int m, int k) {
 
 // ------------------------------------------------------------------------------------------------ gemv
 
-// y[row * m_total + col0 + c] = row . column (col0 + c), c < m <= 8. A quad a row, 64 rows a workgroup.
-template <int WT, int U, int NB>
+// y[row * m_total + col0 + c] = row . column (col0 + c), c < m <= M. A quad a row, 64 rows a workgroup. M = 1 is the
+// one-column form of the row dot, which reads a super-block's activation operands a super-block ahead.
+template <int WT, int U, int NB, int M>
 __global__ __launch_bounds__(256) void k_gemv(const uint8_t *w, long rows, int nb, const uint8_t *act, int m_total,
                                               int col0, int m, float *y) {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -152,11 +153,11 @@ __global__ __launch_bounds__(256) void k_gemv(const uint8_t *w, long rows, int n
     uint8_t *cols = lds + tab_bytes<WT>();
     stage_bytes(cols, act + (size_t)col0 * col_bytes, m * col_bytes);
     __syncthreads();
-    float out[8];
-    row_dot<WT, U, NB, 8>(b, wrow, cols, col_bytes, m, n, q, tb, out, NoTap{});
+    float out[M];
+    row_dot<WT, U, NB, M>(b, wrow, cols, col_bytes, m, n, q, tb, out, NoTap{});
     if (q == 0 && active) {
 #pragma unroll
-        for (int c = 0; c < 8; c++)
+        for (int c = 0; c < M; c++)
             if (c < m) y[(size_t)row * m_total + col0 + c] = out[c];
     }
 }
@@ -821,7 +822,7 @@ hipError_t gemv(const Launch &L, int wtype, const uint8_t *w, int64_t rows, int 
     const int nb = k / 256;
     const size_t lds = tab_bytes_rt(wtype) + (size_t)m * act_col_bytes(wtype, k);
 #define CALL_BODY                                                                                                      \
-    auto kern = k_gemv<WT, U, NB>;                                                                                     \
+    auto kern = m == 1 ? k_gemv<WT, U, NB, 1> : k_gemv<WT, U, NB, 8>;                                                  \
     hipError_t e = allow_lds(kern, lds);                                                                               \
     if (e != hipSuccess) return e;                                                                                     \
     hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 63) / 64)), dim3(256), lds, L.stream, w, (long)rows, nb, act,     \

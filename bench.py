@@ -234,8 +234,7 @@ def bench_grouped(args, bm, ora, threads):
         dg, du, dd = layers[i % len(layers)]
         s_ptr = sel.ptr + 4 * st * n_slots
         if "tables" in which:
-            gpu.enqueue_buckets(s_ptr, n_slots, N_EXPERTS, order, start)
-            gpu.enqueue_tiles(start, N_EXPERTS, n_slots, tiles)
+            gpu.enqueue_tables(s_ptr, n_slots, N_EXPERTS, order, start, tiles)
         if "quant" in which:
             gpu.enqueue_quantize(xd.ptr + 4 * st * m * HIDDEN, m, act)
         if "gate_up" in which:
@@ -263,7 +262,7 @@ def bench_grouped(args, bm, ora, threads):
          "Qwen3-30B-A3B-shaped MoE layer, batched decode of 16 tokens grouped by expert, router logits N(0,1) + expert bias "
          "N(0,0.5) (BASELINE.json configs[2])",
          {"event_ms_per_step": ev, "kernel_us": kernel_us, "parity": parity, "distinct_experts_per_step": float(hit),
-          "algorithmic_bytes_per_step": nbytes, "hbm_tbps": nbytes / (wall * 1e-3) / 1e12, "launches_per_step": 6},
+          "algorithmic_bytes_per_step": nbytes, "hbm_tbps": nbytes / (wall * 1e-3) / 1e12, "launches_per_step": 5},
          {"bound": "hbm", "kernel": "k_gate_up_tiles<Q4_K>", "achieved": ach,
           "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None}, cpu)
     gpu.close()
@@ -379,8 +378,7 @@ def bench_dsv3(args, bm, ora, threads):
         st = i % sets
         s_ptr, x_ptr = sel.ptr + 4 * st * n_slots, xd.ptr + 4 * st * m * hidden
         if "routed" in which:
-            gpu.enqueue_buckets(s_ptr, n_slots, n_experts, order, start)
-            gpu.enqueue_tiles(start, n_experts, n_slots, tiles)
+            gpu.enqueue_tables(s_ptr, n_slots, n_experts, order, start, tiles)
             gpu.enqueue_quantize(x_ptr, m, act)
             gpu.enqueue_gate_up_tiles(dg, du, act, order, start, tiles, n_slots, ff, TOP_K, h)
             gpu.enqueue_quantize_ord(h, start, n_experts, n_slots, act_h)
@@ -413,7 +411,7 @@ def bench_dsv3(args, bm, ora, threads):
          "Q6_K shared expert; random legal blocks (BASELINE.json configs[4])",
          {"event_ms_per_step": ev, "kernel_us": kernel_us, "parity": parity, "distinct_experts_per_step": float(hit),
           "algorithmic_bytes_per_step": nbytes, "hbm_tbps": ach / 1e3},
-         {"bound": "hbm", "kernel": "whole step (11 launches)", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+         {"bound": "hbm", "kernel": "whole step (10 launches)", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
           "frac": ach / HBM_PEAK_GBS, "traffic": None}, cpu)
     gpu.close()
 

@@ -619,6 +619,16 @@ int bm_tiles(bm_ctx *ctx, const uint32_t *start_dev, int n_experts, int n_slots,
     return driver(ctx, what, bmk::tiles(launch_of(ctx), start_dev, n_experts, n_slots, tiles_dev));
 }
 
+int bm_tables(bm_ctx *ctx, const uint32_t *sel_dev, int n_slots, int n_experts, uint32_t *order_dev, uint32_t *start_dev,
+              uint32_t *tiles_dev) {
+    const char *what = "bm_tables";
+    if (!ctx || !sel_dev || !order_dev || !start_dev || !tiles_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (n_experts < 1 || n_experts > bmk::kBucketExperts || n_slots < 1 || n_slots > bmk::kTileMaxSlots)
+        return fail(ctx, BM_ESHAPE, "%s: %d places over %d experts (1..=%d experts, 1..=%d places)", what, n_slots, n_experts,
+                    bmk::kBucketExperts, bmk::kTileMaxSlots);
+    return driver(ctx, what, bmk::tables(launch_of(ctx), sel_dev, n_slots, n_experts, order_dev, start_dev, tiles_dev));
+}
+
 int bm_quantize_ord(bm_ctx *ctx, const float *x_dev, const uint32_t *start_dev, int n_experts, int m_cols, bm_act *act) {
     const char *what = "bm_quantize_ord";
     if (!ctx || !x_dev || !start_dev || !act) return fail(ctx, BM_EARG, "%s: NULL argument", what);

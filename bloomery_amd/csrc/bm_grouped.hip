@@ -32,8 +32,8 @@ __global__ __launch_bounds__(1024) void k_buckets(const u32 *sel, u32 n_slots, u
 
 // crates/gpu/src/q4k_sel.rs:562-680 grouped_tiles. A run outside 0 .. start[n_experts] <= n_slots, or more tiles
 // than `cap`, raise ExpertId and leave a count of 0.
-__global__ __launch_bounds__(1024) void k_tiles(const u32 *start, u32 n_experts, u32 n_slots, u32 cap, u32 *tiles,
-                                                u32 *fault, u32 layer) {
+__device__ __forceinline__ void tiles_body(const u32 *start, u32 n_experts, u32 n_slots, u32 cap, u32 *tiles, u32 *fault,
+                                           u32 layer) {
     __shared__ u32 scan[17];
     __shared__ u32 bad;
     const u32 tid = threadIdx.x;
@@ -58,6 +58,34 @@ __global__ __launch_bounds__(1024) void k_tiles(const u32 *start, u32 n_experts,
     }
     if (tid < n_experts && !refuse)
         for (u32 j = j0; j < j1; j += kTileCols) tiles[1 + g++] = (tid << kTileExpertShift) | j;
+}
+
+__global__ __launch_bounds__(1024) void k_tiles(const u32 *start, u32 n_experts, u32 n_slots, u32 cap, u32 *tiles,
+                                                u32 *fault, u32 layer) {
+    tiles_body(start, n_experts, n_slots, cap, tiles, fault, layer);
+}
+
+// k_buckets, then k_tiles over the runs it has just written: the grouped step's two table launches as one.
+__global__ __launch_bounds__(1024) void k_tables(const u32 *sel, u32 n_slots, u32 n_experts, u32 cap, u32 *order, u32 *start,
+                                                 u32 *tiles, u32 *fault, u32 layer) {
+    __shared__ GroupLds g;
+    group_slots(g, n_slots, n_experts, order, [&](u32 s) {
+        const u32 p = sel[s];
+        if (p < n_experts) return p;
+        if (p != kHostSlot) bm_raise(fault, layer, kSiteExpertId);
+        return kNoBucket;
+    });
+    for (u32 e = threadIdx.x; e <= n_experts; e += blockDim.x) start[e] = g.base[e];
+    __threadfence_block();
+    __syncthreads(); // the runs are the workgroup's own writes: visible to it past the barrier
+    tiles_body(start, n_experts, n_slots, cap, tiles, fault, layer);
+}
+
+hipError_t tables(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start,
+                  uint32_t *tiles_out) {
+    hipLaunchKernelGGL(k_tables, dim3(1), dim3(1024), 0, L.stream, sel, (u32)n_slots, (u32)n_experts,
+                       (u32)tile_cap(n_slots, n_experts), order, start, tiles_out, L.fault, L.layer);
+    return hipGetLastError();
 }
 
 hipError_t buckets(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start) {

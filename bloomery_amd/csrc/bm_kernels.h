@@ -92,6 +92,9 @@ int tile_cap(int n_slots, int n_experts);
 
 hipError_t buckets(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start);
 hipError_t tiles(const Launch &L, const uint32_t *start, int n_experts, int n_slots, uint32_t *tiles);
+// buckets, then tiles, in one launch
+hipError_t tables(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start,
+                  uint32_t *tiles);
 // LDS bytes a tile launch of this type and k asks for (0 if eight columns do not fit a workgroup's LDS).
 size_t tiles_lds(int wtype, int k);
 hipError_t gate_up_tiles(const Launch &L, int wtype, const uint8_t *wg, const uint8_t *wu, int n_experts, int k,

@@ -230,6 +230,9 @@ int bm_buckets(bm_ctx *ctx, const uint32_t *sel_dev, int n_slots, int n_experts,
 /* Q4kSelKernels::enqueue_grouped_tiles (crates/gpu/src/q4k_sel.rs:1152): the tile table of start_dev. A run
  * outside the table raises BM_SITE_EXPERT_ID and leaves a count of 0. */
 int bm_tiles(bm_ctx *ctx, const uint32_t *start_dev, int n_experts, int n_slots, uint32_t *tiles_dev);
+/* bm_buckets then bm_tiles as one launch: order_dev, start_dev and tiles_dev hold what the two calls would leave. */
+int bm_tables(bm_ctx *ctx, const uint32_t *sel_dev, int n_slots, int n_experts, uint32_t *order_dev, uint32_t *start_dev,
+              uint32_t *tiles_dev);
 /* Q4kSelKernels::enqueue_quantize_ord (crates/gpu/src/q4k_sel.rs:1255): the first start_dev[n_experts] columns
  * of x_dev (at most m_cols, the columns launched) into the same columns of act, bm_quantize's bytes; every other
  * column keeps what it held. */

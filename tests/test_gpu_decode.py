@@ -607,7 +607,13 @@ def test_grouped_tables_are_the_definition(gpu, n_experts, n_slots, seed):
     got_tiles = tiles.download()
     assert got_tiles[0] == want_tiles[0] and np.array_equal(got_tiles[1:1 + got_tiles[0]], want_tiles[1:1 + want_tiles[0]])
     assert not refused and gpu.fault() == (bm.FAULT_NONE, 0)
-    for b in (sel, order, start, tiles):
+    # the two launches as one leave the same three tables
+    o2, s2 = gpu.buffer(np.uint32, n_slots).fill_bytes(0), gpu.buffer(np.uint32, n_experts + 1).fill_bytes(0xFF)
+    t2 = gpu.buffer(np.uint32, gpu.tile_cap(n_slots, n_experts) + 1).fill_bytes(0)
+    gpu.enqueue_tables(sel, n_slots, n_experts, o2, s2, t2)
+    assert np.array_equal(s2.download(), want_start) and np.array_equal(o2.download()[:listed], want_order[:listed])
+    assert np.array_equal(t2.download()[:1 + got_tiles[0]], got_tiles[:1 + got_tiles[0]]) and gpu.fault() == (bm.FAULT_NONE, 0)
+    for b in (sel, order, start, tiles, o2, s2, t2):
         b.free()
 
 

@@ -252,6 +252,19 @@ def bench_grouped(args, bm, ora, threads):
     step(0)  # leave set 0's tables for the single-kernel graphs
     kernel_us = {k: timed_graph(gpu, lambda i, k=k: step(i - i % sets, (k,)) if k in ("gate_up", "down") else step(i, (k,)),
                                 64, 512, 64)[1] * 1e3 for k in ("tables", "quant", "gate_up", "down", "combine")}
+    # the same 16 tokens through the per-slot fused step (bm_moe_decode, two launches): every slot reads its expert's rows
+    # for itself, repeats come from the caches
+    y2 = gpu.buffer(np.float32, m * sets * HIDDEN)
+
+    def per_slot(i):
+        st = i % sets
+        dg, du, dd = layers[i % len(layers)]
+        gpu.enqueue_moe_decode(dg, du, dd, xd.ptr + 4 * st * m * HIDDEN, sel.ptr + 4 * st * n_slots, wt.ptr + 4 * st * n_slots, None,
+                               TOP_K, m, act_h, y2.ptr + 4 * st * m * HIDDEN)
+
+    per_slot(0)
+    per_slot_parity = parity_of(y2.download()[:m * HIDDEN].reshape(m, HIDDEN), want)
+    per_slot_us = timed_graph(gpu, per_slot, 64, 512, 64)[1] * 1e3
     hit = np.mean([len(np.unique(ids[s * m:(s + 1) * m])) for s in range(sets)])
     per_expert = 2 * FF * bm.row_bytes(bm.Q4_K, HIDDEN) + HIDDEN * bm.row_bytes(bm.Q6_K, FF)
     nbytes = hit * per_expert
@@ -262,7 +275,9 @@ def bench_grouped(args, bm, ora, threads):
          "Qwen3-30B-A3B-shaped MoE layer, batched decode of 16 tokens grouped by expert, router logits N(0,1) + expert bias "
          "N(0,0.5) (BASELINE.json configs[2])",
          {"event_ms_per_step": ev, "kernel_us": kernel_us, "parity": parity, "distinct_experts_per_step": float(hit),
-          "algorithmic_bytes_per_step": nbytes, "hbm_tbps": nbytes / (wall * 1e-3) / 1e12, "launches_per_step": 5},
+          "algorithmic_bytes_per_step": nbytes, "hbm_tbps": nbytes / (wall * 1e-3) / 1e12, "launches_per_step": 5,
+          "per_slot_two_launches": {"us_per_step": per_slot_us, "us_per_token": per_slot_us / m, "parity": per_slot_parity,
+                                    "note": "bm_moe_decode over the same tokens: not grouped, each slot streams its expert"}},
          {"bound": "hbm", "kernel": "k_gate_up_tiles<Q4_K>", "achieved": ach,
           "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None}, cpu)
     gpu.close()

@@ -415,6 +415,21 @@ def bench_dsv3(args, bm, ora, threads):
     parity = parity_of(y.download()[:m * hidden].reshape(m, hidden), want)
     wall, ev, steps, warm = timed_graph(gpu, step, 16, min(args.steps, 256), min(args.warmup, 32))
     kernel_us = {k: timed_graph(gpu, lambda i, k=k: step(i, (k,)), 16, 64, 16)[1] * 1e3 for k in ("routed", "shared", "combine")}
+    # the same tokens through the per-slot fused step: the shared expert first, its rows the term bm_moe_decode adds to
+    # the slots' sum ((sum + shared), the same grouping); five launches, no tables
+    y2 = gpu.buffer(np.float32, m * sets * hidden)
+
+    def per_slot(i):
+        st = i % sets
+        s_ptr, x_ptr = sel.ptr + 4 * st * n_slots, xd.ptr + 4 * st * m * hidden
+        gpu.enqueue_quantize(x_ptr, m, act6)
+        gpu.enqueue_gate_up(dsg, dsu, act6, zeros, m, ff, 1, None, act_sh)
+        gpu.enqueue_gemv_sel(dsd, act_sh, zeros, m, hidden, sdown)
+        gpu.enqueue_moe_decode(dg, du, dd, x_ptr, s_ptr, wt.ptr + 4 * st * n_slots, sdown, TOP_K, m, act_h, y2.ptr + 4 * st * m * hidden, h=h)
+
+    per_slot(0)
+    per_slot_parity = parity_of(y2.download()[:m * hidden].reshape(m, hidden), want)
+    per_slot_us = timed_graph(gpu, per_slot, 16, 128, 16)[1] * 1e3
     hit = np.mean([len(np.unique(ids[s * m:(s + 1) * m])) for s in range(sets)])
     per_expert = (2 * ff * bm.row_bytes(bm.IQ2_XXS, hidden) + hidden * bm.row_bytes(bm.IQ2_XXS, ff))
     shared_bytes = 2 * ff * bm.row_bytes(bm.Q6_K, hidden) + hidden * bm.row_bytes(bm.Q6_K, ff)
@@ -425,7 +440,9 @@ def bench_dsv3(args, bm, ora, threads):
          "DeepSeek-V3-shaped MoE layer decode, 4 tokens: hidden 7168, 256 IQ2_XXS experts of ff 2048 top-8 grouped by expert + one "
          "Q6_K shared expert; random legal blocks (BASELINE.json configs[4])",
          {"event_ms_per_step": ev, "kernel_us": kernel_us, "parity": parity, "distinct_experts_per_step": float(hit),
-          "algorithmic_bytes_per_step": nbytes, "hbm_tbps": ach / 1e3},
+          "algorithmic_bytes_per_step": nbytes, "hbm_tbps": ach / 1e3,
+          "per_slot_five_launches": {"us_per_step": per_slot_us, "us_per_token": per_slot_us / m, "parity": per_slot_parity,
+                                     "note": "shared expert, then bm_moe_decode over the slots with its rows as the added term"}},
          {"bound": "hbm", "kernel": "whole step (10 launches)", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
           "frac": ach / HBM_PEAK_GBS, "traffic": None}, cpu)
     gpu.close()

@@ -107,14 +107,20 @@ hipError_t tiles(const Launch &L, const uint32_t *start, int n_experts, int n_sl
 // that names no run of the table, which raises ExpertId).
 struct Tile {
     int e, j, m, row_block;
+    u32 entry; // threads 0 .. 7: order[j + thread] (0 past the table), requested together with the run's end
 };
-__device__ __forceinline__ bool tile_of_block(const u32 *tiles, const u32 *start, u32 n_experts, u32 n_slots, u32 cap,
-                                              Tile *t, u32 *fault, u32 layer) {
+// The lookups are a chain of memory round trips in front of everything a workgroup does, so each step asks for all it
+// can: the count and the word together (the table holds cap + 1 words, so word g is there whatever the count), then
+// the run's end together with the tile's entries of `order`.
+__device__ __forceinline__ bool tile_of_block(const u32 *tiles, const u32 *start, const u32 *order, u32 n_experts, u32 n_slots,
+                                              u32 cap, Tile *t, u32 *fault, u32 layer) {
     const u32 g = blockIdx.x % cap;
     t->row_block = (int)(blockIdx.x / cap);
-    if (g >= tiles[0]) return false;
-    const u32 word = tiles[1 + g];
+    const u32 count = tiles[0], word = tiles[1 + g];
+    if (g >= count) return false;
     const u32 e = word >> kTileExpertShift, j = word & ((1u << kTileExpertShift) - 1);
+    const u32 at = j + threadIdx.x;
+    t->entry = threadIdx.x < (u32)kTileCols && at < n_slots ? order[at] : 0;
     const u32 j1 = e < n_experts ? start[e + 1] : 0;
     if (!(j < j1 && j1 <= n_slots)) {
         if (threadIdx.x == 0) bm_raise(fault, layer, kSiteExpertId);
@@ -151,7 +157,7 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
     Tile t;
-    if (!tile_of_block(tiles, start, n_experts, n_slots, cap, &t, fault, layer)) return; // raising twice is raising once
+    if (!tile_of_block(tiles, start, order, n_experts, n_slots, cap, &t, fault, layer)) return; // raising twice is raising once
     if (t.m <= m_lo || t.m > MC) return;
     const int rb = t.row_block;
     const int r = rb * 32 + (tid >> 3);
@@ -168,7 +174,7 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
     float *hbuf = reinterpret_cast<float *>(cols + (size_t)MC * col_bytes); // [MC][32]
     u32 *bad = reinterpret_cast<u32 *>(hbuf + MC * 32);                      // [MC]: entry names no slot
     if (tid < MC) {
-        const u32 s = tid < t.m ? order[t.j + tid] : 0;
+        const u32 s = tid < t.m ? t.entry : 0;
         const bool none = tid < t.m && (s >= n_slots || (int)(s / slots_per_col) >= act_cols);
         if (none) bm_raise(fault, layer, kSiteExpertId);
         bad[tid] = none ? 0xffffffffu : s / slots_per_col;
@@ -205,7 +211,7 @@ __global__ __launch_bounds__(256) void k_gemv_tiles(const uint8_t *w, u32 n_expe
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, q = tid & 3;
     Tile t;
-    if (!tile_of_block(tiles, start, n_experts, n_slots, cap, &t, fault, layer)) return;
+    if (!tile_of_block(tiles, start, order, n_experts, n_slots, cap, &t, fault, layer)) return;
     if (t.m <= m_lo || t.m > MC) return;
     const int r = t.row_block * 64 + (tid >> 2);
     const bool active = r < rpe;
@@ -219,7 +225,7 @@ __global__ __launch_bounds__(256) void k_gemv_tiles(const uint8_t *w, u32 n_expe
     uint8_t *cols = lds + tab_bytes<WT>();
     u32 *slot_of = reinterpret_cast<u32 *>(cols + (size_t)MC * col_bytes); // [MC]
     if (tid < MC) {
-        const u32 s = tid < t.m ? order[t.j + tid] : 0;
+        const u32 s = tid < t.m ? t.entry : 0;
         if (tid < t.m && s >= n_slots && t.row_block == 0) bm_raise(fault, layer, kSiteExpertId);
         slot_of[tid] = s;
     }

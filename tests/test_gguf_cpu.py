@@ -238,3 +238,13 @@ def test_a_split_sets_first_shard_must_carry_the_sets_name(tmp_path):
     with pytest.raises(bm.GpuError) as e:
         bm.Gguf(odd, split=True)
     assert "does not end in -00001-of-00003.gguf" in str(e.value)
+
+
+def test_a_set_of_a_dozen_shards(tmp_path):
+    """Two-digit shard numbers: the siblings' names are zero-padded to five digits on both sides of "-of-"."""
+    first, made = split_set(str(tmp_path), count=12, per=(1,) * 12, prefix="big.model-v2")
+    assert first.endswith("big.model-v2-00001-of-00012.gguf") and os.path.exists(first.replace("-00001-", "-00012-"))
+    g = bm.Gguf(first, split=True)
+    assert [t["name"] for t in g.tensors()] == [f"blk.{i}.w" for i in range(12)]
+    assert np.array_equal(g.data("blk.11.w"), made["blk.11.w"])
+    g.close()

@@ -720,6 +720,24 @@ def main():
         gpu.graph_destroy(g1)
     gate_up_bytes = TOP_K * 2 * FF * bm.row_bytes(gate_t, HIDDEN)
     down_bytes = TOP_K * HIDDEN * bm.row_bytes(down_t, FF)
+    # what the launches' times are to be read against, measured here: an empty launch, and launches that only fetch the
+    # gate . up launch's bytes (cold: a different part of a different layer copy each time) with plain loads
+    sink = gpu.buffer(np.uint32, 4096)
+    stack_bytes = N_EXPERTS * FF * bm.row_bytes(gate_t, HIDDEN)
+    spans = max(1, stack_bytes // gate_up_bytes)
+
+    def plain_read(n_wg, nbytes):
+        def enqueue(i):
+            base = layers[i % len(layers)][(i // len(layers)) % 2].dev_ptr
+            gpu.enqueue_probe_read(base + ((i * 5) % spans) * gate_up_bytes, nbytes, n_wg, sink)
+        return timed_graph(gpu, enqueue, 64, 1024, 64)[1] * 1e3
+
+    calibration = {"empty_launch_us": plain_read(192, 0),
+                   "plain_read_of_gate_up_bytes_us": {str(n): plain_read(n, gate_up_bytes) for n in (192, 256, 1024)},
+                   "note": "bm_probe_read under the same graph replay: n workgroups fetch the gate . up launch's "
+                           f"{gate_up_bytes} bytes and do nothing else"}
+    best = min(calibration["plain_read_of_gate_up_bytes_us"].values())
+    calibration["plain_read_gbps"] = gate_up_bytes / (best * 1e-6) / 1e9
     if single:
         dominant, dom_bytes = "k_moe_decode<Q4_K, Q6_K>", bytes_per_token
         achieved = dom_bytes / (kernel_us["step"] * 1e-6) / 1e9
@@ -776,6 +794,7 @@ def main():
         "kernel_us": kernel_us,
         "kernel_gbps": kernel_gbps,
         "router_kernel_us": router_us,
+        "calibration": calibration,
         "parity": parity,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,

@@ -60,6 +60,7 @@ SYMBOLS = {
     "bm_quantize": (_i, [_vp, _vp, _i, _vp]),
     "bm_gemv": (_i, [_vp, _vp, _vp, _i, _vp]),
     "bm_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
+    "bm_probe_read": (_i, [_vp, _vp, C.c_size_t, _i, _vp]),
     "bm_tables": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp]),
     "bm_gemv_x": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
     "bm_gemv_sel": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
@@ -564,6 +565,10 @@ class Gpu:
         self._check(self.lib.bm_router_logits(self.ctx, _ptr(router), _ptr(x), _ptr(gain) if gain is not None else None,
                                               float(eps), n_tokens, n_experts, hidden,
                                               _ptr(normed) if normed is not None else None, _ptr(logits)))
+
+    def enqueue_probe_read(self, src, nbytes, n_workgroups, sink):
+        """Measurement only: a launch that fetches nbytes with plain loads (0: an empty launch)."""
+        self._check(self.lib.bm_probe_read(self.ctx, _ptr(src), nbytes, n_workgroups, _ptr(sink)))
 
     def enqueue_block_sums(self, w, row, act, col, out):
         self._check(self.lib.bm_block_sums(self.ctx, w.handle, row, act.handle, col, _ptr(out)))

@@ -917,6 +917,14 @@ int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *a
     return driver(ctx, what, bmk::block_sums(launch_of(ctx), w->wtype, wrow, w->k, c, out_dev));
 }
 
+int bm_probe_read(bm_ctx *ctx, const void *src_dev, size_t bytes, int n_workgroups, uint32_t *sink_dev) {
+    const char *what = "bm_probe_read";
+    if (!ctx || !sink_dev || (!src_dev && bytes)) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (bytes % 16 != 0 || ((uintptr_t)src_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: %zu bytes at %p: both multiples of 16", what, bytes, src_dev);
+    if (n_workgroups < 1 || n_workgroups > 65536) return fail(ctx, BM_ESHAPE, "%s: %d workgroups (1 .. 65536)", what, n_workgroups);
+    return driver(ctx, what, bmk::probe_read(launch_of(ctx), src_dev, bytes, n_workgroups, sink_dev));
+}
+
 // ------------------------------------------------------------------------------------ the card rule
 
 static int check_card_planes(bm_ctx *ctx, const char *what, const void *codes, const void *d8, const void *s8) {

@@ -27,6 +27,8 @@ struct Launch {
 constexpr int kMaxLds = 160 * 1024;
 
 hipError_t fill_u32(const Launch &L, uint32_t *dst, uint32_t value, size_t n);
+// Measurement only: n_wg workgroups read `bytes` with plain loads (bytes = 0: an empty launch); sink holds n_wg words.
+hipError_t probe_read(const Launch &L, const void *src, size_t bytes, int n_wg, uint32_t *sink);
 
 // Bytes of one activation column of k values on the device, in the form weight type `wtype` dots against: the CPU
 // path's bytes, and for the Q8_2_X4 form two tables after them (bm_device.cuh).

@@ -14,6 +14,30 @@ __global__ void k_fill_u32(u32 *dst, u32 value, size_t n) {
     if (i < n) dst[i] = value;
 }
 
+// Measurement only: n_wg workgroups read `bytes` (a multiple of 16) as plain 16-byte loads, workgroup b the b-th equal
+// share, four loads a thread in flight, and leave one word a workgroup in `sink`. With bytes = 0 it is an empty launch.
+// What a decode launch's time is to be read against: its bytes fetched by a kernel that does nothing else.
+__global__ __launch_bounds__(256) void k_probe_read(const uint4 *src, size_t n16, u32 *sink) {
+    const size_t per = (n16 + gridDim.x - 1) / gridDim.x;
+    const size_t lo = per * blockIdx.x, hi = lo + per < n16 ? lo + per : n16;
+    u32 acc = 0;
+    size_t i = lo + threadIdx.x;
+    for (; i + 768 < hi; i += 1024) {
+        const uint4 a = src[i], b = src[i + 256], c = src[i + 512], d = src[i + 768];
+        acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    }
+    for (; i < hi; i += 256) {
+        const uint4 a = src[i];
+        acc ^= a.x ^ a.y ^ a.z ^ a.w;
+    }
+    if (acc == 0x9e3779b9u && threadIdx.x == 0) sink[blockIdx.x] = acc; // the loads must happen; the store almost never does
+}
+
+hipError_t probe_read(const Launch &L, const void *src, size_t bytes, int n_wg, uint32_t *sink) {
+    hipLaunchKernelGGL(k_probe_read, dim3((unsigned)n_wg), dim3(256), 0, L.stream, static_cast<const uint4 *>(src), bytes / 16, sink);
+    return hipGetLastError();
+}
+
 hipError_t fill_u32(const Launch &L, uint32_t *dst, uint32_t value, size_t n) {
     if (n == 0) return hipSuccess;
     hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, L.stream, dst, value, n);

@@ -398,6 +398,12 @@ int bm_weights_from_gguf(bm_ctx *ctx, const bm_gguf *g, const char *name, bm_wei
 
 /* ------------------------------------------------------------------------------------------- verification */
 
+/* Measurement only (no counterpart in the reference): n_workgroups workgroups fetch `bytes` from src_dev with plain
+ * 16-byte loads and do nothing else; with bytes = 0 it is an empty launch. The time of a decode launch is to be read
+ * against this: the same bytes by a kernel without arithmetic, tables or dependent reads. sink_dev: n_workgroups words. */
+int bm_probe_read(bm_ctx *ctx, const void *src_dev, size_t bytes, int n_workgroups, uint32_t *sink_dev);
+
+
 /* The exact per-block integers the kernels above form for row `row` of w against column `col` of act, written
  * to out_dev as i32, through the same device code the launchers run:
  *   Q4_K, Q5_K: per super-block 8 sums A[s] = sum q * a over sub-block s (q the 4- or 5-bit code), then the 8

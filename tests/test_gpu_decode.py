@@ -843,3 +843,22 @@ def test_shape_refusals_are_named(gpu):
         assert e.value.code == code and word in str(e.value), str(e.value)
     for b in (w4, a512, a256, aq8k, buf, sel):
         b.free()
+
+
+def test_probe_read_runs_and_refuses_by_name(gpu):
+    """bm_probe_read is a measurement launch: it fetches and leaves the source as it is; its geometry is checked."""
+    src = gpu.upload(np.arange(1 << 16, dtype=np.uint32), np.uint32)
+    sink = gpu.buffer(np.uint32, 64).fill_bytes(0)
+    gpu.enqueue_probe_read(src, 0, 64, sink)
+    gpu.enqueue_probe_read(src, 4 << 16, 64, sink)
+    gpu.enqueue_probe_read(src, 4096 + 16, 7, sink)
+    gpu.sync()
+    assert np.array_equal(src.download(), np.arange(1 << 16, dtype=np.uint32))
+    for call, word in ((lambda: gpu.enqueue_probe_read(src, 24, 4, sink), "multiples of 16"),
+                       (lambda: gpu.enqueue_probe_read(src.ptr + 4, 64, 4, sink), "multiples of 16"),
+                       (lambda: gpu.enqueue_probe_read(src, 64, 0, sink), "workgroups")):
+        with pytest.raises(bm.GpuError) as e:
+            call()
+        assert e.value.code == bm.ESHAPE and word in str(e.value)
+    src.free()
+    sink.free()

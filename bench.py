@@ -506,6 +506,9 @@ def bench_card(args, bm, ora, threads):
     gpu.enqueue_card_quantize(xb, 1, k_big, cb, db, sb)
     big_ms = timed_graph(gpu, lambda i: gpu.enqueue_card_gemv(big[i % 4], cb, db, sb, 1, yb), 8, 64, 8)[1]
     big_gbs = rows_big * bm.row_bytes(bm.Q4_K, k_big) / (big_ms * 1e-3) / 1e9
+    cq, dq, sq, _ = ora.card_q8_1(xb.download())
+    rb = bm.row_bytes(bm.Q4_K, k_big)
+    big_parity = parity_of(yb.download()[-64:], ora.card_gemv(ora.Q4_K, wb[-64 * rb:], 64, k_big, cq, dq, sq))
     cpu = None
     if not args.no_cpu:
         n, t0 = 0, time.perf_counter()
@@ -520,7 +523,7 @@ def bench_card(args, bm, ora, threads):
          "the card rule's MoE down step: 8 slots x 768 values, q8_1 quantizer + 32-lane Q4_K walks over 2048 rows of 8 of 128 "
          "experts; random legal blocks (not a BASELINE.json configuration)",
          {"event_ms_per_step": ev, "kernel_us": kernel_us, "parity": parity, "algorithmic_bytes_per_launch": nbytes,
-          "large_gemv": {"rows": rows_big, "k": k_big, "ms": big_ms, "gb_per_s": big_gbs}},
+          "large_gemv": {"rows": rows_big, "k": k_big, "ms": big_ms, "gb_per_s": big_gbs, "parity_last_64_rows": big_parity}},
          {"bound": "hbm", "kernel": "k_card_gemv_sel<Q4_K>", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
           "frac": ach / HBM_PEAK_GBS, "traffic": None}, cpu)
     gpu.close()

@@ -14,6 +14,10 @@
 //   dequantizers    the reference's ggml-made IQ2_XXS block (66 bytes -> 256 f32 bit patterns), table digests,
 //                   independent decoders written from the layout text in the test suite (all five types);
 //   expf / SwiGLU   libm band and special-case paths;
+//   card rule       (card.c) the quantizer by the worked cases of the reference's own test (ties, near ties, the clamp,
+//                   zero / subnormal / underflowed scales, refused blocks, the sums) and a numpy restatement; the
+//                   32-lane walks by a second spelling from the device's loops over independently decoded blocks,
+//                   one-lane rows that separate the split order from the fused one, and the reference test's f64 band;
 //   weight quantizers   PARITY UNPINNED as bytes: the reference holds no golden bytes for them (it pins them
 //                   against ggml on its own machine). They are held to the reference tests' round-trip bounds,
 //                   zero-row and on-grid properties. Their output is an input shared by the oracle and the GPU

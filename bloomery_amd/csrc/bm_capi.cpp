@@ -479,18 +479,15 @@ int bm_down_combine_h(bm_ctx *ctx, const bm_weights *w, const float *h_dev, bm_a
                       float *y_dev) {
     const char *what = "bm_down_combine_h";
     if (!ctx || !w || !h_dev || !sel_dev || !w_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
-    if (act_form(w->wtype) == 0)
-        return fail(ctx, BM_ETYPE, "%s: folds the Q8_K quantizer; weight type %d takes Q8_2_X4 columns, which bm_gate_up and "
-                    "bm_gate_up_x already write: use bm_down_combine", what, w->wtype);
     int n_experts = 0;
     int rc = check_stack(ctx, what, w, rows_per_expert, &n_experts);
     if (rc) return rc;
     if (n_slots_per_token < 1 || n_slots_per_token > bmk::kMaxCombineSlots)
         return fail(ctx, BM_ESHAPE, "%s: %d slots a token outside 1..=%d", what, n_slots_per_token, bmk::kMaxCombineSlots);
     if (m < 1) return fail(ctx, BM_ESHAPE, "%s: need m >= 1 tokens, got %d", what, m);
-    if (act_h && (act_form(act_h->wtype) != 1 || act_h->k != w->k || (int64_t)act_h->m_cap < (int64_t)m * n_slots_per_token))
-        return fail(ctx, BM_ESHAPE, "%s: act_h must hold %d Q8_K columns of k = %d; it holds %d of k = %d (type %d)", what,
-                    m * n_slots_per_token, w->k, act_h->m_cap, act_h->k, act_h->wtype);
+    if (act_h && (act_form(act_h->wtype) != act_form(w->wtype) || act_h->k != w->k || (int64_t)act_h->m_cap < (int64_t)m * n_slots_per_token))
+        return fail(ctx, BM_ESHAPE, "%s: act_h must hold %d columns of k = %d in the form type %d dots against; it holds %d of k = %d (type %d)",
+                    what, m * n_slots_per_token, w->k, w->wtype, act_h->m_cap, act_h->k, act_h->wtype);
     if (((uintptr_t)h_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: h_dev %p is not 16-byte aligned", what, (const void *)h_dev);
     const size_t lds = (size_t)n_slots_per_token * dev_col_bytes(w->wtype, w->k) + 12288;
     if (lds > (size_t)bmk::kMaxLds)

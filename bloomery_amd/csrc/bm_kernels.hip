@@ -648,6 +648,34 @@ __device__ __forceinline__ void q8k_stage_cols(const float *x, uint8_t *dst, int
     }
 }
 
+// `cols` columns of nb super-blocks each, f32 rows at x (column c at x + c * nb * 256), into LDS at `dst` as Q8_2_X4
+// columns with their tables: a 32-value block is four consecutive lanes of eight values; four blocks' loads a thread
+// are in flight before the first is encoded.
+__device__ __forceinline__ void q82_stage_cols(const float *x, uint8_t *dst, int cols, int nb, u32 *fault, u32 layer) {
+    const int per_col = nb * 32, total = cols * per_col; // tasks of eight values; a multiple of four a column
+    const int col_bytes = nb * BM_Q82_SB_EXT;
+    constexpr int kAhead = 4;
+    for (int t0 = threadIdx.x; t0 < total; t0 += kAhead * (int)blockDim.x) {
+        float4 lo[kAhead], hi[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; u++) {
+            const int task = t0 + u * (int)blockDim.x;
+            const float *p = x + (size_t)(task < total ? task : t0) * 8;
+            lo[u] = *reinterpret_cast<const float4 *>(p);
+            hi[u] = *reinterpret_cast<const float4 *>(p + 4);
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; u++) {
+            const int task = t0 + u * (int)blockDim.x;
+            if (task < total) { // whole quads: the tasks of a block are four neighbours
+                const int c = task / per_col, at = task % per_col;
+                const float v8[8] = {lo[u].x, lo[u].y, lo[u].z, lo[u].w, hi[u].x, hi[u].y, hi[u].z, hi[u].w};
+                q82_quad8(v8, dst + (size_t)c * col_bytes, nb, at >> 2, task & 3, fault, layer);
+            }
+        }
+    }
+}
+
 // k_gate_up_x for gate / up stacks that dot against Q8_K columns (Q3_K, IQ2_XXS, IQ3_XXS, IQ4_XS): the token's row is
 // quantized by every workgroup into LDS, h is written as f32 rows, and where the down stack takes Q8_2_X4 columns
 // (act_h given) the workgroup's 32 values also become their block of the slot's column.
@@ -761,7 +789,8 @@ __global__ __launch_bounds__(256) void k_down_combine_hq(const uint8_t *w, u32 n
     float *part = reinterpret_cast<float *>(cols + (size_t)spt * col_bytes); // [D][spt]
     float *s_w = part + D * spt;                                              // [spt]
     u32 *s_sel = reinterpret_cast<u32 *>(s_w + spt);                          // [spt]
-    q8k_stage_cols(h + (size_t)t * spt * n * 256, cols, spt, n, fault, layer);
+    if constexpr (bm_takes_q8k(WT)) q8k_stage_cols(h + (size_t)t * spt * n * 256, cols, spt, n, fault, layer);
+    else q82_stage_cols(h + (size_t)t * spt * n * 256, cols, spt, n, fault, layer);
     if (tid < spt) {
         s_w[tid] = my_w;
         s_sel[tid] = my_sel;
@@ -988,7 +1017,6 @@ hipError_t down_combine_hq(const Launch &L, int wtype, const uint8_t *w, int n_e
     const int D = 64 / spt;
     const size_t lds = down_combine_lds(wtype, k, spt);
     const unsigned grid = (unsigned)m * (unsigned)((rpe + D - 1) / D);
-    if (!bm_takes_q8k(wtype)) return hipErrorInvalidValue;
 #define CALL_BODY                                                                                                      \
     auto kern = k_down_combine_hq<WT, U, NB>;                                                                          \
     hipError_t e = allow_lds(kern, lds);                                                                               \

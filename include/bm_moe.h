@@ -173,10 +173,12 @@ int bm_down_combine(bm_ctx *ctx, const bm_weights *w, const bm_act *act, const u
                     const float *w_dev, const float *resid_dev, int n_slots_per_token, int m, int rows_per_expert,
                     float *y_dev);
 
-/* bm_quantize of the slots' f32 rows of h and bm_down_combine in one launch, for a down stack that takes Q8_K
- * columns (Q3_K and the IQ types; the K-quants on Q8_2_X4 columns get theirs from bm_gate_up / bm_gate_up_x): slot s
- * reads h_dev[s * k .. (s + 1) * k), k = w's k, 16-byte aligned. act_h (optional) receives the quantized columns.
- * Same bits as the two calls. No counterpart launch in the reference. */
+/* bm_quantize of the slots' f32 rows of h and bm_down_combine in one launch, in the column form w's type dots against.
+ * It is how a down stack on Q8_K columns (Q3_K and the IQ types) joins the fused step; for the K-quants on Q8_2_X4
+ * columns it serves a caller that holds f32 rows only (where bm_gate_up / bm_gate_up_x can write the columns, that is
+ * the faster way: every workgroup here quantizes its token's rows again). Slot s reads h_dev[s * k .. (s + 1) * k),
+ * k = w's k, 16-byte aligned. act_h (optional) receives the quantized columns. Same bits as the two calls. No
+ * counterpart launch in the reference. */
 int bm_down_combine_h(bm_ctx *ctx, const bm_weights *w, const float *h_dev, bm_act *act_h, const uint32_t *sel_dev,
                       const float *w_dev, const float *resid_dev, int n_slots_per_token, int m, int rows_per_expert,
                       float *y_dev);

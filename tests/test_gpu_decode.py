@@ -862,3 +862,42 @@ def test_probe_read_runs_and_refuses_by_name(gpu):
         assert e.value.code == bm.ESHAPE and word in str(e.value)
     src.free()
     sink.free()
+
+
+@pytest.mark.parametrize("down_type,hidden,ff,n_experts,m,top_k", ((bm.Q6_K, 2048, 768, 10, 3, 8), (bm.Q4_K, 512, 512, 5, 4, 2),
+                                                                    (bm.Q5_K, 768, 256, 4, 2, 3), (bm.IQ4_XS, 1024, 512, 6, 2, 4)))
+def test_down_combine_from_f32_rows_for_either_column_form(gpu, down_type, hidden, ff, n_experts, m, top_k):
+    """bm_down_combine_h quantizes the f32 rows of h itself, in the form the down stack dots against (Q8_2_X4 or Q8_K):
+    y and the columns it leaves in act_h are the oracle's, for a stack of either form; a row that is not finite raises
+    QuantColumn."""
+    rng = np.random.default_rng(900 + ff)
+    wd = stack(down_type, n_experts * hidden, ff, 901 + ff)
+    dd = gpu.weights(down_type, n_experts * hidden, ff, wd)
+    n_slots = m * top_k
+    h = normal_f32(rng, (n_slots, ff))
+    h[1] *= np.float32(1e-3)
+    ids, wts = route(rng, m, n_experts, top_k)
+    resid = normal_f32(rng, (m, hidden))
+    hd, sel, wt, rd = gpu.upload(h, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32), gpu.upload(resid, np.float32)
+    act_h = gpu.act(down_type, ff, n_slots)
+    y = gpu.buffer(np.float32, m * hidden).fill_bytes(0xFF)
+    gpu.fault_clear()
+    gpu.enqueue_down_combine_h(dd, hd, act_h, sel, wt, rd, top_k, m, hidden, y)
+    cols = [ora.quantize_col(down_type, h[s]) for s in range(n_slots)]
+    for s in range(n_slots):
+        assert np.array_equal(act_h.download(s), cols[s]), f"column {s}"
+    rb = ora.row_bytes(down_type, ff)
+    down = np.concatenate([ora.gemv(down_type, wd[int(ids.reshape(-1)[s]) * hidden * rb:], hidden, ff, cols[s]) for s in range(n_slots)])
+    assert_f32(y.download(), ora.combine_tokens(down, wts, resid, hidden, top_k, m), "y")
+    # against the launch that takes ready columns: the same bits
+    y2 = gpu.buffer(np.float32, m * hidden).fill_bytes(0xFF)
+    gpu.enqueue_down_combine(dd, act_h, sel, wt, rd, top_k, m, hidden, y2)
+    assert np.array_equal(y.download().view(np.uint32), y2.download().view(np.uint32))
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    h[0, 3] = np.inf
+    hd.upload(h)
+    gpu.enqueue_down_combine_h(dd, hd, None, sel, wt, rd, top_k, m, hidden, y)
+    assert (gpu.fault()[0] & 0xFF) == bm.SITE_QUANT_COLUMN
+    gpu.fault_clear()
+    for b in (dd, hd, sel, wt, rd, act_h, y, y2):
+        b.free()

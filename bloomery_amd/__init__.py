@@ -471,7 +471,7 @@ class Gpu:
                                              n_slots_per_token, m, rows_per_expert, _ptr(y)))
 
     def enqueue_down_combine_h(self, w, h, act_h, sel, wts, resid, n_slots_per_token, m, rows_per_expert, y):
-        """bm_down_combine from the f32 rows of h, for a down stack on Q8_K columns (act_h may be None)."""
+        """bm_down_combine from the f32 rows of h, quantized in the launch in the form the stack dots against (act_h may be None)."""
         self._check(self.lib.bm_down_combine_h(self.ctx, w.handle, _ptr(h), act_h.handle if act_h is not None else None,
                                                _ptr(sel), _ptr(wts), _ptr(resid), n_slots_per_token, m, rows_per_expert,
                                                _ptr(y)))

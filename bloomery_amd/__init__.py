@@ -225,11 +225,11 @@ class Gguf:
         h = _vp()
         rc = (self.lib.bm_gguf_open_split if split else self.lib.bm_gguf_open)(os.fsencode(path), C.byref(h))
         if rc:
-            raise GpuError(rc, self.lib.bm_gguf_last_error().decode())
+            raise GpuError(rc, self.lib.bm_gguf_last_error().decode(errors="replace"))
         self.handle = h.value
 
     def _tensor(self, t):
-        return {"name": t.name.decode(), "type": t.type, "dims": [int(t.dims[d]) for d in range(t.n_dims)],
+        return {"name": t.name.decode(errors="replace"), "type": t.type, "dims": [int(t.dims[d]) for d in range(t.n_dims)],
                 "offset": int(t.offset), "nbytes": int(t.nbytes), "data": t.data}
 
     @property
@@ -242,7 +242,7 @@ class Gguf:
             t = _GgufTensor()
             rc = self.lib.bm_gguf_tensor_at(self.handle, i, C.byref(t))
             if rc:
-                raise GpuError(rc, self.lib.bm_gguf_last_error().decode())
+                raise GpuError(rc, self.lib.bm_gguf_last_error().decode(errors="replace"))
             out.append(self._tensor(t))
         return out
 
@@ -250,7 +250,7 @@ class Gguf:
         t = _GgufTensor()
         rc = self.lib.bm_gguf_find(self.handle, name.encode(), C.byref(t))
         if rc:
-            raise GpuError(rc, self.lib.bm_gguf_last_error().decode())
+            raise GpuError(rc, self.lib.bm_gguf_last_error().decode(errors="replace"))
         return self._tensor(t)
 
     def data(self, name):
@@ -263,19 +263,19 @@ class Gguf:
         v = C.c_uint64()
         rc = self.lib.bm_gguf_get_u64(self.handle, key.encode(), C.byref(v))
         if rc:
-            raise GpuError(rc, self.lib.bm_gguf_last_error().decode())
+            raise GpuError(rc, self.lib.bm_gguf_last_error().decode(errors="replace"))
         return v.value
 
     def get_f32(self, key):
         v = C.c_float()
         rc = self.lib.bm_gguf_get_f32(self.handle, key.encode(), C.byref(v))
         if rc:
-            raise GpuError(rc, self.lib.bm_gguf_last_error().decode())
+            raise GpuError(rc, self.lib.bm_gguf_last_error().decode(errors="replace"))
         return v.value
 
     def get_str(self, key):
         v = self.lib.bm_gguf_get_str(self.handle, key.encode())
-        return v.decode() if v is not None else None
+        return v.decode(errors="replace") if v is not None else None
 
     def weights(self, gpu, name):
         """The tensor as a DeviceTensor on `gpu`, with (rows_per_expert, n_experts) of an expert stack."""
@@ -366,12 +366,12 @@ class Gpu:
         else:
             rc = self.lib.bm_ctx_create_on_stream(device, stream, C.byref(ctx))
         if rc != OK:
-            raise GpuError(rc, self.lib.bm_last_error(None).decode())
+            raise GpuError(rc, self.lib.bm_last_error(None).decode(errors="replace"))
         self.ctx = ctx.value
 
     def _check(self, rc):
         if rc != OK:
-            raise GpuError(rc, self.lib.bm_last_error(self.ctx).decode())
+            raise GpuError(rc, self.lib.bm_last_error(self.ctx).decode(errors="replace"))
 
     def close(self):
         if self.ctx:

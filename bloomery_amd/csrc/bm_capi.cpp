@@ -289,6 +289,7 @@ int bm_act_create(bm_ctx *ctx, int wtype, int k, int m_cap, bm_act **out) {
     const size_t bytes = (size_t)m_cap * dev_col_bytes(wtype, k);
     hipError_t e = hipMalloc((void **)&a->dev, bytes);
     if (e == hipSuccess) e = hipMemset(a->dev, 0, bytes);
+    if (e == hipSuccess) e = hipDeviceSynchronize(); // the fill runs on the null stream; the context's does not wait for it
     if (e != hipSuccess) {
         if (a->dev) (void)hipFree(a->dev);
         delete a;
@@ -723,6 +724,7 @@ int bm_route_create(bm_ctx *ctx, int max_slots, int n_experts, bm_route **out) {
     const size_t words = (size_t)max_slots + 2 * (size_t)bmk::gemm_max_tiles(max_slots, n_experts) + 2;
     hipError_t e = hipMalloc((void **)&r->cols, words * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMemset(r->cols, 0, words * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipDeviceSynchronize(); // as in bm_act_create
     if (e != hipSuccess) {
         if (r->cols) (void)hipFree(r->cols);
         delete r;

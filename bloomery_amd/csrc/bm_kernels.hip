@@ -209,6 +209,7 @@ __global__ __launch_bounds__(256) void k_gate_up(const uint8_t *wg, const uint8_
     Stage<2> st;
     st.load(act_col, col_bytes);
     if (id >= n_experts) { // uniform over the workgroup: no weight is read (crates/gpu/src/kquant/sel.rs:22-28)
+        if (id == 0xffffffffu) return; // a slot served elsewhere: nothing written, nothing raised (sel.rs:153-161)
         if (tid == 0) bm_raise(fault, layer, kSiteExpertId);
         if (h && active && (tid & 7) == 0) h[(size_t)slot * rpe + r] = bm_bits_f32(0x7fc00000u);
         if (act_h && tid < 32) q82_store(hcol, nb_h, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);
@@ -479,6 +480,7 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
     __asm__ volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     if (id >= n_experts) { // uniform over the workgroup
+        if (id == 0xffffffffu) return; // a slot served elsewhere: nothing written, nothing raised
         if (tid == 0) bm_raise(fault, layer, kSiteExpertId);
         if (h && (tid & 7) == 0) h[(size_t)slot * ff + r] = bm_bits_f32(0x7fc00000u);
         if (hcol && tid < 32) q82_store(hcol, nh, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);
@@ -694,6 +696,7 @@ __global__ __launch_bounds__(256) void k_gate_up_xq(const float *x, const uint8_
     const u32 id = sel[slot];
     uint8_t *hcol = act_h ? act_h + (size_t)slot * nh * BM_Q82_SB_EXT : nullptr;
     if (id >= n_experts) { // uniform over the workgroup
+        if (id == 0xffffffffu) return; // a slot served elsewhere: nothing written, nothing raised
         if (tid == 0) bm_raise(fault, layer, kSiteExpertId);
         if (h && (tid & 7) == 0) h[(size_t)slot * ff + r] = bm_bits_f32(0x7fc00000u);
         if (hcol && tid < 32) q82_store(hcol, nh, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);

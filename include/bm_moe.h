@@ -53,7 +53,9 @@ extern "C" {
 #define BM_SITE_F32_PRODUCT 21 /* a gate or up sum that is not finite met a clamped gate rule: the value is NaN */
 #define BM_SITE_STALLED 31     /* ours: a bm_moe_decode consumer gave up waiting for its producers */
 
-/* The id of a slot served elsewhere (crates/gpu/src/host/slots.rs:10): the down projections skip it silently. */
+/* The id of a slot served elsewhere (crates/gpu/src/host/slots.rs:10): every routed entry skips it silently - the
+ * gate . up entries write nothing for it (no h rows, no activation block) and the down entries leave its rows as they
+ * were; nothing is raised (crates/gpu/src/kquant/sel.rs:22-28,153-161). */
 #define BM_HOST_SLOT 0xFFFFFFFFu
 
 typedef struct bm_ctx bm_ctx;         /* crates/gpu/src/lib.rs:2529 Gpu: device, stream, fault word */
@@ -141,7 +143,8 @@ int bm_gemv_x(bm_ctx *ctx, const bm_weights *w, const float *x_dev, int m, bm_ac
  * slot s < n_slots reads expert sel_dev[s]'s rows of both stacks against activation column s / slots_per_col and
  * writes h_dev[s * rows_per_expert + r] = silu(gate_r) * up_r in the CPU path's SwiGLU
  * (crates/qdot/src/lib.rs:11467). An id at or past the stack raises BM_SITE_EXPERT_ID and writes NaN into the
- * slot's rows. h_dev may be NULL when act_h is given.
+ * slot's rows (and a NaN-scaled block into act_h); BM_HOST_SLOT is skipped: nothing written, nothing raised.
+ * h_dev may be NULL when act_h is given.
  * act_h (optional, NULL to skip): the down projection's activation, quantized in the same launch from the rows
  * just written, column s of act_h for slot s, in the form of act_h's type (Q8_2_X4 only; rows_per_expert must
  * then be act_h's k). The reference runs this as a separate quantizer launch (dispatch.rs:1343). */
@@ -188,7 +191,9 @@ int bm_down_combine_h(bm_ctx *ctx, const bm_weights *w, const float *h_dev, bm_a
  * holds m rows of hidden = wg's k f32 values (16-byte aligned); token t's slots are sel_dev / w_dev[t *
  * n_slots_per_token ..]; y_dev[t * hidden + d] gets bm_combine_tokens' value. Same bits as bm_quantize, bm_gate_up
  * (with act_h) and bm_down_combine run one after the other. Gate and up are of one type; every type of this library
- * goes on either side (BM_PLAN_ONE_LAUNCH: Q4_K gate/up with Q6_K or Q4_K down only). act_h is caller-held scratch
+ * goes on either side (BM_PLAN_ONE_LAUNCH: Q4_K gate/up with Q6_K or Q4_K down only). A slot whose id is BM_HOST_SLOT
+ * is skipped by both halves (its h rows and activation column keep what they held, it adds nothing to the sum, nothing is
+ * raised); any other id at or past the stack raises BM_SITE_EXPERT_ID and adds nothing. act_h is caller-held scratch
  * (m * n_slots_per_token columns of ff = wd's k, in the form wd dots against) and holds the quantized h afterwards;
  * act_x (optional, in the form wg dots against) receives the quantized x columns; h_dev receives the f32 h rows:
  * optional, except that a down stack on Q8_K columns needs it (16-byte aligned): a Q8_K block spans eight gate . up
@@ -207,7 +212,8 @@ int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const
 int bm_set_decode_plan(bm_ctx *ctx, int plan);
 /* The first launch of BM_PLAN_TWO_LAUNCHES on its own: bm_quantize, bm_gate_up and the quantizer of h in one
  * launch, from the f32 token rows (gate and up of one type; rows_per_expert = ff a multiple of 256). act_h: Q8_2_X4
- * columns for the down stack, or NULL; h_dev: the f32 h rows, or NULL; one of the two at least. Follow it with
+ * columns for the down stack, or NULL; h_dev: the f32 h rows, or NULL; one of the two at least. Ids as bm_gate_up
+ * takes them (BM_HOST_SLOT skipped silently). Follow it with
  * bm_down_combine or bm_gemv_sel over act_h, or bm_down_combine_h over h_dev. */
 int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const float *x_dev, const uint32_t *sel_dev,
                  int n_slots_per_token, int m, int rows_per_expert, bm_act *act_h, bm_act *act_x, float *h_dev);

@@ -99,7 +99,7 @@ def test_gemm_fast_mode_is_within_the_tolerance(gpu):
 
 
 @pytest.mark.parametrize("types,hidden,ff,n_experts,m,top_k,cheap", (
-    ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 6, 70, 3, False),      # runs past 64 slots: several tiles an expert
+    ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 6, 70, 3, False),      # 210 slots over 6 experts: runs of about 35, a tile each
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 16, 48, 8, True),     # config 4's layer shape, 384 slots
     ((bm.Q6_K, bm.Q6_K, bm.Q4_K), 768, 512, 3, 9, 2, False),       # the other type on each side; ragged tiles
     ((bm.Q5_K, bm.Q5_K, bm.Q5_K), 768, 512, 3, 40, 2, False),      # Q5_K on both sides: the Q4_K walk with a fifth bit

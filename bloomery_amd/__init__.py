@@ -68,6 +68,7 @@ SYMBOLS = {
     "bm_down_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_down_combine_h": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_moe_decode": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp]),
+    "bm_moe_decode_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
     "bm_set_spin_limit": (_i, [_vp, _u32]),
     "bm_set_decode_plan": (_i, [_vp, _i]),
     "bm_gate_up_x": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
@@ -482,6 +483,11 @@ class Gpu:
         self._check(self.lib.bm_moe_decode(self.ctx, wg.handle, wu.handle, wd.handle, _ptr(x), _ptr(sel), _ptr(wts),
                                            _ptr(resid), n_slots_per_token, m, act_h.handle,
                                            act_x.handle if act_x is not None else None, _ptr(h), _ptr(y)))
+
+    def enqueue_moe_decode_noalloc(self, wg, wu, wd, x, sel, wts, resid, n_slots_per_token, m, y):
+        """bm_moe_decode in two launches with the scratch between them held by the library: nothing is allocated."""
+        self._check(self.lib.bm_moe_decode_noalloc(self.ctx, wg.handle, wu.handle, wd.handle, _ptr(x), _ptr(sel), _ptr(wts),
+                                                   _ptr(resid), n_slots_per_token, m, _ptr(y)))
 
     def enqueue_gate_up_x(self, wg, wu, x, sel, n_slots_per_token, m, rows_per_expert, act_h, act_x=None, h=None):
         self._check(self.lib.bm_gate_up_x(self.ctx, wg.handle, wu.handle, _ptr(x), _ptr(sel), n_slots_per_token, m,

@@ -93,6 +93,9 @@ static int ctx_make(int device, hipStream_t stream, bool own, bm_ctx **out) {
     *out = nullptr;
     hipError_t e = hipSetDevice(device);
     if (e != hipSuccess) return fail(nullptr, BM_EDRIVER, "bm_ctx_create: hipSetDevice(%d): %s", device, hipGetErrorString(e));
+    // the device address of the library's static scratch (bm_moe_decode_noalloc), looked up once a device
+    e = bmk::static_scratch_init(device);
+    if (e != hipSuccess) return fail(nullptr, BM_EDRIVER, "bm_ctx_create: hipGetSymbolAddress(scratch) on device %d: %s", device, hipGetErrorString(e));
     bm_ctx *c = new (std::nothrow) bm_ctx();
     if (!c) return fail(nullptr, BM_EDRIVER, "bm_ctx_create: out of host memory");
     c->device = device;
@@ -590,6 +593,43 @@ int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const
                   bmk::moe_decode(launch_of(ctx), ctx->decode_plan, wg->wtype, wd->wtype, x_dev, wg->dev, wu->dev, wd->dev, n_experts, hidden, ff, sel_dev,
                                   w_dev, resid_dev, n_slots_per_token, m, act_x ? act_x->dev : nullptr, act_h->dev, h_dev, y_dev,
                                   ctx->counters, ctx->spin_limit));
+}
+
+int bm_moe_decode_noalloc(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_weights *wd, const float *x_dev,
+                          const uint32_t *sel_dev, const float *w_dev, const float *resid_dev, int n_slots_per_token, int m,
+                          float *y_dev) {
+    const char *what = "bm_moe_decode_noalloc";
+    if (!ctx || !wg || !wu || !wd || !x_dev || !sel_dev || !w_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (wg->wtype != wu->wtype)
+        return fail(ctx, BM_ETYPE, "%s: gate is type %d and up type %d; one launch reads one type", what, wg->wtype, wu->wtype);
+    if (!bmk::moe_decode_supported(bmk::kPlanTwoLaunches, wg->wtype, wd->wtype))
+        return fail(ctx, BM_ETYPE, "%s: no kernel for gate/up type %d with down type %d", what, wg->wtype, wd->wtype);
+    if (wu->k != wg->k || wu->rows != wg->rows)
+        return fail(ctx, BM_ESHAPE, "%s: gate is %lld x %d, up %lld x %d", what, (long long)wg->rows, wg->k, (long long)wu->rows, wu->k);
+    const int hidden = wg->k, ff = wd->k;
+    int n_experts = 0, n_down = 0;
+    int rc = check_stack(ctx, what, wg, ff, &n_experts);
+    if (!rc) rc = check_stack(ctx, what, wd, hidden, &n_down);
+    if (rc) return rc;
+    if (n_down != n_experts)
+        return fail(ctx, BM_ESHAPE, "%s: gate/up hold %d experts of %d rows, down %d experts of %d rows", what, n_experts, ff, n_down, hidden);
+    if (n_slots_per_token < 1 || n_slots_per_token > bmk::kMaxCombineSlots)
+        return fail(ctx, BM_ESHAPE, "%s: %d slots a token outside 1..=%d", what, n_slots_per_token, bmk::kMaxCombineSlots);
+    if (m < 1 || m > bmk::kMaxDecodeTokens)
+        return fail(ctx, BM_ESHAPE, "%s: m = %d tokens outside 1..=%d", what, m, bmk::kMaxDecodeTokens);
+    if ((size_t)m * (size_t)n_slots_per_token * (size_t)ff > bmk::kStaticValues)
+        return fail(ctx, BM_ESHAPE, "%s: %d tokens x %d slots x ff = %d is %zu values of h; the library's static scratch holds %zu "
+                    "(use bm_moe_decode with caller-held act_h past that)", what, m, n_slots_per_token, ff,
+                    (size_t)m * (size_t)n_slots_per_token * (size_t)ff, (size_t)bmk::kStaticValues);
+    if (((uintptr_t)x_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: x_dev %p is not 16-byte aligned", what, (const void *)x_dev);
+    const size_t lds_a = dev_col_bytes(wg->wtype, hidden) + 8192;
+    const size_t lds_b = (size_t)n_slots_per_token * dev_col_bytes(wd->wtype, ff) + 12288;
+    if (lds_a > (size_t)bmk::kMaxLds || lds_b > (size_t)bmk::kMaxLds)
+        return fail(ctx, BM_ESHAPE, "%s: hidden = %d or %d columns of ff = %d do not fit the workgroup's LDS; use the separate launches", what,
+                    hidden, n_slots_per_token, ff);
+    return driver(ctx, what,
+                  bmk::moe_decode_static(launch_of(ctx), ctx->device, wg->wtype, wd->wtype, x_dev, wg->dev, wu->dev, wd->dev, n_experts,
+                                         hidden, ff, sel_dev, w_dev, resid_dev, n_slots_per_token, m, y_dev));
 }
 
 // ------------------------------------------------------------------------------------------ grouped decode

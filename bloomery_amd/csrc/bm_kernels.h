@@ -83,6 +83,16 @@ hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, c
                       const float *wts, const float *resid, int slots_per_token, int m, uint8_t *act_x,
                       uint8_t *act_h, float *h, float *y, uint32_t *counters, uint32_t spin_limit);
 
+// moe_decode's two launches with act_h and h in a file-scope device array instead of caller memory: no allocation
+// anywhere on the way. static_scratch_init(device), called with that device current (the context's creation does),
+// looks the array's address up once a device; kStaticValues = the most values of h (tokens x slots x ff) a call may ask
+// for. Calls on one device share the array: two that overlap race.
+constexpr size_t kStaticValues = 65536;
+hipError_t static_scratch_init(int device);
+hipError_t moe_decode_static(const Launch &L, int device, int gate_type, int down_type, const float *x, const uint8_t *wg,
+                             const uint8_t *wu, const uint8_t *wd, int n_experts, int hidden, int ff, const uint32_t *sel,
+                             const float *wts, const float *resid, int slots_per_token, int m, float *y);
+
 // ------------------------------------------------------------------------------ grouped decode (bm_grouped.hip)
 
 // crates/gpu/src/q4k_sel.rs:68-97: a tile is up to 8 consecutive entries of one expert's run; word (e << 22) | j.

@@ -1075,6 +1075,46 @@ hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, c
     return hipGetLastError();
 }
 
+// --------------------------------------------------------------- the fused step on scratch the library holds
+
+// What bm_moe_decode takes from its caller as act_h (and h, for a down stack on Q8_K columns), held here instead: one
+// array a device for as long as the process lives, so the entry that uses it calls no allocator. Room for
+// kStaticValues values of h (slots x ff): their activation columns in the wider of the two column forms first, their
+// f32 rows after them.
+constexpr size_t kStaticColBytes = kStaticValues / 256 * BM_Q82_SB_EXT; // Q8_K columns (296 a super-block) fit too
+constexpr size_t kStaticBytes = kStaticColBytes + kStaticValues * sizeof(float);
+static __device__ __align__(256) uint8_t scratch[kStaticBytes];
+
+// The array's address on each device. Host code may not hand the symbol itself to a kernel (on the host it names a
+// stand-in, not device memory): the address is asked for once a device, with that device current, and every launch
+// takes it from here.
+constexpr int kStaticMaxDevices = 64;
+static uint8_t *g_scratch_at[kStaticMaxDevices];
+
+hipError_t static_scratch_init(int device) {
+    if (device < 0 || device >= kStaticMaxDevices) return hipErrorInvalidDevice;
+    if (g_scratch_at[device]) return hipSuccess;
+    void *at = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&at, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!at) return hipErrorInvalidSymbol;
+    g_scratch_at[device] = static_cast<uint8_t *>(at);
+    return hipSuccess;
+}
+
+hipError_t moe_decode_static(const Launch &L, int device, int gate_type, int down_type, const float *x, const uint8_t *wg,
+                             const uint8_t *wu, const uint8_t *wd, int n_experts, int hidden, int ff, const uint32_t *sel,
+                             const float *wts, const float *resid, int slots_per_token, int m, float *y) {
+    if (device < 0 || device >= kStaticMaxDevices || !g_scratch_at[device]) return hipErrorNotInitialized;
+    if ((size_t)m * (size_t)slots_per_token * (size_t)ff > kStaticValues) return hipErrorInvalidValue;
+    uint8_t *act_h = g_scratch_at[device];
+    float *h = reinterpret_cast<float *>(g_scratch_at[device] + kStaticColBytes);
+    // every live slot's column (or f32 rows) is written whole by the first launch before the second reads it, and a
+    // slot that is not live is never read into a sum: nothing here has to start at zero
+    return moe_decode(L, kPlanTwoLaunches, gate_type, down_type, x, wg, wu, wd, n_experts, hidden, ff, sel, wts, resid,
+                      slots_per_token, m, nullptr, act_h, bm_takes_q8k(down_type) ? h : nullptr, y, nullptr, 0);
+}
+
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out) {
     const int nb = k / 256;
     const size_t lds = tab_bytes_rt(wtype) + (size_t)act_col_bytes(wtype, k);

@@ -217,6 +217,18 @@ int bm_set_decode_plan(bm_ctx *ctx, int plan);
  * bm_down_combine or bm_gemv_sel over act_h, or bm_down_combine_h over h_dev. */
 int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const float *x_dev, const uint32_t *sel_dev,
                  int n_slots_per_token, int m, int rows_per_expert, bm_act *act_h, bm_act *act_x, float *h_dev);
+/* bm_moe_decode (BM_PLAN_TWO_LAUNCHES) for callers that cannot allocate device memory or hold a scratch handle: code
+ * under HIP graph capture, serving loops and harnesses that forbid hipMalloc. It has no counterpart in the reference,
+ * whose callers make their Q8Act scratch at load time. The quantized h between the two launches (bm_moe_decode's act_h,
+ * and its h_dev rows for a down stack on Q8_K columns) lives in an array the library holds on each device for the life
+ * of the process (about 360 KiB), so the call allocates nothing, on the device or through any library. Same arguments
+ * and same bits in y_dev as bm_moe_decode. Limit: m * n_slots_per_token * ff <= 65536 values of h (8 slots of ff 8192,
+ * 32 of ff 2048, 85 of ff 768); more is refused with BM_ESHAPE. Every call on a device shares that device's array, which
+ * keeps the last call's contents: calls that overlap on one device (two streams, two contexts) race; calls in stream
+ * order do not, and nothing in the array has to start at zero. */
+int bm_moe_decode_noalloc(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_weights *wd, const float *x_dev,
+                          const uint32_t *sel_dev, const float *w_dev, const float *resid_dev, int n_slots_per_token, int m,
+                          float *y_dev);
 /* Polls (a memory round trip each, about a microsecond) a BM_PLAN_ONE_LAUNCH consumer waits before it gives up;
  * the default is 1 << 18. */
 int bm_set_spin_limit(bm_ctx *ctx, uint32_t spins);

@@ -4,6 +4,8 @@
 // bit-equal to the scalar restatement in qdot.c (two independently written paths through the same arithmetic,
 // the reference's own first gate, crates/qdot/tests/qdot.rs:346,738,818,2664), and the benchmark times it as the
 // CPU baseline. Build with -mavx2 -mfma -mf16c -ffp-contract=off.
+#define _GNU_SOURCE
+#include <sched.h>
 #include <immintrin.h>
 #include <pthread.h>
 #include <stdlib.h>
@@ -615,6 +617,10 @@ int ora_avx2_dot_row(int wtype, const uint8_t *wrow, const uint8_t *acol, int k,
 
 // --------------------------------------------------------------------------------- multi-threaded layer baseline
 
+// One phase of the layer step: a list of matrix x columns products (one per expert hit and matrix) whose rows, taken
+// together, are split evenly over the pool's threads - the reference's pool splits an expert matrix's rows statically
+// (crates/threads/src/lib.rs:1-30); here a phase's matrices are laid end to end first, so one dispatch serves them all -
+// or a list of per-slot jobs (SwiGLU and the quantizer of h).
 typedef struct {
     int wtype, k, rows, cols;
     const uint8_t *w;
@@ -623,16 +629,44 @@ typedef struct {
 } mt_gemv;
 
 typedef struct {
+    const mt_gemv *jobs; // kind 0
+    int n_jobs;
+    long total_rows;
+    // kind 1: slot s: h = swiglu(g, u), then its column for the down stack
+    int kind, n_slots, ff, down_type, cb_d;
+    const float *g, *u;
+    float *h;
+    uint8_t *ad;
+    volatile int *rc;
+} mt_phase;
+
+struct ora_pool;
+typedef struct {
     pthread_t th;
-    int tid, n_threads;
-    pthread_barrier_t *bar;
-    volatile int *quit;
-    const mt_gemv *volatile *job;
+    int tid;
+    struct ora_pool *pool;
 } worker;
 
-static void run_slice(const mt_gemv *g, int tid, int n_threads) {
-    int per = (g->rows + n_threads - 1) / n_threads;
-    int r0 = tid * per, r1 = r0 + per > g->rows ? g->rows : r0 + per;
+struct ora_pool {
+    int n_threads;
+    worker *ws;
+    volatile int quit;
+    const mt_phase *volatile phase;
+    // a sense-reversing barrier the threads spin on: a phase lasts tens of microseconds, a futex wake as long
+    volatile int arrived, sense;
+};
+
+static void spin_barrier(struct ora_pool *p, int *my_sense) {
+    *my_sense = !*my_sense;
+    if (__atomic_add_fetch(&p->arrived, 1, __ATOMIC_ACQ_REL) == p->n_threads) {
+        p->arrived = 0;
+        __atomic_store_n(&p->sense, *my_sense, __ATOMIC_RELEASE);
+    } else {
+        while (__atomic_load_n(&p->sense, __ATOMIC_ACQUIRE) != *my_sense) _mm_pause();
+    }
+}
+
+static void run_rows(const mt_gemv *g, int r0, int r1) {
     int rb = ora_row_bytes(g->wtype, g->k);
     float tmp[8];
     for (int r = r0; r < r1; r++) {
@@ -644,63 +678,100 @@ static void run_slice(const mt_gemv *g, int tid, int n_threads) {
     }
 }
 
-static void *worker_main(void *arg) {
-    worker *w = (worker *)arg;
-    for (;;) {
-        pthread_barrier_wait(w->bar);
-        if (*w->quit) return NULL;
-        run_slice((const mt_gemv *)*w->job, w->tid, w->n_threads);
-        pthread_barrier_wait(w->bar);
+static void run_share(const mt_phase *ph, int tid, int n_threads) {
+    if (ph->kind == 1) {
+        for (int s = tid; s < ph->n_slots; s += n_threads) {
+            ora_swiglu(ph->g + (size_t)s * ph->ff, ph->u + (size_t)s * ph->ff, ph->ff, ph->h + (size_t)s * ph->ff);
+            int rc = ora_avx2_quantize_col(ph->down_type, ph->h + (size_t)s * ph->ff, ph->ff, ph->ad + (size_t)s * ph->cb_d);
+            if (rc) *ph->rc = rc;
+        }
+        return;
+    }
+    long per = (ph->total_rows + n_threads - 1) / n_threads;
+    long lo = (long)tid * per, hi = lo + per > ph->total_rows ? ph->total_rows : lo + per;
+    long at = 0;
+    for (int j = 0; j < ph->n_jobs && at < hi; j++) {
+        long end = at + ph->jobs[j].rows;
+        long a = lo > at ? lo : at, b = hi < end ? hi : end;
+        if (a < b) run_rows(&ph->jobs[j], (int)(a - at), (int)(b - at));
+        at = end;
     }
 }
 
-struct ora_pool {
-    int n_threads;
-    worker *ws;
-    pthread_barrier_t bar;
-    volatile int quit;
-    const mt_gemv *volatile job;
-};
+static void *worker_main(void *arg) {
+    worker *w = (worker *)arg;
+    struct ora_pool *p = w->pool;
+    int sense = 0;
+    for (;;) {
+        spin_barrier(p, &sense);
+        if (p->quit) return NULL;
+        run_share((const mt_phase *)p->phase, w->tid, p->n_threads);
+        spin_barrier(p, &sense);
+    }
+}
 
-// A resident pool (the role of crates/threads): n_threads - 1 workers plus the caller.
+// A resident pool (the role of crates/threads): n_threads - 1 workers plus the caller, each pinned to a CPU of the
+// process's set where the system allows it.
 ora_pool *ora_pool_create(int n_threads) {
     if (n_threads < 1) n_threads = 1;
     ora_pool *p = (ora_pool *)calloc(1, sizeof(ora_pool));
     p->n_threads = n_threads;
-    pthread_barrier_init(&p->bar, NULL, (unsigned)n_threads);
     p->ws = (worker *)calloc((size_t)n_threads, sizeof(worker));
+    cpu_set_t all;
+    int have = sched_getaffinity(0, sizeof all, &all) == 0 ? CPU_COUNT(&all) : 0;
     for (int t = 1; t < n_threads; t++) {
-        p->ws[t] = (worker){0, t, n_threads, &p->bar, &p->quit, &p->job};
+        p->ws[t].tid = t;
+        p->ws[t].pool = p;
         pthread_create(&p->ws[t].th, NULL, worker_main, &p->ws[t]);
+        if (have >= n_threads) { // the t-th CPU of the set
+            int seen = 0;
+            for (int c = 0; c < CPU_SETSIZE; c++)
+                if (CPU_ISSET(c, &all) && seen++ == t) {
+                    cpu_set_t one;
+                    CPU_ZERO(&one);
+                    CPU_SET(c, &one);
+                    (void)pthread_setaffinity_np(p->ws[t].th, sizeof one, &one);
+                    break;
+                }
+        }
     }
     return p;
 }
 
+// The caller's barrier sense: the caller is one thread for the pool's life.
+static __thread int g_caller_sense;
+static __thread const ora_pool *g_caller_pool;
+
 void ora_pool_destroy(ora_pool *p) {
     if (!p) return;
     p->quit = 1;
-    if (p->n_threads > 1) pthread_barrier_wait(&p->bar);
+    if (p->n_threads > 1) {
+        if (g_caller_pool != p) g_caller_pool = p, g_caller_sense = p->sense;
+        spin_barrier(p, &g_caller_sense);
+    }
     for (int t = 1; t < p->n_threads; t++) pthread_join(p->ws[t].th, NULL);
-    pthread_barrier_destroy(&p->bar);
     free(p->ws);
     free(p);
 }
 
-static void pool_gemv(ora_pool *p, const mt_gemv *g) {
+static void pool_run(ora_pool *p, const mt_phase *ph) {
     if (p->n_threads == 1) {
-        run_slice(g, 0, 1);
+        run_share(ph, 0, 1);
         return;
     }
-    p->job = g;
-    pthread_barrier_wait(&p->bar);
-    run_slice(g, 0, p->n_threads);
-    pthread_barrier_wait(&p->bar);
+    if (g_caller_pool != p) g_caller_pool = p, g_caller_sense = p->sense;
+    p->phase = ph;
+    spin_barrier(p, &g_caller_sense);
+    run_share(ph, 0, p->n_threads);
+    spin_barrier(p, &g_caller_sense);
 }
 
 // The layer step of ora_moe_forward on the AVX2 kernels and the pool, slots grouped by expert so a weight row is
-// read once for up to eight of its columns (crates/model/src/moe.rs:617-749 with dot_row_cols tiles). The values
-// are ora_moe_forward's bit for bit: every (row, column) dot is the one-column kernel's and the combine keeps
-// its slot order.
+// read once for up to eight of its columns (crates/model/src/moe.rs:617-749 with dot_row_cols tiles). Only the experts
+// the routing names are visited, and the step is three dispatches of the pool whatever their number: every hit
+// expert's gate and up rows, the slots' SwiGLU and quantizer, every hit expert's down rows. The values are
+// ora_moe_forward's bit for bit: every (row, column) dot is the one-column kernel's and the combine keeps its slot
+// order.
 int ora_avx2_moe_forward(ora_pool *p, const ora_moe_layer *L, const float *x, int m, const uint32_t *ids,
                          const float *wts, int top_k, float *y, float *h_out) {
     int hidden = L->hidden, ff = L->ff, n_slots = m * top_k;
@@ -718,45 +789,64 @@ int ora_avx2_moe_forward(ora_pool *p, const ora_moe_layer *L, const float *x, in
     float *u = (float *)malloc(sizeof(float) * (size_t)ff * n_slots);
     float *h = h_out ? h_out : (float *)malloc(sizeof(float) * (size_t)ff * n_slots);
     float *down = (float *)malloc(sizeof(float) * (size_t)hidden * n_slots);
+    int *start = (int *)calloc((size_t)L->n_experts + 1, sizeof(int));
+    int *fill = (int *)malloc(sizeof(int) * (size_t)L->n_experts);
     int *order = (int *)malloc(sizeof(int) * (size_t)n_slots);
-    const uint8_t **cols = (const uint8_t **)malloc(sizeof(void *) * (size_t)n_slots);
-    float **outs = (float **)malloc(sizeof(void *) * (size_t)n_slots);
-    int rc = 0;
+    const uint8_t **cols_g = (const uint8_t **)malloc(sizeof(void *) * (size_t)n_slots);
+    const uint8_t **cols_u = (const uint8_t **)malloc(sizeof(void *) * (size_t)n_slots);
+    const uint8_t **cols_d = (const uint8_t **)malloc(sizeof(void *) * (size_t)n_slots);
+    float **outs_g = (float **)malloc(sizeof(void *) * (size_t)n_slots);
+    float **outs_u = (float **)malloc(sizeof(void *) * (size_t)n_slots);
+    float **outs_d = (float **)malloc(sizeof(void *) * (size_t)n_slots);
+    mt_gemv *jobs = (mt_gemv *)malloc(sizeof(mt_gemv) * 2 * (size_t)(n_slots < L->n_experts ? n_slots : L->n_experts));
+    volatile int rc = 0;
     for (int t = 0; t < m && !rc; t++) {
         rc = ora_avx2_quantize_col(L->gate_type, x + (size_t)t * hidden, hidden, ag + (size_t)t * cb_g);
         if (!rc && !same_enc)
             rc = ora_avx2_quantize_col(L->up_type, x + (size_t)t * hidden, hidden, au + (size_t)t * cb_u);
     }
-    // Slots grouped by expert, ascending slot order inside an expert (the bucket table, moe.rs:281-304).
-    int n = 0;
-    for (int e = 0; e < L->n_experts && !rc; e++) {
-        int first = n;
-        for (int s = 0; s < n_slots; s++)
-            if (ids[s] == (uint32_t)e) order[n++] = s;
-        int cnt = n - first;
-        if (!cnt) continue;
-        for (int pass = 0; pass < 2; pass++) {
-            for (int j = 0; j < cnt; j++) {
-                int s = order[first + j];
-                cols[j] = (pass ? au + (size_t)(s / top_k) * cb_u : ag + (size_t)(s / top_k) * cb_g);
-                outs[j] = (pass ? u : g) + (size_t)s * ff;
-            }
-            mt_gemv job = {pass ? L->up_type : L->gate_type, hidden, ff, cnt,
-                           (pass ? L->wu + (size_t)e * ff * rb_u : L->wg + (size_t)e * ff * rb_g), cols, outs};
-            pool_gemv(p, &job);
-        }
-        for (int j = 0; j < cnt && !rc; j++) {
-            int s = order[first + j];
-            ora_swiglu(g + (size_t)s * ff, u + (size_t)s * ff, ff, h + (size_t)s * ff);
-            rc = ora_avx2_quantize_col(L->down_type, h + (size_t)s * ff, ff, ad + (size_t)s * cb_d);
-            cols[j] = ad + (size_t)s * cb_d;
-            outs[j] = down + (size_t)s * hidden;
-        }
-        if (rc) break;
-        mt_gemv job = {L->down_type, ff, hidden, cnt, L->wd + (size_t)e * hidden * rb_d, cols, outs};
-        pool_gemv(p, &job);
+    // Slots grouped by expert, ascending slot order inside an expert (the bucket table, moe.rs:281-304): a counting
+    // sort over the ids.
+    for (int s = 0; s < n_slots; s++) start[ids[s] + 1]++;
+    for (int e = 0; e < L->n_experts; e++) start[e + 1] += start[e], fill[e] = start[e];
+    for (int s = 0; s < n_slots; s++) order[fill[ids[s]]++] = s;
+    for (int j = 0; j < n_slots; j++) {
+        int s = order[j];
+        cols_g[j] = ag + (size_t)(s / top_k) * cb_g;
+        cols_u[j] = au + (size_t)(s / top_k) * cb_u;
+        cols_d[j] = ad + (size_t)s * cb_d;
+        outs_g[j] = g + (size_t)s * ff;
+        outs_u[j] = u + (size_t)s * ff;
+        outs_d[j] = down + (size_t)s * hidden;
     }
-    if (!rc) ora_combine_tokens(down, wts, NULL, hidden, top_k, m, y);
+    if (!rc) {
+        mt_phase ph = {0};
+        for (int e = 0; e < L->n_experts; e++) {
+            int first = start[e], cnt = start[e + 1] - first;
+            if (!cnt) continue;
+            jobs[ph.n_jobs++] = (mt_gemv){L->gate_type, hidden, ff, cnt, L->wg + (size_t)e * ff * rb_g, cols_g + first, outs_g + first};
+            jobs[ph.n_jobs++] = (mt_gemv){L->up_type, hidden, ff, cnt, L->wu + (size_t)e * ff * rb_u, cols_u + first, outs_u + first};
+            ph.total_rows += 2L * ff;
+        }
+        ph.jobs = jobs;
+        pool_run(p, &ph);
+        mt_phase act = {0};
+        act.kind = 1, act.n_slots = n_slots, act.ff = ff, act.down_type = L->down_type, act.cb_d = cb_d;
+        act.g = g, act.u = u, act.h = h, act.ad = ad, act.rc = &rc;
+        pool_run(p, &act);
+    }
+    if (!rc) {
+        mt_phase ph = {0};
+        for (int e = 0; e < L->n_experts; e++) {
+            int first = start[e], cnt = start[e + 1] - first;
+            if (!cnt) continue;
+            jobs[ph.n_jobs++] = (mt_gemv){L->down_type, ff, hidden, cnt, L->wd + (size_t)e * hidden * rb_d, cols_d + first, outs_d + first};
+            ph.total_rows += hidden;
+        }
+        ph.jobs = jobs;
+        pool_run(p, &ph);
+        ora_combine_tokens(down, wts, NULL, hidden, top_k, m, y);
+    }
     free(ag);
     if (!same_enc) free(au);
     free(ad);
@@ -764,8 +854,15 @@ int ora_avx2_moe_forward(ora_pool *p, const ora_moe_layer *L, const float *x, in
     free(u);
     if (!h_out) free(h);
     free(down);
+    free(start);
+    free(fill);
     free(order);
-    free(cols);
-    free(outs);
+    free(cols_g);
+    free(cols_u);
+    free(cols_d);
+    free(outs_g);
+    free(outs_u);
+    free(outs_d);
+    free(jobs);
     return rc;
 }

@@ -631,7 +631,8 @@ __device__ __forceinline__ void q8k_wave_block(const float4 x4, uint8_t *o, int 
 
 // `cols` columns of nb blocks each, f32 rows at x (column c at x + c * nb * 256), into LDS at `dst` by the workgroup's
 // waves, block by block.
-__device__ __forceinline__ void q8k_stage_cols(const float *x, uint8_t *dst, int cols, int nb, u32 *fault, u32 layer) {
+__device__ __forceinline__ void q8k_stage_cols(const float *x, uint8_t *dst, int cols, int nb, u32 *fault, u32 layer,
+                                               const u32 *ids = nullptr, u32 n_experts = 0) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
     const int total = cols * nb;
     constexpr int kAhead = 6; // blocks whose loads a wave has in flight
@@ -645,38 +646,59 @@ __device__ __forceinline__ void q8k_stage_cols(const float *x, uint8_t *dst, int
 #pragma unroll
         for (int u = 0; u < kAhead; u++) {
             const int b = b0 + u * n_waves;
-            if (b < total) q8k_wave_block(x4[u], dst + (size_t)b * BM_Q8K_STRIDE, lane, fault, layer);
+            // with ids: a column whose slot is not live is not encoded (its rows may hold anything)
+            if (b < total && (!ids || ids[b / nb] < n_experts)) q8k_wave_block(x4[u], dst + (size_t)b * BM_Q8K_STRIDE, lane, fault, layer);
         }
     }
 }
 
 // `cols` columns of nb super-blocks each, f32 rows at x (column c at x + c * nb * 256), into LDS at `dst` as Q8_2_X4
-// columns with their tables: a 32-value block is four consecutive lanes of eight values; four blocks' loads a thread
-// are in flight before the first is encoded.
-__device__ __forceinline__ void q82_stage_cols(const float *x, uint8_t *dst, int cols, int nb, u32 *fault, u32 layer) {
-    const int per_col = nb * 32, total = cols * per_col; // tasks of eight values; a multiple of four a column
-    const int col_bytes = nb * BM_Q82_SB_EXT;
-    constexpr int kAhead = 4;
-    for (int t0 = threadIdx.x; t0 < total; t0 += kAhead * (int)blockDim.x) {
-        float4 lo[kAhead], hi[kAhead];
+// columns with their tables: a 32-value block is four consecutive lanes of eight values. In two steps, for a workgroup
+// that has something else to request in between: the f32 values of the
+// first R tasks a thread are requested at once (memory answers in order, so they are back before anything asked for
+// after them), and encoded into LDS later, when those other requests are on their way; tasks past the first R a thread
+// go through the plain loop afterwards.
+// T: the workgroup's thread count, a constant here: the built-in is read from memory, and a read after the weight
+// requests would wait for all of them.
+template <int R, int T>
+struct Q82Cols {
+    float4 lo[R], hi[R];
+    u32 id[R]; // the expert of a task's column: a column whose slot is not live is not encoded (its rows may hold anything)
+    __device__ __forceinline__ void load(const float *x, int total, int per_col, const u32 *ids) {
 #pragma unroll
-        for (int u = 0; u < kAhead; u++) {
-            const int task = t0 + u * (int)blockDim.x;
-            const float *p = x + (size_t)(task < total ? task : t0) * 8;
+        for (int u = 0; u < R; u++) {
+            int task = (int)threadIdx.x + u * T;
+            task = task < total ? task : total - 1; // a read that stays inside the token's rows; the value is not used
+            const float *p = x + (size_t)task * 8;
             lo[u] = *reinterpret_cast<const float4 *>(p);
             hi[u] = *reinterpret_cast<const float4 *>(p + 4);
+            id[u] = ids[task / per_col];
         }
+        __asm__ volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    __device__ __forceinline__ void encode(const float *x, uint8_t *dst, int cols, int nb, const u32 *ids, u32 n_experts,
+                                           u32 *fault, u32 layer) const {
+        const int per_col = nb * 32, total = cols * per_col, col_bytes = nb * BM_Q82_SB_EXT;
 #pragma unroll
-        for (int u = 0; u < kAhead; u++) {
-            const int task = t0 + u * (int)blockDim.x;
-            if (task < total) { // whole quads: the tasks of a block are four neighbours
+        for (int u = 0; u < R; u++) {
+            const int task = (int)threadIdx.x + u * T;
+            if (task < total && id[u] < n_experts) { // whole quads: the tasks of a block are four neighbours
                 const int c = task / per_col, at = task % per_col;
                 const float v8[8] = {lo[u].x, lo[u].y, lo[u].z, lo[u].w, hi[u].x, hi[u].y, hi[u].z, hi[u].w};
                 q82_quad8(v8, dst + (size_t)c * col_bytes, nb, at >> 2, task & 3, fault, layer);
             }
         }
+        for (int task = (int)threadIdx.x + R * T; task < total; task += T) {
+            const int c = task / per_col, at = task % per_col;
+            if (ids[c] >= n_experts) continue;
+            const float *p = x + (size_t)task * 8;
+            const float4 l4 = *reinterpret_cast<const float4 *>(p), h4 = *reinterpret_cast<const float4 *>(p + 4);
+            const float v8[8] = {l4.x, l4.y, l4.z, l4.w, h4.x, h4.y, h4.z, h4.w};
+            q82_quad8(v8, dst + (size_t)c * col_bytes, nb, at >> 2, task & 3, fault, layer);
+        }
     }
-}
+};
 
 // k_gate_up_x for gate / up stacks that dot against Q8_K columns (Q3_K, IQ2_XXS, IQ3_XXS, IQ4_XS): the token's row is
 // quantized by every workgroup into LDS, h is written as f32 rows, and where the down stack takes Q8_2_X4 columns
@@ -774,14 +796,18 @@ __global__ __launch_bounds__(256) void k_down_combine_hq(const uint8_t *w, u32 n
     const int t = blockIdx.x / blocks_per_token, rb = blockIdx.x % blocks_per_token;
     const int e = quad % spt, dl = quad / spt;
     const int r = rb * D + dl;
+    const int n = NB > 0 ? NB : nb;
     const u32 id = sel[t * spt + e];
+    // Q8_2_X4 columns: the token's f32 rows of h are asked for before anything that waits for the expert id, so they
+    // arrive with it and are encoded while the weight rows are on their way
+    Q82Cols<4, 256> hrows;
+    if constexpr (!bm_takes_q8k(WT)) hrows.load(h + (size_t)t * spt * n * 256, spt * n * 32, n * 32, sel + t * spt);
     const int si = tid < spt ? tid : 0;
     const u32 my_sel = sel[t * spt + si];
     const float my_w = wts[t * spt + si];
     const bool live = id < n_experts;
     const bool active = dl < D && r < rpe && live;
     if (!live && id != 0xffffffffu && rb == 0 && dl == 0 && q == 0) bm_raise(fault, layer, kSiteExpertId);
-    const int n = NB > 0 ? NB : nb;
     const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
     const int col_bytes = bm_act_col_bytes<WT>(n);
     const uint8_t *wrow = w + ((size_t)(live ? id : 0) * rpe + (active ? r : 0)) * row_bytes;
@@ -792,14 +818,16 @@ __global__ __launch_bounds__(256) void k_down_combine_hq(const uint8_t *w, u32 n
     float *part = reinterpret_cast<float *>(cols + (size_t)spt * col_bytes); // [D][spt]
     float *s_w = part + D * spt;                                              // [spt]
     u32 *s_sel = reinterpret_cast<u32 *>(s_w + spt);                          // [spt]
-    if constexpr (bm_takes_q8k(WT)) q8k_stage_cols(h + (size_t)t * spt * n * 256, cols, spt, n, fault, layer);
-    else q82_stage_cols(h + (size_t)t * spt * n * 256, cols, spt, n, fault, layer);
+    if constexpr (bm_takes_q8k(WT)) q8k_stage_cols(h + (size_t)t * spt * n * 256, cols, spt, n, fault, layer, sel + t * spt, n_experts);
+    else hrows.encode(h + (size_t)t * spt * n * 256, cols, spt, n, sel + t * spt, n_experts, fault, layer);
     if (tid < spt) {
         s_w[tid] = my_w;
         s_sel[tid] = my_sel;
     }
     __syncthreads();
-    if (act_h && rb == 0) stage_bytes(act_h + (size_t)t * spt * col_bytes, cols, spt * col_bytes);
+    if (act_h && rb == 0) // the live slots' columns; the others keep what they held
+        for (int c = 0; c < spt; c++)
+            if (s_sel[c] < n_experts) stage_bytes(act_h + ((size_t)t * spt + c) * col_bytes, cols + (size_t)c * col_bytes, col_bytes);
     float v[1];
     row_dot<WT, U, NB, 1>(b, wrow, cols + (size_t)e * col_bytes, col_bytes, 1, n, q, tb, v, NoTap{});
     if (q == 0 && dl < D) part[dl * spt + e] = v[0];
@@ -1044,6 +1072,9 @@ hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, c
     if (plan == kPlanTwoLaunches) {
         // a down stack on Q8_K columns cannot get them from the gate . up launch (a column's block spans eight of
         // its workgroups): that launch leaves h as f32 rows and the down launch quantizes them itself
+        // (for a down stack on Q8_2_X4 columns the same split measures slower, 12.2 us a token against 11.3 at the
+        // Qwen3 shape: the gate . up launch loses its quantizer epilogue, 0.5 us, but every down workgroup then encodes
+        // the token's 6144 values, 700 instructions a wave that do not hide behind its weight stream)
         const bool hq = bm_takes_q8k(down_type);
         hipError_t e = gate_up_x(L, gate_type, x, wg, wu, n_experts, hidden, ff, sel, spt, m, act_x, hq ? nullptr : act_h, h);
         if (e != hipSuccess) return e;
@@ -1112,7 +1143,7 @@ hipError_t moe_decode_static(const Launch &L, int device, int gate_type, int dow
     // every live slot's column (or f32 rows) is written whole by the first launch before the second reads it, and a
     // slot that is not live is never read into a sum: nothing here has to start at zero
     return moe_decode(L, kPlanTwoLaunches, gate_type, down_type, x, wg, wu, wd, n_experts, hidden, ff, sel, wts, resid,
-                      slots_per_token, m, nullptr, act_h, bm_takes_q8k(down_type) ? h : nullptr, y, nullptr, 0);
+                      slots_per_token, m, nullptr, act_h, h, y, nullptr, 0);
 }
 
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out) {

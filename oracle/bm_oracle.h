@@ -18,10 +18,10 @@
 //                   zero / subnormal / underflowed scales, refused blocks, the sums) and a numpy restatement; the
 //                   32-lane walks by a second spelling from the device's loops over independently decoded blocks,
 //                   one-lane rows that separate the split order from the fused one, and the reference test's f64 band;
-//   weight quantizers   PARITY UNPINNED as bytes: the reference holds no golden bytes for them (it pins them
-//                   against ggml on its own machine). They are held to the reference tests' round-trip bounds,
-//                   zero-row and on-grid properties. Their output is an input shared by the oracle and the GPU
-//                   path, so it does not enter any parity claim.
+//   weight quantizers   no golden bytes exist (the reference checks them against ggml on its own machine): a second
+//                   spelling in numpy written from the reference's text gives the same bytes (K-quants and IQ2_XXS) and
+//                   notices a wrong step count or tie rule; exactly representable rows read back exactly; an IQ2_XXS
+//                   group's signs are the input's but for the flip its parity bit forces; the reference tests' bounds.
 #ifndef BM_ORACLE_H
 #define BM_ORACLE_H
 

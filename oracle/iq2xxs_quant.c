@@ -2,8 +2,10 @@
 // `quantize_row_iq2_xxs_impl` as the reference restates it (crates/gguf/src/iq_quant.rs), every f32 operation
 // rounded on its own (build with -ffp-contract=off), ggml's candidate order and strict tie-breaks.
 //
-// PARITY UNPINNED as bytes: the reference holds no golden bytes for it; it is held to the reference tests'
-// properties (grid tables equal a naive sort, every emitted word on the grid, cosine of the round trip).
+// Pinned without golden bytes (the reference holds none): a second spelling written from the reference's text in
+// numpy gives the same bytes on the reference tests' tie-heavy rows and on N(0, 0.02) rows, and notices a shorter scale
+// search; the stored signs are the input's but for the one flip a group's parity bit forces, at the value the rule
+// names; plus the reference tests' own properties (grid tables equal a naive sort, cosine of the round trip).
 #include <pthread.h>
 #include <stdlib.h>
 

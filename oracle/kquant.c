@@ -3,8 +3,11 @@
 // and square root is its own f32 operation (build with -ffp-contract=off); MAX/MIN are `a > b ? a : b` forms and
 // the searches keep the reference's candidate order and strict tie-breaks.
 //
-// PARITY UNPINNED as bytes: the reference pins these only against ggml on its own machine; here they are held
-// to its round-trip error bounds (crates/gguf/src/kquant/tests.rs:5-60).
+// Pinned without golden bytes (the reference checks these against ggml on its own machine only): a second spelling
+// written from the reference's text in numpy, vectors over all sub-blocks at once, gives the same bytes on the reference
+// tests' row generators, on N(0, 0.02) rows and on rows with zero, flat and all-positive sub-blocks, and notices one
+// search step more or fewer and the other tie rule; rows built from legal blocks whose products are exact read back
+// exactly; plus the reference tests' round-trip bounds (crates/gguf/src/kquant/tests.rs:5-60).
 #include <pthread.h>
 #include <stdlib.h>
 

@@ -654,6 +654,7 @@ struct ora_pool {
     const mt_phase *volatile phase;
     // a sense-reversing barrier the threads spin on: a phase lasts tens of microseconds, a futex wake as long
     volatile int arrived, sense;
+    int caller_sense; // the calling thread's side of the barrier (one caller for the pool's life)
 };
 
 static void spin_barrier(struct ora_pool *p, int *my_sense) {
@@ -738,17 +739,10 @@ ora_pool *ora_pool_create(int n_threads) {
     return p;
 }
 
-// The caller's barrier sense: the caller is one thread for the pool's life.
-static __thread int g_caller_sense;
-static __thread const ora_pool *g_caller_pool;
-
 void ora_pool_destroy(ora_pool *p) {
     if (!p) return;
     p->quit = 1;
-    if (p->n_threads > 1) {
-        if (g_caller_pool != p) g_caller_pool = p, g_caller_sense = p->sense;
-        spin_barrier(p, &g_caller_sense);
-    }
+    if (p->n_threads > 1) spin_barrier(p, &p->caller_sense);
     for (int t = 1; t < p->n_threads; t++) pthread_join(p->ws[t].th, NULL);
     free(p->ws);
     free(p);
@@ -759,11 +753,10 @@ static void pool_run(ora_pool *p, const mt_phase *ph) {
         run_share(ph, 0, 1);
         return;
     }
-    if (g_caller_pool != p) g_caller_pool = p, g_caller_sense = p->sense;
     p->phase = ph;
-    spin_barrier(p, &g_caller_sense);
+    spin_barrier(p, &p->caller_sense);
     run_share(ph, 0, p->n_threads);
-    spin_barrier(p, &g_caller_sense);
+    spin_barrier(p, &p->caller_sense);
 }
 
 // The layer step of ora_moe_forward on the AVX2 kernels and the pool, slots grouped by expert so a weight row is

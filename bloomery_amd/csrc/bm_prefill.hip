@@ -14,6 +14,8 @@
 // Activation scales come per 32 values in this form, so every group's sum is scaled on the vector ALU before it is
 // added: three operations a (row, slot, group) against one matrix instruction per 1024 of them. The kernel is bound
 // by that arithmetic, not by the matrix cores.
+#include <type_traits>
+
 #include "bm_stream.cuh"
 
 namespace bmk {
@@ -604,6 +606,227 @@ __global__ __launch_bounds__(256) void k_gemm_fast(const uint8_t *w, int rpe, in
     }
 }
 
+// ---------------------------------------------------------------- Q4_K, one accumulator a value, 32 x 32 x 32 products
+
+// The tolerance mode's Q4_K kernel. A 32-value sub-block of a row against a 32-value block of a column is exactly one
+// v_mfma_i32_32x32x32_i8 over 32 rows and 32 slots: every issued multiply is a useful one, and what is left for the
+// vector ALU is three operations a (row, slot, block) - the integer to a float, the row's d * sc times the column's d8,
+// the multiply-add. The min terms, sum over a super-block's eight sub-blocks of -(dmin m)[row] x (d8 isum)[slot], are a
+// product of two thin matrices and go to the f32 matrix instruction (v_mfma_f32_32x32x2_f32, four a super-block), into
+// the same accumulators.
+// A workgroup of four waves takes 128 rows and a tile's 64 slots; wave w owns rows 32 w .. and both halves of the
+// slots, so a block's weight operand and its sixteen row scales are read from LDS once for two products. LDS holds one
+// super-block: the columns' codes, the slab's codes unpacked to a byte each, and the scale tables transposed so that a
+// lane's four consecutive result rows are one 16-byte read. Two workgroups share a CU and fill each other's staging
+// gaps; the next super-block's global loads are in flight during the arithmetic on the present one.
+constexpr int kFastRows = 128;
+constexpr int kFastCodeStride = 256 + 16;    // a row's or a column's 256 codes; + 16 keeps 16-byte reads off each other's banks
+constexpr int kFastRowLine = kFastRows + 4;  // floats a line of the row tables (sv, mn: [sub-block][row])
+constexpr int kFastColLine = kGemmBN + 4;    // floats a line of the column tables (d8, d8 * isum: [block][slot])
+constexpr size_t kFastLds = sizeof(GemmLds) + (size_t)kGemmBN * kFastCodeStride + 2 * 8 * kFastColLine * sizeof(float) +
+                            (size_t)kFastRows * kFastCodeStride + 2 * 8 * kFastRowLine * sizeof(float);
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256, 2) void k_gemm_q4k_fast(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
+                                                          const u32 *tiles, const u32 *n_tiles, u32 n_slabs, u32 slot_div,
+                                                          u32 n_slots, float *y) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
+    uint8_t *a_codes = lds + sizeof(GemmLds);
+    float *d8_t = reinterpret_cast<float *>(a_codes + (size_t)kGemmBN * kFastCodeStride);
+    float *my_t = d8_t + 8 * kFastColLine;
+    uint8_t *w_codes = reinterpret_cast<uint8_t *>(my_t + 8 * kFastColLine);
+    float *sv_t = reinterpret_cast<float *>(w_codes + (size_t)kFastRows * kFastCodeStride);
+    float *mn_t = sv_t + 8 * kFastRowLine;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const u32 g = tile_of_block(blockIdx.x, n_slabs);
+    const int row0 = (int)slab_of_block(blockIdx.x, n_slabs) * kFastRows;
+    const u32 count = n_tiles[0];
+    if (g > count) return;
+    if (g == count) { // the refused slots' rows: NaN (crates/gpu/src/gemm/grouped.rs:2283-2287)
+        const u32 refused = n_tiles[1];
+        for (u32 i = tid; i < refused * kFastRows; i += 256) {
+            const u32 s = cols[n_slots - refused + i / kFastRows];
+            const int r = row0 + (int)(i % kFastRows);
+            if (r < rpe) y[(size_t)s * rpe + r] = bm_bits_f32(0x7fc00000u);
+        }
+        return;
+    }
+    const u32 e = tiles[2 * g], word = tiles[2 * g + 1];
+    const int start = (int)(word & 0xffffu), len = (int)(word >> 16);
+    if (tid < kGemmBN) {
+        const u32 s = cols[start + (tid < len ? tid : 0)];
+        tab->slot[tid] = s;
+        tab->col[tid] = s / slot_div;
+    }
+    __syncthreads();
+    const u32 row_bytes = (u32)nb * BM_Q4K_BLOCK, col_bytes = (u32)nb * BM_Q82_SB_EXT;
+    // what this thread stages of every super-block:
+    //   four 16-byte pieces of column codes (column tid / 16 + 16 j, piece tid % 16 of the sixteen: a column's
+    //   super-block is two groups of 144 bytes whose first 16 are scales and sums, skipped here),
+    //   one 16-byte piece of two (d8, d8 * isum) pairs (column tid / 4, pairs 2 (tid % 4) ..),
+    //   half a weight row's nibbles (row tid / 2, 64 bytes) and the row's header
+    const int ac = tid >> 4, ap = tid & 15;
+    u32 src_a[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) src_a[j] = tab->col[ac + 16 * j] * col_bytes + 16u * (u32)(1 + ap + (ap >> 3));
+    const int pcol = tid >> 2, pp = tid & 3;
+    const u32 src_p = tab->col[pcol] * col_bytes + (u32)nb * BM_Q82_SB_REF + 16u * (u32)pp;
+    const int wr = tid >> 1, wh = tid & 1;
+    const uint8_t *we = w + (size_t)e * rpe * row_bytes;
+    const u32 src_w = (u32)(row0 + wr < rpe ? row0 + wr : rpe - 1) * row_bytes;
+    uint4 ra0, ra1, ra2, ra3, rp, rq[4], rh;
+    auto fetch = [&](int i) {
+        ra0 = *reinterpret_cast<const uint4 *>(act + (src_a[0] + (u32)i * BM_Q82_SB_REF));
+        ra1 = *reinterpret_cast<const uint4 *>(act + (src_a[1] + (u32)i * BM_Q82_SB_REF));
+        ra2 = *reinterpret_cast<const uint4 *>(act + (src_a[2] + (u32)i * BM_Q82_SB_REF));
+        ra3 = *reinterpret_cast<const uint4 *>(act + (src_a[3] + (u32)i * BM_Q82_SB_REF));
+        rp = *reinterpret_cast<const uint4 *>(act + (src_p + (u32)i * 64u));
+        const uint8_t *blk = we + (src_w + (u32)i * BM_Q4K_BLOCK);
+        rh = *reinterpret_cast<const uint4 *>(blk);
+#pragma unroll
+        for (int c = 0; c < 4; c++) rq[c] = *reinterpret_cast<const uint4 *>(blk + 16 + 64 * wh + 16 * c);
+    };
+    auto stash = [&]() {
+        uint8_t *acol = a_codes + ac * kFastCodeStride + 16 * ap;
+        *reinterpret_cast<uint4 *>(acol) = ra0;
+        *reinterpret_cast<uint4 *>(acol + 16 * kFastCodeStride) = ra1;
+        *reinterpret_cast<uint4 *>(acol + 32 * kFastCodeStride) = ra2;
+        *reinterpret_cast<uint4 *>(acol + 48 * kFastCodeStride) = ra3;
+        d8_t[(2 * pp) * kFastColLine + pcol] = bm_bits_f32(rp.x);
+        my_t[(2 * pp) * kFastColLine + pcol] = bm_bits_f32(rp.y);
+        d8_t[(2 * pp + 1) * kFastColLine + pcol] = bm_bits_f32(rp.z);
+        my_t[(2 * pp + 1) * kFastColLine + pcol] = bm_bits_f32(rp.w);
+        // nibble piece c of this half: code bytes 64 wh + 16 c ..: the low nibbles are sub-block 2 p, values 16 (c % 2) ..,
+        // the high nibbles sub-block 2 p + 1, the same values, with p = 2 wh + c / 2
+        const u32 ml = 0x0f0f0f0fu;
+        uint8_t *row = w_codes + wr * kFastCodeStride;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int p = 2 * wh + (c >> 1), at = 16 * (c & 1);
+            *reinterpret_cast<uint4 *>(row + 64 * p + at) = make_uint4(rq[c].x & ml, rq[c].y & ml, rq[c].z & ml, rq[c].w & ml);
+            *reinterpret_cast<uint4 *>(row + 64 * p + 32 + at) =
+                make_uint4((rq[c].x >> 4) & ml, (rq[c].y >> 4) & ml, (rq[c].z >> 4) & ml, (rq[c].w >> 4) & ml);
+        }
+        // scale and min of sub-blocks 4 wh .. 4 wh + 3 (crates/gguf/src/quant.rs:620-628 get_scale_min_k4)
+        const float d = bm_half_to_f32(rh.x & 0xffffu), dmin = bm_half_to_f32(rh.x >> 16);
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const u32 qa = (rh.y >> (8 * jj)) & 0xffu, qb = (rh.z >> (8 * jj)) & 0xffu, qc = (rh.w >> (8 * jj)) & 0xffu;
+            const u32 scv = wh ? ((qc & 15u) | ((qa >> 6) << 4)) : (qa & 63u);
+            const u32 mv = wh ? ((qc >> 4) | ((qb >> 6) << 4)) : (qb & 63u);
+            sv_t[(4 * wh + jj) * kFastRowLine + wr] = d * (float)scv;
+            mn_t[(4 * wh + jj) * kFastRowLine + wr] = -(dmin * (float)mv);
+        }
+    };
+    // this lane in a 32 x 32 product: operand row / slot lane % 32, the 16 values 16 (lane / 32) .. of a block; result v
+    // is row 8 (v / 4) + 4 (lane / 32) + v % 4 of slot lane % 32
+    const int l32 = lane & 31, kh = lane >> 5;
+    const uint8_t *my_w = w_codes + (32 * wv + l32) * kFastCodeStride + 16 * kh;
+    const uint8_t *my_a = a_codes + l32 * kFastCodeStride + 16 * kh;
+    const float *my_sv = sv_t + 32 * wv + 4 * kh;
+    const bool two = len > 32; // else the second half of the slots is all padding
+    v16f acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[t][v] = 0.0f;
+
+    // One super-block's products. A unit is a (block, half of the slots): its matrix instruction is issued one unit
+    // ahead of the vector work that scales its sums, and its LDS operands are read two units ahead, so the three engines
+    // (LDS, matrix cores, vector ALU) work on consecutive units at the same time from inside one wave.
+    auto blocks = [&](auto two_tiles) __attribute__((always_inline)) {
+        constexpr bool kTwo = decltype(two_tiles)::value;
+        constexpr int kUnits = kTwo ? 16 : 8;
+        v4i a[2], b[2];
+        float4 sv[2][4];
+        float d8[3];
+        v16i sum[2];
+        auto rd_a = [&](int sb) { a[sb & 1] = *reinterpret_cast<const v4i *>(my_w + 32 * sb); };
+        auto rd_sv = [&](int sb) {
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) sv[sb & 1][q4] = *reinterpret_cast<const float4 *>(my_sv + sb * kFastRowLine + 8 * q4);
+        };
+        auto rd_b = [&](int u) { // unit u's column operand and column scale
+            const int sb = kTwo ? u >> 1 : u, t = kTwo ? u & 1 : 0;
+            b[u & 1] = *reinterpret_cast<const v4i *>(my_a + 32 * t * kFastCodeStride + 32 * sb);
+            d8[u % 3] = d8_t[sb * kFastColLine + 32 * t + l32];
+        };
+        auto product = [&](int u) {
+            const int sb = kTwo ? u >> 1 : u;
+            const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            sum[u & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb & 1], b[u & 1], z, 0, 0, 0);
+        };
+        rd_a(0);
+        rd_b(0);
+        rd_sv(0);
+        product(0);
+        rd_b(1);
+        if (!kTwo) rd_a(1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < kUnits; u++) {
+            const int sb = kTwo ? u >> 1 : u, t = kTwo ? u & 1 : 0;
+            if (u + 1 < kUnits) product(u + 1);
+            if (u + 2 < kUnits) rd_b(u + 2);
+            // the row side of the block after: its codes before its first product is issued (the next unit), its scales
+            // before its first scaling
+            if (kTwo && t == 0 && sb + 1 < 8) rd_a(sb + 1);
+            if (!kTwo && sb + 2 < 8) rd_a(sb + 2);
+            if ((!kTwo || t == 1) && sb + 1 < 8) rd_sv(sb + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            const float dc = d8[u % 3];
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                const float4 r = sv[sb & 1][q4];
+                acc[t][4 * q4 + 0] = fmaf(r.x * dc, (float)sum[u & 1][4 * q4 + 0], acc[t][4 * q4 + 0]);
+                acc[t][4 * q4 + 1] = fmaf(r.y * dc, (float)sum[u & 1][4 * q4 + 1], acc[t][4 * q4 + 1]);
+                acc[t][4 * q4 + 2] = fmaf(r.z * dc, (float)sum[u & 1][4 * q4 + 2], acc[t][4 * q4 + 2]);
+                acc[t][4 * q4 + 3] = fmaf(r.w * dc, (float)sum[u & 1][4 * q4 + 3], acc[t][4 * q4 + 3]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // the min terms last, into the same accumulators: a 32 x 8 by 8 x 32 product in f32, two of the eight sub-blocks an
+        // instruction; they run on the matrix cores while the workgroup goes through its barrier and the next staging
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float mn = mn_t[(2 * j + kh) * kFastRowLine + 32 * wv + l32];
+            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(mn, my_t[(2 * j + kh) * kFastColLine + l32], acc[0], 0, 0, 0);
+            if (kTwo) acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(mn, my_t[(2 * j + kh) * kFastColLine + 32 + l32], acc[1], 0, 0, 0);
+        }
+    };
+
+    fetch(0);
+    for (int i = 0; i < nb; i++) {
+        if (i) __syncthreads(); // the readers of the super-block before are done
+        stash();
+        __syncthreads();
+        if (i + 1 < nb) fetch(i + 1);
+        if (two) blocks(std::true_type{});
+        else blocks(std::false_type{});
+    }
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int n = 32 * t + l32;
+        if (n < len) {
+            float *out = y + (size_t)tab->slot[n] * rpe + row0 + 32 * wv + 4 * kh;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                const int r = row0 + 32 * wv + 4 * kh + 8 * q4;
+                const float4 v4 = make_float4(acc[t][4 * q4 + 0], acc[t][4 * q4 + 1], acc[t][4 * q4 + 2], acc[t][4 * q4 + 3]);
+                if (r + 3 < rpe) {
+                    *reinterpret_cast<float4 *>(out + 8 * q4) = v4; // rows_per_expert is a multiple of 16: 16-byte aligned
+                } else {
+                    if (r + 0 < rpe) out[8 * q4 + 0] = v4.x;
+                    if (r + 1 < rpe) out[8 * q4 + 1] = v4.y;
+                    if (r + 2 < rpe) out[8 * q4 + 2] = v4.z;
+                }
+            }
+        }
+    }
+}
+
 bool gemm_supported(int wtype) { return wtype == BM_Q4K || wtype == BM_Q5K || wtype == BM_Q6K; }
 
 hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int rows_per_expert, int k,
@@ -623,7 +846,15 @@ hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int
         return hipGetLastError();
     };
     if (mode == 1) { // Q5_K has no kernel of this kind and takes the exact one
-        if (wtype == BM_Q4K) return launch(k_gemm_fast<BM_Q4K>, 256, gemm_lds_bytes<BM_Q4K>(), 1);
+        if (wtype == BM_Q4K) {
+            hipError_t e = allow_lds(k_gemm_q4k_fast, kFastLds);
+            if (e != hipSuccess) return e;
+            const u32 n_slabs_f = (u32)((rows_per_expert + kFastRows - 1) / kFastRows);
+            const unsigned grid = ((max_tiles + 7) / 8) * 8 * n_slabs_f;
+            hipLaunchKernelGGL(k_gemm_q4k_fast, dim3(grid), dim3(256), kFastLds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
+                               n_tiles, n_slabs_f, (u32)slot_div, (u32)n_slots, y);
+            return hipGetLastError();
+        }
         if (wtype == BM_Q6K) return launch(k_gemm_fast<BM_Q6K>, 256, gemm_lds_bytes<BM_Q6K>(), 1);
     }
     // 512 threads on 32 slots of a tile for both types (Q4_K 114 registers, Q6_K 121): two workgroups a CU. Measured

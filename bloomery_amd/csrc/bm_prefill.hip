@@ -101,24 +101,11 @@ hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, 
 // rows' scale products. Strides are padded off the 128-byte bank period.
 constexpr int kActSb = BM_Q82_SB_REF + 64;   // a column's super-block: its two groups and its (d8, d8 * isum) pairs
 constexpr int kActStride = kActSb + 8;       // 360
-template <int WT>
-__host__ __device__ constexpr int wt_stride() {
-    return WT == BM_Q4K ? 152 : 232; // 144 and 224 (14 chunks of 16) padded
-}
-template <int WT>
-__host__ __device__ constexpr int wt_chunks() {
-    return WT == BM_Q4K ? 9 : 14;
-}
 
 struct GemmLds {
     u32 col[kGemmBN];  // the tile's activation columns
     u32 slot[kGemmBN]; // and slots
 };
-
-template <int WT>
-__host__ __device__ constexpr size_t gemm_lds_bytes() {
-    return sizeof(GemmLds) + (size_t)kGemmBN * kActStride + (size_t)kGemmBM * wt_stride<WT>() + 16 * kGemmBM * sizeof(float);
-}
 
 // Workgroup b of a GEMM grid: tile and row slab. Workgroups go to the chip's eight dies in turn (b to die b % 8,
 // each with its own L2), so a tile's row slabs are consecutive workgroups of one die: the tile's activation columns
@@ -401,244 +388,62 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
     }
 }
 
-// The same product with one accumulator a value: each 32-value block's integer sum (Q4_K: two chained matrix
-// instructions) or 16-value group's (Q6_K) is scaled and added in increasing k, a block's min term just before it.
-// The integers are the exact ones; the f32 sum is not in the CPU path's eight-lane order, so a value differs from
-// the exact kernel's by rounding only (a few 1e-7 of the row's magnitude; the contract's tolerance is 1e-4). A third
-// fewer vector operations and an eighth of the accumulator registers: 32 x 32 tiles, four waves, several
-// workgroups a CU.
+// ------------------------------------------------------ one accumulator a value: whole-block matrix instructions
+
 typedef int v16i __attribute__((ext_vector_type(16)));
-
-template <int WT>
-__global__ __launch_bounds__(256) void k_gemm_fast(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
-                                                   const u32 *tiles, const u32 *n_tiles, u32 n_slabs, u32 slot_div,
-                                                   u32 n_slots, float *y) {
-    extern __shared__ __align__(16) uint8_t lds[];
-    GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
-    uint8_t *acts = lds + sizeof(GemmLds);
-    uint8_t *wts = acts + (size_t)kGemmBN * kActStride;
-    float *rs = reinterpret_cast<float *>(wts + (size_t)kGemmBM * wt_stride<WT>()); // [16][64]
-    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    const u32 g = tile_of_block(blockIdx.x, n_slabs);
-    const int row0 = (int)slab_of_block(blockIdx.x, n_slabs) * kGemmBM;
-    const u32 count = n_tiles[0];
-    if (g > count) return;
-    if (g == count) {
-        const u32 refused = n_tiles[1];
-        for (u32 i = tid; i < refused * kGemmBM; i += blockDim.x) {
-            const u32 s = cols[n_slots - refused + i / kGemmBM];
-            const int r = row0 + (int)(i % kGemmBM);
-            if (r < rpe) y[(size_t)s * rpe + r] = bm_bits_f32(0x7fc00000u);
-        }
-        return;
-    }
-    const u32 e = tiles[2 * g], word = tiles[2 * g + 1];
-    const int start = (int)(word & 0xffffu), len = (int)(word >> 16);
-    if (tid < kGemmBN) {
-        const u32 s = cols[start + (tid < len ? tid : 0)];
-        tab->slot[tid] = s;
-        tab->col[tid] = s / slot_div;
-    }
-    __syncthreads();
-    constexpr int kBlock = WT == BM_Q4K ? BM_Q4K_BLOCK : BM_Q6K_BLOCK;
-    constexpr int kWc = wt_chunks<WT>();
-    const size_t row_bytes = (size_t)nb * kBlock;
-    const int col_bytes = nb * BM_Q82_SB_EXT;
-    constexpr int kAc = kActSb / 16; // 22
-    constexpr int kActLoads = (kGemmBN * kAc + 255) / 256, kWtLoads = (kGemmBM * kWc + 255) / 256;
-    uint4 ra[kActLoads], rw[kWtLoads];
-    auto fetch = [&](int i) {
-#pragma unroll
-        for (int t = 0; t < kActLoads; t++) {
-            int c = t * 256 + tid;
-            c = c < kGemmBN * kAc ? c : kGemmBN * kAc - 1;
-            const int n = c / kAc, k = c % kAc;
-            const uint8_t *colp = act + (size_t)tab->col[n] * col_bytes;
-            const uint8_t *src = k < 18 ? colp + (size_t)i * BM_Q82_SB_REF + 16 * k
-                                        : colp + (size_t)nb * BM_Q82_SB_REF + (size_t)i * 64 + 16 * (k - 18);
-            ra[t] = *reinterpret_cast<const uint4 *>(src);
-        }
-#pragma unroll
-        for (int t = 0; t < kWtLoads; t++) {
-            int c = t * 256 + tid;
-            c = c < kGemmBM * kWc ? c : kGemmBM * kWc - 1;
-            int r = row0 + c / kWc;
-            const int k = c % kWc;
-            r = r < rpe ? r : rpe - 1;
-            const uint8_t *blk = w + ((size_t)e * rpe + r) * row_bytes + (size_t)i * kBlock;
-            rw[t] = bm_ld16u(blk + ((WT == BM_Q6K && k == 13) ? 194 : 16 * k));
-        }
-    };
-    auto stash = [&]() {
-#pragma unroll
-        for (int t = 0; t < kActLoads; t++) {
-            const int c = t * 256 + tid;
-            if (c < kGemmBN * kAc) {
-                uint8_t *dst = acts + (c / kAc) * kActStride + 16 * (c % kAc);
-                *reinterpret_cast<uint2 *>(dst) = make_uint2(ra[t].x, ra[t].y);
-                *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(ra[t].z, ra[t].w);
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < kWtLoads; t++) {
-            const int c = t * 256 + tid;
-            if (c < kGemmBM * kWc) {
-                uint8_t *dst = wts + (c / kWc) * wt_stride<WT>() + 16 * (c % kWc);
-                *reinterpret_cast<uint2 *>(dst) = make_uint2(rw[t].x, rw[t].y);
-                *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(rw[t].z, rw[t].w);
-            }
-        }
-    };
-    // v_mfma_i32_32x32x16_i8: operand row / slot lane % 32, values 8 * (lane / 32) .. + 8 of a 16-value group; result v
-    // is row 8 * (v / 4) + 4 * (lane / 32) + v % 4 of slot lane % 32
-    const int wr = wv & 1, wc = wv >> 1, l32 = lane & 31, kh = lane >> 5;
-    const uint8_t *my_act = acts + (32 * wc + l32) * kActStride;
-    const uint8_t *my_wt = wts + (32 * wr + l32) * wt_stride<WT>();
-    const int rbase = 32 * wr + 4 * kh;
-    float acc[16];
-#pragma unroll
-    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
-
-    fetch(0);
-    for (int i = 0; i < nb; i++) {
-        __syncthreads();
-        stash();
-        __syncthreads();
-        if (i + 1 < nb) fetch(i + 1);
-        {
-            const int r = tid >> 2, part = tid & 3;
-            const uint8_t *blk = wts + r * wt_stride<WT>();
-            if constexpr (WT == BM_Q4K) {
-                const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk));
-                const float dmin = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk + 2));
-                const uint8_t *sc = blk + 4;
-#pragma unroll
-                for (int t = 0; t < 2; t++) { // crates/gguf/src/quant.rs:620-628 get_scale_min_k4
-                    const int s = 2 * part + t;
-                    int scv, mv;
-                    if (s < 4) {
-                        scv = sc[s] & 63;
-                        mv = sc[s + 4] & 63;
-                    } else {
-                        scv = (sc[s + 4] & 15) | ((sc[s - 4] >> 6) << 4);
-                        mv = (sc[s + 4] >> 4) | ((sc[s] >> 6) << 4);
-                    }
-                    rs[s * kGemmBM + r] = d * (float)scv;
-                    rs[(8 + s) * kGemmBM + r] = -(dmin * (float)mv);
-                }
-            } else {
-                const float d = bm_half_to_f32(*reinterpret_cast<const unsigned short *>(blk + 222));
-#pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    const int gq = 4 * part + t;
-                    rs[gq * kGemmBM + r] = d * (float)(int)(signed char)blk[192 + gq];
-                }
-            }
-        }
-        __syncthreads();
-        if (32 * wc >= len) continue; // none of this wave's slots is real (the barriers above are the loop's only ones)
-        const float2 *pair = reinterpret_cast<const float2 *>(my_act + BM_Q82_SB_REF);
-        if constexpr (WT == BM_Q4K) {
-#pragma unroll
-            for (int p = 0; p < 4; p++) {
-                uint2 wq[2];
-#pragma unroll
-                for (int h = 0; h < 2; h++) wq[h] = *reinterpret_cast<const uint2 *>(my_wt + 16 + 32 * p + 16 * h + 8 * kh);
-#pragma unroll
-                for (int en = 0; en < 2; en++) {
-                    const int s = 2 * p + en;
-                    v16i sum = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-                    for (int h = 0; h < 2; h++) {
-                        const u32 ax = (wq[h].x >> (4 * en)) & 0x0f0f0f0fu, ay = (wq[h].y >> (4 * en)) & 0x0f0f0f0fu;
-                        const uint2 bq = *reinterpret_cast<const uint2 *>(my_act + (s >> 2) * BM_Q82X4_STRIDE + 16 +
-                                                                          32 * (s & 3) + 16 * h + 8 * kh);
-                        sum = __builtin_amdgcn_mfma_i32_32x32x16_i8((long)(((unsigned long long)ay << 32) | ax),
-                                                                    (long)(((unsigned long long)bq.y << 32) | bq.x), sum, 0, 0, 0);
-                    }
-                    const float d8 = pair[s].x, my = pair[s].y;
-#pragma unroll
-                    for (int qd = 0; qd < 4; qd++) {
-                        const float4 mn = *reinterpret_cast<const float4 *>(&rs[(8 + s) * kGemmBM + rbase + 8 * qd]);
-                        const float4 sv = *reinterpret_cast<const float4 *>(&rs[s * kGemmBM + rbase + 8 * qd]);
-                        acc[4 * qd + 0] = fmaf(sv.x * d8, (float)sum[4 * qd + 0], fmaf(my, mn.x, acc[4 * qd + 0]));
-                        acc[4 * qd + 1] = fmaf(sv.y * d8, (float)sum[4 * qd + 1], fmaf(my, mn.y, acc[4 * qd + 1]));
-                        acc[4 * qd + 2] = fmaf(sv.z * d8, (float)sum[4 * qd + 2], fmaf(my, mn.z, acc[4 * qd + 2]));
-                        acc[4 * qd + 3] = fmaf(sv.w * d8, (float)sum[4 * qd + 3], fmaf(my, mn.w, acc[4 * qd + 3]));
-                    }
-                }
-            }
-        } else {
-#pragma unroll
-            for (int gq = 0; gq < 16; gq++) {
-                const int c2 = gq >> 3, a4 = (gq & 7) >> 1, hh = gq & 1, bk = gq >> 1;
-                const int l0 = 16 * hh + 8 * kh;
-                const uint2 ql = *reinterpret_cast<const uint2 *>(my_wt + 64 * c2 + 32 * (a4 & 1) + l0);
-                const uint2 qh = *reinterpret_cast<const uint2 *>(my_wt + 128 + 32 * c2 + l0);
-                const int ns = 4 * (a4 >> 1), hs = 2 * a4;
-                const u32 ax = q6_minus_32(((ql.x >> ns) & 0x0f0f0f0fu) | (((qh.x >> hs) & 0x03030303u) << 4));
-                const u32 ay = q6_minus_32(((ql.y >> ns) & 0x0f0f0f0fu) | (((qh.y >> hs) & 0x03030303u) << 4));
-                const uint2 bq = *reinterpret_cast<const uint2 *>(my_act + (bk >> 2) * BM_Q82X4_STRIDE + 16 + 32 * (bk & 3) +
-                                                                  16 * hh + 8 * kh);
-                const float d8 = pair[bk].x;
-                const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                const v16i sum = __builtin_amdgcn_mfma_i32_32x32x16_i8((long)(((unsigned long long)ay << 32) | ax),
-                                                                       (long)(((unsigned long long)bq.y << 32) | bq.x), z, 0, 0, 0);
-#pragma unroll
-                for (int qd = 0; qd < 4; qd++) {
-                    const float4 sv = *reinterpret_cast<const float4 *>(&rs[gq * kGemmBM + rbase + 8 * qd]);
-                    acc[4 * qd + 0] = fmaf(sv.x * d8, (float)sum[4 * qd + 0], acc[4 * qd + 0]);
-                    acc[4 * qd + 1] = fmaf(sv.y * d8, (float)sum[4 * qd + 1], acc[4 * qd + 1]);
-                    acc[4 * qd + 2] = fmaf(sv.z * d8, (float)sum[4 * qd + 2], acc[4 * qd + 2]);
-                    acc[4 * qd + 3] = fmaf(sv.w * d8, (float)sum[4 * qd + 3], acc[4 * qd + 3]);
-                }
-            }
-        }
-    }
-    const int n = 32 * wc + l32;
-    if (n < len) {
-        const size_t out = (size_t)tab->slot[n] * rpe + row0;
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int r = rbase + 8 * (v >> 2) + (v & 3);
-            if (row0 + r < rpe) y[out + r] = acc[v];
-        }
-    }
-}
-
-// ---------------------------------------------------------------- Q4_K, one accumulator a value, 32 x 32 x 32 products
-
-// The tolerance mode's Q4_K kernel. A 32-value sub-block of a row against a 32-value block of a column is exactly one
-// v_mfma_i32_32x32x32_i8 over 32 rows and 32 slots: every issued multiply is a useful one, and what is left for the
-// vector ALU is three operations a (row, slot, block) - the integer to a float, the row's d * sc times the column's d8,
-// the multiply-add. The min terms, sum over a super-block's eight sub-blocks of -(dmin m)[row] x (d8 isum)[slot], are a
-// product of two thin matrices and go to the f32 matrix instruction (v_mfma_f32_32x32x2_f32, four a super-block), into
-// the same accumulators.
-// A workgroup of four waves takes 128 rows and a tile's 64 slots; wave w owns rows 32 w .. and both halves of the
-// slots, so a block's weight operand and its sixteen row scales are read from LDS once for two products. LDS holds one
-// super-block: the columns' codes, the slab's codes unpacked to a byte each, and the scale tables transposed so that a
-// lane's four consecutive result rows are one 16-byte read. Two workgroups share a CU and fill each other's staging
-// gaps; the next super-block's global loads are in flight during the arithmetic on the present one.
-constexpr int kFastRows = 128;
-constexpr int kFastCodeStride = 256 + 16;    // a row's or a column's 256 codes; + 16 keeps 16-byte reads off each other's banks
-constexpr int kFastRowLine = kFastRows + 4;  // floats a line of the row tables (sv, mn: [sub-block][row])
-constexpr int kFastColLine = kGemmBN + 4;    // floats a line of the column tables (d8, d8 * isum: [block][slot])
-constexpr size_t kFastLds = sizeof(GemmLds) + (size_t)kGemmBN * kFastCodeStride + 2 * 8 * kFastColLine * sizeof(float) +
-                            (size_t)kFastRows * kFastCodeStride + 2 * 8 * kFastRowLine * sizeof(float);
-
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-__global__ __launch_bounds__(256, 2) void k_gemm_q4k_fast(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
-                                                          const u32 *tiles, const u32 *n_tiles, u32 n_slabs, u32 slot_div,
-                                                          u32 n_slots, float *y) {
+// The tolerance mode (BM_GEMM_FAST). The integer sums are the exact ones, formed by matrix instructions whose K is
+// exactly the span one scale covers, so no issued multiply is wasted:
+//   Q4_K, Q5_K: a 32-value sub-block of a row against a 32-value block of a column is one v_mfma_i32_32x32x32_i8 over 32
+//         rows and 32 slots; the min terms, sum over a super-block's eight sub-blocks of -(dmin m)[row] x (d8 isum)[slot],
+//         are a product of two thin matrices and go to v_mfma_f32_32x32x2_f32 (four a super-block), into the same
+//         accumulators;
+//   Q6_K: a 16-value group, whose scale is its own, is one v_mfma_i32_32x32x16_i8.
+// What is left for the vector ALU is three operations a (row, slot, unit): the integer to a float, the row's d * sc times
+// the column's d8, the multiply-add into the one accumulator a value (the CPU path keeps eight and a fixed order: that
+// is the exact mode; this one differs from it by f32 rounding only).
+// A workgroup of four waves takes 128 rows and a tile's 64 slots; wave w owns rows 32 w .. and both halves of the slots,
+// so a unit's weight operand and its sixteen row scales are read from LDS once for two products. LDS holds one
+// super-block: the columns' codes, the slab's codes unpacked to a signed byte each, and the scale tables transposed so
+// that a lane's four consecutive result rows are one 16-byte read. Two workgroups share a CU and fill each other's
+// staging gaps; the next super-block's global loads are in flight during the arithmetic on the present one. Inside a
+// wave a unit's matrix instruction is issued one unit ahead of the vector work that scales its sums, and its LDS
+// operands are read two units ahead.
+constexpr int kFastRows = 128;
+constexpr int kFastRowLine = kFastRows + 4; // floats a line of the row tables ([unit][row])
+constexpr int kFastColLine = kGemmBN + 4;   // floats a line of the column tables ([block][slot])
+// a row's or a column's 256 codes, padded so that the operand reads of consecutive rows fall on different banks: the
+// reads are 16 bytes a lane for K = 32 and 8 bytes a lane for K = 16
+template <int WT>
+__host__ __device__ constexpr int fast_code_stride() {
+    return WT == BM_Q6K ? 256 + 8 : 256 + 16;
+}
+template <int WT>
+__host__ __device__ constexpr int fast_units() { // scaled units a super-block
+    return WT == BM_Q6K ? 16 : 8;
+}
+template <int WT>
+__host__ __device__ constexpr size_t fast_lds_bytes() {
+    return sizeof(GemmLds) + (size_t)(kGemmBN + kFastRows) * fast_code_stride<WT>() + 2 * 8 * kFastColLine * sizeof(float) +
+           2 * (size_t)fast_units<WT>() * kFastRowLine * sizeof(float);
+}
+
+template <int WT>
+__global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
+                                                      const u32 *tiles, const u32 *n_tiles, u32 n_slabs, u32 slot_div,
+                                                      u32 n_slots, float *y) {
+    constexpr bool kQ45 = WT == BM_Q4K || WT == BM_Q5K;
+    constexpr int kStride = fast_code_stride<WT>(), kUnitsSb = fast_units<WT>(), kBlock = bm_block_bytes<WT>();
+    constexpr int kOp = kQ45 ? 16 : 8; // operand bytes a lane
     extern __shared__ __align__(16) uint8_t lds[];
     GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
     uint8_t *a_codes = lds + sizeof(GemmLds);
-    float *d8_t = reinterpret_cast<float *>(a_codes + (size_t)kGemmBN * kFastCodeStride);
+    uint8_t *w_codes = a_codes + (size_t)kGemmBN * kStride;
+    float *d8_t = reinterpret_cast<float *>(w_codes + (size_t)kFastRows * kStride);
     float *my_t = d8_t + 8 * kFastColLine;
-    uint8_t *w_codes = reinterpret_cast<uint8_t *>(my_t + 8 * kFastColLine);
-    float *sv_t = reinterpret_cast<float *>(w_codes + (size_t)kFastRows * kFastCodeStride);
-    float *mn_t = sv_t + 8 * kFastRowLine;
+    float *sv_t = my_t + 8 * kFastColLine;
+    float *mn_t = sv_t + kUnitsSb * kFastRowLine; // Q4_K, Q5_K only
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const u32 g = tile_of_block(blockIdx.x, n_slabs);
     const int row0 = (int)slab_of_block(blockIdx.x, n_slabs) * kFastRows;
@@ -661,12 +466,12 @@ __global__ __launch_bounds__(256, 2) void k_gemm_q4k_fast(const uint8_t *w, int 
         tab->col[tid] = s / slot_div;
     }
     __syncthreads();
-    const u32 row_bytes = (u32)nb * BM_Q4K_BLOCK, col_bytes = (u32)nb * BM_Q82_SB_EXT;
+    const u32 row_bytes = (u32)nb * kBlock, col_bytes = (u32)nb * BM_Q82_SB_EXT;
     // what this thread stages of every super-block:
     //   four 16-byte pieces of column codes (column tid / 16 + 16 j, piece tid % 16 of the sixteen: a column's
     //   super-block is two groups of 144 bytes whose first 16 are scales and sums, skipped here),
     //   one 16-byte piece of two (d8, d8 * isum) pairs (column tid / 4, pairs 2 (tid % 4) ..),
-    //   half a weight row's nibbles (row tid / 2, 64 bytes) and the row's header
+    //   half a weight row (row tid / 2): its half of the codes and what the row's scales need
     const int ac = tid >> 4, ap = tid & 15;
     u32 src_a[4];
 #pragma unroll
@@ -676,55 +481,118 @@ __global__ __launch_bounds__(256, 2) void k_gemm_q4k_fast(const uint8_t *w, int 
     const int wr = tid >> 1, wh = tid & 1;
     const uint8_t *we = w + (size_t)e * rpe * row_bytes;
     const u32 src_w = (u32)(row0 + wr < rpe ? row0 + wr : rpe - 1) * row_bytes;
-    uint4 ra0, ra1, ra2, ra3, rp, rq[4], rh;
+    uint4 ra0, ra1, ra2, ra3, rp, rq[4], rh, rx0, rx1;
     auto fetch = [&](int i) {
         ra0 = *reinterpret_cast<const uint4 *>(act + (src_a[0] + (u32)i * BM_Q82_SB_REF));
         ra1 = *reinterpret_cast<const uint4 *>(act + (src_a[1] + (u32)i * BM_Q82_SB_REF));
         ra2 = *reinterpret_cast<const uint4 *>(act + (src_a[2] + (u32)i * BM_Q82_SB_REF));
         ra3 = *reinterpret_cast<const uint4 *>(act + (src_a[3] + (u32)i * BM_Q82_SB_REF));
         rp = *reinterpret_cast<const uint4 *>(act + (src_p + (u32)i * 64u));
-        const uint8_t *blk = we + (src_w + (u32)i * BM_Q4K_BLOCK);
-        rh = *reinterpret_cast<const uint4 *>(blk);
+        const uint8_t *blk = we + (src_w + (u32)i * kBlock);
+        if constexpr (kQ45) {
+            constexpr int kCodesAt = WT == BM_Q5K ? 48 : 16;
+            rh = *reinterpret_cast<const uint4 *>(blk); // d, dmin, the twelve scale bytes
 #pragma unroll
-        for (int c = 0; c < 4; c++) rq[c] = *reinterpret_cast<const uint4 *>(blk + 16 + 64 * wh + 16 * c);
+            for (int c = 0; c < 4; c++) rq[c] = *reinterpret_cast<const uint4 *>(blk + kCodesAt + 64 * wh + 16 * c);
+            if constexpr (WT == BM_Q5K) { // the 32 high-bit bytes: value n's fifth bit is bit n / 32 of byte n % 32
+                rx0 = *reinterpret_cast<const uint4 *>(blk + 16);
+                rx1 = *reinterpret_cast<const uint4 *>(blk + 32);
+            }
+        } else { // half wh of the block: ql bytes 64 wh .. (four pieces), qh bytes 32 wh .. (two), the sixteen scales, d
+#pragma unroll
+            for (int c = 0; c < 4; c++) rq[c] = bm_ld16u(blk + 64 * wh + 16 * c);
+            rx0 = bm_ld16u(blk + 128 + 32 * wh);
+            rx1 = bm_ld16u(blk + 128 + 32 * wh + 16);
+            rh = bm_ld16u(blk + 192);
+            rh.x = wh ? rh.z : rh.x; // this half's eight scale bytes
+            rh.y = wh ? rh.w : rh.y;
+            rh.z = bm_ld2u(blk + 208); // d
+        }
+    };
+    auto put16 = [](uint8_t *dst, u32 a, u32 b, u32 c, u32 d) {
+        if constexpr (kOp == 16) {
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(a, b, c, d);
+        } else { // rows 8 bytes apart modulo 16
+            *reinterpret_cast<uint2 *>(dst) = make_uint2(a, b);
+            *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(c, d);
+        }
     };
     auto stash = [&]() {
-        uint8_t *acol = a_codes + ac * kFastCodeStride + 16 * ap;
-        *reinterpret_cast<uint4 *>(acol) = ra0;
-        *reinterpret_cast<uint4 *>(acol + 16 * kFastCodeStride) = ra1;
-        *reinterpret_cast<uint4 *>(acol + 32 * kFastCodeStride) = ra2;
-        *reinterpret_cast<uint4 *>(acol + 48 * kFastCodeStride) = ra3;
+        uint8_t *acol = a_codes + ac * kStride + 16 * ap;
+        put16(acol, ra0.x, ra0.y, ra0.z, ra0.w);
+        put16(acol + 16 * kStride, ra1.x, ra1.y, ra1.z, ra1.w);
+        put16(acol + 32 * kStride, ra2.x, ra2.y, ra2.z, ra2.w);
+        put16(acol + 48 * kStride, ra3.x, ra3.y, ra3.z, ra3.w);
         d8_t[(2 * pp) * kFastColLine + pcol] = bm_bits_f32(rp.x);
-        my_t[(2 * pp) * kFastColLine + pcol] = bm_bits_f32(rp.y);
         d8_t[(2 * pp + 1) * kFastColLine + pcol] = bm_bits_f32(rp.z);
-        my_t[(2 * pp + 1) * kFastColLine + pcol] = bm_bits_f32(rp.w);
-        // nibble piece c of this half: code bytes 64 wh + 16 c ..: the low nibbles are sub-block 2 p, values 16 (c % 2) ..,
-        // the high nibbles sub-block 2 p + 1, the same values, with p = 2 wh + c / 2
-        const u32 ml = 0x0f0f0f0fu;
-        uint8_t *row = w_codes + wr * kFastCodeStride;
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const int p = 2 * wh + (c >> 1), at = 16 * (c & 1);
-            *reinterpret_cast<uint4 *>(row + 64 * p + at) = make_uint4(rq[c].x & ml, rq[c].y & ml, rq[c].z & ml, rq[c].w & ml);
-            *reinterpret_cast<uint4 *>(row + 64 * p + 32 + at) =
-                make_uint4((rq[c].x >> 4) & ml, (rq[c].y >> 4) & ml, (rq[c].z >> 4) & ml, (rq[c].w >> 4) & ml);
+        if constexpr (kQ45) {
+            my_t[(2 * pp) * kFastColLine + pcol] = bm_bits_f32(rp.y);
+            my_t[(2 * pp + 1) * kFastColLine + pcol] = bm_bits_f32(rp.w);
         }
-        // scale and min of sub-blocks 4 wh .. 4 wh + 3 (crates/gguf/src/quant.rs:620-628 get_scale_min_k4)
-        const float d = bm_half_to_f32(rh.x & 0xffffu), dmin = bm_half_to_f32(rh.x >> 16);
+        const u32 ml = 0x0f0f0f0fu;
+        uint8_t *row = w_codes + wr * kStride;
+        if constexpr (kQ45) {
+            // nibble piece c of this half: code bytes 64 wh + 16 c ..: the low nibbles are sub-block 2 p, values
+            // 16 (c % 2) .., the high nibbles sub-block 2 p + 1, the same values, with p = 2 wh + c / 2
 #pragma unroll
-        for (int jj = 0; jj < 4; jj++) {
-            const u32 qa = (rh.y >> (8 * jj)) & 0xffu, qb = (rh.z >> (8 * jj)) & 0xffu, qc = (rh.w >> (8 * jj)) & 0xffu;
-            const u32 scv = wh ? ((qc & 15u) | ((qa >> 6) << 4)) : (qa & 63u);
-            const u32 mv = wh ? ((qc >> 4) | ((qb >> 6) << 4)) : (qb & 63u);
-            sv_t[(4 * wh + jj) * kFastRowLine + wr] = d * (float)scv;
-            mn_t[(4 * wh + jj) * kFastRowLine + wr] = -(dmin * (float)mv);
+            for (int c = 0; c < 4; c++) {
+                const int p = 2 * wh + (c >> 1), at = 16 * (c & 1);
+                u32 lo[4] = {rq[c].x & ml, rq[c].y & ml, rq[c].z & ml, rq[c].w & ml};
+                u32 hi[4] = {(rq[c].x >> 4) & ml, (rq[c].y >> 4) & ml, (rq[c].z >> 4) & ml, (rq[c].w >> 4) & ml};
+                if constexpr (WT == BM_Q5K) { // high-bit bytes 16 (c % 2) ..: bit 2 p for the low nibbles, 2 p + 1 for the high
+                    const uint4 hb = (c & 1) ? rx1 : rx0;
+                    const u32 hw[4] = {hb.x, hb.y, hb.z, hb.w};
+                    const u32 one = 0x01010101u;
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        lo[k] |= ((hw[k] >> (2 * p)) & one) << 4;
+                        hi[k] |= ((hw[k] >> (2 * p + 1)) & one) << 4;
+                    }
+                }
+                put16(row + 64 * p + at, lo[0], lo[1], lo[2], lo[3]);
+                put16(row + 64 * p + 32 + at, hi[0], hi[1], hi[2], hi[3]);
+            }
+            // scale and min of sub-blocks 4 wh .. 4 wh + 3 (crates/gguf/src/quant.rs:620-628 get_scale_min_k4)
+            const float d = bm_half_to_f32(rh.x & 0xffffu), dmin = bm_half_to_f32(rh.x >> 16);
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) {
+                const u32 qa = (rh.y >> (8 * jj)) & 0xffu, qb = (rh.z >> (8 * jj)) & 0xffu, qc = (rh.w >> (8 * jj)) & 0xffu;
+                const u32 scv = wh ? ((qc & 15u) | ((qa >> 6) << 4)) : (qa & 63u);
+                const u32 mv = wh ? ((qc >> 4) | ((qb >> 6) << 4)) : (qb & 63u);
+                sv_t[(4 * wh + jj) * kFastRowLine + wr] = d * (float)scv;
+                mn_t[(4 * wh + jj) * kFastRowLine + wr] = -(dmin * (float)mv);
+            }
+        } else {
+            // ql piece c of this half (bytes 64 wh + 16 c ..) with qh piece c % 2: the low nibbles are quarter c / 2 of the
+            // half, values 16 (c % 2) .., the high nibbles quarter 2 + c / 2; a quarter's high bits are bits 2 a .. of qh
+            // (crates/gguf/src/quant.rs:826-859). Each is one 16-value group: group 8 wh + 2 a + c % 2.
+            const u32 mh = 0x03030303u;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const uint4 hq = (c & 1) ? rx1 : rx0;
+#pragma unroll
+                for (int hn = 0; hn < 2; hn++) {
+                    const int a4 = (c >> 1) + 2 * hn, ns = 4 * hn, hs = 2 * a4;
+                    put16(row + 128 * wh + 32 * a4 + 16 * (c & 1),
+                          q6_minus_32(((rq[c].x >> ns) & ml) | (((hq.x >> hs) & mh) << 4)),
+                          q6_minus_32(((rq[c].y >> ns) & ml) | (((hq.y >> hs) & mh) << 4)),
+                          q6_minus_32(((rq[c].z >> ns) & ml) | (((hq.z >> hs) & mh) << 4)),
+                          q6_minus_32(((rq[c].w >> ns) & ml) | (((hq.w >> hs) & mh) << 4)));
+                }
+            }
+            const float d = bm_half_to_f32(rh.z & 0xffffu);
+#pragma unroll
+            for (int jj = 0; jj < 8; jj++) {
+                const u32 word = jj < 4 ? rh.x : rh.y;
+                sv_t[(8 * wh + jj) * kFastRowLine + wr] = d * (float)(int)(signed char)((word >> (8 * (jj & 3))) & 0xffu);
+            }
         }
     };
-    // this lane in a 32 x 32 product: operand row / slot lane % 32, the 16 values 16 (lane / 32) .. of a block; result v
+    // this lane in a 32 x 32 product: operand row / slot lane % 32, its share of the unit's values (lane / 32); result v
     // is row 8 (v / 4) + 4 (lane / 32) + v % 4 of slot lane % 32
     const int l32 = lane & 31, kh = lane >> 5;
-    const uint8_t *my_w = w_codes + (32 * wv + l32) * kFastCodeStride + 16 * kh;
-    const uint8_t *my_a = a_codes + l32 * kFastCodeStride + 16 * kh;
+    const uint8_t *my_w = w_codes + (32 * wv + l32) * kStride + kOp * kh;
+    const uint8_t *my_a = a_codes + l32 * kStride + kOp * kh;
     const float *my_sv = sv_t + 32 * wv + 4 * kh;
     const bool two = len > 32; // else the second half of the slots is all padding
     v16f acc[2];
@@ -733,30 +601,30 @@ __global__ __launch_bounds__(256, 2) void k_gemm_q4k_fast(const uint8_t *w, int 
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[t][v] = 0.0f;
 
-    // One super-block's products. A unit is a (block, half of the slots): its matrix instruction is issued one unit
-    // ahead of the vector work that scales its sums, and its LDS operands are read two units ahead, so the three engines
-    // (LDS, matrix cores, vector ALU) work on consecutive units at the same time from inside one wave.
+    // One super-block's products. A step is a (unit, half of the slots).
     auto blocks = [&](auto two_tiles) __attribute__((always_inline)) {
         constexpr bool kTwo = decltype(two_tiles)::value;
-        constexpr int kUnits = kTwo ? 16 : 8;
-        v4i a[2], b[2];
+        constexpr int kSteps = (kTwo ? 2 : 1) * kUnitsSb;
+        typedef typename std::conditional<kQ45, v4i, long>::type Operand;
+        Operand a[2], b[2];
         float4 sv[2][4];
         float d8[3];
         v16i sum[2];
-        auto rd_a = [&](int sb) { a[sb & 1] = *reinterpret_cast<const v4i *>(my_w + 32 * sb); };
-        auto rd_sv = [&](int sb) {
+        auto rd_a = [&](int un) { a[un & 1] = *reinterpret_cast<const Operand *>(my_w + 2 * kOp * un); };
+        auto rd_sv = [&](int un) {
 #pragma unroll
-            for (int q4 = 0; q4 < 4; q4++) sv[sb & 1][q4] = *reinterpret_cast<const float4 *>(my_sv + sb * kFastRowLine + 8 * q4);
+            for (int q4 = 0; q4 < 4; q4++) sv[un & 1][q4] = *reinterpret_cast<const float4 *>(my_sv + un * kFastRowLine + 8 * q4);
         };
-        auto rd_b = [&](int u) { // unit u's column operand and column scale
-            const int sb = kTwo ? u >> 1 : u, t = kTwo ? u & 1 : 0;
-            b[u & 1] = *reinterpret_cast<const v4i *>(my_a + 32 * t * kFastCodeStride + 32 * sb);
-            d8[u % 3] = d8_t[sb * kFastColLine + 32 * t + l32];
+        auto rd_b = [&](int u) { // step u's column operand and column scale
+            const int un = kTwo ? u >> 1 : u, t = kTwo ? u & 1 : 0;
+            b[u & 1] = *reinterpret_cast<const Operand *>(my_a + 32 * t * kStride + 2 * kOp * un);
+            d8[u % 3] = d8_t[(kQ45 ? un : un >> 1) * kFastColLine + 32 * t + l32];
         };
         auto product = [&](int u) {
-            const int sb = kTwo ? u >> 1 : u;
+            const int un = kTwo ? u >> 1 : u;
             const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            sum[u & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[sb & 1], b[u & 1], z, 0, 0, 0);
+            if constexpr (kQ45) sum[u & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[un & 1], b[u & 1], z, 0, 0, 0);
+            else sum[u & 1] = __builtin_amdgcn_mfma_i32_32x32x16_i8(a[un & 1], b[u & 1], z, 0, 0, 0);
         };
         rd_a(0);
         rd_b(0);
@@ -766,20 +634,20 @@ __global__ __launch_bounds__(256, 2) void k_gemm_q4k_fast(const uint8_t *w, int 
         if (!kTwo) rd_a(1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int u = 0; u < kUnits; u++) {
-            const int sb = kTwo ? u >> 1 : u, t = kTwo ? u & 1 : 0;
-            if (u + 1 < kUnits) product(u + 1);
-            if (u + 2 < kUnits) rd_b(u + 2);
-            // the row side of the block after: its codes before its first product is issued (the next unit), its scales
+        for (int u = 0; u < kSteps; u++) {
+            const int un = kTwo ? u >> 1 : u, t = kTwo ? u & 1 : 0;
+            if (u + 1 < kSteps) product(u + 1);
+            if (u + 2 < kSteps) rd_b(u + 2);
+            // the row side of the unit after: its codes before its first product is issued (the next step), its scales
             // before its first scaling
-            if (kTwo && t == 0 && sb + 1 < 8) rd_a(sb + 1);
-            if (!kTwo && sb + 2 < 8) rd_a(sb + 2);
-            if ((!kTwo || t == 1) && sb + 1 < 8) rd_sv(sb + 1);
+            if (kTwo && t == 0 && un + 1 < kUnitsSb) rd_a(un + 1);
+            if (!kTwo && un + 2 < kUnitsSb) rd_a(un + 2);
+            if ((!kTwo || t == 1) && un + 1 < kUnitsSb) rd_sv(un + 1);
             __builtin_amdgcn_sched_barrier(0);
             const float dc = d8[u % 3];
 #pragma unroll
             for (int q4 = 0; q4 < 4; q4++) {
-                const float4 r = sv[sb & 1][q4];
+                const float4 r = sv[un & 1][q4];
                 acc[t][4 * q4 + 0] = fmaf(r.x * dc, (float)sum[u & 1][4 * q4 + 0], acc[t][4 * q4 + 0]);
                 acc[t][4 * q4 + 1] = fmaf(r.y * dc, (float)sum[u & 1][4 * q4 + 1], acc[t][4 * q4 + 1]);
                 acc[t][4 * q4 + 2] = fmaf(r.z * dc, (float)sum[u & 1][4 * q4 + 2], acc[t][4 * q4 + 2]);
@@ -787,13 +655,16 @@ __global__ __launch_bounds__(256, 2) void k_gemm_q4k_fast(const uint8_t *w, int 
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        // the min terms last, into the same accumulators: a 32 x 8 by 8 x 32 product in f32, two of the eight sub-blocks an
-        // instruction; they run on the matrix cores while the workgroup goes through its barrier and the next staging
+        if constexpr (kQ45) {
+            // the min terms last, into the same accumulators: a 32 x 8 by 8 x 32 product in f32, two of the eight
+            // sub-blocks an instruction; they run on the matrix cores while the workgroup goes through its barrier and the
+            // next staging
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const float mn = mn_t[(2 * j + kh) * kFastRowLine + 32 * wv + l32];
-            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(mn, my_t[(2 * j + kh) * kFastColLine + l32], acc[0], 0, 0, 0);
-            if (kTwo) acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(mn, my_t[(2 * j + kh) * kFastColLine + 32 + l32], acc[1], 0, 0, 0);
+            for (int j = 0; j < 4; j++) {
+                const float mn = mn_t[(2 * j + kh) * kFastRowLine + 32 * wv + l32];
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(mn, my_t[(2 * j + kh) * kFastColLine + l32], acc[0], 0, 0, 0);
+                if (kTwo) acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(mn, my_t[(2 * j + kh) * kFastColLine + 32 + l32], acc[1], 0, 0, 0);
+            }
         }
     };
 
@@ -813,15 +684,10 @@ __global__ __launch_bounds__(256, 2) void k_gemm_q4k_fast(const uint8_t *w, int 
             float *out = y + (size_t)tab->slot[n] * rpe + row0 + 32 * wv + 4 * kh;
 #pragma unroll
             for (int q4 = 0; q4 < 4; q4++) {
-                const int r = row0 + 32 * wv + 4 * kh + 8 * q4;
-                const float4 v4 = make_float4(acc[t][4 * q4 + 0], acc[t][4 * q4 + 1], acc[t][4 * q4 + 2], acc[t][4 * q4 + 3]);
-                if (r + 3 < rpe) {
-                    *reinterpret_cast<float4 *>(out + 8 * q4) = v4; // rows_per_expert is a multiple of 16: 16-byte aligned
-                } else {
-                    if (r + 0 < rpe) out[8 * q4 + 0] = v4.x;
-                    if (r + 1 < rpe) out[8 * q4 + 1] = v4.y;
-                    if (r + 2 < rpe) out[8 * q4 + 2] = v4.z;
-                }
+                // rows_per_expert is a multiple of 16 and these four rows start at a multiple of 4: all inside or all outside
+                if (row0 + 32 * wv + 4 * kh + 8 * q4 < rpe)
+                    *reinterpret_cast<float4 *>(out + 8 * q4) =
+                        make_float4(acc[t][4 * q4 + 0], acc[t][4 * q4 + 1], acc[t][4 * q4 + 2], acc[t][4 * q4 + 3]);
             }
         }
     }
@@ -845,17 +711,19 @@ hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int
                            n_units, (u32)slot_div, (u32)n_slots, y);
         return hipGetLastError();
     };
-    if (mode == 1) { // Q5_K has no kernel of this kind and takes the exact one
-        if (wtype == BM_Q4K) {
-            hipError_t e = allow_lds(k_gemm_q4k_fast, kFastLds);
+    if (mode == 1) {
+        auto launch_fast = [&](auto kern, size_t lds) {
+            hipError_t e = allow_lds(kern, lds);
             if (e != hipSuccess) return e;
             const u32 n_slabs_f = (u32)((rows_per_expert + kFastRows - 1) / kFastRows);
             const unsigned grid = ((max_tiles + 7) / 8) * 8 * n_slabs_f;
-            hipLaunchKernelGGL(k_gemm_q4k_fast, dim3(grid), dim3(256), kFastLds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev,
-                               n_tiles, n_slabs_f, (u32)slot_div, (u32)n_slots, y);
+            hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev, n_tiles,
+                               n_slabs_f, (u32)slot_div, (u32)n_slots, y);
             return hipGetLastError();
-        }
-        if (wtype == BM_Q6K) return launch(k_gemm_fast<BM_Q6K>, 256, gemm_lds_bytes<BM_Q6K>(), 1);
+        };
+        if (wtype == BM_Q4K) return launch_fast(k_gemm_fast<BM_Q4K>, fast_lds_bytes<BM_Q4K>());
+        if (wtype == BM_Q5K) return launch_fast(k_gemm_fast<BM_Q5K>, fast_lds_bytes<BM_Q5K>());
+        if (wtype == BM_Q6K) return launch_fast(k_gemm_fast<BM_Q6K>, fast_lds_bytes<BM_Q6K>());
     }
     // 512 threads on 32 slots of a tile for both types (Q4_K 114 registers, Q6_K 121): two workgroups a CU. Measured
     // against 1024 threads on all 64 slots (Q4_K gate 362 -> 342 us), 512 threads with two slot groups a wave on 64

@@ -69,7 +69,7 @@ def test_gemm_fast_mode_is_within_the_tolerance(gpu):
     from common import max_abs_normalised
     rng = np.random.default_rng(2200)
     worst = 0.0
-    for wtype, k, rpe in ((bm.Q4_K, 2048, 768), (bm.Q6_K, 768, 2048)):
+    for wtype, k, rpe in ((bm.Q4_K, 2048, 768), (bm.Q6_K, 768, 2048), (bm.Q5_K, 1024, 80)):
         n_experts, n_slots = 6, 150
         w = stack(wtype, n_experts * rpe, k, 2201)
         ids = rng.integers(0, n_experts, n_slots).astype(np.uint32)

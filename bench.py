@@ -89,6 +89,18 @@ def make_tokens(ora, n_tokens, seed):
     return x, ids, wts
 
 
+def load_probe():
+    """The calibration launches: a library of their own beside the product's, built by the same Makefile."""
+    import ctypes as C
+    path = os.path.join(ROOT, "bloomery_amd", "libbm_bench_probe.so")
+    if not os.path.exists(path):
+        sys.exit(f"bench.py: {path} is not built (make -C bloomery_amd/csrc)")
+    lib = C.CDLL(path)
+    lib.bm_bench_probe_read.restype = C.c_int
+    lib.bm_bench_probe_read.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
+    return lib
+
+
 def timed_graph(gpu, enqueue, unit, steps, warmup):
     """Capture `unit` steps into one graph, replay it for about `steps` timed steps; ms per step by wall clock
     (bracketed by synchronisation) and by events on the launch stream."""
@@ -580,9 +592,8 @@ def main():
     ap.add_argument("--types", default="q4_k,q6_k",
                     help="config 2 only: gate/up and down weight types (q3_k, q4_k, q5_k, q6_k, iq2_xxs, iq3_xxs, iq4_xs); other than the default is "
                          "a side measurement of that type, not the headline workload")
-    ap.add_argument("--mode", choices=("two", "single", "chain"), default="two",
-                    help="two: bm_moe_decode in two launches (quantizers folded in); single: bm_moe_decode in one "
-                         "launch; chain: quantize, gate_up, down_combine")
+    ap.add_argument("--mode", choices=("two", "chain"), default="two",
+                    help="two: bm_moe_decode, two launches with the quantizers folded in; chain: quantize, gate_up, down_combine")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus above 1 is not supported (nothing here shards)")
@@ -602,8 +613,6 @@ def main():
     label = {v: k.upper() for k, v in names.items()}
     gate_n, down_n = label[gate_t], label[down_t]
     q8k = (bm.Q3_K, bm.IQ2_XXS, bm.IQ3_XXS, bm.IQ4_XS)
-    if args.mode == "single" and (gate_t, down_t) != (bm.Q4_K, bm.Q6_K):
-        sys.exit("bench.py: --mode single takes the default types")
     types3 = (gate_t, gate_t, down_t)
     t0 = time.time()
     wg, wu, wd = make_layer(ora, 0xB1000001, threads, gate_t, down_t)
@@ -625,10 +634,8 @@ def main():
     fold_h = down_t not in q8k  # gate . up writes the down activation itself when that is a Q8_2_X4 column
     h = None if fold_h else gpu.buffer(np.float32, TOP_K * FF)  # else f32 rows, quantized by the down launch
 
-    single = args.mode == "single"
-    kernels = {"single": ("step",), "two": ("gate_up_x", "down"),
+    kernels = {"two": ("gate_up_x", "down"),
                "chain": ("quant", "gate_up", "down") if fold_h else ("quant", "gate_up", "quant_h", "down")}[args.mode]
-    gpu.set_decode_plan(bm.PLAN_ONE_LAUNCH if single else bm.PLAN_TWO_LAUNCHES)
 
     def enqueue_step(i, which=kernels):
         t = i % n_tok
@@ -644,9 +651,6 @@ def main():
             gpu.enqueue_down_combine_h(dd, h, act_h, sel.ptr + 4 * t * TOP_K, wt.ptr + 4 * t * TOP_K, None, TOP_K, 1, HIDDEN,
                                        y.ptr + 4 * t * HIDDEN)
             return
-        if "step" in which:
-            gpu.enqueue_moe_decode(dg, du, dd, xd.ptr + 4 * t * HIDDEN, sel.ptr + 4 * t * TOP_K, wt.ptr + 4 * t * TOP_K,
-                                   None, TOP_K, 1, act_h, y.ptr + 4 * t * HIDDEN)
         if "quant" in which:
             gpu.enqueue_quantize(xd.ptr + 4 * t * HIDDEN, 1, act)
         if "gate_up" in which:
@@ -763,6 +767,8 @@ def main():
     # what the launches' times are to be read against, measured here: an empty launch, and launches that only fetch the
     # gate . up launch's bytes (cold: a different part of a different layer copy each time) with plain loads
     sink = gpu.buffer(np.uint32, 4096)
+    probe = load_probe()
+    stream = gpu.lib.bm_ctx_stream(gpu.ctx)
     stack_bytes = N_EXPERTS * FF * bm.row_bytes(gate_t, HIDDEN)
     spans = max(1, stack_bytes // gate_up_bytes)
 
@@ -772,13 +778,14 @@ def main():
         def enqueue(i):
             j = i % (len(layers) * 2 * spans)
             base = layers[j % len(layers)][(j // len(layers)) % 2].dev_ptr
-            gpu.enqueue_probe_read(base + (j // (2 * len(layers))) * gate_up_bytes, nbytes, n_wg, sink)
+            rc = probe.bm_bench_probe_read(stream, base + (j // (2 * len(layers))) * gate_up_bytes, nbytes, n_wg, sink.ptr)
+            assert rc == 0, f"bm_bench_probe_read: {rc}"
         return min(timed_graph(gpu, enqueue, 64, 1024, 64)[1] * 1e3 for _ in range(2))
 
     calibration = {"empty_launch_us": plain_read(192, 0),
                    "plain_read_of_gate_up_bytes_us": {str(n): plain_read(n, gate_up_bytes) for n in (192, 1024, 2048)},
                    "plain_read_of_half_us": {str(n): plain_read(n, gate_up_bytes // 2) for n in (2048,)},
-                   "note": "bm_probe_read under the same graph replay, cold: n workgroups fetch the gate . up launch's "
+                   "note": "a plain read kernel (bloomery_amd/csrc/bench_probe.hip) under the same graph replay, cold: n workgroups fetch the gate . up launch's "
                            f"{gate_up_bytes} bytes (or half of them) with plain loads and do nothing else: no expert ids to read "
                            "first, no arithmetic, no output"}
     best = min(calibration["plain_read_of_gate_up_bytes_us"].values())
@@ -787,15 +794,10 @@ def main():
     full = calibration["plain_read_of_gate_up_bytes_us"]["2048"]
     if full > half:
         calibration["streaming_gbps_between_half_and_whole"] = (gate_up_bytes - gate_up_bytes // 2) / ((full - half) * 1e-6) / 1e9
-    if single:
-        dominant, dom_bytes = "k_moe_decode<Q4_K, Q6_K>", bytes_per_token
-        achieved = dom_bytes / (kernel_us["step"] * 1e-6) / 1e9
-        kernel_gbps = {"step": achieved}
-    else:
-        gk = "gate_up_x" if args.mode == "two" else "gate_up"
-        dominant, dom_bytes = (f"k_gate_up_x<{gate_n}>" if args.mode == "two" else f"k_gate_up<{gate_n}>"), gate_up_bytes
-        achieved = dom_bytes / (kernel_us[gk] * 1e-6) / 1e9
-        kernel_gbps = {gk: achieved, "down": down_bytes / (kernel_us["down"] * 1e-6) / 1e9}
+    gk = "gate_up_x" if args.mode == "two" else "gate_up"
+    dominant, dom_bytes = (f"k_gate_up_x<{gate_n}>" if args.mode == "two" else f"k_gate_up<{gate_n}>"), gate_up_bytes
+    achieved = dom_bytes / (kernel_us[gk] * 1e-6) / 1e9
+    kernel_gbps = {gk: achieved, "down": down_bytes / (kernel_us["down"] * 1e-6) / 1e9}
     assert gpu.fault() == (bm.FAULT_NONE, 0)
 
     cpu = None

@@ -19,10 +19,9 @@ LIB_PATH = os.path.join(HERE, "libbm_moe_hip.so")
 Q3_K, Q4_K, Q5_K, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_XS = 11, 12, 13, 14, 16, 18, 23
 FAULT_NONE = 0xFFFFFFFF
 LAYER_NONE = 0xFFFF
-SITE_QUANT_COLUMN, SITE_ROUTER, SITE_EXPERT_ID, SITE_STALLED = 1, 5, 7, 31
-PLAN_ONE_LAUNCH, PLAN_TWO_LAUNCHES = 1, 2
+SITE_QUANT_COLUMN, SITE_ROUTER, SITE_EXPERT_ID = 1, 5, 7
 GEMM_EXACT, GEMM_FAST = 0, 1
-ACT_SILU_MUL, ACT_SWIGLU_CLAMP, ACT_SWIGLU_OAI, ACT_SWIGLU_GCLAMP = 0, 1, 2, 4
+ACT_SILU_MUL, ACT_SWIGLU_CLAMP, ACT_SWIGLU_OAI, ACT_SITU, ACT_SWIGLU_GCLAMP = 0, 1, 2, 3, 4
 SITE_F32_PRODUCT = 21
 HOST_SLOT = 0xFFFFFFFF
 
@@ -59,31 +58,28 @@ SYMBOLS = {
     "bm_act_upload": (_i, [_vp, _vp, _i, _vp]),
     "bm_quantize": (_i, [_vp, _vp, _i, _vp]),
     "bm_gemv": (_i, [_vp, _vp, _vp, _i, _vp]),
-    "bm_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
-    "bm_probe_read": (_i, [_vp, _vp, C.c_size_t, _i, _vp]),
+    "bm_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
     "bm_tables": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp]),
     "bm_gemv_x": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
     "bm_gemv_sel": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "bm_combine_tokens": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_down_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_down_combine_h": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
-    "bm_moe_decode": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp]),
-    "bm_moe_decode_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
-    "bm_set_spin_limit": (_i, [_vp, _u32]),
-    "bm_set_decode_plan": (_i, [_vp, _i]),
-    "bm_gate_up_x": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
+    "bm_moe_decode": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
+    "bm_moe_decode_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
+    "bm_gate_up_x": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "bm_tile_cap": (_i, [_i, _i]),
     "bm_buckets": (_i, [_vp, _vp, _i, _i, _vp, _vp]),
     "bm_tiles": (_i, [_vp, _vp, _i, _i, _vp]),
     "bm_quantize_ord": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
-    "bm_gate_up_tiles": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
+    "bm_gate_up_tiles": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
     "bm_gemv_tiles": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
     "bm_route_create": (_i, [_vp, _i, _i, C.POINTER(_vp)]),
     "bm_route_destroy": (None, [_vp]),
     "bm_route_fill": (_i, [_vp, _vp, _i, _vp]),
     "bm_route_read": (_i, [_vp, _vp, _vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
     "bm_gemm": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp]),
-    "bm_swiglu_quant": (_i, [_vp, _vp, _vp, _i, _vp]),
+    "bm_swiglu_quant": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
     "bm_moe_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_set_gate_rule": (_i, [_vp, _i, C.c_float]),
     "bm_route_softmax": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
@@ -356,6 +352,19 @@ def _ptr(x):
     return x  # a raw device address (e.g. torch.Tensor.data_ptr())
 
 
+class GateAct(C.Structure):
+    """bm_gate_act: a gate . up launch's own rule and its limit (SiTU: the gate's beta)."""
+    _fields_ = [("rule", C.c_int), ("limit", C.c_float)]
+
+
+def _rule(rule):
+    """None (the context's rule) or (ACT_*, limit) as the bm_gate_act a launch takes."""
+    if rule is None:
+        return None
+    code, limit = rule
+    return C.cast(C.pointer(GateAct(int(code), float(limit))), C.c_void_p)
+
+
 class Gpu:
     """A device context: stream, fault word and the launchers (the reference's `Gpu` and its kernel structs)."""
 
@@ -452,9 +461,10 @@ class Gpu:
     def enqueue_gemv(self, w, act, m, y):
         self._check(self.lib.bm_gemv(self.ctx, w.handle, act.handle, m, _ptr(y)))
 
-    def enqueue_gate_up(self, wg, wu, act, sel, n_slots, rows_per_expert, slots_per_col, h, act_h=None):
+    def enqueue_gate_up(self, wg, wu, act, sel, n_slots, rows_per_expert, slots_per_col, h, act_h=None, rule=None):
+        """rule: (ACT_*, limit) for this launch (GateUpArgs' act), None for the context's."""
         self._check(self.lib.bm_gate_up(self.ctx, wg.handle, wu.handle, act.handle, _ptr(sel), n_slots, rows_per_expert,
-                                        slots_per_col, _ptr(h), act_h.handle if act_h is not None else None))
+                                        slots_per_col, _rule(rule), _ptr(h), act_h.handle if act_h is not None else None))
 
     def enqueue_gemv_sel(self, w, act, sel, n_slots, rows_per_expert, y):
         self._check(self.lib.bm_gemv_sel(self.ctx, w.handle, act.handle, _ptr(sel), n_slots, rows_per_expert, _ptr(y)))
@@ -477,21 +487,21 @@ class Gpu:
                                                _ptr(sel), _ptr(wts), _ptr(resid), n_slots_per_token, m, rows_per_expert,
                                                _ptr(y)))
 
-    def enqueue_moe_decode(self, wg, wu, wd, x, sel, wts, resid, n_slots_per_token, m, act_h, y, act_x=None, h=None):
-        """The whole layer step with the quantizers folded in (bm_moe_decode): two launches, or one under
-        PLAN_ONE_LAUNCH. A down stack on Q8_K columns needs h (f32 scratch of m * n_slots_per_token * ff values)."""
+    def enqueue_moe_decode(self, wg, wu, wd, x, sel, wts, resid, n_slots_per_token, m, act_h, y, act_x=None, h=None, rule=None):
+        """The whole layer step with the quantizers folded in (bm_moe_decode), two launches. A down stack on Q8_K
+        columns needs h (f32 scratch of m * n_slots_per_token * ff values)."""
         self._check(self.lib.bm_moe_decode(self.ctx, wg.handle, wu.handle, wd.handle, _ptr(x), _ptr(sel), _ptr(wts),
-                                           _ptr(resid), n_slots_per_token, m, act_h.handle,
+                                           _ptr(resid), n_slots_per_token, m, _rule(rule), act_h.handle,
                                            act_x.handle if act_x is not None else None, _ptr(h), _ptr(y)))
 
-    def enqueue_moe_decode_noalloc(self, wg, wu, wd, x, sel, wts, resid, n_slots_per_token, m, y):
+    def enqueue_moe_decode_noalloc(self, wg, wu, wd, x, sel, wts, resid, n_slots_per_token, m, y, rule=None):
         """bm_moe_decode in two launches with the scratch between them held by the library: nothing is allocated."""
         self._check(self.lib.bm_moe_decode_noalloc(self.ctx, wg.handle, wu.handle, wd.handle, _ptr(x), _ptr(sel), _ptr(wts),
-                                                   _ptr(resid), n_slots_per_token, m, _ptr(y)))
+                                                   _ptr(resid), n_slots_per_token, m, _rule(rule), _ptr(y)))
 
-    def enqueue_gate_up_x(self, wg, wu, x, sel, n_slots_per_token, m, rows_per_expert, act_h, act_x=None, h=None):
+    def enqueue_gate_up_x(self, wg, wu, x, sel, n_slots_per_token, m, rows_per_expert, act_h, act_x=None, h=None, rule=None):
         self._check(self.lib.bm_gate_up_x(self.ctx, wg.handle, wu.handle, _ptr(x), _ptr(sel), n_slots_per_token, m,
-                                          rows_per_expert, act_h.handle if act_h is not None else None,
+                                          rows_per_expert, _rule(rule), act_h.handle if act_h is not None else None,
                                           act_x.handle if act_x is not None else None, _ptr(h)))
 
     def enqueue_gemv_x(self, w, x, m, y, act_out=None):
@@ -508,12 +518,6 @@ class Gpu:
     def enqueue_card_gemv_sel(self, w, codes, d8, s8, sel, n_slots, rows_per_expert, y):
         self._check(self.lib.bm_card_gemv_sel(self.ctx, w.handle, _ptr(codes), _ptr(d8), _ptr(s8), _ptr(sel), n_slots,
                                               rows_per_expert, _ptr(y)))
-
-    def set_decode_plan(self, plan):
-        self._check(self.lib.bm_set_decode_plan(self.ctx, plan))
-
-    def set_spin_limit(self, spins):
-        self._check(self.lib.bm_set_spin_limit(self.ctx, spins))
 
     # -- grouped decode: the slot table by expert and the tile launchers
     def tile_cap(self, n_slots, n_experts):
@@ -533,9 +537,9 @@ class Gpu:
         self._check(self.lib.bm_quantize_ord(self.ctx, _ptr(x), _ptr(start), n_experts, m_cols, act.handle))
 
     def enqueue_gate_up_tiles(self, wg, wu, act, order, start, tiles, n_slots, rows_per_expert, slots_per_col, h,
-                              act_h=None):
+                              act_h=None, rule=None):
         self._check(self.lib.bm_gate_up_tiles(self.ctx, wg.handle, wu.handle, act.handle, _ptr(order), _ptr(start),
-                                              _ptr(tiles), n_slots, rows_per_expert, slots_per_col, _ptr(h),
+                                              _ptr(tiles), n_slots, rows_per_expert, slots_per_col, _rule(rule), _ptr(h),
                                               act_h.handle if act_h is not None else None))
 
     def enqueue_gemv_tiles(self, w, act, order, start, tiles, n_slots, rows_per_expert, y):
@@ -551,14 +555,14 @@ class Gpu:
         self._check(self.lib.bm_gemm(self.ctx, w.handle, rows_per_expert, act.handle, route.handle, top_k, _ptr(y)))
 
     def set_gate_rule(self, rule, limit=0.0):
-        """The Act of the gate . up launches that follow (crates/gpu/src/kquant/act.rs:21-57)."""
+        """The Act of the gate . up launches that follow and pass no rule of their own (crates/gpu/src/kquant/act.rs:21-57)."""
         self._check(self.lib.bm_set_gate_rule(self.ctx, rule, float(limit)))
 
     def set_gemm_mode(self, mode):
         self._check(self.lib.bm_set_gemm_mode(self.ctx, mode))
 
-    def enqueue_swiglu_quant(self, g, u, n_cols, act):
-        self._check(self.lib.bm_swiglu_quant(self.ctx, _ptr(g), _ptr(u), n_cols, act.handle))
+    def enqueue_swiglu_quant(self, g, u, n_cols, act, rule=None):
+        self._check(self.lib.bm_swiglu_quant(self.ctx, _ptr(g), _ptr(u), n_cols, _rule(rule), act.handle))
 
     def enqueue_route_softmax(self, logits, n_tokens, n_experts, top_k, renorm, probs, ids, weights):
         """RouterKernels::enqueue_route (crates/gpu/src/route_softmax.rs:1643): softmax, top-k, renormalised weights."""
@@ -571,10 +575,6 @@ class Gpu:
         self._check(self.lib.bm_router_logits(self.ctx, _ptr(router), _ptr(x), _ptr(gain) if gain is not None else None,
                                               float(eps), n_tokens, n_experts, hidden,
                                               _ptr(normed) if normed is not None else None, _ptr(logits)))
-
-    def enqueue_probe_read(self, src, nbytes, n_workgroups, sink):
-        """Measurement only: a launch that fetches nbytes with plain loads (0: an empty launch)."""
-        self._check(self.lib.bm_probe_read(self.ctx, _ptr(src), nbytes, n_workgroups, _ptr(sink)))
 
     def enqueue_block_sums(self, w, row, act, col, out):
         self._check(self.lib.bm_block_sums(self.ctx, w.handle, row, act.handle, col, _ptr(out)))

@@ -19,11 +19,8 @@ struct bm_ctx {
     bool own_stream = false;
     uint32_t *fault = nullptr;
     uint32_t layer = BM_LAYER_NONE;
-    uint32_t *counters = nullptr; // bm_moe_decode's producer/consumer counts, zero between launches
-    int decode_plan = BM_PLAN_TWO_LAUNCHES;
     int gemm_mode = BM_GEMM_EXACT;
     bmk::GateRule rule = {0u, 0.0f}; // silu(g) * u
-    uint32_t spin_limit = 1u << 18; // a poll is a round trip to memory: some tenths of a second of waiting
     std::string err;
 };
 
@@ -115,15 +112,9 @@ static int ctx_make(int device, hipStream_t stream, bool own, bm_ctx **out) {
         e = hipMemset(c->fault, 0, sizeof(uint32_t) * BM_FAULT_WORDS);
         if (e == hipSuccess) e = hipMemset(c->fault, 0xff, sizeof(uint32_t));
     }
-    if (e == hipSuccess) {
-        const size_t cb = sizeof(uint32_t) * (bmk::kMaxDecodeTokens + 1);
-        e = hipMalloc((void **)&c->counters, cb);
-        if (e == hipSuccess) e = hipMemset(c->counters, 0, cb);
-    }
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
         if (c->fault) (void)hipFree(c->fault);
-        if (c->counters) (void)hipFree(c->counters);
         if (c->own_stream) (void)hipStreamDestroy(c->stream);
         delete c;
         return fail(nullptr, BM_EDRIVER, "bm_ctx_create: fault word: %s", hipGetErrorString(e));
@@ -143,7 +134,6 @@ void bm_ctx_destroy(bm_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(ctx->fault);
-    (void)hipFree(ctx->counters);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -175,14 +165,18 @@ int bm_fault_read(bm_ctx *ctx, uint32_t layer, uint32_t *word0, uint32_t *mask) 
 }
 
 static bmk::Launch launch_of(bm_ctx *ctx) { return bmk::Launch{ctx->stream, ctx->fault, ctx->layer, ctx->rule}; }
+static int rule_checked(bm_ctx *ctx, const char *what, int rule, float limit, bmk::GateRule *out);
+// The launch state of a gate . up entry: the entry's own rule when the caller passes one, else the context's.
+static int launch_under(bm_ctx *ctx, const char *what, const bm_gate_act *act, bmk::Launch *L) {
+    *L = launch_of(ctx);
+    return act ? rule_checked(ctx, what, act->rule, act->limit, &L->rule) : BM_OK;
+}
 
 int bm_fault_clear(bm_ctx *ctx) {
     if (!ctx) return fail(nullptr, BM_EARG, "bm_fault_clear: ctx is NULL");
     bmk::Launch L = launch_of(ctx);
     hipError_t e = bmk::fill_u32(L, ctx->fault + 1, 0u, BM_FAULT_WORDS - 1);
     if (e == hipSuccess) e = bmk::fill_u32(L, ctx->fault, BM_FAULT_NONE, 1);
-    // a launch that gave up waiting may have left its counts behind
-    if (e == hipSuccess) e = bmk::fill_u32(L, ctx->counters, 0u, bmk::kMaxDecodeTokens + 1);
     return driver(ctx, "bm_fault_clear", e);
 }
 
@@ -388,7 +382,7 @@ static int check_stack(bm_ctx *ctx, const char *what, const bm_weights *w, int r
 }
 
 int bm_gate_up(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_act *act, const uint32_t *sel_dev,
-               int n_slots, int rows_per_expert, int slots_per_col, float *h_dev, bm_act *act_h) {
+               int n_slots, int rows_per_expert, int slots_per_col, const bm_gate_act *rule, float *h_dev, bm_act *act_h) {
     const char *what = "bm_gate_up";
     if (!ctx || !wg || !wu || !act || !sel_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
     if (!h_dev && !act_h) return fail(ctx, BM_EARG, "%s: neither h_dev nor act_h to write", what);
@@ -416,7 +410,9 @@ int bm_gate_up(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm
             return fail(ctx, BM_ESHAPE, "%s: a column of act_h per slot: %d slots, act_h holds %d", what, n_slots, act_h->m_cap);
         ah = act_h->dev;
     }
-    return driver(ctx, what, bmk::gate_up(launch_of(ctx), wg->wtype, wg->dev, wu->dev, n_experts, wg->k, act->dev, sel_dev,
+    bmk::Launch L;
+    if ((rc = launch_under(ctx, what, rule, &L)) != 0) return rc;
+    return driver(ctx, what, bmk::gate_up(L, wg->wtype, wg->dev, wu->dev, n_experts, wg->k, act->dev, sel_dev,
                                           n_slots, rows_per_expert, slots_per_col, h_dev, ah));
 }
 
@@ -501,14 +497,9 @@ int bm_down_combine_h(bm_ctx *ctx, const bm_weights *w, const float *h_dev, bm_a
                                                   sel_dev, w_dev, resid_dev, n_slots_per_token, m, rows_per_expert, y_dev));
 }
 
-int bm_set_spin_limit(bm_ctx *ctx, uint32_t spins) {
-    if (!ctx) return fail(nullptr, BM_EARG, "bm_set_spin_limit: ctx is NULL");
-    ctx->spin_limit = spins;
-    return BM_OK;
-}
-
 int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const float *x_dev, const uint32_t *sel_dev,
-                 int n_slots_per_token, int m, int rows_per_expert, bm_act *act_h, bm_act *act_x, float *h_dev) {
+                 int n_slots_per_token, int m, int rows_per_expert, const bm_gate_act *rule, bm_act *act_h, bm_act *act_x,
+                 float *h_dev) {
     const char *what = "bm_gate_up_x";
     if (!ctx || !wg || !wu || !x_dev || !sel_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
     if (!act_h && !h_dev) return fail(ctx, BM_EARG, "%s: neither act_h nor h_dev: the launch would have no output", what);
@@ -534,32 +525,23 @@ int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const 
     if (((uintptr_t)x_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: x_dev %p is not 16-byte aligned", what, (const void *)x_dev);
     if (dev_col_bytes(wg->wtype, hidden) + 8192 > (size_t)bmk::kMaxLds)
         return fail(ctx, BM_ESHAPE, "%s: a column of hidden = %d does not fit the workgroup's LDS", what, hidden);
+    bmk::Launch L;
+    if ((rc = launch_under(ctx, what, rule, &L)) != 0) return rc;
     return driver(ctx, what,
-                  bmk::gate_up_x(launch_of(ctx), wg->wtype, x_dev, wg->dev, wu->dev, n_experts, hidden, ff, sel_dev, n_slots_per_token, m,
+                  bmk::gate_up_x(L, wg->wtype, x_dev, wg->dev, wu->dev, n_experts, hidden, ff, sel_dev, n_slots_per_token, m,
                                  act_x ? act_x->dev : nullptr, act_h ? act_h->dev : nullptr, h_dev));
-}
-
-int bm_set_decode_plan(bm_ctx *ctx, int plan) {
-    if (!ctx) return fail(nullptr, BM_EARG, "bm_set_decode_plan: ctx is NULL");
-    if (plan != BM_PLAN_ONE_LAUNCH && plan != BM_PLAN_TWO_LAUNCHES)
-        return fail(ctx, BM_EARG, "bm_set_decode_plan: plan %d is neither BM_PLAN_ONE_LAUNCH nor BM_PLAN_TWO_LAUNCHES", plan);
-    ctx->decode_plan = plan;
-    return BM_OK;
 }
 
 int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_weights *wd, const float *x_dev,
                   const uint32_t *sel_dev, const float *w_dev, const float *resid_dev, int n_slots_per_token, int m,
-                  bm_act *act_h, bm_act *act_x, float *h_dev, float *y_dev) {
+                  const bm_gate_act *rule, bm_act *act_h, bm_act *act_x, float *h_dev, float *y_dev) {
     const char *what = "bm_moe_decode";
     if (!ctx || !wg || !wu || !wd || !x_dev || !sel_dev || !w_dev || !act_h || !y_dev)
         return fail(ctx, BM_EARG, "%s: NULL argument", what);
     if (wg->wtype != wu->wtype)
         return fail(ctx, BM_ETYPE, "%s: gate is type %d and up type %d; one launch reads one type", what, wg->wtype, wu->wtype);
-    if (!bmk::moe_decode_supported(ctx->decode_plan, wg->wtype, wd->wtype))
-        return fail(ctx, BM_ETYPE,
-                    "%s: as one launch the fused step takes Q4_K gate/up with Q6_K or Q4_K down (as two: every type), got %d and %d; "
-                    "use BM_PLAN_TWO_LAUNCHES or the separate launches",
-                    what, wg->wtype, wd->wtype);
+    if (!bmk::moe_decode_supported(wg->wtype, wd->wtype))
+        return fail(ctx, BM_ETYPE, "%s: no kernel for gate/up type %d with down type %d", what, wg->wtype, wd->wtype);
     if (wu->k != wg->k || wu->rows != wg->rows)
         return fail(ctx, BM_ESHAPE, "%s: gate is %lld x %d, up %lld x %d", what, (long long)wg->rows, wg->k, (long long)wu->rows, wu->k);
     const int hidden = wg->k, ff = wd->k;
@@ -589,20 +571,21 @@ int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const
     if (lds_a > (size_t)bmk::kMaxLds || lds_b > (size_t)bmk::kMaxLds)
         return fail(ctx, BM_ESHAPE, "%s: hidden = %d or %d columns of ff = %d do not fit the workgroup's LDS; use the separate launches", what,
                     hidden, n_slots_per_token, ff);
+    bmk::Launch L;
+    if ((rc = launch_under(ctx, what, rule, &L)) != 0) return rc;
     return driver(ctx, what,
-                  bmk::moe_decode(launch_of(ctx), ctx->decode_plan, wg->wtype, wd->wtype, x_dev, wg->dev, wu->dev, wd->dev, n_experts, hidden, ff, sel_dev,
-                                  w_dev, resid_dev, n_slots_per_token, m, act_x ? act_x->dev : nullptr, act_h->dev, h_dev, y_dev,
-                                  ctx->counters, ctx->spin_limit));
+                  bmk::moe_decode(L, wg->wtype, wd->wtype, x_dev, wg->dev, wu->dev, wd->dev, n_experts, hidden, ff, sel_dev,
+                                  w_dev, resid_dev, n_slots_per_token, m, act_x ? act_x->dev : nullptr, act_h->dev, h_dev, y_dev));
 }
 
 int bm_moe_decode_noalloc(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_weights *wd, const float *x_dev,
                           const uint32_t *sel_dev, const float *w_dev, const float *resid_dev, int n_slots_per_token, int m,
-                          float *y_dev) {
+                          const bm_gate_act *rule, float *y_dev) {
     const char *what = "bm_moe_decode_noalloc";
     if (!ctx || !wg || !wu || !wd || !x_dev || !sel_dev || !w_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
     if (wg->wtype != wu->wtype)
         return fail(ctx, BM_ETYPE, "%s: gate is type %d and up type %d; one launch reads one type", what, wg->wtype, wu->wtype);
-    if (!bmk::moe_decode_supported(bmk::kPlanTwoLaunches, wg->wtype, wd->wtype))
+    if (!bmk::moe_decode_supported(wg->wtype, wd->wtype))
         return fail(ctx, BM_ETYPE, "%s: no kernel for gate/up type %d with down type %d", what, wg->wtype, wd->wtype);
     if (wu->k != wg->k || wu->rows != wg->rows)
         return fail(ctx, BM_ESHAPE, "%s: gate is %lld x %d, up %lld x %d", what, (long long)wg->rows, wg->k, (long long)wu->rows, wu->k);
@@ -627,8 +610,10 @@ int bm_moe_decode_noalloc(bm_ctx *ctx, const bm_weights *wg, const bm_weights *w
     if (lds_a > (size_t)bmk::kMaxLds || lds_b > (size_t)bmk::kMaxLds)
         return fail(ctx, BM_ESHAPE, "%s: hidden = %d or %d columns of ff = %d do not fit the workgroup's LDS; use the separate launches", what,
                     hidden, n_slots_per_token, ff);
+    bmk::Launch L;
+    if ((rc = launch_under(ctx, what, rule, &L)) != 0) return rc;
     return driver(ctx, what,
-                  bmk::moe_decode_static(launch_of(ctx), ctx->device, wg->wtype, wd->wtype, x_dev, wg->dev, wu->dev, wd->dev, n_experts,
+                  bmk::moe_decode_static(L, ctx->device, wg->wtype, wd->wtype, x_dev, wg->dev, wu->dev, wd->dev, n_experts,
                                          hidden, ff, sel_dev, w_dev, resid_dev, n_slots_per_token, m, y_dev));
 }
 
@@ -689,7 +674,7 @@ static int check_table(bm_ctx *ctx, const char *what, const uint32_t *order, con
 
 int bm_gate_up_tiles(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_act *act, const uint32_t *order_dev,
                      const uint32_t *start_dev, const uint32_t *tiles_dev, int n_slots, int rows_per_expert,
-                     int slots_per_col, float *h_dev, bm_act *act_h) {
+                     int slots_per_col, const bm_gate_act *rule, float *h_dev, bm_act *act_h) {
     const char *what = "bm_gate_up_tiles";
     if (!ctx || !wg || !wu || !act) return fail(ctx, BM_EARG, "%s: NULL argument", what);
     if (!h_dev && !act_h) return fail(ctx, BM_EARG, "%s: neither h_dev nor act_h to write", what);
@@ -719,7 +704,9 @@ int bm_gate_up_tiles(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, co
     }
     if (bmk::tiles_lds(wg->wtype, wg->k) == 0)
         return fail(ctx, BM_ESHAPE, "%s: eight columns of k = %d do not fit the workgroup's LDS; use bm_gate_up", what, wg->k);
-    return driver(ctx, what, bmk::gate_up_tiles(launch_of(ctx), wg->wtype, wg->dev, wu->dev, n_experts, wg->k, act->dev, act->m_cap,
+    bmk::Launch L;
+    if ((rc = launch_under(ctx, what, rule, &L)) != 0) return rc;
+    return driver(ctx, what, bmk::gate_up_tiles(L, wg->wtype, wg->dev, wu->dev, n_experts, wg->k, act->dev, act->m_cap,
                                                 order_dev, start_dev, tiles_dev, n_slots, rows_per_expert, slots_per_col, h_dev, ah));
 }
 
@@ -842,10 +829,8 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
                                        route->tiles, route->n_tiles, n_slots, slot_div, y_dev, ctx->gemm_mode));
 }
 
-int bm_set_gate_rule(bm_ctx *ctx, int rule, float limit) {
-    const char *what = "bm_set_gate_rule";
-    if (!ctx) return fail(nullptr, BM_EARG, "%s: ctx is NULL", what);
-    // crates/gpu/src/kquant/act.rs:71-125 Act::code: what the device rules can run
+// crates/gpu/src/kquant/act.rs:71-125 Act::code: what the device rules can run, refused by name otherwise.
+static int rule_checked(bm_ctx *ctx, const char *what, int rule, float limit, bmk::GateRule *out) {
     switch (rule) {
     case BM_ACT_SILU_MUL:
         limit = 0.0f;
@@ -858,17 +843,27 @@ int bm_set_gate_rule(bm_ctx *ctx, int rule, float limit) {
             return fail(ctx, BM_ESHAPE, "%s: swigluoai runs at alpha 1.702 and a finite limit of at least 0, got limit %g", what,
                         (double)limit);
         break;
+    case BM_ACT_SITU:
+        if (!std::isfinite(limit) || !(limit > 0.0f))
+            return fail(ctx, BM_ESHAPE, "%s: situ runs at linear beta 25 and a finite positive beta, got beta %g", what, (double)limit);
+        break;
     case BM_ACT_SWIGLU_GCLAMP:
         if (!std::isfinite(limit) || !(limit > 0.0f))
             return fail(ctx, BM_ESHAPE, "%s: the gate-first clamp limit must be finite and positive, got %g; a caller that clamps "
                         "nothing runs BM_ACT_SWIGLU_CLAMP", what, (double)limit);
         break;
     default:
-        return fail(ctx, BM_ETYPE, "%s: rule %d is not one of BM_ACT_SILU_MUL, BM_ACT_SWIGLU_CLAMP, BM_ACT_SWIGLU_OAI, "
-                    "BM_ACT_SWIGLU_GCLAMP (SiTU-GLU, code 3, is not built)", what, rule);
+        return fail(ctx, BM_ETYPE, "%s: rule %d is not one of BM_ACT_SILU_MUL, BM_ACT_SWIGLU_CLAMP, BM_ACT_SWIGLU_OAI, BM_ACT_SITU, "
+                    "BM_ACT_SWIGLU_GCLAMP", what, rule);
     }
-    ctx->rule = bmk::GateRule{(uint32_t)rule, limit};
+    *out = bmk::GateRule{(uint32_t)rule, limit};
     return BM_OK;
+}
+
+int bm_set_gate_rule(bm_ctx *ctx, int rule, float limit) {
+    const char *what = "bm_set_gate_rule";
+    if (!ctx) return fail(nullptr, BM_EARG, "%s: ctx is NULL", what);
+    return rule_checked(ctx, what, rule, limit, &ctx->rule);
 }
 
 int bm_set_gemm_mode(bm_ctx *ctx, int mode) {
@@ -879,14 +874,16 @@ int bm_set_gemm_mode(bm_ctx *ctx, int mode) {
     return BM_OK;
 }
 
-int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, bm_act *act) {
+int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, const bm_gate_act *rule, bm_act *act) {
     const char *what = "bm_swiglu_quant";
     if (!ctx || !g_dev || !u_dev || !act) return fail(ctx, BM_EARG, "%s: NULL argument", what);
     if (act_form(act->wtype) != 0)
         return fail(ctx, BM_ETYPE, "%s: writes Q8_2_X4 columns; act was made for type %d (Q8_K)", what, act->wtype);
     if (n_cols < 1 || n_cols > act->m_cap)
         return fail(ctx, BM_ESHAPE, "%s: n_cols = %d columns, act holds %d", what, n_cols, act->m_cap);
-    return driver(ctx, what, bmk::swiglu_quant(launch_of(ctx), g_dev, u_dev, n_cols, act->k, act->dev));
+    bmk::Launch L;
+    if (int rc = launch_under(ctx, what, rule, &L)) return rc;
+    return driver(ctx, what, bmk::swiglu_quant(L, g_dev, u_dev, n_cols, act->k, act->dev));
 }
 
 int bm_weights_from_gguf(bm_ctx *ctx, const bm_gguf *g, const char *name, bm_weights **out, int *rows_per_expert, int *n_experts) {
@@ -954,14 +951,6 @@ int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *a
     const uint8_t *wrow = w->dev + (size_t)row * (size_t)bm_row_bytes(w->wtype, w->k);
     const uint8_t *c = act->dev + (size_t)col * dev_col_bytes(act->wtype, act->k);
     return driver(ctx, what, bmk::block_sums(launch_of(ctx), w->wtype, wrow, w->k, c, out_dev));
-}
-
-int bm_probe_read(bm_ctx *ctx, const void *src_dev, size_t bytes, int n_workgroups, uint32_t *sink_dev) {
-    const char *what = "bm_probe_read";
-    if (!ctx || !sink_dev || (!src_dev && bytes)) return fail(ctx, BM_EARG, "%s: NULL argument", what);
-    if (bytes % 16 != 0 || ((uintptr_t)src_dev & 15) != 0) return fail(ctx, BM_ESHAPE, "%s: %zu bytes at %p: both multiples of 16", what, bytes, src_dev);
-    if (n_workgroups < 1 || n_workgroups > 65536) return fail(ctx, BM_ESHAPE, "%s: %d workgroups (1 .. 65536)", what, n_workgroups);
-    return driver(ctx, what, bmk::probe_read(launch_of(ctx), src_dev, bytes, n_workgroups, sink_dev));
 }
 
 // ------------------------------------------------------------------------------------ the card rule

@@ -1100,7 +1100,18 @@ __device__ __forceinline__ float bm_swiglu_gclamp(float g, float u, float limit)
     return __fmul_rn(bm_silu(x), y);
 }
 
-// A row's value under rule `act` (crates/gpu/src/kquant/act.rs:136-149 apply). Under the clamped rules a sum that is
+// SiTU-GLU: (beta tanh(g / beta) * sigmoid(g)) * (25 tanh(u / 25)), each scale by the f32 reciprocal, the tanh, the
+// scale back, then the products (crates/gpu/src/kquant/act.rs:152-163 situ; crates/model/src/ops.rs:2345-2360 on the
+// host). The sigmoid is ik's; the tanh is the device library's f32 one, which can differ from the host libm's in the
+// last bits, as the reference's own card and host do.
+__device__ __forceinline__ float bm_situ(float g, float u, float beta) {
+    const float a = __fmul_rn(tanhf(__fmul_rn(g, __fdiv_rn(1.0f, beta))), beta);
+    const float s = __fdiv_rn(1.0f, __fadd_rn(1.0f, bm_expf_ik(__fsub_rn(0.0f, g))));
+    const float v = __fmul_rn(tanhf(__fmul_rn(u, __fdiv_rn(1.0f, 25.0f))), 25.0f);
+    return __fmul_rn(__fmul_rn(a, s), v);
+}
+
+// A row's value under rule `act` (crates/gpu/src/kquant/act.rs:136-149 apply). Under the clamped rules and SiTU a sum that is
 // not finite would come out finite: `odd` reports it and the value is NaN (:166-175 apply_checked; the CPU path's
 // rules return false for such a block). The plain rule lets it through as it is, as the CPU path's swiglu does.
 __device__ __forceinline__ float bm_gate_rule(u32 act, float limit, float g, float u, bool &odd) {
@@ -1112,6 +1123,7 @@ __device__ __forceinline__ float bm_gate_rule(u32 act, float limit, float g, flo
     }
     if (act == 1u) return bm_swiglu_clamp(g, u, limit);
     if (act == 2u) return bm_swiglu_oai(g, u, limit);
+    if (act == 3u) return bm_situ(g, u, limit);
     return bm_swiglu_gclamp(g, u, limit);
 }
 

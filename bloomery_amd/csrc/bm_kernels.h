@@ -9,12 +9,13 @@
 namespace bmk {
 
 // The rule a gate . up launch applies to a row's two sums (crates/gpu/src/kquant/act.rs:21-57 Act and its device
-// codes): silu(g) * u, ik's clamped SwiGLU, the gpt-oss / MiniMax SwiGLU at alpha 1.702, ggml's gate-first clamp.
+// codes): silu(g) * u, ik's clamped SwiGLU, the gpt-oss / MiniMax SwiGLU at alpha 1.702, SiTU-GLU at linear beta 25
+// (limit carries the gate's beta), ggml's gate-first clamp.
 struct GateRule {
     uint32_t act;
     float limit;
 };
-constexpr uint32_t kActSiluMul = 0, kActSwigluClamp = 1, kActSwigluOai = 2, kActSwigluGclamp = 4;
+constexpr uint32_t kActSiluMul = 0, kActSwigluClamp = 1, kActSwigluOai = 2, kActSitu = 3, kActSwigluGclamp = 4;
 
 struct Launch {
     hipStream_t stream;
@@ -27,8 +28,6 @@ struct Launch {
 constexpr int kMaxLds = 160 * 1024;
 
 hipError_t fill_u32(const Launch &L, uint32_t *dst, uint32_t value, size_t n);
-// Measurement only: n_wg workgroups read `bytes` with plain loads (bytes = 0: an empty launch); sink holds n_wg words.
-hipError_t probe_read(const Launch &L, const void *src, size_t bytes, int n_wg, uint32_t *sink);
 
 // Bytes of one activation column of k values on the device, in the form weight type `wtype` dots against: the CPU
 // path's bytes, and for the Q8_2_X4 form two tables after them (bm_device.cuh).
@@ -62,14 +61,11 @@ hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_expe
                         const uint32_t *sel, const float *wts, const float *resid, int slots_per_token, int m,
                         int rows_per_expert, float *y);
 
-// The whole decode step: quantize x, gate . up . SwiGLU, quantize h, down, weighted slot sum.
-//   kPlanOneLaunch:   one launch; the down workgroups stream their rows while gate . up runs and wait on device
-//                     counters (`counters`: m + 1 zeroed words, left zeroed; spin_limit bounds the wait);
-//   kPlanTwoLaunches: gate . up with the quantizers folded in, then down + combine (no counters).
-constexpr int kPlanOneLaunch = 1, kPlanTwoLaunches = 2;
+// The whole decode step: quantize x, gate . up . SwiGLU, quantize h, down, weighted slot sum, in two launches: gate . up
+// with the quantizers folded in, then down + combine.
 constexpr int kMaxDecodeTokens = 1024;
-bool moe_decode_supported(int plan, int gate_type, int down_type);
-// gate . up . SwiGLU from f32 token rows, the token quantizer folded in: the first launch of kPlanTwoLaunches. act_h
+bool moe_decode_supported(int gate_type, int down_type);
+// gate . up . SwiGLU from f32 token rows, the token quantizer folded in: the first launch of moe_decode. act_h
 // (Q8_2_X4 columns, or NULL when the down stack takes Q8_K ones) is quantized in the same launch; h (f32 rows) is
 // optional beside act_h and the output without it.
 hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8_t *wg, const uint8_t *wu,
@@ -78,10 +74,9 @@ hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8
 hipError_t down_combine_hq(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const float *h,
                            uint8_t *act_h, const uint32_t *sel, const float *wts, const float *resid,
                            int slots_per_token, int m, int rows_per_expert, float *y);
-hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, const float *x, const uint8_t *wg,
-                      const uint8_t *wu, const uint8_t *wd, int n_experts, int hidden, int ff, const uint32_t *sel,
-                      const float *wts, const float *resid, int slots_per_token, int m, uint8_t *act_x,
-                      uint8_t *act_h, float *h, float *y, uint32_t *counters, uint32_t spin_limit);
+hipError_t moe_decode(const Launch &L, int gate_type, int down_type, const float *x, const uint8_t *wg, const uint8_t *wu,
+                      const uint8_t *wd, int n_experts, int hidden, int ff, const uint32_t *sel, const float *wts,
+                      const float *resid, int slots_per_token, int m, uint8_t *act_x, uint8_t *act_h, float *h, float *y);
 
 // moe_decode's two launches with act_h and h in a file-scope device array instead of caller memory: no allocation
 // anywhere on the way. static_scratch_init(device), called with that device current (the context's creation does),

@@ -14,30 +14,6 @@ __global__ void k_fill_u32(u32 *dst, u32 value, size_t n) {
     if (i < n) dst[i] = value;
 }
 
-// Measurement only: n_wg workgroups read `bytes` (a multiple of 16) as plain 16-byte loads, workgroup b the b-th equal
-// share, four loads a thread in flight, and leave one word a workgroup in `sink`. With bytes = 0 it is an empty launch.
-// What a decode launch's time is to be read against: its bytes fetched by a kernel that does nothing else.
-__global__ __launch_bounds__(256) void k_probe_read(const uint4 *src, size_t n16, u32 *sink) {
-    const size_t per = (n16 + gridDim.x - 1) / gridDim.x;
-    const size_t lo = per * blockIdx.x, hi = lo + per < n16 ? lo + per : n16;
-    u32 acc = 0;
-    size_t i = lo + threadIdx.x;
-    for (; i + 768 < hi; i += 1024) {
-        const uint4 a = src[i], b = src[i + 256], c = src[i + 512], d = src[i + 768];
-        acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
-    }
-    for (; i < hi; i += 256) {
-        const uint4 a = src[i];
-        acc ^= a.x ^ a.y ^ a.z ^ a.w;
-    }
-    if (acc == 0x9e3779b9u && threadIdx.x == 0) sink[blockIdx.x] = acc; // the loads must happen; the store almost never does
-}
-
-hipError_t probe_read(const Launch &L, const void *src, size_t bytes, int n_wg, uint32_t *sink) {
-    hipLaunchKernelGGL(k_probe_read, dim3((unsigned)n_wg), dim3(256), 0, L.stream, static_cast<const uint4 *>(src), bytes / 16, sink);
-    return hipGetLastError();
-}
-
 hipError_t fill_u32(const Launch &L, uint32_t *dst, uint32_t value, size_t n) {
     if (n == 0) return hipSuccess;
     hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, L.stream, dst, value, n);
@@ -298,12 +274,12 @@ hipError_t combine_tokens(const Launch &L, const float *down, const float *w, co
 // --------------------------------------------------------------------------- down + combine in one launch
 
 // The shared body of the down + combine workgroup: token t, output rows rb * D .. + D with D = 64 / spt, a quad for
-// every (row, slot). `wait` runs after the weight requests and before the activation columns are read.
-template <int WT, int U, int NB, class Wait>
+// every (row, slot).
+template <int WT, int U, int NB>
 __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w, u32 n_experts, int nb,
                                                   const uint8_t *act, const u32 *sel, const float *wts,
                                                   const float *resid, int spt, int rpe, float *y, int t, int rb,
-                                                  u32 *fault, u32 layer, const Wait &wait) {
+                                                  u32 *fault, u32 layer) {
     const int tid = threadIdx.x, q = tid & 3, quad = tid >> 2;
     const int D = 64 / spt;
     const int e = quad % spt, dl = quad / spt;
@@ -328,17 +304,10 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
     float *s_w = part + D * spt;                                              // [spt]
     u32 *s_sel = reinterpret_cast<u32 *>(s_w + spt);                          // [spt]
     Blk<WT> b[U];
-    if constexpr (Wait::kWaits) {
-        // the rows do not depend on the activations: request them, then wait for the producers
-        preload<WT, U>(b, wrow, q);
-        wait();
-        stage_bytes(cols, act_cols, spt * col_bytes);
-    } else {
-        Stage<5> st;
-        st.load(act_cols, spt * col_bytes);
-        preload<WT, U>(b, wrow, q);
-        st.store(cols, act_cols, spt * col_bytes);
-    }
+    Stage<5> st;
+    st.load(act_cols, spt * col_bytes);
+    preload<WT, U>(b, wrow, q);
+    st.store(cols, act_cols, spt * col_bytes);
     if (tid < spt) {
         s_w[tid] = my_w;
         s_sel[tid] = my_sel;
@@ -357,11 +326,6 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
     }
 }
 
-struct NoWait {
-    static constexpr bool kWaits = false;
-    __device__ __forceinline__ void operator()() const {}
-};
-
 template <int WT, int U, int NB>
 __global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_experts, int nb, const uint8_t *act,
                                                       const u32 *sel, const float *wts, const float *resid, int spt,
@@ -370,34 +334,8 @@ __global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_ex
     const int D = 64 / spt;
     const int blocks_per_token = (rpe + D - 1) / D;
     down_combine_body<WT, U, NB>(lds, w, n_experts, nb, act, sel, wts, resid, spt, rpe, y,
-                                 blockIdx.x / blocks_per_token, blockIdx.x % blocks_per_token, fault, layer, NoWait{});
+                                 blockIdx.x / blocks_per_token, blockIdx.x % blocks_per_token, fault, layer);
 }
-
-// ------------------------------------------------------------------------- the whole layer step, one launch
-
-// Waits until the token's gate.up workgroups have all published their activation blocks.
-struct CounterWait {
-    static constexpr bool kWaits = true;
-    u32 *counter;
-    u32 need, spin_limit;
-    u32 *fault;
-    u32 layer;
-    __device__ __forceinline__ void operator()() const {
-        if (threadIdx.x == 0) {
-            u32 spins = 0;
-            // relaxed polls (an acquiring poll would invalidate the caches on every turn); one fence afterwards
-            while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) {
-                __builtin_amdgcn_s_sleep(2);
-                if (++spins > spin_limit) { // every wave leaves: the launch ends with a fault, never a hang
-                    bm_raise(fault, layer, kSiteStalled);
-                    break;
-                }
-            }
-        }
-        __syncthreads();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    }
-};
 
 // One 32-value q8_2 block held eight values a lane by four consecutive lanes (the in-kernel token quantizer).
 __device__ __forceinline__ void q82_quad8(const float (&v)[8], uint8_t *col, int nb, int blk, int lane4, u32 *fault,
@@ -524,51 +462,6 @@ __global__ __launch_bounds__(256) void k_gate_up_x(const float *x, const uint8_t
     const int blocks_per_slot = nh * 8;
     gate_up_x_body<WA, UA, NBA>(lds, x, wg, wu, n_experts, NBA > 0 ? NBA : nba, nh, sel, spt, act_x, act_h, h,
                                 blockIdx.x / blocks_per_slot, blockIdx.x % blocks_per_slot, rule, fault, layer);
-}
-
-// The decode step of one MoE layer for m tokens in one launch. The first n_a workgroups are the gate . up ones
-// above; once its block of the down activation is written each bumps the token's counter. The workgroups after
-// them are the down + combine ones: they request their rows at once - the rows do not depend on the activations,
-// so the down stack streams from HBM while gate . up still runs - and read the activations when the counter says
-// all are there. Workgroups are dispatched in index order, so every producer is resident or finished before any
-// consumer waits. The last consumer resets the counters, so a replay starts clean without a memset node.
-template <int WA, int UA, int NBA, int WB, int UB, int NBB>
-__global__ __launch_bounds__(256) void k_moe_decode(const float *x, const uint8_t *wg, const uint8_t *wu,
-                                                    const uint8_t *wd, u32 n_experts, int nba, int nbb,
-                                                    const u32 *sel, const float *wts, const float *resid, int spt,
-                                                    int m, uint8_t *act_x, uint8_t *act_h, float *h, float *y,
-                                                    u32 *counters, u32 spin_limit, GateRule rule, u32 *fault,
-                                                    u32 layer) {
-    extern __shared__ __align__(16) uint8_t lds[];
-    const int tid = threadIdx.x;
-    const int na = NBA > 0 ? NBA : nba, nh = NBB > 0 ? NBB : nbb;
-    const int hidden = na * 256;
-    const int blocks_per_slot = nh * 8;
-    const int n_a = m * spt * blocks_per_slot;
-    if ((int)blockIdx.x < n_a) {
-        const int slot = blockIdx.x / blocks_per_slot;
-        gate_up_x_body<WA, UA, NBA>(lds, x, wg, wu, n_experts, na, nh, sel, spt, act_x, act_h, h, slot,
-                                    blockIdx.x % blocks_per_slot, rule, fault, layer);
-        // publish: the block's stores (complete at the barrier), then the count with agent-scope release
-        __syncthreads();
-        if (tid == 0)
-            __hip_atomic_fetch_add(&counters[1 + slot / spt], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        return;
-    }
-    const int D = 64 / spt;
-    const int blocks_per_token = (hidden + D - 1) / D;
-    const int bi = (int)blockIdx.x - n_a;
-    const int t = bi / blocks_per_token, rb = bi % blocks_per_token;
-    down_combine_body<WB, UB, NBB>(lds, wd, n_experts, nh, act_h, sel, wts, resid, spt, hidden, y, t, rb, fault, layer,
-                                   CounterWait{&counters[1 + t], (u32)(spt * blocks_per_slot), spin_limit, fault, layer});
-    // the last consumer to finish leaves the counters clean for the next launch
-    __syncthreads();
-    if (tid == 0) {
-        const u32 done = __hip_atomic_fetch_add(&counters[0], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        if (done == (u32)(m * blocks_per_token) - 1) {
-            for (int i = 0; i <= m; i++) __hip_atomic_store(&counters[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
 }
 
 // ------------------------------------------------------------- the fused step for the types that take Q8_K columns
@@ -993,11 +886,8 @@ static bool tab_known(int t) {
     return t == BM_Q3K || t == BM_Q4K || t == BM_Q5K || t == BM_Q6K || t == BM_IQ2XXS || t == BM_IQ3XXS || t == BM_IQ4XS;
 }
 
-bool moe_decode_supported(int plan, int gate_type, int down_type) {
-    if (plan == kPlanOneLaunch) return gate_type == BM_Q4K && (down_type == BM_Q6K || down_type == BM_Q4K);
-    // two launches: every type this library has a row dot for, on either side
-    return tab_known(gate_type) && tab_known(down_type);
-}
+// every type this library has a row dot for goes on either side of the fused step
+bool moe_decode_supported(int gate_type, int down_type) { return tab_known(gate_type) && tab_known(down_type); }
 
 hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8_t *wg, const uint8_t *wu,
                      int n_experts, int hidden, int ff, const uint32_t *sel, int slots_per_token, int m,
@@ -1059,51 +949,21 @@ hipError_t down_combine_hq(const Launch &L, int wtype, const uint8_t *w, int n_e
     return hipGetLastError();
 }
 
-hipError_t moe_decode(const Launch &L, int plan, int gate_type, int down_type, const float *x, const uint8_t *wg,
-                      const uint8_t *wu, const uint8_t *wd, int n_experts, int hidden, int ff, const uint32_t *sel,
-                      const float *wts, const float *resid, int slots_per_token, int m, uint8_t *act_x,
-                      uint8_t *act_h, float *h, float *y, uint32_t *counters, uint32_t spin_limit) {
-    const int nba = hidden / 256, nbb = ff / 256, spt = slots_per_token;
-    const int D = 64 / spt;
-    const size_t lds_a = (size_t)act_col_bytes(gate_type, hidden) + 32 * sizeof(float);
-    const size_t lds_b = down_combine_lds(down_type, ff, spt);
-    const unsigned grid_a = (unsigned)m * (unsigned)spt * (unsigned)(ff / 32);
-    if (!moe_decode_supported(plan, gate_type, down_type)) return hipErrorInvalidValue;
-    if (plan == kPlanTwoLaunches) {
-        // a down stack on Q8_K columns cannot get them from the gate . up launch (a column's block spans eight of
-        // its workgroups): that launch leaves h as f32 rows and the down launch quantizes them itself
-        // (for a down stack on Q8_2_X4 columns the same split measures slower, 12.2 us a token against 11.3 at the
-        // Qwen3 shape: the gate . up launch loses its quantizer epilogue, 0.5 us, but every down workgroup then encodes
-        // the token's 6144 values, 700 instructions a wave that do not hide behind its weight stream)
-        const bool hq = bm_takes_q8k(down_type);
-        hipError_t e = gate_up_x(L, gate_type, x, wg, wu, n_experts, hidden, ff, sel, spt, m, act_x, hq ? nullptr : act_h, h);
-        if (e != hipSuccess) return e;
-        if (hq) return down_combine_hq(L, down_type, wd, n_experts, ff, h, act_h, sel, wts, resid, spt, m, hidden, y);
-        return down_combine(L, down_type, wd, n_experts, ff, act_h, sel, wts, resid, spt, m, hidden, y);
-    }
-    const size_t lds = lds_a > lds_b ? lds_a : lds_b;
-    const unsigned grid = grid_a + (unsigned)m * (unsigned)((hidden + D - 1) / D);
-#define BM_FUSED(WA, UA, NA, WB, UB, NBB_)                                                                             \
-    {                                                                                                                  \
-        auto kern = k_moe_decode<WA, UA, NA, WB, UB, NBB_>;                                                            \
-        hipError_t e = allow_lds(kern, lds);                                                                           \
-        if (e != hipSuccess) return e;                                                                                 \
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, x, wg, wu, wd, (u32)n_experts, nba, nbb, sel,   \
-                           wts, resid, spt, m, act_x, act_h, h, y, counters, spin_limit, L.rule, L.fault, L.layer);    \
-    }
-    if (down_type == BM_Q6K) {
-        if (nba == 8 && nbb == 3) BM_FUSED(BM_Q4K, kRingQ4K, 8, BM_Q6K, kRingQ6K, 3)
-        else if (nba == 8) BM_FUSED(BM_Q4K, kRingQ4K, 8, BM_Q6K, 1, 0)
-        else if (nbb == 3) BM_FUSED(BM_Q4K, 1, 0, BM_Q6K, kRingQ6K, 3)
-        else BM_FUSED(BM_Q4K, 1, 0, BM_Q6K, 1, 0)
-    } else if (down_type == BM_Q4K) {
-        if (nba == 8) BM_FUSED(BM_Q4K, kRingQ4K, 8, BM_Q4K, 1, 0)
-        else BM_FUSED(BM_Q4K, 1, 0, BM_Q4K, 1, 0)
-    } else {
-        return hipErrorInvalidValue;
-    }
-#undef BM_FUSED
-    return hipGetLastError();
+hipError_t moe_decode(const Launch &L, int gate_type, int down_type, const float *x, const uint8_t *wg, const uint8_t *wu,
+                      const uint8_t *wd, int n_experts, int hidden, int ff, const uint32_t *sel, const float *wts,
+                      const float *resid, int slots_per_token, int m, uint8_t *act_x, uint8_t *act_h, float *h, float *y) {
+    const int spt = slots_per_token;
+    if (!moe_decode_supported(gate_type, down_type)) return hipErrorInvalidValue;
+    // a down stack on Q8_K columns cannot get them from the gate . up launch (a column's block spans eight of
+    // its workgroups): that launch leaves h as f32 rows and the down launch quantizes them itself
+    // (for a down stack on Q8_2_X4 columns the same split measures slower, 12.2 us a token against 11.3 at the
+    // Qwen3 shape: the gate . up launch loses its quantizer epilogue, 0.5 us, but every down workgroup then encodes
+    // the token's 6144 values, 700 instructions a wave that do not hide behind its weight stream)
+    const bool hq = bm_takes_q8k(down_type);
+    hipError_t e = gate_up_x(L, gate_type, x, wg, wu, n_experts, hidden, ff, sel, spt, m, act_x, hq ? nullptr : act_h, h);
+    if (e != hipSuccess) return e;
+    if (hq) return down_combine_hq(L, down_type, wd, n_experts, ff, h, act_h, sel, wts, resid, spt, m, hidden, y);
+    return down_combine(L, down_type, wd, n_experts, ff, act_h, sel, wts, resid, spt, m, hidden, y);
 }
 
 // --------------------------------------------------------------- the fused step on scratch the library holds
@@ -1142,8 +1002,8 @@ hipError_t moe_decode_static(const Launch &L, int device, int gate_type, int dow
     float *h = reinterpret_cast<float *>(g_scratch_at[device] + kStaticColBytes);
     // every live slot's column (or f32 rows) is written whole by the first launch before the second reads it, and a
     // slot that is not live is never read into a sum: nothing here has to start at zero
-    return moe_decode(L, kPlanTwoLaunches, gate_type, down_type, x, wg, wu, wd, n_experts, hidden, ff, sel, wts, resid,
-                      slots_per_token, m, nullptr, act_h, h, y, nullptr, 0);
+    return moe_decode(L, gate_type, down_type, x, wg, wu, wd, n_experts, hidden, ff, sel, wts, resid,
+                      slots_per_token, m, nullptr, act_h, h, y);
 }
 
 hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, const uint8_t *col, int32_t *out) {

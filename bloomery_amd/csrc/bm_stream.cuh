@@ -25,7 +25,6 @@ namespace bmk {
 constexpr u32 kSiteQuantColumn = 1; // crates/device/src/fault.rs:73-76
 constexpr u32 kSiteExpertId = 7;    // crates/device/src/fault.rs:89
 constexpr u32 kSiteF32Product = 21; // crates/device/src/fault.rs:151-155: a gate or up sum that is not finite under a clamp
-constexpr u32 kSiteStalled = 31;    // ours: a fused launch's down workgroup gave up waiting for its activations
 
 // LDS bytes of the IQ2_XXS tables: 256 grid entries of 16 + 128 sign entries of 8.
 constexpr int kTabBytes = 256 * 16 + 128 * 8;

@@ -51,7 +51,6 @@ extern "C" {
 #define BM_SITE_ROUTER 5       /* a token's logits hold a value that is not finite */
 #define BM_SITE_EXPERT_ID 7    /* an expert id at or past the stack */
 #define BM_SITE_F32_PRODUCT 21 /* a gate or up sum that is not finite met a clamped gate rule: the value is NaN */
-#define BM_SITE_STALLED 31     /* ours: a bm_moe_decode consumer gave up waiting for its producers */
 
 /* The id of a slot served elsewhere (crates/gpu/src/host/slots.rs:10): every routed entry skips it silently - the
  * gate . up entries write nothing for it (no h rows, no activation block) and the down entries leave its rows as they
@@ -61,6 +60,35 @@ extern "C" {
 typedef struct bm_ctx bm_ctx;         /* crates/gpu/src/lib.rs:2529 Gpu: device, stream, fault word */
 typedef struct bm_weights bm_weights; /* crates/gpu/src/tensor.rs:588-616 DeviceTensor<u32>: rows of block bytes */
 typedef struct bm_act bm_act;         /* crates/gpu/src/tensor.rs:811-948 Q8Act: m quantized columns of k values */
+
+/* The rule a gate . up entry (bm_gate_up, bm_gate_up_x, bm_moe_decode, bm_moe_decode_noalloc, bm_gate_up_tiles,
+ * bm_swiglu_quant) applies to a row's gate sum g and up sum u: the Act argument of the reference's launchers
+ * (crates/gpu/src/kquant/act.rs:21-57 Act, device codes :46-56; GateUpAct.rule of crates/gpu/src/kquant/sel.rs), passed
+ * with each launch. An entry whose rule argument is NULL takes the context's rule, which bm_set_gate_rule sets
+ * (BM_ACT_SILU_MUL until then). The numbers are the CPU path's (crates/qdot/src/lib.rs:11467 swiglu, :11492
+ * swiglu_clamp, swiglu_oai, :11617 swiglu_gclamp; crates/model/src/ops.rs:2345 situ_into), every exponential ik's.
+ *   BM_ACT_SILU_MUL       silu(g) * u (the default; limit ignored)
+ *   BM_ACT_SWIGLU_CLAMP   min(silu(g), limit) * clamp(u, -limit, limit); limit <= 1e-6 clamps nothing; limit finite
+ *   BM_ACT_SWIGLU_OAI     x = min(g, limit), y = clamp(u, -limit, limit): x / (1 + e^(-1.702 x)) * (y + 1); limit finite, >= 0
+ *   BM_ACT_SITU           (beta tanh(g / beta) * sigmoid(g)) * (25 tanh(u / 25)), beta = limit, finite and positive; each
+ *                         scale by the f32 reciprocal, the products in that order (act.rs:152-163 situ). The tanh is the
+ *                         device library's f32 one where the CPU path calls the host's: a value can differ from the CPU
+ *                         path's in its last bits (the reference says the same of its own card and host), so under this rule
+ *                         the contract is 1e-5 relative on h (crates/model/src/ops.rs:7124-7131), not bits
+ *   BM_ACT_SWIGLU_GCLAMP  silu(min(g, limit)) * clamp(u, -limit, limit); limit finite and positive
+ * Under every rule but the first a sum that is not finite raises BM_SITE_F32_PRODUCT and its value is NaN (act.rs:166-175
+ * apply_checked; the CPU path's rules refuse such a block). A rule or limit outside the above is refused by the entry
+ * (BM_ETYPE / BM_ESHAPE) before anything is enqueued, as Act::code refuses it (act.rs:71-125). */
+#define BM_ACT_SILU_MUL 0
+#define BM_ACT_SWIGLU_CLAMP 1
+#define BM_ACT_SWIGLU_OAI 2
+#define BM_ACT_SITU 3
+#define BM_ACT_SWIGLU_GCLAMP 4
+typedef struct bm_gate_act {
+    int rule;    /* one of BM_ACT_* */
+    float limit; /* the clamp limit, or SiTU's beta */
+} bm_gate_act;
+int bm_set_gate_rule(bm_ctx *ctx, int rule, float limit);
 
 /* ------------------------------------------------------------------------------------------------ context */
 
@@ -141,15 +169,15 @@ int bm_gemv_x(bm_ctx *ctx, const bm_weights *w, const float *x_dev, int m, bm_ac
 /* ExpertKernels::enqueue_gate_up(GateUpArgs) (crates/gpu/src/arch/qwen3moe/experts.rs:326-335,462), for Q4_K,
  * Q5_K (crates/gpu/src/kquant/tiles.rs:120-190), Q6_K (crates/gpu/src/q6k_sel.rs:633), IQ2_XXS (crates/gpu/src/iq_sel.rs:1357) and IQ4_XS (iq_sel.rs, iq4_xs_gate_up_sel) stacks of one type:
  * slot s < n_slots reads expert sel_dev[s]'s rows of both stacks against activation column s / slots_per_col and
- * writes h_dev[s * rows_per_expert + r] = silu(gate_r) * up_r in the CPU path's SwiGLU
- * (crates/qdot/src/lib.rs:11467). An id at or past the stack raises BM_SITE_EXPERT_ID and writes NaN into the
+ * writes h_dev[s * rows_per_expert + r] = the rule's value of (gate_r, up_r) - rule is GateUpArgs' act, NULL for the
+ * context's; silu(gate_r) * up_r in the CPU path's SwiGLU (crates/qdot/src/lib.rs:11467) by default. An id at or past the stack raises BM_SITE_EXPERT_ID and writes NaN into the
  * slot's rows (and a NaN-scaled block into act_h); BM_HOST_SLOT is skipped: nothing written, nothing raised.
  * h_dev may be NULL when act_h is given.
  * act_h (optional, NULL to skip): the down projection's activation, quantized in the same launch from the rows
  * just written, column s of act_h for slot s, in the form of act_h's type (Q8_2_X4 only; rows_per_expert must
  * then be act_h's k). The reference runs this as a separate quantizer launch (dispatch.rs:1343). */
 int bm_gate_up(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_act *act, const uint32_t *sel_dev,
-               int n_slots, int rows_per_expert, int slots_per_col, float *h_dev, bm_act *act_h);
+               int n_slots, int rows_per_expert, int slots_per_col, const bm_gate_act *rule, float *h_dev, bm_act *act_h);
 
 /* Q4kSelKernels::enqueue_gemv_q4k_sel (crates/gpu/src/q4k_sel.rs:978), Q6kSelKernels::enqueue_gemv_q6k_sel
  * (crates/gpu/src/q6k_sel.rs:513), QuantSelKernels::enqueue_down (crates/gpu/src/iq_sel.rs:1557): slot s writes
@@ -191,33 +219,26 @@ int bm_down_combine_h(bm_ctx *ctx, const bm_weights *w, const float *h_dev, bm_a
  * holds m rows of hidden = wg's k f32 values (16-byte aligned); token t's slots are sel_dev / w_dev[t *
  * n_slots_per_token ..]; y_dev[t * hidden + d] gets bm_combine_tokens' value. Same bits as bm_quantize, bm_gate_up
  * (with act_h) and bm_down_combine run one after the other. Gate and up are of one type; every type of this library
- * goes on either side (BM_PLAN_ONE_LAUNCH: Q4_K gate/up with Q6_K or Q4_K down only). A slot whose id is BM_HOST_SLOT
+ * goes on either side. A slot whose id is BM_HOST_SLOT
  * is skipped by both halves (its h rows and activation column keep what they held, it adds nothing to the sum, nothing is
  * raised); any other id at or past the stack raises BM_SITE_EXPERT_ID and adds nothing. act_h is caller-held scratch
  * (m * n_slots_per_token columns of ff = wd's k, in the form wd dots against) and holds the quantized h afterwards;
  * act_x (optional, in the form wg dots against) receives the quantized x columns; h_dev receives the f32 h rows:
  * optional, except that a down stack on Q8_K columns needs it (16-byte aligned): a Q8_K block spans eight gate . up
  * workgroups, so that launch leaves f32 rows and the down launch quantizes them (bm_down_combine_h). m <= 1024.
- * Two plans (bm_set_decode_plan):
- *   BM_PLAN_TWO_LAUNCHES (default): gate . up with both quantizers folded in, then down + combine;
- *   BM_PLAN_ONE_LAUNCH: one launch; the down workgroups start streaming their rows at once and wait on a
- *     per-token device counter for that token's gate/up workgroups. A wait that outlasts the context's spin
- *     limit raises BM_SITE_STALLED and the launch still ends (y is then not valid; bm_fault_clear re-arms the
- *     counters). Launches of this plan that share a context must not overlap. */
-#define BM_PLAN_ONE_LAUNCH 1
-#define BM_PLAN_TWO_LAUNCHES 2
+ * Two launches: gate . up with both quantizers folded in (bm_gate_up_x), then down + combine (bm_down_combine). */
 int bm_moe_decode(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_weights *wd, const float *x_dev,
                   const uint32_t *sel_dev, const float *w_dev, const float *resid_dev, int n_slots_per_token, int m,
-                  bm_act *act_h, bm_act *act_x, float *h_dev, float *y_dev);
-int bm_set_decode_plan(bm_ctx *ctx, int plan);
-/* The first launch of BM_PLAN_TWO_LAUNCHES on its own: bm_quantize, bm_gate_up and the quantizer of h in one
+                  const bm_gate_act *rule, bm_act *act_h, bm_act *act_x, float *h_dev, float *y_dev);
+/* The first launch of bm_moe_decode on its own: bm_quantize, bm_gate_up and the quantizer of h in one
  * launch, from the f32 token rows (gate and up of one type; rows_per_expert = ff a multiple of 256). act_h: Q8_2_X4
  * columns for the down stack, or NULL; h_dev: the f32 h rows, or NULL; one of the two at least. Ids as bm_gate_up
  * takes them (BM_HOST_SLOT skipped silently). Follow it with
  * bm_down_combine or bm_gemv_sel over act_h, or bm_down_combine_h over h_dev. */
 int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const float *x_dev, const uint32_t *sel_dev,
-                 int n_slots_per_token, int m, int rows_per_expert, bm_act *act_h, bm_act *act_x, float *h_dev);
-/* bm_moe_decode (BM_PLAN_TWO_LAUNCHES) for callers that cannot allocate device memory or hold a scratch handle: code
+                 int n_slots_per_token, int m, int rows_per_expert, const bm_gate_act *rule, bm_act *act_h, bm_act *act_x,
+                 float *h_dev);
+/* bm_moe_decode for callers that cannot allocate device memory or hold a scratch handle: code
  * under HIP graph capture, serving loops and harnesses that forbid hipMalloc. It has no counterpart in the reference,
  * whose callers make their Q8Act scratch at load time. The quantized h between the two launches (bm_moe_decode's act_h,
  * and its h_dev rows for a down stack on Q8_K columns) lives in an array the library holds on each device for the life
@@ -228,10 +249,7 @@ int bm_gate_up_x(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const 
  * order do not, and nothing in the array has to start at zero. */
 int bm_moe_decode_noalloc(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_weights *wd, const float *x_dev,
                           const uint32_t *sel_dev, const float *w_dev, const float *resid_dev, int n_slots_per_token, int m,
-                          float *y_dev);
-/* Polls (a memory round trip each, about a microsecond) a BM_PLAN_ONE_LAUNCH consumer waits before it gives up;
- * the default is 1 << 18. */
-int bm_set_spin_limit(bm_ctx *ctx, uint32_t spins);
+                          const bm_gate_act *rule, float *y_dev);
 
 /* ------------------------------------------------------------- decode of several tokens: grouped by expert */
 
@@ -265,7 +283,7 @@ int bm_quantize_ord(bm_ctx *ctx, const float *x_dev, const uint32_t *start_dev, 
  * slot raises BM_SITE_EXPERT_ID and writes NaN. */
 int bm_gate_up_tiles(bm_ctx *ctx, const bm_weights *wg, const bm_weights *wu, const bm_act *act, const uint32_t *order_dev,
                      const uint32_t *start_dev, const uint32_t *tiles_dev, int n_slots, int rows_per_expert,
-                     int slots_per_col, float *h_dev, bm_act *act_h);
+                     int slots_per_col, const bm_gate_act *rule, float *h_dev, bm_act *act_h);
 /* Q4kSelKernels::enqueue_gemv_q4k_tiles (crates/gpu/src/q4k_sel.rs:1208; Q5K/Q6K/IQ forms kquant/tiles.rs:120-190):
  * the grouped down. Entry j reads column j of act and writes y_dev[order[j] * rows_per_expert + r], bm_gemv_sel's
  * value for that slot. An entry that names no slot raises BM_SITE_EXPERT_ID and writes nothing. */
@@ -307,23 +325,8 @@ int bm_set_gemm_mode(bm_ctx *ctx, int mode);
 /* GemmKernels::enqueue_swiglu_quant (crates/gpu/src/gemm/swiglu.rs:46): column c of act = the quantized
  * silu(g) * u of g_dev / u_dev[c * k .. (c + 1) * k), k = act's k, slot-major as the gate and up GEMMs write them;
  * bm_quantize's bytes of the CPU path's SwiGLU. Q8_2_X4 columns only. */
-int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, bm_act *act);
+int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, const bm_gate_act *rule, bm_act *act);
 
-/* The rule the gate . up entries (bm_gate_up, bm_gate_up_x, bm_moe_decode, bm_gate_up_tiles, bm_swiglu_quant) apply to
- * a row's gate sum g and up sum u: the Act argument of the reference's launchers (crates/gpu/src/kquant/act.rs:21-57,
- * device codes :46-56), set on the context and read by each launch as it is enqueued. The numbers are the CPU path's
- * (crates/qdot/src/lib.rs:11467 swiglu, :11492 swiglu_clamp, swiglu_oai, :11617 swiglu_gclamp), every exponential ik's.
- *   BM_ACT_SILU_MUL       silu(g) * u (the default; limit ignored)
- *   BM_ACT_SWIGLU_CLAMP   min(silu(g), limit) * clamp(u, -limit, limit); limit <= 1e-6 clamps nothing; limit finite
- *   BM_ACT_SWIGLU_OAI     x = min(g, limit), y = clamp(u, -limit, limit): x / (1 + e^(-1.702 x)) * (y + 1); limit finite, >= 0
- *   BM_ACT_SWIGLU_GCLAMP  silu(min(g, limit)) * clamp(u, -limit, limit); limit finite and positive
- * Under the three clamped rules a sum that is not finite raises BM_SITE_F32_PRODUCT and its value is NaN (act.rs:166-175
- * apply_checked; the CPU path's rules return false for such a block). SiTU-GLU (code 3) is not built. */
-#define BM_ACT_SILU_MUL 0
-#define BM_ACT_SWIGLU_CLAMP 1
-#define BM_ACT_SWIGLU_OAI 2
-#define BM_ACT_SWIGLU_GCLAMP 4
-int bm_set_gate_rule(bm_ctx *ctx, int rule, float limit);
 
 /* ------------------------------------------------------------------------------------------------- router */
 
@@ -417,12 +420,6 @@ const char *bm_gguf_get_str(const bm_gguf *g, const char *key);
 int bm_weights_from_gguf(bm_ctx *ctx, const bm_gguf *g, const char *name, bm_weights **out, int *rows_per_expert, int *n_experts);
 
 /* ------------------------------------------------------------------------------------------- verification */
-
-/* Measurement only (no counterpart in the reference): n_workgroups workgroups fetch `bytes` from src_dev with plain
- * 16-byte loads and do nothing else; with bytes = 0 it is an empty launch. The time of a decode launch is to be read
- * against this: the same bytes by a kernel without arithmetic, tables or dependent reads. sink_dev: n_workgroups words. */
-int bm_probe_read(bm_ctx *ctx, const void *src_dev, size_t bytes, int n_workgroups, uint32_t *sink_dev);
-
 
 /* The exact per-block integers the kernels above form for row `row` of w against column `col` of act, written
  * to out_dev as i32, through the same device code the launchers run:

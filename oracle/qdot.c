@@ -752,14 +752,17 @@ void ora_swiglu(const float *gate, const float *up, int n, float *out) {
 // limit) * clamp(u), nothing clamped at limit <= 1e-6. rule 2: swiglu_oai / swiglu_oai_1 at alpha 1.702 (the value the
 // launchers run, crates/gpu/src/kquant/act.rs:58-60): x = min(g, limit), y = clamp(u), x / (1 + e^(alpha (0 - x))) *
 // (y + 1). rule 4: swiglu_gclamp / swiglu_gclamp_1 (:11617-11660): silu(min(g, limit)) * clamp(u), nothing clamped at
-// limit <= 1e-6. rule 0: ora_swiglu. Returns what the reference's functions return: 0 when a clamping rule met a gate
+// limit <= 1e-6. rule 3: SiTU-GLU at linear beta 25, limit = the gate's beta (crates/model/src/ops.rs:2345-2360
+// situ_into: each scale by the f32 reciprocal, the host libm's tanhf, the scale back, 1 / (1 + e^(0 - g)), (a * s) * v);
+// its tanh is whatever libm this file is linked with, so the rule is pinned to the closed form in f64 at the
+// reference's own bound (1e-5 relative, ops.rs:7124-7160), not to bits. rule 0: ora_swiglu. Returns what the reference's functions return: 0 when a clamping rule met a gate
 // or up value that is not finite (the caller refuses the block), else 1; -1 for a rule this file does not hold.
 int ora_gate_rule(int rule, float limit, const float *gate, const float *up, int n, float *out) {
     if (rule == 0) {
         ora_swiglu(gate, up, n, out);
         return 1;
     }
-    if (rule != 1 && rule != 2 && rule != 4) return -1;
+    if (rule < 1 || rule > 4) return -1;
     if ((rule == 1 || rule == 4) && !(limit > 1e-6f)) { // a NaN limit clamps nothing either
         ora_swiglu(gate, up, n, out);
         return 1;
@@ -768,7 +771,12 @@ int ora_gate_rule(int rule, float limit, const float *gate, const float *up, int
     for (int i = 0; i < n; i++) {
         const float g = gate[i], u = up[i];
         if (!isfinite(g) || !isfinite(u)) finite = 0;
-        if (rule == 1) {
+        if (rule == 3) {
+            const float a = tanhf(g * (1.0f / limit)) * limit;
+            const float sg = 1.0f / (1.0f + ora_expf_ik(0.0f - g));
+            const float v = tanhf(u * (1.0f / 25.0f)) * 25.0f;
+            out[i] = (a * sg) * v;
+        } else if (rule == 1) {
             float s = g / (1.0f + ora_expf_ik(0.0f - g));
             s = limit < s ? limit : s;
             float c = u < limit ? u : limit;

@@ -11,7 +11,7 @@ import bloomery_amd as bm
 import ora
 from common import normal_f32
 from test_gpu_decode import (Layer, assert_f32, gpu, grouped_tables_on_device, random_blocks, route,  # noqa: F401
-                             run_single_launch)
+                             run_fused_step)
 from test_gpu_prefill import run_prefill
 
 pytestmark = pytest.mark.gpu
@@ -87,7 +87,6 @@ def test_deepseek_shaped_layer_slot_by_slot(gpu, ds_layer):
     act_h = gpu.act(bm.IQ2_XXS, DS_FF, n_slots)
     h = gpu.buffer(np.float32, n_slots * DS_FF).fill_bytes(0xFF)
     y = gpu.buffer(np.float32, m * DS_HIDDEN).fill_bytes(0xFF)
-    gpu.set_decode_plan(bm.PLAN_TWO_LAUNCHES)
     gpu.enqueue_moe_decode(routed.dg, routed.du, routed.dd, xd, sel, wd, sdown, DS_TOPK, m, act_h, y, h=h)
     assert_f32(h.download(), want_h, "h")
     for s in (0, n_slots // 2, n_slots - 1):
@@ -157,8 +156,7 @@ def test_prefill_layer_shape_under_skewed_routing(gpu):
 
 # ------------------------------------------------------------------------ a host-served slot through gate . up
 
-@pytest.mark.parametrize("plan", (bm.PLAN_ONE_LAUNCH, bm.PLAN_TWO_LAUNCHES))
-def test_gate_up_entries_skip_a_host_slot(gpu, plan):
+def test_gate_up_entries_skip_a_host_slot(gpu):
     """BM_HOST_SLOT through bm_gate_up, bm_gate_up_x and bm_moe_decode: no fault, the slot's rows of h and its
     activation column keep what they held, and y is the oracle's sum over the live slots."""
     L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 4, 3400)
@@ -172,7 +170,7 @@ def test_gate_up_entries_skip_a_host_slot(gpu, plan):
     want1, want_h1 = L.oracle(x[1:], ids[1:], wts[1:], 3)
     gpu.fault_clear()
     # the fused step
-    y, h, act_h, _ = run_single_launch(gpu, L, x, ids, wts, top_k, plan=plan)
+    y, h, act_h, _ = run_fused_step(gpu, L, x, ids, wts, top_k)
     assert gpu.fault() == (bm.FAULT_NONE, 0)
     h = h.reshape(m * top_k, 256)
     assert np.all(h[1].view(np.uint32) == 0xFFFFFFFF), "the host's slot keeps its rows of h"
@@ -201,7 +199,6 @@ def test_gate_up_entries_skip_a_host_slot(gpu, plan):
             assert np.array_equal(ah.download(s), ora.quantize_col(bm.Q6_K, want_h1[(s - 3) * 256:(s - 2) * 256])), f"{entry} act_h {s}"
         ah.free()
         hb.free()
-    gpu.set_decode_plan(bm.PLAN_TWO_LAUNCHES)
     for b in (xd, sel, act):
         b.free()
     L.free()

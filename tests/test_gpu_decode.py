@@ -414,10 +414,9 @@ def test_layers_of_every_type_and_several_tokens(gpu, types, hidden, ff, n_exper
     L.free()
 
 
-def run_single_launch(gpu, L, x, ids, wts, top_k, resid=None, replays=1, plan=bm.PLAN_ONE_LAUNCH):
-    """bm_moe_decode: the whole step with the quantizers folded in, in one launch or two. Returns (y, h, act_h
-    columns, act_x columns) of the last replay."""
-    gpu.set_decode_plan(plan)
+def run_fused_step(gpu, L, x, ids, wts, top_k, resid=None, replays=1):
+    """bm_moe_decode: the whole step with the quantizers folded in. Returns (y, h, act_h columns, act_x columns) of the
+    last replay."""
     m = x.shape[0]
     n_slots = m * top_k
     act_x = gpu.act(L.types[0], L.hidden, m)
@@ -443,7 +442,7 @@ def run_single_launch(gpu, L, x, ids, wts, top_k, resid=None, replays=1, plan=bm
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 1024, 512, 6, 3, 6),    # 64 / 6 rows a consumer workgroup: a ragged tail
     ((bm.Q4_K, bm.Q4_K, bm.Q4_K), 512, 512, 5, 4, 2),
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 4096, 256, 4, 2, 3),    # rows longer than one quantizer pass
-    ((bm.Q5_K, bm.Q5_K, bm.Q6_K), 2048, 512, 4, 3, 4),    # Q5_K gate/up at the whole-row shape (two launches only)
+    ((bm.Q5_K, bm.Q5_K, bm.Q6_K), 2048, 512, 4, 3, 4),    # Q5_K gate/up at the whole-row shape
     ((bm.Q5_K, bm.Q5_K, bm.Q5_K), 768, 256, 3, 2, 2),
     # the types on Q8_K columns: their quantizers folded into the two launches (the token's in every gate . up
     # workgroup, h's in every down workgroup), and the mixes of the two column forms
@@ -454,26 +453,15 @@ def run_single_launch(gpu, L, x, ids, wts, top_k, resid=None, replays=1, plan=bm
     ((bm.Q5_K, bm.Q5_K, bm.Q3_K), 512, 768, 3, 2, 3),
     ((bm.Q6_K, bm.Q6_K, bm.Q4_K), 768, 256, 3, 2, 2),
 ))
-@pytest.mark.parametrize("plan", (bm.PLAN_ONE_LAUNCH, bm.PLAN_TWO_LAUNCHES))
-def test_single_launch_step_matches_the_chain_and_the_oracle(gpu, types, hidden, ff, n_experts, m, top_k, plan):
-    # the one-launch plan takes Q4_K gate/up with Q6_K or Q4_K down only, and says so
-    if (types[0] != bm.Q4_K or types[2] not in (bm.Q4_K, bm.Q6_K)) and plan == bm.PLAN_ONE_LAUNCH:
-        L = Layer(gpu, types, hidden, ff, n_experts, 600 + hidden + ff, cheap=True)
-        x = np.zeros((m, hidden), np.float32)
-        with pytest.raises(bm.GpuError) as e:
-            run_single_launch(gpu, L, x, np.zeros((m, top_k), np.uint32), np.ones((m, top_k), np.float32), top_k, plan=plan)
-        assert e.value.code == bm.ETYPE and "bm_moe_decode" in str(e.value)
-        gpu.set_decode_plan(bm.PLAN_TWO_LAUNCHES)
-        L.free()
-        return
+def test_fused_step_matches_the_chain_and_the_oracle(gpu, types, hidden, ff, n_experts, m, top_k):
     L = Layer(gpu, types, hidden, ff, n_experts, 600 + hidden + ff)
     rng = np.random.default_rng(601)
     x = normal_f32(rng, (m, hidden))
     resid = normal_f32(rng, (m, hidden))
     ids, wts = route(rng, m, n_experts, top_k)
     gpu.fault_clear()
-    # three launches in a row: the counters must come back clean each time
-    y, h, act_h, act_x = run_single_launch(gpu, L, x, ids, wts, top_k, resid, replays=3, plan=plan)
+    # three launches in a row over the same scratch
+    y, h, act_h, act_x = run_fused_step(gpu, L, x, ids, wts, top_k, resid, replays=3)
     want_y, want_h = L.oracle(x, ids, wts, top_k)
     for t in range(m):
         assert np.array_equal(act_x[t], ora.quantize_col(types[0], x[t])), f"act_x token {t}"
@@ -493,7 +481,7 @@ def test_fused_step_at_the_token_limit(gpu):
     x = normal_f32(rng, (m, L.hidden))
     ids, wts = route(rng, m, L.n_experts, top_k)
     gpu.fault_clear()
-    y, h, _, _ = run_single_launch(gpu, L, x, ids, wts, top_k, plan=bm.PLAN_TWO_LAUNCHES)
+    y, h, _, _ = run_fused_step(gpu, L, x, ids, wts, top_k)
     want_y, want_h = L.oracle(x, ids, wts, top_k)
     assert_f32(h, want_h, "h")
     assert_f32(y, want_y, "y")
@@ -509,8 +497,7 @@ def test_fused_step_at_the_token_limit(gpu):
     L.free()
 
 
-@pytest.mark.parametrize("plan", (bm.PLAN_ONE_LAUNCH, bm.PLAN_TWO_LAUNCHES))
-def test_single_launch_refused_ids_and_host_slots(gpu, plan):
+def test_fused_step_refused_ids(gpu):
     L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 4, 700)
     rng = np.random.default_rng(701)
     x = normal_f32(rng, (2, 512))
@@ -518,7 +505,7 @@ def test_single_launch_refused_ids_and_host_slots(gpu, plan):
     wts = np.array([[0.5, 0.3, 0.2], [0.2, 0.5, 0.3]], np.float32)
     gpu.fault_clear()
     gpu.set_layer(4)
-    y, h, _, _ = run_single_launch(gpu, L, x, ids, wts, 3, plan=plan)
+    y, h, _, _ = run_fused_step(gpu, L, x, ids, wts, 3)
     assert gpu.fault(4) == ((4 << 8) | bm.SITE_EXPERT_ID, 1 << bm.SITE_EXPERT_ID)
     assert np.isnan(h.reshape(6, 256)[1]).all()
     # the refused slot adds nothing: the same as the oracle over the live slots with the same weights
@@ -529,32 +516,6 @@ def test_single_launch_refused_ids_and_host_slots(gpu, plan):
     assert_f32(y[512:], want1, "clean token")
     gpu.set_layer(bm.LAYER_NONE)
     gpu.fault_clear()
-    L.free()
-
-
-def test_single_launch_gives_up_waiting_and_recovers(gpu):
-    """A consumer that may not wait at all (spin limit 0) raises BM_SITE_STALLED and the launch still ends;
-    after bm_fault_clear the next launch is whole again."""
-    L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 8, 800)
-    rng = np.random.default_rng(801)
-    x = normal_f32(rng, (1, 2048))
-    ids, wts = route(rng, 1, 8, 8)
-    want_y, _ = L.oracle(x, ids, wts, 8)
-    gpu.fault_clear()
-    gpu.set_spin_limit(0)
-    y, _, _, _ = run_single_launch(gpu, L, x, ids, wts, 8)
-    word0, mask = gpu.fault()
-    gpu.set_spin_limit(1 << 18)
-    stalled = word0 == ((bm.LAYER_NONE << 8) | bm.SITE_STALLED)
-    if not stalled:  # every producer happened to finish first
-        assert word0 == bm.FAULT_NONE
-        assert_f32(y, want_y, "y of the launch that did not stall")
-    else:
-        assert mask == 1 << bm.SITE_STALLED
-    gpu.fault_clear()
-    y, _, _, _ = run_single_launch(gpu, L, x, ids, wts, 8, replays=2)
-    assert_f32(y, want_y, "y after recovery")
-    assert gpu.fault() == (bm.FAULT_NONE, 0)
     L.free()
 
 
@@ -845,21 +806,27 @@ def test_shape_refusals_are_named(gpu):
         b.free()
 
 
-def test_probe_read_runs_and_refuses_by_name(gpu):
-    """bm_probe_read is a measurement launch: it fetches and leaves the source as it is; its geometry is checked."""
+def test_bench_probe_runs_and_refuses(gpu):
+    """The benchmark's calibration launch (a library of its own, not the product's ABI): it fetches and leaves the
+    source as it is; its geometry is checked on the host."""
+    import ctypes as C
+    import os
+    path = os.path.join(os.path.dirname(bm.LIB_PATH), "libbm_bench_probe.so")
+    assert os.path.exists(path), f"{path} is not built (make -C bloomery_amd/csrc)"
+    lib = C.CDLL(path)
+    lib.bm_bench_probe_read.restype = C.c_int
+    lib.bm_bench_probe_read.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
     src = gpu.upload(np.arange(1 << 16, dtype=np.uint32), np.uint32)
     sink = gpu.buffer(np.uint32, 64).fill_bytes(0)
-    gpu.enqueue_probe_read(src, 0, 64, sink)
-    gpu.enqueue_probe_read(src, 4 << 16, 64, sink)
-    gpu.enqueue_probe_read(src, 4096 + 16, 7, sink)
+    stream = gpu.stream()
+    assert lib.bm_bench_probe_read(stream, src.ptr, 0, 64, sink.ptr) == 0
+    assert lib.bm_bench_probe_read(stream, src.ptr, 4 << 16, 64, sink.ptr) == 0
+    assert lib.bm_bench_probe_read(stream, src.ptr, 4096 + 16, 7, sink.ptr) == 0
     gpu.sync()
     assert np.array_equal(src.download(), np.arange(1 << 16, dtype=np.uint32))
-    for call, word in ((lambda: gpu.enqueue_probe_read(src, 24, 4, sink), "multiples of 16"),
-                       (lambda: gpu.enqueue_probe_read(src.ptr + 4, 64, 4, sink), "multiples of 16"),
-                       (lambda: gpu.enqueue_probe_read(src, 64, 0, sink), "workgroups")):
-        with pytest.raises(bm.GpuError) as e:
-            call()
-        assert e.value.code == bm.ESHAPE and word in str(e.value)
+    assert lib.bm_bench_probe_read(stream, src.ptr, 24, 4, sink.ptr) == -1
+    assert lib.bm_bench_probe_read(stream, src.ptr + 4, 64, 4, sink.ptr) == -1
+    assert lib.bm_bench_probe_read(stream, src.ptr, 64, 0, sink.ptr) == -1
     src.free()
     sink.free()
 

@@ -189,7 +189,6 @@ def test_layer_from_the_residual_row(gpu):
     ids, wts = gpu.buffer(np.uint32, m * top_k), gpu.buffer(np.float32, m * top_k)
     act_h, y = gpu.act(bm.Q6_K, ff, m * top_k), gpu.buffer(np.float32, m * hidden).fill_bytes(0xFF)
     gpu.fault_clear()
-    gpu.set_decode_plan(bm.PLAN_TWO_LAUNCHES)
     gpu.enqueue_router_logits(rd, xd, gd, 1e-6, m, n_experts, hidden, normed, logits)
     gpu.enqueue_route_softmax(logits, m, n_experts, top_k, True, None, ids, wts)
     gpu.enqueue_moe_decode(L.dg, L.du, L.dd, normed, ids, wts, xd, top_k, m, act_h, y)   # the residual: the input rows

@@ -96,7 +96,7 @@ def test_gate_rules_by_their_definitions():
     # rule 0 is swiglu; an unknown rule is refused
     assert ora.gate_rule(0, 5.0, g, u)[0].tobytes() == plain.tobytes()
     with pytest.raises(ValueError):
-        ora.gate_rule(3, 1.0, g, u)
+        ora.gate_rule(5, 1.0, g, u)
     # NaN through the comparisons: ik's clamp turns a NaN up into the limit and lets a NaN silu through; the other two
     # let a NaN up through (std::clamp); every clamping rule reports the block
     nan, inf = f(np.nan), f(np.inf)
@@ -114,6 +114,37 @@ def test_gate_rules_by_their_definitions():
         o, _ = ora.gate_rule(rule, 5.0, gg, uu)
         for i in (0, 7, 8, 332):
             assert ora.gate_rule(rule, 5.0, gg[i:i + 1], uu[i:i + 1])[0][0].tobytes() == o[i].tobytes()
+
+
+def test_situ_rule_against_its_closed_form():
+    """SiTU-GLU (rule 3) on the inputs and at the bound of the reference's own test (crates/model/src/ops.rs:7133-7153):
+    beta tanh(g / beta) sigmoid(g) * 25 tanh(u / 25) in f64, 1e-5 relative. The bound notices the mistakes a restatement
+    could make: the gate scaled by the up's beta, a missing sigmoid, the +1 of another rule, the betas swapped."""
+    f = np.float32
+    beta, lb, n = f(8.0), 25.0, 1024
+    i = np.arange(n)
+    g = ((i.astype(f) - f(512.0)) * f(0.07)).astype(f)
+    u = (((i * 37 % n).astype(f) - f(512.0)) * f(0.1)).astype(f)
+    out, ok = ora.gate_rule(3, beta, g, u)
+    g64, u64 = g.astype(np.float64), u.astype(np.float64)
+    want = 8.0 * np.tanh(g64 / 8.0) / (1.0 + np.exp(-g64)) * (lb * np.tanh(u64 / lb))
+    assert ok and np.all(np.abs(out - want) <= 1e-5 * np.abs(want) + 1e-30)
+    for wrong in (25.0 * np.tanh(g64 / 25.0) / (1.0 + np.exp(-g64)) * (lb * np.tanh(u64 / lb)),
+                  8.0 * np.tanh(g64 / 8.0) * (lb * np.tanh(u64 / lb)),
+                  lb * np.tanh(g64 / lb) / (1.0 + np.exp(-g64)) * (8.0 * np.tanh(u64 / 8.0))):
+        assert not np.all(np.abs(out - wrong) <= 1e-5 * np.abs(wrong) + 1e-30)
+    # op order at one value: scale by the f32 reciprocal, tanh, scale back, then (a * s) * v
+    e = ora.expf_ik(f(0.0) - f(1.5))
+    a = f(np.tanh(np.float64(f(f(1.5) * f(f(1.0) / beta)))))  # a correctly rounded tanh; libm's may sit an ulp away
+    sg = f(f(1.0) / f(f(1.0) + e))
+    v = f(np.tanh(np.float64(f(f(-3.0) * f(f(1.0) / f(25.0))))))
+    one, _ = ora.gate_rule(3, beta, np.array([1.5], f), np.array([-3.0], f))
+    want1 = f(f(f(a * beta) * sg) * f(v * f(25.0)))
+    assert abs(float(one[0]) - float(want1)) <= 4 * np.spacing(abs(want1))
+    # a value that is not finite is reported, as situ_into refuses it
+    for bad in (np.nan, np.inf, -np.inf):
+        assert not ora.gate_rule(3, beta, np.array([1.0, bad], f), np.array([1.0, 1.0], f))[1]
+        assert not ora.gate_rule(3, beta, np.array([1.0, 1.0], f), np.array([bad, 1.0], f))[1]
 
 
 # ------------------------------------------------------------------------------------------- router and combine

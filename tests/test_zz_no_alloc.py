@@ -21,7 +21,6 @@ def test_noalloc_matches_bm_moe_decode_on_two_calls_in_a_row(types, hidden, ff, 
     gpu = bm.Gpu(0)
     L = Layer(gpu, types, hidden, ff, n_experts, 4100 + hidden, cheap=True)
     rng = np.random.default_rng(4101)
-    gpu.set_decode_plan(bm.PLAN_TWO_LAUNCHES)
     for m in (5, 2):   # the second call is the smaller one
         x, resid = normal_f32(rng, (m, hidden)), normal_f32(rng, (m, hidden))
         ids, wts = route(rng, m, n_experts, top_k)

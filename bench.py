@@ -489,6 +489,77 @@ def bench_dsv3(args, bm, ora, threads):
     gpu.close()
 
 
+def bench_dsv3_prefill(args, bm, ora, threads):
+    """Config 7: the DeepSeek-V3-shaped routed experts at prefill, 2048 tokens: IQ2_XXS stacks on Q8_K columns through
+    bm_gemm, in both f32 summing modes. A side measurement: BASELINE.json holds no prefill figure for this shape."""
+    hidden, ff, n_experts, m = 7168, 2048, 256, 2048
+    rng = np.random.default_rng(0xB1000007)
+    t0 = time.time()
+    wg = random_blocks(rng, ora.IQ2_XXS, n_experts * ff, hidden, 66, 0)
+    wu = random_blocks(rng, ora.IQ2_XXS, n_experts * ff, hidden, 66, 0)
+    wd = random_blocks(rng, ora.IQ2_XXS, n_experts * hidden, ff, 66, 0)
+    log(f"[bench] stacks drawn ({(wg.nbytes * 2 + wd.nbytes) / 1e9:.2f} GB) in {time.time() - t0:.1f}s")
+    x = np.random.default_rng(0xAC70007).standard_normal((m, hidden), dtype=np.float32)
+    ids, wts = biased_routes(ora, m, n_experts, TOP_K, 0x707E0007, zipf=1.1)
+    n_slots = m * TOP_K
+    gpu = bm.Gpu(0)
+    dg, du, dd = (gpu.weights(bm.IQ2_XXS, n_experts * ff, hidden, wg), gpu.weights(bm.IQ2_XXS, n_experts * ff, hidden, wu),
+                  gpu.weights(bm.IQ2_XXS, n_experts * hidden, ff, wd))
+    xd, sel, wt = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32)
+    act, act_h = gpu.act(bm.IQ2_XXS, hidden, m), gpu.act(bm.IQ2_XXS, ff, n_slots)
+    g, u = gpu.buffer(np.float32, n_slots * ff), gpu.buffer(np.float32, n_slots * ff)
+    down, y = gpu.buffer(np.float32, n_slots * hidden), gpu.buffer(np.float32, m * hidden)
+    table = gpu.route(n_slots, n_experts)
+    names = ("quant", "route", "gate", "up", "swiglu_quant", "down", "combine")
+
+    def step(i, which=names):
+        if "quant" in which:
+            gpu.enqueue_quantize(xd, m, act)
+        if "route" in which:
+            table.fill(sel, n_slots)
+        if "gate" in which:
+            gpu.enqueue_gemm(dg, ff, act, table, TOP_K, g)
+        if "up" in which:
+            gpu.enqueue_gemm(du, ff, act, table, TOP_K, u)
+        if "swiglu_quant" in which:
+            gpu.enqueue_swiglu_quant(g, u, n_slots, act_h)
+        if "down" in which:
+            gpu.enqueue_gemm(dd, hidden, act_h, table, 0, down)
+        if "combine" in which:
+            gpu.enqueue_combine_tokens(down, wt, None, hidden, TOP_K, m, y)
+
+    n_chk = 2
+    types = (ora.IQ2_XXS, ora.IQ2_XXS, ora.IQ2_XXS)
+    want = ora.moe_forward(hidden, ff, n_experts, types, wg, wu, wd, x[:n_chk], ids[:n_chk], wts[:n_chk], TOP_K,
+                           n_threads=threads).reshape(n_chk, hidden)
+    ops = 2.0 * n_slots * 3 * ff * hidden
+    gate_ops = 2.0 * n_slots * ff * hidden
+    out = {}
+    for mode, code in (("fast", bm.GEMM_FAST), ("exact", bm.GEMM_EXACT)):
+        gpu.set_gemm_mode(code)
+        step(0)
+        parity = parity_of(y.download()[:n_chk * hidden].reshape(n_chk, hidden), want)
+        wall, ev, steps, warm = timed_graph(gpu, step, 1, 6, 2)
+        kernel_us = {k: timed_graph(gpu, lambda i, k=k: step(i, (k,)), 1, 4, 1)[1] * 1e3 for k in names}
+        out[mode] = {"ms_per_step": wall, "event_ms_per_step": ev, "steps": steps, "warmup": warm,
+                     "tops": ops / (wall * 1e-3) / 1e12, "frac_of_5.0_POPs": ops / (wall * 1e-3) / 5.0e15,
+                     "gate_gemm_tops": gate_ops / (kernel_us["gate"] * 1e-6) / 1e12,
+                     "gate_gemm_frac_of_5.0_POPs": gate_ops / (kernel_us["gate"] * 1e-6) / 5.0e15,
+                     "kernel_us": kernel_us, "parity": parity}
+        log(f"[bench] {mode}: {out[mode]}")
+    gpu.set_gemm_mode(bm.GEMM_EXACT)
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    f = out["fast"]
+    emit("moe_layer_prefill_int8_tops", f["tops"], "TOP/s", f["steps"], f["warmup"], f["ms_per_step"],
+         "DeepSeek-V3-shaped routed experts, prefill of 2048 tokens: hidden 7168, 256 IQ2_XXS experts of ff 2048 top-8, Zipf(1.1) "
+         "popularity, Q8_K columns; random legal blocks (a side measurement; the shape is BASELINE.json configs[4]'s)",
+         {"mode": "fast (BM_GEMM_FAST); `exact` beside it", "int8_ops_per_step": ops, "distinct_experts": int(len(np.unique(ids))),
+          "fast": f, "exact": out["exact"]},
+         {"bound": "mfma", "kernel": "k_gemm_iq2<fast> (gate)", "achieved": f["gate_gemm_tops"], "peak": 5000.0, "unit": "TOP/s",
+          "frac": f["gate_gemm_frac_of_5.0_POPs"], "traffic": None}, None, higher=True)
+    gpu.close()
+
+
 def bench_card(args, bm, ora, threads):
     """Config 6 (a side measurement, not a BASELINE.json line): the card rule. The MoE down step of the reference's GPU
     tier at the headline layer's down shape (8 slots of 768 values against 2048 Q4_K rows of 8 of 128 resident experts:
@@ -572,10 +643,11 @@ def bench_card(args, bm, ora, threads):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5, 6),
+    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5, 6, 7),
                     help="1: one Q4_K gemv; 2 (default, the headline): Qwen3-shaped layer, 1 token; 3: the same layer, 16 tokens "
                          "grouped by expert; 4: prefill of 2048 tokens (int8 MFMA GEMM); 5: DeepSeek-V3-shaped layer, 4 tokens; "
-                         "6: the card rule's down step (a side measurement)")
+                         "6: the card rule's down step (a side measurement); 7: DeepSeek-V3-shaped IQ2_XXS experts at prefill (a side "
+                         "measurement)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--traffic-probe", action="store_true",
                     help="config 2 only: no timing; 8 copies of 64 MiB by a plain kernel (the counters' calibration), then "
@@ -603,7 +675,7 @@ def main():
 
     threads = host_threads()
     if args.config != 2:
-        return {1: bench_gemv, 3: bench_grouped, 4: bench_prefill, 5: bench_dsv3, 6: bench_card}[args.config](args, bm, ora, threads)
+        return {1: bench_gemv, 3: bench_grouped, 4: bench_prefill, 5: bench_dsv3, 6: bench_card, 7: bench_dsv3_prefill}[args.config](args, bm, ora, threads)
     names = {"q3_k": bm.Q3_K, "q4_k": bm.Q4_K, "q5_k": bm.Q5_K, "q6_k": bm.Q6_K, "iq2_xxs": bm.IQ2_XXS,
              "iq3_xxs": bm.IQ3_XXS, "iq4_xs": bm.IQ4_XS}
     try:

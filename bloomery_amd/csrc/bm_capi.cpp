@@ -802,7 +802,7 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
     if (!ctx || !w || !act || !route || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
     if (!route->filled) return fail(ctx, BM_ESHAPE, "%s: a filled route table (bm_route_fill first)", what);
     if (!bmk::gemm_supported(w->wtype))
-        return fail(ctx, BM_ETYPE, "%s: weight type %d has no grouped GEMM here (Q4_K, Q5_K and Q6_K do); use the tile launchers", what, w->wtype);
+        return fail(ctx, BM_ETYPE, "%s: weight type %d has no grouped GEMM here (Q4_K, Q5_K, Q6_K and IQ2_XXS do); use the tile launchers", what, w->wtype);
     int rc = check_pair(ctx, what, w, act);
     if (rc) return rc;
     if (rows_per_expert <= 0 || rows_per_expert % 16 != 0)
@@ -877,13 +877,11 @@ int bm_set_gemm_mode(bm_ctx *ctx, int mode) {
 int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, const bm_gate_act *rule, bm_act *act) {
     const char *what = "bm_swiglu_quant";
     if (!ctx || !g_dev || !u_dev || !act) return fail(ctx, BM_EARG, "%s: NULL argument", what);
-    if (act_form(act->wtype) != 0)
-        return fail(ctx, BM_ETYPE, "%s: writes Q8_2_X4 columns; act was made for type %d (Q8_K)", what, act->wtype);
     if (n_cols < 1 || n_cols > act->m_cap)
         return fail(ctx, BM_ESHAPE, "%s: n_cols = %d columns, act holds %d", what, n_cols, act->m_cap);
     bmk::Launch L;
     if (int rc = launch_under(ctx, what, rule, &L)) return rc;
-    return driver(ctx, what, bmk::swiglu_quant(L, g_dev, u_dev, n_cols, act->k, act->dev));
+    return driver(ctx, what, bmk::swiglu_quant(L, g_dev, u_dev, n_cols, act->k, act->dev, act_form(act->wtype) != 0));
 }
 
 int bm_weights_from_gguf(bm_ctx *ctx, const bm_gguf *g, const char *name, bm_weights **out, int *rows_per_expert, int *n_experts) {

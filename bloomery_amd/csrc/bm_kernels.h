@@ -121,7 +121,8 @@ int gemm_max_tiles(int n_slots, int n_experts);
 // cols[n_slots], tiles[2 * gemm_max_tiles], n_tiles[2]
 hipError_t route(const Launch &L, const uint32_t *ids, int n_slots, int n_experts, uint32_t *cols, uint32_t *tiles,
                  uint32_t *n_tiles);
-hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act);
+// q8k: the columns are Q8_K ones (else Q8_2_X4)
+hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act, bool q8k);
 bool gemm_supported(int wtype);
 // slot_div: slots a token when every slot of a token reads the token's column, 1 when each slot reads its own.
 // mode 0: the CPU path's eight-accumulator f32 order (bit-identical to the row dots); 1: one accumulator a value.

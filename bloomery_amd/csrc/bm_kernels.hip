@@ -41,58 +41,10 @@ __global__ __launch_bounds__(256) void k_quantize_q82x4(const float *x, int m, i
 // x: m columns of k values -> Q8_K columns (crates/qdot/src/lib.rs:1787-1809). One workgroup a 256-value block.
 __global__ __launch_bounds__(256) void k_quantize_q8k(const float *x, int m, int k, uint8_t *act, const u32 *live,
                                                       u32 *fault, u32 layer) {
-    __shared__ unsigned long long s_key[4];
-    __shared__ int s_codes[256];
     const int bpc = k / 256;
-    const int col = blockIdx.x / bpc, blk = blockIdx.x % bpc, tid = threadIdx.x;
+    const int col = blockIdx.x / bpc, blk = blockIdx.x % bpc;
     if (live && (u32)col >= *live) return;
-    const float *xb = x + (size_t)col * k + 256 * blk;
-    uint8_t *o = act + ((size_t)col * bpc + blk) * BM_Q8K_STRIDE;
-    const float v = xb[tid];
-    // the largest magnitude, first on ties: maximise (|bits|, 255 - index)
-    unsigned long long key = ((unsigned long long)(bm_f32_bits(v) & 0x7fffffffu) << 32) | (u32)(255 - tid);
-#pragma unroll
-    for (int s = 32; s >= 1; s >>= 1) {
-        unsigned long long other = __shfl_xor(key, s, 64);
-        key = other > key ? other : key;
-    }
-    if ((tid & 63) == 0) s_key[tid >> 6] = key;
-    __syncthreads();
-    key = s_key[0];
-    for (int w = 1; w < 4; w++) key = s_key[w] > key ? s_key[w] : key;
-    const u32 ab = (u32)(key >> 32);
-    const int first = 255 - (int)(key & 0xffffffffu);
-    float d;
-    int code = 0;
-    if (ab > 0x7f7fffffu) {
-        if (tid == 0) bm_raise(fault, layer, kSiteQuantColumn);
-        d = bm_bits_f32(0x7fc00000u);
-    } else if (ab == 0) {
-        d = 0.0f;
-    } else {
-        const float max = xb[first];
-        const float iscale = __fdiv_rn(-127.0f, max);
-        int q = bm_nearest_int(__fmul_rn(iscale, v));
-        q = q > 127 ? 127 : q;
-        code = (int)(signed char)(q & 0xff); // `as i8`: the low byte
-        d = __fdiv_rn(1.0f, iscale);
-    }
-    s_codes[tid] = code;
-    __syncthreads();
-    if ((tid & 3) == 0) {
-        const u32 c = (u32)(s_codes[tid] & 0xff) | ((u32)(s_codes[tid + 1] & 0xff) << 8) |
-                      ((u32)(s_codes[tid + 2] & 0xff) << 16) | ((u32)(s_codes[tid + 3] & 0xff) << 24);
-        *reinterpret_cast<u32 *>(o + 8 + tid) = c;
-    }
-    if (tid < 16) {
-        int sum = 0;
-        for (int ii = 0; ii < 16; ii++) sum += s_codes[16 * tid + ii];
-        *reinterpret_cast<unsigned short *>(o + 264 + 2 * tid) = (unsigned short)(short)sum;
-    }
-    if (tid == 0) {
-        *reinterpret_cast<float *>(o) = d;
-        *reinterpret_cast<u32 *>(o + 4) = 0u;
-    }
+    q8k_block_by_workgroup(x[(size_t)col * k + 256 * blk + threadIdx.x], act + ((size_t)col * bpc + blk) * BM_Q8K_STRIDE, fault, layer);
 }
 
 hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, uint8_t *act, const uint32_t *live) {

@@ -88,7 +88,24 @@ __global__ __launch_bounds__(256) void k_swiglu_quant(const float *g, const floa
     q82_store(act + (size_t)col * (k / 256) * BM_Q82_SB_EXT, k / 256, blk, lane32, code, hd, s16);
 }
 
-hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act) {
+// The same into Q8_K columns, for a down stack that dots against those (IQ2_XXS, ...): one workgroup a 256-value block.
+__global__ __launch_bounds__(256) void k_swiglu_quant_q8k(const float *g, const float *u, int m, int k, uint8_t *act,
+                                                          GateRule rule, u32 *fault, u32 layer) {
+    const int bpc = k / 256;
+    const int col = blockIdx.x / bpc, blk = blockIdx.x % bpc;
+    const size_t at = (size_t)col * k + 256 * blk + threadIdx.x;
+    bool odd;
+    const float v = bm_gate_rule(rule.act, rule.limit, g[at], u[at], odd);
+    if (odd) bm_raise(fault, layer, kSiteF32Product);
+    q8k_block_by_workgroup(v, act + ((size_t)col * bpc + blk) * BM_Q8K_STRIDE, fault, layer);
+}
+
+hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act, bool q8k) {
+    if (q8k) {
+        hipLaunchKernelGGL(k_swiglu_quant_q8k, dim3((unsigned)(m * (k / 256))), dim3(256), 0, L.stream, g, u, m, k, act, L.rule,
+                           L.fault, L.layer);
+        return hipGetLastError();
+    }
     const long blocks = (long)m * (k / 32);
     hipLaunchKernelGGL(k_swiglu_quant, dim3((unsigned)((blocks + 7) / 8)), dim3(256), 0, L.stream, g, u, m, k, act,
                        L.rule, L.fault, L.layer);
@@ -693,7 +710,271 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
     }
 }
 
-bool gemm_supported(int wtype) { return wtype == BM_Q4K || wtype == BM_Q5K || wtype == BM_Q6K; }
+// ------------------------------------------------------------------------------------- IQ2_XXS on Q8_K columns
+
+// The grouped GEMM for IQ2_XXS stacks (crates/gpu/src/gemm/kernels.rs:867 gemm_iq2xxs; the arithmetic is
+// crates/gpu/src/gemm/grouped.rs:33-58 with the CPU path's lanes, crates/qdot/src/lib.rs:8677-8724). A super-block of a
+// row against a super-block of a Q8_K column is, in the CPU path, eight accumulators: accumulator l first takes
+// (dmin dy) (2 s_l + 1) (bsum[2l] + bsum[2l + 1]), then (d dy) sumi[l] with
+//     sumi[l] = sum over the eight sub-blocks b of (2 s_b + 1) * sum over i < 4 of u[b][4l + i] a[b][4l + i],
+// u = +-grid + 43 the unsigned code byte. sumi[l] is a 32-term integer dot whose weight-side terms (2 s_b + 1) u are at most
+// 31 * 86 = 2666: too wide for an int8 operand, so each is split into two signed bytes, 256 h + lo with lo = the low byte
+// read as signed and h = (term + 128) >> 8 (0 .. 10), and the dot is two v_mfma_i32_32x32x32_i8 whose sums meet as
+// (H << 8) + L, exactly. The LDS copy of a row's (and a column's) super-block is laid out lane-major, [l][b][i], so a matrix
+// operand is 16 consecutive bytes. With EXACT the eight accumulators and their order are the CPU path's, bit for bit
+// (the value bm_gemv_sel gives); without it one accumulator takes d dy times the super-block's whole sum
+// sum_b (2 s_b + 1) sum_n (u - 43) a, the 43s taken out in integers through two more matrix instructions over the
+// column's 32-value sums (split into two bytes the same way): f32 rounding is the only difference.
+// A workgroup of four waves takes 64 rows and a tile's 64 slots, a wave 32 x 32 of them.
+constexpr int kIqRows = 64;
+constexpr int kIqStride = 256 + 16; // bytes a row's or a column's 256 codes take in LDS
+constexpr int kIqLine = 64 + 4;     // floats a line of the per-lane tables
+template <bool EXACT>
+__host__ __device__ constexpr size_t gemm_iq2_lds_bytes() {
+    return sizeof(GemmLds) + (size_t)tab_bytes<BM_IQ2XXS>() + 3 * (size_t)64 * kIqStride + 2 * 64 * sizeof(float) +
+           (EXACT ? 2 * 8 * kIqLine * sizeof(float) : 3 * 64 * 16);
+}
+
+// (2 s + 1) u for the four code bytes of `u`, each product split into the signed low byte (lo) and what is left over 256
+// (hi): 256 hi + lo is the product.
+__device__ __forceinline__ void iq2_planes(u32 u, u32 sc, u32 &hi, u32 &lo) {
+    const u32 even = __builtin_amdgcn_perm(0u, u, 0x0c020c00u), odd = __builtin_amdgcn_perm(0u, u, 0x0c030c01u);
+    const u32 pe = even * sc, po = odd * sc; // two 16-bit fields each, at most 2666
+    lo = __builtin_amdgcn_perm(po, pe, 0x06020400u);
+    hi = __builtin_amdgcn_perm(po + 0x00800080u, pe + 0x00800080u, 0x07030501u);
+}
+
+template <bool EXACT>
+__global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
+                                                     const u32 *tiles, const u32 *n_tiles, u32 n_slabs, u32 slot_div,
+                                                     u32 n_slots, float *y) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
+    const Iq2Tables tb = stage_tables<BM_IQ2XXS>(lds + sizeof(GemmLds));
+    uint8_t *a_codes = lds + sizeof(GemmLds) + tab_bytes<BM_IQ2XXS>();
+    uint8_t *w_hi = a_codes + 64 * kIqStride;
+    uint8_t *w_lo = w_hi + 64 * kIqStride;
+    float *dy_t = reinterpret_cast<float *>(w_lo + 64 * kIqStride); // [slot]
+    float *d_t = dy_t + 64;                                          // [row]
+    float *bs_t = d_t + 64;                                          // EXACT: [l][slot] the 32-value sums, as floats
+    float *sc_t = bs_t + 8 * kIqLine;                                // EXACT: [l][row] the scales 2 s + 1, as floats
+    uint8_t *x_sc = reinterpret_cast<uint8_t *>(d_t + 64);           // else: [row][16] the scales as bytes, zeros behind
+    uint8_t *x_bl = x_sc + 64 * 16;                                  // [slot][16] the sums' low bytes, zeros behind
+    uint8_t *x_bh = x_bl + 64 * 16;                                  // [slot][16] what is left of the sums over 256
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const u32 g = tile_of_block(blockIdx.x, n_slabs);
+    const int row0 = (int)slab_of_block(blockIdx.x, n_slabs) * kIqRows;
+    const u32 count = n_tiles[0];
+    if (g > count) return;
+    if (g == count) { // the refused slots' rows: NaN (crates/gpu/src/gemm/grouped.rs:2283-2287)
+        const u32 refused = n_tiles[1];
+        for (u32 i = tid; i < refused * kIqRows; i += 256) {
+            const u32 s = cols[n_slots - refused + i / kIqRows];
+            const int r = row0 + (int)(i % kIqRows);
+            if (r < rpe) y[(size_t)s * rpe + r] = bm_bits_f32(0x7fc00000u);
+        }
+        return;
+    }
+    const u32 e = tiles[2 * g], word = tiles[2 * g + 1];
+    const int start = (int)(word & 0xffffu), len = (int)(word >> 16);
+    if (tid < kGemmBN) {
+        const u32 s = cols[start + (tid < len ? tid : 0)];
+        tab->slot[tid] = s;
+        tab->col[tid] = s / slot_div;
+    }
+    __syncthreads();
+    const u32 row_bytes = (u32)nb * BM_IQ2XXS_BLOCK, col_bytes = (u32)nb * BM_Q8K_STRIDE;
+    // what this thread stages of every super-block:
+    //   four 16-byte pieces of column codes (column tid / 16 + 16 j, piece tid % 16 of the sixteen): values 16 (piece % 2) ..
+    //   of sub-block piece / 2, i.e. the four-value groups of lanes 4 (piece % 2) .. + 3, one word each;
+    //   threads below 64: column tid's scale and its sixteen 16-value sums;
+    //   two sub-blocks of a weight row (row tid / 4, sub-blocks 2 (tid % 4) and the one after), the first of the four
+    //   also the row's d
+    const int ac = tid >> 4, ap = tid & 15;
+    u32 src_a[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) src_a[j] = tab->col[ac + 16 * j] * col_bytes + 8u + 16u * (u32)ap;
+    const u32 src_c = tab->col[tid & 63] * col_bytes;
+    const int wr = tid >> 2, wq = tid & 3;
+    const uint8_t *we = w + (size_t)e * rpe * row_bytes;
+    const u32 src_w = (u32)(row0 + wr < rpe ? row0 + wr : rpe - 1) * row_bytes;
+    const int a_dst = ac * kIqStride + 32 * (4 * (ap & 1)) + 4 * (ap >> 1); // word k of a piece: + 32 k
+
+    auto stage = [&](int i) {
+        uint4 ra[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) __builtin_memcpy(&ra[j], act + (src_a[j] + (u32)i * BM_Q8K_STRIDE), 16);
+        const uint8_t *blk = we + (src_w + (u32)i * BM_IQ2XXS_BLOCK);
+        const uint4 rq = bm_ld16u(blk + 2 + 16 * wq);
+        const u32 rd = bm_ld2u(blk);
+        float cdy = 0.0f;
+        uint4 cb0 = make_uint4(0, 0, 0, 0), cb1 = cb0;
+        if (tid < 64) {
+            const uint8_t *cs = act + (src_c + (u32)i * BM_Q8K_STRIDE);
+            cdy = *reinterpret_cast<const float *>(cs);
+            __builtin_memcpy(&cb0, cs + 264, 16);
+            __builtin_memcpy(&cb1, cs + 280, 16);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint8_t *dst = a_codes + a_dst + 16 * j * kIqStride;
+            *reinterpret_cast<u32 *>(dst) = ra[j].x;
+            *reinterpret_cast<u32 *>(dst + 32) = ra[j].y;
+            *reinterpret_cast<u32 *>(dst + 64) = ra[j].z;
+            *reinterpret_cast<u32 *>(dst + 96) = ra[j].w;
+        }
+        if (tid < 64) {
+            dy_t[tid] = cdy;
+            const u32 bw[8] = {cb0.x, cb0.y, cb0.z, cb0.w, cb1.x, cb1.y, cb1.z, cb1.w};
+            u32 bl[2] = {0, 0}, bh[2] = {0, 0};
+#pragma unroll
+            for (int l = 0; l < 8; l++) { // the two 16-value sums of sub-block l
+                const int bs = (int)(short)(bw[l] & 0xffffu) + (int)(short)(bw[l] >> 16);
+                if constexpr (EXACT) {
+                    bs_t[l * kIqLine + tid] = (float)bs;
+                } else { // 256 hi + lo with lo the low byte read as signed
+                    bl[l >> 2] |= ((u32)bs & 0xffu) << (8 * (l & 3));
+                    bh[l >> 2] |= ((u32)((bs + 128) >> 8) & 0xffu) << (8 * (l & 3));
+                }
+            }
+            if constexpr (!EXACT) {
+                *reinterpret_cast<uint4 *>(x_bl + 16 * tid) = make_uint4(bl[0], bl[1], 0u, 0u);
+                *reinterpret_cast<uint4 *>(x_bh + 16 * tid) = make_uint4(bh[0], bh[1], 0u, 0u);
+            }
+        }
+        if (wq == 0) d_t[wr] = 0.125f * bm_half_to_f32((unsigned short)rd);
+        u32 scs[2];
+#pragma unroll
+        for (int e2 = 0; e2 < 2; e2++) {
+            const int b = 2 * wq + e2;
+            const u32 idx = e2 ? rq.z : rq.x, aux = e2 ? rq.w : rq.y;
+            const u32 sc = 2u * (aux >> 28) + 1u;
+            scs[e2] = sc;
+            if constexpr (EXACT) sc_t[b * kIqLine + wr] = (float)sc;
+#pragma unroll
+            for (int q = 0; q < 4; q++) { // values 8 q .. 8 q + 7: lanes 2 q and 2 q + 1
+                const uint4 gp = tb.grid[(idx >> (8 * q)) & 0xffu];
+                const uint2 sg = tb.signs[(aux >> (7 * q)) & 127u];
+                u32 h0, l0, h1, l1;
+                iq2_planes(gp.x - (gp.z & sg.x), sc, h0, l0);
+                iq2_planes(gp.y - (gp.w & sg.y), sc, h1, l1);
+                const int at = wr * kIqStride + 32 * (2 * q) + 4 * b;
+                *reinterpret_cast<u32 *>(w_hi + at) = h0;
+                *reinterpret_cast<u32 *>(w_lo + at) = l0;
+                *reinterpret_cast<u32 *>(w_hi + at + 32) = h1;
+                *reinterpret_cast<u32 *>(w_lo + at + 32) = l1;
+            }
+        }
+        if constexpr (!EXACT) { // the row's eight scales as bytes: the thread of sub-blocks 2 wq, 2 wq + 1 writes its two
+            *reinterpret_cast<unsigned short *>(x_sc + 16 * wr + 2 * wq) = (unsigned short)(scs[0] | (scs[1] << 8));
+            if (wq == 0) *reinterpret_cast<uint2 *>(x_sc + 16 * wr + 8) = make_uint2(0u, 0u);
+        }
+    };
+
+    // this lane in its wave's 32 x 32 product: operand row / slot lane % 32, terms 16 (lane / 32) .. of the 32; result v
+    // is row 8 (v / 4) + 4 (lane / 32) + v % 4 of slot lane % 32
+    const int l32 = lane & 31, kh = lane >> 5;
+    const int wrow = 32 * (wv & 1), wslot = 32 * (wv >> 1);
+    const uint8_t *my_h = w_hi + (wrow + l32) * kIqStride + 16 * kh;
+    const uint8_t *my_l = w_lo + (wrow + l32) * kIqStride + 16 * kh;
+    const uint8_t *my_a = a_codes + (wslot + l32) * kIqStride + 16 * kh;
+    const bool live = wslot < len; // else none of this wave's slots is real
+    const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    constexpr int kAcc = EXACT ? 8 : 1;
+    v16f acc[kAcc];
+#pragma unroll
+    for (int l = 0; l < kAcc; l++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[l][v] = 0.0f;
+
+    for (int i = 0; i < nb; i++) {
+        if (i) __syncthreads(); // the readers of the super-block before are done
+        stage(i);
+        __syncthreads();
+        if (!live) continue;
+        const float dy = dy_t[wslot + l32];
+        float dd[16];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            const float4 d4 = *reinterpret_cast<const float4 *>(d_t + wrow + 8 * q4 + 4 * kh);
+            dd[4 * q4 + 0] = d4.x;
+            dd[4 * q4 + 1] = d4.y;
+            dd[4 * q4 + 2] = d4.z;
+            dd[4 * q4 + 3] = d4.w;
+        }
+        if constexpr (EXACT) {
+            // the fold of the 43s first: accumulator l takes sub-block l's scale on its two sums
+            // (crates/qdot/src/lib.rs:8691-8694); the product of the two small integers is exact in f32
+#pragma unroll
+            for (int l = 0; l < 8; l++) {
+                const float bs = bs_t[l * kIqLine + wslot + l32];
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const float4 s4 = *reinterpret_cast<const float4 *>(sc_t + l * kIqLine + wrow + 8 * q4 + 4 * kh);
+                    const float sv[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        const float dmin = -dd[4 * q4 + k] * 43.0f;
+                        acc[l][4 * q4 + k] = fmaf(dmin * dy, sv[k] * bs, acc[l][4 * q4 + k]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int l = 0; l < 8; l++) {
+                const v4i b = *reinterpret_cast<const v4i *>(my_a + 32 * l);
+                const v16i hs = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i *>(my_h + 32 * l), b, z, 0, 0, 0);
+                const v16i ls = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i *>(my_l + 32 * l), b, z, 0, 0, 0);
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[l][v] = fmaf(dd[v] * dy, (float)((hs[v] << 8) + ls[v]), acc[l][v]);
+            }
+        } else {
+            v16i hs = z, ls = z;
+#pragma unroll
+            for (int l = 0; l < 8; l++) {
+                const v4i b = *reinterpret_cast<const v4i *>(my_a + 32 * l);
+                hs = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i *>(my_h + 32 * l), b, hs, 0, 0, 0);
+                ls = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i *>(my_l + 32 * l), b, ls, 0, 0, 0);
+            }
+            // sum_b (2 s_b + 1) (the sub-block's sum of a): the scales against the sums' two bytes, terms 8 .. 31 zero
+            const v4i zero4 = {0, 0, 0, 0};
+            const v4i xs = kh ? zero4 : *reinterpret_cast<const v4i *>(x_sc + 16 * (wrow + l32));
+            const v4i xl = kh ? zero4 : *reinterpret_cast<const v4i *>(x_bl + 16 * (wslot + l32));
+            const v4i xh = kh ? zero4 : *reinterpret_cast<const v4i *>(x_bh + 16 * (wslot + l32));
+            const v16i ml = __builtin_amdgcn_mfma_i32_32x32x32_i8(xs, xl, z, 0, 0, 0);
+            const v16i mh = __builtin_amdgcn_mfma_i32_32x32x32_i8(xs, xh, z, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int total = ((hs[v] << 8) + ls[v]) - 43 * ((mh[v] << 8) + ml[v]);
+                acc[0][v] = fmaf(dd[v] * dy, (float)total, acc[0][v]);
+            }
+        }
+    }
+    const int n = wslot + l32;
+    if (live && n < len) {
+        float *out = y + (size_t)tab->slot[n] * rpe + row0 + wrow + 4 * kh;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            // rows_per_expert is a multiple of 16 and these four rows start at a multiple of 4: all inside or all outside
+            if (row0 + wrow + 4 * kh + 8 * q4 < rpe) {
+                float r[4];
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const int v = 4 * q4 + k;
+                    if constexpr (EXACT) { // the closing sum of the eight lanes (crates/qdot/src/lib.rs:4128 hsum_float_8's order)
+                        const float t0 = acc[0][v] + acc[4][v], t1 = acc[1][v] + acc[5][v];
+                        const float t2 = acc[2][v] + acc[6][v], t3 = acc[3][v] + acc[7][v];
+                        r[k] = (t0 + t2) + (t1 + t3);
+                    } else {
+                        r[k] = acc[0][v];
+                    }
+                }
+                *reinterpret_cast<float4 *>(out + 8 * q4) = make_float4(r[0], r[1], r[2], r[3]);
+            }
+        }
+    }
+}
+
+bool gemm_supported(int wtype) { return wtype == BM_Q4K || wtype == BM_Q5K || wtype == BM_Q6K || wtype == BM_IQ2XXS; }
 
 hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int rows_per_expert, int k,
                 const uint8_t *act, const uint32_t *cols, const uint32_t *tiles_dev, const uint32_t *n_tiles, int n_slots,
@@ -711,6 +992,19 @@ hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int
                            n_units, (u32)slot_div, (u32)n_slots, y);
         return hipGetLastError();
     };
+    if (wtype == BM_IQ2XXS) {
+        auto launch_iq = [&](auto kern, size_t lds) {
+            hipError_t e = allow_lds(kern, lds);
+            if (e != hipSuccess) return e;
+            const u32 n_slabs_q = (u32)((rows_per_expert + kIqRows - 1) / kIqRows);
+            const unsigned grid = ((max_tiles + 7) / 8) * 8 * n_slabs_q;
+            hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev, n_tiles,
+                               n_slabs_q, (u32)slot_div, (u32)n_slots, y);
+            return hipGetLastError();
+        };
+        if (mode == 1) return launch_iq(k_gemm_iq2<false>, gemm_iq2_lds_bytes<false>());
+        return launch_iq(k_gemm_iq2<true>, gemm_iq2_lds_bytes<true>());
+    }
     if (mode == 1) {
         auto launch_fast = [&](auto kern, size_t lds) {
             hipError_t e = allow_lds(kern, lds);

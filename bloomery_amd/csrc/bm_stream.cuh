@@ -477,6 +477,61 @@ constexpr int kRingQ4K = 4, kRingQ5K = 4, kRingQ6K = 3;
         return hipErrorInvalidValue;                                                                                   \
     }
 
+// One 256-value block of a Q8_K column by a workgroup of 256 threads, thread t holding value t (crates/qdot/src/lib.rs:
+// 1787-1809): the scale from the largest magnitude, the first on ties; codes nearest(iscale v) capped at 127; the sixteen
+// 16-value sums. `o`: the block's 296 bytes.
+__device__ __forceinline__ void q8k_block_by_workgroup(float v, uint8_t *o, u32 *fault, u32 layer) {
+    __shared__ unsigned long long s_key[4];
+    __shared__ int s_codes[256];
+    __shared__ float s_vals[256];
+    const int tid = threadIdx.x;
+    s_vals[tid] = v;
+    // the largest magnitude, first on ties: maximise (|bits|, 255 - index)
+    unsigned long long key = ((unsigned long long)(bm_f32_bits(v) & 0x7fffffffu) << 32) | (u32)(255 - tid);
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) {
+        unsigned long long other = __shfl_xor(key, s, 64);
+        key = other > key ? other : key;
+    }
+    if ((tid & 63) == 0) s_key[tid >> 6] = key;
+    __syncthreads();
+    key = s_key[0];
+    for (int w = 1; w < 4; w++) key = s_key[w] > key ? s_key[w] : key;
+    const u32 ab = (u32)(key >> 32);
+    const int first = 255 - (int)(key & 0xffffffffu);
+    float d;
+    int code = 0;
+    if (ab > 0x7f7fffffu) {
+        if (tid == 0) bm_raise(fault, layer, kSiteQuantColumn);
+        d = bm_bits_f32(0x7fc00000u);
+    } else if (ab == 0) {
+        d = 0.0f;
+    } else {
+        const float max = s_vals[first];
+        const float iscale = __fdiv_rn(-127.0f, max);
+        int q = bm_nearest_int(__fmul_rn(iscale, v));
+        q = q > 127 ? 127 : q;
+        code = (int)(signed char)(q & 0xff); // `as i8`: the low byte
+        d = __fdiv_rn(1.0f, iscale);
+    }
+    s_codes[tid] = code;
+    __syncthreads();
+    if ((tid & 3) == 0) {
+        const u32 c = (u32)(s_codes[tid] & 0xff) | ((u32)(s_codes[tid + 1] & 0xff) << 8) |
+                      ((u32)(s_codes[tid + 2] & 0xff) << 16) | ((u32)(s_codes[tid + 3] & 0xff) << 24);
+        *reinterpret_cast<u32 *>(o + 8 + tid) = c;
+    }
+    if (tid < 16) {
+        int sum = 0;
+        for (int ii = 0; ii < 16; ii++) sum += s_codes[16 * tid + ii];
+        *reinterpret_cast<unsigned short *>(o + 264 + 2 * tid) = (unsigned short)(short)sum;
+    }
+    if (tid == 0) {
+        *reinterpret_cast<float *>(o) = d;
+        *reinterpret_cast<u32 *>(o + 4) = 0u;
+    }
+}
+
 static inline int tab_bytes_rt(int wtype) { return wtype == BM_IQ2XXS ? kTabBytes : wtype == BM_IQ3XXS ? kTabBytes3 : 0; }
 
 } // namespace bmk

@@ -307,7 +307,8 @@ int bm_route_fill(bm_ctx *ctx, const uint32_t *ids_dev, int n_slots, bm_route *r
  * takes the n_slots slot list (refused slots last); tiles_host (optional) two words a tile: expert, then
  * first index | length << 16. */
 int bm_route_read(bm_ctx *ctx, const bm_route *route, uint32_t *cols_host, uint32_t *tiles_host, int *n_tiles, int *n_refused);
-/* GemmKernels::enqueue_gemm(GemmArgs) (crates/gpu/src/gemm/grouped.rs:2125-2133,2300), Q4_K, Q5_K and Q6_K stacks:
+/* GemmKernels::enqueue_gemm(GemmArgs) (crates/gpu/src/gemm/grouped.rs:2125-2133,2300), Q4_K, Q5_K and Q6_K stacks against
+ * Q8_2_X4 columns and IQ2_XXS stacks (crates/gpu/src/gemm/kernels.rs:867 gemm_iq2xxs) against Q8_K columns:
  * y_dev[s * rows_per_expert + r] = row r of expert e(s) . column c(s) of act for every slot s of the table's last
  * fill; c(s) = s / top_k (GemmInput::Shared) or s when top_k is 0 (GemmInput::PerSlot). rows_per_expert a
  * multiple of 16. Every value is bm_gemv_sel's for that slot, bit for bit; the integer sums are formed on the int8
@@ -317,14 +318,14 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
 /* How bm_gemm sums in f32 (the integer block sums are exact either way):
  *   BM_GEMM_EXACT (default): the CPU path's eight accumulators and closing order; bit-identical to bm_gemv_sel;
  *   BM_GEMM_FAST: one accumulator a value, blocks in increasing k; differs from the exact value by f32 rounding
- *     only (observed below 1e-6 of the row's largest magnitude; the contract's tolerance is 1e-4), about 1.4x the
- *     speed. No counterpart in the reference, whose grouped GEMM has one order (gemm/grouped.rs:33-58). */
+ *     only (observed below 1e-6 of the row's largest magnitude; the contract's tolerance is 1e-4), about 1.6x the
+ *     speed of a Q4_K / Q6_K layer step. No counterpart in the reference, whose grouped GEMM has one order (gemm/grouped.rs:33-58). */
 #define BM_GEMM_EXACT 0
 #define BM_GEMM_FAST 1
 int bm_set_gemm_mode(bm_ctx *ctx, int mode);
 /* GemmKernels::enqueue_swiglu_quant (crates/gpu/src/gemm/swiglu.rs:46): column c of act = the quantized
  * silu(g) * u of g_dev / u_dev[c * k .. (c + 1) * k), k = act's k, slot-major as the gate and up GEMMs write them;
- * bm_quantize's bytes of the CPU path's SwiGLU. Q8_2_X4 columns only. */
+ * bm_quantize's bytes of the CPU path's SwiGLU, in the column form of act's type (Q8_2_X4 or Q8_K). */
 int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, const bm_gate_act *rule, bm_act *act);
 
 

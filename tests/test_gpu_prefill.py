@@ -69,7 +69,7 @@ def test_gemm_fast_mode_is_within_the_tolerance(gpu):
     from common import max_abs_normalised
     rng = np.random.default_rng(2200)
     worst = 0.0
-    for wtype, k, rpe in ((bm.Q4_K, 2048, 768), (bm.Q6_K, 768, 2048), (bm.Q5_K, 1024, 80)):
+    for wtype, k, rpe in ((bm.Q4_K, 2048, 768), (bm.Q6_K, 768, 2048), (bm.Q5_K, 1024, 80), (bm.IQ2_XXS, 1792, 208)):
         n_experts, n_slots = 6, 150
         w = stack(wtype, n_experts * rpe, k, 2201)
         ids = rng.integers(0, n_experts, n_slots).astype(np.uint32)
@@ -103,6 +103,9 @@ def test_gemm_fast_mode_is_within_the_tolerance(gpu):
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 16, 48, 8, True),     # config 4's layer shape, 384 slots
     ((bm.Q6_K, bm.Q6_K, bm.Q4_K), 768, 512, 3, 9, 2, False),       # the other type on each side; ragged tiles
     ((bm.Q5_K, bm.Q5_K, bm.Q5_K), 768, 512, 3, 40, 2, False),      # Q5_K on both sides: the Q4_K walk with a fifth bit
+    ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ2_XXS), 1024, 512, 5, 60, 3, False),  # Q8_K columns on both sides; runs past one 32-slot half
+    ((bm.IQ2_XXS, bm.IQ2_XXS, bm.Q6_K), 768, 256, 3, 11, 2, False),      # the two column forms in one layer
+    ((bm.Q4_K, bm.Q4_K, bm.IQ2_XXS), 512, 768, 4, 30, 4, False),
 ))
 def test_prefill_layer_matches_the_oracle(gpu, types, hidden, ff, n_experts, m, top_k, cheap):
     L = Layer(gpu, types, hidden, ff, n_experts, 2000 + hidden, cheap=cheap)
@@ -128,7 +131,7 @@ def test_prefill_layer_matches_the_oracle(gpu, types, hidden, ff, n_experts, m, 
 def test_gemm_rows_not_a_whole_slab_and_refused_slots(gpu):
     """rows_per_expert = 80 (a multiple of 16, a slab and a quarter); a refused id gets NaN rows and ExpertId."""
     rng = np.random.default_rng(2100)
-    for wtype, k in ((bm.Q4_K, 1024), (bm.Q5_K, 512), (bm.Q6_K, 768)):
+    for wtype, k in ((bm.Q4_K, 1024), (bm.Q5_K, 512), (bm.Q6_K, 768), (bm.IQ2_XXS, 768)):
         rpe, n_experts, n_slots = 80, 4, 23
         w = stack(wtype, n_experts * rpe, k, 2101)
         ids = rng.integers(0, n_experts, n_slots).astype(np.uint32)
@@ -162,8 +165,8 @@ def test_gemm_rows_not_a_whole_slab_and_refused_slots(gpu):
 
 def test_prefill_refusals_are_named(gpu):
     w4 = gpu.weights(bm.Q4_K, 64, 512, np.zeros(64 * bm.row_bytes(bm.Q4_K, 512), np.uint8))
-    wi = gpu.weights(bm.IQ2_XXS, 64, 512, np.zeros(64 * bm.row_bytes(bm.IQ2_XXS, 512), np.uint8))
-    a512, aq8k = gpu.act(bm.Q4_K, 512, 8), gpu.act(bm.IQ2_XXS, 512, 8)
+    wi = gpu.weights(bm.IQ4_XS, 64, 512, np.zeros(64 * bm.row_bytes(bm.IQ4_XS, 512), np.uint8))
+    a512, aq8k = gpu.act(bm.Q4_K, 512, 8), gpu.act(bm.IQ4_XS, 512, 8)
     buf = gpu.buffer(np.float32, 4096)
     ids = gpu.upload(np.zeros(8, np.uint32))
     table = gpu.route(8, 2)
@@ -179,7 +182,6 @@ def test_prefill_refusals_are_named(gpu):
         (lambda: gpu.enqueue_gemm(w4, 32, a512, table, 3, buf), bm.ESHAPE, "whole tokens"),
         (lambda: gpu.enqueue_gemm(wi, 32, aq8k, table, 0, buf), bm.ETYPE, "bm_gemm"),
         (lambda: gpu.enqueue_swiglu_quant(buf, buf, 9, a512), bm.ESHAPE, "n_cols"),
-        (lambda: gpu.enqueue_swiglu_quant(buf, buf, 2, aq8k), bm.ETYPE, "Q8_2_X4"),
         (lambda: table.fill(ids, 9), bm.ESHAPE, "n_slots"),
         (lambda: gpu.route(50000, 2), bm.ESHAPE, "max_slots"),
         (lambda: gpu.route(8, 2000), bm.ESHAPE, "n_experts"),

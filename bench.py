@@ -816,14 +816,17 @@ def main():
     normed_d, logits_d = gpu.buffer(np.float32, HIDDEN), gpu.buffer(np.float32, N_EXPERTS)
     ids_d, wts_d = gpu.buffer(np.uint32, TOP_K), gpu.buffer(np.float32, TOP_K)
     router_us = {}
-    for name in ("router_logits", "route_softmax"):
+    for name in ("router_logits", "route_softmax", "norm_route_one_launch"):
         gpu.capture_begin()
         for i in range(unit):
             if name == "router_logits":
                 gpu.enqueue_router_logits(router_d, xd.ptr + 4 * (i % n_tok) * HIDDEN, gain_d, 1e-6, 1, N_EXPERTS, HIDDEN,
                                           normed_d, logits_d)
-            else:
+            elif name == "route_softmax":
                 gpu.enqueue_route_softmax(logits_d, 1, N_EXPERTS, TOP_K, True, None, ids_d, wts_d)
+            else:
+                gpu.enqueue_norm_route(router_d, xd.ptr + 4 * (i % n_tok) * HIDDEN, gain_d, 1e-6, 1, N_EXPERTS, HIDDEN, TOP_K,
+                                       True, normed_d, logits_d, None, ids_d, wts_d)
         g1 = gpu.capture_end()
         gpu.graph_launch(g1)
         gpu.sync()

@@ -84,6 +84,7 @@ SYMBOLS = {
     "bm_set_gate_rule": (_i, [_vp, _i, C.c_float]),
     "bm_route_softmax": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "bm_router_logits": (_i, [_vp, _vp, _vp, _vp, C.c_float, _i, _i, _i, _vp, _vp]),
+    "bm_norm_route": (_i, [_vp, _vp, _vp, _vp, C.c_float, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "bm_card_quantize": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp]),
     "bm_card_gemv": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp]),
     "bm_card_gemv_sel": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
@@ -568,6 +569,13 @@ class Gpu:
         """RouterKernels::enqueue_route (crates/gpu/src/route_softmax.rs:1643): softmax, top-k, renormalised weights."""
         self._check(self.lib.bm_route_softmax(self.ctx, _ptr(logits), n_tokens, n_experts, top_k, int(bool(renorm)),
                                               _ptr(probs) if probs is not None else None, _ptr(ids), _ptr(weights)))
+
+    def enqueue_norm_route(self, router, x, gain, eps, n_tokens, n_experts, hidden, top_k, renorm, normed, logits, probs, ids, weights):
+        """enqueue_router_logits and enqueue_route_softmax as one launch (bm_norm_route): the same bits in every output."""
+        self._check(self.lib.bm_norm_route(self.ctx, _ptr(router), _ptr(x), _ptr(gain) if gain is not None else None, float(eps),
+                                           n_tokens, n_experts, hidden, top_k, int(bool(renorm)),
+                                           _ptr(normed) if normed is not None else None, _ptr(logits),
+                                           _ptr(probs) if probs is not None else None, _ptr(ids), _ptr(weights)))
 
     def enqueue_router_logits(self, router, x, gain, eps, n_tokens, n_experts, hidden, normed, logits):
         """The FFN norm (gain None: none) and the router's f32 logits, the step before enqueue_route_softmax

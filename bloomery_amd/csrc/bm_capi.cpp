@@ -19,6 +19,7 @@ struct bm_ctx {
     bool own_stream = false;
     uint32_t *fault = nullptr;
     uint32_t layer = BM_LAYER_NONE;
+    uint32_t *route_counts = nullptr; // bm_norm_route's finished-workgroup counts, a word a token, zero between launches
     int gemm_mode = BM_GEMM_EXACT;
     bmk::GateRule rule = {0u, 0.0f}; // silu(g) * u
     std::string err;
@@ -112,9 +113,15 @@ static int ctx_make(int device, hipStream_t stream, bool own, bm_ctx **out) {
         e = hipMemset(c->fault, 0, sizeof(uint32_t) * BM_FAULT_WORDS);
         if (e == hipSuccess) e = hipMemset(c->fault, 0xff, sizeof(uint32_t));
     }
+    if (e == hipSuccess) {
+        const size_t cb = sizeof(uint32_t) * bmk::kNormRouteMaxTokens;
+        e = hipMalloc((void **)&c->route_counts, cb);
+        if (e == hipSuccess) e = hipMemset(c->route_counts, 0, cb);
+    }
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
         if (c->fault) (void)hipFree(c->fault);
+        if (c->route_counts) (void)hipFree(c->route_counts);
         if (c->own_stream) (void)hipStreamDestroy(c->stream);
         delete c;
         return fail(nullptr, BM_EDRIVER, "bm_ctx_create: fault word: %s", hipGetErrorString(e));
@@ -134,6 +141,7 @@ void bm_ctx_destroy(bm_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(ctx->fault);
+    (void)hipFree(ctx->route_counts);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -177,6 +185,8 @@ int bm_fault_clear(bm_ctx *ctx) {
     bmk::Launch L = launch_of(ctx);
     hipError_t e = bmk::fill_u32(L, ctx->fault + 1, 0u, BM_FAULT_WORDS - 1);
     if (e == hipSuccess) e = bmk::fill_u32(L, ctx->fault, BM_FAULT_NONE, 1);
+    // a launch that did not run to its end may have left its counts behind
+    if (e == hipSuccess) e = bmk::fill_u32(L, ctx->route_counts, 0u, bmk::kNormRouteMaxTokens);
     return driver(ctx, "bm_fault_clear", e);
 }
 
@@ -937,6 +947,30 @@ int bm_router_logits(bm_ctx *ctx, const float *router_dev, const float *x_dev, c
     if (gain_dev && !(eps >= 0.0f)) return fail(ctx, BM_EARG, "%s: eps = %g is negative or not a number", what, (double)eps);
     return driver(ctx, what, bmk::router_logits(launch_of(ctx), router_dev, x_dev, gain_dev, eps, n_tokens, n_experts, hidden, normed_dev,
                                                 logits_dev));
+}
+
+int bm_norm_route(bm_ctx *ctx, const float *router_dev, const float *x_dev, const float *gain_dev, float eps, int n_tokens,
+                  int n_experts, int hidden, int top_k, int renorm, float *normed_dev, float *logits_dev, float *probs_dev,
+                  uint32_t *ids_dev, float *weights_dev) {
+    const char *what = "bm_norm_route";
+    if (!ctx || !router_dev || !x_dev || !logits_dev || !ids_dev || !weights_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (n_tokens < 1 || n_tokens > bmk::kNormRouteMaxTokens)
+        return fail(ctx, BM_ESHAPE, "%s: n_tokens = %d, the fused launch takes 1 to %d (past that: bm_router_logits, then bm_route_softmax)",
+                    what, n_tokens, bmk::kNormRouteMaxTokens);
+    if (n_experts < 1 || n_experts > bmk::kRouteMaxExperts)
+        return fail(ctx, BM_ESHAPE, "%s: n_experts = %d, the router takes 1 to %d", what, n_experts, bmk::kRouteMaxExperts);
+    if (top_k < 1 || top_k > bmk::kRouteMaxPicks || top_k > n_experts)
+        return fail(ctx, BM_ESHAPE, "%s: top_k = %d of %d experts, the router picks 1 to %d", what, top_k, n_experts,
+                    bmk::kRouteMaxPicks);
+    if (hidden < 8 || hidden % 8 != 0)
+        return fail(ctx, BM_ESHAPE, "%s: hidden = %d is not a positive multiple of 8 (the f32 row dot's eight lanes)", what, hidden);
+    if (!bmk::router_logits_fits(hidden)) return fail(ctx, BM_ESHAPE, "%s: two rows of hidden = %d do not fit the workgroup's LDS", what, hidden);
+    if ((((uintptr_t)router_dev | (uintptr_t)x_dev | (uintptr_t)gain_dev | (uintptr_t)normed_dev) & 15) != 0)
+        return fail(ctx, BM_ESHAPE, "%s: router_dev %p, x_dev %p, gain_dev %p and normed_dev %p must be 16-byte aligned", what,
+                    (const void *)router_dev, (const void *)x_dev, (const void *)gain_dev, (const void *)normed_dev);
+    if (gain_dev && !(eps >= 0.0f)) return fail(ctx, BM_EARG, "%s: eps = %g is negative or not a number", what, (double)eps);
+    return driver(ctx, what, bmk::norm_route(launch_of(ctx), router_dev, x_dev, gain_dev, eps, n_tokens, n_experts, hidden, normed_dev,
+                                             logits_dev, top_k, renorm != 0, probs_dev, ids_dev, weights_dev, ctx->route_counts));
 }
 
 int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *act, int col, int32_t *out_dev) {

@@ -140,6 +140,12 @@ hipError_t route_softmax(const Launch &L, const float *logits, int n_tok, int n_
 // The FFN norm (gain NULL: none) and the router's f32 logits: router[n_exp * hidden], x[m * hidden], logits[m * n_exp],
 // normed_out (optional) [m * hidden]. hidden a multiple of 8.
 bool router_logits_fits(int hidden);
+// router_logits and route_softmax as one launch: the last of a token's workgroups to finish routes it. counts: a zeroed
+// word a token, left zeroed; launches that share them must not overlap.
+constexpr int kNormRouteMaxTokens = 4096;
+hipError_t norm_route(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
+                      int hidden, float *normed_out, float *logits, int used, int renorm, float *probs, uint32_t *ids,
+                      float *weights, uint32_t *counts);
 hipError_t router_logits(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                          int hidden, float *normed_out, float *logits);
 

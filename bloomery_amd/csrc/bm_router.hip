@@ -33,12 +33,11 @@ __device__ __forceinline__ void key_max(u32 &hi, u32 &lo, u32 ohi, u32 olo) {
     lo = take ? olo : lo;
 }
 
-// One wave a token; lane L owns experts L + 64 j, j < PER.
+// Token t's routing by one wave; lane L owns experts L + 64 j, j < PER.
 template <int PER>
-__global__ __launch_bounds__(256) void k_route_softmax(const float *logits, u32 n_tok, u32 n_exp, u32 used, u32 renorm,
-                                                       float *probs, u32 *ids, float *weights, u32 *fault, u32 layer) {
-    const u32 lane = threadIdx.x & 63, t = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (t >= n_tok) return; // whole waves leave
+__device__ __forceinline__ void route_softmax_wave(const float *logits, u32 t, u32 n_exp, u32 used, u32 renorm, float *probs,
+                                                   u32 *ids, float *weights, u32 *fault, u32 layer) {
+    const u32 lane = threadIdx.x & 63;
     const float *row = logits + (size_t)t * n_exp;
     float v[PER];
     bool odd = false;
@@ -113,6 +112,15 @@ __global__ __launch_bounds__(256) void k_route_softmax(const float *logits, u32 
     if (lane < used) weights[(size_t)t * used + lane] = renorm ? mine / (float)chosen : mine;
 }
 
+// One wave a token.
+template <int PER>
+__global__ __launch_bounds__(256) void k_route_softmax(const float *logits, u32 n_tok, u32 n_exp, u32 used, u32 renorm,
+                                                       float *probs, u32 *ids, float *weights, u32 *fault, u32 layer) {
+    const u32 t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= n_tok) return; // whole waves leave
+    route_softmax_wave<PER>(logits, t, n_exp, used, renorm, probs, ids, weights, fault, layer);
+}
+
 hipError_t route_softmax(const Launch &L, const float *logits, int n_tok, int n_exp, int used, int renorm, float *probs,
                          uint32_t *ids, float *weights) {
     const dim3 grid((unsigned)((n_tok + 3) / 4)), block(256);
@@ -142,9 +150,8 @@ hipError_t route_softmax(const Launch &L, const float *logits, int n_tok, int n_
 // A workgroup takes one token and R router rows: the token's row is normed into LDS by all 256 threads while the rows'
 // bytes arrive (both requested at once), then eight lanes a row walk it, lane l the accumulator l.
 template <int R>
-__global__ __launch_bounds__(256) void k_router_logits(const float *router, const float *x, const float *gain, float eps,
-                                                       int n_exp, int hidden, float *normed_out, float *logits) {
-    extern __shared__ __align__(16) uint8_t lds[];
+__device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *router, const float *x, const float *gain, float eps,
+                                                   int n_exp, int hidden, float *normed_out, float *logits) {
     float *xs = reinterpret_cast<float *>(lds);  // [hidden]
     float *ws = xs + hidden;                     // [R][hidden + 8]: rows eight banks apart, the R x 8 readers on 8 R banks
     __shared__ double s_part[4];
@@ -226,26 +233,64 @@ __global__ __launch_bounds__(256) void k_router_logits(const float *router, cons
     __syncthreads();
     if (!gain && normed_out && e0 == 0) // the rows as they are (read after the barrier: other threads staged them)
         for (int i = tid; i < hidden; i += 256) normed_out[(size_t)t * hidden + i] = xs[i];
-    if (tid >= 8 * R) return;
-    const int r = tid >> 3, l = tid & 7;
-    const float *wr = ws + (size_t)r * (hidden + 8);
-    float acc = __fmul_rn(xs[l], wr[l]);
-    // the chain is serial by the order's definition; the reads are not: sixteen steps' operands a batch
-    const int steps = hidden / 8;
-    int i = 1;
-    for (; i + 16 <= steps; i += 16) {
-        float a[16], b[16];
+    if (tid < 8 * R) {
+        const int r = tid >> 3, l = tid & 7;
+        const float *wr = ws + (size_t)r * (hidden + 8);
+        float acc = __fmul_rn(xs[l], wr[l]);
+        // the chain is serial by the order's definition; the reads are not: sixteen steps' operands a batch
+        // (reading the next batch under the present batch's chain measured slower: 8.1 us against 7.1 at 128 x 2048)
+        const int steps = hidden / 8;
+        int i = 1;
+        for (; i + 16 <= steps; i += 16) {
+            float a[16], b[16];
 #pragma unroll
-        for (int u = 0; u < 16; u++) a[u] = xs[8 * (i + u) + l], b[u] = wr[8 * (i + u) + l];
+            for (int u = 0; u < 16; u++) a[u] = xs[8 * (i + u) + l], b[u] = wr[8 * (i + u) + l];
 #pragma unroll
-        for (int u = 0; u < 16; u++) acc = fmaf(a[u], b[u], acc);
+            for (int u = 0; u < 16; u++) acc = fmaf(a[u], b[u], acc);
+        }
+        for (; i < steps; i++) acc = fmaf(xs[8 * i + l], wr[8 * i + l], acc);
+        // s_l = acc_l + acc_{l+4} on lanes 0..3 of the row's eight, then (s0 + s2) + (s1 + s3)
+        const float s = __fadd_rn(acc, __shfl_down(acc, 4, 8));
+        const float pair = __fadd_rn(s, __shfl_down(s, 2, 8)); // lane 0: s0 + s2, lane 1: s1 + s3
+        const float out = __fadd_rn(pair, __shfl_down(pair, 1, 8));
+        if (l == 0 && e0 + r < n_exp) logits[(size_t)t * n_exp + e0 + r] = out;
     }
-    for (; i < steps; i++) acc = fmaf(xs[8 * i + l], wr[8 * i + l], acc);
-    // s_l = acc_l + acc_{l+4} on lanes 0..3 of the row's eight, then (s0 + s2) + (s1 + s3)
-    const float s = __fadd_rn(acc, __shfl_down(acc, 4, 8));
-    const float pair = __fadd_rn(s, __shfl_down(s, 2, 8)); // lane 0: s0 + s2, lane 1: s1 + s3
-    const float out = __fadd_rn(pair, __shfl_down(pair, 1, 8));
-    if (l == 0 && e0 + r < n_exp) logits[(size_t)t * n_exp + e0 + r] = out;
+}
+
+template <int R>
+__global__ __launch_bounds__(256) void k_router_logits(const float *router, const float *x, const float *gain, float eps,
+                                                       int n_exp, int hidden, float *normed_out, float *logits) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    router_logits_body<R>(lds, router, x, gain, eps, n_exp, hidden, normed_out, logits);
+}
+
+// Norm, logits and routing in one launch (crates/gpu/src/route_softmax.rs:1667-1674 enqueue_norm_fused; the quantizer of
+// that launch is folded into the expert launches here). The workgroups are k_router_logits's; each, once its logits are
+// stored, adds one to the token's count with release at device scope, and the workgroup that brings the count to the number
+// of the token's workgroups - the last to finish, whichever it is - reads the token's logits back with acquire and routes
+// it with its first wave, k_route_softmax's numbers. No workgroup waits for another: every one runs to its end whatever the
+// order they are dispatched in. The last one leaves the count at zero for the next launch, so a graph replay needs no
+// memset. Launches over the same counts must not overlap.
+template <int R, int PER>
+__global__ __launch_bounds__(256) void k_norm_route(const float *router, const float *x, const float *gain, float eps, int n_exp,
+                                                    int hidden, float *normed_out, float *logits, u32 used, u32 renorm,
+                                                    float *probs, u32 *ids, float *weights, u32 *counts, u32 *fault,
+                                                    u32 layer) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    __shared__ u32 s_last;
+    router_logits_body<R>(lds, router, x, gain, eps, n_exp, hidden, normed_out, logits);
+    const u32 blocks_per_token = (u32)((n_exp + R - 1) / R);
+    const u32 t = blockIdx.x / blocks_per_token;
+    __syncthreads(); // the workgroup's stores are issued
+    if (threadIdx.x == 0) {
+        const u32 before = __hip_atomic_fetch_add(&counts[t], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = before == blocks_per_token - 1;
+        if (s_last) __hip_atomic_store(&counts[t], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last || threadIdx.x >= 64) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    route_softmax_wave<PER>(logits, t, (u32)n_exp, used, renorm, probs, ids, weights, fault, layer);
 }
 
 // Rows a workgroup takes: four where they fit the LDS beside the token's row, else two, else one.
@@ -275,6 +320,35 @@ hipError_t router_logits(const Launch &L, const float *router, const float *x, c
     else if (rows == 2) BM_RL(2)
     else BM_RL(1)
 #undef BM_RL
+    return hipGetLastError();
+}
+
+hipError_t norm_route(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
+                      int hidden, float *normed_out, float *logits, int used, int renorm, float *probs, uint32_t *ids,
+                      float *weights, uint32_t *counts) {
+    const int rows = router_rows(hidden);
+    if (rows == 0) return hipErrorInvalidValue;
+    const size_t lds = ((size_t)(rows + 1) * hidden + 8 * rows) * sizeof(float);
+    const unsigned grid = (unsigned)m * (unsigned)((n_exp + rows - 1) / rows);
+#define BM_NR(R, PER)                                                                                                  \
+    {                                                                                                                  \
+        auto kern = k_norm_route<R, PER>;                                                                              \
+        hipError_t e = allow_lds(kern, lds);                                                                           \
+        if (e != hipSuccess) return e;                                                                                 \
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, router, x, gain, eps, n_exp, hidden, normed_out, \
+                           logits, (u32)used, (u32)renorm, probs, ids, weights, counts, L.fault, L.layer);             \
+    }
+#define BM_NR_ROWS(PER)                                                                                                \
+    {                                                                                                                  \
+        if (rows == 4) BM_NR(4, PER)                                                                                   \
+        else if (rows == 2) BM_NR(2, PER)                                                                              \
+        else BM_NR(1, PER)                                                                                             \
+    }
+    if (n_exp <= 128) BM_NR_ROWS(2)
+    else if (n_exp <= 256) BM_NR_ROWS(4)
+    else BM_NR_ROWS(16)
+#undef BM_NR_ROWS
+#undef BM_NR
     return hipGetLastError();
 }
 

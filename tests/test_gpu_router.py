@@ -204,3 +204,94 @@ def test_layer_from_the_residual_row(gpu):
     for b in (rd, xd, gd, normed, logits, ids, wts, act_h, y):
         b.free()
     L.free()
+
+
+@pytest.mark.parametrize("n_experts,hidden,m,top_k,with_gain,seed", ((128, 2048, 5, 8, True, 21), (256, 7168, 3, 8, True, 22),
+                                                                      (10, 64, 70, 3, False, 23), (600, 256, 9, 6, True, 24),
+                                                                      (7, 16384, 2, 2, True, 25), (3, 64, 4096, 1, True, 26)))
+def test_norm_route_is_the_two_launches_in_one(gpu, n_experts, hidden, m, top_k, with_gain, seed):
+    """bm_norm_route against bm_router_logits followed by bm_route_softmax on the same inputs: every output the same bits
+    (normed rows, logits, probabilities, ids, weights), three launches in a row over the same counts and then a smaller
+    one, and under a graph replayed several times (the counts come back to zero without a memset)."""
+    rng = np.random.default_rng(seed)
+    router = normal_f32(rng, (n_experts, hidden), 0.05)
+    x = np.stack([normal_f32(rng, hidden) * np.float32(10.0 ** rng.uniform(-1, 1)) for _ in range(m)])
+    gain = (1.0 + normal_f32(rng, hidden, 0.2)).astype(np.float32) if with_gain else None
+    eps = 1e-6
+    rd, xd = gpu.upload(router, np.float32), gpu.upload(x, np.float32)
+    gd = gpu.upload(gain, np.float32) if with_gain else None
+    bufs = {}
+    for tag in ("two", "one"):
+        bufs[tag] = (gpu.buffer(np.float32, m * hidden), gpu.buffer(np.float32, m * n_experts), gpu.buffer(np.float32, m * n_experts),
+                     gpu.buffer(np.uint32, m * top_k), gpu.buffer(np.float32, m * top_k))
+    normed, logits, probs, ids, wts = bufs["two"]
+    gpu.fault_clear()
+    gpu.enqueue_router_logits(rd, xd, gd, eps, m, n_experts, hidden, normed, logits)
+    gpu.enqueue_route_softmax(logits, m, n_experts, top_k, True, probs, ids, wts)
+    want = [b.download() for b in bufs["two"]]
+    normed, logits, probs, ids, wts = bufs["one"]
+
+    def fused(tokens):
+        gpu.enqueue_norm_route(rd, xd, gd, eps, tokens, n_experts, hidden, top_k, True, normed, logits, probs, ids, wts)
+
+    def check(tokens, what):
+        for b, w, per, name in zip(bufs["one"], want, (hidden, n_experts, n_experts, top_k, top_k),
+                                   ("normed", "logits", "probs", "ids", "weights")):
+            got = b.download()
+            assert np.array_equal(got[:tokens * per].view(np.uint32), w[:tokens * per].view(np.uint32)), f"{what}: {name}"
+
+    for rep in range(3):
+        for b in bufs["one"]:
+            b.fill_bytes(0xFF)
+        fused(m)
+        check(m, f"launch {rep}")
+    few = max(1, m // 2)
+    for b in bufs["one"]:
+        b.fill_bytes(0xFF)
+    fused(few)
+    check(few, "a smaller launch after a larger one")
+    gpu.capture_begin()
+    fused(m)
+    g = gpu.capture_end()
+    for rep in range(3):
+        for b in bufs["one"]:
+            b.fill_bytes(0xFF)
+        gpu.graph_launch(g)
+        gpu.sync()
+        check(m, f"replay {rep}")
+    gpu.graph_destroy(g)
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    for b in (rd, xd, gd) + bufs["two"] + bufs["one"]:
+        if b is not None:
+            b.free()
+
+
+def test_norm_route_raises_and_refuses_like_its_parts(gpu):
+    """A logit that is not finite (a NaN in the token's row) raises Router from the fused launch too, and the other
+    tokens are routed; the argument checks are the two entries' own, by name."""
+    n_experts, hidden, m, top_k = 16, 256, 3, 4
+    rng = np.random.default_rng(31)
+    router, x = normal_f32(rng, (n_experts, hidden), 0.05), normal_f32(rng, (m, hidden))
+    x[1, 7] = np.nan
+    rd, xd = gpu.upload(router, np.float32), gpu.upload(x, np.float32)
+    logits, ids, wts = gpu.buffer(np.float32, m * n_experts), gpu.buffer(np.uint32, m * top_k).fill_bytes(0), gpu.buffer(np.float32, m * top_k)
+    gpu.fault_clear()
+    gpu.set_layer(3)
+    gpu.enqueue_norm_route(rd, xd, None, 0.0, m, n_experts, hidden, top_k, True, None, logits, None, ids, wts)
+    assert gpu.fault(3) == ((3 << 8) | bm.SITE_ROUTER, 1 << bm.SITE_ROUTER)
+    got_w = wts.download().reshape(m, top_k)
+    assert np.isnan(got_w[1]).all() and np.isfinite(got_w[0]).all() and np.isfinite(got_w[2]).all()
+    _, want_l = ora.router_logits(router, x, None, 0.0)
+    for t in (0, 2):
+        want_ids, _ = ora.route_softmax_topk(want_l[t], top_k)
+        assert list(ids.download().reshape(m, top_k)[t]) == list(want_ids)
+    gpu.set_layer(bm.LAYER_NONE)
+    gpu.fault_clear()
+    for call, word in ((lambda: gpu.enqueue_norm_route(rd, xd, None, 0.0, 4097, n_experts, hidden, top_k, True, None, logits, None, ids, wts), "4096"),
+                       (lambda: gpu.enqueue_norm_route(rd, xd, None, 0.0, m, n_experts, hidden, 17, True, None, logits, None, ids, wts), "top_k"),
+                       (lambda: gpu.enqueue_norm_route(rd, xd, None, 0.0, m, n_experts, 12, top_k, True, None, logits, None, ids, wts), "multiple of 8")):
+        with pytest.raises(bm.GpuError) as e:
+            call()
+        assert e.value.code == bm.ESHAPE and word in str(e.value) and "bm_norm_route" in str(e.value)
+    for b in (rd, xd, logits, ids, wts):
+        b.free()

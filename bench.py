@@ -560,6 +560,57 @@ def bench_dsv3_prefill(args, bm, ora, threads):
     gpu.close()
 
 
+def bench_paths(args, bm, ora, threads):
+    """Config 8: bm_moe_forward's three paths over the number of tokens, on the headline layer with config 3's routing: the
+    crossovers behind its automatic choice. A side measurement."""
+    wg, wu, wd = make_layer(ora, 0xB1000001, threads)
+    counts = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256, 512, 1024)
+    m_max, sets = counts[-1], 4
+    x = np.random.default_rng(0xAC70001).standard_normal((m_max, HIDDEN), dtype=np.float32)
+    ids, wts = biased_routes(ora, m_max * sets, N_EXPERTS, TOP_K, 0x707E0001, bias_sigma=0.5)
+    gpu = bm.Gpu(0)
+    layers = [(gpu.weights(bm.Q4_K, N_EXPERTS * FF, HIDDEN, wg), gpu.weights(bm.Q4_K, N_EXPERTS * FF, HIDDEN, wu),
+               gpu.weights(bm.Q6_K, N_EXPERTS * HIDDEN, FF, wd)) for _ in range(args.layers)]
+    xd, sel, wt = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32)
+    y = gpu.buffer(np.float32, m_max * HIDDEN)
+    sc = gpu.scratch(bm.Q4_K, bm.Q6_K, HIDDEN, FF, N_EXPERTS, TOP_K, m_max)
+    want = ora.moe_forward(HIDDEN, FF, N_EXPERTS, (ora.Q4_K, ora.Q4_K, ora.Q6_K), wg, wu, wd, x[:4], ids[:4], wts[:4], TOP_K,
+                           n_threads=threads).reshape(4, HIDDEN)
+    rows = []
+    for m in counts:
+        row = {"tokens": m}
+        for name, path, mode in (("per_slot", bm.PATH_PER_SLOT, bm.GEMM_EXACT), ("grouped", bm.PATH_GROUPED, bm.GEMM_EXACT),
+                                 ("gemm_exact", bm.PATH_GEMM, bm.GEMM_EXACT), ("gemm_fast", bm.PATH_GEMM, bm.GEMM_FAST)):
+            sc.set_path(path)
+            gpu.set_gemm_mode(mode)
+
+            def step(i, m=m):
+                dg, du, dd = layers[i % len(layers)]
+                st = i % sets
+                gpu.enqueue_moe_forward(sc, dg, du, dd, xd, sel.ptr + 4 * st * m * TOP_K, wt.ptr + 4 * st * m * TOP_K, None, m, y)
+
+            step(0)
+            if m >= 4:
+                p = parity_of(y.download()[:4 * HIDDEN].reshape(4, HIDDEN), want)
+                assert p["max_abs_normalised_err"] <= 1e-4, (name, m, p)
+            unit = 16 if m <= 64 else 4
+            row[name] = timed_graph(gpu, step, unit, max(2 * unit, min(256, 8192 // m)), unit)[1] * 1e3
+        row["fastest_exact"] = min(("per_slot", "grouped", "gemm_exact"), key=lambda k: row[k])
+        rows.append(row)
+        log(f"[bench] {row}")
+    gpu.set_gemm_mode(bm.GEMM_EXACT)
+    sc.set_path(bm.PATH_AUTO)
+    auto = {m: {bm.PATH_PER_SLOT: "per_slot", bm.PATH_GROUPED: "grouped", bm.PATH_GEMM: "gemm_exact"}[sc.path_for(m)] for m in counts}
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    worst = max(r[auto[r["tokens"]]] / r[r["fastest_exact"]] for r in rows)
+    emit("moe_layer_us_per_step_by_path", rows[5]["per_slot"], "us/step", 0, 0, rows[5]["per_slot"] * 1e-3,
+         "Qwen3-30B-A3B-shaped MoE layer, 1 to 1024 tokens a step through each path of bm_moe_forward, config 3's routing "
+         "(a side measurement: which path for how many tokens)",
+         {"us_per_step": rows, "automatic_choice": auto, "automatic_over_fastest_worst_case": worst},
+         {"bound": "hbm", "kernel": "n/a", "achieved": None, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": None, "traffic": None}, None)
+    gpu.close()
+
+
 def bench_card(args, bm, ora, threads):
     """Config 6 (a side measurement, not a BASELINE.json line): the card rule. The MoE down step of the reference's GPU
     tier at the headline layer's down shape (8 slots of 768 values against 2048 Q4_K rows of 8 of 128 resident experts:
@@ -643,11 +694,11 @@ def bench_card(args, bm, ora, threads):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5, 6, 7),
+    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5, 6, 7, 8),
                     help="1: one Q4_K gemv; 2 (default, the headline): Qwen3-shaped layer, 1 token; 3: the same layer, 16 tokens "
                          "grouped by expert; 4: prefill of 2048 tokens (int8 MFMA GEMM); 5: DeepSeek-V3-shaped layer, 4 tokens; "
                          "6: the card rule's down step (a side measurement); 7: DeepSeek-V3-shaped IQ2_XXS experts at prefill (a side "
-                         "measurement)")
+                         "measurement); 8: the three paths of bm_moe_forward over the number of tokens (a side measurement)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--traffic-probe", action="store_true",
                     help="config 2 only: no timing; 8 copies of 64 MiB by a plain kernel (the counters' calibration), then "
@@ -675,7 +726,7 @@ def main():
 
     threads = host_threads()
     if args.config != 2:
-        return {1: bench_gemv, 3: bench_grouped, 4: bench_prefill, 5: bench_dsv3, 6: bench_card, 7: bench_dsv3_prefill}[args.config](args, bm, ora, threads)
+        return {1: bench_gemv, 3: bench_grouped, 4: bench_prefill, 5: bench_dsv3, 6: bench_card, 7: bench_dsv3_prefill, 8: bench_paths}[args.config](args, bm, ora, threads)
     names = {"q3_k": bm.Q3_K, "q4_k": bm.Q4_K, "q5_k": bm.Q5_K, "q6_k": bm.Q6_K, "iq2_xxs": bm.IQ2_XXS,
              "iq3_xxs": bm.IQ3_XXS, "iq4_xs": bm.IQ4_XS}
     try:

@@ -21,6 +21,7 @@ FAULT_NONE = 0xFFFFFFFF
 LAYER_NONE = 0xFFFF
 SITE_QUANT_COLUMN, SITE_ROUTER, SITE_EXPERT_ID = 1, 5, 7
 GEMM_EXACT, GEMM_FAST = 0, 1
+PATH_AUTO, PATH_PER_SLOT, PATH_GROUPED, PATH_GEMM = 0, 1, 2, 3
 ACT_SILU_MUL, ACT_SWIGLU_CLAMP, ACT_SWIGLU_OAI, ACT_SITU, ACT_SWIGLU_GCLAMP = 0, 1, 2, 3, 4
 SITE_F32_PRODUCT = 21
 HOST_SLOT = 0xFFFFFFFF
@@ -84,6 +85,11 @@ SYMBOLS = {
     "bm_set_gate_rule": (_i, [_vp, _i, C.c_float]),
     "bm_route_softmax": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "bm_router_logits": (_i, [_vp, _vp, _vp, _vp, C.c_float, _i, _i, _i, _vp, _vp]),
+    "bm_scratch_create": (_i, [_vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "bm_scratch_destroy": (None, [_vp]),
+    "bm_scratch_set_path": (_i, [_vp, _i, _i, _i]),
+    "bm_scratch_path_for": (_i, [_vp, _i]),
+    "bm_moe_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     "bm_norm_route": (_i, [_vp, _vp, _vp, _vp, C.c_float, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "bm_card_quantize": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp]),
     "bm_card_gemv": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp]),
@@ -366,6 +372,28 @@ def _rule(rule):
     return C.cast(C.pointer(GateAct(int(code), float(limit))), C.c_void_p)
 
 
+class Scratch:
+    """bm_scratch: what bm_moe_forward's three paths keep between their launches, for up to max_tokens tokens."""
+
+    def __init__(self, gpu, gate_type, down_type, hidden, ff, n_experts, n_slots_per_token, max_tokens):
+        self.gpu = gpu
+        h = _vp()
+        gpu._check(gpu.lib.bm_scratch_create(gpu.ctx, gate_type, down_type, hidden, ff, n_experts, n_slots_per_token, max_tokens,
+                                             C.byref(h)))
+        self.handle = h.value
+
+    def set_path(self, path, grouped_from=0, gemm_from=0):
+        self.gpu._check(self.gpu.lib.bm_scratch_set_path(self.handle, path, grouped_from, gemm_from))
+
+    def path_for(self, m):
+        return self.gpu.lib.bm_scratch_path_for(self.handle, m)
+
+    def free(self):
+        if self.handle:
+            self.gpu.lib.bm_scratch_destroy(self.handle)
+            self.handle = None
+
+
 class Gpu:
     """A device context: stream, fault word and the launchers (the reference's `Gpu` and its kernel structs)."""
 
@@ -569,6 +597,15 @@ class Gpu:
         """RouterKernels::enqueue_route (crates/gpu/src/route_softmax.rs:1643): softmax, top-k, renormalised weights."""
         self._check(self.lib.bm_route_softmax(self.ctx, _ptr(logits), n_tokens, n_experts, top_k, int(bool(renorm)),
                                               _ptr(probs) if probs is not None else None, _ptr(ids), _ptr(weights)))
+
+    def scratch(self, gate_type, down_type, hidden, ff, n_experts, n_slots_per_token, max_tokens):
+        return Scratch(self, gate_type, down_type, hidden, ff, n_experts, n_slots_per_token, max_tokens)
+
+    def enqueue_moe_forward(self, scratch, wg, wu, wd, x, sel, wts, resid, m, y, rule=None):
+        """The expert step for any number of tokens (bm_moe_forward): per slot, grouped by expert or the grouped GEMM,
+        by the number of tokens."""
+        self._check(self.lib.bm_moe_forward(self.ctx, scratch.handle, wg.handle, wu.handle, wd.handle, _ptr(x), _ptr(sel), _ptr(wts),
+                                            _ptr(resid), m, _rule(rule), _ptr(y)))
 
     def enqueue_norm_route(self, router, x, gain, eps, n_tokens, n_experts, hidden, top_k, renorm, normed, logits, probs, ids, weights):
         """enqueue_router_logits and enqueue_route_softmax as one launch (bm_norm_route): the same bits in every output."""

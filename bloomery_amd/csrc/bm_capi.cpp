@@ -839,6 +839,162 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
                                        route->tiles, route->n_tiles, n_slots, slot_div, y_dev, ctx->gemm_mode));
 }
 
+// ------------------------------------------------------------------------- one entry for every batch size
+
+struct bm_scratch {
+    bm_ctx *ctx;
+    int gate_type, down_type, hidden, ff, n_experts, spt, max_tokens;
+    bm_act *act_x, *act_h;
+    float *g, *u, *down;           // f32 rows: g (also the per-slot and grouped paths' h) and u of slots x ff, down of slots x hidden
+    uint32_t *order, *start, *tiles; // the grouped table
+    bm_route *route;               // the GEMM path's table
+    int path, grouped_from, gemm_from, gemm_from_fast;
+};
+
+void bm_scratch_destroy(bm_scratch *s) {
+    if (!s) return;
+    bm_act_destroy(s->act_x);
+    bm_act_destroy(s->act_h);
+    (void)hipFree(s->g);
+    (void)hipFree(s->u);
+    (void)hipFree(s->down);
+    (void)hipFree(s->order);
+    bm_route_destroy(s->route);
+    delete s;
+}
+
+int bm_scratch_create(bm_ctx *ctx, int gate_type, int down_type, int hidden, int ff, int n_experts, int n_slots_per_token,
+                      int max_tokens, bm_scratch **out) {
+    const char *what = "bm_scratch_create";
+    if (!ctx || !out) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    *out = nullptr;
+    if (!bmk::moe_decode_supported(gate_type, down_type))
+        return fail(ctx, BM_ETYPE, "%s: no kernels for gate/up type %d with down type %d", what, gate_type, down_type);
+    if (hidden < 256 || hidden % 256 != 0 || ff < 256 || ff % 256 != 0)
+        return fail(ctx, BM_ESHAPE, "%s: hidden = %d and ff = %d must be positive multiples of 256", what, hidden, ff);
+    if (n_experts < 1 || n_experts > bmk::kBucketExperts)
+        return fail(ctx, BM_ESHAPE, "%s: n_experts = %d outside 1..=%d", what, n_experts, bmk::kBucketExperts);
+    if (n_slots_per_token < 1 || n_slots_per_token > bmk::kMaxCombineSlots)
+        return fail(ctx, BM_ESHAPE, "%s: %d slots a token outside 1..=%d", what, n_slots_per_token, bmk::kMaxCombineSlots);
+    if (max_tokens < 1 || (int64_t)max_tokens * n_slots_per_token > bmk::kGemmMaxSlots)
+        return fail(ctx, BM_ESHAPE, "%s: max_tokens = %d at %d slots a token is outside 1..=%d slots", what, max_tokens,
+                    n_slots_per_token, bmk::kGemmMaxSlots);
+    bm_scratch *s = new (std::nothrow) bm_scratch{};
+    if (!s) return fail(ctx, BM_EDRIVER, "%s: out of host memory", what);
+    s->ctx = ctx;
+    s->gate_type = gate_type, s->down_type = down_type, s->hidden = hidden, s->ff = ff, s->n_experts = n_experts;
+    s->spt = n_slots_per_token, s->max_tokens = max_tokens;
+    // the crossovers measured on MI355X at the Qwen3-30B-A3B layer shape (Q4_K gate/up, Q6_K down, top-8 of 128):
+    // tokens   per slot   grouped   GEMM exact   GEMM tolerance mode   (us a step)
+    //     16       67        86        190          118
+    //     24       92        88        217          130
+    //    128      400       188        336          201
+    //    192      580       246        370          214
+    //    256      767       296        392          230
+    //    512     1491       534        481          289
+    s->path = BM_PATH_AUTO, s->grouped_from = 22, s->gemm_from = 448, s->gemm_from_fast = 160;
+    const size_t slots = (size_t)max_tokens * n_slots_per_token;
+    int rc = bm_act_create(ctx, gate_type, hidden, max_tokens, &s->act_x);
+    if (!rc) rc = bm_act_create(ctx, down_type, ff, (int)slots, &s->act_h);
+    if (!rc) rc = bm_route_create(ctx, (int)slots, n_experts, &s->route);
+    if (!rc) {
+        (void)hipSetDevice(ctx->device);
+        const size_t table = slots + (size_t)n_experts + 1 + (size_t)bmk::tile_cap((int)slots, n_experts) + 1;
+        hipError_t e = hipMalloc((void **)&s->g, slots * ff * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc((void **)&s->u, slots * ff * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc((void **)&s->down, slots * hidden * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc((void **)&s->order, table * sizeof(uint32_t));
+        if (e == hipSuccess) e = hipMemset(s->order, 0, table * sizeof(uint32_t));
+        if (e == hipSuccess) e = hipDeviceSynchronize();
+        if (e != hipSuccess) rc = fail(ctx, BM_EDRIVER, "%s: %zu slots of scratch: %s", what, slots, hipGetErrorString(e));
+        s->start = s->order + slots;
+        s->tiles = s->start + n_experts + 1;
+    }
+    if (rc) {
+        const std::string keep = ctx->err;
+        bm_scratch_destroy(s);
+        ctx->err = keep;
+        return rc;
+    }
+    *out = s;
+    return BM_OK;
+}
+
+int bm_scratch_set_path(bm_scratch *s, int path, int grouped_from, int gemm_from) {
+    const char *what = "bm_scratch_set_path";
+    if (!s) return fail(nullptr, BM_EARG, "%s: scratch is NULL", what);
+    if (path != BM_PATH_AUTO && path != BM_PATH_PER_SLOT && path != BM_PATH_GROUPED && path != BM_PATH_GEMM)
+        return fail(s->ctx, BM_EARG, "%s: path %d is not one of BM_PATH_AUTO, BM_PATH_PER_SLOT, BM_PATH_GROUPED, BM_PATH_GEMM", what, path);
+    if (path == BM_PATH_GEMM && !(bmk::gemm_supported(s->gate_type) && bmk::gemm_supported(s->down_type)))
+        return fail(s->ctx, BM_ETYPE, "%s: no grouped GEMM for types %d / %d", what, s->gate_type, s->down_type);
+    if (grouped_from < 0 || gemm_from < 0)
+        return fail(s->ctx, BM_ESHAPE, "%s: the crossovers are token counts (0: keep), got %d and %d", what, grouped_from, gemm_from);
+    s->path = path;
+    if (grouped_from) s->grouped_from = grouped_from;
+    if (gemm_from) s->gemm_from = s->gemm_from_fast = gemm_from;
+    return BM_OK;
+}
+
+int bm_scratch_path_for(const bm_scratch *s, int m) {
+    if (!s || m < 1 || m > s->max_tokens) return BM_ESHAPE;
+    const bool gemm_ok = bmk::gemm_supported(s->gate_type) && bmk::gemm_supported(s->down_type);
+    if (s->path != BM_PATH_AUTO) {
+        if (s->path == BM_PATH_PER_SLOT && m > bmk::kMaxDecodeTokens) return BM_PATH_GROUPED;
+        return s->path;
+    }
+    if (m < s->grouped_from && m <= bmk::kMaxDecodeTokens) return BM_PATH_PER_SLOT;
+    if (m < (s->ctx->gemm_mode == BM_GEMM_FAST ? s->gemm_from_fast : s->gemm_from) || !gemm_ok) return BM_PATH_GROUPED;
+    return BM_PATH_GEMM;
+}
+
+int bm_moe_forward(bm_ctx *ctx, bm_scratch *s, const bm_weights *wg, const bm_weights *wu, const bm_weights *wd,
+                   const float *x_dev, const uint32_t *sel_dev, const float *w_dev, const float *resid_dev, int m,
+                   const bm_gate_act *rule, float *y_dev) {
+    const char *what = "bm_moe_forward";
+    if (!ctx || !s || !wg || !wu || !wd || !x_dev || !sel_dev || !w_dev || !y_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (s->ctx != ctx) return fail(ctx, BM_EARG, "%s: the scratch was made on another context", what);
+    if (wg->wtype != s->gate_type || wu->wtype != s->gate_type || wd->wtype != s->down_type || wg->k != s->hidden || wd->k != s->ff)
+        return fail(ctx, BM_ESHAPE, "%s: the scratch was made for types %d / %d at hidden %d, ff %d; the stacks are %d / %d / %d at %d, %d",
+                    what, s->gate_type, s->down_type, s->hidden, s->ff, wg->wtype, wu->wtype, wd->wtype, wg->k, wd->k);
+    if (wg->rows != (int64_t)s->n_experts * s->ff || wu->rows != wg->rows || wd->rows != (int64_t)s->n_experts * s->hidden)
+        return fail(ctx, BM_ESHAPE, "%s: the scratch was made for %d experts; the stacks hold %lld, %lld and %lld rows", what,
+                    s->n_experts, (long long)wg->rows, (long long)wu->rows, (long long)wd->rows);
+    if (m < 1 || m > s->max_tokens) return fail(ctx, BM_ESHAPE, "%s: m = %d tokens, the scratch holds 1..=%d", what, m, s->max_tokens);
+    const int spt = s->spt, n_slots = m * spt, hidden = s->hidden, ff = s->ff, n_experts = s->n_experts;
+    const bool down_q8k = act_form(s->down_type) != 0;
+    switch (bm_scratch_path_for(s, m)) {
+    case BM_PATH_PER_SLOT:
+        return bm_moe_decode(ctx, wg, wu, wd, x_dev, sel_dev, w_dev, resid_dev, spt, m, rule, s->act_h, nullptr,
+                             down_q8k ? s->g : nullptr, y_dev);
+    case BM_PATH_GROUPED: {
+        int rc = bm_tables(ctx, sel_dev, n_slots, n_experts, s->order, s->start, s->tiles);
+        if (!rc) rc = bm_quantize(ctx, x_dev, m, s->act_x);
+        if (!rc && !down_q8k)
+            rc = bm_gate_up_tiles(ctx, wg, wu, s->act_x, s->order, s->start, s->tiles, n_slots, ff, spt, rule, nullptr, s->act_h);
+        if (!rc && down_q8k) {
+            rc = bm_gate_up_tiles(ctx, wg, wu, s->act_x, s->order, s->start, s->tiles, n_slots, ff, spt, rule, s->g, nullptr);
+            if (!rc) rc = bm_quantize_ord(ctx, s->g, s->start, n_experts, n_slots, s->act_h);
+        }
+        if (!rc) rc = bm_gemv_tiles(ctx, wd, s->act_h, s->order, s->start, s->tiles, n_slots, hidden, s->down);
+        if (rc) return rc;
+        break;
+    }
+    default: {
+        int rc = bm_quantize(ctx, x_dev, m, s->act_x);
+        if (!rc) rc = bm_route_fill(ctx, sel_dev, n_slots, s->route);
+        if (!rc) rc = bm_gemm(ctx, wg, ff, s->act_x, s->route, spt, s->g);
+        if (!rc) rc = bm_gemm(ctx, wu, ff, s->act_x, s->route, spt, s->u);
+        if (!rc) rc = bm_swiglu_quant(ctx, s->g, s->u, n_slots, rule, s->act_h);
+        if (!rc) rc = bm_gemm(ctx, wd, hidden, s->act_h, s->route, 0, s->down);
+        if (rc) return rc;
+        break;
+    }
+    }
+    // the slots' weighted sum; a slot that names no expert of the stack adds nothing, as in the per-slot path
+    return driver(ctx, what, bmk::combine_tokens(launch_of(ctx), s->down, w_dev, nullptr, resid_dev, hidden, spt, m, y_dev, sel_dev,
+                                                 (uint32_t)n_experts));
+}
+
 // crates/gpu/src/kquant/act.rs:71-125 Act::code: what the device rules can run, refused by name otherwise.
 static int rule_checked(bm_ctx *ctx, const char *what, int rule, float limit, bmk::GateRule *out) {
     switch (rule) {

@@ -52,8 +52,9 @@ hipError_t gate_up(const Launch &L, int wtype, const uint8_t *wg, const uint8_t 
 hipError_t gemv_sel(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const uint8_t *act,
                     const uint32_t *sel, int n_slots, int rows_per_expert, float *y);
 
+// sel (optional): a slot whose id is at or past n_experts adds nothing
 hipError_t combine_tokens(const Launch &L, const float *down, const float *w, const float *shexp, const float *resid,
-                          int rows, int n_slots, int m, float *y);
+                          int rows, int n_slots, int m, float *y, const uint32_t *sel = nullptr, uint32_t n_experts = 0);
 
 // Slots a token may have in the fused down + combine launch.
 constexpr int kMaxCombineSlots = 64;

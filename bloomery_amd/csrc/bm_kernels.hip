@@ -203,23 +203,26 @@ __global__ __launch_bounds__(256) void k_gemv_sel(const uint8_t *w, u32 n_expert
 // crates/gpu/src/arch/qwen3moe/experts.rs:293-318 with crates/gpu/src/elem.rs:658-697: one thread a value.
 // With a shared expert's rows: (sum + shexp) + resid, grouped as the reference groups its two adds
 // (crates/gpu/src/moe_fused.rs:129-170 moe_combine).
+// `sel` (optional): a slot whose id is at or past n_experts adds nothing, as in the fused down + combine launch.
 __global__ __launch_bounds__(256) void k_combine(const float *down, const float *w, const float *shexp, const float *resid,
-                                                 int rows, int n_slots, int m, float *y) {
+                                                 int rows, int n_slots, int m, float *y, const u32 *sel, u32 n_experts) {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (long)rows * m) return;
     const int t = (int)(i / rows), d = (int)(i % rows);
     float acc = 0.0f;
-    for (int e = 0; e < n_slots; e++)
+    for (int e = 0; e < n_slots; e++) {
+        if (sel && sel[(size_t)t * n_slots + e] >= n_experts) continue;
         acc = fmaf(w[(size_t)t * n_slots + e], down[((size_t)t * n_slots + e) * rows + d], acc);
+    }
     if (shexp) acc = __fadd_rn(acc, shexp[i]);
     y[i] = resid ? __fadd_rn(acc, resid[i]) : acc;
 }
 
 hipError_t combine_tokens(const Launch &L, const float *down, const float *w, const float *shexp, const float *resid,
-                          int rows, int n_slots, int m, float *y) {
+                          int rows, int n_slots, int m, float *y, const uint32_t *sel, uint32_t n_experts) {
     const long n = (long)rows * m;
     hipLaunchKernelGGL(k_combine, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, L.stream, down, w, shexp, resid, rows,
-                       n_slots, m, y);
+                       n_slots, m, y, sel, n_experts);
     return hipGetLastError();
 }
 

@@ -329,6 +329,39 @@ int bm_set_gemm_mode(bm_ctx *ctx, int mode);
 int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, const bm_gate_act *rule, bm_act *act);
 
 
+/* ------------------------------------------------------------------ one entry for every number of tokens */
+
+/* The expert step of a layer for any number of tokens through one call, which picks among the three ways above by the
+ * number of tokens - the reference's cut between its gemv arm and its wide arm (crates/gpu/src/arch/qwen3moe/wide.rs:75-77
+ * GEMV_COLS, prefill.rs:602-604 WIDE_FROM, :147 wide_steps), here with a grouped arm between the two:
+ *   BM_PATH_PER_SLOT  bm_moe_decode: two launches, every slot streams its expert's rows (repeats come from the caches);
+ *   BM_PATH_GROUPED   bm_tables, bm_quantize, bm_gate_up_tiles (bm_quantize_ord for a down stack on Q8_K columns),
+ *                     bm_gemv_tiles, the slots' sum: an expert's rows are read once for all of its slots;
+ *   BM_PATH_GEMM      bm_quantize, bm_route_fill, bm_gemm twice, bm_swiglu_quant, bm_gemm, the slots' sum: the int8 matrix
+ *                     cores (in the f32 order bm_set_gemm_mode sets; Q4_K, Q5_K, Q6_K and IQ2_XXS stacks).
+ * In the exact mode all three give the same bits in y_dev. bm_scratch holds what the paths need between their launches for
+ * up to max_tokens tokens (made at load time and shared by every layer of the same shape, as the reference's Q8Act scratch
+ * is): max_tokens * n_slots_per_token <= 40960. BM_PATH_AUTO (the default) takes the per-slot path below grouped_from
+ * tokens, the grouped path below gemm_from and the GEMM from there; the defaults are the crossovers measured on MI355X at
+ * the Qwen3-30B-A3B layer shape: 22 tokens, and 448 tokens in the exact mode of bm_gemm or 160 in its tolerance mode.
+ * bm_scratch_set_path sets others (0 keeps a value; gemm_from then holds for both modes) or forces one path.
+ * bm_scratch_path_for: the path a call with m tokens takes. A slot whose id names no expert of the stack adds nothing to
+ * the sum (and raises BM_SITE_EXPERT_ID unless it is BM_HOST_SLOT, which the GEMM path's route table raises as well:
+ * batches with host-served slots go through the separate launches). Calls that share a scratch must not overlap. */
+typedef struct bm_scratch bm_scratch;
+#define BM_PATH_AUTO 0
+#define BM_PATH_PER_SLOT 1
+#define BM_PATH_GROUPED 2
+#define BM_PATH_GEMM 3
+int bm_scratch_create(bm_ctx *ctx, int gate_type, int down_type, int hidden, int ff, int n_experts, int n_slots_per_token,
+                      int max_tokens, bm_scratch **out);
+void bm_scratch_destroy(bm_scratch *scratch);
+int bm_scratch_set_path(bm_scratch *scratch, int path, int grouped_from, int gemm_from);
+int bm_scratch_path_for(const bm_scratch *scratch, int m);
+int bm_moe_forward(bm_ctx *ctx, bm_scratch *scratch, const bm_weights *wg, const bm_weights *wu, const bm_weights *wd,
+                   const float *x_dev, const uint32_t *sel_dev, const float *w_dev, const float *resid_dev, int m,
+                   const bm_gate_act *rule, float *y_dev);
+
 /* ------------------------------------------------------------------------------------------------- router */
 
 /* The step before the experts: RouterKernels::enqueue_route, kernel softmax_router_route

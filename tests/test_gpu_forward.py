@@ -1,0 +1,119 @@
+"""GPU parity tests of bm_moe_forward, the one entry for any number of tokens: each of its three paths (per slot, grouped
+by expert, the grouped GEMM) gives the oracle's layer output bit for bit on the same seeded inputs, so the choice among
+them by batch size changes no bit; the automatic choice follows the crossovers; ids that name no expert add nothing."""
+import numpy as np
+import pytest
+
+import bloomery_amd as bm
+import ora
+from common import normal_f32
+from test_gpu_decode import Layer, assert_f32, gpu, route  # noqa: F401  (gpu: module fixture)
+
+pytestmark = pytest.mark.gpu
+
+PATHS = ((bm.PATH_PER_SLOT, "per slot"), (bm.PATH_GROUPED, "grouped"), (bm.PATH_GEMM, "gemm"))
+
+
+@pytest.mark.parametrize("types,hidden,ff,n_experts,top_k,m", (
+    ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 12, 8, 19),     # the headline layer's rows
+    ((bm.Q5_K, bm.Q5_K, bm.Q4_K), 512, 512, 5, 3, 40),
+    ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ2_XXS), 1024, 512, 6, 4, 9),  # Q8_K columns on both sides
+    ((bm.Q4_K, bm.Q4_K, bm.IQ2_XXS), 512, 768, 4, 2, 33),    # the two column forms in one layer
+))
+def test_every_path_gives_the_oracles_bits(gpu, types, hidden, ff, n_experts, top_k, m):
+    L = Layer(gpu, types, hidden, ff, n_experts, 5100 + hidden)
+    rng = np.random.default_rng(5101)
+    x, resid = normal_f32(rng, (m, hidden)), normal_f32(rng, (m, hidden))
+    ids, wts = route(rng, m, n_experts, top_k)
+    want_y, _ = L.oracle(x, ids, wts, top_k)
+    want = (want_y.reshape(m, hidden) + resid).astype(np.float32).reshape(-1)
+    xd, sel, wd, rd = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32), gpu.upload(resid, np.float32)
+    y = gpu.buffer(np.float32, m * hidden)
+    sc = gpu.scratch(types[0], types[2], hidden, ff, n_experts, top_k, 64)
+    gpu.fault_clear()
+    try:
+        for path, name in PATHS:
+            sc.set_path(path)
+            assert sc.path_for(m) == path
+            for rep in range(2):  # the scratch is reused as it stands
+                y.fill_bytes(0xFF)
+                gpu.enqueue_moe_forward(sc, L.dg, L.du, L.dd, xd, sel, wd, rd, m, y)
+                assert_f32(y.download(), want, f"{name}, call {rep}")
+            # fewer tokens after more, over the same scratch
+            y.fill_bytes(0xFF)
+            gpu.enqueue_moe_forward(sc, L.dg, L.du, L.dd, xd, sel, wd, rd, 3, y)
+            assert_f32(y.download()[:3 * hidden], want[:3 * hidden], f"{name}, three tokens")
+        assert gpu.fault() == (bm.FAULT_NONE, 0)
+    finally:
+        sc.free()
+        for b in (xd, sel, wd, rd, y):
+            b.free()
+        L.free()
+
+
+def test_the_automatic_choice_follows_the_crossovers(gpu):
+    sc = gpu.scratch(bm.Q4_K, bm.Q6_K, 2048, 768, 128, 8, 4096)
+    try:
+        assert [sc.path_for(m) for m in (1, 21, 22, 447, 448, 4096)] == [bm.PATH_PER_SLOT, bm.PATH_PER_SLOT, bm.PATH_GROUPED,
+                                                                       bm.PATH_GROUPED, bm.PATH_GEMM, bm.PATH_GEMM]
+        gpu.set_gemm_mode(bm.GEMM_FAST)  # the tolerance mode's GEMM is faster: its cut comes earlier
+        try:
+            assert [sc.path_for(m) for m in (21, 22, 159, 160)] == [bm.PATH_PER_SLOT, bm.PATH_GROUPED, bm.PATH_GROUPED, bm.PATH_GEMM]
+        finally:
+            gpu.set_gemm_mode(bm.GEMM_EXACT)
+        sc.set_path(bm.PATH_AUTO, 4, 2000)
+        assert [sc.path_for(m) for m in (3, 4, 1999, 2000)] == [bm.PATH_PER_SLOT, bm.PATH_GROUPED, bm.PATH_GROUPED, bm.PATH_GEMM]
+        sc.set_path(bm.PATH_PER_SLOT)
+        assert sc.path_for(1024) == bm.PATH_PER_SLOT and sc.path_for(1025) == bm.PATH_GROUPED  # past the fused step's token limit
+        assert sc.path_for(0) == bm.ESHAPE and sc.path_for(4097) == bm.ESHAPE
+        with pytest.raises(bm.GpuError) as e:
+            sc.set_path(7)
+        assert "bm_scratch_set_path" in str(e.value)
+    finally:
+        sc.free()
+    # a type without a grouped GEMM never takes that path, and says so when asked to
+    sc = gpu.scratch(bm.IQ4_XS, bm.IQ4_XS, 512, 256, 4, 2, 512)
+    try:
+        assert sc.path_for(500) == bm.PATH_GROUPED
+        with pytest.raises(bm.GpuError) as e:
+            sc.set_path(bm.PATH_GEMM)
+        assert e.value.code == bm.ETYPE
+    finally:
+        sc.free()
+    for call, word in ((lambda: gpu.scratch(bm.Q4_K, bm.Q6_K, 2048, 768, 128, 8, 5121), "40960"),
+                       (lambda: gpu.scratch(bm.Q4_K, bm.Q6_K, 2000, 768, 128, 8, 16), "256"),
+                       (lambda: gpu.scratch(bm.Q4_K, 99, 2048, 768, 128, 8, 16), "type")):
+        with pytest.raises(bm.GpuError) as e:
+            call()
+        assert word in str(e.value) and "bm_scratch_create" in str(e.value)
+
+
+def test_a_slot_without_an_expert_adds_nothing_on_every_path(gpu):
+    """A host-served slot and an id past the stack: the token's sum is the oracle's over its live slots on each path (the
+    id past the stack raises ExpertId; the grouped GEMM's route table raises it for the host's slot as well)."""
+    L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 4, 5200)
+    rng = np.random.default_rng(5201)
+    m, top_k = 3, 3
+    x = normal_f32(rng, (m, 512))
+    ids = np.array([[1, bm.HOST_SLOT, 3], [2, 0, 1], [0, 9, 2]], np.uint32)
+    wts = np.array([[0.5, 0.3, 0.2], [0.2, 0.5, 0.3], [0.1, 0.6, 0.3]], np.float32)
+    want = np.concatenate([L.oracle(x[:1], np.array([[1, 3]], np.uint32), np.array([[0.5, 0.2]], np.float32), 2)[0],
+                           L.oracle(x[1:2], ids[1:2], wts[1:2], 3)[0],
+                           L.oracle(x[2:], np.array([[0, 2]], np.uint32), np.array([[0.1, 0.3]], np.float32), 2)[0]])
+    xd, sel, wd = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32)
+    y = gpu.buffer(np.float32, m * 512)
+    sc = gpu.scratch(bm.Q4_K, bm.Q6_K, 512, 256, 4, top_k, 8)
+    try:
+        for path, name in PATHS:
+            sc.set_path(path)
+            gpu.fault_clear()
+            y.fill_bytes(0xFF)
+            gpu.enqueue_moe_forward(sc, L.dg, L.du, L.dd, xd, sel, wd, None, m, y)
+            assert_f32(y.download(), want, name)
+            assert gpu.fault()[1] & (1 << bm.SITE_EXPERT_ID)  # (the refused slot's NaN rows may raise the quantizer's site too)
+        gpu.fault_clear()
+    finally:
+        sc.free()
+        for b in (xd, sel, wd, y):
+            b.free()
+        L.free()

@@ -591,10 +591,21 @@ __device__ __forceinline__ Blk<BM_IQ2XXS> bm_load_iq2xxs(const uint8_t *wrow, in
 }
 
 // LDS tables of the IQ2_XXS decode. The CPU path dots the unsigned bytes u = +-mag + 43 (0 .. 86) and takes the 43s
-// back out through the column's sums, so the tables give u with two operations a word: a grid point is kept as its
-// eight magnitudes + 43 (x, y) and its eight doubled magnitudes (z, w), a sign index as eight byte masks (0xff where
-// the value is negative): u = (mag + 43) - (2 mag & mask), byte by byte without a borrow.
-// IQ3_XXS: the same with the offset 64 and grid points of four magnitudes: an entry is (magnitudes + 64, doubled).
+// back out through the column's sums, so the tables give u with one operation a word: a grid point is kept as its
+// eight bytes 43 + mag (x, y) and its eight bytes 43 - mag (z, w), a sign index as eight byte masks (0xff where the
+// value is negative), and u is a bitwise pick between the two by the mask (v_bfi_b32).
+// IQ3_XXS: the same with the offset 64 and grid points of four magnitudes: an entry is (64 + mag, 64 - mag).
+__device__ __forceinline__ u32 bm_iq_pick(u32 plus, u32 minus, u32 mask) { return (minus & mask) | (plus & ~mask); }
+
+// a * b + c over 24-bit factors as one multiply-add: the empty statement pins the running sum, so the compiler cannot
+// regroup a chain of these into multiplies and three-operand adds (three instructions for two products where two do).
+// (The instruction itself is not written by hand: the compiler places the wait states a dot product's result needs
+// before another kind of instruction reads it, and cannot see into a hand-written one.)
+__device__ __forceinline__ int bm_mad24_chain(int a, int b, int c) {
+    int r = __mul24(a, b) + c;
+    asm volatile("" : "+v"(r));
+    return r;
+}
 struct Iq2Tables {
     const uint4 *grid;  // IQ2_XXS
     const uint2 *grid3; // IQ3_XXS
@@ -639,8 +650,8 @@ __device__ __forceinline__ Iq2Dec bm_decode_iq2xxs(const Blk<BM_IQ2XXS> &b, int 
             dec.sc[sb] = 2 * (int)(aux >> 28) + 1;
             const uint4 g = tb.grid[(idx >> (8 * q)) & 0xffu];
             const uint2 sg = tb.signs[(aux >> (7 * q)) & 127u];
-            dec.u_lo[sb] = g.x - (g.z & sg.x);
-            dec.u_hi[sb] = g.y - (g.w & sg.y);
+            dec.u_lo[sb] = bm_iq_pick(g.x, g.z, sg.x);
+            dec.u_hi[sb] = bm_iq_pick(g.y, g.w, sg.y);
         }
     }
     return dec;
@@ -671,8 +682,8 @@ __device__ __forceinline__ void bm_dot_iqx_dec(float d, int sca, int scb, const 
         // the reference sums sc * u * a (the offsets come back out through the fold above); sums within 4 * 126 * 128
         // and sc <= 31 lie inside 24 bits
         const int d_lo = bm_sdot4(dec.u_lo[sb], a.x, 0), d_hi = bm_sdot4(dec.u_hi[sb], a.y, 0);
-        sumi0 = bm_mad24(dec.sc[sb], d_lo, sumi0);
-        sumi1 = bm_mad24(dec.sc[sb], d_hi, sumi1);
+        sumi0 = bm_mad24_chain(dec.sc[sb], d_lo, sumi0);
+        sumi1 = bm_mad24_chain(dec.sc[sb], d_hi, sumi1);
         if constexpr (Tap::kActive) // the signed sum: less the offset times the eight codes
             tap.iq2(i, sb, q, d_lo + d_hi - OFF * (bm_sdot4(0x01010101u, a.x, 0) + bm_sdot4(0x01010101u, a.y, 0)));
     }
@@ -735,8 +746,8 @@ __device__ __forceinline__ Iq2Dec bm_decode_iq3xxs(const Blk<BM_IQ3XXS> &b, int 
             dec.sc[sb] = 2 * (int)(aux >> 28) + 1;
             const uint2 g0 = tb.grid3[pair & 0xffu], g1 = tb.grid3[(pair >> 8) & 0xffu];
             const uint2 sg = tb.signs[(aux >> (7 * q)) & 127u];
-            dec.u_lo[sb] = g0.x - (g0.y & sg.x);
-            dec.u_hi[sb] = g1.x - (g1.y & sg.y);
+            dec.u_lo[sb] = bm_iq_pick(g0.x, g0.y, sg.x);
+            dec.u_hi[sb] = bm_iq_pick(g1.x, g1.y, sg.y);
         }
     }
     return dec;

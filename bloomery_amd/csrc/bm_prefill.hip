@@ -856,8 +856,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, 
                 const uint4 gp = tb.grid[(idx >> (8 * q)) & 0xffu];
                 const uint2 sg = tb.signs[(aux >> (7 * q)) & 127u];
                 u32 h0, l0, h1, l1;
-                iq2_planes(gp.x - (gp.z & sg.x), sc, h0, l0);
-                iq2_planes(gp.y - (gp.w & sg.y), sc, h1, l1);
+                iq2_planes(bm_iq_pick(gp.x, gp.z, sg.x), sc, h0, l0);
+                iq2_planes(bm_iq_pick(gp.y, gp.w, sg.y), sc, h1, l1);
                 const int at = wr * kIqStride + 32 * (2 * q) + 4 * b;
                 *reinterpret_cast<u32 *>(w_hi + at) = h0;
                 *reinterpret_cast<u32 *>(w_lo + at) = l0;

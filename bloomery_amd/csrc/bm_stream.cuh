@@ -55,9 +55,9 @@ __device__ __forceinline__ Iq2Tables stage_tables(uint8_t *lds) {
         uint4 *grid = reinterpret_cast<uint4 *>(lds);
         uint2 *signs = reinterpret_cast<uint2 *>(lds + 256 * 16);
         for (int t = threadIdx.x; t < 256; t += blockDim.x) {
-            const uint64_t g = BM_IQ2XXS_GRID[t]; // bytes 8, 25 or 43: + 43 and doubled stay inside a byte
+            const uint64_t g = BM_IQ2XXS_GRID[t]; // bytes 8, 25 or 43: 43 + and 43 - stay inside a byte
             const u32 lo = (u32)g, hi = (u32)(g >> 32);
-            grid[t] = make_uint4(lo + 0x2b2b2b2bu, hi + 0x2b2b2b2bu, lo << 1, hi << 1);
+            grid[t] = make_uint4(0x2b2b2b2bu + lo, 0x2b2b2b2bu + hi, 0x2b2b2b2bu - lo, 0x2b2b2b2bu - hi);
         }
         for (int t = threadIdx.x; t < 128; t += blockDim.x) signs[t] = iq_sign_masks(t);
         tb.grid = grid;
@@ -67,8 +67,8 @@ __device__ __forceinline__ Iq2Tables stage_tables(uint8_t *lds) {
         uint2 *grid = reinterpret_cast<uint2 *>(lds);
         uint2 *signs = reinterpret_cast<uint2 *>(lds + 256 * 8);
         for (int t = threadIdx.x; t < 256; t += blockDim.x) {
-            const u32 g = BM_IQ3XXS_GRID[t]; // bytes 4 .. 62: + 64 and doubled stay inside a byte
-            grid[t] = make_uint2(g + 0x40404040u, g << 1);
+            const u32 g = BM_IQ3XXS_GRID[t]; // bytes 4 .. 62: 64 + and 64 - stay inside a byte
+            grid[t] = make_uint2(0x40404040u + g, 0x40404040u - g);
         }
         for (int t = threadIdx.x; t < 128; t += blockDim.x) signs[t] = iq_sign_masks(t);
         tb.grid3 = grid;

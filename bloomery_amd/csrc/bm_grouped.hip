@@ -147,7 +147,9 @@ __device__ __forceinline__ void stage_tile_cols(uint8_t *cols, const uint8_t *ac
 // the activation column of the token of slot order[j + c] and writes h[(j + c) * rpe + r]: by entry, not by slot.
 // With act_h the 32 values of each column become block rb of column j + c of act_h in the same launch.
 // MC: the columns this launch has LDS for; it takes the tiles of m_lo < m <= MC columns and leaves the others to the
-// launch of the other width (see tile_widths below).
+// launch of the other width (see tile_widths below). m_lo < 0: it takes every tile, MC columns at a pass over the rows
+// (a wider tile's rows are then read and unpacked again for every pass: the form for batches whose tiles are nearly all
+// narrow, where it saves the second launch).
 template <int WT, int U, int NB, int MC>
 __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const uint8_t *wu, u32 n_experts, int nb,
                                                        const uint8_t *act, int act_cols, const u32 *order,
@@ -158,7 +160,9 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
     const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
     Tile t;
     if (!tile_of_block(tiles, start, order, n_experts, n_slots, cap, &t, fault, layer)) return; // raising twice is raising once
-    if (t.m <= m_lo || t.m > MC) return;
+    if (m_lo >= 0 && (t.m <= m_lo || t.m > MC)) return;
+    __shared__ u32 s_entry[kTileCols];
+    if (tid < kTileCols) s_entry[tid] = t.entry;
     const int rb = t.row_block;
     const int r = rb * 32 + (tid >> 3);
     const bool active = r < rpe;
@@ -173,32 +177,37 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
     uint8_t *cols = lds + tab_bytes<WT>();
     float *hbuf = reinterpret_cast<float *>(cols + (size_t)MC * col_bytes); // [MC][32]
     u32 *bad = reinterpret_cast<u32 *>(hbuf + MC * 32);                      // [MC]: entry names no slot
-    if (tid < MC) {
-        const u32 s = tid < t.m ? t.entry : 0;
-        const bool none = tid < t.m && (s >= n_slots || (int)(s / slots_per_col) >= act_cols);
-        if (none) bm_raise(fault, layer, kSiteExpertId);
-        bad[tid] = none ? 0xffffffffu : s / slots_per_col;
-    }
-    __syncthreads();
-    stage_tile_cols(cols, act, col_bytes, t.m, [&](int c) { return bad[c] == 0xffffffffu ? 0 : (int)bad[c]; });
-    __syncthreads();
-    float v[MC];
-    row_dot<WT, U, NB, MC>(b, wrow, cols, col_bytes, t.m, n, q, tb, v, NoTap{});
-#pragma unroll
-    for (int c = 0; c < MC; c++) {
-        float hv = swiglu_of_pair(c < t.m ? v[c] : 0.0f, which, rule, fault, layer);
-        if (c < t.m) {
-            if (bad[c] == 0xffffffffu) hv = bm_bits_f32(0x7fc00000u);
-            if (h && active && (tid & 7) == 0) h[(size_t)(t.j + c) * rpe + r] = hv;
-            if (act_h && (tid & 7) == 0) hbuf[c * 32 + (tid >> 3)] = hv;
+    for (int c0 = 0; c0 < t.m; c0 += MC) { // one pass, but for a tile wider than MC under m_lo < 0
+        const int mc = t.m - c0 < MC ? t.m - c0 : MC;
+        __syncthreads(); // s_entry is written; the pass before is done with cols, hbuf and bad
+        if (c0) preload<WT, U>(b, wrow, q);
+        if (tid < MC) {
+            const u32 s = tid < mc ? s_entry[c0 + tid] : 0;
+            const bool none = tid < mc && (s >= n_slots || (int)(s / slots_per_col) >= act_cols);
+            if (none) bm_raise(fault, layer, kSiteExpertId);
+            bad[tid] = none ? 0xffffffffu : s / slots_per_col;
         }
-    }
-    if (act_h) { // rpe is a multiple of 256 here, so every row of the block is live
         __syncthreads();
-        const int c = tid >> 5; // half wave c: column c
-        if (c < t.m)
-            quantize_h_block(hbuf + c * 32, act_h + (size_t)(t.j + c) * nb_h * BM_Q82_SB_EXT, nb_h, rb, tid & 31, fault,
-                             layer);
+        stage_tile_cols(cols, act, col_bytes, mc, [&](int c) { return bad[c] == 0xffffffffu ? 0 : (int)bad[c]; });
+        __syncthreads();
+        float v[MC];
+        row_dot<WT, U, NB, MC>(b, wrow, cols, col_bytes, mc, n, q, tb, v, NoTap{});
+#pragma unroll
+        for (int c = 0; c < MC; c++) {
+            float hv = swiglu_of_pair(c < mc ? v[c] : 0.0f, which, rule, fault, layer);
+            if (c < mc) {
+                if (bad[c] == 0xffffffffu) hv = bm_bits_f32(0x7fc00000u);
+                if (h && active && (tid & 7) == 0) h[(size_t)(t.j + c0 + c) * rpe + r] = hv;
+                if (act_h && (tid & 7) == 0) hbuf[c * 32 + (tid >> 3)] = hv;
+            }
+        }
+        if (act_h) { // rpe is a multiple of 256 here, so every row of the block is live
+            __syncthreads();
+            const int c = tid >> 5; // half wave c: column c
+            if (c < mc)
+                quantize_h_block(hbuf + c * 32, act_h + (size_t)(t.j + c0 + c) * nb_h * BM_Q82_SB_EXT, nb_h, rb, tid & 31, fault,
+                                 layer);
+        }
     }
 }
 
@@ -212,7 +221,9 @@ __global__ __launch_bounds__(256) void k_gemv_tiles(const uint8_t *w, u32 n_expe
     const int tid = threadIdx.x, q = tid & 3;
     Tile t;
     if (!tile_of_block(tiles, start, order, n_experts, n_slots, cap, &t, fault, layer)) return;
-    if (t.m <= m_lo || t.m > MC) return;
+    if (m_lo >= 0 && (t.m <= m_lo || t.m > MC)) return;
+    __shared__ u32 s_entry[kTileCols];
+    if (tid < kTileCols) s_entry[tid] = t.entry;
     const int r = t.row_block * 64 + (tid >> 2);
     const bool active = r < rpe;
     const int n = NB > 0 ? NB : nb;
@@ -224,19 +235,24 @@ __global__ __launch_bounds__(256) void k_gemv_tiles(const uint8_t *w, u32 n_expe
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *cols = lds + tab_bytes<WT>();
     u32 *slot_of = reinterpret_cast<u32 *>(cols + (size_t)MC * col_bytes); // [MC]
-    if (tid < MC) {
-        const u32 s = tid < t.m ? t.entry : 0;
-        if (tid < t.m && s >= n_slots && t.row_block == 0) bm_raise(fault, layer, kSiteExpertId);
-        slot_of[tid] = s;
-    }
-    stage_bytes(cols, act + (size_t)t.j * col_bytes, t.m * col_bytes); // the tile's columns lie side by side
-    __syncthreads();
-    float v[MC];
-    row_dot<WT, U, NB, MC>(b, wrow, cols, col_bytes, t.m, n, q, tb, v, NoTap{});
-    if (q == 0 && active) {
+    for (int c0 = 0; c0 < t.m; c0 += MC) { // one pass, but for a tile wider than MC under m_lo < 0
+        const int mc = t.m - c0 < MC ? t.m - c0 : MC;
+        __syncthreads(); // s_entry is written; the pass before is done with cols and slot_of
+        if (c0) preload<WT, U>(b, wrow, q);
+        if (tid < MC) {
+            const u32 s = tid < mc ? s_entry[c0 + tid] : 0;
+            if (tid < mc && s >= n_slots && t.row_block == 0) bm_raise(fault, layer, kSiteExpertId);
+            slot_of[tid] = s;
+        }
+        stage_bytes(cols, act + (size_t)(t.j + c0) * col_bytes, mc * col_bytes); // the tile's columns lie side by side
+        __syncthreads();
+        float v[MC];
+        row_dot<WT, U, NB, MC>(b, wrow, cols, col_bytes, mc, n, q, tb, v, NoTap{});
+        if (q == 0 && active) {
 #pragma unroll
-        for (int c = 0; c < MC; c++)
-            if (c < t.m && slot_of[c] < n_slots) y[(size_t)slot_of[c] * rpe + r] = v[c];
+            for (int c = 0; c < MC; c++)
+                if (c < mc && slot_of[c] < n_slots) y[(size_t)slot_of[c] * rpe + r] = v[c];
+        }
     }
 }
 
@@ -253,18 +269,20 @@ size_t tiles_lds(int wtype, int k) {
 // Eight columns of a long row take most of a CU's LDS (IQ2_XXS at 7168 values: 66 KB, two workgroups a CU), and with
 // few tokens over many experts most tiles hold one or two slots. Past kTileSplitLds a tile launch therefore goes as two:
 // one with LDS for two columns takes the tiles of up to two slots at several times the occupancy, one with LDS for
-// eight takes the rest; a workgroup whose tile is the other launch's returns at once. Values do not depend on the
-// width: every column is its own row dot.
+// eight takes the rest; a workgroup whose tile is the other launch's returns at once. With no more than two slots an
+// expert of the stack on average nearly every tile is narrow, and the narrow launch alone takes them all, a wider tile
+// in passes of two columns: one launch instead of two. Values do not depend on the width: every column is its own row dot.
 constexpr size_t kTileSplitLds = 40 * 1024;
 constexpr int kTileNarrow = 2;
 static bool tile_widths_split(int wtype, int k) { return tiles_lds_of(wtype, k, kTileCols) > kTileSplitLds; }
+static bool tiles_mostly_narrow(int n_slots, int n_experts) { return n_slots <= kTileNarrow * n_experts; }
 
 hipError_t gate_up_tiles(const Launch &L, int wtype, const uint8_t *wg, const uint8_t *wu, int n_experts, int k,
                          const uint8_t *act, int act_cols, const uint32_t *order, const uint32_t *start,
                          const uint32_t *tiles_dev, int n_slots, int rows_per_expert, int slots_per_col, float *h,
                          uint8_t *act_h) {
     const int nb = k / 256, rpe = rows_per_expert;
-    const bool split = tile_widths_split(wtype, k);
+    const bool split = tile_widths_split(wtype, k), narrow = tiles_mostly_narrow(n_slots, n_experts);
     const u32 cap = (u32)tile_cap(n_slots, n_experts);
     const unsigned grid = cap * (unsigned)((rpe + 31) / 32);
 #define BM_TILE_LAUNCH(MC, M_LO)                                                                                       \
@@ -278,8 +296,11 @@ hipError_t gate_up_tiles(const Launch &L, int wtype, const uint8_t *wg, const ui
                            L.fault, L.layer);                                                                          \
     }
 #define CALL_BODY                                                                                                      \
-    if (split) BM_TILE_LAUNCH(kTileNarrow, 0)                                                                          \
-    BM_TILE_LAUNCH(kTileCols, split ? kTileNarrow : 0)
+    if (split && narrow) BM_TILE_LAUNCH(kTileNarrow, -1)                                                               \
+    else {                                                                                                             \
+        if (split) BM_TILE_LAUNCH(kTileNarrow, 0)                                                                      \
+        BM_TILE_LAUNCH(kTileCols, split ? kTileNarrow : 0)                                                             \
+    }
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
 #undef BM_TILE_LAUNCH
@@ -290,7 +311,7 @@ hipError_t gemv_tiles(const Launch &L, int wtype, const uint8_t *w, int n_expert
                       const uint32_t *order, const uint32_t *start, const uint32_t *tiles_dev, int n_slots,
                       int rows_per_expert, float *y) {
     const int nb = k / 256, rpe = rows_per_expert;
-    const bool split = tile_widths_split(wtype, k);
+    const bool split = tile_widths_split(wtype, k), narrow = tiles_mostly_narrow(n_slots, n_experts);
     const u32 cap = (u32)tile_cap(n_slots, n_experts);
     const unsigned grid = cap * (unsigned)((rpe + 63) / 64);
 #define BM_TILE_LAUNCH(MC, M_LO)                                                                                       \
@@ -303,8 +324,11 @@ hipError_t gemv_tiles(const Launch &L, int wtype, const uint8_t *w, int n_expert
                            tiles_dev, (u32)n_slots, cap, rpe, y, M_LO, L.fault, L.layer);                              \
     }
 #define CALL_BODY                                                                                                      \
-    if (split) BM_TILE_LAUNCH(kTileNarrow, 0)                                                                          \
-    BM_TILE_LAUNCH(kTileCols, split ? kTileNarrow : 0)
+    if (split && narrow) BM_TILE_LAUNCH(kTileNarrow, -1)                                                               \
+    else {                                                                                                             \
+        if (split) BM_TILE_LAUNCH(kTileNarrow, 0)                                                                      \
+        BM_TILE_LAUNCH(kTileCols, split ? kTileNarrow : 0)                                                             \
+    }
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
 #undef BM_TILE_LAUNCH

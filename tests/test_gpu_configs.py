@@ -76,6 +76,40 @@ def test_deepseek_shaped_layer_grouped(gpu, ds_layer):
         b.free()
 
 
+def test_long_rows_few_slots_an_expert_one_tile_launch(gpu, ds_layer):
+    """With rows this long a tile launch has LDS for two columns, and with no more than two slots an expert of the stack
+    on average the one launch takes every tile, a wider one in passes of two columns: three tokens that all name expert
+    5 make a tile of three (two passes, the second of one column); every slot's h and down rows against the oracle."""
+    routed = ds_layer[0]
+    rng = np.random.default_rng(3150)
+    m, top_k = 3, DS_TOPK
+    n_slots = m * top_k  # 24 = 2 x the 12 experts of the stack
+    x = normal_f32(rng, (m, DS_HIDDEN))
+    ids = np.stack([np.concatenate([[5], rng.permutation([e for e in range(DS_RESIDENT) if e != 5])[:top_k - 1]]) for _ in range(m)])
+    ids = np.stack([rng.permutation(row) for row in ids]).astype(np.uint32)
+    wts = rng.uniform(0.05, 0.3, (m, top_k)).astype(np.float32)
+    want_y, want_h = routed.oracle(x, ids, wts, top_k)
+    gpu.fault_clear()
+    sel, order, start, tiles = grouped_tables_on_device(gpu, ids.reshape(-1), DS_RESIDENT)
+    counts = np.diff(start.download())
+    assert counts[5] == 3 and n_slots <= 2 * DS_RESIDENT
+    xd, wd = gpu.upload(x, np.float32), gpu.upload(wts, np.float32)
+    act, act_h = gpu.act(bm.IQ2_XXS, DS_HIDDEN, m), gpu.act(bm.IQ2_XXS, DS_FF, n_slots)
+    h = gpu.buffer(np.float32, n_slots * DS_FF).fill_bytes(0xFF)
+    down = gpu.buffer(np.float32, n_slots * DS_HIDDEN).fill_bytes(0xFF)
+    y = gpu.buffer(np.float32, m * DS_HIDDEN).fill_bytes(0xFF)
+    gpu.enqueue_quantize(xd, m, act)
+    gpu.enqueue_gate_up_tiles(routed.dg, routed.du, act, order, start, tiles, n_slots, DS_FF, top_k, h)
+    gpu.enqueue_quantize_ord(h, start, DS_RESIDENT, n_slots, act_h)
+    gpu.enqueue_gemv_tiles(routed.dd, act_h, order, start, tiles, n_slots, DS_HIDDEN, down)
+    gpu.enqueue_combine_tokens(down, wd, None, DS_HIDDEN, top_k, m, y)
+    assert_f32(h.download().reshape(n_slots, DS_FF), want_h.reshape(n_slots, DS_FF)[order.download()], "h by table entry")
+    assert_f32(y.download(), want_y, "y")
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    for b in (sel, order, start, tiles, xd, wd, act, act_h, h, down, y):
+        b.free()
+
+
 def test_deepseek_shaped_layer_slot_by_slot(gpu, ds_layer):
     """The same tokens through bm_moe_decode (its residual argument carrying the shared expert's rows, the same
     grouping of the adds) and through the plain chain bm_gate_up, bm_quantize, bm_gemv_sel, bm_moe_combine."""

@@ -711,6 +711,9 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--one-interval", action="store_true",
+                    help="config 2 only: exactly --steps steps (rounded up to whole replays) with one event interval around them all, instead "
+                         "of at least 32 replays with an interval each: for runs under a profiler")
     ap.add_argument("--no-prefill", action="store_true", help="config 2 only: leave the prefill leg (config 4's step) out of the line")
     ap.add_argument("--types", default="q4_k,q6_k",
                     help="config 2 only: gate/up and down weight types (q3_k, q4_k, q5_k, q6_k, iq2_xxs, iq3_xxs, iq4_xs); other than the default is "
@@ -819,27 +822,31 @@ def main():
         enqueue_step(i)
     graph = gpu.capture_end()
     reps_w = max(1, -(-args.warmup // unit))
-    reps = max(32, -(-max(args.steps, 2048) // unit))
+    reps = -(-args.steps // unit) if args.one_interval else max(32, -(-max(args.steps, 2048) // unit))
     steps = reps * unit
     for _ in range(reps_w):
         gpu.graph_launch(graph)
     gpu.sync()
-    marks = [gpu.event() for _ in range(reps + 1)]
+    # an event after every replay (--one-interval: only around them all, for runs under a profiler, whose interception
+    # of a graph launch has crashed here when events were recorded between the launches)
+    stride = reps if args.one_interval else 1
+    marks = [gpu.event() for _ in range(reps // stride + 1)]
     t_start = time.perf_counter()
     gpu.event_record(marks[0])
     for r in range(reps):
         gpu.graph_launch(graph)
-        gpu.event_record(marks[r + 1])
+        if (r + 1) % stride == 0:
+            gpu.event_record(marks[(r + 1) // stride])
     gpu.sync()
     wall_ms = (time.perf_counter() - t_start) * 1e3
-    ev_ms = gpu.event_elapsed_ms(marks[0], marks[reps])
-    replay_us = sorted(gpu.event_elapsed_ms(marks[r], marks[r + 1]) * 1e3 / unit for r in range(reps))
+    ev_ms = gpu.event_elapsed_ms(marks[0], marks[-1])
+    replay_us = sorted(gpu.event_elapsed_ms(marks[r], marks[r + 1]) * 1e3 / (unit * stride) for r in range(len(marks) - 1))
     for ev in marks:
         gpu.event_destroy(ev)
     e0, e1 = gpu.event(), gpu.event()
     ms_per_step = wall_ms / steps
     us_per_token = ms_per_step * 1e3
-    replay_stats = {"replays": reps, "steps_per_replay": unit, "median_us_per_token": replay_us[reps // 2],
+    replay_stats = {"replays": reps, "steps_per_replay": unit, "median_us_per_token": replay_us[len(replay_us) // 2],
                     "min_us_per_token": replay_us[0], "max_us_per_token": replay_us[-1]}
     bytes_per_token = TOP_K * (2 * FF * bm.row_bytes(gate_t, HIDDEN) + HIDDEN * bm.row_bytes(down_t, FF))
 

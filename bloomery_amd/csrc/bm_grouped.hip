@@ -147,10 +147,10 @@ __device__ __forceinline__ void stage_tile_cols(uint8_t *cols, const uint8_t *ac
 // the activation column of the token of slot order[j + c] and writes h[(j + c) * rpe + r]: by entry, not by slot.
 // With act_h the 32 values of each column become block rb of column j + c of act_h in the same launch.
 // MC: the columns this launch has LDS for; it takes the tiles of m_lo < m <= MC columns and leaves the others to the
-// launch of the other width (see tile_widths below). m_lo < 0: it takes every tile, MC columns at a pass over the rows
+// launch of the other width (see tile_widths below). PASSES: it takes every tile, MC columns at a pass over the rows
 // (a wider tile's rows are then read and unpacked again for every pass: the form for batches whose tiles are nearly all
-// narrow, where it saves the second launch).
-template <int WT, int U, int NB, int MC>
+// narrow, where it saves the second launch; a variant of its own, so that the one-pass kernels stay straight-line code).
+template <int WT, int U, int NB, int MC, bool PASSES>
 __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const uint8_t *wu, u32 n_experts, int nb,
                                                        const uint8_t *act, int act_cols, const u32 *order,
                                                        const u32 *start, const u32 *tiles, u32 n_slots, u32 cap,
@@ -160,9 +160,9 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
     const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
     Tile t;
     if (!tile_of_block(tiles, start, order, n_experts, n_slots, cap, &t, fault, layer)) return; // raising twice is raising once
-    if (m_lo >= 0 && (t.m <= m_lo || t.m > MC)) return;
+    if (!PASSES && (t.m <= m_lo || t.m > MC)) return;
     __shared__ u32 s_entry[kTileCols];
-    if (tid < kTileCols) s_entry[tid] = t.entry;
+    if (PASSES && tid < kTileCols) s_entry[tid] = t.entry;
     const int rb = t.row_block;
     const int r = rb * 32 + (tid >> 3);
     const bool active = r < rpe;
@@ -177,12 +177,12 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
     uint8_t *cols = lds + tab_bytes<WT>();
     float *hbuf = reinterpret_cast<float *>(cols + (size_t)MC * col_bytes); // [MC][32]
     u32 *bad = reinterpret_cast<u32 *>(hbuf + MC * 32);                      // [MC]: entry names no slot
-    for (int c0 = 0; c0 < t.m; c0 += MC) { // one pass, but for a tile wider than MC under m_lo < 0
-        const int mc = t.m - c0 < MC ? t.m - c0 : MC;
-        __syncthreads(); // s_entry is written; the pass before is done with cols, hbuf and bad
-        if (c0) preload<WT, U>(b, wrow, q);
+    for (int c0 = 0; c0 < (PASSES ? t.m : 1); c0 += MC) { // one pass, but for a tile wider than MC under PASSES
+        const int mc = !PASSES ? t.m : t.m - c0 < MC ? t.m - c0 : MC;
+        if (PASSES) __syncthreads(); // s_entry is written; the pass before is done with cols, hbuf and bad
+        if (PASSES && c0) preload<WT, U>(b, wrow, q);
         if (tid < MC) {
-            const u32 s = tid < mc ? s_entry[c0 + tid] : 0;
+            const u32 s = tid < mc ? (PASSES ? s_entry[c0 + tid] : t.entry) : 0;
             const bool none = tid < mc && (s >= n_slots || (int)(s / slots_per_col) >= act_cols);
             if (none) bm_raise(fault, layer, kSiteExpertId);
             bad[tid] = none ? 0xffffffffu : s / slots_per_col;
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
 
 // crates/gpu/src/kquant/tiles.rs:120-190 GemvTiles: workgroup = tile x 64 rows (a quad a row); entry j + c reads
 // column j + c of act and writes row r of its slot order[j + c]. An entry that names no slot raises ExpertId.
-template <int WT, int U, int NB, int MC>
+template <int WT, int U, int NB, int MC, bool PASSES>
 __global__ __launch_bounds__(256) void k_gemv_tiles(const uint8_t *w, u32 n_experts, int nb, const uint8_t *act,
                                                     const u32 *order, const u32 *start, const u32 *tiles, u32 n_slots,
                                                     u32 cap, int rpe, float *y, int m_lo, u32 *fault, u32 layer) {
@@ -221,9 +221,9 @@ __global__ __launch_bounds__(256) void k_gemv_tiles(const uint8_t *w, u32 n_expe
     const int tid = threadIdx.x, q = tid & 3;
     Tile t;
     if (!tile_of_block(tiles, start, order, n_experts, n_slots, cap, &t, fault, layer)) return;
-    if (m_lo >= 0 && (t.m <= m_lo || t.m > MC)) return;
+    if (!PASSES && (t.m <= m_lo || t.m > MC)) return;
     __shared__ u32 s_entry[kTileCols];
-    if (tid < kTileCols) s_entry[tid] = t.entry;
+    if (PASSES && tid < kTileCols) s_entry[tid] = t.entry;
     const int r = t.row_block * 64 + (tid >> 2);
     const bool active = r < rpe;
     const int n = NB > 0 ? NB : nb;
@@ -235,12 +235,12 @@ __global__ __launch_bounds__(256) void k_gemv_tiles(const uint8_t *w, u32 n_expe
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *cols = lds + tab_bytes<WT>();
     u32 *slot_of = reinterpret_cast<u32 *>(cols + (size_t)MC * col_bytes); // [MC]
-    for (int c0 = 0; c0 < t.m; c0 += MC) { // one pass, but for a tile wider than MC under m_lo < 0
-        const int mc = t.m - c0 < MC ? t.m - c0 : MC;
-        __syncthreads(); // s_entry is written; the pass before is done with cols and slot_of
-        if (c0) preload<WT, U>(b, wrow, q);
+    for (int c0 = 0; c0 < (PASSES ? t.m : 1); c0 += MC) { // one pass, but for a tile wider than MC under PASSES
+        const int mc = !PASSES ? t.m : t.m - c0 < MC ? t.m - c0 : MC;
+        if (PASSES) __syncthreads(); // s_entry is written; the pass before is done with cols and slot_of
+        if (PASSES && c0) preload<WT, U>(b, wrow, q);
         if (tid < MC) {
-            const u32 s = tid < mc ? s_entry[c0 + tid] : 0;
+            const u32 s = tid < mc ? (PASSES ? s_entry[c0 + tid] : t.entry) : 0;
             if (tid < mc && s >= n_slots && t.row_block == 0) bm_raise(fault, layer, kSiteExpertId);
             slot_of[tid] = s;
         }
@@ -285,10 +285,10 @@ hipError_t gate_up_tiles(const Launch &L, int wtype, const uint8_t *wg, const ui
     const bool split = tile_widths_split(wtype, k), narrow = tiles_mostly_narrow(n_slots, n_experts);
     const u32 cap = (u32)tile_cap(n_slots, n_experts);
     const unsigned grid = cap * (unsigned)((rpe + 31) / 32);
-#define BM_TILE_LAUNCH(MC, M_LO)                                                                                       \
+#define BM_TILE_LAUNCH(MC, M_LO, PASSES)                                                                               \
     {                                                                                                                  \
         const size_t lds = tiles_lds_of(wtype, k, MC);                                                                 \
-        auto kern = k_gate_up_tiles<WT, U, NB, MC>;                                                                    \
+        auto kern = k_gate_up_tiles<WT, U, NB, MC, PASSES>;                                                                    \
         hipError_t e = allow_lds(kern, lds);                                                                           \
         if (e != hipSuccess) return e;                                                                                 \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, wg, wu, (u32)n_experts, nb, act, act_cols,      \
@@ -296,10 +296,10 @@ hipError_t gate_up_tiles(const Launch &L, int wtype, const uint8_t *wg, const ui
                            L.fault, L.layer);                                                                          \
     }
 #define CALL_BODY                                                                                                      \
-    if (split && narrow) BM_TILE_LAUNCH(kTileNarrow, -1)                                                               \
+    if (split && narrow) BM_TILE_LAUNCH(kTileNarrow, 0, true)                                                          \
     else {                                                                                                             \
-        if (split) BM_TILE_LAUNCH(kTileNarrow, 0)                                                                      \
-        BM_TILE_LAUNCH(kTileCols, split ? kTileNarrow : 0)                                                             \
+        if (split) BM_TILE_LAUNCH(kTileNarrow, 0, false)                                                               \
+        BM_TILE_LAUNCH(kTileCols, split ? kTileNarrow : 0, false)                                                      \
     }
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
@@ -314,20 +314,20 @@ hipError_t gemv_tiles(const Launch &L, int wtype, const uint8_t *w, int n_expert
     const bool split = tile_widths_split(wtype, k), narrow = tiles_mostly_narrow(n_slots, n_experts);
     const u32 cap = (u32)tile_cap(n_slots, n_experts);
     const unsigned grid = cap * (unsigned)((rpe + 63) / 64);
-#define BM_TILE_LAUNCH(MC, M_LO)                                                                                       \
+#define BM_TILE_LAUNCH(MC, M_LO, PASSES)                                                                               \
     {                                                                                                                  \
         const size_t lds = tiles_lds_of(wtype, k, MC);                                                                 \
-        auto kern = k_gemv_tiles<WT, U, NB, MC>;                                                                       \
+        auto kern = k_gemv_tiles<WT, U, NB, MC, PASSES>;                                                                       \
         hipError_t e = allow_lds(kern, lds);                                                                           \
         if (e != hipSuccess) return e;                                                                                 \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act, order, start,       \
                            tiles_dev, (u32)n_slots, cap, rpe, y, M_LO, L.fault, L.layer);                              \
     }
 #define CALL_BODY                                                                                                      \
-    if (split && narrow) BM_TILE_LAUNCH(kTileNarrow, -1)                                                               \
+    if (split && narrow) BM_TILE_LAUNCH(kTileNarrow, 0, true)                                                          \
     else {                                                                                                             \
-        if (split) BM_TILE_LAUNCH(kTileNarrow, 0)                                                                      \
-        BM_TILE_LAUNCH(kTileCols, split ? kTileNarrow : 0)                                                             \
+        if (split) BM_TILE_LAUNCH(kTileNarrow, 0, false)                                                               \
+        BM_TILE_LAUNCH(kTileCols, split ? kTileNarrow : 0, false)                                                      \
     }
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY

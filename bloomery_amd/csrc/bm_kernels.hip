@@ -47,7 +47,29 @@ __global__ __launch_bounds__(256) void k_quantize_q8k(const float *x, int m, int
     q8k_block_by_workgroup(x[(size_t)col * k + 256 * blk + threadIdx.x], act + ((size_t)col * bpc + blk) * BM_Q8K_STRIDE, fault, layer);
 }
 
+// The same columns with eight values a thread, a block a quad of lanes (two 16-byte loads a thread, fewer and fatter
+// workgroups): the form for many columns at once, where the launch is bound by its traffic and not by its latency.
+__global__ __launch_bounds__(256) void k_quantize_q82x4_wide(const float *x, int m, int k, uint8_t *act, const u32 *live,
+                                                             u32 *fault, u32 layer) {
+    const long at = ((long)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (at >= (long)m * k) return;
+    const int col = (int)(at / k), o = (int)(at % k);
+    if (live && (u32)col >= *live) return;
+    const float4 a = *reinterpret_cast<const float4 *>(x + at), b = *reinterpret_cast<const float4 *>(x + at + 4);
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    q82_quad8(v, act + (size_t)col * (k / 256) * BM_Q82_SB_EXT, k / 256, o >> 5, threadIdx.x & 3, fault, layer);
+}
+
+// Columns from which on the wide form is launched (and only for 16-byte aligned rows).
+constexpr long kWideQuantValues = 1 << 18;
+
 hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, uint8_t *act, const uint32_t *live) {
+    if (!bm_takes_q8k(wtype) && (long)m * k >= kWideQuantValues && ((uintptr_t)x & 15) == 0) {
+        const long threads = (long)m * k / 8;
+        hipLaunchKernelGGL(k_quantize_q82x4_wide, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, L.stream, x, m, k, act,
+                           live, L.fault, L.layer);
+        return hipGetLastError();
+    }
     if (bm_takes_q8k(wtype)) {
         hipLaunchKernelGGL(k_quantize_q8k, dim3((unsigned)(m * (k / 256))), dim3(256), 0, L.stream, x, m, k, act,
                            live, L.fault, L.layer);
@@ -290,56 +312,6 @@ __global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_ex
     const int blocks_per_token = (rpe + D - 1) / D;
     down_combine_body<WT, U, NB>(lds, w, n_experts, nb, act, sel, wts, resid, spt, rpe, y,
                                  blockIdx.x / blocks_per_token, blockIdx.x % blocks_per_token, fault, layer);
-}
-
-// One 32-value q8_2 block held eight values a lane by four consecutive lanes (the in-kernel token quantizer).
-__device__ __forceinline__ void q82_quad8(const float (&v)[8], uint8_t *col, int nb, int blk, int lane4, u32 *fault,
-                                          u32 layer) {
-    u32 ab = 0;
-#pragma unroll
-    for (int k = 0; k < 8; k++) {
-        const u32 a = bm_f32_bits(v[k]) & 0x7fffffffu;
-        ab = a > ab ? a : ab;
-    }
-    u32 o;
-    o = bm_dpp<kDppXor1>(ab), ab = o > ab ? o : ab;
-    o = bm_dpp<kDppXor2>(ab), ab = o > ab ? o : ab;
-    uint8_t *group = col + (size_t)(blk >> 2) * BM_Q82X4_STRIDE;
-    const int ir = blk & 3;
-    u32 t;
-    int isum = 0, csum = 0;
-    u32 c0 = 0, c1 = 0;
-    if (ab > 0x7f7fffffu) {
-        t = 0x7fc0u;
-        if (lane4 == 0) bm_raise(fault, layer, kSiteQuantColumn);
-    } else {
-        t = bm_fp32_to_bf16_bits(__fdiv_rn(bm_bits_f32(ab), 127.0f));
-        const float id = bm_q82_inverse(t);
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            const int qv = bm_nearest_int(__fmul_rn(v[k], id));
-            const int code = qv < -128 ? -128 : (qv > 127 ? 127 : qv);
-            isum += qv;
-            csum += code;
-            if (k < 4)
-                c0 |= (u32)(code & 0xff) << (8 * k);
-            else
-                c1 |= (u32)(code & 0xff) << (8 * (k - 4));
-        }
-    }
-    isum += (int)bm_dpp<kDppXor1>((u32)isum);
-    isum += (int)bm_dpp<kDppXor2>((u32)isum);
-    csum += (int)bm_dpp<kDppXor1>((u32)csum); // lanes (0,1): first 16 values, lanes (2,3): second
-    *reinterpret_cast<uint2 *>(group + 16 + 32 * ir + 8 * lane4) = make_uint2(c0, c1);
-    if ((lane4 & 1) == 0)
-        *reinterpret_cast<int *>(col + (size_t)nb * (BM_Q82_SB_REF + 64) + 4 * (2 * blk + (lane4 >> 1))) = csum;
-    if (lane4 == 0) {
-        *reinterpret_cast<unsigned short *>(group + 2 * ir) = (unsigned short)t;
-        *reinterpret_cast<unsigned short *>(group + 8 + 2 * ir) = (unsigned short)(short)isum;
-        const float d8 = bm_bf16_to_f32(t);
-        *reinterpret_cast<float2 *>(col + (size_t)nb * BM_Q82_SB_REF + 8 * blk) =
-            make_float2(d8, __fmul_rn(d8, (float)(short)isum));
-    }
 }
 
 // The gate . up . SwiGLU workgroup of the fused step: as k_gate_up's, except that it quantizes its token's f32 row

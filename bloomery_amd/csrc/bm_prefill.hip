@@ -100,7 +100,35 @@ __global__ __launch_bounds__(256) void k_swiglu_quant_q8k(const float *g, const 
     q8k_block_by_workgroup(v, act + ((size_t)col * bpc + blk) * BM_Q8K_STRIDE, fault, layer);
 }
 
+// The Q8_2_X4 form with eight values a thread, a block a quad of lanes: two 16-byte loads of each input a thread.
+__global__ __launch_bounds__(256) void k_swiglu_quant_wide(const float *g, const float *u, int m, int k, uint8_t *act,
+                                                           GateRule rule, u32 *fault, u32 layer) {
+    const long at = ((long)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (at >= (long)m * k) return;
+    const int col = (int)(at / k), o = (int)(at % k);
+    const float4 g0 = *reinterpret_cast<const float4 *>(g + at), g1 = *reinterpret_cast<const float4 *>(g + at + 4);
+    const float4 u0 = *reinterpret_cast<const float4 *>(u + at), u1 = *reinterpret_cast<const float4 *>(u + at + 4);
+    const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+    const float uv[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+    float v[8];
+    bool any_odd = false;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        bool odd;
+        v[i] = bm_gate_rule(rule.act, rule.limit, gv[i], uv[i], odd);
+        any_odd |= odd;
+    }
+    if (any_odd) bm_raise(fault, layer, kSiteF32Product);
+    q82_quad8(v, act + (size_t)col * (k / 256) * BM_Q82_SB_EXT, k / 256, o >> 5, threadIdx.x & 3, fault, layer);
+}
+
 hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act, bool q8k) {
+    if (!q8k && (((uintptr_t)g | (uintptr_t)u) & 15) == 0) {
+        const long threads = (long)m * k / 8;
+        hipLaunchKernelGGL(k_swiglu_quant_wide, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, L.stream, g, u, m, k, act,
+                           L.rule, L.fault, L.layer);
+        return hipGetLastError();
+    }
     if (q8k) {
         hipLaunchKernelGGL(k_swiglu_quant_q8k, dim3((unsigned)(m * (k / 256))), dim3(256), 0, L.stream, g, u, m, k, act, L.rule,
                            L.fault, L.layer);

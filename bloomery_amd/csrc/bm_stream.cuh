@@ -298,6 +298,56 @@ __device__ __forceinline__ void q82_store(uint8_t *col, int nb, int blk, int lan
     }
 }
 
+// One 32-value q8_2 block held eight values a lane by four consecutive lanes (the in-kernel token quantizer).
+__device__ __forceinline__ void q82_quad8(const float (&v)[8], uint8_t *col, int nb, int blk, int lane4, u32 *fault,
+                                          u32 layer) {
+    u32 ab = 0;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const u32 a = bm_f32_bits(v[k]) & 0x7fffffffu;
+        ab = a > ab ? a : ab;
+    }
+    u32 o;
+    o = bm_dpp<kDppXor1>(ab), ab = o > ab ? o : ab;
+    o = bm_dpp<kDppXor2>(ab), ab = o > ab ? o : ab;
+    uint8_t *group = col + (size_t)(blk >> 2) * BM_Q82X4_STRIDE;
+    const int ir = blk & 3;
+    u32 t;
+    int isum = 0, csum = 0;
+    u32 c0 = 0, c1 = 0;
+    if (ab > 0x7f7fffffu) {
+        t = 0x7fc0u;
+        if (lane4 == 0) bm_raise(fault, layer, kSiteQuantColumn);
+    } else {
+        t = bm_fp32_to_bf16_bits(__fdiv_rn(bm_bits_f32(ab), 127.0f));
+        const float id = bm_q82_inverse(t);
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int qv = bm_nearest_int(__fmul_rn(v[k], id));
+            const int code = qv < -128 ? -128 : (qv > 127 ? 127 : qv);
+            isum += qv;
+            csum += code;
+            if (k < 4)
+                c0 |= (u32)(code & 0xff) << (8 * k);
+            else
+                c1 |= (u32)(code & 0xff) << (8 * (k - 4));
+        }
+    }
+    isum += (int)bm_dpp<kDppXor1>((u32)isum);
+    isum += (int)bm_dpp<kDppXor2>((u32)isum);
+    csum += (int)bm_dpp<kDppXor1>((u32)csum); // lanes (0,1): first 16 values, lanes (2,3): second
+    *reinterpret_cast<uint2 *>(group + 16 + 32 * ir + 8 * lane4) = make_uint2(c0, c1);
+    if ((lane4 & 1) == 0)
+        *reinterpret_cast<int *>(col + (size_t)nb * (BM_Q82_SB_REF + 64) + 4 * (2 * blk + (lane4 >> 1))) = csum;
+    if (lane4 == 0) {
+        *reinterpret_cast<unsigned short *>(group + 2 * ir) = (unsigned short)t;
+        *reinterpret_cast<unsigned short *>(group + 8 + 2 * ir) = (unsigned short)(short)isum;
+        const float d8 = bm_bf16_to_f32(t);
+        *reinterpret_cast<float2 *>(col + (size_t)nb * BM_Q82_SB_REF + 8 * blk) =
+            make_float2(d8, __fmul_rn(d8, (float)(short)isum));
+    }
+}
+
 // The gate/up exchange of the eight lanes of an output: lanes 0..3 hold the gate dot, 4..7 the up dot.
 __device__ __forceinline__ float swiglu_of_pair(float v, int which, GateRule rule, u32 *fault, u32 layer) {
     // both moves run on every lane: a lane-crossing move under a divergent branch reads switched-off lanes as 0

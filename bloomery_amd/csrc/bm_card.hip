@@ -5,7 +5,7 @@
 // give the same values on this GPU: a 64-lane wave carries two of the rule's 32-lane walks, one row each, with every
 // lane's integer chain, f32 operations and the butterfly's order kept as the rule states them. The column planes lie
 // in value order: codes i8 [m][k], d8 f32 [m][k / 128], s8 i32 [m][k / 32].
-#include "bm_stream.cuh"
+#include "bm_stream.hpp"
 
 namespace bmk {
 

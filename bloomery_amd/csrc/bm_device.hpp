@@ -17,8 +17,8 @@
 //
 // Build: -ffp-contract=off (a product meets a sum in one rounding only where fmaf is written), f32 denormals
 // kept, correctly rounded f32 divide (hipcc's defaults for gfx950).
-#ifndef BM_DEVICE_CUH
-#define BM_DEVICE_CUH
+#ifndef BM_DEVICE_HPP
+#define BM_DEVICE_HPP
 
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
@@ -1138,4 +1138,4 @@ __device__ __forceinline__ float bm_gate_rule(u32 act, float limit, float g, flo
     return bm_swiglu_gclamp(g, u, limit);
 }
 
-#endif // BM_DEVICE_CUH
+#endif // BM_DEVICE_HPP

@@ -3,7 +3,7 @@
 // expert, expert e's run is order[start[e] .. start[e + 1]], and the tile table cuts every run into tiles of up to
 // eight consecutive entries, tile g the word (e << 22) | j at tiles[1 + g], their count at tiles[0]. Every slot's
 // value is its slot-by-slot launch's, bit for bit: a column of the multi-column dot is the one-column dot.
-#include "bm_stream.cuh"
+#include "bm_stream.hpp"
 
 namespace bmk {
 

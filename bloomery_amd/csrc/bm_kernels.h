@@ -30,7 +30,7 @@ constexpr int kMaxLds = 160 * 1024;
 hipError_t fill_u32(const Launch &L, uint32_t *dst, uint32_t value, size_t n);
 
 // Bytes of one activation column of k values on the device, in the form weight type `wtype` dots against: the CPU
-// path's bytes, and for the Q8_2_X4 form two tables after them (bm_device.cuh).
+// path's bytes, and for the Q8_2_X4 form two tables after them (bm_device.hpp).
 int act_col_bytes(int wtype, int k);
 
 // `live` (optional): a device word holding how many of the m columns to quantize; the rest keep what they held.

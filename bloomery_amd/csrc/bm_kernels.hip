@@ -3,7 +3,7 @@
 // its fused forms, and the block-sum verification kernel.
 #include "bm_kernels.h"
 
-#include "bm_stream.cuh"
+#include "bm_stream.hpp"
 
 namespace bmk {
 

@@ -7,7 +7,7 @@
 // refused count}.
 //
 // The GEMM's numbers are the decode path's, bit for bit: every (row, slot) value is the one-column row dot of
-// bm_device.cuh. The integer sums of each 16-value group come out of v_mfma_i32_16x16x32_i8 (16 rows x 16 slots,
+// bm_device.hpp. The integer sums of each 16-value group come out of v_mfma_i32_16x16x32_i8 (16 rows x 16 slots,
 // exact; the other half of the 32 values zeroed on the weight side), and each enters the f32 accumulator of the CPU path's lane that
 // owns it, in the CPU path's order (crates/qdot/src/lib.rs:4363-4447 Q4_K, :4776-4874 Q6_K): eight accumulators a
 // value, the min term first, then the groups in increasing k, and the closing sum (t0 + t2) + (t1 + t3).
@@ -16,7 +16,7 @@
 // by that arithmetic, not by the matrix cores.
 #include <type_traits>
 
-#include "bm_stream.cuh"
+#include "bm_stream.hpp"
 
 namespace bmk {
 

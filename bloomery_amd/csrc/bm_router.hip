@@ -13,7 +13,7 @@
 //
 // A token with a logit that is not finite has no defined routing: it raises Router on the fault word, gets NaN
 // probabilities and weights, and keeps its ids as they stand (crates/gpu/src/route_softmax.rs:53-62).
-#include "bm_stream.cuh"
+#include "bm_stream.hpp"
 
 namespace bmk {
 

@@ -1,7 +1,7 @@
 // Shared device pieces of the dot kernels: staging of activation columns and IQ2_XXS tables into LDS, the register
 // ring a weight row streams through, the Q8_2 block quantizer, and the host-side variant dispatch.
 //
-// Every dot kernel follows one plan: a quad of lanes per weight row (bm_device.cuh); the token's quantized
+// Every dot kernel follows one plan: a quad of lanes per weight row (bm_device.hpp); the token's quantized
 // activation column requested first, then the row's super-blocks (128-bit loads) through a small ring of
 // registers, a few super-blocks ahead of the arithmetic, all from straight-line code so the hardware's in-order
 // load counter lets the arithmetic of one super-block run while the later ones are still in flight. Weights are
@@ -10,15 +10,15 @@
 // Variants: a kernel is instantiated per weight type and per (U, NB): U the ring's size in super-blocks, NB the
 // row's super-block count when it is known at compile time (0: a run-time count that U divides). The hot shapes
 // (Q4_K rows of 2048 values, Q6_K rows of 768) have NB set and their stages unrolled.
-#ifndef BM_STREAM_CUH
-#define BM_STREAM_CUH
+#ifndef BM_STREAM_HPP
+#define BM_STREAM_HPP
 
 #include "bm_kernels.h"
 
 #define BM_TABLE_QUAL static __device__ const
 #include "iq2xxs_tables.h"
 
-#include "bm_device.cuh"
+#include "bm_device.hpp"
 
 namespace bmk {
 
@@ -586,4 +586,4 @@ static inline int tab_bytes_rt(int wtype) { return wtype == BM_IQ2XXS ? kTabByte
 
 } // namespace bmk
 
-#endif // BM_STREAM_CUH
+#endif // BM_STREAM_HPP

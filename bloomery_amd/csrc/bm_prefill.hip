@@ -470,9 +470,30 @@ __host__ __device__ constexpr int fast_units() { // scaled units a super-block
 }
 template <int WT>
 __host__ __device__ constexpr size_t fast_lds_bytes() {
-    return sizeof(GemmLds) + (size_t)(kGemmBN + kFastRows) * fast_code_stride<WT>() + 2 * 8 * kFastColLine * sizeof(float) +
-           2 * (size_t)fast_units<WT>() * kFastRowLine * sizeof(float);
+    // codes of both sides; the columns' scale operands ([block][half of the lanes][slot], 8 bytes) and d8 * isum; the rows'
+    // scale operands ([unit][row], 8 bytes) and mins
+    constexpr bool mins = WT != BM_Q6K;
+    return sizeof(GemmLds) + (size_t)(kGemmBN + kFastRows) * fast_code_stride<WT>() + 2 * 8 * kFastColLine * 8 +
+           (mins ? 8 * kFastColLine * sizeof(float) : 0) + (size_t)fast_units<WT>() * kFastRowLine * (8 + (mins ? sizeof(float) : 0));
 }
+
+// The product of a row's scale and a column's d8 for a whole 32 x 32 tile is an outer product, so it goes to the matrix
+// cores too: v_mfma_f32_32x32x8_bf16_1k over K slots that hold the row scale as three bf16 pieces (8 + 8 + 8 bits: the
+// f32 exactly) against the column's d8 (a bf16 value as it stands) in the same three slots. Each of the three products
+// is exact in f32; their sum is the f32 product to within a rounding. Lanes 32 .. 63 carry K slots 4 .. 7: the column
+// side holds zeros there.
+__device__ __forceinline__ uint2 scale_operand_row(float v) {
+    const u32 hi = bm_f32_bits(v) & 0xffff0000u;
+    const float r1 = v - bm_bits_f32(hi);
+    const u32 mid = bm_f32_bits(r1) & 0xffff0000u;
+    const float r2 = r1 - bm_bits_f32(mid);
+    return make_uint2((hi >> 16) | mid, bm_f32_bits(r2) >> 16);
+}
+__device__ __forceinline__ uint2 scale_operand_col(u32 d8_bits) {
+    const u32 h = d8_bits >> 16;
+    return make_uint2(h | (h << 16), h);
+}
+typedef short v4s __attribute__((ext_vector_type(4)));
 
 template <int WT>
 __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
@@ -485,10 +506,10 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
     GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
     uint8_t *a_codes = lds + sizeof(GemmLds);
     uint8_t *w_codes = a_codes + (size_t)kGemmBN * kStride;
-    float *d8_t = reinterpret_cast<float *>(w_codes + (size_t)kFastRows * kStride);
-    float *my_t = d8_t + 8 * kFastColLine;
-    float *sv_t = my_t + 8 * kFastColLine;
-    float *mn_t = sv_t + kUnitsSb * kFastRowLine; // Q4_K, Q5_K only
+    uint2 *d8_t = reinterpret_cast<uint2 *>(w_codes + (size_t)kFastRows * kStride); // [block][lane / 32][slot]
+    uint2 *sv_t = d8_t + 2 * 8 * kFastColLine;                                       // [unit][row]
+    float *my_t = reinterpret_cast<float *>(sv_t + kUnitsSb * kFastRowLine);
+    float *mn_t = my_t + 8 * kFastColLine; // Q4_K, Q5_K only
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const u32 g = tile_of_block(blockIdx.x, n_slabs);
     const int row0 = (int)slab_of_block(blockIdx.x, n_slabs) * kFastRows;
@@ -516,7 +537,9 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
     //   four 16-byte pieces of column codes (column tid / 16 + 16 j, piece tid % 16 of the sixteen: a column's
     //   super-block is two groups of 144 bytes whose first 16 are scales and sums, skipped here),
     //   one 16-byte piece of two (d8, d8 * isum) pairs (column tid / 4, pairs 2 (tid % 4) ..),
-    //   half a weight row (row tid / 2): its half of the codes and what the row's scales need
+    //   what the scales of half a weight row need (row tid / 2),
+    //   four 16-byte pieces of weight codes (row tid / 8 + 32 j, piece tid % 8 of the row's eight: eight consecutive lanes
+    //   read 128 consecutive bytes, so a wave's load touches eight rows' lines, not sixty-four)
     const int ac = tid >> 4, ap = tid & 15;
     u32 src_a[4];
 #pragma unroll
@@ -526,7 +549,16 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
     const int wr = tid >> 1, wh = tid & 1;
     const uint8_t *we = w + (size_t)e * rpe * row_bytes;
     const u32 src_w = (u32)(row0 + wr < rpe ? row0 + wr : rpe - 1) * row_bytes;
-    uint4 ra0, ra1, ra2, ra3, rp, rq[4], rh, rx0, rx1;
+    const int crow = tid >> 3, cc = tid & 7;
+    constexpr int kCodesAt = WT == BM_Q5K ? 48 : WT == BM_Q4K ? 16 : 0;
+    u32 src_c[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        src_c[j] = (u32)(row0 + crow + 32 * j < rpe ? row0 + crow + 32 * j : rpe - 1) * row_bytes + kCodesAt + 16u * (u32)cc;
+    // the bytes that carry the high bits of piece cc, from the piece's own address: Q5_K's 32 high-bit bytes (value n's
+    // fifth bit is bit n / 32 of byte n % 32), Q6_K's qh (piece cc of ql goes with qh piece cc % 2 of its half)
+    const int high_at = WT == BM_Q5K ? 16 * (cc & 1) - 32 - 16 * cc : 128 + 32 * (cc >> 2) + 16 * (cc & 1) - 16 * cc;
+    uint4 ra0, ra1, ra2, ra3, rp, rq[4], rh, rx[WT == BM_Q4K ? 1 : 4];
     auto fetch = [&](int i) {
         ra0 = *reinterpret_cast<const uint4 *>(act + (src_a[0] + (u32)i * BM_Q82_SB_REF));
         ra1 = *reinterpret_cast<const uint4 *>(act + (src_a[1] + (u32)i * BM_Q82_SB_REF));
@@ -535,21 +567,22 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
         rp = *reinterpret_cast<const uint4 *>(act + (src_p + (u32)i * 64u));
         const uint8_t *blk = we + (src_w + (u32)i * kBlock);
         if constexpr (kQ45) {
-            constexpr int kCodesAt = WT == BM_Q5K ? 48 : 16;
             rh = *reinterpret_cast<const uint4 *>(blk); // d, dmin, the twelve scale bytes
 #pragma unroll
-            for (int c = 0; c < 4; c++) rq[c] = *reinterpret_cast<const uint4 *>(blk + kCodesAt + 64 * wh + 16 * c);
-            if constexpr (WT == BM_Q5K) { // the 32 high-bit bytes: value n's fifth bit is bit n / 32 of byte n % 32
-                rx0 = *reinterpret_cast<const uint4 *>(blk + 16);
-                rx1 = *reinterpret_cast<const uint4 *>(blk + 32);
+            for (int j = 0; j < 4; j++) {
+                const uint8_t *piece = we + (src_c[j] + (u32)i * kBlock);
+                rq[j] = *reinterpret_cast<const uint4 *>(piece);
+                if constexpr (WT == BM_Q5K) rx[j] = *reinterpret_cast<const uint4 *>(piece + high_at);
             }
-        } else { // half wh of the block: ql bytes 64 wh .. (four pieces), qh bytes 32 wh .. (two), the sixteen scales, d
+        } else {
 #pragma unroll
-            for (int c = 0; c < 4; c++) rq[c] = bm_ld16u(blk + 64 * wh + 16 * c);
-            rx0 = bm_ld16u(blk + 128 + 32 * wh);
-            rx1 = bm_ld16u(blk + 128 + 32 * wh + 16);
-            rh = bm_ld16u(blk + 192);
-            rh.x = wh ? rh.z : rh.x; // this half's eight scale bytes
+            for (int j = 0; j < 4; j++) {
+                const uint8_t *piece = we + (src_c[j] + (u32)i * kBlock);
+                rq[j] = bm_ld16u(piece);
+                rx[j] = bm_ld16u(piece + high_at);
+            }
+            rh = bm_ld16u(blk + 192); // the sixteen scales
+            rh.x = wh ? rh.z : rh.x;  // this half's eight scale bytes
             rh.y = wh ? rh.w : rh.y;
             rh.z = bm_ld2u(blk + 208); // d
         }
@@ -568,25 +601,24 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
         put16(acol + 16 * kStride, ra1.x, ra1.y, ra1.z, ra1.w);
         put16(acol + 32 * kStride, ra2.x, ra2.y, ra2.z, ra2.w);
         put16(acol + 48 * kStride, ra3.x, ra3.y, ra3.z, ra3.w);
-        d8_t[(2 * pp) * kFastColLine + pcol] = bm_bits_f32(rp.x);
-        d8_t[(2 * pp + 1) * kFastColLine + pcol] = bm_bits_f32(rp.z);
+        d8_t[(2 * (2 * pp)) * kFastColLine + pcol] = scale_operand_col(rp.x);
+        d8_t[(2 * (2 * pp + 1)) * kFastColLine + pcol] = scale_operand_col(rp.z);
         if constexpr (kQ45) {
             my_t[(2 * pp) * kFastColLine + pcol] = bm_bits_f32(rp.y);
             my_t[(2 * pp + 1) * kFastColLine + pcol] = bm_bits_f32(rp.w);
         }
         const u32 ml = 0x0f0f0f0fu;
-        uint8_t *row = w_codes + wr * kStride;
         if constexpr (kQ45) {
-            // nibble piece c of this half: code bytes 64 wh + 16 c ..: the low nibbles are sub-block 2 p, values
-            // 16 (c % 2) .., the high nibbles sub-block 2 p + 1, the same values, with p = 2 wh + c / 2
+            // nibble piece cc of a row: code bytes 16 cc ..: the low nibbles are sub-block 2 p, values 16 (cc % 2) .., the
+            // high nibbles sub-block 2 p + 1, the same values, with p = cc / 2
+            const int p = cc >> 1, at = 16 * (cc & 1);
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const int p = 2 * wh + (c >> 1), at = 16 * (c & 1);
-                u32 lo[4] = {rq[c].x & ml, rq[c].y & ml, rq[c].z & ml, rq[c].w & ml};
-                u32 hi[4] = {(rq[c].x >> 4) & ml, (rq[c].y >> 4) & ml, (rq[c].z >> 4) & ml, (rq[c].w >> 4) & ml};
-                if constexpr (WT == BM_Q5K) { // high-bit bytes 16 (c % 2) ..: bit 2 p for the low nibbles, 2 p + 1 for the high
-                    const uint4 hb = (c & 1) ? rx1 : rx0;
-                    const u32 hw[4] = {hb.x, hb.y, hb.z, hb.w};
+            for (int j = 0; j < 4; j++) {
+                uint8_t *row = w_codes + (crow + 32 * j) * kStride;
+                u32 lo[4] = {rq[j].x & ml, rq[j].y & ml, rq[j].z & ml, rq[j].w & ml};
+                u32 hi[4] = {(rq[j].x >> 4) & ml, (rq[j].y >> 4) & ml, (rq[j].z >> 4) & ml, (rq[j].w >> 4) & ml};
+                if constexpr (WT == BM_Q5K) { // high-bit bytes 16 (cc % 2) ..: bit 2 p for the low nibbles, 2 p + 1 for the high
+                    const u32 hw[4] = {rx[j].x, rx[j].y, rx[j].z, rx[j].w};
                     const u32 one = 0x01010101u;
 #pragma unroll
                     for (int k = 0; k < 4; k++) {
@@ -604,32 +636,35 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
                 const u32 qa = (rh.y >> (8 * jj)) & 0xffu, qb = (rh.z >> (8 * jj)) & 0xffu, qc = (rh.w >> (8 * jj)) & 0xffu;
                 const u32 scv = wh ? ((qc & 15u) | ((qa >> 6) << 4)) : (qa & 63u);
                 const u32 mv = wh ? ((qc >> 4) | ((qb >> 6) << 4)) : (qb & 63u);
-                sv_t[(4 * wh + jj) * kFastRowLine + wr] = d * (float)scv;
+                sv_t[(4 * wh + jj) * kFastRowLine + wr] = scale_operand_row(d * (float)scv);
                 mn_t[(4 * wh + jj) * kFastRowLine + wr] = -(dmin * (float)mv);
             }
         } else {
-            // ql piece c of this half (bytes 64 wh + 16 c ..) with qh piece c % 2: the low nibbles are quarter c / 2 of the
-            // half, values 16 (c % 2) .., the high nibbles quarter 2 + c / 2; a quarter's high bits are bits 2 a .. of qh
-            // (crates/gguf/src/quant.rs:826-859). Each is one 16-value group: group 8 wh + 2 a + c % 2.
+            // ql piece cc of a row (bytes 16 cc ..: half cc / 4, piece c = cc % 4 of it) with qh piece c % 2 of that half: the
+            // low nibbles are quarter c / 2 of the half, values 16 (c % 2) .., the high nibbles quarter 2 + c / 2; a quarter's
+            // high bits are bits 2 a .. of qh (crates/gguf/src/quant.rs:826-859). Each is one 16-value group: group
+            // 8 (cc / 4) + 2 a + c % 2.
             const u32 mh = 0x03030303u;
+            const int half = cc >> 2, c = cc & 3;
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const uint4 hq = (c & 1) ? rx1 : rx0;
+            for (int j = 0; j < 4; j++) {
+                uint8_t *row = w_codes + (crow + 32 * j) * kStride;
+                const uint4 hq = rx[j];
 #pragma unroll
                 for (int hn = 0; hn < 2; hn++) {
                     const int a4 = (c >> 1) + 2 * hn, ns = 4 * hn, hs = 2 * a4;
-                    put16(row + 128 * wh + 32 * a4 + 16 * (c & 1),
-                          q6_minus_32(((rq[c].x >> ns) & ml) | (((hq.x >> hs) & mh) << 4)),
-                          q6_minus_32(((rq[c].y >> ns) & ml) | (((hq.y >> hs) & mh) << 4)),
-                          q6_minus_32(((rq[c].z >> ns) & ml) | (((hq.z >> hs) & mh) << 4)),
-                          q6_minus_32(((rq[c].w >> ns) & ml) | (((hq.w >> hs) & mh) << 4)));
+                    put16(row + 128 * half + 32 * a4 + 16 * (c & 1),
+                          q6_minus_32(((rq[j].x >> ns) & ml) | (((hq.x >> hs) & mh) << 4)),
+                          q6_minus_32(((rq[j].y >> ns) & ml) | (((hq.y >> hs) & mh) << 4)),
+                          q6_minus_32(((rq[j].z >> ns) & ml) | (((hq.z >> hs) & mh) << 4)),
+                          q6_minus_32(((rq[j].w >> ns) & ml) | (((hq.w >> hs) & mh) << 4)));
                 }
             }
             const float d = bm_half_to_f32(rh.z & 0xffffu);
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) {
                 const u32 word = jj < 4 ? rh.x : rh.y;
-                sv_t[(8 * wh + jj) * kFastRowLine + wr] = d * (float)(int)(signed char)((word >> (8 * (jj & 3))) & 0xffu);
+                sv_t[(8 * wh + jj) * kFastRowLine + wr] = scale_operand_row(d * (float)(int)(signed char)((word >> (8 * (jj & 3))) & 0xffu));
             }
         }
     };
@@ -638,7 +673,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
     const int l32 = lane & 31, kh = lane >> 5;
     const uint8_t *my_w = w_codes + (32 * wv + l32) * kStride + kOp * kh;
     const uint8_t *my_a = a_codes + l32 * kStride + kOp * kh;
-    const float *my_sv = sv_t + 32 * wv + 4 * kh;
+    const uint2 *my_sv = sv_t + 32 * wv + l32;
+    const uint2 *my_d8 = d8_t + kh * kFastColLine + l32;
     const bool two = len > 32; // else the second half of the slots is all padding
     v16f acc[2];
 #pragma unroll
@@ -646,24 +682,25 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[t][v] = 0.0f;
 
-    // One super-block's products. A step is a (unit, half of the slots).
+    // One super-block's products. A step is a (unit, half of the slots): its integer sums (one matrix instruction, issued a
+    // step ahead), its scale products (another, issued at the end of the step before, behind that step's last use of the
+    // one buffer), and on the vector ALU the sums to floats and the multiply-adds: two operations a (row, slot, unit).
     auto blocks = [&](auto two_tiles) __attribute__((always_inline)) {
         constexpr bool kTwo = decltype(two_tiles)::value;
         constexpr int kSteps = (kTwo ? 2 : 1) * kUnitsSb;
         typedef typename std::conditional<kQ45, v4i, long>::type Operand;
         Operand a[2], b[2];
-        float4 sv[2][4];
-        float d8[3];
+        uint2 sa[2], sb[3];
         v16i sum[2];
-        auto rd_a = [&](int un) { a[un & 1] = *reinterpret_cast<const Operand *>(my_w + 2 * kOp * un); };
-        auto rd_sv = [&](int un) {
-#pragma unroll
-            for (int q4 = 0; q4 < 4; q4++) sv[un & 1][q4] = *reinterpret_cast<const float4 *>(my_sv + un * kFastRowLine + 8 * q4);
+        v16f pr;
+        auto rd_a = [&](int un) {
+            a[un & 1] = *reinterpret_cast<const Operand *>(my_w + 2 * kOp * un);
+            sa[un & 1] = my_sv[un * kFastRowLine];
         };
         auto rd_b = [&](int u) { // step u's column operand and column scale
             const int un = kTwo ? u >> 1 : u, t = kTwo ? u & 1 : 0;
             b[u & 1] = *reinterpret_cast<const Operand *>(my_a + 32 * t * kStride + 2 * kOp * un);
-            d8[u % 3] = d8_t[(kQ45 ? un : un >> 1) * kFastColLine + 32 * t + l32];
+            sb[u % 3] = my_d8[2 * (kQ45 ? un : un >> 1) * kFastColLine + 32 * t];
         };
         auto product = [&](int u) {
             const int un = kTwo ? u >> 1 : u;
@@ -671,34 +708,34 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
             if constexpr (kQ45) sum[u & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[un & 1], b[u & 1], z, 0, 0, 0);
             else sum[u & 1] = __builtin_amdgcn_mfma_i32_32x32x16_i8(a[un & 1], b[u & 1], z, 0, 0, 0);
         };
+        auto scales = [&](int u) {
+            const int un = kTwo ? u >> 1 : u;
+            const v16f z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            pr = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(v4s, sa[un & 1]), __builtin_bit_cast(v4s, sb[u % 3]), z, 0,
+                                                         0, 0);
+        };
         rd_a(0);
         rd_b(0);
-        rd_sv(0);
         product(0);
+        scales(0);
         rd_b(1);
-        if (!kTwo) rd_a(1);
+        rd_a(1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < kSteps; u++) {
             const int un = kTwo ? u >> 1 : u, t = kTwo ? u & 1 : 0;
             if (u + 1 < kSteps) product(u + 1);
             if (u + 2 < kSteps) rd_b(u + 2);
-            // the row side of the unit after: its codes before its first product is issued (the next step), its scales
-            // before its first scaling
-            if (kTwo && t == 0 && un + 1 < kUnitsSb) rd_a(un + 1);
-            if (!kTwo && un + 2 < kUnitsSb) rd_a(un + 2);
-            if ((!kTwo || t == 1) && un + 1 < kUnitsSb) rd_sv(un + 1);
+            // the row side two units on, into the buffer of this unit, whose last instructions have been issued
+            if ((!kTwo || t == 1) && un + 2 < kUnitsSb) rd_a(un + 2);
             __builtin_amdgcn_sched_barrier(0);
-            const float dc = d8[u % 3];
+            float f[16];
 #pragma unroll
-            for (int q4 = 0; q4 < 4; q4++) {
-                const float4 r = sv[un & 1][q4];
-                acc[t][4 * q4 + 0] = fmaf(r.x * dc, (float)sum[u & 1][4 * q4 + 0], acc[t][4 * q4 + 0]);
-                acc[t][4 * q4 + 1] = fmaf(r.y * dc, (float)sum[u & 1][4 * q4 + 1], acc[t][4 * q4 + 1]);
-                acc[t][4 * q4 + 2] = fmaf(r.z * dc, (float)sum[u & 1][4 * q4 + 2], acc[t][4 * q4 + 2]);
-                acc[t][4 * q4 + 3] = fmaf(r.w * dc, (float)sum[u & 1][4 * q4 + 3], acc[t][4 * q4 + 3]);
-            }
+            for (int v = 0; v < 16; v++) f[v] = (float)sum[u & 1][v];
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[t][v] = fmaf(pr[v], f[v], acc[t][v]);
             __builtin_amdgcn_sched_barrier(0);
+            if (u + 1 < kSteps) scales(u + 1);
         }
         if constexpr (kQ45) {
             // the min terms last, into the same accumulators: a 32 x 8 by 8 x 32 product in f32, two of the eight
@@ -713,6 +750,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
         }
     };
 
+    for (int i = tid; i < 8 * kGemmBN; i += 256) d8_t[(2 * (i / kGemmBN) + 1) * kFastColLine + i % kGemmBN] = make_uint2(0u, 0u);
     fetch(0);
     for (int i = 0; i < nb; i++) {
         if (i) __syncthreads(); // the readers of the super-block before are done

@@ -445,19 +445,24 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 //         are a product of two thin matrices and go to v_mfma_f32_32x32x2_f32 (four a super-block), into the same
 //         accumulators;
 //   Q6_K: a 16-value group, whose scale is its own, is one v_mfma_i32_32x32x16_i8.
-// What is left for the vector ALU is three operations a (row, slot, unit): the integer to a float, the row's d * sc times
-// the column's d8, the multiply-add into the one accumulator a value (the CPU path keeps eight and a fixed order: that
-// is the exact mode; this one differs from it by f32 rounding only).
-// A workgroup of four waves takes 128 rows and a tile's 64 slots; wave w owns rows 32 w .. and both halves of the slots,
-// so a unit's weight operand and its sixteen row scales are read from LDS once for two products. LDS holds one
-// super-block: the columns' codes, the slab's codes unpacked to a signed byte each, and the scale tables transposed so
-// that a lane's four consecutive result rows are one 16-byte read. Two workgroups share a CU and fill each other's
-// staging gaps; the next super-block's global loads are in flight during the arithmetic on the present one. Inside a
-// wave a unit's matrix instruction is issued one unit ahead of the vector work that scales its sums, and its LDS
-// operands are read two units ahead.
+// The product of a row's scale and a column's d8 for a whole 32 x 32 tile is an outer product, so it goes to the matrix
+// cores too: v_mfma_f32_32x32x8_bf16_1k over K slots that hold the row scale as three bf16 pieces (8 + 8 + 8 bits: the
+// f32 exactly) against the column's d8 (a bf16 value as it stands) in the same three slots. Each of the three products
+// is exact in f32; their sum is the f32 product to within a rounding. Lanes 32 .. 63 carry K slots 4 .. 7: the row side
+// reads a zero there.
+// What is left for the vector ALU is two operations a (row, slot, unit): the integer to a float and the multiply-add into
+// the one accumulator a value (the CPU path keeps eight and a fixed order: that is the exact mode; this one differs from
+// it by f32 rounding only).
+// A workgroup of eight waves takes 128 rows and a tile's 64 slots, a wave 32 x 32 of them. LDS holds one super-block: the
+// columns' codes, the slab's codes unpacked to a signed byte each, and the scale operands; 72 KB and at most 128 registers,
+// so two workgroups, four waves a SIMD, share a CU and fill each other's staging gaps and waits (a wave alone issues a
+// vector instruction every five to six cycles, the SIMD takes one every four). The next super-block's global loads are in flight during the
+// arithmetic on the present one. Inside a wave a unit's matrix instructions are issued one unit ahead of the vector work
+// on their results, and its LDS operands are read two units ahead.
 constexpr int kFastRows = 128;
-constexpr int kFastRowLine = kFastRows + 4; // floats a line of the row tables ([unit][row])
-constexpr int kFastColLine = kGemmBN + 4;   // floats a line of the column tables ([block][slot])
+constexpr int kFastThreads = 512;
+constexpr int kFastRowLine = kFastRows + 4; // entries a line of the row tables ([unit][row]); entry kFastRows of a line holds zero
+constexpr int kFastColLine = kGemmBN + 4;   // entries a line of the column tables ([block][slot])
 // a row's or a column's 256 codes, padded so that the operand reads of consecutive rows fall on different banks: the
 // reads are 16 bytes a lane for K = 32 and 8 bytes a lane for K = 16
 template <int WT>
@@ -470,18 +475,13 @@ __host__ __device__ constexpr int fast_units() { // scaled units a super-block
 }
 template <int WT>
 __host__ __device__ constexpr size_t fast_lds_bytes() {
-    // codes of both sides; the columns' scale operands ([block][half of the lanes][slot], 8 bytes) and d8 * isum; the rows'
-    // scale operands ([unit][row], 8 bytes) and mins
+    // codes of both sides; the columns' scale operands ([block][slot], 8 bytes) and d8 * isum; the rows' scale operands
+    // ([unit][row], 8 bytes) and mins
     constexpr bool mins = WT != BM_Q6K;
-    return sizeof(GemmLds) + (size_t)(kGemmBN + kFastRows) * fast_code_stride<WT>() + 2 * 8 * kFastColLine * 8 +
-           (mins ? 8 * kFastColLine * sizeof(float) : 0) + (size_t)fast_units<WT>() * kFastRowLine * (8 + (mins ? sizeof(float) : 0));
+    return sizeof(GemmLds) + (size_t)(kGemmBN + kFastRows) * fast_code_stride<WT>() + 8 * kFastColLine * (8 + (mins ? sizeof(float) : 0)) +
+           (size_t)fast_units<WT>() * kFastRowLine * (8 + (mins ? sizeof(float) : 0));
 }
 
-// The product of a row's scale and a column's d8 for a whole 32 x 32 tile is an outer product, so it goes to the matrix
-// cores too: v_mfma_f32_32x32x8_bf16_1k over K slots that hold the row scale as three bf16 pieces (8 + 8 + 8 bits: the
-// f32 exactly) against the column's d8 (a bf16 value as it stands) in the same three slots. Each of the three products
-// is exact in f32; their sum is the f32 product to within a rounding. Lanes 32 .. 63 carry K slots 4 .. 7: the column
-// side holds zeros there.
 __device__ __forceinline__ uint2 scale_operand_row(float v) {
     const u32 hi = bm_f32_bits(v) & 0xffff0000u;
     const float r1 = v - bm_bits_f32(hi);
@@ -496,7 +496,7 @@ __device__ __forceinline__ uint2 scale_operand_col(u32 d8_bits) {
 typedef short v4s __attribute__((ext_vector_type(4)));
 
 template <int WT>
-__global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
+__global__ __launch_bounds__(kFastThreads, 2) void k_gemm_fast(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
                                                       const u32 *tiles, const u32 *n_tiles, u32 n_slabs, u32 slot_div,
                                                       u32 n_slots, float *y) {
     constexpr bool kQ45 = WT == BM_Q4K || WT == BM_Q5K;
@@ -506,10 +506,10 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
     GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
     uint8_t *a_codes = lds + sizeof(GemmLds);
     uint8_t *w_codes = a_codes + (size_t)kGemmBN * kStride;
-    uint2 *d8_t = reinterpret_cast<uint2 *>(w_codes + (size_t)kFastRows * kStride); // [block][lane / 32][slot]
-    uint2 *sv_t = d8_t + 2 * 8 * kFastColLine;                                       // [unit][row]
-    float *my_t = reinterpret_cast<float *>(sv_t + kUnitsSb * kFastRowLine);
-    float *mn_t = my_t + 8 * kFastColLine; // Q4_K, Q5_K only
+    uint2 *d8_t = reinterpret_cast<uint2 *>(w_codes + (size_t)kFastRows * kStride); // [block][slot]
+    uint2 *sv_t = d8_t + 8 * kFastColLine;                                           // [unit][row]
+    float *my_t = reinterpret_cast<float *>(sv_t + kUnitsSb * kFastRowLine);         // Q4_K, Q5_K only, as is mn_t
+    float *mn_t = my_t + 8 * kFastColLine;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const u32 g = tile_of_block(blockIdx.x, n_slabs);
     const int row0 = (int)slab_of_block(blockIdx.x, n_slabs) * kFastRows;
@@ -517,7 +517,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
     if (g > count) return;
     if (g == count) { // the refused slots' rows: NaN (crates/gpu/src/gemm/grouped.rs:2283-2287)
         const u32 refused = n_tiles[1];
-        for (u32 i = tid; i < refused * kFastRows; i += 256) {
+        for (u32 i = tid; i < refused * kFastRows; i += kFastThreads) {
             const u32 s = cols[n_slots - refused + i / kFastRows];
             const int r = row0 + (int)(i % kFastRows);
             if (r < rpe) y[(size_t)s * rpe + r] = bm_bits_f32(0x7fc00000u);
@@ -531,60 +531,57 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
         tab->slot[tid] = s;
         tab->col[tid] = s / slot_div;
     }
+    if (tid < kUnitsSb) sv_t[tid * kFastRowLine + kFastRows] = make_uint2(0u, 0u);
     __syncthreads();
     const u32 row_bytes = (u32)nb * kBlock, col_bytes = (u32)nb * BM_Q82_SB_EXT;
     // what this thread stages of every super-block:
-    //   four 16-byte pieces of column codes (column tid / 16 + 16 j, piece tid % 16 of the sixteen: a column's
+    //   two 16-byte pieces of column codes (column tid / 16 + 32 j, piece tid % 16 of the sixteen: a column's
     //   super-block is two groups of 144 bytes whose first 16 are scales and sums, skipped here),
-    //   one 16-byte piece of two (d8, d8 * isum) pairs (column tid / 4, pairs 2 (tid % 4) ..),
-    //   what the scales of half a weight row need (row tid / 2),
-    //   four 16-byte pieces of weight codes (row tid / 8 + 32 j, piece tid % 8 of the row's eight: eight consecutive lanes
-    //   read 128 consecutive bytes, so a wave's load touches eight rows' lines, not sixty-four)
+    //   one (d8, d8 * isum) pair (column tid / 8, block tid % 8),
+    //   two 16-byte pieces of weight codes (row tid / 8 + 64 j, piece tid % 8 of the row's eight: eight consecutive lanes
+    //   read 128 consecutive bytes),
+    //   a quarter of a weight row's scales (row tid / 4)
     const int ac = tid >> 4, ap = tid & 15;
-    u32 src_a[4];
+    u32 src_a[2];
 #pragma unroll
-    for (int j = 0; j < 4; j++) src_a[j] = tab->col[ac + 16 * j] * col_bytes + 16u * (u32)(1 + ap + (ap >> 3));
-    const int pcol = tid >> 2, pp = tid & 3;
-    const u32 src_p = tab->col[pcol] * col_bytes + (u32)nb * BM_Q82_SB_REF + 16u * (u32)pp;
-    const int wr = tid >> 1, wh = tid & 1;
+    for (int j = 0; j < 2; j++) src_a[j] = tab->col[ac + 32 * j] * col_bytes + 16u * (u32)(1 + ap + (ap >> 3));
+    const int pcol = tid >> 3, pb = tid & 7;
+    const u32 src_p = tab->col[pcol] * col_bytes + (u32)nb * BM_Q82_SB_REF + 8u * (u32)pb;
+    const int wr = tid >> 2, wq = tid & 3;
     const uint8_t *we = w + (size_t)e * rpe * row_bytes;
     const u32 src_w = (u32)(row0 + wr < rpe ? row0 + wr : rpe - 1) * row_bytes;
     const int crow = tid >> 3, cc = tid & 7;
     constexpr int kCodesAt = WT == BM_Q5K ? 48 : WT == BM_Q4K ? 16 : 0;
-    u32 src_c[4];
+    u32 src_c[2];
 #pragma unroll
-    for (int j = 0; j < 4; j++)
-        src_c[j] = (u32)(row0 + crow + 32 * j < rpe ? row0 + crow + 32 * j : rpe - 1) * row_bytes + kCodesAt + 16u * (u32)cc;
+    for (int j = 0; j < 2; j++)
+        src_c[j] = (u32)(row0 + crow + 64 * j < rpe ? row0 + crow + 64 * j : rpe - 1) * row_bytes + kCodesAt + 16u * (u32)cc;
     // the bytes that carry the high bits of piece cc, from the piece's own address: Q5_K's 32 high-bit bytes (value n's
     // fifth bit is bit n / 32 of byte n % 32), Q6_K's qh (piece cc of ql goes with qh piece cc % 2 of its half)
     const int high_at = WT == BM_Q5K ? 16 * (cc & 1) - 32 - 16 * cc : 128 + 32 * (cc >> 2) + 16 * (cc & 1) - 16 * cc;
-    uint4 ra0, ra1, ra2, ra3, rp, rq[4], rh, rx[WT == BM_Q4K ? 1 : 4];
+    uint4 ra0, ra1, rq[2], rh, rx[WT == BM_Q4K ? 1 : 2];
+    uint2 rp;
     auto fetch = [&](int i) {
         ra0 = *reinterpret_cast<const uint4 *>(act + (src_a[0] + (u32)i * BM_Q82_SB_REF));
         ra1 = *reinterpret_cast<const uint4 *>(act + (src_a[1] + (u32)i * BM_Q82_SB_REF));
-        ra2 = *reinterpret_cast<const uint4 *>(act + (src_a[2] + (u32)i * BM_Q82_SB_REF));
-        ra3 = *reinterpret_cast<const uint4 *>(act + (src_a[3] + (u32)i * BM_Q82_SB_REF));
-        rp = *reinterpret_cast<const uint4 *>(act + (src_p + (u32)i * 64u));
+        rp = *reinterpret_cast<const uint2 *>(act + (src_p + (u32)i * 64u));
         const uint8_t *blk = we + (src_w + (u32)i * kBlock);
-        if constexpr (kQ45) {
-            rh = *reinterpret_cast<const uint4 *>(blk); // d, dmin, the twelve scale bytes
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const uint8_t *piece = we + (src_c[j] + (u32)i * kBlock);
+        for (int j = 0; j < 2; j++) {
+            const uint8_t *piece = we + (src_c[j] + (u32)i * kBlock);
+            if constexpr (kQ45) {
                 rq[j] = *reinterpret_cast<const uint4 *>(piece);
                 if constexpr (WT == BM_Q5K) rx[j] = *reinterpret_cast<const uint4 *>(piece + high_at);
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const uint8_t *piece = we + (src_c[j] + (u32)i * kBlock);
+            } else {
                 rq[j] = bm_ld16u(piece);
                 rx[j] = bm_ld16u(piece + high_at);
             }
-            rh = bm_ld16u(blk + 192); // the sixteen scales
-            rh.x = wh ? rh.z : rh.x;  // this half's eight scale bytes
-            rh.y = wh ? rh.w : rh.y;
-            rh.z = bm_ld2u(blk + 208); // d
+        }
+        if constexpr (kQ45) {
+            rh = *reinterpret_cast<const uint4 *>(blk); // d, dmin, the twelve scale bytes
+        } else { // scales 4 wq .. 4 wq + 3 of the sixteen, and d
+            rh.x = bm_ld2u(blk + 192 + 4 * wq) | (bm_ld2u(blk + 194 + 4 * wq) << 16);
+            rh.y = bm_ld2u(blk + 208);
         }
     };
     auto put16 = [](uint8_t *dst, u32 a, u32 b, u32 c, u32 d) {
@@ -598,23 +595,17 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
     auto stash = [&]() {
         uint8_t *acol = a_codes + ac * kStride + 16 * ap;
         put16(acol, ra0.x, ra0.y, ra0.z, ra0.w);
-        put16(acol + 16 * kStride, ra1.x, ra1.y, ra1.z, ra1.w);
-        put16(acol + 32 * kStride, ra2.x, ra2.y, ra2.z, ra2.w);
-        put16(acol + 48 * kStride, ra3.x, ra3.y, ra3.z, ra3.w);
-        d8_t[(2 * (2 * pp)) * kFastColLine + pcol] = scale_operand_col(rp.x);
-        d8_t[(2 * (2 * pp + 1)) * kFastColLine + pcol] = scale_operand_col(rp.z);
-        if constexpr (kQ45) {
-            my_t[(2 * pp) * kFastColLine + pcol] = bm_bits_f32(rp.y);
-            my_t[(2 * pp + 1) * kFastColLine + pcol] = bm_bits_f32(rp.w);
-        }
+        put16(acol + 32 * kStride, ra1.x, ra1.y, ra1.z, ra1.w);
+        d8_t[pb * kFastColLine + pcol] = scale_operand_col(rp.x);
+        if constexpr (kQ45) my_t[pb * kFastColLine + pcol] = bm_bits_f32(rp.y);
         const u32 ml = 0x0f0f0f0fu;
         if constexpr (kQ45) {
             // nibble piece cc of a row: code bytes 16 cc ..: the low nibbles are sub-block 2 p, values 16 (cc % 2) .., the
             // high nibbles sub-block 2 p + 1, the same values, with p = cc / 2
             const int p = cc >> 1, at = 16 * (cc & 1);
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                uint8_t *row = w_codes + (crow + 32 * j) * kStride;
+            for (int j = 0; j < 2; j++) {
+                uint8_t *row = w_codes + (crow + 64 * j) * kStride;
                 u32 lo[4] = {rq[j].x & ml, rq[j].y & ml, rq[j].z & ml, rq[j].w & ml};
                 u32 hi[4] = {(rq[j].x >> 4) & ml, (rq[j].y >> 4) & ml, (rq[j].z >> 4) & ml, (rq[j].w >> 4) & ml};
                 if constexpr (WT == BM_Q5K) { // high-bit bytes 16 (cc % 2) ..: bit 2 p for the low nibbles, 2 p + 1 for the high
@@ -629,15 +620,19 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
                 put16(row + 64 * p + at, lo[0], lo[1], lo[2], lo[3]);
                 put16(row + 64 * p + 32 + at, hi[0], hi[1], hi[2], hi[3]);
             }
-            // scale and min of sub-blocks 4 wh .. 4 wh + 3 (crates/gguf/src/quant.rs:620-628 get_scale_min_k4)
+            // scale and min of sub-blocks 2 wq and 2 wq + 1 (crates/gguf/src/quant.rs:620-628 get_scale_min_k4): with the
+            // twelve bytes as q[0 .. 11], sub-block j < 4 has q[j] & 63 and q[j + 4] & 63; j >= 4 has
+            // (q[j + 4] & 15) | (q[j - 4] >> 6) << 4 and (q[j + 4] >> 4) | (q[j] >> 6) << 4
             const float d = bm_half_to_f32(rh.x & 0xffffu), dmin = bm_half_to_f32(rh.x >> 16);
+            const bool upper = wq >= 2;
 #pragma unroll
-            for (int jj = 0; jj < 4; jj++) {
-                const u32 qa = (rh.y >> (8 * jj)) & 0xffu, qb = (rh.z >> (8 * jj)) & 0xffu, qc = (rh.w >> (8 * jj)) & 0xffu;
-                const u32 scv = wh ? ((qc & 15u) | ((qa >> 6) << 4)) : (qa & 63u);
-                const u32 mv = wh ? ((qc >> 4) | ((qb >> 6) << 4)) : (qb & 63u);
-                sv_t[(4 * wh + jj) * kFastRowLine + wr] = scale_operand_row(d * (float)scv);
-                mn_t[(4 * wh + jj) * kFastRowLine + wr] = -(dmin * (float)mv);
+            for (int i = 0; i < 2; i++) {
+                const u32 sh = 8u * (u32)(2 * (wq & 1) + i);
+                const u32 qa = (rh.y >> sh) & 0xffu, qb = (rh.z >> sh) & 0xffu, qc = (rh.w >> sh) & 0xffu;
+                const u32 scv = upper ? ((qc & 15u) | ((qa >> 6) << 4)) : (qa & 63u);
+                const u32 mv = upper ? ((qc >> 4) | ((qb >> 6) << 4)) : (qb & 63u);
+                sv_t[(2 * wq + i) * kFastRowLine + wr] = scale_operand_row(d * (float)scv);
+                mn_t[(2 * wq + i) * kFastRowLine + wr] = -(dmin * (float)mv);
             }
         } else {
             // ql piece cc of a row (bytes 16 cc ..: half cc / 4, piece c = cc % 4 of it) with qh piece c % 2 of that half: the
@@ -647,8 +642,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
             const u32 mh = 0x03030303u;
             const int half = cc >> 2, c = cc & 3;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                uint8_t *row = w_codes + (crow + 32 * j) * kStride;
+            for (int j = 0; j < 2; j++) {
+                uint8_t *row = w_codes + (crow + 64 * j) * kStride;
                 const uint4 hq = rx[j];
 #pragma unroll
                 for (int hn = 0; hn < 2; hn++) {
@@ -660,118 +655,96 @@ __global__ __launch_bounds__(256, 2) void k_gemm_fast(const uint8_t *w, int rpe,
                           q6_minus_32(((rq[j].w >> ns) & ml) | (((hq.w >> hs) & mh) << 4)));
                 }
             }
-            const float d = bm_half_to_f32(rh.z & 0xffffu);
+            const float d = bm_half_to_f32(rh.y & 0xffffu);
 #pragma unroll
-            for (int jj = 0; jj < 8; jj++) {
-                const u32 word = jj < 4 ? rh.x : rh.y;
-                sv_t[(8 * wh + jj) * kFastRowLine + wr] = scale_operand_row(d * (float)(int)(signed char)((word >> (8 * (jj & 3))) & 0xffu));
-            }
+            for (int jj = 0; jj < 4; jj++)
+                sv_t[(4 * wq + jj) * kFastRowLine + wr] = scale_operand_row(d * (float)(int)(signed char)((rh.x >> (8 * jj)) & 0xffu));
         }
     };
-    // this lane in a 32 x 32 product: operand row / slot lane % 32, its share of the unit's values (lane / 32); result v
-    // is row 8 (v / 4) + 4 (lane / 32) + v % 4 of slot lane % 32
+    // this wave's 32 rows (32 rg ..) and 32 slots (32 t ..); this lane in the 32 x 32 product: operand row / slot lane % 32,
+    // its share of the unit's values (lane / 32); result v is row 8 (v / 4) + 4 (lane / 32) + v % 4 of slot lane % 32
+    const int rg = wv & 3, t = wv >> 2;
     const int l32 = lane & 31, kh = lane >> 5;
-    const uint8_t *my_w = w_codes + (32 * wv + l32) * kStride + kOp * kh;
-    const uint8_t *my_a = a_codes + l32 * kStride + kOp * kh;
-    const uint2 *my_sv = sv_t + 32 * wv + l32;
-    const uint2 *my_d8 = d8_t + kh * kFastColLine + l32;
-    const bool two = len > 32; // else the second half of the slots is all padding
-    v16f acc[2];
+    const uint8_t *my_w = w_codes + (32 * rg + l32) * kStride + kOp * kh;
+    const uint8_t *my_a = a_codes + (32 * t + l32) * kStride + kOp * kh;
+    const uint2 *my_sv = sv_t + (kh ? kFastRows : 32 * rg + l32); // lanes 32 .. 63: the line's zero
+    const uint2 *my_d8 = d8_t + 32 * t + l32;
+    const bool live = t == 0 || len > 32; // else this wave's slots are all padding
+    v16f acc;
 #pragma unroll
-    for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) acc[t][v] = 0.0f;
+    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
 
-    // One super-block's products. A step is a (unit, half of the slots): its integer sums (one matrix instruction, issued a
-    // step ahead), its scale products (another, issued at the end of the step before, behind that step's last use of the
-    // one buffer), and on the vector ALU the sums to floats and the multiply-adds: two operations a (row, slot, unit).
-    auto blocks = [&](auto two_tiles) __attribute__((always_inline)) {
-        constexpr bool kTwo = decltype(two_tiles)::value;
-        constexpr int kSteps = (kTwo ? 2 : 1) * kUnitsSb;
+    // One super-block's products. A step is a unit: its integer sums (one matrix instruction, issued a step ahead), its
+    // scale products (another, issued at the end of the step before, behind that step's last use of the one buffer), and on
+    // the vector ALU the sums to floats and the multiply-adds.
+    auto blocks = [&]() __attribute__((always_inline)) {
         typedef typename std::conditional<kQ45, v4i, long>::type Operand;
         Operand a[2], b[2];
-        uint2 sa[2], sb[3];
+        uint2 sa[2], sb[2];
         v16i sum[2];
         v16f pr;
-        auto rd_a = [&](int un) {
-            a[un & 1] = *reinterpret_cast<const Operand *>(my_w + 2 * kOp * un);
-            sa[un & 1] = my_sv[un * kFastRowLine];
-        };
-        auto rd_b = [&](int u) { // step u's column operand and column scale
-            const int un = kTwo ? u >> 1 : u, t = kTwo ? u & 1 : 0;
-            b[u & 1] = *reinterpret_cast<const Operand *>(my_a + 32 * t * kStride + 2 * kOp * un);
-            sb[u % 3] = my_d8[2 * (kQ45 ? un : un >> 1) * kFastColLine + 32 * t];
+        auto rd = [&](int u) {
+            a[u & 1] = *reinterpret_cast<const Operand *>(my_w + 2 * kOp * u);
+            b[u & 1] = *reinterpret_cast<const Operand *>(my_a + 2 * kOp * u);
+            sa[u & 1] = my_sv[u * kFastRowLine];
+            sb[u & 1] = my_d8[(kQ45 ? u : u >> 1) * kFastColLine];
         };
         auto product = [&](int u) {
-            const int un = kTwo ? u >> 1 : u;
             const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            if constexpr (kQ45) sum[u & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[un & 1], b[u & 1], z, 0, 0, 0);
-            else sum[u & 1] = __builtin_amdgcn_mfma_i32_32x32x16_i8(a[un & 1], b[u & 1], z, 0, 0, 0);
+            if constexpr (kQ45) sum[u & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[u & 1], b[u & 1], z, 0, 0, 0);
+            else sum[u & 1] = __builtin_amdgcn_mfma_i32_32x32x16_i8(a[u & 1], b[u & 1], z, 0, 0, 0);
         };
         auto scales = [&](int u) {
-            const int un = kTwo ? u >> 1 : u;
             const v16f z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            pr = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(v4s, sa[un & 1]), __builtin_bit_cast(v4s, sb[u % 3]), z, 0,
-                                                         0, 0);
+            pr = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(v4s, sa[u & 1]), __builtin_bit_cast(v4s, sb[u & 1]), z, 0, 0,
+                                                         0);
         };
-        rd_a(0);
-        rd_b(0);
+        rd(0);
+        rd(1);
         product(0);
         scales(0);
-        rd_b(1);
-        rd_a(1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int u = 0; u < kSteps; u++) {
-            const int un = kTwo ? u >> 1 : u, t = kTwo ? u & 1 : 0;
-            if (u + 1 < kSteps) product(u + 1);
-            if (u + 2 < kSteps) rd_b(u + 2);
-            // the row side two units on, into the buffer of this unit, whose last instructions have been issued
-            if ((!kTwo || t == 1) && un + 2 < kUnitsSb) rd_a(un + 2);
+        for (int u = 0; u < kUnitsSb; u++) {
+            if (u + 1 < kUnitsSb) product(u + 1);
             __builtin_amdgcn_sched_barrier(0);
             float f[16];
 #pragma unroll
             for (int v = 0; v < 16; v++) f[v] = (float)sum[u & 1][v];
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc[t][v] = fmaf(pr[v], f[v], acc[t][v]);
+            for (int v = 0; v < 16; v++) acc[v] = fmaf(pr[v], f[v], acc[v]);
             __builtin_amdgcn_sched_barrier(0);
-            if (u + 1 < kSteps) scales(u + 1);
+            if (u + 1 < kUnitsSb) scales(u + 1);
+            // the operands two units on, into the buffers of this unit, whose last instructions have been issued
+            if (u + 2 < kUnitsSb) rd(u + 2);
         }
         if constexpr (kQ45) {
             // the min terms last, into the same accumulators: a 32 x 8 by 8 x 32 product in f32, two of the eight
             // sub-blocks an instruction; they run on the matrix cores while the workgroup goes through its barrier and the
             // next staging
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float mn = mn_t[(2 * j + kh) * kFastRowLine + 32 * wv + l32];
-                acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(mn, my_t[(2 * j + kh) * kFastColLine + l32], acc[0], 0, 0, 0);
-                if (kTwo) acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(mn, my_t[(2 * j + kh) * kFastColLine + 32 + l32], acc[1], 0, 0, 0);
-            }
+            for (int j = 0; j < 4; j++)
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(mn_t[(2 * j + kh) * kFastRowLine + 32 * rg + l32],
+                                                           my_t[(2 * j + kh) * kFastColLine + 32 * t + l32], acc, 0, 0, 0);
         }
     };
 
-    for (int i = tid; i < 8 * kGemmBN; i += 256) d8_t[(2 * (i / kGemmBN) + 1) * kFastColLine + i % kGemmBN] = make_uint2(0u, 0u);
     fetch(0);
     for (int i = 0; i < nb; i++) {
         if (i) __syncthreads(); // the readers of the super-block before are done
         stash();
         __syncthreads();
         if (i + 1 < nb) fetch(i + 1);
-        if (two) blocks(std::true_type{});
-        else blocks(std::false_type{});
+        if (live) blocks();
     }
+    const int n = 32 * t + l32;
+    if (n < len) {
+        float *out = y + (size_t)tab->slot[n] * rpe + row0 + 32 * rg + 4 * kh;
 #pragma unroll
-    for (int t = 0; t < 2; t++) {
-        const int n = 32 * t + l32;
-        if (n < len) {
-            float *out = y + (size_t)tab->slot[n] * rpe + row0 + 32 * wv + 4 * kh;
-#pragma unroll
-            for (int q4 = 0; q4 < 4; q4++) {
-                // rows_per_expert is a multiple of 16 and these four rows start at a multiple of 4: all inside or all outside
-                if (row0 + 32 * wv + 4 * kh + 8 * q4 < rpe)
-                    *reinterpret_cast<float4 *>(out + 8 * q4) =
-                        make_float4(acc[t][4 * q4 + 0], acc[t][4 * q4 + 1], acc[t][4 * q4 + 2], acc[t][4 * q4 + 3]);
-            }
+        for (int q4 = 0; q4 < 4; q4++) {
+            // rows_per_expert is a multiple of 16 and these four rows start at a multiple of 4: all inside or all outside
+            if (row0 + 32 * rg + 4 * kh + 8 * q4 < rpe)
+                *reinterpret_cast<float4 *>(out + 8 * q4) = make_float4(acc[4 * q4 + 0], acc[4 * q4 + 1], acc[4 * q4 + 2], acc[4 * q4 + 3]);
         }
     }
 }
@@ -1077,7 +1050,7 @@ hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int
             if (e != hipSuccess) return e;
             const u32 n_slabs_f = (u32)((rows_per_expert + kFastRows - 1) / kFastRows);
             const unsigned grid = ((max_tiles + 7) / 8) * 8 * n_slabs_f;
-            hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev, n_tiles,
+            hipLaunchKernelGGL(kern, dim3(grid), dim3(kFastThreads), lds, L.stream, w, rows_per_expert, nb, act, cols, tiles_dev, n_tiles,
                                n_slabs_f, (u32)slot_div, (u32)n_slots, y);
             return hipGetLastError();
         };

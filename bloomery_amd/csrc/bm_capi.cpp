@@ -892,7 +892,7 @@ int bm_scratch_create(bm_ctx *ctx, int gate_type, int down_type, int hidden, int
     //    192      580       246        370          214
     //    256      767       296        392          230
     //    512     1491       534        481          289
-    s->path = BM_PATH_AUTO, s->grouped_from = 22, s->gemm_from = 448, s->gemm_from_fast = 160;
+    s->path = BM_PATH_AUTO, s->grouped_from = 22, s->gemm_from = 448, s->gemm_from_fast = 96;
     const size_t slots = (size_t)max_tokens * n_slots_per_token;
     int rc = bm_act_create(ctx, gate_type, hidden, max_tokens, &s->act_x);
     if (!rc) rc = bm_act_create(ctx, down_type, ff, (int)slots, &s->act_h);

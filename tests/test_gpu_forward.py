@@ -58,7 +58,7 @@ def test_the_automatic_choice_follows_the_crossovers(gpu):
                                                                        bm.PATH_GROUPED, bm.PATH_GEMM, bm.PATH_GEMM]
         gpu.set_gemm_mode(bm.GEMM_FAST)  # the tolerance mode's GEMM is faster: its cut comes earlier
         try:
-            assert [sc.path_for(m) for m in (21, 22, 159, 160)] == [bm.PATH_PER_SLOT, bm.PATH_GROUPED, bm.PATH_GROUPED, bm.PATH_GEMM]
+            assert [sc.path_for(m) for m in (21, 22, 95, 96)] == [bm.PATH_PER_SLOT, bm.PATH_GROUPED, bm.PATH_GROUPED, bm.PATH_GEMM]
         finally:
             gpu.set_gemm_mode(bm.GEMM_EXACT)
         sc.set_path(bm.PATH_AUTO, 4, 2000)

@@ -318,7 +318,7 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
 /* How bm_gemm sums in f32 (the integer block sums are exact either way):
  *   BM_GEMM_EXACT (default): the CPU path's eight accumulators and closing order; bit-identical to bm_gemv_sel;
  *   BM_GEMM_FAST: one accumulator a value, blocks in increasing k; differs from the exact value by f32 rounding
- *     only (observed below 1e-6 of the row's largest magnitude; the contract's tolerance is 1e-4), about 1.6x the
+ *     only (observed below 1e-6 of the row's largest magnitude; the contract's tolerance is 1e-4), about 1.9x the
  *     speed of a Q4_K / Q6_K layer step. No counterpart in the reference, whose grouped GEMM has one order (gemm/grouped.rs:33-58). */
 #define BM_GEMM_EXACT 0
 #define BM_GEMM_FAST 1

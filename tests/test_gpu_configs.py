@@ -188,6 +188,104 @@ def test_prefill_layer_shape_under_skewed_routing(gpu):
     L.free()
 
 
+def test_prefill_at_the_benchmarks_full_size_equals_the_slot_path(gpu):
+    """The prefill configuration at its full size: 2048 tokens, top-8 of 128 resident experts under a Zipf routing, Q4_K
+    gate / up (768 rows, K 2048), Q6_K down (2048 rows, K 768). The oracle would take minutes over 16384 slots, so the
+    size-independent property stands in: the grouped GEMM step and the per-slot step are separate kernels over the same
+    arithmetic and must agree bit for bit on every slot's down row and on every token's y; sampled slots' h columns are
+    compared as bytes and their gate rows against the oracle's row dots. The tolerance mode's gate rows are held to the
+    exact mode's, every slot."""
+    hidden, ff, n_experts, m, top_k = 2048, 768, 128, 2048, 8
+    n_slots = m * top_k
+    L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), hidden, ff, n_experts, 3500, cheap=True)
+    rng = np.random.default_rng(3501)
+    x = normal_f32(rng, (m, hidden))
+    bias = np.empty(n_experts, np.float32)
+    bias[rng.permutation(n_experts)] = (-1.1 * np.log(np.arange(1, n_experts + 1))).astype(np.float32)
+    ids, wts = route(rng, m, n_experts, top_k, bias)
+    runs = np.bincount(ids.reshape(-1), minlength=n_experts)
+    assert runs.max() > 1024 and runs.min() < 32, (runs.max(), runs.min())  # many tiles an expert, and less than a tile
+    gpu.fault_clear()
+    xd, sel, wd = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32)
+    act = gpu.act(bm.Q4_K, hidden, m)
+    gpu.enqueue_quantize(xd, m, act)
+    table = gpu.route(n_slots, n_experts)
+    table.fill(sel, n_slots)
+    g = gpu.buffer(np.float32, n_slots * ff).fill_bytes(0xFF)
+    u = gpu.buffer(np.float32, n_slots * ff).fill_bytes(0xFF)
+    sample = list(range(0, n_slots, 1021)) + [n_slots - 1]
+
+    def gemm_step(fast):
+        act_h = gpu.act(bm.Q6_K, ff, n_slots)
+        down = gpu.buffer(np.float32, n_slots * hidden).fill_bytes(0xFF)
+        y = gpu.buffer(np.float32, m * hidden).fill_bytes(0xFF)
+        gpu.set_gemm_mode(bm.GEMM_FAST if fast else bm.GEMM_EXACT)
+        try:
+            gpu.enqueue_gemm(L.dg, ff, act, table, top_k, g)
+            gpu.enqueue_gemm(L.du, ff, act, table, top_k, u)
+            gpu.enqueue_swiglu_quant(g, u, n_slots, act_h)
+            gpu.enqueue_gemm(L.dd, hidden, act_h, table, 0, down)
+            gpu.enqueue_combine_tokens(down, wd, None, hidden, top_k, m, y)
+            out = y.download(), down.download(), [act_h.download(s) for s in sample], g.download()
+        finally:
+            gpu.set_gemm_mode(bm.GEMM_EXACT)
+        for b in (act_h, down, y):
+            b.free()
+        return out
+
+    y_gemm, down_gemm, cols_gemm, g_gemm = gemm_step(False)
+    # the per-slot step: gate . up with its folded quantizer, the slot gemv, the slot sum
+    act_h = gpu.act(bm.Q6_K, ff, n_slots)
+    down = gpu.buffer(np.float32, n_slots * hidden).fill_bytes(0xFF)
+    y = gpu.buffer(np.float32, m * hidden).fill_bytes(0xFF)
+    gpu.enqueue_gate_up(L.dg, L.du, act, sel, n_slots, ff, top_k, None, act_h)
+    gpu.enqueue_gemv_sel(L.dd, act_h, sel, n_slots, hidden, down)
+    gpu.enqueue_combine_tokens(down, wd, None, hidden, top_k, m, y)
+    y_slot, down_slot = y.download(), down.download()
+    cols_slot = [act_h.download(s) for s in sample]
+    assert np.array_equal(down_gemm.view(np.uint32), down_slot.view(np.uint32)), "down rows: GEMM against slot gemv"
+    assert np.array_equal(y_gemm.view(np.uint32), y_slot.view(np.uint32)), "y: GEMM step against per-slot step"
+    for s, a, b in zip(sample, cols_gemm, cols_slot):
+        assert np.array_equal(a, b), f"h column of slot {s}"
+    assert np.isfinite(y_gemm).all() and gpu.fault() == (bm.FAULT_NONE, 0)
+    rb = ora.row_bytes(bm.Q4_K, hidden)
+    flat = ids.reshape(-1)
+    for s in sample[::4]:
+        e, col = int(flat[s]), ora.quantize_col(bm.Q4_K, x[s // top_k])
+        assert_f32(g_gemm[s * ff:(s + 1) * ff], ora.gemv(bm.Q4_K, L.wg[e * ff * rb:(e + 1) * ff * rb], ff, hidden, col, 1), f"gate slot {s}")
+    # the tolerance mode, GEMM by GEMM on the same columns (through the layer a last-bit difference can flip a code of h)
+    g_fast = gemm_step(True)[3].reshape(n_slots, ff)
+    g_exact = g_gemm.reshape(n_slots, ff)
+    worst = float((np.abs(g_fast - g_exact).max(axis=1) / np.abs(g_exact).max(axis=1)).max())
+    assert worst <= 1e-5, f"tolerance mode, gate rows: {worst}"
+    for b in (xd, sel, wd, act, table, g, u, act_h, down, y):
+        b.free()
+    L.free()
+
+
+@pytest.mark.parametrize("m", (1, 16))
+def test_decode_layer_with_all_128_experts_resident(gpu, m):
+    """The headline configuration's layer with every one of its 128 experts resident (random legal blocks: the size is
+    what is under test), one token and the sixteen of the grouped configuration: the fused per-slot step against the
+    oracle, bit for bit, h columns included."""
+    hidden, ff, n_experts, top_k = 2048, 768, 128, 8
+    L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), hidden, ff, n_experts, 3600, cheap=True)
+    rng = np.random.default_rng(3601 + m)
+    x = normal_f32(rng, (m, hidden))
+    ids, wts = route(rng, m, n_experts, top_k)
+    resid = normal_f32(rng, (m, hidden))
+    gpu.fault_clear()
+    y, h, cols_h, cols_x = run_fused_step(gpu, L, x, ids, wts, top_k, resid=resid)
+    want_y, want_h = L.oracle(x, ids, wts, top_k)
+    assert_f32(h, want_h, "h")
+    for s in range(m * top_k):
+        assert np.array_equal(cols_h[s], ora.quantize_col(bm.Q6_K, want_h[s * ff:(s + 1) * ff])), f"act_h slot {s}"
+    want = (np.asarray(want_y, np.float32).reshape(m, hidden) + resid).astype(np.float32)
+    assert_f32(y, want.reshape(-1), "y")
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    L.free()
+
+
 # ------------------------------------------------------------------------ a host-served slot through gate . up
 
 def test_gate_up_entries_skip_a_host_slot(gpu):

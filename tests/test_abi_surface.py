@@ -1,11 +1,12 @@
-"""The C header and the binding notes name the same surface: every function include/bm_moe.h declares appears in
-INTEGRATION.md's extern "C" block with the same number of arguments under the same names, in the same order, and the
-block binds nothing the header does not declare. (That the built library exports every declared symbol is
+"""The C header and the binding notes at the repository root name the same surface: every function include/bm_moe.h
+declares appears in the notes' extern "C" block with the same number of arguments under the same names, in the same
+order, and the block binds nothing the header does not declare. (That the built library exports every declared symbol is
 test_capi_cpu.py's part.)"""
 import os
 import re
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+NOTES = os.path.join(ROOT, "INTEGRATION.md")
 
 
 def header_functions():
@@ -23,7 +24,7 @@ def header_functions():
 
 
 def bound_functions():
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    text = open(NOTES).read()
     block = re.search(r'extern "C" \{(.*?)\n\}', text, flags=re.S).group(1)
     out = {}
     for name, params in re.findall(r"pub fn (bm_\w+)\s*\((.*?)\)\s*(?:->[^;]*)?;", block, flags=re.S):
@@ -37,8 +38,8 @@ def bound_functions():
 def test_every_declared_function_is_bound_with_the_same_arguments():
     declared, bound = header_functions(), bound_functions()
     assert len(declared) > 60
-    assert sorted(set(declared) - set(bound)) == [], "declared in include/bm_moe.h, missing from INTEGRATION.md"
-    assert sorted(set(bound) - set(declared)) == [], "bound in INTEGRATION.md, not declared in include/bm_moe.h"
+    assert sorted(set(declared) - set(bound)) == [], "declared in include/bm_moe.h, missing from the binding notes"
+    assert sorted(set(bound) - set(declared)) == [], "bound in the notes, not declared in include/bm_moe.h"
     for name, names in declared.items():
         assert bound[name] == names, f"{name}: the header has ({', '.join(names)}), the binding ({', '.join(bound[name])})"
 
@@ -47,7 +48,7 @@ def test_the_build_recipe_names_every_source_of_the_library():
     """The build.rs shown compiles what the Makefile compiles."""
     mk = open(os.path.join(ROOT, "bloomery_amd", "csrc", "Makefile")).read()
     srcs = re.search(r"^SRCS = (.*)$", mk, flags=re.M).group(1).split()
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    text = open(NOTES).read()
     recipe = re.search(r"## build\.rs(.*?)## extern", text, flags=re.S).group(1)
     assert len(srcs) >= 7
     for s in srcs:

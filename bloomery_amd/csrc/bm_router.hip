@@ -149,11 +149,23 @@ hipError_t route_softmax(const Launch &L, const float *logits, int n_tok, int n_
 //
 // A workgroup takes one token and R router rows: the token's row is normed into LDS by all 256 threads while the rows'
 // bytes arrive (both requested at once), then eight lanes a row walk it, lane l the accumulator l.
+// Floats a line of the accumulator-major LDS rows.
+__host__ __device__ inline int router_line(int hidden) { return ((hidden / 8 + 3) & ~3) + 8; }
+
 template <int R>
 __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *router, const float *x, const float *gain, float eps,
                                                    int n_exp, int hidden, float *normed_out, float *logits) {
-    float *xs = reinterpret_cast<float *>(lds);  // [hidden]
-    float *ws = xs + hidden;                     // [R][hidden + 8]: rows eight banks apart, the R x 8 readers on 8 R banks
+    // The token's row and the R router rows lie accumulator-major in LDS: value k at line k % 8, place k / 8, so that the
+    // lane that owns accumulator l reads four consecutive steps' operands as 16 bytes. A line is hidden / 8 floats, rounded up
+    // to whole 16 bytes, + 8 (the eight lines of a row 8 banks apart), a router row four floats past the one before (rows r
+    // and r + 1 on different banks).
+    const int line = router_line(hidden), wrow_floats = 8 * line + 4;
+    float *xs = reinterpret_cast<float *>(lds);  // [8][line]
+    float *ws = xs + 8 * line;                   // [R][8][line] (+ 4 a row)
+    auto put4 = [&](float *base, int c, const float4 v) { // the four values 4 c .. 4 c + 3 of a row
+        float *at = base + (4 * (c & 1)) * line + (c >> 1);
+        at[0] = v.x, at[line] = v.y, at[2 * line] = v.z, at[3 * line] = v.w;
+    };
     __shared__ double s_part[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int blocks_per_token = (n_exp + R - 1) / R;
@@ -164,7 +176,7 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
     for (int i = tid; i < R * n4; i += 256) {
         const int r = i / n4, c = i % n4;
         const int e = e0 + r < n_exp ? e0 + r : n_exp - 1;
-        reinterpret_cast<float4 *>(ws + (size_t)r * (hidden + 8))[c] = reinterpret_cast<const float4 *>(router + (size_t)e * hidden)[c];
+        put4(ws + (size_t)r * wrow_floats, c, reinterpret_cast<const float4 *>(router + (size_t)e * hidden)[c]);
     }
     double sum = 0.0;
     constexpr int kInRegs = 8; // float4s of the row a thread can hold: rows of up to 8192 values stay in registers
@@ -200,14 +212,14 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
             if (i < n4) {
                 const float4 v = make_float4(__fmul_rn(__fmul_rn(scale, gv[j].x), xv[j].x), __fmul_rn(__fmul_rn(scale, gv[j].y), xv[j].y),
                                              __fmul_rn(__fmul_rn(scale, gv[j].z), xv[j].z), __fmul_rn(__fmul_rn(scale, gv[j].w), xv[j].w));
-                reinterpret_cast<float4 *>(xs)[i] = v;
+                put4(xs, i, v);
                 if (normed_out && e0 == 0) reinterpret_cast<float4 *>(normed_out + (size_t)t * hidden)[i] = v;
             }
         }
     } else {
         for (int i = tid; i < n4; i += 256) {
             const float4 v = reinterpret_cast<const float4 *>(xt)[i];
-            reinterpret_cast<float4 *>(xs)[i] = v;
+            put4(xs, i, v);
             if (gain) {
                 sum += (double)__fmul_rn(v.x, v.x);
                 sum += (double)__fmul_rn(v.y, v.y);
@@ -224,31 +236,39 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
             const float mean = (float)(total / (double)hidden);
             const float scale = __fdiv_rn(1.0f, bm_sqrt_rn(__fadd_rn(mean, eps)));
             for (int i = tid; i < hidden; i += 256) {
-                const float v = __fmul_rn(__fmul_rn(scale, gain[i]), xs[i]); // written before the barrier above
-                xs[i] = v;
+                float *at = xs + (i & 7) * line + (i >> 3);
+                const float v = __fmul_rn(__fmul_rn(scale, gain[i]), *at); // written before the barrier above
+                *at = v;
                 if (normed_out && e0 == 0) normed_out[(size_t)t * hidden + i] = v;
             }
         }
     }
     __syncthreads();
     if (!gain && normed_out && e0 == 0) // the rows as they are (read after the barrier: other threads staged them)
-        for (int i = tid; i < hidden; i += 256) normed_out[(size_t)t * hidden + i] = xs[i];
+        for (int i = tid; i < hidden; i += 256) normed_out[(size_t)t * hidden + i] = xs[(i & 7) * line + (i >> 3)];
     if (tid < 8 * R) {
         const int r = tid >> 3, l = tid & 7;
-        const float *wr = ws + (size_t)r * (hidden + 8);
-        float acc = __fmul_rn(xs[l], wr[l]);
-        // the chain is serial by the order's definition; the reads are not: sixteen steps' operands a batch
+        const float4 *xl = reinterpret_cast<const float4 *>(xs + l * line);
+        const float4 *wl = reinterpret_cast<const float4 *>(ws + (size_t)r * wrow_floats + l * line);
+        // the chain is serial by the order's definition (a product, then fused multiply-adds in increasing k); the reads
+        // are not: sixteen steps' operands, four 16-byte reads a side, a batch
         // (reading the next batch under the present batch's chain measured slower: 8.1 us against 7.1 at 128 x 2048)
+        const float *xf = xs + l * line, *wf = ws + (size_t)r * wrow_floats + l * line;
         const int steps = hidden / 8;
+        float acc = __fmul_rn(xf[0], wf[0]);
         int i = 1;
+        for (; i < 4 && i < steps; i++) acc = fmaf(xf[i], wf[i], acc);
         for (; i + 16 <= steps; i += 16) {
-            float a[16], b[16];
+            float4 a[4], b[4];
 #pragma unroll
-            for (int u = 0; u < 16; u++) a[u] = xs[8 * (i + u) + l], b[u] = wr[8 * (i + u) + l];
+            for (int u = 0; u < 4; u++) a[u] = xl[i / 4 + u], b[u] = wl[i / 4 + u];
 #pragma unroll
-            for (int u = 0; u < 16; u++) acc = fmaf(a[u], b[u], acc);
+            for (int u = 0; u < 4; u++) {
+                acc = fmaf(a[u].x, b[u].x, acc), acc = fmaf(a[u].y, b[u].y, acc);
+                acc = fmaf(a[u].z, b[u].z, acc), acc = fmaf(a[u].w, b[u].w, acc);
+            }
         }
-        for (; i < steps; i++) acc = fmaf(xs[8 * i + l], wr[8 * i + l], acc);
+        for (; i < steps; i++) acc = fmaf(xf[i], wf[i], acc);
         // s_l = acc_l + acc_{l+4} on lanes 0..3 of the row's eight, then (s0 + s2) + (s1 + s3)
         const float s = __fadd_rn(acc, __shfl_down(acc, 4, 8));
         const float pair = __fadd_rn(s, __shfl_down(s, 2, 8)); // lane 0: s0 + s2, lane 1: s1 + s3
@@ -293,10 +313,15 @@ __global__ __launch_bounds__(256) void k_norm_route(const float *router, const f
     route_softmax_wave<PER>(logits, t, (u32)n_exp, used, renorm, probs, ids, weights, fault, layer);
 }
 
+// LDS of a workgroup of R rows: the token's row and the router rows, each as eight lines.
+static size_t router_lds_bytes(int rows, int hidden) {
+    return ((size_t)(rows + 1) * 8 * router_line(hidden) + 4 * (size_t)rows) * sizeof(float);
+}
+
 // Rows a workgroup takes: four where they fit the LDS beside the token's row, else two, else one.
 static int router_rows(int hidden) {
     for (int r = 4; r >= 1; r >>= 1)
-        if (((size_t)(r + 1) * hidden + 8 * r) * sizeof(float) <= (size_t)kMaxLds - 1024) return r;
+        if (router_lds_bytes(r, hidden) <= (size_t)kMaxLds - 1024) return r;
     return 0;
 }
 
@@ -306,7 +331,7 @@ hipError_t router_logits(const Launch &L, const float *router, const float *x, c
                          int hidden, float *normed_out, float *logits) {
     const int rows = router_rows(hidden);
     if (rows == 0) return hipErrorInvalidValue;
-    const size_t lds = ((size_t)(rows + 1) * hidden + 8 * rows) * sizeof(float);
+    const size_t lds = router_lds_bytes(rows, hidden);
     const unsigned grid = (unsigned)m * (unsigned)((n_exp + rows - 1) / rows);
 #define BM_RL(R)                                                                                                       \
     {                                                                                                                  \
@@ -328,7 +353,7 @@ hipError_t norm_route(const Launch &L, const float *router, const float *x, cons
                       float *weights, uint32_t *counts) {
     const int rows = router_rows(hidden);
     if (rows == 0) return hipErrorInvalidValue;
-    const size_t lds = ((size_t)(rows + 1) * hidden + 8 * rows) * sizeof(float);
+    const size_t lds = router_lds_bytes(rows, hidden);
     const unsigned grid = (unsigned)m * (unsigned)((n_exp + rows - 1) / rows);
 #define BM_NR(R, PER)                                                                                                  \
     {                                                                                                                  \

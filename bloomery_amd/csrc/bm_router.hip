@@ -26,13 +26,6 @@ __device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
     return __hiloint2double(hi, lo);
 }
 
-// The larger of two (high, low) keys into the first.
-__device__ __forceinline__ void key_max(u32 &hi, u32 &lo, u32 ohi, u32 olo) {
-    const bool take = ohi > hi || (ohi == hi && olo > lo);
-    hi = take ? ohi : hi;
-    lo = take ? olo : lo;
-}
-
 // Token t's routing by one wave; lane L owns experts L + 64 j, j < PER.
 template <int PER>
 __device__ __forceinline__ void route_softmax_wave(const float *logits, u32 t, u32 n_exp, u32 used, u32 renorm, float *probs,
@@ -78,32 +71,35 @@ __device__ __forceinline__ void route_softmax_wave(const float *logits, u32 t, u
         p[j] = p[j] / inv;
         if (probs && lane + 64 * j < n_exp) probs[(size_t)t * n_exp + lane + 64 * j] = p[j];
     }
-    // `used` rounds of a wave argmax under (probability descending, id ascending); the winning lane marks its entry
+    // `used` rounds of a wave argmax under (probability descending, id ascending): the largest probability left (its bits
+    // order as its value: not negative) as one unsigned maximum over the wave, then the smallest id that holds it: expert
+    // lane + 64 j, so the first j with a holder and that ballot's lowest lane. The winning lane marks its entry.
     u32 taken = 0;
     double chosen = 0.0;
     float mine = 0.0f;
     for (u32 s = 0; s < used; s++) {
-        // the order as one unsigned key: a probability's bits (not negative, so ordered as its value) over the
-        // complement of the id; none left: key 0, which reads back as id 0xffffffff
-        u32 khi = 0, klo = 0;
+        u32 best = 0;
+        bool any = false;
 #pragma unroll
         for (int j = 0; j < PER; j++) {
-            const u32 e = lane + 64 * j;
-            if (e < n_exp && !((taken >> j) & 1u)) key_max(khi, klo, bm_f32_bits(p[j]), 0xffffffffu - e);
+            const bool open = lane + 64 * j < n_exp && !((taken >> j) & 1u);
+            const u32 bits = bm_f32_bits(p[j]);
+            best = open && bits > best ? bits : best;
+            any |= open;
         }
-        // the wave's maximum: four exchanges inside each row of sixteen lanes, one between the rows of a half, the two
-        // halves through their first lanes
-        key_max(khi, klo, bm_dpp<kDppXor1>(khi), bm_dpp<kDppXor1>(klo));
-        key_max(khi, klo, bm_dpp<kDppXor2>(khi), bm_dpp<kDppXor2>(klo));
-        key_max(khi, klo, bm_dpp<kDppHalfMirror>(khi), bm_dpp<kDppHalfMirror>(klo));
-        key_max(khi, klo, bm_dpp<kDppMirror>(khi), bm_dpp<kDppMirror>(klo));
-        key_max(khi, klo, bm_swap16(khi), bm_swap16(klo));
-        const u32 h0 = (u32)__builtin_amdgcn_readlane((int)khi, 0), l0 = (u32)__builtin_amdgcn_readlane((int)klo, 0);
-        const u32 h1 = (u32)__builtin_amdgcn_readlane((int)khi, 32), l1 = (u32)__builtin_amdgcn_readlane((int)klo, 32);
-        khi = h0, klo = l0;
-        key_max(khi, klo, h1, l1);
-        const float bv = bm_bits_f32(khi);
-        const u32 bi = 0xffffffffu - klo;
+        const u32 half = bm_max32(best);
+        const u32 m0 = (u32)__builtin_amdgcn_readlane((int)half, 0), m1 = (u32)__builtin_amdgcn_readlane((int)half, 32);
+        const u32 top = m0 > m1 ? m0 : m1;
+        u32 bi = 0xffffffffu; // none left
+        if (__ballot(any) != 0) {
+#pragma unroll
+            for (int j = PER - 1; j >= 0; j--) {
+                const bool open = lane + 64 * j < n_exp && !((taken >> j) & 1u);
+                const unsigned long long holders = __ballot(open && bm_f32_bits(p[j]) == top);
+                if (holders) bi = (u32)(64 * j + __builtin_ctzll(holders)); // uniform; the smallest j wins: it comes last
+            }
+        }
+        const float bv = bi != 0xffffffffu ? bm_bits_f32(top) : 0.0f;
         if ((bi & 63u) == lane && bi != 0xffffffffu) taken |= 1u << (bi >> 6);
         if (lane == 0) ids[(size_t)t * used + s] = bi;
         chosen += (double)bv;

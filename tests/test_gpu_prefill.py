@@ -173,6 +173,51 @@ def test_gemm_rows_not_a_whole_slab_and_refused_slots(gpu, fast):
             b.free()
 
 
+@pytest.mark.parametrize("fast", (False, True))
+def test_gemm_column_that_is_not_finite(gpu, fast):
+    """A token row with an infinity: the quantizer raises QuantColumn and leaves a NaN scale with zero codes
+    (crates/gpu/src/lib.rs:925-933); the GEMM rows of that token's slots are NaN in either mode, and every other slot's
+    rows are what they are without it."""
+    from common import max_abs_normalised
+    rng = np.random.default_rng(2150)
+    wtype, k, rpe, n_experts, m, top_k = bm.Q4_K, 512, 96, 3, 20, 2
+    n_slots = m * top_k
+    w = stack(wtype, n_experts * rpe, k, 2151)
+    ids = rng.integers(0, n_experts, (m, top_k)).astype(np.uint32)
+    x = normal_f32(rng, (m, k))
+    x[7, 100] = np.inf
+    dw, act = gpu.weights(wtype, n_experts * rpe, k, w), gpu.act(wtype, k, m)
+    xd, sel = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32)
+    table = gpu.route(n_slots, n_experts)
+    gpu.fault_clear()
+    gpu.set_layer(4)
+    gpu.enqueue_quantize(xd, m, act)
+    table.fill(sel, n_slots)
+    y = gpu.buffer(np.float32, n_slots * rpe).fill_bytes(0)
+    gpu.set_gemm_mode(bm.GEMM_FAST if fast else bm.GEMM_EXACT)
+    try:
+        gpu.enqueue_gemm(dw, rpe, act, table, top_k, y)
+        got = y.download().reshape(n_slots, rpe)
+    finally:
+        gpu.set_gemm_mode(bm.GEMM_EXACT)
+    assert gpu.fault(4)[1] & (1 << bm.SITE_QUANT_COLUMN)
+    rb = ora.row_bytes(wtype, k)
+    for s in range(n_slots):
+        t, e = s // top_k, int(ids.reshape(-1)[s])
+        if t == 7:
+            assert np.isnan(got[s]).all(), f"slot {s} of the token that is not finite"
+            continue
+        want = ora.gemv(wtype, w[e * rpe * rb:(e + 1) * rpe * rb], rpe, k, ora.quantize_col(wtype, x[t]), 1)
+        if fast:
+            assert max_abs_normalised(got[s], want) <= 1e-4, f"slot {s}"
+        else:
+            assert_f32(got[s], want, f"slot {s}")
+    gpu.set_layer(bm.LAYER_NONE)
+    gpu.fault_clear()
+    for b in (dw, act, xd, sel, table, y):
+        b.free()
+
+
 def test_prefill_refusals_are_named(gpu):
     w4 = gpu.weights(bm.Q4_K, 64, 512, np.zeros(64 * bm.row_bytes(bm.Q4_K, 512), np.uint8))
     wi = gpu.weights(bm.IQ4_XS, 64, 512, np.zeros(64 * bm.row_bytes(bm.IQ4_XS, 512), np.uint8))

@@ -66,3 +66,12 @@ def test_a_missing_library_raises():
         assert "not built" in str(e.value)
     finally:
         bm._lib = saved
+
+
+def test_the_benchmark_refuses_more_than_one_gpu():
+    """Nothing in this build shards: bench.py --gpus 2 ends with a message that says so, before it touches a device."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""

@@ -376,6 +376,46 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
                 }
             }
         }
+        if constexpr (T == 1) {
+            // one product a 16-value group, sixteen a super-block: a group's matrix instruction is issued one group ahead
+            // of the vector work on its sums, and a block's LDS operands are read two blocks ahead
+            long a[2][2], b[2];
+            float d8[2];
+            float4 sv[2][2];
+            v4i sum[2];
+            auto rd = [&](int bk) {
+#pragma unroll
+                for (int h = 0; h < 2; h++) a[bk & 1][h] = *reinterpret_cast<const long *>(my_a[h] + 32 * bk);
+                b[bk & 1] = *reinterpret_cast<const long *>(buf + my_act[0] + (bk >> 2) * BM_Q82X4_STRIDE + 16 + 32 * (bk & 3) + 8 * kg);
+                d8[bk & 1] = pair[0][bk].x;
+                sv[bk & 1][0] = *reinterpret_cast<const float4 *>(&rs[(kQ45 ? bk : 2 * bk) * kRsStride + rbase]);
+                if constexpr (!kQ45) sv[bk & 1][1] = *reinterpret_cast<const float4 *>(&rs[(2 * bk + 1) * kRsStride + rbase]);
+            };
+            auto product = [&](int g) {
+                const v4i z = {0, 0, 0, 0};
+                sum[g & 1] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[(g >> 1) & 1][g & 1], b[(g >> 1) & 1], z, 0, 0, 0);
+            };
+            rd(0);
+            rd(1);
+            product(0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g = 0; g < 16; g++) {
+                const int bk = g >> 1, h = g & 1, l = 4 * h + (bk & 3);
+                if (g + 1 < 16) product(g + 1);
+                __builtin_amdgcn_sched_barrier(0);
+                // Q4_K, Q5_K: one scale a block; Q6_K: one a group (crates/qdot/src/lib.rs:4403-4440, :4794-4809)
+                const float4 r = sv[bk & 1][kQ45 ? 0 : h];
+                const float dc = d8[bk & 1];
+                acc[0][0][l] = fmaf(r.x * dc, (float)sum[g & 1][0], acc[0][0][l]);
+                acc[0][1][l] = fmaf(r.y * dc, (float)sum[g & 1][1], acc[0][1][l]);
+                acc[0][2][l] = fmaf(r.z * dc, (float)sum[g & 1][2], acc[0][2][l]);
+                acc[0][3][l] = fmaf(r.w * dc, (float)sum[g & 1][3], acc[0][3][l]);
+                __builtin_amdgcn_sched_barrier(0);
+                if (h == 1 && bk + 2 < 8) rd(bk + 2);
+            }
+            return;
+        }
 #pragma unroll
         for (int bk = 0; bk < 8; bk++) { // 32-value block bk of the super-block: groups 2 bk (half 0) and 2 bk + 1
             long a[2], b[T];

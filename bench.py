@@ -813,10 +813,10 @@ def main():
         log(f"[bench] parity {parity}")
         assert err <= 1e-4, parity
 
-    # one graph of `unit` steps; the timed region replays it at least 32 times and for at least 2048 steps, whatever
+    # one graph of `unit` steps; the timed region replays it at least 32 times (8192 steps), whatever
     # --steps asks for below that: a replay is under a millisecond of GPU time, and the figure is a median, not one sample
     unit = max(len(layers) * n_tok // np.gcd(len(layers), n_tok), 1)
-    unit = min(max(int(unit), 64), 256)  # a graph of at least 64 steps: the replay call itself costs microseconds
+    unit = min(max(int(unit), 256), 256)  # a graph of 256 steps (a token's graph in a model of this size holds as many launches): the replay call itself costs microseconds
     gpu.capture_begin()
     for i in range(unit):
         enqueue_step(i)

@@ -692,6 +692,44 @@ def bench_card(args, bm, ora, threads):
     gpu.close()
 
 
+def timeline(args, bm, gpu, enqueue_step, type_names):
+    """The decode step's two launches seen from inside: the measurement build's kernels leave the device's constant-rate
+    counter (100 MHz) at marks in every workgroup; a graph of 193 steps is replayed three times and the last step's marks are
+    read (cold rows: a different token and layer copy every step)."""
+    import ctypes as C
+    lib = gpu.lib
+    lib.bm_timeline_read.restype = C.c_int
+    lib.bm_timeline_read.argtypes = [C.c_void_p]
+    gpu.capture_begin()
+    for i in range(193):
+        enqueue_step(i)
+    graph = gpu.capture_end()
+    for _ in range(3):
+        gpu.graph_launch(graph)
+    gpu.sync()
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    rows = 4096
+    tr = np.zeros(rows * 8, np.uint64)
+    rc = lib.bm_timeline_read(tr.ctypes.data)
+    assert rc == 0, f"bm_timeline_read: {rc}"
+    tr = tr.reshape(rows, 8).astype(np.int64)
+    n_a, n_b = TOP_K * FF // 32, HIDDEN // (64 // TOP_K)
+    a, b = tr[:n_a, :5], tr[rows // 2:rows // 2 + n_b, :4]
+    t0 = a[:, 0].min()
+
+    def stat(v):
+        v = (v - t0) / 100.0
+        return {"min": round(float(v.min()), 2), "median": round(float(np.median(v)), 2), "max": round(float(v.max()), 2)}
+    out = {"unit": "us after the first workgroup of k_gate_up_x started", "gate": type_names[0], "down": type_names[1],
+           "k_gate_up_x": {"workgroups": n_a,
+                           **{name: stat(a[:, i]) for i, name in enumerate(("start", "expert_id_known", "token_quantized", "rows_dotted", "h_block_stored"))}},
+           "k_down_combine": {"workgroups": n_b,
+                              **{name: stat(b[:, i]) for i, name in enumerate(("start", "columns_in_lds", "rows_dotted", "sum_stored"))}}}
+    out["launch_boundary_us"] = round(out["k_down_combine"]["start"]["min"] - out["k_gate_up_x"]["h_block_stored"]["max"], 2)
+    print(json.dumps(out, indent=1), flush=True)
+    gpu.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5, 6, 7, 8),
@@ -718,6 +756,10 @@ def main():
     ap.add_argument("--types", default="q4_k,q6_k",
                     help="config 2 only: gate/up and down weight types (q3_k, q4_k, q5_k, q6_k, iq2_xxs, iq3_xxs, iq4_xs); other than the default is "
                          "a side measurement of that type, not the headline workload")
+    ap.add_argument("--timeline", action="store_true",
+                    help="config 2 only: no timing by events; the step's two launches through the measurement build of the library "
+                         "(libbm_moe_hip_timeline.so), whose kernels leave the device's 100 MHz counter at marks inside every "
+                         "workgroup; prints when each phase of each launch is reached")
     ap.add_argument("--mode", choices=("two", "chain"), default="two",
                     help="two: bm_moe_decode, two launches with the quantizers folded in; chain: quantize, gate_up, down_combine")
     args = ap.parse_args()
@@ -727,6 +769,8 @@ def main():
     import bloomery_amd as bm
     import ora
 
+    if args.timeline:
+        bm.load_library(os.path.join(ROOT, "bloomery_amd", "libbm_moe_hip_timeline.so"))
     threads = host_threads()
     if args.config != 2:
         return {1: bench_gemv, 3: bench_grouped, 4: bench_prefill, 5: bench_dsv3, 6: bench_card, 7: bench_dsv3_prefill, 8: bench_paths}[args.config](args, bm, ora, threads)
@@ -787,6 +831,8 @@ def main():
             gpu.enqueue_down_combine(dd, act_h, sel.ptr + 4 * t * TOP_K, wt.ptr + 4 * t * TOP_K, None, TOP_K, 1, HIDDEN,
                                      y.ptr + 4 * t * HIDDEN)
 
+    if args.timeline:
+        return timeline(args, bm, gpu, enqueue_step, (gate_n, down_n))
     if args.traffic_probe:
         n = 1 << 24  # 64 MiB of f32 in, 64 MiB out: combine over one slot of weight 1 is a copy
         src, dst, one = gpu.buffer(np.float32, n).fill_bytes(0), gpu.buffer(np.float32, n), gpu.upload(np.ones(16, np.float32))

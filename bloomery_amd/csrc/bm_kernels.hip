@@ -7,6 +7,25 @@
 
 namespace bmk {
 
+// Timeline of the two decode launches, in measurement builds only (-DBM_TIMELINE: `make timeline` builds
+// libbm_moe_hip_timeline.so, which bench.py --timeline loads; the library proper holds none of this). Thread 0 of
+// workgroup b of k_gate_up_x leaves the device's constant-rate counter (100 MHz) in row b at marks 0 .. 4 (start, expert
+// id known, token quantized, rows dotted, block of h stored); of k_down_combine in row kTimelineRows / 2 + b at marks
+// 0 .. 3 (start, columns in LDS, rows dotted, sum stored). The last launch of each kernel is what the table holds.
+#ifdef BM_TIMELINE
+constexpr int kTimelineRows = 4096;
+__device__ unsigned long long g_timeline[kTimelineRows * 8];
+#define BM_MARK(base, mark)                                                                                            \
+    do {                                                                                                               \
+        if (threadIdx.x == 0 && (base) + blockIdx.x < (unsigned)kTimelineRows)                                         \
+            g_timeline[((base) + blockIdx.x) * 8 + (mark)] = wall_clock64();                                           \
+    } while (0)
+#else
+#define BM_MARK(base, mark)                                                                                            \
+    do {                                                                                                               \
+    } while (0)
+#endif
+
 // ----------------------------------------------------------------------------------------------- fill
 
 __global__ void k_fill_u32(u32 *dst, u32 value, size_t n) {
@@ -283,6 +302,32 @@ hipError_t combine_tokens(const Launch &L, const float *down, const float *w, co
 
 // --------------------------------------------------------------------------- down + combine in one launch
 
+// A row's closing sum over its token's slots in slot order, acc = fma(w_s, v_s, acc) for the live slots, then the
+// residual (crates/gpu/src/arch/qwen3moe/experts.rs:293-318). v, w and ids lie in LDS. With eight slots every operand is
+// read before the first multiply-add (six 16-byte reads in flight at once); a loop that reads as it goes pays an LDS
+// round trip a slot, 0.4 us at the end of the launch.
+__device__ __forceinline__ float slot_sum(const float *v, const float *w, const u32 *ids, int spt, u32 n_experts,
+                                          float resid_v, bool with_resid) {
+    float acc = 0.0f;
+    if (spt == 8) {
+        const float4 v0 = *reinterpret_cast<const float4 *>(v), v1 = *reinterpret_cast<const float4 *>(v + 4);
+        const float4 w0 = *reinterpret_cast<const float4 *>(w), w1 = *reinterpret_cast<const float4 *>(w + 4);
+        const uint4 i0 = *reinterpret_cast<const uint4 *>(ids), i1 = *reinterpret_cast<const uint4 *>(ids + 4);
+        acc = i0.x < n_experts ? fmaf(w0.x, v0.x, acc) : acc;
+        acc = i0.y < n_experts ? fmaf(w0.y, v0.y, acc) : acc;
+        acc = i0.z < n_experts ? fmaf(w0.z, v0.z, acc) : acc;
+        acc = i0.w < n_experts ? fmaf(w0.w, v0.w, acc) : acc;
+        acc = i1.x < n_experts ? fmaf(w1.x, v1.x, acc) : acc;
+        acc = i1.y < n_experts ? fmaf(w1.y, v1.y, acc) : acc;
+        acc = i1.z < n_experts ? fmaf(w1.z, v1.z, acc) : acc;
+        acc = i1.w < n_experts ? fmaf(w1.w, v1.w, acc) : acc;
+    } else {
+        for (int s = 0; s < spt; s++)
+            if (ids[s] < n_experts) acc = fmaf(w[s], v[s], acc);
+    }
+    return with_resid ? __fadd_rn(acc, resid_v) : acc;
+}
+
 // The shared body of the down + combine workgroup: token t, output rows rb * D .. + D with D = 64 / spt, a quad for
 // every (row, slot).
 template <int WT, int U, int NB>
@@ -291,6 +336,7 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
                                                   const float *resid, int spt, int rpe, float *y, int t, int rb,
                                                   u32 *fault, u32 layer) {
     const int tid = threadIdx.x, q = tid & 3, quad = tid >> 2;
+    BM_MARK(2048, 0);
     const int D = 64 / spt;
     const int e = quad % spt, dl = quad / spt;
     const int r = rb * D + dl;
@@ -302,6 +348,8 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
     const float my_w = wts[t * spt + si];
     const bool live = id < n_experts;
     const bool active = dl < D && r < rpe && live;
+    // the residual value of the row this thread closes, asked for now: at the end it would be a memory round trip
+    const float resid_v = resid && tid < D && rb * D + tid < rpe ? resid[(size_t)t * rpe + rb * D + tid] : 0.0f;
     if (!live && id != 0xffffffffu && rb == 0 && dl == 0 && q == 0) bm_raise(fault, layer, kSiteExpertId);
     const int n = NB > 0 ? NB : nb;
     const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
@@ -323,17 +371,14 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
         s_sel[tid] = my_sel;
     }
     __syncthreads();
+    BM_MARK(2048, 1);
     float v[1];
     row_dot<WT, U, NB, 1>(b, wrow, cols + (size_t)e * col_bytes, col_bytes, 1, n, q, tb, v, NoTap{});
+    BM_MARK(2048, 2);
     if (q == 0 && dl < D) part[dl * spt + e] = v[0];
     __syncthreads();
-    if (tid < D && rb * D + tid < rpe) {
-        float acc = 0.0f;
-        for (int s = 0; s < spt; s++)
-            if (s_sel[s] < n_experts) acc = fmaf(s_w[s], part[tid * spt + s], acc);
-        const size_t o = (size_t)t * rpe + rb * D + tid;
-        y[o] = resid ? __fadd_rn(acc, resid[o]) : acc;
-    }
+    if (tid < D && rb * D + tid < rpe) y[(size_t)t * rpe + rb * D + tid] = slot_sum(part + tid * spt, s_w, s_sel, spt, n_experts, resid_v, resid != nullptr);
+    BM_MARK(2048, 3);
 }
 
 template <int WT, int U, int NB>
@@ -356,6 +401,7 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
                                                uint8_t *act_h, float *h, int slot, int rb, GateRule rule, u32 *fault,
                                                u32 layer) {
     const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
+    BM_MARK(0, 0);
     const int hidden = na * 256, ff = nh * 256;
     const int t = slot / spt;
     const int r = rb * 32 + (tid >> 3);
@@ -384,6 +430,7 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
         if (hcol && tid < 32) q82_store(hcol, nh, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);
         return;
     }
+    BM_MARK(0, 1);
     const size_t row_bytes = (size_t)na * bm_block_bytes<WA>();
     const uint8_t *wrow = (which ? wu : wg) + ((size_t)id * ff + r) * row_bytes;
     Blk<WA> b[UA];
@@ -402,8 +449,10 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
     }
     __syncthreads();
     if (act_x && rb == 0 && slot % spt == 0) stage_bytes(act_x + (size_t)t * col_bytes, col, col_bytes);
+    BM_MARK(0, 2);
     float v[1];
     row_dot<WA, UA, NBA, 1>(b, wrow, col, col_bytes, 1, na, q, Iq2Tables{}, v, NoTap{});
+    BM_MARK(0, 3);
     const float hv = swiglu_of_pair(v[0], which, rule, fault, layer);
     if (h && (tid & 7) == 0) h[(size_t)slot * ff + r] = hv;
     if (!hcol) return;
@@ -411,6 +460,7 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
     if ((tid & 7) == 0) hbuf[tid >> 3] = hv;
     __syncthreads();
     if (tid < 32) quantize_h_block(hbuf, hcol, nh, rb, tid, fault, layer);
+    BM_MARK(0, 4);
 }
 
 // The first half of the fused step as a launch of its own: x -> quantized h, slot by slot.
@@ -660,6 +710,7 @@ __global__ __launch_bounds__(256) void k_down_combine_hq(const uint8_t *w, u32 n
     const float my_w = wts[t * spt + si];
     const bool live = id < n_experts;
     const bool active = dl < D && r < rpe && live;
+    const float resid_v = resid && tid < D && rb * D + tid < rpe ? resid[(size_t)t * rpe + rb * D + tid] : 0.0f;
     if (!live && id != 0xffffffffu && rb == 0 && dl == 0 && q == 0) bm_raise(fault, layer, kSiteExpertId);
     const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
     const int col_bytes = bm_act_col_bytes<WT>(n);
@@ -685,13 +736,7 @@ __global__ __launch_bounds__(256) void k_down_combine_hq(const uint8_t *w, u32 n
     row_dot<WT, U, NB, 1>(b, wrow, cols + (size_t)e * col_bytes, col_bytes, 1, n, q, tb, v, NoTap{});
     if (q == 0 && dl < D) part[dl * spt + e] = v[0];
     __syncthreads();
-    if (tid < D && rb * D + tid < rpe) {
-        float acc = 0.0f;
-        for (int s = 0; s < spt; s++)
-            if (s_sel[s] < n_experts) acc = fmaf(s_w[s], part[tid * spt + s], acc);
-        const size_t o = (size_t)t * rpe + rb * D + tid;
-        y[o] = resid ? __fadd_rn(acc, resid[o]) : acc;
-    }
+    if (tid < D && rb * D + tid < rpe) y[(size_t)t * rpe + rb * D + tid] = slot_sum(part + tid * spt, s_w, s_sel, spt, n_experts, resid_v, resid != nullptr);
 }
 
 // ------------------------------------------------------------------------------------------ verification
@@ -980,3 +1025,10 @@ hipError_t block_sums(const Launch &L, int wtype, const uint8_t *wrow, int k, co
 }
 
 } // namespace bmk
+
+#ifdef BM_TIMELINE
+// The table above, copied to the host: dst holds kTimelineRows * 8 words. Measurement builds only; not part of the C ABI.
+extern "C" int bm_timeline_read(unsigned long long *dst) {
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(bmk::g_timeline), sizeof(unsigned long long) * bmk::kTimelineRows * 8);
+}
+#endif

@@ -20,7 +20,7 @@ Q3_K, Q4_K, Q5_K, Q6_K, IQ2_XXS, IQ3_XXS, IQ4_XS = 11, 12, 13, 14, 16, 18, 23
 FAULT_NONE = 0xFFFFFFFF
 LAYER_NONE = 0xFFFF
 SITE_QUANT_COLUMN, SITE_ROUTER, SITE_EXPERT_ID = 1, 5, 7
-GEMM_EXACT, GEMM_FAST = 0, 1
+GEMM_EXACT, GEMM_FAST, GEMM_FAST_F16 = 0, 1, 2
 PATH_AUTO, PATH_PER_SLOT, PATH_GROUPED, PATH_GEMM = 0, 1, 2, 3
 ACT_SILU_MUL, ACT_SWIGLU_CLAMP, ACT_SWIGLU_OAI, ACT_SITU, ACT_SWIGLU_GCLAMP = 0, 1, 2, 3, 4
 SITE_F32_PRODUCT = 21

@@ -943,7 +943,7 @@ int bm_scratch_path_for(const bm_scratch *s, int m) {
         return s->path;
     }
     if (m < s->grouped_from && m <= bmk::kMaxDecodeTokens) return BM_PATH_PER_SLOT;
-    if (m < (s->ctx->gemm_mode == BM_GEMM_FAST ? s->gemm_from_fast : s->gemm_from) || !gemm_ok) return BM_PATH_GROUPED;
+    if (m < (s->ctx->gemm_mode != BM_GEMM_EXACT ? s->gemm_from_fast : s->gemm_from) || !gemm_ok) return BM_PATH_GROUPED;
     return BM_PATH_GEMM;
 }
 
@@ -1034,8 +1034,8 @@ int bm_set_gate_rule(bm_ctx *ctx, int rule, float limit) {
 
 int bm_set_gemm_mode(bm_ctx *ctx, int mode) {
     if (!ctx) return fail(nullptr, BM_EARG, "bm_set_gemm_mode: ctx is NULL");
-    if (mode != BM_GEMM_EXACT && mode != BM_GEMM_FAST)
-        return fail(ctx, BM_EARG, "bm_set_gemm_mode: mode %d is neither BM_GEMM_EXACT nor BM_GEMM_FAST", mode);
+    if (mode != BM_GEMM_EXACT && mode != BM_GEMM_FAST && mode != BM_GEMM_FAST_F16)
+        return fail(ctx, BM_EARG, "bm_set_gemm_mode: mode %d is none of BM_GEMM_EXACT, BM_GEMM_FAST, BM_GEMM_FAST_F16", mode);
     ctx->gemm_mode = mode;
     return BM_OK;
 }

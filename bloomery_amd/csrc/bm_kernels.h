@@ -126,10 +126,17 @@ hipError_t route(const Launch &L, const uint32_t *ids, int n_slots, int n_expert
 hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act, bool q8k);
 bool gemm_supported(int wtype);
 // slot_div: slots a token when every slot of a token reads the token's column, 1 when each slot reads its own.
-// mode 0: the CPU path's eight-accumulator f32 order (bit-identical to the row dots); 1: one accumulator a value.
+// mode 0: the CPU path's eight-accumulator f32 order (bit-identical to the row dots); 1: one accumulator a value, int8
+// matrix instructions; 2: one accumulator, f16 matrix instructions with the scales in the operands (Q4_K; else as 1).
 hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int rows_per_expert, int k,
                 const uint8_t *act, const uint32_t *cols, const uint32_t *tiles, const uint32_t *n_tiles, int n_slots,
                 int slot_div, float *y, int mode);
+
+// The tolerance mode on f16 matrix instructions with both scales folded into the operands (bm_gemm_half.hip): gemm()'s
+// mode 2 where a type has that form; mode 1 is the int8 form.
+bool gemm_half_supported(int wtype);
+hipError_t gemm_half(const Launch &L, int wtype, const uint8_t *w, int n_experts, int rows_per_expert, int k, const uint8_t *act,
+                     const uint32_t *cols, const uint32_t *tiles, const uint32_t *n_tiles, int n_slots, int slot_div, float *y);
 
 // ---------------------------------------------------------------------------------------- router (bm_router.hip)
 

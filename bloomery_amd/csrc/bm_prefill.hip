@@ -16,7 +16,7 @@
 // by that arithmetic, not by the matrix cores.
 #include <type_traits>
 
-#include "bm_stream.hpp"
+#include "bm_gemm.hpp"
 
 namespace bmk {
 
@@ -146,17 +146,6 @@ hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, 
 // rows' scale products. Strides are padded off the 128-byte bank period.
 constexpr int kActSb = BM_Q82_SB_REF + 64;   // a column's super-block: its two groups and its (d8, d8 * isum) pairs
 constexpr int kActStride = kActSb + 8;       // 360
-
-struct GemmLds {
-    u32 col[kGemmBN];  // the tile's activation columns
-    u32 slot[kGemmBN]; // and slots
-};
-
-// Workgroup b of a GEMM grid: tile and row slab. Workgroups go to the chip's eight dies in turn (b to die b % 8,
-// each with its own L2), so a tile's row slabs are consecutive workgroups of one die: the tile's activation columns
-// come from memory once and serve all the slabs from that L2. The grid is 8 * ceil(tiles / 8) * n_slabs workgroups.
-__device__ __forceinline__ u32 tile_of_block(u32 b, u32 n_slabs) { return ((b >> 3) / n_slabs) * 8 + (b & 7); }
-__device__ __forceinline__ u32 slab_of_block(u32 b, u32 n_slabs) { return (b >> 3) % n_slabs; }
 
 // (q6 - 32) of four codes a word, as signed bytes: q6 in 0..63.
 __device__ __forceinline__ u32 q6_minus_32(u32 q) {
@@ -1081,10 +1070,12 @@ hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int
                                n_slabs_q, (u32)slot_div, (u32)n_slots, y);
             return hipGetLastError();
         };
-        if (mode == 1) return launch_iq(k_gemm_iq2<false>, gemm_iq2_lds_bytes<false>());
+        if (mode != 0) return launch_iq(k_gemm_iq2<false>, gemm_iq2_lds_bytes<false>());
         return launch_iq(k_gemm_iq2<true>, gemm_iq2_lds_bytes<true>());
     }
-    if (mode == 1) {
+    if (mode == 2 && gemm_half_supported(wtype)) // the f16 form of the tolerance mode, where the type has one
+        return gemm_half(L, wtype, w, n_experts, rows_per_expert, k, act, cols, tiles_dev, n_tiles, n_slots, slot_div, y);
+    if (mode == 1 || mode == 2) {
         auto launch_fast = [&](auto kern, size_t lds) {
             hipError_t e = allow_lds(kern, lds);
             if (e != hipSuccess) return e;

@@ -319,9 +319,15 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
  *   BM_GEMM_EXACT (default): the CPU path's eight accumulators and closing order; bit-identical to bm_gemv_sel;
  *   BM_GEMM_FAST: one accumulator a value, blocks in increasing k; differs from the exact value by f32 rounding
  *     only (observed below 1e-6 of the row's largest magnitude; the contract's tolerance is 1e-4), about 1.9x the
- *     speed of a Q4_K / Q6_K layer step. No counterpart in the reference, whose grouped GEMM has one order (gemm/grouped.rs:33-58). */
+ *     speed of a Q4_K / Q6_K layer step. No counterpart in the reference, whose grouped GEMM has one order (gemm/grouped.rs:33-58).
+ *   BM_GEMM_FAST_F16: the tolerance mode with both scales folded into f16 matrix operands (the sub-scale times the 4-bit
+ *     code on the weight side, the block scale times the int8 code as an f16 value and its remainder on the column side), so
+ *     the matrix cores deliver scaled sums and the vector ALU is left with two multiply-adds a super-block. The same
+ *     tolerance (observed 3e-7). Q4_K stacks only; other types run as under BM_GEMM_FAST. Measured slower than BM_GEMM_FAST on
+ *     MI355X (167 against 125 us for the 2048-token gate GEMM) and kept as the measured alternative form. */
 #define BM_GEMM_EXACT 0
 #define BM_GEMM_FAST 1
+#define BM_GEMM_FAST_F16 2
 int bm_set_gemm_mode(bm_ctx *ctx, int mode);
 /* GemmKernels::enqueue_swiglu_quant (crates/gpu/src/gemm/swiglu.rs:46): column c of act = the quantized
  * silu(g) * u of g_dev / u_dev[c * k .. (c + 1) * k), k = act's k, slot-major as the gate and up GEMMs write them;

@@ -69,10 +69,15 @@ def test_gemm_fast_mode_is_within_the_tolerance(gpu):
     from common import max_abs_normalised
     rng = np.random.default_rng(2200)
     worst = 0.0
-    for wtype, k, rpe in ((bm.Q4_K, 2048, 768), (bm.Q6_K, 768, 2048), (bm.Q5_K, 1024, 80), (bm.IQ2_XXS, 1792, 208)):
+    # the last cases: the f16 form of the tolerance mode (Q4_K), full slabs and a ragged one, tiles wider and narrower than 32 slots
+    for wtype, k, rpe, mode in ((bm.Q4_K, 2048, 768, bm.GEMM_FAST), (bm.Q6_K, 768, 2048, bm.GEMM_FAST), (bm.Q5_K, 1024, 80, bm.GEMM_FAST),
+                                (bm.IQ2_XXS, 1792, 208, bm.GEMM_FAST), (bm.Q4_K, 2048, 768, bm.GEMM_FAST_F16),
+                                (bm.Q4_K, 512, 272, bm.GEMM_FAST_F16), (bm.Q6_K, 768, 96, bm.GEMM_FAST_F16)):
         n_experts, n_slots = 6, 150
         w = stack(wtype, n_experts * rpe, k, 2201)
         ids = rng.integers(0, n_experts, n_slots).astype(np.uint32)
+        ids[ids == 5] = rng.integers(0, 2, int((ids == 5).sum())).astype(np.uint32)  # expert 5 idle, 0 and 1 past 32 slots
+        ids[:3] = 5                                                                    # but for three slots: a narrow tile
         x = normal_f32(rng, (n_slots, k))
         dw, act = gpu.weights(wtype, n_experts * rpe, k, w), gpu.act(wtype, k, n_slots)
         xd, sel = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32)
@@ -80,7 +85,7 @@ def test_gemm_fast_mode_is_within_the_tolerance(gpu):
         gpu.enqueue_quantize(xd, n_slots, act)
         table.fill(sel, n_slots)
         y = gpu.buffer(np.float32, n_slots * rpe).fill_bytes(0)
-        gpu.set_gemm_mode(bm.GEMM_FAST)
+        gpu.set_gemm_mode(mode)
         try:
             gpu.enqueue_gemm(dw, rpe, act, table, 0, y)
             got = y.download().reshape(n_slots, rpe)
@@ -128,7 +133,7 @@ def test_prefill_layer_matches_the_oracle(gpu, types, hidden, ff, n_experts, m, 
     L.free()
 
 
-@pytest.mark.parametrize("fast", (False, True))
+@pytest.mark.parametrize("fast", (0, 1, 2))
 def test_gemm_rows_not_a_whole_slab_and_refused_slots(gpu, fast):
     """rows_per_expert = 80 (a multiple of 16, not a whole slab of either mode's kernel); a refused id gets NaN rows and
     ExpertId. In the tolerance mode the live rows are held to the tolerance instead of to bits."""
@@ -148,7 +153,7 @@ def test_gemm_rows_not_a_whole_slab_and_refused_slots(gpu, fast):
         gpu.enqueue_quantize(xd, n_slots, act)
         table.fill(sel, n_slots)
         y = gpu.buffer(np.float32, n_slots * rpe).fill_bytes(0)
-        gpu.set_gemm_mode(bm.GEMM_FAST if fast else bm.GEMM_EXACT)
+        gpu.set_gemm_mode(fast)  # 0: exact, 1: tolerance mode, 2: its f16 form
         try:
             gpu.enqueue_gemm(dw, rpe, act, table, 0, y)
             got = y.download().reshape(n_slots, rpe)
@@ -173,7 +178,7 @@ def test_gemm_rows_not_a_whole_slab_and_refused_slots(gpu, fast):
             b.free()
 
 
-@pytest.mark.parametrize("fast", (False, True))
+@pytest.mark.parametrize("fast", (0, 1, 2))
 def test_gemm_column_that_is_not_finite(gpu, fast):
     """A token row with an infinity: the quantizer raises QuantColumn and leaves a NaN scale with zero codes
     (crates/gpu/src/lib.rs:925-933); the GEMM rows of that token's slots are NaN in either mode, and every other slot's
@@ -194,7 +199,7 @@ def test_gemm_column_that_is_not_finite(gpu, fast):
     gpu.enqueue_quantize(xd, m, act)
     table.fill(sel, n_slots)
     y = gpu.buffer(np.float32, n_slots * rpe).fill_bytes(0)
-    gpu.set_gemm_mode(bm.GEMM_FAST if fast else bm.GEMM_EXACT)
+    gpu.set_gemm_mode(fast)  # 0: exact, 1: tolerance mode, 2: its f16 form
     try:
         gpu.enqueue_gemm(dw, rpe, act, table, top_k, y)
         got = y.download().reshape(n_slots, rpe)

@@ -81,6 +81,7 @@ SYMBOLS = {
     "bm_route_read": (_i, [_vp, _vp, _vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
     "bm_gemm": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp]),
     "bm_swiglu_quant": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
+    "bm_swiglu_quant_sel": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "bm_moe_combine": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "bm_set_gate_rule": (_i, [_vp, _i, C.c_float]),
     "bm_route_softmax": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
@@ -590,7 +591,11 @@ class Gpu:
     def set_gemm_mode(self, mode):
         self._check(self.lib.bm_set_gemm_mode(self.ctx, mode))
 
-    def enqueue_swiglu_quant(self, g, u, n_cols, act, rule=None):
+    def enqueue_swiglu_quant(self, g, u, n_cols, act, rule=None, sel=None, n_experts=0):
+        """With sel: only the columns of slots whose expert is on the stack (a host-served slot's column is left as it is)."""
+        if sel is not None:
+            self._check(self.lib.bm_swiglu_quant_sel(self.ctx, _ptr(g), _ptr(u), _ptr(sel), n_experts, n_cols, _rule(rule), act.handle))
+            return
         self._check(self.lib.bm_swiglu_quant(self.ctx, _ptr(g), _ptr(u), n_cols, _rule(rule), act.handle))
 
     def enqueue_route_softmax(self, logits, n_tokens, n_experts, top_k, renorm, probs, ids, weights):

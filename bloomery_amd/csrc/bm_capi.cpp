@@ -758,7 +758,7 @@ int bm_route_create(bm_ctx *ctx, int max_slots, int n_experts, bm_route **out) {
         return fail(ctx, BM_ESHAPE, "%s: 1 <= n_experts <= %d, got %d", what, bmk::kGemmMaxExperts, n_experts);
     bm_route *r = new (std::nothrow) bm_route{ctx, max_slots, n_experts, 0, nullptr, nullptr, nullptr};
     if (!r) return fail(ctx, BM_EDRIVER, "%s: out of host memory", what);
-    const size_t words = (size_t)max_slots + 2 * (size_t)bmk::gemm_max_tiles(max_slots, n_experts) + 2;
+    const size_t words = (size_t)max_slots + 2 * (size_t)bmk::gemm_max_tiles(max_slots, n_experts) + 3;
     hipError_t e = hipMalloc((void **)&r->cols, words * sizeof(uint32_t));
     if (e == hipSuccess) e = hipMemset(r->cols, 0, words * sizeof(uint32_t));
     if (e == hipSuccess) e = hipDeviceSynchronize(); // as in bm_act_create
@@ -935,14 +935,23 @@ int bm_scratch_set_path(bm_scratch *s, int path, int grouped_from, int gemm_from
     return BM_OK;
 }
 
+// Whether the per-slot step's two launches fit a workgroup's LDS at this shape (bm_moe_decode refuses a shape past it: the
+// token's column beside the quantizer's staging, and a token's slot columns beside the closing sum's operands).
+static bool per_slot_fits(const bm_scratch *s) {
+    const size_t lds_a = dev_col_bytes(s->gate_type, s->hidden) + 8192;
+    const size_t lds_b = (size_t)s->spt * dev_col_bytes(s->down_type, s->ff) + 12288;
+    return lds_a <= (size_t)bmk::kMaxLds && lds_b <= (size_t)bmk::kMaxLds;
+}
+
 int bm_scratch_path_for(const bm_scratch *s, int m) {
     if (!s || m < 1 || m > s->max_tokens) return BM_ESHAPE;
     const bool gemm_ok = bmk::gemm_supported(s->gate_type) && bmk::gemm_supported(s->down_type);
+    const bool per_slot_ok = m <= bmk::kMaxDecodeTokens && per_slot_fits(s);
     if (s->path != BM_PATH_AUTO) {
-        if (s->path == BM_PATH_PER_SLOT && m > bmk::kMaxDecodeTokens) return BM_PATH_GROUPED;
+        if (s->path == BM_PATH_PER_SLOT && !per_slot_ok) return BM_PATH_GROUPED;
         return s->path;
     }
-    if (m < s->grouped_from && m <= bmk::kMaxDecodeTokens) return BM_PATH_PER_SLOT;
+    if (m < s->grouped_from && per_slot_ok) return BM_PATH_PER_SLOT;
     if (m < (s->ctx->gemm_mode != BM_GEMM_EXACT ? s->gemm_from_fast : s->gemm_from) || !gemm_ok) return BM_PATH_GROUPED;
     return BM_PATH_GEMM;
 }
@@ -984,7 +993,7 @@ int bm_moe_forward(bm_ctx *ctx, bm_scratch *s, const bm_weights *wg, const bm_we
         if (!rc) rc = bm_route_fill(ctx, sel_dev, n_slots, s->route);
         if (!rc) rc = bm_gemm(ctx, wg, ff, s->act_x, s->route, spt, s->g);
         if (!rc) rc = bm_gemm(ctx, wu, ff, s->act_x, s->route, spt, s->u);
-        if (!rc) rc = bm_swiglu_quant(ctx, s->g, s->u, n_slots, rule, s->act_h);
+        if (!rc) rc = bm_swiglu_quant_sel(ctx, s->g, s->u, sel_dev, n_experts, n_slots, rule, s->act_h);
         if (!rc) rc = bm_gemm(ctx, wd, hidden, s->act_h, s->route, 0, s->down);
         if (rc) return rc;
         break;
@@ -1048,6 +1057,19 @@ int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_c
     bmk::Launch L;
     if (int rc = launch_under(ctx, what, rule, &L)) return rc;
     return driver(ctx, what, bmk::swiglu_quant(L, g_dev, u_dev, n_cols, act->k, act->dev, act_form(act->wtype) != 0));
+}
+
+int bm_swiglu_quant_sel(bm_ctx *ctx, const float *g_dev, const float *u_dev, const uint32_t *sel_dev, int n_experts, int n_cols,
+                        const bm_gate_act *rule, bm_act *act) {
+    const char *what = "bm_swiglu_quant_sel";
+    if (!ctx || !g_dev || !u_dev || !sel_dev || !act) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (n_experts < 1) return fail(ctx, BM_ESHAPE, "%s: n_experts = %d", what, n_experts);
+    if (n_cols < 1 || n_cols > act->m_cap) return fail(ctx, BM_ESHAPE, "%s: %d columns, the activation holds %d", what, n_cols, act->m_cap);
+    bmk::Launch L;
+    int rc = launch_under(ctx, what, rule, &L);
+    if (rc) return rc;
+    return driver(ctx, what,
+                  bmk::swiglu_quant(L, g_dev, u_dev, n_cols, act->k, act->dev, act_form(act->wtype) != 0, sel_dev, (uint32_t)n_experts));
 }
 
 int bm_weights_from_gguf(bm_ctx *ctx, const bm_gguf *g, const char *name, bm_weights **out, int *rows_per_expert, int *n_experts) {

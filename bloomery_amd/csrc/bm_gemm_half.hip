@@ -107,7 +107,7 @@ __global__ __launch_bounds__(kHThreads, 2) void k_gemm_half(const uint8_t *w, in
     if (g == count) { // the refused slots' rows: NaN (crates/gpu/src/gemm/grouped.rs:2283-2287)
         const u32 refused = n_tiles[1];
         for (u32 i = tid; i < refused * kHRows; i += kHThreads) {
-            const u32 s = cols[n_slots - refused + i / kHRows];
+            const u32 s = cols[n_slots - n_tiles[2] - refused + i / kHRows];
             const int r = row0 + (int)(i % kHRows);
             if (r < rpe) y[(size_t)s * rpe + r] = bm_bits_f32(0x7fc00000u);
         }

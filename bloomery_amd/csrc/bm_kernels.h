@@ -119,11 +119,13 @@ hipError_t gemv_tiles(const Launch &L, int wtype, const uint8_t *w, int n_expert
 constexpr int kGemmBN = 64, kGemmBM = 64;
 constexpr int kGemmMaxSlots = 40960, kGemmMaxExperts = 1024;
 int gemm_max_tiles(int n_slots, int n_experts);
-// cols[n_slots], tiles[2 * gemm_max_tiles], n_tiles[2]
+// cols[n_slots], tiles[2 * gemm_max_tiles], n_tiles[3]: tiles, refused slots, slots served elsewhere (not listed)
 hipError_t route(const Launch &L, const uint32_t *ids, int n_slots, int n_experts, uint32_t *cols, uint32_t *tiles,
                  uint32_t *n_tiles);
 // q8k: the columns are Q8_K ones (else Q8_2_X4)
-hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act, bool q8k);
+// sel (optional): column c is slot c's; a slot served elsewhere is left as it stands, another id at or past n_experts raises
+hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act, bool q8k,
+                        const uint32_t *sel = nullptr, uint32_t n_experts = 0);
 bool gemm_supported(int wtype);
 // slot_div: slots a token when every slot of a token reads the token's column, 1 when each slot reads its own.
 // mode 0: the CPU path's eight-accumulator f32 order (bit-identical to the row dots); 1: one accumulator a value, int8

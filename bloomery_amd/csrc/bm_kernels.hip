@@ -3,6 +3,8 @@
 // its fused forms, and the block-sum verification kernel.
 #include "bm_kernels.h"
 
+#include <atomic>
+
 #include "bm_stream.hpp"
 
 namespace bmk {
@@ -985,26 +987,28 @@ static __device__ __align__(256) uint8_t scratch[kStaticBytes];
 // stand-in, not device memory): the address is asked for once a device, with that device current, and every launch
 // takes it from here.
 constexpr int kStaticMaxDevices = 64;
-static uint8_t *g_scratch_at[kStaticMaxDevices];
+static std::atomic<uint8_t *> g_scratch_at[kStaticMaxDevices]; // contexts may be made from several threads at once
 
 hipError_t static_scratch_init(int device) {
     if (device < 0 || device >= kStaticMaxDevices) return hipErrorInvalidDevice;
-    if (g_scratch_at[device]) return hipSuccess;
+    if (g_scratch_at[device].load(std::memory_order_acquire)) return hipSuccess;
     void *at = nullptr;
     const hipError_t e = hipGetSymbolAddress(&at, HIP_SYMBOL(scratch));
     if (e != hipSuccess) return e;
     if (!at) return hipErrorInvalidSymbol;
-    g_scratch_at[device] = static_cast<uint8_t *>(at);
+    g_scratch_at[device].store(static_cast<uint8_t *>(at), std::memory_order_release); // every thread finds the same address
     return hipSuccess;
 }
 
 hipError_t moe_decode_static(const Launch &L, int device, int gate_type, int down_type, const float *x, const uint8_t *wg,
                              const uint8_t *wu, const uint8_t *wd, int n_experts, int hidden, int ff, const uint32_t *sel,
                              const float *wts, const float *resid, int slots_per_token, int m, float *y) {
-    if (device < 0 || device >= kStaticMaxDevices || !g_scratch_at[device]) return hipErrorNotInitialized;
+    uint8_t *base = device < 0 || device >= kStaticMaxDevices ? nullptr : g_scratch_at[device].load(std::memory_order_acquire);
+    if (!base) return hipErrorNotInitialized;
     if ((size_t)m * (size_t)slots_per_token * (size_t)ff > kStaticValues) return hipErrorInvalidValue;
-    uint8_t *act_h = g_scratch_at[device];
-    float *h = reinterpret_cast<float *>(g_scratch_at[device] + kStaticColBytes);
+    uint8_t *act_h = base;
+    // the f32 rows of h are only read by a down stack on Q8_K columns: no other call writes them
+    float *h = bm_takes_q8k(down_type) ? reinterpret_cast<float *>(base + kStaticColBytes) : nullptr;
     // every live slot's column (or f32 rows) is written whole by the first launch before the second reads it, and a
     // slot that is not live is never read into a sum: nothing here has to start at zero
     return moe_decode(L, gate_type, down_type, x, wg, wu, wd, n_experts, hidden, ff, sel, wts, resid,

@@ -31,15 +31,19 @@ int gemm_max_tiles(int n_slots, int n_experts) { // crates/gpu/src/gemm/route.rs
 // ------------------------------------------------------------------------------------------------ route
 
 // One workgroup: the slots listed by expert in ascending slot order (group_slots), bucket n_experts collecting the
-// refused ones at the list's end; then the tiles, an expert's run cut into runs of at most 64.
+// refused ones at the list's end; then the tiles, an expert's run cut into runs of at most 64. A slot served elsewhere
+// (id 0xffffffff, crates/gpu/src/kquant/sel.rs:22-28) is not listed and raises nothing: the list is that many entries
+// shorter, the entries past it hold 0xffffffff, and n_tiles[2] counts them.
 __global__ __launch_bounds__(kRouteThreads) void k_route(const u32 *ids, u32 n_slots, u32 n_experts, u32 *cols,
                                                          u32 *tiles, u32 *n_tiles, u32 *fault, u32 layer) {
     __shared__ GroupLds g;
     const u32 tid = threadIdx.x;
     group_slots(g, n_slots, n_experts + 1, cols, [&](u32 s) {
         const u32 id = ids[s];
-        return id < n_experts ? id : n_experts;
+        return id < n_experts ? id : id == 0xffffffffu ? kNoBucket : n_experts;
     });
+    const u32 listed = g.base[n_experts + 1];
+    for (u32 i = listed + tid; i < n_slots; i += kRouteThreads) cols[i] = 0xffffffffu;
     u32 j0 = 0, j1 = 0;
     if (tid < n_experts) {
         j0 = g.base[tid];
@@ -57,6 +61,7 @@ __global__ __launch_bounds__(kRouteThreads) void k_route(const u32 *ids, u32 n_s
         if (refused) bm_raise(fault, layer, kSiteExpertId);
         n_tiles[0] = total;
         n_tiles[1] = refused;
+        n_tiles[2] = n_slots - listed;
     }
 }
 
@@ -71,12 +76,24 @@ hipError_t route(const Launch &L, const uint32_t *ids, int n_slots, int n_expert
 
 // crates/gpu/src/gemm/swiglu.rs:46-58 in the CPU path's rules: column c of act = Q8_2_X4(swiglu(g, u)) over the k
 // values g[c * k ..], u[c * k ..]. One half wave a 32-value block.
+// `sel` (optional; crates/gpu/src/gemm/swiglu.rs:96-140 enqueue_swiglu_act_quant_sel): column c belongs to slot c; a slot
+// served elsewhere (id 0xffffffff) keeps its column as it stands and raises nothing, any other id at or past n_experts
+// raises ExpertId with nothing stored.
+__device__ __forceinline__ bool swiglu_column_skipped(const u32 *sel, u32 n_experts, int col, bool first, u32 *fault, u32 layer) {
+    if (!sel) return false;
+    const u32 id = sel[col];
+    if (id < n_experts) return false;
+    if (id != 0xffffffffu && first) bm_raise(fault, layer, kSiteExpertId);
+    return true;
+}
+
 __global__ __launch_bounds__(256) void k_swiglu_quant(const float *g, const float *u, int m, int k, uint8_t *act,
-                                                      GateRule rule, u32 *fault, u32 layer) {
+                                                      GateRule rule, const u32 *sel, u32 n_experts, u32 *fault, u32 layer) {
     const int bpc = k / 32;
     const long gblk = (long)blockIdx.x * 8 + (threadIdx.x >> 5);
     if (gblk >= (long)m * bpc) return;
     const int col = (int)(gblk / bpc), blk = (int)(gblk % bpc), lane32 = threadIdx.x & 31;
+    if (swiglu_column_skipped(sel, n_experts, col, blk == 0 && lane32 == 0, fault, layer)) return; // uniform over the half wave
     const size_t at = (size_t)col * k + 32 * blk + lane32;
     bool odd;
     const float v = bm_gate_rule(rule.act, rule.limit, g[at], u[at], odd);
@@ -90,9 +107,10 @@ __global__ __launch_bounds__(256) void k_swiglu_quant(const float *g, const floa
 
 // The same into Q8_K columns, for a down stack that dots against those (IQ2_XXS, ...): one workgroup a 256-value block.
 __global__ __launch_bounds__(256) void k_swiglu_quant_q8k(const float *g, const float *u, int m, int k, uint8_t *act,
-                                                          GateRule rule, u32 *fault, u32 layer) {
+                                                          GateRule rule, const u32 *sel, u32 n_experts, u32 *fault, u32 layer) {
     const int bpc = k / 256;
     const int col = blockIdx.x / bpc, blk = blockIdx.x % bpc;
+    if (swiglu_column_skipped(sel, n_experts, col, blk == 0 && threadIdx.x == 0, fault, layer)) return; // uniform over the workgroup
     const size_t at = (size_t)col * k + 256 * blk + threadIdx.x;
     bool odd;
     const float v = bm_gate_rule(rule.act, rule.limit, g[at], u[at], odd);
@@ -102,10 +120,11 @@ __global__ __launch_bounds__(256) void k_swiglu_quant_q8k(const float *g, const 
 
 // The Q8_2_X4 form with eight values a thread, a block a quad of lanes: two 16-byte loads of each input a thread.
 __global__ __launch_bounds__(256) void k_swiglu_quant_wide(const float *g, const float *u, int m, int k, uint8_t *act,
-                                                           GateRule rule, u32 *fault, u32 layer) {
+                                                           GateRule rule, const u32 *sel, u32 n_experts, u32 *fault, u32 layer) {
     const long at = ((long)blockIdx.x * 256 + threadIdx.x) * 8;
     if (at >= (long)m * k) return;
     const int col = (int)(at / k), o = (int)(at % k);
+    if (swiglu_column_skipped(sel, n_experts, col, o == 0, fault, layer)) return; // uniform over a block's quad of lanes
     const float4 g0 = *reinterpret_cast<const float4 *>(g + at), g1 = *reinterpret_cast<const float4 *>(g + at + 4);
     const float4 u0 = *reinterpret_cast<const float4 *>(u + at), u1 = *reinterpret_cast<const float4 *>(u + at + 4);
     const float gv[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
@@ -122,21 +141,22 @@ __global__ __launch_bounds__(256) void k_swiglu_quant_wide(const float *g, const
     q82_quad8(v, act + (size_t)col * (k / 256) * BM_Q82_SB_EXT, k / 256, o >> 5, threadIdx.x & 3, fault, layer);
 }
 
-hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act, bool q8k) {
+hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act, bool q8k, const uint32_t *sel,
+                        uint32_t n_experts) {
     if (!q8k && (((uintptr_t)g | (uintptr_t)u) & 15) == 0) {
         const long threads = (long)m * k / 8;
         hipLaunchKernelGGL(k_swiglu_quant_wide, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, L.stream, g, u, m, k, act,
-                           L.rule, L.fault, L.layer);
+                           L.rule, sel, n_experts, L.fault, L.layer);
         return hipGetLastError();
     }
     if (q8k) {
         hipLaunchKernelGGL(k_swiglu_quant_q8k, dim3((unsigned)(m * (k / 256))), dim3(256), 0, L.stream, g, u, m, k, act, L.rule,
-                           L.fault, L.layer);
+                           sel, n_experts, L.fault, L.layer);
         return hipGetLastError();
     }
     const long blocks = (long)m * (k / 32);
     hipLaunchKernelGGL(k_swiglu_quant, dim3((unsigned)((blocks + 7) / 8)), dim3(256), 0, L.stream, g, u, m, k, act,
-                       L.rule, L.fault, L.layer);
+                       L.rule, sel, n_experts, L.fault, L.layer);
     return hipGetLastError();
 }
 
@@ -208,7 +228,7 @@ __global__ __launch_bounds__(256 * CH) void k_gemm(const uint8_t *w, int rpe, in
     if (g == count) { // the refused slots' rows: NaN (crates/gpu/src/gemm/grouped.rs:2283-2287)
         const u32 refused = part0 == 0 ? n_tiles[1] : 0u;
         for (u32 i = tid; i < refused * kGemmBM; i += blockDim.x) {
-            const u32 s = cols[n_slots - refused + i / kGemmBM];
+            const u32 s = cols[n_slots - n_tiles[2] - refused + i / kGemmBM];
             const int r = row0 + (int)(i % kGemmBM);
             if (r < rpe) y[(size_t)s * rpe + r] = bm_bits_f32(0x7fc00000u);
         }
@@ -547,7 +567,7 @@ __global__ __launch_bounds__(kFastThreads, 2) void k_gemm_fast(const uint8_t *w,
     if (g == count) { // the refused slots' rows: NaN (crates/gpu/src/gemm/grouped.rs:2283-2287)
         const u32 refused = n_tiles[1];
         for (u32 i = tid; i < refused * kFastRows; i += kFastThreads) {
-            const u32 s = cols[n_slots - refused + i / kFastRows];
+            const u32 s = cols[n_slots - n_tiles[2] - refused + i / kFastRows];
             const int r = row0 + (int)(i % kFastRows);
             if (r < rpe) y[(size_t)s * rpe + r] = bm_bits_f32(0x7fc00000u);
         }
@@ -837,7 +857,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, 
     if (g == count) { // the refused slots' rows: NaN (crates/gpu/src/gemm/grouped.rs:2283-2287)
         const u32 refused = n_tiles[1];
         for (u32 i = tid; i < refused * kIqRows; i += 256) {
-            const u32 s = cols[n_slots - refused + i / kIqRows];
+            const u32 s = cols[n_slots - n_tiles[2] - refused + i / kIqRows];
             const int r = row0 + (int)(i % kIqRows);
             if (r < rpe) y[(size_t)s * rpe + r] = bm_bits_f32(0x7fc00000u);
         }

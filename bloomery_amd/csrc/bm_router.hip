@@ -242,6 +242,9 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
     __syncthreads();
     if (!gain && normed_out && e0 == 0) // the rows as they are (read after the barrier: other threads staged them)
         for (int i = tid; i < hidden; i += 256) normed_out[(size_t)t * hidden + i] = xs[(i & 7) * line + (i >> 3)];
+    // every thread that stores a logit below is of the first wave: k_norm_route's hand-over (a device-scope count updated by
+    // thread 0 behind the workgroup's barrier) publishes that wave's stores and relies on it
+    static_assert(8 * R <= 64, "the logits of a workgroup are stored by its first wave");
     if (tid < 8 * R) {
         const int r = tid >> 3, l = tid & 7;
         const float4 *xl = reinterpret_cast<const float4 *>(xs + l * line);

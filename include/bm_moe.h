@@ -301,11 +301,12 @@ void bm_route_destroy(bm_route *route);
 /* GemmKernels::enqueue_route (crates/gpu/src/gemm/route.rs:351): the table of ids_dev[0 .. n_slots) (slot =
  * token * top_k + k), built on the device: the slots grouped by expert, ascending inside an expert, cut into
  * tiles of at most 64. An id at or past the stack raises BM_SITE_EXPERT_ID; its slot is left out of the tiles
- * and listed as refused, and every bm_gemm over the table writes NaN into its rows. */
+ * and listed as refused, and every bm_gemm over the table writes NaN into its rows. A slot whose id is BM_HOST_SLOT is
+ * not listed at all and raises nothing (crates/gpu/src/kquant/sel.rs:22-28): no bm_gemm over the table touches its rows. */
 int bm_route_fill(bm_ctx *ctx, const uint32_t *ids_dev, int n_slots, bm_route *route);
 /* GemmRoute::read_back / refused_back (route.rs:188-245): synchronise and copy the table out. cols_host (optional)
- * takes the n_slots slot list (refused slots last); tiles_host (optional) two words a tile: expert, then
- * first index | length << 16. */
+ * takes the n_slots slot list (refused slots last; behind them BM_HOST_SLOT once for every slot that is not listed);
+ * tiles_host (optional) two words a tile: expert, then first index | length << 16. */
 int bm_route_read(bm_ctx *ctx, const bm_route *route, uint32_t *cols_host, uint32_t *tiles_host, int *n_tiles, int *n_refused);
 /* GemmKernels::enqueue_gemm(GemmArgs) (crates/gpu/src/gemm/grouped.rs:2125-2133,2300), Q4_K, Q5_K and Q6_K stacks against
  * Q8_2_X4 columns and IQ2_XXS stacks (crates/gpu/src/gemm/kernels.rs:867 gemm_iq2xxs) against Q8_K columns:
@@ -333,6 +334,13 @@ int bm_set_gemm_mode(bm_ctx *ctx, int mode);
  * silu(g) * u of g_dev / u_dev[c * k .. (c + 1) * k), k = act's k, slot-major as the gate and up GEMMs write them;
  * bm_quantize's bytes of the CPU path's SwiGLU, in the column form of act's type (Q8_2_X4 or Q8_K). */
 int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_cols, const bm_gate_act *rule, bm_act *act);
+/* GemmKernels::enqueue_swiglu_act_quant_sel (crates/gpu/src/gemm/swiglu.rs:96-140): bm_swiglu_quant over the columns of
+ * slots 0 .. n_cols whose expert sel_dev[c] is on the stack. The column of a slot served elsewhere (BM_HOST_SLOT) is left
+ * exactly as it stands, whatever its g / u rows hold, and raises nothing (a bm_gemm over the route reads listed columns
+ * only); any other id at or past n_experts raises BM_SITE_EXPERT_ID with nothing stored. The written columns' bytes are
+ * bm_swiglu_quant's. */
+int bm_swiglu_quant_sel(bm_ctx *ctx, const float *g_dev, const float *u_dev, const uint32_t *sel_dev, int n_experts, int n_cols,
+                        const bm_gate_act *rule, bm_act *act);
 
 
 /* ------------------------------------------------------------------ one entry for every number of tokens */
@@ -343,7 +351,7 @@ int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_c
  *   BM_PATH_PER_SLOT  bm_moe_decode: two launches, every slot streams its expert's rows (repeats come from the caches);
  *   BM_PATH_GROUPED   bm_tables, bm_quantize, bm_gate_up_tiles (bm_quantize_ord for a down stack on Q8_K columns),
  *                     bm_gemv_tiles, the slots' sum: an expert's rows are read once for all of its slots;
- *   BM_PATH_GEMM      bm_quantize, bm_route_fill, bm_gemm twice, bm_swiglu_quant, bm_gemm, the slots' sum: the int8 matrix
+ *   BM_PATH_GEMM      bm_quantize, bm_route_fill, bm_gemm twice, bm_swiglu_quant_sel, bm_gemm, the slots' sum: the int8 matrix
  *                     cores (in the f32 order bm_set_gemm_mode sets; Q4_K, Q5_K, Q6_K and IQ2_XXS stacks).
  * In the exact mode all three give the same bits in y_dev. bm_scratch holds what the paths need between their launches for
  * up to max_tokens tokens (made at load time and shared by every layer of the same shape, as the reference's Q8Act scratch
@@ -352,8 +360,8 @@ int bm_swiglu_quant(bm_ctx *ctx, const float *g_dev, const float *u_dev, int n_c
  * the Qwen3-30B-A3B layer shape: 22 tokens, and 448 tokens in the exact mode of bm_gemm or 96 in its tolerance mode.
  * bm_scratch_set_path sets others (0 keeps a value; gemm_from then holds for both modes) or forces one path.
  * bm_scratch_path_for: the path a call with m tokens takes. A slot whose id names no expert of the stack adds nothing to
- * the sum (and raises BM_SITE_EXPERT_ID unless it is BM_HOST_SLOT, which the GEMM path's route table raises as well:
- * batches with host-served slots go through the separate launches). Calls that share a scratch must not overlap. */
+ * the sum and raises BM_SITE_EXPERT_ID unless it is BM_HOST_SLOT, which every path skips silently (the GEMM path's route
+ * table does not list it, and its SwiGLU quantizer is bm_swiglu_quant_sel). Calls that share a scratch must not overlap. */
 typedef struct bm_scratch bm_scratch;
 #define BM_PATH_AUTO 0
 #define BM_PATH_PER_SLOT 1

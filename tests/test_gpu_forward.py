@@ -71,6 +71,14 @@ def test_the_automatic_choice_follows_the_crossovers(gpu):
         assert "bm_scratch_set_path" in str(e.value)
     finally:
         sc.free()
+    # a shape whose slot columns do not fit the per-slot step's LDS (64 slots of ff 2048) goes grouped from the first token
+    sc = gpu.scratch(bm.Q4_K, bm.Q6_K, 512, 2048, 4, 64, 8)
+    try:
+        assert [sc.path_for(m) for m in (1, 8)] == [bm.PATH_GROUPED, bm.PATH_GROUPED]
+        sc.set_path(bm.PATH_PER_SLOT)
+        assert sc.path_for(1) == bm.PATH_GROUPED
+    finally:
+        sc.free()
     # a type without a grouped GEMM never takes that path, and says so when asked to
     sc = gpu.scratch(bm.IQ4_XS, bm.IQ4_XS, 512, 256, 4, 2, 512)
     try:
@@ -89,8 +97,9 @@ def test_the_automatic_choice_follows_the_crossovers(gpu):
 
 
 def test_a_slot_without_an_expert_adds_nothing_on_every_path(gpu):
-    """A host-served slot and an id past the stack: the token's sum is the oracle's over its live slots on each path (the
-    id past the stack raises ExpertId; the grouped GEMM's route table raises it for the host's slot as well)."""
+    """A host-served slot and an id past the stack: the token's sum is the oracle's over its live slots on each path, and
+    the id past the stack raises ExpertId. With host-served slots only, no path raises anything (the GEMM path's route table
+    does not list them and its SwiGLU quantizer leaves their columns alone, crates/gpu/src/gemm/swiglu.rs:96-140)."""
     L = Layer(gpu, (bm.Q4_K, bm.Q4_K, bm.Q6_K), 512, 256, 4, 5200)
     rng = np.random.default_rng(5201)
     m, top_k = 3, 3
@@ -112,6 +121,19 @@ def test_a_slot_without_an_expert_adds_nothing_on_every_path(gpu):
             assert_f32(y.download(), want, name)
             assert gpu.fault()[1] & (1 << bm.SITE_EXPERT_ID)  # (the refused slot's NaN rows may raise the quantizer's site too)
         gpu.fault_clear()
+        # host-served slots only: the same sums over the live slots, and no fault on any path
+        ids_h = np.array([[1, bm.HOST_SLOT, 3], [bm.HOST_SLOT, 0, bm.HOST_SLOT], [0, 2, 1]], np.uint32)
+        want_h = np.concatenate([L.oracle(x[:1], np.array([[1, 3]], np.uint32), np.array([[0.5, 0.2]], np.float32), 2)[0],
+                                 L.oracle(x[1:2], np.array([[0]], np.uint32), np.array([[0.5]], np.float32), 1)[0],
+                                 L.oracle(x[2:], ids_h[2:], wts[2:], 3)[0]])
+        sel_h = gpu.upload(ids_h, np.uint32)
+        for path, name in PATHS:
+            sc.set_path(path)
+            y.fill_bytes(0xFF)
+            gpu.enqueue_moe_forward(sc, L.dg, L.du, L.dd, xd, sel_h, wd, None, m, y)
+            assert_f32(y.download(), want_h, name + ", host-served slots")
+            assert gpu.fault() == (bm.FAULT_NONE, 0), name
+        sel_h.free()
     finally:
         sc.free()
         for b in (xd, sel, wd, y):

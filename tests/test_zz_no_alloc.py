@@ -38,6 +38,29 @@ def test_noalloc_matches_bm_moe_decode_on_two_calls_in_a_row(types, hidden, ff, 
         assert gpu.fault() == (bm.FAULT_NONE, 0)
         for b in (xd, sel, wd, rd, act_h, h, y_ref, y_new):
             b.free()
+    # under graph capture (where an allocation would fail the capture), replayed twice with other work between the replays
+    m = 2
+    x, resid = normal_f32(rng, (m, hidden)), normal_f32(rng, (m, hidden))
+    ids, wts = route(rng, m, n_experts, top_k)
+    xd, sel, wd, rd = (gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32), gpu.upload(resid, np.float32))
+    act_h, h = gpu.act(types[2], ff, m * top_k), gpu.buffer(np.float32, m * top_k * ff)
+    y_ref, y_new = gpu.buffer(np.float32, m * hidden).fill_bytes(0xFF), gpu.buffer(np.float32, m * hidden)
+    gpu.enqueue_moe_decode(L.dg, L.du, L.dd, xd, sel, wd, rd, top_k, m, act_h, y_ref, h=h)
+    want = y_ref.download()
+    gpu.capture_begin()
+    gpu.enqueue_moe_decode_noalloc(L.dg, L.du, L.dd, xd, sel, wd, rd, top_k, m, y_new)
+    graph = gpu.capture_end()
+    for replay in range(2):
+        y_new.fill_bytes(0xFF)
+        gpu.graph_launch(graph)
+        got = y_new.download()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), f"replay {replay}"
+        gpu.enqueue_moe_decode(L.dg, L.du, L.dd, xd, sel, wd, rd, top_k, m, act_h, y_ref, h=h)  # eager work between the replays
+        gpu.sync()
+    gpu.graph_destroy(graph)
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    for b in (xd, sel, wd, rd, act_h, h, y_ref, y_new):
+        b.free()
     # past the array's size: refused by name before any launch
     m = 65536 // (top_k * ff) + 1
     xd, sel, wd = gpu.upload(np.zeros((m, hidden), np.float32)), gpu.upload(np.zeros((m, top_k), np.uint32)), \

@@ -744,14 +744,18 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2048)
     ap.add_argument("--warmup", type=int, default=256)
-    ap.add_argument("--layers", type=int, default=4, help="distinct device copies of the layer cycled through")
+    ap.add_argument("--layers", type=int, default=32,
+                    help="distinct device copies of the layer cycled through: step i takes copy i %% layers, so with 64 tokens and 32 "
+                         "copies two reads of the same expert of the same copy lie 32 steps = 780 MB apart, three times the memory-side "
+                         "cache")
     ap.add_argument("--tokens", type=int, default=64, help="distinct tokens (and routings) cycled through")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
     ap.add_argument("--one-interval", action="store_true",
-                    help="config 2 only: exactly --steps steps (rounded up to whole replays) with one event interval around them all, instead "
-                         "of at least 32 replays with an interval each: for runs under a profiler")
+                    help="config 2 only: leave out the 32 replays with an event after each that give the median beside `value` (one replay "
+                         "instead): for runs under a profiler, whose interception of a graph launch has crashed with events recorded between "
+                         "the launches")
     ap.add_argument("--no-prefill", action="store_true", help="config 2 only: leave the prefill leg (config 4's step) out of the line")
     ap.add_argument("--types", default="q4_k,q6_k",
                     help="config 2 only: gate/up and down weight types (q3_k, q4_k, q5_k, q6_k, iq2_xxs, iq3_xxs, iq4_xs); other than the default is "
@@ -859,39 +863,55 @@ def main():
         log(f"[bench] parity {parity}")
         assert err <= 1e-4, parity
 
-    # one graph of `unit` steps; the timed region replays it at least 32 times (8192 steps), whatever
-    # --steps asks for below that: a replay is under a millisecond of GPU time, and the figure is a median, not one sample
-    unit = max(len(layers) * n_tok // np.gcd(len(layers), n_tok), 1)
-    unit = min(max(int(unit), 256), 256)  # a graph of 256 steps (a token's graph in a model of this size holds as many launches): the replay call itself costs microseconds
-    gpu.capture_begin()
-    for i in range(unit):
-        enqueue_step(i)
-    graph = gpu.capture_end()
-    reps_w = max(1, -(-args.warmup // unit))
-    reps = -(-args.steps // unit) if args.one_interval else max(32, -(-max(args.steps, 2048) // unit))
-    steps = reps * unit
-    for _ in range(reps_w):
-        gpu.graph_launch(graph)
+    # The timed region is exactly --steps steps behind exactly --warmup untimed ones: graphs of up to 256 steps (a token's
+    # graph in a model of this size holds as many launches) replayed back to back, the remainder as a shorter graph. Everything
+    # is enqueued before the first event can fire (two replays of the 256-step graph go first, untimed, so the device is busy
+    # meanwhile), so the events bracket device time only; `value` is the event time of the region over its steps. Beside it, whatever --steps says: at least 32 replays of the 256-step graph with an event after
+    # each, and their median, minimum and maximum (a replay is under three milliseconds of device time).
+    unit = 256
+    graphs = {}
+
+    def graph_of(n):
+        if n not in graphs:
+            gpu.capture_begin()
+            for i in range(n):
+                enqueue_step(i)
+            graphs[n] = gpu.capture_end()
+        return graphs[n]
+
+    def run_steps(n):
+        for _ in range(n // unit):
+            gpu.graph_launch(graph_of(unit))
+        if n % unit:
+            gpu.graph_launch(graph_of(n % unit))
+
+    steps, warm = max(1, args.steps), max(0, args.warmup)
+    for n in {unit, steps % unit, warm % unit} - {0}:
+        graph_of(n)
     gpu.sync()
-    # an event after every replay (--one-interval: only around them all, for runs under a profiler, whose interception
-    # of a graph launch has crashed here when events were recorded between the launches)
-    stride = reps if args.one_interval else 1
-    marks = [gpu.event() for _ in range(reps // stride + 1)]
+    e0, e1 = gpu.event(), gpu.event()
     t_start = time.perf_counter()
+    run_steps(2 * unit)  # a lead-in that keeps the device busy while the host enqueues what follows: the events then see no idle gap
+    run_steps(warm)
+    gpu.event_record(e0)
+    run_steps(steps)
+    gpu.event_record(e1)
+    gpu.sync()
+    wall_ms = (time.perf_counter() - t_start) * 1e3
+    ev_ms = gpu.event_elapsed_ms(e0, e1)
+    ms_per_step = ev_ms / steps
+    us_per_token = ms_per_step * 1e3
+    graph = graph_of(unit)
+    reps = 1 if args.one_interval else 32
+    marks = [gpu.event() for _ in range(reps + 1)]
     gpu.event_record(marks[0])
     for r in range(reps):
         gpu.graph_launch(graph)
-        if (r + 1) % stride == 0:
-            gpu.event_record(marks[(r + 1) // stride])
+        gpu.event_record(marks[r + 1])
     gpu.sync()
-    wall_ms = (time.perf_counter() - t_start) * 1e3
-    ev_ms = gpu.event_elapsed_ms(marks[0], marks[-1])
-    replay_us = sorted(gpu.event_elapsed_ms(marks[r], marks[r + 1]) * 1e3 / (unit * stride) for r in range(len(marks) - 1))
+    replay_us = sorted(gpu.event_elapsed_ms(marks[r], marks[r + 1]) * 1e3 / unit for r in range(reps))
     for ev in marks:
         gpu.event_destroy(ev)
-    e0, e1 = gpu.event(), gpu.event()
-    ms_per_step = wall_ms / steps
-    us_per_token = ms_per_step * 1e3
     replay_stats = {"replays": reps, "steps_per_replay": unit, "median_us_per_token": replay_us[len(replay_us) // 2],
                     "min_us_per_token": replay_us[0], "max_us_per_token": replay_us[-1]}
     bytes_per_token = TOP_K * (2 * FF * bm.row_bytes(gate_t, HIDDEN) + HIDDEN * bm.row_bytes(down_t, FF))
@@ -996,8 +1016,24 @@ def main():
                     break
         finally:
             ora.lib.ora_pool_destroy(pool)
+        # the same on one thread, a shorter sample
+        pool1 = ora.lib.ora_pool_create(1)
+        try:
+            ora.moe_forward(HIDDEN, FF, N_EXPERTS, types3, wg, wu, wd, x[0], ids[0], wts[0], TOP_K, avx2_pool=pool1)
+            n1, t1 = 0, time.perf_counter()
+            while True:
+                ora.moe_forward(HIDDEN, FF, N_EXPERTS, types3, wg, wu, wd, x[n1 % n_tok], ids[n1 % n_tok], wts[n1 % n_tok], TOP_K,
+                                avx2_pool=pool1)
+                n1 += 1
+                el1 = time.perf_counter() - t1
+                if el1 >= args.cpu_seconds / 3 and n1 >= 10:
+                    break
+        finally:
+            ora.lib.ora_pool_destroy(pool1)
         gbs = bytes_per_token * n / el / 1e9
-        cpu = {"value": el / n * 1e6, "unit": "us/token", "cores": threads, "kind": "port",
+        single = {"value": el1 / n1 * 1e6, "unit": "us/token", "cores": 1, "gb_per_s": bytes_per_token * n1 / el1 / 1e9,
+                  "sample": f"{n1} tokens on one thread, {el1:.1f}s"}
+        cpu = {"value": el / n * 1e6, "unit": "us/token", "cores": threads, "kind": "port", "single_thread": single,
                "sample": f"{n} tokens of the same layer and routings, AVX2 restatement of qdot on {threads} threads (the "
                          f"box's worker-pool size), {el:.1f}s; {gbs:.1f} GB/s of expert rows = {gbs / threads:.2f} GB/s a thread "
                          "(the reference documents about 12 GB/s a core and 130 GB/s on 32 cores for its own build, "
@@ -1010,7 +1046,7 @@ def main():
         "unit": "us/token",
         "n_gpus": 1,
         "steps": steps,
-        "warmup": reps_w * unit,
+        "warmup": warm,
         "ms_per_step": ms_per_step,
         "higher_is_better": False,
         "scaling": "weak",
@@ -1024,7 +1060,7 @@ def main():
                    "layer_copies": len(layers), "distinct_tokens": n_tok, "launches_per_step": len(kernels), "mode": "hipGraph replay"},
         "hbm_tbps": bytes_per_token / (us_per_token * 1e-6) / 1e12,
         "algorithmic_bytes_per_token": bytes_per_token,
-        "event_ms_per_step": ev_ms / steps,
+        "wall_ms_lead_in_warmup_and_steps": wall_ms,
         "replay_us_per_token": replay_stats,
         "kernel_us": kernel_us,
         "kernel_gbps": kernel_gbps,

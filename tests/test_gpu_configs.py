@@ -1,6 +1,6 @@
 """GPU parity tests at the shapes the benchmark's configurations name, through the C ABI, against the CPU oracle on the
-same seeded inputs: the DeepSeek-V3-shaped layer (IQ2_XXS routed experts over a resident subset, one Q6_K shared expert,
-the shared-expert combine) on the grouped and on the per-slot path, and the prefill GEMMs at the Qwen3-shaped layer's
+same seeded inputs: the DeepSeek-V3-shaped layer (IQ2_XXS routed experts over a resident subset, and over all 256, one Q6_K
+shared expert, the shared-expert combine) on the grouped and on the per-slot path, and the prefill GEMMs at the Qwen3-shaped layer's
 two matrix shapes under a skewed routing (an expert with three tiles, an expert with none). Also: a slot the host
 serves through every gate . up entry, and stacks wrapped in place. Contracts: crates/gpu/src/iq_sel.rs:1357,1557,
 crates/gpu/src/gemm/route.rs:351, crates/gpu/src/kquant/sel.rs:22-28, crates/gpu/src/moe_fused.rs:129-170."""
@@ -74,6 +74,54 @@ def test_deepseek_shaped_layer_grouped(gpu, ds_layer):
     assert gpu.fault() == (bm.FAULT_NONE, 0)
     for b in (sel, order, start, tiles, xd, wd, act, act_h, h, down, y, sdown) + keep:
         b.free()
+
+
+def test_deepseek_shaped_layer_with_all_256_experts_resident(gpu):
+    """BASELINE configs[4] with its whole routed stack on the card: 256 IQ2_XXS experts of hidden 7168 / ff 2048 (2.9 GB of
+    random legal blocks), 4 tokens, top-8 drawn over all 256. The grouped step and the per-slot step are separate kernels and
+    must agree bit for bit on every slot's h and every token's y, and both are the oracle's (which only visits the 32 slots'
+    experts, so the full comparison is affordable)."""
+    n_experts, m, top_k = 256, DS_TOKENS, DS_TOPK
+    n_slots = m * top_k
+    routed = Layer(gpu, (bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ2_XXS), DS_HIDDEN, DS_FF, n_experts, 3300, cheap=True)
+    try:
+        rng = np.random.default_rng(3301)
+        x = normal_f32(rng, (m, DS_HIDDEN))
+        ids, wts = route(rng, m, n_experts, top_k)
+        ids[1, 3] = 255  # the stack's last expert takes part
+        ids[2, 0] = ids[0, 0]  # and one expert has two slots: a tile of two
+        assert len(np.unique(ids[1])) == top_k and len(np.unique(ids[2])) == top_k
+        want_y, want_h = routed.oracle(x, ids, wts, top_k)
+        gpu.fault_clear()
+        xd, sel_d, wd = gpu.upload(x, np.float32), gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32)
+        # the per-slot step
+        act_h = gpu.act(bm.IQ2_XXS, DS_FF, n_slots)
+        h = gpu.buffer(np.float32, n_slots * DS_FF).fill_bytes(0xFF)
+        y = gpu.buffer(np.float32, m * DS_HIDDEN).fill_bytes(0xFF)
+        gpu.enqueue_moe_decode(routed.dg, routed.du, routed.dd, xd, sel_d, wd, None, top_k, m, act_h, y, h=h)
+        h_slot, y_slot = h.download(), y.download()
+        # the grouped step
+        sel, order, start, tiles = grouped_tables_on_device(gpu, ids.reshape(-1), n_experts)
+        act = gpu.act(bm.IQ2_XXS, DS_HIDDEN, m)
+        act_g = gpu.act(bm.IQ2_XXS, DS_FF, n_slots)
+        hg = gpu.buffer(np.float32, n_slots * DS_FF).fill_bytes(0xFF)
+        down = gpu.buffer(np.float32, n_slots * DS_HIDDEN).fill_bytes(0xFF)
+        yg = gpu.buffer(np.float32, m * DS_HIDDEN).fill_bytes(0xFF)
+        gpu.enqueue_quantize(xd, m, act)
+        gpu.enqueue_gate_up_tiles(routed.dg, routed.du, act, order, start, tiles, n_slots, DS_FF, top_k, hg)
+        gpu.enqueue_quantize_ord(hg, start, n_experts, n_slots, act_g)
+        gpu.enqueue_gemv_tiles(routed.dd, act_g, order, start, tiles, n_slots, DS_HIDDEN, down)
+        gpu.enqueue_combine_tokens(down, wd, None, DS_HIDDEN, top_k, m, yg)
+        h_grouped = hg.download().reshape(n_slots, DS_FF)
+        assert np.array_equal(h_grouped.view(np.uint32), h_slot.reshape(n_slots, DS_FF)[order.download()].view(np.uint32)), "h: grouped against per slot"
+        assert np.array_equal(yg.download().view(np.uint32), y_slot.view(np.uint32)), "y: grouped against per slot"
+        assert_f32(h_slot, want_h, "h against the oracle")
+        assert_f32(y_slot, want_y, "y against the oracle")
+        assert gpu.fault() == (bm.FAULT_NONE, 0)
+        for b in (xd, sel_d, wd, act_h, h, y, sel, order, start, tiles, act, act_g, hg, down, yg):
+            b.free()
+    finally:
+        routed.free()
 
 
 def test_long_rows_few_slots_an_expert_one_tile_launch(gpu, ds_layer):

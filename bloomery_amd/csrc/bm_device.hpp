@@ -590,11 +590,11 @@ __device__ __forceinline__ Blk<BM_IQ2XXS> bm_load_iq2xxs(const uint8_t *wrow, in
     return b;
 }
 
-// LDS tables of the IQ2_XXS decode. The CPU path dots the unsigned bytes u = +-mag + 43 (0 .. 86) and takes the 43s
-// back out through the column's sums, so the tables give u with one operation a word: a grid point is kept as its
-// eight bytes 43 + mag (x, y) and its eight bytes 43 - mag (z, w), a sign index as eight byte masks (0xff where the
-// value is negative), and u is a bitwise pick between the two by the mask (v_bfi_b32).
-// IQ3_XXS: the same with the offset 64 and grid points of four magnitudes: an entry is (64 + mag, 64 - mag).
+// LDS tables of the IQ decodes. The CPU path dots the unsigned bytes u = +-mag + off (IQ2_XXS: off 43, IQ3_XXS: 64) and
+// takes the offsets back out through the column's sums. IQ2_XXS: selector tables and a byte permute (bm_iq2_codes below).
+// IQ3_XXS: a grid point of four magnitudes is kept as its four bytes 64 + mag and its four bytes 64 - mag, a sign index as
+// eight byte masks (0xff where the value is negative), and u is a bitwise pick between the two by the mask (one operation a
+// word).
 __device__ __forceinline__ u32 bm_iq_pick(u32 plus, u32 minus, u32 mask) { return (minus & mask) | (plus & ~mask); }
 
 // a * b + c over 24-bit factors as one multiply-add: the empty statement pins the running sum, so the compiler cannot
@@ -607,10 +607,22 @@ __device__ __forceinline__ int bm_mad24_chain(int a, int b, int c) {
     return r;
 }
 struct Iq2Tables {
-    const uint4 *grid;  // IQ2_XXS
-    const uint2 *grid3; // IQ3_XXS
-    const uint2 *signs;
+    const uint2 *grid;  // IQ2_XXS: a grid point's eight magnitude selectors (0, 1, 2), a byte each
+    const uint2 *grid3; // IQ3_XXS: (64 + magnitudes, 64 - magnitudes) of a four-value grid point
+    const uint2 *signs; // IQ2_XXS: 4 in the bytes of the negative values; IQ3_XXS: 0xff there
 };
+
+// The eight code bytes 43 +- magnitude of an IQ2_XXS group (what the CPU path dots, crates/qdot/src/lib.rs:8677-8724): two
+// 8-byte table reads, a grid point's magnitude selectors and a sign index's bytes of 4, whose sum is a byte selector into the
+// six possible codes: 0 .. 2 pick 43 + {8, 25, 43}, 4 .. 6 pick 43 - {8, 25, 43} (the reference's card kernels decode the same
+// way, crates/gpu/src/iq.rs:473-512). A third less LDS traffic than ready-made code bytes of both signs and half the banks
+// an entry, for two more vector instructions a group.
+constexpr u32 kIq2Plus = 0x00564433u, kIq2Minus = 0x00001223u;
+__device__ __forceinline__ void bm_iq2_codes(const Iq2Tables &tb, u32 grid_idx, u32 sign_idx, u32 &lo, u32 &hi) {
+    const uint2 g = tb.grid[grid_idx], sg = tb.signs[sign_idx];
+    lo = __builtin_amdgcn_perm(kIq2Minus, kIq2Plus, g.x | sg.x);
+    hi = __builtin_amdgcn_perm(kIq2Minus, kIq2Plus, g.y | sg.y);
+}
 
 template <>
 struct Act<BM_IQ2XXS> {
@@ -648,10 +660,7 @@ __device__ __forceinline__ Iq2Dec bm_decode_iq2xxs(const Blk<BM_IQ2XXS> &b, int 
             const int sb = 2 * k + e;
             const u32 idx = e ? idx_b : idx_a, aux = e ? aux_b : aux_a;
             dec.sc[sb] = 2 * (int)(aux >> 28) + 1;
-            const uint4 g = tb.grid[(idx >> (8 * q)) & 0xffu];
-            const uint2 sg = tb.signs[(aux >> (7 * q)) & 127u];
-            dec.u_lo[sb] = bm_iq_pick(g.x, g.z, sg.x);
-            dec.u_hi[sb] = bm_iq_pick(g.y, g.w, sg.y);
+            bm_iq2_codes(tb, (idx >> (8 * q)) & 0xffu, (aux >> (7 * q)) & 127u, dec.u_lo[sb], dec.u_hi[sb]);
         }
     }
     return dec;

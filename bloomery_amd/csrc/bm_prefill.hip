@@ -941,11 +941,11 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, 
             if constexpr (EXACT) sc_t[b * kIqLine + wr] = (float)sc;
 #pragma unroll
             for (int q = 0; q < 4; q++) { // values 8 q .. 8 q + 7: lanes 2 q and 2 q + 1
-                const uint4 gp = tb.grid[(idx >> (8 * q)) & 0xffu];
-                const uint2 sg = tb.signs[(aux >> (7 * q)) & 127u];
+                u32 c_lo, c_hi;
+                bm_iq2_codes(tb, (idx >> (8 * q)) & 0xffu, (aux >> (7 * q)) & 127u, c_lo, c_hi);
                 u32 h0, l0, h1, l1;
-                iq2_planes(bm_iq_pick(gp.x, gp.z, sg.x), sc, h0, l0);
-                iq2_planes(bm_iq_pick(gp.y, gp.w, sg.y), sc, h1, l1);
+                iq2_planes(c_lo, sc, h0, l0);
+                iq2_planes(c_hi, sc, h1, l1);
                 const int at = wr * kIqStride + 32 * (2 * q) + 4 * b;
                 *reinterpret_cast<u32 *>(w_hi + at) = h0;
                 *reinterpret_cast<u32 *>(w_lo + at) = l0;

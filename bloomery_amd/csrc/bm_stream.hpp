@@ -26,8 +26,8 @@ constexpr u32 kSiteQuantColumn = 1; // crates/device/src/fault.rs:73-76
 constexpr u32 kSiteExpertId = 7;    // crates/device/src/fault.rs:89
 constexpr u32 kSiteF32Product = 21; // crates/device/src/fault.rs:151-155: a gate or up sum that is not finite under a clamp
 
-// LDS bytes of the IQ2_XXS tables: 256 grid entries of 16 + 128 sign entries of 8.
-constexpr int kTabBytes = 256 * 16 + 128 * 8;
+// LDS bytes of the IQ2_XXS tables: 256 grid entries of 8 + 128 sign entries of 8.
+constexpr int kTabBytes = 256 * 8 + 128 * 8;
 
 constexpr int kTabBytes3 = 256 * 8 + 128 * 8; // IQ3_XXS: 256 grid entries of 8 + 128 sign entries of 8
 
@@ -52,14 +52,20 @@ template <int WT>
 __device__ __forceinline__ Iq2Tables stage_tables(uint8_t *lds) {
     Iq2Tables tb{nullptr, nullptr, nullptr};
     if constexpr (WT == BM_IQ2XXS) {
-        uint4 *grid = reinterpret_cast<uint4 *>(lds);
-        uint2 *signs = reinterpret_cast<uint2 *>(lds + 256 * 16);
+        // a grid point as eight byte selectors over the three magnitudes (8, 25, 43 -> 0, 1, 2), a sign index as eight bytes
+        // of 4 where the value is negative: their sum picks a value's code byte 43 +- magnitude out of six (bm_iq2_codes)
+        uint2 *grid = reinterpret_cast<uint2 *>(lds);
+        uint2 *signs = reinterpret_cast<uint2 *>(lds + 256 * 8);
         for (int t = threadIdx.x; t < 256; t += blockDim.x) {
-            const uint64_t g = BM_IQ2XXS_GRID[t]; // bytes 8, 25 or 43: 43 + and 43 - stay inside a byte
+            const uint64_t g = BM_IQ2XXS_GRID[t];
             const u32 lo = (u32)g, hi = (u32)(g >> 32);
-            grid[t] = make_uint4(0x2b2b2b2bu + lo, 0x2b2b2b2bu + hi, 0x2b2b2b2bu - lo, 0x2b2b2b2bu - hi);
+            // 0x08 -> 0, 0x19 -> 1, 0x2b -> 2: bit 0 of the byte is 1 for 0x19 and 0x2b, bit 1 for 0x2b only
+            grid[t] = make_uint2(((lo & 0x01010101u) + ((lo >> 1) & 0x01010101u)), ((hi & 0x01010101u) + ((hi >> 1) & 0x01010101u)));
         }
-        for (int t = threadIdx.x; t < 128; t += blockDim.x) signs[t] = iq_sign_masks(t);
+        for (int t = threadIdx.x; t < 128; t += blockDim.x) {
+            const uint2 m = iq_sign_masks(t);
+            signs[t] = make_uint2(m.x & 0x04040404u, m.y & 0x04040404u);
+        }
         tb.grid = grid;
         tb.signs = signs;
     }

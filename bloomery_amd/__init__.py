@@ -91,7 +91,7 @@ SYMBOLS = {
     "bm_scratch_set_path": (_i, [_vp, _i, _i, _i]),
     "bm_scratch_path_for": (_i, [_vp, _i]),
     "bm_moe_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
-    "bm_norm_route": (_i, [_vp, _vp, _vp, _vp, C.c_float, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
+    "bm_norm_route": (_i, [_vp, _vp, _vp, _vp, C.c_float, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "bm_card_quantize": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp]),
     "bm_card_gemv": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp]),
     "bm_card_gemv_sel": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp]),
@@ -612,12 +612,15 @@ class Gpu:
         self._check(self.lib.bm_moe_forward(self.ctx, scratch.handle, wg.handle, wu.handle, wd.handle, _ptr(x), _ptr(sel), _ptr(wts),
                                             _ptr(resid), m, _rule(rule), _ptr(y)))
 
-    def enqueue_norm_route(self, router, x, gain, eps, n_tokens, n_experts, hidden, top_k, renorm, normed, logits, probs, ids, weights):
-        """enqueue_router_logits and enqueue_route_softmax as one launch (bm_norm_route): the same bits in every output."""
+    def enqueue_norm_route(self, router, x, gain, eps, n_tokens, n_experts, hidden, top_k, renorm, normed, logits, probs, ids, weights,
+                           act_x=None):
+        """enqueue_router_logits and enqueue_route_softmax as one launch (bm_norm_route): the same bits in every output. With act_x
+        the launch also leaves the normed rows as quantized columns (the bytes enqueue_quantize makes of `normed`)."""
         self._check(self.lib.bm_norm_route(self.ctx, _ptr(router), _ptr(x), _ptr(gain) if gain is not None else None, float(eps),
                                            n_tokens, n_experts, hidden, top_k, int(bool(renorm)),
                                            _ptr(normed) if normed is not None else None, _ptr(logits),
-                                           _ptr(probs) if probs is not None else None, _ptr(ids), _ptr(weights)))
+                                           _ptr(probs) if probs is not None else None, _ptr(ids), _ptr(weights),
+                                           act_x.handle if act_x is not None else None))
 
     def enqueue_router_logits(self, router, x, gain, eps, n_tokens, n_experts, hidden, normed, logits):
         """The FFN norm (gain None: none) and the router's f32 logits, the step before enqueue_route_softmax

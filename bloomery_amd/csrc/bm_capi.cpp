@@ -1129,7 +1129,7 @@ int bm_router_logits(bm_ctx *ctx, const float *router_dev, const float *x_dev, c
 
 int bm_norm_route(bm_ctx *ctx, const float *router_dev, const float *x_dev, const float *gain_dev, float eps, int n_tokens,
                   int n_experts, int hidden, int top_k, int renorm, float *normed_dev, float *logits_dev, float *probs_dev,
-                  uint32_t *ids_dev, float *weights_dev) {
+                  uint32_t *ids_dev, float *weights_dev, bm_act *act_x) {
     const char *what = "bm_norm_route";
     if (!ctx || !router_dev || !x_dev || !logits_dev || !ids_dev || !weights_dev) return fail(ctx, BM_EARG, "%s: NULL argument", what);
     if (n_tokens < 1 || n_tokens > bmk::kNormRouteMaxTokens)
@@ -1147,8 +1147,12 @@ int bm_norm_route(bm_ctx *ctx, const float *router_dev, const float *x_dev, cons
         return fail(ctx, BM_ESHAPE, "%s: router_dev %p, x_dev %p, gain_dev %p and normed_dev %p must be 16-byte aligned", what,
                     (const void *)router_dev, (const void *)x_dev, (const void *)gain_dev, (const void *)normed_dev);
     if (gain_dev && !(eps >= 0.0f)) return fail(ctx, BM_EARG, "%s: eps = %g is negative or not a number", what, (double)eps);
+    if (act_x && (act_x->k != hidden || act_x->m_cap < n_tokens))
+        return fail(ctx, BM_ESHAPE, "%s: act_x must hold %d columns of k = %d; it holds %d of k = %d", what, n_tokens, hidden, act_x->m_cap,
+                    act_x->k);
     return driver(ctx, what, bmk::norm_route(launch_of(ctx), router_dev, x_dev, gain_dev, eps, n_tokens, n_experts, hidden, normed_dev,
-                                             logits_dev, top_k, renorm != 0, probs_dev, ids_dev, weights_dev, ctx->route_counts));
+                                             logits_dev, top_k, renorm != 0, probs_dev, ids_dev, weights_dev, ctx->route_counts,
+                                             act_x ? act_x->dev : nullptr, act_x && act_form(act_x->wtype) != 0));
 }
 
 int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *act, int col, int32_t *out_dev) {

@@ -153,9 +153,10 @@ bool router_logits_fits(int hidden);
 // router_logits and route_softmax as one launch: the last of a token's workgroups to finish routes it. counts: a zeroed
 // word a token, left zeroed; launches that share them must not overlap.
 constexpr int kNormRouteMaxTokens = 4096;
+// act_x (optional; hidden a multiple of 256): the tokens' normed rows as quantized columns (q8k: Q8_K, else Q8_2_X4 with tables)
 hipError_t norm_route(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                       int hidden, float *normed_out, float *logits, int used, int renorm, float *probs, uint32_t *ids,
-                      float *weights, uint32_t *counts);
+                      float *weights, uint32_t *counts, uint8_t *act_x = nullptr, bool q8k = false);
 hipError_t router_logits(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                          int hidden, float *normed_out, float *logits);
 

@@ -478,62 +478,6 @@ __global__ __launch_bounds__(256) void k_gate_up_x(const float *x, const uint8_t
 
 // ------------------------------------------------------------- the fused step for the types that take Q8_K columns
 
-// One 256-value block of a Q8_K column by one wave, four consecutive values a lane: k_quantize_q8k's operations on the
-// same operands (crates/qdot/src/lib.rs:1787-1809), the block's maximum and the sums met through lane exchanges.
-// `o` is the block's 296 bytes (LDS or global memory).
-__device__ __forceinline__ void q8k_wave_block(const float4 x4, uint8_t *o, int lane, u32 *fault, u32 layer) {
-    const float v[4] = {x4.x, x4.y, x4.z, x4.w};
-    // the largest magnitude: a maximum of the sign-less bit patterns over the wave
-    u32 mine_ab = 0;
-#pragma unroll
-    for (int k = 0; k < 4; k++) {
-        const u32 a = bm_f32_bits(v[k]) & 0x7fffffffu;
-        mine_ab = a > mine_ab ? a : mine_ab;
-    }
-    const u32 half_ab = bm_max32(mine_ab); // over each half of the wave
-    const u32 lo_ab = (u32)__builtin_amdgcn_readlane((int)half_ab, 0), hi_ab = (u32)__builtin_amdgcn_readlane((int)half_ab, 32);
-    const u32 ab = lo_ab > hi_ab ? lo_ab : hi_ab;
-    // its first holder (value 4 * lane + k): the lowest lane among those that hold it at k, the lowest such value
-    int first = 1 << 20;
-    float max = 0.0f;
-#pragma unroll
-    for (int k = 0; k < 4; k++) {
-        const unsigned long long holders = __ballot((bm_f32_bits(v[k]) & 0x7fffffffu) == ab);
-        if (holders) { // uniform over the wave
-            const int at = __builtin_ctzll(holders);
-            const float val = bm_bits_f32((u32)__builtin_amdgcn_readlane((int)bm_f32_bits(v[k]), at));
-            if (4 * at + k < first) first = 4 * at + k, max = val;
-        }
-    }
-    float d;
-    int code[4] = {0, 0, 0, 0};
-    if (ab > 0x7f7fffffu) {
-        if (lane == 0) bm_raise(fault, layer, kSiteQuantColumn);
-        d = bm_bits_f32(0x7fc00000u);
-    } else if (ab == 0) {
-        d = 0.0f;
-    } else {
-        const float iscale = __fdiv_rn(-127.0f, max);
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            int qv = bm_nearest_int(__fmul_rn(iscale, v[k]));
-            qv = qv > 127 ? 127 : qv;
-            code[k] = (int)(signed char)(qv & 0xff); // `as i8`: the low byte
-        }
-        d = __fdiv_rn(1.0f, iscale);
-    }
-    *reinterpret_cast<u32 *>(o + 8 + 4 * lane) = (u32)(code[0] & 0xff) | ((u32)(code[1] & 0xff) << 8) |
-                                                 ((u32)(code[2] & 0xff) << 16) | ((u32)(code[3] & 0xff) << 24);
-    int sum = code[0] + code[1] + code[2] + code[3]; // sixteen codes a sum: four lanes
-    sum += (int)bm_dpp<kDppXor1>((u32)sum);
-    sum += (int)bm_dpp<kDppXor2>((u32)sum);
-    if ((lane & 3) == 0) *reinterpret_cast<unsigned short *>(o + 264 + 2 * (lane >> 2)) = (unsigned short)(short)sum;
-    if (lane == 0) {
-        *reinterpret_cast<float *>(o) = d;
-        *reinterpret_cast<u32 *>(o + 4) = 0u;
-    }
-}
-
 // `cols` columns of nb blocks each, f32 rows at x (column c at x + c * nb * 256), into LDS at `dst` by the workgroup's
 // waves, block by block.
 __device__ __forceinline__ void q8k_stage_cols(const float *x, uint8_t *dst, int cols, int nb, u32 *fault, u32 layer,

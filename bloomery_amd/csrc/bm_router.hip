@@ -148,9 +148,11 @@ hipError_t route_softmax(const Launch &L, const float *logits, int n_tok, int n_
 // Floats a line of the accumulator-major LDS rows.
 __host__ __device__ inline int router_line(int hidden) { return ((hidden / 8 + 3) & ~3) + 8; }
 
+// t: the token; e0: the first of the workgroup's R router rows, or -1 for a workgroup that only norms the token's row into LDS
+// (k_norm_route's quantizer workgroups): no router rows, no logits.
 template <int R>
 __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *router, const float *x, const float *gain, float eps,
-                                                   int n_exp, int hidden, float *normed_out, float *logits) {
+                                                   int n_exp, int hidden, float *normed_out, float *logits, int t, int e0) {
     // The token's row and the R router rows lie accumulator-major in LDS: value k at line k % 8, place k / 8, so that the
     // lane that owns accumulator l reads four consecutive steps' operands as 16 bytes. A line is hidden / 8 floats, rounded up
     // to whole 16 bytes, + 8 (the eight lines of a row 8 banks apart), a router row four floats past the one before (rows r
@@ -164,12 +166,10 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
     };
     __shared__ double s_part[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int blocks_per_token = (n_exp + R - 1) / R;
-    const int t = blockIdx.x / blocks_per_token, e0 = (blockIdx.x % blocks_per_token) * R;
     const float *xt = x + (size_t)t * hidden;
     // the rows' bytes on their way first: they do not depend on the norm
     const int n4 = hidden / 4;
-    for (int i = tid; i < R * n4; i += 256) {
+    for (int i = tid; i < (e0 >= 0 ? R * n4 : 0); i += 256) {
         const int r = i / n4, c = i % n4;
         const int e = e0 + r < n_exp ? e0 + r : n_exp - 1;
         put4(ws + (size_t)r * wrow_floats, c, reinterpret_cast<const float4 *>(router + (size_t)e * hidden)[c]);
@@ -245,7 +245,7 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
     // every thread that stores a logit below is of the first wave: k_norm_route's hand-over (a device-scope count updated by
     // thread 0 behind the workgroup's barrier) publishes that wave's stores and relies on it
     static_assert(8 * R <= 64, "the logits of a workgroup are stored by its first wave");
-    if (tid < 8 * R) {
+    if (e0 >= 0 && tid < 8 * R) {
         const int r = tid >> 3, l = tid & 7;
         const float4 *xl = reinterpret_cast<const float4 *>(xs + l * line);
         const float4 *wl = reinterpret_cast<const float4 *>(ws + (size_t)r * wrow_floats + l * line);
@@ -280,7 +280,9 @@ template <int R>
 __global__ __launch_bounds__(256) void k_router_logits(const float *router, const float *x, const float *gain, float eps,
                                                        int n_exp, int hidden, float *normed_out, float *logits) {
     extern __shared__ __align__(16) uint8_t lds[];
-    router_logits_body<R>(lds, router, x, gain, eps, n_exp, hidden, normed_out, logits);
+    const int blocks_per_token = (n_exp + R - 1) / R;
+    router_logits_body<R>(lds, router, x, gain, eps, n_exp, hidden, normed_out, logits, blockIdx.x / blocks_per_token,
+                          (blockIdx.x % blocks_per_token) * R);
 }
 
 // Norm, logits and routing in one launch (crates/gpu/src/route_softmax.rs:1667-1674 enqueue_norm_fused; the quantizer of
@@ -290,16 +292,42 @@ __global__ __launch_bounds__(256) void k_router_logits(const float *router, cons
 // it with its first wave, k_route_softmax's numbers. No workgroup waits for another: every one runs to its end whatever the
 // order they are dispatched in. The last one leaves the count at zero for the next launch, so a graph replay needs no
 // memset. Launches over the same counts must not overlap.
+// With act_x (the reference launch's quantizer, route_softmax.rs:1679): one more workgroup a token, behind the others in the
+// grid, norms the token's row the same way and leaves it as the token's quantized column (q8k: a Q8_K column, else a Q8_2_X4
+// one with its tables), the bytes bm_quantize makes of normed_out. It takes part in no count, so the routing waits for none of it.
 template <int R, int PER>
 __global__ __launch_bounds__(256) void k_norm_route(const float *router, const float *x, const float *gain, float eps, int n_exp,
                                                     int hidden, float *normed_out, float *logits, u32 used, u32 renorm,
-                                                    float *probs, u32 *ids, float *weights, u32 *counts, u32 *fault,
-                                                    u32 layer) {
+                                                    float *probs, u32 *ids, float *weights, u32 *counts, uint8_t *act_x,
+                                                    int q8k, int m, u32 *fault, u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
     __shared__ u32 s_last;
-    router_logits_body<R>(lds, router, x, gain, eps, n_exp, hidden, normed_out, logits);
     const u32 blocks_per_token = (u32)((n_exp + R - 1) / R);
+    if (blockIdx.x >= (u32)m * blocks_per_token) { // a quantizer workgroup
+        const int tq = (int)(blockIdx.x - (u32)m * blocks_per_token);
+        router_logits_body<R>(lds, router, x, gain, eps, n_exp, hidden, nullptr, nullptr, tq, -1);
+        const int line = router_line(hidden), nb = hidden / 256, tid = threadIdx.x;
+        const float *xs = reinterpret_cast<const float *>(lds); // value k at line k % 8, place k / 8
+        if (q8k) {
+            uint8_t *col = act_x + (size_t)tq * nb * BM_Q8K_STRIDE;
+            for (int b = tid >> 6; b < nb; b += 4) { // a wave a 256-value block, four consecutive values a lane
+                const int k = 256 * b + 4 * (tid & 63);
+                const float *at = xs + (k & 7) * line + (k >> 3);
+                q8k_wave_block(make_float4(at[0], at[line], at[2 * line], at[3 * line]), col + (size_t)b * BM_Q8K_STRIDE, tid & 63, fault, layer);
+            }
+        } else {
+            uint8_t *col = act_x + (size_t)tq * nb * BM_Q82_SB_EXT;
+            for (int k = 8 * tid; k < hidden; k += 2048) { // a quad of lanes a 32-value block, eight consecutive values a lane
+                float v8[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) v8[j] = xs[j * line + (k >> 3)];
+                q82_quad8(v8, col, nb, k >> 5, tid & 3, fault, layer);
+            }
+        }
+        return;
+    }
     const u32 t = blockIdx.x / blocks_per_token;
+    router_logits_body<R>(lds, router, x, gain, eps, n_exp, hidden, normed_out, logits, (int)t, (int)(blockIdx.x % blocks_per_token) * R);
     __syncthreads(); // the workgroup's stores are issued
     if (threadIdx.x == 0) {
         const u32 before = __hip_atomic_fetch_add(&counts[t], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
@@ -349,18 +377,19 @@ hipError_t router_logits(const Launch &L, const float *router, const float *x, c
 
 hipError_t norm_route(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                       int hidden, float *normed_out, float *logits, int used, int renorm, float *probs, uint32_t *ids,
-                      float *weights, uint32_t *counts) {
+                      float *weights, uint32_t *counts, uint8_t *act_x, bool q8k) {
     const int rows = router_rows(hidden);
     if (rows == 0) return hipErrorInvalidValue;
+    if (act_x && hidden % 256 != 0) return hipErrorInvalidValue;
     const size_t lds = router_lds_bytes(rows, hidden);
-    const unsigned grid = (unsigned)m * (unsigned)((n_exp + rows - 1) / rows);
+    const unsigned grid = (unsigned)m * (unsigned)((n_exp + rows - 1) / rows) + (act_x ? (unsigned)m : 0u);
 #define BM_NR(R, PER)                                                                                                  \
     {                                                                                                                  \
         auto kern = k_norm_route<R, PER>;                                                                              \
         hipError_t e = allow_lds(kern, lds);                                                                           \
         if (e != hipSuccess) return e;                                                                                 \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, router, x, gain, eps, n_exp, hidden, normed_out, \
-                           logits, (u32)used, (u32)renorm, probs, ids, weights, counts, L.fault, L.layer);             \
+                           logits, (u32)used, (u32)renorm, probs, ids, weights, counts, act_x, q8k ? 1 : 0, m, L.fault, L.layer); \
     }
 #define BM_NR_ROWS(PER)                                                                                                \
     {                                                                                                                  \

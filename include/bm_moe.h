@@ -400,14 +400,16 @@ int bm_route_softmax(bm_ctx *ctx, const float *logits_dev, int n_tokens, int n_e
 int bm_router_logits(bm_ctx *ctx, const float *router_dev, const float *x_dev, const float *gain_dev, float eps, int n_tokens,
                      int n_experts, int hidden, float *normed_dev, float *logits_dev);
 /* bm_router_logits and bm_route_softmax as one launch (RouterKernels::enqueue_norm_fused / enqueue_norm_fused_m,
- * crates/gpu/src/route_softmax.rs:1667-1679: norm, logits and routing of the tokens in one launch; that launch's
- * quantizer rides in bm_moe_decode / bm_gate_up_x over normed_dev here). Same arguments and the same bits in every output
- * as the two calls one after the other. The workgroup that finishes a token's last logits routes the token; none waits
+ * crates/gpu/src/route_softmax.rs:1667-1679: norm, logits, routing and the activation quantizer of the tokens in one
+ * launch). Same arguments and the same bits in every output as the two calls one after the other. act_x (optional; hidden a
+ * multiple of 256): the tokens' normed rows as quantized columns in the form the bm_act was made for, the bytes bm_quantize
+ * makes of normed_dev (the launch's act_ffn), written by one more workgroup a token that the routing does not wait for:
+ * bm_gate_up over act_x then takes the place of bm_gate_up_x / bm_moe_decode's first launch over normed_dev. The workgroup that finishes a token's last logits routes the token; none waits
  * for another. logits_dev is required (the token's logits meet there); 1 .. 4096 tokens a launch. Launches of this entry
  * that share a context must not overlap (they count finished workgroups in words the context holds). */
 int bm_norm_route(bm_ctx *ctx, const float *router_dev, const float *x_dev, const float *gain_dev, float eps, int n_tokens,
                   int n_experts, int hidden, int top_k, int renorm, float *normed_dev, float *logits_dev, float *probs_dev,
-                  uint32_t *ids_dev, float *weights_dev);
+                  uint32_t *ids_dev, float *weights_dev, bm_act *act_x);
 
 
 /* ------------------------------------------------------------------------------------------- the card rule */

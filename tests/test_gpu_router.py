@@ -200,8 +200,16 @@ def test_layer_from_the_residual_row(gpu):
         assert_ulp(got_w[t], want_w, f"weights of token {t}", odd_share=1.0)
     want_y, _ = L.oracle(want_n, got_ids, got_w, top_k)
     assert_f32(y.download(), (want_y.reshape(m, hidden) + x).astype(np.float32).reshape(-1), "y + residual")
+    # the same layer as three launches: the router launch leaves the quantized columns (with the tables the dots read), gate . up
+    # takes them, down + combine closes
+    act_x, y3 = gpu.act(bm.Q4_K, hidden, m), gpu.buffer(np.float32, m * hidden).fill_bytes(0xFF)
+    ids3, wts3 = gpu.buffer(np.uint32, m * top_k), gpu.buffer(np.float32, m * top_k)
+    gpu.enqueue_norm_route(rd, xd, gd, 1e-6, m, n_experts, hidden, top_k, True, None, logits, None, ids3, wts3, act_x=act_x)
+    gpu.enqueue_gate_up(L.dg, L.du, act_x, ids3, m * top_k, ff, top_k, None, act_h)
+    gpu.enqueue_down_combine(L.dd, act_h, ids3, wts3, xd, top_k, m, hidden, y3)
+    assert np.array_equal(y3.download().view(np.uint32), y.download().view(np.uint32)), "three launches against four"
     assert gpu.fault() == (bm.FAULT_NONE, 0)
-    for b in (rd, xd, gd, normed, logits, ids, wts, act_h, y):
+    for b in (rd, xd, gd, normed, logits, ids, wts, act_h, y, act_x, y3, ids3, wts3):
         b.free()
     L.free()
 
@@ -231,8 +239,14 @@ def test_norm_route_is_the_two_launches_in_one(gpu, n_experts, hidden, m, top_k,
     want = [b.download() for b in bufs["two"]]
     normed, logits, probs, ids, wts = bufs["one"]
 
+    # where the rows are whole super-blocks the launch also leaves the quantized columns, in either column form
+    acts = [gpu.act(wt, hidden, m) for wt in (bm.Q4_K, bm.IQ2_XXS)] if hidden % 256 == 0 else [None]
+    which = [0]
+
     def fused(tokens):
-        gpu.enqueue_norm_route(rd, xd, gd, eps, tokens, n_experts, hidden, top_k, True, normed, logits, probs, ids, wts)
+        gpu.enqueue_norm_route(rd, xd, gd, eps, tokens, n_experts, hidden, top_k, True, normed, logits, probs, ids, wts,
+                               act_x=acts[which[0] % len(acts)])
+        which[0] += 1
 
     def check(tokens, what):
         for b, w, per, name in zip(bufs["one"], want, (hidden, n_experts, n_experts, top_k, top_k),
@@ -245,6 +259,16 @@ def test_norm_route_is_the_two_launches_in_one(gpu, n_experts, hidden, m, top_k,
             b.fill_bytes(0xFF)
         fused(m)
         check(m, f"launch {rep}")
+    if acts[0] is not None:  # the columns are the CPU path's bytes of the normed rows, and what bm_quantize makes of them
+        normed_rows = want[0].reshape(m, hidden)
+        for act, wt in zip(acts, (bm.Q4_K, bm.IQ2_XXS)):
+            ref = gpu.act(wt, hidden, m)
+            gpu.enqueue_quantize(bufs["two"][0], m, ref)
+            for t in (0, m // 2, m - 1):
+                col = act.download(t)
+                assert np.array_equal(col, ora.quantize_col(wt, normed_rows[t])), f"act_x column {t}, type {wt}"
+                assert np.array_equal(col, ref.download(t))
+            ref.free()
     few = max(1, m // 2)
     for b in bufs["one"]:
         b.fill_bytes(0xFF)
@@ -261,7 +285,7 @@ def test_norm_route_is_the_two_launches_in_one(gpu, n_experts, hidden, m, top_k,
         check(m, f"replay {rep}")
     gpu.graph_destroy(g)
     assert gpu.fault() == (bm.FAULT_NONE, 0)
-    for b in (rd, xd, gd) + bufs["two"] + bufs["one"]:
+    for b in (rd, xd, gd) + bufs["two"] + bufs["one"] + tuple(acts):
         if b is not None:
             b.free()
 

@@ -730,6 +730,42 @@ def timeline(args, bm, gpu, enqueue_step, type_names):
     gpu.close()
 
 
+def handoff(bm, gpu, src, src_bytes):
+    """What handing data from one workgroup to others costs inside a launch (a flag and 64 words through memory with device-scope
+    stores and loads, the only scope another compute unit sees), to be read against the launch boundary of the decode step:
+    pollers on the writer's XCD and on others, the rest of the chip idle, streaming reads, or the pollers' own compute units
+    streaming too. Times from the writer's flag store to the poller holding the words, 20 launches a case."""
+    import ctypes as C
+    probe = load_probe()
+    probe.bm_bench_probe_handoff.restype = C.c_int
+    probe.bm_bench_probe_handoff.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_int, C.c_int]
+    stream = gpu.lib.bm_ctx_stream(gpu.ctx)
+    flag, out_d, sink = gpu.buffer(np.uint32, 128).fill_bytes(0), gpu.buffer(np.uint64, 2048), gpu.buffer(np.uint32, 256)
+    same, other = (8, 16, 248), (1, 4, 255)
+    res, gen = {"unit": "ns", "launches_a_case": 20, "writer": 0, "pollers_on_the_writers_xcd": list(same), "pollers_on_other_xcds": list(other)}, 0
+    for load, name in ((0, "idle"), (1, "other_compute_units_stream"), (2, "every_compute_unit_streams")):
+        lat = {w: [] for w in same + other}
+        ack = []
+        for _ in range(20):
+            gen += 1
+            out_d.fill_bytes(0)
+            rc = probe.bm_bench_probe_handoff(stream, src, src_bytes, flag.ptr, out_d.ptr, sink.ptr, gen, load, 400)
+            assert rc == 0, f"bm_bench_probe_handoff: {rc}"
+            gpu.sync()
+            o = out_d.download().reshape(256, 8).astype(np.int64)
+            if gen == 1:
+                res["workgroups_on_the_xcd_of_their_index_mod_8"] = int(sum(o[w, 0] == o[w % 8, 0] for w in range(256)))
+            ack.append((o[0, 3] - o[0, 2]) * 10)
+            for w in lat:
+                assert o[w, 4] == 1, f"workgroup {w} did not see the words (polls {o[w, 5]})"
+                lat[w].append((o[w, 3] - o[0, 2]) * 10)
+        res[name] = {"flag_store_acknowledged": float(np.mean(ack)),
+                     "same_xcd_mean": float(np.mean([lat[w] for w in same])), "same_xcd_max": float(np.max([lat[w] for w in same])),
+                     "other_xcd_mean": float(np.mean([lat[w] for w in other])), "other_xcd_max": float(np.max([lat[w] for w in other]))}
+    print(json.dumps(res, indent=1), flush=True)
+    gpu.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5, 6, 7, 8),
@@ -764,6 +800,8 @@ def main():
                     help="config 2 only: no timing by events; the step's two launches through the measurement build of the library "
                          "(libbm_moe_hip_timeline.so), whose kernels leave the device's 100 MHz counter at marks inside every "
                          "workgroup; prints when each phase of each launch is reached")
+    ap.add_argument("--handoff", action="store_true",
+                    help="config 2 only: no timing of the step; what a hand-over between workgroups inside one launch costs (--layers 1 is enough)")
     ap.add_argument("--mode", choices=("two", "chain"), default="two",
                     help="two: bm_moe_decode, two launches with the quantizers folded in; chain: quantize, gate_up, down_combine")
     args = ap.parse_args()
@@ -835,6 +873,8 @@ def main():
             gpu.enqueue_down_combine(dd, act_h, sel.ptr + 4 * t * TOP_K, wt.ptr + 4 * t * TOP_K, None, TOP_K, 1, HIDDEN,
                                      y.ptr + 4 * t * HIDDEN)
 
+    if args.handoff:
+        return handoff(bm, gpu, layers[0][0].dev_ptr, N_EXPERTS * FF * bm.row_bytes(gate_t, HIDDEN))
     if args.timeline:
         return timeline(args, bm, gpu, enqueue_step, (gate_n, down_n))
     if args.traffic_probe:
@@ -940,7 +980,7 @@ def main():
     normed_d, logits_d = gpu.buffer(np.float32, HIDDEN), gpu.buffer(np.float32, N_EXPERTS)
     ids_d, wts_d = gpu.buffer(np.uint32, TOP_K), gpu.buffer(np.float32, TOP_K)
     router_us = {}
-    for name in ("router_logits", "route_softmax", "norm_route_one_launch"):
+    for name in ("router_logits", "route_softmax", "norm_route_one_launch", "norm_route_with_column"):
         gpu.capture_begin()
         for i in range(unit):
             if name == "router_logits":
@@ -948,9 +988,12 @@ def main():
                                           normed_d, logits_d)
             elif name == "route_softmax":
                 gpu.enqueue_route_softmax(logits_d, 1, N_EXPERTS, TOP_K, True, None, ids_d, wts_d)
-            else:
+            elif name == "norm_route_one_launch":
                 gpu.enqueue_norm_route(router_d, xd.ptr + 4 * (i % n_tok) * HIDDEN, gain_d, 1e-6, 1, N_EXPERTS, HIDDEN, TOP_K,
                                        True, normed_d, logits_d, None, ids_d, wts_d)
+            else:  # the launch also leaves the token's quantized column; the normed f32 row is not stored
+                gpu.enqueue_norm_route(router_d, xd.ptr + 4 * (i % n_tok) * HIDDEN, gain_d, 1e-6, 1, N_EXPERTS, HIDDEN, TOP_K,
+                                       True, None, logits_d, None, ids_d, wts_d, act_x=act)
         g1 = gpu.capture_end()
         gpu.graph_launch(g1)
         gpu.sync()
@@ -961,6 +1004,34 @@ def main():
         gpu.event_record(e1)
         router_us[name] = gpu.event_elapsed_ms(e0, e1) * 1e3 / (r * unit)
         gpu.graph_destroy(g1)
+    # The layer from its residual row, router and experts together (three launches either way, the ids and weights the router's
+    # own): the router launch leaves the normed f32 row and the fused expert step quantizes it in its first launch, or the
+    # router launch leaves the quantized column and gate . up reads it. The residual added back is the input row.
+    def from_residual(with_column):
+        def enqueue(i):
+            t = i % n_tok
+            dg, du, dd = layers[i % len(layers)]
+            xrow, yrow = xd.ptr + 4 * t * HIDDEN, y.ptr + 4 * t * HIDDEN
+            if with_column:
+                gpu.enqueue_norm_route(router_d, xrow, gain_d, 1e-6, 1, N_EXPERTS, HIDDEN, TOP_K, True, None, logits_d, None, ids_d,
+                                       wts_d, act_x=act)
+                gpu.enqueue_gate_up(dg, du, act, ids_d, TOP_K, FF, TOP_K, None, act_h)
+                gpu.enqueue_down_combine(dd, act_h, ids_d, wts_d, xrow, TOP_K, 1, HIDDEN, yrow)
+            else:
+                gpu.enqueue_norm_route(router_d, xrow, gain_d, 1e-6, 1, N_EXPERTS, HIDDEN, TOP_K, True, normed_d, logits_d, None, ids_d,
+                                       wts_d)
+                gpu.enqueue_moe_decode(dg, du, dd, normed_d, ids_d, wts_d, xrow, TOP_K, 1, act_h, yrow, h=h)
+        return enqueue
+
+    residual_us = {"column_made_in_gate_up_x": timed_graph(gpu, from_residual(False), unit, 2048, 512)[1] * 1e3}
+    if fold_h:
+        residual_us["column_from_norm_route"] = timed_graph(gpu, from_residual(True), unit, 2048, 512)[1] * 1e3
+        rows = []
+        for way in (False, True):  # the two ways give the same bits
+            from_residual(way)(0)
+            rows.append(y.download()[:HIDDEN].copy())
+        assert np.array_equal(rows[0].view(np.uint32), rows[1].view(np.uint32)), "the layer from its residual row, the two ways"
+        residual_us["same_bits_both_ways"] = True
     gate_up_bytes = TOP_K * 2 * FF * bm.row_bytes(gate_t, HIDDEN)
     down_bytes = TOP_K * HIDDEN * bm.row_bytes(down_t, FF)
     # what the launches' times are to be read against, measured here: an empty launch, and launches that only fetch the
@@ -1065,6 +1136,7 @@ def main():
         "kernel_us": kernel_us,
         "kernel_gbps": kernel_gbps,
         "router_kernel_us": router_us,
+        "layer_from_residual_row_us": residual_us,
         "calibration": calibration,
         "parity": parity,
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS,

@@ -829,6 +829,23 @@ def test_bench_probe_runs_and_refuses(gpu):
     assert lib.bm_bench_probe_read(stream, src.ptr, 64, 0, sink.ptr) == -1
     src.free()
     sink.free()
+    # the hand-over probe: every poller ends holding the writer's words, whatever the other workgroups do meanwhile
+    lib.bm_bench_probe_handoff.restype = C.c_int
+    lib.bm_bench_probe_handoff.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_int, C.c_int]
+    big = gpu.buffer(np.uint32, 16 << 20).fill_bytes(1)
+    flag, out, sink = gpu.buffer(np.uint32, 128).fill_bytes(0), gpu.buffer(np.uint64, 2048), gpu.buffer(np.uint32, 256)
+    for gen, load in ((1, 0), (2, 1), (3, 2)):
+        out.fill_bytes(0)
+        assert lib.bm_bench_probe_handoff(stream, big.ptr, 64 << 20, flag.ptr, out.ptr, sink.ptr, gen, load, 100) == 0
+        gpu.sync()
+        o = out.download().reshape(256, 8)
+        assert all(o[w, 4] == 1 for w in (8, 16, 248, 1, 4, 255)), o[[8, 16, 248, 1, 4, 255], 2:6]
+        assert flag.download()[0] == gen
+    assert lib.bm_bench_probe_handoff(stream, big.ptr, 1 << 20, flag.ptr, out.ptr, sink.ptr, 4, 0, 100) == -1
+    assert lib.bm_bench_probe_handoff(stream, big.ptr, 64 << 20, flag.ptr, out.ptr, sink.ptr, 4, 3, 100) == -1
+    assert lib.bm_bench_probe_handoff(stream, big.ptr, 64 << 20, None, out.ptr, sink.ptr, 4, 0, 100) == -1
+    for b in (big, flag, out, sink):
+        b.free()
 
 
 @pytest.mark.parametrize("down_type,hidden,ff,n_experts,m,top_k", ((bm.Q6_K, 2048, 768, 10, 3, 8), (bm.Q4_K, 512, 512, 5, 4, 2),

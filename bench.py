@@ -714,7 +714,7 @@ def timeline(args, bm, gpu, enqueue_step, type_names):
     assert rc == 0, f"bm_timeline_read: {rc}"
     tr = tr.reshape(rows, 8).astype(np.int64)
     n_a, n_b = TOP_K * FF // 32, HIDDEN // (64 // TOP_K)
-    a, b = tr[:n_a, :5], tr[rows // 2:rows // 2 + n_b, :4]
+    a, b = tr[:n_a, :5], tr[rows // 2:rows // 2 + n_b, :7]
     t0 = a[:, 0].min()
 
     def stat(v):
@@ -724,7 +724,9 @@ def timeline(args, bm, gpu, enqueue_step, type_names):
            "k_gate_up_x": {"workgroups": n_a,
                            **{name: stat(a[:, i]) for i, name in enumerate(("start", "expert_id_known", "token_quantized", "rows_dotted", "h_block_stored"))}},
            "k_down_combine": {"workgroups": n_b,
-                              **{name: stat(b[:, i]) for i, name in enumerate(("start", "columns_in_lds", "rows_dotted", "sum_stored"))}}}
+                              **{name: stat(b[:, i]) for i, name in ((0, "start"), (4, "expert_id_known"), (5, "ring_asked_for"),
+                                                                        (6, "columns_arrived"), (1, "columns_in_lds"),
+                                                                        (2, "rows_dotted"), (3, "sum_stored"))}}}
     out["launch_boundary_us"] = round(out["k_down_combine"]["start"]["min"] - out["k_gate_up_x"]["h_block_stored"]["max"], 2)
     print(json.dumps(out, indent=1), flush=True)
     gpu.close()

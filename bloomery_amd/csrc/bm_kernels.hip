@@ -13,7 +13,9 @@ namespace bmk {
 // libbm_moe_hip_timeline.so, which bench.py --timeline loads; the library proper holds none of this). Thread 0 of
 // workgroup b of k_gate_up_x leaves the device's constant-rate counter (100 MHz) in row b at marks 0 .. 4 (start, expert
 // id known, token quantized, rows dotted, block of h stored); of k_down_combine in row kTimelineRows / 2 + b at marks
-// 0 .. 3 (start, columns in LDS, rows dotted, sum stored). The last launch of each kernel is what the table holds.
+// 0 .. 3 (start, columns in LDS, rows dotted, sum stored) and, taken into registers and stored behind the barrier so that no
+// store stands among the loads they time, 4 .. 6 (expert id known, the ring's first super-blocks asked for, columns arrived).
+// The last launch of each kernel is what the table holds.
 #ifdef BM_TIMELINE
 constexpr int kTimelineRows = 4096;
 __device__ unsigned long long g_timeline[kTimelineRows * 8];
@@ -22,8 +24,26 @@ __device__ unsigned long long g_timeline[kTimelineRows * 8];
         if (threadIdx.x == 0 && (base) + blockIdx.x < (unsigned)kTimelineRows)                                         \
             g_timeline[((base) + blockIdx.x) * 8 + (mark)] = wall_clock64();                                           \
     } while (0)
+// BM_TICK keeps the counter in a register once `dep` has arrived (no store among the loads it times); BM_TOCK stores it.
+#define BM_TICK(var, dep)                                                                                              \
+    unsigned long long var;                                                                                            \
+    do {                                                                                                               \
+        __asm__ volatile("" ::"v"(dep) : "memory");                                                                    \
+        var = wall_clock64();                                                                                          \
+    } while (0)
+#define BM_TOCK(base, mark, var)                                                                                       \
+    do {                                                                                                               \
+        if (threadIdx.x == 0 && (base) + blockIdx.x < (unsigned)kTimelineRows)                                         \
+            g_timeline[((base) + blockIdx.x) * 8 + (mark)] = var;                                                      \
+    } while (0)
 #else
 #define BM_MARK(base, mark)                                                                                            \
+    do {                                                                                                               \
+    } while (0)
+#define BM_TICK(var, dep)                                                                                              \
+    do {                                                                                                               \
+    } while (0)
+#define BM_TOCK(base, mark, var)                                                                                       \
     do {                                                                                                               \
     } while (0)
 #endif
@@ -352,11 +372,14 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
     const bool active = dl < D && r < rpe && live;
     // the residual value of the row this thread closes, asked for now: at the end it would be a memory round trip
     const float resid_v = resid && tid < D && rb * D + tid < rpe ? resid[(size_t)t * rpe + rb * D + tid] : 0.0f;
-    if (!live && id != 0xffffffffu && rb == 0 && dl == 0 && q == 0) bm_raise(fault, layer, kSiteExpertId);
     const int n = NB > 0 ? NB : nb;
     const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
     const int col_bytes = bm_act_col_bytes<WT>(n);
     const uint8_t *act_cols = act + (size_t)t * spt * col_bytes;
+    // the token's columns are asked for before anything waits for the expert id: they arrive with it
+    Stage<5> st;
+    st.load(act_cols, spt * col_bytes);
+    if (!live && id != 0xffffffffu && rb == 0 && dl == 0 && q == 0) bm_raise(fault, layer, kSiteExpertId);
     const uint8_t *wrow = w + ((size_t)(live ? id : 0) * rpe + (active ? r : 0)) * row_bytes;
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *cols = lds + tab_bytes<WT>();
@@ -364,9 +387,10 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
     float *s_w = part + D * spt;                                              // [spt]
     u32 *s_sel = reinterpret_cast<u32 *>(s_w + spt);                          // [spt]
     Blk<WT> b[U];
-    Stage<5> st;
-    st.load(act_cols, spt * col_bytes);
+    BM_TICK(t_id, id);
     preload<WT, U>(b, wrow, q);
+    BM_TICK(t_asked, tid);
+    BM_TICK(t_cols, st.v[4].x);
     st.store(cols, act_cols, spt * col_bytes);
     if (tid < spt) {
         s_w[tid] = my_w;
@@ -374,6 +398,9 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
     }
     __syncthreads();
     BM_MARK(2048, 1);
+    BM_TOCK(2048, 4, t_id);
+    BM_TOCK(2048, 5, t_asked);
+    BM_TOCK(2048, 6, t_cols);
     float v[1];
     row_dot<WT, U, NB, 1>(b, wrow, cols + (size_t)e * col_bytes, col_bytes, 1, n, q, tb, v, NoTap{});
     BM_MARK(2048, 2);

@@ -135,9 +135,9 @@ __device__ __forceinline__ void preload(Blk<WT> (&b)[U], const uint8_t *wrow, in
 template <int WT, int U, class Tap>
 __device__ __forceinline__ void stage_one(Blk<WT> (&b)[U], int slot, int fill, const uint8_t *wrow, int ahead,
                                           const ActView &av, int i, int act_next, int q, const Iq2Tables &tb,
-                                          Act<WT> &cur, float &a0, float &a1, const Tap &tap) {
+                                          Act<WT> &cur, float &a0, float &a1, const Tap &tap, bool fetch = true) {
     __asm__ volatile("" ::: "memory");
-    if (U > 1) b[fill] = bm_load_blk<WT>(wrow, ahead, q);
+    if (U > 1 && fetch) b[fill] = bm_load_blk<WT>(wrow, ahead, q);
     const Act<WT> next = bm_load_act<WT, Tap::kActive>(av, act_next, q);
     __asm__ volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
@@ -169,7 +169,7 @@ __device__ __forceinline__ void row_dot(Blk<WT> (&b)[U], const uint8_t *wrow, co
             for (int i = 0; i < NB; i++) {
                 const int ahead = i + U - 1 < NB ? i + U - 1 : NB - 1;
                 stage_one<WT, U>(b, i % U, (i + U - 1) % U, wrow, ahead, av[0], i, i + 1 < NB ? i + 1 : i, q, tb, cur,
-                                 a0[0], a1[0], tap);
+                                 a0[0], a1[0], tap, i + U - 1 < NB); // the count is known here: nothing is asked for past the end
             }
         } else {
             for (int i0 = 0; i0 < n; i0 += U) {
@@ -186,7 +186,7 @@ __device__ __forceinline__ void row_dot(Blk<WT> (&b)[U], const uint8_t *wrow, co
         // several columns: the same ring for the weights, the activation operands read where they are used
         auto stage = [&](int slot, int fill, int i) {
             const int ahead = i + U - 1 < n ? i + U - 1 : n - 1;
-            b[fill] = bm_load_blk<WT>(wrow, U > 1 ? ahead : i, q);
+            if (NB == 0 || U == 1 || i + U - 1 < NB) b[fill] = bm_load_blk<WT>(wrow, U > 1 ? ahead : i, q);
             if constexpr (WT == BM_IQ2XXS) { // the table lookups once, not once a column
                 const Iq2Dec dec = bm_decode_iq2xxs(b[slot], q, tb);
 #pragma unroll

@@ -453,22 +453,42 @@ __device__ __forceinline__ void bm_dot_q45k_dec(const Q45Dec &x, const Act<BM_Q4
 // ---- Q6_K: lane (c, h) owns accumulators l = 4h + c and 4h + c + 2. Per 128-value half j it reads ql bytes
 // [64j + 32c + 16h, +16) (low nibbles: quarter c, high nibbles: quarter c + 2, both half h) and qh bytes
 // [32j + 16h, +16) (bits 2a of quarter a).
+// Four loads a lane and super-block, nothing fetched twice by a quad: the two ql pieces; one of the two qh pieces (lane c
+// of a pair takes half c's, its neighbour the other, and they exchange on use); and for the scales and d, lane 0 of the quad
+// takes the 16 scale bytes, lane 1 the 16 bytes that end with d (the address unit works through a load 64 bytes at a time
+// whether the lanes ask for different bytes or the same: with every lane asking for qh twice, the scales and d, a quad's
+// 210 bytes cost six passes instead of four; measured on the headline layer's down stack, 16 tokens slot by slot: 66.2 -> 64.1 us).
 template <>
 struct Blk<BM_Q6K> {
-    uint4 ql0, qh0, ql1, qh1, sc;
-    u32 d;
+    uint4 ql0, ql1, qhx, scd;
 };
 
 __device__ __forceinline__ Blk<BM_Q6K> bm_load_q6k(const uint8_t *wrow, int i, int c, int h) {
     const uint8_t *wb = wrow + (size_t)i * BM_Q6K_BLOCK;
     Blk<BM_Q6K> b;
     b.ql0 = bm_ld16u(wb + 32 * c + 16 * h);
-    b.qh0 = bm_ld16u(wb + 128 + 16 * h);
     b.ql1 = bm_ld16u(wb + 64 + 32 * c + 16 * h);
-    b.qh1 = bm_ld16u(wb + 128 + 32 + 16 * h);
-    b.sc = bm_ld16u(wb + 192);
-    b.d = bm_ld2u(wb + 208);
+    b.qhx = bm_ld16u(wb + 128 + 32 * c + 16 * h);
+    b.scd = bm_ld16u(wb + 192 + ((c & ~h & 1) ? 2 : 0)); // lane (c, h) = (1, 0): bytes 194 .. 210, d the last two
     return b;
+}
+
+// What the lane computes with, exchanged inside the quad once the loads are back: qh of both halves, the scales, d.
+struct Q6Parts {
+    uint4 qh0, qh1, sc;
+    u32 d;
+};
+template <int CTRL>
+__device__ __forceinline__ uint4 bm_dpp4(uint4 v) {
+    return make_uint4(bm_dpp<CTRL>(v.x), bm_dpp<CTRL>(v.y), bm_dpp<CTRL>(v.z), bm_dpp<CTRL>(v.w));
+}
+__device__ __forceinline__ Q6Parts bm_q6k_parts(const Blk<BM_Q6K> &b) {
+    Q6Parts p;
+    p.qh0 = bm_dpp4<0xA0>(b.qhx); // quad_perm [0,0,2,2]: the pair's lane c = 0 holds half 0's piece
+    p.qh1 = bm_dpp4<0xF5>(b.qhx); // quad_perm [1,1,3,3]
+    p.sc = bm_dpp4<0x00>(b.scd);  // quad lane 0
+    p.d = bm_dpp<0x55>(b.scd.w) >> 16; // quad lane 1: bytes 208, 209
+    return p;
 }
 
 // The two 16-value dots of one half: quarter c (low nibbles, high bits 2c) against aa and quarter c + 2 (high
@@ -513,17 +533,18 @@ __device__ __forceinline__ Act<BM_Q6K> bm_act_q6k(const ActView &av, int i, int 
 template <class Tap>
 __device__ __forceinline__ void bm_dot_q6k(const Blk<BM_Q6K> &b, const Act<BM_Q6K> &a, int i, int c, int h,
                                            float &acc0, float &acc1, const Tap &tap) {
-    const float d = bm_half_to_f32(b.d);
+    const Q6Parts p = bm_q6k_parts(b);
+    const float d = bm_half_to_f32(p.d);
     const int bi = 8 * (2 * c + h); // this lane's scale byte inside each word of four
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         int s0, s1;
-        bm_q6_dot16x2(j ? b.ql1 : b.ql0, j ? b.qh1 : b.qh0, 2 * c, a.aa[j], a.ab[j], s0, s1);
+        bm_q6_dot16x2(j ? b.ql1 : b.ql0, j ? p.qh1 : p.qh0, 2 * c, a.aa[j], a.ab[j], s0, s1);
         s0 -= 32 * a.sa[j]; // sum (q6 - 32) * a
         s1 -= 32 * a.sb[j];
         // scale bytes 8j + 2c + h and 8j + 4 + 2c + h (crates/qdot/src/lib.rs:4455 K_SHUFFLE_Q6K, :4794-4809)
-        const int sc0 = __builtin_amdgcn_sbfe((int)(j ? b.sc.z : b.sc.x), bi, 8);
-        const int sc1 = __builtin_amdgcn_sbfe((int)(j ? b.sc.w : b.sc.y), bi, 8);
+        const int sc0 = __builtin_amdgcn_sbfe((int)(j ? p.sc.z : p.sc.x), bi, 8);
+        const int sc1 = __builtin_amdgcn_sbfe((int)(j ? p.sc.w : p.sc.y), bi, 8);
         acc0 = fmaf((d * (float)sc0) * a.d8a[j], (float)s0, acc0);
         acc1 = fmaf((d * (float)sc1) * a.d8b[j], (float)s1, acc1);
         tap.q6k(i, 8 * j + 2 * c + h, s0);
@@ -539,21 +560,22 @@ struct Q6Dec {
 };
 
 __device__ __forceinline__ Q6Dec bm_decode_q6k(const Blk<BM_Q6K> &b, int c, int h) {
-    const float d = bm_half_to_f32(b.d);
+    const Q6Parts p = bm_q6k_parts(b);
+    const float d = bm_half_to_f32(p.d);
     const int bi = 8 * (2 * c + h), hs = 2 * c;
     const u32 ml = 0x0f0f0f0fu, mh = 0x30303030u;
     Q6Dec x;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
-        const uint4 ql = j ? b.ql1 : b.ql0, qh = j ? b.qh1 : b.qh0;
+        const uint4 ql = j ? b.ql1 : b.ql0, qh = j ? p.qh1 : p.qh0;
         const u32 l[4] = {ql.x, ql.y, ql.z, ql.w}, hh[4] = {qh.x >> hs, qh.y >> hs, qh.z >> hs, qh.w >> hs};
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             x.wa[j][t] = (l[t] & ml) | ((hh[t] << 4) & mh);
             x.wb[j][t] = ((l[t] >> 4) & ml) | (hh[t] & mh);
         }
-        const int sc0 = __builtin_amdgcn_sbfe((int)(j ? b.sc.z : b.sc.x), bi, 8); // the builtin's type is unsigned
-        const int sc1 = __builtin_amdgcn_sbfe((int)(j ? b.sc.w : b.sc.y), bi, 8);
+        const int sc0 = __builtin_amdgcn_sbfe((int)(j ? p.sc.z : p.sc.x), bi, 8); // the builtin's type is unsigned
+        const int sc1 = __builtin_amdgcn_sbfe((int)(j ? p.sc.w : p.sc.y), bi, 8);
         x.fa[j] = d * (float)sc0;
         x.fb[j] = d * (float)sc1;
     }

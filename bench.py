@@ -728,6 +728,35 @@ def timeline(args, bm, gpu, enqueue_step, type_names):
                                                                         (6, "columns_arrived"), (1, "columns_in_lds"),
                                                                         (2, "rows_dotted"), (3, "sum_stored"))}}}
     out["launch_boundary_us"] = round(out["k_down_combine"]["start"]["min"] - out["k_gate_up_x"]["h_block_stored"]["max"], 2)
+    # the router launch of one token (norm, logits, routing: bm_norm_route), the same way: 65 launches in a graph, the last one's marks
+    rng = np.random.default_rng(0x707E0001)
+    router_d = gpu.upload(rng.standard_normal((N_EXPERTS, HIDDEN), dtype=np.float32) * np.float32(0.05), np.float32)
+    xr = gpu.upload(rng.standard_normal((64, HIDDEN), dtype=np.float32), np.float32)
+    gain_d = gpu.upload(np.ones(HIDDEN, np.float32), np.float32)
+    normed_d, logits_d = gpu.buffer(np.float32, HIDDEN), gpu.buffer(np.float32, N_EXPERTS)
+    ids_d, wts_d = gpu.buffer(np.uint32, TOP_K), gpu.buffer(np.float32, TOP_K)
+    gpu.capture_begin()
+    for i in range(65):
+        gpu.enqueue_norm_route(router_d, xr.ptr + 4 * (i % 64) * HIDDEN, gain_d, 1e-6, 1, N_EXPERTS, HIDDEN, TOP_K, True, normed_d,
+                               logits_d, None, ids_d, wts_d)
+    graph = gpu.capture_end()
+    for _ in range(3):
+        gpu.graph_launch(graph)
+    gpu.sync()
+    lib.bm_router_timeline_read.restype = C.c_int
+    lib.bm_router_timeline_read.argtypes = [C.c_void_p]
+    rt = np.zeros(1024 * 8, np.uint64)
+    rc = lib.bm_router_timeline_read(rt.ctypes.data)
+    assert rc == 0, f"bm_router_timeline_read: {rc}"
+    rt = rt.reshape(1024, 8).astype(np.int64)
+    n_r = int(np.count_nonzero(rt[:, 0]))
+    rt = rt[:n_r]
+    r0 = rt[:, 0].min()
+    out["k_norm_route"] = {"unit": "us after the launch's first workgroup started", "workgroups": n_r,
+                           **{name: {"min": round(float((rt[:, i].min() - r0) / 100.0), 2), "median": round(float(np.median(rt[:, i] - r0) / 100.0), 2),
+                                     "max": round(float((rt[:, i].max() - r0) / 100.0), 2)}
+                              for i, name in enumerate(("start", "token_row_arrived", "normed", "rows_and_token_in_lds", "dots_done"))},
+                           "routed_by_the_last_workgroup": round(float((rt[:, 5].max() - r0) / 100.0), 2)}
     print(json.dumps(out, indent=1), flush=True)
     gpu.close()
 

@@ -17,6 +17,32 @@
 
 namespace bmk {
 
+// Timeline of the router launch, in measurement builds only (-DBM_TIMELINE, the library bench.py --timeline loads): thread 0 of
+// workgroup b keeps the device's constant-rate counter (100 MHz) in registers at six points of router_logits_body and stores
+// them at its end in row b: start, the token's row arrived, normed, rows and token in LDS (behind the barrier), dots done,
+// the routing done (the workgroup that routes).
+#ifdef BM_TIMELINE
+constexpr int kRouterTimelineRows = 1024;
+__device__ unsigned long long g_router_timeline[kRouterTimelineRows * 8];
+#define BM_RTICK(var, dep)                                                                                             \
+    do {                                                                                                               \
+        __asm__ volatile("" ::"v"(dep) : "memory");                                                                    \
+        var = wall_clock64();                                                                                          \
+    } while (0)
+#define BM_RTOCK(mark, var)                                                                                            \
+    do {                                                                                                               \
+        if (threadIdx.x == 0 && blockIdx.x < (unsigned)kRouterTimelineRows) g_router_timeline[blockIdx.x * 8 + (mark)] = var; \
+    } while (0)
+#else
+#define BM_RTICK(var, dep)                                                                                             \
+    do {                                                                                                               \
+    } while (0)
+#define BM_RTOCK(mark, var)                                                                                            \
+    do {                                                                                                               \
+    } while (0)
+#endif
+
+
 constexpr u32 kSiteRouter = 5; // crates/device/src/fault.rs:84-86
 
 __device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
@@ -26,8 +52,9 @@ __device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
     return __hiloint2double(hi, lo);
 }
 
-// Token t's routing by one wave; lane L owns experts L + 64 j, j < PER.
-template <int PER>
+// Token t's routing by one wave; lane L owns experts L + 64 j, j < PER. COH: the logits were stored by other workgroups of
+// this launch with device-scope stores and are read with device-scope loads (no cache of this compute unit's own is asked).
+template <int PER, bool COH = false>
 __device__ __forceinline__ void route_softmax_wave(const float *logits, u32 t, u32 n_exp, u32 used, u32 renorm, float *probs,
                                                    u32 *ids, float *weights, u32 *fault, u32 layer) {
     const u32 lane = threadIdx.x & 63;
@@ -37,7 +64,8 @@ __device__ __forceinline__ void route_softmax_wave(const float *logits, u32 t, u
 #pragma unroll
     for (int j = 0; j < PER; j++) {
         const u32 e = lane + 64 * j;
-        v[j] = e < n_exp ? row[e] : -INFINITY;
+        if constexpr (COH) v[j] = e < n_exp ? __hip_atomic_load(row + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
+        else v[j] = e < n_exp ? row[e] : -INFINITY;
         odd |= e < n_exp && !(fabsf(v[j]) <= 3.402823466e38f);
     }
     if (__ballot(odd) != 0) {
@@ -150,7 +178,7 @@ __host__ __device__ inline int router_line(int hidden) { return ((hidden / 8 + 3
 
 // t: the token; e0: the first of the workgroup's R router rows, or -1 for a workgroup that only norms the token's row into LDS
 // (k_norm_route's quantizer workgroups): no router rows, no logits.
-template <int R>
+template <int R, bool COH = false>
 __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *router, const float *x, const float *gain, float eps,
                                                    int n_exp, int hidden, float *normed_out, float *logits, int t, int e0) {
     // The token's row and the R router rows lie accumulator-major in LDS: value k at line k % 8, place k / 8, so that the
@@ -166,14 +194,34 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
     };
     __shared__ double s_part[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    [[maybe_unused]] unsigned long long tl_start = 0, tl_row = 0, tl_norm = 0, tl_lds = 0, tl_dots = 0;
+    BM_RTICK(tl_start, tid);
     const float *xt = x + (size_t)t * hidden;
-    // the rows' bytes on their way first: they do not depend on the norm
+    // the rows' bytes on their way first: they do not depend on the norm. Eight 16-byte loads a thread are asked for together
+    // and go to LDS once the token's row has been asked for too and normed
     const int n4 = hidden / 4;
-    for (int i = tid; i < (e0 >= 0 ? R * n4 : 0); i += 256) {
-        const int r = i / n4, c = i % n4;
-        const int e = e0 + r < n_exp ? e0 + r : n_exp - 1;
-        put4(ws + (size_t)r * wrow_floats, c, reinterpret_cast<const float4 *>(router + (size_t)e * hidden)[c]);
-    }
+    const int total = e0 >= 0 ? R * n4 : 0;
+    constexpr int kBatch = 8;
+    float4 rv[kBatch];
+    auto ask = [&](int i0) {
+#pragma unroll
+        for (int u = 0; u < kBatch; u++) {
+            const int i = i0 + tid + 256 * u;
+            if (i < total) {
+                const int r = i / n4, c = i % n4;
+                const int e = e0 + r < n_exp ? e0 + r : n_exp - 1;
+                rv[u] = reinterpret_cast<const float4 *>(router + (size_t)e * hidden)[c];
+            }
+        }
+    };
+    auto park = [&](int i0) {
+#pragma unroll
+        for (int u = 0; u < kBatch; u++) {
+            const int i = i0 + tid + 256 * u;
+            if (i < total) put4(ws + (size_t)(i / n4) * wrow_floats, i % n4, rv[u]);
+        }
+    };
+    ask(0);
     double sum = 0.0;
     constexpr int kInRegs = 8; // float4s of the row a thread can hold: rows of up to 8192 values stay in registers
     if (gain && n4 <= 256 * kInRegs) {
@@ -195,6 +243,7 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
                 sum += (double)__fmul_rn(xv[j].z, xv[j].z);
                 sum += (double)__fmul_rn(xv[j].w, xv[j].w);
             }
+        BM_RTICK(tl_row, sum);
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) sum += shfl_xor_f64(sum, off);
         if (lane == 0) s_part[wave] = sum;
@@ -202,6 +251,7 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
         const double total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
         const float mean = (float)(total / (double)hidden);
         const float scale = __fdiv_rn(1.0f, bm_sqrt_rn(__fadd_rn(mean, eps)));
+        BM_RTICK(tl_norm, scale);
 #pragma unroll
         for (int j = 0; j < kInRegs; j++) {
             const int i = tid + 256 * j;
@@ -239,7 +289,13 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
             }
         }
     }
+    park(0);
+    for (int i0 = 256 * kBatch; i0 < total; i0 += 256 * kBatch) {
+        ask(i0);
+        park(i0);
+    }
     __syncthreads();
+    BM_RTICK(tl_lds, tid);
     if (!gain && normed_out && e0 == 0) // the rows as they are (read after the barrier: other threads staged them)
         for (int i = tid; i < hidden; i += 256) normed_out[(size_t)t * hidden + i] = xs[(i & 7) * line + (i >> 3)];
     // every thread that stores a logit below is of the first wave: k_norm_route's hand-over (a device-scope count updated by
@@ -251,20 +307,41 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
         const float4 *wl = reinterpret_cast<const float4 *>(ws + (size_t)r * wrow_floats + l * line);
         // the chain is serial by the order's definition (a product, then fused multiply-adds in increasing k); the reads
         // are not: sixteen steps' operands, four 16-byte reads a side, a batch
-        // (reading the next batch under the present batch's chain measured slower: 8.1 us against 7.1 at 128 x 2048)
         const float *xf = xs + l * line, *wf = ws + (size_t)r * wrow_floats + l * line;
         const int steps = hidden / 8;
         float acc = __fmul_rn(xf[0], wf[0]);
         int i = 1;
         for (; i < 4 && i < steps; i++) acc = fmaf(xf[i], wf[i], acc);
-        for (; i + 16 <= steps; i += 16) {
-            float4 a[4], b[4];
+        auto rd = [&](float4(&a)[4], float4(&b)[4], int at) {
 #pragma unroll
-            for (int u = 0; u < 4; u++) a[u] = xl[i / 4 + u], b[u] = wl[i / 4 + u];
+            for (int u = 0; u < 4; u++) a[u] = xl[at / 4 + u], b[u] = wl[at / 4 + u];
+        };
+        auto chain = [&](const float4(&a)[4], const float4(&b)[4]) {
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 acc = fmaf(a[u].x, b[u].x, acc), acc = fmaf(a[u].y, b[u].y, acc);
                 acc = fmaf(a[u].z, b[u].z, acc), acc = fmaf(a[u].w, b[u].w, acc);
+            }
+        };
+        if (i + 16 <= steps) {
+            // two batches a turn in two sets of registers: a batch's operands are read while the batch before runs its chain
+            float4 a0[4], b0[4], a1[4], b1[4];
+            rd(a0, b0, i);
+            for (; i + 48 <= steps; i += 32) {
+                rd(a1, b1, i + 16);
+                __builtin_amdgcn_sched_barrier(0);
+                chain(a0, b0);
+                __builtin_amdgcn_sched_barrier(0);
+                rd(a0, b0, i + 32);
+                __builtin_amdgcn_sched_barrier(0);
+                chain(a1, b1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            chain(a0, b0);
+            i += 16;
+            for (; i + 16 <= steps; i += 16) {
+                rd(a0, b0, i);
+                chain(a0, b0);
             }
         }
         for (; i < steps; i++) acc = fmaf(xf[i], wf[i], acc);
@@ -272,8 +349,17 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
         const float s = __fadd_rn(acc, __shfl_down(acc, 4, 8));
         const float pair = __fadd_rn(s, __shfl_down(s, 2, 8)); // lane 0: s0 + s2, lane 1: s1 + s3
         const float out = __fadd_rn(pair, __shfl_down(pair, 1, 8));
-        if (l == 0 && e0 + r < n_exp) logits[(size_t)t * n_exp + e0 + r] = out;
+        BM_RTICK(tl_dots, out);
+        if (l == 0 && e0 + r < n_exp) {
+            if constexpr (COH) __hip_atomic_store(logits + (size_t)t * n_exp + e0 + r, out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            else logits[(size_t)t * n_exp + e0 + r] = out;
+        }
     }
+    BM_RTOCK(0, tl_start);
+    BM_RTOCK(1, tl_row);
+    BM_RTOCK(2, tl_norm);
+    BM_RTOCK(3, tl_lds);
+    BM_RTOCK(4, tl_dots);
 }
 
 template <int R>
@@ -286,10 +372,10 @@ __global__ __launch_bounds__(256) void k_router_logits(const float *router, cons
 }
 
 // Norm, logits and routing in one launch (crates/gpu/src/route_softmax.rs:1667-1674 enqueue_norm_fused; the quantizer of
-// that launch is folded into the expert launches here). The workgroups are k_router_logits's; each, once its logits are
-// stored, adds one to the token's count with release at device scope, and the workgroup that brings the count to the number
-// of the token's workgroups - the last to finish, whichever it is - reads the token's logits back with acquire and routes
-// it with its first wave, k_route_softmax's numbers. No workgroup waits for another: every one runs to its end whatever the
+// that launch is an option here, see below). The workgroups are k_router_logits's; each stores its logits with device-scope
+// stores, waits for their acknowledgement and adds one to the token's count, and the workgroup that brings the count to the
+// number of the token's workgroups - the last to finish, whichever it is - reads the token's logits back with device-scope
+// loads and routes it with its first wave, k_route_softmax's numbers. No workgroup waits for another: every one runs to its end whatever the
 // order they are dispatched in. The last one leaves the count at zero for the next launch, so a graph replay needs no
 // memset. Launches over the same counts must not overlap.
 // With act_x (the reference launch's quantizer, route_softmax.rs:1679): one more workgroup a token, behind the others in the
@@ -327,17 +413,23 @@ __global__ __launch_bounds__(256) void k_norm_route(const float *router, const f
         return;
     }
     const u32 t = blockIdx.x / blocks_per_token;
-    router_logits_body<R>(lds, router, x, gain, eps, n_exp, hidden, normed_out, logits, (int)t, (int)(blockIdx.x % blocks_per_token) * R);
-    __syncthreads(); // the workgroup's stores are issued
+    router_logits_body<R, true>(lds, router, x, gain, eps, n_exp, hidden, normed_out, logits, (int)t, (int)(blockIdx.x % blocks_per_token) * R);
     if (threadIdx.x == 0) {
-        const u32 before = __hip_atomic_fetch_add(&counts[t], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        // the workgroup's logits were stored by this wave with device-scope stores: once they are acknowledged they are where
+        // a device-scope load of any compute unit finds them, and only then is the count raised (no cache is written back or
+        // dropped as a whole, which an acquire/release pair at this scope does and which cost more than the routing itself)
+        __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const u32 before = __hip_atomic_fetch_add(&counts[t], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = before == blocks_per_token - 1;
         if (s_last) __hip_atomic_store(&counts[t], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (!s_last || threadIdx.x >= 64) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    route_softmax_wave<PER>(logits, t, (u32)n_exp, used, renorm, probs, ids, weights, fault, layer);
+    __asm__ volatile("" ::: "memory"); // the loads below stay behind the count
+    route_softmax_wave<PER, true>(logits, t, (u32)n_exp, used, renorm, probs, ids, weights, fault, layer);
+    [[maybe_unused]] unsigned long long tl_routed = 0;
+    BM_RTICK(tl_routed, threadIdx.x);
+    BM_RTOCK(5, tl_routed);
 }
 
 // LDS of a workgroup of R rows: the token's row and the router rows, each as eight lines.
@@ -345,18 +437,25 @@ static size_t router_lds_bytes(int rows, int hidden) {
     return ((size_t)(rows + 1) * 8 * router_line(hidden) + 4 * (size_t)rows) * sizeof(float);
 }
 
-// Rows a workgroup takes: four where they fit the LDS beside the token's row, else two, else one.
-static int router_rows(int hidden) {
+// Rows a workgroup takes: four where they fit the LDS beside the token's row, else two, else one - and no more than leaves
+// a workgroup for every compute unit: a workgroup's time goes to bringing its rows in and laying them out in LDS (the dots of
+// its rows run side by side on one wave), so with few tokens fewer rows a workgroup is the shorter launch.
+static int router_rows(int hidden, int m = 1 << 20, int n_exp = 1 << 20) {
+    int fit = 0;
     for (int r = 4; r >= 1; r >>= 1)
-        if (router_lds_bytes(r, hidden) <= (size_t)kMaxLds - 1024) return r;
-    return 0;
+        if (router_lds_bytes(r, hidden) <= (size_t)kMaxLds - 1024) {
+            fit = r;
+            break;
+        }
+    while (fit > 1 && (long)m * ((n_exp + fit - 1) / fit) < 256) fit >>= 1;
+    return fit;
 }
 
 bool router_logits_fits(int hidden) { return router_rows(hidden) > 0; }
 
 hipError_t router_logits(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                          int hidden, float *normed_out, float *logits) {
-    const int rows = router_rows(hidden);
+    const int rows = router_rows(hidden, m, n_exp);
     if (rows == 0) return hipErrorInvalidValue;
     const size_t lds = router_lds_bytes(rows, hidden);
     const unsigned grid = (unsigned)m * (unsigned)((n_exp + rows - 1) / rows);
@@ -378,7 +477,7 @@ hipError_t router_logits(const Launch &L, const float *router, const float *x, c
 hipError_t norm_route(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                       int hidden, float *normed_out, float *logits, int used, int renorm, float *probs, uint32_t *ids,
                       float *weights, uint32_t *counts, uint8_t *act_x, bool q8k) {
-    const int rows = router_rows(hidden);
+    const int rows = router_rows(hidden, m, n_exp);
     if (rows == 0) return hipErrorInvalidValue;
     if (act_x && hidden % 256 != 0) return hipErrorInvalidValue;
     const size_t lds = router_lds_bytes(rows, hidden);
@@ -406,3 +505,10 @@ hipError_t norm_route(const Launch &L, const float *router, const float *x, cons
 }
 
 } // namespace bmk
+
+#ifdef BM_TIMELINE
+// The router's table, copied to the host: dst holds 1024 * 8 words. Measurement builds only; not part of the C ABI.
+extern "C" int bm_router_timeline_read(unsigned long long *dst) {
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(bmk::g_router_timeline), sizeof(unsigned long long) * bmk::kRouterTimelineRows * 8);
+}
+#endif

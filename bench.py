@@ -721,6 +721,7 @@ def timeline(args, bm, gpu, enqueue_step, type_names):
         v = (v - t0) / 100.0
         return {"min": round(float(v.min()), 2), "median": round(float(np.median(v)), 2), "max": round(float(v.max()), 2)}
     out = {"unit": "us after the first workgroup of k_gate_up_x started", "gate": type_names[0], "down": type_names[1],
+           "down_form": args.down_form,
            "k_gate_up_x": {"workgroups": n_a,
                            **{name: stat(a[:, i]) for i, name in enumerate(("start", "expert_id_known", "token_quantized", "rows_dotted", "h_block_stored"))}},
            "k_down_combine": {"workgroups": n_b,
@@ -797,6 +798,44 @@ def handoff(bm, gpu, src, src_bytes):
     gpu.close()
 
 
+def read_patterns(bm, gpu, layers, sel, n_tok):
+    """What the two decode launches' requests cost with nothing computed, and what other ways of asking for the same bytes would
+    (bloomery_amd/csrc/bench_probe.hip): graph replay over the cycling routings and layer copies as the timed step, us a launch."""
+    import ctypes as C
+    probe = load_probe()
+    probe.bm_bench_probe_gate_up_rows.restype = C.c_int
+    probe.bm_bench_probe_gate_up_rows.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    probe.bm_bench_probe_down_rows.restype = C.c_int
+    probe.bm_bench_probe_down_rows.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
+    stream = gpu.lib.bm_ctx_stream(gpu.ctx)
+    sink = gpu.buffer(np.uint32, 4096)
+
+    def timed(enqueue):
+        return round(min(timed_graph(gpu, enqueue, 256, 1024, 256)[1] * 1e3 for _ in range(2)), 3)
+
+    res = {"unit": "us a launch, graph replay, cold rows", "gate_up_bytes": TOP_K * 2 * FF * bm.row_bytes(bm.Q4_K, HIDDEN),
+           "down_bytes": TOP_K * HIDDEN * bm.row_bytes(bm.Q6_K, FF), "gate_up": {}, "down": {}}
+    for name, pattern, threads, ahead in (("quad_a_row_4_ahead_192x256_as_k_gate_up_x", 0, 256, 4), ("quad_a_row_8_ahead_192x256", 0, 256, 8),
+                                          ("quad_a_row_4_ahead_256x192", 0, 192, 4), ("quad_a_row_8_ahead_256x192", 0, 192, 8),
+                                          ("octet_a_row_pair_192x256", 1, 256, 8), ("octet_a_row_pair_256x192", 1, 192, 8),
+                                          ("workgroup_contiguous_192x256", 2, 256, 8), ("workgroup_contiguous_256x192", 2, 192, 8)):
+        def enqueue(i):
+            dg, du, _ = layers[i % len(layers)]
+            rc = probe.bm_bench_probe_gate_up_rows(stream, dg.dev_ptr, du.dev_ptr, sel.ptr + 4 * TOP_K * (i % n_tok), FF, pattern, threads,
+                                                   ahead, sink.ptr)
+            assert rc == 0, f"bm_bench_probe_gate_up_rows: {rc}"
+        res["gate_up"][name] = timed(enqueue)
+    planes = [gpu.buffer(np.uint8, N_EXPERTS * HIDDEN * 640).fill_bytes(0x11) for _ in range(4)]
+    for name, layout in (("rows_of_630_bytes_as_they_are", 0), ("rows_as_planes_of_640_bytes", 1)):
+        def enqueue(i):
+            base = layers[i % len(layers)][2].dev_ptr if layout == 0 else planes[i % len(planes)].ptr
+            rc = probe.bm_bench_probe_down_rows(stream, base, sel.ptr + 4 * TOP_K * (i % n_tok), HIDDEN, layout, sink.ptr)
+            assert rc == 0, f"bm_bench_probe_down_rows: {rc}"
+        res["down"][name] = timed(enqueue)
+    print(json.dumps(res, indent=1), flush=True)
+    gpu.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5, 6, 7, 8),
@@ -831,6 +870,11 @@ def main():
                     help="config 2 only: no timing by events; the step's two launches through the measurement build of the library "
                          "(libbm_moe_hip_timeline.so), whose kernels leave the device's 100 MHz counter at marks inside every "
                          "workgroup; prints when each phase of each launch is reached")
+    ap.add_argument("--down-form", choices=("ring", "split"), default="ring",
+                    help="config 2 only: how the down launch walks a row (bm_set_down_form); `split` is the measured alternative, a side measurement")
+    ap.add_argument("--read-patterns", action="store_true",
+                    help="config 2 only (Q4_K / Q6_K): no timing of the step; the decode launches' read patterns with nothing computed, "
+                         "and other ways of asking for the same bytes")
     ap.add_argument("--handoff", action="store_true",
                     help="config 2 only: no timing of the step; what a hand-over between workgroups inside one launch costs (--layers 1 is enough)")
     ap.add_argument("--mode", choices=("two", "chain"), default="two",
@@ -904,6 +948,11 @@ def main():
             gpu.enqueue_down_combine(dd, act_h, sel.ptr + 4 * t * TOP_K, wt.ptr + 4 * t * TOP_K, None, TOP_K, 1, HIDDEN,
                                      y.ptr + 4 * t * HIDDEN)
 
+    if args.down_form == "split":
+        gpu.set_down_form(bm.DOWN_SPLIT)
+    if args.read_patterns:
+        assert (gate_t, down_t) == (bm.Q4_K, bm.Q6_K), "--read-patterns reads Q4_K gate/up and Q6_K down rows"
+        return read_patterns(bm, gpu, layers, sel, n_tok)
     if args.handoff:
         return handoff(bm, gpu, layers[0][0].dev_ptr, N_EXPERTS * FF * bm.row_bytes(gate_t, HIDDEN))
     if args.timeline:
@@ -1159,7 +1208,8 @@ def main():
                                f"{gate_n} gate/up + {down_n} down, softmax top-8 renormalised "
                                + ("(BASELINE.json configs[1])" if (gate_t, down_t) == (bm.Q4_K, bm.Q6_K)
                                   else "(BASELINE.json configs[1]'s shape with other weight types: a side measurement)"),
-                   "layer_copies": len(layers), "distinct_tokens": n_tok, "launches_per_step": len(kernels), "mode": "hipGraph replay"},
+                   "layer_copies": len(layers), "distinct_tokens": n_tok, "launches_per_step": len(kernels), "mode": "hipGraph replay",
+                   "down_form": args.down_form},
         "hbm_tbps": bytes_per_token / (us_per_token * 1e-6) / 1e12,
         "algorithmic_bytes_per_token": bytes_per_token,
         "wall_ms_lead_in_warmup_and_steps": wall_ms,

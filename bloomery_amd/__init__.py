@@ -21,6 +21,7 @@ FAULT_NONE = 0xFFFFFFFF
 LAYER_NONE = 0xFFFF
 SITE_QUANT_COLUMN, SITE_ROUTER, SITE_EXPERT_ID = 1, 5, 7
 GEMM_EXACT, GEMM_FAST, GEMM_FAST_F16 = 0, 1, 2
+DOWN_RING, DOWN_SPLIT = 0, 1
 PATH_AUTO, PATH_PER_SLOT, PATH_GROUPED, PATH_GEMM = 0, 1, 2, 3
 ACT_SILU_MUL, ACT_SWIGLU_CLAMP, ACT_SWIGLU_OAI, ACT_SITU, ACT_SWIGLU_GCLAMP = 0, 1, 2, 3, 4
 SITE_F32_PRODUCT = 21
@@ -108,6 +109,7 @@ SYMBOLS = {
     "bm_gguf_get_str": (C.c_char_p, [_vp, C.c_char_p]),
     "bm_weights_from_gguf": (_i, [_vp, _vp, C.c_char_p, C.POINTER(_vp), C.POINTER(_i), C.POINTER(_i)]),
     "bm_set_gemm_mode": (_i, [_vp, _i]),
+    "bm_set_down_form": (_i, [_vp, _i]),
     "bm_block_sums": (_i, [_vp, _vp, _i64, _vp, _i, _vp]),
     "bm_capture_begin": (_i, [_vp]),
     "bm_capture_end": (_i, [_vp, C.POINTER(_vp)]),
@@ -590,6 +592,10 @@ class Gpu:
 
     def set_gemm_mode(self, mode):
         self._check(self.lib.bm_set_gemm_mode(self.ctx, mode))
+
+    def set_down_form(self, form):
+        """DOWN_RING (default) or DOWN_SPLIT: how the down + combine launch walks a row; the same bits (bm_set_down_form)."""
+        self._check(self.lib.bm_set_down_form(self.ctx, form))
 
     def enqueue_swiglu_quant(self, g, u, n_cols, act, rule=None, sel=None, n_experts=0):
         """With sel: only the columns of slots whose expert is on the stack (a host-served slot's column is left as it is)."""

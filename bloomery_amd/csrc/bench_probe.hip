@@ -84,7 +84,148 @@ __global__ __launch_bounds__(256) void k_probe_handoff(uint32_t gen, int load, c
     if (lane == 0) out[wg * 8 + 2] = t1, out[wg * 8 + 3] = t2, out[wg * 8 + 4] = right ? 1 : 0, out[wg * 8 + 5] = polls;
 }
 
+// The read patterns of the two decode launches with nothing computed, to be read against their times: what the requests
+// alone cost, and what other ways of asking for the same bytes would.
+// Gate . up (rows of 8 super-blocks of 144 bytes, a workgroup of T threads takes T / 8 row pairs (gate row, up row) of one slot):
+//   pattern 0: a quad a row as k_gate_up_x asks: lane q of the quad the 16 bytes at 16 + 32 q and at 32 + 32 q and the 4 at 4 q of
+//              a super-block, `ahead` super-blocks asked for up front and one more behind every one consumed;
+//   pattern 1: eight lanes a row pair: lane k the 16 code bytes at 16 + 16 k of the gate row's and of the up row's super-block
+//              and the two 16-byte headers (four requests a super-block, every one of a row 16-byte contiguous over the octet);
+//   pattern 2: the workgroup's rows of each matrix are contiguous in memory: plain 16-byte loads over them, thread by thread.
+template <int T, int PATTERN, int AHEAD>
+__global__ __launch_bounds__(T) void k_probe_gate_up_rows(const uint8_t *wg, const uint8_t *wu, const uint32_t *sel, int ff,
+                                                          uint32_t *sink) {
+    constexpr int RP = T / 8;
+    const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
+    const int per_slot = ff / RP;
+    const int slot = blockIdx.x / per_slot, rb = blockIdx.x % per_slot;
+    const uint32_t id = sel[slot];
+    uint4 acc = make_uint4(0, 0, 0, 0);
+    if constexpr (PATTERN == 0) {
+        const uint8_t *wrow = (which ? wu : wg) + ((size_t)id * ff + rb * RP + (tid >> 3)) * 1152;
+        uint4 a[8], b[8];
+        uint32_t c[8];
+        auto ask = [&](int i) {
+            const uint8_t *p = wrow + i * 144;
+            a[i] = *reinterpret_cast<const uint4 *>(p + 16 + 32 * q);
+            b[i] = *reinterpret_cast<const uint4 *>(p + 32 + 32 * q);
+            c[i] = *reinterpret_cast<const uint32_t *>(p + 4 * q);
+        };
+#pragma unroll
+        for (int i = 0; i < AHEAD; i++) ask(i);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            acc.x ^= a[i].x ^ b[i].x ^ c[i], acc.y ^= a[i].y ^ b[i].y, acc.z ^= a[i].z ^ b[i].z, acc.w ^= a[i].w ^ b[i].w;
+            if (i + AHEAD < 8) ask(i + AHEAD);
+        }
+    } else if constexpr (PATTERN == 1) {
+        const int k = tid & 7;
+        const size_t row = ((size_t)id * ff + rb * RP + (tid >> 3)) * 1152;
+        uint4 qg[8], qu[8], hg[8], hu[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            qg[i] = *reinterpret_cast<const uint4 *>(wg + row + i * 144 + 16 + 16 * k);
+            hg[i] = *reinterpret_cast<const uint4 *>(wg + row + i * 144);
+            qu[i] = *reinterpret_cast<const uint4 *>(wu + row + i * 144 + 16 + 16 * k);
+            hu[i] = *reinterpret_cast<const uint4 *>(wu + row + i * 144);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            acc.x ^= qg[i].x ^ qu[i].x ^ hg[i].x ^ hu[i].x, acc.y ^= qg[i].y ^ qu[i].y ^ hg[i].y ^ hu[i].y;
+            acc.z ^= qg[i].z ^ qu[i].z ^ hg[i].z ^ hu[i].z, acc.w ^= qg[i].w ^ qu[i].w ^ hg[i].w ^ hu[i].w;
+        }
+    } else {
+        constexpr int N16 = RP * 1152 / 16, PER = (2 * N16 + T - 1) / T;
+        const uint8_t *g0 = wg + ((size_t)id * ff + rb * RP) * 1152, *u0 = wu + ((size_t)id * ff + rb * RP) * 1152;
+        uint4 v[PER];
+#pragma unroll
+        for (int k = 0; k < PER; k++) {
+            int ch = k * T + tid;
+            ch = ch < 2 * N16 ? ch : 2 * N16 - 1;
+            v[k] = *reinterpret_cast<const uint4 *>((ch < N16 ? g0 : u0) + (size_t)(ch % N16) * 16);
+        }
+#pragma unroll
+        for (int k = 0; k < PER; k++) acc.x ^= v[k].x, acc.y ^= v[k].y, acc.z ^= v[k].z, acc.w ^= v[k].w;
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[tid] = acc.x;
+}
+
+// Down (rows of 3 Q6_K super-blocks; a workgroup of 256 threads takes 8 rows of each of the token's 8 experts, a quad a
+// (row, expert)): layout 0: the rows as they are, super-blocks of 210 bytes back to back, the six requests a lane and
+// super-block of the six-load form (ql, qh, ql, qh, scales, d); layout 1: the same requests over rows laid out as planes (ql of
+// the three super-blocks, then qh, scales, d) in 640 bytes, every piece 16-byte aligned; `w` must hold n_experts * rpe rows
+// of 630 or 640 bytes.
+template <int LAYOUT>
+__global__ __launch_bounds__(256) void k_probe_down_rows(const uint8_t *w, const uint32_t *sel, int rpe, uint32_t *sink) {
+    const int tid = threadIdx.x, q = tid & 3, quad = tid >> 2, c = q & 1, h = q >> 1;
+    const int e = quad % 8, r = blockIdx.x * 8 + quad / 8;
+    const uint32_t id = sel[e];
+    const uint8_t *wrow = w + ((size_t)id * rpe + r) * (LAYOUT == 0 ? 630 : 640);
+    auto ld16 = [](const uint8_t *p) {
+        uint4 v;
+        __builtin_memcpy(&v, p, 16);
+        return v;
+    };
+    uint4 v[3][5];
+    uint32_t d[3];
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+        const uint8_t *ql = LAYOUT == 0 ? wrow + i * 210 : wrow + i * 128;
+        const uint8_t *qh = LAYOUT == 0 ? wrow + i * 210 + 128 : wrow + 384 + i * 64;
+        const uint8_t *sc = LAYOUT == 0 ? wrow + i * 210 + 192 : wrow + 576 + i * 16;
+        const uint8_t *dd = LAYOUT == 0 ? wrow + i * 210 + 208 : wrow + 624 + i * 2;
+        v[i][0] = ld16(ql + 32 * c + 16 * h), v[i][1] = ld16(qh + 16 * h), v[i][2] = ld16(ql + 64 + 32 * c + 16 * h);
+        v[i][3] = ld16(qh + 32 + 16 * h), v[i][4] = ld16(sc);
+        unsigned short d16;
+        __builtin_memcpy(&d16, dd, 2);
+        d[i] = d16;
+    }
+    uint4 acc = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+#pragma unroll
+        for (int j = 0; j < 5; j++) acc.x ^= v[i][j].x, acc.y ^= v[i][j].y, acc.z ^= v[i][j].z, acc.w ^= v[i][j].w;
+        acc.x ^= d[i];
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[tid] = acc.x;
+}
+
 } // namespace
+
+// Enqueues a gate . up read pattern over 8 slots of sel_dev: pattern 0 .. 2 as above, threads 256 or 192 a workgroup (ff a
+// multiple of threads / 8), ahead 4 or 8 (pattern 0 only). Returns 0, -1 for a refused argument, or the HIP error.
+extern "C" int bm_bench_probe_gate_up_rows(void *hip_stream, const void *wg_dev, const void *wu_dev, const uint32_t *sel_dev, int ff,
+                                           int pattern, int threads, int ahead, uint32_t *sink_dev) {
+    if (!wg_dev || !wu_dev || !sel_dev || !sink_dev || ff < 1) return -1;
+    if ((threads != 256 && threads != 192) || ff % (threads / 8) != 0) return -1;
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    const uint8_t *g = static_cast<const uint8_t *>(wg_dev), *u = static_cast<const uint8_t *>(wu_dev);
+    const dim3 grid((unsigned)(8 * ff / (threads / 8)));
+#define BM_PROBE_ROWS(T, P, A) hipLaunchKernelGGL((k_probe_gate_up_rows<T, P, A>), grid, dim3(T), 0, s, g, u, sel_dev, ff, sink_dev)
+    if (pattern == 0 && threads == 256 && ahead == 4) BM_PROBE_ROWS(256, 0, 4);
+    else if (pattern == 0 && threads == 256 && ahead == 8) BM_PROBE_ROWS(256, 0, 8);
+    else if (pattern == 0 && threads == 192 && ahead == 4) BM_PROBE_ROWS(192, 0, 4);
+    else if (pattern == 0 && threads == 192 && ahead == 8) BM_PROBE_ROWS(192, 0, 8);
+    else if (pattern == 1 && threads == 256) BM_PROBE_ROWS(256, 1, 8);
+    else if (pattern == 1 && threads == 192) BM_PROBE_ROWS(192, 1, 8);
+    else if (pattern == 2 && threads == 256) BM_PROBE_ROWS(256, 2, 8);
+    else if (pattern == 2 && threads == 192) BM_PROBE_ROWS(192, 2, 8);
+    else return -1;
+#undef BM_PROBE_ROWS
+    return (int)hipGetLastError();
+}
+
+// Enqueues the down read pattern over the 8 experts of sel_dev: rows_per_expert a multiple of 8, layout 0 or 1 as above.
+extern "C" int bm_bench_probe_down_rows(void *hip_stream, const void *w_dev, const uint32_t *sel_dev, int rows_per_expert, int layout,
+                                        uint32_t *sink_dev) {
+    if (!w_dev || !sel_dev || !sink_dev || rows_per_expert < 8 || rows_per_expert % 8 != 0) return -1;
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    const dim3 grid((unsigned)(rows_per_expert / 8));
+    if (layout == 0) hipLaunchKernelGGL(k_probe_down_rows<0>, grid, dim3(256), 0, s, static_cast<const uint8_t *>(w_dev), sel_dev, rows_per_expert, sink_dev);
+    else if (layout == 1) hipLaunchKernelGGL(k_probe_down_rows<1>, grid, dim3(256), 0, s, static_cast<const uint8_t *>(w_dev), sel_dev, rows_per_expert, sink_dev);
+    else return -1;
+    return (int)hipGetLastError();
+}
 
 // Enqueues the hand-over probe: src_dev of src_bytes (at least 64 MiB, a multiple of 16), flag_dev of 65 words (the flag,
 // then the words; `gen` must differ from what the flag holds: count launches from 1 over a zeroed flag), out_dev of 2048

@@ -21,6 +21,7 @@ struct bm_ctx {
     uint32_t layer = BM_LAYER_NONE;
     uint32_t *route_counts = nullptr; // bm_norm_route's finished-workgroup counts, a word a token, zero between launches
     int gemm_mode = BM_GEMM_EXACT;
+    int down_form = BM_DOWN_RING;
     bmk::GateRule rule = {0u, 0.0f}; // silu(g) * u
     std::string err;
 };
@@ -172,7 +173,7 @@ int bm_fault_read(bm_ctx *ctx, uint32_t layer, uint32_t *word0, uint32_t *mask) 
     return rc;
 }
 
-static bmk::Launch launch_of(bm_ctx *ctx) { return bmk::Launch{ctx->stream, ctx->fault, ctx->layer, ctx->rule}; }
+static bmk::Launch launch_of(bm_ctx *ctx) { return bmk::Launch{ctx->stream, ctx->fault, ctx->layer, ctx->rule, ctx->down_form}; }
 static int rule_checked(bm_ctx *ctx, const char *what, int rule, float limit, bmk::GateRule *out);
 // The launch state of a gate . up entry: the entry's own rule when the caller passes one, else the context's.
 static int launch_under(bm_ctx *ctx, const char *what, const bm_gate_act *act, bmk::Launch *L) {
@@ -1046,6 +1047,14 @@ int bm_set_gemm_mode(bm_ctx *ctx, int mode) {
     if (mode != BM_GEMM_EXACT && mode != BM_GEMM_FAST && mode != BM_GEMM_FAST_F16)
         return fail(ctx, BM_EARG, "bm_set_gemm_mode: mode %d is none of BM_GEMM_EXACT, BM_GEMM_FAST, BM_GEMM_FAST_F16", mode);
     ctx->gemm_mode = mode;
+    return BM_OK;
+}
+
+int bm_set_down_form(bm_ctx *ctx, int form) {
+    if (!ctx) return fail(nullptr, BM_EARG, "bm_set_down_form: ctx is NULL");
+    if (form != BM_DOWN_RING && form != BM_DOWN_SPLIT)
+        return fail(ctx, BM_EARG, "bm_set_down_form: form %d is neither BM_DOWN_RING nor BM_DOWN_SPLIT", form);
+    ctx->down_form = form;
     return BM_OK;
 }
 

@@ -552,6 +552,27 @@ __device__ __forceinline__ void bm_dot_q6k(const Blk<BM_Q6K> &b, const Act<BM_Q6
     }
 }
 
+// The operands of bm_dot_q6k's four multiply-adds, in its order: (half 0: accumulator 0, accumulator 1), (half 1: the same);
+// acc = fmaf(p, s, acc) over them is bm_dot_q6k.
+__device__ __forceinline__ void bm_q6k_terms(const Blk<BM_Q6K> &b, const Act<BM_Q6K> &a, int c, int h, float (&p)[4], float (&s)[4]) {
+    const Q6Parts parts = bm_q6k_parts(b);
+    const float d = bm_half_to_f32(parts.d);
+    const int bi = 8 * (2 * c + h);
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        int s0, s1;
+        bm_q6_dot16x2(j ? b.ql1 : b.ql0, j ? parts.qh1 : parts.qh0, 2 * c, a.aa[j], a.ab[j], s0, s1);
+        s0 -= 32 * a.sa[j];
+        s1 -= 32 * a.sb[j];
+        const int sc0 = __builtin_amdgcn_sbfe((int)(j ? parts.sc.z : parts.sc.x), bi, 8);
+        const int sc1 = __builtin_amdgcn_sbfe((int)(j ? parts.sc.w : parts.sc.y), bi, 8);
+        p[2 * j] = (d * (float)sc0) * a.d8a[j];
+        s[2 * j] = (float)s0;
+        p[2 * j + 1] = (d * (float)sc1) * a.d8b[j];
+        s[2 * j + 1] = (float)s1;
+    }
+}
+
 // A Q6_K super-block's weight side, formed once for several columns: the 6-bit code words of the lane's four
 // 16-value groups and the four products d * scale.
 struct Q6Dec {

@@ -22,6 +22,7 @@ struct Launch {
     uint32_t *fault; // device fault word, u32[BM_FAULT_WORDS]
     uint32_t layer;  // layer the launch raises with
     GateRule rule;   // what the gate . up launches apply
+    int down_form = 0; // BM_DOWN_RING or BM_DOWN_SPLIT: how down_combine walks a row (bm_set_down_form)
 };
 
 // Largest dynamic LDS a launch may ask for (gfx950 has 160 KiB a workgroup).

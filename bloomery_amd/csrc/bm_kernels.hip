@@ -421,6 +421,94 @@ __global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_ex
                                  blockIdx.x / blocks_per_token, blockIdx.x % blocks_per_token, fault, layer);
 }
 
+// k_down_combine for a Q6_K stack of NB super-blocks a row with the row's super-blocks dealt to the waves (BM_DOWN_SPLIT, the
+// measured alternative: 5.6 us against the ring's 5.2 at the headline shape): a workgroup of 256 NB threads, the same 64
+// (row, slot) pairs as k_down_combine's, wave w super-block w % NB of quads 16 (w / NB) .. + 16. Under the ring one wave a SIMD
+// runs its loads, its wait and its arithmetic one after the other; here every super-block of every row is asked for at once by
+// a wave of its own and NB waves a SIMD overlap. What it shows: the launch is bound by how fast a compute unit's address unit
+// takes the quads' scattered 16-byte requests, not by waves to overlap - the twelve waves' requests queue for it, the first
+// barrier (every wave's requests issued) comes 2.3 us after the start against 1.9, and the shorter arithmetic behind it (0.95
+// us against 1.4) does not win that back. The numbers are the same:
+// a wave leaves the operands of its super-block's multiply-adds (the f32 scale product and the integer sum as a float, two
+// halves by two accumulators a lane) in LDS, and the wave of the last super-block runs the chain in the CPU path's order,
+// super-block by super-block, then closes the quad as bm_quad_finish does.
+template <int NB>
+__global__ __launch_bounds__(256 * NB) void k_down_combine_q6k_split(const uint8_t *w, u32 n_experts, const uint8_t *act,
+                                                                     const u32 *sel, const float *wts, const float *resid,
+                                                                     int spt, int rpe, float *y, u32 *fault, u32 layer) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    constexpr int WT = BM_Q6K;
+    const int tid = threadIdx.x, q = tid & 3, wave = tid >> 6;
+    BM_MARK(2048, 0);
+    const int i = wave % NB, quad = 16 * (wave / NB) + ((tid & 63) >> 2);
+    const int D = 64 / spt;
+    const int blocks_per_token = (rpe + D - 1) / D;
+    const int t = blockIdx.x / blocks_per_token, rb = blockIdx.x % blocks_per_token;
+    const int e = quad % spt, dl = quad / spt;
+    const int r = rb * D + dl;
+    const u32 id = sel[t * spt + e];
+    const int si = tid < spt ? tid : 0;
+    const u32 my_sel = sel[t * spt + si];
+    const float my_w = wts[t * spt + si];
+    const bool live = id < n_experts;
+    const bool active = dl < D && r < rpe && live;
+    const float resid_v = resid && tid < D && rb * D + tid < rpe ? resid[(size_t)t * rpe + rb * D + tid] : 0.0f;
+    constexpr size_t row_bytes = (size_t)NB * BM_Q6K_BLOCK;
+    constexpr int col_bytes = bm_act_col_bytes<WT>(NB);
+    const uint8_t *act_cols = act + (size_t)t * spt * col_bytes;
+    Stage<2> st; // 16 bytes a thread of 768: the eight columns of 1248 bytes
+    st.load(act_cols, spt * col_bytes);
+    if (!live && id != 0xffffffffu && rb == 0 && dl == 0 && q == 0 && i == 0) bm_raise(fault, layer, kSiteExpertId);
+    const uint8_t *wrow = w + ((size_t)(live ? id : 0) * rpe + (active ? r : 0)) * row_bytes;
+    uint8_t *cols = lds;
+    float *terms = reinterpret_cast<float *>(cols + (size_t)spt * col_bytes); // [64 quads][NB - 1][4 lanes][8]
+    float *part = terms + 64 * (NB - 1) * 32;                                  // [D][spt]
+    float *s_w = part + D * spt;                                               // [spt]
+    u32 *s_sel = reinterpret_cast<u32 *>(s_w + spt);                           // [spt]
+    BM_TICK(t_id, id);
+    const Blk<WT> b = bm_load_blk<WT>(wrow, i, q);
+    BM_TICK(t_asked, tid);
+    st.store(cols, act_cols, spt * col_bytes);
+    if (tid < spt) {
+        s_w[tid] = my_w;
+        s_sel[tid] = my_sel;
+    }
+    __syncthreads();
+    BM_MARK(2048, 1);
+    BM_TOCK(2048, 4, t_id);
+    BM_TOCK(2048, 5, t_asked);
+    const int c = q & 1, h = q >> 1;
+    const Act<WT> a = bm_act_q6k(bm_act_view<WT>(cols + (size_t)e * col_bytes, NB), i, c, h);
+    float p[4], s[4]; // (half 0: accumulator 0, accumulator 1), (half 1: ...)
+    bm_q6k_terms(b, a, c, h, p, s);
+    BM_TICK(t_terms, p[3]);
+    float *mine = terms + ((size_t)(quad * (NB - 1) + i) * 4 + q) * 8;
+    if (i < NB - 1) {
+        *reinterpret_cast<float4 *>(mine) = make_float4(p[0], s[0], p[1], s[1]);
+        *reinterpret_cast<float4 *>(mine + 4) = make_float4(p[2], s[2], p[3], s[3]);
+    }
+    __syncthreads();
+    BM_MARK(2048, 2);
+    BM_TOCK(2048, 6, t_terms);
+    if (i == NB - 1) {
+        float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+        for (int u = 0; u < NB - 1; u++) {
+            const float *o = terms + ((size_t)(quad * (NB - 1) + u) * 4 + q) * 8;
+            const float4 lo = *reinterpret_cast<const float4 *>(o), hi = *reinterpret_cast<const float4 *>(o + 4);
+            a0 = fmaf(lo.x, lo.y, a0), a1 = fmaf(lo.z, lo.w, a1);
+            a0 = fmaf(hi.x, hi.y, a0), a1 = fmaf(hi.z, hi.w, a1);
+        }
+        a0 = fmaf(p[0], s[0], a0), a1 = fmaf(p[1], s[1], a1);
+        a0 = fmaf(p[2], s[2], a0), a1 = fmaf(p[3], s[3], a1);
+        const float v = bm_quad_finish<WT>(a0, a1);
+        if (q == 0 && dl < D) part[dl * spt + e] = v;
+    }
+    __syncthreads();
+    if (tid < D && rb * D + tid < rpe) y[(size_t)t * rpe + rb * D + tid] = slot_sum(part + tid * spt, s_w, s_sel, spt, n_experts, resid_v, resid != nullptr);
+    BM_MARK(2048, 3);
+}
+
 // The gate . up . SwiGLU workgroup of the fused step: as k_gate_up's, except that it quantizes its token's f32 row
 // itself (into LDS; no quantizer launch, no activation column in memory) and always writes its q8_2 block of the
 // slot's down activation.
@@ -849,6 +937,13 @@ hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_expe
     const int D = 64 / spt;
     const size_t lds = down_combine_lds(wtype, k, spt);
     const unsigned grid = (unsigned)m * (unsigned)((rpe + D - 1) / D);
+    if (L.down_form == 1 && wtype == BM_Q6K && nb == 3 && 64 % spt == 0) { // BM_DOWN_SPLIT where it is built: the super-blocks of a row dealt to the waves
+        constexpr int NB = 3;
+        const size_t lds_split = (size_t)spt * bm_act_col_bytes<BM_Q6K>(NB) + (64 * (NB - 1) * 32 + D * spt + 2 * spt) * sizeof(float);
+        hipLaunchKernelGGL(k_down_combine_q6k_split<NB>, dim3(grid), dim3(256 * NB), lds_split, L.stream, w, (u32)n_experts, act, sel, wts,
+                           resid, spt, rpe, y, L.fault, L.layer);
+        return hipGetLastError();
+    }
 #define CALL_BODY                                                                                                      \
     auto kern = k_down_combine<WT, U, NB>;                                                                             \
     hipError_t e = allow_lds(kern, lds);                                                                               \

@@ -330,6 +330,17 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
 #define BM_GEMM_FAST 1
 #define BM_GEMM_FAST_F16 2
 int bm_set_gemm_mode(bm_ctx *ctx, int mode);
+/* How the down + combine launch (bm_down_combine, the second launch of bm_moe_decode and of the per-slot path of bm_moe_forward)
+ * walks a weight row; the bits of y are the same either way. No counterpart in the reference (its down launch has one form,
+ * crates/gpu/src/arch/qwen3moe/experts.rs:227-318): a measurement switch.
+ *   BM_DOWN_RING (default): four lanes a (row, slot), the row's super-blocks one after the other through a ring of registers;
+ *   BM_DOWN_SPLIT: the row's super-blocks dealt to the waves of a larger workgroup (every super-block asked for at once, three
+ *     waves a SIMD), the f32 chain run by the last super-block's wave in the CPU path's order. Built for Q6_K stacks of 768-value
+ *     rows with 1, 2, 4 or 8 slots a token; every other launch runs as under BM_DOWN_RING. Measured slower on MI355X (5.6 against
+ *     5.2 us at 2048 rows x 8 slots) and kept as the measured alternative form. */
+#define BM_DOWN_RING 0
+#define BM_DOWN_SPLIT 1
+int bm_set_down_form(bm_ctx *ctx, int form);
 /* GemmKernels::enqueue_swiglu_quant (crates/gpu/src/gemm/swiglu.rs:46): column c of act = the quantized
  * silu(g) * u of g_dev / u_dev[c * k .. (c + 1) * k), k = act's k, slot-major as the gate and up GEMMs write them;
  * bm_quantize's bytes of the CPU path's SwiGLU, in the column form of act's type (Q8_2_X4 or Q8_K). */

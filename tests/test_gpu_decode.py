@@ -848,6 +848,50 @@ def test_bench_probe_runs_and_refuses(gpu):
         b.free()
 
 
+@pytest.mark.parametrize("top_k,m,hidden", ((8, 3, 2048), (4, 2, 512), (2, 5, 72), (1, 1, 64), (3, 2, 256)))
+def test_down_form_split_gives_the_rings_bits(gpu, top_k, m, hidden):
+    """bm_set_down_form(BM_DOWN_SPLIT): the down + combine launch with a row's super-blocks dealt to the waves gives the bits of
+    the default form (and so the oracle's), with a residual, a host-served slot and an id past the stack among the slots, at
+    every number of slots a token it is built for; with three slots a token (64 is no multiple) the launch runs in the default
+    form and the switch changes nothing. It refuses a form it does not know."""
+    ff, n_experts = 768, 10
+    rng = np.random.default_rng(9100 + top_k)
+    wd = ora.quantize_rows(bm.Q6_K, normal_f32(rng, (n_experts * hidden, ff), 0.05), n_experts * hidden, ff)
+    dd = gpu.weights(bm.Q6_K, n_experts * hidden, ff, wd)
+    hrows = normal_f32(rng, (m * top_k, ff))
+    act = gpu.act(bm.Q6_K, ff, m * top_k)
+    hd = gpu.upload(hrows, np.float32)
+    gpu.enqueue_quantize(hd, m * top_k, act)
+    ids, wts = route(rng, m, n_experts, top_k)
+    if top_k >= 2:
+        ids[0, 1] = bm.HOST_SLOT
+    if m >= 2:
+        ids[1, 0] = n_experts + 3
+    resid = normal_f32(rng, (m, hidden))
+    sel, wt, rd = gpu.upload(ids, np.uint32), gpu.upload(wts, np.float32), gpu.upload(resid, np.float32)
+    ys = []
+    try:
+        for form in (bm.DOWN_RING, bm.DOWN_SPLIT, bm.DOWN_RING):
+            gpu.set_down_form(form)
+            gpu.fault_clear()
+            y = gpu.buffer(np.float32, m * hidden).fill_bytes(0xFF)
+            for _ in range(2):
+                gpu.enqueue_down_combine(dd, act, sel, wt, rd, top_k, m, hidden, y)
+            ys.append(y.download().copy())
+            y.free()
+            assert (gpu.fault()[0] != bm.FAULT_NONE) == (m >= 2)
+        assert np.array_equal(ys[0].view(np.uint32), ys[1].view(np.uint32)), "split against ring"
+        assert np.array_equal(ys[0].view(np.uint32), ys[2].view(np.uint32))
+        with pytest.raises(bm.GpuError) as e:
+            gpu.set_down_form(2)
+        assert "bm_set_down_form" in str(e.value)
+    finally:
+        gpu.set_down_form(bm.DOWN_RING)
+        gpu.fault_clear()
+        for b in (dd, act, hd, sel, wt, rd):
+            b.free()
+
+
 @pytest.mark.parametrize("down_type,hidden,ff,n_experts,m,top_k", ((bm.Q6_K, 2048, 768, 10, 3, 8), (bm.Q4_K, 512, 512, 5, 4, 2),
                                                                     (bm.Q5_K, 768, 256, 4, 2, 3), (bm.IQ4_XS, 1024, 512, 6, 2, 4)))
 def test_down_combine_from_f32_rows_for_either_column_form(gpu, down_type, hidden, ff, n_experts, m, top_k):

@@ -29,7 +29,7 @@ HIDDEN, FF, N_EXPERTS, TOP_K = 2048, 768, 128, 8
 HBM_PEAK_GBS = 8000.0
 # HBM bytes a launch of the headline configuration's dominant kernel moves (read + written), from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE summary under profiles/ (counter x the copy-kernel calibration measured in the same run).
-GATE_UP_X_TRAFFIC_BYTES = 14430680
+GATE_UP_X_TRAFFIC_BYTES = 14430300
 
 
 def host_threads():
@@ -345,7 +345,8 @@ def prefill_leg(args, bm, ora, threads, gpu, stacks, layer, m, reps=16):
     ops = 2.0 * n_slots * (2 * FF * HIDDEN + HIDDEN * FF)
     gate_ops = 2.0 * n_slots * FF * HIDDEN
     out = {}
-    for mode, code in (("fast", bm.GEMM_FAST), ("exact", bm.GEMM_EXACT)):
+    modes = (("fast", bm.GEMM_FAST), ("exact", bm.GEMM_EXACT)) + ((("fast_f16", bm.GEMM_FAST_F16),) if args.gemm_f16 else ())
+    for mode, code in modes:
         gpu.set_gemm_mode(code)
         step(0)
         parity = parity_of(y.download()[:n_chk * HIDDEN].reshape(n_chk, HIDDEN), want)
@@ -368,6 +369,8 @@ def prefill_leg(args, bm, ora, threads, gpu, stacks, layer, m, reps=16):
     res.update({k: out["fast"][k] for k in ("tops", "frac_of_5.0_POPs", "ms_per_step", "steps", "warmup", "parity", "gate_gemm_tops",
                                             "gate_gemm_frac_of_5.0_POPs", "kernel_us")})
     res["exact"] = out["exact"]
+    if "fast_f16" in out:
+        res["fast_f16"] = out["fast_f16"]
     for b in (xd, sel, wt, act, act_h, g, u, down, y, table):
         b.free()
     return res, (x, ids, wts)
@@ -385,7 +388,7 @@ def bench_prefill(args, bm, ora, threads):
                              TOP_K, min(m, 64), 0)
     emit("prefill_int8_tops", res["tops"], "TOP/s", res["steps"], res["warmup"], res["ms_per_step"], res["workload"],
          {k: res[k] for k in ("mode", "int8_ops_per_step", "distinct_experts", "weight_bytes_hit", "us_per_token", "kernel_us",
-                              "parity", "exact")},
+                              "parity", "exact", "fast_f16") if k in res},
          {"bound": "mfma", "kernel": "k_gemm (gate GEMM, fast mode)", "achieved": res["gate_gemm_tops"], "peak": 5000.0,
           "unit": "TOP/s", "frac": res["gate_gemm_frac_of_5.0_POPs"], "traffic": None}, cpu, higher=True)
     gpu.close()
@@ -872,6 +875,8 @@ def main():
                          "workgroup; prints when each phase of each launch is reached")
     ap.add_argument("--down-form", choices=("ring", "split"), default="ring",
                     help="config 2 only: how the down launch walks a row (bm_set_down_form); `split` is the measured alternative, a side measurement")
+    ap.add_argument("--gemm-f16", action="store_true",
+                    help="prefill leg: also time the tolerance mode's f16-operand form (BM_GEMM_FAST_F16, Q4_K GEMMs), under `fast_f16`")
     ap.add_argument("--read-patterns", action="store_true",
                     help="config 2 only (Q4_K / Q6_K): no timing of the step; the decode launches' read patterns with nothing computed, "
                          "and other ways of asking for the same bytes")

@@ -558,7 +558,7 @@ def bench_dsv3_prefill(args, bm, ora, threads):
          "popularity, Q8_K columns; random legal blocks (a side measurement; the shape is BASELINE.json configs[4]'s)",
          {"mode": "fast (BM_GEMM_FAST); `exact` beside it", "int8_ops_per_step": ops, "distinct_experts": int(len(np.unique(ids))),
           "fast": f, "exact": out["exact"]},
-         {"bound": "mfma", "kernel": "k_gemm_iq2<fast> (gate)", "achieved": f["gate_gemm_tops"], "peak": 5000.0, "unit": "TOP/s",
+         {"bound": "mfma", "kernel": "k_gemm_iq<IQ2_XXS, fast> (gate)", "achieved": f["gate_gemm_tops"], "peak": 5000.0, "unit": "TOP/s",
           "frac": f["gate_gemm_frac_of_5.0_POPs"], "traffic": None}, None, higher=True)
     gpu.close()
 

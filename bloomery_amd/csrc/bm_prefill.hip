@@ -817,9 +817,9 @@ __global__ __launch_bounds__(kFastThreads, 2) void k_gemm_fast(const uint8_t *w,
 constexpr int kIqRows = 64;
 constexpr int kIqStride = 256 + 16; // bytes a row's or a column's 256 codes take in LDS
 constexpr int kIqLine = 64 + 4;     // floats a line of the per-lane tables
-template <bool EXACT>
-__host__ __device__ constexpr size_t gemm_iq2_lds_bytes() {
-    return sizeof(GemmLds) + (size_t)tab_bytes<BM_IQ2XXS>() + 3 * (size_t)64 * kIqStride + 2 * 64 * sizeof(float) +
+template <int WT, bool EXACT>
+__host__ __device__ constexpr size_t gemm_iq_lds_bytes() {
+    return sizeof(GemmLds) + (size_t)tab_bytes<WT>() + 3 * (size_t)64 * kIqStride + 2 * 64 * sizeof(float) +
            (EXACT ? 2 * 8 * kIqLine * sizeof(float) : 3 * 64 * 16);
 }
 
@@ -832,14 +832,44 @@ __device__ __forceinline__ void iq2_planes(u32 u, u32 sc, u32 &hi, u32 &lo) {
     hi = __builtin_amdgcn_perm(po + 0x00800080u, pe + 0x00800080u, 0x07030501u);
 }
 
-template <bool EXACT>
-__global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
-                                                     const u32 *tiles, const u32 *n_tiles, u32 n_slabs, u32 slot_div,
-                                                     u32 n_slots, float *y) {
+// The same split for a product of four signed bytes with a signed scale (|product| <= 4064): lo the low byte read as signed,
+// hi what is left over 256.
+__device__ __forceinline__ void iq_planes_signed(u32 v, int sc, u32 &hi, u32 &lo) {
+    const int p0 = bm_mul24(__builtin_amdgcn_sbfe((int)v, 0, 8), sc), p1 = bm_mul24(__builtin_amdgcn_sbfe((int)v, 8, 8), sc);
+    const int p2 = bm_mul24(__builtin_amdgcn_sbfe((int)v, 16, 8), sc), p3 = bm_mul24(__builtin_amdgcn_sbfe((int)v, 24, 8), sc);
+    lo = ((u32)p0 & 0xffu) | (((u32)p1 & 0xffu) << 8) | (((u32)p2 & 0xffu) << 16) | ((u32)p3 << 24);
+    hi = ((u32)((p0 + 128) >> 8) & 0xffu) | (((u32)((p1 + 128) >> 8) & 0xffu) << 8) | (((u32)((p2 + 128) >> 8) & 0xffu) << 16) |
+         ((u32)((p3 + 128) >> 8) << 24);
+}
+
+// The types that dot against Q8_K columns (crates/gpu/src/gemm/kernels.rs:867 gemm_iq2xxs, :759 gemm_q3k, :1139 gemm_iq3xxs,
+// :1248 gemm_iq4xs). What differs between them is how a row's super-block becomes signed code x scale terms (the staging) and
+// the f32 step a super-block; the columns, the lane-major operands, the two byte planes and the products are the same.
+//   IQ2_XXS, IQ3_XXS: terms (2 s + 1) (offset + u), offset 43 / 64, the offsets folded out through the column's sums first,
+//     eight accumulators, d = f16 / 8 and f16 / 4;
+//   IQ4_XS: terms scale x level (scale -32 .. 31, the sixteen levels), eight accumulators, one multiply-add a super-block each
+//     (crates/qdot/src/lib.rs:11171-11173);
+//   Q3_K: terms scale x (u - 4) over the sixteen 16-value groups, one integer a super-block and one accumulator, the float step
+//     acc + (dcol d) sum with every operation rounded on its own (crates/qdot/src/lib.rs:2223-2245).
+// EXACT only for the three added types: the tolerance mode runs them in this order too.
+template <int WT>
+struct IqGemm {
+    static constexpr bool kFold = WT == BM_IQ2XXS || WT == BM_IQ3XXS;
+    static constexpr int kOff = WT == BM_IQ2XXS ? 43 : 64;
+    static constexpr int kLanes = WT == BM_Q3K ? 1 : 8;
+    static constexpr int kBlock = WT == BM_IQ2XXS ? BM_IQ2XXS_BLOCK : WT == BM_IQ3XXS ? BM_IQ3XXS_BLOCK : WT == BM_IQ4XS ? BM_IQ4XS_BLOCK : BM_Q3K_BLOCK;
+};
+
+template <int WT, bool EXACT>
+__global__ __launch_bounds__(256, 2) void k_gemm_iq(const uint8_t *w, int rpe, int nb, const uint8_t *act, const u32 *cols,
+                                                    const u32 *tiles, const u32 *n_tiles, u32 n_slabs, u32 slot_div,
+                                                    u32 n_slots, float *y) {
+    static_assert(EXACT || WT == BM_IQ2XXS, "the one-accumulator form is IQ2_XXS's");
+    using G = IqGemm<WT>;
     extern __shared__ __align__(16) uint8_t lds[];
     GemmLds *tab = reinterpret_cast<GemmLds *>(lds);
-    const Iq2Tables tb = stage_tables<BM_IQ2XXS>(lds + sizeof(GemmLds));
-    uint8_t *a_codes = lds + sizeof(GemmLds) + tab_bytes<BM_IQ2XXS>();
+    [[maybe_unused]] const Iq2Tables tb = stage_tables<WT>(lds + sizeof(GemmLds));
+    uint8_t *a_codes = lds + sizeof(GemmLds) + tab_bytes<WT>();
     uint8_t *w_hi = a_codes + 64 * kIqStride;
     uint8_t *w_lo = w_hi + 64 * kIqStride;
     float *dy_t = reinterpret_cast<float *>(w_lo + 64 * kIqStride); // [slot]
@@ -871,7 +901,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, 
         tab->col[tid] = s / slot_div;
     }
     __syncthreads();
-    const u32 row_bytes = (u32)nb * BM_IQ2XXS_BLOCK, col_bytes = (u32)nb * BM_Q8K_STRIDE;
+    const u32 row_bytes = (u32)nb * G::kBlock, col_bytes = (u32)nb * BM_Q8K_STRIDE;
     // what this thread stages of every super-block:
     //   four 16-byte pieces of column codes (column tid / 16 + 16 j, piece tid % 16 of the sixteen): values 16 (piece % 2) ..
     //   of sub-block piece / 2, i.e. the four-value groups of lanes 4 (piece % 2) .. + 3, one word each;
@@ -892,9 +922,33 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, 
         uint4 ra[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) __builtin_memcpy(&ra[j], act + (src_a[j] + (u32)i * BM_Q8K_STRIDE), 16);
-        const uint8_t *blk = we + (src_w + (u32)i * BM_IQ2XXS_BLOCK);
-        const uint4 rq = bm_ld16u(blk + 2 + 16 * wq);
-        const u32 rd = bm_ld2u(blk);
+        const uint8_t *blk = we + (src_w + (u32)i * G::kBlock);
+        // the row's two sub-blocks 2 wq and 2 wq + 1, as the type lays them out
+        uint4 rq = make_uint4(0, 0, 0, 0), rq2 = rq, rq3 = rq, rq4 = rq;
+        uint2 rx = make_uint2(0, 0);
+        u32 rd = 0, ra2 = 0;
+        if constexpr (WT == BM_IQ2XXS) {
+            rq = bm_ld16u(blk + 2 + 16 * wq);
+            rd = bm_ld2u(blk);
+        } else if constexpr (WT == BM_IQ3XXS) {
+            rq = bm_ld16u(blk + 2 + 16 * wq); // the index bytes of the two sub-blocks
+            __builtin_memcpy(&rx, blk + 66 + 8 * wq, 8); // their sign/scale words
+            rd = bm_ld2u(blk);
+        } else if constexpr (WT == BM_IQ4XS) {
+            __builtin_memcpy(&rx, blk, 8); // d | scales_h << 16, scales_l
+            rq = bm_ld16u(blk + 8 + 32 * wq);
+            rq2 = bm_ld16u(blk + 24 + 32 * wq);
+            rd = rx.x & 0xffffu;
+        } else { // Q3_K: the 32 field bytes of half wq / 2, the 32 high-bit bytes, the scales and d
+            rq = bm_ld16u(blk + 32 + 32 * (wq >> 1));
+            rq2 = bm_ld16u(blk + 48 + 32 * (wq >> 1));
+            rq3 = bm_ld16u(blk);
+            rq4 = bm_ld16u(blk + 16);
+            const uint4 tail = bm_ld16u(blk + 94); // the twelve scale bytes at 2 .., d at 14
+            rx = make_uint2((tail.x >> 16) | (tail.y << 16), (tail.y >> 16) | (tail.z << 16)); // scale words a0, a1
+            ra2 = (tail.z >> 16) | (tail.w << 16);                                             // a2: their high bits
+            rd = tail.w >> 16;
+        }
         float cdy = 0.0f;
         uint4 cb0 = make_uint4(0, 0, 0, 0), cb1 = cb0;
         if (tid < 64) {
@@ -919,7 +973,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, 
             for (int l = 0; l < 8; l++) { // the two 16-value sums of sub-block l
                 const int bs = (int)(short)(bw[l] & 0xffffu) + (int)(short)(bw[l] >> 16);
                 if constexpr (EXACT) {
-                    bs_t[l * kIqLine + tid] = (float)bs;
+                    if constexpr (G::kFold) bs_t[l * kIqLine + tid] = (float)bs;
                 } else { // 256 hi + lo with lo the low byte read as signed
                     bl[l >> 2] |= ((u32)bs & 0xffu) << (8 * (l & 3));
                     bh[l >> 2] |= ((u32)((bs + 128) >> 8) & 0xffu) << (8 * (l & 3));
@@ -930,27 +984,77 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, 
                 *reinterpret_cast<uint4 *>(x_bh + 16 * tid) = make_uint4(bh[0], bh[1], 0u, 0u);
             }
         }
-        if (wq == 0) d_t[wr] = 0.125f * bm_half_to_f32((unsigned short)rd);
-        u32 scs[2];
+        if (wq == 0) {
+            const float dh = bm_half_to_f32((unsigned short)rd);
+            d_t[wr] = WT == BM_IQ2XXS ? 0.125f * dh : WT == BM_IQ3XXS ? 0.25f * dh : dh;
+        }
+        [[maybe_unused]] u32 scs[2] = {0, 0};
 #pragma unroll
         for (int e2 = 0; e2 < 2; e2++) {
             const int b = 2 * wq + e2;
-            const u32 idx = e2 ? rq.z : rq.x, aux = e2 ? rq.w : rq.y;
-            const u32 sc = 2u * (aux >> 28) + 1u;
-            scs[e2] = sc;
-            if constexpr (EXACT) sc_t[b * kIqLine + wr] = (float)sc;
+            // the four values 4 l .. 4 l + 3 of sub-block b, times the scale, as the two byte planes at lane l's place
+            auto put = [&](int l, u32 h, u32 lo) {
+                const int at = wr * kIqStride + 32 * l + 4 * b;
+                *reinterpret_cast<u32 *>(w_hi + at) = h;
+                *reinterpret_cast<u32 *>(w_lo + at) = lo;
+            };
+            if constexpr (WT == BM_IQ2XXS || WT == BM_IQ3XXS) {
+                const u32 aux = WT == BM_IQ2XXS ? (e2 ? rq.w : rq.y) : (e2 ? rx.y : rx.x);
+                const u32 sc = 2u * (aux >> 28) + 1u;
+                scs[e2] = sc;
+                if constexpr (EXACT) sc_t[b * kIqLine + wr] = (float)sc;
 #pragma unroll
-            for (int q = 0; q < 4; q++) { // values 8 q .. 8 q + 7: lanes 2 q and 2 q + 1
-                u32 c_lo, c_hi;
-                bm_iq2_codes(tb, (idx >> (8 * q)) & 0xffu, (aux >> (7 * q)) & 127u, c_lo, c_hi);
-                u32 h0, l0, h1, l1;
-                iq2_planes(c_lo, sc, h0, l0);
-                iq2_planes(c_hi, sc, h1, l1);
-                const int at = wr * kIqStride + 32 * (2 * q) + 4 * b;
-                *reinterpret_cast<u32 *>(w_hi + at) = h0;
-                *reinterpret_cast<u32 *>(w_lo + at) = l0;
-                *reinterpret_cast<u32 *>(w_hi + at + 32) = h1;
-                *reinterpret_cast<u32 *>(w_lo + at + 32) = l1;
+                for (int q = 0; q < 4; q++) { // values 8 q .. 8 q + 7: lanes 2 q and 2 q + 1
+                    u32 c_lo, c_hi;
+                    if constexpr (WT == BM_IQ2XXS) {
+                        const u32 idx = e2 ? rq.z : rq.x;
+                        bm_iq2_codes(tb, (idx >> (8 * q)) & 0xffu, (aux >> (7 * q)) & 127u, c_lo, c_hi);
+                    } else { // index bytes 2 q and 2 q + 1 of the sub-block's eight, sign group q
+                        const u32 word = e2 ? ((q & 2) ? rq.w : rq.z) : ((q & 2) ? rq.y : rq.x);
+                        const u32 pair = word >> (16 * (q & 1));
+                        const uint2 g0 = tb.grid3[pair & 0xffu], g1 = tb.grid3[(pair >> 8) & 0xffu];
+                        const uint2 sg = tb.signs[(aux >> (7 * q)) & 127u];
+                        c_lo = bm_iq_pick(g0.x, g0.y, sg.x);
+                        c_hi = bm_iq_pick(g1.x, g1.y, sg.y);
+                    }
+                    u32 h0, l0, h1, l1;
+                    iq2_planes(c_lo, sc, h0, l0);
+                    iq2_planes(c_hi, sc, h1, l1);
+                    put(2 * q, h0, l0);
+                    put(2 * q + 1, h1, l1);
+                }
+            } else if constexpr (WT == BM_IQ4XS) {
+                // crates/gguf/src/quant.rs:1989-1991: nibble b % 2 of scales_l[b / 2] under bits 2b .. of scales_h, less 32
+                const u32 sl = (rx.y >> (8 * wq + 4 * e2)) & 15u, sh = (rx.x >> (16 + 4 * wq + 2 * e2)) & 3u;
+                const int sc = (int)(sl | (sh << 4)) - 32;
+                const uint4 cw = e2 ? rq2 : rq;
+                const u32 qw[4] = {cw.x, cw.y, cw.z, cw.w};
+#pragma unroll
+                for (int l = 0; l < 4; l++) { // low nibbles: values 4 l ..; high nibbles: values 16 + 4 l ..
+                    u32 h, lo;
+                    iq_planes_signed(bm_iq4_levels<0>(qw[l]), sc, h, lo);
+                    put(l, h, lo);
+                    iq_planes_signed(bm_iq4_levels<4>(qw[l]), sc, h, lo);
+                    put(4 + l, h, lo);
+                }
+            } else { // Q3_K: sub-block b = 4 j + f is field f of the half's 32 cells; cell p is value p of the sub-block
+                const int j = wq >> 1, f = 2 * (wq & 1) + e2;
+                // the sixteen six-bit scales (crates/qdot/src/lib.rs:2162-2174): group 8 j + 2 f + odd
+                const u32 lo4 = j ? (rx.x >> 4) : rx.x, lo41 = j ? (rx.y >> 4) : rx.y, hi2 = ra2 >> (4 * j);
+                const u32 w0 = (lo4 & 0x0f0f0f0fu) | ((hi2 & 0x03030303u) << 4);
+                const u32 w1 = (lo41 & 0x0f0f0f0fu) | (((hi2 >> 2) & 0x03030303u) << 4);
+                const u32 sword = (f >> 1) ? w1 : w0;
+                const u32 qs[8] = {rq.x, rq.y, rq.z, rq.w, rq2.x, rq2.y, rq2.z, rq2.w};
+                const u32 hm[8] = {rq3.x, rq3.y, rq3.z, rq3.w, rq4.x, rq4.y, rq4.z, rq4.w};
+#pragma unroll
+                for (int t = 0; t < 8; t++) { // cells 4 t .. 4 t + 3: lane t
+                    const int sc = (int)((sword >> (8 * (2 * (f & 1) + (t >> 2)))) & 0xffu) - 32;
+                    const u32 low = (qs[t] >> (2 * f)) & 0x03030303u, high = (hm[t] >> (4 * j + f)) & 0x01010101u;
+                    const u32 v = __builtin_amdgcn_perm(0x03020100u, 0xfffefdfcu, (high << 2) | low); // u - 4
+                    u32 h, lo;
+                    iq_planes_signed(v, sc, h, lo);
+                    put(t, h, lo);
+                }
             }
         }
         if constexpr (!EXACT) { // the row's eight scales as bytes: the thread of sub-blocks 2 wq, 2 wq + 1 writes its two
@@ -968,7 +1072,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, 
     const uint8_t *my_a = a_codes + (wslot + l32) * kIqStride + 16 * kh;
     const bool live = wslot < len; // else none of this wave's slots is real
     const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    constexpr int kAcc = EXACT ? 8 : 1;
+    constexpr int kAcc = EXACT ? G::kLanes : 1;
     v16f acc[kAcc];
 #pragma unroll
     for (int l = 0; l < kAcc; l++)
@@ -990,20 +1094,34 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, 
             dd[4 * q4 + 2] = d4.z;
             dd[4 * q4 + 3] = d4.w;
         }
-        if constexpr (EXACT) {
-            // the fold of the 43s first: accumulator l takes sub-block l's scale on its two sums
-            // (crates/qdot/src/lib.rs:8691-8694); the product of the two small integers is exact in f32
+        if constexpr (EXACT && G::kLanes == 1) {
+            // Q3_K: one integer a super-block, then acc + (dcol d) sum, each operation rounded on its own
+            v16i hs = z, ls = z;
 #pragma unroll
             for (int l = 0; l < 8; l++) {
-                const float bs = bs_t[l * kIqLine + wslot + l32];
+                const v4i b = *reinterpret_cast<const v4i *>(my_a + 32 * l);
+                hs = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i *>(my_h + 32 * l), b, hs, 0, 0, 0);
+                ls = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i *>(my_l + 32 * l), b, ls, 0, 0, 0);
+            }
 #pragma unroll
-                for (int q4 = 0; q4 < 4; q4++) {
-                    const float4 s4 = *reinterpret_cast<const float4 *>(sc_t + l * kIqLine + wrow + 8 * q4 + 4 * kh);
-                    const float sv[4] = {s4.x, s4.y, s4.z, s4.w};
+            for (int v = 0; v < 16; v++)
+                acc[0][v] = __fadd_rn(acc[0][v], __fmul_rn(__fmul_rn(dy, dd[v]), (float)(hs[v] * 256 + ls[v])));
+        } else if constexpr (EXACT) {
+            if constexpr (G::kFold) {
+                // the fold of the offsets first: accumulator l takes sub-block l's scale on its two sums
+                // (crates/qdot/src/lib.rs:8691-8694); the product of the two small integers is exact in f32
 #pragma unroll
-                    for (int k = 0; k < 4; k++) {
-                        const float dmin = -dd[4 * q4 + k] * 43.0f;
-                        acc[l][4 * q4 + k] = fmaf(dmin * dy, sv[k] * bs, acc[l][4 * q4 + k]);
+                for (int l = 0; l < 8; l++) {
+                    const float bs = bs_t[l * kIqLine + wslot + l32];
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        const float4 s4 = *reinterpret_cast<const float4 *>(sc_t + l * kIqLine + wrow + 8 * q4 + 4 * kh);
+                        const float sv[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+                        for (int k = 0; k < 4; k++) {
+                            const float dmin = -dd[4 * q4 + k] * (float)G::kOff;
+                            acc[l][4 * q4 + k] = fmaf(dmin * dy, sv[k] * bs, acc[l][4 * q4 + k]);
+                        }
                     }
                 }
             }
@@ -1013,7 +1131,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, 
                 const v16i hs = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i *>(my_h + 32 * l), b, z, 0, 0, 0);
                 const v16i ls = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i *>(my_l + 32 * l), b, z, 0, 0, 0);
 #pragma unroll
-                for (int v = 0; v < 16; v++) acc[l][v] = fmaf(dd[v] * dy, (float)((hs[v] << 8) + ls[v]), acc[l][v]);
+                for (int v = 0; v < 16; v++) acc[l][v] = fmaf(dd[v] * dy, (float)(hs[v] * 256 + ls[v]), acc[l][v]);
             }
         } else {
             v16i hs = z, ls = z;
@@ -1048,7 +1166,7 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, 
 #pragma unroll
                 for (int k = 0; k < 4; k++) {
                     const int v = 4 * q4 + k;
-                    if constexpr (EXACT) { // the closing sum of the eight lanes (crates/qdot/src/lib.rs:4128 hsum_float_8's order)
+                    if constexpr (EXACT && G::kLanes == 8) { // the closing sum of the eight lanes (crates/qdot/src/lib.rs:4128 hsum_float_8's order)
                         const float t0 = acc[0][v] + acc[4][v], t1 = acc[1][v] + acc[5][v];
                         const float t2 = acc[2][v] + acc[6][v], t3 = acc[3][v] + acc[7][v];
                         r[k] = (t0 + t2) + (t1 + t3);
@@ -1062,7 +1180,10 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq2(const uint8_t *w, int rpe, 
     }
 }
 
-bool gemm_supported(int wtype) { return wtype == BM_Q4K || wtype == BM_Q5K || wtype == BM_Q6K || wtype == BM_IQ2XXS; }
+bool gemm_supported(int wtype) {
+    return wtype == BM_Q4K || wtype == BM_Q5K || wtype == BM_Q6K || wtype == BM_IQ2XXS || wtype == BM_IQ3XXS || wtype == BM_IQ4XS ||
+           wtype == BM_Q3K;
+}
 
 hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int rows_per_expert, int k,
                 const uint8_t *act, const uint32_t *cols, const uint32_t *tiles_dev, const uint32_t *n_tiles, int n_slots,
@@ -1080,7 +1201,7 @@ hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int
                            n_units, (u32)slot_div, (u32)n_slots, y);
         return hipGetLastError();
     };
-    if (wtype == BM_IQ2XXS) {
+    if (bm_takes_q8k(wtype)) {
         auto launch_iq = [&](auto kern, size_t lds) {
             hipError_t e = allow_lds(kern, lds);
             if (e != hipSuccess) return e;
@@ -1090,8 +1211,12 @@ hipError_t gemm(const Launch &L, int wtype, const uint8_t *w, int n_experts, int
                                n_slabs_q, (u32)slot_div, (u32)n_slots, y);
             return hipGetLastError();
         };
-        if (mode != 0) return launch_iq(k_gemm_iq2<false>, gemm_iq2_lds_bytes<false>());
-        return launch_iq(k_gemm_iq2<true>, gemm_iq2_lds_bytes<true>());
+        if (wtype == BM_IQ3XXS) return launch_iq(k_gemm_iq<BM_IQ3XXS, true>, gemm_iq_lds_bytes<BM_IQ3XXS, true>());
+        if (wtype == BM_IQ4XS) return launch_iq(k_gemm_iq<BM_IQ4XS, true>, gemm_iq_lds_bytes<BM_IQ4XS, true>());
+        if (wtype == BM_Q3K) return launch_iq(k_gemm_iq<BM_Q3K, true>, gemm_iq_lds_bytes<BM_Q3K, true>());
+        if (wtype != BM_IQ2XXS) return hipErrorInvalidValue;
+        if (mode != 0) return launch_iq(k_gemm_iq<BM_IQ2XXS, false>, gemm_iq_lds_bytes<BM_IQ2XXS, false>());
+        return launch_iq(k_gemm_iq<BM_IQ2XXS, true>, gemm_iq_lds_bytes<BM_IQ2XXS, true>());
     }
     if (mode == 2 && gemm_half_supported(wtype)) // the f16 form of the tolerance mode, where the type has one
         return gemm_half(L, wtype, w, n_experts, rows_per_expert, k, act, cols, tiles_dev, n_tiles, n_slots, slot_div, y);

@@ -309,7 +309,8 @@ int bm_route_fill(bm_ctx *ctx, const uint32_t *ids_dev, int n_slots, bm_route *r
  * tiles_host (optional) two words a tile: expert, then first index | length << 16. */
 int bm_route_read(bm_ctx *ctx, const bm_route *route, uint32_t *cols_host, uint32_t *tiles_host, int *n_tiles, int *n_refused);
 /* GemmKernels::enqueue_gemm(GemmArgs) (crates/gpu/src/gemm/grouped.rs:2125-2133,2300), Q4_K, Q5_K and Q6_K stacks against
- * Q8_2_X4 columns and IQ2_XXS stacks (crates/gpu/src/gemm/kernels.rs:867 gemm_iq2xxs) against Q8_K columns:
+ * Q8_2_X4 columns and IQ2_XXS, IQ3_XXS, IQ4_XS and Q3_K stacks (crates/gpu/src/gemm/kernels.rs:867 gemm_iq2xxs, :1139
+ * gemm_iq3xxs, :1248 gemm_iq4xs, :759 gemm_q3k) against Q8_K columns:
  * y_dev[s * rows_per_expert + r] = row r of expert e(s) . column c(s) of act for every slot s of the table's last
  * fill; c(s) = s / top_k (GemmInput::Shared) or s when top_k is 0 (GemmInput::PerSlot). rows_per_expert a
  * multiple of 16. Every value is bm_gemv_sel's for that slot, bit for bit; the integer sums are formed on the int8
@@ -321,6 +322,7 @@ int bm_gemm(bm_ctx *ctx, const bm_weights *w, int rows_per_expert, const bm_act 
  *   BM_GEMM_FAST: one accumulator a value, blocks in increasing k; differs from the exact value by f32 rounding
  *     only (observed below 1e-6 of the row's largest magnitude; the contract's tolerance is 1e-4), about 1.9x the
  *     speed of a Q4_K / Q6_K layer step. No counterpart in the reference, whose grouped GEMM has one order (gemm/grouped.rs:33-58).
+ *     IQ3_XXS, IQ4_XS and Q3_K stacks have the exact order only and run in it under every mode.
  *   BM_GEMM_FAST_F16: the tolerance mode with both scales folded into f16 matrix operands (the sub-scale times the 4-bit
  *     code on the weight side, the block scale times the int8 code as an f16 value and its remainder on the column side), so
  *     the matrix cores deliver scaled sums and the vector ALU is left with two multiply-adds a super-block. The same

@@ -19,6 +19,8 @@ PATHS = ((bm.PATH_PER_SLOT, "per slot"), (bm.PATH_GROUPED, "grouped"), (bm.PATH_
     ((bm.Q5_K, bm.Q5_K, bm.Q4_K), 512, 512, 5, 3, 40),
     ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ2_XXS), 1024, 512, 6, 4, 9),  # Q8_K columns on both sides
     ((bm.Q4_K, bm.Q4_K, bm.IQ2_XXS), 512, 768, 4, 2, 33),    # the two column forms in one layer
+    ((bm.IQ4_XS, bm.IQ4_XS, bm.Q3_K), 512, 512, 5, 3, 25),   # the added types through the GEMM path as well
+    ((bm.IQ3_XXS, bm.IQ3_XXS, bm.Q6_K), 768, 256, 4, 2, 18),
 ))
 def test_every_path_gives_the_oracles_bits(gpu, types, hidden, ff, n_experts, top_k, m):
     L = Layer(gpu, types, hidden, ff, n_experts, 5100 + hidden)
@@ -79,13 +81,12 @@ def test_the_automatic_choice_follows_the_crossovers(gpu):
         assert sc.path_for(1) == bm.PATH_GROUPED
     finally:
         sc.free()
-    # a type without a grouped GEMM never takes that path, and says so when asked to
-    sc = gpu.scratch(bm.IQ4_XS, bm.IQ4_XS, 512, 256, 4, 2, 512)
+    # every type has a grouped GEMM: the same cut for a layer of the added types
+    sc = gpu.scratch(bm.IQ4_XS, bm.Q3_K, 512, 256, 4, 2, 512)
     try:
-        assert sc.path_for(500) == bm.PATH_GROUPED
-        with pytest.raises(bm.GpuError) as e:
-            sc.set_path(bm.PATH_GEMM)
-        assert e.value.code == bm.ETYPE
+        assert [sc.path_for(m) for m in (21, 447, 448, 500)] == [bm.PATH_PER_SLOT, bm.PATH_GROUPED, bm.PATH_GEMM, bm.PATH_GEMM]
+        sc.set_path(bm.PATH_GEMM)
+        assert sc.path_for(3) == bm.PATH_GEMM
     finally:
         sc.free()
     for call, word in ((lambda: gpu.scratch(bm.Q4_K, bm.Q6_K, 2048, 768, 128, 8, 5121), "40960"),

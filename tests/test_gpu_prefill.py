@@ -111,6 +111,11 @@ def test_gemm_fast_mode_is_within_the_tolerance(gpu):
     ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ2_XXS), 1024, 512, 5, 60, 3, False),  # Q8_K columns on both sides; runs past one 32-slot half
     ((bm.IQ2_XXS, bm.IQ2_XXS, bm.Q6_K), 768, 256, 3, 11, 2, False),      # the two column forms in one layer
     ((bm.Q4_K, bm.Q4_K, bm.IQ2_XXS), 512, 768, 4, 30, 4, False),
+    ((bm.IQ4_XS, bm.IQ4_XS, bm.IQ4_XS), 768, 512, 4, 50, 3, False),    # the other types on Q8_K columns: the IQ2_XXS kernel's
+    ((bm.IQ3_XXS, bm.IQ3_XXS, bm.IQ3_XXS), 512, 768, 3, 44, 2, False),  # products over their own staging and f32 steps
+    ((bm.Q3_K, bm.Q3_K, bm.Q3_K), 1024, 256, 5, 37, 4, False),
+    ((bm.IQ3_XXS, bm.IQ3_XXS, bm.Q3_K), 768, 768, 3, 20, 3, False),
+    ((bm.Q3_K, bm.Q3_K, bm.IQ4_XS), 512, 512, 6, 70, 2, False),
 ))
 def test_prefill_layer_matches_the_oracle(gpu, types, hidden, ff, n_experts, m, top_k, cheap):
     L = Layer(gpu, types, hidden, ff, n_experts, 2000 + hidden, cheap=cheap)
@@ -139,7 +144,8 @@ def test_gemm_rows_not_a_whole_slab_and_refused_slots(gpu, fast):
     ExpertId. In the tolerance mode the live rows are held to the tolerance instead of to bits."""
     from common import max_abs_normalised
     rng = np.random.default_rng(2100)
-    for wtype, k in ((bm.Q4_K, 1024), (bm.Q5_K, 512), (bm.Q6_K, 768), (bm.IQ2_XXS, 768)):
+    for wtype, k in ((bm.Q4_K, 1024), (bm.Q5_K, 512), (bm.Q6_K, 768), (bm.IQ2_XXS, 768), (bm.IQ3_XXS, 512), (bm.IQ4_XS, 768),
+                     (bm.Q3_K, 1024)):
         rpe, n_experts, n_slots = 80, 4, 23
         w = stack(wtype, n_experts * rpe, k, 2101)
         ids = rng.integers(0, n_experts, n_slots).astype(np.uint32)
@@ -240,7 +246,6 @@ def test_prefill_refusals_are_named(gpu):
         (lambda: gpu.enqueue_gemm(w4, 24, a512, table, 0, buf), bm.ESHAPE, "multiple of 16"),
         (lambda: gpu.enqueue_gemm(w4, 16, a512, table, 0, buf), bm.ESHAPE, "experts"),
         (lambda: gpu.enqueue_gemm(w4, 32, a512, table, 3, buf), bm.ESHAPE, "whole tokens"),
-        (lambda: gpu.enqueue_gemm(wi, 32, aq8k, table, 0, buf), bm.ETYPE, "bm_gemm"),
         (lambda: gpu.enqueue_swiglu_quant(buf, buf, 9, a512), bm.ESHAPE, "n_cols"),
         (lambda: table.fill(ids, 9), bm.ESHAPE, "n_slots"),
         (lambda: gpu.route(50000, 2), bm.ESHAPE, "max_slots"),

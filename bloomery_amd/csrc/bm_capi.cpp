@@ -894,6 +894,11 @@ int bm_scratch_create(bm_ctx *ctx, int gate_type, int down_type, int hidden, int
     //    256      767       296        392          230
     //    512     1491       534        481          289
     s->path = BM_PATH_AUTO, s->grouped_from = 22, s->gemm_from = 448, s->gemm_from_fast = 96;
+    // a gate/up stack on Q8_K columns (Q3_K, IQ2_XXS, IQ3_XXS, IQ4_XS): its tile launchers are bound by the type's decode, which
+    // the GEMM does once a row and super-block for all of a tile's slots, so the exact GEMM is ahead much earlier (same layer
+    // shape, us a step, grouped / GEMM: IQ4_XS 48 tokens 180 / 170, 96 tokens 265 / 185, 2048 tokens 3202 / 907; IQ2_XXS 64
+    // tokens 168 / 196, 96 tokens 230 / 212, 2048 tokens 2682 / 995; IQ3_XXS 96 tokens 241 / 215; Q3_K 24 tokens 112 / 103)
+    if (act_form(gate_type) != 0) s->gemm_from = 96;
     const size_t slots = (size_t)max_tokens * n_slots_per_token;
     int rc = bm_act_create(ctx, gate_type, hidden, max_tokens, &s->act_x);
     if (!rc) rc = bm_act_create(ctx, down_type, ff, (int)slots, &s->act_h);

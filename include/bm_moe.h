@@ -370,7 +370,8 @@ int bm_swiglu_quant_sel(bm_ctx *ctx, const float *g_dev, const float *u_dev, con
  * up to max_tokens tokens (made at load time and shared by every layer of the same shape, as the reference's Q8Act scratch
  * is): max_tokens * n_slots_per_token <= 40960. BM_PATH_AUTO (the default) takes the per-slot path below grouped_from
  * tokens, the grouped path below gemm_from and the GEMM from there; the defaults are the crossovers measured on MI355X at
- * the Qwen3-30B-A3B layer shape: 22 tokens, and 448 tokens in the exact mode of bm_gemm or 96 in its tolerance mode.
+ * the Qwen3-30B-A3B layer shape: 22 tokens, and 448 tokens in the exact mode of bm_gemm or 96 in its tolerance mode (96 in
+ * either mode where the gate/up stack dots against Q8_K columns: Q3_K, IQ2_XXS, IQ3_XXS, IQ4_XS).
  * bm_scratch_set_path sets others (0 keeps a value; gemm_from then holds for both modes) or forces one path.
  * bm_scratch_path_for: the path a call with m tokens takes. A slot whose id names no expert of the stack adds nothing to
  * the sum and raises BM_SITE_EXPERT_ID unless it is BM_HOST_SLOT, which every path skips silently (the GEMM path's route

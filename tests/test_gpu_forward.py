@@ -84,7 +84,8 @@ def test_the_automatic_choice_follows_the_crossovers(gpu):
     # every type has a grouped GEMM: the same cut for a layer of the added types
     sc = gpu.scratch(bm.IQ4_XS, bm.Q3_K, 512, 256, 4, 2, 512)
     try:
-        assert [sc.path_for(m) for m in (21, 447, 448, 500)] == [bm.PATH_PER_SLOT, bm.PATH_GROUPED, bm.PATH_GEMM, bm.PATH_GEMM]
+        # (a gate/up stack on Q8_K columns: the exact GEMM is ahead from 96 tokens)
+        assert [sc.path_for(m) for m in (21, 95, 96, 500)] == [bm.PATH_PER_SLOT, bm.PATH_GROUPED, bm.PATH_GEMM, bm.PATH_GEMM]
         sc.set_path(bm.PATH_GEMM)
         assert sc.path_for(3) == bm.PATH_GEMM
     finally:

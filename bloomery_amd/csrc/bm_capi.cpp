@@ -899,6 +899,12 @@ int bm_scratch_create(bm_ctx *ctx, int gate_type, int down_type, int hidden, int
     // shape, us a step, grouped / GEMM: IQ4_XS 48 tokens 180 / 170, 96 tokens 265 / 185, 2048 tokens 3202 / 907; IQ2_XXS 64
     // tokens 168 / 196, 96 tokens 230 / 212, 2048 tokens 2682 / 995; IQ3_XXS 96 tokens 241 / 215; Q3_K 24 tokens 112 / 103)
     if (act_form(gate_type) != 0) s->gemm_from = 96;
+    // ... and where the down stack is on Q8_K columns too and the experts are large, the grouped step - for few slots an
+    // expert the per-slot gate . up launch and the down tiles, see bm_moe_forward - is ahead of the per-slot step from the first
+    // token: every workgroup of the per-slot down launch encodes all of a token's h rows itself, work that grows with hidden x ff
+    // (DeepSeek-V3 shape, hidden 7168, ff 2048, IQ2_XXS, us a step per slot / grouped: 1 token 61.5 / 57.9, 4 tokens 171 / 147,
+    // 16 tokens 589 / 481; at hidden 2048, ff 768 the per-slot step leads up to 12 tokens: 1 token 16.0 / 23.7)
+    if (act_form(gate_type) != 0 && act_form(down_type) != 0 && (int64_t)hidden * ff >= ((int64_t)1 << 23)) s->grouped_from = 1;
     const size_t slots = (size_t)max_tokens * n_slots_per_token;
     int rc = bm_act_create(ctx, gate_type, hidden, max_tokens, &s->act_x);
     if (!rc) rc = bm_act_create(ctx, down_type, ff, (int)slots, &s->act_h);
@@ -983,6 +989,25 @@ int bm_moe_forward(bm_ctx *ctx, bm_scratch *s, const bm_weights *wg, const bm_we
                              down_q8k ? s->g : nullptr, y_dev);
     case BM_PATH_GROUPED: {
         int rc = bm_tables(ctx, sel_dev, n_slots, n_experts, s->order, s->start, s->tiles);
+        // Few slots an expert (no more slots than experts: nearly every tile is one slot) and h on its way through f32 rows:
+        // the per-slot gate . up launch from the token rows is the faster one there (its one-column walk reads the activation
+        // operands a super-block ahead: 83 against 102 us at the DeepSeek-V3 shape, 4 tokens) and the tile launch the faster down
+        // (54 against 84 us), so the step takes one of each; the down tiles then read their columns in slot order.
+        if (!rc && down_q8k && act_form(s->gate_type) != 0 && n_slots <= n_experts && m <= bmk::kMaxDecodeTokens && per_slot_fits(s)) {
+            bmk::Launch L;
+            rc = launch_under(ctx, what, rule, &L);
+            if (!rc)
+                rc = driver(ctx, what, bmk::gate_up_x(L, wg->wtype, x_dev, wg->dev, wu->dev, n_experts, hidden, ff, sel_dev, spt, m, nullptr,
+                                                      nullptr, s->g));
+            if (!rc) // (a slot without an expert of the stack: its rows of h hold nothing, its column is left alone)
+                rc = driver(ctx, what, bmk::quantize(launch_of(ctx), s->down_type, s->g, n_slots, ff, s->act_h->dev, nullptr, sel_dev,
+                                                     (uint32_t)n_experts));
+            if (!rc)
+                rc = driver(ctx, what, bmk::gemv_tiles(launch_of(ctx), wd->wtype, wd->dev, n_experts, ff, s->act_h->dev, s->order, s->start,
+                                                       s->tiles, n_slots, hidden, s->down, true));
+            if (rc) return rc;
+            break;
+        }
         if (!rc) rc = bm_quantize(ctx, x_dev, m, s->act_x);
         if (!rc && !down_q8k)
             rc = bm_gate_up_tiles(ctx, wg, wu, s->act_x, s->order, s->start, s->tiles, n_slots, ff, spt, rule, nullptr, s->act_h);

@@ -213,10 +213,12 @@ __global__ __launch_bounds__(256) void k_gate_up_tiles(const uint8_t *wg, const 
 
 // crates/gpu/src/kquant/tiles.rs:120-190 GemvTiles: workgroup = tile x 64 rows (a quad a row); entry j + c reads
 // column j + c of act and writes row r of its slot order[j + c]. An entry that names no slot raises ExpertId.
+// by_slot: the columns of act lie in slot order instead (entry j + c reads column order[j + c]): what a per-slot gate . up launch
+// leaves, so a step can take that launch for gate . up and this one for down.
 template <int WT, int U, int NB, int MC, bool PASSES>
 __global__ __launch_bounds__(256) void k_gemv_tiles(const uint8_t *w, u32 n_experts, int nb, const uint8_t *act,
                                                     const u32 *order, const u32 *start, const u32 *tiles, u32 n_slots,
-                                                    u32 cap, int rpe, float *y, int m_lo, u32 *fault, u32 layer) {
+                                                    u32 cap, int rpe, float *y, int m_lo, int by_slot, u32 *fault, u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, q = tid & 3;
     Tile t;
@@ -244,7 +246,13 @@ __global__ __launch_bounds__(256) void k_gemv_tiles(const uint8_t *w, u32 n_expe
             if (tid < mc && s >= n_slots && t.row_block == 0) bm_raise(fault, layer, kSiteExpertId);
             slot_of[tid] = s;
         }
-        stage_bytes(cols, act + (size_t)(t.j + c0) * col_bytes, mc * col_bytes); // the tile's columns lie side by side
+        if (by_slot) {
+            __syncthreads(); // slot_of is written
+            for (int c = 0; c < mc; c++)
+                stage_bytes(cols + (size_t)c * col_bytes, act + (size_t)(slot_of[c] < n_slots ? slot_of[c] : 0) * col_bytes, col_bytes);
+        } else {
+            stage_bytes(cols, act + (size_t)(t.j + c0) * col_bytes, mc * col_bytes); // the tile's columns lie side by side
+        }
         __syncthreads();
         float v[MC];
         row_dot<WT, U, NB, MC>(b, wrow, cols, col_bytes, mc, n, q, tb, v, NoTap{});
@@ -309,7 +317,7 @@ hipError_t gate_up_tiles(const Launch &L, int wtype, const uint8_t *wg, const ui
 
 hipError_t gemv_tiles(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const uint8_t *act,
                       const uint32_t *order, const uint32_t *start, const uint32_t *tiles_dev, int n_slots,
-                      int rows_per_expert, float *y) {
+                      int rows_per_expert, float *y, bool by_slot) {
     const int nb = k / 256, rpe = rows_per_expert;
     const bool split = tile_widths_split(wtype, k), narrow = tiles_mostly_narrow(n_slots, n_experts);
     const u32 cap = (u32)tile_cap(n_slots, n_experts);
@@ -321,7 +329,7 @@ hipError_t gemv_tiles(const Launch &L, int wtype, const uint8_t *w, int n_expert
         hipError_t e = allow_lds(kern, lds);                                                                           \
         if (e != hipSuccess) return e;                                                                                 \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act, order, start,       \
-                           tiles_dev, (u32)n_slots, cap, rpe, y, M_LO, L.fault, L.layer);                              \
+                           tiles_dev, (u32)n_slots, cap, rpe, y, M_LO, by_slot ? 1 : 0, L.fault, L.layer);             \
     }
 #define CALL_BODY                                                                                                      \
     if (split && narrow) BM_TILE_LAUNCH(kTileNarrow, 0, true)                                                          \

@@ -36,7 +36,7 @@ int act_col_bytes(int wtype, int k);
 
 // `live` (optional): a device word holding how many of the m columns to quantize; the rest keep what they held.
 hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, uint8_t *act,
-                    const uint32_t *live = nullptr);
+                    const uint32_t *live = nullptr, const uint32_t *sel = nullptr, uint32_t n_experts = 0);
 
 // Rebuilds the tables of m Q8_2_X4 device columns whose reference bytes were just written by a copy.
 hipError_t q82_tables(const Launch &L, uint8_t *act, int m, int k);
@@ -112,7 +112,7 @@ hipError_t gate_up_tiles(const Launch &L, int wtype, const uint8_t *wg, const ui
                          uint8_t *act_h);
 hipError_t gemv_tiles(const Launch &L, int wtype, const uint8_t *w, int n_experts, int k, const uint8_t *act,
                       const uint32_t *order, const uint32_t *start, const uint32_t *tiles, int n_slots,
-                      int rows_per_expert, float *y);
+                      int rows_per_expert, float *y, bool by_slot = false);
 
 // ------------------------------------------------------------------------------------- prefill (bm_prefill.hip)
 

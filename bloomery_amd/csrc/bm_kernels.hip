@@ -80,11 +80,14 @@ __global__ __launch_bounds__(256) void k_quantize_q82x4(const float *x, int m, i
 }
 
 // x: m columns of k values -> Q8_K columns (crates/qdot/src/lib.rs:1787-1809). One workgroup a 256-value block.
+// sel (optional): column c belongs to slot c; a slot whose id names no expert of the stack (served elsewhere, or refused) keeps
+// its column as it stands and raises nothing here: its rows of x need not hold anything.
 __global__ __launch_bounds__(256) void k_quantize_q8k(const float *x, int m, int k, uint8_t *act, const u32 *live,
-                                                      u32 *fault, u32 layer) {
+                                                      const u32 *sel, u32 n_experts, u32 *fault, u32 layer) {
     const int bpc = k / 256;
     const int col = blockIdx.x / bpc, blk = blockIdx.x % bpc;
     if (live && (u32)col >= *live) return;
+    if (sel && sel[col] >= n_experts) return;
     q8k_block_by_workgroup(x[(size_t)col * k + 256 * blk + threadIdx.x], act + ((size_t)col * bpc + blk) * BM_Q8K_STRIDE, fault, layer);
 }
 
@@ -104,7 +107,9 @@ __global__ __launch_bounds__(256) void k_quantize_q82x4_wide(const float *x, int
 // Columns from which on the wide form is launched (and only for 16-byte aligned rows).
 constexpr long kWideQuantValues = 1 << 18;
 
-hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, uint8_t *act, const uint32_t *live) {
+hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, uint8_t *act, const uint32_t *live,
+                    const uint32_t *sel, uint32_t n_experts) {
+    if (sel && !bm_takes_q8k(wtype)) return hipErrorInvalidValue; // the slot-aware form is the Q8_K quantizer's
     if (!bm_takes_q8k(wtype) && (long)m * k >= kWideQuantValues && ((uintptr_t)x & 15) == 0) {
         const long threads = (long)m * k / 8;
         hipLaunchKernelGGL(k_quantize_q82x4_wide, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, L.stream, x, m, k, act,
@@ -113,7 +118,7 @@ hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, ui
     }
     if (bm_takes_q8k(wtype)) {
         hipLaunchKernelGGL(k_quantize_q8k, dim3((unsigned)(m * (k / 256))), dim3(256), 0, L.stream, x, m, k, act,
-                           live, L.fault, L.layer);
+                           live, sel, n_experts, L.fault, L.layer);
     } else {
         const long blocks = (long)m * (k / 32);
         hipLaunchKernelGGL(k_quantize_q82x4, dim3((unsigned)((blocks + 7) / 8)), dim3(256), 0, L.stream, x, m, k, act,

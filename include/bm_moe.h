@@ -365,13 +365,15 @@ int bm_swiglu_quant_sel(bm_ctx *ctx, const float *g_dev, const float *u_dev, con
  *   BM_PATH_GROUPED   bm_tables, bm_quantize, bm_gate_up_tiles (bm_quantize_ord for a down stack on Q8_K columns),
  *                     bm_gemv_tiles, the slots' sum: an expert's rows are read once for all of its slots;
  *   BM_PATH_GEMM      bm_quantize, bm_route_fill, bm_gemm twice, bm_swiglu_quant_sel, bm_gemm, the slots' sum: the int8 matrix
- *                     cores (in the f32 order bm_set_gemm_mode sets; Q4_K, Q5_K, Q6_K and IQ2_XXS stacks).
+ *                     cores (in the f32 order bm_set_gemm_mode sets; every stack type bm_gemm takes).
  * In the exact mode all three give the same bits in y_dev. bm_scratch holds what the paths need between their launches for
  * up to max_tokens tokens (made at load time and shared by every layer of the same shape, as the reference's Q8Act scratch
  * is): max_tokens * n_slots_per_token <= 40960. BM_PATH_AUTO (the default) takes the per-slot path below grouped_from
  * tokens, the grouped path below gemm_from and the GEMM from there; the defaults are the crossovers measured on MI355X at
  * the Qwen3-30B-A3B layer shape: 22 tokens, and 448 tokens in the exact mode of bm_gemm or 96 in its tolerance mode (96 in
- * either mode where the gate/up stack dots against Q8_K columns: Q3_K, IQ2_XXS, IQ3_XXS, IQ4_XS).
+ * either mode where the gate/up stack dots against Q8_K columns: Q3_K, IQ2_XXS, IQ3_XXS, IQ4_XS; where the down stack does so
+ * too and hidden x ff is 2^23 or more, the grouped path from the first token). On the grouped path a batch with no more slots
+ * than experts whose h crosses in f32 rows takes the per-slot gate . up launch and the tile launch for down.
  * bm_scratch_set_path sets others (0 keeps a value; gemm_from then holds for both modes) or forces one path.
  * bm_scratch_path_for: the path a call with m tokens takes. A slot whose id names no expert of the stack adds nothing to
  * the sum and raises BM_SITE_EXPERT_ID unless it is BM_HOST_SLOT, which every path skips silently (the GEMM path's route

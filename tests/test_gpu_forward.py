@@ -21,6 +21,8 @@ PATHS = ((bm.PATH_PER_SLOT, "per slot"), (bm.PATH_GROUPED, "grouped"), (bm.PATH_
     ((bm.Q4_K, bm.Q4_K, bm.IQ2_XXS), 512, 768, 4, 2, 33),    # the two column forms in one layer
     ((bm.IQ4_XS, bm.IQ4_XS, bm.Q3_K), 512, 512, 5, 3, 25),   # the added types through the GEMM path as well
     ((bm.IQ3_XXS, bm.IQ3_XXS, bm.Q6_K), 768, 256, 4, 2, 18),
+    ((bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ2_XXS), 512, 512, 40, 4, 6),  # no more slots than experts, Q8_K columns on both sides: the
+    ((bm.IQ4_XS, bm.IQ4_XS, bm.Q3_K), 512, 256, 64, 3, 7),       # grouped path's per-slot gate . up launch and slot-ordered down tiles
 ))
 def test_every_path_gives_the_oracles_bits(gpu, types, hidden, ff, n_experts, top_k, m):
     L = Layer(gpu, types, hidden, ff, n_experts, 5100 + hidden)
@@ -96,6 +98,46 @@ def test_the_automatic_choice_follows_the_crossovers(gpu):
         with pytest.raises(bm.GpuError) as e:
             call()
         assert word in str(e.value) and "bm_scratch_create" in str(e.value)
+
+
+def test_a_slot_without_an_expert_on_the_grouped_path_of_few_slots(gpu):
+    """The grouped path with no more slots than experts and Q8_K columns on both sides (the per-slot gate . up launch, the
+    slot-aware quantizer of h, the down tiles reading their columns in slot order): a host-served slot and an id past the stack
+    add nothing, the sums over the live slots are the oracle's, only the id past the stack raises; the scratch is poisoned first so
+    that a stale row of h would show."""
+    hidden, ff, n_experts, top_k, m = 512, 256, 16, 3, 3
+    L = Layer(gpu, (bm.IQ2_XXS, bm.IQ2_XXS, bm.IQ4_XS), hidden, ff, n_experts, 5300)
+    rng = np.random.default_rng(5301)
+    x = normal_f32(rng, (m, hidden))
+    wts = np.array([[0.5, 0.3, 0.2], [0.2, 0.5, 0.3], [0.1, 0.6, 0.3]], np.float32)
+    xd, wd = gpu.upload(x, np.float32), gpu.upload(wts, np.float32)
+    y = gpu.buffer(np.float32, m * hidden)
+    sc = gpu.scratch(bm.IQ2_XXS, bm.IQ4_XS, hidden, ff, n_experts, top_k, 4)
+    sc.set_path(bm.PATH_GROUPED)
+    try:
+        for ids, live, raises in ((np.array([[1, bm.HOST_SLOT, 3], [bm.HOST_SLOT, 0, bm.HOST_SLOT], [0, 2, 15]], np.uint32),
+                                   ([(1, 0.5), (3, 0.2)], [(0, 0.5)], [(0, 0.1), (2, 0.6), (15, 0.3)]), False),
+                                  (np.array([[1, 99, 3], [2, 0, 1], [0, 16, 2]], np.uint32),
+                                   ([(1, 0.5), (3, 0.2)], [(2, 0.2), (0, 0.5), (1, 0.3)], [(0, 0.1), (2, 0.3)]), True)):
+            want = np.concatenate([L.oracle(x[t:t + 1], np.array([[e for e, _ in live[t]]], np.uint32),
+                                            np.array([[w for _, w in live[t]]], np.float32), len(live[t]))[0] for t in range(m)])
+            sel = gpu.upload(ids, np.uint32)
+            gpu.fault_clear()
+            for rep in range(2):
+                y.fill_bytes(0xFF)
+                gpu.enqueue_moe_forward(sc, L.dg, L.du, L.dd, xd, sel, wd, None, m, y)
+                assert_f32(y.download(), want, f"call {rep}")
+            if raises:
+                assert gpu.fault()[1] & (1 << bm.SITE_EXPERT_ID)
+            else:
+                assert gpu.fault() == (bm.FAULT_NONE, 0)
+            sel.free()
+        gpu.fault_clear()
+    finally:
+        sc.free()
+        for b in (xd, wd, y):
+            b.free()
+        L.free()
 
 
 def test_a_slot_without_an_expert_adds_nothing_on_every_path(gpu):

@@ -30,18 +30,26 @@ int gemm_max_tiles(int n_slots, int n_experts) { // crates/gpu/src/gemm/route.rs
 
 // ------------------------------------------------------------------------------------------------ route
 
-// One workgroup: the slots listed by expert in ascending slot order (group_slots), bucket n_experts collecting the
-// refused ones at the list's end; then the tiles, an expert's run cut into runs of at most 64. A slot served elsewhere
-// (id 0xffffffff, crates/gpu/src/kquant/sel.rs:22-28) is not listed and raises nothing: the list is that many entries
-// shorter, the entries past it hold 0xffffffff, and n_tiles[2] counts them.
+// The slots listed by expert in ascending slot order, bucket n_experts collecting the refused ones at the list's end
+// (group_slots_part: as many workgroups as the list has parts, each placing its part; one workgroup on a single compute
+// unit took 23 us over 16384 slots, bound by that unit's instruction rate and by lanes queueing on a popular expert's
+// counter); one workgroup more places nothing and writes the tiles, an expert's run cut into runs of at most 64. A slot served elsewhere (id 0xffffffff, crates/gpu/src/kquant/sel.rs:22-28) is not
+// listed and raises nothing: the list is that many entries shorter, the entries past it hold 0xffffffff, and n_tiles[2]
+// counts them.
+struct RouteLds {
+    GroupLds g;
+    u32 off[kGroupBuckets];
+};
 __global__ __launch_bounds__(kRouteThreads) void k_route(const u32 *ids, u32 n_slots, u32 n_experts, u32 *cols,
                                                          u32 *tiles, u32 *n_tiles, u32 *fault, u32 layer) {
-    __shared__ GroupLds g;
+    __shared__ RouteLds lds;
+    GroupLds &g = lds.g;
     const u32 tid = threadIdx.x;
-    group_slots(g, n_slots, n_experts + 1, cols, [&](u32 s) {
+    group_slots_part(g, lds.off, n_slots, n_experts + 1, blockIdx.x, cols, [&](u32 s) {
         const u32 id = ids[s];
         return id < n_experts ? id : id == 0xffffffffu ? kNoBucket : n_experts;
     });
+    if (blockIdx.x + 1 != gridDim.x) return;
     const u32 listed = g.base[n_experts + 1];
     for (u32 i = listed + tid; i < n_slots; i += kRouteThreads) cols[i] = 0xffffffffu;
     u32 j0 = 0, j1 = 0;
@@ -67,8 +75,8 @@ __global__ __launch_bounds__(kRouteThreads) void k_route(const u32 *ids, u32 n_s
 
 hipError_t route(const Launch &L, const uint32_t *ids, int n_slots, int n_experts, uint32_t *cols, uint32_t *tiles_out,
                  uint32_t *n_tiles) {
-    hipLaunchKernelGGL(k_route, dim3(1), dim3(kRouteThreads), 0, L.stream, ids, (u32)n_slots, (u32)n_experts, cols,
-                       tiles_out, n_tiles, L.fault, L.layer);
+    hipLaunchKernelGGL(k_route, dim3(group_parts((u32)n_slots, (u32)n_experts + 1) + 1), dim3(kRouteThreads), 0, L.stream, ids,
+                       (u32)n_slots, (u32)n_experts, cols, tiles_out, n_tiles, L.fault, L.layer);
     return hipGetLastError();
 }
 

@@ -472,6 +472,18 @@ struct GroupLds {
     u32 scan[17];
 };
 
+// The lanes of the wave whose bucket is this lane's (a lane that is not live: the lanes that are not), read off the
+// ballots of the bucket's bits.
+__device__ __forceinline__ unsigned long long lanes_of_my_bucket(u32 b, bool live, int bits) {
+    const unsigned long long all_live = __ballot(live);
+    unsigned long long same = live ? all_live : ~all_live;
+    for (int k = 0; k < bits; k++) {
+        const unsigned long long set = __ballot(live && ((b >> k) & 1u));
+        same &= (live && ((b >> k) & 1u)) ? set : ~set;
+    }
+    return same;
+}
+
 // bucket_of(s): slot s's bucket below n_buckets, or kNoBucket for a slot that joins no run. Called twice a slot.
 // Every thread of the workgroup calls group_slots; afterwards g.base holds the runs' bounds.
 template <class BucketOf>
@@ -529,6 +541,114 @@ __device__ __forceinline__ void group_slots(GroupLds &g, u32 n, u32 n_buckets, u
             if (live && lane == (u32)leader) first = atomicAdd(&g.hist[wave * n_buckets + b], (u32)__builtin_popcountll(same));
             first = (u32)__shfl((int)first, leader, 64);
             if (live) list[g.base[b] + first + (u32)__builtin_popcountll(same & ((1ull << lane) - 1ull))] = s;
+        }
+    }
+    __syncthreads();
+}
+
+// The same list made by several workgroups of 1024 threads, none waiting for another: the slots are cut into
+// group_parts(n, n_buckets) parts and workgroup `part` places the slots of its part. Every workgroup counts all the slots
+// (light work: two counters a bucket, the ids come from the cache after the first reader), so each knows every run's start
+// and how many of a bucket's slots lie in the parts before its own; it then counts its own part once more, a sub-part a
+// wave, and its waves place their sub-parts as group_slots' waves place their chunks. `off` holds n_buckets words of LDS.
+// Afterwards g.base holds the runs' bounds in every workgroup; a workgroup whose `part` is group_parts(..) or more places
+// nothing and has the bounds sooner than the others are done (for what a caller makes of the bounds alone).
+__host__ __device__ inline u32 group_chunks(u32 n_buckets) {
+    const u32 chunks = (u32)kGroupHist / n_buckets;
+    return chunks < (u32)kGroupWaves ? chunks : (u32)kGroupWaves;
+}
+__host__ __device__ inline u32 group_chunk_len(u32 n, u32 chunks) { return ((n + chunks - 1) / chunks + 63) & ~63u; }
+__host__ __device__ inline u32 group_parts(u32 n, u32 n_buckets) {
+    const u32 per = group_chunk_len(n, group_chunks(n_buckets));
+    return n ? (n + per - 1) / per : 1;
+}
+
+template <class BucketOf>
+__device__ __forceinline__ void group_slots_part(GroupLds &g, u32 *off, u32 n, u32 n_buckets, u32 part, u32 *list,
+                                                 const BucketOf &bucket_of) {
+    const u32 tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const u32 chunks = group_chunks(n_buckets);
+    const u32 per = group_chunk_len(n, chunks);
+    const u32 p_lo = part * per < n ? part * per : n, p_hi = p_lo + per < n ? p_lo + per : n;
+    const int bits = 32 - __builtin_clz(n_buckets | 1u);
+    // All the slots, thread by thread, four loads at a time: a bucket's count in the parts before this one, and its count
+    // from this part on. A lane adds to one of up to 16 copies of the counters, picked by its number, on banks of their
+    // own (an odd stride): with a popular expert a quarter of a wave's lanes would otherwise queue up on one word.
+    const u32 rstride = 2 * n_buckets + 1;
+    u32 reps = 16;
+    while (reps > 1 && reps * rstride > (u32)kGroupHist) reps >>= 1;
+    u32 *mine = g.hist + (lane & (reps - 1)) * rstride;
+    for (u32 i = tid; i < reps * rstride; i += blockDim.x) g.hist[i] = 0;
+    __syncthreads();
+    for (u32 s0 = tid; s0 < n; s0 += 4 * blockDim.x) {
+        u32 b[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const u32 s = s0 + (u32)j * blockDim.x;
+            b[j] = s < n ? bucket_of(s) : kNoBucket;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (b[j] != kNoBucket) atomicAdd(&mine[(s0 + (u32)j * blockDim.x < p_lo ? 0u : n_buckets) + b[j]], 1u);
+    }
+    __syncthreads();
+    u32 count = 0;
+    for (u32 b = tid; b < n_buckets; b += blockDim.x) {
+        u32 bef = 0, aft = 0;
+        for (u32 r = 0; r < reps; r++) {
+            bef += g.hist[r * rstride + b];
+            aft += g.hist[r * rstride + n_buckets + b];
+        }
+        off[b] = bef;
+        if (b < 1024) count = bef + aft;
+        else g.base[kGroupBuckets] = bef + aft; // bucket 1024's count, parked
+    }
+    u32 total;
+    const u32 at = block_scan_1024(count, g.scan, &total);
+    if (tid < n_buckets) g.base[tid] = at;
+    if (tid == 0) {
+        if (n_buckets == (u32)kGroupBuckets) {
+            const u32 last = g.base[kGroupBuckets];
+            g.base[1024] = total;
+            g.base[kGroupBuckets] = total + last;
+        } else {
+            g.base[n_buckets] = total;
+        }
+    }
+    for (u32 i = tid; i < chunks * n_buckets; i += blockDim.x) g.hist[i] = 0; // (its readers passed the scan's barriers)
+    __syncthreads();
+    if (p_lo >= n) return; // a workgroup past the last part: the bounds only
+    // this part once more, a sub-part a wave
+    const u32 sub = group_chunk_len(p_hi - p_lo, chunks);
+    const u32 lo = p_lo + wave * sub < p_hi ? p_lo + wave * sub : p_hi, hi = lo + sub < p_hi ? lo + sub : p_hi;
+    if (wave < chunks)
+        for (u32 s0 = lo; s0 < hi; s0 += 64) {
+            const u32 s = s0 + lane;
+            const u32 b = s < hi ? bucket_of(s) : kNoBucket;
+            const unsigned long long same = lanes_of_my_bucket(b, b != kNoBucket, bits);
+            if (b != kNoBucket && lane == (u32)__builtin_ctzll(same)) atomicAdd(&g.hist[wave * n_buckets + b], (u32)__builtin_popcountll(same));
+        }
+    __syncthreads();
+    for (u32 b = tid; b < n_buckets; b += blockDim.x) { // a sub-part's count -> its first place in the list
+        u32 sum = g.base[b] + off[b];
+        for (u32 c = 0; c < chunks; c++) {
+            const u32 v = g.hist[c * n_buckets + b];
+            g.hist[c * n_buckets + b] = sum;
+            sum += v;
+        }
+    }
+    __syncthreads();
+    if (wave < chunks) {
+        for (u32 s0 = lo; s0 < hi; s0 += 64) {
+            const u32 s = s0 + lane;
+            const u32 b = s < hi ? bucket_of(s) : kNoBucket;
+            const bool live = b != kNoBucket;
+            const unsigned long long same = lanes_of_my_bucket(b, live, bits);
+            const int leader = live ? __builtin_ctzll(same) : (int)lane;
+            u32 first = 0;
+            if (live && lane == (u32)leader) first = atomicAdd(&g.hist[wave * n_buckets + b], (u32)__builtin_popcountll(same));
+            first = (u32)__shfl((int)first, leader, 64);
+            if (live) list[first + (u32)__builtin_popcountll(same & ((1ull << lane) - 1ull))] = s;
         }
     }
     __syncthreads();

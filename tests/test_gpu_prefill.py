@@ -35,6 +35,43 @@ def test_route_table_is_the_definition(gpu, n_experts, n_slots, seed):
     ids_d.free()
 
 
+@pytest.mark.parametrize("n_experts,n_slots,seed", ((128, 40960, 11), (256, 16385, 12), (1024, 40960, 13), (511, 33000, 14),
+                                                    (512, 2049, 15), (600, 8191, 16), (5, 129, 17)))
+def test_route_table_made_by_several_workgroups(gpu, n_experts, n_slots, seed):
+    """Lists long enough for several workgroups (each places a part of the slots), with host-served slots and refused ids
+    among them, against the definition spelt with a stable sort: the live slots by expert, ascending inside an expert, then
+    the refused ones ascending, then 0xffffffff for as many entries as slots are served elsewhere; tiles of at most 64."""
+    rng = np.random.default_rng(seed)
+    p = 1.0 / np.arange(1, n_experts + 1) ** 1.1
+    ids = rng.permutation(n_experts)[rng.choice(n_experts, n_slots, p=p / p.sum())].astype(np.uint32)
+    odd = rng.random(n_slots)
+    ids[odd < 0.02] = bm.HOST_SLOT
+    ids[(odd >= 0.02) & (odd < 0.03)] = n_experts + rng.integers(0, 1000, int(((odd >= 0.02) & (odd < 0.03)).sum()))
+    live = np.flatnonzero(ids < n_experts)
+    refused = np.flatnonzero((ids >= n_experts) & (ids != bm.HOST_SLOT))
+    listed = live[np.argsort(ids[live], kind="stable")]
+    want_cols = np.concatenate([listed, refused, np.full(n_slots - listed.size - refused.size, 0xFFFFFFFF)]).astype(np.uint32)
+    counts = np.bincount(ids[live], minlength=n_experts)
+    want_tiles, at = [], 0
+    for e in range(n_experts):
+        for j in range(0, int(counts[e]), 64):
+            want_tiles.append((e, at + j, min(64, int(counts[e]) - j)))
+        at += int(counts[e])
+    gpu.fault_clear()
+    table = gpu.route(n_slots, n_experts)
+    ids_d = gpu.upload(ids, np.uint32)
+    for rep in range(2):  # the second fill over the first one's table
+        table.fill(ids_d, n_slots)
+        cols, tiles, n_refused = table.read()
+        assert n_refused == refused.size
+        assert np.array_equal(cols, want_cols)
+        assert np.array_equal(tiles, np.asarray(want_tiles, np.uint32).reshape(-1, 3))
+    assert (gpu.fault()[1] & (1 << bm.SITE_EXPERT_ID)) != 0 if refused.size else gpu.fault() == (bm.FAULT_NONE, 0)
+    gpu.fault_clear()
+    table.free()
+    ids_d.free()
+
+
 def run_prefill(gpu, L, x, ids, wts, top_k):
     """quantize -> route -> gate GEMM, up GEMM (Shared) -> swiglu_quant -> down GEMM (PerSlot) -> combine
     (crates/gpu/src/arch/qwen3moe/wide.rs:1171-1225)."""

@@ -840,7 +840,9 @@ def read_patterns(bm, gpu, layers, sel, n_tok):
     for name, pattern, threads, ahead in (("quad_a_row_4_ahead_192x256_as_k_gate_up_x", 0, 256, 4), ("quad_a_row_8_ahead_192x256", 0, 256, 8),
                                           ("quad_a_row_4_ahead_256x192", 0, 192, 4), ("quad_a_row_8_ahead_256x192", 0, 192, 8),
                                           ("octet_a_row_pair_192x256", 1, 256, 8), ("octet_a_row_pair_256x192", 1, 192, 8),
-                                          ("workgroup_contiguous_192x256", 2, 256, 8), ("workgroup_contiguous_256x192", 2, 192, 8)):
+                                          ("workgroup_contiguous_192x256", 2, 256, 8), ("workgroup_contiguous_256x192", 2, 192, 8),
+                                          ("into_lds_nine_lanes_a_row_super_block_192x256", 3, 256, 8),
+                                          ("into_lds_wave_rows_contiguous_192x256", 4, 256, 8)):
         def enqueue(i):
             dg, du, _ = layers[i % len(layers)]
             rc = probe.bm_bench_probe_gate_up_rows(stream, dg.dev_ptr, du.dev_ptr, sel.ptr + 4 * TOP_K * (i % n_tok), FF, pattern, threads,

@@ -92,6 +92,12 @@ __global__ __launch_bounds__(256) void k_probe_handoff(uint32_t gen, int load, c
 //   pattern 1: eight lanes a row pair: lane k the 16 code bytes at 16 + 16 k of the gate row's and of the up row's super-block
 //              and the two 16-byte headers (four requests a super-block, every one of a row 16-byte contiguous over the octet);
 //   pattern 2: the workgroup's rows of each matrix are contiguous in memory: plain 16-byte loads over them, thread by thread.
+//   pattern 3: loads that land in LDS (global_load_lds_dwordx4: no register holds them, any lane may ask for any piece): a wave
+//              takes its own 8 row pairs, super-block by super-block, nine lanes a (row, super-block)'s 144 contiguous bytes,
+//              all asked for up front; the bytes are then read back from LDS;
+//   pattern 4: the same loads over the wave's rows as they lie (8 gate rows, then 8 up rows: 9 KB contiguous each).
+typedef __attribute__((address_space(1))) const void probe_gptr;
+typedef __attribute__((address_space(3))) void probe_lptr;
 template <int T, int PATTERN, int AHEAD>
 __global__ __launch_bounds__(T) void k_probe_gate_up_rows(const uint8_t *wg, const uint8_t *wu, const uint32_t *sel, int ff,
                                                           uint32_t *sink) {
@@ -133,6 +139,45 @@ __global__ __launch_bounds__(T) void k_probe_gate_up_rows(const uint8_t *wg, con
         for (int i = 0; i < 8; i++) {
             acc.x ^= qg[i].x ^ qu[i].x ^ hg[i].x ^ hu[i].x, acc.y ^= qg[i].y ^ qu[i].y ^ hg[i].y ^ hu[i].y;
             acc.z ^= qg[i].z ^ qu[i].z ^ hg[i].z ^ hu[i].z, acc.w ^= qg[i].w ^ qu[i].w ^ hg[i].w ^ hu[i].w;
+        }
+    } else if constexpr (PATTERN == 3 || PATTERN == 4) {
+        static_assert(T == 256, "four waves of 8 row pairs");
+        extern __shared__ __align__(16) uint8_t lds[];
+        const int lane = tid & 63, wave = tid >> 6;
+        uint8_t *mine = lds + wave * 24576; // 16 rows of 1152 bytes (pattern 3: 24 requests of 1 KB)
+        const size_t row0 = ((size_t)id * ff + rb * RP + 8 * wave) * 1152;
+        if constexpr (PATTERN == 3) {
+            // piece P = 64 j + lane of a super-block's 144: row P / 9 of the wave's 16 (8 gate, 8 up), part P % 9
+            const uint8_t *src[3];
+#pragma unroll
+            for (int j = 0; j < 3; j++) {
+                int pc = 64 * j + lane;
+                pc = pc < 144 ? pc : 143;
+                const int r16 = pc / 9, part = pc % 9;
+                src[j] = (r16 < 8 ? wg : wu) + row0 + (size_t)(r16 & 7) * 1152 + 16 * part;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+#pragma unroll
+                for (int j = 0; j < 3; j++)
+                    __builtin_amdgcn_global_load_lds((probe_gptr *)(src[j] + 144 * i), (probe_lptr *)(mine + (3 * i + j) * 1024), 16, 0, 0);
+            __builtin_amdgcn_s_waitcnt(0);
+#pragma unroll
+            for (int k = 0; k < 24; k++) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(mine + k * 1024 + 16 * lane);
+                acc.x ^= v.x, acc.y ^= v.y, acc.z ^= v.z, acc.w ^= v.w;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 18; k++)
+                __builtin_amdgcn_global_load_lds((probe_gptr *)((k < 9 ? wg : wu) + row0 + (size_t)(k % 9) * 1024 + 16 * lane),
+                                                 (probe_lptr *)(mine + k * 1024), 16, 0, 0);
+            __builtin_amdgcn_s_waitcnt(0);
+#pragma unroll
+            for (int k = 0; k < 18; k++) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(mine + k * 1024 + 16 * lane);
+                acc.x ^= v.x, acc.y ^= v.y, acc.z ^= v.z, acc.w ^= v.w;
+            }
         }
     } else {
         constexpr int N16 = RP * 1152 / 16, PER = (2 * N16 + T - 1) / T;
@@ -192,8 +237,8 @@ __global__ __launch_bounds__(256) void k_probe_down_rows(const uint8_t *w, const
 
 } // namespace
 
-// Enqueues a gate . up read pattern over 8 slots of sel_dev: pattern 0 .. 2 as above, threads 256 or 192 a workgroup (ff a
-// multiple of threads / 8), ahead 4 or 8 (pattern 0 only). Returns 0, -1 for a refused argument, or the HIP error.
+// Enqueues a gate . up read pattern over 8 slots of sel_dev: pattern 0 .. 4 as above, threads 256 or 192 a workgroup (ff a
+// multiple of threads / 8; patterns 3 and 4: 256), ahead 4 or 8 (pattern 0 only). Returns 0, -1 for a refused argument, or the HIP error.
 extern "C" int bm_bench_probe_gate_up_rows(void *hip_stream, const void *wg_dev, const void *wu_dev, const uint32_t *sel_dev, int ff,
                                            int pattern, int threads, int ahead, uint32_t *sink_dev) {
     if (!wg_dev || !wu_dev || !sel_dev || !sink_dev || ff < 1) return -1;
@@ -210,7 +255,15 @@ extern "C" int bm_bench_probe_gate_up_rows(void *hip_stream, const void *wg_dev,
     else if (pattern == 1 && threads == 192) BM_PROBE_ROWS(192, 1, 8);
     else if (pattern == 2 && threads == 256) BM_PROBE_ROWS(256, 2, 8);
     else if (pattern == 2 && threads == 192) BM_PROBE_ROWS(192, 2, 8);
-    else return -1;
+    else if ((pattern == 3 || pattern == 4) && threads == 256) {
+        constexpr int kLds = 4 * 24 * 1024; // a wave: 24 KB (pattern 3 leaves the third request of a super-block a quarter full)
+        auto k3 = k_probe_gate_up_rows<256, 3, 8>;
+        auto k4 = k_probe_gate_up_rows<256, 4, 8>;
+        auto kern = pattern == 3 ? k3 : k4;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+        if (e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL(kern, grid, dim3(256), kLds, s, g, u, sel_dev, ff, sink_dev);
+    } else return -1;
 #undef BM_PROBE_ROWS
     return (int)hipGetLastError();
 }

@@ -773,13 +773,15 @@ def timeline(args, bm, gpu, enqueue_step, type_names):
     assert rc == 0, f"bm_router_timeline_read: {rc}"
     rt = rt.reshape(1024, 8).astype(np.int64)
     n_r = int(np.count_nonzero(rt[:, 0]))
-    rt = rt[:n_r]
-    r0 = rt[:, 0].min()
+    rt, wave = rt[:n_r - 1], rt[n_r - 1]  # the logits' workgroups, and behind them in the grid the token's routing workgroup
+    r0 = min(rt[:, 0].min(), wave[0])
     out["k_norm_route"] = {"unit": "us after the launch's first workgroup started", "workgroups": n_r,
                            **{name: {"min": round(float((rt[:, i].min() - r0) / 100.0), 2), "median": round(float(np.median(rt[:, i] - r0) / 100.0), 2),
                                      "max": round(float((rt[:, i].max() - r0) / 100.0), 2)}
                               for i, name in enumerate(("start", "token_row_arrived", "normed", "rows_and_token_in_lds", "dots_done"))},
-                           "routed_by_the_last_workgroup": round(float((rt[:, 5].max() - r0) / 100.0), 2)}
+                           "routing_wave": {"start": round(float((wave[0] - r0) / 100.0), 2),
+                                            "holds_every_logit": round(float((wave[4] - r0) / 100.0), 2),
+                                            "routed": round(float((wave[5] - r0) / 100.0), 2)}}
     print(json.dumps(out, indent=1), flush=True)
     gpu.close()
 

@@ -13,13 +13,16 @@
 #include "../../include/bm_moe.h"
 #include "bm_kernels.h"
 
+// bm_norm_route's hand-over words: one a (token, expert) of the largest launch it takes
+static constexpr size_t kRouteHandWords = (size_t)bmk::kNormRouteMaxTokens * bmk::kRouteMaxExperts;
+
 struct bm_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
     bool own_stream = false;
     uint32_t *fault = nullptr;
     uint32_t layer = BM_LAYER_NONE;
-    uint32_t *route_counts = nullptr; // bm_norm_route's finished-workgroup counts, a word a token, zero between launches
+    uint32_t *route_hand = nullptr; // bm_norm_route's hand-over words, one a (token, expert), bmk::kRouteArmed between launches
     int gemm_mode = BM_GEMM_EXACT;
     int down_form = BM_DOWN_RING;
     bmk::GateRule rule = {0u, 0.0f}; // silu(g) * u
@@ -115,14 +118,13 @@ static int ctx_make(int device, hipStream_t stream, bool own, bm_ctx **out) {
         if (e == hipSuccess) e = hipMemset(c->fault, 0xff, sizeof(uint32_t));
     }
     if (e == hipSuccess) {
-        const size_t cb = sizeof(uint32_t) * bmk::kNormRouteMaxTokens;
-        e = hipMalloc((void **)&c->route_counts, cb);
-        if (e == hipSuccess) e = hipMemset(c->route_counts, 0, cb);
+        e = hipMalloc((void **)&c->route_hand, sizeof(uint32_t) * kRouteHandWords);
+        if (e == hipSuccess) e = hipMemsetD32(reinterpret_cast<hipDeviceptr_t>(c->route_hand), (int)bmk::kRouteArmed, kRouteHandWords);
     }
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
         if (c->fault) (void)hipFree(c->fault);
-        if (c->route_counts) (void)hipFree(c->route_counts);
+        if (c->route_hand) (void)hipFree(c->route_hand);
         if (c->own_stream) (void)hipStreamDestroy(c->stream);
         delete c;
         return fail(nullptr, BM_EDRIVER, "bm_ctx_create: fault word: %s", hipGetErrorString(e));
@@ -142,7 +144,7 @@ void bm_ctx_destroy(bm_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipFree(ctx->fault);
-    (void)hipFree(ctx->route_counts);
+    (void)hipFree(ctx->route_hand);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -186,8 +188,8 @@ int bm_fault_clear(bm_ctx *ctx) {
     bmk::Launch L = launch_of(ctx);
     hipError_t e = bmk::fill_u32(L, ctx->fault + 1, 0u, BM_FAULT_WORDS - 1);
     if (e == hipSuccess) e = bmk::fill_u32(L, ctx->fault, BM_FAULT_NONE, 1);
-    // a launch that did not run to its end may have left its counts behind
-    if (e == hipSuccess) e = bmk::fill_u32(L, ctx->route_counts, 0u, bmk::kNormRouteMaxTokens);
+    // a launch that did not run to its end may have left words of its hand-over behind
+    if (e == hipSuccess) e = bmk::fill_u32(L, ctx->route_hand, bmk::kRouteArmed, kRouteHandWords);
     return driver(ctx, "bm_fault_clear", e);
 }
 
@@ -1190,7 +1192,7 @@ int bm_norm_route(bm_ctx *ctx, const float *router_dev, const float *x_dev, cons
         return fail(ctx, BM_ESHAPE, "%s: act_x must hold %d columns of k = %d; it holds %d of k = %d", what, n_tokens, hidden, act_x->m_cap,
                     act_x->k);
     return driver(ctx, what, bmk::norm_route(launch_of(ctx), router_dev, x_dev, gain_dev, eps, n_tokens, n_experts, hidden, normed_dev,
-                                             logits_dev, top_k, renorm != 0, probs_dev, ids_dev, weights_dev, ctx->route_counts,
+                                             logits_dev, top_k, renorm != 0, probs_dev, ids_dev, weights_dev, ctx->route_hand,
                                              act_x ? act_x->dev : nullptr, act_x && act_form(act_x->wtype) != 0));
 }
 

@@ -151,13 +151,15 @@ hipError_t route_softmax(const Launch &L, const float *logits, int n_tok, int n_
 // The FFN norm (gain NULL: none) and the router's f32 logits: router[n_exp * hidden], x[m * hidden], logits[m * n_exp],
 // normed_out (optional) [m * hidden]. hidden a multiple of 8.
 bool router_logits_fits(int hidden);
-// router_logits and route_softmax as one launch: the last of a token's workgroups to finish routes it. counts: a zeroed
-// word a token, left zeroed; launches that share them must not overlap.
+// router_logits and route_softmax as one launch: a token's logits reach its routing wave through `hand`, a word a (token,
+// expert) of the launch (m * n_exp of them) that holds kRouteArmed between launches (left so); launches that share it must
+// not overlap. kRouteArmed is a signalling NaN's pattern: no logit has it, arithmetic only ever leaves the quiet form.
 constexpr int kNormRouteMaxTokens = 4096;
+constexpr uint32_t kRouteArmed = 0x7fa00001u;
 // act_x (optional; hidden a multiple of 256): the tokens' normed rows as quantized columns (q8k: Q8_K, else Q8_2_X4 with tables)
 hipError_t norm_route(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                       int hidden, float *normed_out, float *logits, int used, int renorm, float *probs, uint32_t *ids,
-                      float *weights, uint32_t *counts, uint8_t *act_x = nullptr, bool q8k = false);
+                      float *weights, uint32_t *hand, uint8_t *act_x = nullptr, bool q8k = false);
 hipError_t router_logits(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                          int hidden, float *normed_out, float *logits);
 

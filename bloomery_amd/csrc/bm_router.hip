@@ -54,20 +54,14 @@ __device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
 
 // Token t's routing by one wave; lane L owns experts L + 64 j, j < PER. COH: the logits were stored by other workgroups of
 // this launch with device-scope stores and are read with device-scope loads (no cache of this compute unit's own is asked).
-template <int PER, bool COH = false>
-__device__ __forceinline__ void route_softmax_wave(const float *logits, u32 t, u32 n_exp, u32 used, u32 renorm, float *probs,
+// `v`: this lane's logits, expert lane + 64 j in v[j] (-inf past n_exp).
+template <int PER>
+__device__ __forceinline__ void route_softmax_wave(const float (&v)[PER], u32 t, u32 n_exp, u32 used, u32 renorm, float *probs,
                                                    u32 *ids, float *weights, u32 *fault, u32 layer) {
     const u32 lane = threadIdx.x & 63;
-    const float *row = logits + (size_t)t * n_exp;
-    float v[PER];
     bool odd = false;
 #pragma unroll
-    for (int j = 0; j < PER; j++) {
-        const u32 e = lane + 64 * j;
-        if constexpr (COH) v[j] = e < n_exp ? __hip_atomic_load(row + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
-        else v[j] = e < n_exp ? row[e] : -INFINITY;
-        odd |= e < n_exp && !(fabsf(v[j]) <= 3.402823466e38f);
-    }
+    for (int j = 0; j < PER; j++) odd |= lane + 64 * j < n_exp && !(fabsf(v[j]) <= 3.402823466e38f);
     if (__ballot(odd) != 0) {
         const float nan = bm_bits_f32(0x7fc00000u);
         if (probs) {
@@ -142,7 +136,13 @@ __global__ __launch_bounds__(256) void k_route_softmax(const float *logits, u32 
                                                        float *probs, u32 *ids, float *weights, u32 *fault, u32 layer) {
     const u32 t = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= n_tok) return; // whole waves leave
-    route_softmax_wave<PER>(logits, t, n_exp, used, renorm, probs, ids, weights, fault, layer);
+    float v[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const u32 e = (threadIdx.x & 63) + 64 * j;
+        v[j] = e < n_exp ? logits[(size_t)t * n_exp + e] : -INFINITY;
+    }
+    route_softmax_wave<PER>(v, t, n_exp, used, renorm, probs, ids, weights, fault, layer);
 }
 
 hipError_t route_softmax(const Launch &L, const float *logits, int n_tok, int n_exp, int used, int renorm, float *probs,
@@ -180,7 +180,8 @@ __host__ __device__ inline int router_line(int hidden) { return ((hidden / 8 + 3
 // (k_norm_route's quantizer workgroups): no router rows, no logits.
 template <int R, bool COH = false>
 __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *router, const float *x, const float *gain, float eps,
-                                                   int n_exp, int hidden, float *normed_out, float *logits, int t, int e0) {
+                                                   int n_exp, int hidden, float *normed_out, float *logits, int t, int e0,
+                                                   [[maybe_unused]] u32 *hand = nullptr) {
     // The token's row and the R router rows lie accumulator-major in LDS: value k at line k % 8, place k / 8, so that the
     // lane that owns accumulator l reads four consecutive steps' operands as 16 bytes. A line is hidden / 8 floats, rounded up
     // to whole 16 bytes, + 8 (the eight lines of a row 8 banks apart), a router row four floats past the one before (rows r
@@ -351,8 +352,9 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
         const float out = __fadd_rn(pair, __shfl_down(pair, 1, 8));
         BM_RTICK(tl_dots, out);
         if (l == 0 && e0 + r < n_exp) {
-            if constexpr (COH) __hip_atomic_store(logits + (size_t)t * n_exp + e0 + r, out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            else logits[(size_t)t * n_exp + e0 + r] = out;
+            logits[(size_t)t * n_exp + e0 + r] = out;
+            // k_norm_route's hand-over: the logit as a device-scope store of its own, into a word that held the armed pattern
+            if constexpr (COH) __hip_atomic_store(hand + (size_t)t * n_exp + e0 + r, bm_f32_bits(out), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     BM_RTOCK(0, tl_start);
@@ -372,25 +374,66 @@ __global__ __launch_bounds__(256) void k_router_logits(const float *router, cons
 }
 
 // Norm, logits and routing in one launch (crates/gpu/src/route_softmax.rs:1667-1674 enqueue_norm_fused; the quantizer of
-// that launch is an option here, see below). The workgroups are k_router_logits's; each stores its logits with device-scope
-// stores, waits for their acknowledgement and adds one to the token's count, and the workgroup that brings the count to the
-// number of the token's workgroups - the last to finish, whichever it is - reads the token's logits back with device-scope
-// loads and routes it with its first wave, k_route_softmax's numbers. No workgroup waits for another: every one runs to its end whatever the
-// order they are dispatched in. The last one leaves the count at zero for the next launch, so a graph replay needs no
-// memset. Launches over the same counts must not overlap.
-// With act_x (the reference launch's quantizer, route_softmax.rs:1679): one more workgroup a token, behind the others in the
-// grid, norms the token's row the same way and leaves it as the token's quantized column (q8k: a Q8_K column, else a Q8_2_X4
-// one with its tables), the bytes bm_quantize makes of normed_out. It takes part in no count, so the routing waits for none of it.
+// that launch is an option here, see below). The workgroups are k_router_logits's, and behind them in the grid one more a
+// token, whose first wave routes it with k_route_softmax's numbers. The hand-over is one trip through memory: `hand` holds a
+// word a (token, expert) that is armed between launches - kRouteArmed, a signalling NaN pattern, which no arithmetic
+// leaves behind (an operation on it gives the quiet form) - each logit is stored over its word with a device-scope store as
+// soon as it is formed, and the routing wave reads its words with device-scope loads until none is armed, so it has the
+// logits the moment the last one lands: no acknowledgement is waited for, no count is kept, nothing is read back (the form
+// before, a count raised behind acknowledged stores by the last workgroup to finish, which then read the logits back: 10.3
+// us a token against this one's figure in the bench line). The wave arms its words again before it ends, so a graph replay
+// needs no memset. A routing workgroup comes after every workgroup it waits for in the grid, so those are dispatched
+// whatever else the card runs; the wait is bounded all the same (kRouteSpins polls, then BM_SITE_ROUTER and NaN weights), and
+// every wave ends. Launches over the same `hand` must not overlap.
+// With act_x (the reference launch's quantizer, route_softmax.rs:1679): one more workgroup a token, between the two kinds in
+// the grid, norms the token's row the same way and leaves it as the token's quantized column (q8k: a Q8_K column, else a
+// Q8_2_X4 one with its tables), the bytes bm_quantize makes of normed_out. The routing waits for none of it.
+constexpr u32 kRouteSpins = 1u << 20;
 template <int R, int PER>
 __global__ __launch_bounds__(256) void k_norm_route(const float *router, const float *x, const float *gain, float eps, int n_exp,
                                                     int hidden, float *normed_out, float *logits, u32 used, u32 renorm,
-                                                    float *probs, u32 *ids, float *weights, u32 *counts, uint8_t *act_x,
+                                                    float *probs, u32 *ids, float *weights, u32 *hand, uint8_t *act_x,
                                                     int q8k, int m, u32 *fault, u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
-    __shared__ u32 s_last;
     const u32 blocks_per_token = (u32)((n_exp + R - 1) / R);
-    if (blockIdx.x >= (u32)m * blocks_per_token) { // a quantizer workgroup
-        const int tq = (int)(blockIdx.x - (u32)m * blocks_per_token);
+    const u32 n_logit_blocks = (u32)m * blocks_per_token, n_quant_blocks = act_x ? (u32)m : 0u;
+    if (blockIdx.x >= n_logit_blocks + n_quant_blocks) { // a routing workgroup: its first wave
+        if (threadIdx.x >= 64) return;
+        const u32 t = blockIdx.x - n_logit_blocks - n_quant_blocks, lane = threadIdx.x;
+        u32 *mine = hand + (size_t)t * n_exp;
+        [[maybe_unused]] unsigned long long tl_start = 0, tl_seen = 0;
+        BM_RTICK(tl_start, lane);
+        u32 w[PER];
+        bool late = true;
+        for (u32 spin = 0; spin < kRouteSpins && late; spin++) {
+            bool armed = false;
+#pragma unroll
+            for (int j = 0; j < PER; j++) {
+                const u32 e = lane + 64 * j;
+                w[j] = e < (u32)n_exp ? __hip_atomic_load(mine + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+                armed |= w[j] == kRouteArmed;
+            }
+            late = __ballot(armed) != 0;
+        }
+        BM_RTICK(tl_seen, w[0]);
+        BM_RTOCK(0, tl_start);
+        BM_RTOCK(4, tl_seen);
+        float v[PER];
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const u32 e = lane + 64 * j;
+            // (a word still armed after the last poll: the NaN it is, which the routing refuses as it refuses any)
+            v[j] = e < (u32)n_exp ? bm_bits_f32(w[j]) : -INFINITY;
+            if (e < (u32)n_exp) __hip_atomic_store(mine + e, kRouteArmed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        route_softmax_wave<PER>(v, t, (u32)n_exp, used, renorm, probs, ids, weights, fault, layer);
+        [[maybe_unused]] unsigned long long tl_routed = 0;
+        BM_RTICK(tl_routed, threadIdx.x);
+        BM_RTOCK(5, tl_routed);
+        return;
+    }
+    if (blockIdx.x >= n_logit_blocks) { // a quantizer workgroup
+        const int tq = (int)(blockIdx.x - n_logit_blocks);
         router_logits_body<R>(lds, router, x, gain, eps, n_exp, hidden, nullptr, nullptr, tq, -1);
         const int line = router_line(hidden), nb = hidden / 256, tid = threadIdx.x;
         const float *xs = reinterpret_cast<const float *>(lds); // value k at line k % 8, place k / 8
@@ -413,23 +456,8 @@ __global__ __launch_bounds__(256) void k_norm_route(const float *router, const f
         return;
     }
     const u32 t = blockIdx.x / blocks_per_token;
-    router_logits_body<R, true>(lds, router, x, gain, eps, n_exp, hidden, normed_out, logits, (int)t, (int)(blockIdx.x % blocks_per_token) * R);
-    if (threadIdx.x == 0) {
-        // the workgroup's logits were stored by this wave with device-scope stores: once they are acknowledged they are where
-        // a device-scope load of any compute unit finds them, and only then is the count raised (no cache is written back or
-        // dropped as a whole, which an acquire/release pair at this scope does and which cost more than the routing itself)
-        __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        const u32 before = __hip_atomic_fetch_add(&counts[t], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = before == blocks_per_token - 1;
-        if (s_last) __hip_atomic_store(&counts[t], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (!s_last || threadIdx.x >= 64) return;
-    __asm__ volatile("" ::: "memory"); // the loads below stay behind the count
-    route_softmax_wave<PER, true>(logits, t, (u32)n_exp, used, renorm, probs, ids, weights, fault, layer);
-    [[maybe_unused]] unsigned long long tl_routed = 0;
-    BM_RTICK(tl_routed, threadIdx.x);
-    BM_RTOCK(5, tl_routed);
+    router_logits_body<R, true>(lds, router, x, gain, eps, n_exp, hidden, normed_out, logits, (int)t, (int)(blockIdx.x % blocks_per_token) * R,
+                                hand);
 }
 
 // LDS of a workgroup of R rows: the token's row and the router rows, each as eight lines.
@@ -476,19 +504,19 @@ hipError_t router_logits(const Launch &L, const float *router, const float *x, c
 
 hipError_t norm_route(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                       int hidden, float *normed_out, float *logits, int used, int renorm, float *probs, uint32_t *ids,
-                      float *weights, uint32_t *counts, uint8_t *act_x, bool q8k) {
+                      float *weights, uint32_t *hand, uint8_t *act_x, bool q8k) {
     const int rows = router_rows(hidden, m, n_exp);
     if (rows == 0) return hipErrorInvalidValue;
     if (act_x && hidden % 256 != 0) return hipErrorInvalidValue;
     const size_t lds = router_lds_bytes(rows, hidden);
-    const unsigned grid = (unsigned)m * (unsigned)((n_exp + rows - 1) / rows) + (act_x ? (unsigned)m : 0u);
+    const unsigned grid = (unsigned)m * (unsigned)((n_exp + rows - 1) / rows) + (act_x ? (unsigned)m : 0u) + (unsigned)m;
 #define BM_NR(R, PER)                                                                                                  \
     {                                                                                                                  \
         auto kern = k_norm_route<R, PER>;                                                                              \
         hipError_t e = allow_lds(kern, lds);                                                                           \
         if (e != hipSuccess) return e;                                                                                 \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, router, x, gain, eps, n_exp, hidden, normed_out, \
-                           logits, (u32)used, (u32)renorm, probs, ids, weights, counts, act_x, q8k ? 1 : 0, m, L.fault, L.layer); \
+                           logits, (u32)used, (u32)renorm, probs, ids, weights, hand, act_x, q8k ? 1 : 0, m, L.fault, L.layer); \
     }
 #define BM_NR_ROWS(PER)                                                                                                \
     {                                                                                                                  \

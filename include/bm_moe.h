@@ -420,9 +420,11 @@ int bm_router_logits(bm_ctx *ctx, const float *router_dev, const float *x_dev, c
  * launch). Same arguments and the same bits in every output as the two calls one after the other. act_x (optional; hidden a
  * multiple of 256): the tokens' normed rows as quantized columns in the form the bm_act was made for, the bytes bm_quantize
  * makes of normed_dev (the launch's act_ffn), written by one more workgroup a token that the routing does not wait for:
- * bm_gate_up over act_x then takes the place of bm_gate_up_x / bm_moe_decode's first launch over normed_dev. The workgroup that finishes a token's last logits routes the token; none waits
- * for another. logits_dev is required (the token's logits meet there); 1 .. 4096 tokens a launch. Launches of this entry
- * that share a context must not overlap (they count finished workgroups in words the context holds). */
+ * bm_gate_up over act_x then takes the place of bm_gate_up_x / bm_moe_decode's first launch over normed_dev. One workgroup
+ * a token, behind the logits' workgroups in the grid, takes the token's logits as they land (words of the context that
+ * hold an armed pattern between launches; its wait is bounded: BM_SITE_ROUTER and NaN weights if a logit never came) and
+ * routes the token. logits_dev is required; 1 .. 4096 tokens a launch. Launches of this entry that share a context must not
+ * overlap (they share those words). */
 int bm_norm_route(bm_ctx *ctx, const float *router_dev, const float *x_dev, const float *gain_dev, float eps, int n_tokens,
                   int n_experts, int hidden, int top_k, int renorm, float *normed_dev, float *logits_dev, float *probs_dev,
                   uint32_t *ids_dev, float *weights_dev, bm_act *act_x);

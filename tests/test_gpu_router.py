@@ -219,8 +219,8 @@ def test_layer_from_the_residual_row(gpu):
                                                                       (7, 16384, 2, 2, True, 25), (3, 64, 4096, 1, True, 26)))
 def test_norm_route_is_the_two_launches_in_one(gpu, n_experts, hidden, m, top_k, with_gain, seed):
     """bm_norm_route against bm_router_logits followed by bm_route_softmax on the same inputs: every output the same bits
-    (normed rows, logits, probabilities, ids, weights), three launches in a row over the same counts and then a smaller
-    one, and under a graph replayed several times (the counts come back to zero without a memset)."""
+    (normed rows, logits, probabilities, ids, weights), three launches in a row over the same hand-over words and then a
+    smaller one, and under a graph replayed several times (the routing waves arm their words again without a memset)."""
     rng = np.random.default_rng(seed)
     router = normal_f32(rng, (n_experts, hidden), 0.05)
     x = np.stack([normal_f32(rng, hidden) * np.float32(10.0 ** rng.uniform(-1, 1)) for _ in range(m)])

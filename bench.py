@@ -781,6 +781,11 @@ def timeline(args, bm, gpu, enqueue_step, type_names):
                               for i, name in enumerate(("start", "token_row_arrived", "normed", "rows_and_token_in_lds", "dots_done"))},
                            "routing_wave": {"start": round(float((wave[0] - r0) / 100.0), 2),
                                             "holds_every_logit": round(float((wave[4] - r0) / 100.0), 2),
+                                            "maximum_known": round(float((wave[1] - r0) / 100.0), 2),
+                                            "exponentials_summed": round(float((wave[2] - r0) / 100.0), 2),
+                                            "probabilities_stored": round(float((wave[3] - r0) / 100.0), 2),
+                                            "entries_ahead_counted_by_its_wave": round(float((wave[6] - r0) / 100.0), 2),
+                                            "and_by_every_wave": round(float((wave[7] - r0) / 100.0), 2),
                                             "routed": round(float((wave[5] - r0) / 100.0), 2)}}
     print(json.dumps(out, indent=1), flush=True)
     gpu.close()

@@ -45,19 +45,40 @@ __device__ unsigned long long g_router_timeline[kRouterTimelineRows * 8];
 
 constexpr u32 kSiteRouter = 5; // crates/device/src/fault.rs:84-86
 
-__device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
-    int lo = __double2loint(v), hi = __double2hiint(v);
-    lo = __shfl_xor(lo, mask);
-    hi = __shfl_xor(hi, mask);
-    return __hiloint2double(hi, lo);
+// Sum / maximum over the wave, every lane ending with it: pairs, quads, eights and sixteens by data-parallel-primitive moves
+// (a few cycles each, where a shuffle through the LDS crossbar is a hundred), the two sixteens of a half by one swizzle, the
+// halves by two lane reads. The sum's association: ((pairs) quads) ... halves, lower half first.
+template <int CTRL>
+__device__ __forceinline__ double dpp_f64(double v) {
+    return __hiloint2double((int)bm_dpp<CTRL>((u32)__double2hiint(v)), (int)bm_dpp<CTRL>((u32)__double2loint(v)));
+}
+__device__ __forceinline__ double wave_sum_f64(double v) {
+    v += dpp_f64<kDppXor1>(v);
+    v += dpp_f64<kDppXor2>(v);
+    v += dpp_f64<kDppHalfMirror>(v);
+    v += dpp_f64<kDppMirror>(v);
+    v += __hiloint2double((int)bm_swap16((u32)__double2hiint(v)), (int)bm_swap16((u32)__double2loint(v)));
+    const int lo = __double2loint(v), hi = __double2hiint(v);
+    const double a = __hiloint2double(__builtin_amdgcn_readlane(hi, 0), __builtin_amdgcn_readlane(lo, 0));
+    const double b = __hiloint2double(__builtin_amdgcn_readlane(hi, 32), __builtin_amdgcn_readlane(lo, 32));
+    return a + b;
+}
+__device__ __forceinline__ float wave_max_f32(float v) {
+    v = fmaxf(v, bm_dppf<kDppXor1>(v));
+    v = fmaxf(v, bm_dppf<kDppXor2>(v));
+    v = fmaxf(v, bm_dppf<kDppHalfMirror>(v));
+    v = fmaxf(v, bm_dppf<kDppMirror>(v));
+    v = fmaxf(v, bm_bits_f32(bm_swap16(bm_f32_bits(v))));
+    const int bits = (int)bm_f32_bits(v);
+    return fmaxf(bm_bits_f32((u32)__builtin_amdgcn_readlane(bits, 0)), bm_bits_f32((u32)__builtin_amdgcn_readlane(bits, 32)));
 }
 
-// Token t's routing by one wave; lane L owns experts L + 64 j, j < PER. COH: the logits were stored by other workgroups of
-// this launch with device-scope stores and are read with device-scope loads (no cache of this compute unit's own is asked).
-// `v`: this lane's logits, expert lane + 64 j in v[j] (-inf past n_exp).
+// Token t's routing by one wave; lane L owns experts L + 64 j, j < PER. `v`: this lane's logits, expert lane + 64 j in v[j]
+// (-inf past n_exp). First the probabilities (p[j]; stored if asked for): false, with NaN probabilities and weights and
+// BM_SITE_ROUTER raised, when a logit is not finite.
 template <int PER>
-__device__ __forceinline__ void route_softmax_wave(const float (&v)[PER], u32 t, u32 n_exp, u32 used, u32 renorm, float *probs,
-                                                   u32 *ids, float *weights, u32 *fault, u32 layer) {
+__device__ __forceinline__ bool route_probs_wave(const float (&v)[PER], u32 t, u32 n_exp, u32 used, float *probs, float *weights,
+                                                 u32 *fault, u32 layer, float (&p)[PER]) {
     const u32 lane = threadIdx.x & 63;
     bool odd = false;
 #pragma unroll
@@ -71,31 +92,43 @@ __device__ __forceinline__ void route_softmax_wave(const float (&v)[PER], u32 t,
         }
         if (lane < used) weights[(size_t)t * used + lane] = nan;
         if (lane == 0) bm_raise(fault, layer, kSiteRouter);
-        return;
+        return false;
     }
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < PER; j++) mx = fmaxf(mx, v[j]);
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    float p[PER];
+    mx = wave_max_f32(mx);
+    [[maybe_unused]] unsigned long long tl_a = 0, tl_b = 0, tl_c = 0;
+    BM_RTICK(tl_a, mx);
     double sum = 0.0;
 #pragma unroll
     for (int j = 0; j < PER; j++) {
         p[j] = lane + 64 * j < n_exp ? (float)exp((double)(v[j] - mx)) : 0.0f;
         sum += (double)p[j];
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) sum += shfl_xor_f64(sum, off);
+    sum = wave_sum_f64(sum);
+    BM_RTICK(tl_b, sum);
     const float inv = (float)sum;
 #pragma unroll
     for (int j = 0; j < PER; j++) {
         p[j] = p[j] / inv;
         if (probs && lane + 64 * j < n_exp) probs[(size_t)t * n_exp + lane + 64 * j] = p[j];
     }
-    // `used` rounds of a wave argmax under (probability descending, id ascending): the largest probability left (its bits
-    // order as its value: not negative) as one unsigned maximum over the wave, then the smallest id that holds it: expert
-    // lane + 64 j, so the first j with a holder and that ballot's lowest lane. The winning lane marks its entry.
+    BM_RTICK(tl_c, p[0]);
+    BM_RTOCK(1, tl_a);
+    BM_RTOCK(2, tl_b);
+    BM_RTOCK(3, tl_c);
+    return true;
+}
+
+// Then the picks, by the wave alone: `used` rounds of a wave argmax under (probability descending, id ascending): the
+// largest probability left (its bits order as its value: not negative) as one unsigned maximum over the wave, then the
+// smallest id that holds it: expert lane + 64 j, so the first j with a holder and that ballot's lowest lane. The winning
+// lane marks its entry.
+template <int PER>
+__device__ __forceinline__ void route_pick_rounds(const float (&p)[PER], u32 t, u32 n_exp, u32 used, u32 renorm, u32 *ids,
+                                                  float *weights) {
+    const u32 lane = threadIdx.x & 63;
     u32 taken = 0;
     double chosen = 0.0;
     float mine = 0.0f;
@@ -128,6 +161,91 @@ __device__ __forceinline__ void route_softmax_wave(const float (&v)[PER], u32 t,
         if (lane == s) mine = bv;
     }
     if (lane < used) weights[(size_t)t * used + lane] = renorm ? mine / (float)chosen : mine;
+}
+
+template <int PER>
+__device__ __forceinline__ void route_softmax_wave(const float (&v)[PER], u32 t, u32 n_exp, u32 used, u32 renorm, float *probs,
+                                                   u32 *ids, float *weights, u32 *fault, u32 layer) {
+    float p[PER];
+    if (route_probs_wave<PER>(v, t, n_exp, used, probs, weights, fault, layer, p)) route_pick_rounds<PER>(p, t, n_exp, used, renorm, ids, weights);
+}
+
+// The same picks by a workgroup of 256 threads for up to 256 experts (n_exp >= used), the probabilities in LDS: an entry's
+// place in the order (probability descending, id ascending) is the number of entries ahead of it, counted by comparing it
+// with every other - independent instructions spread over four waves, where the wave's rounds are a chain of some eighty
+// dependent ones each (2.0 us of a 2.6 us routing at 128 experts, 8 picks). What is counted is the entries not smaller
+// (one compare and one add with carry an entry; probabilities are not negative, so their bits order as signed integers,
+// and the places past n_exp hold -1): without the entry itself that is its place unless another entry has its bits, and then
+// some place below `used` is taken twice or not at all - seen by counting the takers of every place - and the first wave
+// picks by its rounds instead. The entry with `s` ahead of it is pick s: the rounds' ids, and the same weights from the
+// same sums (the chosen probabilities added in pick order).
+// A barrier that waits for the wave's LDS traffic only: the routing workgroup's waves meet over LDS while the first wave's
+// stores to memory (the words armed again, the probabilities) are still on their way, and a barrier that waited for those to
+// be acknowledged cost the routing 1 us.
+__device__ __forceinline__ void lds_barrier() { __asm__ volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+struct PickLds {
+    __align__(16) float p[256];      // entry e's probability, -1 past n_exp
+    u32 ahead[256];    // zero on entry
+    u32 takers[32];    // zero on entry
+    u32 pick_id[32];
+    __align__(16) float pick_p[32];
+    u32 ok;
+};
+// Every thread of the workgroup calls it; true: the picks are written; false (first wave: pick by rounds): two entries tie.
+__device__ __forceinline__ bool route_pick_ranks(PickLds &L, u32 t, u32 n_exp, u32 used, u32 renorm, u32 *ids, float *weights) {
+    const u32 tid = threadIdx.x;
+    // the entries padded to 64 << k; a thread an (entry, part of the others): 4 >> k parts of 16 << 2 k entries, a wave's
+    // threads all of one part, so its reads of the others are broadcasts
+    const u32 k = n_exp <= 64 ? 0u : n_exp <= 128 ? 1u : 2u;
+    const u32 n_pad = 64u << k, chunk = 16u << (2 * k);
+    const u32 i = tid & (n_pad - 1), j0 = (tid >> (6 + k)) * chunk;
+    if (i < n_exp) {
+        const int ki = (int)bm_f32_bits(L.p[i]);
+        u32 cnt = 0;
+        for (u32 j = j0; j < j0 + chunk; j += 16) { // sixteen entries' reads in flight, then their compares (chunk: 16, 64 or 256)
+            float4 o[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) o[k] = *reinterpret_cast<const float4 *>(&L.p[j + 4 * k]);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                cnt += (int)bm_f32_bits(o[k].x) >= ki;
+                cnt += (int)bm_f32_bits(o[k].y) >= ki;
+                cnt += (int)bm_f32_bits(o[k].z) >= ki;
+                cnt += (int)bm_f32_bits(o[k].w) >= ki;
+            }
+        }
+        if (cnt) atomicAdd(&L.ahead[i], cnt);
+    }
+    [[maybe_unused]] unsigned long long tl_cnt = 0, tl_place = 0;
+    BM_RTICK(tl_cnt, tid);
+    lds_barrier();
+    BM_RTICK(tl_place, tid);
+    BM_RTOCK(6, tl_cnt);
+    BM_RTOCK(7, tl_place);
+    if (tid < n_exp) {
+        const u32 r = L.ahead[tid] - 1; // (itself among the counted)
+        if (r < used) {
+            L.pick_id[r] = tid, L.pick_p[r] = L.p[tid];
+            atomicAdd(&L.takers[r], 1u);
+        }
+    }
+    lds_barrier();
+    if (tid >= 64) return true;
+    if (__ballot(tid < used && L.takers[tid] != 1u) != 0) return false;
+    if (tid < used) {
+        double chosen = 0.0;
+        for (u32 s0 = 0; s0 < used; s0 += 8) { // eight reads at a time, then their adds in pick order
+            const float4 a = *reinterpret_cast<const float4 *>(&L.pick_p[s0]), b = *reinterpret_cast<const float4 *>(&L.pick_p[s0 + 4]);
+            const float q[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int k = 0; k < 8; k++)
+                if (s0 + k < used) chosen += (double)q[k];
+        }
+        ids[(size_t)t * used + tid] = L.pick_id[tid];
+        weights[(size_t)t * used + tid] = renorm ? L.pick_p[tid] / (float)chosen : L.pick_p[tid];
+    }
+    return true;
 }
 
 // One wave a token.
@@ -245,8 +363,7 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
                 sum += (double)__fmul_rn(xv[j].w, xv[j].w);
             }
         BM_RTICK(tl_row, sum);
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) sum += shfl_xor_f64(sum, off);
+        sum = wave_sum_f64(sum);
         if (lane == 0) s_part[wave] = sum;
         __syncthreads();
         const double total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
@@ -275,8 +392,7 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
             }
         }
         if (gain) {
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) sum += shfl_xor_f64(sum, off);
+            sum = wave_sum_f64(sum);
             if (lane == 0) s_part[wave] = sum;
             __syncthreads();
             const double total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
@@ -347,9 +463,10 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
         }
         for (; i < steps; i++) acc = fmaf(xf[i], wf[i], acc);
         // s_l = acc_l + acc_{l+4} on lanes 0..3 of the row's eight, then (s0 + s2) + (s1 + s3)
-        const float s = __fadd_rn(acc, __shfl_down(acc, 4, 8));
-        const float pair = __fadd_rn(s, __shfl_down(s, 2, 8)); // lane 0: s0 + s2, lane 1: s1 + s3
-        const float out = __fadd_rn(pair, __shfl_down(pair, 1, 8));
+        // (lane i reads lane i + n of its sixteen: right for the lanes of the eight whose value is used)
+        const float s = __fadd_rn(acc, bm_dppf<kDppShl4>(acc));
+        const float pair = __fadd_rn(s, bm_dppf<kDppShl2>(s)); // lane 0: s0 + s2, lane 1: s1 + s3
+        const float out = __fadd_rn(pair, bm_dppf<kDppShl1>(pair));
         BM_RTICK(tl_dots, out);
         if (l == 0 && e0 + r < n_exp) {
             logits[(size_t)t * n_exp + e0 + r] = out;
@@ -397,36 +514,59 @@ __global__ __launch_bounds__(256) void k_norm_route(const float *router, const f
     extern __shared__ __align__(16) uint8_t lds[];
     const u32 blocks_per_token = (u32)((n_exp + R - 1) / R);
     const u32 n_logit_blocks = (u32)m * blocks_per_token, n_quant_blocks = act_x ? (u32)m : 0u;
-    if (blockIdx.x >= n_logit_blocks + n_quant_blocks) { // a routing workgroup: its first wave
-        if (threadIdx.x >= 64) return;
+    if (blockIdx.x >= n_logit_blocks + n_quant_blocks) { // a routing workgroup: its first wave takes the logits
+        __shared__ PickLds pick;
         const u32 t = blockIdx.x - n_logit_blocks - n_quant_blocks, lane = threadIdx.x;
-        u32 *mine = hand + (size_t)t * n_exp;
-        [[maybe_unused]] unsigned long long tl_start = 0, tl_seen = 0;
-        BM_RTICK(tl_start, lane);
-        u32 w[PER];
-        bool late = true;
-        for (u32 spin = 0; spin < kRouteSpins && late; spin++) {
-            bool armed = false;
+        constexpr bool kRanks = PER <= 4; // up to 256 experts: the picks by the whole workgroup
+        if constexpr (kRanks) {
+            pick.p[threadIdx.x] = -1.0f, pick.ahead[threadIdx.x] = 0;
+            if (threadIdx.x < 32) pick.takers[threadIdx.x] = 0;
+            lds_barrier();
+        } else {
+            if (threadIdx.x >= 64) return;
+        }
+        [[maybe_unused]] float p[PER];
+        if (threadIdx.x < 64) {
+            u32 *mine = hand + (size_t)t * n_exp;
+            [[maybe_unused]] unsigned long long tl_start = 0, tl_seen = 0;
+            BM_RTICK(tl_start, lane);
+            u32 w[PER];
+            bool late = true;
+            for (u32 spin = 0; spin < kRouteSpins && late; spin++) {
+                bool armed = false;
+#pragma unroll
+                for (int j = 0; j < PER; j++) {
+                    const u32 e = lane + 64 * j;
+                    w[j] = e < (u32)n_exp ? __hip_atomic_load(mine + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+                    armed |= w[j] == kRouteArmed;
+                }
+                late = __ballot(armed) != 0;
+            }
+            BM_RTICK(tl_seen, w[0]);
+            BM_RTOCK(0, tl_start);
+            BM_RTOCK(4, tl_seen);
+            float v[PER];
 #pragma unroll
             for (int j = 0; j < PER; j++) {
                 const u32 e = lane + 64 * j;
-                w[j] = e < (u32)n_exp ? __hip_atomic_load(mine + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-                armed |= w[j] == kRouteArmed;
+                // (a word still armed after the last poll: the NaN it is, which the routing refuses as it refuses any)
+                v[j] = e < (u32)n_exp ? bm_bits_f32(w[j]) : -INFINITY;
+                if (e < (u32)n_exp) __hip_atomic_store(mine + e, kRouteArmed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-            late = __ballot(armed) != 0;
-        }
-        BM_RTICK(tl_seen, w[0]);
-        BM_RTOCK(0, tl_start);
-        BM_RTOCK(4, tl_seen);
-        float v[PER];
+            if constexpr (!kRanks) route_softmax_wave<PER>(v, t, (u32)n_exp, used, renorm, probs, ids, weights, fault, layer);
+            if constexpr (kRanks) {
+                const bool ok = route_probs_wave<PER>(v, t, (u32)n_exp, used, probs, weights, fault, layer, p);
+                if (lane == 0) pick.ok = ok;
 #pragma unroll
-        for (int j = 0; j < PER; j++) {
-            const u32 e = lane + 64 * j;
-            // (a word still armed after the last poll: the NaN it is, which the routing refuses as it refuses any)
-            v[j] = e < (u32)n_exp ? bm_bits_f32(w[j]) : -INFINITY;
-            if (e < (u32)n_exp) __hip_atomic_store(mine + e, kRouteArmed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int j = 0; j < PER; j++)
+                    if (ok && lane + 64 * j < (u32)n_exp) pick.p[lane + 64 * j] = p[j];
+            }
         }
-        route_softmax_wave<PER>(v, t, (u32)n_exp, used, renorm, probs, ids, weights, fault, layer);
+        if constexpr (kRanks) {
+            lds_barrier();
+            if (pick.ok && !route_pick_ranks(pick, t, (u32)n_exp, used, renorm, ids, weights))
+                route_pick_rounds<PER>(p, t, (u32)n_exp, used, renorm, ids, weights); // (the first wave, which holds p)
+        }
         [[maybe_unused]] unsigned long long tl_routed = 0;
         BM_RTICK(tl_routed, threadIdx.x);
         BM_RTOCK(5, tl_routed);

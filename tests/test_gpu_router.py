@@ -290,6 +290,46 @@ def test_norm_route_is_the_two_launches_in_one(gpu, n_experts, hidden, m, top_k,
             b.free()
 
 
+@pytest.mark.parametrize("n_experts,top_k", ((128, 8), (200, 6), (40, 4), (300, 8)))
+def test_norm_route_picks_among_equal_probabilities(gpu, n_experts, top_k):
+    """Router rows that repeat give logits that are equal bit for bit: the fused launch's picks (by counting, for up to 256
+    experts, with the wave's rounds behind it when two entries tie) go to the smaller id as the two launches' and the
+    oracle's do: a token whose winners tie, one whose ties lie past the picks, one whose row is zero (every expert ties),
+    one without ties."""
+    hidden, m = 256, 4
+    rng = np.random.default_rng(4100 + n_experts)
+    router = normal_f32(rng, (n_experts, hidden), 0.05)
+    x = normal_f32(rng, (m, hidden))
+    x[2] = 0.0
+    l0 = ora.router_logits(router, x[:1], None, 0.0)[1][0]
+    order = np.argsort(-l0, kind="stable")
+    router[order[1]] = router[order[0]]            # token 0's two best tie (and every token's at those two ids)
+    router[order[-1]] = router[order[-2]]          # and two of its worst
+    rd, xd = gpu.upload(router, np.float32), gpu.upload(x, np.float32)
+    out = {}
+    for tag in ("two", "one"):
+        out[tag] = (gpu.buffer(np.float32, m * n_experts), gpu.buffer(np.float32, m * n_experts), gpu.buffer(np.uint32, m * top_k).fill_bytes(0xFF),
+                    gpu.buffer(np.float32, m * top_k))
+    gpu.fault_clear()
+    logits, probs, ids, wts = out["two"]
+    gpu.enqueue_router_logits(rd, xd, None, 0.0, m, n_experts, hidden, None, logits)
+    gpu.enqueue_route_softmax(logits, m, n_experts, top_k, True, probs, ids, wts)
+    logits, probs, ids, wts = out["one"]
+    for rep in range(2):
+        gpu.enqueue_norm_route(rd, xd, None, 0.0, m, n_experts, hidden, top_k, True, None, logits, probs, ids, wts)
+        for a, b, name in zip(out["one"], out["two"], ("logits", "probs", "ids", "weights")):
+            assert np.array_equal(a.download().view(np.uint32), b.download().view(np.uint32)), f"call {rep}: {name}"
+    got_l, got_ids = logits.download().reshape(m, n_experts), ids.download().reshape(m, top_k)
+    assert got_l[0, order[0]] == got_l[0, order[1]] and sorted(got_ids[0, :2]) == sorted(order[:2]) and got_ids[0, 0] < got_ids[0, 1]
+    assert got_ids[2].tolist() == list(range(top_k))
+    for t in range(m):
+        want_ids, _ = ora.route_softmax_topk(got_l[t], top_k)
+        assert np.array_equal(got_ids[t], want_ids), f"token {t}"
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    for b in (rd, xd) + out["two"] + out["one"]:
+        b.free()
+
+
 def test_norm_route_raises_and_refuses_like_its_parts(gpu):
     """A logit that is not finite (a NaN in the token's row) raises Router from the fused launch too, and the other
     tokens are routed; the argument checks are the two entries' own, by name."""

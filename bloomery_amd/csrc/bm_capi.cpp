@@ -990,17 +990,23 @@ int bm_moe_forward(bm_ctx *ctx, bm_scratch *s, const bm_weights *wg, const bm_we
         return bm_moe_decode(ctx, wg, wu, wd, x_dev, sel_dev, w_dev, resid_dev, spt, m, rule, s->act_h, nullptr,
                              down_q8k ? s->g : nullptr, y_dev);
     case BM_PATH_GROUPED: {
-        int rc = bm_tables(ctx, sel_dev, n_slots, n_experts, s->order, s->start, s->tiles);
         // Few slots an expert (no more slots than experts: nearly every tile is one slot) and h on its way through f32 rows:
-        // the per-slot gate . up launch from the token rows is the faster one there (its one-column walk reads the activation
-        // operands a super-block ahead: 83 against 102 us at the DeepSeek-V3 shape, 4 tokens) and the tile launch the faster down
-        // (54 against 84 us), so the step takes one of each; the down tiles then read their columns in slot order.
-        if (!rc && down_q8k && act_form(s->gate_type) != 0 && n_slots <= n_experts && m <= bmk::kMaxDecodeTokens && per_slot_fits(s)) {
-            bmk::Launch L;
-            rc = launch_under(ctx, what, rule, &L);
-            if (!rc)
-                rc = driver(ctx, what, bmk::gate_up_x(L, wg->wtype, x_dev, wg->dev, wu->dev, n_experts, hidden, ff, sel_dev, spt, m, nullptr,
-                                                      nullptr, s->g));
+        // the per-slot gate . up launch is the faster one there (its one-column walk reads the activation operands a
+        // super-block ahead: 83 against 102 us at the DeepSeek-V3 shape, 4 tokens) and the tile launch the faster down (54
+        // against 84 us), so the step takes one of each; the down tiles then read their columns in slot order. The tokens'
+        // columns are quantized once, beside the tables in their launch, not by every workgroup of the gate . up launch
+        // (whose vector ALU is what bounds it at these types: 180 -> 172 us a step).
+        if (down_q8k && act_form(s->gate_type) != 0 && n_slots <= n_experts && m <= bmk::kMaxDecodeTokens && per_slot_fits(s) &&
+            n_experts <= bmk::kBucketExperts && n_slots <= bmk::kTileMaxSlots) {
+            int rc;
+            if ((reinterpret_cast<uintptr_t>(x_dev) & 15) == 0) {
+                rc = driver(ctx, what, bmk::tables_q8k(launch_of(ctx), sel_dev, n_slots, n_experts, s->order, s->start, s->tiles, x_dev, m,
+                                                       hidden, s->act_x->dev));
+            } else {
+                rc = bm_tables(ctx, sel_dev, n_slots, n_experts, s->order, s->start, s->tiles);
+                if (!rc) rc = bm_quantize(ctx, x_dev, m, s->act_x);
+            }
+            if (!rc) rc = bm_gate_up(ctx, wg, wu, s->act_x, sel_dev, n_slots, ff, spt, rule, s->g, nullptr);
             if (!rc) // (a slot without an expert of the stack: its rows of h hold nothing, its column is left alone)
                 rc = driver(ctx, what, bmk::quantize(launch_of(ctx), s->down_type, s->g, n_slots, ff, s->act_h->dev, nullptr, sel_dev,
                                                      (uint32_t)n_experts));
@@ -1010,6 +1016,7 @@ int bm_moe_forward(bm_ctx *ctx, bm_scratch *s, const bm_weights *wg, const bm_we
             if (rc) return rc;
             break;
         }
+        int rc = bm_tables(ctx, sel_dev, n_slots, n_experts, s->order, s->start, s->tiles);
         if (!rc) rc = bm_quantize(ctx, x_dev, m, s->act_x);
         if (!rc && !down_q8k)
             rc = bm_gate_up_tiles(ctx, wg, wu, s->act_x, s->order, s->start, s->tiles, n_slots, ff, spt, rule, nullptr, s->act_h);

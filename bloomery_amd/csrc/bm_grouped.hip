@@ -81,6 +81,38 @@ __global__ __launch_bounds__(1024) void k_tables(const u32 *sel, u32 n_slots, u3
     tiles_body(start, n_experts, n_slots, cap, tiles, fault, layer);
 }
 
+// k_tables with a quantizer beside it: workgroup 0 makes the tables, the others the Q8_K columns of m rows of k f32 values
+// (a wave a 256-value block, the bytes of k_quantize_q8k) - two short launches that do not depend on each other as one.
+__global__ __launch_bounds__(1024) void k_tables_q8k(const u32 *sel, u32 n_slots, u32 n_experts, u32 cap, u32 *order, u32 *start,
+                                                     u32 *tiles, const float *x, int n_blocks, uint8_t *act, u32 *fault, u32 layer) {
+    if (blockIdx.x != 0) {
+        const int b = (int)(blockIdx.x - 1) * 16 + (int)(threadIdx.x >> 6), lane = (int)(threadIdx.x & 63);
+        if (b >= n_blocks) return; // whole waves leave
+        q8k_wave_block(*reinterpret_cast<const float4 *>(x + (size_t)b * 256 + 4 * lane), act + (size_t)b * BM_Q8K_STRIDE, lane, fault, layer);
+        return;
+    }
+    __shared__ GroupLds g;
+    group_slots(g, n_slots, n_experts, order, [&](u32 s) {
+        const u32 p = sel[s];
+        if (p < n_experts) return p;
+        if (p != kHostSlot) bm_raise(fault, layer, kSiteExpertId);
+        return kNoBucket;
+    });
+    for (u32 e = threadIdx.x; e <= n_experts; e += blockDim.x) start[e] = g.base[e];
+    __threadfence_block();
+    __syncthreads();
+    tiles_body(start, n_experts, n_slots, cap, tiles, fault, layer);
+}
+
+hipError_t tables_q8k(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start,
+                      uint32_t *tiles_out, const float *x, int m, int k, uint8_t *act) {
+    if (k % 256 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0) return hipErrorInvalidValue;
+    const int n_blocks = m * (k / 256);
+    hipLaunchKernelGGL(k_tables_q8k, dim3(1 + (unsigned)((n_blocks + 15) / 16)), dim3(1024), 0, L.stream, sel, (u32)n_slots,
+                       (u32)n_experts, (u32)tile_cap(n_slots, n_experts), order, start, tiles_out, x, n_blocks, act, L.fault, L.layer);
+    return hipGetLastError();
+}
+
 hipError_t tables(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start,
                   uint32_t *tiles_out) {
     hipLaunchKernelGGL(k_tables, dim3(1), dim3(1024), 0, L.stream, sel, (u32)n_slots, (u32)n_experts,

@@ -373,7 +373,8 @@ int bm_swiglu_quant_sel(bm_ctx *ctx, const float *g_dev, const float *u_dev, con
  * the Qwen3-30B-A3B layer shape: 22 tokens, and 448 tokens in the exact mode of bm_gemm or 96 in its tolerance mode (96 in
  * either mode where the gate/up stack dots against Q8_K columns: Q3_K, IQ2_XXS, IQ3_XXS, IQ4_XS; where the down stack does so
  * too and hidden x ff is 2^23 or more, the grouped path from the first token). On the grouped path a batch with no more slots
- * than experts whose h crosses in f32 rows takes the per-slot gate . up launch and the tile launch for down.
+ * than experts whose h crosses in f32 rows takes the per-slot gate . up launch (over columns made in the tables' launch) and
+ * the tile launch for down.
  * bm_scratch_set_path sets others (0 keeps a value; gemm_from then holds for both modes) or forces one path.
  * bm_scratch_path_for: the path a call with m tokens takes. A slot whose id names no expert of the stack adds nothing to
  * the sum and raises BM_SITE_EXPERT_ID unless it is BM_HOST_SLOT, which every path skips silently (the GEMM path's route

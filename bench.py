@@ -256,9 +256,11 @@ def bench_grouped(args, bm, ora, threads):
         st = i % sets
         dg, du, dd = layers[i % len(layers)]
         s_ptr = sel.ptr + 4 * st * n_slots
-        if "tables" in which:
+        if "tables" in which and "quant" in which:  # the whole step: the two as one launch
+            gpu.enqueue_tables_quantize(s_ptr, n_slots, N_EXPERTS, order, start, tiles, xd.ptr + 4 * st * m * HIDDEN, m, act)
+        elif "tables" in which:
             gpu.enqueue_tables(s_ptr, n_slots, N_EXPERTS, order, start, tiles)
-        if "quant" in which:
+        elif "quant" in which:
             gpu.enqueue_quantize(xd.ptr + 4 * st * m * HIDDEN, m, act)
         if "gate_up" in which:
             gpu.enqueue_gate_up_tiles(dg, du, act, order, start, tiles, n_slots, FF, TOP_K, None, act_h)

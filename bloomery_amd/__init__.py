@@ -62,6 +62,7 @@ SYMBOLS = {
     "bm_gemv": (_i, [_vp, _vp, _vp, _i, _vp]),
     "bm_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
     "bm_tables": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp]),
+    "bm_tables_quantize": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _vp]),
     "bm_gemv_x": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
     "bm_gemv_sel": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "bm_combine_tokens": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -561,6 +562,11 @@ class Gpu:
     def enqueue_tables(self, sel, n_slots, n_experts, order, start, tiles):
         """enqueue_buckets and enqueue_tiles as one launch."""
         self._check(self.lib.bm_tables(self.ctx, _ptr(sel), n_slots, n_experts, _ptr(order), _ptr(start), _ptr(tiles)))
+
+    def enqueue_tables_quantize(self, sel, n_slots, n_experts, order, start, tiles, x, m, act):
+        """enqueue_tables and enqueue_quantize as one launch (same tables, same column bytes)."""
+        self._check(self.lib.bm_tables_quantize(self.ctx, _ptr(sel), n_slots, n_experts, _ptr(order), _ptr(start), _ptr(tiles), _ptr(x), m,
+                                                act.handle))
 
     def enqueue_tiles(self, start, n_experts, n_slots, tiles):
         self._check(self.lib.bm_tiles(self.ctx, _ptr(start), n_experts, n_slots, _ptr(tiles)))

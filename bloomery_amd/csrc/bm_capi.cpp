@@ -665,6 +665,22 @@ int bm_tables(bm_ctx *ctx, const uint32_t *sel_dev, int n_slots, int n_experts, 
     return driver(ctx, what, bmk::tables(launch_of(ctx), sel_dev, n_slots, n_experts, order_dev, start_dev, tiles_dev));
 }
 
+int bm_tables_quantize(bm_ctx *ctx, const uint32_t *sel_dev, int n_slots, int n_experts, uint32_t *order_dev, uint32_t *start_dev,
+                       uint32_t *tiles_dev, const float *x_dev, int m, bm_act *act) {
+    const char *what = "bm_tables_quantize";
+    if (!ctx || !sel_dev || !order_dev || !start_dev || !tiles_dev || !x_dev || !act) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (n_experts < 1 || n_experts > bmk::kBucketExperts || n_slots < 1 || n_slots > bmk::kTileMaxSlots)
+        return fail(ctx, BM_ESHAPE, "%s: %d places over %d experts (1..=%d experts, 1..=%d places)", what, n_slots, n_experts,
+                    bmk::kBucketExperts, bmk::kTileMaxSlots);
+    if (m < 1 || m > act->m_cap) return fail(ctx, BM_ESHAPE, "%s: m = %d columns, act holds %d", what, m, act->m_cap);
+    if ((reinterpret_cast<uintptr_t>(x_dev) & 15) != 0 || act->k % 256 != 0) { // rows the one launch does not read: the two launches
+        int rc = bm_tables(ctx, sel_dev, n_slots, n_experts, order_dev, start_dev, tiles_dev);
+        return rc ? rc : bm_quantize(ctx, x_dev, m, act);
+    }
+    return driver(ctx, what, bmk::tables_quant(launch_of(ctx), sel_dev, n_slots, n_experts, order_dev, start_dev, tiles_dev, act->wtype,
+                                               x_dev, m, act->k, act->dev));
+}
+
 int bm_quantize_ord(bm_ctx *ctx, const float *x_dev, const uint32_t *start_dev, int n_experts, int m_cols, bm_act *act) {
     const char *what = "bm_quantize_ord";
     if (!ctx || !x_dev || !start_dev || !act) return fail(ctx, BM_EARG, "%s: NULL argument", what);
@@ -998,14 +1014,7 @@ int bm_moe_forward(bm_ctx *ctx, bm_scratch *s, const bm_weights *wg, const bm_we
         // (whose vector ALU is what bounds it at these types: 180 -> 172 us a step).
         if (down_q8k && act_form(s->gate_type) != 0 && n_slots <= n_experts && m <= bmk::kMaxDecodeTokens && per_slot_fits(s) &&
             n_experts <= bmk::kBucketExperts && n_slots <= bmk::kTileMaxSlots) {
-            int rc;
-            if ((reinterpret_cast<uintptr_t>(x_dev) & 15) == 0) {
-                rc = driver(ctx, what, bmk::tables_q8k(launch_of(ctx), sel_dev, n_slots, n_experts, s->order, s->start, s->tiles, x_dev, m,
-                                                       hidden, s->act_x->dev));
-            } else {
-                rc = bm_tables(ctx, sel_dev, n_slots, n_experts, s->order, s->start, s->tiles);
-                if (!rc) rc = bm_quantize(ctx, x_dev, m, s->act_x);
-            }
+            int rc = bm_tables_quantize(ctx, sel_dev, n_slots, n_experts, s->order, s->start, s->tiles, x_dev, m, s->act_x);
             if (!rc) rc = bm_gate_up(ctx, wg, wu, s->act_x, sel_dev, n_slots, ff, spt, rule, s->g, nullptr);
             if (!rc) // (a slot without an expert of the stack: its rows of h hold nothing, its column is left alone)
                 rc = driver(ctx, what, bmk::quantize(launch_of(ctx), s->down_type, s->g, n_slots, ff, s->act_h->dev, nullptr, sel_dev,
@@ -1016,8 +1025,7 @@ int bm_moe_forward(bm_ctx *ctx, bm_scratch *s, const bm_weights *wg, const bm_we
             if (rc) return rc;
             break;
         }
-        int rc = bm_tables(ctx, sel_dev, n_slots, n_experts, s->order, s->start, s->tiles);
-        if (!rc) rc = bm_quantize(ctx, x_dev, m, s->act_x);
+        int rc = bm_tables_quantize(ctx, sel_dev, n_slots, n_experts, s->order, s->start, s->tiles, x_dev, m, s->act_x);
         if (!rc && !down_q8k)
             rc = bm_gate_up_tiles(ctx, wg, wu, s->act_x, s->order, s->start, s->tiles, n_slots, ff, spt, rule, nullptr, s->act_h);
         if (!rc && down_q8k) {

@@ -81,14 +81,25 @@ __global__ __launch_bounds__(1024) void k_tables(const u32 *sel, u32 n_slots, u3
     tiles_body(start, n_experts, n_slots, cap, tiles, fault, layer);
 }
 
-// k_tables with a quantizer beside it: workgroup 0 makes the tables, the others the Q8_K columns of m rows of k f32 values
-// (a wave a 256-value block, the bytes of k_quantize_q8k) - two short launches that do not depend on each other as one.
-__global__ __launch_bounds__(1024) void k_tables_q8k(const u32 *sel, u32 n_slots, u32 n_experts, u32 cap, u32 *order, u32 *start,
-                                                     u32 *tiles, const float *x, int n_blocks, uint8_t *act, u32 *fault, u32 layer) {
+// k_tables with a quantizer beside it: workgroup 0 makes the tables, the others the quantized columns of m rows of k f32
+// values - Q8_K: a wave a 256-value block, the bytes of k_quantize_q8k; Q8_2_X4: eight values a thread, a block a quad of
+// lanes, the bytes of k_quantize_q82x4 - two short launches that do not depend on each other as one.
+template <bool Q8K>
+__global__ __launch_bounds__(1024) void k_tables_quant(const u32 *sel, u32 n_slots, u32 n_experts, u32 cap, u32 *order, u32 *start,
+                                                       u32 *tiles, const float *x, int m, int k, uint8_t *act, u32 *fault, u32 layer) {
     if (blockIdx.x != 0) {
-        const int b = (int)(blockIdx.x - 1) * 16 + (int)(threadIdx.x >> 6), lane = (int)(threadIdx.x & 63);
-        if (b >= n_blocks) return; // whole waves leave
-        q8k_wave_block(*reinterpret_cast<const float4 *>(x + (size_t)b * 256 + 4 * lane), act + (size_t)b * BM_Q8K_STRIDE, lane, fault, layer);
+        if constexpr (Q8K) {
+            const int b = (int)(blockIdx.x - 1) * 16 + (int)(threadIdx.x >> 6), lane = (int)(threadIdx.x & 63);
+            if (b >= m * (k / 256)) return; // whole waves leave
+            q8k_wave_block(*reinterpret_cast<const float4 *>(x + (size_t)b * 256 + 4 * lane), act + (size_t)b * BM_Q8K_STRIDE, lane, fault, layer);
+        } else {
+            const long at = ((long)(blockIdx.x - 1) * 1024 + threadIdx.x) * 8;
+            if (at >= (long)m * k) return; // whole quads leave: a block is 32 values, k a multiple of 256
+            const int col = (int)(at / k), o = (int)(at % k);
+            const float4 a = *reinterpret_cast<const float4 *>(x + at), b = *reinterpret_cast<const float4 *>(x + at + 4);
+            const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+            q82_quad8(v, act + (size_t)col * (k / 256) * BM_Q82_SB_EXT, k / 256, o >> 5, threadIdx.x & 3, fault, layer);
+        }
         return;
     }
     __shared__ GroupLds g;
@@ -104,12 +115,19 @@ __global__ __launch_bounds__(1024) void k_tables_q8k(const u32 *sel, u32 n_slots
     tiles_body(start, n_experts, n_slots, cap, tiles, fault, layer);
 }
 
-hipError_t tables_q8k(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start,
-                      uint32_t *tiles_out, const float *x, int m, int k, uint8_t *act) {
+hipError_t tables_quant(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start,
+                        uint32_t *tiles_out, int wtype, const float *x, int m, int k, uint8_t *act) {
     if (k % 256 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0) return hipErrorInvalidValue;
-    const int n_blocks = m * (k / 256);
-    hipLaunchKernelGGL(k_tables_q8k, dim3(1 + (unsigned)((n_blocks + 15) / 16)), dim3(1024), 0, L.stream, sel, (u32)n_slots,
-                       (u32)n_experts, (u32)tile_cap(n_slots, n_experts), order, start, tiles_out, x, n_blocks, act, L.fault, L.layer);
+    const u32 cap = (u32)tile_cap(n_slots, n_experts);
+    if (bm_takes_q8k(wtype)) {
+        const unsigned grid = 1 + (unsigned)((m * (k / 256) + 15) / 16);
+        hipLaunchKernelGGL(k_tables_quant<true>, dim3(grid), dim3(1024), 0, L.stream, sel, (u32)n_slots, (u32)n_experts, cap, order, start,
+                           tiles_out, x, m, k, act, L.fault, L.layer);
+    } else {
+        const unsigned grid = 1 + (unsigned)(((long)m * k + 8191) / 8192);
+        hipLaunchKernelGGL(k_tables_quant<false>, dim3(grid), dim3(1024), 0, L.stream, sel, (u32)n_slots, (u32)n_experts, cap, order, start,
+                           tiles_out, x, m, k, act, L.fault, L.layer);
+    }
     return hipGetLastError();
 }
 

@@ -106,9 +106,10 @@ hipError_t tables(const Launch &L, const uint32_t *sel, int n_slots, int n_exper
                   uint32_t *tiles);
 // LDS bytes a tile launch of this type and k asks for (0 if eight columns do not fit a workgroup's LDS).
 size_t tiles_lds(int wtype, int k);
-// tables() and the Q8_K columns of m rows of k f32 values (k a multiple of 256, x 16-byte aligned) as one launch.
-hipError_t tables_q8k(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start,
-                      uint32_t *tiles_out, const float *x, int m, int k, uint8_t *act);
+// tables() and quantize() of m rows of k f32 values (k a multiple of 256, x 16-byte aligned) into the column form wtype
+// dots against, as one launch.
+hipError_t tables_quant(const Launch &L, const uint32_t *sel, int n_slots, int n_experts, uint32_t *order, uint32_t *start,
+                        uint32_t *tiles_out, int wtype, const float *x, int m, int k, uint8_t *act);
 hipError_t gate_up_tiles(const Launch &L, int wtype, const uint8_t *wg, const uint8_t *wu, int n_experts, int k,
                          const uint8_t *act, int act_cols, const uint32_t *order, const uint32_t *start,
                          const uint32_t *tiles, int n_slots, int rows_per_expert, int slots_per_col, float *h,

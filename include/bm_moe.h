@@ -271,6 +271,12 @@ int bm_tiles(bm_ctx *ctx, const uint32_t *start_dev, int n_experts, int n_slots,
 /* bm_buckets then bm_tiles as one launch: order_dev, start_dev and tiles_dev hold what the two calls would leave. */
 int bm_tables(bm_ctx *ctx, const uint32_t *sel_dev, int n_slots, int n_experts, uint32_t *order_dev, uint32_t *start_dev,
               uint32_t *tiles_dev);
+/* bm_tables and bm_quantize(ctx, x_dev, m, act) as one launch: the two depend on nothing of each other and are each a few
+ * microseconds of latency, so the grouped step starts one launch sooner. The same tables and the same column bytes. No
+ * counterpart in the reference, which enqueues the two separately (crates/gpu/src/q4k_sel.rs:1103,1152 and the card's
+ * quantizer). Rows that are not 16-byte aligned or not whole super-blocks go through the two launches. */
+int bm_tables_quantize(bm_ctx *ctx, const uint32_t *sel_dev, int n_slots, int n_experts, uint32_t *order_dev, uint32_t *start_dev,
+                       uint32_t *tiles_dev, const float *x_dev, int m, bm_act *act);
 /* Q4kSelKernels::enqueue_quantize_ord (crates/gpu/src/q4k_sel.rs:1255): the first start_dev[n_experts] columns
  * of x_dev (at most m_cols, the columns launched) into the same columns of act, bm_quantize's bytes; every other
  * column keeps what it held. */
@@ -362,7 +368,7 @@ int bm_swiglu_quant_sel(bm_ctx *ctx, const float *g_dev, const float *u_dev, con
  * number of tokens - the reference's cut between its gemv arm and its wide arm (crates/gpu/src/arch/qwen3moe/wide.rs:75-77
  * GEMV_COLS, prefill.rs:602-604 WIDE_FROM, :147 wide_steps), here with a grouped arm between the two:
  *   BM_PATH_PER_SLOT  bm_moe_decode: two launches, every slot streams its expert's rows (repeats come from the caches);
- *   BM_PATH_GROUPED   bm_tables, bm_quantize, bm_gate_up_tiles (bm_quantize_ord for a down stack on Q8_K columns),
+ *   BM_PATH_GROUPED   bm_tables_quantize, bm_gate_up_tiles (bm_quantize_ord for a down stack on Q8_K columns),
  *                     bm_gemv_tiles, the slots' sum: an expert's rows are read once for all of its slots;
  *   BM_PATH_GEMM      bm_quantize, bm_route_fill, bm_gemm twice, bm_swiglu_quant_sel, bm_gemm, the slots' sum: the int8 matrix
  *                     cores (in the f32 order bm_set_gemm_mode sets; every stack type bm_gemm takes).

@@ -578,6 +578,51 @@ def test_grouped_tables_are_the_definition(gpu, n_experts, n_slots, seed):
         b.free()
 
 
+@pytest.mark.parametrize("wtype,k,m,n_experts,top_k,seed", ((bm.Q4_K, 2048, 16, 128, 8, 1), (bm.IQ2_XXS, 1792, 5, 40, 3, 2),
+                                                          (bm.Q6_K, 256, 1, 3, 2, 3), (bm.IQ4_XS, 7168, 33, 256, 8, 4), (bm.Q5_K, 512, 70, 9, 4, 5)))
+def test_tables_and_quantizer_as_one_launch(gpu, wtype, k, m, n_experts, top_k, seed):
+    """bm_tables_quantize leaves what bm_tables and bm_quantize leave: the three tables word for word and every column's bytes,
+    in either column form, with a host-served slot and an id past the stack among the slots (the one raises nothing, the other
+    ExpertId, as in bm_tables), twice in a row; rows that are not 16-byte aligned go through the two launches and give the same."""
+    rng = np.random.default_rng(7700 + seed)
+    n_slots = m * top_k
+    ids = rng.integers(0, n_experts, n_slots).astype(np.uint32)
+    if n_slots > 4:
+        ids[1], ids[3] = bm.HOST_SLOT, n_experts + 5
+    x = normal_f32(rng, (m, k))
+    x[0, 5] = 0.0
+    sel, xd = gpu.upload(ids, np.uint32), gpu.upload(np.concatenate([np.zeros(1, np.float32), x.reshape(-1)]), np.float32)
+    cap = gpu.tile_cap(n_slots, n_experts)
+    want = (gpu.buffer(np.uint32, n_slots).fill_bytes(0), gpu.buffer(np.uint32, n_experts + 1).fill_bytes(0xFF), gpu.buffer(np.uint32, cap + 1).fill_bytes(0))
+    want_act = gpu.act(wtype, k, m)
+    gpu.fault_clear()
+    gpu.enqueue_tables(sel, n_slots, n_experts, *want)
+    want_fault = gpu.fault()
+    gpu.enqueue_quantize(xd.ptr + 4, m, want_act)
+    for x_ptr, what in ((xd.ptr + 4, "rows 4 bytes off a 16-byte boundary"), (None, "aligned rows")):
+        xa = gpu.upload(x, np.float32) if x_ptr is None else None
+        got = (gpu.buffer(np.uint32, n_slots).fill_bytes(0), gpu.buffer(np.uint32, n_experts + 1).fill_bytes(0xFF), gpu.buffer(np.uint32, cap + 1).fill_bytes(0))
+        act = gpu.act(wtype, k, m)
+        for rep in range(2):
+            gpu.fault_clear()
+            gpu.enqueue_tables_quantize(sel, n_slots, n_experts, *got, xa if xa is not None else x_ptr, m, act)
+            listed = int(want[1].download()[-1])
+            assert np.array_equal(got[1].download(), want[1].download()), what
+            assert np.array_equal(got[0].download()[:listed], want[0].download()[:listed]), what
+            n_t = int(want[2].download()[0])
+            assert np.array_equal(got[2].download()[:1 + n_t], want[2].download()[:1 + n_t]), what
+            for c in range(m):
+                assert np.array_equal(act.download(c), want_act.download(c)), f"{what}: column {c}"
+                if c in (0, m - 1):
+                    assert np.array_equal(act.download(c), ora.quantize_col(wtype, x[c])), f"{what}: column {c} against the oracle"
+            assert gpu.fault() == want_fault, what
+        for b in got + (act,) + ((xa,) if xa is not None else ()):
+            b.free()
+    gpu.fault_clear()
+    for b in want + (want_act, sel, xd):
+        b.free()
+
+
 def test_grouped_tables_refuse_bad_ids_and_bad_runs(gpu):
     ids = np.array([2, 9, 1, 2], np.uint32)   # 9 is past a stack of 4
     gpu.fault_clear()

@@ -926,15 +926,28 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq(const uint8_t *w, int rpe, i
     const u32 src_w = (u32)(row0 + wr < rpe ? row0 + wr : rpe - 1) * row_bytes;
     const int a_dst = ac * kIqStride + 32 * (4 * (ap & 1)) + 4 * (ap >> 1); // word k of a piece: + 32 k
 
-    auto stage = [&](int i) {
-        uint4 ra[4];
+    // A super-block's bytes are asked for one super-block ahead (fetch_rows, fetch_cols: into registers, behind the staging of
+    // the present one and before its products) and unpacked into LDS when their turn comes (stage): the loads' way through memory runs
+    // under the matrix work instead of in front of it.
+    uint4 ra[4];
+    uint4 rq = make_uint4(0, 0, 0, 0), rq2 = rq, rq3 = rq, rq4 = rq;
+    uint2 rx = make_uint2(0, 0);
+    u32 rd = 0, ra2 = 0;
+    float cdy = 0.0f;
+    uint4 cb0 = make_uint4(0, 0, 0, 0), cb1 = cb0;
+    auto fetch_cols = [&](int i) {
 #pragma unroll
         for (int j = 0; j < 4; j++) __builtin_memcpy(&ra[j], act + (src_a[j] + (u32)i * BM_Q8K_STRIDE), 16);
+        if (tid < 64) {
+            const uint8_t *cs = act + (src_c + (u32)i * BM_Q8K_STRIDE);
+            cdy = *reinterpret_cast<const float *>(cs);
+            __builtin_memcpy(&cb0, cs + 264, 16);
+            __builtin_memcpy(&cb1, cs + 280, 16);
+        }
+    };
+    auto fetch_rows = [&](int i) {
         const uint8_t *blk = we + (src_w + (u32)i * G::kBlock);
         // the row's two sub-blocks 2 wq and 2 wq + 1, as the type lays them out
-        uint4 rq = make_uint4(0, 0, 0, 0), rq2 = rq, rq3 = rq, rq4 = rq;
-        uint2 rx = make_uint2(0, 0);
-        u32 rd = 0, ra2 = 0;
         if constexpr (WT == BM_IQ2XXS) {
             rq = bm_ld16u(blk + 2 + 16 * wq);
             rd = bm_ld2u(blk);
@@ -957,14 +970,8 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq(const uint8_t *w, int rpe, i
             ra2 = (tail.z >> 16) | (tail.w << 16);                                             // a2: their high bits
             rd = tail.w >> 16;
         }
-        float cdy = 0.0f;
-        uint4 cb0 = make_uint4(0, 0, 0, 0), cb1 = cb0;
-        if (tid < 64) {
-            const uint8_t *cs = act + (src_c + (u32)i * BM_Q8K_STRIDE);
-            cdy = *reinterpret_cast<const float *>(cs);
-            __builtin_memcpy(&cb0, cs + 264, 16);
-            __builtin_memcpy(&cb1, cs + 280, 16);
-        }
+    };
+    auto stage = [&]() {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             uint8_t *dst = a_codes + a_dst + 16 * j * kIqStride;
@@ -1087,9 +1094,20 @@ __global__ __launch_bounds__(256, 2) void k_gemm_iq(const uint8_t *w, int rpe, i
 #pragma unroll
         for (int v = 0; v < 16; v++) acc[l][v] = 0.0f;
 
+    // (the columns' bytes too where the registers allow: the exact forms of the types with eight accumulators a value have few
+    // to spare - with everything held over they spilled and ran 6 % slower - so there only the rows' bytes, which come from
+    // HBM, are asked for ahead, and the columns', which the cache holds, when their turn comes)
+    constexpr bool kColsAhead = !EXACT || G::kLanes == 1;
+    fetch_rows(0);
+    if constexpr (kColsAhead) fetch_cols(0);
     for (int i = 0; i < nb; i++) {
         if (i) __syncthreads(); // the readers of the super-block before are done
-        stage(i);
+        if constexpr (!kColsAhead) fetch_cols(i);
+        stage();
+        if (i + 1 < nb) {
+            fetch_rows(i + 1);
+            if constexpr (kColsAhead) fetch_cols(i + 1);
+        }
         __syncthreads();
         if (!live) continue;
         const float dy = dy_t[wslot + l32];

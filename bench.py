@@ -326,9 +326,11 @@ def prefill_leg(args, bm, ora, threads, gpu, stacks, layer, m, reps=16):
     names = ("quant", "route", "gate", "up", "swiglu_quant", "down", "combine")
 
     def step(i, which=names):
-        if "quant" in which:
+        if "quant" in which and "route" in which:  # the whole step: the two as one launch
+            table.fill_quantize(sel, n_slots, xd, m, act)
+        elif "quant" in which:
             gpu.enqueue_quantize(xd, m, act)
-        if "route" in which:
+        elif "route" in which:
             table.fill(sel, n_slots)
         if "gate" in which:
             gpu.enqueue_gemm(dg, FF, act, table, TOP_K, g)
@@ -537,9 +539,11 @@ def bench_dsv3_prefill(args, bm, ora, threads):
     names = ("quant", "route", "gate", "up", "swiglu_quant", "down", "combine")
 
     def step(i, which=names):
-        if "quant" in which:
+        if "quant" in which and "route" in which:  # the whole step: the two as one launch
+            table.fill_quantize(sel, n_slots, xd, m, act)
+        elif "quant" in which:
             gpu.enqueue_quantize(xd, m, act)
-        if "route" in which:
+        elif "route" in which:
             table.fill(sel, n_slots)
         if "gate" in which:
             gpu.enqueue_gemm(dg, ff, act, table, TOP_K, g)

@@ -80,6 +80,7 @@ SYMBOLS = {
     "bm_route_create": (_i, [_vp, _i, _i, C.POINTER(_vp)]),
     "bm_route_destroy": (None, [_vp]),
     "bm_route_fill": (_i, [_vp, _vp, _i, _vp]),
+    "bm_route_fill_quantize": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp]),
     "bm_route_read": (_i, [_vp, _vp, _vp, _vp, C.POINTER(_i), C.POINTER(_i)]),
     "bm_gemm": (_i, [_vp, _vp, _i, _vp, _vp, _i, _vp]),
     "bm_swiglu_quant": (_i, [_vp, _vp, _vp, _i, _vp, _vp]),
@@ -336,6 +337,11 @@ class Route:
 
     def fill(self, ids, n_slots):
         self.gpu._check(self.gpu.lib.bm_route_fill(self.gpu.ctx, _ptr(ids), n_slots, self.handle))
+        self.n_slots = n_slots
+
+    def fill_quantize(self, ids, n_slots, x, m, act):
+        """fill and Gpu.enqueue_quantize(x, m, act) as one launch (same table, same column bytes)."""
+        self.gpu._check(self.gpu.lib.bm_route_fill_quantize(self.gpu.ctx, _ptr(ids), n_slots, self.handle, _ptr(x), m, act.handle))
         self.n_slots = n_slots
 
     def read(self):

@@ -808,6 +808,22 @@ int bm_route_fill(bm_ctx *ctx, const uint32_t *ids_dev, int n_slots, bm_route *r
     return rc;
 }
 
+int bm_route_fill_quantize(bm_ctx *ctx, const uint32_t *ids_dev, int n_slots, bm_route *route, const float *x_dev, int m, bm_act *act) {
+    const char *what = "bm_route_fill_quantize";
+    if (!ctx || !ids_dev || !route || !x_dev || !act) return fail(ctx, BM_EARG, "%s: NULL argument", what);
+    if (n_slots < 1 || n_slots > route->max_slots)
+        return fail(ctx, BM_ESHAPE, "%s: 1 <= n_slots <= the table's %d slots, got %d", what, route->max_slots, n_slots);
+    if (m < 1 || m > act->m_cap) return fail(ctx, BM_ESHAPE, "%s: m = %d columns, act holds %d", what, m, act->m_cap);
+    if ((reinterpret_cast<uintptr_t>(x_dev) & 15) != 0 || act->k % 256 != 0) { // rows the one launch does not read: the two launches
+        int rc = bm_quantize(ctx, x_dev, m, act);
+        return rc ? rc : bm_route_fill(ctx, ids_dev, n_slots, route);
+    }
+    int rc = driver(ctx, what, bmk::route(launch_of(ctx), ids_dev, n_slots, route->n_experts, route->cols, route->tiles, route->n_tiles,
+                                          act->wtype, x_dev, m, act->k, act->dev));
+    if (!rc) route->filled = n_slots;
+    return rc;
+}
+
 int bm_route_read(bm_ctx *ctx, const bm_route *route, uint32_t *cols_host, uint32_t *tiles_host, int *n_tiles, int *n_refused) {
     const char *what = "bm_route_read";
     if (!ctx || !route || !n_tiles || !n_refused) return fail(ctx, BM_EARG, "%s: NULL argument", what);
@@ -1037,8 +1053,7 @@ int bm_moe_forward(bm_ctx *ctx, bm_scratch *s, const bm_weights *wg, const bm_we
         break;
     }
     default: {
-        int rc = bm_quantize(ctx, x_dev, m, s->act_x);
-        if (!rc) rc = bm_route_fill(ctx, sel_dev, n_slots, s->route);
+        int rc = bm_route_fill_quantize(ctx, sel_dev, n_slots, s->route, x_dev, m, s->act_x);
         if (!rc) rc = bm_gemm(ctx, wg, ff, s->act_x, s->route, spt, s->g);
         if (!rc) rc = bm_gemm(ctx, wu, ff, s->act_x, s->route, spt, s->u);
         if (!rc) rc = bm_swiglu_quant_sel(ctx, s->g, s->u, sel_dev, n_experts, n_slots, rule, s->act_h);

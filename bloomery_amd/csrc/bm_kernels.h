@@ -125,8 +125,10 @@ constexpr int kGemmBN = 64, kGemmBM = 64;
 constexpr int kGemmMaxSlots = 40960, kGemmMaxExperts = 1024;
 int gemm_max_tiles(int n_slots, int n_experts);
 // cols[n_slots], tiles[2 * gemm_max_tiles], n_tiles[3]: tiles, refused slots, slots served elsewhere (not listed)
+// x (optional; 16-byte aligned, k a multiple of 256): in the same launch, quantize() of m rows of k f32 values into act, the
+// column form wtype dots against.
 hipError_t route(const Launch &L, const uint32_t *ids, int n_slots, int n_experts, uint32_t *cols, uint32_t *tiles,
-                 uint32_t *n_tiles);
+                 uint32_t *n_tiles, int wtype = 0, const float *x = nullptr, int m = 0, int k = 0, uint8_t *act = nullptr);
 // q8k: the columns are Q8_K ones (else Q8_2_X4)
 // sel (optional): column c is slot c's; a slot served elsewhere is left as it stands, another id at or past n_experts raises
 hipError_t swiglu_quant(const Launch &L, const float *g, const float *u, int m, int k, uint8_t *act, bool q8k,

@@ -40,8 +40,28 @@ struct RouteLds {
     GroupLds g;
     u32 off[kGroupBuckets];
 };
+// With `x`: behind the table's workgroups (route_blocks of them) further ones quantize m rows of k f32 values into `act`,
+// the column form picked by q8k (Q8_K: a wave a 256-value block; Q8_2_X4: eight values a thread): the prefill step's two
+// first launches, which depend on nothing of each other, as one.
 __global__ __launch_bounds__(kRouteThreads) void k_route(const u32 *ids, u32 n_slots, u32 n_experts, u32 *cols,
-                                                         u32 *tiles, u32 *n_tiles, u32 *fault, u32 layer) {
+                                                         u32 *tiles, u32 *n_tiles, u32 route_blocks, const float *x, int m, int k,
+                                                         int q8k, uint8_t *act, u32 *fault, u32 layer) {
+    if (blockIdx.x >= route_blocks) {
+        const u32 qb = blockIdx.x - route_blocks;
+        if (q8k) {
+            const int b = (int)qb * 16 + (int)(threadIdx.x >> 6), lane = (int)(threadIdx.x & 63);
+            if (b >= m * (k / 256)) return; // whole waves leave
+            q8k_wave_block(*reinterpret_cast<const float4 *>(x + (size_t)b * 256 + 4 * lane), act + (size_t)b * BM_Q8K_STRIDE, lane, fault, layer);
+        } else {
+            const long at = ((long)qb * kRouteThreads + threadIdx.x) * 8;
+            if (at >= (long)m * k) return; // whole quads leave: a block is 32 values, k a multiple of 256
+            const int col = (int)(at / k), o = (int)(at % k);
+            const float4 a = *reinterpret_cast<const float4 *>(x + at), b = *reinterpret_cast<const float4 *>(x + at + 4);
+            const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+            q82_quad8(v, act + (size_t)col * (k / 256) * BM_Q82_SB_EXT, k / 256, o >> 5, threadIdx.x & 3, fault, layer);
+        }
+        return;
+    }
     __shared__ RouteLds lds;
     GroupLds &g = lds.g;
     const u32 tid = threadIdx.x;
@@ -49,7 +69,7 @@ __global__ __launch_bounds__(kRouteThreads) void k_route(const u32 *ids, u32 n_s
         const u32 id = ids[s];
         return id < n_experts ? id : id == 0xffffffffu ? kNoBucket : n_experts;
     });
-    if (blockIdx.x + 1 != gridDim.x) return;
+    if (blockIdx.x + 1 != route_blocks) return;
     const u32 listed = g.base[n_experts + 1];
     for (u32 i = listed + tid; i < n_slots; i += kRouteThreads) cols[i] = 0xffffffffu;
     u32 j0 = 0, j1 = 0;
@@ -74,9 +94,16 @@ __global__ __launch_bounds__(kRouteThreads) void k_route(const u32 *ids, u32 n_s
 }
 
 hipError_t route(const Launch &L, const uint32_t *ids, int n_slots, int n_experts, uint32_t *cols, uint32_t *tiles_out,
-                 uint32_t *n_tiles) {
-    hipLaunchKernelGGL(k_route, dim3(group_parts((u32)n_slots, (u32)n_experts + 1) + 1), dim3(kRouteThreads), 0, L.stream, ids,
-                       (u32)n_slots, (u32)n_experts, cols, tiles_out, n_tiles, L.fault, L.layer);
+                 uint32_t *n_tiles, int wtype, const float *x, int m, int k, uint8_t *act) {
+    const u32 route_blocks = group_parts((u32)n_slots, (u32)n_experts + 1) + 1;
+    u32 quant_blocks = 0;
+    const bool q8k = x && bm_takes_q8k(wtype);
+    if (x) {
+        if (k % 256 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0) return hipErrorInvalidValue;
+        quant_blocks = q8k ? (u32)((m * (k / 256) + 15) / 16) : (u32)(((long)m * k + 8 * kRouteThreads - 1) / (8 * kRouteThreads));
+    }
+    hipLaunchKernelGGL(k_route, dim3(route_blocks + quant_blocks), dim3(kRouteThreads), 0, L.stream, ids, (u32)n_slots, (u32)n_experts,
+                       cols, tiles_out, n_tiles, route_blocks, x, m, k, q8k ? 1 : 0, act, L.fault, L.layer);
     return hipGetLastError();
 }
 

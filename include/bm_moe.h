@@ -310,6 +310,11 @@ void bm_route_destroy(bm_route *route);
  * and listed as refused, and every bm_gemm over the table writes NaN into its rows. A slot whose id is BM_HOST_SLOT is
  * not listed at all and raises nothing (crates/gpu/src/kquant/sel.rs:22-28): no bm_gemm over the table touches its rows. */
 int bm_route_fill(bm_ctx *ctx, const uint32_t *ids_dev, int n_slots, bm_route *route);
+/* bm_route_fill and bm_quantize(ctx, x_dev, m, act) as one launch (the prefill step's two first launches depend on nothing of
+ * each other): the same table and the same column bytes. No counterpart in the reference, which enqueues the two separately
+ * (crates/gpu/src/gemm/route.rs:351 and the card's quantizer). Rows that are not 16-byte aligned or not whole super-blocks go
+ * through the two launches. */
+int bm_route_fill_quantize(bm_ctx *ctx, const uint32_t *ids_dev, int n_slots, bm_route *route, const float *x_dev, int m, bm_act *act);
 /* GemmRoute::read_back / refused_back (route.rs:188-245): synchronise and copy the table out. cols_host (optional)
  * takes the n_slots slot list (refused slots last; behind them BM_HOST_SLOT once for every slot that is not listed);
  * tiles_host (optional) two words a tile: expert, then first index | length << 16. */
@@ -370,7 +375,7 @@ int bm_swiglu_quant_sel(bm_ctx *ctx, const float *g_dev, const float *u_dev, con
  *   BM_PATH_PER_SLOT  bm_moe_decode: two launches, every slot streams its expert's rows (repeats come from the caches);
  *   BM_PATH_GROUPED   bm_tables_quantize, bm_gate_up_tiles (bm_quantize_ord for a down stack on Q8_K columns),
  *                     bm_gemv_tiles, the slots' sum: an expert's rows are read once for all of its slots;
- *   BM_PATH_GEMM      bm_quantize, bm_route_fill, bm_gemm twice, bm_swiglu_quant_sel, bm_gemm, the slots' sum: the int8 matrix
+ *   BM_PATH_GEMM      bm_route_fill_quantize, bm_gemm twice, bm_swiglu_quant_sel, bm_gemm, the slots' sum: the int8 matrix
  *                     cores (in the f32 order bm_set_gemm_mode sets; every stack type bm_gemm takes).
  * In the exact mode all three give the same bits in y_dev. bm_scratch holds what the paths need between their launches for
  * up to max_tokens tokens (made at load time and shared by every layer of the same shape, as the reference's Q8Act scratch

@@ -72,6 +72,45 @@ def test_route_table_made_by_several_workgroups(gpu, n_experts, n_slots, seed):
     ids_d.free()
 
 
+@pytest.mark.parametrize("wtype,k,m,n_experts,top_k,seed", ((bm.Q4_K, 2048, 300, 128, 8, 1), (bm.IQ2_XXS, 1792, 5, 40, 3, 2),
+                                                          (bm.Q6_K, 256, 1, 3, 2, 3), (bm.IQ4_XS, 512, 2100, 256, 8, 4)))
+def test_route_table_and_quantizer_as_one_launch(gpu, wtype, k, m, n_experts, top_k, seed):
+    """bm_route_fill_quantize leaves what bm_route_fill and bm_quantize leave: the table word for word and every column's
+    bytes, in either column form, with a host-served slot and a refused id among the slots, twice in a row; rows that are not
+    16-byte aligned go through the two launches and give the same."""
+    rng = np.random.default_rng(7800 + seed)
+    n_slots = m * top_k
+    ids = rng.integers(0, n_experts, n_slots).astype(np.uint32)
+    if n_slots > 4:
+        ids[1], ids[3] = bm.HOST_SLOT, n_experts + 5
+    x = normal_f32(rng, (m, k))
+    sel, xd = gpu.upload(ids, np.uint32), gpu.upload(np.concatenate([np.zeros(1, np.float32), x.reshape(-1)]), np.float32)
+    xa = gpu.upload(x, np.float32)
+    want_t, want_act = gpu.route(n_slots, n_experts), gpu.act(wtype, k, m)
+    gpu.fault_clear()
+    want_t.fill(sel, n_slots)
+    want_fault = gpu.fault()
+    gpu.enqueue_quantize(xa, m, want_act)
+    want = want_t.read()
+    cols_to_check = sorted({0, m // 3, m // 2, m - 1})
+    for x_ptr, what in ((xd.ptr + 4, "rows 4 bytes off a 16-byte boundary"), (xa, "aligned rows")):
+        t, act = gpu.route(n_slots, n_experts), gpu.act(wtype, k, m)
+        for rep in range(2):
+            gpu.fault_clear()
+            t.fill_quantize(sel, n_slots, x_ptr, m, act)
+            got = t.read()
+            assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]) and got[2] == want[2], what
+            for c in cols_to_check:
+                assert np.array_equal(act.download(c), want_act.download(c)), f"{what}: column {c}"
+            assert np.array_equal(act.download(m - 1), ora.quantize_col(wtype, x[m - 1])), what
+            assert gpu.fault() == want_fault, what
+        t.free()
+        act.free()
+    gpu.fault_clear()
+    for b in (want_t, want_act, sel, xd, xa):
+        b.free()
+
+
 def run_prefill(gpu, L, x, ids, wts, top_k):
     """quantize -> route -> gate GEMM, up GEMM (Shared) -> swiglu_quant -> down GEMM (PerSlot) -> combine
     (crates/gpu/src/arch/qwen3moe/wide.rs:1171-1225)."""

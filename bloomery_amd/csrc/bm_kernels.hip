@@ -17,12 +17,13 @@ namespace bmk {
 // store stands among the loads they time, 4 .. 6 (expert id known, the ring's first super-blocks asked for, columns arrived).
 // The last launch of each kernel is what the table holds.
 #ifdef BM_TIMELINE
+__device__ __forceinline__ unsigned bm_block_linear() { return (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x; }
 constexpr int kTimelineRows = 4096;
 __device__ unsigned long long g_timeline[kTimelineRows * 8];
 #define BM_MARK(base, mark)                                                                                            \
     do {                                                                                                               \
-        if (threadIdx.x == 0 && (base) + blockIdx.x < (unsigned)kTimelineRows)                                         \
-            g_timeline[((base) + blockIdx.x) * 8 + (mark)] = wall_clock64();                                           \
+        if (threadIdx.x == 0 && (base) + bm_block_linear() < (unsigned)kTimelineRows)                                  \
+            g_timeline[((base) + bm_block_linear()) * 8 + (mark)] = wall_clock64();                                           \
     } while (0)
 // BM_TICK keeps the counter in a register once `dep` has arrived (no store among the loads it times); BM_TOCK stores it.
 #define BM_TICK(var, dep)                                                                                              \
@@ -33,8 +34,8 @@ __device__ unsigned long long g_timeline[kTimelineRows * 8];
     } while (0)
 #define BM_TOCK(base, mark, var)                                                                                       \
     do {                                                                                                               \
-        if (threadIdx.x == 0 && (base) + blockIdx.x < (unsigned)kTimelineRows)                                         \
-            g_timeline[((base) + blockIdx.x) * 8 + (mark)] = var;                                                      \
+        if (threadIdx.x == 0 && (base) + bm_block_linear() < (unsigned)kTimelineRows)                                  \
+            g_timeline[((base) + bm_block_linear()) * 8 + (mark)] = var;                                                      \
     } while (0)
 #else
 #define BM_MARK(base, mark)                                                                                            \
@@ -361,11 +362,13 @@ template <int WT, int U, int NB>
 __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w, u32 n_experts, int nb,
                                                   const uint8_t *act, const u32 *sel, const float *wts,
                                                   const float *resid, int spt, int rpe, float *y, int t, int rb,
-                                                  u32 *fault, u32 layer) {
+                                                  u32 *fault, u32 layer, int spt_shift = -1) {
     const int tid = threadIdx.x, q = tid & 3, quad = tid >> 2;
     BM_MARK(2048, 0);
-    const int D = 64 / spt;
-    const int e = quad % spt, dl = quad / spt;
+    // (spt_shift: log2 of a power-of-two spt, else -1: the divisions by a count only known at run time are some eighty
+    // instructions at the head of a workgroup whose first request waits for them)
+    const int D = spt_shift >= 0 ? 64 >> spt_shift : 64 / spt;
+    const int e = spt_shift >= 0 ? quad & (spt - 1) : quad % spt, dl = spt_shift >= 0 ? quad >> spt_shift : quad / spt;
     const int r = rb * D + dl;
     const int slot = t * spt + e;
     const u32 id = sel[slot];
@@ -418,12 +421,11 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
 template <int WT, int U, int NB>
 __global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_experts, int nb, const uint8_t *act,
                                                       const u32 *sel, const float *wts, const float *resid, int spt,
-                                                      int rpe, float *y, u32 *fault, u32 layer) {
+                                                      int rpe, float *y, u32 *fault, u32 layer, int spt_shift) {
     extern __shared__ __align__(16) uint8_t lds[];
-    const int D = 64 / spt;
-    const int blocks_per_token = (rpe + D - 1) / D;
-    down_combine_body<WT, U, NB>(lds, w, n_experts, nb, act, sel, wts, resid, spt, rpe, y,
-                                 blockIdx.x / blocks_per_token, blockIdx.x % blocks_per_token, fault, layer);
+    // the grid: (row blocks of a token, tokens)
+    down_combine_body<WT, U, NB>(lds, w, n_experts, nb, act, sel, wts, resid, spt, rpe, y, (int)blockIdx.y, (int)blockIdx.x, fault, layer,
+                                 spt_shift);
 }
 
 // k_down_combine for a Q6_K stack of NB super-blocks a row with the row's super-blocks dealt to the waves (BM_DOWN_SPLIT, the
@@ -520,12 +522,11 @@ __global__ __launch_bounds__(256 * NB) void k_down_combine_q6k_split(const uint8
 template <int WA, int UA, int NBA>
 __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, const uint8_t *wg, const uint8_t *wu,
                                                u32 n_experts, int na, int nh, const u32 *sel, int spt, uint8_t *act_x,
-                                               uint8_t *act_h, float *h, int slot, int rb, GateRule rule, u32 *fault,
+                                               uint8_t *act_h, float *h, int slot, int rb, int t, GateRule rule, u32 *fault,
                                                u32 layer) {
     const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
     BM_MARK(0, 0);
     const int hidden = na * 256, ff = nh * 256;
-    const int t = slot / spt;
     const int r = rb * 32 + (tid >> 3);
     const u32 id = sel[slot];
     const int col_bytes = bm_act_col_bytes<WA>(na);
@@ -591,9 +592,9 @@ __global__ __launch_bounds__(256) void k_gate_up_x(const float *x, const uint8_t
                                                    int nba, int nh, const u32 *sel, int spt, uint8_t *act_x,
                                                    uint8_t *act_h, float *h, GateRule rule, u32 *fault, u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
-    const int blocks_per_slot = nh * 8;
+    // the grid: (blocks of 32 rows, slots of a token, tokens): no division stands before the workgroup's first request
     gate_up_x_body<WA, UA, NBA>(lds, x, wg, wu, n_experts, NBA > 0 ? NBA : nba, nh, sel, spt, act_x, act_h, h,
-                                blockIdx.x / blocks_per_slot, blockIdx.x % blocks_per_slot, rule, fault, layer);
+                                (int)(blockIdx.z * gridDim.y + blockIdx.y), (int)blockIdx.x, (int)blockIdx.z, rule, fault, layer);
 }
 
 // ------------------------------------------------------------- the fused step for the types that take Q8_K columns
@@ -940,6 +941,7 @@ hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_expe
                         int rows_per_expert, float *y) {
     const int nb = k / 256, rpe = rows_per_expert, spt = slots_per_token;
     const int D = 64 / spt;
+    const int spt_shift = (spt & (spt - 1)) == 0 ? __builtin_ctz((unsigned)spt) : -1;
     const size_t lds = down_combine_lds(wtype, k, spt);
     const unsigned grid = (unsigned)m * (unsigned)((rpe + D - 1) / D);
     if (L.down_form == 1 && wtype == BM_Q6K && nb == 3 && 64 % spt == 0) { // BM_DOWN_SPLIT where it is built: the super-blocks of a row dealt to the waves
@@ -953,8 +955,8 @@ hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_expe
     auto kern = k_down_combine<WT, U, NB>;                                                                             \
     hipError_t e = allow_lds(kern, lds);                                                                               \
     if (e != hipSuccess) return e;                                                                                     \
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act, sel, wts, resid, spt,   \
-                       rpe, y, L.fault, L.layer);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((rpe + D - 1) / D), (unsigned)m), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act,  \
+                       sel, wts, resid, spt, rpe, y, L.fault, L.layer, spt_shift);
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
     return hipGetLastError();
@@ -978,8 +980,8 @@ hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8
         auto kern = k_gate_up_x<WA, UA, NA>;                                                                           \
         hipError_t e = allow_lds(kern, lds_a);                                                                         \
         if (e != hipSuccess) return e;                                                                                 \
-        hipLaunchKernelGGL(kern, dim3(grid_a), dim3(256), lds_a, L.stream, x, wg, wu, (u32)n_experts, nba, nbb, sel,   \
-                           spt, act_x, act_h, h, L.rule, L.fault, L.layer);                                            \
+        hipLaunchKernelGGL(kern, dim3((unsigned)(ff / 32), (unsigned)spt, (unsigned)m), dim3(256), lds_a, L.stream, x, wg, wu,          \
+                           (u32)n_experts, nba, nbb, sel, spt, act_x, act_h, h, L.rule, L.fault, L.layer);                                 \
     }
     if (gate_type == BM_Q4K) {
         if (nba == 8) BM_GUX(BM_Q4K, kRingQ4K, 8)

@@ -23,6 +23,9 @@ struct bm_ctx {
     uint32_t *fault = nullptr;
     uint32_t layer = BM_LAYER_NONE;
     uint32_t *route_hand = nullptr; // bm_norm_route's hand-over words, one a (token, expert), bmk::kRouteArmed between launches
+    // polls a routing wave of bm_norm_route waits for its logits (BM_NORM_ROUTE_POLLS in the environment when the context is
+    // made, for the tests of the give-up path: the kernels end normally either way)
+    uint32_t route_polls = bmk::kRoutePolls;
     int gemm_mode = BM_GEMM_EXACT;
     int down_form = BM_DOWN_RING;
     bmk::GateRule rule = {0u, 0.0f}; // silu(g) * u
@@ -101,6 +104,10 @@ static int ctx_make(int device, hipStream_t stream, bool own, bm_ctx **out) {
     bm_ctx *c = new (std::nothrow) bm_ctx();
     if (!c) return fail(nullptr, BM_EDRIVER, "bm_ctx_create: out of host memory");
     c->device = device;
+    if (const char *polls = getenv("BM_NORM_ROUTE_POLLS")) {
+        const long v = atol(polls);
+        if (v >= 1 && v <= (long)bmk::kRoutePolls) c->route_polls = (uint32_t)v;
+    }
     if (own) {
         e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking); // default priority
         if (e != hipSuccess) {
@@ -1223,7 +1230,7 @@ int bm_norm_route(bm_ctx *ctx, const float *router_dev, const float *x_dev, cons
                     act_x->k);
     return driver(ctx, what, bmk::norm_route(launch_of(ctx), router_dev, x_dev, gain_dev, eps, n_tokens, n_experts, hidden, normed_dev,
                                              logits_dev, top_k, renorm != 0, probs_dev, ids_dev, weights_dev, ctx->route_hand,
-                                             act_x ? act_x->dev : nullptr, act_x && act_form(act_x->wtype) != 0));
+                                             act_x ? act_x->dev : nullptr, act_x && act_form(act_x->wtype) != 0, ctx->route_polls));
 }
 
 int bm_block_sums(bm_ctx *ctx, const bm_weights *w, int64_t row, const bm_act *act, int col, int32_t *out_dev) {

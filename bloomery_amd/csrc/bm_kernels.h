@@ -162,10 +162,13 @@ bool router_logits_fits(int hidden);
 // not overlap. kRouteArmed is a signalling NaN's pattern: no logit has it, arithmetic only ever leaves the quiet form.
 constexpr int kNormRouteMaxTokens = 4096;
 constexpr uint32_t kRouteArmed = 0x7fa00001u;
+// polls after which a routing wave gives a token up (BM_SITE_ROUTER, NaN weights): some ten seconds; only a launch that
+// lost its other workgroups gets there
+constexpr uint32_t kRoutePolls = 1u << 24;
 // act_x (optional; hidden a multiple of 256): the tokens' normed rows as quantized columns (q8k: Q8_K, else Q8_2_X4 with tables)
 hipError_t norm_route(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                       int hidden, float *normed_out, float *logits, int used, int renorm, float *probs, uint32_t *ids,
-                      float *weights, uint32_t *hand, uint8_t *act_x = nullptr, bool q8k = false);
+                      float *weights, uint32_t *hand, uint8_t *act_x = nullptr, bool q8k = false, uint32_t max_polls = kRoutePolls);
 hipError_t router_logits(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                          int hidden, float *normed_out, float *logits);
 

@@ -500,17 +500,17 @@ __global__ __launch_bounds__(256) void k_router_logits(const float *router, cons
 // before, a count raised behind acknowledged stores by the last workgroup to finish, which then read the logits back: 10.3
 // us a token against this one's figure in the bench line). The wave arms its words again before it ends, so a graph replay
 // needs no memset. A routing workgroup comes after every workgroup it waits for in the grid, so those are dispatched
-// whatever else the card runs; the wait is bounded all the same (kRouteSpins polls, then BM_SITE_ROUTER and NaN weights), and
+// whatever else the card runs; the wait is bounded all the same (max_polls polls, kRoutePolls = 2^24 or some ten seconds unless the caller says otherwise - an XCD busy with another stream's work may hold some of them back for
+// a while - then BM_SITE_ROUTER and NaN weights), and
 // every wave ends. Launches over the same `hand` must not overlap.
 // With act_x (the reference launch's quantizer, route_softmax.rs:1679): one more workgroup a token, between the two kinds in
 // the grid, norms the token's row the same way and leaves it as the token's quantized column (q8k: a Q8_K column, else a
 // Q8_2_X4 one with its tables), the bytes bm_quantize makes of normed_out. The routing waits for none of it.
-constexpr u32 kRouteSpins = 1u << 20;
 template <int R, int PER>
 __global__ __launch_bounds__(256) void k_norm_route(const float *router, const float *x, const float *gain, float eps, int n_exp,
                                                     int hidden, float *normed_out, float *logits, u32 used, u32 renorm,
                                                     float *probs, u32 *ids, float *weights, u32 *hand, uint8_t *act_x,
-                                                    int q8k, int m, u32 *fault, u32 layer) {
+                                                    int q8k, int m, u32 *fault, u32 layer, u32 max_polls) {
     extern __shared__ __align__(16) uint8_t lds[];
     const u32 blocks_per_token = (u32)((n_exp + R - 1) / R);
     const u32 n_logit_blocks = (u32)m * blocks_per_token, n_quant_blocks = act_x ? (u32)m : 0u;
@@ -532,7 +532,7 @@ __global__ __launch_bounds__(256) void k_norm_route(const float *router, const f
             BM_RTICK(tl_start, lane);
             u32 w[PER];
             bool late = true;
-            for (u32 spin = 0; spin < kRouteSpins && late; spin++) {
+            for (u32 spin = 0; spin < max_polls && late; spin++) {
                 bool armed = false;
 #pragma unroll
                 for (int j = 0; j < PER; j++) {
@@ -644,7 +644,7 @@ hipError_t router_logits(const Launch &L, const float *router, const float *x, c
 
 hipError_t norm_route(const Launch &L, const float *router, const float *x, const float *gain, float eps, int m, int n_exp,
                       int hidden, float *normed_out, float *logits, int used, int renorm, float *probs, uint32_t *ids,
-                      float *weights, uint32_t *hand, uint8_t *act_x, bool q8k) {
+                      float *weights, uint32_t *hand, uint8_t *act_x, bool q8k, uint32_t max_polls) {
     const int rows = router_rows(hidden, m, n_exp);
     if (rows == 0) return hipErrorInvalidValue;
     if (act_x && hidden % 256 != 0) return hipErrorInvalidValue;
@@ -656,7 +656,7 @@ hipError_t norm_route(const Launch &L, const float *router, const float *x, cons
         hipError_t e = allow_lds(kern, lds);                                                                           \
         if (e != hipSuccess) return e;                                                                                 \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, router, x, gain, eps, n_exp, hidden, normed_out, \
-                           logits, (u32)used, (u32)renorm, probs, ids, weights, hand, act_x, q8k ? 1 : 0, m, L.fault, L.layer); \
+                           logits, (u32)used, (u32)renorm, probs, ids, weights, hand, act_x, q8k ? 1 : 0, m, L.fault, L.layer, max_polls); \
     }
 #define BM_NR_ROWS(PER)                                                                                                \
     {                                                                                                                  \

@@ -435,7 +435,8 @@ int bm_router_logits(bm_ctx *ctx, const float *router_dev, const float *x_dev, c
  * bm_gate_up over act_x then takes the place of bm_gate_up_x / bm_moe_decode's first launch over normed_dev. One workgroup
  * a token, behind the logits' workgroups in the grid, takes the token's logits as they land (words of the context that
  * hold an armed pattern between launches; its wait is bounded: BM_SITE_ROUTER and NaN weights if a logit never came) and
- * routes the token. logits_dev is required; 1 .. 4096 tokens a launch. Launches of this entry that share a context must not
+ * routes the token (after a wait that ran out: bm_fault_clear, which arms the words again, before the next call).
+ * logits_dev is required; 1 .. 4096 tokens a launch. Launches of this entry that share a context must not
  * overlap (they share those words). */
 int bm_norm_route(bm_ctx *ctx, const float *router_dev, const float *x_dev, const float *gain_dev, float eps, int n_tokens,
                   int n_experts, int hidden, int top_k, int renorm, float *normed_dev, float *logits_dev, float *probs_dev,

@@ -330,6 +330,44 @@ def test_norm_route_picks_among_equal_probabilities(gpu, n_experts, top_k):
         b.free()
 
 
+def test_norm_route_gives_a_token_up_when_its_logits_do_not_come(gpu, monkeypatch):
+    """The routing wave's wait is bounded: a context made with BM_NORM_ROUTE_POLLS=1 lets it look once, right after the
+    launch started, when no logit of a single token's launch can be there yet; it then raises Router, leaves NaN weights,
+    and every workgroup ends (the call returns, the context stays usable); bm_fault_clear arms the words again, and the
+    module's own context, made without the variable, routes the same token."""
+    n_experts, hidden, top_k = 128, 2048, 8
+    rng = np.random.default_rng(77)
+    router, x = normal_f32(rng, (n_experts, hidden), 0.05), normal_f32(rng, (1, hidden))
+    monkeypatch.setenv("BM_NORM_ROUTE_POLLS", "1")
+    hasty = bm.Gpu(0)
+    monkeypatch.delenv("BM_NORM_ROUTE_POLLS")
+    try:
+        rd, xd = hasty.upload(router, np.float32), hasty.upload(x, np.float32)
+        logits, ids, wts = hasty.buffer(np.float32, n_experts), hasty.buffer(np.uint32, top_k).fill_bytes(0), hasty.buffer(np.float32, top_k)
+        for rep in range(2):
+            hasty.fault_clear()
+            wts.fill_bytes(0)
+            hasty.enqueue_norm_route(rd, xd, None, 0.0, 1, n_experts, hidden, top_k, True, None, logits, None, ids, wts)
+            assert hasty.fault()[1] == 1 << bm.SITE_ROUTER, f"call {rep}"
+            assert np.isnan(wts.download()).all(), f"call {rep}"
+            # the logits themselves are written whatever became of the routing
+            assert np.array_equal(logits.download().view(np.uint32), ora.router_logits(router, x, None, 0.0)[1][0].view(np.uint32))
+        hasty.fault_clear()
+        for b in (rd, xd, logits, ids, wts):
+            b.free()
+    finally:
+        hasty.close()
+    rd, xd = gpu.upload(router, np.float32), gpu.upload(x, np.float32)
+    logits, ids, wts = gpu.buffer(np.float32, n_experts), gpu.buffer(np.uint32, top_k), gpu.buffer(np.float32, top_k)
+    gpu.fault_clear()
+    gpu.enqueue_norm_route(rd, xd, None, 0.0, 1, n_experts, hidden, top_k, True, None, logits, None, ids, wts)
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    want_ids, _ = ora.route_softmax_topk(logits.download(), top_k)
+    assert np.array_equal(ids.download(), want_ids)
+    for b in (rd, xd, logits, ids, wts):
+        b.free()
+
+
 def test_norm_route_raises_and_refuses_like_its_parts(gpu):
     """A logit that is not finite (a NaN in the token's row) raises Router from the fused launch too, and the other
     tokens are routed; the argument checks are the two entries' own, by name."""

@@ -593,6 +593,9 @@ def bench_paths(args, bm, ora, threads):
     crossovers behind its automatic choice. A side measurement."""
     wg, wu, wd = make_layer(ora, 0xB1000001, threads)
     counts = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256, 512, 1024)
+    if args.path_tokens:  # a few counts only (the run to put under a profiler)
+        counts = tuple(sorted(int(t) for t in args.path_tokens.split(",")))
+        assert all(1 <= t <= 1024 for t in counts), "--path-tokens: counts of 1 .. 1024"
     m_max, sets = counts[-1], 4
     x = np.random.default_rng(0xAC70001).standard_normal((m_max, HIDDEN), dtype=np.float32)
     ids, wts = biased_routes(ora, m_max * sets, N_EXPERTS, TOP_K, 0x707E0001, bias_sigma=0.5)
@@ -631,7 +634,8 @@ def bench_paths(args, bm, ora, threads):
     auto = {m: {bm.PATH_PER_SLOT: "per_slot", bm.PATH_GROUPED: "grouped", bm.PATH_GEMM: "gemm_exact"}[sc.path_for(m)] for m in counts}
     assert gpu.fault() == (bm.FAULT_NONE, 0)
     worst = max(r[auto[r["tokens"]]] / r[r["fastest_exact"]] for r in rows)
-    emit("moe_layer_us_per_step_by_path", rows[5]["per_slot"], "us/step", 0, 0, rows[5]["per_slot"] * 1e-3,
+    head = next((r for r in rows if r["tokens"] == 16), rows[0])
+    emit("moe_layer_us_per_step_by_path", head["per_slot"], "us/step", 0, 0, head["per_slot"] * 1e-3,
          "Qwen3-30B-A3B-shaped MoE layer, 1 to 1024 tokens a step through each path of bm_moe_forward, config 3's routing "
          "(a side measurement: which path for how many tokens)",
          {"us_per_step": rows, "automatic_choice": auto, "automatic_over_fastest_worst_case": worst},
@@ -881,6 +885,7 @@ def main():
                          "6: the card rule's down step (a side measurement); 7: DeepSeek-V3-shaped IQ2_XXS experts at prefill (a side "
                          "measurement); 8: the three paths of bm_moe_forward over the number of tokens (a side measurement)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--path-tokens", default="", help="config 8 only: the token counts to run, comma separated (default: the whole sweep)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="config 2 only: no timing; 8 copies of 64 MiB by a plain kernel (the counters' calibration), then "
                          "256 eager steps - the run to put under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")

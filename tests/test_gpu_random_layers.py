@@ -1,6 +1,6 @@
 """Layers of random shape through every path of the library against the CPU oracle, bit for bit: weight types drawn from
 all that the path takes, hidden and ff any number of super-blocks, 1 .. 79 tokens, 1 .. 4 slots a token over 1 .. 8 experts
-(so runs from a single slot to several GEMM tiles). Each case runs the per-slot chain or its fused form, the fused
+(so runs from a single slot to several GEMM tiles), in three cases of ten a few tokens over up to 40 experts. Each case runs the per-slot chain or its fused form, the fused
 two-launch step, the grouped GEMM step in both f32 modes where the types have one, and bm_moe_forward on each of its
 paths. The fixed-shape tests beside this one hold the named configurations; this one holds what lies between them."""
 import numpy as np
@@ -14,9 +14,7 @@ from test_gpu_prefill import run_prefill
 
 pytestmark = pytest.mark.gpu
 
-K_TYPES = (bm.Q4_K, bm.Q5_K, bm.Q6_K)
-GEMM_TYPES = K_TYPES + (bm.IQ2_XXS,)
-ALL_TYPES = GEMM_TYPES + (bm.Q3_K, bm.IQ3_XXS, bm.IQ4_XS)
+ALL_TYPES = (bm.Q4_K, bm.Q5_K, bm.Q6_K, bm.IQ2_XXS, bm.Q3_K, bm.IQ3_XXS, bm.IQ4_XS)
 
 
 def same_bits(got, want, what):
@@ -29,10 +27,11 @@ def test_random_layers_every_path(gpu, seed):
     rng = np.random.default_rng(9000 + seed)
     for case in range(8):
         with_gemm = rng.random() < 0.6
-        pool = GEMM_TYPES if with_gemm else ALL_TYPES
-        tg, td = pool[rng.integers(len(pool))], pool[rng.integers(len(pool))]
+        tg, td = ALL_TYPES[rng.integers(len(ALL_TYPES))], ALL_TYPES[rng.integers(len(ALL_TYPES))]
         hidden, ff = 256 * int(rng.integers(1, 9)), 256 * int(rng.integers(1, 5))
         n_experts, m = int(rng.integers(1, 9)), int(rng.integers(1, 80))
+        if rng.random() < 0.3:  # more experts than slots: bm_moe_forward's grouped form of few slots an expert among the cases
+            n_experts, m = int(rng.integers(9, 41)), int(rng.integers(1, 9))
         top_k = min(int(rng.integers(1, 5)), n_experts)
         tag = f"seed {seed} case {case}: types {tg}/{td}, hidden {hidden}, ff {ff}, {n_experts} experts, {m} tokens, top-{top_k}"
         L = Layer(gpu, (tg, tg, td), hidden, ff, n_experts, 9100 + 16 * seed + case, cheap=True)

@@ -421,9 +421,10 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
 template <int WT, int U, int NB>
 __global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_experts, int nb, const uint8_t *act,
                                                       const u32 *sel, const float *wts, const float *resid, int spt,
-                                                      int rpe, float *y, u32 *fault, u32 layer, int spt_shift) {
+                                                      int rpe, int spt_shift, float *y, u32 *fault, u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
-    // the grid: (row blocks of a token, tokens)
+    // the grid: (row blocks of a token, tokens). (spt_shift stands among the first sixteen argument words, which are in
+    // registers when the wave starts: behind them it was a load from memory in front of the workgroup's first request)
     down_combine_body<WT, U, NB>(lds, w, n_experts, nb, act, sel, wts, resid, spt, rpe, y, (int)blockIdx.y, (int)blockIdx.x, fault, layer,
                                  spt_shift);
 }
@@ -463,7 +464,7 @@ __global__ __launch_bounds__(256 * NB) void k_down_combine_q6k_split(const uint8
     constexpr size_t row_bytes = (size_t)NB * BM_Q6K_BLOCK;
     constexpr int col_bytes = bm_act_col_bytes<WT>(NB);
     const uint8_t *act_cols = act + (size_t)t * spt * col_bytes;
-    Stage<2> st; // 16 bytes a thread of 768: the eight columns of 1248 bytes
+    Stage<2, 256 * NB> st; // 16 bytes a thread of 768: the eight columns of 1248 bytes
     st.load(act_cols, spt * col_bytes);
     if (!live && id != 0xffffffffu && rb == 0 && dl == 0 && q == 0 && i == 0) bm_raise(fault, layer, kSiteExpertId);
     const uint8_t *wrow = w + ((size_t)(live ? id : 0) * rpe + (active ? r : 0)) * row_bytes;
@@ -530,9 +531,10 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
     const int r = rb * 32 + (tid >> 3);
     const u32 id = sel[slot];
     const int col_bytes = bm_act_col_bytes<WA>(na);
-    uint8_t *hcol = act_h ? act_h + (size_t)slot * nh * BM_Q82_SB_EXT : nullptr; // none: the down stack takes Q8_K columns
     uint8_t *col = lds;
-    // the token's row: eight consecutive values a lane, 2048 a pass
+    // the token's row: eight consecutive values a lane, 2048 a pass. Asked for before anything reads an argument that is
+    // not in a register when the wave starts (the first thirteen words are): scalar loads come back in any order, so the
+    // first wait for one of them is a wait for the expert id as well, and the row's loads would stand behind it
     constexpr int kPasses = NBA > 0 ? (NBA * 256 + 2047) / 2048 : 1;
     float xv[kPasses][8];
 #pragma unroll
@@ -546,6 +548,7 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
     }
     __asm__ volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
+    uint8_t *hcol = act_h ? act_h + (size_t)slot * nh * BM_Q82_SB_EXT : nullptr; // none: the down stack takes Q8_K columns
     if (id >= n_experts) { // uniform over the workgroup
         if (id == 0xffffffffu) return; // a slot served elsewhere: nothing written, nothing raised
         if (tid == 0) bm_raise(fault, layer, kSiteExpertId);
@@ -592,9 +595,10 @@ __global__ __launch_bounds__(256) void k_gate_up_x(const float *x, const uint8_t
                                                    int nba, int nh, const u32 *sel, int spt, uint8_t *act_x,
                                                    uint8_t *act_h, float *h, GateRule rule, u32 *fault, u32 layer) {
     extern __shared__ __align__(16) uint8_t lds[];
-    // the grid: (blocks of 32 rows, slots of a token, tokens): no division stands before the workgroup's first request
+    // the grid: (blocks of 32 rows, slots of a token, tokens): no division stands before the workgroup's first request (and no
+    // read of the grid's size, which comes from the dispatch packet in memory: spt is an argument, in a register at the start)
     gate_up_x_body<WA, UA, NBA>(lds, x, wg, wu, n_experts, NBA > 0 ? NBA : nba, nh, sel, spt, act_x, act_h, h,
-                                (int)(blockIdx.z * gridDim.y + blockIdx.y), (int)blockIdx.x, (int)blockIdx.z, rule, fault, layer);
+                                (int)blockIdx.z * spt + (int)blockIdx.y, (int)blockIdx.x, (int)blockIdx.z, rule, fault, layer);
 }
 
 // ------------------------------------------------------------- the fused step for the types that take Q8_K columns
@@ -956,7 +960,7 @@ hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_expe
     hipError_t e = allow_lds(kern, lds);                                                                               \
     if (e != hipSuccess) return e;                                                                                     \
     hipLaunchKernelGGL(kern, dim3((unsigned)((rpe + D - 1) / D), (unsigned)m), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act,  \
-                       sel, wts, resid, spt, rpe, y, L.fault, L.layer, spt_shift);
+                       sel, wts, resid, spt, rpe, spt_shift, y, L.fault, L.layer);
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
     return hipGetLastError();

@@ -91,15 +91,16 @@ __device__ __forceinline__ void stage_bytes(uint8_t *dst, const uint8_t *src, in
 
 // The same copy in two halves: R unconditional loads a thread (offsets past the end are clamped onto the last
 // word, so no branch stands between them and the weight loads that follow), then the LDS stores. Memory returns
-// in order, so the stores wait for these loads only. Bytes past R * 8 * blockDim are copied afterwards by
-// stage_bytes' loop (that part waits for everything in flight).
-template <int R>
+// in order, so the stores wait for these loads only. Bytes past R * 8 * T are copied afterwards by
+// stage_bytes' loop (that part waits for everything in flight). T: the workgroup's thread count, a constant here: the
+// built-in is read from memory, a round trip in front of the workgroup's first requests.
+template <int R, int T = 256>
 struct Stage {
     uint2 v[R];
     __device__ __forceinline__ void load(const uint8_t *src, int bytes) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            int o = (r * (int)blockDim.x + (int)threadIdx.x) * 8;
+            int o = (r * T + (int)threadIdx.x) * 8;
             o = o < bytes ? o : bytes - 8;
             v[r] = *reinterpret_cast<const uint2 *>(src + o);
         }
@@ -110,10 +111,10 @@ struct Stage {
     __device__ __forceinline__ void store(uint8_t *dst, const uint8_t *src, int bytes) const {
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const int o = (r * (int)blockDim.x + (int)threadIdx.x) * 8;
+            const int o = (r * T + (int)threadIdx.x) * 8;
             if (o < bytes) *reinterpret_cast<uint2 *>(dst + o) = v[r];
         }
-        for (int o = (R * (int)blockDim.x + (int)threadIdx.x) * 8; o < bytes; o += (int)blockDim.x * 8)
+        for (int o = (R * T + (int)threadIdx.x) * 8; o < bytes; o += T * 8)
             *reinterpret_cast<uint2 *>(dst + o) = *reinterpret_cast<const uint2 *>(src + o);
     }
 };

@@ -328,6 +328,66 @@ hipError_t combine_tokens(const Launch &L, const float *down, const float *w, co
     return hipGetLastError();
 }
 
+// An argument read from the launch's argument block at the place in the code where this call stands. The first fourteen
+// words of the block are in registers when a wave starts; an argument behind them is a scalar load, and the compiler asks
+// for it at the top of the kernel: scalar loads come back in any order, so the first wait for one of them - the expert id's -
+// would be a wait for those words as well. The arguments the head of a decode launch does not need stand at the end of its
+// list as one struct, which the kernel does not touch, and are read through this behind the launch's first requests.
+template <class T>
+__device__ __forceinline__ T bm_kernarg_at(unsigned offset) {
+    static_assert(sizeof(T) % 4 == 0, "whole words");
+    typedef __attribute__((address_space(4))) const uint8_t *Block;
+    typedef __attribute__((address_space(4))) const u32 *Words;
+    const Words from = (Words)((Block)__builtin_amdgcn_kernarg_segment_ptr() + offset);
+    struct Raw {
+        u32 w[sizeof(T) / 4];
+    } raw;
+#pragma unroll
+    for (unsigned i = 0; i < sizeof(T) / 4; i++) raw.w[i] = from[i];
+    return __builtin_bit_cast(T, raw);
+}
+
+// A pointer that came out of bm_kernarg_at's words, as what a pointer argument is: an address in global memory (without this
+// the compiler takes it for one that may also lie in LDS or scratch, and every wait for a vector load behind its first use is
+// a wait for all of them).
+template <class P>
+__device__ __forceinline__ P *bm_global(P *p) {
+    return (P *)(__attribute__((address_space(1))) P *)(uintptr_t)p;
+}
+
+struct DownLate { // the end of k_down_combine's arguments
+    float *y;
+    u32 *fault;
+    u32 layer;
+};
+struct DownArgs { // k_down_combine's argument block
+    const uint8_t *w;
+    u32 n_experts;
+    int nb;
+    const uint8_t *act;
+    const u32 *sel;
+    const float *wts, *resid;
+    int spt_word, rpe;
+    DownLate late;
+};
+struct GateUpLate { // the end of k_gate_up_x's arguments
+    uint8_t *act_x, *act_h;
+    float *h;
+    GateRule rule;
+    u32 *fault;
+    u32 layer;
+};
+struct GateUpArgs { // k_gate_up_x's argument block
+    const float *x;
+    const uint8_t *wg, *wu;
+    u32 n_experts;
+    int nba, nh;
+    const u32 *sel;
+    int spt;
+    GateUpLate late;
+};
+static_assert(offsetof(DownArgs, late) == 56 && offsetof(GateUpArgs, late) == 56, "fourteen words in front of the late arguments");
+
 // --------------------------------------------------------------------------- down + combine in one launch
 
 // A row's closing sum over its token's slots in slot order, acc = fma(w_s, v_s, acc) for the live slots, then the
@@ -358,26 +418,35 @@ __device__ __forceinline__ float slot_sum(const float *v, const float *w, const 
 
 // The shared body of the down + combine workgroup: token t, output rows rb * D .. + D with D = 64 / spt, a quad for
 // every (row, slot).
-template <int WT, int U, int NB>
+template <int WT, int U, int NB, bool EIGHT = false>
 __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w, u32 n_experts, int nb,
                                                   const uint8_t *act, const u32 *sel, const float *wts,
-                                                  const float *resid, int spt, int rpe, float *y, int t, int rb,
-                                                  u32 *fault, u32 layer, int spt_shift = -1) {
+                                                  const float *resid, int spt, int rpe, int t, int rb, int spt_shift = -1) {
     const int tid = threadIdx.x, q = tid & 3, quad = tid >> 2;
     BM_MARK(2048, 0);
+    if constexpr (EIGHT) spt = 8, spt_shift = 3; // what the launcher has checked: constants from here on
     // (spt_shift: log2 of a power-of-two spt, else -1: the divisions by a count only known at run time are some eighty
     // instructions at the head of a workgroup whose first request waits for them)
     const int D = spt_shift >= 0 ? 64 >> spt_shift : 64 / spt;
     const int e = spt_shift >= 0 ? quad & (spt - 1) : quad % spt, dl = spt_shift >= 0 ? quad >> spt_shift : quad / spt;
     const int r = rb * D + dl;
     const int slot = t * spt + e;
-    const u32 id = sel[slot];
+    // eight slots a token: the token's ids through the scalar cache (one request a wave, a shorter way than a vector load's);
+    // the lane picks its own out of the eight registers further down, behind the vector requests that do not wait for it
+    constexpr bool eight = EIGHT; // (a variant of its own: a run-time choice leaves the id's register waiting for either way's load)
+    u32 i8[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    u32 id = 0;
+    if constexpr (eight) {
+        const u32 *s8 = sel + (size_t)t * 8;
+#pragma unroll
+        for (int k = 0; k < 8; k++) i8[k] = s8[k];
+    } else {
+        id = sel[slot];
+    }
     // the token's ids and weights for the closing sum, requested now and parked in LDS
     const int si = tid < spt ? tid : 0;
     const u32 my_sel = sel[t * spt + si];
     const float my_w = wts[t * spt + si];
-    const bool live = id < n_experts;
-    const bool active = dl < D && r < rpe && live;
     // the residual value of the row this thread closes, asked for now: at the end it would be a memory round trip
     const float resid_v = resid && tid < D && rb * D + tid < rpe ? resid[(size_t)t * rpe + rb * D + tid] : 0.0f;
     const int n = NB > 0 ? NB : nb;
@@ -387,7 +456,14 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
     // the token's columns are asked for before anything waits for the expert id: they arrive with it
     Stage<5> st;
     st.load(act_cols, spt * col_bytes);
-    if (!live && id != 0xffffffffu && rb == 0 && dl == 0 && q == 0) bm_raise(fault, layer, kSiteExpertId);
+    if constexpr (eight) {
+        __builtin_amdgcn_sched_barrier(0);
+        const u32 a = (e & 1) ? i8[1] : i8[0], b2 = (e & 1) ? i8[3] : i8[2], c = (e & 1) ? i8[5] : i8[4], d = (e & 1) ? i8[7] : i8[6];
+        const u32 ab = (e & 2) ? b2 : a, cd = (e & 2) ? d : c;
+        id = (e & 4) ? cd : ab;
+    }
+    const bool live = id < n_experts;
+    const bool active = dl < D && r < rpe && live;
     const uint8_t *wrow = w + ((size_t)(live ? id : 0) * rpe + (active ? r : 0)) * row_bytes;
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *cols = lds + tab_bytes<WT>();
@@ -396,6 +472,9 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
     u32 *s_sel = reinterpret_cast<u32 *>(s_w + spt);                          // [spt]
     Blk<WT> b[U];
     BM_TICK(t_id, id);
+    // behind the wait for the ids, and nothing reads them before the barrier: their way through memory runs under the columns'
+    __builtin_amdgcn_sched_barrier(0);
+    const DownLate late = bm_kernarg_at<DownLate>(offsetof(DownArgs, late));
     preload<WT, U>(b, wrow, q);
     BM_TICK(t_asked, tid);
     BM_TICK(t_cols, st.v[4].x);
@@ -405,6 +484,8 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
         s_sel[tid] = my_sel;
     }
     __syncthreads();
+    float *y = bm_global(late.y);
+    if (!live && id != 0xffffffffu && rb == 0 && dl == 0 && q == 0) bm_raise(bm_global(late.fault), late.layer, kSiteExpertId);
     BM_MARK(2048, 1);
     BM_TOCK(2048, 4, t_id);
     BM_TOCK(2048, 5, t_asked);
@@ -418,15 +499,16 @@ __device__ __forceinline__ void down_combine_body(uint8_t *lds, const uint8_t *w
     BM_MARK(2048, 3);
 }
 
-template <int WT, int U, int NB>
+template <int WT, int U, int NB, bool EIGHT>
 __global__ __launch_bounds__(256) void k_down_combine(const uint8_t *w, u32 n_experts, int nb, const uint8_t *act,
-                                                      const u32 *sel, const float *wts, const float *resid, int spt,
-                                                      int rpe, int spt_shift, float *y, u32 *fault, u32 layer) {
+                                                      const u32 *sel, const float *wts, const float *resid, int spt_word,
+                                                      int rpe, DownLate) {
     extern __shared__ __align__(16) uint8_t lds[];
-    // the grid: (row blocks of a token, tokens). (spt_shift stands among the first sixteen argument words, which are in
-    // registers when the wave starts: behind them it was a load from memory in front of the workgroup's first request)
-    down_combine_body<WT, U, NB>(lds, w, n_experts, nb, act, sel, wts, resid, spt, rpe, y, (int)blockIdx.y, (int)blockIdx.x, fault, layer,
-                                 spt_shift);
+    // the grid: (row blocks of a token, tokens). spt_word: the slot count, and above bit 16 one more than its log2 where it is
+    // a power of two - one word, so that both stand among the first fourteen argument words, which are in registers when the
+    // wave starts (an argument behind them is a load from memory in front of the workgroup's first request)
+    down_combine_body<WT, U, NB, EIGHT>(lds, w, n_experts, nb, act, sel, wts, resid, spt_word & 0xffff, rpe, (int)blockIdx.y, (int)blockIdx.x,
+                                        (spt_word >> 16) - 1);
 }
 
 // k_down_combine for a Q6_K stack of NB super-blocks a row with the row's super-blocks dealt to the waves (BM_DOWN_SPLIT, the
@@ -522,9 +604,7 @@ __global__ __launch_bounds__(256 * NB) void k_down_combine_q6k_split(const uint8
 // slot's down activation.
 template <int WA, int UA, int NBA>
 __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, const uint8_t *wg, const uint8_t *wu,
-                                               u32 n_experts, int na, int nh, const u32 *sel, int spt, uint8_t *act_x,
-                                               uint8_t *act_h, float *h, int slot, int rb, int t, GateRule rule, u32 *fault,
-                                               u32 layer) {
+                                               u32 n_experts, int na, int nh, const u32 *sel, int spt, int slot, int rb, int t) {
     const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
     BM_MARK(0, 0);
     const int hidden = na * 256, ff = nh * 256;
@@ -548,32 +628,44 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
     }
     __asm__ volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    uint8_t *hcol = act_h ? act_h + (size_t)slot * nh * BM_Q82_SB_EXT : nullptr; // none: the down stack takes Q8_K columns
     if (id >= n_experts) { // uniform over the workgroup
         if (id == 0xffffffffu) return; // a slot served elsewhere: nothing written, nothing raised
-        if (tid == 0) bm_raise(fault, layer, kSiteExpertId);
-        if (h && (tid & 7) == 0) h[(size_t)slot * ff + r] = bm_bits_f32(0x7fc00000u);
-        if (hcol && tid < 32) q82_store(hcol, nh, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);
+        const GateUpLate late = bm_kernarg_at<GateUpLate>(offsetof(GateUpArgs, late));
+        if (tid == 0) bm_raise(bm_global(late.fault), late.layer, kSiteExpertId);
+        if (late.h && (tid & 7) == 0) bm_global(late.h)[(size_t)slot * ff + r] = bm_bits_f32(0x7fc00000u);
+        if (late.act_h && tid < 32)
+            q82_store(bm_global(late.act_h) + (size_t)slot * nh * BM_Q82_SB_EXT, nh, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);
         return;
     }
     BM_MARK(0, 1);
     const size_t row_bytes = (size_t)na * bm_block_bytes<WA>();
     const uint8_t *wrow = (which ? wu : wg) + ((size_t)id * ff + r) * row_bytes;
     Blk<WA> b[UA];
+    // behind the wait for the id, and nothing reads them before the token's column stands in LDS: their way through memory runs
+    // under the quantizer's work
+    const GateUpLate late = bm_kernarg_at<GateUpLate>(offsetof(GateUpArgs, late));
     preload<WA, UA>(b, wrow, q);
+    bool bad = false;
 #pragma unroll
     for (int p = 0; p < kPasses; p++) {
         const int o = p * 2048 + tid * 8;
-        if (o < hidden) q82_quad8(xv[p], col, na, o >> 5, tid & 3, fault, layer);
+        if (o < hidden) bad |= q82_quad8<false>(xv[p], col, na, o >> 5, tid & 3, nullptr, 0);
     }
     if constexpr (NBA == 0) { // longer rows: the passes past the first, straight from memory
         for (int o = 2048 + tid * 8; o < hidden; o += 2048) {
             float v8[8];
             for (int k = 0; k < 8; k++) v8[k] = x[(size_t)t * hidden + o + k];
-            q82_quad8(v8, col, na, o >> 5, tid & 3, fault, layer);
+            bad |= q82_quad8<false>(v8, col, na, o >> 5, tid & 3, nullptr, 0);
         }
     }
     __syncthreads();
+    uint8_t *const act_x = bm_global(late.act_x), *const act_h = bm_global(late.act_h);
+    float *const h = bm_global(late.h);
+    const GateRule rule = late.rule;
+    u32 *const fault = bm_global(late.fault);
+    const u32 layer = late.layer;
+    uint8_t *hcol = act_h ? act_h + (size_t)slot * nh * BM_Q82_SB_EXT : nullptr; // none: the down stack takes Q8_K columns
+    if (bad && (tid & 3) == 0) bm_raise(fault, layer, kSiteQuantColumn);
     if (act_x && rb == 0 && slot % spt == 0) stage_bytes(act_x + (size_t)t * col_bytes, col, col_bytes);
     BM_MARK(0, 2);
     float v[1];
@@ -592,13 +684,12 @@ __device__ __forceinline__ void gate_up_x_body(uint8_t *lds, const float *x, con
 // The first half of the fused step as a launch of its own: x -> quantized h, slot by slot.
 template <int WA, int UA, int NBA>
 __global__ __launch_bounds__(256) void k_gate_up_x(const float *x, const uint8_t *wg, const uint8_t *wu, u32 n_experts,
-                                                   int nba, int nh, const u32 *sel, int spt, uint8_t *act_x,
-                                                   uint8_t *act_h, float *h, GateRule rule, u32 *fault, u32 layer) {
+                                                   int nba, int nh, const u32 *sel, int spt, GateUpLate) {
     extern __shared__ __align__(16) uint8_t lds[];
     // the grid: (blocks of 32 rows, slots of a token, tokens): no division stands before the workgroup's first request (and no
     // read of the grid's size, which comes from the dispatch packet in memory: spt is an argument, in a register at the start)
-    gate_up_x_body<WA, UA, NBA>(lds, x, wg, wu, n_experts, NBA > 0 ? NBA : nba, nh, sel, spt, act_x, act_h, h,
-                                (int)blockIdx.z * spt + (int)blockIdx.y, (int)blockIdx.x, (int)blockIdx.z, rule, fault, layer);
+    gate_up_x_body<WA, UA, NBA>(lds, x, wg, wu, n_experts, NBA > 0 ? NBA : nba, nh, sel, spt,
+                                (int)blockIdx.z * spt + (int)blockIdx.y, (int)blockIdx.x, (int)blockIdx.z);
 }
 
 // ------------------------------------------------------------- the fused step for the types that take Q8_K columns
@@ -955,14 +1046,20 @@ hipError_t down_combine(const Launch &L, int wtype, const uint8_t *w, int n_expe
                            resid, spt, rpe, y, L.fault, L.layer);
         return hipGetLastError();
     }
+#define BM_DOWN_LAUNCH(EIGHT)                                                                                          \
+    {                                                                                                                  \
+        auto kern = k_down_combine<WT, U, NB, EIGHT>;                                                                  \
+        hipError_t e = allow_lds(kern, lds);                                                                           \
+        if (e != hipSuccess) return e;                                                                                 \
+        hipLaunchKernelGGL(kern, dim3((unsigned)((rpe + D - 1) / D), (unsigned)m), dim3(256), lds, L.stream, w, (u32)n_experts, nb,    \
+                           act, sel, wts, resid, spt | ((spt_shift + 1) << 16), rpe, DownLate{y, L.fault, L.layer});   \
+    }
+    // (eight slots a token: the form that takes the token's ids through the scalar cache)
 #define CALL_BODY                                                                                                      \
-    auto kern = k_down_combine<WT, U, NB>;                                                                             \
-    hipError_t e = allow_lds(kern, lds);                                                                               \
-    if (e != hipSuccess) return e;                                                                                     \
-    hipLaunchKernelGGL(kern, dim3((unsigned)((rpe + D - 1) / D), (unsigned)m), dim3(256), lds, L.stream, w, (u32)n_experts, nb, act,  \
-                       sel, wts, resid, spt, rpe, spt_shift, y, L.fault, L.layer);
+    if (spt == 8) BM_DOWN_LAUNCH(true) else BM_DOWN_LAUNCH(false)
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
+#undef BM_DOWN_LAUNCH
     return hipGetLastError();
 }
 
@@ -985,7 +1082,7 @@ hipError_t gate_up_x(const Launch &L, int gate_type, const float *x, const uint8
         hipError_t e = allow_lds(kern, lds_a);                                                                         \
         if (e != hipSuccess) return e;                                                                                 \
         hipLaunchKernelGGL(kern, dim3((unsigned)(ff / 32), (unsigned)spt, (unsigned)m), dim3(256), lds_a, L.stream, x, wg, wu,          \
-                           (u32)n_experts, nba, nbb, sel, spt, act_x, act_h, h, L.rule, L.fault, L.layer);                                 \
+                           (u32)n_experts, nba, nbb, sel, spt, GateUpLate{act_x, act_h, h, L.rule, L.fault, L.layer});                    \
     }
     if (gate_type == BM_Q4K) {
         if (nba == 8) BM_GUX(BM_Q4K, kRingQ4K, 8)

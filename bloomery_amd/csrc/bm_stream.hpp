@@ -305,8 +305,11 @@ __device__ __forceinline__ void q82_store(uint8_t *col, int nb, int blk, int lan
     }
 }
 
-// One 32-value q8_2 block held eight values a lane by four consecutive lanes (the in-kernel token quantizer).
-__device__ __forceinline__ void q82_quad8(const float (&v)[8], uint8_t *col, int nb, int blk, int lane4, u32 *fault,
+// One 32-value q8_2 block held eight values a lane by four consecutive lanes (the in-kernel token quantizer). Returns whether
+// the block holds a value that is not finite; RAISE: raises QuantColumn for it as well (without: the caller does, where the
+// fault word's address has come in).
+template <bool RAISE = true>
+__device__ __forceinline__ bool q82_quad8(const float (&v)[8], uint8_t *col, int nb, int blk, int lane4, u32 *fault,
                                           u32 layer) {
     u32 ab = 0;
 #pragma unroll
@@ -322,9 +325,11 @@ __device__ __forceinline__ void q82_quad8(const float (&v)[8], uint8_t *col, int
     u32 t;
     int isum = 0, csum = 0;
     u32 c0 = 0, c1 = 0;
-    if (ab > 0x7f7fffffu) {
+    const bool bad = ab > 0x7f7fffffu;
+    if (bad) {
         t = 0x7fc0u;
-        if (lane4 == 0) bm_raise(fault, layer, kSiteQuantColumn);
+        if constexpr (RAISE)
+            if (lane4 == 0) bm_raise(fault, layer, kSiteQuantColumn);
     } else {
         t = bm_fp32_to_bf16_bits(__fdiv_rn(bm_bits_f32(ab), 127.0f));
         const float id = bm_q82_inverse(t);
@@ -353,6 +358,7 @@ __device__ __forceinline__ void q82_quad8(const float (&v)[8], uint8_t *col, int
         *reinterpret_cast<float2 *>(col + (size_t)nb * BM_Q82_SB_REF + 8 * blk) =
             make_float2(d8, __fmul_rn(d8, (float)(short)isum));
     }
+    return bad;
 }
 
 // One 256-value block of a Q8_K column by one wave, four consecutive values a lane: k_quantize_q8k's operations on the

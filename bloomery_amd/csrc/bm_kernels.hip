@@ -328,33 +328,6 @@ hipError_t combine_tokens(const Launch &L, const float *down, const float *w, co
     return hipGetLastError();
 }
 
-// An argument read from the launch's argument block at the place in the code where this call stands. The first fourteen
-// words of the block are in registers when a wave starts; an argument behind them is a scalar load, and the compiler asks
-// for it at the top of the kernel: scalar loads come back in any order, so the first wait for one of them - the expert id's -
-// would be a wait for those words as well. The arguments the head of a decode launch does not need stand at the end of its
-// list as one struct, which the kernel does not touch, and are read through this behind the launch's first requests.
-template <class T>
-__device__ __forceinline__ T bm_kernarg_at(unsigned offset) {
-    static_assert(sizeof(T) % 4 == 0, "whole words");
-    typedef __attribute__((address_space(4))) const uint8_t *Block;
-    typedef __attribute__((address_space(4))) const u32 *Words;
-    const Words from = (Words)((Block)__builtin_amdgcn_kernarg_segment_ptr() + offset);
-    struct Raw {
-        u32 w[sizeof(T) / 4];
-    } raw;
-#pragma unroll
-    for (unsigned i = 0; i < sizeof(T) / 4; i++) raw.w[i] = from[i];
-    return __builtin_bit_cast(T, raw);
-}
-
-// A pointer that came out of bm_kernarg_at's words, as what a pointer argument is: an address in global memory (without this
-// the compiler takes it for one that may also lie in LDS or scratch, and every wait for a vector load behind its first use is
-// a wait for all of them).
-template <class P>
-__device__ __forceinline__ P *bm_global(P *p) {
-    return (P *)(__attribute__((address_space(1))) P *)(uintptr_t)p;
-}
-
 struct DownLate { // the end of k_down_combine's arguments
     float *y;
     u32 *fault;
@@ -826,15 +799,28 @@ __global__ __launch_bounds__(256) void k_gemv_x(const float *x, const uint8_t *w
     const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
     const int col_bytes = bm_act_col_bytes<WT>(n);
     const uint8_t *wrow = w + (size_t)(active ? row : 0) * row_bytes;
+    const float *xc = x + (size_t)c * k;
+    // the column's first 2048 values are asked for in front of the rows: vector loads come back in the order they were asked
+    // for, and behind the rows' requests the quantizer would wait for those as well
+    float4 x_lo = make_float4(0, 0, 0, 0), x_hi = x_lo;
+    if constexpr (!bm_takes_q8k(WT)) {
+        const int o = tid * 8 < k ? tid * 8 : k - 8;
+        x_lo = *reinterpret_cast<const float4 *>(xc + o), x_hi = *reinterpret_cast<const float4 *>(xc + o + 4);
+        __asm__ volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    }
     Blk<WT> b[U];
     preload<WT, U>(b, wrow, q);
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *col = lds + tab_bytes<WT>();
-    const float *xc = x + (size_t)c * k;
     if constexpr (bm_takes_q8k(WT)) {
         q8k_stage_cols(xc, col, 1, n, fault, layer);
     } else { // a q8_2 block is four lanes of eight values; 2048 values a pass
-        for (int o = tid * 8; o < k; o += 2048) {
+        if (tid * 8 < k) {
+            const float v8[8] = {x_lo.x, x_lo.y, x_lo.z, x_lo.w, x_hi.x, x_hi.y, x_hi.z, x_hi.w};
+            q82_quad8(v8, col, n, tid >> 2, tid & 3, fault, layer);
+        }
+        for (int o = 2048 + tid * 8; o < k; o += 2048) {
             const float4 lo = *reinterpret_cast<const float4 *>(xc + o), hi = *reinterpret_cast<const float4 *>(xc + o + 4);
             float v8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
             q82_quad8(v8, col, n, o >> 5, tid & 3, fault, layer);

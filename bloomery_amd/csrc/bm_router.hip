@@ -294,12 +294,36 @@ hipError_t route_softmax(const Launch &L, const float *logits, int n_tok, int n_
 // Floats a line of the accumulator-major LDS rows.
 __host__ __device__ inline int router_line(int hidden) { return ((hidden / 8 + 3) & ~3) + 8; }
 
+// (k_norm_route's arguments: what the head of a logits workgroup needs stands in the first fourteen words, which are in registers when a
+// wave starts - m_word is the token count, bit 31 set where the quantized column is asked for - and the rest travels as one
+// struct behind them that a workgroup reads when it gets there: see bm_kernarg_at.)
+struct NormRouteLate {
+    u32 used, renorm;
+    float *probs;
+    u32 *ids;
+    float *weights;
+    u32 *hand;
+    uint8_t *act_x;
+    int q8k;
+    u32 layer;
+    u32 *fault;
+    u32 max_polls, unused;
+};
+struct NormRouteArgs { // k_norm_route's argument block
+    const float *router, *x, *gain;
+    float eps;
+    int n_exp, hidden;
+    u32 m_word;
+    float *normed_out, *logits;
+    NormRouteLate late;
+};
+static_assert(offsetof(NormRouteArgs, late) == 56, "fourteen words in front of the late arguments");
+
 // t: the token; e0: the first of the workgroup's R router rows, or -1 for a workgroup that only norms the token's row into LDS
 // (k_norm_route's quantizer workgroups): no router rows, no logits.
 template <int R, bool COH = false>
 __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *router, const float *x, const float *gain, float eps,
-                                                   int n_exp, int hidden, float *normed_out, float *logits, int t, int e0,
-                                                   [[maybe_unused]] u32 *hand = nullptr) {
+                                                   int n_exp, int hidden, float *normed_out, float *logits, int t, int e0) {
     // The token's row and the R router rows lie accumulator-major in LDS: value k at line k % 8, place k / 8, so that the
     // lane that owns accumulator l reads four consecutive steps' operands as 16 bytes. A line is hidden / 8 floats, rounded up
     // to whole 16 bytes, + 8 (the eight lines of a row 8 banks apart), a router row four floats past the one before (rows r
@@ -319,28 +343,41 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
     // the rows' bytes on their way first: they do not depend on the norm. Eight 16-byte loads a thread are asked for together
     // and go to LDS once the token's row has been asked for too and normed
     const int n4 = hidden / 4;
-    const int total = e0 >= 0 ? R * n4 : 0;
+    // A thread's pieces of the R rows: row 0's pieces tid, tid + 256, ..., then row 1's, ...: piece n of the thread is (row, place)
+    // by counting on, no division by a length only known at run time in front of the first request.
     constexpr int kBatch = 8;
     float4 rv[kBatch];
-    auto ask = [&](int i0) {
+    struct Piece {
+        int r, c;
+    };
+    const int rows_here = e0 >= 0 ? R : 0;
+    auto step = [&](Piece &p) {
+        p.c += 256;
+        if (p.c >= n4) p.r++, p.c = tid;
+    };
+    const Piece first = {tid < n4 ? 0 : rows_here, tid};
+    auto ask = [&](Piece p) { // asks for the next kBatch pieces from p on; returns the piece behind them
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
-            const int i = i0 + tid + 256 * u;
-            if (i < total) {
-                const int r = i / n4, c = i % n4;
-                const int e = e0 + r < n_exp ? e0 + r : n_exp - 1;
-                rv[u] = reinterpret_cast<const float4 *>(router + (size_t)e * hidden)[c];
+            if (p.r < rows_here) {
+                const int e = e0 + p.r < n_exp ? e0 + p.r : n_exp - 1;
+                rv[u] = reinterpret_cast<const float4 *>(router + (size_t)e * hidden)[p.c];
+                step(p);
             }
         }
+        return p;
     };
-    auto park = [&](int i0) {
+    auto park = [&](Piece p) {
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
-            const int i = i0 + tid + 256 * u;
-            if (i < total) put4(ws + (size_t)(i / n4) * wrow_floats, i % n4, rv[u]);
+            if (p.r < rows_here) {
+                put4(ws + (size_t)p.r * wrow_floats, p.c, rv[u]);
+                step(p);
+            }
         }
+        return p;
     };
-    ask(0);
+    ask(first);
     double sum = 0.0;
     constexpr int kInRegs = 8; // float4s of the row a thread can hold: rows of up to 8192 values stay in registers
     if (gain && n4 <= 256 * kInRegs) {
@@ -406,13 +443,17 @@ __device__ __forceinline__ void router_logits_body(uint8_t *lds, const float *ro
             }
         }
     }
-    park(0);
-    for (int i0 = 256 * kBatch; i0 < total; i0 += 256 * kBatch) {
-        ask(i0);
-        park(i0);
+    Piece parked = park(first);
+    while (parked.r < rows_here) { // (no barrier inside: a thread with fewer pieces leaves earlier)
+        ask(parked);
+        parked = park(parked);
     }
     __syncthreads();
     BM_RTICK(tl_lds, tid);
+    // (k_norm_route's hand-over words: an argument behind the preloaded ones, read here, where its way through memory runs under
+    // the dots)
+    [[maybe_unused]] u32 *hand = nullptr;
+    if constexpr (COH) hand = bm_global(bm_kernarg_at<u32 *>(offsetof(NormRouteArgs, late) + offsetof(NormRouteLate, hand)));
     if (!gain && normed_out && e0 == 0) // the rows as they are (read after the barrier: other threads staged them)
         for (int i = tid; i < hidden; i += 256) normed_out[(size_t)t * hidden + i] = xs[(i & 7) * line + (i >> 3)];
     // every thread that stores a logit below is of the first wave: k_norm_route's hand-over (a device-scope count updated by
@@ -508,15 +549,18 @@ __global__ __launch_bounds__(256) void k_router_logits(const float *router, cons
 // Q8_2_X4 one with its tables), the bytes bm_quantize makes of normed_out. The routing waits for none of it.
 template <int R, int PER>
 __global__ __launch_bounds__(256) void k_norm_route(const float *router, const float *x, const float *gain, float eps, int n_exp,
-                                                    int hidden, float *normed_out, float *logits, u32 used, u32 renorm,
-                                                    float *probs, u32 *ids, float *weights, u32 *hand, uint8_t *act_x,
-                                                    int q8k, int m, u32 *fault, u32 layer, u32 max_polls) {
+                                                    int hidden, u32 m_word, float *normed_out, float *logits, NormRouteLate) {
     extern __shared__ __align__(16) uint8_t lds[];
     const u32 blocks_per_token = (u32)((n_exp + R - 1) / R);
-    const u32 n_logit_blocks = (u32)m * blocks_per_token, n_quant_blocks = act_x ? (u32)m : 0u;
+    const u32 m = m_word & 0x7fffffffu;
+    const u32 n_logit_blocks = m * blocks_per_token, n_quant_blocks = (m_word >> 31) ? m : 0u;
     if (blockIdx.x >= n_logit_blocks + n_quant_blocks) { // a routing workgroup: its first wave takes the logits
         __shared__ PickLds pick;
         const u32 t = blockIdx.x - n_logit_blocks - n_quant_blocks, lane = threadIdx.x;
+        const NormRouteLate late = bm_kernarg_at<NormRouteLate>(offsetof(NormRouteArgs, late));
+        const u32 used = late.used, renorm = late.renorm, layer = late.layer, max_polls = late.max_polls;
+        float *const probs = bm_global(late.probs), *const weights = bm_global(late.weights);
+        u32 *const ids = bm_global(late.ids), *const hand = bm_global(late.hand), *const fault = bm_global(late.fault);
         constexpr bool kRanks = PER <= 4; // up to 256 experts: the picks by the whole workgroup
         if constexpr (kRanks) {
             pick.p[threadIdx.x] = -1.0f, pick.ahead[threadIdx.x] = 0;
@@ -575,6 +619,11 @@ __global__ __launch_bounds__(256) void k_norm_route(const float *router, const f
     if (blockIdx.x >= n_logit_blocks) { // a quantizer workgroup
         const int tq = (int)(blockIdx.x - n_logit_blocks);
         router_logits_body<R>(lds, router, x, gain, eps, n_exp, hidden, nullptr, nullptr, tq, -1);
+        const NormRouteLate late = bm_kernarg_at<NormRouteLate>(offsetof(NormRouteArgs, late));
+        uint8_t *const act_x = bm_global(late.act_x);
+        u32 *const fault = bm_global(late.fault);
+        const u32 layer = late.layer;
+        const int q8k = late.q8k;
         const int line = router_line(hidden), nb = hidden / 256, tid = threadIdx.x;
         const float *xs = reinterpret_cast<const float *>(lds); // value k at line k % 8, place k / 8
         if (q8k) {
@@ -596,8 +645,7 @@ __global__ __launch_bounds__(256) void k_norm_route(const float *router, const f
         return;
     }
     const u32 t = blockIdx.x / blocks_per_token;
-    router_logits_body<R, true>(lds, router, x, gain, eps, n_exp, hidden, normed_out, logits, (int)t, (int)(blockIdx.x % blocks_per_token) * R,
-                                hand);
+    router_logits_body<R, true>(lds, router, x, gain, eps, n_exp, hidden, normed_out, logits, (int)t, (int)(blockIdx.x % blocks_per_token) * R);
 }
 
 // LDS of a workgroup of R rows: the token's row and the router rows, each as eight lines.
@@ -655,8 +703,9 @@ hipError_t norm_route(const Launch &L, const float *router, const float *x, cons
         auto kern = k_norm_route<R, PER>;                                                                              \
         hipError_t e = allow_lds(kern, lds);                                                                           \
         if (e != hipSuccess) return e;                                                                                 \
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, router, x, gain, eps, n_exp, hidden, normed_out, \
-                           logits, (u32)used, (u32)renorm, probs, ids, weights, hand, act_x, q8k ? 1 : 0, m, L.fault, L.layer, max_polls); \
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, router, x, gain, eps, n_exp, hidden,           \
+                           (u32)m | (act_x ? 0x80000000u : 0u), normed_out, logits,                                    \
+                           NormRouteLate{(u32)used, (u32)renorm, probs, ids, weights, hand, act_x, q8k ? 1 : 0, L.layer, L.fault, max_polls, 0u}); \
     }
 #define BM_NR_ROWS(PER)                                                                                                \
     {                                                                                                                  \

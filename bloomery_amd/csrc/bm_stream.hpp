@@ -427,6 +427,33 @@ __device__ __forceinline__ float swiglu_of_pair(float v, int which, GateRule rul
     return hv;
 }
 
+// An argument read from the launch's argument block at the place in the code where this call stands. The first fourteen
+// words of the block are in registers when a wave starts; an argument behind them is a scalar load, and the compiler asks
+// for it at the top of the kernel: scalar loads come back in any order, so the first wait for one of them - the expert id's -
+// would be a wait for those words as well. The arguments the head of a decode launch does not need stand at the end of its
+// list as one struct, which the kernel does not touch, and are read through this behind the launch's first requests.
+template <class T>
+__device__ __forceinline__ T bm_kernarg_at(unsigned offset) {
+    static_assert(sizeof(T) % 4 == 0, "whole words");
+    typedef __attribute__((address_space(4))) const uint8_t *Block;
+    typedef __attribute__((address_space(4))) const u32 *Words;
+    const Words from = (Words)((Block)__builtin_amdgcn_kernarg_segment_ptr() + offset);
+    struct Raw {
+        u32 w[sizeof(T) / 4];
+    } raw;
+#pragma unroll
+    for (unsigned i = 0; i < sizeof(T) / 4; i++) raw.w[i] = from[i];
+    return __builtin_bit_cast(T, raw);
+}
+
+// A pointer that came out of bm_kernarg_at's words, as what a pointer argument is: an address in global memory (without this
+// the compiler takes it for one that may also lie in LDS or scratch, and every wait for a vector load behind its first use is
+// a wait for all of them).
+template <class P>
+__device__ __forceinline__ P *bm_global(P *p) {
+    return (P *)(__attribute__((address_space(1))) P *)(uintptr_t)p;
+}
+
 // The 32 values a workgroup produced (hbuf, LDS) as block `rb` of column `hcol`, by the first 32 threads.
 __device__ __forceinline__ void quantize_h_block(const float *hbuf, uint8_t *hcol, int nb_h, int rb, int tid,
                                                  u32 *fault, u32 layer) {

@@ -27,7 +27,7 @@ __global__ __launch_bounds__(1024) void k_buckets(const u32 *sel, u32 n_slots, u
         if (p != kHostSlot) bm_raise(fault, layer, kSiteExpertId);
         return kNoBucket;
     });
-    for (u32 e = threadIdx.x; e <= n_experts; e += blockDim.x) start[e] = g.base[e];
+    for (u32 e = threadIdx.x; e <= n_experts; e += kGroupThreads) start[e] = g.base[e];
 }
 
 // crates/gpu/src/q4k_sel.rs:562-680 grouped_tiles. A run outside 0 .. start[n_experts] <= n_slots, or more tiles
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(1024) void k_tables(const u32 *sel, u32 n_slots, u3
         if (p != kHostSlot) bm_raise(fault, layer, kSiteExpertId);
         return kNoBucket;
     });
-    for (u32 e = threadIdx.x; e <= n_experts; e += blockDim.x) start[e] = g.base[e];
+    for (u32 e = threadIdx.x; e <= n_experts; e += kGroupThreads) start[e] = g.base[e];
     __threadfence_block();
     __syncthreads(); // the runs are the workgroup's own writes: visible to it past the barrier
     tiles_body(start, n_experts, n_slots, cap, tiles, fault, layer);
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(1024) void k_tables_quant(const u32 *sel, u32 n_slo
         if (p != kHostSlot) bm_raise(fault, layer, kSiteExpertId);
         return kNoBucket;
     });
-    for (u32 e = threadIdx.x; e <= n_experts; e += blockDim.x) start[e] = g.base[e];
+    for (u32 e = threadIdx.x; e <= n_experts; e += kGroupThreads) start[e] = g.base[e];
     __threadfence_block();
     __syncthreads();
     tiles_body(start, n_experts, n_slots, cap, tiles, fault, layer);

@@ -52,7 +52,7 @@ __device__ unsigned long long g_timeline[kTimelineRows * 8];
 // ----------------------------------------------------------------------------------------------- fill
 
 __global__ void k_fill_u32(u32 *dst, u32 value, size_t n) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) dst[i] = value;
 }
 
@@ -130,7 +130,7 @@ hipError_t quantize(const Launch &L, int wtype, const float *x, int m, int k, ui
 
 // Fills the two tables of `m` device Q8_2_X4 columns from their reference bytes (after an upload of those bytes).
 __global__ __launch_bounds__(256) void k_q82_tables(uint8_t *act, int m, int nb) {
-    const long g = (long)blockIdx.x * blockDim.x + threadIdx.x; // one 16-value group a thread
+    const long g = (long)blockIdx.x * 256 + threadIdx.x; // one 16-value group a thread
     if (g >= (long)m * nb * 16) return;
     const int col = (int)(g / (nb * 16)), g16 = (int)(g % (nb * 16)), blk = g16 >> 1, half = g16 & 1;
     uint8_t *c = act + (size_t)col * nb * BM_Q82_SB_EXT;
@@ -187,42 +187,75 @@ __global__ __launch_bounds__(256) void k_gemv(const uint8_t *w, long rows, int n
 
 // One workgroup = 32 consecutive rows of one slot; eight lanes a row: a quad on the gate row, a quad on the up row.
 // With act_h the 32 values are quantized to one q8_2 block of the slot's down activation in the same launch.
+struct GateUpColLate { // the end of k_gate_up's arguments (see bm_kernarg_at)
+    float *h;
+    uint8_t *act_h;
+    GateRule rule;
+    u32 *fault;
+    u32 layer;
+};
+struct GateUpColArgs { // k_gate_up's argument block
+    const uint8_t *wg, *wu;
+    u32 n_experts;
+    int nb;
+    const uint8_t *act;
+    const u32 *sel;
+    int rpe, spc_word;
+    u32 n_slots;
+    GateUpColLate late;
+};
+static_assert(offsetof(GateUpColArgs, late) == 56, "fourteen words in front of the late arguments");
+constexpr unsigned kGateUpGridY = 32768; // slots along the grid's second dimension; the third counts the rest
+
+// The grid: (blocks of 32 rows, slots, slots / kGateUpGridY): no division stands before the workgroup's first request.
+// spc_word: slots_per_col, and above bit 24 one more than its log2 where it is a power of two.
 template <int WT, int U, int NB>
 __global__ __launch_bounds__(256) void k_gate_up(const uint8_t *wg, const uint8_t *wu, u32 n_experts, int nb,
-                                                 const uint8_t *act, const u32 *sel, int rpe, int slots_per_col,
-                                                 float *h, uint8_t *act_h, GateRule rule, u32 *fault, u32 layer) {
+                                                 const uint8_t *act, const u32 *sel, int rpe, int spc_word, u32 n_slots,
+                                                 GateUpColLate) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, q = tid & 3, which = (tid >> 2) & 1;
-    const int blocks_per_slot = (rpe + 31) / 32;
-    const int slot = blockIdx.x / blocks_per_slot, rb = blockIdx.x % blocks_per_slot;
+    const int slot = (int)(blockIdx.z * kGateUpGridY + blockIdx.y), rb = (int)blockIdx.x;
+    if ((u32)slot >= n_slots) return;
     const int r = rb * 32 + (tid >> 3);
     const bool active = r < rpe;
     const u32 id = sel[slot];
     const int n = NB > 0 ? NB : nb;
     const int nb_h = rpe / 256;
     const int col_bytes = bm_act_col_bytes<WT>(n);
-    const uint8_t *act_col = act + (size_t)(slot / slots_per_col) * col_bytes;
-    uint8_t *hcol = act_h ? act_h + (size_t)slot * nb_h * BM_Q82_SB_EXT : nullptr;
+    const int spc_shift = (spc_word >> 24) - 1;
+    const int token = spc_shift >= 0 ? slot >> spc_shift : slot / (spc_word & 0xffffff);
+    const uint8_t *act_col = act + (size_t)token * col_bytes;
     Stage<2> st;
     st.load(act_col, col_bytes);
     if (id >= n_experts) { // uniform over the workgroup: no weight is read (crates/gpu/src/kquant/sel.rs:22-28)
         if (id == 0xffffffffu) return; // a slot served elsewhere: nothing written, nothing raised (sel.rs:153-161)
-        if (tid == 0) bm_raise(fault, layer, kSiteExpertId);
+        const GateUpColLate late = bm_kernarg_at<GateUpColLate>(offsetof(GateUpColArgs, late));
+        float *const h = bm_global(late.h);
+        uint8_t *const act_h = bm_global(late.act_h);
+        if (tid == 0) bm_raise(bm_global(late.fault), late.layer, kSiteExpertId);
         if (h && active && (tid & 7) == 0) h[(size_t)slot * rpe + r] = bm_bits_f32(0x7fc00000u);
-        if (act_h && tid < 32) q82_store(hcol, nb_h, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);
+        if (act_h && tid < 32) q82_store(act_h + (size_t)slot * nb_h * BM_Q82_SB_EXT, nb_h, rb, tid, 0, Q82Head{0x7fc0u, 0, true}, 0);
         return;
     }
     const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
     const uint8_t *wrow = (which ? wu : wg) + ((size_t)id * rpe + (active ? r : 0)) * row_bytes;
     Blk<WT> b[U];
+    // (behind the wait for the id; nothing reads them before the column stands in LDS)
+    const GateUpColLate late = bm_kernarg_at<GateUpColLate>(offsetof(GateUpColArgs, late));
     preload<WT, U>(b, wrow, q);
     const Iq2Tables tb = stage_tables<WT>(lds);
     uint8_t *col = lds + tab_bytes<WT>();
     st.store(col, act_col, col_bytes);
     __syncthreads();
+    float *const h = bm_global(late.h);
+    uint8_t *const act_h = bm_global(late.act_h);
+    u32 *const fault = bm_global(late.fault);
+    const u32 layer = late.layer;
+    uint8_t *hcol = act_h ? act_h + (size_t)slot * nb_h * BM_Q82_SB_EXT : nullptr;
     float v[1];
     row_dot<WT, U, NB, 1>(b, wrow, col, col_bytes, 1, n, q, tb, v, NoTap{});
-    const float hv = swiglu_of_pair(v[0], which, rule, fault, layer);
+    const float hv = swiglu_of_pair(v[0], which, late.rule, fault, layer);
     if (h && active && (tid & 7) == 0) h[(size_t)slot * rpe + r] = hv;
     if (act_h) { // rpe is a multiple of 256 here, so every row of the block is live
         float *hbuf = reinterpret_cast<float *>(col + col_bytes);
@@ -275,7 +308,7 @@ __global__ __launch_bounds__(256) void k_gemv_sel(const uint8_t *w, u32 n_expert
 // `sel` (optional): a slot whose id is at or past n_experts adds nothing, as in the fused down + combine launch.
 __global__ __launch_bounds__(256) void k_combine(const float *down, const float *w, const float *shexp, const float *resid,
                                                  int rows, int n_slots, int m, float *y, const u32 *sel, u32 n_experts) {
-    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long i = (long)blockIdx.x * 256 + threadIdx.x; // (the launcher's 256 threads: blockDim.x is a load from memory)
     if (i >= (long)rows * m) return;
     const int t = (int)(i / rows), d = (int)(i % rows);
     float acc = 0.0f;
@@ -290,7 +323,7 @@ __global__ __launch_bounds__(256) void k_combine(const float *down, const float 
 // The same with four consecutive values a thread (16-byte loads): the form for many tokens.
 __global__ __launch_bounds__(256) void k_combine4(const float *down, const float *w, const float *shexp, const float *resid,
                                                   int rows, int n_slots, int m, float *y, const u32 *sel, u32 n_experts) {
-    const long i = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= (long)rows * m) return;
     const int t = (int)(i / rows), d = (int)(i % rows);
     float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -671,7 +704,7 @@ __global__ __launch_bounds__(256) void k_gate_up_x(const float *x, const uint8_t
 // waves, block by block.
 __device__ __forceinline__ void q8k_stage_cols(const float *x, uint8_t *dst, int cols, int nb, u32 *fault, u32 layer,
                                                const u32 *ids = nullptr, u32 n_experts = 0) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = 4; // (256 threads: every caller's workgroup)
     const int total = cols * nb;
     constexpr int kAhead = 6; // blocks whose loads a wave has in flight
     for (int b0 = wave; b0 < total; b0 += kAhead * n_waves) {
@@ -909,10 +942,10 @@ __global__ __launch_bounds__(64) void k_block_sums(const uint8_t *wrow, int nb, 
     const int tid = threadIdx.x, q = tid & 3;
     const int n = NB > 0 ? NB : nb;
     const int col_bytes = bm_act_col_bytes<WT>(n);
-    for (int i = tid; i < 16 * n; i += blockDim.x) out[i] = 0;
-    const Iq2Tables tb = stage_tables<WT>(lds);
+    for (int i = tid; i < 16 * n; i += 64) out[i] = 0;
+    const Iq2Tables tb = stage_tables<WT, 64>(lds);
     uint8_t *col = lds + tab_bytes<WT>();
-    stage_bytes(col, act_col, col_bytes);
+    stage_bytes<64>(col, act_col, col_bytes);
     __threadfence();
     __syncthreads();
     if (tid >= 4) return;
@@ -984,13 +1017,21 @@ hipError_t gate_up(const Launch &L, int wtype, const uint8_t *wg, const uint8_t 
                    float *h, uint8_t *act_h) {
     const int nb = k / 256, rpe = rows_per_expert;
     const size_t lds = tab_bytes_rt(wtype) + (size_t)act_col_bytes(wtype, k) + 32 * sizeof(float);
-    const unsigned grid = (unsigned)n_slots * (unsigned)((rpe + 31) / 32);
+    if (n_slots <= 0 || slots_per_col <= 0) return hipErrorInvalidValue;
+    if (slots_per_col > 0xffffff) { // (more slots a column than there are slots: column 0 either way)
+        if (n_slots > 0xffffff) return hipErrorInvalidValue;
+        slots_per_col = 0xffffff;
+    }
+    const unsigned grid_y = (unsigned)n_slots < kGateUpGridY ? (unsigned)n_slots : kGateUpGridY;
+    const unsigned grid_z = ((unsigned)n_slots + kGateUpGridY - 1) / kGateUpGridY;
+    const int spc_shift = (slots_per_col & (slots_per_col - 1)) == 0 ? __builtin_ctz((unsigned)slots_per_col) : -1;
 #define CALL_BODY                                                                                                      \
     auto kern = k_gate_up<WT, U, NB>;                                                                                  \
     hipError_t e = allow_lds(kern, lds);                                                                               \
     if (e != hipSuccess) return e;                                                                                     \
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, L.stream, wg, wu, (u32)n_experts, nb, act, sel, rpe,          \
-                       slots_per_col, h, act_h, L.rule, L.fault, L.layer);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((rpe + 31) / 32), grid_y, grid_z), dim3(256), lds, L.stream, wg, wu, (u32)n_experts, nb, \
+                       act, sel, rpe, slots_per_col | ((spc_shift + 1) << 24), (u32)n_slots,                           \
+                       GateUpColLate{h, act_h, L.rule, L.fault, L.layer});
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
     return hipGetLastError();

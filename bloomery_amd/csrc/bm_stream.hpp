@@ -48,7 +48,8 @@ __device__ __forceinline__ uint2 iq_sign_masks(int t) {
     return make_uint2(m[0], m[1]);
 }
 
-template <int WT>
+// (T: the workgroup's thread count, a constant: blockDim.x is a load from the dispatch packet, in front of whatever comes next)
+template <int WT, int T = 256>
 __device__ __forceinline__ Iq2Tables stage_tables(uint8_t *lds) {
     Iq2Tables tb{nullptr, nullptr, nullptr};
     if constexpr (WT == BM_IQ2XXS) {
@@ -56,13 +57,13 @@ __device__ __forceinline__ Iq2Tables stage_tables(uint8_t *lds) {
         // of 4 where the value is negative: their sum picks a value's code byte 43 +- magnitude out of six (bm_iq2_codes)
         uint2 *grid = reinterpret_cast<uint2 *>(lds);
         uint2 *signs = reinterpret_cast<uint2 *>(lds + 256 * 8);
-        for (int t = threadIdx.x; t < 256; t += blockDim.x) {
+        for (int t = threadIdx.x; t < 256; t += T) {
             const uint64_t g = BM_IQ2XXS_GRID[t];
             const u32 lo = (u32)g, hi = (u32)(g >> 32);
             // 0x08 -> 0, 0x19 -> 1, 0x2b -> 2: bit 0 of the byte is 1 for 0x19 and 0x2b, bit 1 for 0x2b only
             grid[t] = make_uint2(((lo & 0x01010101u) + ((lo >> 1) & 0x01010101u)), ((hi & 0x01010101u) + ((hi >> 1) & 0x01010101u)));
         }
-        for (int t = threadIdx.x; t < 128; t += blockDim.x) {
+        for (int t = threadIdx.x; t < 128; t += T) {
             const uint2 m = iq_sign_masks(t);
             signs[t] = make_uint2(m.x & 0x04040404u, m.y & 0x04040404u);
         }
@@ -72,20 +73,21 @@ __device__ __forceinline__ Iq2Tables stage_tables(uint8_t *lds) {
     if constexpr (WT == BM_IQ3XXS) {
         uint2 *grid = reinterpret_cast<uint2 *>(lds);
         uint2 *signs = reinterpret_cast<uint2 *>(lds + 256 * 8);
-        for (int t = threadIdx.x; t < 256; t += blockDim.x) {
+        for (int t = threadIdx.x; t < 256; t += T) {
             const u32 g = BM_IQ3XXS_GRID[t]; // bytes 4 .. 62: 64 + and 64 - stay inside a byte
             grid[t] = make_uint2(0x40404040u + g, 0x40404040u - g);
         }
-        for (int t = threadIdx.x; t < 128; t += blockDim.x) signs[t] = iq_sign_masks(t);
+        for (int t = threadIdx.x; t < 128; t += T) signs[t] = iq_sign_masks(t);
         tb.grid3 = grid;
         tb.signs = signs;
     }
     return tb;
 }
 
-// `bytes` (a multiple of 8) from 8-byte aligned global memory to 8-byte aligned LDS, by the whole workgroup.
+// `bytes` (a multiple of 8) from 8-byte aligned global memory to 8-byte aligned LDS, by the whole workgroup of T threads.
+template <int T = 256>
 __device__ __forceinline__ void stage_bytes(uint8_t *dst, const uint8_t *src, int bytes) {
-    for (int o = threadIdx.x * 8; o < bytes; o += blockDim.x * 8)
+    for (int o = threadIdx.x * 8; o < bytes; o += T * 8)
         *reinterpret_cast<uint2 *>(dst + o) = *reinterpret_cast<const uint2 *>(src + o);
 }
 
@@ -500,6 +502,7 @@ __device__ __forceinline__ u32 block_scan_1024(u32 v, u32 *scratch, u32 *total) 
 // rank among the lanes of its bucket read off the ballots of the bucket's bits.
 constexpr u32 kNoBucket = 0xffffffffu;
 constexpr int kGroupHist = 8192, kGroupWaves = 16, kGroupBuckets = 1025;
+constexpr u32 kGroupThreads = 1024; // the workgroups these routines run in (a constant: blockDim.x is a load from the dispatch packet)
 struct GroupLds {
     u32 hist[kGroupHist + kGroupWaves]; // [chunk][bucket]: the chunk's next place inside the bucket's run
     u32 base[kGroupBuckets + 1];        // bucket b's run is list[base[b] .. base[b + 1]]
@@ -527,7 +530,7 @@ __device__ __forceinline__ void group_slots(GroupLds &g, u32 n, u32 n_buckets, u
     chunks = chunks < (u32)kGroupWaves ? chunks : (u32)kGroupWaves;
     const u32 per = ((n + chunks - 1) / chunks + 63) & ~63u; // whole batches of 64 a chunk
     const u32 lo = wave * per, hi = lo + per < n ? lo + per : n;
-    for (u32 i = tid; i < chunks * n_buckets; i += blockDim.x) g.hist[i] = 0;
+    for (u32 i = tid; i < chunks * n_buckets; i += kGroupThreads) g.hist[i] = 0;
     __syncthreads();
     if (wave < chunks)
         for (u32 s = lo + lane; s < hi; s += 64) {
@@ -536,7 +539,7 @@ __device__ __forceinline__ void group_slots(GroupLds &g, u32 n, u32 n_buckets, u
         }
     __syncthreads();
     u32 count = 0;
-    for (u32 b = tid; b < n_buckets; b += blockDim.x) { // a chunk's count -> its offset inside the bucket's run
+    for (u32 b = tid; b < n_buckets; b += kGroupThreads) { // a chunk's count -> its offset inside the bucket's run
         u32 sum = 0;
         for (u32 c = 0; c < chunks; c++) {
             const u32 v = g.hist[c * n_buckets + b];
@@ -612,22 +615,22 @@ __device__ __forceinline__ void group_slots_part(GroupLds &g, u32 *off, u32 n, u
     u32 reps = 16;
     while (reps > 1 && reps * rstride > (u32)kGroupHist) reps >>= 1;
     u32 *mine = g.hist + (lane & (reps - 1)) * rstride;
-    for (u32 i = tid; i < reps * rstride; i += blockDim.x) g.hist[i] = 0;
+    for (u32 i = tid; i < reps * rstride; i += kGroupThreads) g.hist[i] = 0;
     __syncthreads();
-    for (u32 s0 = tid; s0 < n; s0 += 4 * blockDim.x) {
+    for (u32 s0 = tid; s0 < n; s0 += 4 * kGroupThreads) {
         u32 b[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const u32 s = s0 + (u32)j * blockDim.x;
+            const u32 s = s0 + (u32)j * kGroupThreads;
             b[j] = s < n ? bucket_of(s) : kNoBucket;
         }
 #pragma unroll
         for (int j = 0; j < 4; j++)
-            if (b[j] != kNoBucket) atomicAdd(&mine[(s0 + (u32)j * blockDim.x < p_lo ? 0u : n_buckets) + b[j]], 1u);
+            if (b[j] != kNoBucket) atomicAdd(&mine[(s0 + (u32)j * kGroupThreads < p_lo ? 0u : n_buckets) + b[j]], 1u);
     }
     __syncthreads();
     u32 count = 0;
-    for (u32 b = tid; b < n_buckets; b += blockDim.x) {
+    for (u32 b = tid; b < n_buckets; b += kGroupThreads) {
         u32 bef = 0, aft = 0;
         for (u32 r = 0; r < reps; r++) {
             bef += g.hist[r * rstride + b];
@@ -649,7 +652,7 @@ __device__ __forceinline__ void group_slots_part(GroupLds &g, u32 *off, u32 n, u
             g.base[n_buckets] = total;
         }
     }
-    for (u32 i = tid; i < chunks * n_buckets; i += blockDim.x) g.hist[i] = 0; // (its readers passed the scan's barriers)
+    for (u32 i = tid; i < chunks * n_buckets; i += kGroupThreads) g.hist[i] = 0; // (its readers passed the scan's barriers)
     __syncthreads();
     if (p_lo >= n) return; // a workgroup past the last part: the bounds only
     // this part once more, a sub-part a wave
@@ -663,7 +666,7 @@ __device__ __forceinline__ void group_slots_part(GroupLds &g, u32 *off, u32 n, u
             if (b != kNoBucket && lane == (u32)__builtin_ctzll(same)) atomicAdd(&g.hist[wave * n_buckets + b], (u32)__builtin_popcountll(same));
         }
     __syncthreads();
-    for (u32 b = tid; b < n_buckets; b += blockDim.x) { // a sub-part's count -> its first place in the list
+    for (u32 b = tid; b < n_buckets; b += kGroupThreads) { // a sub-part's count -> its first place in the list
         u32 sum = g.base[b] + off[b];
         for (u32 c = 0; c < chunks; c++) {
             const u32 v = g.hist[c * n_buckets + b];

@@ -29,7 +29,7 @@ HIDDEN, FF, N_EXPERTS, TOP_K = 2048, 768, 128, 8
 HBM_PEAK_GBS = 8000.0
 # HBM bytes a launch of the headline configuration's dominant kernel moves (read + written), from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE summary under profiles/ (counter x the copy-kernel calibration measured in the same run).
-GATE_UP_X_TRAFFIC_BYTES = 14430300
+GATE_UP_X_TRAFFIC_BYTES = 14425174
 
 
 def host_threads():

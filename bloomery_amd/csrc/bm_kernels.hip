@@ -157,22 +157,28 @@ hipError_t q82_tables(const Launch &L, uint8_t *act, int m, int k) {
 
 // y[row * m_total + col0 + c] = row . column (col0 + c), c < m <= M. A quad a row, 64 rows a workgroup. M = 1 is the
 // one-column form of the row dot, which reads a super-block's activation operands a super-block ahead.
-template <int WT, int U, int NB, int M>
-__global__ __launch_bounds__(256) void k_gemv(const uint8_t *w, long rows, int nb, const uint8_t *act, int m_total,
-                                              int col0, int m, float *y) {
+// T: the workgroup's threads, T / 4 rows: 256, or 64 for a matrix of so few rows that workgroups of 64 rows would leave most of
+// the card idle (768 rows are 12 of them, on 12 of 256 compute units, each streaming its 64 rows through one address unit).
+template <int WT, int U, int NB, int M, int T = 256>
+__global__ __launch_bounds__(T) void k_gemv(const uint8_t *w, long rows, int nb, const uint8_t *act, int m_total,
+                                            int col0, int m, float *y) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, q = tid & 3;
-    const long row = (long)blockIdx.x * 64 + (tid >> 2);
+    const long row = (long)blockIdx.x * (T / 4) + (tid >> 2);
     const bool active = row < rows;
     const int n = NB > 0 ? NB : nb;
     const size_t row_bytes = (size_t)n * bm_block_bytes<WT>();
     const int col_bytes = bm_act_col_bytes<WT>(n);
     const uint8_t *wrow = w + (size_t)(active ? row : 0) * row_bytes;
+    // the columns' first bytes are asked for in front of the rows (vector loads come back in the order they were asked for:
+    // behind the rows' requests the columns would wait for those as well); what a thread's few loads do not cover comes after
+    Stage<(T == 64 ? 5 : 2), T> st;
+    st.load(act + (size_t)col0 * col_bytes, m * col_bytes);
     Blk<WT> b[U];
     preload<WT, U>(b, wrow, q);
-    const Iq2Tables tb = stage_tables<WT>(lds);
+    const Iq2Tables tb = stage_tables<WT, T>(lds);
     uint8_t *cols = lds + tab_bytes<WT>();
-    stage_bytes(cols, act + (size_t)col0 * col_bytes, m * col_bytes);
+    st.store(cols, act + (size_t)col0 * col_bytes, m * col_bytes);
     __syncthreads();
     float out[M];
     row_dot<WT, U, NB, M>(b, wrow, cols, col_bytes, m, n, q, tb, out, NoTap{});
@@ -817,6 +823,8 @@ __global__ __launch_bounds__(256) void k_gate_up_xq(const float *x, const uint8_
     }
 }
 
+// (Workgroups of 64 or 128 threads, as k_gemv takes for a matrix of few rows, measure slower here: 4.35 and 3.89 us against
+// 3.55 at 768 x 2048 - a wave then quantizes four or two times as much of the column before its first product.)
 // k_gemv with the activation quantizer folded in: grid row c is column c, an f32 row of k values that every workgroup
 // quantizes into LDS for itself (the form its weight type dots against), so a matrix-vector product from f32 is one
 // launch and no column passes through memory. With act_out the first workgroup of a column leaves its bytes there.
@@ -970,6 +978,8 @@ __global__ __launch_bounds__(64) void k_block_sums(const uint8_t *wrow, int nb, 
 
 // ---------------------------------------------------------------------------------------- launch helpers
 
+constexpr unsigned kCardUnits = 256; // compute units of the card these kernels are written for
+
 int act_col_bytes(int wtype, int k) {
     const int nb = k / 256;
     return bm_takes_q8k(wtype) ? nb * BM_Q8K_STRIDE : nb * BM_Q82_SB_EXT;
@@ -984,12 +994,21 @@ hipError_t gemv(const Launch &L, int wtype, const uint8_t *w, int64_t rows, int 
                 int col0, int m, float *y) {
     const int nb = k / 256;
     const size_t lds = tab_bytes_rt(wtype) + (size_t)m * act_col_bytes(wtype, k);
+    const bool few = m == 1 && (rows + 63) / 64 < (int64_t)kCardUnits; // one column of a matrix whose 64-row blocks do not fill the card
 #define CALL_BODY                                                                                                      \
-    auto kern = m == 1 ? k_gemv<WT, U, NB, 1> : k_gemv<WT, U, NB, 8>;                                                  \
-    hipError_t e = allow_lds(kern, lds);                                                                               \
-    if (e != hipSuccess) return e;                                                                                     \
-    hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 63) / 64)), dim3(256), lds, L.stream, w, (long)rows, nb, act,     \
-                       m_total, col0, m, y);
+    if (few) {                                                                                                         \
+        auto kern = k_gemv<WT, U, NB, 1, 64>;                                                                          \
+        hipError_t e = allow_lds(kern, lds);                                                                           \
+        if (e != hipSuccess) return e;                                                                                 \
+        hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 15) / 16)), dim3(64), lds, L.stream, w, (long)rows, nb, act,  \
+                           m_total, col0, m, y);                                                                       \
+    } else {                                                                                                           \
+        auto kern = m == 1 ? k_gemv<WT, U, NB, 1> : k_gemv<WT, U, NB, 8>;                                              \
+        hipError_t e = allow_lds(kern, lds);                                                                           \
+        if (e != hipSuccess) return e;                                                                                 \
+        hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 63) / 64)), dim3(256), lds, L.stream, w, (long)rows, nb, act, \
+                           m_total, col0, m, y);                                                                       \
+    }
     BM_DISPATCH(wtype, nb)
 #undef CALL_BODY
     return hipGetLastError();

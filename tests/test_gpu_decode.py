@@ -385,6 +385,26 @@ def test_qwen3_shaped_layer_one_token(gpu, fused):
     L.free()
 
 
+@pytest.mark.parametrize("fused", (False, True))
+def test_gate_up_over_more_slots_than_one_grid_dimension_holds(gpu, fused):
+    """bm_gate_up's grid counts the slots along its second dimension up to 32768 and the rest along the third: 4101 tokens of
+    eight slots are 32808 slots, so the last 40 lie in the second plane. A small layer, every slot against the oracle."""
+    types, hidden, ff, n_experts, m, top_k = (bm.Q4_K, bm.Q4_K, bm.Q6_K), 256, 256, 3, 4101, 8
+    L = Layer(gpu, types, hidden, ff, n_experts, 977)
+    rng = np.random.default_rng(978)
+    x = normal_f32(rng, (m, hidden))
+    ids = rng.integers(0, n_experts, size=(m, top_k)).astype(np.uint32)
+    wts = (rng.random((m, top_k), dtype=np.float32) + np.float32(0.1)).astype(np.float32)
+    y, h, act_h = run_chain(gpu, L, x, ids, wts, top_k, fused)
+    want_y, want_h = L.oracle(x, ids, wts, top_k)
+    assert_f32(h, want_h, "h")
+    for s in (0, 1, 32767, 32768, 32769, 32807):
+        assert np.array_equal(act_h[s], ora.quantize_col(types[2], want_h[s * ff:(s + 1) * ff])), f"act_h slot {s}"
+    assert_f32(y, want_y, "y")
+    assert gpu.fault() == (bm.FAULT_NONE, 0)
+    L.free()
+
+
 @pytest.mark.parametrize("types,hidden,ff,n_experts,m,top_k", (
     ((bm.Q4_K, bm.Q4_K, bm.Q6_K), 2048, 768, 12, 5, 4),
     ((bm.Q6_K, bm.Q6_K, bm.Q4_K), 512, 512, 5, 3, 2),

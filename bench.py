@@ -496,6 +496,35 @@ def bench_dsv3(args, bm, ora, threads):
     per_slot(0)
     per_slot_parity = parity_of(y2.download()[:m * hidden].reshape(m, hidden), want)
     per_slot_us = timed_graph(gpu, per_slot, 16, 128, 16)[1] * 1e3
+    # the shared expert on a stream of its own beside the routed experts (a second context; fork and join by events, one graph):
+    # the routed step without an added term, then (routed sum + shared) as a closing launch over one "slot" of weight 1
+    side = bm.Gpu(0)
+    forked, joined = gpu.event(), gpu.event()
+    y3, routed_rows = gpu.buffer(np.float32, m * sets * hidden), gpu.buffer(np.float32, m * hidden)
+
+    def two_streams(i):
+        st = i % sets
+        s_ptr, x_ptr = sel.ptr + 4 * st * n_slots, xd.ptr + 4 * st * m * hidden
+        gpu.event_record(forked)
+        side.event_wait(forked)
+        side.enqueue_quantize(x_ptr, m, act6)
+        side.enqueue_gate_up(dsg, dsu, act6, zeros, m, ff, 1, None, act_sh)
+        side.enqueue_gemv_sel(dsd, act_sh, zeros, m, hidden, sdown)
+        side.event_record(joined)
+        gpu.enqueue_moe_forward(sc, dg, du, dd, x_ptr, s_ptr, wt.ptr + 4 * st * n_slots, None, m, routed_rows)
+        gpu.event_wait(joined)
+        gpu.enqueue_combine_tokens(routed_rows, ones, sdown, hidden, 1, m, y3.ptr + 4 * st * m * hidden)
+
+    gpu.capture_begin()
+    two_streams(0)
+    g0 = gpu.capture_end()
+    gpu.graph_launch(g0)
+    gpu.sync()
+    gpu.graph_destroy(g0)
+    two_streams_parity = parity_of(y3.download()[:m * hidden].reshape(m, hidden), want)
+    two_streams_us = timed_graph(gpu, two_streams, 16, 128, 16)[1] * 1e3
+    assert side.fault() == (bm.FAULT_NONE, 0)
+    side.close()
     hit = np.mean([len(np.unique(ids[s * m:(s + 1) * m])) for s in range(sets)])
     per_expert = (2 * ff * bm.row_bytes(bm.IQ2_XXS, hidden) + hidden * bm.row_bytes(bm.IQ2_XXS, ff))
     shared_bytes = 2 * ff * bm.row_bytes(bm.Q6_K, hidden) + hidden * bm.row_bytes(bm.Q6_K, ff)
@@ -509,7 +538,10 @@ def bench_dsv3(args, bm, ora, threads):
           "algorithmic_bytes_per_step": nbytes, "hbm_tbps": ach / 1e3,
           "tile_launchers_only_ten_launches": {"us_per_step": tiles_us, "us_per_token": tiles_us / m, "parity": tiles_parity},
           "per_slot_five_launches": {"us_per_step": per_slot_us, "us_per_token": per_slot_us / m, "parity": per_slot_parity,
-                                     "note": "shared expert, then bm_moe_decode over the slots with its rows as the added term"}},
+                                     "note": "shared expert, then bm_moe_decode over the slots with its rows as the added term"},
+          "shared_expert_on_a_stream_of_its_own": {"us_per_step": two_streams_us, "us_per_token": two_streams_us / m,
+                                                   "parity": two_streams_parity,
+                                                   "note": "two contexts forked and joined by events inside one graph; nine launches"}},
          {"bound": "hbm", "kernel": "whole step (8 launches)", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
           "frac": ach / HBM_PEAK_GBS, "traffic": None}, cpu)
     gpu.close()

@@ -119,6 +119,7 @@ SYMBOLS = {
     "bm_graph_destroy": (None, [_vp]),
     "bm_event_create": (_i, [_vp, C.POINTER(_vp)]),
     "bm_event_record": (_i, [_vp, _vp]),
+    "bm_event_wait": (_i, [_vp, _vp]),
     "bm_event_elapsed_ms": (_i, [_vp, _vp, _vp, C.POINTER(C.c_float)]),
     "bm_event_destroy": (None, [_vp]),
 }
@@ -484,6 +485,10 @@ class Gpu:
 
     def event_record(self, event):
         self._check(self.lib.bm_event_record(self.ctx, event))
+
+    def event_wait(self, event):
+        """What is enqueued on this context's stream from here on waits for `event` (another context's record): Stream::wait."""
+        self._check(self.lib.bm_event_wait(self.ctx, event))
 
     def event_elapsed_ms(self, start, stop):
         ms = C.c_float()

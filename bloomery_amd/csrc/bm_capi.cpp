@@ -1369,6 +1369,11 @@ int bm_event_record(bm_ctx *ctx, bm_event *event) {
     return driver(ctx, "bm_event_record", hipEventRecord(event->ev, ctx->stream));
 }
 
+int bm_event_wait(bm_ctx *ctx, bm_event *event) {
+    if (!ctx || !event) return fail(ctx, BM_EARG, "bm_event_wait: NULL argument");
+    return driver(ctx, "bm_event_wait", hipStreamWaitEvent(ctx->stream, event->ev, 0));
+}
+
 int bm_event_elapsed_ms(bm_ctx *ctx, bm_event *start, bm_event *stop, float *ms) {
     if (!ctx || !start || !stop || !ms) return fail(ctx, BM_EARG, "bm_event_elapsed_ms: NULL argument");
     int rc = driver(ctx, "bm_event_elapsed_ms: sync", hipEventSynchronize(stop->ev));

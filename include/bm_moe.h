@@ -541,6 +541,12 @@ void bm_graph_destroy(bm_graph *graph);
 
 int bm_event_create(bm_ctx *ctx, bm_event **out);
 int bm_event_record(bm_ctx *ctx, bm_event *event);
+/* The work enqueued on the context's stream after this call waits for `event`, which another context may have recorded on
+ * its own stream (`Stream::wait`, crates/device/src/lib.rs:821, crates/gpu/src/device.rs:244): the fork and join of two
+ * streams. Under capture a wait for an event recorded on the capturing stream draws the waiting context's stream into the same
+ * graph, where the two streams' launches become branches that may run side by side (the capturing context must wait for an
+ * event recorded at the end of the other stream's work before bm_capture_end). */
+int bm_event_wait(bm_ctx *ctx, bm_event *event);
 /* Waits for `stop`, then the milliseconds from `start` to `stop`. */
 int bm_event_elapsed_ms(bm_ctx *ctx, bm_event *start, bm_event *stop, float *ms);
 void bm_event_destroy(bm_event *event);
